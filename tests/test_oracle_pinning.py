@@ -1,0 +1,379 @@
+"""Pins the CPU oracle against things that do not share its code: float64 closed
+forms, library routines, brute force on tiny inputs, invariants and the
+independent formulations (literal loop / counting sort / C).  The reference's
+own tests hold no numeric fixtures for this path, so these checks are what
+fixes the oracle.  A dropped term, wrong sign, swapped gate/up half or
+transposed weight fails at least one test here.
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import c_oracle
+from oracle import sparse_layer_oracle as O
+
+
+def g(seed):
+    return torch.Generator().manual_seed(seed)
+
+
+# ------------------------------------------------------------------ RMSNorm
+def test_rmsnorm_closed_form_f64():
+    x = torch.randn(7, 96, generator=g(0))
+    w = 1 + 0.1 * torch.randn(96, generator=g(1))
+    xd = x.double().numpy()
+    ref = xd / np.sqrt((xd ** 2).mean(-1, keepdims=True) + 1e-6) * w.double().numpy()
+    got = O.rmsnorm(x, w, 1e-6).double().numpy()
+    assert np.max(np.abs(got - ref)) <= 1e-5 * np.max(np.abs(ref))
+
+
+def test_rmsnorm_unit_rms_and_library():
+    x = torch.randn(5, 3, 128, generator=g(2)) * 3.0
+    y = O.rmsnorm(x, None, 1e-6)
+    assert torch.allclose(y.pow(2).mean(-1).sqrt(), torch.ones(5, 3), atol=1e-5)
+    w = torch.rand(128, generator=g(3)) + 0.5
+    assert torch.allclose(O.rmsnorm(x, w, 1e-6), F.rms_norm(x, (128,), w, 1e-6), rtol=1e-5, atol=1e-6)
+
+
+def test_rmsnorm_extreme_scales_and_dtype():
+    # the reference's own stability test (Src/tests/test_model.py:31-43)
+    for s in (1e-6, 1e6):
+        y = O.rmsnorm(torch.randn(2, 10, 128, generator=g(4)) * s, torch.ones(128))
+        assert torch.isfinite(y).all()
+    xb = torch.randn(4, 64, generator=g(5)).bfloat16()
+    assert O.rmsnorm(xb, torch.ones(64)).dtype == torch.bfloat16
+
+
+def test_rmsnorm_scale_equivariance():
+    x = torch.randn(3, 256, generator=g(6))
+    assert torch.allclose(O.rmsnorm(x, None), O.rmsnorm(x * 37.0, None), rtol=1e-5, atol=1e-6)
+
+
+# ------------------------------------------------------------------ RoPE table
+def test_rope_table_closed_form():
+    L, D, theta = 300, 64, 10000.0
+    cos, sin = O.rope_table(L, D, theta)
+    assert cos.shape == (L, D) and cos.dtype == torch.float32
+    for pos in (0, 1, 2, 17, 299):
+        for d in (0, 1, 5, 31):
+            ang = float(np.float32(pos)) * (1.0 / theta ** (2 * d / D))
+            for half in (0, D // 2):
+                assert abs(cos[pos, d + half].item() - math.cos(ang)) <= 2e-7
+                assert abs(sin[pos, d + half].item() - math.sin(ang)) <= 2e-7
+    assert torch.all(cos[0] == 1) and torch.all(sin[0] == 0)
+    # d = 0 has unit frequency: angle == position
+    assert abs(sin[7, 0].item() - math.sin(7.0)) <= 2e-7
+
+
+def test_rope_table_scaling_factor():
+    c1, s1 = O.rope_table(64, 32, 10000.0, scaling_factor=2.0)
+    c2, s2 = O.rope_table(32, 32, 10000.0)
+    assert torch.allclose(c1[::2], c2, atol=1e-6) and torch.allclose(s1[::2], s2, atol=1e-6)
+
+
+# ------------------------------------------------------------------ RoPE apply
+def _rot_closed_form(x, cos, sin):
+    B, Hh, L, D = x.shape
+    out = np.zeros((B, Hh, L, D))
+    xd = x.double().numpy()
+    c = cos.double().numpy()
+    s = sin.double().numpy()
+    for l in range(L):
+        for d in range(D // 2):
+            a, b = xd[:, :, l, d], xd[:, :, l, d + D // 2]
+            out[:, :, l, d] = a * c[l, d] - b * s[l, d]
+            out[:, :, l, d + D // 2] = a * s[l, d] + b * c[l, d]
+    return out
+
+
+def test_rope_apply_closed_form_and_gqa():
+    B, Hq, Hkv, L, D = 2, 4, 2, 9, 16
+    q = torch.randn(B, Hq, L, D, generator=g(7))
+    k = torch.randn(B, Hkv, L, D, generator=g(8))
+    cos, sin = O.rope_table(L, D)
+    qr, kr = O.rope_apply(q, k, cos, sin)
+    assert np.max(np.abs(qr.double().numpy() - _rot_closed_form(q, cos, sin))) < 1e-6
+    assert np.max(np.abs(kr.double().numpy() - _rot_closed_form(k, cos, sin))) < 1e-6
+    # k is independent of the number of query heads
+    _, kr2 = O.rope_apply(q[:, :1], k, cos, sin)
+    assert torch.equal(kr, kr2)
+
+
+def test_rope_invariants():
+    B, Hh, L, D = 1, 2, 33, 32
+    q = torch.randn(B, Hh, L, D, generator=g(9))
+    k = torch.randn(B, Hh, L, D, generator=g(10))
+    cos, sin = O.rope_table(L, D)
+    qr, kr = O.rope_apply(q, k, cos, sin)
+    # per-pair norm preservation (the reference's own smoke check, cuda_opt_wrapper.py:537-538)
+    def pair_norm(x):
+        return x[..., : D // 2] ** 2 + x[..., D // 2:] ** 2
+    assert torch.allclose(pair_norm(q), pair_norm(qr), rtol=1e-5, atol=1e-5)
+    # inverse rotation
+    qb, _ = O.rope_apply(qr, kr, cos, -sin)
+    assert torch.allclose(qb, q, atol=1e-5)
+    # relative-position property: <R(m)q, R(n)k> = <R(m-n)q, k>
+    qv, kv = q[0, 0, 0], k[0, 0, 0]
+    qs = qv.expand(1, 1, L, D).contiguous()
+    ks = kv.expand(1, 1, L, D).contiguous()
+    qall, kall = O.rope_apply(qs, ks, cos, sin)
+    m, n = 20, 7
+    lhs = (qall[0, 0, m] * kall[0, 0, n]).sum()
+    rhs = (qall[0, 0, m - n] * kv).sum()
+    assert abs(lhs.item() - rhs.item()) < 1e-4
+
+
+def test_fused_rope_matches_full_table_form():
+    B, Hq, Hkv, L, D = 1, 2, 1, 6, 8
+    q = torch.randn(B, Hq, L, D, generator=g(11))
+    k = torch.randn(B, Hkv, L, D, generator=g(12))
+    ch, sh = O.fused_rope_table(32, D)
+    off = 5
+    qf, kf = O.fused_rope_apply(q, k, ch, sh, off)
+    cos = torch.cat([ch, ch], -1)[off:off + L]
+    sin = torch.cat([sh, sh], -1)[off:off + L]
+    qr, kr = O.rope_apply(q, k, cos, sin)
+    assert torch.equal(qf, qr) and torch.equal(kf, kr)
+    # half table agrees with the float64-derived one to float32 trig accuracy at small angles
+    c64, s64 = O.rope_table(32, D)
+    assert torch.allclose(ch, c64[:, : D // 2], atol=1e-5)
+
+
+def test_rope_bf16_single_rounding():
+    q = torch.randn(1, 2, 4, 8, generator=g(13)).bfloat16()
+    k = torch.randn(1, 1, 4, 8, generator=g(14)).bfloat16()
+    cos, sin = O.rope_table(4, 8)
+    qr, kr = O.rope_apply(q, k, cos, sin)
+    assert qr.dtype == torch.bfloat16
+    q32, _ = O.rope_apply(q.float(), k.float(), cos, sin)
+    assert torch.equal(qr, q32.bfloat16())
+
+
+# ------------------------------------------------------------------ router + routing
+def test_router_logits_f64():
+    x = torch.randn(33, 40, generator=g(15))
+    w = torch.randn(6, 40, generator=g(16)) * 0.02
+    ref = x.double() @ w.double().T
+    assert torch.allclose(O.router_logits(x, w).double(), ref, rtol=1e-5, atol=1e-7)
+
+
+def _brute_topk(vals, k):
+    # full descending sort, lower index first among equals
+    order = sorted(range(len(vals)), key=lambda i: (-vals[i], i))
+    return order[:k]
+
+
+@pytest.mark.parametrize("E,k", [(4, 1), (4, 2), (8, 2), (8, 3), (64, 6)])
+def test_routing_brute_force(E, k):
+    logits = torch.randn(50, E, generator=g(17 + E + k))
+    for temp in (1.0, 0.7):
+        i1, w1 = O.route_softmax_topk_renorm(logits, k, temp)
+        i2, w2 = O.route_topk_softmax(logits, k, temp)
+        assert torch.equal(i1, i2)
+        for t in range(50):
+            row = (logits[t].double() / temp)
+            assert i1[t].tolist() == _brute_topk(row.tolist(), k)
+            p = torch.softmax(row, -1)
+            sel = p[i1[t]]
+            assert torch.allclose(w1[t].double(), sel / sel.sum(), atol=1e-6)
+            assert torch.allclose(w2[t].double(), torch.softmax(row[i2[t]], -1), atol=1e-6)
+        assert torch.allclose(w1.sum(-1), torch.ones(50), atol=1e-5)
+        assert torch.allclose(w2.sum(-1), torch.ones(50), atol=1e-5)
+        assert torch.allclose(w1, w2, atol=1e-6)
+        assert i1.dtype == torch.int64
+
+
+def test_capacity_known_values():
+    assert O.capacity(512, 2, 8, 1.25) == 160
+    assert O.capacity(64, 2, 8, 1.25) == 20
+    assert O.capacity(16384, 2, 8, 1.25) == 5120
+    assert O.capacity(4096, 6, 64, 1.5) == 576
+    assert O.capacity(512, 2, 8, 1.1) == 140      # 140.8 truncates; 128*1.1 is not 141
+    assert O.capacity(7, 2, 4, 1.25) == 4
+
+
+# ------------------------------------------------------------------ dispatch
+@pytest.mark.parametrize("T,E,k,C", [(16, 4, 2, 5), (16, 8, 3, 4), (9, 4, 1, 100), (12, 4, 2, 0),
+                                     (40, 8, 2, 10), (64, 64, 6, 9)])
+def test_dispatch_three_formulations(T, E, k, C):
+    gen = g(100 + T + E + k + C)
+    logits = torch.randn(T, E, generator=gen)
+    idx = torch.topk(logits, k, -1)[1]
+    x = torch.randn(T, 6, generator=gen)
+    ei_l, tm_l = O.dispatch_loop(x, idx, E, C)
+    ei_v, tm_v = O.dispatch_vectorized(x, idx, E, C)
+    tm_c, slot_c, hist_c, kept_c, dropped_c = c_oracle.fcfs_dispatch(idx.numpy(), E, C)
+    assert torch.equal(tm_l, tm_v) and torch.equal(ei_l, ei_v)
+    assert np.array_equal(tm_l.numpy(), tm_c)
+    _, slot_v, hist_v, kept_v = O.dispatch_plan_vectorized(idx, E, C)
+    assert np.array_equal(slot_v.numpy(), slot_c)
+    assert np.array_equal(hist_v.numpy(), hist_c) and np.array_equal(kept_v.numpy(), kept_c)
+    # invariants
+    hist = torch.bincount(idx.reshape(-1), minlength=E)
+    assert np.array_equal(hist.numpy(), hist_c)
+    assert np.array_equal(np.minimum(hist.numpy(), C), kept_c)
+    assert kept_c.sum() + dropped_c == T * k
+    for e in range(E):
+        row = tm_c[e]
+        n = kept_c[e]
+        assert (row[:n] >= 0).all() and (row[n:] == -1).all()
+        assert (np.diff(row[:n]) > 0).all()
+        assert all(idx.reshape(-1)[m] == e for m in row[:n])
+    occ = tm_c[tm_c >= 0]
+    assert len(set(occ.tolist())) == len(occ)
+    # padded rows are zero, occupied rows are the source tokens
+    for e in range(E):
+        for pos in range(C):
+            m = tm_c[e, pos]
+            if m < 0:
+                assert torch.all(ei_l[e, pos] == 0)
+            else:
+                assert torch.equal(ei_l[e, pos], x[m // k])
+
+
+def test_dispatch_special_cases():
+    # everything to one expert: first C assignments in order survive
+    idx = torch.zeros(10, 1, dtype=torch.int64)
+    tm, slot, hist, kept, dropped = c_oracle.fcfs_dispatch(idx.numpy(), 4, 3)
+    assert tm[0].tolist() == [0, 1, 2] and dropped == 7 and hist[0] == 10
+    assert slot.tolist() == [0, 1, 2] + [-1] * 7
+    # hand-worked example, T=4, k=2, E=3, C=2
+    idx = torch.tensor([[0, 1], [0, 2], [0, 1], [1, 2]])
+    tm, slot, hist, kept, dropped = c_oracle.fcfs_dispatch(idx.numpy(), 3, 2)
+    assert tm.tolist() == [[0, 2], [1, 5], [3, 7]]
+    assert slot.tolist() == [0, 0, 1, 0, -1, 1, -1, 1]
+    assert hist.tolist() == [3, 3, 2] and kept.tolist() == [2, 2, 2] and dropped == 2
+
+
+# ------------------------------------------------------------------ experts
+def test_swiglu_expert_f64():
+    H, I = 12, 20
+    x = torch.randn(5, H, generator=g(20))
+    wgu = torch.randn(2 * I, H, generator=g(21)) * 0.3
+    wd = torch.randn(H, I, generator=g(22)) * 0.3
+    xd = x.double()
+    gate = xd @ wgu[:I].double().T
+    up = xd @ wgu[I:].double().T
+    ref = ((gate / (1 + torch.exp(-gate))) * up) @ wd.double().T
+    assert torch.allclose(O.swiglu_expert(x, wgu, wd).double(), ref, rtol=1e-5, atol=1e-6)
+    # swapping the halves must change the answer (guards the gate/up convention)
+    swapped = torch.cat([wgu[I:], wgu[:I]], 0)
+    assert not torch.allclose(O.swiglu_expert(x, swapped, wd).double(), ref, rtol=1e-3, atol=1e-4)
+
+
+# ------------------------------------------------------------------ combine + whole layer
+def _tiny_layer(seed, T=24, H=16, I=24, E=4):
+    gen = g(seed)
+    x = torch.randn(T, H, generator=gen)
+    wg = torch.randn(E, H, generator=gen) * 0.5
+    wgu = [torch.randn(2 * I, H, generator=gen) * 0.2 for _ in range(E)]
+    wd = [torch.randn(H, I, generator=gen) * 0.2 for _ in range(E)]
+    return x, wg, wgu, wd
+
+
+def test_combine_formulations_and_linearity():
+    x, wg, wgu, wd = _tiny_layer(30)
+    r = O.moe_forward_capacity(x, wg, wgu, wd, k=2, capacity_factor=0.75, literal_loops=True)
+    assert (r["slot"] < 0).any(), "case must drop something"
+    T, k = r["indices"].shape
+    out_v = O.combine_vectorized(r["expert_outputs"], r["token_map"], r["weights"], T, k)
+    assert torch.equal(out_v, r["out"])
+    out_c = c_oracle.combine_f32(r["expert_outputs"].numpy(), r["token_map"].numpy(),
+                                 r["weights"].numpy(), T, k)
+    assert np.array_equal(out_c, r["out"].numpy())
+    out2 = O.combine_loop(r["expert_outputs"], r["token_map"], 2.0 * r["weights"], T, k)
+    assert torch.allclose(out2, 2.0 * r["out"], rtol=1e-6, atol=1e-7)
+    # brute force: sum over kept assignments
+    bf = torch.zeros_like(r["out"]).double()
+    for a in range(T * k):
+        s = r["slot"][a].item()
+        if s >= 0:
+            e = r["indices"].reshape(-1)[a].item()
+            bf[a // k] += r["weights"].reshape(-1)[a].double() * r["expert_outputs"][e, s].double()
+    assert torch.allclose(r["out"].double(), bf, rtol=1e-5, atol=1e-6)
+    # fully dropped tokens stay zero; weights not renormalised
+    for t in range(T):
+        if (r["slot"][t * k:(t + 1) * k] < 0).all():
+            assert torch.all(r["out"][t] == 0)
+
+
+def test_capacity_layer_equals_nocap_when_nothing_dropped():
+    x, wg, wgu, wd = _tiny_layer(31)
+    a = O.moe_forward_capacity(x, wg, wgu, wd, k=2, capacity_factor=100.0, literal_loops=True)
+    b = O.moe_forward_nocap(x, wg, wgu, wd, k=2)
+    assert torch.equal(a["indices"], b["indices"])
+    assert (a["slot"] >= 0).all()
+    assert torch.allclose(a["out"], b["out"], rtol=1e-5, atol=1e-6)
+    assert torch.equal(a["aux"], b["aux"])
+
+
+def test_nocap_dense_brute_force():
+    x, wg, wgu, wd = _tiny_layer(32)
+    r = O.moe_forward_nocap(x.view(2, 12, 16), wg, wgu, wd, k=2)
+    assert r["out"].shape == (2, 12, 16)
+    dense = torch.zeros(24, 16, dtype=torch.float64)
+    for e in range(4):
+        y = O.swiglu_expert(x, wgu[e], wd[e]).double()
+        wsel = ((r["indices"] == e).double() * r["weights"].double()).sum(-1, keepdim=True)
+        dense += wsel * y
+    assert torch.allclose(r["out"].reshape(24, 16).double(), dense, rtol=1e-5, atol=1e-6)
+
+
+def test_aux_loss_uniform_and_closed_form():
+    E, T, k = 8, 64, 2
+    logits = torch.zeros(T, E)                       # uniform importance 1/E
+    idx = torch.stack([torch.arange(T) % E, (torch.arange(T) + 1) % E], -1)   # uniform usage
+    assert abs(O.aux_loss(logits, idx, E, 0.01).item() - 0.01) < 1e-8
+    logits = torch.randn(T, E, generator=g(33))
+    idx = torch.topk(logits, k, -1)[1]
+    usage = torch.bincount(idx.reshape(-1), minlength=E).double() / (T * k)
+    imp = torch.softmax(logits.double(), -1).mean(0)
+    ref = min(float((usage * imp).sum() * E * 0.01), 1.0)
+    assert abs(O.aux_loss(logits, idx, E, 0.01).item() - ref) < 1e-7
+    assert O.aux_loss(logits, idx, E, 1e6).item() == 1.0     # clamp
+
+
+def test_temperature_changes_weights_not_indices():
+    x, wg, wgu, wd = _tiny_layer(34)
+    a = O.moe_forward_capacity(x, wg, wgu, wd, k=2, temperature=1.0)
+    b = O.moe_forward_capacity(x, wg, wgu, wd, k=2, temperature=2.0)
+    assert torch.equal(a["indices"], b["indices"])
+    assert not torch.allclose(a["weights"], b["weights"])
+
+
+# ------------------------------------------------------------------ MoD
+def test_mod_eval_mask_threshold():
+    p = torch.rand(2, 16, 1, generator=g(35))
+    mask = O.mod_router_eval_mask(p, 0.5)
+    n, cap = 32, 16
+    srt = sorted(p.flatten().tolist())
+    thr = srt[max(1, n - cap) - 1]
+    assert mask.flatten().tolist() == [1.0 if v >= thr else 0.0 for v in p.flatten().tolist()]
+    assert int(mask.sum()) == cap + 1        # the reference's off-by-one
+
+
+def test_mod_select_per_sequence():
+    s = torch.randn(3, 40, generator=g(36))
+    sel = O.mod_select_per_sequence(s, 5)
+    for b in range(3):
+        order = sorted(range(40), key=lambda i: (-s[b, i].item(), i))[:5]
+        assert sel[b].tolist() == sorted(order)
+    # ties go to the lower position
+    assert O.mod_select_per_sequence(torch.tensor([[1.0, 2.0, 2.0, 2.0]]), 2).tolist() == [[1, 2]]
+
+
+def test_mod_moe_block_skip_tokens_untouched():
+    gen = g(37)
+    B, L, H, I, E = 2, 16, 16, 24, 4
+    x = torch.randn(B, L, H, generator=gen)
+    wm = torch.randn(1, H, generator=gen)
+    _, wg, wgu, wd = _tiny_layer(38, H=H, I=I, E=E)
+    r = O.mod_moe_block(x, wm, None, 4, dict(gate_weight=wg, gate_up_weights=wgu, down_weights=wd,
+                                             k=2, capacity_factor=1.5))
+    keep = torch.zeros(B, L, dtype=torch.bool)
+    keep.scatter_(1, r["selected"], True)
+    assert torch.equal(r["block_out"][~keep], x[~keep])
+    assert torch.allclose(r["block_out"][keep] - x[keep], r["out"].reshape(-1, H), atol=1e-6)
