@@ -1,0 +1,86 @@
+"""ctypes binding of libats_gfx950.so.
+
+The library is the only compute path of this package: if it is missing or a
+call fails, an exception is raised.  There is no PyTorch or CPU fallback.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from ctypes import c_char_p, c_double, c_float, c_int, c_int64, c_size_t, c_void_p
+
+LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libats_gfx950.so")
+
+ATS_F32, ATS_BF16 = 0, 1
+ROUTE_SOFTMAX_TOPK, ROUTE_TOPK_SOFTMAX = 0, 1
+IDX_I32, IDX_I64 = 0, 1
+
+
+class AtsError(RuntimeError):
+    """A libats_gfx950 entry point returned an error code."""
+
+
+_SIGNATURES = {
+    "ats_version": (c_int, []),
+    "ats_last_error_string": (c_char_p, []),
+    "ats_rmsnorm_fwd": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int, c_float, c_int, c_int, c_void_p]),
+    "ats_rope_table": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_double, c_double, c_void_p]),
+    "ats_rope_fwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
+                             c_int, c_int, c_int, c_int, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int,
+                             c_void_p]),
+    "ats_router_logits": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_void_p]),
+    "ats_route_topk_workspace": (c_size_t, [c_int64, c_int]),
+    "ats_route_topk": (c_int, [c_void_p, c_int64, c_int, c_int, c_float, c_int, c_void_p, c_void_p, c_void_p,
+                               c_void_p, c_void_p, c_float, c_void_p, c_size_t, c_void_p]),
+    "ats_dispatch_plan_workspace": (c_size_t, [c_int64, c_int, c_int]),
+    "ats_dispatch_plan": (c_int, [c_void_p, c_int, c_int64, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p,
+                                  c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "ats_gather_rows": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_int64, c_int, c_int, c_void_p]),
+    "ats_invert_token_map": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p]),
+    "ats_grouped_gateup_swiglu": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
+                                          c_int64, c_int, c_int, c_int, c_void_p]),
+    "ats_grouped_down": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int, c_int,
+                                 c_int, c_int, c_void_p]),
+    "ats_combine": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_int,
+                            c_void_p]),
+    "ats_row_dot": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_int64, c_int, c_int,
+                            c_void_p]),
+    "ats_select_topk_per_sequence": (c_int, [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p]),
+    "ats_scatter_add_rows": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int, c_void_p]),
+    "ats_kth_value_mask": (c_int, [c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "ats_swiglu_mul": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int, c_void_p]),
+    "ats_debug_decode_tile": (c_int, [c_int64, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p]),
+    "ats_debug_grid_blocks": (c_int64, [c_int64, c_int, c_int, c_int, c_int, c_int]),
+}
+
+_lib = None
+
+
+def is_built() -> bool:
+    return os.path.exists(LIB_PATH)
+
+
+def load() -> ctypes.CDLL:
+    """Loads the library (once).  Raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not is_built():
+            raise AtsError(
+                f"{LIB_PATH} is missing: build it with `python -m adaptivetrainingsystem_amd.build` "
+                "(needs hipcc); this package has no fallback path")
+        lib = ctypes.CDLL(LIB_PATH)
+        for name, (res, args) in _SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = lib
+    return _lib
+
+
+def last_error() -> str:
+    return load().ats_last_error_string().decode("utf-8", "replace")
+
+
+def check(rc: int, what: str) -> None:
+    if rc != 0:
+        raise AtsError(f"{what} failed with code {rc}: {last_error()}")

@@ -1,0 +1,529 @@
+// Capacity dispatch plan, row gather, token-map inversion and token-major
+// combine for gfx950.
+//
+// The plan is a stable counting sort of the T*k assignments by expert id, in
+// (token, choice) order, so that the slot of an assignment equals the number of
+// earlier assignments to the same expert - exactly what a sequential
+// first-come-first-served loop produces, but without ordered atomics:
+//   1. per-chunk histograms (chunk = kPlanChunk consecutive assignments),
+//   2. an exclusive scan over chunks per expert (+ totals, kept, offsets),
+//   3. per-chunk ranking: inside a wave the rank among equal ids comes from
+//      ballots; across the steps of a wave and the waves of a block from small
+//      LDS counters that are only ever advanced in program order.
+// A single chunk (T*k <= kPlanChunk) runs all three steps in one launch.
+#include <limits.h>
+
+#include "ats_common.hpp"
+
+namespace ats {
+
+constexpr int kPlanChunk = 1024;     // assignments per block
+constexpr int kPlanPerWave = 256;    // assignments per wave (4 steps of 64)
+constexpr int kPlanMaxE = 1024;
+
+template <typename IdxT>
+__device__ __forceinline__ int load_expert(const IdxT* idx, int64_t a, int64_t n, int E, bool* bad) {
+    if (a >= n) return -1;
+    const long long e = (long long)idx[a];
+    if (e < 0 || e >= E) {
+        *bad = true;
+        return -1;
+    }
+    return (int)e;
+}
+
+// step 1: counts of one chunk into LDS (s_cnt[w*E + e] per wave), returns via LDS
+template <typename IdxT>
+__device__ void chunk_wave_counts(const IdxT* idx, int64_t n, int E, int64_t chunk_base, int* s_cnt, bool* bad) {
+    const int lane = lane_id();
+    const int wave = threadIdx.x >> 6;
+    for (int i = threadIdx.x; i < 4 * E; i += 256) s_cnt[i] = 0;
+    __syncthreads();
+    for (int step = 0; step < kPlanPerWave / kWave; ++step) {
+        const int64_t a = chunk_base + wave * kPlanPerWave + step * kWave + lane;
+        const int e = load_expert(idx, a, n, E, bad);
+        if (e >= 0) atomicAdd(&s_cnt[wave * E + e], 1);
+    }
+    __syncthreads();
+}
+
+template <typename IdxT>
+__global__ __launch_bounds__(256) void plan_hist_kernel(const IdxT* __restrict__ idx, int64_t n, int E,
+                                                        int32_t* __restrict__ chunk_hist,
+                                                        int32_t* __restrict__ status) {
+    extern __shared__ int s_cnt[];
+    bool bad = false;
+    chunk_wave_counts(idx, n, E, (int64_t)blockIdx.x * kPlanChunk, s_cnt, &bad);
+    for (int e = threadIdx.x; e < E; e += 256)
+        chunk_hist[(int64_t)blockIdx.x * E + e] = s_cnt[e] + s_cnt[E + e] + s_cnt[2 * E + e] + s_cnt[3 * E + e];
+    if (bad) status[0] = 1;
+}
+
+// step 2 (one block): chunk_hist -> exclusive chunk bases (in place), hist, kept, offsets
+__device__ void scan_totals(int32_t* chunk_hist, int nchunks, int E, int C, int32_t* hist, int32_t* kept,
+                            int32_t* offsets, int* s_tot) {
+    for (int e = threadIdx.x; e < E; e += blockDim.x) {
+        int run = 0;
+        for (int c = 0; c < nchunks; ++c) {
+            const int v = chunk_hist[(int64_t)c * E + e];
+            chunk_hist[(int64_t)c * E + e] = run;
+            run += v;
+        }
+        hist[e] = run;
+        const int kp = run < C ? run : C;
+        kept[e] = kp;
+        s_tot[e] = kp;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int run = 0;
+        for (int e = 0; e < E; ++e) {
+            offsets[e] = run;
+            run += s_tot[e];
+        }
+        offsets[E] = run;
+    }
+    __syncthreads();
+}
+
+__global__ __launch_bounds__(256) void plan_scan_kernel(int32_t* __restrict__ chunk_hist, int nchunks, int E, int C,
+                                                        int32_t* __restrict__ hist, int32_t* __restrict__ kept,
+                                                        int32_t* __restrict__ offsets) {
+    extern __shared__ int s_tot[];
+    scan_totals(chunk_hist, nchunks, E, C, hist, kept, offsets, s_tot);
+}
+
+// step 3: ranks of one chunk.  s_cnt holds the per-wave counts of this chunk
+// (from chunk_wave_counts); they are turned into per-wave running bases.
+template <typename IdxT>
+__device__ void chunk_rank_and_write(const IdxT* idx, int64_t n, int k, int E, int C, int64_t chunk_base,
+                                     const int32_t* chunk_excl /* [E] for this chunk */,
+                                     const int32_t* offsets, int* s_cnt, int32_t* slot, int32_t* token_map,
+                                     int32_t* row_src, int32_t* row_of) {
+    const int lane = lane_id();
+    const int wave = threadIdx.x >> 6;
+    // per-wave running base = chunk base + counts of the earlier waves
+    for (int e = threadIdx.x; e < E; e += 256) {
+        int run = chunk_excl[e];
+        for (int w = 0; w < 4; ++w) {
+            const int v = s_cnt[w * E + e];
+            s_cnt[w * E + e] = run;
+            run += v;
+        }
+    }
+    __syncthreads();
+    int* my_base = s_cnt + wave * E;
+    const unsigned long long lt_mask = lane == 0 ? 0ull : (~0ull >> (64 - lane));
+    for (int step = 0; step < kPlanPerWave / kWave; ++step) {
+        const int64_t a = chunk_base + wave * kPlanPerWave + step * kWave + lane;
+        bool bad = false;
+        const int e = load_expert(idx, a, n, E, &bad);
+        int rank = -1;
+        unsigned long long remaining = __ballot(e >= 0);
+        while (remaining) {
+            const int leader = __ffsll((long long)remaining) - 1;
+            const int le = __shfl(e, leader, 64);
+            const unsigned long long same = __ballot(e == le);
+            if (e == le) rank = my_base[le] + __popcll(same & lt_mask);
+            remaining &= ~same;
+            // all lanes have read my_base[le]; the leader advances it for the next step
+            if (lane == leader) my_base[le] += __popcll(same);
+        }
+        if (a < n) {
+            if (e >= 0 && rank < C) {
+                const int row = offsets[e] + rank;
+                slot[a] = rank;
+                token_map[(int64_t)e * C + rank] = (int32_t)a;
+                row_src[row] = (int32_t)a;
+                row_of[a] = row;
+            } else {
+                slot[a] = -1;
+                row_of[a] = -1;
+            }
+        }
+    }
+}
+
+template <typename IdxT>
+__global__ __launch_bounds__(256) void plan_rank_kernel(const IdxT* __restrict__ idx, int64_t n, int k, int E, int C,
+                                                        const int32_t* __restrict__ chunk_excl,
+                                                        const int32_t* __restrict__ kept,
+                                                        const int32_t* __restrict__ offsets,
+                                                        int32_t* __restrict__ slot, int32_t* __restrict__ token_map,
+                                                        int32_t* __restrict__ row_src, int32_t* __restrict__ row_of,
+                                                        int64_t row_src_len) {
+    extern __shared__ int s_cnt[];
+    bool bad = false;
+    const int64_t chunk_base = (int64_t)blockIdx.x * kPlanChunk;
+    chunk_wave_counts(idx, n, E, chunk_base, s_cnt, &bad);
+    chunk_rank_and_write(idx, n, k, E, C, chunk_base, chunk_excl + (int64_t)blockIdx.x * E, offsets, s_cnt, slot,
+                         token_map, row_src, row_of);
+    // empty slots and unused compact rows
+    const int64_t stride = (int64_t)gridDim.x * 256;
+    const int64_t ec = (int64_t)E * C;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < ec; i += stride) {
+        const int e = (int)(i / C);
+        const int pos = (int)(i - (int64_t)e * C);
+        if (pos >= kept[e]) token_map[i] = -1;
+    }
+    const int total = offsets[E];
+    for (int64_t i = total + (int64_t)blockIdx.x * 256 + threadIdx.x; i < row_src_len; i += stride) row_src[i] = -1;
+}
+
+// Whole plan in one block (n <= kPlanChunk).
+template <typename IdxT>
+__global__ __launch_bounds__(256) void plan_single_kernel(const IdxT* idx, int64_t n, int k, int E,
+                                                          int C, int32_t* chunk_hist,
+                                                          int32_t* hist, int32_t* kept,
+                                                          int32_t* offsets, int32_t* slot,
+                                                          int32_t* token_map,
+                                                          int32_t* row_src, int32_t* row_of,
+                                                          int64_t row_src_len, int32_t* status) {
+    extern __shared__ int s_all[];
+    int* s_cnt = s_all;          // [4*E]
+    int* s_tot = s_all + 4 * E;  // [E]
+    bool bad = false;
+    chunk_wave_counts(idx, n, E, 0, s_cnt, &bad);
+    if (bad) status[0] = 1;
+    for (int e = threadIdx.x; e < E; e += 256)
+        chunk_hist[e] = s_cnt[e] + s_cnt[E + e] + s_cnt[2 * E + e] + s_cnt[3 * E + e];
+    __syncthreads();
+    scan_totals(chunk_hist, 1, E, C, hist, kept, offsets, s_tot);
+    __threadfence_block();
+    chunk_rank_and_write(idx, n, k, E, C, 0, chunk_hist, offsets, s_cnt, slot, token_map, row_src, row_of);
+    const int64_t ec = (int64_t)E * C;
+    for (int64_t i = threadIdx.x; i < ec; i += 256) {
+        const int e = (int)(i / C);
+        const int pos = (int)(i - (int64_t)e * C);
+        if (pos >= kept[e]) token_map[i] = -1;
+    }
+    const int total = offsets[E];
+    for (int64_t i = total + threadIdx.x; i < row_src_len; i += 256) row_src[i] = -1;
+}
+
+__global__ void plan_clear_status_kernel(int32_t* status) { status[0] = 0; }
+
+// ------------------------------------------------------------------ row gather
+// One wave per output row; 16-byte accesses; zero rows for negative map entries.
+template <typename T>
+__global__ __launch_bounds__(256) void gather_rows_kernel(const T* __restrict__ src, const int32_t* __restrict__ map,
+                                                          int div, T* __restrict__ out, int64_t n_rows, int H,
+                                                          bool vec) {
+    constexpr int V = Elem<T>::kVec;
+    const int lane = lane_id();
+    const int64_t wave = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    const int64_t nwaves = (int64_t)gridDim.x * (blockDim.x >> 6);
+    for (int64_t r = wave; r < n_rows; r += nwaves) {
+        const int m = map[r];
+        const int64_t srow = m < 0 ? -1 : (int64_t)(m / div);
+        if (vec) {
+            const int nvec = H / V;
+            uint4* o = reinterpret_cast<uint4*>(out + r * H);
+            if (srow < 0) {
+                for (int v = lane; v < nvec; v += kWave) o[v] = make_uint4(0, 0, 0, 0);
+            } else {
+                const uint4* s = reinterpret_cast<const uint4*>(src + srow * H);
+                for (int v = lane; v < nvec; v += kWave) o[v] = s[v];
+            }
+        } else {
+            for (int h = lane; h < H; h += kWave) {
+                if (srow < 0) Elem<T>::store(out + r * H + h, 0.f);
+                else out[r * H + h] = src[srow * H + h];
+            }
+        }
+    }
+}
+
+__global__ __launch_bounds__(256) void fill_i32_kernel(int32_t* p, int64_t n, int32_t v) {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
+        p[i] = v;
+}
+__global__ __launch_bounds__(256) void invert_map_kernel(const int32_t* __restrict__ token_map, int64_t n_slots,
+                                                         int32_t* __restrict__ row_of, int64_t n_assign) {
+    for (int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; r < n_slots;
+         r += (int64_t)gridDim.x * blockDim.x) {
+        const int m = token_map[r];
+        if (m >= 0 && m < n_assign) row_of[m] = (int32_t)r;
+    }
+}
+
+// ------------------------------------------------------------------ combine
+// One wave per token.  Lanes 0..k-1 hold (row, weight) of the k choices and
+// rank them by row; rows then come out in ascending order as wave-uniform
+// values, and every lane accumulates its 16-byte column slices in float32 with
+// separately rounded product and sum.
+template <typename TY, typename TO>
+__global__ __launch_bounds__(256) void combine_kernel(const TY* __restrict__ y, const int32_t* __restrict__ row_of,
+                                                      const float* __restrict__ w, const TO* __restrict__ residual,
+                                                      TO* __restrict__ out, int64_t T, int k, int H) {
+    const int lane = lane_id();
+    const int64_t wave = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    const int64_t nwaves = (int64_t)gridDim.x * (blockDim.x >> 6);
+    for (int64_t t = wave; t < T; t += nwaves) {
+        int my_row = -1;
+        float my_w = 0.f;
+        if (lane < k) {
+            my_row = row_of[t * k + lane];
+            my_w = w[t * k + lane];
+        }
+        // position of this lane's row among the kept rows of the token
+        int my_rank = 0;
+        for (int j = 0; j < k; ++j) {
+            const int rj = __shfl(my_row, j, 64);
+            if (rj >= 0 && (rj < my_row || (rj == my_row && j < lane))) ++my_rank;
+        }
+        const int n_kept = __popcll(__ballot(my_row >= 0));
+        for (int h0 = lane * 4; h0 < H; h0 += kWave * 4) {
+            float acc[4] = {0.f, 0.f, 0.f, 0.f};
+            const int nh = min(4, H - h0);
+            for (int n = 0; n < n_kept; ++n) {
+                const unsigned long long who = __ballot(my_row >= 0 && my_rank == n);
+                const int src = __ffsll((long long)who) - 1;
+                const int64_t row = __shfl(my_row, src, 64);
+                const float wt = __shfl(my_w, src, 64);
+                const TY* yr = y + row * H + h0;
+                for (int j = 0; j < nh; ++j) acc[j] = __fadd_rn(acc[j], __fmul_rn(wt, Elem<TY>::load(yr + j)));
+            }
+            for (int j = 0; j < nh; ++j) {
+                float v = acc[j];
+                if (residual) v = __fadd_rn(Elem<TO>::load(residual + t * H + h0 + j), v);
+                Elem<TO>::store(out + t * H + h0 + j, v);
+            }
+        }
+    }
+}
+
+// Vector form: H multiple of the 16-byte vector width of both types, aligned.
+template <typename TY, typename TO, int MAXK>
+__global__ __launch_bounds__(256) void combine_vec_kernel(const TY* __restrict__ y, const int32_t* __restrict__ row_of,
+                                                          const float* __restrict__ w,
+                                                          const TO* __restrict__ residual, TO* __restrict__ out,
+                                                          int64_t T, int k, int H) {
+    constexpr int V = 8;  // columns per lane per step (one 16-byte bf16 vector or two float vectors)
+    const int lane = lane_id();
+    const int64_t wave = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    const int64_t nwaves = (int64_t)gridDim.x * (blockDim.x >> 6);
+    for (int64_t t = wave; t < T; t += nwaves) {
+        int my_row = -1;
+        float my_w = 0.f;
+        if (lane < k) {
+            my_row = row_of[t * k + lane];
+            my_w = w[t * k + lane];
+        }
+        int my_rank = 0;
+        for (int j = 0; j < k; ++j) {
+            const int rj = __shfl(my_row, j, 64);
+            if (rj >= 0 && (rj < my_row || (rj == my_row && j < lane))) ++my_rank;
+        }
+        const int n_kept = __popcll(__ballot(my_row >= 0));
+        int64_t rows[MAXK];
+        float wts[MAXK];
+#pragma unroll
+        for (int n = 0; n < MAXK; ++n) {
+            const unsigned long long who = __ballot(my_row >= 0 && my_rank == n);
+            const int src = who ? __ffsll((long long)who) - 1 : 0;
+            rows[n] = __shfl(my_row, src, 64);
+            wts[n] = __shfl(my_w, src, 64);
+        }
+        for (int h0 = lane * V; h0 < H; h0 += kWave * V) {
+            float acc[V];
+#pragma unroll
+            for (int j = 0; j < V; ++j) acc[j] = 0.f;
+            float yv[MAXK][V];
+#pragma unroll
+            for (int n = 0; n < MAXK; ++n) {
+                if (n < n_kept) {
+                    const TY* yr = y + rows[n] * H + h0;
+                    if constexpr (sizeof(TY) == 2) {
+                        Elem<TY>::unpack(*reinterpret_cast<const uint4*>(yr), yv[n]);
+                    } else {
+                        Elem<TY>::unpack(*reinterpret_cast<const uint4*>(yr), yv[n]);
+                        Elem<TY>::unpack(*reinterpret_cast<const uint4*>(yr + 4), yv[n] + 4);
+                    }
+                }
+            }
+#pragma unroll
+            for (int n = 0; n < MAXK; ++n) {
+                if (n < n_kept) {
+#pragma unroll
+                    for (int j = 0; j < V; ++j) acc[j] = __fadd_rn(acc[j], __fmul_rn(wts[n], yv[n][j]));
+                }
+            }
+            if (residual) {
+                float rv[V];
+                const TO* rr = residual + t * H + h0;
+                if constexpr (sizeof(TO) == 2) {
+                    Elem<TO>::unpack(*reinterpret_cast<const uint4*>(rr), rv);
+                } else {
+                    Elem<TO>::unpack(*reinterpret_cast<const uint4*>(rr), rv);
+                    Elem<TO>::unpack(*reinterpret_cast<const uint4*>(rr + 4), rv + 4);
+                }
+#pragma unroll
+                for (int j = 0; j < V; ++j) acc[j] = __fadd_rn(rv[j], acc[j]);
+            }
+            TO* o = out + t * H + h0;
+            if constexpr (sizeof(TO) == 2) {
+                *reinterpret_cast<uint4*>(o) = Elem<TO>::pack(acc);
+            } else {
+                *reinterpret_cast<uint4*>(o) = Elem<TO>::pack(acc);
+                *reinterpret_cast<uint4*>(o + 4) = Elem<TO>::pack(acc + 4);
+            }
+        }
+    }
+}
+
+template <typename TY, typename TO>
+static void launch_combine(const void* y, const int32_t* row_of, const float* w, const void* residual, void* out,
+                           int64_t T, int k, int H, hipStream_t s) {
+    int64_t blocks = (T + 3) / 4;
+    if (blocks > 16384) blocks = 16384;
+    const TY* yp = static_cast<const TY*>(y);
+    const TO* rp = static_cast<const TO*>(residual);
+    TO* op = static_cast<TO*>(out);
+    const bool vec = H % 8 == 0 && aligned16(y) && aligned16(out) && (!residual || aligned16(residual)) && k <= 8;
+    if (vec && k <= 2)
+        hipLaunchKernelGGL((combine_vec_kernel<TY, TO, 2>), dim3((unsigned)blocks), dim3(256), 0, s, yp, row_of, w, rp,
+                           op, T, k, H);
+    else if (vec && k <= 4)
+        hipLaunchKernelGGL((combine_vec_kernel<TY, TO, 4>), dim3((unsigned)blocks), dim3(256), 0, s, yp, row_of, w, rp,
+                           op, T, k, H);
+    else if (vec)
+        hipLaunchKernelGGL((combine_vec_kernel<TY, TO, 8>), dim3((unsigned)blocks), dim3(256), 0, s, yp, row_of, w, rp,
+                           op, T, k, H);
+    else
+        hipLaunchKernelGGL((combine_kernel<TY, TO>), dim3((unsigned)blocks), dim3(256), 0, s, yp, row_of, w, rp, op, T,
+                           k, H);
+}
+
+}  // namespace ats
+
+extern "C" size_t ats_dispatch_plan_workspace(int64_t T, int k, int E) {
+    if (T <= 0 || k <= 0 || E <= 0) return 0;
+    const int64_t n = T * k;
+    const int64_t nchunks = (n + ats::kPlanChunk - 1) / ats::kPlanChunk;
+    return (size_t)nchunks * E * sizeof(int32_t);
+}
+
+extern "C" int ats_dispatch_plan(const void* idx, int idx_dtype, int64_t T, int k, int E, int C, int32_t* slot,
+                                 int32_t* token_map, int32_t* hist, int32_t* kept, int32_t* offsets, int32_t* row_src,
+                                 int32_t* row_of, int32_t* status, void* workspace, size_t workspace_bytes,
+                                 ats_stream_t stream) {
+    using namespace ats;
+    ATS_REQUIRE(T >= 0 && k > 0 && E > 0 && E <= kPlanMaxE && C >= 0, ATS_ERR_INVALID_ARG,
+                "ats_dispatch_plan: T=%lld k=%d E=%d C=%d (E <= %d)", (long long)T, k, E, C, kPlanMaxE);
+    ATS_REQUIRE(idx_dtype == ATS_IDX_I32 || idx_dtype == ATS_IDX_I64, ATS_ERR_INVALID_ARG,
+                "ats_dispatch_plan: idx dtype tag %d", idx_dtype);
+    ATS_REQUIRE(T * (int64_t)k < (int64_t)INT_MAX && (int64_t)E * C < (int64_t)INT_MAX, ATS_ERR_UNSUPPORTED,
+                "ats_dispatch_plan: T*k and E*C must fit in int32");
+    ATS_REQUIRE(slot && token_map && hist && kept && offsets && row_src && row_of && status, ATS_ERR_INVALID_ARG,
+                "ats_dispatch_plan: null output pointer");
+    ATS_REQUIRE(T == 0 || idx, ATS_ERR_INVALID_ARG, "ats_dispatch_plan: null idx");
+    const int64_t n = T * k;
+    const int64_t nchunks = n == 0 ? 1 : (n + kPlanChunk - 1) / kPlanChunk;
+    const size_t need = (size_t)nchunks * E * sizeof(int32_t);
+    ATS_REQUIRE(workspace && workspace_bytes >= need, ATS_ERR_WORKSPACE,
+                "ats_dispatch_plan: workspace %zu bytes, need %zu", workspace_bytes, need);
+    hipStream_t s = as_stream(stream);
+    int32_t* chunk_hist = static_cast<int32_t*>(workspace);
+    int64_t row_src_len = n < (int64_t)E * C ? n : (int64_t)E * C;
+    if (row_src_len < 1) row_src_len = 1;
+    hipLaunchKernelGGL(plan_clear_status_kernel, dim3(1), dim3(1), 0, s, status);
+    const size_t smem = (size_t)5 * E * sizeof(int);
+    if (nchunks == 1) {
+        if (idx_dtype == ATS_IDX_I32)
+            hipLaunchKernelGGL((plan_single_kernel<int32_t>), dim3(1), dim3(256), smem, s,
+                               static_cast<const int32_t*>(idx), n, k, E, C, chunk_hist, hist, kept, offsets, slot,
+                               token_map, row_src, row_of, row_src_len, status);
+        else
+            hipLaunchKernelGGL((plan_single_kernel<int64_t>), dim3(1), dim3(256), smem, s,
+                               static_cast<const int64_t*>(idx), n, k, E, C, chunk_hist, hist, kept, offsets, slot,
+                               token_map, row_src, row_of, row_src_len, status);
+        ATS_CHECK_LAUNCH("ats_dispatch_plan(single)");
+        return ATS_OK;
+    }
+    if (idx_dtype == ATS_IDX_I32)
+        hipLaunchKernelGGL((plan_hist_kernel<int32_t>), dim3((unsigned)nchunks), dim3(256), smem, s,
+                           static_cast<const int32_t*>(idx), n, E, chunk_hist, status);
+    else
+        hipLaunchKernelGGL((plan_hist_kernel<int64_t>), dim3((unsigned)nchunks), dim3(256), smem, s,
+                           static_cast<const int64_t*>(idx), n, E, chunk_hist, status);
+    ATS_CHECK_LAUNCH("ats_dispatch_plan(hist)");
+    hipLaunchKernelGGL(plan_scan_kernel, dim3(1), dim3(256), (size_t)E * sizeof(int), s, chunk_hist, (int)nchunks, E,
+                       C, hist, kept, offsets);
+    ATS_CHECK_LAUNCH("ats_dispatch_plan(scan)");
+    if (idx_dtype == ATS_IDX_I32)
+        hipLaunchKernelGGL((plan_rank_kernel<int32_t>), dim3((unsigned)nchunks), dim3(256), smem, s,
+                           static_cast<const int32_t*>(idx), n, k, E, C, chunk_hist, kept, offsets, slot, token_map,
+                           row_src, row_of, row_src_len);
+    else
+        hipLaunchKernelGGL((plan_rank_kernel<int64_t>), dim3((unsigned)nchunks), dim3(256), smem, s,
+                           static_cast<const int64_t*>(idx), n, k, E, C, chunk_hist, kept, offsets, slot, token_map,
+                           row_src, row_of, row_src_len);
+    ATS_CHECK_LAUNCH("ats_dispatch_plan(rank)");
+    return ATS_OK;
+}
+
+extern "C" int ats_gather_rows(const void* src, const int32_t* map, int div, void* out, int64_t n_rows, int H,
+                               int dtype, ats_stream_t stream) {
+    using namespace ats;
+    ATS_REQUIRE(n_rows >= 0 && H > 0 && div > 0, ATS_ERR_INVALID_ARG, "ats_gather_rows: n_rows=%lld H=%d div=%d",
+                (long long)n_rows, H, div);
+    ATS_REQUIRE(dtype == ATS_F32 || dtype == ATS_BF16, ATS_ERR_UNSUPPORTED, "ats_gather_rows: dtype tag %d", dtype);
+    if (n_rows == 0) return ATS_OK;
+    ATS_REQUIRE(src && map && out, ATS_ERR_INVALID_ARG, "ats_gather_rows: null pointer");
+    int64_t blocks = (n_rows + 3) / 4;
+    if (blocks > 32768) blocks = 32768;
+    const int V = dtype == ATS_F32 ? 4 : 8;
+    const bool vec = H % V == 0 && aligned16(src) && aligned16(out);
+    if (dtype == ATS_F32)
+        hipLaunchKernelGGL((gather_rows_kernel<float>), dim3((unsigned)blocks), dim3(256), 0, as_stream(stream),
+                           static_cast<const float*>(src), map, div, static_cast<float*>(out), n_rows, H, vec);
+    else
+        hipLaunchKernelGGL((gather_rows_kernel<bf16_t>), dim3((unsigned)blocks), dim3(256), 0, as_stream(stream),
+                           static_cast<const bf16_t*>(src), map, div, static_cast<bf16_t*>(out), n_rows, H, vec);
+    ATS_CHECK_LAUNCH("ats_gather_rows");
+    return ATS_OK;
+}
+
+extern "C" int ats_invert_token_map(const int32_t* token_map, int64_t n_slots, int32_t* row_of, int64_t n_assign,
+                                    ats_stream_t stream) {
+    using namespace ats;
+    ATS_REQUIRE(n_slots >= 0 && n_assign >= 0 && n_slots < INT_MAX, ATS_ERR_INVALID_ARG,
+                "ats_invert_token_map: n_slots=%lld n_assign=%lld", (long long)n_slots, (long long)n_assign);
+    if (n_assign == 0) return ATS_OK;
+    ATS_REQUIRE(row_of && (n_slots == 0 || token_map), ATS_ERR_INVALID_ARG, "ats_invert_token_map: null pointer");
+    hipStream_t s = as_stream(stream);
+    int64_t b1 = (n_assign + 255) / 256;
+    if (b1 > 4096) b1 = 4096;
+    hipLaunchKernelGGL(fill_i32_kernel, dim3((unsigned)b1), dim3(256), 0, s, row_of, n_assign, -1);
+    ATS_CHECK_LAUNCH("ats_invert_token_map(fill)");
+    if (n_slots > 0) {
+        int64_t b2 = (n_slots + 255) / 256;
+        if (b2 > 4096) b2 = 4096;
+        hipLaunchKernelGGL(invert_map_kernel, dim3((unsigned)b2), dim3(256), 0, s, token_map, n_slots, row_of,
+                           n_assign);
+        ATS_CHECK_LAUNCH("ats_invert_token_map");
+    }
+    return ATS_OK;
+}
+
+extern "C" int ats_combine(const void* y, const int32_t* row_of, const float* w, const void* residual, void* out,
+                           int64_t T, int k, int H, int y_dtype, int out_dtype, ats_stream_t stream) {
+    using namespace ats;
+    ATS_REQUIRE(T >= 0 && k > 0 && k <= 64 && H > 0, ATS_ERR_INVALID_ARG, "ats_combine: T=%lld k=%d H=%d",
+                (long long)T, k, H);
+    ATS_REQUIRE((y_dtype == ATS_F32 || y_dtype == ATS_BF16) && (out_dtype == ATS_F32 || out_dtype == ATS_BF16),
+                ATS_ERR_UNSUPPORTED, "ats_combine: dtype tags %d/%d", y_dtype, out_dtype);
+    if (T == 0) return ATS_OK;
+    ATS_REQUIRE(y && row_of && w && out, ATS_ERR_INVALID_ARG, "ats_combine: null pointer");
+    hipStream_t s = as_stream(stream);
+    if (y_dtype == ATS_F32 && out_dtype == ATS_F32) launch_combine<float, float>(y, row_of, w, residual, out, T, k, H, s);
+    else if (y_dtype == ATS_BF16 && out_dtype == ATS_BF16)
+        launch_combine<bf16_t, bf16_t>(y, row_of, w, residual, out, T, k, H, s);
+    else if (y_dtype == ATS_F32 && out_dtype == ATS_BF16)
+        launch_combine<float, bf16_t>(y, row_of, w, residual, out, T, k, H, s);
+    else
+        launch_combine<bf16_t, float>(y, row_of, w, residual, out, T, k, H, s);
+    ATS_CHECK_LAUNCH("ats_combine");
+    return ATS_OK;
+}

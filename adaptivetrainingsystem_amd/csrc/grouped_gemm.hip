@@ -1,0 +1,391 @@
+// Grouped expert GEMMs for gfx950 (CDNA4 MFMA, wave64).
+//
+//   gate/up + SwiGLU : h[r, i] = silu(a_r . Wgu[e][i,:]) * (a_r . Wgu[e][I+i,:])
+//   down             : y[r, :] = h[r,:] . Wd[e]^T
+//
+// Both are "NT" products: activations [rows, K] and weights [N, K] have K
+// contiguous, so both operands are fetched with 16-byte loads along K and fed to
+// v_mfma_f32_32x32x16_bf16 (bf16) or v_mfma_f32_32x32x2_f32 (f32) without any
+// transpose.  The weight fragment is passed as the first MFMA operand, so the
+// accumulator of a lane holds 4 consecutive output columns of one output row
+// and the epilogue stores 8/16 contiguous bytes per lane.
+//
+// Block tile BM x BN (BN counts weight rows; with SwiGLU the tile holds BN/2
+// gate rows and the matching BN/2 up rows, so silu(g)*u is formed in registers
+// and the [rows, 2I] intermediate never exists).  K is consumed in 128-byte
+// slabs per row, staged through LDS with a 144-byte row pitch (bank-conflict
+// free for 16-byte reads), double buffered: the global loads of slab t+1 are in
+// flight while slab t feeds the matrix cores; one barrier per slab.
+// The permutation gather is fused into the A load (row index table).
+#include <math.h>
+
+#include "ats_common.hpp"
+#include "tile_schedule.hpp"
+
+namespace ats {
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
+
+struct GroupedArgs {
+    const void* a;           // [*, K] activations
+    const int32_t* a_rows;   // optional gather table over the row space
+    int a_row_div;
+    int64_t lda;             // elements
+    const void* const* b;    // per expert weight [N_total, K]
+    void* out;               // [*, N_out]
+    int64_t ldo;
+    const int32_t* row_start;
+    const int32_t* row_count;
+    int E, K, N_out, up_offset, n_tiles;
+};
+
+constexpr int kRowPitch = 144;  // bytes per staged row: 128 data + 16 pad
+
+template <typename T>
+__device__ __forceinline__ void mma_step(const uint4& wfrag, const uint4& afrag, f32x16_t& c);
+
+template <>
+__device__ __forceinline__ void mma_step<bf16_t>(const uint4& wfrag, const uint4& afrag, f32x16_t& c) {
+    union {
+        uint4 u;
+        bf16x8_t v;
+    } w, a;
+    w.u = wfrag;
+    a.u = afrag;
+    c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(w.v, a.v, c, 0, 0, 0);
+}
+template <>
+__device__ __forceinline__ void mma_step<float>(const uint4& wfrag, const uint4& afrag, f32x16_t& c) {
+    c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(wfrag.x), __uint_as_float(afrag.x), c, 0, 0, 0);
+    c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(wfrag.y), __uint_as_float(afrag.y), c, 0, 0, 0);
+    c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(wfrag.z), __uint_as_float(afrag.z), c, 0, 0, 0);
+    c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(wfrag.w), __uint_as_float(afrag.w), c, 0, 0, 0);
+}
+
+__device__ __forceinline__ float silu_f(float g) { return g / (1.0f + expf(-g)); }
+
+template <typename TO>
+__device__ __forceinline__ void store4(TO* p, const float* v, int n_valid);
+template <>
+__device__ __forceinline__ void store4<float>(float* p, const float* v, int n_valid) {
+    if (n_valid >= 4 && (reinterpret_cast<uintptr_t>(p) & 15u) == 0) {
+        *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
+    } else {
+        for (int i = 0; i < 4; ++i)
+            if (i < n_valid) p[i] = v[i];
+    }
+}
+template <>
+__device__ __forceinline__ void store4<bf16_t>(bf16_t* p, const float* v, int n_valid) {
+    if (n_valid >= 4 && (reinterpret_cast<uintptr_t>(p) & 7u) == 0) {
+        uint2 u;
+        u.x = float_to_bf16_bits(v[0]) | (float_to_bf16_bits(v[1]) << 16);
+        u.y = float_to_bf16_bits(v[2]) | (float_to_bf16_bits(v[3]) << 16);
+        *reinterpret_cast<uint2*>(p) = u;
+    } else {
+        for (int i = 0; i < 4; ++i)
+            if (i < n_valid) p[i].bits = (uint16_t)float_to_bf16_bits(v[i]);
+    }
+}
+
+template <typename T, typename TO, int BM, int BN, int WM, int WN, int SM, int SN, bool SWIGLU>
+__global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_kernel(GroupedArgs p) {
+    constexpr int NT = WM * WN * 64;
+    constexpr int VEC = 16 / (int)sizeof(T);
+    constexpr int BK = 128 / (int)sizeof(T);
+    constexpr int TM = BM / WM / 32;
+    constexpr int TN = BN / WN / 32;
+    constexpr int RPP = NT / 8;  // rows loaded per pass (8 threads x 16 B per row)
+    constexpr int PA = BM / RPP;
+    constexpr int PB = BN / RPP;
+    constexpr int STAGE = (BM + BN) * kRowPitch;
+    static_assert(BM % (WM * 32) == 0 && BN % (WN * 32) == 0, "wave tiling");
+    static_assert(BM % RPP == 0 && BN % RPP == 0, "loader tiling");
+    static_assert(!SWIGLU || TN % 2 == 0, "SwiGLU needs gate and up tiles in the same wave");
+    static_assert(SM * SN == kSuperBlocks, "supertile");
+
+    extern __shared__ __align__(16) unsigned char smem[];
+
+    TileCoord tc;
+    if (!decode_tile(blockIdx.x, p.row_count, p.E, BM, p.n_tiles, SM, SN, &tc)) return;
+    const int count = p.row_count[tc.e];
+    const int row0 = p.row_start[tc.e];
+    const int K = p.K;
+    const T* Bexp = static_cast<const T*>(p.b[tc.e]);
+    const T* A = static_cast<const T*>(p.a);
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wm = wave / WN, wn = wave % WN;
+    const int lrow = tid >> 3;   // loader: row inside a pass
+    const int lchunk = tid & 7;  // loader: 16-byte chunk inside the 128-byte slab
+
+    // ---- loader row pointers (nullptr = row does not exist -> zeros)
+    const T* ap[PA];
+#pragma unroll
+    for (int i = 0; i < PA; ++i) {
+        const int m = tc.mt * BM + lrow + i * RPP;
+        ap[i] = nullptr;
+        if (m < count) {
+            int64_t src = row0 + m;
+            if (p.a_rows) src = p.a_rows[src] / p.a_row_div;
+            ap[i] = A + src * p.lda + lchunk * VEC;
+        }
+    }
+    constexpr int HALF = BN / 2;
+    const T* bp[PB];
+#pragma unroll
+    for (int i = 0; i < PB; ++i) {
+        const int rb = lrow + i * RPP;
+        int n, brow;
+        if (SWIGLU) {
+            const bool up = rb >= HALF;
+            n = tc.nt * HALF + (up ? rb - HALF : rb);
+            brow = up ? p.up_offset + n : n;
+        } else {
+            n = tc.nt * BN + rb;
+            brow = n;
+        }
+        bp[i] = n < p.N_out ? Bexp + (int64_t)brow * K + lchunk * VEC : nullptr;
+    }
+
+    f32x16_t acc[TN][TM];
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[j][i][v] = 0.f;
+
+    const int nk = (K + BK - 1) / BK;
+    const uint4 zero4 = make_uint4(0, 0, 0, 0);
+    uint4 ra[PA], rb[PB];
+
+#define ATS_LOAD_GLOBAL(kt_)                                                                       \
+    {                                                                                              \
+        const int koff = (kt_) * BK;                                                               \
+        const bool kok = koff + lchunk * VEC < K;                                                  \
+        _Pragma("unroll") for (int i = 0; i < PA; ++i) {                                           \
+            ra[i] = zero4;                                                                         \
+            if (ap[i] && kok) ra[i] = *reinterpret_cast<const uint4*>(ap[i] + koff);               \
+        }                                                                                          \
+        _Pragma("unroll") for (int i = 0; i < PB; ++i) {                                           \
+            rb[i] = zero4;                                                                         \
+            if (bp[i] && kok) rb[i] = *reinterpret_cast<const uint4*>(bp[i] + koff);               \
+        }                                                                                          \
+    }
+#define ATS_STORE_LDS(stage_)                                                                      \
+    {                                                                                              \
+        unsigned char* sA_ = smem + (stage_) * STAGE;                                              \
+        unsigned char* sB_ = sA_ + BM * kRowPitch;                                                 \
+        _Pragma("unroll") for (int i = 0; i < PA; ++i)                                             \
+            *reinterpret_cast<uint4*>(sA_ + (lrow + i * RPP) * kRowPitch + lchunk * 16) = ra[i];   \
+        _Pragma("unroll") for (int i = 0; i < PB; ++i)                                             \
+            *reinterpret_cast<uint4*>(sB_ + (lrow + i * RPP) * kRowPitch + lchunk * 16) = rb[i];   \
+    }
+
+    // fragment rows of this wave inside the staged tiles
+    const int frow = lane & 31;
+    const int fgrp = lane >> 5;
+    int a_row_off[TM], b_row_off[TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i) a_row_off[i] = (wm * (BM / WM) + i * 32 + frow) * kRowPitch + fgrp * 16;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+        int r;
+        if (SWIGLU) {
+            constexpr int WH = BN / WN / 2;  // gate (or up) rows per wave
+            r = j < TN / 2 ? wn * WH + j * 32 : HALF + wn * WH + (j - TN / 2) * 32;
+        } else {
+            r = wn * (BN / WN) + j * 32;
+        }
+        b_row_off[j] = (r + frow) * kRowPitch + fgrp * 16;
+    }
+
+    ATS_LOAD_GLOBAL(0);
+    ATS_STORE_LDS(0);
+    __syncthreads();
+    for (int kt = 0; kt < nk; ++kt) {
+        const int cur = kt & 1;
+        if (kt + 1 < nk) ATS_LOAD_GLOBAL(kt + 1);
+        const unsigned char* sA = smem + cur * STAGE;
+        const unsigned char* sB = sA + BM * kRowPitch;
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+            uint4 fa[TM], fb[TN];
+#pragma unroll
+            for (int i = 0; i < TM; ++i) fa[i] = *reinterpret_cast<const uint4*>(sA + a_row_off[i] + ks * 32);
+#pragma unroll
+            for (int j = 0; j < TN; ++j) fb[j] = *reinterpret_cast<const uint4*>(sB + b_row_off[j] + ks * 32);
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+#pragma unroll
+                for (int i = 0; i < TM; ++i) mma_step<T>(fb[j], fa[i], acc[j][i]);
+        }
+        if (kt + 1 < nk) ATS_STORE_LDS(cur ^ 1);
+        __syncthreads();
+    }
+
+    // ---- epilogue.  acc[j][i][v]: output row m = tile row (lane & 31), output
+    // column n = 8*(v/4) + 4*(lane>>5) + (v%4) inside the 32x32 tile.
+    TO* out = static_cast<TO*>(p.out);
+    constexpr int TNO = SWIGLU ? TN / 2 : TN;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+        const int m = tc.mt * BM + wm * (BM / WM) + i * 32 + frow;
+        if (m >= count) continue;
+        TO* orow = out + (int64_t)(row0 + m) * p.ldo;
+#pragma unroll
+        for (int j = 0; j < TNO; ++j) {
+            const int ncol0 = SWIGLU ? tc.nt * HALF + wn * (BN / WN / 2) + j * 32 : tc.nt * BN + wn * (BN / WN) + j * 32;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int n = ncol0 + 8 * q + 4 * fgrp;
+                float v[4];
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    if (SWIGLU) v[c] = silu_f(acc[j][i][q * 4 + c]) * acc[j + TN / 2][i][q * 4 + c];
+                    else v[c] = acc[j][i][q * 4 + c];
+                }
+                const int n_valid = p.N_out - n;
+                if (n_valid > 0) store4<TO>(orow + n, v, n_valid);
+            }
+        }
+    }
+}
+
+template <typename T, typename TO, int BM, int BN, int WM, int WN, int SM, int SN, bool SWIGLU>
+static int launch_cfg(const GroupedArgs& p0, int64_t max_rows, hipStream_t s) {
+    GroupedArgs p = p0;
+    constexpr int n_per_tile = SWIGLU ? BN / 2 : BN;
+    p.n_tiles = (p.N_out + n_per_tile - 1) / n_per_tile;
+    constexpr size_t smem = 2 * (size_t)(BM + BN) * kRowPitch;
+    auto kern = grouped_gemm_kernel<T, TO, BM, BN, WM, WN, SM, SN, SWIGLU>;
+    static bool attr_done = false;
+    if (!attr_done) {
+        if (smem > 64 * 1024) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+            if (e != hipSuccess) {
+                set_error("grouped GEMM: cannot reserve %zu bytes of LDS: %s", smem, hipGetErrorString(e));
+                return ATS_ERR_LAUNCH;
+            }
+        }
+        attr_done = true;
+    }
+    const int64_t blocks = grid_blocks(max_rows, p.E, BM, p.n_tiles, SM, SN);
+    if (blocks > 0x7fffffffLL) {
+        set_error("grouped GEMM: grid of %lld blocks", (long long)blocks);
+        return ATS_ERR_UNSUPPORTED;
+    }
+    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(WM * WN * 64), smem, s, p);
+    return ATS_OK;
+}
+
+// Tile configuration by rows per expert: decode-sized groups stream weights
+// with 32-row tiles, mid-sized groups use 128-row tiles, prefill uses 256x256.
+template <typename T, typename TO, bool SWIGLU>
+static int launch_grouped(const GroupedArgs& p, int64_t max_rows, hipStream_t s) {
+    const int64_t avg = max_rows / (p.E > 0 ? p.E : 1);
+    if (avg <= 48) {
+        if constexpr (SWIGLU) return launch_cfg<T, TO, 32, 256, 1, 4, 1, 32, SWIGLU>(p, max_rows, s);
+        else return launch_cfg<T, TO, 32, 128, 1, 4, 1, 32, SWIGLU>(p, max_rows, s);
+    }
+    if (avg <= 768) return launch_cfg<T, TO, 128, 256, 2, 2, 4, 8, SWIGLU>(p, max_rows, s);
+    return launch_cfg<T, TO, 256, 256, 2, 2, 4, 8, SWIGLU>(p, max_rows, s);
+}
+
+static int check_common(const char* name, const void* a, const void* const* w, const void* out,
+                        const int32_t* row_start, const int32_t* row_count, int E, int64_t max_rows, int H, int I,
+                        int dtype) {
+    ATS_REQUIRE(E > 0 && E <= 4096 && max_rows >= 0 && H > 0 && I > 0, ATS_ERR_INVALID_ARG,
+                "%s: E=%d max_rows=%lld H=%d I=%d", name, E, (long long)max_rows, H, I);
+    ATS_REQUIRE(dtype == ATS_F32 || dtype == ATS_BF16, ATS_ERR_UNSUPPORTED, "%s: dtype tag %d", name, dtype);
+    ATS_REQUIRE(a && w && out && row_start && row_count, ATS_ERR_INVALID_ARG, "%s: null pointer", name);
+    const int vec = dtype == ATS_F32 ? 4 : 8;
+    ATS_REQUIRE(H % vec == 0 && I % vec == 0, ATS_ERR_UNSUPPORTED,
+                "%s: H=%d and I=%d must be multiples of %d (16-byte rows)", name, H, I, vec);
+    ATS_REQUIRE(aligned16(a) && aligned16(out), ATS_ERR_INVALID_ARG, "%s: operands must be 16-byte aligned", name);
+    return ATS_OK;
+}
+
+}  // namespace ats
+
+extern "C" int ats_grouped_gateup_swiglu(const void* a, const int32_t* a_rows, int a_row_div,
+                                         const void* const* w_gu, void* h, const int32_t* row_start,
+                                         const int32_t* row_count, int E, int64_t max_rows, int H, int I, int dtype,
+                                         ats_stream_t stream) {
+    using namespace ats;
+    int rc = check_common("ats_grouped_gateup_swiglu", a, w_gu, h, row_start, row_count, E, max_rows, H, I, dtype);
+    if (rc != ATS_OK) return rc;
+    ATS_REQUIRE(!a_rows || a_row_div > 0, ATS_ERR_INVALID_ARG, "ats_grouped_gateup_swiglu: a_row_div=%d", a_row_div);
+    if (max_rows == 0) return ATS_OK;
+    GroupedArgs p{};
+    p.a = a;
+    p.a_rows = a_rows;
+    p.a_row_div = a_rows ? a_row_div : 1;
+    p.lda = H;
+    p.b = w_gu;
+    p.out = h;
+    p.ldo = I;
+    p.row_start = row_start;
+    p.row_count = row_count;
+    p.E = E;
+    p.K = H;
+    p.N_out = I;
+    p.up_offset = I;
+    hipStream_t s = as_stream(stream);
+    rc = dtype == ATS_F32 ? launch_grouped<float, float, true>(p, max_rows, s)
+                          : launch_grouped<bf16_t, bf16_t, true>(p, max_rows, s);
+    if (rc != ATS_OK) return rc;
+    ATS_CHECK_LAUNCH("ats_grouped_gateup_swiglu");
+    return ATS_OK;
+}
+
+extern "C" int ats_grouped_down(const void* h, const void* const* w_d, void* y, const int32_t* row_start,
+                                const int32_t* row_count, int E, int64_t max_rows, int H, int I, int dtype,
+                                int y_dtype, ats_stream_t stream) {
+    using namespace ats;
+    int rc = check_common("ats_grouped_down", h, w_d, y, row_start, row_count, E, max_rows, H, I, dtype);
+    if (rc != ATS_OK) return rc;
+    ATS_REQUIRE(y_dtype == ATS_F32 || y_dtype == dtype, ATS_ERR_UNSUPPORTED,
+                "ats_grouped_down: y dtype tag %d (float32 or the operand type)", y_dtype);
+    if (max_rows == 0) return ATS_OK;
+    GroupedArgs p{};
+    p.a = h;
+    p.a_rows = nullptr;
+    p.a_row_div = 1;
+    p.lda = I;
+    p.b = w_d;
+    p.out = y;
+    p.ldo = H;
+    p.row_start = row_start;
+    p.row_count = row_count;
+    p.E = E;
+    p.K = I;
+    p.N_out = H;
+    p.up_offset = 0;
+    hipStream_t s = as_stream(stream);
+    if (dtype == ATS_F32) rc = launch_grouped<float, float, false>(p, max_rows, s);
+    else if (y_dtype == ATS_F32) rc = launch_grouped<bf16_t, float, false>(p, max_rows, s);
+    else rc = launch_grouped<bf16_t, bf16_t, false>(p, max_rows, s);
+    if (rc != ATS_OK) return rc;
+    ATS_CHECK_LAUNCH("ats_grouped_down");
+    return ATS_OK;
+}
+
+// Host-side view of the tile schedule (for tests of the block -> tile map).
+extern "C" int ats_debug_decode_tile(int64_t block, const int32_t* row_count_host, int E, int BM, int n_tiles,
+                                     int SM, int SN, int32_t* out3) {
+    ats::TileCoord tc;
+    if (!ats::decode_tile(block, row_count_host, E, BM, n_tiles, SM, SN, &tc)) return 0;
+    out3[0] = tc.e;
+    out3[1] = tc.mt;
+    out3[2] = tc.nt;
+    return 1;
+}
+extern "C" int64_t ats_debug_grid_blocks(int64_t max_rows, int E, int BM, int n_tiles, int SM, int SN) {
+    return ats::grid_blocks(max_rows, E, BM, n_tiles, SM, SN);
+}

@@ -1,0 +1,329 @@
+// Mixture-of-Depths helpers for gfx950: per-token router score (H -> 1 linear,
+// HBM-bound: x is read once), per-sequence top-`keep` selection, and the
+// scatter-add of the block output onto the residual stream.
+#include <limits.h>
+#include <math.h>
+
+#include "ats_common.hpp"
+
+namespace ats {
+
+// One wave per token row; 16-byte loads; weight vector re-read from L2.
+template <typename T>
+__global__ __launch_bounds__(256) void row_dot_kernel(const T* __restrict__ x, const T* __restrict__ w,
+                                                      const float* __restrict__ bias, float* __restrict__ score,
+                                                      float* __restrict__ prob, float temperature, int64_t Tn, int H,
+                                                      bool vec) {
+    constexpr int V = Elem<T>::kVec;
+    const int lane = lane_id();
+    const int64_t wave = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    const int64_t nwaves = (int64_t)gridDim.x * (blockDim.x >> 6);
+    for (int64_t t = wave; t < Tn; t += nwaves) {
+        float acc = 0.f;
+        if (vec) {
+            const uint4* xr = reinterpret_cast<const uint4*>(x + t * H);
+            const uint4* wr = reinterpret_cast<const uint4*>(w);
+            for (int v = lane; v < H / V; v += kWave) {
+                float a[V], b[V];
+                Elem<T>::unpack(xr[v], a);
+                Elem<T>::unpack(wr[v], b);
+#pragma unroll
+                for (int j = 0; j < V; ++j) acc += a[j] * b[j];
+            }
+        } else {
+            for (int h = lane; h < H; h += kWave) acc += Elem<T>::load(x + t * H + h) * Elem<T>::load(w + h);
+        }
+        acc = wave_sum(acc);
+        if (lane == 0) {
+            const float sc = acc + (bias ? bias[0] : 0.f);
+            if (score) score[t] = sc;
+            if (prob) prob[t] = 1.0f / (1.0f + expf(-__fdiv_rn(sc, temperature)));
+        }
+    }
+}
+
+// One block per sequence.  Bitonic sort of (score desc, position asc) keys in
+// LDS, then the first `keep` positions are flagged and compacted in position
+// order with a block-wide prefix sum.
+__global__ __launch_bounds__(1024) void select_topk_seq_kernel(const float* __restrict__ score, int L, int Lpow2,
+                                                               int keep, int32_t* __restrict__ sel) {
+    extern __shared__ unsigned char smem_raw[];
+    float* s_val = reinterpret_cast<float*>(smem_raw);      // [Lpow2]
+    int* s_pos = reinterpret_cast<int*>(s_val + Lpow2);      // [Lpow2]
+    int* s_flag = s_pos + Lpow2;                             // [Lpow2] then prefix sums
+    const int b = blockIdx.x;
+    const int nthr = blockDim.x;
+    for (int i = threadIdx.x; i < Lpow2; i += nthr) {
+        s_val[i] = i < L ? score[(int64_t)b * L + i] : -INFINITY;
+        s_pos[i] = i < L ? i : INT_MAX;
+        s_flag[i] = 0;
+    }
+    __syncthreads();
+    // "a before b": larger score first (NaN above all), lower position among equals
+    auto before = [](float va, int pa, float vb, int pb) {
+        const bool na = va != va, nb = vb != vb;
+        if (na != nb) return na;
+        if (!na && va != vb) return va > vb;
+        return pa < pb;
+    };
+    for (int size = 2; size <= Lpow2; size <<= 1) {
+        for (int stride = size >> 1; stride > 0; stride >>= 1) {
+            for (int i = threadIdx.x; i < (Lpow2 >> 1); i += nthr) {
+                const int lo = 2 * i - (i & (stride - 1));
+                const int hi = lo + stride;
+                const bool asc_block = ((lo & size) == 0);  // this block sorts "before"-first
+                const float va = s_val[lo], vb = s_val[hi];
+                const int pa = s_pos[lo], pb = s_pos[hi];
+                const bool swap = asc_block ? before(vb, pb, va, pa) : before(va, pa, vb, pb);
+                if (swap) {
+                    s_val[lo] = vb;
+                    s_val[hi] = va;
+                    s_pos[lo] = pb;
+                    s_pos[hi] = pa;
+                }
+            }
+            __syncthreads();
+        }
+    }
+    for (int i = threadIdx.x; i < keep; i += nthr) s_flag[s_pos[i]] = 1;
+    __syncthreads();
+    // inclusive prefix sum of the flags (Hillis-Steele over LDS, two buffers folded into s_val as int)
+    int* s_a = s_flag;
+    int* s_b = reinterpret_cast<int*>(s_val);
+    for (int off = 1; off < Lpow2; off <<= 1) {
+        for (int i = threadIdx.x; i < Lpow2; i += nthr) s_b[i] = s_a[i] + (i >= off ? s_a[i - off] : 0);
+        __syncthreads();
+        int* t = s_a;
+        s_a = s_b;
+        s_b = t;
+    }
+    for (int i = threadIdx.x; i < L; i += nthr) {
+        const int incl = s_a[i];
+        const int prev = i > 0 ? s_a[i - 1] : 0;
+        if (incl != prev) sel[(int64_t)b * keep + prev] = b * L + i;
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void scatter_add_rows_kernel(T* __restrict__ base, const int32_t* __restrict__ rows,
+                                                               const T* __restrict__ delta, int64_t n, int H,
+                                                               bool vec) {
+    constexpr int V = Elem<T>::kVec;
+    const int lane = lane_id();
+    const int64_t wave = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    const int64_t nwaves = (int64_t)gridDim.x * (blockDim.x >> 6);
+    for (int64_t i = wave; i < n; i += nwaves) {
+        const int64_t r = rows[i];
+        if (r < 0) continue;
+        if (vec) {
+            uint4* bp = reinterpret_cast<uint4*>(base + r * H);
+            const uint4* dp = reinterpret_cast<const uint4*>(delta + i * H);
+            for (int v = lane; v < H / V; v += kWave) {
+                float a[V], d[V];
+                Elem<T>::unpack(bp[v], a);
+                Elem<T>::unpack(dp[v], d);
+#pragma unroll
+                for (int j = 0; j < V; ++j) a[j] = __fadd_rn(a[j], d[j]);
+                bp[v] = Elem<T>::pack(a);
+            }
+        } else {
+            for (int h = lane; h < H; h += kWave)
+                Elem<T>::store(base + r * H + h, __fadd_rn(Elem<T>::load(base + r * H + h), Elem<T>::load(delta + i * H + h)));
+        }
+    }
+}
+
+// k-th smallest value (1-based) of n floats by a 4-pass, 8-bit radix select in one
+// block, then a threshold mask.  Keys are the usual order-preserving unsigned
+// image of the float bits.
+__device__ __forceinline__ uint32_t order_key(float f) {
+    const uint32_t u = __float_as_uint(f);
+    return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+
+__global__ __launch_bounds__(1024) void kth_value_kernel(const float* __restrict__ v, int64_t n, int64_t kth,
+                                                         uint32_t* __restrict__ key_out) {
+    __shared__ unsigned int hist[256];
+    __shared__ uint32_t s_prefix;
+    __shared__ long long s_rank;
+    if (threadIdx.x == 0) {
+        s_prefix = 0;
+        s_rank = kth;
+    }
+    for (int pass = 3; pass >= 0; --pass) {
+        for (int i = threadIdx.x; i < 256; i += blockDim.x) hist[i] = 0;
+        __syncthreads();
+        const uint32_t prefix = s_prefix;
+        const uint32_t hi_mask = pass == 3 ? 0u : (0xffffffffu << (8 * (pass + 1)));
+        for (int64_t i = threadIdx.x; i < n; i += blockDim.x) {
+            const uint32_t key = order_key(v[i]);
+            if ((key & hi_mask) == prefix) atomicAdd(&hist[(key >> (8 * pass)) & 255u], 1u);
+        }
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            long long rank = s_rank;
+            int b = 0;
+            for (; b < 255; ++b) {
+                if (rank <= (long long)hist[b]) break;
+                rank -= hist[b];
+            }
+            s_rank = rank;
+            s_prefix = prefix | ((uint32_t)b << (8 * pass));
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) key_out[0] = s_prefix;
+}
+
+__global__ __launch_bounds__(256) void threshold_mask_kernel(const float* __restrict__ v, int64_t n,
+                                                             const uint32_t* __restrict__ key, float* __restrict__ mask) {
+    const uint32_t thr = key[0];
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
+        mask[i] = order_key(v[i]) >= thr ? 1.0f : 0.0f;
+}
+
+// Dense-FFN activation of the fused wrapper: out = gate * silu(up).
+template <typename T>
+__global__ __launch_bounds__(256) void swiglu_mul_kernel(const T* __restrict__ gate, const T* __restrict__ up,
+                                                         T* __restrict__ out, int64_t n, bool vec) {
+    constexpr int V = Elem<T>::kVec;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    const int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (vec) {
+        const int64_t nv = n / V;
+        for (int64_t i = tid; i < nv; i += stride) {
+            float g[V], u[V];
+            Elem<T>::unpack(reinterpret_cast<const uint4*>(gate)[i], g);
+            Elem<T>::unpack(reinterpret_cast<const uint4*>(up)[i], u);
+#pragma unroll
+            for (int j = 0; j < V; ++j) g[j] = g[j] * (u[j] / (1.0f + expf(-u[j])));
+            reinterpret_cast<uint4*>(out)[i] = Elem<T>::pack(g);
+        }
+        for (int64_t i = nv * V + tid; i < n; i += stride) {
+            const float u = Elem<T>::load(up + i);
+            Elem<T>::store(out + i, Elem<T>::load(gate + i) * (u / (1.0f + expf(-u))));
+        }
+    } else {
+        for (int64_t i = tid; i < n; i += stride) {
+            const float u = Elem<T>::load(up + i);
+            Elem<T>::store(out + i, Elem<T>::load(gate + i) * (u / (1.0f + expf(-u))));
+        }
+    }
+}
+
+}  // namespace ats
+
+extern "C" int ats_row_dot(const void* x, const void* w, const float* bias, float* score, float* prob,
+                           float temperature, int64_t T, int H, int dtype, ats_stream_t stream) {
+    using namespace ats;
+    ATS_REQUIRE(T >= 0 && H > 0, ATS_ERR_INVALID_ARG, "ats_row_dot: T=%lld H=%d", (long long)T, H);
+    ATS_REQUIRE(dtype == ATS_F32 || dtype == ATS_BF16, ATS_ERR_UNSUPPORTED, "ats_row_dot: dtype tag %d", dtype);
+    ATS_REQUIRE(!prob || temperature > 0.f, ATS_ERR_INVALID_ARG, "ats_row_dot: temperature %g", temperature);
+    if (T == 0) return ATS_OK;
+    ATS_REQUIRE(x && w && (score || prob), ATS_ERR_INVALID_ARG, "ats_row_dot: null pointer");
+    int64_t blocks = (T + 3) / 4;
+    if (blocks > 16384) blocks = 16384;
+    const int V = dtype == ATS_F32 ? 4 : 8;
+    const bool vec = H % V == 0 && aligned16(x) && aligned16(w);
+    if (dtype == ATS_F32)
+        hipLaunchKernelGGL((row_dot_kernel<float>), dim3((unsigned)blocks), dim3(256), 0, as_stream(stream),
+                           static_cast<const float*>(x), static_cast<const float*>(w), bias, score, prob, temperature,
+                           T, H, vec);
+    else
+        hipLaunchKernelGGL((row_dot_kernel<bf16_t>), dim3((unsigned)blocks), dim3(256), 0, as_stream(stream),
+                           static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), bias, score, prob,
+                           temperature, T, H, vec);
+    ATS_CHECK_LAUNCH("ats_row_dot");
+    return ATS_OK;
+}
+
+extern "C" int ats_select_topk_per_sequence(const float* score, int B, int L, int keep, int32_t* sel,
+                                            ats_stream_t stream) {
+    using namespace ats;
+    ATS_REQUIRE(B >= 0 && L > 0 && L <= 8192 && keep >= 0 && keep <= L, ATS_ERR_INVALID_ARG,
+                "ats_select_topk_per_sequence: B=%d L=%d keep=%d (L <= 8192, keep <= L)", B, L, keep);
+    ATS_REQUIRE((int64_t)B * L < INT_MAX, ATS_ERR_UNSUPPORTED, "ats_select_topk_per_sequence: B*L must fit in int32");
+    if (B == 0 || keep == 0) return ATS_OK;
+    ATS_REQUIRE(score && sel, ATS_ERR_INVALID_ARG, "ats_select_topk_per_sequence: null pointer");
+    int lp2 = 2;
+    while (lp2 < L) lp2 <<= 1;
+    const int threads = lp2 / 2 < 64 ? 64 : (lp2 / 2 > 1024 ? 1024 : lp2 / 2);
+    const size_t smem = (size_t)lp2 * 12;
+    if (smem > 64 * 1024) {
+        static bool attr_done = false;
+        if (!attr_done) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(select_topk_seq_kernel),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, 8192 * 12);
+            ATS_REQUIRE(e == hipSuccess, ATS_ERR_LAUNCH, "ats_select_topk_per_sequence: LDS attribute: %s",
+                        hipGetErrorString(e));
+            attr_done = true;
+        }
+    }
+    hipLaunchKernelGGL(select_topk_seq_kernel, dim3(B), dim3(threads), smem, as_stream(stream), score, L, lp2, keep,
+                       sel);
+    ATS_CHECK_LAUNCH("ats_select_topk_per_sequence");
+    return ATS_OK;
+}
+
+extern "C" int ats_scatter_add_rows(void* base, const int32_t* rows, const void* delta, int64_t n, int H, int dtype,
+                                    ats_stream_t stream) {
+    using namespace ats;
+    ATS_REQUIRE(n >= 0 && H > 0, ATS_ERR_INVALID_ARG, "ats_scatter_add_rows: n=%lld H=%d", (long long)n, H);
+    ATS_REQUIRE(dtype == ATS_F32 || dtype == ATS_BF16, ATS_ERR_UNSUPPORTED, "ats_scatter_add_rows: dtype tag %d", dtype);
+    if (n == 0) return ATS_OK;
+    ATS_REQUIRE(base && rows && delta, ATS_ERR_INVALID_ARG, "ats_scatter_add_rows: null pointer");
+    int64_t blocks = (n + 3) / 4;
+    if (blocks > 16384) blocks = 16384;
+    const int V = dtype == ATS_F32 ? 4 : 8;
+    const bool vec = H % V == 0 && aligned16(base) && aligned16(delta);
+    if (dtype == ATS_F32)
+        hipLaunchKernelGGL((scatter_add_rows_kernel<float>), dim3((unsigned)blocks), dim3(256), 0, as_stream(stream),
+                           static_cast<float*>(base), rows, static_cast<const float*>(delta), n, H, vec);
+    else
+        hipLaunchKernelGGL((scatter_add_rows_kernel<bf16_t>), dim3((unsigned)blocks), dim3(256), 0, as_stream(stream),
+                           static_cast<bf16_t*>(base), rows, static_cast<const bf16_t*>(delta), n, H, vec);
+    ATS_CHECK_LAUNCH("ats_scatter_add_rows");
+    return ATS_OK;
+}
+
+extern "C" int ats_kth_value_mask(const float* v, int64_t n, int64_t kth, float* mask, void* workspace,
+                                  size_t workspace_bytes, ats_stream_t stream) {
+    using namespace ats;
+    ATS_REQUIRE(n >= 0 && (n == 0 || (kth >= 1 && kth <= n)), ATS_ERR_INVALID_ARG,
+                "ats_kth_value_mask: n=%lld kth=%lld", (long long)n, (long long)kth);
+    if (n == 0) return ATS_OK;
+    ATS_REQUIRE(v && mask, ATS_ERR_INVALID_ARG, "ats_kth_value_mask: null pointer");
+    ATS_REQUIRE(workspace && workspace_bytes >= sizeof(uint32_t), ATS_ERR_WORKSPACE,
+                "ats_kth_value_mask: workspace of at least 4 bytes needed");
+    hipStream_t s = as_stream(stream);
+    uint32_t* key = static_cast<uint32_t*>(workspace);
+    hipLaunchKernelGGL(kth_value_kernel, dim3(1), dim3(1024), 0, s, v, n, kth, key);
+    ATS_CHECK_LAUNCH("ats_kth_value_mask(select)");
+    int64_t blocks = (n + 255) / 256;
+    if (blocks > 4096) blocks = 4096;
+    hipLaunchKernelGGL(threshold_mask_kernel, dim3((unsigned)blocks), dim3(256), 0, s, v, n, key, mask);
+    ATS_CHECK_LAUNCH("ats_kth_value_mask(mask)");
+    return ATS_OK;
+}
+
+extern "C" int ats_swiglu_mul(const void* gate, const void* up, void* out, int64_t n, int dtype,
+                              ats_stream_t stream) {
+    using namespace ats;
+    ATS_REQUIRE(n >= 0, ATS_ERR_INVALID_ARG, "ats_swiglu_mul: n=%lld", (long long)n);
+    ATS_REQUIRE(dtype == ATS_F32 || dtype == ATS_BF16, ATS_ERR_UNSUPPORTED, "ats_swiglu_mul: dtype tag %d", dtype);
+    if (n == 0) return ATS_OK;
+    ATS_REQUIRE(gate && up && out, ATS_ERR_INVALID_ARG, "ats_swiglu_mul: null pointer");
+    const bool vec = aligned16(gate) && aligned16(up) && aligned16(out);
+    int64_t blocks = (n / (dtype == ATS_F32 ? 4 : 8) + 255) / 256 + 1;
+    if (blocks > 16384) blocks = 16384;
+    if (dtype == ATS_F32)
+        hipLaunchKernelGGL((swiglu_mul_kernel<float>), dim3((unsigned)blocks), dim3(256), 0, as_stream(stream),
+                           static_cast<const float*>(gate), static_cast<const float*>(up), static_cast<float*>(out),
+                           n, vec);
+    else
+        hipLaunchKernelGGL((swiglu_mul_kernel<bf16_t>), dim3((unsigned)blocks), dim3(256), 0, as_stream(stream),
+                           static_cast<const bf16_t*>(gate), static_cast<const bf16_t*>(up),
+                           static_cast<bf16_t*>(out), n, vec);
+    ATS_CHECK_LAUNCH("ats_swiglu_mul");
+    return ATS_OK;
+}

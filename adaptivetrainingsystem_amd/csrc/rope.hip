@@ -1,0 +1,211 @@
+// Rotary position embedding (rotate-half, grouped-query aware) for gfx950.
+// HBM-bound: q and k are read once and written once.  A group of lanes owns one
+// (batch, position); it loads that position's cos/sin once and walks a chunk of
+// heads, so the float32 table costs one L2 read per HEADS_PER_ITEM rows.  Lanes
+// of a wave cover consecutive positions of one head, i.e. one contiguous span
+// of memory per head, with 16-byte accesses per lane.
+#include <math.h>
+
+#include "ats_common.hpp"
+
+namespace ats {
+
+constexpr int kRopeHeadsPerItem = 4;
+
+struct RopeSeg {
+    const void* in;
+    void* out;
+    int64_t sb, sh, sl;  // input element strides: batch, head, position
+    int heads;
+    int chunks;  // ceil(heads / kRopeHeadsPerItem)
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void rope_vec_kernel(RopeSeg q, RopeSeg k, const float* __restrict__ cos_tab,
+                                                       const float* __restrict__ sin_tab, int table_stride,
+                                                       int L, int D, int pos_offset, int lanes_per_row,
+                                                       int pos_per_wave, int n_pos_groups, int64_t n_items) {
+    constexpr int V = Elem<T>::kVec;
+    const int lane = lane_id();
+    const int64_t item = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (item >= n_items) return;
+    const int pg = (int)(item % n_pos_groups);
+    const int64_t rest = item / n_pos_groups;
+    const int total_chunks = q.chunks + k.chunks;
+    int chunk = (int)(rest % total_chunks);
+    const int b = (int)(rest / total_chunks);
+    const RopeSeg& seg = chunk < q.chunks ? q : k;
+    if (chunk >= q.chunks) chunk -= q.chunks;
+
+    const int prow = lane / lanes_per_row;
+    const int c = lane - prow * lanes_per_row;
+    const int pos = pg * pos_per_wave + prow;
+    if (prow >= pos_per_wave || pos >= L) return;
+
+    const int half = D >> 1;
+    float cs[V], sn[V];
+    {
+        const float* cp = cos_tab + (int64_t)(pos_offset + pos) * table_stride + c * V;
+        const float* sp = sin_tab + (int64_t)(pos_offset + pos) * table_stride + c * V;
+#pragma unroll
+        for (int j = 0; j < V; ++j) {
+            cs[j] = cp[j];
+            sn[j] = sp[j];
+        }
+    }
+    const int h0 = chunk * kRopeHeadsPerItem;
+    const T* in = static_cast<const T*>(seg.in);
+    T* out = static_cast<T*>(seg.out);
+    uint4 lo[kRopeHeadsPerItem], hi[kRopeHeadsPerItem];
+#pragma unroll
+    for (int i = 0; i < kRopeHeadsPerItem; ++i) {
+        const int h = h0 + i;
+        if (h < seg.heads) {
+            const T* p = in + b * seg.sb + h * seg.sh + pos * seg.sl + c * V;
+            lo[i] = *reinterpret_cast<const uint4*>(p);
+            hi[i] = *reinterpret_cast<const uint4*>(p + half);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < kRopeHeadsPerItem; ++i) {
+        const int h = h0 + i;
+        if (h < seg.heads) {
+            float a[V], bb[V], o1[V], o2[V];
+            Elem<T>::unpack(lo[i], a);
+            Elem<T>::unpack(hi[i], bb);
+#pragma unroll
+            for (int j = 0; j < V; ++j) {
+                o1[j] = __fsub_rn(__fmul_rn(a[j], cs[j]), __fmul_rn(bb[j], sn[j]));
+                o2[j] = __fadd_rn(__fmul_rn(a[j], sn[j]), __fmul_rn(bb[j], cs[j]));
+            }
+            T* p = out + (((int64_t)b * seg.heads + h) * L + pos) * D + c * V;
+            *reinterpret_cast<uint4*>(p) = Elem<T>::pack(o1);
+            *reinterpret_cast<uint4*>(p + half) = Elem<T>::pack(o2);
+        }
+    }
+}
+
+// Any even D / alignment: one thread per rotated pair.
+template <typename T>
+__global__ __launch_bounds__(256) void rope_scalar_kernel(RopeSeg q, RopeSeg k, const float* __restrict__ cos_tab,
+                                                          const float* __restrict__ sin_tab, int table_stride,
+                                                          int B, int L, int D, int pos_offset) {
+    const int half = D >> 1;
+    const int64_t per_b = (int64_t)(q.heads + k.heads) * L * half;
+    const int64_t total = per_b * B;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+         i += (int64_t)gridDim.x * blockDim.x) {
+        const int d = (int)(i % half);
+        int64_t r = i / half;
+        const int pos = (int)(r % L);
+        r /= L;
+        const int hh = (int)(r % (q.heads + k.heads));
+        const int b = (int)(r / (q.heads + k.heads));
+        const RopeSeg& seg = hh < q.heads ? q : k;
+        const int h = hh < q.heads ? hh : hh - q.heads;
+        const T* p = static_cast<const T*>(seg.in) + b * seg.sb + h * seg.sh + pos * seg.sl + d;
+        const float a = Elem<T>::load(p), bb = Elem<T>::load(p + half);
+        const float cs = cos_tab[(int64_t)(pos_offset + pos) * table_stride + d];
+        const float sn = sin_tab[(int64_t)(pos_offset + pos) * table_stride + d];
+        T* o = static_cast<T*>(seg.out) + (((int64_t)b * seg.heads + h) * L + pos) * D + d;
+        Elem<T>::store(o, __fsub_rn(__fmul_rn(a, cs), __fmul_rn(bb, sn)));
+        Elem<T>::store(o + half, __fadd_rn(__fmul_rn(a, sn), __fmul_rn(bb, cs)));
+    }
+}
+
+// cos/sin table in float64, stored as float32.
+__global__ __launch_bounds__(256) void rope_table_kernel(float* __restrict__ cos_out, float* __restrict__ sin_out,
+                                                         int seq_len, int dim, int cols, double theta,
+                                                         double scaling) {
+    const int half = dim >> 1;
+    const int64_t total = (int64_t)seq_len * half;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+         i += (int64_t)gridDim.x * blockDim.x) {
+        const int d = (int)(i % half);
+        const int pos = (int)(i / half);
+        const double inv_freq = 1.0 / pow(theta, (double)(2 * d) / (double)dim);
+        float t = (float)pos;
+        if (scaling != 1.0) t = t / (float)scaling;
+        const double ang = (double)t * inv_freq;
+        const float cv = (float)cos(ang), sv = (float)sin(ang);
+        cos_out[(int64_t)pos * cols + d] = cv;
+        sin_out[(int64_t)pos * cols + d] = sv;
+        if (cols == dim) {
+            cos_out[(int64_t)pos * cols + d + half] = cv;
+            sin_out[(int64_t)pos * cols + d + half] = sv;
+        }
+    }
+}
+
+template <typename T>
+static void launch_rope(RopeSeg q, RopeSeg k, const float* cos_tab, const float* sin_tab, int table_stride, int B,
+                        int L, int D, int pos_offset, bool vec_ok, hipStream_t s) {
+    constexpr int V = Elem<T>::kVec;
+    if (vec_ok) {
+        const int lanes_per_row = (D / 2) / V;
+        const int pos_per_wave = kWave / lanes_per_row;
+        const int n_pos_groups = (L + pos_per_wave - 1) / pos_per_wave;
+        const int64_t n_items = (int64_t)n_pos_groups * (q.chunks + k.chunks) * B;
+        const int64_t blocks = (n_items + 3) / 4;
+        hipLaunchKernelGGL((rope_vec_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, s, q, k, cos_tab, sin_tab,
+                           table_stride, L, D, pos_offset, lanes_per_row, pos_per_wave, n_pos_groups, n_items);
+    } else {
+        const int64_t total = (int64_t)B * (q.heads + k.heads) * L * (D / 2);
+        int64_t blocks = (total + 255) / 256;
+        if (blocks > 65536) blocks = 65536;
+        hipLaunchKernelGGL((rope_scalar_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, s, q, k, cos_tab, sin_tab,
+                           table_stride, B, L, D, pos_offset);
+    }
+}
+
+}  // namespace ats
+
+extern "C" int ats_rope_table(float* cos_out, float* sin_out, int seq_len, int dim, int cols, double theta,
+                              double scaling_factor, ats_stream_t stream) {
+    using namespace ats;
+    ATS_REQUIRE(cos_out && sin_out, ATS_ERR_INVALID_ARG, "ats_rope_table: null pointer");
+    ATS_REQUIRE(seq_len >= 0 && dim > 0 && dim % 2 == 0 && (cols == dim || cols == dim / 2) && theta > 0 &&
+                    scaling_factor > 0,
+                ATS_ERR_INVALID_ARG, "ats_rope_table: seq_len=%d dim=%d cols=%d theta=%g scaling=%g", seq_len, dim,
+                cols, theta, scaling_factor);
+    if (seq_len == 0) return ATS_OK;
+    const int64_t total = (int64_t)seq_len * (dim / 2);
+    int64_t blocks = (total + 255) / 256;
+    if (blocks > 65536) blocks = 65536;
+    hipLaunchKernelGGL(rope_table_kernel, dim3((unsigned)blocks), dim3(256), 0, as_stream(stream), cos_out, sin_out,
+                       seq_len, dim, cols, theta, scaling_factor);
+    ATS_CHECK_LAUNCH("ats_rope_table");
+    return ATS_OK;
+}
+
+extern "C" int ats_rope_fwd(const void* q_in, const void* k_in, void* q_out, void* k_out, const float* cos_tab,
+                            const float* sin_tab, int table_stride, int table_len, int B, int Hq, int Hkv, int L,
+                            int D, int pos_offset, int64_t q_sb, int64_t q_sh, int64_t q_sl, int64_t k_sb,
+                            int64_t k_sh, int64_t k_sl, int dtype, ats_stream_t stream) {
+    using namespace ats;
+    ATS_REQUIRE(B >= 0 && Hq >= 0 && Hkv >= 0 && L >= 0 && D > 0 && D % 2 == 0, ATS_ERR_INVALID_ARG,
+                "ats_rope_fwd: B=%d Hq=%d Hkv=%d L=%d D=%d", B, Hq, Hkv, L, D);
+    ATS_REQUIRE(dtype == ATS_F32 || dtype == ATS_BF16, ATS_ERR_UNSUPPORTED, "ats_rope_fwd: dtype tag %d", dtype);
+    if (B == 0 || L == 0 || Hq + Hkv == 0) return ATS_OK;
+    ATS_REQUIRE(cos_tab && sin_tab && table_stride >= D / 2, ATS_ERR_INVALID_ARG,
+                "ats_rope_fwd: table pointers/stride (stride=%d, need >= %d)", table_stride, D / 2);
+    ATS_REQUIRE(pos_offset >= 0 && (int64_t)pos_offset + L <= table_len, ATS_ERR_INVALID_ARG,
+                "ats_rope_fwd: positions %d..%d exceed table length %d", pos_offset, pos_offset + L - 1, table_len);
+    ATS_REQUIRE((Hq == 0 || (q_in && q_out)) && (Hkv == 0 || (k_in && k_out)), ATS_ERR_INVALID_ARG,
+                "ats_rope_fwd: null tensor pointer");
+    RopeSeg q{q_in, q_out, q_sb, q_sh, q_sl, Hq, (Hq + kRopeHeadsPerItem - 1) / kRopeHeadsPerItem};
+    RopeSeg k{k_in, k_out, k_sb, k_sh, k_sl, Hkv, (Hkv + kRopeHeadsPerItem - 1) / kRopeHeadsPerItem};
+    const int V = dtype == ATS_F32 ? 4 : 8;
+    auto seg_ok = [&](const RopeSeg& sgm) {
+        return sgm.heads == 0 || (aligned16(sgm.in) && aligned16(sgm.out) && sgm.sb % V == 0 && sgm.sh % V == 0 &&
+                                  sgm.sl % V == 0);
+    };
+    const int half = D / 2;
+    const bool vec_ok = half % V == 0 && half / V <= kWave && seg_ok(q) && seg_ok(k);
+    if (dtype == ATS_F32)
+        launch_rope<float>(q, k, cos_tab, sin_tab, table_stride, B, L, D, pos_offset, vec_ok, as_stream(stream));
+    else
+        launch_rope<bf16_t>(q, k, cos_tab, sin_tab, table_stride, B, L, D, pos_offset, vec_ok, as_stream(stream));
+    ATS_CHECK_LAUNCH("ats_rope_fwd");
+    return ATS_OK;
+}

@@ -1,0 +1,460 @@
+// Router for gfx950: gate GEMM (tokens x experts, float32 logits) and the fused
+// softmax / top-k / histogram / importance pass.
+//
+// Gate GEMM.  N = E is tiny, so the kernel is bound by reading x once from HBM.
+// bf16: a block owns 16 tokens; its 4 waves split the hidden dimension in
+// quarters (4x more loads in flight than one wave per tile), each feeding
+// v_mfma_f32_16x16x32_bf16 straight from global memory with 16-byte loads, and
+// the four partial tiles are summed in a fixed order through LDS.  Any bijection
+// of the k index onto (lane group, step) gives the same dot product as long as
+// A and B use the same one, so every lane reads 64 contiguous bytes per step.
+// f32 (and odd shapes): one wave per token with plain FMAs.
+//
+// Routing pass.  A group of G = pow2 >= min(E,64) lanes owns one token; values
+// stay in registers, maxima / sums / arg-max run over xor-shuffles inside the
+// group.  Per-block histogram and probability column sums go to a workspace and
+// a second tiny kernel reduces them in a fixed order (bit-reproducible, no
+// float atomics) and evaluates the auxiliary loss.
+#include <limits.h>
+#include <math.h>
+
+#include "ats_common.hpp"
+
+namespace ats {
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
+
+union Frag16 {
+    uint4 u;
+    bf16x8_t v;
+};
+
+constexpr int kGateKC = 128;  // k elements consumed per wave per step
+
+// NT = number of 16-wide expert tiles.
+template <int NT>
+__global__ __launch_bounds__(256) void gate_gemm_bf16_kernel(const bf16_t* __restrict__ x,
+                                                             const bf16_t* __restrict__ wg,
+                                                             const float* __restrict__ bias,
+                                                             float* __restrict__ logits, int64_t T, int H,
+                                                             int E) {
+    __shared__ float red[4][NT][16 * 16];
+    const int lane = lane_id();
+    const int wave = threadIdx.x >> 6;
+    const int r = lane & 15;   // A: token row inside the tile; B: expert inside the tile
+    const int g = lane >> 4;   // lane group -> 32-element k slice of each 128-element step
+    const int64_t t0 = (int64_t)blockIdx.x * 16;
+    const int64_t trow = t0 + r;
+    const bool row_ok = trow < T;
+
+    // this wave's k range (multiple of kGateKC per wave, tail handled by predicates)
+    const int steps_total = (H + kGateKC - 1) / kGateKC;
+    const int steps_per_wave = (steps_total + 3) / 4;
+    const int s_begin = wave * steps_per_wave;
+    const int s_end = min(steps_total, s_begin + steps_per_wave);
+
+    f32x4_t acc[NT];
+#pragma unroll
+    for (int n = 0; n < NT; ++n) acc[n] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+    const bf16_t* xrow = x + (row_ok ? trow : 0) * (int64_t)H;
+    const uint4 zero4 = make_uint4(0, 0, 0, 0);
+
+    for (int s = s_begin; s < s_end; ++s) {
+        const int kb = s * kGateKC + g * 32;
+        Frag16 a[4];
+        Frag16 b[NT][4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int kk = kb + i * 8;
+            a[i].u = (row_ok && kk < H) ? *reinterpret_cast<const uint4*>(xrow + kk) : zero4;
+        }
+#pragma unroll
+        for (int n = 0; n < NT; ++n) {
+            const int e = n * 16 + r;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int kk = kb + i * 8;
+                b[n][i].u = (e < E && kk < H) ? *reinterpret_cast<const uint4*>(wg + (int64_t)e * H + kk) : zero4;
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+#pragma unroll
+            for (int n = 0; n < NT; ++n)
+                acc[n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i].v, b[n][i].v, acc[n], 0, 0, 0);
+        }
+    }
+    // D layout of the 16x16 tile: lane holds column (lane & 15), rows 4*(lane>>4) + v.
+#pragma unroll
+    for (int n = 0; n < NT; ++n) {
+#pragma unroll
+        for (int v = 0; v < 4; ++v) red[wave][n][(4 * g + v) * 16 + r] = acc[n][v];
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < NT * 256; i += 256) {
+        const int n = i >> 8;
+        const int row = (i & 255) >> 4;
+        const int col = i & 15;
+        const int e = n * 16 + col;
+        const int64_t t = t0 + row;
+        if (t < T && e < E) {
+            float v = ((red[0][n][i & 255] + red[1][n][i & 255]) + red[2][n][i & 255]) + red[3][n][i & 255];
+            if (bias) v += bias[e];
+            logits[t * E + e] = v;
+        }
+    }
+}
+
+// One wave per token, 8 experts at a time.  Works for every dtype / shape.
+template <typename T>
+__global__ __launch_bounds__(256) void gate_gemm_generic_kernel(const T* __restrict__ x, const T* __restrict__ wg,
+                                                                const float* __restrict__ bias,
+                                                                float* __restrict__ logits, int64_t Tn, int H,
+                                                                int E) {
+    const int lane = lane_id();
+    const int64_t wave = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    const int64_t nwaves = (int64_t)gridDim.x * (blockDim.x >> 6);
+    for (int64_t t = wave; t < Tn; t += nwaves) {
+        const T* xr = x + t * H;
+        for (int e0 = 0; e0 < E; e0 += 8) {
+            float acc[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) acc[j] = 0.f;
+            for (int h = lane; h < H; h += kWave) {
+                const float xv = Elem<T>::load(xr + h);
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    if (e0 + j < E) acc[j] += xv * Elem<T>::load(wg + (int64_t)(e0 + j) * H + h);
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const float s = wave_sum(acc[j]);
+                if (lane == 0 && e0 + j < E) logits[t * E + e0 + j] = s + (bias ? bias[e0 + j] : 0.f);
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------ routing pass
+__device__ __forceinline__ float group_max(float v, int G) {
+    for (int off = G >> 1; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+    return v;
+}
+__device__ __forceinline__ float group_sum(float v, int G) {
+    for (int off = G >> 1; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+// Order used for selection: larger value first, lower index among equals; NaN
+// ranks above every number (as torch.topk does).
+__device__ __forceinline__ bool key_before(float va, int ia, float vb, int ib) {
+    const bool na = va != va, nb = vb != vb;
+    if (na != nb) return na;
+    if (!na && va != vb) return va > vb;
+    return ia < ib;
+}
+
+constexpr int kRouteMaxK = 16;
+
+template <int VPL>
+__global__ __launch_bounds__(256) void route_topk_kernel(const float* __restrict__ logits, int64_t T, int E, int k,
+                                                         float temperature, int variant, int G, int iters,
+                                                         int32_t* __restrict__ idx_out, float* __restrict__ w_out,
+                                                         int32_t* __restrict__ part_hist,
+                                                         float* __restrict__ part_colsum) {
+    extern __shared__ unsigned char smem_raw[];
+    int* s_hist = reinterpret_cast<int*>(smem_raw);            // [E]
+    float* s_col = reinterpret_cast<float*>(s_hist + E);        // [4][E]
+    const bool want_stats = part_hist != nullptr;
+    const int lane = lane_id();
+    const int wave = threadIdx.x >> 6;
+    const int gl = lane & (G - 1);          // lane inside the group
+    const int grp = lane / G;               // group inside the wave
+    const int groups_per_wave = kWave / G;
+    const int groups_per_block = 4 * groups_per_wave;
+
+    if (want_stats) {
+        for (int i = threadIdx.x; i < E; i += 256) s_hist[i] = 0;
+        __syncthreads();
+    }
+    float col[VPL];
+#pragma unroll
+    for (int i = 0; i < VPL; ++i) col[i] = 0.f;
+
+    const float neg_inf = -INFINITY;
+    for (int it = 0; it < iters; ++it) {
+        const int64_t t = ((int64_t)blockIdx.x * iters + it) * groups_per_block + wave * groups_per_wave + grp;
+        const bool tok_ok = t < T;
+        float v[VPL];
+#pragma unroll
+        for (int i = 0; i < VPL; ++i) {
+            const int e = gl + i * G;
+            v[i] = (tok_ok && e < E) ? logits[t * E + e] : neg_inf;
+        }
+        // softmax of the raw logits (importance term of the auxiliary loss)
+        float m0 = neg_inf;
+#pragma unroll
+        for (int i = 0; i < VPL; ++i) m0 = fmaxf(m0, v[i]);
+        m0 = group_max(m0, G);
+        float p0[VPL];
+        float s0 = 0.f;
+#pragma unroll
+        for (int i = 0; i < VPL; ++i) {
+            p0[i] = (gl + i * G < E) ? expf(v[i] - m0) : 0.f;
+            s0 += p0[i];
+        }
+        s0 = group_sum(s0, G);
+#pragma unroll
+        for (int i = 0; i < VPL; ++i) {
+            p0[i] = p0[i] / s0;
+            if (tok_ok) col[i] += p0[i];
+        }
+        // tempered values and (variant 0) their softmax
+        float sv[VPL], p[VPL];
+        if (temperature == 1.0f) {
+#pragma unroll
+            for (int i = 0; i < VPL; ++i) {
+                sv[i] = v[i];
+                p[i] = p0[i];
+            }
+        } else {
+            float m = neg_inf;
+#pragma unroll
+            for (int i = 0; i < VPL; ++i) {
+                sv[i] = (gl + i * G < E) ? __fdiv_rn(v[i], temperature) : neg_inf;
+                m = fmaxf(m, sv[i]);
+            }
+            m = group_max(m, G);
+            float s = 0.f;
+#pragma unroll
+            for (int i = 0; i < VPL; ++i) {
+                p[i] = (gl + i * G < E) ? expf(sv[i] - m) : 0.f;
+                s += p[i];
+            }
+            s = group_sum(s, G);
+#pragma unroll
+            for (int i = 0; i < VPL; ++i) p[i] = p[i] / s;
+        }
+        // k rounds of group-wide arg-max
+        unsigned taken = 0;   // bit i: v[i] already selected
+        float sel_val = 0.f;  // lane j < k of the group keeps choice j: value ...
+        float sel_p = 0.f;    // ... its softmax probability ...
+        int sel_idx = 0;      // ... and expert id
+        for (int j = 0; j < k; ++j) {
+            float bv = neg_inf;
+            int bi = INT_MAX;
+            float bp = 0.f;
+#pragma unroll
+            for (int i = 0; i < VPL; ++i) {
+                const int e = gl + i * G;
+                if (e < E && !((taken >> i) & 1u) && key_before(sv[i], e, bv, bi)) {
+                    bv = sv[i];
+                    bi = e;
+                    bp = p[i];
+                }
+            }
+            for (int off = G >> 1; off > 0; off >>= 1) {
+                const float ov = __shfl_xor(bv, off, 64);
+                const int oi = __shfl_xor(bi, off, 64);
+                const float op = __shfl_xor(bp, off, 64);
+                if (key_before(ov, oi, bv, bi)) {
+                    bv = ov;
+                    bi = oi;
+                    bp = op;
+                }
+            }
+            // owner marks its value as used
+#pragma unroll
+            for (int i = 0; i < VPL; ++i)
+                if (gl + i * G == bi) taken |= 1u << i;
+            // k <= G always holds: G >= min(E, 64) and k <= min(E, kRouteMaxK)
+            if (gl == j) {
+                sel_val = bv;
+                sel_p = bp;
+                sel_idx = bi;
+            }
+            if (want_stats && tok_ok && gl == 0) atomicAdd(&s_hist[bi], 1);
+        }
+        // weights: lanes 0..k-1 of the group hold the choices in rank order
+        float wsel;
+        const bool is_sel = gl < k;
+        if (variant == ATS_ROUTE_SOFTMAX_TOPK) {
+            float tot = 0.f;
+            for (int j = 0; j < k; ++j) tot += __shfl(sel_p, grp * G + j, 64);
+            wsel = sel_p / (tot + 1e-9f);
+        } else {
+            const float mx = __shfl(sel_val, grp * G, 64);
+            const float ex = is_sel ? expf(sel_val - mx) : 0.f;
+            float tot = 0.f;
+            for (int j = 0; j < k; ++j) tot += __shfl(ex, grp * G + j, 64);
+            wsel = ex / tot;
+        }
+        if (tok_ok && is_sel) {
+            idx_out[t * k + gl] = sel_idx;
+            w_out[t * k + gl] = wsel;
+        }
+    }
+    if (want_stats) {
+        // fold the groups of a wave together (fixed butterfly), then the 4 waves via LDS
+#pragma unroll
+        for (int i = 0; i < VPL; ++i) {
+            float c = col[i];
+            for (int off = 32; off >= G; off >>= 1) c += __shfl_xor(c, off, 64);
+            const int e = gl + i * G;
+            if (grp == 0 && e < E) s_col[wave * E + e] = c;
+        }
+        __syncthreads();
+        for (int e = threadIdx.x; e < E; e += 256) {
+            part_hist[(int64_t)blockIdx.x * E + e] = s_hist[e];
+            part_colsum[(int64_t)blockIdx.x * E + e] = ((s_col[e] + s_col[E + e]) + s_col[2 * E + e]) + s_col[3 * E + e];
+        }
+    }
+}
+
+// Reduces the per-block partials in a fixed order and evaluates the auxiliary loss.
+__global__ __launch_bounds__(256) void route_finalize_kernel(const int32_t* __restrict__ part_hist,
+                                                             const float* __restrict__ part_colsum, int nblocks,
+                                                             int E, int64_t T, int k, float lbw,
+                                                             int32_t* __restrict__ hist, float* __restrict__ colsum,
+                                                             float* __restrict__ aux) {
+    extern __shared__ unsigned char smem_raw[];
+    float* s_term = reinterpret_cast<float*>(smem_raw);  // [E]
+    const int lane = lane_id();
+    const int wave = threadIdx.x >> 6;
+    for (int e = wave; e < E; e += 4) {
+        int hsum = 0;
+        float csum = 0.f;
+        for (int b = lane; b < nblocks; b += kWave) {
+            hsum += part_hist[(int64_t)b * E + e];
+            csum += part_colsum[(int64_t)b * E + e];
+        }
+        for (int off = 32; off > 0; off >>= 1) {
+            hsum += __shfl_xor(hsum, off, 64);
+            csum += __shfl_xor(csum, off, 64);
+        }
+        if (lane == 0) {
+            hist[e] = hsum;
+            colsum[e] = csum;
+            const float usage = (float)hsum / (float)((double)T * k + 1e-9);
+            const float importance = csum / (float)T;
+            s_term[e] = usage * importance;
+        }
+    }
+    __syncthreads();
+    if (threadIdx.x == 0 && aux) {
+        float s = 0.f;
+        for (int e = 0; e < E; ++e) s += s_term[e];
+        aux[0] = fminf(s * (float)E * lbw, 1.0f);
+    }
+}
+
+static int route_grid(int64_t T, int E, int* G_out, int* iters_out) {
+    int G = 1;
+    while (G < E && G < kWave) G <<= 1;
+    const int groups_per_block = 4 * (kWave / G);
+    int64_t iters = (T + (int64_t)512 * groups_per_block - 1) / ((int64_t)512 * groups_per_block);
+    if (iters < 1) iters = 1;
+    if (iters > 64) iters = 64;
+    const int64_t per_block = (int64_t)groups_per_block * iters;
+    *G_out = G;
+    *iters_out = (int)iters;
+    return (int)((T + per_block - 1) / per_block);
+}
+
+}  // namespace ats
+
+extern "C" int ats_router_logits(const void* x, const void* wg, const float* bias, float* logits, int64_t T, int H,
+                                 int E, int dtype, ats_stream_t stream) {
+    using namespace ats;
+    ATS_REQUIRE(T >= 0 && H > 0 && E > 0, ATS_ERR_INVALID_ARG, "ats_router_logits: T=%lld H=%d E=%d", (long long)T, H,
+                E);
+    ATS_REQUIRE(dtype == ATS_F32 || dtype == ATS_BF16, ATS_ERR_UNSUPPORTED, "ats_router_logits: dtype tag %d", dtype);
+    if (T == 0) return ATS_OK;
+    ATS_REQUIRE(x && wg && logits, ATS_ERR_INVALID_ARG, "ats_router_logits: null pointer");
+    hipStream_t s = as_stream(stream);
+    const bool mfma_ok = dtype == ATS_BF16 && H % 8 == 0 && aligned16(x) && aligned16(wg) && E <= 128;
+    if (mfma_ok) {
+        const unsigned blocks = (unsigned)((T + 15) / 16);
+        const bf16_t* xp = static_cast<const bf16_t*>(x);
+        const bf16_t* wp = static_cast<const bf16_t*>(wg);
+        const int nt = (E + 15) / 16;
+        if (nt <= 1)
+            hipLaunchKernelGGL((gate_gemm_bf16_kernel<1>), dim3(blocks), dim3(256), 0, s, xp, wp, bias, logits, T, H, E);
+        else if (nt <= 2)
+            hipLaunchKernelGGL((gate_gemm_bf16_kernel<2>), dim3(blocks), dim3(256), 0, s, xp, wp, bias, logits, T, H, E);
+        else if (nt <= 4)
+            hipLaunchKernelGGL((gate_gemm_bf16_kernel<4>), dim3(blocks), dim3(256), 0, s, xp, wp, bias, logits, T, H, E);
+        else
+            hipLaunchKernelGGL((gate_gemm_bf16_kernel<8>), dim3(blocks), dim3(256), 0, s, xp, wp, bias, logits, T, H, E);
+    } else {
+        int64_t blocks = (T + 3) / 4;
+        if (blocks > 8192) blocks = 8192;
+        if (dtype == ATS_F32)
+            hipLaunchKernelGGL((gate_gemm_generic_kernel<float>), dim3((unsigned)blocks), dim3(256), 0, s,
+                               static_cast<const float*>(x), static_cast<const float*>(wg), bias, logits, T, H, E);
+        else
+            hipLaunchKernelGGL((gate_gemm_generic_kernel<bf16_t>), dim3((unsigned)blocks), dim3(256), 0, s,
+                               static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(wg), bias, logits, T, H, E);
+    }
+    ATS_CHECK_LAUNCH("ats_router_logits");
+    return ATS_OK;
+}
+
+extern "C" size_t ats_route_topk_workspace(int64_t T, int E) {
+    using namespace ats;
+    if (T <= 0 || E <= 0) return 0;
+    int G, iters;
+    const int nblocks = route_grid(T, E, &G, &iters);
+    return (size_t)nblocks * E * (sizeof(int32_t) + sizeof(float));
+}
+
+extern "C" int ats_route_topk(const float* logits, int64_t T, int E, int k, float temperature, int variant,
+                              int32_t* idx_out, float* w_out, int32_t* hist, float* prob_colsum, float* aux,
+                              float load_balancing_weight, void* workspace, size_t workspace_bytes,
+                              ats_stream_t stream) {
+    using namespace ats;
+    ATS_REQUIRE(T >= 0 && E > 0 && E <= 1024 && k > 0 && k <= E && k <= kRouteMaxK, ATS_ERR_INVALID_ARG,
+                "ats_route_topk: T=%lld E=%d k=%d (need 1 <= k <= min(E,%d), E <= 1024)", (long long)T, E, k,
+                kRouteMaxK);
+    ATS_REQUIRE(variant == ATS_ROUTE_SOFTMAX_TOPK || variant == ATS_ROUTE_TOPK_SOFTMAX, ATS_ERR_INVALID_ARG,
+                "ats_route_topk: variant %d", variant);
+    ATS_REQUIRE(temperature > 0.f, ATS_ERR_INVALID_ARG, "ats_route_topk: temperature %g", temperature);
+    const bool stats = hist != nullptr;
+    ATS_REQUIRE((hist != nullptr) == (prob_colsum != nullptr), ATS_ERR_INVALID_ARG,
+                "ats_route_topk: hist and prob_colsum must be given together");
+    ATS_REQUIRE(stats || aux == nullptr, ATS_ERR_INVALID_ARG, "ats_route_topk: aux needs hist and prob_colsum");
+    if (T == 0) return ATS_OK;
+    ATS_REQUIRE(logits && idx_out && w_out, ATS_ERR_INVALID_ARG, "ats_route_topk: null pointer");
+    int G, iters;
+    const int nblocks = route_grid(T, E, &G, &iters);
+    int32_t* part_hist = nullptr;
+    float* part_col = nullptr;
+    if (stats) {
+        const size_t need = (size_t)nblocks * E * (sizeof(int32_t) + sizeof(float));
+        ATS_REQUIRE(workspace && workspace_bytes >= need, ATS_ERR_WORKSPACE,
+                    "ats_route_topk: workspace %zu bytes, need %zu", workspace_bytes, need);
+        part_hist = static_cast<int32_t*>(workspace);
+        part_col = reinterpret_cast<float*>(part_hist + (size_t)nblocks * E);
+    }
+    hipStream_t s = as_stream(stream);
+    const size_t smem = (size_t)E * 5 * sizeof(float);
+    const int vpl = (E + G - 1) / G;
+    if (vpl <= 1)
+        hipLaunchKernelGGL((route_topk_kernel<1>), dim3(nblocks), dim3(256), smem, s, logits, T, E, k, temperature,
+                           variant, G, iters, idx_out, w_out, part_hist, part_col);
+    else if (vpl <= 4)
+        hipLaunchKernelGGL((route_topk_kernel<4>), dim3(nblocks), dim3(256), smem, s, logits, T, E, k, temperature,
+                           variant, G, iters, idx_out, w_out, part_hist, part_col);
+    else
+        hipLaunchKernelGGL((route_topk_kernel<16>), dim3(nblocks), dim3(256), smem, s, logits, T, E, k, temperature,
+                           variant, G, iters, idx_out, w_out, part_hist, part_col);
+    ATS_CHECK_LAUNCH("ats_route_topk");
+    if (stats) {
+        hipLaunchKernelGGL(route_finalize_kernel, dim3(1), dim3(256), (size_t)E * sizeof(float), s, part_hist,
+                           part_col, nblocks, E, T, k, load_balancing_weight, hist, prob_colsum, aux);
+        ATS_CHECK_LAUNCH("ats_route_topk(finalize)");
+    }
+    return ATS_OK;
+}

@@ -1,0 +1,409 @@
+"""Module-level API of the sparse-layer path, with the reference's names and
+call signatures, backed only by the gfx950 HIP kernels.
+
+Reference interfaces mirrored here (paths relative to the reference checkout,
+MS = Src/Main_Scripts):
+  RMSNorm                MS/core/model.py:228-305
+  RotaryEmbedding        MS/core/model.py:334-467
+  apply_rotary_pos_emb   MS/core/model.py:527-558
+  SwiGLUExpert           MS/core/model.py:1027-1088
+  MoEFFNLayer            MS/core/model.py:1090-1302  (routing: softmax -> top-k -> renormalise)
+  CapacityMoEFFNLayer    MS/core/moe_cuda_wrapper.py:362-526 (routing: top-k -> softmax, FCFS capacity)
+  MoECUDAOps             MS/core/moe_cuda_wrapper.py:162-359
+  FusedRMSNorm/FusedRoPE/FusedSwiGLU   MS/core/cuda_opt_wrapper.py:261-478
+  MoDRouter              MS/core/model.py:860-1020
+
+Differences that are deliberate:
+  * no PyTorch/CPU fallback: CPU tensors or a missing library raise AtsError
+    (the reference silently falls back);
+  * forward only: outputs carry no autograd graph;
+  * no device synchronisation inside any op (the reference synchronises after
+    every kernel);
+  * FusedRMSNorm returns the input dtype (the reference's fused wrapper
+    returns float32 for every input dtype);
+  * routing ties are broken toward the lower expert id.
+"""
+from __future__ import annotations
+
+import math
+from typing import Any, Dict, Optional, Tuple
+
+import torch
+import torch.nn as nn
+
+from . import ops
+from ._lib import ROUTE_SOFTMAX_TOPK, ROUTE_TOPK_SOFTMAX, AtsError
+
+
+# ============================================================================ normalisation
+class RMSNorm(nn.Module):
+    """y = x * rsqrt(mean(x^2) + eps) * weight, float32 math, result in x's dtype."""
+
+    def __init__(self, dim: int, eps: float = 1e-6, elementwise_affine: bool = True):
+        super().__init__()
+        self.dim = dim
+        self.eps = eps
+        self.elementwise_affine = elementwise_affine
+        if elementwise_affine:
+            self.weight = nn.Parameter(torch.ones(dim))
+        else:
+            self.register_parameter("weight", None)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        if x.shape[-1] != self.dim:
+            raise AtsError(f"RMSNorm: last dimension {x.shape[-1]} != {self.dim}")
+        return ops.rmsnorm(x, self.weight if self.elementwise_affine else None, self.eps)
+
+    def extra_repr(self) -> str:
+        return f"dim={self.dim}, eps={self.eps}, elementwise_affine={self.elementwise_affine}, backend=gfx950"
+
+
+class FusedRMSNorm(nn.Module):
+    """Constructor and attributes of the reference's FusedRMSNorm(hidden_size, eps)."""
+
+    def __init__(self, hidden_size: int, eps: float = 1e-6):
+        super().__init__()
+        self.hidden_size = hidden_size
+        self.eps = eps
+        self.weight = nn.Parameter(torch.ones(hidden_size))
+        self.cuda_enabled = True
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return ops.rmsnorm(x, self.weight, self.eps)
+
+
+# ============================================================================ rotary embedding
+class RotaryEmbedding(nn.Module):
+    """cos/sin tables [seq_len, dim] (float32, halves duplicated), evaluated in
+    float64 by a GPU kernel, cached per device and extended on demand."""
+
+    def __init__(self, dim: int, max_seq_len: int = 8192, theta: float = 10000.0,
+                 scaling_factor: Optional[float] = None):
+        super().__init__()
+        self.dim = dim
+        self.max_seq_len = max_seq_len
+        self.theta = theta
+        self.scaling_factor = scaling_factor
+        inv_freq = 1.0 / (theta ** (torch.arange(0, dim, 2, dtype=torch.float64) / dim))
+        self.register_buffer("inv_freq", inv_freq.float(), persistent=False)
+        self._tables: Dict[Any, Tuple[torch.Tensor, torch.Tensor]] = {}
+
+    def _extend_cache(self, seq_len: int) -> None:
+        if seq_len > self.max_seq_len:
+            self.max_seq_len = seq_len
+            self._tables.clear()
+
+    def forward(self, seq_len: int, device) -> Tuple[torch.Tensor, torch.Tensor]:
+        device = torch.device(device)
+        if device.type != "cuda":
+            raise AtsError("RotaryEmbedding: tables are built on the GPU; pass a cuda device")
+        self._extend_cache(seq_len)
+        key = (device.type, device.index if device.index is not None else torch.cuda.current_device())
+        if key not in self._tables:
+            self._tables[key] = ops.rope_table(self.max_seq_len, self.dim, self.theta, self.scaling_factor,
+                                               half=False, device=device)
+        cos, sin = self._tables[key]
+        return cos[:seq_len], sin[:seq_len]
+
+    def extra_repr(self) -> str:
+        return f"dim={self.dim}, max_seq_len={self.max_seq_len}, theta={self.theta}, backend=gfx950"
+
+
+def apply_rotary_pos_emb(q: torch.Tensor, k: torch.Tensor, cos: torch.Tensor,
+                         sin: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """q [B,Hq,L,D], k [B,Hkv,L,D], cos/sin [L, D] -> rotated (q, k) in the input dtype."""
+    return ops.rope(q, k, cos, sin, 0)
+
+
+class FusedRoPE(nn.Module):
+    """Constructor, cache attributes ([max_seq, head_dim/2]) and forward(q, k, position_offset)
+    of the reference's FusedRoPE.  The table is the float64-evaluated one."""
+
+    def __init__(self, head_dim: int, max_seq_len: int = 8192, theta: float = 10000.0):
+        super().__init__()
+        self.head_dim = head_dim
+        self.max_seq_len = max_seq_len
+        self.theta = theta
+        self.cuda_enabled = True
+        self.cos_cache, self.sin_cache = ops.rope_table(max_seq_len, head_dim, theta, None, half=True)
+
+    def forward(self, q: torch.Tensor, k: torch.Tensor, position_offset: int = 0):
+        if self.cos_cache.device != q.device:
+            self.cos_cache = self.cos_cache.to(q.device)
+            self.sin_cache = self.sin_cache.to(q.device)
+        return ops.rope(q, k, self.cos_cache, self.sin_cache, position_offset)
+
+
+# ============================================================================ experts
+class SwiGLUExpert(nn.Module):
+    """down(silu(gate) * up) with the fused [2I, H] gate/up weight (gate = first I rows)."""
+
+    def __init__(self, config):
+        super().__init__()
+        self.gate_up_proj = nn.Linear(config.hidden_size, config.intermediate_size * 2, bias=False)
+        self.down_proj = nn.Linear(config.intermediate_size, config.hidden_size, bias=False)
+        self._param_count = sum(p.numel() for p in self.parameters())
+        self._init_weights(config)
+
+    def _init_weights(self, config) -> None:
+        std = getattr(config, "init_std", 0.02)
+        nn.init.normal_(self.gate_up_proj.weight, mean=0.0, std=std)
+        down_std = std / math.sqrt(2 * getattr(config, "num_layers", 1))
+        if hasattr(config, "expert_output_scaling"):
+            down_std *= config.expert_output_scaling
+        nn.init.normal_(self.down_proj.weight, mean=0.0, std=down_std)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        """One expert over every row of x, through the grouped kernels with a single group."""
+        shape = x.shape
+        x2 = x.reshape(-1, shape[-1]).contiguous()
+        n = x2.shape[0]
+        H, I = self.gate_up_proj.in_features, self.down_proj.in_features
+        wgu = _as_dtype(self.gate_up_proj.weight, x2.dtype)
+        wd = _as_dtype(self.down_proj.weight, x2.dtype)
+        start = torch.zeros(1, dtype=torch.int32, device=x.device)
+        count = torch.full((1,), n, dtype=torch.int32, device=x.device)
+        h = ops.grouped_gateup_swiglu(x2, ops.weight_pointer_table([wgu]), start, count, n, n, H, I)
+        y = ops.grouped_down(h, ops.weight_pointer_table([wd]), start, count, n, H, I)
+        return y.view(shape)
+
+
+def _as_dtype(w: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
+    w = w.detach()
+    if w.dtype != dtype:
+        w = w.to(dtype)
+    return w.contiguous()
+
+
+# ============================================================================ MoE layer
+class MoEFFNLayer(nn.Module):
+    """Mixture-of-experts FFN: gate Linear -> routing -> (capacity) dispatch -> SwiGLU experts ->
+    weighted combine, plus the load-balancing auxiliary loss.  forward(x [B,L,H]) -> (out, aux).
+
+    Attributes read on every call, so a trainer may change them between steps:
+    num_experts, top_k, capacity_factor, routing_temperature, noise_std,
+    load_balancing_weight, experts (ModuleList), gate.
+
+    routing:        "softmax_topk" (softmax over experts, top-k, renormalise) or
+                    "topk_softmax" (top-k of logits, softmax over the k)
+    capacity_mode:  "none" (no token is dropped) or "fcfs" (per-expert capacity
+                    int(T*k/E * capacity_factor), first come first served in
+                    (token, choice) order; dropped choices contribute nothing)
+    """
+
+    default_routing = "softmax_topk"
+    default_capacity_mode = "none"
+
+    def __init__(self, config):
+        super().__init__()
+        self.config = config
+        self.num_experts = config.num_experts
+        self.top_k = config.moe_top_k
+        self.hidden_size = config.hidden_size
+        self.capacity_factor = getattr(config, "capacity_factor", 1.25)
+        self.use_cuda_ops = True
+        self.routing = getattr(config, "moe_routing", self.default_routing)
+        self.capacity_mode = getattr(config, "moe_capacity_mode", self.default_capacity_mode)
+        self.gate = nn.Linear(config.hidden_size, config.num_experts, bias=False)
+        self.experts = nn.ModuleList([SwiGLUExpert(config) for _ in range(config.num_experts)])
+        self.load_balancing_weight = getattr(config, "load_balancing_weight", 0.01)
+        self.routing_temperature = getattr(config, "routing_temperature", 1.0)
+        self.noise_std = getattr(config, "routing_noise_std", 0.1)
+        self.router_logit_bias: Optional[torch.Tensor] = None   # optional per-expert skew (benchmarks)
+        self._gate_param_count = sum(p.numel() for p in self.gate.parameters())
+        self._expert_param_count = self.experts[0]._param_count
+        self._routing_stats = {"expert_usage": torch.zeros(config.num_experts), "total_routed": 0,
+                               "dropped_tokens": 0}
+        self._wcache_key = None
+        self._wcache = None
+        self.last_plan = None
+        nn.init.normal_(self.gate.weight, mean=0.0, std=0.01)
+
+    # ---- expert weight tables (device arrays of pointers; rebuilt when a weight moves or changes dtype)
+    def _weight_tables(self, dtype: torch.dtype, device: torch.device):
+        params = []
+        for ex in self.experts:
+            params.append(ex.gate_up_proj.weight)
+            params.append(ex.down_proj.weight)
+        key = (dtype, device, tuple((p.data_ptr(), p._version if p.dtype != dtype else 0) for p in params))
+        if key != self._wcache_key:
+            wgu = [_as_dtype(ex.gate_up_proj.weight, dtype) for ex in self.experts]
+            wd = [_as_dtype(ex.down_proj.weight, dtype) for ex in self.experts]
+            self._wcache = (ops.weight_pointer_table(wgu), ops.weight_pointer_table(wd), wgu, wd)
+            self._wcache_key = key
+        return self._wcache
+
+    def forward(self, x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+        if x.dim() != 3 or x.shape[-1] != self.hidden_size:
+            raise AtsError(f"MoEFFNLayer: expected [batch, seq, {self.hidden_size}], got {tuple(x.shape)}")
+        if len(self.experts) != self.num_experts or self.gate.weight.shape[0] != self.num_experts:
+            raise AtsError("MoEFFNLayer: num_experts, experts and gate disagree")
+        B, L, H = x.shape
+        x_flat = x.reshape(-1, H).contiguous()
+        T = x_flat.shape[0]
+        E, k = self.num_experts, self.top_k
+        I = self.experts[0].down_proj.in_features
+
+        logits = ops.router_logits(x_flat, _as_dtype(self.gate.weight, x.dtype), self.router_logit_bias)
+        if self.training and self.noise_std > 0:
+            logits = logits + torch.randn_like(logits) * self.noise_std
+        variant = {"softmax_topk": ROUTE_SOFTMAX_TOPK, "topk_softmax": ROUTE_TOPK_SOFTMAX}[self.routing]
+        route = ops.route_topk(logits, k, self.routing_temperature, variant, self.load_balancing_weight)
+
+        if self.capacity_mode == "fcfs":
+            C = ops.expert_capacity(T, k, E, self.capacity_factor)
+        elif self.capacity_mode == "none":
+            C = T
+        else:
+            raise AtsError(f"MoEFFNLayer: capacity_mode {self.capacity_mode!r}")
+        plan = ops.dispatch_plan(route["indices"], E, C)
+        rows = min(T * k, E * C)
+        wgu_ptrs, wd_ptrs, _, _ = self._weight_tables(x.dtype, x.device)
+        if rows > 0:
+            h = ops.grouped_gateup_swiglu(x_flat, wgu_ptrs, plan["offsets"], plan["kept"], rows, rows, H, I,
+                                          a_rows=plan["row_src"], a_row_div=k)
+            y = ops.grouped_down(h, wd_ptrs, plan["offsets"], plan["kept"], rows, H, I)
+        else:
+            y = torch.zeros(1, H, dtype=x.dtype, device=x.device)
+        out = ops.combine(y, plan["row_of"], route["weights"], T, k, out_dtype=x.dtype)
+
+        self.last_plan = {"logits": logits, "capacity": C, **route, **plan}
+        if self.training:
+            self._update_routing_stats(plan, T)
+        return out.view(B, L, H), route["aux"][0]
+
+    def _update_routing_stats(self, plan, total_tokens: int) -> None:
+        hist = plan["hist"].cpu()
+        kept = plan["kept"].cpu()
+        self._routing_stats["expert_usage"] += hist.float()
+        self._routing_stats["total_routed"] += total_tokens
+        self._routing_stats["dropped_tokens"] += int((hist - kept).sum())
+
+    def get_routing_stats(self) -> Dict[str, Any]:
+        total = self._routing_stats["total_routed"]
+        if total == 0:
+            return {"error": "No routing statistics available"}
+        usage = self._routing_stats["expert_usage"].clone()
+        pct = (usage / total * 100).tolist()
+        return {
+            "expert_usage_percentages": pct, "total_tokens_routed": total,
+            "dropped_tokens": self._routing_stats["dropped_tokens"],
+            "usage_std": float(torch.std(usage / total)), "usage_min": min(pct), "usage_max": max(pct),
+            "imbalance_ratio": max(pct) / max(min(pct), 0.1),
+        }
+
+    def reset_routing_stats(self) -> None:
+        self._routing_stats = {"expert_usage": torch.zeros(self.num_experts), "total_routed": 0,
+                               "dropped_tokens": 0}
+
+
+class CapacityMoEFFNLayer(MoEFFNLayer):
+    """The capacity-factor variant: top-k on the tempered logits, softmax over the k selected,
+    first-come-first-served capacity dispatch."""
+
+    default_routing = "topk_softmax"
+    default_capacity_mode = "fcfs"
+
+
+# ============================================================================ MoECUDAOps
+class MoECUDAOps:
+    """Static operator interface of the reference's MoECUDAOps.  `use_cuda` is accepted for
+    signature compatibility; the gfx950 kernels are the only path."""
+
+    CUDA_THRESHOLD_TOKENS = 256
+    CUDA_THRESHOLD_EXPERTS = 8
+    CUDA_THRESHOLD_HIDDEN = 128
+
+    @staticmethod
+    def should_use_cuda(num_tokens: int, num_experts: int, hidden_dim: int, use_cuda: bool,
+                        device_is_cuda: bool) -> bool:
+        return bool(use_cuda and device_is_cuda)
+
+    @staticmethod
+    def topk_gating(gate_logits: torch.Tensor, k: int, temperature: float = 1.0, use_cuda: bool = True):
+        """-> (indices int64 [T,k], weights float32 [T,k]); top-k of logits/temperature, softmax over the k."""
+        r = ops.route_topk(gate_logits.float(), k, temperature, ROUTE_TOPK_SOFTMAX, with_stats=False)
+        return r["indices"].long(), r["weights"]
+
+    @staticmethod
+    def dispatch_tokens(tokens: torch.Tensor, top_k_indices: torch.Tensor, num_experts: int, capacity: int,
+                        use_cuda: bool = True):
+        """-> (expert_inputs [E,C,H] zero padded, token_map [E,C] int32, -1 = empty)."""
+        plan = ops.dispatch_plan(top_k_indices, num_experts, capacity)
+        k = top_k_indices.shape[1]
+        H = tokens.shape[1]
+        expert_inputs = ops.gather_rows(tokens, plan["token_map"].view(-1), div=k)
+        return expert_inputs.view(num_experts, capacity, H), plan["token_map"]
+
+    @staticmethod
+    def combine_expert_outputs(expert_outputs: torch.Tensor, token_map: torch.Tensor, top_k_weights: torch.Tensor,
+                               num_tokens: int, k: int, use_cuda: bool = True) -> torch.Tensor:
+        """-> [num_tokens, H]; ascending expert order, dropped choices contribute nothing."""
+        row_of = ops.invert_token_map(token_map.to(torch.int32), num_tokens * k)
+        return ops.combine(expert_outputs, row_of, top_k_weights.float(), num_tokens, k,
+                           out_dtype=expert_outputs.dtype)
+
+
+# ============================================================================ Mixture of Depths
+class MoDRouter(nn.Module):
+    """Token-level compute/skip router: sigmoid(Linear(H,1)(x) / temperature), inference branch
+    (k-th value threshold over all tokens of the batch).  forward -> (routing_weights [B,L,1],
+    routing_probs [B,L,1], None)."""
+
+    def __init__(self, hidden_size: int, capacity_factor: float = 0.5, routing_temperature: float = 1.0):
+        super().__init__()
+        self.hidden_size = hidden_size
+        self.capacity_factor = capacity_factor
+        self.routing_temperature = routing_temperature
+        self.router = nn.Linear(hidden_size, 1, bias=True)
+        self._routing_stats = {"total_tokens": 0, "computed_tokens": 0, "skipped_tokens": 0}
+        nn.init.normal_(self.router.weight, mean=0.0, std=0.01)
+        nn.init.zeros_(self.router.bias)
+
+    def forward(self, x: torch.Tensor):
+        if self.training:
+            raise NotImplementedError("MoDRouter: the training branch needs autograd, which this forward-only "
+                                      "path does not provide")
+        B, L, H = x.shape
+        _, probs = ops.row_dot(x, _as_dtype(self.router.weight, x.dtype), self.router.bias.detach(),
+                               self.routing_temperature, want_prob=True)
+        total = B * L
+        capacity = int(total * self.capacity_factor)
+        mask = ops.kth_value_mask(probs, max(1, total - capacity))
+        self._routing_stats["total_tokens"] += total
+        return mask.view(B, L, 1), probs.view(B, L, 1), None
+
+    def get_routing_stats(self) -> Dict[str, Any]:
+        total = self._routing_stats["total_tokens"]
+        if total == 0:
+            return {"error": "No routing statistics available"}
+        return {"total_tokens_routed": total, "target_capacity": self.capacity_factor}
+
+    def reset_routing_stats(self) -> None:
+        self._routing_stats = {"total_tokens": 0, "computed_tokens": 0, "skipped_tokens": 0}
+
+
+class MoDMoEBlock(nn.Module):
+    """Mixture-of-Depths in front of a capacity MoE layer: score every token with Linear(H,1),
+    keep the `keep_fraction` best per sequence (ascending position), run the MoE layer on the
+    gathered tokens and add its output onto the residual stream at the kept positions; the
+    other tokens pass through unchanged.  forward(x [B,L,H]) -> (out [B,L,H], aux)."""
+
+    def __init__(self, config):
+        super().__init__()
+        self.keep_fraction = getattr(config, "mod_keep_fraction", 0.125)
+        self.router = nn.Linear(config.hidden_size, 1, bias=False)
+        self.moe = CapacityMoEFFNLayer(config)
+        self.last_selected = None
+
+    def forward(self, x: torch.Tensor):
+        B, L, H = x.shape
+        keep = int(L * self.keep_fraction)
+        scores = ops.row_dot(x, _as_dtype(self.router.weight, x.dtype))
+        sel = ops.select_topk_per_sequence(scores.view(B, L), keep)
+        gathered = ops.gather_rows(x.reshape(-1, H), sel)
+        delta, aux = self.moe(gathered.view(1, B * keep, H))
+        out = x.reshape(-1, H).clone()
+        ops.scatter_add_rows(out, sel, delta.view(-1, H))
+        self.last_selected = sel
+        return out.view(B, L, H), aux

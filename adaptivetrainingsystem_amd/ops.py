@@ -1,0 +1,344 @@
+"""Tensor-level wrappers of the libats_gfx950 entry points.
+
+PyTorch is used for device memory and streams only: every function here
+validates shapes on the host, allocates outputs with torch, and enqueues the
+hand-written HIP kernels on torch's current stream.  Tensors must live on the
+GPU; there is no CPU path.
+"""
+from __future__ import annotations
+
+from typing import Optional, Sequence, Tuple
+
+import torch
+
+from . import _lib
+from ._lib import ATS_BF16, ATS_F32, IDX_I32, IDX_I64, ROUTE_SOFTMAX_TOPK, ROUTE_TOPK_SOFTMAX, AtsError, check
+
+_DT = {torch.float32: ATS_F32, torch.bfloat16: ATS_BF16}
+
+
+def _tag(t: torch.Tensor) -> int:
+    try:
+        return _DT[t.dtype]
+    except KeyError:
+        raise AtsError(f"unsupported dtype {t.dtype}: the gfx950 kernels take float32 or bfloat16") from None
+
+
+def _need_gpu(*tensors: Optional[torch.Tensor]) -> None:
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise AtsError("tensor is not on the GPU: the gfx950 path has no CPU fallback")
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+# --------------------------------------------------------------------------- RMSNorm
+def rmsnorm(x: torch.Tensor, weight: Optional[torch.Tensor], eps: float = 1e-6) -> torch.Tensor:
+    _need_gpu(x, weight)
+    H = x.shape[-1]
+    xc = x.contiguous()
+    if weight is not None:
+        if weight.numel() != H:
+            raise AtsError(f"rmsnorm: weight has {weight.numel()} elements, hidden size is {H}")
+        weight = weight.contiguous()
+    y = torch.empty_like(xc)
+    rows = xc.numel() // H if H else 0
+    check(_lib.load().ats_rmsnorm_fwd(xc.data_ptr(), _ptr(weight), y.data_ptr(), rows, H, float(eps), _tag(xc),
+                                      _tag(weight) if weight is not None else ATS_F32, _stream()), "ats_rmsnorm_fwd")
+    return y.view(x.shape)
+
+
+# --------------------------------------------------------------------------- RoPE
+def rope_table(seq_len: int, dim: int, theta: float = 10000.0, scaling_factor: Optional[float] = None,
+               half: bool = False, device=None) -> Tuple[torch.Tensor, torch.Tensor]:
+    device = torch.device("cuda") if device is None else torch.device(device)
+    if device.type != "cuda":
+        raise AtsError("rope_table: the table is built by a GPU kernel; pass a cuda device")
+    cols = dim // 2 if half else dim
+    cos = torch.empty(seq_len, cols, dtype=torch.float32, device=device)
+    sin = torch.empty(seq_len, cols, dtype=torch.float32, device=device)
+    with torch.cuda.device(device):
+        check(_lib.load().ats_rope_table(cos.data_ptr(), sin.data_ptr(), seq_len, dim, cols, float(theta),
+                                         1.0 if scaling_factor is None else float(scaling_factor), _stream()),
+              "ats_rope_table")
+    return cos, sin
+
+
+def _bhl_strides(t: torch.Tensor):
+    if t.stride(3) != 1:
+        t = t.contiguous()
+    return t, t.stride(0), t.stride(1), t.stride(2)
+
+
+def rope(q: torch.Tensor, k: Optional[torch.Tensor], cos: torch.Tensor, sin: torch.Tensor,
+         position_offset: int = 0) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+    """q [B,Hq,L,D], k [B,Hkv,L,D] (any batch/head/position strides), cos/sin float32
+    [>= offset+L, D or D/2].  Returns new contiguous tensors."""
+    _need_gpu(q, k, cos, sin)
+    if q.dim() != 4 or (k is not None and k.dim() != 4):
+        raise AtsError("rope: q and k must be [batch, heads, seq, head_dim]")
+    B, Hq, L, D = q.shape
+    Hkv = 0
+    if k is not None:
+        if k.shape[0] != B or k.shape[2] != L or k.shape[3] != D or k.dtype != q.dtype:
+            raise AtsError(f"rope: k {tuple(k.shape)}/{k.dtype} does not match q {tuple(q.shape)}/{q.dtype}")
+        Hkv = k.shape[1]
+    if cos.dtype != torch.float32 or sin.dtype != torch.float32 or cos.shape != sin.shape or cos.dim() != 2:
+        raise AtsError("rope: cos/sin must be float32 2-D tables of equal shape")
+    if cos.stride(1) != 1 or sin.stride(1) != 1 or cos.stride(0) != sin.stride(0):
+        cos, sin = cos.contiguous(), sin.contiguous()
+    q, qsb, qsh, qsl = _bhl_strides(q)
+    q_out = torch.empty((B, Hq, L, D), dtype=q.dtype, device=q.device)
+    k_out = None
+    ksb = ksh = ksl = 0
+    if k is not None:
+        k, ksb, ksh, ksl = _bhl_strides(k)
+        k_out = torch.empty((B, Hkv, L, D), dtype=k.dtype, device=k.device)
+    check(_lib.load().ats_rope_fwd(q.data_ptr(), _ptr(k), q_out.data_ptr(), _ptr(k_out), cos.data_ptr(),
+                                   sin.data_ptr(), cos.stride(0), cos.shape[0], B, Hq, Hkv, L, D,
+                                   int(position_offset), qsb, qsh, qsl, ksb, ksh, ksl, _tag(q), _stream()),
+          "ats_rope_fwd")
+    return q_out, k_out
+
+
+# --------------------------------------------------------------------------- router
+def router_logits(x: torch.Tensor, gate_weight: torch.Tensor, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """x [T,H], gate_weight [E,H] (same dtype) -> float32 logits [T,E]."""
+    _need_gpu(x, gate_weight, bias)
+    if x.dim() != 2 or gate_weight.dim() != 2 or x.shape[1] != gate_weight.shape[1] or x.dtype != gate_weight.dtype:
+        raise AtsError(f"router_logits: x {tuple(x.shape)}/{x.dtype} vs weight {tuple(gate_weight.shape)}/{gate_weight.dtype}")
+    T, H = x.shape
+    E = gate_weight.shape[0]
+    x, gate_weight = x.contiguous(), gate_weight.contiguous()
+    if bias is not None:
+        if bias.numel() != E:
+            raise AtsError("router_logits: bias must have one entry per expert")
+        bias = bias.to(torch.float32).contiguous()
+    logits = torch.empty(T, E, dtype=torch.float32, device=x.device)
+    check(_lib.load().ats_router_logits(x.data_ptr(), gate_weight.data_ptr(), _ptr(bias), logits.data_ptr(), T, H, E,
+                                        _tag(x), _stream()), "ats_router_logits")
+    return logits
+
+
+def route_topk(logits: torch.Tensor, k: int, temperature: float = 1.0, variant: int = ROUTE_SOFTMAX_TOPK,
+               load_balancing_weight: float = 0.01, with_stats: bool = True):
+    """float32 logits [T,E] -> dict(indices int32 [T,k], weights f32 [T,k], hist int32 [E],
+    prob_colsum f32 [E], aux f32 [1])."""
+    _need_gpu(logits)
+    if logits.dim() != 2 or logits.dtype != torch.float32:
+        raise AtsError("route_topk: logits must be a float32 [tokens, experts] tensor")
+    logits = logits.contiguous()
+    T, E = logits.shape
+    dev = logits.device
+    idx = torch.empty(T, k, dtype=torch.int32, device=dev)
+    w = torch.empty(T, k, dtype=torch.float32, device=dev)
+    hist = colsum = aux = ws = None
+    ws_bytes = 0
+    lib = _lib.load()
+    if with_stats:
+        hist = torch.zeros(E, dtype=torch.int32, device=dev)
+        colsum = torch.zeros(E, dtype=torch.float32, device=dev)
+        aux = torch.zeros(1, dtype=torch.float32, device=dev)
+        ws_bytes = lib.ats_route_topk_workspace(T, E)
+        ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
+    check(lib.ats_route_topk(logits.data_ptr(), T, E, int(k), float(temperature), int(variant), idx.data_ptr(),
+                             w.data_ptr(), _ptr(hist), _ptr(colsum), _ptr(aux), float(load_balancing_weight),
+                             _ptr(ws), ws_bytes, _stream()), "ats_route_topk")
+    return {"indices": idx, "weights": w, "hist": hist, "prob_colsum": colsum, "aux": aux}
+
+
+# --------------------------------------------------------------------------- dispatch
+def expert_capacity(total_tokens: int, top_k: int, num_experts: int, capacity_factor: float) -> int:
+    """Host-side integer, in double arithmetic then truncated, exactly as the reference computes it."""
+    return int((total_tokens * top_k / num_experts) * capacity_factor)
+
+
+def dispatch_plan(indices: torch.Tensor, num_experts: int, capacity: int):
+    """indices [T,k] int32/int64 -> dict of int32 tensors: slot [T*k], token_map [E,C], hist [E],
+    kept [E], offsets [E+1], row_src [min(T*k,E*C)], row_of [T*k], status [1]."""
+    _need_gpu(indices)
+    if indices.dim() != 2 or indices.dtype not in (torch.int32, torch.int64):
+        raise AtsError("dispatch_plan: indices must be an int32/int64 [tokens, k] tensor")
+    indices = indices.contiguous()
+    T, k = indices.shape
+    E, C = int(num_experts), int(capacity)
+    dev = indices.device
+    i32 = dict(dtype=torch.int32, device=dev)
+    n = T * k
+    out = {
+        "slot": torch.empty(n, **i32), "token_map": torch.empty(E, C, **i32), "hist": torch.empty(E, **i32),
+        "kept": torch.empty(E, **i32), "offsets": torch.empty(E + 1, **i32),
+        "row_src": torch.empty(max(1, min(n, E * C)), **i32), "row_of": torch.empty(n, **i32),
+        "status": torch.empty(1, **i32),
+    }
+    lib = _lib.load()
+    ws_bytes = max(lib.ats_dispatch_plan_workspace(max(T, 1), k, E), 4 * E)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    check(lib.ats_dispatch_plan(indices.data_ptr(), IDX_I64 if indices.dtype == torch.int64 else IDX_I32, T, k, E, C,
+                                out["slot"].data_ptr(), out["token_map"].data_ptr(), out["hist"].data_ptr(),
+                                out["kept"].data_ptr(), out["offsets"].data_ptr(), out["row_src"].data_ptr(),
+                                out["row_of"].data_ptr(), out["status"].data_ptr(), ws.data_ptr(), ws_bytes,
+                                _stream()), "ats_dispatch_plan")
+    return out
+
+
+def gather_rows(src: torch.Tensor, row_map: torch.Tensor, div: int = 1) -> torch.Tensor:
+    """out[r] = src[row_map[r] // div] (zeros where row_map[r] < 0)."""
+    _need_gpu(src, row_map)
+    if src.dim() != 2 or row_map.dtype != torch.int32:
+        raise AtsError("gather_rows: src must be 2-D and row_map int32")
+    src, row_map = src.contiguous(), row_map.contiguous()
+    n, H = row_map.numel(), src.shape[1]
+    out = torch.empty(n, H, dtype=src.dtype, device=src.device)
+    check(_lib.load().ats_gather_rows(src.data_ptr(), row_map.data_ptr(), int(div), out.data_ptr(), n, H, _tag(src),
+                                      _stream()), "ats_gather_rows")
+    return out
+
+
+def invert_token_map(token_map: torch.Tensor, n_assign: int) -> torch.Tensor:
+    _need_gpu(token_map)
+    if token_map.dtype != torch.int32:
+        raise AtsError("invert_token_map: token_map must be int32")
+    token_map = token_map.contiguous()
+    row_of = torch.empty(n_assign, dtype=torch.int32, device=token_map.device)
+    check(_lib.load().ats_invert_token_map(token_map.data_ptr(), token_map.numel(), row_of.data_ptr(), n_assign,
+                                           _stream()), "ats_invert_token_map")
+    return row_of
+
+
+# --------------------------------------------------------------------------- expert FFN
+def weight_pointer_table(weights: Sequence[torch.Tensor]) -> torch.Tensor:
+    """Device array of the experts' weight base addresses (int64)."""
+    for w in weights:
+        _need_gpu(w)
+        if not w.is_contiguous():
+            raise AtsError("expert weights must be contiguous")
+    return torch.tensor([w.data_ptr() for w in weights], dtype=torch.int64, device=weights[0].device)
+
+
+def grouped_gateup_swiglu(a: torch.Tensor, w_gu_ptrs: torch.Tensor, row_start: torch.Tensor, row_count: torch.Tensor,
+                          n_rows_out: int, max_rows: int, H: int, I: int, a_rows: Optional[torch.Tensor] = None,
+                          a_row_div: int = 1) -> torch.Tensor:
+    _need_gpu(a, w_gu_ptrs, row_start, row_count, a_rows)
+    if a.dim() != 2 or a.shape[1] != H or not a.is_contiguous():
+        raise AtsError("grouped_gateup_swiglu: activations must be a contiguous [rows, H] tensor")
+    E = w_gu_ptrs.numel()
+    if row_start.numel() < E or row_count.numel() < E or row_start.dtype != torch.int32 or row_count.dtype != torch.int32:
+        raise AtsError("grouped_gateup_swiglu: row_start/row_count must be int32 with one entry per expert")
+    h = torch.empty(n_rows_out, I, dtype=a.dtype, device=a.device)
+    check(_lib.load().ats_grouped_gateup_swiglu(a.data_ptr(), _ptr(a_rows), int(a_row_div), w_gu_ptrs.data_ptr(),
+                                                h.data_ptr(), row_start.data_ptr(), row_count.data_ptr(), E,
+                                                int(max_rows), H, I, _tag(a), _stream()), "ats_grouped_gateup_swiglu")
+    return h
+
+
+def grouped_down(h: torch.Tensor, w_d_ptrs: torch.Tensor, row_start: torch.Tensor, row_count: torch.Tensor,
+                 max_rows: int, H: int, I: int, out: Optional[torch.Tensor] = None,
+                 out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    _need_gpu(h, w_d_ptrs, row_start, row_count, out)
+    if h.dim() != 2 or h.shape[1] != I or not h.is_contiguous():
+        raise AtsError("grouped_down: h must be a contiguous [rows, I] tensor")
+    E = w_d_ptrs.numel()
+    if out is None:
+        out = torch.empty(h.shape[0], H, dtype=out_dtype or h.dtype, device=h.device)
+    check(_lib.load().ats_grouped_down(h.data_ptr(), w_d_ptrs.data_ptr(), out.data_ptr(), row_start.data_ptr(),
+                                       row_count.data_ptr(), E, int(max_rows), H, I, _tag(h), _tag(out), _stream()),
+          "ats_grouped_down")
+    return out
+
+
+# --------------------------------------------------------------------------- combine
+def combine(y: torch.Tensor, row_of: torch.Tensor, weights: torch.Tensor, num_tokens: int, k: int,
+            out_dtype: Optional[torch.dtype] = None, residual: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """y [rows, H]; row_of int32 [T*k]; weights f32 [T,k] -> out [T,H]."""
+    _need_gpu(y, row_of, weights, residual)
+    if row_of.dtype != torch.int32 or weights.dtype != torch.float32:
+        raise AtsError("combine: row_of must be int32 and weights float32")
+    if row_of.numel() != num_tokens * k or weights.numel() != num_tokens * k:
+        raise AtsError("combine: row_of/weights must have tokens*k entries")
+    y2 = y.reshape(-1, y.shape[-1]).contiguous()
+    H = y2.shape[1]
+    out = torch.empty(num_tokens, H, dtype=out_dtype or y.dtype, device=y.device)
+    if residual is not None:
+        residual = residual.reshape(num_tokens, H).contiguous()
+        if residual.dtype != out.dtype:
+            raise AtsError("combine: residual must have the output dtype")
+    check(_lib.load().ats_combine(y2.data_ptr(), row_of.contiguous().data_ptr(), weights.contiguous().data_ptr(),
+                                  _ptr(residual), out.data_ptr(), num_tokens, int(k), H, _tag(y2), _tag(out),
+                                  _stream()), "ats_combine")
+    return out
+
+
+# --------------------------------------------------------------------------- MoD helpers
+def row_dot(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, temperature: float = 1.0,
+            want_prob: bool = False):
+    """score[t] = x[t,:] . w (+ bias); optionally sigmoid(score / temperature)."""
+    _need_gpu(x, w, bias)
+    x2 = x.reshape(-1, x.shape[-1]).contiguous()
+    T, H = x2.shape
+    w = w.reshape(-1).contiguous()
+    if w.numel() != H or w.dtype != x2.dtype:
+        raise AtsError("row_dot: weight must have H elements of x's dtype")
+    if bias is not None:
+        bias = bias.reshape(-1).to(torch.float32).contiguous()
+    score = torch.empty(T, dtype=torch.float32, device=x.device)
+    prob = torch.empty(T, dtype=torch.float32, device=x.device) if want_prob else None
+    check(_lib.load().ats_row_dot(x2.data_ptr(), w.data_ptr(), _ptr(bias), score.data_ptr(), _ptr(prob),
+                                  float(temperature), T, H, _tag(x2), _stream()), "ats_row_dot")
+    return (score, prob) if want_prob else score
+
+
+def select_topk_per_sequence(scores: torch.Tensor, keep: int) -> torch.Tensor:
+    """scores f32 [B,L] -> flat token ids (b*L+pos) of the `keep` best per sequence, ascending, int32 [B*keep]."""
+    _need_gpu(scores)
+    if scores.dim() != 2 or scores.dtype != torch.float32:
+        raise AtsError("select_topk_per_sequence: scores must be float32 [batch, seq]")
+    scores = scores.contiguous()
+    B, L = scores.shape
+    sel = torch.empty(B * keep, dtype=torch.int32, device=scores.device)
+    check(_lib.load().ats_select_topk_per_sequence(scores.data_ptr(), B, L, int(keep), sel.data_ptr(), _stream()),
+          "ats_select_topk_per_sequence")
+    return sel
+
+
+def scatter_add_rows(base: torch.Tensor, rows: torch.Tensor, delta: torch.Tensor) -> torch.Tensor:
+    """base[rows[i]] += delta[i] in place (rows distinct); returns base."""
+    _need_gpu(base, rows, delta)
+    if not base.is_contiguous() or base.dim() != 2 or rows.dtype != torch.int32 or delta.dtype != base.dtype:
+        raise AtsError("scatter_add_rows: base must be contiguous 2-D, rows int32, delta of base's dtype")
+    delta = delta.reshape(-1, base.shape[1]).contiguous()
+    check(_lib.load().ats_scatter_add_rows(base.data_ptr(), rows.contiguous().data_ptr(), delta.data_ptr(),
+                                           rows.numel(), base.shape[1], _tag(base), _stream()),
+          "ats_scatter_add_rows")
+    return base
+
+
+def kth_value_mask(values: torch.Tensor, kth: int) -> torch.Tensor:
+    """float32 mask of values >= the kth smallest value (1-based), same shape as `values`."""
+    _need_gpu(values)
+    if values.dtype != torch.float32:
+        raise AtsError("kth_value_mask: values must be float32")
+    v = values.contiguous()
+    mask = torch.empty_like(v)
+    ws = torch.empty(16, dtype=torch.uint8, device=v.device)
+    check(_lib.load().ats_kth_value_mask(v.data_ptr(), v.numel(), int(kth), mask.data_ptr(), ws.data_ptr(), 16,
+                                         _stream()), "ats_kth_value_mask")
+    return mask
+
+
+def swiglu_mul(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
+    """gate * silu(up) (dense-FFN convention of the fused wrapper)."""
+    _need_gpu(gate, up)
+    if gate.shape != up.shape or gate.dtype != up.dtype:
+        raise AtsError("swiglu_mul: gate and up must match")
+    g, u = gate.contiguous(), up.contiguous()
+    out = torch.empty_like(g)
+    check(_lib.load().ats_swiglu_mul(g.data_ptr(), u.data_ptr(), out.data_ptr(), g.numel(), _tag(g), _stream()),
+          "ats_swiglu_mul")
+    return out

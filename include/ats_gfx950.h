@@ -1,0 +1,196 @@
+/* libats_gfx950 — C ABI of the MI355X (gfx950) sparse-layer kernels.
+ *
+ * Every entry point
+ *   - takes raw device pointers, sizes and a hipStream_t (passed as void*),
+ *   - enqueues work on that stream and returns without synchronising,
+ *   - never allocates, frees or retains memory (scratch comes in through a
+ *     workspace pointer whose size a *_workspace() call reports),
+ *   - returns ATS_OK or a negative error code and never terminates the
+ *     process; ats_last_error_string() describes the last failure of the
+ *     calling thread.
+ *
+ * This replaces, for the sparse-layer path, the two native interfaces of the
+ * reference (paths relative to the reference checkout):
+ *   - the extern "C" launchers of Src/Main_Scripts/core/transformer_ops.cu:331-436
+ *     (rms_norm_launcher, rope_precompute_launcher, rope_apply_launcher), which
+ *     return void and exit() on error (transformer_ops.cu:321-329);
+ *   - the pybind11 module `moe_cuda_ops` of Src/Main_Scripts/core/moe_cuda_ops.cu:436-442
+ *     (topk_gating, dispatch_tokens, combine_expert_outputs).
+ * Data types: ATS_F32 / ATS_BF16 element tags; all accumulation is float32.
+ */
+#ifndef ATS_GFX950_H
+#define ATS_GFX950_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define ATS_OK 0
+#define ATS_ERR_INVALID_ARG (-1)
+#define ATS_ERR_UNSUPPORTED (-2)
+#define ATS_ERR_LAUNCH (-3)
+#define ATS_ERR_WORKSPACE (-4)
+
+#define ATS_F32 0
+#define ATS_BF16 1
+
+#define ATS_ROUTE_SOFTMAX_TOPK 0 /* softmax over all experts, top-k, renormalise */
+#define ATS_ROUTE_TOPK_SOFTMAX 1 /* top-k of the logits, softmax over the k     */
+
+#define ATS_IDX_I32 0
+#define ATS_IDX_I64 1
+
+typedef void* ats_stream_t; /* hipStream_t */
+
+/* Library identification and error text (no reference counterpart: the
+ * reference prints to stderr and exits, transformer_ops.cu:321-329). */
+int ats_version(void);
+const char* ats_last_error_string(void);
+
+/* ---- RMSNorm ------------------------------------------------------------
+ * Replaces rms_norm_launcher (transformer_ops.cu:333-351); numerics follow
+ * RMSNorm.forward of Src/Main_Scripts/core/model.py:263-299:
+ *   y = ((float)x * rsqrt(mean(x^2) + eps) * (float)w) cast to x's type.
+ * x, y: [rows, hidden] of x_dtype; w: [hidden] of w_dtype or NULL. */
+int ats_rmsnorm_fwd(const void* x, const void* w, void* y, int64_t rows, int hidden, float eps,
+                    int x_dtype, int w_dtype, ats_stream_t stream);
+
+/* ---- RoPE ---------------------------------------------------------------
+ * ats_rope_table replaces rope_precompute_launcher (transformer_ops.cu:353-370)
+ * with the float64 evaluation of RotaryEmbedding._build_pytorch_cache
+ * (model.py:378-402): angle = (float)pos / scaling * theta^(-2d/dim), cos/sin in
+ * float64, stored as float32.  cols == dim writes both (duplicated) halves,
+ * cols == dim/2 writes the half table of FusedRoPE (cuda_opt_wrapper.py:350-363). */
+int ats_rope_table(float* cos_out, float* sin_out, int seq_len, int dim, int cols, double theta,
+                   double scaling_factor, ats_stream_t stream);
+
+/* ats_rope_fwd replaces rope_apply_launcher (transformer_ops.cu:372-392) and
+ * follows apply_rotary_pos_emb_optimized (model.py:470-524): rotate-half with
+ * separately rounded products and sum, float32 math, one rounding to the
+ * element type.  q: [B,Hq,L,D], k: [B,Hkv,L,D] (Hq != Hkv allowed), inputs
+ * addressed through element strides (batch, head, position; D contiguous),
+ * outputs contiguous; in-place (out == in, contiguous) is allowed.  cos/sin:
+ * float32 [table_len, >= D/2 used] with row stride table_stride; position of
+ * row l is pos_offset + l and must be < table_len.  k_in may be NULL (Hkv = 0). */
+int ats_rope_fwd(const void* q_in, const void* k_in, void* q_out, void* k_out, const float* cos_tab,
+                 const float* sin_tab, int table_stride, int table_len, int B, int Hq, int Hkv, int L,
+                 int D, int pos_offset, int64_t q_sb, int64_t q_sh, int64_t q_sl, int64_t k_sb,
+                 int64_t k_sh, int64_t k_sl, int dtype, ats_stream_t stream);
+
+/* ---- Router -------------------------------------------------------------
+ * logits[T,E] (float32) = x[T,H] . wg[E,H]^T (+ bias[E] if not NULL): the
+ * nn.Linear(H, E, bias=False) gate of model.py:1124,1169. */
+int ats_router_logits(const void* x, const void* wg, const float* bias, float* logits, int64_t T,
+                      int H, int E, int dtype, ats_stream_t stream);
+
+/* Routing.  Replaces moe_cuda_ops.topk_gating (moe_cuda_ops.cu:316-348) with the
+ * semantics of the PyTorch paths: variant ATS_ROUTE_SOFTMAX_TOPK = model.py:1200-1217,
+ * ATS_ROUTE_TOPK_SOFTMAX = moe_cuda_wrapper.py:229-233.  Selection is by
+ * descending logit/temperature, lower expert id first among equal values.
+ * Also produces what the auxiliary loss needs (model.py:1244-1263): hist[E]
+ * (pre-capacity assignment counts), prob_colsum[E] (sum over tokens of
+ * softmax(un-tempered logits)) and aux[1] = min(sum_e hist/(T*k) * colsum/T * E * lbw, 1).
+ * idx_out: [T,k] int32; w_out: [T,k] float32.  hist/prob_colsum/aux may be NULL together. */
+size_t ats_route_topk_workspace(int64_t T, int E);
+int ats_route_topk(const float* logits, int64_t T, int E, int k, float temperature, int variant,
+                   int32_t* idx_out, float* w_out, int32_t* hist, float* prob_colsum, float* aux,
+                   float load_balancing_weight, void* workspace, size_t workspace_bytes,
+                   ats_stream_t stream);
+
+/* ---- Capacity dispatch ---------------------------------------------------
+ * Deterministic restatement of the first-come-first-served loop of
+ * MoECUDAOps._pytorch_dispatch (moe_cuda_wrapper.py:295-326), replacing
+ * moe_cuda_ops.dispatch_tokens (moe_cuda_ops.cu:350-387, atomic order).
+ * idx: [T,k] expert ids (int32 or int64).  Outputs (all int32, any may not be NULL):
+ *   slot[T*k]       slot inside the expert, -1 when dropped
+ *   token_map[E*C]  assignment id t*k+j per slot, -1 when empty
+ *   hist[E], kept[E] = min(hist, C), offsets[E+1] = exclusive prefix of kept
+ *   row_src[max(1,min(T*k, E*C))]  compact row (offsets[e]+slot) -> assignment id
+ *   row_of[T*k]     assignment id -> compact row, -1 when dropped
+ * status[1]: 0, or 1 when an expert id was outside [0,E). */
+size_t ats_dispatch_plan_workspace(int64_t T, int k, int E);
+int ats_dispatch_plan(const void* idx, int idx_dtype, int64_t T, int k, int E, int C, int32_t* slot,
+                      int32_t* token_map, int32_t* hist, int32_t* kept, int32_t* offsets,
+                      int32_t* row_src, int32_t* row_of, int32_t* status, void* workspace,
+                      size_t workspace_bytes, ats_stream_t stream);
+
+/* out[r,:] = src[map[r] / div, :] or zeros when map[r] < 0; r in [0, n_rows).
+ * With map = token_map and div = k this fills expert_inputs[E,C,H]
+ * (moe_cuda_wrapper.py:306-322); with div = 1 it is a plain row gather. */
+int ats_gather_rows(const void* src, const int32_t* map, int div, void* out, int64_t n_rows, int H,
+                    int dtype, ats_stream_t stream);
+
+/* row_of[m] = r for every r in [0, n_slots) with m = token_map[r] >= 0; entries
+ * of row_of not named by token_map are set to -1.  Lets the combine step work
+ * from a bare token_map (moe_cuda_wrapper.py:343-357). */
+int ats_invert_token_map(const int32_t* token_map, int64_t n_slots, int32_t* row_of,
+                         int64_t n_assign, ats_stream_t stream);
+
+/* ---- Expert FFN (grouped GEMMs) -------------------------------------------
+ * SwiGLUExpert.forward (model.py:1071-1088) for all experts in one launch each.
+ * Rows of expert e are row_start[e] .. row_start[e]+row_count[e]-1 of the row
+ * space (compact: row_start = offsets; padded [E,C,*]: row_start = e*C).
+ * gate/up: h[r, i] = silu(a_r . w_gu[e][i,:]) * (a_r . w_gu[e][I+i,:]), where a_r
+ * is row r of `a`, or row a_rows[r]/a_row_div of `a` when a_rows != NULL (the
+ * permutation gather fused into the operand load).  w_gu / w_d are device
+ * arrays of E pointers to [2I,H] / [H,I] matrices.  h: [rows, I] of dtype;
+ * down: y[r,:] = h[r,:] . w_d[e]^T, y of y_dtype (ATS_F32 or dtype).
+ * max_rows bounds sum(row_count) (grid sizing only). */
+int ats_grouped_gateup_swiglu(const void* a, const int32_t* a_rows, int a_row_div,
+                              const void* const* w_gu, void* h, const int32_t* row_start,
+                              const int32_t* row_count, int E, int64_t max_rows, int H, int I,
+                              int dtype, ats_stream_t stream);
+int ats_grouped_down(const void* h, const void* const* w_d, void* y, const int32_t* row_start,
+                     const int32_t* row_count, int E, int64_t max_rows, int H, int I, int dtype,
+                     int y_dtype, ats_stream_t stream);
+
+/* ---- Combine --------------------------------------------------------------
+ * Token-major restatement of MoECUDAOps._pytorch_combine (moe_cuda_wrapper.py:328-359),
+ * replacing moe_cuda_ops.combine_expert_outputs (moe_cuda_ops.cu:389-423, atomic adds):
+ * out[t,:] = sum over the kept choices j of token t, in ascending row (= ascending
+ * expert id) order, of w[t,j] * y[row_of[t*k+j], :]; float32 products and sums
+ * rounded separately; zeros for a token with no kept choice.
+ * If residual != NULL, out[t,:] = residual[t,:] + that sum. */
+int ats_combine(const void* y, const int32_t* row_of, const float* w, const void* residual,
+                void* out, int64_t T, int k, int H, int y_dtype, int out_dtype, ats_stream_t stream);
+
+/* ---- Mixture-of-Depths helpers -------------------------------------------
+ * score[t] = x[t,:] . w[:] (+ bias[0]); optionally prob[t] = sigmoid(score/temperature)
+ * (MoDRouter.forward, model.py:926-936). */
+int ats_row_dot(const void* x, const void* w, const float* bias, float* score, float* prob,
+                float temperature, int64_t T, int H, int dtype, ats_stream_t stream);
+/* Per sequence, positions of the `keep` largest scores (lower position first
+ * among equals), written in ascending order as flat token ids b*L+pos:
+ * sel[B*keep] int32.  L <= 8192. */
+int ats_select_topk_per_sequence(const float* score, int B, int L, int keep, int32_t* sel,
+                                 ats_stream_t stream);
+/* base[rows[i], :] += delta[i, :] for i in [0, n) (rows distinct). */
+int ats_scatter_add_rows(void* base, const int32_t* rows, const void* delta, int64_t n, int H,
+                         int dtype, ats_stream_t stream);
+
+/* mask[i] = 1.0f if v[i] >= (kth smallest of v, 1-based) else 0.0f: the inference
+ * branch of MoDRouter.forward (model.py:984-990, kthvalue threshold).
+ * workspace: at least 4 bytes of device memory. */
+int ats_kth_value_mask(const float* v, int64_t n, int64_t kth, float* mask, void* workspace,
+                       size_t workspace_bytes, ats_stream_t stream);
+
+/* out = gate * silu(up), elementwise over n values: replaces swiglu_launcher
+ * (transformer_ops.cu:394-409), the activation of the dense FusedSwiGLU wrapper
+ * (cuda_opt_wrapper.py:476-478; note the convention differs from the experts'). */
+int ats_swiglu_mul(const void* gate, const void* up, void* out, int64_t n, int dtype, ats_stream_t stream);
+
+/* ---- Host-side views of the grouped-GEMM tile schedule (no device work) ----
+ * No reference counterpart; used to test the block -> (expert, m-tile, n-tile)
+ * map on the CPU.  row_count_host is a host array.  decode returns 1 and fills
+ * out3 = {expert, m_tile, n_tile} when the block owns a tile, else 0. */
+int ats_debug_decode_tile(int64_t block, const int32_t* row_count_host, int E, int BM, int n_tiles,
+                          int SM, int SN, int32_t* out3);
+int64_t ats_debug_grid_blocks(int64_t max_rows, int E, int BM, int n_tiles, int SM, int SN);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ATS_GFX950_H */

@@ -1,0 +1,127 @@
+"""CPU-side checks: the C-ABI library loads and exports every declared symbol, the tile
+schedule covers every tile exactly once, host-side integer logic, error behaviour without a GPU."""
+import ctypes
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "ats_gfx950.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(ats_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from adaptivetrainingsystem_amd import _lib
+    assert _lib.is_built(), "build the library first: python -m adaptivetrainingsystem_amd.build"
+    lib = _lib.load()
+    names = _declared_symbols()
+    assert len(names) >= 20
+    for n in names:
+        assert hasattr(lib, n), n
+        assert n in _lib._SIGNATURES, f"{n} has no ctypes signature"
+    assert lib.ats_version() >= 100
+    assert set(_lib._SIGNATURES) == set(names)
+
+
+def test_argument_errors_return_codes_not_exits():
+    from adaptivetrainingsystem_amd import _lib
+    lib = _lib.load()
+    # invalid arguments are rejected on the host before any device work
+    assert lib.ats_rmsnorm_fwd(None, None, None, 4, 0, 1e-6, 0, 0, None) == -1
+    assert b"hidden" in lib.ats_last_error_string()
+    assert lib.ats_rmsnorm_fwd(None, None, None, 4, 8, 1e-6, 7, 0, None) != 0
+    assert lib.ats_route_topk(None, 4, 8, 9, 1.0, 0, None, None, None, None, None, 0.01, None, 0, None) == -1
+    assert lib.ats_dispatch_plan(None, 0, 4, 2, 5000, 3, None, None, None, None, None, None, None, None, None, 0,
+                                 None) == -1
+    assert lib.ats_rope_fwd(None, None, None, None, None, None, 4, 4, 1, 1, 1, 4, 7, 0, 0, 0, 0, 0, 0, 0, 0,
+                            None) == -1       # odd head_dim
+    assert lib.ats_select_topk_per_sequence(None, 1, 10000, 5, None, None) == -1
+    assert lib.ats_route_topk_workspace(16384, 8) > 0
+    assert lib.ats_dispatch_plan_workspace(16384, 2, 8) == 32 * 8 * 4
+
+
+@pytest.mark.parametrize("counts,BM,n_tiles,SM,SN", [
+    ([5120, 4000, 300, 0, 1, 256, 257, 77], 256, 112, 4, 8),
+    ([20, 16, 0, 3], 32, 112, 1, 32),
+    ([130, 90, 576, 1], 128, 11, 4, 8),
+    ([0, 0, 0], 128, 5, 4, 8),
+    ([1000] * 64, 128, 11, 4, 8),
+])
+def test_tile_schedule_covers_each_tile_once(counts, BM, n_tiles, SM, SN):
+    from adaptivetrainingsystem_amd import _lib
+    lib = _lib.load()
+    rc = np.asarray(counts, dtype=np.int32)
+    E = len(counts)
+    blocks = lib.ats_debug_grid_blocks(int(rc.sum()), E, BM, n_tiles, SM, SN)
+    assert blocks % 256 == 0
+    seen = {}
+    out = np.zeros(3, dtype=np.int32)
+    for b in range(blocks):
+        if lib.ats_debug_decode_tile(b, rc.ctypes.data, E, BM, n_tiles, SM, SN, out.ctypes.data):
+            key = tuple(out.tolist())
+            assert key not in seen, f"tile {key} given to blocks {seen[key]} and {b}"
+            seen[key] = b
+    expect = {(e, mt, nt) for e in range(E) for mt in range(-(-counts[e] // BM)) for nt in range(n_tiles)}
+    assert set(seen) == expect
+    # blocks of one supertile land on one XCD (ids congruent mod 8) and cover SM x SN neighbours
+    if expect:
+        by_xcd = {}
+        for key, b in seen.items():
+            by_xcd.setdefault((b % 8, (b // 8) // 32), []).append(key)
+        for keys in by_xcd.values():
+            assert len({k[0] for k in keys}) == 1
+            assert len({k[1] // SM for k in keys}) == 1 and len({k[2] // SN for k in keys}) == 1
+
+
+def test_capacity_is_python_double_arithmetic():
+    from adaptivetrainingsystem_amd import ops
+    assert ops.expert_capacity(512, 2, 8, 1.25) == 160
+    assert ops.expert_capacity(64, 2, 8, 1.25) == 20
+    assert ops.expert_capacity(16384, 2, 8, 1.25) == 5120
+    assert ops.expert_capacity(4096, 6, 64, 1.5) == 576
+    assert ops.expert_capacity(512, 2, 8, 1.1) == 140
+
+
+def test_no_cpu_fallback_and_module_surface():
+    import adaptivetrainingsystem_amd as A
+    from adaptivetrainingsystem_amd.workloads import LayerConfig
+    with pytest.raises(A.AtsError):
+        A.RMSNorm(16)(torch.randn(2, 16))
+    with pytest.raises(A.AtsError):
+        A.apply_rotary_pos_emb(torch.randn(1, 1, 4, 8), torch.randn(1, 1, 4, 8), torch.ones(4, 8), torch.zeros(4, 8))
+    layer = A.MoEFFNLayer(LayerConfig(32, 64, 4, 2))
+    with pytest.raises(A.AtsError):
+        layer(torch.randn(1, 3, 32))
+    # parameter names and shapes that checkpoints of the reference model carry
+    sd = layer.state_dict()
+    assert sd["gate.weight"].shape == (4, 32)
+    assert sd["experts.0.gate_up_proj.weight"].shape == (128, 32)
+    assert sd["experts.3.down_proj.weight"].shape == (32, 64)
+    assert set(sd) == {"gate.weight"} | {f"experts.{i}.{n}.weight" for i in range(4)
+                                         for n in ("gate_up_proj", "down_proj")}
+    for attr in ("num_experts", "top_k", "capacity_factor", "routing_temperature", "noise_std",
+                 "load_balancing_weight", "use_cuda_ops", "get_routing_stats", "reset_routing_stats"):
+        assert hasattr(layer, attr)
+    assert layer.get_routing_stats() == {"error": "No routing statistics available"}
+    assert A.RMSNorm(8).state_dict()["weight"].shape == (8,)
+    assert list(A.RotaryEmbedding(8).state_dict()) == []           # buffers are non-persistent
+    assert A.MoECUDAOps.should_use_cuda(1, 1, 1, True, False) is False
+
+
+def test_workloads_are_reproducible():
+    from adaptivetrainingsystem_amd import workloads as W
+    a = W.make_moe_workload("c1_cpu_reference", device="cpu")
+    b = W.make_moe_workload("c1_cpu_reference", device="cpu")
+    assert torch.equal(a.x, b.x) and torch.equal(a.down[7], b.down[7])
+    assert a.x.shape == (2, 256, 512) and a.gate_up[0].shape == (2816, 512) and a.gate.shape == (8, 512)
+    c = W.make_moe_workload("c4_prefill", device="cpu", scale_tokens=16, overrides={"hidden": 64, "intermediate": 64})
+    assert torch.allclose(c.logit_bias, 1.5 * torch.log(1.0 / torch.arange(1, 9).float()))
+    n = W.make_norm_rope_workload(device="cpu", batch=1, seq=8)
+    assert n.q.shape == (1, 16, 8, 128) and n.k.shape == (1, 4, 8, 128) and n.norm_weight.dtype == torch.float32
