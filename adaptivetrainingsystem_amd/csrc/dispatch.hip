@@ -15,6 +15,10 @@
 
 #include "ats_common.hpp"
 
+// Products and sums below must round separately (the reference computes them as separate
+// tensor ops); the HIP default would contract a*b+c into one fused multiply-add.
+#pragma clang fp contract(off)
+
 namespace ats {
 
 constexpr int kPlanChunk = 1024;     // assignments per block
@@ -282,11 +286,11 @@ __global__ __launch_bounds__(256) void combine_kernel(const TY* __restrict__ y, 
                 const int64_t row = __shfl(my_row, src, 64);
                 const float wt = __shfl(my_w, src, 64);
                 const TY* yr = y + row * H + h0;
-                for (int j = 0; j < nh; ++j) acc[j] = __fadd_rn(acc[j], __fmul_rn(wt, Elem<TY>::load(yr + j)));
+                for (int j = 0; j < nh; ++j) acc[j] = ((acc[j]) + (((wt) * (Elem<TY>::load(yr + j)))));
             }
             for (int j = 0; j < nh; ++j) {
                 float v = acc[j];
-                if (residual) v = __fadd_rn(Elem<TO>::load(residual + t * H + h0 + j), v);
+                if (residual) v = ((Elem<TO>::load(residual + t * H + h0 + j)) + (v));
                 Elem<TO>::store(out + t * H + h0 + j, v);
             }
         }
@@ -346,7 +350,7 @@ __global__ __launch_bounds__(256) void combine_vec_kernel(const TY* __restrict__
             for (int n = 0; n < MAXK; ++n) {
                 if (n < n_kept) {
 #pragma unroll
-                    for (int j = 0; j < V; ++j) acc[j] = __fadd_rn(acc[j], __fmul_rn(wts[n], yv[n][j]));
+                    for (int j = 0; j < V; ++j) acc[j] = ((acc[j]) + (((wts[n]) * (yv[n][j]))));
                 }
             }
             if (residual) {
@@ -359,7 +363,7 @@ __global__ __launch_bounds__(256) void combine_vec_kernel(const TY* __restrict__
                     Elem<TO>::unpack(*reinterpret_cast<const uint4*>(rr + 4), rv + 4);
                 }
 #pragma unroll
-                for (int j = 0; j < V; ++j) acc[j] = __fadd_rn(rv[j], acc[j]);
+                for (int j = 0; j < V; ++j) acc[j] = ((rv[j]) + (acc[j]));
             }
             TO* o = out + t * H + h0;
             if constexpr (sizeof(TO) == 2) {
@@ -415,8 +419,9 @@ extern "C" int ats_dispatch_plan(const void* idx, int idx_dtype, int64_t T, int 
                 "ats_dispatch_plan: idx dtype tag %d", idx_dtype);
     ATS_REQUIRE(T * (int64_t)k < (int64_t)INT_MAX && (int64_t)E * C < (int64_t)INT_MAX, ATS_ERR_UNSUPPORTED,
                 "ats_dispatch_plan: T*k and E*C must fit in int32");
-    ATS_REQUIRE(slot && token_map && hist && kept && offsets && row_src && row_of && status, ATS_ERR_INVALID_ARG,
-                "ats_dispatch_plan: null output pointer");
+    ATS_REQUIRE((token_map || (int64_t)E * C == 0) && (T == 0 || (slot && row_of)) && hist && kept && offsets &&
+                    row_src && status,
+                ATS_ERR_INVALID_ARG, "ats_dispatch_plan: null output pointer");
     ATS_REQUIRE(T == 0 || idx, ATS_ERR_INVALID_ARG, "ats_dispatch_plan: null idx");
     const int64_t n = T * k;
     const int64_t nchunks = n == 0 ? 1 : (n + kPlanChunk - 1) / kPlanChunk;

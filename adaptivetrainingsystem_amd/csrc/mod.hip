@@ -6,6 +6,9 @@
 
 #include "ats_common.hpp"
 
+// Sums below must not be contracted with a preceding product into a fused multiply-add.
+#pragma clang fp contract(off)
+
 namespace ats {
 
 // One wave per token row; 16-byte loads; weight vector re-read from L2.
@@ -123,12 +126,12 @@ __global__ __launch_bounds__(256) void scatter_add_rows_kernel(T* __restrict__ b
                 Elem<T>::unpack(bp[v], a);
                 Elem<T>::unpack(dp[v], d);
 #pragma unroll
-                for (int j = 0; j < V; ++j) a[j] = __fadd_rn(a[j], d[j]);
+                for (int j = 0; j < V; ++j) a[j] = ((a[j]) + (d[j]));
                 bp[v] = Elem<T>::pack(a);
             }
         } else {
             for (int h = lane; h < H; h += kWave)
-                Elem<T>::store(base + r * H + h, __fadd_rn(Elem<T>::load(base + r * H + h), Elem<T>::load(delta + i * H + h)));
+                Elem<T>::store(base + r * H + h, ((Elem<T>::load(base + r * H + h)) + (Elem<T>::load(delta + i * H + h))));
         }
     }
 }

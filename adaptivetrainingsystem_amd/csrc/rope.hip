@@ -8,6 +8,10 @@
 
 #include "ats_common.hpp"
 
+// Products and sums below must round separately (the reference computes them as separate
+// tensor ops); the HIP default would contract a*b+c into one fused multiply-add.
+#pragma clang fp contract(off)
+
 namespace ats {
 
 constexpr int kRopeHeadsPerItem = 4;
@@ -75,8 +79,8 @@ __global__ __launch_bounds__(256) void rope_vec_kernel(RopeSeg q, RopeSeg k, con
             Elem<T>::unpack(hi[i], bb);
 #pragma unroll
             for (int j = 0; j < V; ++j) {
-                o1[j] = __fsub_rn(__fmul_rn(a[j], cs[j]), __fmul_rn(bb[j], sn[j]));
-                o2[j] = __fadd_rn(__fmul_rn(a[j], sn[j]), __fmul_rn(bb[j], cs[j]));
+                o1[j] = ((((a[j]) * (cs[j]))) - (((bb[j]) * (sn[j]))));
+                o2[j] = ((((a[j]) * (sn[j]))) + (((bb[j]) * (cs[j]))));
             }
             T* p = out + (((int64_t)b * seg.heads + h) * L + pos) * D + c * V;
             *reinterpret_cast<uint4*>(p) = Elem<T>::pack(o1);
@@ -108,8 +112,8 @@ __global__ __launch_bounds__(256) void rope_scalar_kernel(RopeSeg q, RopeSeg k, 
         const float cs = cos_tab[(int64_t)(pos_offset + pos) * table_stride + d];
         const float sn = sin_tab[(int64_t)(pos_offset + pos) * table_stride + d];
         T* o = static_cast<T*>(seg.out) + (((int64_t)b * seg.heads + h) * L + pos) * D + d;
-        Elem<T>::store(o, __fsub_rn(__fmul_rn(a, cs), __fmul_rn(bb, sn)));
-        Elem<T>::store(o + half, __fadd_rn(__fmul_rn(a, sn), __fmul_rn(bb, cs)));
+        Elem<T>::store(o, ((((a) * (cs))) - (((bb) * (sn)))));
+        Elem<T>::store(o + half, ((((a) * (sn))) + (((bb) * (cs)))));
     }
 }
 

@@ -32,6 +32,7 @@ import torch
 import torch.nn as nn
 
 from . import ops
+from .profiling import stage
 from ._lib import ROUTE_SOFTMAX_TOPK, ROUTE_TOPK_SOFTMAX, AtsError
 
 
@@ -217,6 +218,7 @@ class MoEFFNLayer(nn.Module):
         self._wcache_key = None
         self._wcache = None
         self.last_plan = None
+        self.stage_timer = None            # set to a profiling.StageTimer to time each stage with HIP events
         nn.init.normal_(self.gate.weight, mean=0.0, std=0.01)
 
     # ---- expert weight tables (device arrays of pointers; rebuilt when a weight moves or changes dtype)
@@ -244,11 +246,14 @@ class MoEFFNLayer(nn.Module):
         E, k = self.num_experts, self.top_k
         I = self.experts[0].down_proj.in_features
 
-        logits = ops.router_logits(x_flat, _as_dtype(self.gate.weight, x.dtype), self.router_logit_bias)
+        tm = self.stage_timer
+        with stage(tm, "router_logits"):
+            logits = ops.router_logits(x_flat, _as_dtype(self.gate.weight, x.dtype), self.router_logit_bias)
         if self.training and self.noise_std > 0:
             logits = logits + torch.randn_like(logits) * self.noise_std
         variant = {"softmax_topk": ROUTE_SOFTMAX_TOPK, "topk_softmax": ROUTE_TOPK_SOFTMAX}[self.routing]
-        route = ops.route_topk(logits, k, self.routing_temperature, variant, self.load_balancing_weight)
+        with stage(tm, "route_topk"):
+            route = ops.route_topk(logits, k, self.routing_temperature, variant, self.load_balancing_weight)
 
         if self.capacity_mode == "fcfs":
             C = ops.expert_capacity(T, k, E, self.capacity_factor)
@@ -256,16 +261,20 @@ class MoEFFNLayer(nn.Module):
             C = T
         else:
             raise AtsError(f"MoEFFNLayer: capacity_mode {self.capacity_mode!r}")
-        plan = ops.dispatch_plan(route["indices"], E, C)
+        with stage(tm, "dispatch_plan"):
+            plan = ops.dispatch_plan(route["indices"], E, C)
         rows = min(T * k, E * C)
         wgu_ptrs, wd_ptrs, _, _ = self._weight_tables(x.dtype, x.device)
         if rows > 0:
-            h = ops.grouped_gateup_swiglu(x_flat, wgu_ptrs, plan["offsets"], plan["kept"], rows, rows, H, I,
-                                          a_rows=plan["row_src"], a_row_div=k)
-            y = ops.grouped_down(h, wd_ptrs, plan["offsets"], plan["kept"], rows, H, I)
+            with stage(tm, "gateup_swiglu"):
+                h = ops.grouped_gateup_swiglu(x_flat, wgu_ptrs, plan["offsets"], plan["kept"], rows, rows, H, I,
+                                              a_rows=plan["row_src"], a_row_div=k)
+            with stage(tm, "down"):
+                y = ops.grouped_down(h, wd_ptrs, plan["offsets"], plan["kept"], rows, H, I)
         else:
             y = torch.zeros(1, H, dtype=x.dtype, device=x.device)
-        out = ops.combine(y, plan["row_of"], route["weights"], T, k, out_dtype=x.dtype)
+        with stage(tm, "combine"):
+            out = ops.combine(y, plan["row_of"], route["weights"], T, k, out_dtype=x.dtype)
 
         self.last_plan = {"logits": logits, "capacity": C, **route, **plan}
         if self.training:
