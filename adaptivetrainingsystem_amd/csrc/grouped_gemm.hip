@@ -26,6 +26,8 @@ namespace ats {
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
+// Native 16-byte vector (plain IR loads/stores, so staging arrays stay in registers).
+typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
 
 struct GroupedArgs {
     const void* a;           // [*, K] activations
@@ -38,17 +40,18 @@ struct GroupedArgs {
     const int32_t* row_start;
     const int32_t* row_count;
     int E, K, N_out, up_offset, n_tiles;
+    int force_general;  // testing aid: always take the general (k-tail capable) kernel
 };
 
 constexpr int kRowPitch = 144;  // bytes per staged row: 128 data + 16 pad
 
 template <typename T>
-__device__ __forceinline__ void mma_step(const uint4& wfrag, const uint4& afrag, f32x16_t& c);
+__device__ __forceinline__ void mma_step(const u32x4_t& wfrag, const u32x4_t& afrag, f32x16_t& c);
 
 template <>
-__device__ __forceinline__ void mma_step<bf16_t>(const uint4& wfrag, const uint4& afrag, f32x16_t& c) {
+__device__ __forceinline__ void mma_step<bf16_t>(const u32x4_t& wfrag, const u32x4_t& afrag, f32x16_t& c) {
     union {
-        uint4 u;
+        u32x4_t u;
         bf16x8_t v;
     } w, a;
     w.u = wfrag;
@@ -56,14 +59,19 @@ __device__ __forceinline__ void mma_step<bf16_t>(const uint4& wfrag, const uint4
     c = __builtin_amdgcn_mfma_f32_32x32x16_bf16(w.v, a.v, c, 0, 0, 0);
 }
 template <>
-__device__ __forceinline__ void mma_step<float>(const uint4& wfrag, const uint4& afrag, f32x16_t& c) {
+__device__ __forceinline__ void mma_step<float>(const u32x4_t& wfrag, const u32x4_t& afrag, f32x16_t& c) {
     c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(wfrag.x), __uint_as_float(afrag.x), c, 0, 0, 0);
     c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(wfrag.y), __uint_as_float(afrag.y), c, 0, 0, 0);
     c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(wfrag.z), __uint_as_float(afrag.z), c, 0, 0, 0);
     c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(wfrag.w), __uint_as_float(afrag.w), c, 0, 0, 0);
 }
 
-__device__ __forceinline__ float silu_f(float g) { return g / (1.0f + expf(-g)); }
+// silu(g) = g / (1 + exp(-g)) with the hardware exp2 and reciprocal (each about 1 ulp): the
+// result is within ~3e-7 relative of the correctly rounded value, far inside the float32 bar.
+__device__ __forceinline__ float silu_f(float g) {
+    const float e = __builtin_amdgcn_exp2f(g * -1.4426950408889634f);
+    return g * __builtin_amdgcn_rcpf(1.0f + e);
+}
 
 template <typename TO>
 __device__ __forceinline__ void store4(TO* p, const float* v, int n_valid);
@@ -160,8 +168,8 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_kernel(GroupedArgs p
             for (int v = 0; v < 16; ++v) acc[j][i][v] = 0.f;
 
     const int nk = (K + BK - 1) / BK;
-    const uint4 zero4 = make_uint4(0, 0, 0, 0);
-    uint4 ra[PA], rb[PB];
+    const u32x4_t zero4 = {0u, 0u, 0u, 0u};
+    u32x4_t ra[PA], rb[PB];
 
 #define ATS_LOAD_GLOBAL(kt_)                                                                       \
     {                                                                                              \
@@ -169,11 +177,11 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_kernel(GroupedArgs p
         const bool kok = koff + lchunk * VEC < K;                                                  \
         _Pragma("unroll") for (int i = 0; i < PA; ++i) {                                           \
             ra[i] = zero4;                                                                         \
-            if (ap[i] && kok) ra[i] = *reinterpret_cast<const uint4*>(ap[i] + koff);               \
+            if (ap[i] && kok) ra[i] = *reinterpret_cast<const u32x4_t*>(ap[i] + koff);               \
         }                                                                                          \
         _Pragma("unroll") for (int i = 0; i < PB; ++i) {                                           \
             rb[i] = zero4;                                                                         \
-            if (bp[i] && kok) rb[i] = *reinterpret_cast<const uint4*>(bp[i] + koff);               \
+            if (bp[i] && kok) rb[i] = *reinterpret_cast<const u32x4_t*>(bp[i] + koff);               \
         }                                                                                          \
     }
 #define ATS_STORE_LDS(stage_)                                                                      \
@@ -181,9 +189,9 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_kernel(GroupedArgs p
         unsigned char* sA_ = smem + (stage_) * STAGE;                                              \
         unsigned char* sB_ = sA_ + BM * kRowPitch;                                                 \
         _Pragma("unroll") for (int i = 0; i < PA; ++i)                                             \
-            *reinterpret_cast<uint4*>(sA_ + (lrow + i * RPP) * kRowPitch + lchunk * 16) = ra[i];   \
+            *reinterpret_cast<u32x4_t*>(sA_ + (lrow + i * RPP) * kRowPitch + lchunk * 16) = ra[i];   \
         _Pragma("unroll") for (int i = 0; i < PB; ++i)                                             \
-            *reinterpret_cast<uint4*>(sB_ + (lrow + i * RPP) * kRowPitch + lchunk * 16) = rb[i];   \
+            *reinterpret_cast<u32x4_t*>(sB_ + (lrow + i * RPP) * kRowPitch + lchunk * 16) = rb[i];   \
     }
 
     // fragment rows of this wave inside the staged tiles
@@ -214,11 +222,11 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_kernel(GroupedArgs p
         const unsigned char* sB = sA + BM * kRowPitch;
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks) {
-            uint4 fa[TM], fb[TN];
+            u32x4_t fa[TM], fb[TN];
 #pragma unroll
-            for (int i = 0; i < TM; ++i) fa[i] = *reinterpret_cast<const uint4*>(sA + a_row_off[i] + ks * 32);
+            for (int i = 0; i < TM; ++i) fa[i] = *reinterpret_cast<const u32x4_t*>(sA + a_row_off[i] + ks * 32);
 #pragma unroll
-            for (int j = 0; j < TN; ++j) fb[j] = *reinterpret_cast<const uint4*>(sB + b_row_off[j] + ks * 32);
+            for (int j = 0; j < TN; ++j) fb[j] = *reinterpret_cast<const u32x4_t*>(sB + b_row_off[j] + ks * 32);
 #pragma unroll
             for (int j = 0; j < TN; ++j)
 #pragma unroll
@@ -256,25 +264,306 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_kernel(GroupedArgs p
     }
 }
 
+
+// LDS-only barrier: waits for this wave's LDS traffic, not for global loads in flight.
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+// Software-pipelined variant for K % BK == 0.  All loader addresses are valid by
+// construction (rows past the end of the expert / of N are clamped; their results are never
+// stored), so the steady-state loop body is straight-line code:
+//   k-step 0: MFMAs(frag buf 0) while fragments of k-step 1 are read
+//   k-step 1: MFMAs(buf 1) | read k-step 2 | slab t+1: registers -> LDS (other stage)
+//   k-step 2: MFMAs(buf 0) | read k-step 3 | issue global loads of slab t+2
+//   LDS barrier
+//   k-step 3: MFMAs(buf 1) | read k-step 0 of slab t+1
+// Global loads therefore have a whole slab of MFMA time to land before they are needed.
+template <typename T, typename TO, int BM, int BN, int WM, int WN, int SM, int SN, bool SWIGLU>
+__global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_pipelined_kernel(GroupedArgs p) {
+    constexpr int NT = WM * WN * 64;
+    constexpr int VEC = 16 / (int)sizeof(T);
+    constexpr int BK = 128 / (int)sizeof(T);
+    constexpr int TM = BM / WM / 32;
+    constexpr int TN = BN / WN / 32;
+    constexpr int RPP = NT / 8;
+    constexpr int PA = BM / RPP;
+    constexpr int PB = BN / RPP;
+    constexpr int STAGE = (BM + BN) * kRowPitch;
+    constexpr int HALF = BN / 2;
+    static_assert(BM % (WM * 32) == 0 && BN % (WN * 32) == 0, "wave tiling");
+    static_assert(BM % RPP == 0 && BN % RPP == 0, "loader tiling");
+    static_assert(!SWIGLU || TN % 2 == 0, "SwiGLU needs gate and up tiles in the same wave");
+    static_assert(SM * SN == kSuperBlocks, "supertile");
+
+    extern __shared__ __align__(16) unsigned char smem[];
+
+    TileCoord tc;
+    if (!decode_tile(blockIdx.x, p.row_count, p.E, BM, p.n_tiles, SM, SN, &tc)) return;
+    const int count = p.row_count[tc.e];
+    const int row0 = p.row_start[tc.e];
+    const int K = p.K;
+    const T* Bexp = static_cast<const T*>(p.b[tc.e]);
+    const T* A = static_cast<const T*>(p.a);
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wm = wave / WN, wn = wave % WN;
+    const int lrow = tid >> 3;
+    const int lchunk = tid & 7;
+
+    const T* ap[PA];
+#pragma unroll
+    for (int i = 0; i < PA; ++i) {
+        int m = tc.mt * BM + lrow + i * RPP;
+        m = m < count ? m : count - 1;
+        int64_t src = row0 + m;
+        if (p.a_rows) src = p.a_rows[src] / p.a_row_div;
+        ap[i] = A + src * p.lda + lchunk * VEC;
+    }
+    const T* bp[PB];
+#pragma unroll
+    for (int i = 0; i < PB; ++i) {
+        const int rb = lrow + i * RPP;
+        int n, brow;
+        if (SWIGLU) {
+            const bool up = rb >= HALF;
+            n = tc.nt * HALF + (up ? rb - HALF : rb);
+            n = n < p.N_out ? n : p.N_out - 1;
+            brow = up ? p.up_offset + n : n;
+        } else {
+            n = tc.nt * BN + rb;
+            n = n < p.N_out ? n : p.N_out - 1;
+            brow = n;
+        }
+        bp[i] = Bexp + (int64_t)brow * K + lchunk * VEC;
+    }
+
+    // L2 warm-up: each thread touches one 128-byte line of a slab that the loaders will ask
+    // for kPfDist slabs later, so that the loaders' requests hit in L2.  The values are only
+    // folded into a dummy word (which keeps the loads ordered and alive).
+    constexpr int kPfDist = 3;
+    const T* apf;
+    const T* bpf;
+    {
+        int m = tc.mt * BM + tid % BM;
+        m = m < count ? m : count - 1;
+        int64_t src = row0 + m;
+        if (p.a_rows) src = p.a_rows[src] / p.a_row_div;
+        apf = A + src * p.lda;
+        const int rbp = tid % BN;
+        int n, brow;
+        if (SWIGLU) {
+            const bool up = rbp >= HALF;
+            n = tc.nt * HALF + (up ? rbp - HALF : rbp);
+            n = n < p.N_out ? n : p.N_out - 1;
+            brow = up ? p.up_offset + n : n;
+        } else {
+            n = tc.nt * BN + rbp;
+            n = n < p.N_out ? n : p.N_out - 1;
+            brow = n;
+        }
+        bpf = Bexp + (int64_t)brow * K;
+    }
+    unsigned pfa[2] = {0u, 0u}, pfb[2] = {0u, 0u}, junk = 0u;
+
+    f32x16_t acc[TN][TM];
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[j][i][v] = 0.f;
+
+    const int nk = K / BK;
+    u32x4_t ra[PA], rb[PB];
+    const int st_off = lrow * kRowPitch + lchunk * 16;
+
+    const int frow = lane & 31;
+    const int fgrp = lane >> 5;
+    int a_row_off[TM], b_row_off[TN];
+#pragma unroll
+    for (int i = 0; i < TM; ++i) a_row_off[i] = (wm * (BM / WM) + i * 32 + frow) * kRowPitch + fgrp * 16;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+        int r;
+        if (SWIGLU) {
+            constexpr int WH = BN / WN / 2;
+            r = j < TN / 2 ? wn * WH + j * 32 : HALF + wn * WH + (j - TN / 2) * 32;
+        } else {
+            r = wn * (BN / WN) + j * 32;
+        }
+        b_row_off[j] = BM * kRowPitch + (r + frow) * kRowPitch + fgrp * 16;
+    }
+    u32x4_t fa[2][TM], fb[2][TN];
+
+#define PL_LOADG(kt_)                                                                                  \
+    {                                                                                                  \
+        const int koff = (kt_) * BK;                                                                   \
+        _Pragma("unroll") for (int i = 0; i < PA; ++i) ra[i] = *reinterpret_cast<const u32x4_t*>(ap[i] + koff); \
+        _Pragma("unroll") for (int i = 0; i < PB; ++i) rb[i] = *reinterpret_cast<const u32x4_t*>(bp[i] + koff); \
+    }
+#define PL_STORE(stage_)                                                                               \
+    {                                                                                                  \
+        unsigned char* sA_ = smem + (stage_) * STAGE + st_off;                                         \
+        unsigned char* sB_ = sA_ + BM * kRowPitch;                                                     \
+        _Pragma("unroll") for (int i = 0; i < PA; ++i)                                                 \
+            *reinterpret_cast<u32x4_t*>(sA_ + i * RPP * kRowPitch) = ra[i];                              \
+        _Pragma("unroll") for (int i = 0; i < PB; ++i)                                                 \
+            *reinterpret_cast<u32x4_t*>(sB_ + i * RPP * kRowPitch) = rb[i];                              \
+    }
+#define PL_READ(stage_, ks_, buf_)                                                                     \
+    {                                                                                                  \
+        const unsigned char* s_ = smem + (stage_) * STAGE + (ks_) * 32;                                \
+        _Pragma("unroll") for (int i = 0; i < TM; ++i)                                                 \
+            fa[buf_][i] = *reinterpret_cast<const u32x4_t*>(s_ + a_row_off[i]);                          \
+        _Pragma("unroll") for (int j = 0; j < TN; ++j)                                                 \
+            fb[buf_][j] = *reinterpret_cast<const u32x4_t*>(s_ + b_row_off[j]);                          \
+    }
+#define PL_MMA(buf_)                                                                                   \
+    {                                                                                                  \
+        _Pragma("unroll") for (int j = 0; j < TN; ++j)                                                 \
+            _Pragma("unroll") for (int i = 0; i < TM; ++i) mma_step<T>(fb[buf_][j], fa[buf_][i], acc[j][i]); \
+    }
+// Instruction-order control: inside a phase the scheduler is asked to alternate matrix
+// instructions with the memory instructions of that phase (so the memory pipes work in the
+// shadow of the MFMAs); nothing moves across a phase boundary.
+#define SG_MFMA 0x008
+#define SG_VMEM_RD 0x020
+#define SG_DS_RD 0x100
+#define SG_DS_WR 0x200
+#define PL_FENCE() __builtin_amdgcn_sched_barrier(0)
+#define PL_MIX_READS()                                                                  \
+    _Pragma("unroll") for (int g_ = 0; g_ < (TM + TN); ++g_) {                          \
+        __builtin_amdgcn_sched_group_barrier(SG_MFMA, (TM * TN) / (TM + TN), 0);        \
+        __builtin_amdgcn_sched_group_barrier(SG_DS_RD, 1, 0);                           \
+    }
+#define PL_ITER(kt_, HAS1, HAS2, SLOT)                                                    \
+    {                                                                                   \
+        const int cur_ = (kt_) & 1;                                                     \
+        PL_READ(cur_, 1, 1);                                                            \
+        PL_MMA(0);                                                                      \
+        PL_MIX_READS();                                                                 \
+        PL_FENCE();                                                                     \
+        PL_READ(cur_, 2, 0);                                                            \
+        if (HAS1) PL_STORE(cur_ ^ 1);                                                   \
+        PL_MMA(1);                                                                      \
+        if (HAS1) {                                                                     \
+            _Pragma("unroll") for (int g_ = 0; g_ < (TM + TN); ++g_) {                  \
+                __builtin_amdgcn_sched_group_barrier(SG_MFMA, (TM * TN) / (TM + TN), 0); \
+                __builtin_amdgcn_sched_group_barrier(SG_DS_RD, 1, 0);                   \
+                __builtin_amdgcn_sched_group_barrier(SG_DS_WR, (PA + PB) / (TM + TN), 0); \
+            }                                                                           \
+        } else {                                                                        \
+            PL_MIX_READS();                                                             \
+        }                                                                               \
+        PL_FENCE();                                                                     \
+        PL_READ(cur_, 3, 1);                                                            \
+        if (HAS2) {                                                                     \
+            PL_LOADG((kt_) + 2);                                                        \
+            junk ^= pfa[SLOT] ^ pfb[SLOT];                                              \
+            const int kpf_ = min((kt_) + 2 + kPfDist, nk - 1) * BK;                     \
+            pfa[SLOT] = *reinterpret_cast<const unsigned*>(apf + kpf_);                 \
+            pfb[SLOT] = *reinterpret_cast<const unsigned*>(bpf + kpf_);                 \
+        }                                                                               \
+        PL_MMA(0);                                                                      \
+        if (HAS2) {                                                                     \
+            _Pragma("unroll") for (int g_ = 0; g_ < (TM + TN); ++g_) {                  \
+                __builtin_amdgcn_sched_group_barrier(SG_MFMA, (TM * TN) / (TM + TN), 0); \
+                __builtin_amdgcn_sched_group_barrier(SG_DS_RD, 1, 0);                   \
+                __builtin_amdgcn_sched_group_barrier(SG_VMEM_RD, (PA + PB) / (TM + TN), 0); \
+            }                                                                           \
+            __builtin_amdgcn_sched_group_barrier(SG_VMEM_RD, 2, 0);                     \
+        } else {                                                                        \
+            PL_MIX_READS();                                                             \
+        }                                                                               \
+        PL_FENCE();                                                                     \
+        lds_barrier();                                                                  \
+        PL_FENCE();                                                                     \
+        if (HAS1) PL_READ(cur_ ^ 1, 0, 0);                                              \
+        PL_MMA(1);                                                                      \
+        if (HAS1) PL_MIX_READS();                                                       \
+        PL_FENCE();                                                                     \
+    }
+
+    PL_LOADG(0);
+    PL_STORE(0);
+    if (nk > 1) PL_LOADG(1);
+    lds_barrier();
+    PL_READ(0, 0, 0);
+    int kt = 0;
+    for (; kt + 3 < nk; kt += 2) {
+        PL_ITER(kt, true, true, 0);
+        PL_ITER(kt + 1, true, true, 1);
+    }
+    if (kt + 2 < nk) {
+        PL_ITER(kt, true, true, 0);
+        ++kt;
+    }
+    if (kt + 1 < nk) {
+        PL_ITER(kt, true, false, 0);
+        ++kt;
+    }
+    PL_ITER(kt, false, false, 0);
+    junk ^= pfa[0] ^ pfb[0] ^ pfa[1] ^ pfb[1];
+#undef PL_LOADG
+#undef PL_STORE
+#undef PL_READ
+#undef PL_MMA
+#undef PL_ITER
+#undef PL_FENCE
+#undef PL_MIX_READS
+
+    TO* out = static_cast<TO*>(p.out);
+    if (p.E < 0) out[0] = TO{};   // never true; with the next line it keeps the warm-up loads alive
+    if (p.E < 0 && junk == 0x5a5a5a5au) out[1] = TO{};
+    constexpr int TNO = SWIGLU ? TN / 2 : TN;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+        const int m = tc.mt * BM + wm * (BM / WM) + i * 32 + frow;
+        if (m >= count) continue;
+        TO* orow = out + (int64_t)(row0 + m) * p.ldo;
+#pragma unroll
+        for (int j = 0; j < TNO; ++j) {
+            const int ncol0 = SWIGLU ? tc.nt * HALF + wn * (BN / WN / 2) + j * 32 : tc.nt * BN + wn * (BN / WN) + j * 32;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int n = ncol0 + 8 * q + 4 * fgrp;
+                float v[4];
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    if (SWIGLU) v[c] = silu_f(acc[j][i][q * 4 + c]) * acc[j + TN / 2][i][q * 4 + c];
+                    else v[c] = acc[j][i][q * 4 + c];
+                }
+                const int n_valid = p.N_out - n;
+                if (n_valid > 0) store4<TO>(orow + n, v, n_valid);
+            }
+        }
+    }
+}
+
 template <typename T, typename TO, int BM, int BN, int WM, int WN, int SM, int SN, bool SWIGLU>
 static int launch_cfg(const GroupedArgs& p0, int64_t max_rows, hipStream_t s) {
     GroupedArgs p = p0;
     constexpr int n_per_tile = SWIGLU ? BN / 2 : BN;
     p.n_tiles = (p.N_out + n_per_tile - 1) / n_per_tile;
     constexpr size_t smem = 2 * (size_t)(BM + BN) * kRowPitch;
-    auto kern = grouped_gemm_kernel<T, TO, BM, BN, WM, WN, SM, SN, SWIGLU>;
+    constexpr int BK = 128 / (int)sizeof(T);
+    auto kern_general = grouped_gemm_kernel<T, TO, BM, BN, WM, WN, SM, SN, SWIGLU>;
+    auto kern_pipe = grouped_gemm_pipelined_kernel<T, TO, BM, BN, WM, WN, SM, SN, SWIGLU>;
     static bool attr_done = false;
     if (!attr_done) {
         if (smem > 64 * 1024) {
-            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-            if (e != hipSuccess) {
-                set_error("grouped GEMM: cannot reserve %zu bytes of LDS: %s", smem, hipGetErrorString(e));
-                return ATS_ERR_LAUNCH;
+            for (const void* k : {reinterpret_cast<const void*>(kern_general), reinterpret_cast<const void*>(kern_pipe)}) {
+                hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+                if (e != hipSuccess) {
+                    set_error("grouped GEMM: cannot reserve %zu bytes of LDS: %s", smem, hipGetErrorString(e));
+                    return ATS_ERR_LAUNCH;
+                }
             }
         }
         attr_done = true;
     }
+    auto kern = (p.K % BK == 0 && !(p.force_general & 1)) ? kern_pipe : kern_general;
     const int64_t blocks = grid_blocks(max_rows, p.E, BM, p.n_tiles, SM, SN);
     if (blocks > 0x7fffffffLL) {
         set_error("grouped GEMM: grid of %lld blocks", (long long)blocks);
