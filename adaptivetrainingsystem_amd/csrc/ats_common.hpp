@@ -40,13 +40,19 @@ struct bf16_t {
 
 __device__ __forceinline__ float bf16_bits_to_float(uint32_t b) { return __uint_as_float(b << 16); }
 
-// Round to nearest even; NaN stays NaN (quiet).
-__device__ __forceinline__ uint32_t float_to_bf16_bits(float f) {
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return u >> 16;
+// float32 pair -> packed bf16 pair with the hardware converter (v_cvt_pk_bf16_f32: round to
+// nearest even, NaN stays a quiet NaN).  lo goes to bits [15:0].
+typedef __bf16 ats_bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float ats_f32x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
+    union {
+        ats_bf16x2_t b;
+        uint32_t u;
+    } cv;
+    cv.b = __builtin_convertvector(ats_f32x2_t{lo, hi}, ats_bf16x2_t);
+    return cv.u;
 }
+__device__ __forceinline__ uint32_t float_to_bf16_bits(float f) { return pack_bf16x2(f, 0.f) & 0xffffu; }
 
 template <typename T>
 struct Elem;
@@ -84,8 +90,7 @@ struct Elem<bf16_t> {
     __device__ static __forceinline__ uint4 pack(const float* f) {
         uint32_t w[4];
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-            w[i] = float_to_bf16_bits(f[2 * i]) | (float_to_bf16_bits(f[2 * i + 1]) << 16);
+        for (int i = 0; i < 4; ++i) w[i] = pack_bf16x2(f[2 * i], f[2 * i + 1]);
         return make_uint4(w[0], w[1], w[2], w[3]);
     }
 };

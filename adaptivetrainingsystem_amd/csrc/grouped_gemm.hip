@@ -40,7 +40,6 @@ struct GroupedArgs {
     const int32_t* row_start;
     const int32_t* row_count;
     int E, K, N_out, up_offset, n_tiles;
-    int force_general;  // testing aid: always take the general (k-tail capable) kernel
 };
 
 constexpr int kRowPitch = 144;  // bytes per staged row: 128 data + 16 pad
@@ -73,27 +72,57 @@ __device__ __forceinline__ float silu_f(float g) {
     return g * __builtin_amdgcn_rcpf(1.0f + e);
 }
 
-template <typename TO>
-__device__ __forceinline__ void store4(TO* p, const float* v, int n_valid);
-template <>
-__device__ __forceinline__ void store4<float>(float* p, const float* v, int n_valid) {
-    if (n_valid >= 4 && (reinterpret_cast<uintptr_t>(p) & 15u) == 0) {
-        *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]);
-    } else {
-        for (int i = 0; i < 4; ++i)
-            if (i < n_valid) p[i] = v[i];
-    }
-}
-template <>
-__device__ __forceinline__ void store4<bf16_t>(bf16_t* p, const float* v, int n_valid) {
-    if (n_valid >= 4 && (reinterpret_cast<uintptr_t>(p) & 7u) == 0) {
-        uint2 u;
-        u.x = float_to_bf16_bits(v[0]) | (float_to_bf16_bits(v[1]) << 16);
-        u.y = float_to_bf16_bits(v[2]) | (float_to_bf16_bits(v[3]) << 16);
-        *reinterpret_cast<uint2*>(p) = u;
-    } else {
-        for (int i = 0; i < 4; ++i)
-            if (i < n_valid) p[i].bits = (uint16_t)float_to_bf16_bits(v[i]);
+// Epilogue through LDS.  In the accumulator layout a lane owns 4 consecutive columns of one row,
+// so storing straight from registers would issue 8-byte pieces of 64 different cache lines per
+// instruction.  Instead every wave transposes 32-row blocks of its sub-tile through a private LDS
+// region and writes whole rows: 16 bytes per lane, 128-byte lines fully covered.
+// wstage: this wave's private region, 32 * (WCOLS * sizeof(TO) + 16) bytes.
+template <typename TO, int TM, int TN, bool SWIGLU>
+__device__ __forceinline__ void epilogue_staged(f32x16_t (&acc)[TN][TM], unsigned char* wstage, TO* out, int64_t ldo,
+                                                int64_t row_base, int rows_valid, int ncol0, int n_out, int lane) {
+    constexpr int TNO = SWIGLU ? TN / 2 : TN;
+    constexpr int WCOLS = TNO * 32;
+    constexpr int ES = (int)sizeof(TO);
+    constexpr int PITCH = WCOLS * ES + 16;
+    constexpr int LPR = WCOLS * ES / 16;   // lanes per output row
+    constexpr int RPI = 64 / LPR;          // rows per store instruction
+    constexpr int EPC = 16 / ES;           // elements per 16-byte chunk
+    const int frow = lane & 31, fgrp = lane >> 5;
+#pragma unroll
+    for (int i = 0; i < TM; ++i) {
+#pragma unroll
+        for (int j = 0; j < TNO; ++j) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                float v[4];
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    if (SWIGLU) v[c] = silu_f(acc[j][i][q * 4 + c]) * acc[j + TN / 2][i][q * 4 + c];
+                    else v[c] = acc[j][i][q * 4 + c];
+                }
+                unsigned char* dst = wstage + frow * PITCH + (j * 32 + 8 * q + 4 * fgrp) * ES;
+                if constexpr (ES == 2) {
+                    uint2 u;
+                    u.x = pack_bf16x2(v[0], v[1]);
+                    u.y = pack_bf16x2(v[2], v[3]);
+                    *reinterpret_cast<uint2*>(dst) = u;
+                } else {
+                    *reinterpret_cast<float4*>(dst) = make_float4(v[0], v[1], v[2], v[3]);
+                }
+            }
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+        for (int r0 = 0; r0 < 32; r0 += RPI) {
+            const int r = r0 + lane / LPR;
+            const int c = lane % LPR;
+            const u32x4_t data = *reinterpret_cast<const u32x4_t*>(wstage + r * PITCH + c * 16);
+            const int m_local = i * 32 + r;
+            const int col = ncol0 + c * EPC;
+            if (m_local < rows_valid && col < n_out)
+                *reinterpret_cast<u32x4_t*>(out + (row_base + m_local) * ldo + col) = data;
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
     }
 }
 
@@ -236,31 +265,14 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_kernel(GroupedArgs p
         __syncthreads();
     }
 
-    // ---- epilogue.  acc[j][i][v]: output row m = tile row (lane & 31), output
-    // column n = 8*(v/4) + 4*(lane>>5) + (v%4) inside the 32x32 tile.
-    TO* out = static_cast<TO*>(p.out);
-    constexpr int TNO = SWIGLU ? TN / 2 : TN;
-#pragma unroll
-    for (int i = 0; i < TM; ++i) {
-        const int m = tc.mt * BM + wm * (BM / WM) + i * 32 + frow;
-        if (m >= count) continue;
-        TO* orow = out + (int64_t)(row0 + m) * p.ldo;
-#pragma unroll
-        for (int j = 0; j < TNO; ++j) {
-            const int ncol0 = SWIGLU ? tc.nt * HALF + wn * (BN / WN / 2) + j * 32 : tc.nt * BN + wn * (BN / WN) + j * 32;
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const int n = ncol0 + 8 * q + 4 * fgrp;
-                float v[4];
-#pragma unroll
-                for (int c = 0; c < 4; ++c) {
-                    if (SWIGLU) v[c] = silu_f(acc[j][i][q * 4 + c]) * acc[j + TN / 2][i][q * 4 + c];
-                    else v[c] = acc[j][i][q * 4 + c];
-                }
-                const int n_valid = p.N_out - n;
-                if (n_valid > 0) store4<TO>(orow + n, v, n_valid);
-            }
-        }
+    // ---- epilogue (all LDS reads of the K loop are behind the last barrier, so LDS is free)
+    {
+        constexpr int TNO_ = SWIGLU ? TN / 2 : TN;
+        constexpr int WSTAGE = 32 * (TNO_ * 32 * (int)sizeof(TO) + 16);
+        const int wrow = tc.mt * BM + wm * (BM / WM);
+        const int ncol0 = SWIGLU ? tc.nt * HALF + wn * (BN / WN / 2) : tc.nt * BN + wn * (BN / WN);
+        epilogue_staged<TO, TM, TN, SWIGLU>(acc, smem + wave * WSTAGE, static_cast<TO*>(p.out), p.ldo,
+                                            (int64_t)row0 + wrow, count - wrow, ncol0, p.N_out, lane);
     }
 }
 
@@ -506,40 +518,27 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_pipelined_kernel(Gro
     PL_ITER(kt, false, false, 0);
     junk ^= pfa[0] ^ pfb[0] ^ pfa[1] ^ pfb[1];
 #undef PL_LOADG
-#undef PL_STORE
-#undef PL_READ
-#undef PL_MMA
 #undef PL_ITER
-#undef PL_FENCE
-#undef PL_MIX_READS
 
     TO* out = static_cast<TO*>(p.out);
     if (p.E < 0) out[0] = TO{};   // never true; with the next line it keeps the warm-up loads alive
     if (p.E < 0 && junk == 0x5a5a5a5au) out[1] = TO{};
-    constexpr int TNO = SWIGLU ? TN / 2 : TN;
-#pragma unroll
-    for (int i = 0; i < TM; ++i) {
-        const int m = tc.mt * BM + wm * (BM / WM) + i * 32 + frow;
-        if (m >= count) continue;
-        TO* orow = out + (int64_t)(row0 + m) * p.ldo;
-#pragma unroll
-        for (int j = 0; j < TNO; ++j) {
-            const int ncol0 = SWIGLU ? tc.nt * HALF + wn * (BN / WN / 2) + j * 32 : tc.nt * BN + wn * (BN / WN) + j * 32;
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const int n = ncol0 + 8 * q + 4 * fgrp;
-                float v[4];
-#pragma unroll
-                for (int c = 0; c < 4; ++c) {
-                    if (SWIGLU) v[c] = silu_f(acc[j][i][q * 4 + c]) * acc[j + TN / 2][i][q * 4 + c];
-                    else v[c] = acc[j][i][q * 4 + c];
-                }
-                const int n_valid = p.N_out - n;
-                if (n_valid > 0) store4<TO>(orow + n, v, n_valid);
-            }
-        }
+    {
+        constexpr int TNO_ = SWIGLU ? TN / 2 : TN;
+        constexpr int WSTAGE = 32 * (TNO_ * 32 * (int)sizeof(TO) + 16);
+        const int wrow = tc.mt * BM + wm * (BM / WM);
+        const int ncol0 = SWIGLU ? tc.nt * HALF + wn * (BN / WN / 2) : tc.nt * BN + wn * (BN / WN);
+        epilogue_staged<TO, TM, TN, SWIGLU>(acc, smem + wave * WSTAGE, out, p.ldo, (int64_t)row0 + wrow, count - wrow,
+                                            ncol0, p.N_out, lane);
     }
 }
+
+
+#undef PL_STORE
+#undef PL_READ
+#undef PL_MMA
+#undef PL_FENCE
+#undef PL_MIX_READS
 
 template <typename T, typename TO, int BM, int BN, int WM, int WN, int SM, int SN, bool SWIGLU>
 static int launch_cfg(const GroupedArgs& p0, int64_t max_rows, hipStream_t s) {
@@ -563,12 +562,12 @@ static int launch_cfg(const GroupedArgs& p0, int64_t max_rows, hipStream_t s) {
         }
         attr_done = true;
     }
-    auto kern = (p.K % BK == 0 && !(p.force_general & 1)) ? kern_pipe : kern_general;
     const int64_t blocks = grid_blocks(max_rows, p.E, BM, p.n_tiles, SM, SN);
     if (blocks > 0x7fffffffLL) {
         set_error("grouped GEMM: grid of %lld blocks", (long long)blocks);
         return ATS_ERR_UNSUPPORTED;
     }
+    auto kern = (p.K % BK == 0) ? kern_pipe : kern_general;
     hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(WM * WN * 64), smem, s, p);
     return ATS_OK;
 }
