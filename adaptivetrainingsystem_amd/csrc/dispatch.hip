@@ -329,6 +329,7 @@ __global__ __launch_bounds__(256) void combine_vec_kernel(const TY* __restrict__
             rows[n] = __shfl(my_row, src, 64);
             wts[n] = __shfl(my_w, src, 64);
         }
+#pragma unroll 4
         for (int h0 = lane * V; h0 < H; h0 += kWave * V) {
             float acc[V];
 #pragma unroll

@@ -28,7 +28,7 @@ template <typename T>
 __global__ __launch_bounds__(256) void rope_vec_kernel(RopeSeg q, RopeSeg k, const float* __restrict__ cos_tab,
                                                        const float* __restrict__ sin_tab, int table_stride,
                                                        int L, int D, int pos_offset, int lanes_per_row,
-                                                       int pos_per_wave, int n_pos_groups, int64_t n_items) {
+                                                       int pos_per_wave, int n_pos_groups, int64_t n_items, bool tab_vec) {
     constexpr int V = Elem<T>::kVec;
     const int lane = lane_id();
     const int64_t item = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
@@ -51,10 +51,20 @@ __global__ __launch_bounds__(256) void rope_vec_kernel(RopeSeg q, RopeSeg k, con
     {
         const float* cp = cos_tab + (int64_t)(pos_offset + pos) * table_stride + c * V;
         const float* sp = sin_tab + (int64_t)(pos_offset + pos) * table_stride + c * V;
+        if (tab_vec) {   // 16-byte table loads (stride and base are multiples of 4 floats)
 #pragma unroll
-        for (int j = 0; j < V; ++j) {
-            cs[j] = cp[j];
-            sn[j] = sp[j];
+            for (int j = 0; j < V; j += 4) {
+                const float4 cv = *reinterpret_cast<const float4*>(cp + j);
+                const float4 sv = *reinterpret_cast<const float4*>(sp + j);
+                cs[j] = cv.x; cs[j + 1] = cv.y; cs[j + 2] = cv.z; cs[j + 3] = cv.w;
+                sn[j] = sv.x; sn[j + 1] = sv.y; sn[j + 2] = sv.z; sn[j + 3] = sv.w;
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < V; ++j) {
+                cs[j] = cp[j];
+                sn[j] = sp[j];
+            }
         }
     }
     const int h0 = chunk * kRopeHeadsPerItem;
@@ -151,8 +161,9 @@ static void launch_rope(RopeSeg q, RopeSeg k, const float* cos_tab, const float*
         const int n_pos_groups = (L + pos_per_wave - 1) / pos_per_wave;
         const int64_t n_items = (int64_t)n_pos_groups * (q.chunks + k.chunks) * B;
         const int64_t blocks = (n_items + 3) / 4;
+        const bool tab_vec = table_stride % 4 == 0 && aligned16(cos_tab) && aligned16(sin_tab);
         hipLaunchKernelGGL((rope_vec_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, s, q, k, cos_tab, sin_tab,
-                           table_stride, L, D, pos_offset, lanes_per_row, pos_per_wave, n_pos_groups, n_items);
+                           table_stride, L, D, pos_offset, lanes_per_row, pos_per_wave, n_pos_groups, n_items, tab_vec);
     } else {
         const int64_t total = (int64_t)B * (q.heads + k.heads) * L * (D / 2);
         int64_t blocks = (total + 255) / 256;

@@ -5,9 +5,8 @@
 // bf16: a block owns 16 tokens; its 4 waves split the hidden dimension in
 // quarters (4x more loads in flight than one wave per tile), each feeding
 // v_mfma_f32_16x16x32_bf16 straight from global memory with 16-byte loads, and
-// the four partial tiles are summed in a fixed order through LDS.  Any bijection
-// of the k index onto (lane group, step) gives the same dot product as long as
-// A and B use the same one, so every lane reads 64 contiguous bytes per step.
+// the four partial tiles are summed in a fixed order through LDS.  The four lane
+// groups of a row read 64 contiguous bytes per load instruction.
 // f32 (and odd shapes): one wave per token with plain FMAs.
 //
 // Routing pass.  A group of G = pow2 >= min(E,64) lanes owns one token; values
@@ -25,32 +24,39 @@ namespace ats {
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8_t;
 typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
 
-union Frag16 {
-    uint4 u;
-    bf16x8_t v;
-};
+typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ bf16x8_t as_bf16x8(const u32x4_t& u) {
+    union {
+        u32x4_t u;
+        bf16x8_t v;
+    } cv;
+    cv.u = u;
+    return cv.v;
+}
 
 constexpr int kGateKC = 128;  // k elements consumed per wave per step
 
-// NT = number of 16-wide expert tiles.
-template <int NT>
-__global__ __launch_bounds__(256) void gate_gemm_bf16_kernel(const bf16_t* __restrict__ x,
-                                                             const bf16_t* __restrict__ wg,
-                                                             const float* __restrict__ bias,
-                                                             float* __restrict__ logits, int64_t T, int H,
-                                                             int E) {
-    __shared__ float red[4][NT][16 * 16];
+// NT = number of 16-wide expert tiles, KW = waves per block (each owns 1/KW of the hidden
+// dimension).  With PF the loads of step s+1 are issued before the MFMAs of step s.
+template <int NT, int KW, bool PF>
+__global__ __launch_bounds__(KW * 64) void gate_gemm_bf16_kernel(const bf16_t* __restrict__ x,
+                                                               const bf16_t* __restrict__ wg,
+                                                               const float* __restrict__ bias,
+                                                               float* __restrict__ logits, int64_t T, int H,
+                                                               int E) {
+    __shared__ float red[KW][NT][16 * 16];
     const int lane = lane_id();
     const int wave = threadIdx.x >> 6;
     const int r = lane & 15;   // A: token row inside the tile; B: expert inside the tile
-    const int g = lane >> 4;   // lane group -> 32-element k slice of each 128-element step
+    const int g = lane >> 4;   // lane group -> 8-element k slice of each 32-element MFMA step (64 contiguous bytes per row and load)
     const int64_t t0 = (int64_t)blockIdx.x * 16;
     const int64_t trow = t0 + r;
     const bool row_ok = trow < T;
 
-    // this wave's k range (multiple of kGateKC per wave, tail handled by predicates)
+    // this wave's k range (whole steps; the tail is handled by predicates)
     const int steps_total = (H + kGateKC - 1) / kGateKC;
-    const int steps_per_wave = (steps_total + 3) / 4;
+    const int steps_per_wave = (steps_total + KW - 1) / KW;
     const int s_begin = wave * steps_per_wave;
     const int s_end = min(steps_total, s_begin + steps_per_wave);
 
@@ -59,33 +65,59 @@ __global__ __launch_bounds__(256) void gate_gemm_bf16_kernel(const bf16_t* __res
     for (int n = 0; n < NT; ++n) acc[n] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
     const bf16_t* xrow = x + (row_ok ? trow : 0) * (int64_t)H;
-    const uint4 zero4 = make_uint4(0, 0, 0, 0);
+    const u32x4_t zero4 = {0u, 0u, 0u, 0u};
+    u32x4_t a[PF ? 2 : 1][4], b[PF ? 2 : 1][NT][4];
 
-    for (int s = s_begin; s < s_end; ++s) {
-        const int kb = s * kGateKC + g * 32;
-        Frag16 a[4];
-        Frag16 b[NT][4];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int kk = kb + i * 8;
-            a[i].u = (row_ok && kk < H) ? *reinterpret_cast<const uint4*>(xrow + kk) : zero4;
-        }
-#pragma unroll
-        for (int n = 0; n < NT; ++n) {
-            const int e = n * 16 + r;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int kk = kb + i * 8;
-                b[n][i].u = (e < E && kk < H) ? *reinterpret_cast<const uint4*>(wg + (int64_t)e * H + kk) : zero4;
+#define GG_LOAD(s_, buf_)                                                                              \
+    {                                                                                                  \
+        const int kb_ = (s_) * kGateKC + g * 8;                                                        \
+        _Pragma("unroll") for (int i = 0; i < 4; ++i) {                                                \
+            const int kk = kb_ + i * 32;                                                               \
+            a[buf_][i] = zero4;                                                                        \
+            if (row_ok && kk < H) a[buf_][i] = *reinterpret_cast<const u32x4_t*>(xrow + kk);           \
+        }                                                                                              \
+        _Pragma("unroll") for (int n = 0; n < NT; ++n) {                                               \
+            const int e = n * 16 + r;                                                                  \
+            _Pragma("unroll") for (int i = 0; i < 4; ++i) {                                            \
+                const int kk = kb_ + i * 32;                                                           \
+                b[buf_][n][i] = zero4;                                                                 \
+                if (e < E && kk < H) b[buf_][n][i] = *reinterpret_cast<const u32x4_t*>(wg + (int64_t)e * H + kk); \
+            }                                                                                          \
+        }                                                                                              \
+    }
+#define GG_MMA(buf_)                                                                                   \
+    {                                                                                                  \
+        _Pragma("unroll") for (int i = 0; i < 4; ++i) {                                                \
+            _Pragma("unroll") for (int n = 0; n < NT; ++n)                                             \
+                acc[n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a[buf_][i]), as_bf16x8(b[buf_][n][i]), acc[n], 0, 0, 0); \
+        }                                                                                              \
+    }
+    if constexpr (PF) {
+        if (s_begin < s_end) {
+            GG_LOAD(s_begin, 0);
+            int s = s_begin;
+            for (; s + 2 < s_end; s += 2) {
+                GG_LOAD(s + 1, 1);
+                GG_MMA(0);
+                GG_LOAD(s + 2, 0);
+                GG_MMA(1);
+            }
+            if (s + 1 < s_end) {
+                GG_LOAD(s + 1, PF ? 1 : 0);
+                GG_MMA(0);
+                GG_MMA(PF ? 1 : 0);
+            } else {
+                GG_MMA(0);
             }
         }
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-#pragma unroll
-            for (int n = 0; n < NT; ++n)
-                acc[n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i].v, b[n][i].v, acc[n], 0, 0, 0);
+    } else {
+        for (int s = s_begin; s < s_end; ++s) {
+            GG_LOAD(s, 0);
+            GG_MMA(0);
         }
     }
+#undef GG_LOAD
+#undef GG_MMA
     // D layout of the 16x16 tile: lane holds column (lane & 15), rows 4*(lane>>4) + v.
 #pragma unroll
     for (int n = 0; n < NT; ++n) {
@@ -93,14 +125,16 @@ __global__ __launch_bounds__(256) void gate_gemm_bf16_kernel(const bf16_t* __res
         for (int v = 0; v < 4; ++v) red[wave][n][(4 * g + v) * 16 + r] = acc[n][v];
     }
     __syncthreads();
-    for (int i = threadIdx.x; i < NT * 256; i += 256) {
+    for (int i = threadIdx.x; i < NT * 256; i += KW * 64) {
         const int n = i >> 8;
         const int row = (i & 255) >> 4;
         const int col = i & 15;
         const int e = n * 16 + col;
         const int64_t t = t0 + row;
         if (t < T && e < E) {
-            float v = ((red[0][n][i & 255] + red[1][n][i & 255]) + red[2][n][i & 255]) + red[3][n][i & 255];
+            float v = red[0][n][i & 255];
+#pragma unroll
+            for (int w = 1; w < KW; ++w) v += red[w][n][i & 255];
             if (bias) v += bias[e];
             logits[t * E + e] = v;
         }
@@ -380,14 +414,16 @@ extern "C" int ats_router_logits(const void* x, const void* wg, const float* bia
         const bf16_t* xp = static_cast<const bf16_t*>(x);
         const bf16_t* wp = static_cast<const bf16_t*>(wg);
         const int nt = (E + 15) / 16;
+        // Few experts: 8 waves split K (short dependent chains, 32 waves per CU resident);
+        // more expert tiles need more registers per wave and use 4 waves with (NT <= 2) prefetch.
         if (nt <= 1)
-            hipLaunchKernelGGL((gate_gemm_bf16_kernel<1>), dim3(blocks), dim3(256), 0, s, xp, wp, bias, logits, T, H, E);
+            hipLaunchKernelGGL((gate_gemm_bf16_kernel<1, 8, false>), dim3(blocks), dim3(512), 0, s, xp, wp, bias, logits, T, H, E);
         else if (nt <= 2)
-            hipLaunchKernelGGL((gate_gemm_bf16_kernel<2>), dim3(blocks), dim3(256), 0, s, xp, wp, bias, logits, T, H, E);
+            hipLaunchKernelGGL((gate_gemm_bf16_kernel<2, 4, true>), dim3(blocks), dim3(256), 0, s, xp, wp, bias, logits, T, H, E);
         else if (nt <= 4)
-            hipLaunchKernelGGL((gate_gemm_bf16_kernel<4>), dim3(blocks), dim3(256), 0, s, xp, wp, bias, logits, T, H, E);
+            hipLaunchKernelGGL((gate_gemm_bf16_kernel<4, 4, false>), dim3(blocks), dim3(256), 0, s, xp, wp, bias, logits, T, H, E);
         else
-            hipLaunchKernelGGL((gate_gemm_bf16_kernel<8>), dim3(blocks), dim3(256), 0, s, xp, wp, bias, logits, T, H, E);
+            hipLaunchKernelGGL((gate_gemm_bf16_kernel<8, 4, false>), dim3(blocks), dim3(256), 0, s, xp, wp, bias, logits, T, H, E);
     } else {
         int64_t blocks = (T + 3) / 4;
         if (blocks > 8192) blocks = 8192;
