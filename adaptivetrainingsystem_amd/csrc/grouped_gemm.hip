@@ -578,8 +578,10 @@ template <typename T, typename TO, bool SWIGLU>
 static int launch_grouped(const GroupedArgs& p, int64_t max_rows, hipStream_t s) {
     const int64_t avg = max_rows / (p.E > 0 ? p.E : 1);
     if (avg <= 48) {
-        if constexpr (SWIGLU) return launch_cfg<T, TO, 32, 256, 1, 4, 1, 32, SWIGLU>(p, max_rows, s);
-        else return launch_cfg<T, TO, 32, 128, 1, 4, 1, 32, SWIGLU>(p, max_rows, s);
+        // Weight streaming: small tiles give many blocks per CU (loads in flight) and tile counts
+        // that divide evenly over the CUs.
+        if constexpr (SWIGLU) return launch_cfg<T, TO, 32, 128, 1, 2, 1, 32, SWIGLU>(p, max_rows, s);
+        else return launch_cfg<T, TO, 32, 64, 1, 2, 1, 32, SWIGLU>(p, max_rows, s);
     }
     if (avg <= 768) return launch_cfg<T, TO, 128, 256, 2, 2, 4, 8, SWIGLU>(p, max_rows, s);
     return launch_cfg<T, TO, 256, 256, 2, 2, 4, 8, SWIGLU>(p, max_rows, s);
