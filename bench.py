@@ -32,6 +32,9 @@ sys.path.insert(0, ROOT)
 
 PEAK_MFMA_BF16_TFLOPS = 2500.0   # MI355X dense bf16
 PEAK_HBM_GBS = 8000.0            # MI355X HBM3E
+# HBM-side bytes per launch of the gate/up GEMM, from separate hardware-counter runs of this script
+# (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0, factors from a 1 GiB copy; summary under profiles/).
+GATEUP_HBM_BYTES_PER_LAUNCH = {"c4_prefill": 11.17e9}
 
 
 def log(*a):
@@ -113,7 +116,7 @@ def run_moe(args):
                    "kept_assignments": kept, "dropped_assignments": dropped},
         "roofline": {"kernel": "grouped gate/up GEMM + SwiGLU", "bound": "mfma", "achieved": achieved,
                      "peak": PEAK_MFMA_BF16_TFLOPS, "unit": "TFLOP/s", "frac": achieved / PEAK_MFMA_BF16_TFLOPS,
-                     "traffic": None},
+                     "traffic": GATEUP_HBM_BYTES_PER_LAUNCH.get(name)},
         "stages_ms": {s: round(v["mean_ms"], 4) for s, v in stages.items()},
     }
     if not args.no_cpu_baseline:
@@ -190,6 +193,8 @@ def main():
     ap.add_argument("--workload", default="c4_prefill",
                     choices=["c4_prefill", "c3_decode", "c5_finegrained_mod", "c1_cpu_reference", "c2_norm_rope"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--copy-probe", action="store_true",
+                    help="also run a 1 GiB device copy (known traffic) so hardware-counter runs can be scaled")
     ap.add_argument("--cpu-sample-tokens", type=int, default=16384)
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -202,6 +207,13 @@ def main():
     from adaptivetrainingsystem_amd import _lib
     _lib.load()
     torch.cuda.set_device(0)
+    if args.copy_probe:
+        src = torch.empty(1 << 29, dtype=torch.bfloat16, device="cuda:0").normal_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     result = run_norm_rope(args) if args.workload == "c2_norm_rope" else run_moe(args)
     print(json.dumps(result), flush=True)
 
