@@ -289,7 +289,7 @@ __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(
 //   LDS barrier
 //   k-step 3: MFMAs(buf 1) | read k-step 0 of slab t+1
 // Global loads therefore have a whole slab of MFMA time to land before they are needed.
-template <typename T, typename TO, int BM, int BN, int WM, int WN, int SM, int SN, bool SWIGLU>
+template <typename T, typename TO, int BM, int BN, int WM, int WN, int SM, int SN, bool SWIGLU, bool WARM>
 __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_pipelined_kernel(GroupedArgs p) {
     constexpr int NT = WM * WN * 64;
     constexpr int VEC = 16 / (int)sizeof(T);
@@ -472,10 +472,12 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_pipelined_kernel(Gro
         PL_READ(cur_, 3, 1);                                                            \
         if (HAS2) {                                                                     \
             PL_LOADG((kt_) + 2);                                                        \
-            junk ^= pfa[SLOT] ^ pfb[SLOT];                                              \
-            const int kpf_ = min((kt_) + 2 + kPfDist, nk - 1) * BK;                     \
-            pfa[SLOT] = *reinterpret_cast<const unsigned*>(apf + kpf_);                 \
-            pfb[SLOT] = *reinterpret_cast<const unsigned*>(bpf + kpf_);                 \
+            if (WARM) {                                                                 \
+                junk ^= pfa[SLOT] ^ pfb[SLOT];                                          \
+                const int kpf_ = min((kt_) + 2 + kPfDist, nk - 1) * BK;                 \
+                pfa[SLOT] = *reinterpret_cast<const unsigned*>(apf + kpf_);             \
+                pfb[SLOT] = *reinterpret_cast<const unsigned*>(bpf + kpf_);             \
+            }                                                                           \
         }                                                                               \
         PL_MMA(0);                                                                      \
         if (HAS2) {                                                                     \
@@ -484,7 +486,7 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_pipelined_kernel(Gro
                 __builtin_amdgcn_sched_group_barrier(SG_DS_RD, 1, 0);                   \
                 __builtin_amdgcn_sched_group_barrier(SG_VMEM_RD, (PA + PB) / (TM + TN), 0); \
             }                                                                           \
-            __builtin_amdgcn_sched_group_barrier(SG_VMEM_RD, 2, 0);                     \
+            if (WARM) __builtin_amdgcn_sched_group_barrier(SG_VMEM_RD, 2, 0);           \
         } else {                                                                        \
             PL_MIX_READS();                                                             \
         }                                                                               \
@@ -548,7 +550,7 @@ static int launch_cfg(const GroupedArgs& p0, int64_t max_rows, hipStream_t s) {
     constexpr size_t smem = 2 * (size_t)(BM + BN) * kRowPitch;
     constexpr int BK = 128 / (int)sizeof(T);
     auto kern_general = grouped_gemm_kernel<T, TO, BM, BN, WM, WN, SM, SN, SWIGLU>;
-    auto kern_pipe = grouped_gemm_pipelined_kernel<T, TO, BM, BN, WM, WN, SM, SN, SWIGLU>;
+    auto kern_pipe = grouped_gemm_pipelined_kernel<T, TO, BM, BN, WM, WN, SM, SN, SWIGLU, (WM * WN <= 4)>;
     static bool attr_done = false;
     if (!attr_done) {
         if (smem > 64 * 1024) {
@@ -583,8 +585,15 @@ static int launch_grouped(const GroupedArgs& p, int64_t max_rows, hipStream_t s)
         if constexpr (SWIGLU) return launch_cfg<T, TO, 32, 128, 1, 2, 1, 32, SWIGLU>(p, max_rows, s);
         else return launch_cfg<T, TO, 32, 64, 1, 2, 1, 32, SWIGLU>(p, max_rows, s);
     }
-    if (avg <= 768) return launch_cfg<T, TO, 128, 256, 2, 2, 4, 8, SWIGLU>(p, max_rows, s);
-    return launch_cfg<T, TO, 256, 256, 2, 2, 4, 8, SWIGLU>(p, max_rows, s);
+    if (avg <= 768) {
+        // Mid-size groups are short on reuse (a weight panel serves 3-6 row tiles), so loads often
+        // miss L2: favour more resident blocks / waves over tile size.
+        if constexpr (SWIGLU) return launch_cfg<T, TO, 128, 128, 2, 2, 4, 8, SWIGLU>(p, max_rows, s);
+        else return launch_cfg<T, TO, 128, 256, 2, 4, 4, 8, SWIGLU>(p, max_rows, s);
+    }
+    // Prefill: 256 x 256 tile, 8 waves (2 per SIMD: one wave's LDS / memory waits are covered by
+    // the other's MFMAs), 128 accumulator registers per lane.
+    return launch_cfg<T, TO, 256, 256, 2, 4, 4, 8, SWIGLU>(p, max_rows, s);
 }
 
 static int check_common(const char* name, const void* a, const void* const* w, const void* out,
