@@ -10,7 +10,7 @@
 //   3. per-chunk ranking: inside a wave the rank among equal ids comes from
 //      ballots; across the steps of a wave and the waves of a block from small
 //      LDS counters that are only ever advanced in program order.
-// A single chunk (T*k <= kPlanChunk) runs all three steps in one launch.
+// Small plans (T*k <= kPlanSingle) run all three steps in one block, one launch.
 #include <limits.h>
 
 #include "ats_common.hpp"
@@ -21,8 +21,8 @@
 
 namespace ats {
 
-constexpr int kPlanChunk = 1024;     // assignments per block
-constexpr int kPlanPerWave = 256;    // assignments per wave (4 steps of 64)
+constexpr int kPlanChunk = 256;      // assignments per block of the multi-block plan (64 per wave: one step)
+constexpr int kPlanSingle = 1024;    // largest plan done by one block alone (256 per wave: four steps)
 constexpr int kPlanMaxE = 1024;
 
 template <typename IdxT>
@@ -37,14 +37,14 @@ __device__ __forceinline__ int load_expert(const IdxT* idx, int64_t a, int64_t n
 }
 
 // step 1: counts of one chunk into LDS (s_cnt[w*E + e] per wave), returns via LDS
-template <typename IdxT>
+template <typename IdxT, int PERWAVE>
 __device__ void chunk_wave_counts(const IdxT* idx, int64_t n, int E, int64_t chunk_base, int* s_cnt, bool* bad) {
     const int lane = lane_id();
     const int wave = threadIdx.x >> 6;
     for (int i = threadIdx.x; i < 4 * E; i += 256) s_cnt[i] = 0;
     __syncthreads();
-    for (int step = 0; step < kPlanPerWave / kWave; ++step) {
-        const int64_t a = chunk_base + wave * kPlanPerWave + step * kWave + lane;
+    for (int step = 0; step < PERWAVE / kWave; ++step) {
+        const int64_t a = chunk_base + wave * PERWAVE + step * kWave + lane;
         const int e = load_expert(idx, a, n, E, bad);
         if (e >= 0) atomicAdd(&s_cnt[wave * E + e], 1);
     }
@@ -57,26 +57,52 @@ __global__ __launch_bounds__(256) void plan_hist_kernel(const IdxT* __restrict__
                                                         int32_t* __restrict__ status) {
     extern __shared__ int s_cnt[];
     bool bad = false;
-    chunk_wave_counts(idx, n, E, (int64_t)blockIdx.x * kPlanChunk, s_cnt, &bad);
+    chunk_wave_counts<IdxT, kPlanChunk / 4>(idx, n, E, (int64_t)blockIdx.x * kPlanChunk, s_cnt, &bad);
     for (int e = threadIdx.x; e < E; e += 256)
         chunk_hist[(int64_t)blockIdx.x * E + e] = s_cnt[e] + s_cnt[E + e] + s_cnt[2 * E + e] + s_cnt[3 * E + e];
     if (bad) status[0] = 1;
 }
 
-// step 2 (one block): chunk_hist -> exclusive chunk bases (in place), hist, kept, offsets
+// step 2 (one block): chunk_hist -> exclusive chunk bases (in place), hist, kept, offsets.
+// One wave scans one expert at a time: 64 chunks per pass with a shuffle prefix sum, the carry
+// runs across passes.
 __device__ void scan_totals(int32_t* chunk_hist, int nchunks, int E, int C, int32_t* hist, int32_t* kept,
                             int32_t* offsets, int* s_tot) {
-    for (int e = threadIdx.x; e < E; e += blockDim.x) {
-        int run = 0;
-        for (int c = 0; c < nchunks; ++c) {
-            const int v = chunk_hist[(int64_t)c * E + e];
-            chunk_hist[(int64_t)c * E + e] = run;
-            run += v;
+    const int lane = lane_id();
+    const int wave = threadIdx.x >> 6;
+    const int nwaves = blockDim.x >> 6;
+    constexpr int U = 4;   // experts scanned together by a wave (their loads are issued back to back)
+    for (int e0 = wave * U; e0 < E; e0 += nwaves * U) {
+        int carry[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) carry[u] = 0;
+        for (int base = 0; base < nchunks; base += kWave) {
+            const int c = base + lane;
+            int v[U], incl[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) v[u] = (c < nchunks && e0 + u < E) ? chunk_hist[(int64_t)c * E + e0 + u] : 0;
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                incl[u] = v[u];
+                for (int off = 1; off < kWave; off <<= 1) {
+                    const int up = __shfl_up(incl[u], off, 64);
+                    if (lane >= off) incl[u] += up;
+                }
+                if (c < nchunks && e0 + u < E) chunk_hist[(int64_t)c * E + e0 + u] = carry[u] + incl[u] - v[u];
+                carry[u] += __shfl(incl[u], kWave - 1, 64);
+            }
         }
-        hist[e] = run;
-        const int kp = run < C ? run : C;
-        kept[e] = kp;
-        s_tot[e] = kp;
+        if (lane == 0) {
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                if (e0 + u < E) {
+                    hist[e0 + u] = carry[u];
+                    const int kp = carry[u] < C ? carry[u] : C;
+                    kept[e0 + u] = kp;
+                    s_tot[e0 + u] = kp;
+                }
+            }
+        }
     }
     __syncthreads();
     if (threadIdx.x == 0) {
@@ -99,7 +125,7 @@ __global__ __launch_bounds__(256) void plan_scan_kernel(int32_t* __restrict__ ch
 
 // step 3: ranks of one chunk.  s_cnt holds the per-wave counts of this chunk
 // (from chunk_wave_counts); they are turned into per-wave running bases.
-template <typename IdxT>
+template <typename IdxT, int PERWAVE>
 __device__ void chunk_rank_and_write(const IdxT* idx, int64_t n, int k, int E, int C, int64_t chunk_base,
                                      const int32_t* chunk_excl /* [E] for this chunk */,
                                      const int32_t* offsets, int* s_cnt, int32_t* slot, int32_t* token_map,
@@ -118,8 +144,8 @@ __device__ void chunk_rank_and_write(const IdxT* idx, int64_t n, int k, int E, i
     __syncthreads();
     int* my_base = s_cnt + wave * E;
     const unsigned long long lt_mask = lane == 0 ? 0ull : (~0ull >> (64 - lane));
-    for (int step = 0; step < kPlanPerWave / kWave; ++step) {
-        const int64_t a = chunk_base + wave * kPlanPerWave + step * kWave + lane;
+    for (int step = 0; step < PERWAVE / kWave; ++step) {
+        const int64_t a = chunk_base + wave * PERWAVE + step * kWave + lane;
         bool bad = false;
         const int e = load_expert(idx, a, n, E, &bad);
         int rank = -1;
@@ -159,8 +185,8 @@ __global__ __launch_bounds__(256) void plan_rank_kernel(const IdxT* __restrict__
     extern __shared__ int s_cnt[];
     bool bad = false;
     const int64_t chunk_base = (int64_t)blockIdx.x * kPlanChunk;
-    chunk_wave_counts(idx, n, E, chunk_base, s_cnt, &bad);
-    chunk_rank_and_write(idx, n, k, E, C, chunk_base, chunk_excl + (int64_t)blockIdx.x * E, offsets, s_cnt, slot,
+    chunk_wave_counts<IdxT, kPlanChunk / 4>(idx, n, E, chunk_base, s_cnt, &bad);
+    chunk_rank_and_write<IdxT, kPlanChunk / 4>(idx, n, k, E, C, chunk_base, chunk_excl + (int64_t)blockIdx.x * E, offsets, s_cnt, slot,
                          token_map, row_src, row_of);
     // empty slots and unused compact rows
     const int64_t stride = (int64_t)gridDim.x * 256;
@@ -174,7 +200,7 @@ __global__ __launch_bounds__(256) void plan_rank_kernel(const IdxT* __restrict__
     for (int64_t i = total + (int64_t)blockIdx.x * 256 + threadIdx.x; i < row_src_len; i += stride) row_src[i] = -1;
 }
 
-// Whole plan in one block (n <= kPlanChunk).
+// Whole plan in one block (n <= kPlanSingle).
 template <typename IdxT>
 __global__ __launch_bounds__(256) void plan_single_kernel(const IdxT* idx, int64_t n, int k, int E,
                                                           int C, int32_t* chunk_hist,
@@ -187,14 +213,15 @@ __global__ __launch_bounds__(256) void plan_single_kernel(const IdxT* idx, int64
     int* s_cnt = s_all;          // [4*E]
     int* s_tot = s_all + 4 * E;  // [E]
     bool bad = false;
-    chunk_wave_counts(idx, n, E, 0, s_cnt, &bad);
+    chunk_wave_counts<IdxT, kPlanSingle / 4>(idx, n, E, 0, s_cnt, &bad);
     if (bad) status[0] = 1;
     for (int e = threadIdx.x; e < E; e += 256)
         chunk_hist[e] = s_cnt[e] + s_cnt[E + e] + s_cnt[2 * E + e] + s_cnt[3 * E + e];
     __syncthreads();
     scan_totals(chunk_hist, 1, E, C, hist, kept, offsets, s_tot);
     __threadfence_block();
-    chunk_rank_and_write(idx, n, k, E, C, 0, chunk_hist, offsets, s_cnt, slot, token_map, row_src, row_of);
+    chunk_rank_and_write<IdxT, kPlanSingle / 4>(idx, n, k, E, C, 0, chunk_hist, offsets, s_cnt, slot, token_map, row_src,
+                                                row_of);
     const int64_t ec = (int64_t)E * C;
     for (int64_t i = threadIdx.x; i < ec; i += 256) {
         const int e = (int)(i / C);
@@ -425,7 +452,8 @@ extern "C" int ats_dispatch_plan(const void* idx, int idx_dtype, int64_t T, int 
                 ATS_ERR_INVALID_ARG, "ats_dispatch_plan: null output pointer");
     ATS_REQUIRE(T == 0 || idx, ATS_ERR_INVALID_ARG, "ats_dispatch_plan: null idx");
     const int64_t n = T * k;
-    const int64_t nchunks = n == 0 ? 1 : (n + kPlanChunk - 1) / kPlanChunk;
+    const bool single = n <= kPlanSingle;
+    const int64_t nchunks = single ? 1 : (n + kPlanChunk - 1) / kPlanChunk;
     const size_t need = (size_t)nchunks * E * sizeof(int32_t);
     ATS_REQUIRE(workspace && workspace_bytes >= need, ATS_ERR_WORKSPACE,
                 "ats_dispatch_plan: workspace %zu bytes, need %zu", workspace_bytes, need);
@@ -435,7 +463,7 @@ extern "C" int ats_dispatch_plan(const void* idx, int idx_dtype, int64_t T, int 
     if (row_src_len < 1) row_src_len = 1;
     hipLaunchKernelGGL(plan_clear_status_kernel, dim3(1), dim3(1), 0, s, status);
     const size_t smem = (size_t)5 * E * sizeof(int);
-    if (nchunks == 1) {
+    if (single) {
         if (idx_dtype == ATS_IDX_I32)
             hipLaunchKernelGGL((plan_single_kernel<int32_t>), dim3(1), dim3(256), smem, s,
                                static_cast<const int32_t*>(idx), n, k, E, C, chunk_hist, hist, kept, offsets, slot,

@@ -348,35 +348,57 @@ __global__ __launch_bounds__(256) void route_topk_kernel(const float* __restrict
 }
 
 // Reduces the per-block partials in a fixed order and evaluates the auxiliary loss.
+// Thread (e, c) sums blocks c, c+TPE, ... of expert e (consecutive threads read consecutive
+// experts: coalesced); the TPE partial sums of an expert are then added in ascending c.
 __global__ __launch_bounds__(256) void route_finalize_kernel(const int32_t* __restrict__ part_hist,
                                                              const float* __restrict__ part_colsum, int nblocks,
                                                              int E, int64_t T, int k, float lbw,
                                                              int32_t* __restrict__ hist, float* __restrict__ colsum,
                                                              float* __restrict__ aux) {
     extern __shared__ unsigned char smem_raw[];
-    float* s_term = reinterpret_cast<float*>(smem_raw);  // [E]
-    const int lane = lane_id();
-    const int wave = threadIdx.x >> 6;
-    for (int e = wave; e < E; e += 4) {
+    float* s_term = reinterpret_cast<float*>(smem_raw);          // [E]
+    int* s_h = reinterpret_cast<int*>(s_term + E);               // [256]
+    float* s_c = reinterpret_cast<float*>(s_h + 256);            // [256]
+    int tpe = 1;
+    while (tpe * 2 * E <= 256) tpe *= 2;   // threads per expert (power of two), 1 when E > 128
+    for (int e0 = 0; e0 < E; e0 += 256 / tpe) {
+        const int e = e0 + (int)threadIdx.x % (256 / tpe);
+        const int c = (int)threadIdx.x / (256 / tpe);
         int hsum = 0;
         float csum = 0.f;
-        for (int b = lane; b < nblocks; b += kWave) {
-            hsum += part_hist[(int64_t)b * E + e];
-            csum += part_colsum[(int64_t)b * E + e];
+        if (e < E) {
+            for (int b = c; b < nblocks; b += tpe * 8) {   // 8 independent loads in flight, summed in order
+                int hv[8];
+                float cv[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    const int bb = b + u * tpe;
+                    hv[u] = bb < nblocks ? part_hist[(int64_t)bb * E + e] : 0;
+                    cv[u] = bb < nblocks ? part_colsum[(int64_t)bb * E + e] : 0.f;
+                }
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    hsum += hv[u];
+                    csum += cv[u];
+                }
+            }
         }
-        for (int off = 32; off > 0; off >>= 1) {
-            hsum += __shfl_xor(hsum, off, 64);
-            csum += __shfl_xor(csum, off, 64);
-        }
-        if (lane == 0) {
+        s_h[threadIdx.x] = hsum;
+        s_c[threadIdx.x] = csum;
+        __syncthreads();
+        if (c == 0 && e < E) {
+            for (int cc = 1; cc < tpe; ++cc) {
+                hsum += s_h[cc * (256 / tpe) + (int)threadIdx.x];
+                csum += s_c[cc * (256 / tpe) + (int)threadIdx.x];
+            }
             hist[e] = hsum;
             colsum[e] = csum;
             const float usage = (float)hsum / (float)((double)T * k + 1e-9);
             const float importance = csum / (float)T;
             s_term[e] = usage * importance;
         }
+        __syncthreads();
     }
-    __syncthreads();
     if (threadIdx.x == 0 && aux) {
         float s = 0.f;
         for (int e = 0; e < E; ++e) s += s_term[e];
@@ -488,7 +510,7 @@ extern "C" int ats_route_topk(const float* logits, int64_t T, int E, int k, floa
                            variant, G, iters, idx_out, w_out, part_hist, part_col);
     ATS_CHECK_LAUNCH("ats_route_topk");
     if (stats) {
-        hipLaunchKernelGGL(route_finalize_kernel, dim3(1), dim3(256), (size_t)E * sizeof(float), s, part_hist,
+        hipLaunchKernelGGL(route_finalize_kernel, dim3(1), dim3(256), (size_t)(E + 512) * sizeof(float), s, part_hist,
                            part_col, nblocks, E, T, k, load_balancing_weight, hist, prob_colsum, aux);
         ATS_CHECK_LAUNCH("ats_route_topk(finalize)");
     }

@@ -44,7 +44,7 @@ def test_argument_errors_return_codes_not_exits():
                             None) == -1       # odd head_dim
     assert lib.ats_select_topk_per_sequence(None, 1, 10000, 5, None, None) == -1
     assert lib.ats_route_topk_workspace(16384, 8) > 0
-    assert lib.ats_dispatch_plan_workspace(16384, 2, 8) == 32 * 8 * 4
+    assert lib.ats_dispatch_plan_workspace(16384, 2, 8) == (32768 // 256) * 8 * 4
 
 
 @pytest.mark.parametrize("counts,BM,n_tiles,SM,SN", [
