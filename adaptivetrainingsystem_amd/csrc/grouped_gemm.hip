@@ -580,10 +580,11 @@ template <typename T, typename TO, bool SWIGLU>
 static int launch_grouped(const GroupedArgs& p, int64_t max_rows, hipStream_t s) {
     const int64_t avg = max_rows / (p.E > 0 ? p.E : 1);
     if (avg <= 48) {
-        // Weight streaming: small tiles give many blocks per CU (loads in flight) and tile counts
-        // that divide evenly over the CUs.
-        if constexpr (SWIGLU) return launch_cfg<T, TO, 32, 128, 1, 2, 1, 32, SWIGLU>(p, max_rows, s);
-        else return launch_cfg<T, TO, 32, 64, 1, 2, 1, 32, SWIGLU>(p, max_rows, s);
+        // Decode: pure weight streaming, 32-row tiles.  (Measured alternatives: narrower tiles with
+        // more blocks per CU, and MFMA fragments loaded straight from global memory without LDS,
+        // both stream more slowly - the latter is bound by the address rate of 64-line loads.)
+        if constexpr (SWIGLU) return launch_cfg<T, TO, 32, 256, 1, 4, 1, 32, SWIGLU>(p, max_rows, s);
+        else return launch_cfg<T, TO, 32, 128, 1, 4, 1, 32, SWIGLU>(p, max_rows, s);
     }
     if (avg <= 768) {
         // Mid-size groups are short on reuse (a weight panel serves 3-6 row tiles), so loads often
