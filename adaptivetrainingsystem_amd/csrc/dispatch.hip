@@ -60,7 +60,8 @@ __global__ __launch_bounds__(256) void plan_hist_kernel(const IdxT* __restrict__
     chunk_wave_counts<IdxT, kPlanChunk / 4>(idx, n, E, (int64_t)blockIdx.x * kPlanChunk, s_cnt, &bad);
     for (int e = threadIdx.x; e < E; e += 256)
         chunk_hist[(int64_t)blockIdx.x * E + e] = s_cnt[e] + s_cnt[E + e] + s_cnt[2 * E + e] + s_cnt[3 * E + e];
-    if (bad) status[0] = 1;
+    // the status word is cleared here and raised by the ranking kernel, which runs after this one
+    if (blockIdx.x == 0 && threadIdx.x == 0) status[0] = 0;
 }
 
 // step 2 (one block): chunk_hist -> exclusive chunk bases (in place), hist, kept, offsets.
@@ -181,11 +182,12 @@ __global__ __launch_bounds__(256) void plan_rank_kernel(const IdxT* __restrict__
                                                         const int32_t* __restrict__ offsets,
                                                         int32_t* __restrict__ slot, int32_t* __restrict__ token_map,
                                                         int32_t* __restrict__ row_src, int32_t* __restrict__ row_of,
-                                                        int64_t row_src_len) {
+                                                        int64_t row_src_len, int32_t* __restrict__ status) {
     extern __shared__ int s_cnt[];
     bool bad = false;
     const int64_t chunk_base = (int64_t)blockIdx.x * kPlanChunk;
     chunk_wave_counts<IdxT, kPlanChunk / 4>(idx, n, E, chunk_base, s_cnt, &bad);
+    if (bad) status[0] = 1;
     chunk_rank_and_write<IdxT, kPlanChunk / 4>(idx, n, k, E, C, chunk_base, chunk_excl + (int64_t)blockIdx.x * E, offsets, s_cnt, slot,
                          token_map, row_src, row_of);
     // empty slots and unused compact rows
@@ -214,6 +216,8 @@ __global__ __launch_bounds__(256) void plan_single_kernel(const IdxT* idx, int64
     int* s_tot = s_all + 4 * E;  // [E]
     bool bad = false;
     chunk_wave_counts<IdxT, kPlanSingle / 4>(idx, n, E, 0, s_cnt, &bad);
+    if (threadIdx.x == 0) status[0] = 0;
+    __syncthreads();
     if (bad) status[0] = 1;
     for (int e = threadIdx.x; e < E; e += 256)
         chunk_hist[e] = s_cnt[e] + s_cnt[E + e] + s_cnt[2 * E + e] + s_cnt[3 * E + e];
@@ -231,8 +235,6 @@ __global__ __launch_bounds__(256) void plan_single_kernel(const IdxT* idx, int64
     const int total = offsets[E];
     for (int64_t i = total + threadIdx.x; i < row_src_len; i += 256) row_src[i] = -1;
 }
-
-__global__ void plan_clear_status_kernel(int32_t* status) { status[0] = 0; }
 
 // ------------------------------------------------------------------ row gather
 // One wave per output row; 16-byte accesses; zero rows for negative map entries.
@@ -461,7 +463,6 @@ extern "C" int ats_dispatch_plan(const void* idx, int idx_dtype, int64_t T, int 
     int32_t* chunk_hist = static_cast<int32_t*>(workspace);
     int64_t row_src_len = n < (int64_t)E * C ? n : (int64_t)E * C;
     if (row_src_len < 1) row_src_len = 1;
-    hipLaunchKernelGGL(plan_clear_status_kernel, dim3(1), dim3(1), 0, s, status);
     const size_t smem = (size_t)5 * E * sizeof(int);
     if (single) {
         if (idx_dtype == ATS_IDX_I32)
@@ -488,11 +489,11 @@ extern "C" int ats_dispatch_plan(const void* idx, int idx_dtype, int64_t T, int 
     if (idx_dtype == ATS_IDX_I32)
         hipLaunchKernelGGL((plan_rank_kernel<int32_t>), dim3((unsigned)nchunks), dim3(256), smem, s,
                            static_cast<const int32_t*>(idx), n, k, E, C, chunk_hist, kept, offsets, slot, token_map,
-                           row_src, row_of, row_src_len);
+                           row_src, row_of, row_src_len, status);
     else
         hipLaunchKernelGGL((plan_rank_kernel<int64_t>), dim3((unsigned)nchunks), dim3(256), smem, s,
                            static_cast<const int64_t*>(idx), n, k, E, C, chunk_hist, kept, offsets, slot, token_map,
-                           row_src, row_of, row_src_len);
+                           row_src, row_of, row_src_len, status);
     ATS_CHECK_LAUNCH("ats_dispatch_plan(rank)");
     return ATS_OK;
 }
