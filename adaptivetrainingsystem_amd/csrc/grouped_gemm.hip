@@ -40,6 +40,8 @@ struct GroupedArgs {
     const int32_t* row_start;
     const int32_t* row_count;
     int E, K, N_out, up_offset, n_tiles;
+    // direct-to-LDS path only: bytes addressable from the A / B descriptors (0 = path not usable)
+    uint32_t a_extent_bytes, b_extent_bytes;
 };
 
 constexpr int kRowPitch = 144;  // bytes per staged row: 128 data + 16 pad
@@ -440,6 +442,7 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_pipelined_kernel(Gro
 // instructions with the memory instructions of that phase (so the memory pipes work in the
 // shadow of the MFMAs); nothing moves across a phase boundary.
 #define SG_MFMA 0x008
+#define SG_VMEM 0x010
 #define SG_VMEM_RD 0x020
 #define SG_DS_RD 0x100
 #define SG_DS_WR 0x200
@@ -536,25 +539,235 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_pipelined_kernel(Gro
 }
 
 
+// Direct-to-LDS variant for K % BK == 0 (bf16 and f32).  The loads write LDS themselves
+// (buffer_load_dwordx4 ... lds: lane l of a wave deposits its 16 bytes at M0 + 16*l), so a slab
+// never passes through registers: no staging registers, no ds_write instructions.  The loads use
+// buffer addressing (descriptor base + 32-bit lane offset + scalar k offset), so advancing along
+// K costs no vector ALU work - 64-bit per-lane pointer updates would take issue slots from the
+// MFMAs.  The host only selects this kernel when every lane offset fits in 32 bits.
+//
+// One wave instruction fills 1 KiB = 8 rows x 128 bytes, rows unpadded.  Bank conflicts on the
+// fragment reads are avoided by an XOR swizzle applied on the global side: LDS slot s of row R
+// holds the 16-byte chunk  s ^ f(R),  f(R) = (R & 7) ^ ((R >> 3) & 1), and a reader that wants
+// chunk c of row R reads slot c ^ f(R).  For the 16 consecutive rows that one quarter-wave reads,
+// (R & 1, c ^ f(R)) takes 16 different values, i.e. all 64 banks are hit once.
+//
+// LDS map: [A stage 0][A stage 1][B stage 0][B stage 1]; both stages of a fragment row are
+// reachable from one address register through the 16-bit instruction offset.
+//
+// Schedule per slab t (4 k-steps of MFMAs, fragments double buffered in registers):
+//   k-steps 0..2 : MFMAs | fragment reads of the next k-step
+//   wait for the loads of slab t+1, barrier (every wave is done reading slab t)
+//   issue the loads of slab t+2 into the stage slab t occupied
+//   k-step 3     : MFMAs | fragment reads of k-step 0 of slab t+1
+// so a slab has a whole slab of MFMA time to land.
+template <typename T, typename TO, int BM, int BN, int WM, int WN, int SM, int SN, bool SWIGLU>
+__global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_dma_kernel(GroupedArgs p) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    constexpr int NW = WM * WN;
+    constexpr int ES = (int)sizeof(T);
+    constexpr int TM = BM / WM / 32;
+    constexpr int TN = BN / WN / 32;
+    constexpr int NIA = BM / 8 / NW;  // load instructions per wave and slab, A rows
+    constexpr int NIB = BN / 8 / NW;
+    constexpr int HALF = BN / 2;
+    constexpr int A_STAGE = BM * 128;
+    constexpr int B_STAGE = BN * 128;
+    constexpr int B_BASE = 2 * A_STAGE;
+    static_assert(BM % (WM * 32) == 0 && BN % (WN * 32) == 0, "wave tiling");
+    static_assert(BM % (8 * NW) == 0 && BN % (8 * NW) == 0 && NW % 2 == 0, "loader tiling");
+    static_assert(!SWIGLU || TN % 2 == 0, "SwiGLU needs gate and up tiles in the same wave");
+    static_assert(SM * SN == kSuperBlocks, "supertile");
+    static_assert(A_STAGE + (TM - 1) * 4096 + 128 <= 65536 && B_STAGE + (BN / 2 + 32 * TN) * 128 <= 65536, "offset field");
+
+    extern __shared__ __align__(16) unsigned char smem[];
+    typedef __attribute__((address_space(3))) void* lds_ptr_t;
+
+    TileCoord tc;
+    if (!decode_tile(blockIdx.x, p.row_count, p.E, BM, p.n_tiles, SM, SN, &tc)) return;
+    const int count = p.row_count[tc.e];
+    const int row0 = p.row_start[tc.e];
+    const int K = p.K;
+    const T* Bexp = static_cast<const T*>(p.b[tc.e]);
+    const T* A = static_cast<const T*>(p.a);
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / WN, wn = wave % WN;
+
+    // ---- load descriptors and lane offsets: instruction j of this wave covers rows (j*NW + wave)*8 .. +8
+    constexpr int kRsrcFlags = 0x00020000;  // raw buffer, 32-bit data format
+    const bool gather = p.a_rows != nullptr;
+    // without a gather the A descriptor starts at the tile's first row, so lane offsets stay small
+    const T* a_base = gather ? A : A + ((int64_t)row0 + (int64_t)tc.mt * BM) * p.lda;
+    const __amdgpu_buffer_rsrc_t rsrc_a =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(a_base), 0, (int)p.a_extent_bytes, kRsrcFlags);
+    const __amdgpu_buffer_rsrc_t rsrc_b =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(Bexp), 0, (int)p.b_extent_bytes, kRsrcFlags);
+    const int drow = lane >> 3;                         // row inside the 8-row group
+    const int dchunk = (lane & 7) ^ drow ^ (wave & 1);  // global chunk that lands in slot lane&7
+    unsigned ao[NIA], bo[NIB];
+#pragma unroll
+    for (int j = 0; j < NIA; ++j) {
+        int m = tc.mt * BM + (j * NW + wave) * 8 + drow;
+        m = m < count ? m : count - 1;
+        int64_t src = gather ? (int64_t)(p.a_rows[row0 + m] / p.a_row_div) : (int64_t)(m - tc.mt * BM);
+        ao[j] = (unsigned)(src * p.lda * ES + dchunk * 16);
+    }
+#pragma unroll
+    for (int j = 0; j < NIB; ++j) {
+        const int rb = (j * NW + wave) * 8 + drow;
+        int n, brow;
+        if (SWIGLU) {
+            const bool up = rb >= HALF;
+            n = tc.nt * HALF + (up ? rb - HALF : rb);
+            n = n < p.N_out ? n : p.N_out - 1;
+            brow = up ? p.up_offset + n : n;
+        } else {
+            n = tc.nt * BN + rb;
+            n = n < p.N_out ? n : p.N_out - 1;
+            brow = n;
+        }
+        bo[j] = (unsigned)((int64_t)brow * K * ES + dchunk * 16);
+    }
+    unsigned char* const dma_a = smem + wave * 1024;           // + stage*A_STAGE + j*NW*1024
+    unsigned char* const dma_b = smem + B_BASE + wave * 1024;  // + stage*B_STAGE + j*NW*1024
+
+    f32x16_t acc[TN][TM];
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[j][i][v] = 0.f;
+
+    const int nk = K * ES / 128;
+
+    // ---- fragment addresses: one register per k-step and operand; rows and stages by offset
+    const int frow = lane & 31;
+    const int fgrp = lane >> 5;
+    const int fsw = fgrp ^ (frow & 7) ^ ((frow >> 3) & 1);
+    const unsigned char* fa_addr[4];
+    const unsigned char* fb_addr[4];
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+        const int slot = (2 * ks) ^ fsw;
+        fa_addr[ks] = smem + (wm * (BM / WM) + frow) * 128 + slot * 16;
+        fb_addr[ks] = smem + B_BASE + (wn * (SWIGLU ? BN / WN / 2 : BN / WN) + frow) * 128 + slot * 16;
+    }
+    u32x4_t fa[2][TM], fb[2][TN];
+
+#define DM_ISSUE(kt_, stage_)                                                                          \
+    {                                                                                                  \
+        const int soff = (kt_) * 128;                                                                  \
+        _Pragma("unroll") for (int j = 0; j < NIA; ++j)                                                \
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(                                                  \
+                rsrc_a, (lds_ptr_t)(dma_a + (stage_) * A_STAGE + j * NW * 1024), 16, ao[j], soff, 0, 0); \
+        _Pragma("unroll") for (int j = 0; j < NIB; ++j)                                                \
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(                                                  \
+                rsrc_b, (lds_ptr_t)(dma_b + (stage_) * B_STAGE + j * NW * 1024), 16, bo[j], soff, 0, 0); \
+    }
+#define DM_B_ROW(j_) (SWIGLU ? ((j_) < TN / 2 ? (j_) * 32 : HALF + ((j_) - TN / 2) * 32) : (j_) * 32)
+// Read order = use order of the MFMAs (weight fragment 0, all activation fragments, then the
+// other weight fragments), so the first MFMAs of the next k-step wait for few reads.
+#define DM_READ(stage_, ks_, buf_)                                                                     \
+    {                                                                                                  \
+        fb[buf_][0] = *reinterpret_cast<const u32x4_t*>(fb_addr[ks_] + (stage_) * B_STAGE + DM_B_ROW(0) * 128); \
+        _Pragma("unroll") for (int i = 0; i < TM; ++i)                                                 \
+            fa[buf_][i] = *reinterpret_cast<const u32x4_t*>(fa_addr[ks_] + (stage_) * A_STAGE + i * 4096); \
+        _Pragma("unroll") for (int j = 1; j < TN; ++j)                                                 \
+            fb[buf_][j] = *reinterpret_cast<const u32x4_t*>(fb_addr[ks_] + (stage_) * B_STAGE + DM_B_ROW(j) * 128); \
+    }
+// k-step 3: the fragment reads go first (one per MFMA), the loads fill the remaining slots.
+#define DM_MIX_DMA()                                                                    \
+    _Pragma("unroll") for (int g_ = 0; g_ < (TM + TN); ++g_) {                          \
+        __builtin_amdgcn_sched_group_barrier(SG_DS_RD, 1, 0);                           \
+        __builtin_amdgcn_sched_group_barrier(SG_MFMA, 1, 0);                            \
+        __builtin_amdgcn_sched_group_barrier(SG_VMEM, 1, 0);                            \
+    }                                                                                   \
+    _Pragma("unroll") for (int g_ = 0; g_ < TM * TN - (TM + TN); ++g_) {                \
+        __builtin_amdgcn_sched_group_barrier(SG_MFMA, 1, 0);                            \
+        __builtin_amdgcn_sched_group_barrier(SG_VMEM, 1, 0);                            \
+    }
+// STG: stage of slab kt (compile time).  Slabs past the end are clamped to the last one: their
+// loads land in a stage nobody reads again, which keeps the loop body free of special cases.
+#define DM_ITER(kt_, STG)                                                               \
+    {                                                                                   \
+        DM_READ(STG, 1, 1);                                                             \
+        PL_MMA(0);                                                                      \
+        PL_MIX_READS();                                                                 \
+        PL_FENCE();                                                                     \
+        DM_READ(STG, 2, 0);                                                             \
+        PL_MMA(1);                                                                      \
+        PL_MIX_READS();                                                                 \
+        PL_FENCE();                                                                     \
+        DM_READ(STG, 3, 1);                                                             \
+        PL_MMA(0);                                                                      \
+        PL_MIX_READS();                                                                 \
+        PL_FENCE();                                                                     \
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");        \
+        PL_FENCE();                                                                     \
+        DM_READ(STG ^ 1, 0, 0);                                                         \
+        DM_ISSUE(min((kt_) + 2, nk - 1), STG);                                          \
+        PL_MMA(1);                                                                      \
+        DM_MIX_DMA();                                                                   \
+        PL_FENCE();                                                                     \
+    }
+
+    DM_ISSUE(0, 0);
+    DM_ISSUE(min(1, nk - 1), 1);
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(NIA + NIB) : "memory");
+    DM_READ(0, 0, 0);
+    int kt = 0;
+    for (; kt + 1 < nk; kt += 2) {
+        DM_ITER(kt, 0);
+        DM_ITER(kt + 1, 1);
+    }
+    if (kt < nk) DM_ITER(kt, 0);
+    // the clamped loads of the last slabs may still be in flight; the epilogue reuses LDS
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+#undef DM_ISSUE
+#undef DM_READ
+#undef DM_ITER
+#undef DM_B_ROW
+#undef DM_MIX_DMA
+
+    {
+        constexpr int TNO_ = SWIGLU ? TN / 2 : TN;
+        constexpr int WSTAGE = 32 * (TNO_ * 32 * (int)sizeof(TO) + 16);
+        const int wrow = tc.mt * BM + wm * (BM / WM);
+        const int ncol0 = SWIGLU ? tc.nt * HALF + wn * (BN / WN / 2) : tc.nt * BN + wn * (BN / WN);
+        epilogue_staged<TO, TM, TN, SWIGLU>(acc, smem + wave * WSTAGE, static_cast<TO*>(p.out), p.ldo,
+                                            (int64_t)row0 + wrow, count - wrow, ncol0, p.N_out, lane);
+    }
+#endif
+}
+
 #undef PL_STORE
 #undef PL_READ
 #undef PL_MMA
 #undef PL_FENCE
 #undef PL_MIX_READS
 
-template <typename T, typename TO, int BM, int BN, int WM, int WN, int SM, int SN, bool SWIGLU>
+template <typename T, typename TO, int BM, int BN, int WM, int WN, int SM, int SN, bool SWIGLU, bool DMA = false>
 static int launch_cfg(const GroupedArgs& p0, int64_t max_rows, hipStream_t s) {
     GroupedArgs p = p0;
     constexpr int n_per_tile = SWIGLU ? BN / 2 : BN;
     p.n_tiles = (p.N_out + n_per_tile - 1) / n_per_tile;
-    constexpr size_t smem = 2 * (size_t)(BM + BN) * kRowPitch;
+    constexpr size_t smem = 2 * (size_t)(BM + BN) * kRowPitch;  // covers the unpadded DMA layout too
     constexpr int BK = 128 / (int)sizeof(T);
     auto kern_general = grouped_gemm_kernel<T, TO, BM, BN, WM, WN, SM, SN, SWIGLU>;
-    auto kern_pipe = grouped_gemm_pipelined_kernel<T, TO, BM, BN, WM, WN, SM, SN, SWIGLU, (WM * WN <= 4)>;
+    auto kern_pipe = grouped_gemm_pipelined_kernel<T, TO, BM, BN, WM, WN, SM, SN, SWIGLU, true>;
+    auto kern_dma = [] {
+        if constexpr (DMA) return grouped_gemm_dma_kernel<T, TO, BM, BN, WM, WN, SM, SN, SWIGLU>;
+        else return grouped_gemm_pipelined_kernel<T, TO, BM, BN, WM, WN, SM, SN, SWIGLU, true>;
+    }();
     static bool attr_done = false;
     if (!attr_done) {
         if (smem > 64 * 1024) {
-            for (const void* k : {reinterpret_cast<const void*>(kern_general), reinterpret_cast<const void*>(kern_pipe)}) {
+            for (const void* k : {reinterpret_cast<const void*>(kern_general), reinterpret_cast<const void*>(kern_pipe),
+                                  reinterpret_cast<const void*>(kern_dma)}) {
                 hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
                 if (e != hipSuccess) {
                     set_error("grouped GEMM: cannot reserve %zu bytes of LDS: %s", smem, hipGetErrorString(e));
@@ -569,7 +782,9 @@ static int launch_cfg(const GroupedArgs& p0, int64_t max_rows, hipStream_t s) {
         set_error("grouped GEMM: grid of %lld blocks", (long long)blocks);
         return ATS_ERR_UNSUPPORTED;
     }
-    auto kern = (p.K % BK == 0) ? kern_pipe : kern_general;
+    // the direct-to-LDS kernel addresses its operands with 32-bit lane offsets
+    const bool dma_ok = DMA && p.K % BK == 0 && p.a_extent_bytes != 0 && p.b_extent_bytes != 0;
+    auto kern = dma_ok ? kern_dma : (p.K % BK == 0) ? kern_pipe : kern_general;
     hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(WM * WN * 64), smem, s, p);
     return ATS_OK;
 }
@@ -594,7 +809,13 @@ static int launch_grouped(const GroupedArgs& p, int64_t max_rows, hipStream_t s)
     }
     // Prefill: 256 x 256 tile, 8 waves (2 per SIMD: one wave's LDS / memory waits are covered by
     // the other's MFMAs), 128 accumulator registers per lane.
-    return launch_cfg<T, TO, 256, 256, 2, 4, 4, 8, SWIGLU>(p, max_rows, s);
+    return launch_cfg<T, TO, 256, 256, 2, 4, 4, 8, SWIGLU, true>(p, max_rows, s);
+}
+
+// Bytes reachable from a buffer descriptor, or 0 when they do not fit its 32-bit range.
+static uint32_t extent32(int64_t rows, int64_t row_elems, int elem_size) {
+    if (rows <= 0 || rows > (int64_t)0xffffffffLL / (row_elems * elem_size)) return 0;
+    return (uint32_t)(rows * row_elems * elem_size);
 }
 
 static int check_common(const char* name, const void* a, const void* const* w, const void* out,
@@ -613,14 +834,15 @@ static int check_common(const char* name, const void* a, const void* const* w, c
 
 }  // namespace ats
 
-extern "C" int ats_grouped_gateup_swiglu(const void* a, const int32_t* a_rows, int a_row_div,
+extern "C" int ats_grouped_gateup_swiglu(const void* a, int64_t a_num_rows, const int32_t* a_rows, int a_row_div,
                                          const void* const* w_gu, void* h, const int32_t* row_start,
                                          const int32_t* row_count, int E, int64_t max_rows, int H, int I, int dtype,
                                          ats_stream_t stream) {
     using namespace ats;
     int rc = check_common("ats_grouped_gateup_swiglu", a, w_gu, h, row_start, row_count, E, max_rows, H, I, dtype);
     if (rc != ATS_OK) return rc;
-    ATS_REQUIRE(!a_rows || a_row_div > 0, ATS_ERR_INVALID_ARG, "ats_grouped_gateup_swiglu: a_row_div=%d", a_row_div);
+    ATS_REQUIRE(!a_rows || (a_row_div > 0 && a_num_rows > 0), ATS_ERR_INVALID_ARG,
+                "ats_grouped_gateup_swiglu: a_row_div=%d a_num_rows=%lld", a_row_div, (long long)a_num_rows);
     if (max_rows == 0) return ATS_OK;
     GroupedArgs p{};
     p.a = a;
@@ -636,6 +858,9 @@ extern "C" int ats_grouped_gateup_swiglu(const void* a, const int32_t* a_rows, i
     p.K = H;
     p.N_out = I;
     p.up_offset = I;
+    const int es = dtype == ATS_F32 ? 4 : 2;
+    p.a_extent_bytes = a_rows ? extent32(a_num_rows, H, es) : 0xffffffffu;
+    p.b_extent_bytes = extent32(2 * (int64_t)I, H, es);
     hipStream_t s = as_stream(stream);
     rc = dtype == ATS_F32 ? launch_grouped<float, float, true>(p, max_rows, s)
                           : launch_grouped<bf16_t, bf16_t, true>(p, max_rows, s);
@@ -667,6 +892,8 @@ extern "C" int ats_grouped_down(const void* h, const void* const* w_d, void* y, 
     p.K = I;
     p.N_out = H;
     p.up_offset = 0;
+    p.a_extent_bytes = 0xffffffffu;
+    p.b_extent_bytes = extent32(H, I, dtype == ATS_F32 ? 4 : 2);
     hipStream_t s = as_stream(stream);
     if (dtype == ATS_F32) rc = launch_grouped<float, float, false>(p, max_rows, s);
     else if (y_dtype == ATS_F32) rc = launch_grouped<bf16_t, float, false>(p, max_rows, s);

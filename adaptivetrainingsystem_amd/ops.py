@@ -232,7 +232,7 @@ def grouped_gateup_swiglu(a: torch.Tensor, w_gu_ptrs: torch.Tensor, row_start: t
     if row_start.numel() < E or row_count.numel() < E or row_start.dtype != torch.int32 or row_count.dtype != torch.int32:
         raise AtsError("grouped_gateup_swiglu: row_start/row_count must be int32 with one entry per expert")
     h = torch.empty(n_rows_out, I, dtype=a.dtype, device=a.device)
-    check(_lib.load().ats_grouped_gateup_swiglu(a.data_ptr(), _ptr(a_rows), int(a_row_div), w_gu_ptrs.data_ptr(),
+    check(_lib.load().ats_grouped_gateup_swiglu(a.data_ptr(), int(a.shape[0]), _ptr(a_rows), int(a_row_div), w_gu_ptrs.data_ptr(),
                                                 h.data_ptr(), row_start.data_ptr(), row_count.data_ptr(), E,
                                                 int(max_rows), H, I, _tag(a), _stream()), "ats_grouped_gateup_swiglu")
     return h

@@ -135,12 +135,13 @@ int ats_invert_token_map(const int32_t* token_map, int64_t n_slots, int32_t* row
  * space (compact: row_start = offsets; padded [E,C,*]: row_start = e*C).
  * gate/up: h[r, i] = silu(a_r . w_gu[e][i,:]) * (a_r . w_gu[e][I+i,:]), where a_r
  * is row r of `a`, or row a_rows[r]/a_row_div of `a` when a_rows != NULL (the
- * permutation gather fused into the operand load).  w_gu / w_d are device
+ * permutation gather fused into the operand load; a_num_rows = rows of `a`, every
+ * gathered index must be below it; ignored when a_rows == NULL).  w_gu / w_d are device
  * arrays of E pointers to [2I,H] / [H,I] matrices.  h: [rows, I] of dtype;
  * down: y[r,:] = h[r,:] . w_d[e]^T, y of y_dtype (ATS_F32 or dtype).
  * max_rows bounds sum(row_count) (grid sizing only). */
-int ats_grouped_gateup_swiglu(const void* a, const int32_t* a_rows, int a_row_div,
-                              const void* const* w_gu, void* h, const int32_t* row_start,
+int ats_grouped_gateup_swiglu(const void* a, int64_t a_num_rows, const int32_t* a_rows,
+                              int a_row_div, const void* const* w_gu, void* h, const int32_t* row_start,
                               const int32_t* row_count, int E, int64_t max_rows, int H, int I,
                               int dtype, ats_stream_t stream);
 int ats_grouped_down(const void* h, const void* const* w_d, void* y, const int32_t* row_start,
