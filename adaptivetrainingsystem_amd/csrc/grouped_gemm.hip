@@ -31,10 +31,13 @@ typedef unsigned int u32x4_t __attribute__((ext_vector_type(4)));
 
 struct GroupedArgs {
     const void* a;           // [*, K] activations
+    const void* const* a_ptrs;  // optional: per expert A base; its rows are then counted from 0 (no row_start)
     const int32_t* a_rows;   // optional gather table over the row space
     int a_row_div;
     int64_t lda;             // elements
     const void* const* b;    // per expert weight [N_total, K]
+    int64_t ldb;             // elements between rows of b
+    const int32_t* k_count;  // optional: per expert K (a multiple of the K slab), overrides K
     void* out;               // [*, N_out]
     int64_t ldo;
     const int32_t* row_start;
@@ -187,7 +190,7 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_kernel(GroupedArgs p
             n = tc.nt * BN + rb;
             brow = n;
         }
-        bp[i] = n < p.N_out ? Bexp + (int64_t)brow * K + lchunk * VEC : nullptr;
+        bp[i] = n < p.N_out ? Bexp + (int64_t)brow * p.ldb + lchunk * VEC : nullptr;
     }
 
     f32x16_t acc[TN][TM];
@@ -314,9 +317,10 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_pipelined_kernel(Gro
     if (!decode_tile(blockIdx.x, p.row_count, p.E, BM, p.n_tiles, SM, SN, &tc)) return;
     const int count = p.row_count[tc.e];
     const int row0 = p.row_start[tc.e];
-    const int K = p.K;
+    const int K = p.k_count ? p.k_count[tc.e] : p.K;
     const T* Bexp = static_cast<const T*>(p.b[tc.e]);
-    const T* A = static_cast<const T*>(p.a);
+    const T* A = static_cast<const T*>(p.a_ptrs ? p.a_ptrs[tc.e] : p.a);
+    const int arow0 = p.a_ptrs ? 0 : row0;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -330,7 +334,7 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_pipelined_kernel(Gro
     for (int i = 0; i < PA; ++i) {
         int m = tc.mt * BM + lrow + i * RPP;
         m = m < count ? m : count - 1;
-        int64_t src = row0 + m;
+        int64_t src = arow0 + m;
         if (p.a_rows) src = p.a_rows[src] / p.a_row_div;
         ap[i] = A + src * p.lda + lchunk * VEC;
     }
@@ -349,7 +353,7 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_pipelined_kernel(Gro
             n = n < p.N_out ? n : p.N_out - 1;
             brow = n;
         }
-        bp[i] = Bexp + (int64_t)brow * K + lchunk * VEC;
+        bp[i] = Bexp + (int64_t)brow * p.ldb + lchunk * VEC;
     }
 
     // L2 warm-up: each thread touches one 128-byte line of a slab that the loaders will ask
@@ -361,7 +365,7 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_pipelined_kernel(Gro
     {
         int m = tc.mt * BM + tid % BM;
         m = m < count ? m : count - 1;
-        int64_t src = row0 + m;
+        int64_t src = arow0 + m;
         if (p.a_rows) src = p.a_rows[src] / p.a_row_div;
         apf = A + src * p.lda;
         const int rbp = tid % BN;
@@ -376,7 +380,7 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_pipelined_kernel(Gro
             n = n < p.N_out ? n : p.N_out - 1;
             brow = n;
         }
-        bpf = Bexp + (int64_t)brow * K;
+        bpf = Bexp + (int64_t)brow * p.ldb;
     }
     unsigned pfa[2] = {0u, 0u}, pfb[2] = {0u, 0u}, junk = 0u;
 
@@ -587,9 +591,10 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_dma_kernel(GroupedAr
     if (!decode_tile(blockIdx.x, p.row_count, p.E, BM, p.n_tiles, SM, SN, &tc)) return;
     const int count = p.row_count[tc.e];
     const int row0 = p.row_start[tc.e];
-    const int K = p.K;
+    const int K = p.k_count ? p.k_count[tc.e] : p.K;
     const T* Bexp = static_cast<const T*>(p.b[tc.e]);
-    const T* A = static_cast<const T*>(p.a);
+    const T* A = static_cast<const T*>(p.a_ptrs ? p.a_ptrs[tc.e] : p.a);
+    const int arow0 = p.a_ptrs ? 0 : row0;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -600,7 +605,7 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_dma_kernel(GroupedAr
     constexpr int kRsrcFlags = 0x00020000;  // raw buffer, 32-bit data format
     const bool gather = p.a_rows != nullptr;
     // without a gather the A descriptor starts at the tile's first row, so lane offsets stay small
-    const T* a_base = gather ? A : A + ((int64_t)row0 + (int64_t)tc.mt * BM) * p.lda;
+    const T* a_base = gather ? A : A + ((int64_t)arow0 + (int64_t)tc.mt * BM) * p.lda;
     const __amdgpu_buffer_rsrc_t rsrc_a =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(a_base), 0, (int)p.a_extent_bytes, kRsrcFlags);
     const __amdgpu_buffer_rsrc_t rsrc_b =
@@ -612,7 +617,7 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_dma_kernel(GroupedAr
     for (int j = 0; j < NIA; ++j) {
         int m = tc.mt * BM + (j * NW + wave) * 8 + drow;
         m = m < count ? m : count - 1;
-        int64_t src = gather ? (int64_t)(p.a_rows[row0 + m] / p.a_row_div) : (int64_t)(m - tc.mt * BM);
+        int64_t src = gather ? (int64_t)(p.a_rows[arow0 + m] / p.a_row_div) : (int64_t)(m - tc.mt * BM);
         ao[j] = (unsigned)(src * p.lda * ES + dchunk * 16);
     }
 #pragma unroll
@@ -629,7 +634,7 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_dma_kernel(GroupedAr
             n = n < p.N_out ? n : p.N_out - 1;
             brow = n;
         }
-        bo[j] = (unsigned)((int64_t)brow * K * ES + dchunk * 16);
+        bo[j] = (unsigned)((int64_t)brow * p.ldb * ES + dchunk * 16);
     }
     unsigned char* const dma_a = smem + wave * 1024;           // + stage*A_STAGE + j*NW*1024
     unsigned char* const dma_b = smem + B_BASE + wave * 1024;  // + stage*B_STAGE + j*NW*1024
@@ -850,6 +855,7 @@ extern "C" int ats_grouped_gateup_swiglu(const void* a, int64_t a_num_rows, cons
     p.a_row_div = a_rows ? a_row_div : 1;
     p.lda = H;
     p.b = w_gu;
+    p.ldb = H;
     p.out = h;
     p.ldo = I;
     p.row_start = row_start;
@@ -884,6 +890,7 @@ extern "C" int ats_grouped_down(const void* h, const void* const* w_d, void* y, 
     p.a_row_div = 1;
     p.lda = I;
     p.b = w_d;
+    p.ldb = I;
     p.out = y;
     p.ldo = H;
     p.row_start = row_start;
@@ -900,6 +907,63 @@ extern "C" int ats_grouped_down(const void* h, const void* const* w_d, void* y, 
     else rc = launch_grouped<bf16_t, bf16_t, false>(p, max_rows, s);
     if (rc != ATS_OK) return rc;
     ATS_CHECK_LAUNCH("ats_grouped_down");
+    return ATS_OK;
+}
+
+extern "C" int ats_grouped_gemm_nt(const void* a, const void* const* a_ptrs, int64_t lda, int64_t a_num_rows,
+                                   const int32_t* a_rows, int a_row_div, const void* const* b_ptrs, int64_t ldb,
+                                   int64_t b_rows, void* out, int64_t ldo, const int32_t* row_start,
+                                   const int32_t* row_count, const int32_t* k_count, int E, int64_t max_rows, int N,
+                                   int K, int dtype, int out_dtype, ats_stream_t stream) {
+    using namespace ats;
+    const char* name = "ats_grouped_gemm_nt";
+    ATS_REQUIRE(E > 0 && E <= 4096 && max_rows >= 0 && N > 0 && K > 0, ATS_ERR_INVALID_ARG,
+                "%s: E=%d max_rows=%lld N=%d K=%d", name, E, (long long)max_rows, N, K);
+    ATS_REQUIRE(dtype == ATS_F32 || dtype == ATS_BF16, ATS_ERR_UNSUPPORTED, "%s: dtype tag %d", name, dtype);
+    ATS_REQUIRE(out_dtype == ATS_F32 || out_dtype == dtype, ATS_ERR_UNSUPPORTED,
+                "%s: out dtype tag %d (float32 or the operand type)", name, out_dtype);
+    ATS_REQUIRE((a || a_ptrs) && b_ptrs && out && row_start && row_count, ATS_ERR_INVALID_ARG, "%s: null pointer", name);
+    ATS_REQUIRE(!(a_ptrs && a_rows), ATS_ERR_INVALID_ARG, "%s: a gather table needs a single A base", name);
+    ATS_REQUIRE(!a_rows || (a_row_div > 0 && a_num_rows > 0), ATS_ERR_INVALID_ARG, "%s: a_row_div=%d a_num_rows=%lld",
+                name, a_row_div, (long long)a_num_rows);
+    const int vec = dtype == ATS_F32 ? 4 : 8;
+    const int ovec = out_dtype == ATS_F32 ? 4 : 8;
+    ATS_REQUIRE(K % vec == 0 && lda % vec == 0 && ldb % vec == 0 && lda >= K && ldb >= K && N % ovec == 0 &&
+                    ldo % ovec == 0 && ldo >= N,
+                ATS_ERR_UNSUPPORTED, "%s: K=%d N=%d lda=%lld ldb=%lld ldo=%lld must describe 16-byte aligned rows", name, K, N,
+                (long long)lda, (long long)ldb, (long long)ldo);
+    ATS_REQUIRE((!a || aligned16(a)) && aligned16(out), ATS_ERR_INVALID_ARG, "%s: operands must be 16-byte aligned", name);
+    const int slab = dtype == ATS_F32 ? 32 : 64;
+    ATS_REQUIRE((!k_count && !a_ptrs) || K % slab == 0, ATS_ERR_UNSUPPORTED,
+                "%s: per-expert K / A bases need K to be a multiple of %d", name, slab);
+    if (max_rows == 0) return ATS_OK;
+    GroupedArgs p{};
+    p.a = a;
+    p.a_ptrs = a_ptrs;
+    p.a_rows = a_rows;
+    p.a_row_div = a_rows ? a_row_div : 1;
+    p.lda = lda;
+    p.b = b_ptrs;
+    p.ldb = ldb;
+    p.k_count = k_count;
+    p.out = out;
+    p.ldo = ldo;
+    p.row_start = row_start;
+    p.row_count = row_count;
+    p.E = E;
+    p.K = K;
+    p.N_out = N;
+    p.up_offset = 0;
+    const int es = dtype == ATS_F32 ? 4 : 2;
+    p.a_extent_bytes = a_rows ? extent32(a_num_rows, lda, es) : 0xffffffffu;
+    p.b_extent_bytes = extent32(b_rows > 0 ? b_rows : N, ldb, es);
+    hipStream_t s = as_stream(stream);
+    int rc;
+    if (dtype == ATS_F32) rc = launch_grouped<float, float, false>(p, max_rows, s);
+    else if (out_dtype == ATS_F32) rc = launch_grouped<bf16_t, float, false>(p, max_rows, s);
+    else rc = launch_grouped<bf16_t, bf16_t, false>(p, max_rows, s);
+    if (rc != ATS_OK) return rc;
+    ATS_CHECK_LAUNCH(name);
     return ATS_OK;
 }
 

@@ -127,6 +127,209 @@ static int launch_rmsnorm(const void* x, const void* w, void* y, int64_t rows, i
     return ATS_OK;
 }
 
+// ---------------------------------------------------------------- backward
+// y = x * r * w, r = rsqrt(mean(x^2) + eps).  With g = dy * w (dy alone when there is no weight):
+//   dx = r * g - x * r^3 * mean(g * x)          dw = sum over rows of dy * x * r
+// (RMSNormFunction.backward, cuda_opt_wrapper.py:119-142).  HBM-bound: x and dy are read once,
+// dx written once.  A wave keeps its slice of dw in registers over all the rows it processes;
+// the waves of a block add their slices in LDS in a fixed order and the block writes one
+// partial row; a second kernel adds the partial rows in index order (no atomics, so the result
+// does not depend on timing).
+template <typename T, typename WT, int NV, bool HAS_W, bool WREG>
+__global__ __launch_bounds__(256) void rmsnorm_bwd_rows_kernel(const T* __restrict__ x, const WT* __restrict__ w,
+                                                               const T* __restrict__ dy, T* __restrict__ dx,
+                                                               float* __restrict__ dw_partial, int64_t rows,
+                                                               int H, float eps) {
+    constexpr int V = Elem<T>::kVec;
+    extern __shared__ float dw_lds[];  // [H] when dw_partial != nullptr
+    const int lane = lane_id();
+    const int nvec = H / V;
+    const int wave_in_block = threadIdx.x >> 6;
+    const int64_t wave = (int64_t)blockIdx.x * (blockDim.x >> 6) + wave_in_block;
+    const int64_t nwaves = (int64_t)gridDim.x * (blockDim.x >> 6);
+
+    // the weight slice lives in registers unless the row is so long that registers run out;
+    // then it is re-read per row (it stays in the vector cache)
+    float wreg[WREG ? NV : 1][V];
+    float dwacc[NV][V];
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int v = lane + i * kWave;
+#pragma unroll
+        for (int j = 0; j < V; ++j) {
+            dwacc[i][j] = 0.f;
+            if (WREG) {
+                wreg[i][j] = 1.f;
+                if (HAS_W && v < nvec) wreg[i][j] = Elem<WT>::load(w + (int64_t)v * V + j);
+            }
+        }
+    }
+#define ATS_WVAL(i_, j_, v_) (!HAS_W ? 1.f : WREG ? wreg[WREG ? (i_) : 0][j_] : Elem<WT>::load(w + (int64_t)(v_) * V + (j_)))
+
+    for (int64_t row = wave; row < rows; row += nwaves) {
+        const uint4* xr = reinterpret_cast<const uint4*>(x + row * H);
+        const uint4* gr = reinterpret_cast<const uint4*>(dy + row * H);
+        uint4 xraw[NV], graw[NV];
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int v = lane + i * kWave;
+            if (v < nvec) {
+                xraw[i] = xr[v];
+                graw[i] = gr[v];
+            }
+        }
+        float ss = 0.f, dot = 0.f;
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int v = lane + i * kWave;
+            if (v < nvec) {
+                float xf[V], gf[V];
+                Elem<T>::unpack(xraw[i], xf);
+                Elem<T>::unpack(graw[i], gf);
+#pragma unroll
+                for (int j = 0; j < V; ++j) {
+                    ss += xf[j] * xf[j];
+                    dot += gf[j] * ATS_WVAL(i, j, v) * xf[j];
+                }
+            }
+        }
+        ss = wave_sum(ss);
+        dot = wave_sum(dot);
+        const float r = 1.0f / sqrtf(ss / (float)H + eps);
+        const float c = dot / (float)H * r * r * r;
+        uint4* dxr = reinterpret_cast<uint4*>(dx + row * H);
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int v = lane + i * kWave;
+            if (v < nvec) {
+                float xf[V], gf[V], o[V];
+                Elem<T>::unpack(xraw[i], xf);
+                Elem<T>::unpack(graw[i], gf);
+#pragma unroll
+                for (int j = 0; j < V; ++j) {
+                    o[j] = gf[j] * ATS_WVAL(i, j, v) * r - xf[j] * c;
+                    dwacc[i][j] += gf[j] * xf[j] * r;
+                }
+                dxr[v] = Elem<T>::pack(o);
+            }
+        }
+    }
+
+    if (dw_partial) {
+        for (int wv = 0; wv < (int)(blockDim.x >> 6); ++wv) {
+            if (wave_in_block == wv) {
+#pragma unroll
+                for (int i = 0; i < NV; ++i) {
+                    const int v = lane + i * kWave;
+                    if (v < nvec) {
+#pragma unroll
+                        for (int j = 0; j < V; ++j) {
+                            const int h = v * V + j;
+                            dw_lds[h] = (wv == 0 ? 0.f : dw_lds[h]) + dwacc[i][j];
+                        }
+                    }
+                }
+            }
+            __syncthreads();
+        }
+        for (int h = threadIdx.x; h < H; h += blockDim.x) dw_partial[(int64_t)blockIdx.x * H + h] = dw_lds[h];
+    }
+}
+#undef ATS_WVAL
+
+// Any hidden size / alignment: one wave per row, two scalar passes over the row; every wave owns
+// one partial row of dw in global memory and adds to it row after row.
+template <typename T, typename WT, bool HAS_W>
+__global__ __launch_bounds__(256) void rmsnorm_bwd_generic_kernel(const T* __restrict__ x, const WT* __restrict__ w,
+                                                                  const T* __restrict__ dy, T* __restrict__ dx,
+                                                                  float* __restrict__ dw_partial, int64_t rows,
+                                                                  int H, float eps) {
+    const int lane = lane_id();
+    const int64_t wave = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    const int64_t nwaves = (int64_t)gridDim.x * (blockDim.x >> 6);
+    float* mine = dw_partial ? dw_partial + wave * H : nullptr;
+    bool first = true;
+    for (int64_t row = wave; row < rows; row += nwaves) {
+        const T* xr = x + row * H;
+        const T* gr = dy + row * H;
+        float ss = 0.f, dot = 0.f;
+        for (int h = lane; h < H; h += kWave) {
+            const float xf = Elem<T>::load(xr + h);
+            const float wf = HAS_W ? Elem<WT>::load(w + h) : 1.f;
+            ss += xf * xf;
+            dot += Elem<T>::load(gr + h) * wf * xf;
+        }
+        ss = wave_sum(ss);
+        dot = wave_sum(dot);
+        const float r = 1.0f / sqrtf(ss / (float)H + eps);
+        const float c = dot / (float)H * r * r * r;
+        T* dxr = dx + row * H;
+        for (int h = lane; h < H; h += kWave) {
+            const float xf = Elem<T>::load(xr + h);
+            const float gf = Elem<T>::load(gr + h);
+            const float wf = HAS_W ? Elem<WT>::load(w + h) : 1.f;
+            Elem<T>::store(dxr + h, gf * wf * r - xf * c);
+            if (mine) mine[h] = (first ? 0.f : mine[h]) + gf * xf * r;
+        }
+        first = false;
+    }
+    if (mine && first)
+        for (int h = lane; h < H; h += kWave) mine[h] = 0.f;
+}
+
+__global__ __launch_bounds__(256) void rmsnorm_dw_reduce_kernel(const float* __restrict__ partial, int n_partial,
+                                                                float* __restrict__ dw, int H) {
+    const int h = blockIdx.x * blockDim.x + threadIdx.x;
+    if (h >= H) return;
+    float s = 0.f;
+    for (int b = 0; b < n_partial; ++b) s += partial[(int64_t)b * H + h];
+    dw[h] = s;
+}
+
+constexpr int kBwdBlocksVec = 512;      // vector kernel: 2 blocks per CU, one partial row per block
+constexpr int kBwdBlocksGeneric = 64;   // generic kernel: one partial row per wave (256 rows)
+
+static bool rmsnorm_bwd_vec_ok(const void* x, const void* dy, const void* dx, int H, int V) {
+    return (H % V == 0) && aligned16(x) && aligned16(dy) && aligned16(dx) && (H / V) <= 16 * kWave;
+}
+
+template <typename T, typename WT, bool HAS_W>
+static int launch_rmsnorm_bwd(const void* x, const void* w, const void* dy, void* dx, float* dw, float* partial,
+                              int64_t rows, int H, float eps, hipStream_t s) {
+    constexpr int V = Elem<T>::kVec;
+    const T* xp = static_cast<const T*>(x);
+    const WT* wp = static_cast<const WT*>(w);
+    const T* gp = static_cast<const T*>(dy);
+    T* dxp = static_cast<T*>(dx);
+    float* part = dw ? partial : nullptr;
+    int n_partial;
+    if (!rmsnorm_bwd_vec_ok(x, dy, dx, H, V)) {
+        const int64_t want = (rows + 3) / 4;
+        const int blocks = (int)(want < kBwdBlocksGeneric ? want : kBwdBlocksGeneric);
+        hipLaunchKernelGGL((rmsnorm_bwd_generic_kernel<T, WT, HAS_W>), dim3(blocks), dim3(256), 0, s, xp, wp, gp, dxp,
+                           part, rows, H, eps);
+        n_partial = blocks * 4;
+    } else {
+        const int64_t want = (rows + 3) / 4;
+        const int blocks = (int)(want < kBwdBlocksVec ? want : kBwdBlocksVec);
+        const size_t lds = part ? (size_t)H * sizeof(float) : 0;
+        const int per_lane = (H / V + kWave - 1) / kWave;
+#define ATS_RMSB_CASE(NV)                                                                                  \
+    hipLaunchKernelGGL((rmsnorm_bwd_rows_kernel<T, WT, NV, HAS_W, (NV * V <= 32)>), dim3(blocks), dim3(256), lds, \
+                       s, xp, wp, gp, dxp, part, rows, H, eps)
+        if (per_lane <= 1) ATS_RMSB_CASE(1);
+        else if (per_lane <= 2) ATS_RMSB_CASE(2);
+        else if (per_lane <= 4) ATS_RMSB_CASE(4);
+        else if (per_lane <= 8) ATS_RMSB_CASE(8);
+        else ATS_RMSB_CASE(16);
+#undef ATS_RMSB_CASE
+        n_partial = blocks;
+    }
+    if (dw)
+        hipLaunchKernelGGL(rmsnorm_dw_reduce_kernel, dim3((H + 255) / 256), dim3(256), 0, s, partial, n_partial, dw, H);
+    return ATS_OK;
+}
+
 }  // namespace ats
 
 extern "C" int ats_rmsnorm_fwd(const void* x, const void* w, void* y, int64_t rows, int hidden,
@@ -151,5 +354,46 @@ extern "C" int ats_rmsnorm_fwd(const void* x, const void* w, void* y, int64_t ro
     }
     if (rc != ATS_OK) return rc;
     ATS_CHECK_LAUNCH("ats_rmsnorm_fwd");
+    return ATS_OK;
+}
+
+extern "C" size_t ats_rmsnorm_bwd_workspace(int64_t rows, int hidden) {
+    (void)rows;
+    const size_t n = ats::kBwdBlocksVec > ats::kBwdBlocksGeneric * 4 ? ats::kBwdBlocksVec : ats::kBwdBlocksGeneric * 4;
+    return n * (size_t)(hidden > 0 ? hidden : 0) * sizeof(float);
+}
+
+extern "C" int ats_rmsnorm_bwd(const void* x, const void* w, const void* dy, void* dx, float* dw, int64_t rows,
+                               int hidden, float eps, int x_dtype, int w_dtype, void* workspace,
+                               size_t workspace_bytes, ats_stream_t stream) {
+    using namespace ats;
+    ATS_REQUIRE(rows >= 0 && hidden > 0, ATS_ERR_INVALID_ARG, "ats_rmsnorm_bwd: rows=%lld hidden=%d",
+                (long long)rows, hidden);
+    ATS_REQUIRE((x_dtype == ATS_F32 || x_dtype == ATS_BF16) && (w_dtype == ATS_F32 || w_dtype == ATS_BF16),
+                ATS_ERR_UNSUPPORTED, "ats_rmsnorm_bwd: dtype tags %d/%d", x_dtype, w_dtype);
+    hipStream_t s = as_stream(stream);
+    if (rows == 0) {
+        if (dw) hipLaunchKernelGGL(rmsnorm_dw_reduce_kernel, dim3((hidden + 255) / 256), dim3(256), 0, s, nullptr, 0, dw, hidden);
+        ATS_CHECK_LAUNCH("ats_rmsnorm_bwd");
+        return ATS_OK;
+    }
+    ATS_REQUIRE(x && dy && dx, ATS_ERR_INVALID_ARG, "ats_rmsnorm_bwd: null pointer");
+    ATS_REQUIRE(!dw || (workspace && workspace_bytes >= ats_rmsnorm_bwd_workspace(rows, hidden)), ATS_ERR_WORKSPACE,
+                "ats_rmsnorm_bwd: workspace of %zu bytes, need %zu", workspace_bytes,
+                ats_rmsnorm_bwd_workspace(rows, hidden));
+    ATS_REQUIRE(hidden <= 32768 || !dw, ATS_ERR_UNSUPPORTED, "ats_rmsnorm_bwd: hidden=%d", hidden);
+    float* part = static_cast<float*>(workspace);
+    int rc;
+    if (x_dtype == ATS_F32) {
+        if (!w) rc = launch_rmsnorm_bwd<float, float, false>(x, w, dy, dx, dw, part, rows, hidden, eps, s);
+        else if (w_dtype == ATS_F32) rc = launch_rmsnorm_bwd<float, float, true>(x, w, dy, dx, dw, part, rows, hidden, eps, s);
+        else rc = launch_rmsnorm_bwd<float, bf16_t, true>(x, w, dy, dx, dw, part, rows, hidden, eps, s);
+    } else {
+        if (!w) rc = launch_rmsnorm_bwd<bf16_t, float, false>(x, w, dy, dx, dw, part, rows, hidden, eps, s);
+        else if (w_dtype == ATS_F32) rc = launch_rmsnorm_bwd<bf16_t, float, true>(x, w, dy, dx, dw, part, rows, hidden, eps, s);
+        else rc = launch_rmsnorm_bwd<bf16_t, bf16_t, true>(x, w, dy, dx, dw, part, rows, hidden, eps, s);
+    }
+    if (rc != ATS_OK) return rc;
+    ATS_CHECK_LAUNCH("ats_rmsnorm_bwd");
     return ATS_OK;
 }

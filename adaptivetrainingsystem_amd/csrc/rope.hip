@@ -28,7 +28,8 @@ template <typename T>
 __global__ __launch_bounds__(256) void rope_vec_kernel(RopeSeg q, RopeSeg k, const float* __restrict__ cos_tab,
                                                        const float* __restrict__ sin_tab, int table_stride,
                                                        int L, int D, int pos_offset, int lanes_per_row,
-                                                       int pos_per_wave, int n_pos_groups, int64_t n_items, bool tab_vec) {
+                                                       int pos_per_wave, int n_pos_groups, int64_t n_items, bool tab_vec,
+                                                       float sin_sign) {
     constexpr int V = Elem<T>::kVec;
     const int lane = lane_id();
     const int64_t item = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
@@ -66,6 +67,8 @@ __global__ __launch_bounds__(256) void rope_vec_kernel(RopeSeg q, RopeSeg k, con
                 sn[j] = sp[j];
             }
         }
+#pragma unroll
+        for (int j = 0; j < V; ++j) sn[j] *= sin_sign;   // exact: +1 forward, -1 inverse rotation
     }
     const int h0 = chunk * kRopeHeadsPerItem;
     const T* in = static_cast<const T*>(seg.in);
@@ -103,7 +106,7 @@ __global__ __launch_bounds__(256) void rope_vec_kernel(RopeSeg q, RopeSeg k, con
 template <typename T>
 __global__ __launch_bounds__(256) void rope_scalar_kernel(RopeSeg q, RopeSeg k, const float* __restrict__ cos_tab,
                                                           const float* __restrict__ sin_tab, int table_stride,
-                                                          int B, int L, int D, int pos_offset) {
+                                                          int B, int L, int D, int pos_offset, float sin_sign) {
     const int half = D >> 1;
     const int64_t per_b = (int64_t)(q.heads + k.heads) * L * half;
     const int64_t total = per_b * B;
@@ -120,7 +123,7 @@ __global__ __launch_bounds__(256) void rope_scalar_kernel(RopeSeg q, RopeSeg k, 
         const T* p = static_cast<const T*>(seg.in) + b * seg.sb + h * seg.sh + pos * seg.sl + d;
         const float a = Elem<T>::load(p), bb = Elem<T>::load(p + half);
         const float cs = cos_tab[(int64_t)(pos_offset + pos) * table_stride + d];
-        const float sn = sin_tab[(int64_t)(pos_offset + pos) * table_stride + d];
+        const float sn = sin_tab[(int64_t)(pos_offset + pos) * table_stride + d] * sin_sign;
         T* o = static_cast<T*>(seg.out) + (((int64_t)b * seg.heads + h) * L + pos) * D + d;
         Elem<T>::store(o, ((((a) * (cs))) - (((bb) * (sn)))));
         Elem<T>::store(o + half, ((((a) * (sn))) + (((bb) * (cs)))));
@@ -153,7 +156,7 @@ __global__ __launch_bounds__(256) void rope_table_kernel(float* __restrict__ cos
 
 template <typename T>
 static void launch_rope(RopeSeg q, RopeSeg k, const float* cos_tab, const float* sin_tab, int table_stride, int B,
-                        int L, int D, int pos_offset, bool vec_ok, hipStream_t s) {
+                        int L, int D, int pos_offset, bool vec_ok, float sin_sign, hipStream_t s) {
     constexpr int V = Elem<T>::kVec;
     if (vec_ok) {
         const int lanes_per_row = (D / 2) / V;
@@ -163,13 +166,14 @@ static void launch_rope(RopeSeg q, RopeSeg k, const float* cos_tab, const float*
         const int64_t blocks = (n_items + 3) / 4;
         const bool tab_vec = table_stride % 4 == 0 && aligned16(cos_tab) && aligned16(sin_tab);
         hipLaunchKernelGGL((rope_vec_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, s, q, k, cos_tab, sin_tab,
-                           table_stride, L, D, pos_offset, lanes_per_row, pos_per_wave, n_pos_groups, n_items, tab_vec);
+                           table_stride, L, D, pos_offset, lanes_per_row, pos_per_wave, n_pos_groups, n_items, tab_vec,
+                           sin_sign);
     } else {
         const int64_t total = (int64_t)B * (q.heads + k.heads) * L * (D / 2);
         int64_t blocks = (total + 255) / 256;
         if (blocks > 65536) blocks = 65536;
         hipLaunchKernelGGL((rope_scalar_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, s, q, k, cos_tab, sin_tab,
-                           table_stride, B, L, D, pos_offset);
+                           table_stride, B, L, D, pos_offset, sin_sign);
     }
 }
 
@@ -193,21 +197,21 @@ extern "C" int ats_rope_table(float* cos_out, float* sin_out, int seq_len, int d
     return ATS_OK;
 }
 
-extern "C" int ats_rope_fwd(const void* q_in, const void* k_in, void* q_out, void* k_out, const float* cos_tab,
-                            const float* sin_tab, int table_stride, int table_len, int B, int Hq, int Hkv, int L,
-                            int D, int pos_offset, int64_t q_sb, int64_t q_sh, int64_t q_sl, int64_t k_sb,
-                            int64_t k_sh, int64_t k_sl, int dtype, ats_stream_t stream) {
+static int rope_apply(const char* name, float sin_sign, const void* q_in, const void* k_in, void* q_out, void* k_out,
+                      const float* cos_tab, const float* sin_tab, int table_stride, int table_len, int B, int Hq,
+                      int Hkv, int L, int D, int pos_offset, int64_t q_sb, int64_t q_sh, int64_t q_sl, int64_t k_sb,
+                      int64_t k_sh, int64_t k_sl, int dtype, ats_stream_t stream) {
     using namespace ats;
     ATS_REQUIRE(B >= 0 && Hq >= 0 && Hkv >= 0 && L >= 0 && D > 0 && D % 2 == 0, ATS_ERR_INVALID_ARG,
-                "ats_rope_fwd: B=%d Hq=%d Hkv=%d L=%d D=%d", B, Hq, Hkv, L, D);
-    ATS_REQUIRE(dtype == ATS_F32 || dtype == ATS_BF16, ATS_ERR_UNSUPPORTED, "ats_rope_fwd: dtype tag %d", dtype);
+                "%s: B=%d Hq=%d Hkv=%d L=%d D=%d", name, B, Hq, Hkv, L, D);
+    ATS_REQUIRE(dtype == ATS_F32 || dtype == ATS_BF16, ATS_ERR_UNSUPPORTED, "%s: dtype tag %d", name, dtype);
     if (B == 0 || L == 0 || Hq + Hkv == 0) return ATS_OK;
     ATS_REQUIRE(cos_tab && sin_tab && table_stride >= D / 2, ATS_ERR_INVALID_ARG,
-                "ats_rope_fwd: table pointers/stride (stride=%d, need >= %d)", table_stride, D / 2);
+                "%s: table pointers/stride (stride=%d, need >= %d)", name, table_stride, D / 2);
     ATS_REQUIRE(pos_offset >= 0 && (int64_t)pos_offset + L <= table_len, ATS_ERR_INVALID_ARG,
-                "ats_rope_fwd: positions %d..%d exceed table length %d", pos_offset, pos_offset + L - 1, table_len);
+                "%s: positions %d..%d exceed table length %d", name, pos_offset, pos_offset + L - 1, table_len);
     ATS_REQUIRE((Hq == 0 || (q_in && q_out)) && (Hkv == 0 || (k_in && k_out)), ATS_ERR_INVALID_ARG,
-                "ats_rope_fwd: null tensor pointer");
+                "%s: null tensor pointer", name);
     RopeSeg q{q_in, q_out, q_sb, q_sh, q_sl, Hq, (Hq + kRopeHeadsPerItem - 1) / kRopeHeadsPerItem};
     RopeSeg k{k_in, k_out, k_sb, k_sh, k_sl, Hkv, (Hkv + kRopeHeadsPerItem - 1) / kRopeHeadsPerItem};
     const int V = dtype == ATS_F32 ? 4 : 8;
@@ -218,9 +222,25 @@ extern "C" int ats_rope_fwd(const void* q_in, const void* k_in, void* q_out, voi
     const int half = D / 2;
     const bool vec_ok = half % V == 0 && half / V <= kWave && seg_ok(q) && seg_ok(k);
     if (dtype == ATS_F32)
-        launch_rope<float>(q, k, cos_tab, sin_tab, table_stride, B, L, D, pos_offset, vec_ok, as_stream(stream));
+        launch_rope<float>(q, k, cos_tab, sin_tab, table_stride, B, L, D, pos_offset, vec_ok, sin_sign, as_stream(stream));
     else
-        launch_rope<bf16_t>(q, k, cos_tab, sin_tab, table_stride, B, L, D, pos_offset, vec_ok, as_stream(stream));
-    ATS_CHECK_LAUNCH("ats_rope_fwd");
+        launch_rope<bf16_t>(q, k, cos_tab, sin_tab, table_stride, B, L, D, pos_offset, vec_ok, sin_sign, as_stream(stream));
+    ATS_CHECK_LAUNCH(name);
     return ATS_OK;
+}
+
+extern "C" int ats_rope_fwd(const void* q_in, const void* k_in, void* q_out, void* k_out, const float* cos_tab,
+                            const float* sin_tab, int table_stride, int table_len, int B, int Hq, int Hkv, int L,
+                            int D, int pos_offset, int64_t q_sb, int64_t q_sh, int64_t q_sl, int64_t k_sb,
+                            int64_t k_sh, int64_t k_sl, int dtype, ats_stream_t stream) {
+    return rope_apply("ats_rope_fwd", 1.0f, q_in, k_in, q_out, k_out, cos_tab, sin_tab, table_stride, table_len, B, Hq,
+                      Hkv, L, D, pos_offset, q_sb, q_sh, q_sl, k_sb, k_sh, k_sl, dtype, stream);
+}
+
+extern "C" int ats_rope_bwd(const void* dq_out, const void* dk_out, void* dq, void* dk, const float* cos_tab,
+                            const float* sin_tab, int table_stride, int table_len, int B, int Hq, int Hkv, int L,
+                            int D, int pos_offset, int64_t q_sb, int64_t q_sh, int64_t q_sl, int64_t k_sb,
+                            int64_t k_sh, int64_t k_sl, int dtype, ats_stream_t stream) {
+    return rope_apply("ats_rope_bwd", -1.0f, dq_out, dk_out, dq, dk, cos_tab, sin_tab, table_stride, table_len, B, Hq,
+                      Hkv, L, D, pos_offset, q_sb, q_sh, q_sl, k_sb, k_sh, k_sl, dtype, stream);
 }

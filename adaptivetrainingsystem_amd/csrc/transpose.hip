@@ -1,0 +1,154 @@
+// Transposes that put the contraction dimension innermost for the backward GEMMs (gfx950).
+// The grouped GEMM kernels multiply operands that are both contiguous along K ("NT").  The
+// backward pass needs   dX = dY . W   (contraction over W's rows)  and  dW = dY^T . X
+// (contraction over the token rows), so weights and activations are transposed once per step by
+// these HBM-bound kernels: 64 x 64 tiles through LDS, 16-byte accesses on both sides.
+//
+//   ats_transpose_batched      : E matrices [R, C] -> [C, R] (expert weights)
+//   ats_wgrad_plan             : per expert, the padded K extent and its first column
+//   ats_transpose_grouped_rows : rows [A, C] (optionally gathered) -> [C, ld_out]; the rows of expert
+//                                e become columns k_start[e] .. k_start[e] + k_count[e] - 1, zero padded
+#include "ats_common.hpp"
+
+namespace ats {
+
+constexpr int kTile = 64;
+constexpr int kKPad = 64;  // K granularity of the pipelined GEMM kernels (128 bytes of bf16)
+
+// tile[r][c] with a 2-element pad per row: LDS column reads hit different banks.
+template <typename T>
+__device__ __forceinline__ void transpose_tile(const T* __restrict__ in, int64_t ld_in, int rows_valid, int cols_valid,
+                                               const int32_t* __restrict__ gather, int gather_div,
+                                               T* __restrict__ out, int64_t ld_out, int out_cols_store, T* tile) {
+    // in: tile origin (row 0, col 0 of the tile) unless gather != nullptr, then in = matrix base + col offset
+    // and gather[i] / gather_div is the source row of tile row i.
+    constexpr int P = kTile + 2;
+    const int tid = threadIdx.x;
+    for (int i = tid; i < kTile * kTile; i += blockDim.x) {
+        const int r = i / kTile, c = i % kTile;
+        float v = 0.f;
+        if (r < rows_valid && c < cols_valid) {
+            const int64_t src = gather ? (int64_t)(gather[r] / gather_div) : (int64_t)r;
+            v = Elem<T>::load(in + src * ld_in + c);
+        }
+        Elem<T>::store(tile + r * P + c, v);
+    }
+    __syncthreads();
+    for (int i = tid; i < kTile * kTile; i += blockDim.x) {
+        const int c = i / kTile, r = i % kTile;  // out row = c (source column), out col = r (source row)
+        if (c < cols_valid && r < out_cols_store) out[(int64_t)c * ld_out + r] = tile[r * P + c];
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void transpose_batched_kernel(const void* const* __restrict__ in_ptrs,
+                                                                void* const* __restrict__ out_ptrs, int R, int C) {
+    __shared__ T tile[kTile * (kTile + 2)];
+    const int e = blockIdx.z;
+    const int r0 = blockIdx.y * kTile, c0 = blockIdx.x * kTile;
+    const T* in = static_cast<const T*>(in_ptrs[e]) + (int64_t)r0 * C + c0;
+    T* out = static_cast<T*>(out_ptrs[e]) + (int64_t)c0 * R + r0;
+    const int rv = R - r0 < kTile ? R - r0 : kTile;
+    const int cv = C - c0 < kTile ? C - c0 : kTile;
+    transpose_tile<T>(in, C, rv, cv, nullptr, 1, out, R, rv, tile);
+}
+
+__global__ void wgrad_plan_kernel(const int32_t* __restrict__ row_count, int E, int32_t* __restrict__ k_start,
+                                  int32_t* __restrict__ k_count) {
+    if (blockIdx.x != 0 || threadIdx.x != 0) return;
+    int acc = 0;
+    for (int e = 0; e < E; ++e) {
+        const int c = row_count[e];
+        const int kp = c <= 0 ? kKPad : (c + kKPad - 1) / kKPad * kKPad;
+        k_start[e] = acc;
+        k_count[e] = kp;
+        acc += kp;
+    }
+}
+
+// grid.x walks the padded row tiles of all experts (upper bound from max_rows), grid.y the column tiles.
+template <typename T>
+__global__ __launch_bounds__(256) void transpose_grouped_kernel(const T* __restrict__ in, int64_t ld_in, int C,
+                                                                const int32_t* __restrict__ gather, int gather_div,
+                                                                const int32_t* __restrict__ row_start,
+                                                                const int32_t* __restrict__ row_count, int E,
+                                                                T* __restrict__ out, int64_t ld_out) {
+    __shared__ T tile[kTile * (kTile + 2)];
+    int tile_id = blockIdx.x;
+    int e = 0, kstart = 0, kp = 0;
+    for (; e < E; ++e) {
+        const int c = row_count[e];
+        kp = c <= 0 ? kKPad : (c + kKPad - 1) / kKPad * kKPad;
+        const int nt = kp / kTile;
+        if (tile_id < nt) break;
+        tile_id -= nt;
+        kstart += kp;
+    }
+    if (e >= E) return;
+    const int i0 = tile_id * kTile;              // first local row of this tile inside expert e
+    const int count = row_count[e] > 0 ? row_count[e] : 0;
+    const int rv = count - i0 < 0 ? 0 : (count - i0 < kTile ? count - i0 : kTile);
+    const int c0 = blockIdx.y * kTile;
+    const int cv = C - c0 < kTile ? C - c0 : kTile;
+    const int64_t r0 = (int64_t)row_start[e] + i0;
+    const T* src = gather ? in + c0 : in + r0 * ld_in + c0;
+    transpose_tile<T>(src, ld_in, rv, cv, gather ? gather + r0 : nullptr, gather_div,
+                      out + (int64_t)c0 * ld_out + kstart + i0, ld_out, kTile, tile);
+}
+
+}  // namespace ats
+
+extern "C" int ats_transpose_batched(const void* const* in_ptrs, void* const* out_ptrs, int E, int R, int C, int dtype,
+                                     ats_stream_t stream) {
+    using namespace ats;
+    ATS_REQUIRE(E >= 0 && E <= 65535 && R > 0 && C > 0, ATS_ERR_INVALID_ARG, "ats_transpose_batched: E=%d R=%d C=%d", E, R, C);
+    ATS_REQUIRE(dtype == ATS_F32 || dtype == ATS_BF16, ATS_ERR_UNSUPPORTED, "ats_transpose_batched: dtype tag %d", dtype);
+    if (E == 0) return ATS_OK;
+    ATS_REQUIRE(in_ptrs && out_ptrs, ATS_ERR_INVALID_ARG, "ats_transpose_batched: null pointer");
+    const dim3 grid((unsigned)((C + kTile - 1) / kTile), (unsigned)((R + kTile - 1) / kTile), (unsigned)E);
+    ATS_REQUIRE(grid.y <= 65535, ATS_ERR_UNSUPPORTED, "ats_transpose_batched: R=%d", R);
+    if (dtype == ATS_F32)
+        hipLaunchKernelGGL((transpose_batched_kernel<float>), grid, dim3(256), 0, as_stream(stream), in_ptrs, out_ptrs, R, C);
+    else
+        hipLaunchKernelGGL((transpose_batched_kernel<bf16_t>), grid, dim3(256), 0, as_stream(stream), in_ptrs, out_ptrs, R, C);
+    ATS_CHECK_LAUNCH("ats_transpose_batched");
+    return ATS_OK;
+}
+
+extern "C" int64_t ats_wgrad_padded_rows(int64_t max_rows, int E) {
+    // upper bound of sum_e max(64, roundup(count_e, 64)) given sum_e count_e <= max_rows
+    return (max_rows + (int64_t)ats::kKPad * E + ats::kKPad - 1) / ats::kKPad * ats::kKPad;
+}
+
+extern "C" int ats_wgrad_plan(const int32_t* row_count, int E, int32_t* k_start, int32_t* k_count, ats_stream_t stream) {
+    using namespace ats;
+    ATS_REQUIRE(E > 0 && row_count && k_start && k_count, ATS_ERR_INVALID_ARG, "ats_wgrad_plan: E=%d or null pointer", E);
+    hipLaunchKernelGGL(wgrad_plan_kernel, dim3(1), dim3(64), 0, as_stream(stream), row_count, E, k_start, k_count);
+    ATS_CHECK_LAUNCH("ats_wgrad_plan");
+    return ATS_OK;
+}
+
+extern "C" int ats_transpose_grouped_rows(const void* in, int64_t ld_in, int C, const int32_t* gather, int gather_div,
+                                          const int32_t* row_start, const int32_t* row_count, int E, int64_t max_rows,
+                                          void* out, int64_t ld_out, int dtype, ats_stream_t stream) {
+    using namespace ats;
+    ATS_REQUIRE(E > 0 && C > 0 && max_rows >= 0 && ld_in >= C && ld_out >= ats_wgrad_padded_rows(max_rows, E),
+                ATS_ERR_INVALID_ARG, "ats_transpose_grouped_rows: E=%d C=%d max_rows=%lld ld_in=%lld ld_out=%lld", E, C,
+                (long long)max_rows, (long long)ld_in, (long long)ld_out);
+    ATS_REQUIRE(dtype == ATS_F32 || dtype == ATS_BF16, ATS_ERR_UNSUPPORTED, "ats_transpose_grouped_rows: dtype tag %d", dtype);
+    ATS_REQUIRE(in && row_start && row_count && out && (!gather || gather_div > 0), ATS_ERR_INVALID_ARG,
+                "ats_transpose_grouped_rows: null pointer");
+    const int64_t tiles = ats_wgrad_padded_rows(max_rows, E) / kTile;
+    const dim3 grid((unsigned)tiles, (unsigned)((C + kTile - 1) / kTile));
+    ATS_REQUIRE(tiles <= 0x7fffffffLL && grid.y <= 65535, ATS_ERR_UNSUPPORTED, "ats_transpose_grouped_rows: grid");
+    if (dtype == ATS_F32)
+        hipLaunchKernelGGL((transpose_grouped_kernel<float>), grid, dim3(256), 0, as_stream(stream),
+                           static_cast<const float*>(in), ld_in, C, gather, gather_div, row_start, row_count, E,
+                           static_cast<float*>(out), ld_out);
+    else
+        hipLaunchKernelGGL((transpose_grouped_kernel<bf16_t>), grid, dim3(256), 0, as_stream(stream),
+                           static_cast<const bf16_t*>(in), ld_in, C, gather, gather_div, row_start, row_count, E,
+                           static_cast<bf16_t*>(out), ld_out);
+    ATS_CHECK_LAUNCH("ats_transpose_grouped_rows");
+    return ATS_OK;
+}

@@ -77,9 +77,10 @@ def _bhl_strides(t: torch.Tensor):
 
 
 def rope(q: torch.Tensor, k: Optional[torch.Tensor], cos: torch.Tensor, sin: torch.Tensor,
-         position_offset: int = 0) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+         position_offset: int = 0, inverse: bool = False) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
     """q [B,Hq,L,D], k [B,Hkv,L,D] (any batch/head/position strides), cos/sin float32
-    [>= offset+L, D or D/2].  Returns new contiguous tensors."""
+    [>= offset+L, D or D/2].  Returns new contiguous tensors.  inverse=True applies the
+    inverse rotation, i.e. the gradient of the forward rotation."""
     _need_gpu(q, k, cos, sin)
     if q.dim() != 4 or (k is not None and k.dim() != 4):
         raise AtsError("rope: q and k must be [batch, heads, seq, head_dim]")
@@ -100,10 +101,10 @@ def rope(q: torch.Tensor, k: Optional[torch.Tensor], cos: torch.Tensor, sin: tor
     if k is not None:
         k, ksb, ksh, ksl = _bhl_strides(k)
         k_out = torch.empty((B, Hkv, L, D), dtype=k.dtype, device=k.device)
-    check(_lib.load().ats_rope_fwd(q.data_ptr(), _ptr(k), q_out.data_ptr(), _ptr(k_out), cos.data_ptr(),
-                                   sin.data_ptr(), cos.stride(0), cos.shape[0], B, Hq, Hkv, L, D,
-                                   int(position_offset), qsb, qsh, qsl, ksb, ksh, ksl, _tag(q), _stream()),
-          "ats_rope_fwd")
+    name = "ats_rope_bwd" if inverse else "ats_rope_fwd"
+    check(getattr(_lib.load(), name)(q.data_ptr(), _ptr(k), q_out.data_ptr(), _ptr(k_out), cos.data_ptr(),
+                                     sin.data_ptr(), cos.stride(0), cos.shape[0], B, Hq, Hkv, L, D,
+                                     int(position_offset), qsb, qsh, qsl, ksb, ksh, ksl, _tag(q), _stream()), name)
     return q_out, k_out
 
 
@@ -341,4 +342,211 @@ def swiglu_mul(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
     out = torch.empty_like(g)
     check(_lib.load().ats_swiglu_mul(g.data_ptr(), u.data_ptr(), out.data_ptr(), g.numel(), _tag(g), _stream()),
           "ats_swiglu_mul")
+    return out
+
+
+# --------------------------------------------------------------------------- backward pass
+def rmsnorm_bwd(x: torch.Tensor, weight: Optional[torch.Tensor], dy: torch.Tensor, eps: float = 1e-6,
+                need_dw: bool = True) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+    """Gradients of rmsnorm: dx (x's shape and dtype) and dw (float32 [H]) or None."""
+    _need_gpu(x, weight, dy)
+    H = x.shape[-1]
+    if dy.shape != x.shape or dy.dtype != x.dtype:
+        raise AtsError(f"rmsnorm_bwd: dy {tuple(dy.shape)}/{dy.dtype} does not match x {tuple(x.shape)}/{x.dtype}")
+    xc, dyc = x.contiguous(), dy.contiguous()
+    if weight is not None:
+        weight = weight.contiguous()
+    rows = xc.numel() // H if H else 0
+    dx = torch.empty_like(xc)
+    lib = _lib.load()
+    dw = ws = None
+    ws_bytes = 0
+    if need_dw and weight is not None:
+        dw = torch.empty(H, dtype=torch.float32, device=x.device)
+        ws_bytes = lib.ats_rmsnorm_bwd_workspace(rows, H)
+        ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=x.device)
+    check(lib.ats_rmsnorm_bwd(xc.data_ptr(), _ptr(weight), dyc.data_ptr(), dx.data_ptr(), _ptr(dw), rows, H,
+                              float(eps), _tag(xc), _tag(weight) if weight is not None else ATS_F32, _ptr(ws),
+                              ws_bytes, _stream()), "ats_rmsnorm_bwd")
+    return dx.view(x.shape), dw
+
+
+def _rows_2d(t: torch.Tensor, name: str) -> torch.Tensor:
+    if t.dim() != 2 or t.stride(1) != 1:
+        raise AtsError(f"{name}: operands must be 2-D with contiguous rows")
+    return t
+
+
+def silu_mul(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
+    """silu(a) * b for 2-D operands that may be column slices of a wider matrix."""
+    _need_gpu(a, b)
+    a, b = _rows_2d(a, "silu_mul"), _rows_2d(b, "silu_mul")
+    if a.shape != b.shape or a.dtype != b.dtype:
+        raise AtsError("silu_mul: operand shapes / dtypes differ")
+    out = torch.empty(a.shape, dtype=a.dtype, device=a.device)
+    check(_lib.load().ats_silu_mul_fwd(a.data_ptr(), a.stride(0), b.data_ptr(), b.stride(0), out.data_ptr(),
+                                       out.stride(0) if out.numel() else a.shape[1], a.shape[0], a.shape[1], _tag(a),
+                                       _stream()), "ats_silu_mul_fwd")
+    return out
+
+
+def silu_mul_bwd(a: torch.Tensor, b: torch.Tensor, dout: torch.Tensor, da: Optional[torch.Tensor] = None,
+                 db: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Gradients of silu(a) * b; da/db may be preallocated (e.g. the two halves of one matrix)."""
+    _need_gpu(a, b, dout, da, db)
+    a, b, dout = _rows_2d(a, "silu_mul_bwd"), _rows_2d(b, "silu_mul_bwd"), _rows_2d(dout, "silu_mul_bwd")
+    if a.shape != b.shape or a.shape != dout.shape or a.dtype != b.dtype or a.dtype != dout.dtype:
+        raise AtsError("silu_mul_bwd: operand shapes / dtypes differ")
+    if da is None:
+        da = torch.empty(a.shape, dtype=a.dtype, device=a.device)
+    if db is None:
+        db = torch.empty(a.shape, dtype=a.dtype, device=a.device)
+    da, db = _rows_2d(da, "silu_mul_bwd"), _rows_2d(db, "silu_mul_bwd")
+    cols = a.shape[1]
+    st = lambda t: t.stride(0) if t.shape[0] > 1 else max(t.stride(0), cols)
+    check(_lib.load().ats_silu_mul_bwd(a.data_ptr(), st(a), b.data_ptr(), st(b), dout.data_ptr(), st(dout),
+                                       da.data_ptr(), st(da), db.data_ptr(), st(db), a.shape[0], cols, _tag(a),
+                                       _stream()), "ats_silu_mul_bwd")
+    return da, db
+
+
+def combine_bwd(dout: torch.Tensor, y: torch.Tensor, token_map: torch.Tensor, w: torch.Tensor,
+                k: int) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Gradients of combine: dy (y's shape/dtype) and dw float32 [T, k]."""
+    _need_gpu(dout, y, token_map, w)
+    if dout.dim() != 2 or y.dim() != 2 or dout.shape[1] != y.shape[1] or token_map.dtype != torch.int32:
+        raise AtsError("combine_bwd: dout [T,H], y [rows,H], token_map int32 [rows]")
+    T, H = dout.shape
+    n_rows = y.shape[0]
+    if token_map.numel() < n_rows or w.numel() != T * k or w.dtype != torch.float32:
+        raise AtsError("combine_bwd: token_map / weights do not match the row and token counts")
+    dout, y, w = dout.contiguous(), y.contiguous(), w.contiguous()
+    dy = torch.empty_like(y)
+    dw = torch.empty(T, k, dtype=torch.float32, device=y.device)
+    check(_lib.load().ats_combine_bwd(dout.data_ptr(), y.data_ptr(), token_map.data_ptr(), w.data_ptr(), dy.data_ptr(),
+                                      dw.data_ptr(), n_rows, T, int(k), H, _tag(y), _tag(dout), _stream()),
+          "ats_combine_bwd")
+    return dy, dw
+
+
+def route_bwd(logits_route: torch.Tensor, idx: torch.Tensor, w: torch.Tensor, dw: torch.Tensor,
+              temperature: float = 1.0, mode: int = ROUTE_SOFTMAX_TOPK, logits_aux: Optional[torch.Tensor] = None,
+              usage: Optional[torch.Tensor] = None, aux_scale: float = 0.0) -> torch.Tensor:
+    """dlogits [T,E] float32 of the routing rule (and of the load-balancing loss when usage is given)."""
+    _need_gpu(logits_route, idx, w, dw, logits_aux, usage)
+    T, E = logits_route.shape
+    k = idx.shape[1]
+    if (logits_route.dtype != torch.float32 or idx.dtype != torch.int32 or w.dtype != torch.float32
+            or dw.dtype != torch.float32 or w.shape != idx.shape or dw.shape != idx.shape):
+        raise AtsError("route_bwd: logits float32 [T,E], idx int32 [T,k], w/dw float32 [T,k]")
+    logits_route, idx, w, dw = logits_route.contiguous(), idx.contiguous(), w.contiguous(), dw.contiguous()
+    if usage is not None:
+        usage = usage.contiguous().float()
+        logits_aux = (logits_route if logits_aux is None else logits_aux).contiguous()
+    out = torch.empty(T, E, dtype=torch.float32, device=logits_route.device)
+    check(_lib.load().ats_route_bwd(logits_route.data_ptr(), _ptr(logits_aux), idx.data_ptr(), w.data_ptr(),
+                                    dw.data_ptr(), _ptr(usage), float(aux_scale), float(temperature), int(mode),
+                                    out.data_ptr(), T, E, k, _stream()), "ats_route_bwd")
+    return out
+
+
+def router_bwd(dlogits: torch.Tensor, x: torch.Tensor, gate_weight: torch.Tensor,
+               base: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None,
+               need_dx: bool = True, need_dw: bool = True) -> Tuple[Optional[torch.Tensor], Optional[torch.Tensor]]:
+    """Gradients of router_logits: dx = base + dlogits @ Wg (x's dtype) and dWg float32 [E,H]."""
+    _need_gpu(dlogits, x, gate_weight, base, out)
+    T, H = x.shape
+    E = gate_weight.shape[0]
+    if dlogits.shape != (T, E) or dlogits.dtype != torch.float32 or gate_weight.dtype != x.dtype:
+        raise AtsError("router_bwd: dlogits float32 [T,E]; x and the gate weight share a dtype")
+    dlogits, xc, wg = dlogits.contiguous(), x.contiguous(), gate_weight.contiguous()
+    lib = _lib.load()
+    dx = dwg = None
+    if need_dx:
+        if base is not None:
+            base = base.contiguous()
+        dx = out if out is not None else torch.empty_like(xc)
+        check(lib.ats_router_bwd_dx(dlogits.data_ptr(), wg.data_ptr(), _ptr(base), dx.data_ptr(), T, E, H, _tag(xc),
+                                    _stream()), "ats_router_bwd_dx")
+    if need_dw:
+        dwg = torch.empty(E, H, dtype=torch.float32, device=x.device)
+        ws_bytes = lib.ats_router_bwd_dw_workspace(T, E, H)
+        ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=x.device)
+        check(lib.ats_router_bwd_dw(dlogits.data_ptr(), xc.data_ptr(), dwg.data_ptr(), T, E, H, _tag(xc),
+                                    ws.data_ptr(), ws_bytes, _stream()), "ats_router_bwd_dw")
+    return dx, dwg
+
+
+def transpose_batched(mats: Sequence[torch.Tensor]) -> Tuple[list, torch.Tensor]:
+    """Transposes E equally shaped contiguous matrices [R,C]; returns the list of [C,R] views of one
+    buffer and the device pointer table over them."""
+    _need_gpu(*mats)
+    R, C = mats[0].shape
+    for m in mats:
+        if m.shape != (R, C) or m.dtype != mats[0].dtype or not m.is_contiguous():
+            raise AtsError("transpose_batched: matrices must be contiguous and share shape and dtype")
+    E = len(mats)
+    buf = torch.empty(E, C, R, dtype=mats[0].dtype, device=mats[0].device)
+    outs = [buf[e] for e in range(E)]
+    in_tab = weight_pointer_table(list(mats))
+    out_tab = weight_pointer_table(outs)
+    check(_lib.load().ats_transpose_batched(in_tab.data_ptr(), out_tab.data_ptr(), E, R, C, _tag(mats[0]), _stream()),
+          "ats_transpose_batched")
+    return outs, out_tab
+
+
+def wgrad_plan(row_count: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Per expert: first column and padded width of its slice in the transposed activations."""
+    _need_gpu(row_count)
+    E = row_count.numel()
+    k_start = torch.empty(E, dtype=torch.int32, device=row_count.device)
+    k_count = torch.empty(E, dtype=torch.int32, device=row_count.device)
+    check(_lib.load().ats_wgrad_plan(row_count.data_ptr(), E, k_start.data_ptr(), k_count.data_ptr(), _stream()),
+          "ats_wgrad_plan")
+    return k_start, k_count
+
+
+def wgrad_padded_rows(max_rows: int, E: int) -> int:
+    return int(_lib.load().ats_wgrad_padded_rows(int(max_rows), int(E)))
+
+
+def transpose_grouped_rows(src: torch.Tensor, row_start: torch.Tensor, row_count: torch.Tensor, max_rows: int,
+                           gather: Optional[torch.Tensor] = None, gather_div: int = 1) -> torch.Tensor:
+    """[rows, C] -> [C, padded] with expert e in columns k_start[e] .. (see wgrad_plan), zero padded."""
+    _need_gpu(src, row_start, row_count, gather)
+    src = _rows_2d(src, "transpose_grouped_rows")
+    E = row_count.numel()
+    C = src.shape[1]
+    ld = wgrad_padded_rows(max_rows, E)
+    out = torch.empty(C, ld, dtype=src.dtype, device=src.device)
+    check(_lib.load().ats_transpose_grouped_rows(src.data_ptr(), src.stride(0), C, _ptr(gather), int(gather_div),
+                                                 row_start.data_ptr(), row_count.data_ptr(), E, int(max_rows),
+                                                 out.data_ptr(), ld, _tag(src), _stream()),
+          "ats_transpose_grouped_rows")
+    return out
+
+
+def grouped_gemm_nt(b_ptrs: torch.Tensor, ldb: int, b_rows: int, row_start: torch.Tensor, row_count: torch.Tensor,
+                    n_rows_out: int, max_rows: int, N: int, K: int, a: Optional[torch.Tensor] = None,
+                    a_ptrs: Optional[torch.Tensor] = None, lda: Optional[int] = None,
+                    a_rows: Optional[torch.Tensor] = None, a_row_div: int = 1, k_count: Optional[torch.Tensor] = None,
+                    dtype: Optional[torch.dtype] = None, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """out[row_start[e]+m, :N] = A_e[m, :K_e] @ B_e[:N, :K_e]^T (see ats_grouped_gemm_nt)."""
+    _need_gpu(a, a_ptrs, b_ptrs, row_start, row_count, a_rows, k_count)
+    if (a is None) == (a_ptrs is None):
+        raise AtsError("grouped_gemm_nt: give either a or a_ptrs")
+    if a is not None:
+        a = _rows_2d(a, "grouped_gemm_nt")
+        dtype = a.dtype
+        lda = a.stride(0)
+    elif dtype is None or lda is None:
+        raise AtsError("grouped_gemm_nt: a_ptrs needs dtype and lda")
+    out_dtype = dtype if out_dtype is None else out_dtype
+    E = b_ptrs.numel()
+    out = torch.empty(n_rows_out, N, dtype=out_dtype, device=b_ptrs.device)
+    check(_lib.load().ats_grouped_gemm_nt(_ptr(a), _ptr(a_ptrs), int(lda), int(a.shape[0]) if a is not None else 0,
+                                          _ptr(a_rows), int(a_row_div), b_ptrs.data_ptr(), int(ldb), int(b_rows),
+                                          out.data_ptr(), N, row_start.data_ptr(), row_count.data_ptr(), _ptr(k_count),
+                                          E, int(max_rows), int(N), int(K), _DT[dtype], _DT[out_dtype], _stream()),
+          "ats_grouped_gemm_nt")
     return out

@@ -183,6 +183,79 @@ int ats_kth_value_mask(const float* v, int64_t n, int64_t kth, float* mask, void
  * (cuda_opt_wrapper.py:476-478; note the convention differs from the experts'). */
 int ats_swiglu_mul(const void* gate, const void* up, void* out, int64_t n, int dtype, ats_stream_t stream);
 
+/* ---- Backward pass ---------------------------------------------------------
+ * The reference trains through this path with PyTorch autograd (model.py) and,
+ * for its fused ops, with explicit autograd Functions (cuda_opt_wrapper.py:85-254).
+ * These entry points are the gradients of the forward entry points above.
+ *
+ * RMSNormFunction.backward (cuda_opt_wrapper.py:119-142): with g = dy*w,
+ * r = rsqrt(mean(x^2)+eps):  dx = r*g - x*r^3*mean(g*x),  dw[h] = sum_rows dy*x*r
+ * (float32, fixed summation order).  dw may be NULL; otherwise workspace must hold
+ * ats_rmsnorm_bwd_workspace(rows, hidden) bytes. */
+size_t ats_rmsnorm_bwd_workspace(int64_t rows, int hidden);
+int ats_rmsnorm_bwd(const void* x, const void* w, const void* dy, void* dx, float* dw, int64_t rows,
+                    int hidden, float eps, int x_dtype, int w_dtype, void* workspace,
+                    size_t workspace_bytes, ats_stream_t stream);
+/* RoPEFunction.backward (cuda_opt_wrapper.py:180-207): the inverse rotation
+ * (sin negated); arguments as ats_rope_fwd with gradients in place of q/k. */
+int ats_rope_bwd(const void* dq_out, const void* dk_out, void* dq, void* dk, const float* cos_tab,
+                 const float* sin_tab, int table_stride, int table_len, int B, int Hq, int Hkv, int L,
+                 int D, int pos_offset, int64_t q_sb, int64_t q_sh, int64_t q_sl, int64_t k_sb,
+                 int64_t k_sh, int64_t k_sl, int dtype, ats_stream_t stream);
+/* out = silu(a) * b on row-strided [rows, cols] operands (strides in elements), and its
+ * gradient da = dout*b*(s + a*s*(1-s)), db = dout*a*s, s = sigmoid(a)
+ * (SwiGLUFunction.backward, cuda_opt_wrapper.py:237-254; SwiGLUExpert, model.py:1071-1088:
+ * a = gate half, b = up half of the [rows, 2I] projection). */
+int ats_silu_mul_fwd(const void* a, int64_t lda, const void* b, int64_t ldb, void* out, int64_t ldo,
+                     int64_t rows, int cols, int dtype, ats_stream_t stream);
+int ats_silu_mul_bwd(const void* a, int64_t lda, const void* b, int64_t ldb, const void* dout,
+                     int64_t ldd, void* da, int64_t ldda, void* db, int64_t lddb, int64_t rows,
+                     int cols, int dtype, ats_stream_t stream);
+/* Gradient of ats_combine: for expert row r with m = token_map[r] >= 0, t = m / k:
+ * dy[r,:] = w[m] * dout[t,:], dw[m] = dout[t,:] . y[r,:]; rows with m < 0 and the dw of
+ * dropped assignments are zero.  dw: [T*k] float32. */
+int ats_combine_bwd(const void* dout, const void* y, const int32_t* token_map, const float* w, void* dy,
+                    float* dw, int64_t n_rows, int64_t T, int k, int H, int y_dtype, int out_dtype,
+                    ats_stream_t stream);
+/* Gradient of the routing rule w.r.t. the router logits (mode 0: softmax -> top-k ->
+ * renormalise, model.py:1200-1217; mode 1: top-k -> softmax, moe_cuda_wrapper.py:229-233)
+ * plus, when usage != NULL, of the load-balancing loss (model.py:1244-1263) taken on
+ * logits_aux: aux_scale = dL/daux * E * load_balancing_weight / T, usage[e] as in the forward
+ * (treated as a constant).  logits_route are the logits the routing saw (with noise, if any). */
+int ats_route_bwd(const float* logits_route, const float* logits_aux, const int32_t* idx, const float* w,
+                  const float* dw, const float* usage, float aux_scale, float temperature, int mode,
+                  float* dlogits, int64_t T, int E, int k, ats_stream_t stream);
+/* Gradient of ats_router_logits: out[t,:] = base[t,:] + dlogits[t,:] . Wg (base NULL or == out),
+ * dWg[e,:] = sum_t dlogits[t,e] * x[t,:] (float32, fixed order). */
+int ats_router_bwd_dx(const float* dlogits, const void* wg, const void* base, void* out, int64_t T, int E,
+                      int H, int dtype, ats_stream_t stream);
+size_t ats_router_bwd_dw_workspace(int64_t T, int E, int H);
+int ats_router_bwd_dw(const float* dlogits, const void* x, float* dwg, int64_t T, int E, int H, int dtype,
+                      void* workspace, size_t workspace_bytes, ats_stream_t stream);
+/* Transposes that make the contraction dimension contiguous for the backward GEMMs:
+ * E matrices [R, C] -> [C, R]; and grouped rows [*, C] (row r of expert e, optionally
+ * gathered as in ats_grouped_gateup_swiglu) -> [C, ld_out] where expert e owns the columns
+ * k_start[e] .. k_start[e]+k_count[e]-1, k_count[e] = max(64, roundup(row_count[e], 64)),
+ * zero padded (ats_wgrad_plan writes k_start/k_count; ld_out >= ats_wgrad_padded_rows). */
+int ats_transpose_batched(const void* const* in_ptrs, void* const* out_ptrs, int E, int R, int C, int dtype,
+                          ats_stream_t stream);
+int64_t ats_wgrad_padded_rows(int64_t max_rows, int E);
+int ats_wgrad_plan(const int32_t* row_count, int E, int32_t* k_start, int32_t* k_count, ats_stream_t stream);
+int ats_transpose_grouped_rows(const void* in, int64_t ld_in, int C, const int32_t* gather, int gather_div,
+                               const int32_t* row_start, const int32_t* row_count, int E, int64_t max_rows,
+                               void* out, int64_t ld_out, int dtype, ats_stream_t stream);
+/* General grouped product with K contiguous in both operands:
+ * out[row_start[e]+m, n] = sum_k A_e[m,k] * B_e[n,k], m < row_count[e], n < N.
+ * A_e = rows row_start[e].. of `a` (optionally gathered through a_rows), or a_ptrs[e] with rows
+ * counted from 0; B_e = b_ptrs[e] ([b_rows >= N, ldb]); K_e = k_count[e] when given.
+ * Serves the training forward (gate/up pre-activations), dgrad (B = transposed weights)
+ * and wgrad (A, B = transposed activations, one "expert" per weight matrix). */
+int ats_grouped_gemm_nt(const void* a, const void* const* a_ptrs, int64_t lda, int64_t a_num_rows,
+                        const int32_t* a_rows, int a_row_div, const void* const* b_ptrs, int64_t ldb,
+                        int64_t b_rows, void* out, int64_t ldo, const int32_t* row_start,
+                        const int32_t* row_count, const int32_t* k_count, int E, int64_t max_rows, int N,
+                        int K, int dtype, int out_dtype, ats_stream_t stream);
+
 /* ---- Host-side views of the grouped-GEMM tile schedule (no device work) ----
  * No reference counterpart; used to test the block -> (expert, m-tile, n-tile)
  * map on the CPU.  row_count_host is a host array.  decode returns 1 and fills

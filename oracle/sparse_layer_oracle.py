@@ -43,6 +43,11 @@ PINNING = {
     "aux_loss": "uniform routing gives exactly load_balancing_weight; float64 closed form",
     "mod_router_eval_mask": "sorted-threshold brute force",
     "mod_select_per_sequence": "argsort brute force (composition defined by the benchmark config, not a reference function)",
+    "rmsnorm_backward": "torch.autograd of rmsnorm in float64; torch.autograd.gradcheck",
+    "rope_backward": "torch.autograd of rope_apply; R(p)^T = R(-p)",
+    "swiglu_backward": "torch.autograd of gate*silu(up) in float64; gradcheck",
+    "layer_grads": "is torch.autograd over the forward restatements above (what the reference itself trains with); "
+                   "gradcheck in float64 on the no-capacity layer with fixed routing",
 }
 
 
@@ -405,3 +410,54 @@ def mod_moe_block(x, mod_weight, mod_bias, keep, moe_kwargs):
     out[rows] += res["out"].reshape(-1, H)
     res.update({"block_out": out.reshape(B, L, H), "selected": sel, "scores": scores})
     return res
+
+
+# --------------------------------------------------------------------------- backward pass
+def rmsnorm_backward(x: torch.Tensor, weight: Optional[torch.Tensor], dy: torch.Tensor, eps: float = 1e-6):
+    """MS/core/cuda_opt_wrapper.py:119-142 (RMSNormFunction.backward), float32 math.
+    Returns (dx in x's dtype, dw float32 or None)."""
+    xf, gf = x.float().reshape(-1, x.shape[-1]), dy.float().reshape(-1, x.shape[-1])
+    hidden = xf.shape[-1]
+    rstd = torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps)
+    dw = (gf * xf * rstd).sum(0) if weight is not None else None
+    g = gf * weight.float().unsqueeze(0) if weight is not None else gf
+    gi = g * rstd
+    mean_grad = (gi * xf).sum(-1, keepdim=True) / hidden
+    dx = gi - xf * mean_grad * rstd.pow(2)
+    return dx.reshape(x.shape).to(x.dtype), dw
+
+
+def rope_backward(dq: torch.Tensor, dk: torch.Tensor, cos_half: torch.Tensor, sin_half: torch.Tensor,
+                  position_offset: int = 0):
+    """MS/core/cuda_opt_wrapper.py:180-207 (RoPEFunction.backward): inverse rotation."""
+    L = dq.shape[2]
+    pos = torch.arange(position_offset, position_offset + L)
+    def inv(g):
+        half = g.shape[-1] // 2
+        c = cos_half[pos][..., :half].float().unsqueeze(0).unsqueeze(0)
+        s = sin_half[pos][..., :half].float().unsqueeze(0).unsqueeze(0)
+        g1, g2 = g.float()[..., :half], g.float()[..., half:]
+        return torch.cat([g1 * c + g2 * s, -g1 * s + g2 * c], dim=-1).to(g.dtype)
+    return inv(dq), inv(dk)
+
+
+def swiglu_backward(gate: torch.Tensor, up: torch.Tensor, dout: torch.Tensor):
+    """MS/core/cuda_opt_wrapper.py:237-254 (SwiGLUFunction.backward; out = gate * silu(up))."""
+    g, u, d = gate.float(), up.float(), dout.float()
+    sig = torch.sigmoid(u)
+    dgate = d * (u * sig)
+    dup = d * g * (sig + u * sig * (1 - sig))
+    return dgate.to(gate.dtype), dup.to(up.dtype)
+
+
+def layer_grads(forward, tensors, cotangents):
+    """Gradients the reference obtains from PyTorch autograd (it trains the MoE layer through
+    MS/core/model.py with plain autograd): differentiates ``forward(*leaves)`` -- a callable built
+    from the forward restatements above that returns a tuple of tensors -- against ``cotangents``.
+    All leaves are float32 copies with requires_grad; returns the list of their gradients."""
+    leaves = [t.detach().float().clone().requires_grad_() for t in tensors]
+    outs = forward(*leaves)
+    if isinstance(outs, torch.Tensor):
+        outs = (outs,)
+    loss = sum((o.float() * c.float()).sum() for o, c in zip(outs, cotangents))
+    return list(torch.autograd.grad(loss, leaves, allow_unused=True))

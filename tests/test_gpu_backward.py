@@ -1,0 +1,269 @@
+"""Parity of the backward-pass kernels against the CPU oracle, through the C ABI.
+
+The oracle for a gradient is what the reference computes: its explicit backward formulas for the
+fused ops (restated in oracle/sparse_layer_oracle.py) and PyTorch autograd over the forward
+restatement for everything else.  Bars as for the forward pass: float32 within 1e-5 and bfloat16
+within 2e-2 of the oracle relative to its max-abs; the inverse rotation and the transposes are
+bit-exact; float32 GEMM gradients that contract over thousands of rows get 2e-5.
+"""
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import sparse_layer_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+F32_TOL = 1e-5
+BF16_TOL = 2e-2
+
+
+def rel_err(got, ref) -> float:
+    got, ref = got.detach().double().cpu(), ref.detach().double().cpu()
+    denom = ref.abs().max().item()
+    return (got - ref).abs().max().item() / (denom if denom > 0 else 1.0)
+
+
+def tol(dtype):
+    return F32_TOL if dtype == torch.float32 else BF16_TOL
+
+
+def gen(seed):
+    return torch.Generator().manual_seed(seed)
+
+
+@pytest.fixture(scope="module")
+def ops(gpu):
+    from adaptivetrainingsystem_amd import _lib, ops as _ops
+    _lib.load()
+    return _ops
+
+
+# ------------------------------------------------------------------ RMSNorm
+@pytest.mark.parametrize("shape", [(8, 512), (3, 5, 128), (7, 100), (300, 4096), (5, 8192), (3, 12000), (1, 8), (2, 6),
+                                   (1000, 2048)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_rmsnorm_bwd(ops, gpu, shape, dtype):
+    print("case rmsnorm_bwd", shape, dtype, flush=True)
+    g = gen(41)
+    x = torch.randn(*shape, generator=g).to(dtype)
+    dy = torch.randn(*shape, generator=g).to(dtype)
+    w = torch.randn(shape[-1], generator=g) * 0.2 + 1.0
+    dx_ref, dw_ref = O.rmsnorm_backward(x, w, dy, 1e-6)
+    dx, dw = ops.rmsnorm_bwd(x.to(gpu), w.to(gpu), dy.to(gpu), 1e-6)
+    assert dx.dtype == dtype and dx.shape == x.shape and dw.dtype == torch.float32
+    assert rel_err(dx, dx_ref) <= tol(dtype)
+    assert rel_err(dw, dw_ref) <= 2e-5          # float32 sums over the rows in a different order
+    dx2, dw2 = ops.rmsnorm_bwd(x.to(gpu), None, dy.to(gpu), 1e-6)
+    assert dw2 is None and rel_err(dx2, O.rmsnorm_backward(x, None, dy, 1e-6)[0]) <= tol(dtype)
+
+
+def test_rmsnorm_bwd_bf16_weight_and_empty(ops, gpu):
+    g = gen(42)
+    x = torch.randn(33, 256, generator=g).bfloat16()
+    dy = torch.randn(33, 256, generator=g).bfloat16()
+    w = (torch.randn(256, generator=g) * 0.2 + 1.0).bfloat16()
+    dx_ref, dw_ref = O.rmsnorm_backward(x, w, dy)
+    dx, dw = ops.rmsnorm_bwd(x.to(gpu), w.to(gpu), dy.to(gpu))
+    assert rel_err(dx, dx_ref) <= BF16_TOL and rel_err(dw, dw_ref) <= 2e-5
+    e = torch.empty(0, 64, device=gpu)
+    dx0, dw0 = ops.rmsnorm_bwd(e, torch.ones(64, device=gpu), e)
+    assert dx0.shape == (0, 64) and torch.equal(dw0.cpu(), torch.zeros(64))
+
+
+# ------------------------------------------------------------------ RoPE
+@pytest.mark.parametrize("B,Hq,Hkv,L,D", [(2, 4, 2, 9, 16), (1, 16, 4, 130, 128), (2, 3, 1, 33, 64), (1, 2, 2, 5, 6)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_rope_bwd_bit_exact(ops, gpu, B, Hq, Hkv, L, D, dtype):
+    print("case rope_bwd", B, Hq, Hkv, L, D, dtype, flush=True)
+    g = gen(43)
+    dq = torch.randn(B, Hq, L, D, generator=g).to(dtype)
+    dk = torch.randn(B, Hkv, L, D, generator=g).to(dtype)
+    cos, sin = ops.rope_table(L + 7, D, half=True, device=gpu)
+    rq, rk = O.rope_backward(dq, dk, cos.cpu(), sin.cpu(), position_offset=7)
+    gq, gk = ops.rope(dq.to(gpu), dk.to(gpu), cos, sin, position_offset=7, inverse=True)
+    assert torch.equal(gq.cpu(), rq) and torch.equal(gk.cpu(), rk)
+
+
+# ------------------------------------------------------------------ silu(a) * b
+@pytest.mark.parametrize("rows,cols", [(37, 1408), (5, 6), (300, 200), (1, 8), (0, 16)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_silu_mul_fwd_bwd_on_halves(ops, gpu, rows, cols, dtype):
+    print("case silu_mul", rows, cols, dtype, flush=True)
+    g = gen(44)
+    gu = (torch.randn(rows, 2 * cols, generator=g) * 2).to(dtype)
+    dh = torch.randn(rows, cols, generator=g).to(dtype)
+    a, b = gu[:, :cols].float().requires_grad_(), gu[:, cols:].float().requires_grad_()
+    h_ref = F.silu(a) * b
+    da_ref, db_ref = torch.autograd.grad((h_ref * dh.float()).sum(), [a, b]) if rows else (a.detach(), b.detach())
+    gud = gu.to(gpu)
+    h = ops.silu_mul(gud[:, :cols], gud[:, cols:])
+    assert h.shape == (rows, cols) and h.dtype == dtype
+    dgu = torch.empty_like(gud)
+    ops.silu_mul_bwd(gud[:, :cols], gud[:, cols:], dh.to(gpu), da=dgu[:, :cols], db=dgu[:, cols:])
+    if rows:
+        assert rel_err(h, h_ref) <= tol(dtype)
+        assert rel_err(dgu[:, :cols], da_ref) <= tol(dtype) and rel_err(dgu[:, cols:], db_ref) <= tol(dtype)
+        # the dense convention of the fused wrapper (gate * silu(up)) is the same kernel with the roles swapped
+        dg_ref, du_ref = O.swiglu_backward(gu[:, :cols], gu[:, cols:], dh)
+        du, dg = ops.silu_mul_bwd(gud[:, cols:].contiguous(), gud[:, :cols].contiguous(), dh.to(gpu))
+        assert rel_err(dg, dg_ref) <= tol(dtype) and rel_err(du, du_ref) <= tol(dtype)
+
+
+# ------------------------------------------------------------------ combine
+@pytest.mark.parametrize("T,E,k,C,H", [(64, 8, 2, 20, 128), (100, 4, 3, 60, 72), (512, 8, 2, 160, 512), (9, 4, 2, 2, 6)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_combine_bwd(ops, gpu, T, E, k, C, H, dtype):
+    print("case combine_bwd", T, E, k, C, H, dtype, flush=True)
+    g = gen(45)
+    idx = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)]).int()
+    _, token_map = O.dispatch_vectorized(torch.zeros(T, 1), idx, E, C)
+    w = torch.rand(T, k, generator=g)
+    y = torch.randn(E, C, H, generator=g).to(dtype)
+    dout = torch.randn(T, H, generator=g).to(dtype)
+    yl, wl = y.float().requires_grad_(), w.clone().requires_grad_()
+    out = O.combine_vectorized(yl, token_map, wl, T, k)
+    dy_ref, dw_ref = torch.autograd.grad((out * dout.float()).sum(), [yl, wl])
+    dy, dw = ops.combine_bwd(dout.to(gpu), y.reshape(E * C, H).to(gpu), token_map.reshape(-1).int().to(gpu),
+                             w.to(gpu), k)
+    assert rel_err(dy, dy_ref.reshape(E * C, H)) <= tol(dtype)
+    assert rel_err(dw, dw_ref) <= (2e-5 if dtype == torch.float32 else BF16_TOL)
+    dropped = torch.ones(T * k, dtype=torch.bool)
+    dropped[token_map.reshape(-1)[token_map.reshape(-1) >= 0].long()] = False
+    assert torch.equal(dw.cpu().reshape(-1)[dropped], torch.zeros(int(dropped.sum())))
+
+
+# ------------------------------------------------------------------ routing
+@pytest.mark.parametrize("T,E,k,temp", [(300, 8, 2, 1.0), (64, 64, 6, 1.0), (50, 4, 1, 0.7), (129, 128, 4, 1.3)])
+@pytest.mark.parametrize("mode", [0, 1])
+def test_route_bwd(ops, gpu, T, E, k, temp, mode):
+    print("case route_bwd", T, E, k, temp, mode, flush=True)
+    g = gen(46)
+    z = (torch.randn(T, E, generator=g) * 1.5).requires_grad_()
+    noise = torch.randn(T, E, generator=g) * 0.1
+    dw = torch.randn(T, k, generator=g)
+    route = O.route_softmax_topk_renorm if mode == 0 else O.route_topk_softmax
+    idx, w = route(z + noise, k, temp)
+    aux = O.aux_loss(z, idx, E, 0.01)
+    daux = 3.0
+    dz_ref, = torch.autograd.grad((w * dw).sum() + aux * daux, [z])
+    usage = torch.bincount(idx.reshape(-1), minlength=E).float() / (T * k + 1e-9)
+    dz = ops.route_bwd((z + noise).detach().to(gpu), idx.int().to(gpu), w.detach().to(gpu), dw.to(gpu), temp, mode,
+                       logits_aux=z.detach().to(gpu), usage=usage.to(gpu), aux_scale=daux * E * 0.01 / T)
+    # With k = 1 the renormalised weight is p / (p + 1e-9) = 1 up to rounding: its gradient is a
+    # difference of nearly equal float32 numbers (in autograd as well), so rounding noise of the order
+    # eps * |dw| / tau is added to the bar.
+    noise_floor = 2.5e-7 * dw.abs().max().item() / temp
+    err = (dz.cpu() - dz_ref).abs().max().item()
+    assert err <= 2e-5 * dz_ref.abs().max().item() + noise_floor
+    # without the auxiliary term
+    dz_ref2, = torch.autograd.grad((route(z + noise, k, temp)[1] * dw).sum(), [z])
+    dz2 = ops.route_bwd((z + noise).detach().to(gpu), idx.int().to(gpu), w.detach().to(gpu), dw.to(gpu), temp, mode)
+    assert (dz2.cpu() - dz_ref2).abs().max().item() <= 2e-5 * dz_ref2.abs().max().item() + noise_floor
+
+
+@pytest.mark.parametrize("T,H,E", [(512, 512, 8), (100, 1024, 64), (33, 40, 6), (1000, 2048, 128), (1, 64, 4)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_router_bwd(ops, gpu, T, H, E, dtype):
+    print("case router_bwd", T, H, E, dtype, flush=True)
+    g = gen(47)
+    x = torch.randn(T, H, generator=g).to(dtype)
+    wg = (torch.randn(E, H, generator=g) * 0.05).to(dtype)
+    dz = torch.randn(T, E, generator=g)
+    base = torch.randn(T, H, generator=g).to(dtype)
+    dx_ref = base.float() + dz @ wg.float()
+    dw_ref = dz.T @ x.float()
+    dx, dwg = ops.router_bwd(dz.to(gpu), x.to(gpu), wg.to(gpu), base=base.to(gpu))
+    assert dx.dtype == dtype and rel_err(dx, dx_ref) <= tol(dtype)
+    assert dwg.dtype == torch.float32 and rel_err(dwg, dw_ref) <= 2e-5
+    dx0, _ = ops.router_bwd(dz.to(gpu), x.to(gpu), wg.to(gpu), need_dw=False)
+    assert rel_err(dx0, dz @ wg.float()) <= tol(dtype)
+
+
+# ------------------------------------------------------------------ transposes
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_transposes_exact(ops, gpu, dtype):
+    g = gen(48)
+    mats = [torch.randn(100, 72, generator=g).to(dtype).to(gpu) for _ in range(3)]
+    outs, _ = ops.transpose_batched(mats)
+    for m, o in zip(mats, outs):
+        assert torch.equal(o, m.T)
+    counts = torch.tensor([70, 0, 129, 64], dtype=torch.int32)
+    starts = torch.tensor([0, 70, 70, 199], dtype=torch.int32)
+    A, C, E = 263, 40, 4
+    src = torch.randn(A, C, generator=g).to(dtype)
+    ks, kc = ops.wgrad_plan(counts.to(gpu))
+    assert kc.cpu().tolist() == [128, 64, 192, 64] and ks.cpu().tolist() == [0, 128, 192, 384]
+    out = ops.transpose_grouped_rows(src.to(gpu), starts.to(gpu), counts.to(gpu), A)
+    assert out.shape[0] == C and out.shape[1] >= 448 and out.shape[1] == ops.wgrad_padded_rows(A, E)
+    ref = torch.zeros(C, 448, dtype=dtype)
+    for e in range(E):
+        ref[:, ks[e]:ks[e] + counts[e]] = src[starts[e]:starts[e] + counts[e]].T
+    assert torch.equal(out[:, :448].cpu(), ref)
+    # gathered source rows (row = table // div)
+    big = torch.randn(500, C, generator=g).to(dtype)
+    table = (torch.randint(0, 500, (A,), generator=g) * 2 + 1).int()
+    out2 = ops.transpose_grouped_rows(big.to(gpu), starts.to(gpu), counts.to(gpu), A, gather=table.to(gpu), gather_div=2)
+    gathered = big[(table // 2).long()]
+    ref2 = torch.zeros(C, 448, dtype=dtype)
+    for e in range(E):
+        ref2[:, ks[e]:ks[e] + counts[e]] = gathered[starts[e]:starts[e] + counts[e]].T
+    assert torch.equal(out2[:, :448].cpu(), ref2)
+
+
+# ------------------------------------------------------------------ grouped GEMMs of the backward pass
+@pytest.mark.parametrize("counts,H,I", [([70, 0, 129, 64], 128, 72), ([900, 1100], 512, 256), ([30, 20, 10, 4], 64, 136)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_expert_ffn_gradients(ops, gpu, counts, H, I, dtype):
+    """gate/up pre-activation, dgrad and wgrad of the expert FFN against autograd on the oracle's expert."""
+    print("case ffn grads", counts, H, I, dtype, flush=True)
+    g = gen(49)
+    E, A = len(counts), sum(counts)
+    cnt = torch.tensor(counts, dtype=torch.int32)
+    start = torch.cumsum(cnt, 0).int() - cnt
+    xr = torch.randn(A, H, generator=g).to(dtype)
+    wgu = [(torch.randn(2 * I, H, generator=g) * 0.05).to(dtype) for _ in range(E)]
+    wd = [(torch.randn(H, I, generator=g) * 0.05).to(dtype) for _ in range(E)]
+    dy = torch.randn(A, H, generator=g).to(dtype)
+    # oracle: autograd over swiglu_expert per group (float32 math on the stored values)
+    leaves = [t.float().requires_grad_() for t in [xr] + wgu + wd]
+    ys = [O.swiglu_expert(leaves[0][start[e]:start[e] + counts[e]], leaves[1 + e], leaves[1 + E + e]) for e in range(E)]
+    grads = torch.autograd.grad((torch.cat(ys) * dy.float()).sum(), leaves, allow_unused=True)
+    dx_ref, dwgu_ref, dwd_ref = grads[0], grads[1:1 + E], grads[1 + E:]
+
+    d = lambda t: t.to(gpu)
+    xr_d, dy_d, cnt_d, start_d = d(xr), d(dy), d(cnt), d(start)
+    wgu_d, wd_d = [d(w) for w in wgu], [d(w) for w in wd]
+    tab_gu, tab_d = ops.weight_pointer_table(wgu_d), ops.weight_pointer_table(wd_d)
+    # forward with saved pre-activations
+    gu = ops.grouped_gemm_nt(tab_gu, H, 2 * I, start_d, cnt_d, A, A, 2 * I, H, a=xr_d)
+    h = ops.silu_mul(gu[:, :I], gu[:, I:])
+    y = ops.grouped_gemm_nt(tab_d, I, H, start_d, cnt_d, A, A, H, I, a=h)
+    assert rel_err(y, torch.cat(ys)) <= tol(dtype)
+    # dgrad
+    wdT, tab_dT = ops.transpose_batched(wd_d)          # [I, H] each
+    dh = ops.grouped_gemm_nt(tab_dT, H, I, start_d, cnt_d, A, A, I, H, a=dy_d)
+    dgu = torch.empty_like(gu)
+    ops.silu_mul_bwd(gu[:, :I], gu[:, I:], dh, da=dgu[:, :I], db=dgu[:, I:])
+    wguT, tab_guT = ops.transpose_batched(wgu_d)       # [H, 2I] each
+    dx = ops.grouped_gemm_nt(tab_guT, 2 * I, H, start_d, cnt_d, A, A, H, 2 * I, a=dgu)
+    assert rel_err(dx, dx_ref) <= tol(dtype)
+    # wgrad: one "expert" per weight matrix, K = padded rows of the expert
+    ks, kc = ops.wgrad_plan(cnt_d)
+    ld = ops.wgrad_padded_rows(A, E)
+    es = 4 if dtype == torch.float32 else 2
+    def wgrad(lhs, rhs, M, N):
+        lhsT = ops.transpose_grouped_rows(lhs, start_d, cnt_d, A)     # [M, ld]
+        rhsT = ops.transpose_grouped_rows(rhs, start_d, cnt_d, A)     # [N, ld]
+        a_ptrs = (ks.long() * es + lhsT.data_ptr())
+        b_ptrs = (ks.long() * es + rhsT.data_ptr())
+        rs = torch.arange(E, dtype=torch.int32, device=gpu) * M
+        rc = torch.full((E,), M, dtype=torch.int32, device=gpu)
+        out = ops.grouped_gemm_nt(b_ptrs, ld, N, rs, rc, E * M, E * M, N, ld, a_ptrs=a_ptrs, lda=ld, k_count=kc,
+                                  dtype=dtype, out_dtype=torch.float32)
+        return out.view(E, M, N)
+    dwd = wgrad(dy_d, h, H, I)
+    dwgu = wgrad(dgu, xr_d, 2 * I, H)
+    bar = 2e-5 if dtype == torch.float32 else BF16_TOL
+    assert rel_err(dwd, torch.stack(list(dwd_ref))) <= bar
+    assert rel_err(dwgu, torch.stack(list(dwgu_ref))) <= bar

@@ -298,6 +298,32 @@ def test_swiglu_expert_single_group(A, gpu, n, H, I, dtype):
     assert rel_err(got, ref) <= (F32_TOL if dtype == torch.float32 else BF16_TOL)
 
 
+def test_grouped_gateup_gather_small_and_huge_source(ops, gpu):
+    """The fused gather must give the same bits as a GEMM over pre-gathered rows, both when the
+    source fits 32-bit lane offsets (direct-to-LDS kernel) and when it does not (a 4.4 GB source
+    tensor, which selects the 64-bit-pointer kernel)."""
+    print("case gather paths", flush=True)
+    H, I, n = 512, 256, 1100
+    g = gen(23)
+    w = (torch.randn(2 * I, H, generator=g) * 0.05).bfloat16().to(gpu)
+    tab = ops.weight_pointer_table([w])
+    start = torch.zeros(1, dtype=torch.int32, device=gpu)
+    count = torch.full((1,), n, dtype=torch.int32, device=gpu)
+    rows_small = torch.randn(n, H, generator=g).bfloat16().to(gpu)
+    base = ops.grouped_gateup_swiglu(rows_small, tab, start, count, n, n, H, I)
+    ref = O.swiglu_expert(rows_small.cpu(), w.cpu(), torch.zeros(H, I, dtype=torch.bfloat16))  # shape check only
+    assert base.shape == (n, I) and ref.shape == (n, H)
+    for total_rows in (5000, 4_400_000):          # 5 MB and 4.5 GB of source rows
+        src = torch.empty(total_rows, H, dtype=torch.bfloat16, device=gpu)
+        idx = torch.randperm(n, generator=g).to(gpu) * (total_rows // n) + (total_rows // n - 1)
+        src[idx] = rows_small
+        k = 2
+        a_rows = (idx * k + 1).to(torch.int32)     # row index = a_rows // k
+        got = ops.grouped_gateup_swiglu(src, tab, start, count, n, n, H, I, a_rows=a_rows, a_row_div=k)
+        assert same_bits(got, base), f"gather from {total_rows} rows"
+        del src
+
+
 # ------------------------------------------------------------------ whole layer
 def _layer_vs_oracle(A, gpu, name, capacity_mode, routing, tol, scale_tokens=None, overrides=None, temperature=1.0):
     from adaptivetrainingsystem_amd import workloads as W

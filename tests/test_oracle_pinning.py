@@ -377,3 +377,95 @@ def test_mod_moe_block_skip_tokens_untouched():
     keep.scatter_(1, r["selected"], True)
     assert torch.equal(r["block_out"][~keep], x[~keep])
     assert torch.allclose(r["block_out"][keep] - x[keep], r["out"].reshape(-1, H), atol=1e-6)
+
+
+# --------------------------------------------------------------------------- backward restatements
+def test_rmsnorm_backward_matches_autograd_and_gradcheck():
+    g = torch.Generator().manual_seed(31)
+    x = torch.randn(7, 24, generator=g, dtype=torch.float64)
+    w = torch.randn(24, generator=g, dtype=torch.float64) * 0.3 + 1.0
+    dy = torch.randn(7, 24, generator=g, dtype=torch.float64)
+
+    def f64(xx, ww):     # float64 closed form of the forward (O.rmsnorm up-casts to float32 only)
+        return xx * torch.rsqrt(xx.pow(2).mean(-1, keepdim=True) + 1e-6) * ww
+
+    xr, wr = x.clone().requires_grad_(), w.clone().requires_grad_()
+    gx, gw = torch.autograd.grad((f64(xr, wr) * dy).sum(), [xr, wr])
+    dx, dw = O.rmsnorm_backward(x.float(), w.float(), dy.float())
+    assert torch.allclose(dx.double(), gx, rtol=2e-5, atol=2e-6)
+    assert torch.allclose(dw.double(), gw, rtol=2e-5, atol=2e-5)
+    assert torch.autograd.gradcheck(f64, (xr, wr), eps=1e-6, atol=1e-6)
+    # no weight: same formula with w = 1, dw is None
+    dx1, dw1 = O.rmsnorm_backward(x.float(), None, dy.float())
+    gx1, = torch.autograd.grad((f64(xr, torch.ones_like(w)) * dy).sum(), [xr])
+    assert dw1 is None and torch.allclose(dx1.double(), gx1, rtol=2e-5, atol=2e-6)
+
+
+def test_rope_backward_is_transpose_of_forward():
+    g = torch.Generator().manual_seed(32)
+    B, Hq, Hkv, L, D = 2, 3, 1, 9, 8
+    cos, sin = O.fused_rope_table(32, D)
+    q = torch.randn(B, Hq, L, D, generator=g).requires_grad_()
+    k = torch.randn(B, Hkv, L, D, generator=g).requires_grad_()
+    dq_o, dk_o = torch.randn(B, Hq, L, D, generator=g), torch.randn(B, Hkv, L, D, generator=g)
+    qo, ko = O.fused_rope_apply(q, k, cos, sin, position_offset=5)
+    gq, gk = torch.autograd.grad((qo * dq_o).sum() + (ko * dk_o).sum(), [q, k])
+    dq, dk = O.rope_backward(dq_o, dk_o, cos, sin, position_offset=5)
+    assert torch.allclose(dq, gq, rtol=1e-6, atol=1e-6) and torch.allclose(dk, gk, rtol=1e-6, atol=1e-6)
+    # rotating forward and then with the inverse returns the input
+    back_q, back_k = O.rope_backward(qo.detach(), ko.detach(), cos, sin, position_offset=5)
+    assert torch.allclose(back_q, q.detach(), atol=1e-5) and torch.allclose(back_k, k.detach(), atol=1e-5)
+
+
+def test_swiglu_backward_matches_autograd():
+    g = torch.Generator().manual_seed(33)
+    gate = torch.randn(5, 12, generator=g, dtype=torch.float64).requires_grad_()
+    up = (torch.randn(5, 12, generator=g, dtype=torch.float64) * 2).requires_grad_()
+    dout = torch.randn(5, 12, generator=g, dtype=torch.float64)
+    f = lambda a, b: a * torch.nn.functional.silu(b)
+    gg, gu = torch.autograd.grad((f(gate, up) * dout).sum(), [gate, up])
+    dg, du = O.swiglu_backward(gate.detach().float(), up.detach().float(), dout.float())
+    assert torch.allclose(dg.double(), gg, rtol=1e-5, atol=1e-6) and torch.allclose(du.double(), gu, rtol=1e-5, atol=1e-6)
+    assert torch.autograd.gradcheck(f, (gate, up), eps=1e-6, atol=1e-6)
+
+
+def test_layer_grads_gradcheck_fixed_routing():
+    """The layer's gradient oracle is autograd over the forward restatement; with the discrete routing
+    held fixed the forward is smooth, so float64 finite differences must agree with it."""
+    g = torch.Generator().manual_seed(34)
+    T, H, E, I, k = 6, 8, 3, 5, 2
+    x = torch.randn(T, H, generator=g, dtype=torch.float64).requires_grad_()
+    wg = (torch.randn(E, H, generator=g, dtype=torch.float64) * 0.5).requires_grad_()
+    wgu = (torch.randn(E, 2 * I, H, generator=g, dtype=torch.float64) * 0.3).requires_grad_()
+    wd = (torch.randn(E, H, I, generator=g, dtype=torch.float64) * 0.3).requires_grad_()
+    idx = torch.topk(torch.softmax(x.detach() @ wg.detach().T, -1), k, dim=-1).indices
+
+    def f(xx, wgg, wguu, wdd):
+        probs = torch.softmax(xx @ wgg.T, -1)
+        top = probs.gather(1, idx)
+        w = top / (top.sum(-1, keepdim=True) + 1e-9)
+        out = torch.zeros_like(xx)
+        for e in range(E):
+            for j in range(k):
+                m = idx[:, j] == e
+                gu = xx[m] @ wguu[e].T
+                h = torch.nn.functional.silu(gu[:, :I]) * gu[:, I:]
+                out[m] = out[m] + (h @ wdd[e].T) * w[m, j:j + 1]
+        return out
+
+    # the double-precision closed form equals the float32 oracle forward ...
+    ref = O.moe_forward_nocap(x.detach().float(), wg.detach().float(), [w_.float() for w_ in wgu.detach()],
+                              [w_.float() for w_ in wd.detach()], k)
+    assert torch.equal(ref["indices"], idx)
+    assert torch.allclose(ref["out"].double(), f(x, wg, wgu, wd).detach(), rtol=1e-4, atol=1e-5)
+    # ... and its autograd gradient passes the finite-difference check
+    assert torch.autograd.gradcheck(f, (x, wg, wgu, wd), eps=1e-6, atol=1e-5)
+    # layer_grads (autograd over the float32 oracle) agrees with autograd over the closed form
+    cot = torch.randn(T, H, generator=g, dtype=torch.float64)
+    g64 = torch.autograd.grad((f(x, wg, wgu, wd) * cot).sum(), [x, wg, wgu, wd])
+    got = O.layer_grads(lambda xx, wgg, *ws: O.moe_forward_nocap(xx, wgg, list(ws[:E]), list(ws[E:]), k)["out"],
+                        [x, wg] + list(wgu.detach()) + list(wd.detach()), [cot])
+    assert torch.allclose(got[0].double(), g64[0], rtol=1e-3, atol=1e-5)
+    assert torch.allclose(got[1].double(), g64[1], rtol=1e-3, atol=1e-5)
+    assert torch.allclose(torch.stack(got[2:2 + E]).double(), g64[2], rtol=1e-3, atol=1e-5)
+    assert torch.allclose(torch.stack(got[2 + E:]).double(), g64[3], rtol=1e-3, atol=1e-5)
