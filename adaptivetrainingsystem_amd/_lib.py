@@ -53,8 +53,8 @@ _SIGNATURES = {
                                  c_int64, c_int64, c_int, c_int, c_void_p]),
     "ats_combine_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int,
                                 c_int, c_int, c_int, c_void_p]),
-    "ats_route_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_float, c_int,
-                              c_void_p, c_int64, c_int, c_int, c_void_p]),
+    "ats_route_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_float,
+                              c_int, c_void_p, c_int64, c_int, c_int, c_void_p]),
     "ats_router_bwd_dx": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_void_p]),
     "ats_router_bwd_dw_workspace": (c_size_t, [c_int64, c_int, c_int]),
     "ats_router_bwd_dw": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_void_p, c_size_t,

@@ -1,0 +1,249 @@
+"""Autograd functions over the gfx950 kernels, so that a transformer block trains through the HIP
+path.  Every forward and backward step is a kernel of libats_gfx950; torch is used for tensor
+allocation, a handful of E-element scalar expressions and the autograd graph itself.
+
+Reference counterparts (MS = Src/Main_Scripts of the reference checkout):
+  RMSNormFunction / RoPEFunction / SwiGLUFunction   MS/core/cuda_opt_wrapper.py:85-254
+  MoE layer: the reference trains it through plain PyTorch autograd over MS/core/model.py:1160-1263
+  (noise on the routing logits in training mode, model.py:1203-1205; the auxiliary loss is taken on
+  the noise-free logits with the usage histogram as a constant, model.py:1190-1192, 1244-1263).
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+from torch.autograd import Function
+
+from . import ops
+from ._lib import ROUTE_SOFTMAX_TOPK, ROUTE_TOPK_SOFTMAX
+
+
+def _grad_to(g: Optional[torch.Tensor], like: torch.Tensor) -> Optional[torch.Tensor]:
+    if g is None:
+        return None
+    return g if g.dtype == like.dtype else g.to(like.dtype)
+
+
+class RMSNormFunction(Function):
+    @staticmethod
+    def forward(ctx, x, weight, eps):
+        ctx.save_for_backward(x, weight)
+        ctx.eps = eps
+        return ops.rmsnorm(x, weight, eps)
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, weight = ctx.saved_tensors
+        need_dw = weight is not None and ctx.needs_input_grad[1]
+        dx, dw = ops.rmsnorm_bwd(x, weight, dy.to(x.dtype), ctx.eps, need_dw=need_dw)
+        return dx, (_grad_to(dw, weight) if need_dw else None), None
+
+
+class RoPEFunction(Function):
+    @staticmethod
+    def forward(ctx, q, k, cos, sin, position_offset):
+        ctx.save_for_backward(cos, sin)
+        ctx.position_offset = position_offset
+        q_out, k_out = ops.rope(q, k, cos, sin, position_offset)
+        return q_out, k_out
+
+    @staticmethod
+    def backward(ctx, dq, dk):
+        cos, sin = ctx.saved_tensors
+        gq, gk = ops.rope(dq, dk, cos, sin, ctx.position_offset, inverse=True)
+        return gq, gk, None, None, None
+
+
+class SwiGLUFunction(Function):
+    """out = gate * silu(up) (the dense-FFN convention of the fused wrapper)."""
+
+    @staticmethod
+    def forward(ctx, gate, up):
+        shape = gate.shape
+        g2, u2 = gate.reshape(-1, shape[-1]).contiguous(), up.reshape(-1, shape[-1]).contiguous()
+        ctx.save_for_backward(g2, u2)
+        ctx.shape = shape
+        return ops.silu_mul(u2, g2).view(shape)
+
+    @staticmethod
+    def backward(ctx, dout):
+        g2, u2 = ctx.saved_tensors
+        d2 = dout.reshape(g2.shape).to(g2.dtype).contiguous()
+        du, dg = ops.silu_mul_bwd(u2, g2, d2)
+        return dg.view(ctx.shape), du.view(ctx.shape)
+
+
+def _ffn_forward(x, wgu, wd, offsets, kept, rows, row_src, k):
+    """Expert FFN over the grouped rows, keeping the gate/up pre-activations for the backward pass.
+    Returns (gu [rows, 2I], h [rows, I], y [rows, H])."""
+    H, I = x.shape[1], wd[0].shape[1]
+    tab_gu, tab_d = ops.weight_pointer_table(wgu), ops.weight_pointer_table(wd)
+    gu = ops.grouped_gemm_nt(tab_gu, H, 2 * I, offsets, kept, rows, rows, 2 * I, H, a=x, a_rows=row_src,
+                             a_row_div=k)
+    h = ops.silu_mul(gu[:, :I], gu[:, I:])
+    y = ops.grouped_down(h, tab_d, offsets, kept, rows, H, I)
+    return gu, h, y
+
+
+def _ffn_backward(dy, x, wgu, wd, gu, h, offsets, kept, rows, row_src, k, need_x, need_w):
+    """Gradients of _ffn_forward: dx_rows [rows, H] (or None), dWgu [E, 2I, H], dWd [E, H, I] (or None).
+    dgrad multiplies by per-step transposed copies of the weights; wgrad multiplies the transposed,
+    zero-padded activations of each expert (K = its padded row count)."""
+    E = len(wd)
+    H, I = x.shape[1], wd[0].shape[1]
+    dtype, dev = x.dtype, x.device
+    wdT, tab_dT = ops.transpose_batched(wd)                      # [I, H] per expert; kept alive until return
+    dh = ops.grouped_gemm_nt(tab_dT, H, I, offsets, kept, rows, rows, I, H, a=dy)
+    dgu = torch.empty_like(gu)
+    ops.silu_mul_bwd(gu[:, :I], gu[:, I:], dh, da=dgu[:, :I], db=dgu[:, I:])
+    dx_rows = dwgu = dwd = None
+    if need_x:
+        wguT, tab_guT = ops.transpose_batched(wgu)               # [H, 2I] per expert
+        dx_rows = ops.grouped_gemm_nt(tab_guT, 2 * I, H, offsets, kept, rows, rows, H, 2 * I, a=dgu)
+    if need_w:
+        ks, kc = ops.wgrad_plan(kept)
+        ld = ops.wgrad_padded_rows(rows, E)
+        es = x.element_size()
+
+        def wgrad(lhs, rhs, M, N, gather=None):
+            lhsT = ops.transpose_grouped_rows(lhs, offsets, kept, rows)
+            rhsT = ops.transpose_grouped_rows(rhs, offsets, kept, rows, gather=gather, gather_div=k)
+            a_ptrs = ks.long() * es + lhsT.data_ptr()
+            b_ptrs = ks.long() * es + rhsT.data_ptr()
+            rs = torch.arange(E, dtype=torch.int32, device=dev) * M
+            rc = torch.full((E,), M, dtype=torch.int32, device=dev)
+            g = ops.grouped_gemm_nt(b_ptrs, ld, N, rs, rc, E * M, E * M, N, ld, a_ptrs=a_ptrs, lda=ld, k_count=kc,
+                                    dtype=dtype, out_dtype=dtype)
+            return g.view(E, M, N)
+
+        dwd = wgrad(dy, h, H, I)
+        dwgu = wgrad(dgu, x, 2 * I, H, gather=row_src)
+    return dx_rows, dwgu, dwd
+
+
+class ExpertFFNFunction(Function):
+    """One SwiGLU expert over every row of x [n, H]: down(silu(gate) * up)."""
+
+    @staticmethod
+    def forward(ctx, x, w_gate_up, w_down):
+        dtype = x.dtype
+        x = x.contiguous()
+        wgu, wd = [w_gate_up.detach().to(dtype).contiguous()], [w_down.detach().to(dtype).contiguous()]
+        n = x.shape[0]
+        offsets = torch.tensor([0, n], dtype=torch.int32, device=x.device)
+        kept = offsets[1:].clone()
+        gu, h, y = _ffn_forward(x, wgu, wd, offsets, kept, n, None, 1)
+        ctx.save_for_backward(x, offsets, kept, gu, h)
+        ctx.wgu, ctx.wd = wgu, wd
+        ctx.param_dtypes = (w_gate_up.dtype, w_down.dtype)
+        return y
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, offsets, kept, gu, h = ctx.saved_tensors
+        need_x, need_w = ctx.needs_input_grad[0], ctx.needs_input_grad[1] or ctx.needs_input_grad[2]
+        dx, dwgu, dwd = _ffn_backward(dy.to(x.dtype).contiguous(), x, ctx.wgu, ctx.wd, gu, h, offsets, kept,
+                                      x.shape[0], None, 1, need_x, need_w)
+        return (dx, dwgu[0].to(ctx.param_dtypes[0]) if need_w else None,
+                dwd[0].to(ctx.param_dtypes[1]) if need_w else None)
+
+
+class MoEFunction(Function):
+    """The whole MoE FFN layer on [T, H] tokens.  apply(x, gate_weight, cfg, *expert_weights) with
+    expert_weights = E gate/up matrices [2I, H] followed by E down matrices [H, I]; cfg is a dict:
+    top_k, temperature, variant, capacity (C, or T for no dropping), load_balancing_weight,
+    noise_std (0 in eval), logit_bias (tensor or None), stats (dict filled with the plan).
+    Returns (out [T, H], aux scalar)."""
+
+    @staticmethod
+    def forward(ctx, x, gate_weight, cfg, *expert_weights):
+        E = len(expert_weights) // 2
+        k, C = cfg["top_k"], cfg["capacity"]
+        T, H = x.shape
+        dtype = x.dtype
+        wg = gate_weight.detach().to(dtype).contiguous()
+        wgu = [w.detach().to(dtype).contiguous() for w in expert_weights[:E]]
+        wd = [w.detach().to(dtype).contiguous() for w in expert_weights[E:]]
+        I = wd[0].shape[1]
+        x = x.contiguous()
+
+        logits = ops.router_logits(x, wg, cfg.get("logit_bias"))
+        logits_route = logits
+        if cfg.get("noise_std", 0.0) > 0:
+            logits_route = logits + torch.randn_like(logits) * cfg["noise_std"]
+        route = ops.route_topk(logits_route, k, cfg["temperature"], cfg["variant"], cfg["load_balancing_weight"])
+        usage = route["hist"].float() / (T * k + 1e-9)
+        if logits_route is logits:
+            aux = route["aux"][0]
+        else:   # importance from the noise-free logits (model.py:1190-1192)
+            colsum = ops.route_topk(logits, k, 1.0, cfg["variant"], cfg["load_balancing_weight"])["prob_colsum"]
+            aux = torch.clamp((usage * (colsum / T)).sum() * (E * cfg["load_balancing_weight"]), max=1.0)
+        plan = ops.dispatch_plan(route["indices"], E, C)
+        rows = min(T * k, E * C)
+        if rows > 0:
+            gu, h, y = _ffn_forward(x, wgu, wd, plan["offsets"], plan["kept"], rows, plan["row_src"], k)
+        else:
+            gu = torch.zeros(1, 2 * I, dtype=dtype, device=x.device)
+            h = torch.zeros(1, I, dtype=dtype, device=x.device)
+            y = torch.zeros(1, H, dtype=dtype, device=x.device)
+        out = ops.combine(y, plan["row_of"], route["weights"], T, k, out_dtype=dtype)
+
+        ctx.cfg = {key: cfg[key] for key in ("top_k", "temperature", "variant", "load_balancing_weight")}
+        ctx.dims = (T, H, I, E, rows)
+        ctx.n_weights = len(expert_weights)
+        ctx.wgu, ctx.wd = wgu, wd          # dtype copies (or the parameters' own storage); not graph tensors
+        ctx.save_for_backward(x, wg, logits, logits_route, route["indices"], route["weights"], usage, aux.detach(),
+                              plan["offsets"], plan["kept"], plan["row_src"], plan["row_of"], gu, h, y)
+        ctx.param_dtypes = (gate_weight.dtype, [w.dtype for w in expert_weights])
+        if cfg.get("stats") is not None:
+            cfg["stats"].update({"logits": logits, "capacity": C, **route, **plan, "aux": aux.detach().reshape(1)})
+        return out, aux
+
+    @staticmethod
+    def backward(ctx, dout, daux):
+        (x, wg, logits, logits_route, idx, w, usage, aux, offsets, kept, row_src, row_of, gu, h, y) = ctx.saved_tensors
+        T, H, I, E, rows = ctx.dims
+        k = ctx.cfg["top_k"]
+        dtype = x.dtype
+        dev = x.device
+        dout = dout.to(dtype).contiguous()
+        need_x, need_wg = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
+        need_w = any(ctx.needs_input_grad[3:])
+
+        dwgu = dwd = None
+        if rows > 0:
+            dy, dw = ops.combine_bwd(dout, y, row_src, w, k)
+            dx_rows, dwgu, dwd = _ffn_backward(dy, x, ctx.wgu, ctx.wd, gu, h, offsets, kept, rows, row_src, k, need_x,
+                                               need_w)
+            if need_x:
+                ones = torch.ones(T, k, dtype=torch.float32, device=dev)
+                dx = ops.combine(dx_rows, row_of, ones, T, k, out_dtype=dtype)
+        else:
+            dw = torch.zeros(T, k, dtype=torch.float32, device=dev)
+            dx = torch.zeros(T, H, dtype=dtype, device=dev) if need_x else None
+            if need_w:
+                dwd = torch.zeros(E, H, I, dtype=dtype, device=dev)
+                dwgu = torch.zeros(E, 2 * I, H, dtype=dtype, device=dev)
+
+        # routing rule + load-balancing loss -> router logits -> x and the gate weight
+        lbw = ctx.cfg["load_balancing_weight"]
+        scale_dev = (daux.detach().float() * (aux < 1.0).float()).reshape(1).contiguous()
+        dz = ops.route_bwd(logits_route, idx, w, dw, ctx.cfg["temperature"], ctx.cfg["variant"], logits_aux=logits,
+                           usage=usage, aux_scale=E * lbw / T, aux_scale_dev=scale_dev)
+        dx_out, dwg = ops.router_bwd(dz, x, wg, base=dx if need_x else None, out=dx if need_x else None,
+                                     need_dx=need_x, need_dw=need_wg)
+
+        gate_dtype, wdtypes = ctx.param_dtypes
+        grads_w = [None] * ctx.n_weights
+        if need_w:
+            for e in range(E):
+                if ctx.needs_input_grad[3 + e]:
+                    grads_w[e] = dwgu[e].to(wdtypes[e])
+                if ctx.needs_input_grad[3 + E + e]:
+                    grads_w[E + e] = dwd[e].to(wdtypes[E + e])
+        return (dx_out if need_x else None, dwg.to(gate_dtype) if need_wg else None, None, *grads_w)
+
+
+def moe_variant(routing: str) -> int:
+    return {"softmax_topk": ROUTE_SOFTMAX_TOPK, "topk_softmax": ROUTE_TOPK_SOFTMAX}[routing]

@@ -167,12 +167,14 @@ __global__ __launch_bounds__(256) void fill_f32_kernel(float* __restrict__ p, in
 //   dz[i_j] = w_j * (dw_j - sum_m dw_m w_m) / tau
 // Load-balancing loss (model.py:1244-1263) with q = softmax(z_aux), usage constant:
 //   dz_aux[e] += aux_scale * q_e * (usage_e - sum_e' usage_e' q_e'),  aux_scale = dL/daux * E * weight / T
+// (aux_scale = host factor times an optional device scalar, so dL/daux needs no host read-back)
 // One thread per token (E is small).
 __global__ __launch_bounds__(256) void route_bwd_kernel(const float* __restrict__ z_route,
                                                         const float* __restrict__ z_aux,
                                                         const int32_t* __restrict__ idx, const float* __restrict__ w,
                                                         const float* __restrict__ dw, const float* __restrict__ usage,
-                                                        float aux_scale, float inv_tau, int mode,
+                                                        float aux_scale, const float* __restrict__ aux_scale_dev,
+                                                        float inv_tau, int mode,
                                                         float* __restrict__ dz, int64_t T, int E, int k) {
     const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (t >= T) return;
@@ -204,6 +206,7 @@ __global__ __launch_bounds__(256) void route_bwd_kernel(const float* __restrict_
         for (int e = 0; e < E; ++e) out[e] = 0.f;
         for (int j = 0; j < k; ++j) out[it[j]] += wt[j] * (dwt[j] - dot) * inv_tau;
     }
+    if (aux_scale_dev) aux_scale *= aux_scale_dev[0];
     if (usage && aux_scale != 0.f) {
         const float* za = z_aux + t * E;
         float mx = -INFINITY;
@@ -399,8 +402,9 @@ extern "C" int ats_combine_bwd(const void* dout, const void* y, const int32_t* t
 }
 
 extern "C" int ats_route_bwd(const float* logits_route, const float* logits_aux, const int32_t* idx, const float* w,
-                             const float* dw, const float* usage, float aux_scale, float temperature, int mode,
-                             float* dlogits, int64_t T, int E, int k, ats_stream_t stream) {
+                             const float* dw, const float* usage, float aux_scale, const float* aux_scale_dev,
+                             float temperature, int mode, float* dlogits, int64_t T, int E, int k,
+                             ats_stream_t stream) {
     using namespace ats;
     ATS_REQUIRE(T >= 0 && E > 0 && k > 0 && k <= E && temperature > 0.f && (mode == 0 || mode == 1),
                 ATS_ERR_INVALID_ARG, "ats_route_bwd: T=%lld E=%d k=%d temperature=%g mode=%d", (long long)T, E, k,
@@ -409,8 +413,8 @@ extern "C" int ats_route_bwd(const float* logits_route, const float* logits_aux,
     ATS_REQUIRE(logits_route && idx && w && dw && dlogits && (!usage || logits_aux), ATS_ERR_INVALID_ARG,
                 "ats_route_bwd: null pointer");
     hipLaunchKernelGGL(route_bwd_kernel, dim3((unsigned)((T + 255) / 256)), dim3(256), 0, as_stream(stream),
-                       logits_route, logits_aux, idx, w, dw, usage, aux_scale, 1.0f / temperature, mode, dlogits, T, E,
-                       k);
+                       logits_route, logits_aux, idx, w, dw, usage, aux_scale, aux_scale_dev, 1.0f / temperature, mode,
+                       dlogits, T, E, k);
     ATS_CHECK_LAUNCH("ats_route_bwd");
     return ATS_OK;
 }

@@ -16,7 +16,9 @@ MS = Src/Main_Scripts):
 Differences that are deliberate:
   * no PyTorch/CPU fallback: CPU tensors or a missing library raise AtsError
     (the reference silently falls back);
-  * forward only: outputs carry no autograd graph;
+  * when gradients are required (torch.is_grad_enabled() and an input or parameter requires
+    grad) the modules run through the autograd functions of autograd.py, whose backward steps
+    are HIP kernels as well; otherwise the fused inference kernels run and outputs carry no graph;
   * no device synchronisation inside any op (the reference synchronises after
     every kernel);
   * FusedRMSNorm returns the input dtype (the reference's fused wrapper
@@ -31,6 +33,7 @@ from typing import Any, Dict, Optional, Tuple
 import torch
 import torch.nn as nn
 
+from . import autograd as ag
 from . import ops
 from .profiling import stage
 from ._lib import ROUTE_SOFTMAX_TOPK, ROUTE_TOPK_SOFTMAX, AtsError
@@ -53,7 +56,10 @@ class RMSNorm(nn.Module):
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         if x.shape[-1] != self.dim:
             raise AtsError(f"RMSNorm: last dimension {x.shape[-1]} != {self.dim}")
-        return ops.rmsnorm(x, self.weight if self.elementwise_affine else None, self.eps)
+        w = self.weight if self.elementwise_affine else None
+        if _wants_grad(x, w):
+            return ag.RMSNormFunction.apply(x, w, self.eps)
+        return ops.rmsnorm(x, w, self.eps)
 
     def extra_repr(self) -> str:
         return f"dim={self.dim}, eps={self.eps}, elementwise_affine={self.elementwise_affine}, backend=gfx950"
@@ -70,6 +76,8 @@ class FusedRMSNorm(nn.Module):
         self.cuda_enabled = True
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
+        if _wants_grad(x, self.weight):
+            return ag.RMSNormFunction.apply(x, self.weight, self.eps)
         return ops.rmsnorm(x, self.weight, self.eps)
 
 
@@ -113,6 +121,8 @@ class RotaryEmbedding(nn.Module):
 def apply_rotary_pos_emb(q: torch.Tensor, k: torch.Tensor, cos: torch.Tensor,
                          sin: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     """q [B,Hq,L,D], k [B,Hkv,L,D], cos/sin [L, D] -> rotated (q, k) in the input dtype."""
+    if _wants_grad(q, k):
+        return ag.RoPEFunction.apply(q, k, cos, sin, 0)
     return ops.rope(q, k, cos, sin, 0)
 
 
@@ -132,6 +142,8 @@ class FusedRoPE(nn.Module):
         if self.cos_cache.device != q.device:
             self.cos_cache = self.cos_cache.to(q.device)
             self.sin_cache = self.sin_cache.to(q.device)
+        if _wants_grad(q, k):
+            return ag.RoPEFunction.apply(q, k, self.cos_cache, self.sin_cache, position_offset)
         return ops.rope(q, k, self.cos_cache, self.sin_cache, position_offset)
 
 
@@ -160,6 +172,8 @@ class SwiGLUExpert(nn.Module):
         x2 = x.reshape(-1, shape[-1]).contiguous()
         n = x2.shape[0]
         H, I = self.gate_up_proj.in_features, self.down_proj.in_features
+        if n > 0 and _wants_grad(x, self.gate_up_proj.weight, self.down_proj.weight):
+            return ag.ExpertFFNFunction.apply(x2, self.gate_up_proj.weight, self.down_proj.weight).view(shape)
         wgu = _as_dtype(self.gate_up_proj.weight, x2.dtype)
         wd = _as_dtype(self.down_proj.weight, x2.dtype)
         start = torch.zeros(1, dtype=torch.int32, device=x.device)
@@ -167,6 +181,10 @@ class SwiGLUExpert(nn.Module):
         h = ops.grouped_gateup_swiglu(x2, ops.weight_pointer_table([wgu]), start, count, n, n, H, I)
         y = ops.grouped_down(h, ops.weight_pointer_table([wd]), start, count, n, H, I)
         return y.view(shape)
+
+
+def _wants_grad(*tensors: Optional[torch.Tensor]) -> bool:
+    return torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in tensors)
 
 
 def _as_dtype(w: torch.Tensor, dtype: torch.dtype) -> torch.Tensor:
@@ -246,6 +264,27 @@ class MoEFFNLayer(nn.Module):
         E, k = self.num_experts, self.top_k
         I = self.experts[0].down_proj.in_features
 
+        if self.capacity_mode == "fcfs":
+            C = ops.expert_capacity(T, k, E, self.capacity_factor)
+        elif self.capacity_mode == "none":
+            C = T
+        else:
+            raise AtsError(f"MoEFFNLayer: capacity_mode {self.capacity_mode!r}")
+
+        params = [self.gate.weight] + [ex.gate_up_proj.weight for ex in self.experts] + \
+                 [ex.down_proj.weight for ex in self.experts]
+        if _wants_grad(x, *params):
+            stats: Dict[str, Any] = {}
+            cfg = {"top_k": k, "temperature": self.routing_temperature, "variant": ag.moe_variant(self.routing),
+                   "capacity": C, "load_balancing_weight": self.load_balancing_weight,
+                   "noise_std": self.noise_std if self.training else 0.0, "logit_bias": self.router_logit_bias,
+                   "stats": stats}
+            out, aux = ag.MoEFunction.apply(x_flat, self.gate.weight, cfg, *params[1:])
+            self.last_plan = stats
+            if self.training:
+                self._update_routing_stats(stats, T)
+            return out.view(B, L, H), aux
+
         tm = self.stage_timer
         with stage(tm, "router_logits"):
             logits = ops.router_logits(x_flat, _as_dtype(self.gate.weight, x.dtype), self.router_logit_bias)
@@ -254,13 +293,6 @@ class MoEFFNLayer(nn.Module):
         variant = {"softmax_topk": ROUTE_SOFTMAX_TOPK, "topk_softmax": ROUTE_TOPK_SOFTMAX}[self.routing]
         with stage(tm, "route_topk"):
             route = ops.route_topk(logits, k, self.routing_temperature, variant, self.load_balancing_weight)
-
-        if self.capacity_mode == "fcfs":
-            C = ops.expert_capacity(T, k, E, self.capacity_factor)
-        elif self.capacity_mode == "none":
-            C = T
-        else:
-            raise AtsError(f"MoEFFNLayer: capacity_mode {self.capacity_mode!r}")
         with stage(tm, "dispatch_plan"):
             plan = ops.dispatch_plan(route["indices"], E, C)
         rows = min(T * k, E * C)

@@ -431,9 +431,13 @@ def combine_bwd(dout: torch.Tensor, y: torch.Tensor, token_map: torch.Tensor, w:
 
 def route_bwd(logits_route: torch.Tensor, idx: torch.Tensor, w: torch.Tensor, dw: torch.Tensor,
               temperature: float = 1.0, mode: int = ROUTE_SOFTMAX_TOPK, logits_aux: Optional[torch.Tensor] = None,
-              usage: Optional[torch.Tensor] = None, aux_scale: float = 0.0) -> torch.Tensor:
-    """dlogits [T,E] float32 of the routing rule (and of the load-balancing loss when usage is given)."""
-    _need_gpu(logits_route, idx, w, dw, logits_aux, usage)
+              usage: Optional[torch.Tensor] = None, aux_scale: float = 0.0,
+              aux_scale_dev: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """dlogits [T,E] float32 of the routing rule (and of the load-balancing loss when usage is given;
+    its factor is aux_scale times the optional float32 device scalar aux_scale_dev)."""
+    _need_gpu(logits_route, idx, w, dw, logits_aux, usage, aux_scale_dev)
+    if aux_scale_dev is not None and (aux_scale_dev.dtype != torch.float32 or aux_scale_dev.numel() != 1):
+        raise AtsError("route_bwd: aux_scale_dev must be a float32 scalar tensor")
     T, E = logits_route.shape
     k = idx.shape[1]
     if (logits_route.dtype != torch.float32 or idx.dtype != torch.int32 or w.dtype != torch.float32
@@ -445,8 +449,9 @@ def route_bwd(logits_route: torch.Tensor, idx: torch.Tensor, w: torch.Tensor, dw
         logits_aux = (logits_route if logits_aux is None else logits_aux).contiguous()
     out = torch.empty(T, E, dtype=torch.float32, device=logits_route.device)
     check(_lib.load().ats_route_bwd(logits_route.data_ptr(), _ptr(logits_aux), idx.data_ptr(), w.data_ptr(),
-                                    dw.data_ptr(), _ptr(usage), float(aux_scale), float(temperature), int(mode),
-                                    out.data_ptr(), T, E, k, _stream()), "ats_route_bwd")
+                                    dw.data_ptr(), _ptr(usage), float(aux_scale), _ptr(aux_scale_dev),
+                                    float(temperature), int(mode), out.data_ptr(), T, E, k, _stream()),
+          "ats_route_bwd")
     return out
 
 

@@ -10,6 +10,7 @@ import torch
 import torch.nn as nn
 
 from adaptivetrainingsystem_amd import _lib, ops
+from adaptivetrainingsystem_amd.autograd import SwiGLUFunction
 from adaptivetrainingsystem_amd.layers import FusedRMSNorm, FusedRoPE  # noqa: F401
 
 TRANSFORMER_OPS_AVAILABLE = _lib.is_built()
@@ -29,4 +30,7 @@ class FusedSwiGLU(nn.Module):
         self.up_proj = nn.Linear(hidden_size, intermediate_size, bias=use_bias)
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
-        return ops.swiglu_mul(self.gate_proj(x), self.up_proj(x))
+        gate, up = self.gate_proj(x), self.up_proj(x)
+        if torch.is_grad_enabled() and (gate.requires_grad or up.requires_grad):
+            return SwiGLUFunction.apply(gate, up)
+        return ops.swiglu_mul(gate, up)

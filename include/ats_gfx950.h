@@ -220,11 +220,13 @@ int ats_combine_bwd(const void* dout, const void* y, const int32_t* token_map, c
 /* Gradient of the routing rule w.r.t. the router logits (mode 0: softmax -> top-k ->
  * renormalise, model.py:1200-1217; mode 1: top-k -> softmax, moe_cuda_wrapper.py:229-233)
  * plus, when usage != NULL, of the load-balancing loss (model.py:1244-1263) taken on
- * logits_aux: aux_scale = dL/daux * E * load_balancing_weight / T, usage[e] as in the forward
- * (treated as a constant).  logits_route are the logits the routing saw (with noise, if any). */
+ * logits_aux: the factor aux_scale * (aux_scale_dev ? *aux_scale_dev : 1) must equal
+ * dL/daux * E * load_balancing_weight / T (0 where the loss is clamped); usage[e] as in the
+ * forward (a constant).  logits_route are the logits the routing saw (with noise, if any). */
 int ats_route_bwd(const float* logits_route, const float* logits_aux, const int32_t* idx, const float* w,
-                  const float* dw, const float* usage, float aux_scale, float temperature, int mode,
-                  float* dlogits, int64_t T, int E, int k, ats_stream_t stream);
+                  const float* dw, const float* usage, float aux_scale, const float* aux_scale_dev,
+                  float temperature, int mode, float* dlogits, int64_t T, int E, int k,
+                  ats_stream_t stream);
 /* Gradient of ats_router_logits: out[t,:] = base[t,:] + dlogits[t,:] . Wg (base NULL or == out),
  * dWg[e,:] = sum_t dlogits[t,e] * x[t,:] (float32, fixed order). */
 int ats_router_bwd_dx(const float* dlogits, const void* wg, const void* base, void* out, int64_t T, int E,

@@ -267,3 +267,127 @@ def test_expert_ffn_gradients(ops, gpu, counts, H, I, dtype):
     bar = 2e-5 if dtype == torch.float32 else BF16_TOL
     assert rel_err(dwd, torch.stack(list(dwd_ref))) <= bar
     assert rel_err(dwgu, torch.stack(list(dwgu_ref))) <= bar
+
+
+# ------------------------------------------------------------------ whole layer through autograd
+def _layer_grads_vs_oracle(gpu, name, capacity_mode, routing, bar, scale_tokens=None, daux=2.5, temperature=1.0):
+    """Gradients of sum(out * cot) + daux * aux w.r.t. x, the gate and every expert weight: the HIP
+    autograd path against torch autograd over the oracle's forward (the reference's own training path).
+    The discrete routing must coincide, which is asserted first."""
+    from adaptivetrainingsystem_amd import workloads as W
+    w = W.make_moe_workload(name, device="cpu", scale_tokens=scale_tokens)
+    wg = W.make_moe_workload(name, device=gpu, scale_tokens=scale_tokens)
+    w.routing = wg.routing = routing
+    layer = W.build_layer(wg, capacity_mode)
+    layer.routing_temperature = temperature
+    for p in layer.parameters():
+        p.requires_grad_(True)
+    x = wg.x.clone().requires_grad_(True)
+    out, aux = layer(x)                      # eval mode: no routing noise, gradients still flow
+    assert out.requires_grad and aux.requires_grad
+    g = gen(51)
+    cot = torch.randn(w.x.shape, generator=g).to(w.dtype)
+    (out.float() * cot.to(gpu).float()).sum().add(aux * daux).backward()
+
+    E, k = w.num_experts, w.top_k
+
+    def fwd(xx, wgate, *ws):
+        if capacity_mode == "fcfs":
+            r = O.moe_forward_capacity(xx, wgate, list(ws[:E]), list(ws[E:]), k=k, capacity_factor=w.capacity_factor,
+                                       routing=routing, temperature=temperature, logit_bias=w.logit_bias)
+        else:
+            r = O.moe_forward_nocap(xx, wgate, list(ws[:E]), list(ws[E:]), k=k, temperature=temperature)
+        fwd.last = r
+        return r["out"], r["aux"]
+
+    grads = O.layer_grads(fwd, [w.x, w.gate] + list(w.gate_up) + list(w.down), [cot, torch.tensor(daux)])
+    assert torch.equal(layer.last_plan["indices"].cpu().long(), fwd.last["indices"]), "routing differs from the oracle"
+    if capacity_mode == "fcfs":
+        assert torch.equal(layer.last_plan["token_map"].cpu(), fwd.last["token_map"])
+    errs = {"x": rel_err(x.grad, grads[0]), "gate": rel_err(layer.gate.weight.grad, grads[1]),
+            "gate_up": max(rel_err(ex.gate_up_proj.weight.grad, grads[2 + e]) for e, ex in enumerate(layer.experts)),
+            "down": max(rel_err(ex.down_proj.weight.grad, grads[2 + E + e]) for e, ex in enumerate(layer.experts))}
+    print(name, capacity_mode, routing, {n: f"{v:.2e}" for n, v in errs.items()}, flush=True)
+    assert x.grad.dtype == w.dtype and layer.gate.weight.grad.dtype == w.dtype
+    for n, v in errs.items():
+        assert v <= bar, (n, v)
+
+
+def test_layer_grads_c1_fp32(gpu):
+    _layer_grads_vs_oracle(gpu, "c1_cpu_reference", "none", "softmax_topk", 2e-5)
+    _layer_grads_vs_oracle(gpu, "c1_cpu_reference", "fcfs", "softmax_topk", 2e-5)
+    _layer_grads_vs_oracle(gpu, "c1_cpu_reference", "fcfs", "topk_softmax", 2e-5, temperature=0.8)
+
+
+def test_layer_grads_bf16_skewed_drops(gpu):
+    # prefill-shaped skewed routing scaled down to 1024 tokens: expert 0 overflows its capacity
+    _layer_grads_vs_oracle(gpu, "c4_prefill", "fcfs", "softmax_topk", 3e-2, scale_tokens=1024)
+
+
+def test_training_mode_noise_and_stats(gpu):
+    """Training mode: noise on the routing logits only; the auxiliary loss still uses the clean logits."""
+    from adaptivetrainingsystem_amd import workloads as W
+    wg = W.make_moe_workload("c1_cpu_reference", device=gpu)
+    layer = W.build_layer(wg, "none")
+    for p in layer.parameters():
+        p.requires_grad_(True)
+    layer.train()
+    layer.noise_std = 0.5
+    torch.manual_seed(7)
+    out, aux = layer(wg.x)
+    plan = layer.last_plan
+    ref_aux = O.aux_loss(plan["logits"].cpu(), plan["indices"].cpu().long(), wg.num_experts, layer.load_balancing_weight)
+    assert abs(aux.item() - ref_aux.item()) <= 1e-6
+    clean_idx = O.route_softmax_topk_renorm(plan["logits"].cpu(), wg.top_k)[0]
+    assert (clean_idx != plan["indices"].cpu().long()).any(), "noise of 0.5 should change some routing decision"
+    (out.sum() + aux).backward()
+    assert all(p.grad is not None and torch.isfinite(p.grad).all() for p in layer.parameters())
+    stats = layer.get_routing_stats()
+    assert stats["total_tokens_routed"] == wg.tokens
+
+
+def test_module_gradients_norm_rope_expert_swiglu(gpu):
+    import adaptivetrainingsystem_amd as A
+    from adaptivetrainingsystem_amd.seams.cuda_opt_wrapper import FusedSwiGLU
+    from adaptivetrainingsystem_amd.workloads import LayerConfig
+    g = gen(52)
+    # RMSNorm module
+    norm = A.RMSNorm(256).to(gpu)
+    with torch.no_grad():
+        norm.weight.copy_(torch.randn(256, generator=g) * 0.2 + 1)
+    x = torch.randn(4, 9, 256, generator=g)
+    dy = torch.randn(4, 9, 256, generator=g)
+    xg = x.to(gpu).requires_grad_()
+    norm(xg).backward(dy.to(gpu))
+    dx_ref, dw_ref = O.rmsnorm_backward(x, norm.weight.detach().cpu(), dy)
+    assert rel_err(xg.grad, dx_ref) <= F32_TOL and rel_err(norm.weight.grad, dw_ref) <= 2e-5
+    # rotary embedding through apply_rotary_pos_emb
+    rot = A.RotaryEmbedding(32, max_seq_len=64)
+    cos, sin = rot(17, gpu)
+    q = torch.randn(2, 4, 17, 32, generator=g)
+    k = torch.randn(2, 2, 17, 32, generator=g)
+    qg, kg = q.to(gpu).requires_grad_(), k.to(gpu).requires_grad_()
+    qo, ko = A.apply_rotary_pos_emb(qg, kg, cos, sin)
+    dq, dk = torch.randn(2, 4, 17, 32, generator=g), torch.randn(2, 2, 17, 32, generator=g)
+    torch.autograd.backward([qo, ko], [dq.to(gpu), dk.to(gpu)])
+    rq, rk = O.rope_backward(dq, dk, cos.cpu(), sin.cpu())
+    assert torch.equal(qg.grad.cpu(), rq) and torch.equal(kg.grad.cpu(), rk)
+    # one expert
+    ex = A.SwiGLUExpert(LayerConfig(128, 72, 1, 1)).to(gpu)
+    xe = torch.randn(50, 128, generator=g)
+    de = torch.randn(50, 128, generator=g)
+    xeg = xe.to(gpu).requires_grad_()
+    ex(xeg).backward(de.to(gpu))
+    grads = O.layer_grads(lambda a, b, c: O.swiglu_expert(a, b, c),
+                          [xe, ex.gate_up_proj.weight.detach().cpu(), ex.down_proj.weight.detach().cpu()], [de])
+    assert rel_err(xeg.grad, grads[0]) <= 2e-5
+    assert rel_err(ex.gate_up_proj.weight.grad, grads[1]) <= 2e-5 and rel_err(ex.down_proj.weight.grad, grads[2]) <= 2e-5
+    # dense SwiGLU block of the fused wrapper (gate * silu(up))
+    blk = FusedSwiGLU(64, 96).to(gpu)
+    xs = torch.randn(10, 64, generator=g)
+    ds = torch.randn(10, 96, generator=g)
+    xsg = xs.to(gpu).requires_grad_()
+    blk(xsg).backward(ds.to(gpu))
+    wgp, wup = blk.gate_proj.weight.detach().cpu(), blk.up_proj.weight.detach().cpu()
+    ref = O.layer_grads(lambda a, b, c: (a @ b.T) * F.silu(a @ c.T), [xs, wgp, wup], [ds])
+    assert rel_err(xsg.grad, ref[0]) <= 2e-5 and rel_err(blk.gate_proj.weight.grad, ref[1]) <= 2e-5
