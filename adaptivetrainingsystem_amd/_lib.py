@@ -47,10 +47,10 @@ _SIGNATURES = {
     "ats_rope_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
                              c_int, c_int, c_int, c_int, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int,
                              c_void_p]),
-    "ats_silu_mul_fwd": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_int64, c_int, c_int,
-                                 c_void_p]),
+    "ats_silu_mul_fwd": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_int64, c_void_p, c_int,
+                                 c_int, c_void_p]),
     "ats_silu_mul_bwd": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_void_p,
-                                 c_int64, c_int64, c_int, c_int, c_void_p]),
+                                 c_int64, c_int64, c_void_p, c_int, c_int, c_void_p]),
     "ats_combine_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int,
                                 c_int, c_int, c_int, c_void_p]),
     "ats_route_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_float,
@@ -59,7 +59,7 @@ _SIGNATURES = {
     "ats_router_bwd_dw_workspace": (c_size_t, [c_int64, c_int, c_int]),
     "ats_router_bwd_dw": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_void_p, c_size_t,
                                   c_void_p]),
-    "ats_transpose_batched": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
+    "ats_transpose_batched": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "ats_wgrad_padded_rows": (c_int64, [c_int64, c_int]),
     "ats_wgrad_plan": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p]),
     "ats_transpose_grouped_rows": (c_int, [c_void_p, c_int64, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int,

@@ -81,7 +81,7 @@ def _ffn_forward(x, wgu, wd, offsets, kept, rows, row_src, k):
     tab_gu, tab_d = ops.weight_pointer_table(wgu), ops.weight_pointer_table(wd)
     gu = ops.grouped_gemm_nt(tab_gu, H, 2 * I, offsets, kept, rows, rows, 2 * I, H, a=x, a_rows=row_src,
                              a_row_div=k)
-    h = ops.silu_mul(gu[:, :I], gu[:, I:])
+    h = ops.silu_mul(gu[:, :I], gu[:, I:], rows_dev=offsets[-1:])      # only the kept rows
     y = ops.grouped_down(h, tab_d, offsets, kept, rows, H, I)
     return gu, h, y
 
@@ -96,7 +96,7 @@ def _ffn_backward(dy, x, wgu, wd, gu, h, offsets, kept, rows, row_src, k, need_x
     wdT, tab_dT = ops.transpose_batched(wd)                      # [I, H] per expert; kept alive until return
     dh = ops.grouped_gemm_nt(tab_dT, H, I, offsets, kept, rows, rows, I, H, a=dy)
     dgu = torch.empty_like(gu)
-    ops.silu_mul_bwd(gu[:, :I], gu[:, I:], dh, da=dgu[:, :I], db=dgu[:, I:])
+    ops.silu_mul_bwd(gu[:, :I], gu[:, I:], dh, da=dgu[:, :I], db=dgu[:, I:], rows_dev=offsets[-1:])
     dx_rows = dwgu = dwd = None
     if need_x:
         wguT, tab_guT = ops.transpose_batched(wgu)               # [H, 2I] per expert

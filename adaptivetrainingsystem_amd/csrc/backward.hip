@@ -8,29 +8,35 @@
 
 namespace ats {
 
-__device__ __forceinline__ float sigmoid_f(float v) { return 1.0f / (1.0f + expf(-v)); }
+// sigmoid with the hardware exp2 and reciprocal (each about 1 ulp): a few 1e-7 relative, well inside the
+// float32 bar of the gradients.
+__device__ __forceinline__ float sigmoid_f(float v) {
+    return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(v * -1.4426950408889634f));
+}
 
 // ---------------------------------------------------------------- silu(a) * b
 // out[r, c] = silu(a[r, c]) * b[r, c]; operands addressed as base + r * ld + c.
 template <typename T>
 __global__ __launch_bounds__(256) void silu_mul_fwd_kernel(const T* __restrict__ a, int64_t lda,
                                                            const T* __restrict__ b, int64_t ldb, T* __restrict__ out,
-                                                           int64_t ldo, int64_t rows, int cols, bool vec) {
+                                                           int64_t ldo, int64_t rows, const int32_t* __restrict__ rows_dev, int cols,
+                                                           bool vec) {
     constexpr int V = Elem<T>::kVec;
+    if (rows_dev && rows_dev[0] < rows) rows = rows_dev[0] > 0 ? rows_dev[0] : 0;
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     const int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (vec) {
+    if (vec) {   // a block walks whole rows: no 64-bit divisions in the address math
         const int cv = cols / V;
-        const int64_t n = rows * cv;
-        for (int64_t i = tid; i < n; i += stride) {
-            const int64_t r = i / cv;
-            const int c = (int)(i - r * cv) * V;
-            float av[V], bv[V];
-            Elem<T>::unpack(*reinterpret_cast<const uint4*>(a + r * lda + c), av);
-            Elem<T>::unpack(*reinterpret_cast<const uint4*>(b + r * ldb + c), bv);
+        for (int64_t r = blockIdx.x; r < rows; r += gridDim.x) {
+            for (int cvi = threadIdx.x; cvi < cv; cvi += blockDim.x) {
+                const int c = cvi * V;
+                float av[V], bv[V];
+                Elem<T>::unpack(*reinterpret_cast<const uint4*>(a + r * lda + c), av);
+                Elem<T>::unpack(*reinterpret_cast<const uint4*>(b + r * ldb + c), bv);
 #pragma unroll
-            for (int j = 0; j < V; ++j) av[j] = av[j] * sigmoid_f(av[j]) * bv[j];
-            *reinterpret_cast<uint4*>(out + r * ldo + c) = Elem<T>::pack(av);
+                for (int j = 0; j < V; ++j) av[j] = av[j] * sigmoid_f(av[j]) * bv[j];
+                *reinterpret_cast<uint4*>(out + r * ldo + c) = Elem<T>::pack(av);
+            }
         }
     } else {
         const int64_t n = rows * cols;
@@ -50,28 +56,30 @@ __global__ __launch_bounds__(256) void silu_mul_bwd_kernel(const T* __restrict__
                                                            const T* __restrict__ b, int64_t ldb,
                                                            const T* __restrict__ dout, int64_t ldd,
                                                            T* __restrict__ da, int64_t ldda, T* __restrict__ db,
-                                                           int64_t lddb, int64_t rows, int cols, bool vec) {
+                                                           int64_t lddb, int64_t rows, const int32_t* __restrict__ rows_dev, int cols,
+                                                           bool vec) {
     constexpr int V = Elem<T>::kVec;
+    if (rows_dev && rows_dev[0] < rows) rows = rows_dev[0] > 0 ? rows_dev[0] : 0;
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     const int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (vec) {
         const int cv = cols / V;
-        const int64_t n = rows * cv;
-        for (int64_t i = tid; i < n; i += stride) {
-            const int64_t r = i / cv;
-            const int c = (int)(i - r * cv) * V;
-            float av[V], bv[V], gv[V], oa[V], ob[V];
-            Elem<T>::unpack(*reinterpret_cast<const uint4*>(a + r * lda + c), av);
-            Elem<T>::unpack(*reinterpret_cast<const uint4*>(b + r * ldb + c), bv);
-            Elem<T>::unpack(*reinterpret_cast<const uint4*>(dout + r * ldd + c), gv);
+        for (int64_t r = blockIdx.x; r < rows; r += gridDim.x) {
+            for (int cvi = threadIdx.x; cvi < cv; cvi += blockDim.x) {
+                const int c = cvi * V;
+                float av[V], bv[V], gv[V], oa[V], ob[V];
+                Elem<T>::unpack(*reinterpret_cast<const uint4*>(a + r * lda + c), av);
+                Elem<T>::unpack(*reinterpret_cast<const uint4*>(b + r * ldb + c), bv);
+                Elem<T>::unpack(*reinterpret_cast<const uint4*>(dout + r * ldd + c), gv);
 #pragma unroll
-            for (int j = 0; j < V; ++j) {
-                const float s = sigmoid_f(av[j]);
-                oa[j] = gv[j] * bv[j] * (s + av[j] * s * (1.0f - s));
-                ob[j] = gv[j] * (av[j] * s);
+                for (int j = 0; j < V; ++j) {
+                    const float s = sigmoid_f(av[j]);
+                    oa[j] = gv[j] * bv[j] * (s + av[j] * s * (1.0f - s));
+                    ob[j] = gv[j] * (av[j] * s);
+                }
+                *reinterpret_cast<uint4*>(da + r * ldda + c) = Elem<T>::pack(oa);
+                *reinterpret_cast<uint4*>(db + r * lddb + c) = Elem<T>::pack(ob);
             }
-            *reinterpret_cast<uint4*>(da + r * ldda + c) = Elem<T>::pack(oa);
-            *reinterpret_cast<uint4*>(db + r * lddb + c) = Elem<T>::pack(ob);
         }
     } else {
         const int64_t n = rows * cols;
@@ -318,7 +326,7 @@ static int64_t ew_blocks(int64_t items) {
 }  // namespace ats
 
 extern "C" int ats_silu_mul_fwd(const void* a, int64_t lda, const void* b, int64_t ldb, void* out, int64_t ldo,
-                                int64_t rows, int cols, int dtype, ats_stream_t stream) {
+                                int64_t rows, const int32_t* rows_dev, int cols, int dtype, ats_stream_t stream) {
     using namespace ats;
     ATS_REQUIRE(rows >= 0 && cols > 0 && lda >= cols && ldb >= cols && ldo >= cols, ATS_ERR_INVALID_ARG,
                 "ats_silu_mul_fwd: rows=%lld cols=%d strides %lld/%lld/%lld", (long long)rows, cols, (long long)lda,
@@ -329,22 +337,22 @@ extern "C" int ats_silu_mul_fwd(const void* a, int64_t lda, const void* b, int64
     const int V = dtype == ATS_F32 ? 4 : 8;
     const bool vec = cols % V == 0 && lda % V == 0 && ldb % V == 0 && ldo % V == 0 && aligned16(a) && aligned16(b) &&
                      aligned16(out);
-    const int64_t blocks = ew_blocks(rows * (vec ? cols / V : cols));
+    const int64_t blocks = vec ? (rows < 65536 ? rows : 65536) : ew_blocks(rows * cols);
     if (dtype == ATS_F32)
         hipLaunchKernelGGL((silu_mul_fwd_kernel<float>), dim3((unsigned)blocks), dim3(256), 0, as_stream(stream),
                            static_cast<const float*>(a), lda, static_cast<const float*>(b), ldb,
-                           static_cast<float*>(out), ldo, rows, cols, vec);
+                           static_cast<float*>(out), ldo, rows, rows_dev, cols, vec);
     else
         hipLaunchKernelGGL((silu_mul_fwd_kernel<bf16_t>), dim3((unsigned)blocks), dim3(256), 0, as_stream(stream),
                            static_cast<const bf16_t*>(a), lda, static_cast<const bf16_t*>(b), ldb,
-                           static_cast<bf16_t*>(out), ldo, rows, cols, vec);
+                           static_cast<bf16_t*>(out), ldo, rows, rows_dev, cols, vec);
     ATS_CHECK_LAUNCH("ats_silu_mul_fwd");
     return ATS_OK;
 }
 
 extern "C" int ats_silu_mul_bwd(const void* a, int64_t lda, const void* b, int64_t ldb, const void* dout, int64_t ldd,
-                                void* da, int64_t ldda, void* db, int64_t lddb, int64_t rows, int cols, int dtype,
-                                ats_stream_t stream) {
+                                void* da, int64_t ldda, void* db, int64_t lddb, int64_t rows, const int32_t* rows_dev,
+                                int cols, int dtype, ats_stream_t stream) {
     using namespace ats;
     ATS_REQUIRE(rows >= 0 && cols > 0 && lda >= cols && ldb >= cols && ldd >= cols && ldda >= cols && lddb >= cols,
                 ATS_ERR_INVALID_ARG, "ats_silu_mul_bwd: rows=%lld cols=%d", (long long)rows, cols);
@@ -354,17 +362,17 @@ extern "C" int ats_silu_mul_bwd(const void* a, int64_t lda, const void* b, int64
     const int V = dtype == ATS_F32 ? 4 : 8;
     const bool vec = cols % V == 0 && lda % V == 0 && ldb % V == 0 && ldd % V == 0 && ldda % V == 0 && lddb % V == 0 &&
                      aligned16(a) && aligned16(b) && aligned16(dout) && aligned16(da) && aligned16(db);
-    const int64_t blocks = ew_blocks(rows * (vec ? cols / V : cols));
+    const int64_t blocks = vec ? (rows < 65536 ? rows : 65536) : ew_blocks(rows * cols);
     if (dtype == ATS_F32)
         hipLaunchKernelGGL((silu_mul_bwd_kernel<float>), dim3((unsigned)blocks), dim3(256), 0, as_stream(stream),
                            static_cast<const float*>(a), lda, static_cast<const float*>(b), ldb,
                            static_cast<const float*>(dout), ldd, static_cast<float*>(da), ldda,
-                           static_cast<float*>(db), lddb, rows, cols, vec);
+                           static_cast<float*>(db), lddb, rows, rows_dev, cols, vec);
     else
         hipLaunchKernelGGL((silu_mul_bwd_kernel<bf16_t>), dim3((unsigned)blocks), dim3(256), 0, as_stream(stream),
                            static_cast<const bf16_t*>(a), lda, static_cast<const bf16_t*>(b), ldb,
                            static_cast<const bf16_t*>(dout), ldd, static_cast<bf16_t*>(da), ldda,
-                           static_cast<bf16_t*>(db), lddb, rows, cols, vec);
+                           static_cast<bf16_t*>(db), lddb, rows, rows_dev, cols, vec);
     ATS_CHECK_LAUNCH("ats_silu_mul_bwd");
     return ATS_OK;
 }

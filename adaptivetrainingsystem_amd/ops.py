@@ -377,21 +377,23 @@ def _rows_2d(t: torch.Tensor, name: str) -> torch.Tensor:
     return t
 
 
-def silu_mul(a: torch.Tensor, b: torch.Tensor) -> torch.Tensor:
-    """silu(a) * b for 2-D operands that may be column slices of a wider matrix."""
-    _need_gpu(a, b)
+def silu_mul(a: torch.Tensor, b: torch.Tensor, rows_dev: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """silu(a) * b for 2-D operands that may be column slices of a wider matrix.  rows_dev: optional
+    int32 device scalar; rows at or beyond it are left untouched."""
+    _need_gpu(a, b, rows_dev)
     a, b = _rows_2d(a, "silu_mul"), _rows_2d(b, "silu_mul")
     if a.shape != b.shape or a.dtype != b.dtype:
         raise AtsError("silu_mul: operand shapes / dtypes differ")
     out = torch.empty(a.shape, dtype=a.dtype, device=a.device)
     check(_lib.load().ats_silu_mul_fwd(a.data_ptr(), a.stride(0), b.data_ptr(), b.stride(0), out.data_ptr(),
-                                       out.stride(0) if out.numel() else a.shape[1], a.shape[0], a.shape[1], _tag(a),
-                                       _stream()), "ats_silu_mul_fwd")
+                                       out.stride(0) if out.numel() else a.shape[1], a.shape[0], _ptr(rows_dev),
+                                       a.shape[1], _tag(a), _stream()), "ats_silu_mul_fwd")
     return out
 
 
 def silu_mul_bwd(a: torch.Tensor, b: torch.Tensor, dout: torch.Tensor, da: Optional[torch.Tensor] = None,
-                 db: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+                 db: Optional[torch.Tensor] = None,
+                 rows_dev: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:
     """Gradients of silu(a) * b; da/db may be preallocated (e.g. the two halves of one matrix)."""
     _need_gpu(a, b, dout, da, db)
     a, b, dout = _rows_2d(a, "silu_mul_bwd"), _rows_2d(b, "silu_mul_bwd"), _rows_2d(dout, "silu_mul_bwd")
@@ -405,8 +407,8 @@ def silu_mul_bwd(a: torch.Tensor, b: torch.Tensor, dout: torch.Tensor, da: Optio
     cols = a.shape[1]
     st = lambda t: t.stride(0) if t.shape[0] > 1 else max(t.stride(0), cols)
     check(_lib.load().ats_silu_mul_bwd(a.data_ptr(), st(a), b.data_ptr(), st(b), dout.data_ptr(), st(dout),
-                                       da.data_ptr(), st(da), db.data_ptr(), st(db), a.shape[0], cols, _tag(a),
-                                       _stream()), "ats_silu_mul_bwd")
+                                       da.data_ptr(), st(da), db.data_ptr(), st(db), a.shape[0], _ptr(rows_dev), cols,
+                                       _tag(a), _stream()), "ats_silu_mul_bwd")
     return da, db
 
 
@@ -495,8 +497,9 @@ def transpose_batched(mats: Sequence[torch.Tensor]) -> Tuple[list, torch.Tensor]
     outs = [buf[e] for e in range(E)]
     in_tab = weight_pointer_table(list(mats))
     out_tab = weight_pointer_table(outs)
-    check(_lib.load().ats_transpose_batched(in_tab.data_ptr(), out_tab.data_ptr(), E, R, C, _tag(mats[0]), _stream()),
-          "ats_transpose_batched")
+    aligned = all(m.data_ptr() % 16 == 0 for m in mats) and all(o.data_ptr() % 16 == 0 for o in outs)
+    check(_lib.load().ats_transpose_batched(in_tab.data_ptr(), out_tab.data_ptr(), E, R, C, _tag(mats[0]), int(aligned),
+                                            _stream()), "ats_transpose_batched")
     return outs, out_tab
 
 

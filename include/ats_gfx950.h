@@ -205,12 +205,13 @@ int ats_rope_bwd(const void* dq_out, const void* dk_out, void* dq, void* dk, con
 /* out = silu(a) * b on row-strided [rows, cols] operands (strides in elements), and its
  * gradient da = dout*b*(s + a*s*(1-s)), db = dout*a*s, s = sigmoid(a)
  * (SwiGLUFunction.backward, cuda_opt_wrapper.py:237-254; SwiGLUExpert, model.py:1071-1088:
- * a = gate half, b = up half of the [rows, 2I] projection). */
+ * a = gate half, b = up half of the [rows, 2I] projection).  rows_dev (optional device scalar)
+ * lowers the row count to min(rows, *rows_dev), e.g. the number of kept rows of a dispatch plan. */
 int ats_silu_mul_fwd(const void* a, int64_t lda, const void* b, int64_t ldb, void* out, int64_t ldo,
-                     int64_t rows, int cols, int dtype, ats_stream_t stream);
+                     int64_t rows, const int32_t* rows_dev, int cols, int dtype, ats_stream_t stream);
 int ats_silu_mul_bwd(const void* a, int64_t lda, const void* b, int64_t ldb, const void* dout,
                      int64_t ldd, void* da, int64_t ldda, void* db, int64_t lddb, int64_t rows,
-                     int cols, int dtype, ats_stream_t stream);
+                     const int32_t* rows_dev, int cols, int dtype, ats_stream_t stream);
 /* Gradient of ats_combine: for expert row r with m = token_map[r] >= 0, t = m / k:
  * dy[r,:] = w[m] * dout[t,:], dw[m] = dout[t,:] . y[r,:]; rows with m < 0 and the dw of
  * dropped assignments are zero.  dw: [T*k] float32. */
@@ -238,9 +239,10 @@ int ats_router_bwd_dw(const float* dlogits, const void* x, float* dwg, int64_t T
  * E matrices [R, C] -> [C, R]; and grouped rows [*, C] (row r of expert e, optionally
  * gathered as in ats_grouped_gateup_swiglu) -> [C, ld_out] where expert e owns the columns
  * k_start[e] .. k_start[e]+k_count[e]-1, k_count[e] = max(64, roundup(row_count[e], 64)),
- * zero padded (ats_wgrad_plan writes k_start/k_count; ld_out >= ats_wgrad_padded_rows). */
+ * zero padded (ats_wgrad_plan writes k_start/k_count; ld_out >= ats_wgrad_padded_rows).
+ * aligned_bases != 0 promises that every matrix in both pointer tables is 16-byte aligned. */
 int ats_transpose_batched(const void* const* in_ptrs, void* const* out_ptrs, int E, int R, int C, int dtype,
-                          ats_stream_t stream);
+                          int aligned_bases, ats_stream_t stream);
 int64_t ats_wgrad_padded_rows(int64_t max_rows, int E);
 int ats_wgrad_plan(const int32_t* row_count, int E, int32_t* k_start, int32_t* k_count, ats_stream_t stream);
 int ats_transpose_grouped_rows(const void* in, int64_t ld_in, int C, const int32_t* gather, int gather_div,
