@@ -301,11 +301,23 @@ __global__ __launch_bounds__(256) void router_dw_partial_kernel(const float* __r
 
 __global__ __launch_bounds__(256) void router_dw_reduce_kernel(const float* __restrict__ partial, int n_chunks,
                                                                float* __restrict__ dwg, int64_t EH) {
-    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i >= EH) return;
+    // a block owns 32 entries; 8 groups each add every 8th chunk, then the 8 sums are added in order
+    __shared__ float part[8][32];
+    const int col = threadIdx.x & 31, grp = threadIdx.x >> 5;
+    const int64_t i = (int64_t)blockIdx.x * 32 + col;
     float s = 0.f;
-    for (int c = 0; c < n_chunks; ++c) s += partial[(int64_t)c * EH + i];
-    dwg[i] = s;
+    if (i < EH) {
+#pragma unroll 8
+        for (int c = grp; c < n_chunks; c += 8) s += partial[(int64_t)c * EH + i];
+    }
+    part[grp][col] = s;
+    __syncthreads();
+    if (grp == 0 && i < EH) {
+        float t = part[0][col];
+#pragma unroll
+        for (int g = 1; g < 8; ++g) t += part[g][col];
+        dwg[i] = t;
+    }
 }
 
 static int dw_chunks(int64_t T, int* chunk_tokens) {
@@ -483,7 +495,7 @@ extern "C" int ats_router_bwd_dw(const float* dlogits, const void* x, float* dwg
     else
         hipLaunchKernelGGL((router_dw_partial_kernel<bf16_t>), grid, dim3(256), 0, s, dlogits,
                            static_cast<const bf16_t*>(x), partial, T, E, H, chunk_tokens);
-    hipLaunchKernelGGL(router_dw_reduce_kernel, dim3((unsigned)((EH + 255) / 256)), dim3(256), 0, s, partial, n_chunks,
+    hipLaunchKernelGGL(router_dw_reduce_kernel, dim3((unsigned)((EH + 31) / 32)), dim3(256), 0, s, partial, n_chunks,
                        dwg, EH);
     ATS_CHECK_LAUNCH("ats_router_bwd_dw");
     return ATS_OK;

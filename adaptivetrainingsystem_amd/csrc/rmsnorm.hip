@@ -166,16 +166,48 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_rows_kernel(const T* __restri
     }
 #define ATS_WVAL(i_, j_, v_) (!HAS_W ? 1.f : WREG ? wreg[WREG ? (i_) : 0][j_] : Elem<WT>::load(w + (int64_t)(v_) * V + (j_)))
 
-    for (int64_t row = wave; row < rows; row += nwaves) {
-        const uint4* xr = reinterpret_cast<const uint4*>(x + row * H);
-        const uint4* gr = reinterpret_cast<const uint4*>(dy + row * H);
-        uint4 xraw[NV], graw[NV];
+    // short rows: the next row is fetched while the current one is reduced and written
+    constexpr bool kPrefetch = NV <= 4;
+    uint4 xnext[kPrefetch ? NV : 1], gnext[kPrefetch ? NV : 1];
+    if (kPrefetch && wave < rows) {
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
             const int v = lane + i * kWave;
             if (v < nvec) {
-                xraw[i] = xr[v];
-                graw[i] = gr[v];
+                xnext[kPrefetch ? i : 0] = reinterpret_cast<const uint4*>(x + wave * H)[v];
+                gnext[kPrefetch ? i : 0] = reinterpret_cast<const uint4*>(dy + wave * H)[v];
+            }
+        }
+    }
+    for (int64_t row = wave; row < rows; row += nwaves) {
+        const uint4* xr = reinterpret_cast<const uint4*>(x + row * H);
+        const uint4* gr = reinterpret_cast<const uint4*>(dy + row * H);
+        uint4 xraw[NV], graw[NV];
+        if (kPrefetch) {
+#pragma unroll
+            for (int i = 0; i < NV; ++i) {
+                xraw[i] = xnext[kPrefetch ? i : 0];
+                graw[i] = gnext[kPrefetch ? i : 0];
+            }
+            const int64_t nrow = row + nwaves;
+            if (nrow < rows) {
+#pragma unroll
+                for (int i = 0; i < NV; ++i) {
+                    const int v = lane + i * kWave;
+                    if (v < nvec) {
+                        xnext[kPrefetch ? i : 0] = reinterpret_cast<const uint4*>(x + nrow * H)[v];
+                        gnext[kPrefetch ? i : 0] = reinterpret_cast<const uint4*>(dy + nrow * H)[v];
+                    }
+                }
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < NV; ++i) {
+                const int v = lane + i * kWave;
+                if (v < nvec) {
+                    xraw[i] = xr[v];
+                    graw[i] = gr[v];
+                }
             }
         }
         float ss = 0.f, dot = 0.f;
@@ -277,16 +309,29 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_generic_kernel(const T* __res
         for (int h = lane; h < H; h += kWave) mine[h] = 0.f;
 }
 
+// dw[h] = sum over the partial rows, in a fixed order: a block owns 32 columns; its 8 row groups each add
+// every 8th partial row (independent loads, so many are in flight), then the 8 sums are added in order.
 __global__ __launch_bounds__(256) void rmsnorm_dw_reduce_kernel(const float* __restrict__ partial, int n_partial,
                                                                 float* __restrict__ dw, int H) {
-    const int h = blockIdx.x * blockDim.x + threadIdx.x;
-    if (h >= H) return;
+    __shared__ float part[8][32];
+    const int col = threadIdx.x & 31, grp = threadIdx.x >> 5;
+    const int h = blockIdx.x * 32 + col;
     float s = 0.f;
-    for (int b = 0; b < n_partial; ++b) s += partial[(int64_t)b * H + h];
-    dw[h] = s;
+    if (h < H) {
+#pragma unroll 8
+        for (int b = grp; b < n_partial; b += 8) s += partial[(int64_t)b * H + h];
+    }
+    part[grp][col] = s;
+    __syncthreads();
+    if (grp == 0 && h < H) {
+        float t = part[0][col];
+#pragma unroll
+        for (int g = 1; g < 8; ++g) t += part[g][col];
+        dw[h] = t;
+    }
 }
 
-constexpr int kBwdBlocksVec = 512;      // vector kernel: 2 blocks per CU, one partial row per block
+constexpr int kBwdBlocksVec = 512;      // vector kernel: two blocks per CU, one partial row per block
 constexpr int kBwdBlocksGeneric = 64;   // generic kernel: one partial row per wave (256 rows)
 
 static bool rmsnorm_bwd_vec_ok(const void* x, const void* dy, const void* dx, int H, int V) {
@@ -326,7 +371,7 @@ static int launch_rmsnorm_bwd(const void* x, const void* w, const void* dy, void
         n_partial = blocks;
     }
     if (dw)
-        hipLaunchKernelGGL(rmsnorm_dw_reduce_kernel, dim3((H + 255) / 256), dim3(256), 0, s, partial, n_partial, dw, H);
+        hipLaunchKernelGGL(rmsnorm_dw_reduce_kernel, dim3((H + 31) / 32), dim3(256), 0, s, partial, n_partial, dw, H);
     return ATS_OK;
 }
 
@@ -373,7 +418,7 @@ extern "C" int ats_rmsnorm_bwd(const void* x, const void* w, const void* dy, voi
                 ATS_ERR_UNSUPPORTED, "ats_rmsnorm_bwd: dtype tags %d/%d", x_dtype, w_dtype);
     hipStream_t s = as_stream(stream);
     if (rows == 0) {
-        if (dw) hipLaunchKernelGGL(rmsnorm_dw_reduce_kernel, dim3((hidden + 255) / 256), dim3(256), 0, s, nullptr, 0, dw, hidden);
+        if (dw) hipLaunchKernelGGL(rmsnorm_dw_reduce_kernel, dim3((hidden + 31) / 32), dim3(256), 0, s, nullptr, 0, dw, hidden);
         ATS_CHECK_LAUNCH("ats_rmsnorm_bwd");
         return ATS_OK;
     }

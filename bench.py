@@ -244,6 +244,13 @@ def run_norm_rope(args):
         with timer.range("rope"):
             for _ in range(burst):
                 ops.rope(w.q, w.k, cos, sin)
+        # the gradients of the two kernels (x stands in for dy: same shape and type)
+        with timer.range("rmsnorm_bwd"):
+            for _ in range(burst):
+                ops.rmsnorm_bwd(w.x, w.norm_weight, w.x, w.eps)
+        with timer.range("rope_bwd"):
+            for _ in range(burst):
+                ops.rope(w.q, w.k, cos, sin, inverse=True)
     torch.cuda.synchronize()
     st = timer.summary()
     for v in st.values():
@@ -257,6 +264,11 @@ def run_norm_rope(args):
     rope_gbs = rope_bytes / (st["rope"]["mean_ms"] * 1e-3) / 1e9
     log(f"  rmsnorm {st['rmsnorm']['mean_ms']*1e3:.1f} us -> {rms_gbs:.0f} GB/s ({rms_gbs/PEAK_HBM_GBS:.1%}); "
         f"rope {st['rope']['mean_ms']*1e3:.1f} us -> {rope_gbs:.0f} GB/s ({rope_gbs/PEAK_HBM_GBS:.1%})")
+    rmsb_bytes = 3 * T * w.hidden * es + 8 * w.hidden
+    rmsb_gbs = rmsb_bytes / (st["rmsnorm_bwd"]["mean_ms"] * 1e-3) / 1e9
+    ropeb_gbs = rope_bytes / (st["rope_bwd"]["mean_ms"] * 1e-3) / 1e9
+    log(f"  rmsnorm_bwd {st['rmsnorm_bwd']['mean_ms']*1e3:.1f} us -> {rmsb_gbs:.0f} GB/s ({rmsb_gbs/PEAK_HBM_GBS:.1%}); "
+        f"rope_bwd {st['rope_bwd']['mean_ms']*1e3:.1f} us -> {ropeb_gbs:.0f} GB/s ({ropeb_gbs/PEAK_HBM_GBS:.1%})")
     result = {
         "metric": "fused RMSNorm + RoPE tokens/s (config 2)", "value": T * args.steps / dt, "unit": "tokens/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": dt / args.steps * 1e3,
@@ -266,6 +278,10 @@ def run_norm_rope(args):
                      "frac": rope_gbs / PEAK_HBM_GBS, "traffic": None},
         "rmsnorm_roofline": {"bound": "hbm", "achieved": rms_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s",
                              "frac": rms_gbs / PEAK_HBM_GBS},
+        "rmsnorm_bwd_roofline": {"bound": "hbm", "achieved": rmsb_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                                 "frac": rmsb_gbs / PEAK_HBM_GBS},
+        "rope_bwd_roofline": {"bound": "hbm", "achieved": ropeb_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                              "frac": ropeb_gbs / PEAK_HBM_GBS},
         "stages_ms": {s: round(v["mean_ms"], 5) for s, v in st.items()},
     }
     if not args.no_cpu_baseline:
