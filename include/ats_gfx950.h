@@ -260,6 +260,36 @@ int ats_grouped_gemm_nt(const void* a, const void* const* a_ptrs, int64_t lda, i
                         const int32_t* row_count, const int32_t* k_count, int E, int64_t max_rows, int N,
                         int K, int dtype, int out_dtype, ats_stream_t stream);
 
+/* ---- Training-step ops beside the sparse layer --------------------------------
+ * Fused cross-entropy + accuracy.  Replaces fused_cross_entropy_accuracy_launcher
+ * (Src/Main_Scripts/training/fused_loss.cu:179-214); numerics follow FusedLoss._pytorch_fallback
+ * (Src/Main_Scripts/training/cuda_kernels.py:191-249).  A token is ignored when its label equals
+ * pad_id or lies outside [0, V).  Per token: loss_tok = logsumexp(z) - z[label] (10.0 if not
+ * finite), lse, correct (arg-max == label, lower index among equal logits), valid.
+ * sums[5] = {sum w*loss, sum w, sum loss, sum correct, valid count} over valid tokens
+ * (w = weights[t], 1 when weights == NULL), added in a fixed order.  logits: [T, V] of dtype. */
+int ats_cross_entropy_fwd(const void* logits, const int64_t* labels, int64_t pad_id, const float* weights,
+                          float* loss_tok, float* lse, float* correct, float* valid, float* sums, int64_t T,
+                          int V, int dtype, ats_stream_t stream);
+/* Gradient of sums[0] / max(sums[1], 1e-8) w.r.t. the logits, times the device scalar scale[0]:
+ * dlogits[t,v] = scale * w_t * valid_t / max(sums[1], 1e-8) * (exp(z - lse_t) - [v == label_t]).
+ * (The reference's fused loss returns a value without a graph; its fallback uses autograd.) */
+int ats_cross_entropy_bwd(const void* logits, const int64_t* labels, const float* lse, const float* valid,
+                          const float* weights, const float* sums, const float* scale, void* dlogits, int64_t T,
+                          int V, int dtype, ats_stream_t stream);
+/* Multi-tensor gradient norm and clipping.  Replaces fused_grad_clip_launcher
+ * (Src/Main_Scripts/training/fused_grad_clip.cu:117-175) without its synchronisation and atomics.
+ * grad_ptrs/sizes: n_tensors tensors of one dtype; chunk_start[n_tensors+1]: running count of
+ * ats_grad_clip_chunk_elems()-sized chunks (built by the host), n_chunks = chunk_start[n_tensors];
+ * partial: n_chunks floats of scratch.  norm_out[0] = sqrt(extra_sumsq[0] + sum of squares),
+ * norm_out[1] = that sum (so groups of different dtype can be chained through extra_sumsq).
+ * do_clip: 0 = norm only; 1 = norm, then grads *= max_norm / (norm + 1e-6) if that is < 1;
+ * 2 = scale only, with the norm already in norm_out[0]. */
+int ats_grad_clip_chunk_elems(void);
+int ats_grad_norm_clip(void* const* grad_ptrs, const int64_t* sizes, const int32_t* chunk_start, int n_tensors,
+                       int n_chunks, int dtype, const float* extra_sumsq, float* partial, float* norm_out,
+                       float max_norm, int do_clip, ats_stream_t stream);
+
 /* ---- Host-side views of the grouped-GEMM tile schedule (no device work) ----
  * No reference counterpart; used to test the block -> (expert, m-tile, n-tile)
  * map on the CPU.  row_count_host is a host array.  decode returns 1 and fills

@@ -46,6 +46,8 @@ PINNING = {
     "rmsnorm_backward": "torch.autograd of rmsnorm in float64; torch.autograd.gradcheck",
     "rope_backward": "torch.autograd of rope_apply; R(p)^T = R(-p)",
     "swiglu_backward": "torch.autograd of gate*silu(up) in float64; gradcheck",
+    "fused_loss": "float64 logsumexp closed form; uniform logits give log(V); torch.autograd for the gradient",
+    "clip_grad_norm": "closed form sqrt(sum of squares) and scaling by max_norm/(norm+1e-6)",
     "layer_grads": "is torch.autograd over the forward restatements above (what the reference itself trains with); "
                    "gradcheck in float64 on the no-capacity layer with fixed routing",
 }
@@ -461,3 +463,37 @@ def layer_grads(forward, tensors, cotangents):
         outs = (outs,)
     loss = sum((o.float() * c.float()).sum() for o, c in zip(outs, cotangents))
     return list(torch.autograd.grad(loss, leaves, allow_unused=True))
+
+
+# --------------------------------------------------------------------------- training-step ops
+def fused_loss(logits: torch.Tensor, labels: torch.Tensor, loss_weights: Optional[torch.Tensor] = None,
+               pad_token_id: int = -100):
+    """MS/training/cuda_kernels.py:191-249 (FusedLoss._pytorch_fallback), float32 math, with the
+    validity rule of the fused kernel (MS/training/fused_loss.cu:83-84: a label equal to the pad id or
+    outside [0, V) is ignored).  Returns the dict of the reference; ``loss`` is differentiable."""
+    V = logits.shape[-1]
+    lg = logits.reshape(-1, V).float()
+    lb = labels.reshape(-1).long()
+    mask = ((lb != pad_token_id) & (lb >= 0) & (lb < V)).float()
+    n_valid = mask.sum()
+    safe = torch.where(mask.bool(), lb, torch.zeros_like(lb))
+    per_tok = F.cross_entropy(lg, safe, reduction="none")
+    per_tok = torch.where(torch.isfinite(per_tok), per_tok, torch.full_like(per_tok, 10.0))
+    acc = ((lg.argmax(-1) == lb).float() * mask).sum() / n_valid.clamp(min=1.0)
+    raw = (per_tok * mask).sum() / n_valid.clamp(min=1.0)
+    if loss_weights is not None:
+        w = loss_weights.reshape(-1).float()
+        loss = (per_tok * w * mask).sum() / (w * mask).sum().clamp(min=1e-8)
+    else:
+        loss = (per_tok * mask).sum() / n_valid.clamp(min=1e-8)
+    ppl = torch.exp(torch.clamp(raw.detach(), min=0.0, max=15.0)) if n_valid > 0 else torch.tensor(float("inf"))
+    return {"loss": loss, "raw_loss": raw.detach(), "perplexity": ppl, "valid_tokens": n_valid, "accuracy": acc}
+
+
+def clip_grad_norm(grads, max_norm: float):
+    """MS/training/cuda_kernels.py:340-342 (torch.nn.utils.clip_grad_norm_) restated on a list of
+    gradient tensors: returns (total L2 norm float32, list of clipped copies)."""
+    total = torch.sqrt(sum((g.float() ** 2).sum() for g in grads)) if grads else torch.tensor(0.0)
+    coef = max_norm / (total + 1e-6)
+    out = [(g.float() * coef).to(g.dtype) if coef < 1.0 else g.clone() for g in grads]
+    return total, out

@@ -469,3 +469,50 @@ def test_layer_grads_gradcheck_fixed_routing():
     assert torch.allclose(got[1].double(), g64[1], rtol=1e-3, atol=1e-5)
     assert torch.allclose(torch.stack(got[2:2 + E]).double(), g64[2], rtol=1e-3, atol=1e-5)
     assert torch.allclose(torch.stack(got[2 + E:]).double(), g64[3], rtol=1e-3, atol=1e-5)
+
+
+# --------------------------------------------------------------------------- training-step ops
+def test_fused_loss_closed_form_and_masking():
+    g = torch.Generator().manual_seed(61)
+    T, V = 40, 37
+    z = torch.randn(T, V, generator=g, dtype=torch.float64) * 3
+    y = torch.randint(0, V, (T,), generator=g)
+    y[3] = -100
+    y[7] = V + 5            # out of range: ignored like the pad id
+    y[11] = -1
+    r = O.fused_loss(z.float(), y)
+    keep = torch.tensor([i for i in range(T) if i not in (3, 7, 11)])
+    lse = torch.logsumexp(z[keep], -1)
+    ref = (lse - z[keep, y[keep]]).mean()
+    assert abs(r["loss"].item() - ref.item()) < 1e-5 and r["valid_tokens"].item() == T - 3
+    assert abs(r["accuracy"].item() - (z[keep].argmax(-1) == y[keep]).double().mean().item()) < 1e-6
+    assert abs(r["perplexity"].item() - min(math.exp(ref.item()), math.exp(15.0))) / r["perplexity"].item() < 1e-4
+    # uniform logits: loss = log V exactly, accuracy = share of label 0 (first index wins the arg-max)
+    u = O.fused_loss(torch.zeros(T, V), y)
+    assert abs(u["loss"].item() - math.log(V)) < 1e-6
+    # weights: weighted mean over valid tokens
+    w = torch.rand(T, generator=g)
+    rw = O.fused_loss(z.float(), y, loss_weights=w)
+    refw = ((lse - z[keep, y[keep]]) * w[keep].double()).sum() / w[keep].double().sum()
+    assert abs(rw["loss"].item() - refw.item()) < 1e-5
+    # all tokens ignored
+    e = O.fused_loss(z.float(), torch.full((T,), -100))
+    assert e["loss"].item() == 0.0 and e["valid_tokens"].item() == 0 and math.isinf(e["perplexity"].item())
+
+
+def test_clip_grad_norm_closed_form():
+    g = torch.Generator().manual_seed(62)
+    grads = [torch.randn(5, 7, generator=g), torch.randn(11, generator=g) * 3, torch.randn(2, 3, 4, generator=g)]
+    total = math.sqrt(sum(float((x.double() ** 2).sum()) for x in grads))
+    n, clipped = O.clip_grad_norm(grads, max_norm=1.0)
+    assert abs(n.item() - total) < 1e-5
+    new_total = math.sqrt(sum(float((x.double() ** 2).sum()) for x in clipped))
+    assert abs(new_total - 1.0) < 1e-4
+    n2, same = O.clip_grad_norm(grads, max_norm=1e6)
+    assert all(torch.equal(a, b) for a, b in zip(grads, same))
+    params = [torch.nn.Parameter(torch.zeros_like(x)) for x in grads]
+    for p_, x in zip(params, grads):
+        p_.grad = x.clone()
+    lib_norm = torch.nn.utils.clip_grad_norm_(params, 1.0)
+    assert abs(lib_norm.item() - n.item()) < 1e-5
+    assert all(torch.allclose(p_.grad, c, atol=1e-6) for p_, c in zip(params, clipped))
