@@ -316,6 +316,12 @@ class MoEFFNLayer(nn.Module):
     def _update_routing_stats(self, plan, total_tokens: int) -> None:
         hist = plan["hist"].cpu()
         kept = plan["kept"].cpu()
+        usage = self._routing_stats["expert_usage"]
+        if usage.numel() != hist.numel():       # an expert was added or pruned since the last step
+            grown = torch.zeros(hist.numel())
+            n = min(usage.numel(), hist.numel())
+            grown[:n] = usage[:n]
+            self._routing_stats["expert_usage"] = grown
         self._routing_stats["expert_usage"] += hist.float()
         self._routing_stats["total_routed"] += total_tokens
         self._routing_stats["dropped_tokens"] += int((hist - kept).sum())

@@ -391,3 +391,88 @@ def test_module_gradients_norm_rope_expert_swiglu(gpu):
     wgp, wup = blk.gate_proj.weight.detach().cpu(), blk.up_proj.weight.detach().cpu()
     ref = O.layer_grads(lambda a, b, c: (a @ b.T) * F.silu(a @ c.T), [xs, wgp, wup], [ds])
     assert rel_err(xsg.grad, ref[0]) <= 2e-5 and rel_err(blk.gate_proj.weight.grad, ref[1]) <= 2e-5
+
+
+# ------------------------------------------------------------------ trainer-facing management
+def test_trainer_surgery_and_checkpoint_round_trip(gpu):
+    """What the reference trainer does to a live layer between steps (add_expert / prune_expert /
+    adjust_capacity_factor / adjust_routing_temperature, trainer.py:1269-1493) and a state_dict round trip:
+    after every change forward and backward still agree with the oracle on the layer's current weights."""
+    import torch.nn as nn
+    import adaptivetrainingsystem_amd as A
+    from adaptivetrainingsystem_amd import workloads as W
+    from adaptivetrainingsystem_amd.workloads import LayerConfig
+    torch.manual_seed(11)
+    cfg = LayerConfig(128, 72, 4, 2, 1.25, moe_routing="softmax_topk", moe_capacity_mode="fcfs")
+    layer = A.MoEFFNLayer(cfg).to(gpu)
+    layer.eval()
+    g = gen(53)
+    x = torch.randn(3, 50, 128, generator=g)
+    cot = torch.randn(3, 50, 128, generator=g)
+
+    def check():
+        xg = x.to(gpu).requires_grad_()
+        for p in layer.parameters():
+            p.grad = None
+        out, aux = layer(xg)
+        (out * cot.to(gpu)).sum().add(aux).backward()
+        E = layer.num_experts
+        ws = [layer.gate.weight] + [ex.gate_up_proj.weight for ex in layer.experts] + \
+             [ex.down_proj.weight for ex in layer.experts]
+
+        def fwd(xx, wgate, *rest):
+            r = O.moe_forward_capacity(xx, wgate, list(rest[:E]), list(rest[E:]), k=layer.top_k,
+                                       capacity_factor=layer.capacity_factor, temperature=layer.routing_temperature)
+            fwd.last = r
+            return r["out"], r["aux"]
+
+        grads = O.layer_grads(fwd, [x] + [w_.detach().cpu() for w_ in ws], [cot, torch.tensor(1.0)])
+        assert torch.equal(layer.last_plan["indices"].cpu().long(), fwd.last["indices"])
+        assert layer.last_plan["capacity"] == fwd.last["capacity"]
+        assert rel_err(out, fwd.last["out"]) <= F32_TOL
+        assert rel_err(xg.grad, grads[0]) <= 2e-5
+        for w_, g_ in zip(ws, grads[1:]):
+            assert rel_err(w_.grad, g_) <= 2e-5
+        return out.detach()
+
+    check()
+    # add_expert: average of the existing experts plus noise, gate row appended, new nn.Linear gate
+    new = A.SwiGLUExpert(cfg).to(gpu)
+    with torch.no_grad():
+        for name, p in new.named_parameters():
+            p.copy_(torch.stack([dict(e.named_parameters())[name] for e in layer.experts]).mean(0))
+            p.add_(torch.randn_like(p) * 0.01)
+    layer.experts.append(new)
+    layer.num_experts += 1
+    old = layer.gate.weight.data
+    grown = torch.zeros(layer.num_experts, 128, device=gpu)
+    grown[:-1] = old
+    nn.init.normal_(grown[-1], mean=0.0, std=0.01)
+    layer.gate = nn.Linear(128, layer.num_experts, bias=False).to(gpu)
+    layer.gate.weight.data = grown
+    layer.train()                      # statistics follow the new expert count
+    layer.noise_std = 0.0
+    check()
+    assert len(layer.get_routing_stats()["expert_usage_percentages"]) == 5
+    layer.eval()
+    # adjust_capacity_factor / adjust_routing_temperature
+    layer.capacity_factor = 0.6
+    layer.routing_temperature = 1.7
+    check()
+    assert int((layer.last_plan["hist"] - layer.last_plan["kept"]).sum()) > 0       # the tighter capacity drops
+    # prune_expert
+    del layer.experts[1]
+    layer.num_experts -= 1
+    w_old = layer.gate.weight.data
+    layer.gate = nn.Linear(128, layer.num_experts, bias=False).to(gpu)
+    layer.gate.weight.data = torch.cat([w_old[:1], w_old[2:]], dim=0)
+    before = check()
+    # checkpoint round trip: the reference's key names, loaded into a fresh layer
+    sd = {k_: v.cpu() for k_, v in layer.state_dict().items()}
+    assert set(sd) == {"gate.weight"} | {f"experts.{i}.{n}.weight" for i in range(4) for n in ("gate_up_proj", "down_proj")}
+    fresh = A.MoEFFNLayer(cfg).to(gpu).eval()
+    fresh.load_state_dict(sd)
+    fresh.capacity_factor, fresh.routing_temperature = layer.capacity_factor, layer.routing_temperature
+    with torch.no_grad():
+        again, _ = fresh(x.to(gpu))
+    assert torch.equal(again, before)
