@@ -11,6 +11,7 @@ from .layers import (  # noqa: F401
     CapacityMoEFFNLayer,
     FusedRMSNorm,
     FusedRoPE,
+    GroupedQueryAttention,
     MoDMoEBlock,
     MoDRouter,
     MoECUDAOps,

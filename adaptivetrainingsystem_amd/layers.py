@@ -12,6 +12,7 @@ MS = Src/Main_Scripts):
   MoECUDAOps             MS/core/moe_cuda_wrapper.py:162-359
   FusedRMSNorm/FusedRoPE/FusedSwiGLU   MS/core/cuda_opt_wrapper.py:261-478
   MoDRouter              MS/core/model.py:860-1020
+  GroupedQueryAttention  MS/core/model.py:561-839 (forward only)
 
 Differences that are deliberate:
   * no PyTorch/CPU fallback: CPU tensors or a missing library raise AtsError
@@ -145,6 +146,71 @@ class FusedRoPE(nn.Module):
         if _wants_grad(q, k):
             return ag.RoPEFunction.apply(q, k, self.cos_cache, self.sin_cache, position_offset)
         return ops.rope(q, k, self.cos_cache, self.sin_cache, position_offset)
+
+
+# ============================================================================ attention
+class GroupedQueryAttention(nn.Module):
+    """Causal grouped-query attention with the reference's constructor fields, parameter names
+    (q_proj / k_proj / v_proj / o_proj, no bias) and forward(x [B, L, hidden]) -> [B, L, hidden]
+    (MS/core/model.py:561-731).  Projections run through the grouped GEMM kernels (one group), RoPE and the
+    attention itself through their HIP kernels; the score matrix is never materialised.
+
+    Not built yet (raise AtsError): extra attention masks, KV cache, dropout, gradients (forward only),
+    float32 inputs."""
+
+    def __init__(self, config):
+        super().__init__()
+        self.config = config
+        self.hidden_size = config.hidden_size
+        self.num_heads = config.num_heads
+        self.num_kv_heads = getattr(config, "num_kv_heads", config.num_heads)
+        self.head_dim = self.hidden_size // self.num_heads
+        self.num_queries_per_kv = self.num_heads // self.num_kv_heads
+        if self.hidden_size % self.num_heads or self.num_heads % self.num_kv_heads:
+            raise AtsError("GroupedQueryAttention: hidden_size % num_heads and num_heads % num_kv_heads must be 0")
+        self.scale = self.head_dim ** -0.5
+        self.q_proj = nn.Linear(self.hidden_size, self.num_heads * self.head_dim, bias=False)
+        self.k_proj = nn.Linear(self.hidden_size, self.num_kv_heads * self.head_dim, bias=False)
+        self.v_proj = nn.Linear(self.hidden_size, self.num_kv_heads * self.head_dim, bias=False)
+        self.o_proj = nn.Linear(self.hidden_size, self.hidden_size, bias=False)
+        self.rope = RotaryEmbedding(self.head_dim, getattr(config, "seq_length", 8192),
+                                    getattr(config, "rope_theta", 10000.0))
+        std = getattr(config, "init_std", 0.02)
+        gain = math.sqrt(2.0 / (5.0 * self.hidden_size))
+        for proj in (self.q_proj, self.k_proj, self.v_proj):
+            nn.init.normal_(proj.weight, mean=0.0, std=std * gain)
+        nn.init.normal_(self.o_proj.weight, mean=0.0, std=std * gain / math.sqrt(2 * getattr(config, "num_layers", 1)))
+        self._param_count = sum(p.numel() for p in self.parameters())
+        self._calls = 0
+
+    def forward(self, x: torch.Tensor, attention_mask: Optional[torch.Tensor] = None, past_key_value=None,
+                use_cache: bool = False):
+        if attention_mask is not None or past_key_value is not None:
+            raise AtsError("GroupedQueryAttention: attention masks and KV caches are not built in the gfx950 path yet")
+        if x.dim() != 3 or x.shape[-1] != self.hidden_size:
+            raise AtsError(f"GroupedQueryAttention: expected [batch, seq, {self.hidden_size}], got {tuple(x.shape)}")
+        if _wants_grad(x, *self.parameters()):
+            raise AtsError("GroupedQueryAttention: forward only (run under torch.no_grad(); the backward kernels "
+                           "of attention are not built yet)")
+        B, L, H = x.shape
+        nh, nkv, D = self.num_heads, self.num_kv_heads, self.head_dim
+        x2 = x.reshape(B * L, H).contiguous()
+        q = ops.linear_nt(x2, _as_dtype(self.q_proj.weight, x.dtype)).view(B, L, nh, D).transpose(1, 2)
+        k = ops.linear_nt(x2, _as_dtype(self.k_proj.weight, x.dtype)).view(B, L, nkv, D).transpose(1, 2)
+        v = ops.linear_nt(x2, _as_dtype(self.v_proj.weight, x.dtype)).view(B, L, nkv, D).transpose(1, 2)
+        cos, sin = self.rope(L, x.device)
+        q, k = ops.rope(q, k, cos, sin, 0)
+        a = ops.causal_attention(q, k, v, self.scale)               # [B, L, nh*D]
+        out = ops.linear_nt(a.view(B * L, nh * D), _as_dtype(self.o_proj.weight, x.dtype)).view(B, L, H)
+        self._calls += 1
+        if use_cache:
+            return out, (k, v.contiguous())
+        return out
+
+    def get_attention_stats(self) -> Dict[str, Any]:
+        return {"total_calls": self._calls, "flash_attention_calls": self._calls, "standard_attention_calls": 0,
+                "flash_attention_ratio": 1.0 if self._calls else 0.0, "num_heads": self.num_heads,
+                "num_kv_heads": self.num_kv_heads, "head_dim": self.head_dim, "parameter_count": self._param_count}
 
 
 # ============================================================================ experts

@@ -260,6 +260,20 @@ int ats_grouped_gemm_nt(const void* a, const void* const* a_ptrs, int64_t lda, i
                         const int32_t* row_count, const int32_t* k_count, int E, int64_t max_rows, int N,
                         int K, int dtype, int out_dtype, ats_stream_t stream);
 
+/* ---- Causal grouped-query attention (forward) -----------------------------------
+ * Replaces GroupedQueryAttention._standard_attention / _flash_attention
+ * (Src/Main_Scripts/core/model.py:757-839): softmax(q.k^T * scale + causal mask) . v with float32
+ * scores and softmax, probabilities rounded to bf16, output laid out [B, L, Hq*D] (the layout o_proj
+ * consumes).  bf16 only, D = 64 or 128, Hq a multiple of Hkv (query head h reads kv head h / (Hq/Hkv)).
+ * q: [B,Hq,L,D], k: [B,Hkv,L,D] contiguous; vt: [B,Hkv,D,Lp] with Lp = ats_attention_padded_len(L),
+ * written by ats_attention_transpose_v from v addressed as base + b*sb + l*sl + h*sh (+ d).
+ * lse (optional): [B,Hq,L] float32 log-sum-exp of the scaled scores per query. */
+int64_t ats_attention_padded_len(int L);
+int ats_attention_transpose_v(const void* v, int64_t sb, int64_t sl, int64_t sh, void* vt, int B, int Hkv, int L,
+                              int D, ats_stream_t stream);
+int ats_attention_fwd(const void* q, const void* k, const void* vt, void* out, float* lse, int B, int Hq, int Hkv,
+                      int L, int D, float scale, ats_stream_t stream);
+
 /* ---- Training-step ops beside the sparse layer --------------------------------
  * Fused cross-entropy + accuracy.  Replaces fused_cross_entropy_accuracy_launcher
  * (Src/Main_Scripts/training/fused_loss.cu:179-214); numerics follow FusedLoss._pytorch_fallback

@@ -48,6 +48,8 @@ PINNING = {
     "swiglu_backward": "torch.autograd of gate*silu(up) in float64; gradcheck",
     "fused_loss": "float64 logsumexp closed form; uniform logits give log(V); torch.autograd for the gradient",
     "clip_grad_norm": "closed form sqrt(sum of squares) and scaling by max_norm/(norm+1e-6)",
+    "attention_standard": "float64 brute force per query (explicit loop over allowed keys); F.scaled_dot_product_attention(is_causal=True)",
+    "gqa_forward": "composition of pinned parts; equals per-head attention with repeat_interleave done by hand",
     "layer_grads": "is torch.autograd over the forward restatements above (what the reference itself trains with); "
                    "gradcheck in float64 on the no-capacity layer with fixed routing",
 }
@@ -497,3 +499,39 @@ def clip_grad_norm(grads, max_norm: float):
     coef = max_norm / (total + 1e-6)
     out = [(g.float() * coef).to(g.dtype) if coef < 1.0 else g.clone() for g in grads]
     return total, out
+
+
+# --------------------------------------------------------------------------- attention
+def attention_standard(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float) -> torch.Tensor:
+    """MS/core/model.py:757-823 (GroupedQueryAttention._standard_attention, no extra mask, no dropout).
+    q [B,H,L,D], k/v [B,H,L,D] (already expanded to H heads).  Scores and softmax in float32, causal
+    positions filled with -1e4, probabilities cast to the input dtype before the second matmul,
+    output [B, L, H*D] in the input dtype."""
+    B, H, L, D = q.shape
+    scores = torch.matmul(q.float(), k.float().transpose(-2, -1)) * scale
+    causal = torch.triu(torch.ones(L, L, dtype=torch.bool), diagonal=1)
+    scores = scores.masked_fill(causal, -1e4)
+    scores = scores - scores.detach().amax(dim=-1, keepdim=True)
+    w = F.softmax(scores, dim=-1, dtype=torch.float32).to(q.dtype)
+    out = torch.matmul(w.float(), v.float()).to(q.dtype)
+    return out.transpose(1, 2).reshape(B, L, H * D)
+
+
+def gqa_forward(x: torch.Tensor, wq: torch.Tensor, wk: torch.Tensor, wv: torch.Tensor, wo: torch.Tensor,
+                num_heads: int, num_kv_heads: int, theta: float = 10000.0) -> torch.Tensor:
+    """MS/core/model.py:663-731 (GroupedQueryAttention.forward without cache): projections (float32
+    accumulation, rounded to the input dtype like nn.Linear), RoPE, KV heads repeated, attention, o_proj."""
+    B, L, H = x.shape
+    D = wq.shape[0] // num_heads
+    lin = lambda a, w: F.linear(a.float(), w.float()).to(a.dtype)
+    q = lin(x, wq).view(B, L, num_heads, D).transpose(1, 2)
+    k = lin(x, wk).view(B, L, num_kv_heads, D).transpose(1, 2)
+    v = lin(x, wv).view(B, L, num_kv_heads, D).transpose(1, 2)
+    cos, sin = rope_table(L, D, theta)
+    q, k = rope_apply(q, k, cos, sin)
+    rep = num_heads // num_kv_heads
+    if rep > 1:
+        k = k.repeat_interleave(rep, dim=1)
+        v = v.repeat_interleave(rep, dim=1)
+    a = attention_standard(q, k, v, D ** -0.5)
+    return lin(a, wo)

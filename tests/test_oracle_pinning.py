@@ -516,3 +516,53 @@ def test_clip_grad_norm_closed_form():
     lib_norm = torch.nn.utils.clip_grad_norm_(params, 1.0)
     assert abs(lib_norm.item() - n.item()) < 1e-5
     assert all(torch.allclose(p_.grad, c, atol=1e-6) for p_, c in zip(params, clipped))
+
+
+# --------------------------------------------------------------------------- attention
+def test_attention_standard_brute_force_and_sdpa():
+    g = torch.Generator().manual_seed(81)
+    B, H, L, D = 2, 3, 11, 8
+    q = torch.randn(B, H, L, D, generator=g)
+    k = torch.randn(B, H, L, D, generator=g)
+    v = torch.randn(B, H, L, D, generator=g)
+    scale = D ** -0.5
+    out = O.attention_standard(q, k, v, scale)
+    ref = torch.zeros(B, L, H, D, dtype=torch.float64)
+    for b in range(B):
+        for h in range(H):
+            for i in range(L):
+                s = torch.tensor([float(q[b, h, i].double() @ k[b, h, j].double()) * scale for j in range(i + 1)],
+                                 dtype=torch.float64)
+                p = torch.exp(s - s.max())
+                p = p / p.sum()
+                ref[b, i, h] = (p.unsqueeze(1) * v[b, h, :i + 1].double()).sum(0)
+    assert torch.allclose(out.double(), ref.reshape(B, L, H * D), atol=1e-5)
+    sdpa = F.scaled_dot_product_attention(q.double(), k.double(), v.double(), is_causal=True)
+    assert torch.allclose(out.double(), sdpa.transpose(1, 2).reshape(B, L, H * D), atol=1e-5)
+    # the first query attends to the first key only
+    assert torch.allclose(out.view(B, L, H, D)[:, 0], v[:, :, 0].transpose(0, 1).transpose(0, 1), atol=1e-6)
+
+
+def test_gqa_forward_matches_per_head_composition():
+    g = torch.Generator().manual_seed(82)
+    B, L, Hd, nh, nkv = 2, 9, 32, 4, 2
+    D = Hd // nh
+    x = torch.randn(B, L, Hd, generator=g)
+    wq = torch.randn(nh * D, Hd, generator=g) * 0.2
+    wk = torch.randn(nkv * D, Hd, generator=g) * 0.2
+    wv = torch.randn(nkv * D, Hd, generator=g) * 0.2
+    wo = torch.randn(Hd, Hd, generator=g) * 0.2
+    out = O.gqa_forward(x, wq, wk, wv, wo, nh, nkv)
+    q = (x @ wq.T).view(B, L, nh, D).transpose(1, 2)
+    k = (x @ wk.T).view(B, L, nkv, D).transpose(1, 2)
+    v = (x @ wv.T).view(B, L, nkv, D).transpose(1, 2)
+    cos, sin = O.rope_table(L, D)
+    q, k = O.rope_apply(q, k, cos, sin)
+    heads = []
+    for h in range(nh):
+        kv = h // (nh // nkv)           # query head h reads kv head h // group size
+        a = F.scaled_dot_product_attention(q[:, h:h + 1].double(), k[:, kv:kv + 1].double(), v[:, kv:kv + 1].double(),
+                                           is_causal=True)
+        heads.append(a[:, 0])
+    ref = torch.cat(heads, dim=-1) @ wo.double().T
+    assert torch.allclose(out.double(), ref, atol=2e-5)
