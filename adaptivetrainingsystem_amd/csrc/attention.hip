@@ -65,11 +65,12 @@ __global__ __launch_bounds__(256) void attention_vt_kernel(const bf16_t* __restr
     }
 }
 
+// One 128-row query tile of one (batch, query head) against its visible keys.
 template <int D>
-__global__ __launch_bounds__(256) void attention_fwd_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
-                                                            const bf16_t* __restrict__ vt, bf16_t* __restrict__ out,
-                                                            float* __restrict__ lse, int Hq, int Hkv, int L, int Lp,
-                                                            float scale_log2) {
+__device__ __forceinline__ void attention_q_tile(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
+                                                 const bf16_t* __restrict__ vt, bf16_t* __restrict__ out,
+                                                 float* __restrict__ lse, int Hq, int Hkv, int L, int Lp,
+                                                 float scale_log2, int qt, int hq, int b, unsigned char* smem) {
     constexpr int KS = D / 16;              // k-steps of the score product
     constexpr int DB = D / 32;              // 32-row blocks of the output (transposed)
     constexpr int KPITCH = D * 2 + 16;      // bytes per K row in LDS
@@ -78,13 +79,10 @@ __global__ __launch_bounds__(256) void attention_fwd_kernel(const bf16_t* __rest
     constexpr int VTILE = D * VPITCH;
     constexpr int KVEC = kAttBN * (D / 8) / 256;   // 16-byte vectors per thread for a K tile
     constexpr int VVEC = D * (kAttBN / 8) / 256;   // and for a V^T tile
-    extern __shared__ __align__(16) unsigned char smem[];   // [2 stages][K tile | V^T tile]
+    // smem: [2 stages][K tile | V^T tile]
 #define ATT_SK(stage_) (smem + (stage_) * (KTILE + VTILE))
 #define ATT_SV(stage_) (smem + (stage_) * (KTILE + VTILE) + KTILE)
 
-    const int n_qt = (L + kAttBM - 1) / kAttBM;
-    const int qt = n_qt - 1 - blockIdx.x;    // longest rows first
-    const int hq = blockIdx.y, b = blockIdx.z;
     const int hkv = hq / (Hq / Hkv);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int col = lane & 31, g = lane >> 5;
@@ -111,119 +109,173 @@ __global__ __launch_bounds__(256) void attention_fwd_kernel(const bf16_t* __rest
     const int q_wave_first = qt * kAttBM + wave * 32;
     const int q_wave_last = q_wave_first + 31;
 
+    // One barrier per key tile: tile t+1 travels global -> registers while tile t is computed and lands in
+    // the other LDS stage at the end of the iteration.  LDS operand fragments are read kRing MFMAs ahead
+    // of their use through a small register ring; without it every MFMA would wait a full LDS round trip.
+    constexpr int kRing = 6;
     au32x4_t rk[KVEC], rv[VVEC];
-    auto load_tile = [&](int t) {
-        const int n0 = t * kAttBN;
+    au32x4_t ring[kRing];
+    af32x16_t acc_s[2];
+
+    {   // tile 0 -> stage 0
 #pragma unroll
         for (int i = 0; i < KVEC; ++i) {
             const int idx = tid + i * 256;
             const int r = idx / (D / 8), c = idx % (D / 8);
-            int key = n0 + r;
-            key = key < L ? key : L - 1;
+            const int key = r < L ? r : L - 1;
             rk[i] = *reinterpret_cast<const au32x4_t*>(kbase + (int64_t)key * D + c * 8);
         }
 #pragma unroll
         for (int i = 0; i < VVEC; ++i) {
             const int idx = tid + i * 256;
             const int d = idx / (kAttBN / 8), c = idx % (kAttBN / 8);
-            rv[i] = *reinterpret_cast<const au32x4_t*>(vbase + (int64_t)d * Lp + n0 + c * 8);
+            rv[i] = *reinterpret_cast<const au32x4_t*>(vbase + (int64_t)d * Lp + c * 8);
         }
-    };
-    auto store_tile = [&](int stage) {
 #pragma unroll
         for (int i = 0; i < KVEC; ++i) {
             const int idx = tid + i * 256;
             const int r = idx / (D / 8), c = idx % (D / 8);
-            *reinterpret_cast<au32x4_t*>(ATT_SK(stage) + r * KPITCH + c * 16) = rk[i];
+            *reinterpret_cast<au32x4_t*>(ATT_SK(0) + r * KPITCH + c * 16) = rk[i];
         }
 #pragma unroll
         for (int i = 0; i < VVEC; ++i) {
             const int idx = tid + i * 256;
             const int d = idx / (kAttBN / 8), c = idx % (kAttBN / 8);
-            // 8-byte halves: the row pitch keeps 8-byte alignment only
-            au32x2_t lo = {rv[i].x, rv[i].y}, hi = {rv[i].z, rv[i].w};
-            *reinterpret_cast<au32x2_t*>(ATT_SV(stage) + d * VPITCH + c * 16) = lo;
-            *reinterpret_cast<au32x2_t*>(ATT_SV(stage) + d * VPITCH + c * 16 + 8) = hi;
+            const au32x2_t lo = {rv[i].x, rv[i].y}, hi = {rv[i].z, rv[i].w};
+            *reinterpret_cast<au32x2_t*>(ATT_SV(0) + d * VPITCH + c * 16) = lo;
+            *reinterpret_cast<au32x2_t*>(ATT_SV(0) + d * VPITCH + c * 16 + 8) = hi;
         }
-    };
+        __syncthreads();
+    }
 
-    load_tile(0);
-    store_tile(0);
-    __syncthreads();
-    for (int t = 0; t < n_tiles; ++t) {
-        const int st = t & 1;
-        const int n0 = t * kAttBN;
-        if (t + 1 < n_tiles) load_tile(t + 1);
-        if (n0 <= q_wave_last) {   // otherwise every key of the tile is in this wave's future
-            // ---- S^T = K . Q^T for 2 blocks of 32 keys
-            af32x16_t acc_s[2];
+    // Pin the query fragments here: loads left pending into the loop make the compiler's wait-count
+    // bookkeeping hold every score MFMA of every iteration behind that iteration's global loads.
 #pragma unroll
-            for (int kb = 0; kb < 2; ++kb) {
+    for (int s = 0; s < KS; ++s) asm volatile("" : "+v"(qf[s]));
+
+    for (int t = 0; t < n_tiles; ++t) {
+        const int n0 = t * kAttBN;
+        const unsigned char* sk = ATT_SK(t & 1);
+        const unsigned char* sv = ATT_SV(t & 1);
+        const bool has_next = t + 1 < n_tiles;
+        if (has_next) {
+            const int n1 = n0 + kAttBN;
+#pragma unroll
+            for (int i = 0; i < KVEC; ++i) {
+                const int idx = tid + i * 256;
+                const int r = idx / (D / 8), c = idx % (D / 8);
+                int key = n1 + r;
+                key = key < L ? key : L - 1;
+                rk[i] = *reinterpret_cast<const au32x4_t*>(kbase + (int64_t)key * D + c * 8);
+            }
+#pragma unroll
+            for (int i = 0; i < VVEC; ++i) {
+                const int idx = tid + i * 256;
+                const int d = idx / (kAttBN / 8), c = idx % (kAttBN / 8);
+                rv[i] = *reinterpret_cast<const au32x4_t*>(vbase + (int64_t)d * Lp + n1 + c * 8);
+            }
+        }
+
+        if (n0 <= q_wave_last) {   // some key of the tile is visible to this wave
+            // ---- S^T = K . Q^T: fragment f = (k-step f/2, key block f%2)
+            const unsigned char* kr = sk + col * KPITCH + g * 16;
+#define ATT_KFRAG(f_) (*reinterpret_cast<const au32x4_t*>(kr + ((f_) & 1) * 32 * KPITCH + ((f_) >> 1) * 32))
+#pragma unroll
+            for (int f = 0; f < kRing; ++f) ring[f] = ATT_KFRAG(f);
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
                 for (int v = 0; v < 16; ++v) acc_s[kb][v] = 0.f;
 #pragma unroll
-                for (int s = 0; s < KS; ++s) {
-                    const au32x4_t kf = *reinterpret_cast<const au32x4_t*>(ATT_SK(st) + (kb * 32 + col) * KPITCH + s * 32 + g * 16);
-                    acc_s[kb] = att_mma(kf, qf[s], acc_s[kb]);
-                }
+            for (int f = 0; f < 2 * KS; ++f) {
+                acc_s[f & 1] = att_mma(ring[f % kRing], qf[f >> 1], acc_s[f & 1]);
+                if (f + kRing < 2 * KS) ring[f % kRing] = ATT_KFRAG(f + kRing);
             }
-            // ---- scale, causal mask, online softmax (log2 domain)
-            const bool need_mask = n0 + kAttBN - 1 > q_wave_first;
-            float mx = m_run;
+#undef ATT_KFRAG
+            // first V^T fragments travel during the softmax: fragment f = (k-step f/DB, output block f%DB)
+            const unsigned char* vr = sv + col * VPITCH + g * 8;
+#define ATT_VFRAG(f_, dst_)                                                                            \
+    {                                                                                                  \
+        const unsigned char* p_ = vr + ((f_) % DB) * 32 * VPITCH + ((f_) / DB) * 32;                   \
+        const au32x2_t lo_ = *reinterpret_cast<const au32x2_t*>(p_);                                   \
+        const au32x2_t hi_ = *reinterpret_cast<const au32x2_t*>(p_ + 16);                              \
+        dst_ = au32x4_t{lo_.x, lo_.y, hi_.x, hi_.y};                                                   \
+    }
 #pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
+            for (int f = 0; f < kRing; ++f) ATT_VFRAG(f, ring[f]);
+
+            if (n0 + kAttBN - 1 > q_wave_first) {   // diagonal tile: causal mask
 #pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    float s2 = acc_s[kb][v] * scale_log2;
-                    if (need_mask) {
+                for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
                         const int key = n0 + kb * 32 + (v >> 2) * 8 + g * 4 + (v & 3);
-                        if (key > q_row) s2 = -INFINITY;
+                        if (key > q_row) acc_s[kb][v] = -INFINITY;
                     }
-                    acc_s[kb][v] = s2;
-                    mx = fmaxf(mx, s2);
-                }
+            }
+            float mx = -INFINITY;
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) mx = fmaxf(mx, acc_s[kb][v]);
             mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-            const float alpha = __builtin_amdgcn_exp2f(m_run - mx);   // 0 on the first tile (m_run = -inf)
+            const float m_new = fmaxf(m_run, mx * scale_log2);   // scale > 0 keeps the order
+            const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);   // 0 on the first tile
             float psum = 0.f;
+            // p = exp2(s * c - m * c): one fused multiply-add per element, c = scale * log2(e)
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
                 for (int v = 0; v < 16; ++v) {
-                    const float p = __builtin_amdgcn_exp2f(acc_s[kb][v] - mx);
+                    const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(acc_s[kb][v], scale_log2, -m_new));
                     acc_s[kb][v] = p;
                     psum += p;
                 }
             l_run = l_run * alpha + psum;
-            m_run = mx;
+            m_run = m_new;
+            if (!__all(alpha == 1.0f)) {   // the running maximum moved for some row of this wave
 #pragma unroll
-            for (int d = 0; d < DB; ++d)
+                for (int d = 0; d < DB; ++d)
 #pragma unroll
-                for (int v = 0; v < 16; ++v) acc_o[d][v] *= alpha;
-            // ---- P^T as B operand: k-step s holds accumulator values 8*(s&1) .. +7 of key block s>>1
+                    for (int v = 0; v < 16; ++v) acc_o[d][v] *= alpha;
+            }
+            // P^T as B operand: k-step s holds accumulator values 8*(s&1) .. +7 of key block s>>1
             au32x4_t pf[4];
 #pragma unroll
-            for (int s = 0; s < 4; ++s) {
-                const int kb = s >> 1, v0 = (s & 1) * 8;
-                pf[s].x = pack_bf16x2(acc_s[kb][v0 + 0], acc_s[kb][v0 + 1]);
-                pf[s].y = pack_bf16x2(acc_s[kb][v0 + 2], acc_s[kb][v0 + 3]);
-                pf[s].z = pack_bf16x2(acc_s[kb][v0 + 4], acc_s[kb][v0 + 5]);
-                pf[s].w = pack_bf16x2(acc_s[kb][v0 + 6], acc_s[kb][v0 + 7]);
+            for (int s_ = 0; s_ < 4; ++s_) {
+                const int kb = s_ >> 1, v0 = (s_ & 1) * 8;
+                pf[s_].x = pack_bf16x2(acc_s[kb][v0 + 0], acc_s[kb][v0 + 1]);
+                pf[s_].y = pack_bf16x2(acc_s[kb][v0 + 2], acc_s[kb][v0 + 3]);
+                pf[s_].z = pack_bf16x2(acc_s[kb][v0 + 4], acc_s[kb][v0 + 5]);
+                pf[s_].w = pack_bf16x2(acc_s[kb][v0 + 6], acc_s[kb][v0 + 7]);
             }
             // ---- O^T += V^T . P^T
 #pragma unroll
-            for (int d = 0; d < DB; ++d) {
-#pragma unroll
-                for (int s = 0; s < 4; ++s) {
-                    const unsigned char* vr = ATT_SV(st) + (d * 32 + col) * VPITCH + (s * 16 + g * 4) * 2;
-                    const au32x2_t lo = *reinterpret_cast<const au32x2_t*>(vr);
-                    const au32x2_t hi = *reinterpret_cast<const au32x2_t*>(vr + 16);
-                    const au32x4_t vf = {lo.x, lo.y, hi.x, hi.y};
-                    acc_o[d] = att_mma(vf, pf[s], acc_o[d]);
-                }
+            for (int f = 0; f < 4 * DB; ++f) {
+                acc_o[f % DB] = att_mma(ring[f % kRing], pf[f / DB], acc_o[f % DB]);
+                if (f + kRing < 4 * DB) ATT_VFRAG(f + kRing, ring[f % kRing]);
             }
+#undef ATT_VFRAG
         }
-        if (t + 1 < n_tiles) {
-            store_tile(st ^ 1);      // the other stage was last read in iteration t-1, before its barrier
+
+        if (has_next) {   // stage (t+1)&1 was last read in iteration t-1, before its closing barrier
+            unsigned char* dk = ATT_SK((t + 1) & 1);
+            unsigned char* dv = ATT_SV((t + 1) & 1);
+#pragma unroll
+            for (int i = 0; i < KVEC; ++i) {
+                const int idx = tid + i * 256;
+                const int r = idx / (D / 8), c = idx % (D / 8);
+                *reinterpret_cast<au32x4_t*>(dk + r * KPITCH + c * 16) = rk[i];
+            }
+#pragma unroll
+            for (int i = 0; i < VVEC; ++i) {
+                const int idx = tid + i * 256;
+                const int d = idx / (kAttBN / 8), c = idx % (kAttBN / 8);
+                // 8-byte halves: the row pitch keeps 8-byte alignment only
+                const au32x2_t lo = {rv[i].x, rv[i].y}, hi = {rv[i].z, rv[i].w};
+                *reinterpret_cast<au32x2_t*>(dv + d * VPITCH + c * 16) = lo;
+                *reinterpret_cast<au32x2_t*>(dv + d * VPITCH + c * 16 + 8) = hi;
+            }
         }
         __syncthreads();
     }
@@ -246,6 +298,42 @@ __global__ __launch_bounds__(256) void attention_fwd_kernel(const bf16_t* __rest
     }
 #undef ATT_SK
 #undef ATT_SV
+}
+
+// Each workgroup takes a long query tile and its mirror-image short one, so every workgroup of a launch
+// does the same work: the hardware hands workgroups to XCDs and shader engines strictly in turn and waits
+// for the next target to have room, so workgroups of uneven length leave whole shader engines idle.
+// Consecutive ids go to different XCDs; the blocks of one (batch, kv head) are kept on one XCD so that
+// its K and V stay in that XCD's L2.  Two waves per SIMD (register budget 256): one wave's softmax runs
+// in the shadow of the other's MFMAs.
+template <int D>
+__global__ __launch_bounds__(256, 2) void attention_fwd_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
+                                                            const bf16_t* __restrict__ vt, bf16_t* __restrict__ out,
+                                                            float* __restrict__ lse, int Hq, int Hkv, int L, int Lp,
+                                                            float scale_log2, int B) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    const int n_qt = (L + kAttBM - 1) / kAttBM;
+    const int n_pairs = (n_qt + 1) / 2;
+    const int per_group = n_pairs * (Hq / Hkv);          // workgroups sharing one K/V
+    const int n_groups = B * Hkv;
+    int group, within;
+    if (n_groups % 8 == 0) {
+        const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
+        group = (idx / per_group) * 8 + xcd;
+        within = idx % per_group;
+    } else {
+        group = blockIdx.x / per_group;
+        within = blockIdx.x % per_group;
+    }
+    const int b = group / Hkv;
+    const int hq = (group % Hkv) * (Hq / Hkv) + within / n_pairs;
+    const int pair = within % n_pairs;
+    const int qt_long = n_qt - 1 - pair;
+#pragma unroll 1
+    for (int half = 0; half < 2; ++half) {
+        if (half && pair == qt_long) break;   // an odd tile count leaves the middle tile on its own
+        attention_q_tile<D>(q, k, vt, out, lse, Hq, Hkv, L, Lp, scale_log2, half ? pair : qt_long, hq, b, smem);
+    }
 }
 
 }  // namespace ats
@@ -281,9 +369,10 @@ extern "C" int ats_attention_fwd(const void* q, const void* k, const void* vt, v
     if (B == 0 || L == 0) return ATS_OK;
     ATS_REQUIRE(q && k && vt && out && aligned16(q) && aligned16(k) && aligned16(vt) && aligned16(out),
                 ATS_ERR_INVALID_ARG, "ats_attention_fwd: null or misaligned pointer");
-    ATS_REQUIRE(Hq <= 65535 && B <= 65535, ATS_ERR_UNSUPPORTED, "ats_attention_fwd: grid");
     const int Lp = (int)ats_attention_padded_len(L);
-    const dim3 grid((unsigned)((L + kAttBM - 1) / kAttBM), (unsigned)Hq, (unsigned)B);
+    const int64_t n_blocks = (int64_t)(((L + kAttBM - 1) / kAttBM + 1) / 2) * Hq * B;
+    ATS_REQUIRE(n_blocks <= 0x7fffffff, ATS_ERR_UNSUPPORTED, "ats_attention_fwd: %lld workgroups", (long long)n_blocks);
+    const dim3 grid((unsigned)n_blocks);
     const float scale_log2 = scale * 1.4426950408889634f;
     if (D == 128) {
         constexpr int smem = 2 * (kAttBN * (128 * 2 + 16) + 128 * (kAttBN * 2 + 8));
@@ -296,12 +385,12 @@ extern "C" int ats_attention_fwd(const void* q, const void* k, const void* vt, v
         }
         hipLaunchKernelGGL((attention_fwd_kernel<128>), grid, dim3(256), smem, as_stream(stream),
                            static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k), static_cast<const bf16_t*>(vt),
-                           static_cast<bf16_t*>(out), lse, Hq, Hkv, L, Lp, scale_log2);
+                           static_cast<bf16_t*>(out), lse, Hq, Hkv, L, Lp, scale_log2, B);
     } else {
         constexpr int smem = 2 * (kAttBN * (64 * 2 + 16) + 64 * (kAttBN * 2 + 8));
         hipLaunchKernelGGL((attention_fwd_kernel<64>), grid, dim3(256), smem, as_stream(stream),
                            static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k), static_cast<const bf16_t*>(vt),
-                           static_cast<bf16_t*>(out), lse, Hq, Hkv, L, Lp, scale_log2);
+                           static_cast<bf16_t*>(out), lse, Hq, Hkv, L, Lp, scale_log2, B);
     }
     ATS_CHECK_LAUNCH("ats_attention_fwd");
     return ATS_OK;

@@ -279,6 +279,53 @@ def run_loss_clip(args):
     return result
 
 
+def run_attention(args):
+    """Causal GQA attention of the headline model shape: B 8, L 2048, 32 query / 8 kv heads, head_dim 128."""
+    from adaptivetrainingsystem_amd import ops
+    from adaptivetrainingsystem_amd.profiling import StageTimer
+    dev = torch.device("cuda:0")
+    B, L, Hq, Hkv, D = 8, 2048, 32, 8, 128
+    torch.manual_seed(6)
+    q = torch.randn(B, Hq, L, D, device=dev).bfloat16()
+    k = torch.randn(B, Hkv, L, D, device=dev).bfloat16()
+    v = torch.randn(B, L, Hkv, D, device=dev).bfloat16().transpose(1, 2)     # view of a projection output
+    for _ in range(args.warmup):
+        ops.causal_attention(q, k, v)
+    torch.cuda.synchronize()
+    timer = StageTimer()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        with timer.range("attention"):
+            out = ops.causal_attention(q, k, v)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    st = timer.summary()
+    flops = 4.0 * B * Hq * D * L * (L + 1) / 2
+    achieved = flops / (st["attention"]["mean_ms"] * 1e-3) / 1e12
+    log(f"  attention (V transpose + kernel) {st['attention']['mean_ms']*1e3:.1f} us -> {achieved:.1f} TFLOP/s "
+        f"({achieved / PEAK_MFMA_BF16_TFLOPS:.1%} of the bf16 MFMA peak)")
+    result = {
+        "metric": "causal GQA attention tokens/s", "value": B * L * args.steps / dt, "unit": "tokens/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": dt / args.steps * 1e3, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"attention: causal GQA forward, batch {B}, seq {L}, {Hq} query / {Hkv} kv heads, head_dim {D}"},
+        "roofline": {"kernel": "attention_fwd_kernel (+ V transpose)", "bound": "mfma", "achieved": achieved,
+                     "peak": PEAK_MFMA_BF16_TFLOPS, "unit": "TFLOP/s", "frac": achieved / PEAK_MFMA_BF16_TFLOPS,
+                     "traffic": None},
+        "stages_ms": {s_: round(v_["mean_ms"], 4) for s_, v_ in st.items()},
+    }
+    if not args.no_cpu_baseline:
+        from oracle import sparse_layer_oracle as O
+        rep = Hq // Hkv
+        qc, kc, vc = q[:1].float().cpu(), k[:1].float().cpu(), v[:1].float().cpu()
+        t0 = time.perf_counter()
+        O.attention_standard(qc, kc.repeat_interleave(rep, dim=1), vc.repeat_interleave(rep, dim=1), D ** -0.5)
+        cdt = time.perf_counter() - t0
+        result["cpu_baseline"] = {"value": L / cdt, "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
+                                  "sample": f"one sequence of the batch ({L} tokens), float32, one pass ({cdt:.2f} s)"}
+    return result
+
+
 def run_norm_rope(args):
     """Config 2: RMSNorm over x[8192, 2048] and RoPE over q[4,16,2048,128], k[4,4,2048,128], bf16."""
     from adaptivetrainingsystem_amd import ops
@@ -372,7 +419,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="c4_prefill",
                     choices=["c4_prefill", "c3_decode", "c5_finegrained_mod", "c1_cpu_reference", "c2_norm_rope",
-                             "c4_prefill_train", "c1_cpu_reference_train", "loss_clip"])
+                             "c4_prefill_train", "c1_cpu_reference_train", "loss_clip", "attention"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a 1 GiB device copy (known traffic) so hardware-counter runs can be scaled")
@@ -399,6 +446,8 @@ def main():
         result = run_norm_rope(args)
     elif args.workload == "loss_clip":
         result = run_loss_clip(args)
+    elif args.workload == "attention":
+        result = run_attention(args)
     elif args.workload.endswith("_train"):
         result = run_train(args)
     else:
