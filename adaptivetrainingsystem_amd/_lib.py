@@ -78,7 +78,7 @@ _SIGNATURES = {
     "ats_attention_transpose_v": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_int, c_int, c_int, c_int,
                                           c_void_p]),
     "ats_attention_fwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
-                                  c_float, c_void_p]),
+                                  c_int, c_float, c_void_p]),
     "ats_combine": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_int,
                             c_void_p]),
     "ats_row_dot": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_int64, c_int, c_int,

@@ -69,7 +69,7 @@ __global__ __launch_bounds__(256) void attention_vt_kernel(const bf16_t* __restr
 template <int D>
 __device__ __forceinline__ void attention_q_tile(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
                                                  const bf16_t* __restrict__ vt, bf16_t* __restrict__ out,
-                                                 float* __restrict__ lse, int Hq, int Hkv, int L, int Lp,
+                                                 float* __restrict__ lse, int Hq, int Hkv, int L, int Lk, int Lp,
                                                  float scale_log2, int qt, int hq, int b, unsigned char* smem) {
     constexpr int KS = D / 16;              // k-steps of the score product
     constexpr int DB = D / 32;              // 32-row blocks of the output (transposed)
@@ -90,7 +90,7 @@ __device__ __forceinline__ void attention_q_tile(const bf16_t* __restrict__ q, c
     const int q_clamped = q_row < L ? q_row : L - 1;
 
     const bf16_t* qp = q + ((int64_t)(b * Hq + hq) * L + q_clamped) * D;
-    const bf16_t* kbase = k + (int64_t)(b * Hkv + hkv) * L * D;
+    const bf16_t* kbase = k + (int64_t)(b * Hkv + hkv) * Lk * D;
     const bf16_t* vbase = vt + (int64_t)(b * Hkv + hkv) * D * Lp;
 
     au32x4_t qf[KS];
@@ -104,9 +104,12 @@ __device__ __forceinline__ void attention_q_tile(const bf16_t* __restrict__ q, c
         for (int v = 0; v < 16; ++v) acc_o[d][v] = 0.f;
     float m_run = -INFINITY, l_run = 0.f;
 
-    const int q_block_last = min(qt * kAttBM + kAttBM - 1, L - 1);
+    // Query i sits at position i + (Lk - L): with cached keys in front the causal diagonal moves right.
+    const int off = Lk - L;
+    const int q_pos = q_row + off;                              // last key this lane's query sees
+    const int q_block_last = min(qt * kAttBM + kAttBM - 1, L - 1) + off;
     const int n_tiles = q_block_last / kAttBN + 1;
-    const int q_wave_first = qt * kAttBM + wave * 32;
+    const int q_wave_first = qt * kAttBM + wave * 32 + off;
     const int q_wave_last = q_wave_first + 31;
 
     // One barrier per key tile: tile t+1 travels global -> registers while tile t is computed and lands in
@@ -122,7 +125,7 @@ __device__ __forceinline__ void attention_q_tile(const bf16_t* __restrict__ q, c
         for (int i = 0; i < KVEC; ++i) {
             const int idx = tid + i * 256;
             const int r = idx / (D / 8), c = idx % (D / 8);
-            const int key = r < L ? r : L - 1;
+            const int key = r < Lk ? r : Lk - 1;
             rk[i] = *reinterpret_cast<const au32x4_t*>(kbase + (int64_t)key * D + c * 8);
         }
 #pragma unroll
@@ -165,7 +168,7 @@ __device__ __forceinline__ void attention_q_tile(const bf16_t* __restrict__ q, c
                 const int idx = tid + i * 256;
                 const int r = idx / (D / 8), c = idx % (D / 8);
                 int key = n1 + r;
-                key = key < L ? key : L - 1;
+                key = key < Lk ? key : Lk - 1;
                 rk[i] = *reinterpret_cast<const au32x4_t*>(kbase + (int64_t)key * D + c * 8);
             }
 #pragma unroll
@@ -190,6 +193,7 @@ __device__ __forceinline__ void attention_q_tile(const bf16_t* __restrict__ q, c
             for (int f = 0; f < 2 * KS; ++f) {
                 acc_s[f & 1] = att_mma(ring[f % kRing], qf[f >> 1], acc_s[f & 1]);
                 if (f + kRing < 2 * KS) ring[f % kRing] = ATT_KFRAG(f + kRing);
+                __builtin_amdgcn_sched_barrier(0);   // keep the reads kRing fragments ahead of their use
             }
 #undef ATT_KFRAG
             // first V^T fragments travel during the softmax: fragment f = (k-step f/DB, output block f%DB)
@@ -203,6 +207,7 @@ __device__ __forceinline__ void attention_q_tile(const bf16_t* __restrict__ q, c
     }
 #pragma unroll
             for (int f = 0; f < kRing; ++f) ATT_VFRAG(f, ring[f]);
+            __builtin_amdgcn_sched_barrier(0);
 
             if (n0 + kAttBN - 1 > q_wave_first) {   // diagonal tile: causal mask
 #pragma unroll
@@ -210,7 +215,7 @@ __device__ __forceinline__ void attention_q_tile(const bf16_t* __restrict__ q, c
 #pragma unroll
                     for (int v = 0; v < 16; ++v) {
                         const int key = n0 + kb * 32 + (v >> 2) * 8 + g * 4 + (v & 3);
-                        if (key > q_row) acc_s[kb][v] = -INFINITY;
+                        if (key > q_pos) acc_s[kb][v] = -INFINITY;
                     }
             }
             float mx = -INFINITY;
@@ -254,6 +259,7 @@ __device__ __forceinline__ void attention_q_tile(const bf16_t* __restrict__ q, c
             for (int f = 0; f < 4 * DB; ++f) {
                 acc_o[f % DB] = att_mma(ring[f % kRing], pf[f / DB], acc_o[f % DB]);
                 if (f + kRing < 4 * DB) ATT_VFRAG(f + kRing, ring[f % kRing]);
+                __builtin_amdgcn_sched_barrier(0);
             }
 #undef ATT_VFRAG
         }
@@ -309,7 +315,7 @@ __device__ __forceinline__ void attention_q_tile(const bf16_t* __restrict__ q, c
 template <int D>
 __global__ __launch_bounds__(256, 2) void attention_fwd_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
                                                             const bf16_t* __restrict__ vt, bf16_t* __restrict__ out,
-                                                            float* __restrict__ lse, int Hq, int Hkv, int L, int Lp,
+                                                            float* __restrict__ lse, int Hq, int Hkv, int L, int Lk, int Lp,
                                                             float scale_log2, int B) {
     extern __shared__ __align__(16) unsigned char smem[];
     const int n_qt = (L + kAttBM - 1) / kAttBM;
@@ -332,7 +338,7 @@ __global__ __launch_bounds__(256, 2) void attention_fwd_kernel(const bf16_t* __r
 #pragma unroll 1
     for (int half = 0; half < 2; ++half) {
         if (half && pair == qt_long) break;   // an odd tile count leaves the middle tile on its own
-        attention_q_tile<D>(q, k, vt, out, lse, Hq, Hkv, L, Lp, scale_log2, half ? pair : qt_long, hq, b, smem);
+        attention_q_tile<D>(q, k, vt, out, lse, Hq, Hkv, L, Lk, Lp, scale_log2, half ? pair : qt_long, hq, b, smem);
     }
 }
 
@@ -361,15 +367,15 @@ extern "C" int ats_attention_transpose_v(const void* v, int64_t sb, int64_t sl, 
 }
 
 extern "C" int ats_attention_fwd(const void* q, const void* k, const void* vt, void* out, float* lse, int B, int Hq,
-                                 int Hkv, int L, int D, float scale, ats_stream_t stream) {
+                                 int Hkv, int L, int Lk, int D, float scale, ats_stream_t stream) {
     using namespace ats;
-    ATS_REQUIRE(B >= 0 && Hq > 0 && Hkv > 0 && Hq % Hkv == 0 && L >= 0 && scale > 0.f, ATS_ERR_INVALID_ARG,
-                "ats_attention_fwd: B=%d Hq=%d Hkv=%d L=%d scale=%g", B, Hq, Hkv, L, scale);
+    ATS_REQUIRE(B >= 0 && Hq > 0 && Hkv > 0 && Hq % Hkv == 0 && L >= 0 && Lk >= L && scale > 0.f, ATS_ERR_INVALID_ARG,
+                "ats_attention_fwd: B=%d Hq=%d Hkv=%d L=%d Lk=%d scale=%g", B, Hq, Hkv, L, Lk, scale);
     ATS_REQUIRE(D == 64 || D == 128, ATS_ERR_UNSUPPORTED, "ats_attention_fwd: head_dim %d (64 or 128)", D);
     if (B == 0 || L == 0) return ATS_OK;
     ATS_REQUIRE(q && k && vt && out && aligned16(q) && aligned16(k) && aligned16(vt) && aligned16(out),
                 ATS_ERR_INVALID_ARG, "ats_attention_fwd: null or misaligned pointer");
-    const int Lp = (int)ats_attention_padded_len(L);
+    const int Lp = (int)ats_attention_padded_len(Lk);
     const int64_t n_blocks = (int64_t)(((L + kAttBM - 1) / kAttBM + 1) / 2) * Hq * B;
     ATS_REQUIRE(n_blocks <= 0x7fffffff, ATS_ERR_UNSUPPORTED, "ats_attention_fwd: %lld workgroups", (long long)n_blocks);
     const dim3 grid((unsigned)n_blocks);
@@ -385,12 +391,12 @@ extern "C" int ats_attention_fwd(const void* q, const void* k, const void* vt, v
         }
         hipLaunchKernelGGL((attention_fwd_kernel<128>), grid, dim3(256), smem, as_stream(stream),
                            static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k), static_cast<const bf16_t*>(vt),
-                           static_cast<bf16_t*>(out), lse, Hq, Hkv, L, Lp, scale_log2, B);
+                           static_cast<bf16_t*>(out), lse, Hq, Hkv, L, Lk, Lp, scale_log2, B);
     } else {
         constexpr int smem = 2 * (kAttBN * (64 * 2 + 16) + 64 * (kAttBN * 2 + 8));
         hipLaunchKernelGGL((attention_fwd_kernel<64>), grid, dim3(256), smem, as_stream(stream),
                            static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k), static_cast<const bf16_t*>(vt),
-                           static_cast<bf16_t*>(out), lse, Hq, Hkv, L, Lp, scale_log2, B);
+                           static_cast<bf16_t*>(out), lse, Hq, Hkv, L, Lk, Lp, scale_log2, B);
     }
     ATS_CHECK_LAUNCH("ats_attention_fwd");
     return ATS_OK;

@@ -185,8 +185,8 @@ class GroupedQueryAttention(nn.Module):
 
     def forward(self, x: torch.Tensor, attention_mask: Optional[torch.Tensor] = None, past_key_value=None,
                 use_cache: bool = False):
-        if attention_mask is not None or past_key_value is not None:
-            raise AtsError("GroupedQueryAttention: attention masks and KV caches are not built in the gfx950 path yet")
+        if attention_mask is not None:
+            raise AtsError("GroupedQueryAttention: padding masks are not built in the gfx950 path")
         if x.dim() != 3 or x.shape[-1] != self.hidden_size:
             raise AtsError(f"GroupedQueryAttention: expected [batch, seq, {self.hidden_size}], got {tuple(x.shape)}")
         if _wants_grad(x, *self.parameters()):
@@ -198,8 +198,16 @@ class GroupedQueryAttention(nn.Module):
         q = ops.linear_nt(x2, _as_dtype(self.q_proj.weight, x.dtype)).view(B, L, nh, D).transpose(1, 2)
         k = ops.linear_nt(x2, _as_dtype(self.k_proj.weight, x.dtype)).view(B, L, nkv, D).transpose(1, 2)
         v = ops.linear_nt(x2, _as_dtype(self.v_proj.weight, x.dtype)).view(B, L, nkv, D).transpose(1, 2)
+        # positions 0..L-1 also when a cache is passed, as the reference does (model.py:690-698)
         cos, sin = self.rope(L, x.device)
         q, k = ops.rope(q, k, cos, sin, 0)
+        if past_key_value is not None:
+            k_cache, v_cache = past_key_value
+            if (k_cache.dim() != 4 or k_cache.shape[0] != B or k_cache.shape[1] != nkv or k_cache.shape[3] != D
+                    or v_cache.shape != k_cache.shape):
+                raise AtsError(f"GroupedQueryAttention: cache shapes {tuple(k_cache.shape)} / {tuple(v_cache.shape)}")
+            k = torch.cat([k_cache.to(k.dtype), k], dim=2)
+            v = torch.cat([v_cache.to(v.dtype), v], dim=2)
         a = ops.causal_attention(q, k, v, self.scale)               # [B, L, nh*D]
         out = ops.linear_nt(a.view(B * L, nh * D), _as_dtype(self.o_proj.weight, x.dtype)).view(B, L, H)
         self._calls += 1

@@ -563,28 +563,29 @@ def grouped_gemm_nt(b_ptrs: torch.Tensor, ldb: int, b_rows: int, row_start: torc
 # --------------------------------------------------------------------------- attention
 def causal_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: Optional[float] = None,
                      return_lse: bool = False):
-    """Causal grouped-query attention.  q [B,Hq,L,D], k [B,Hkv,L,D] (made contiguous), v [B,Hkv,L,D] in any
-    batch/head/position strides (e.g. a view of a fused projection output); bf16, D 64 or 128.
+    """Causal grouped-query attention.  q [B,Hq,L,D], k [B,Hkv,Lk,D] (made contiguous), v [B,Hkv,Lk,D] in any
+    batch/head/position strides (e.g. a view of a fused projection output); bf16, D 64 or 128, Lk >= L.
+    With Lk > L the leading Lk - L keys are a cache: query i sits at position i + Lk - L.
     Returns out [B, L, Hq*D] (and lse [B,Hq,L] float32 if asked)."""
     _need_gpu(q, k, v)
     if q.dim() != 4 or k.dim() != 4 or v.dim() != 4 or q.dtype != torch.bfloat16 or k.dtype != q.dtype or v.dtype != q.dtype:
         raise AtsError("causal_attention: q, k, v must be 4-D bfloat16 tensors [batch, heads, seq, head_dim]")
     B, Hq, L, D = q.shape
-    Hkv = k.shape[1]
-    if k.shape != (B, Hkv, L, D) or v.shape != (B, Hkv, L, D) or Hq % Hkv != 0:
+    Hkv, Lk = k.shape[1], k.shape[2]
+    if k.shape != (B, Hkv, Lk, D) or v.shape != (B, Hkv, Lk, D) or Hq % Hkv != 0 or Lk < L:
         raise AtsError(f"causal_attention: shapes q {tuple(q.shape)} k {tuple(k.shape)} v {tuple(v.shape)}")
     q, k = q.contiguous(), k.contiguous()
     if v.stride(3) != 1 or any(st % 8 for st in v.stride()[:3]) or v.data_ptr() % 16:
         v = v.contiguous()
     lib = _lib.load()
-    Lp = int(lib.ats_attention_padded_len(L))
+    Lp = int(lib.ats_attention_padded_len(Lk))
     vt = torch.empty(B, Hkv, D, Lp, dtype=q.dtype, device=q.device)
-    check(lib.ats_attention_transpose_v(v.data_ptr(), v.stride(0), v.stride(2), v.stride(1), vt.data_ptr(), B, Hkv, L, D,
+    check(lib.ats_attention_transpose_v(v.data_ptr(), v.stride(0), v.stride(2), v.stride(1), vt.data_ptr(), B, Hkv, Lk, D,
                                         _stream()), "ats_attention_transpose_v")
     out = torch.empty(B, L, Hq * D, dtype=q.dtype, device=q.device)
     lse = torch.empty(B, Hq, L, dtype=torch.float32, device=q.device) if return_lse else None
-    check(lib.ats_attention_fwd(q.data_ptr(), k.data_ptr(), vt.data_ptr(), out.data_ptr(), _ptr(lse), B, Hq, Hkv, L, D,
-                                float(D ** -0.5 if scale is None else scale), _stream()), "ats_attention_fwd")
+    check(lib.ats_attention_fwd(q.data_ptr(), k.data_ptr(), vt.data_ptr(), out.data_ptr(), _ptr(lse), B, Hq, Hkv, L, Lk,
+                                D, float(D ** -0.5 if scale is None else scale), _stream()), "ats_attention_fwd")
     return (out, lse) if return_lse else out
 
 

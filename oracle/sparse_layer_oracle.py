@@ -504,12 +504,17 @@ def clip_grad_norm(grads, max_norm: float):
 # --------------------------------------------------------------------------- attention
 def attention_standard(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float) -> torch.Tensor:
     """MS/core/model.py:757-823 (GroupedQueryAttention._standard_attention, no extra mask, no dropout).
-    q [B,H,L,D], k/v [B,H,L,D] (already expanded to H heads).  Scores and softmax in float32, causal
-    positions filled with -1e4, probabilities cast to the input dtype before the second matmul,
-    output [B, L, H*D] in the input dtype."""
+    q [B,H,L,D], k/v [B,H,Lk,D] (already expanded to H heads), Lk >= L.  Scores and softmax in float32,
+    causal positions filled with -1e4, probabilities cast to the input dtype before the second matmul,
+    output [B, L, H*D] in the input dtype.
+    With cached keys in front (Lk > L, model.py:700-704) query i sits at position i + Lk - L.  The
+    reference's own [L, L] mask only broadcasts against [L, Lk] scores for L = 1 (one new token, which
+    then sees every key); the diagonal used here is that case's generalisation, and equals what slicing
+    the last L query rows out of a full-length call gives."""
     B, H, L, D = q.shape
+    Lk = k.shape[2]
     scores = torch.matmul(q.float(), k.float().transpose(-2, -1)) * scale
-    causal = torch.triu(torch.ones(L, L, dtype=torch.bool), diagonal=1)
+    causal = torch.triu(torch.ones(L, Lk, dtype=torch.bool), diagonal=1 + Lk - L)
     scores = scores.masked_fill(causal, -1e4)
     scores = scores - scores.detach().amax(dim=-1, keepdim=True)
     w = F.softmax(scores, dim=-1, dtype=torch.float32).to(q.dtype)
@@ -518,9 +523,12 @@ def attention_standard(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale:
 
 
 def gqa_forward(x: torch.Tensor, wq: torch.Tensor, wk: torch.Tensor, wv: torch.Tensor, wo: torch.Tensor,
-                num_heads: int, num_kv_heads: int, theta: float = 10000.0) -> torch.Tensor:
-    """MS/core/model.py:663-731 (GroupedQueryAttention.forward without cache): projections (float32
-    accumulation, rounded to the input dtype like nn.Linear), RoPE, KV heads repeated, attention, o_proj."""
+                num_heads: int, num_kv_heads: int, theta: float = 10000.0, past_key_value=None,
+                use_cache: bool = False):
+    """MS/core/model.py:663-731 (GroupedQueryAttention.forward): projections (float32 accumulation,
+    rounded to the input dtype like nn.Linear), RoPE at positions 0..L-1 (also with a cache, 690-698),
+    cached keys/values concatenated in front (700-704), KV heads repeated, attention, o_proj.
+    Returns the output, and the (k, v) cache as well when use_cache is set (706-708, 729-731)."""
     B, L, H = x.shape
     D = wq.shape[0] // num_heads
     lin = lambda a, w: F.linear(a.float(), w.float()).to(a.dtype)
@@ -529,9 +537,14 @@ def gqa_forward(x: torch.Tensor, wq: torch.Tensor, wk: torch.Tensor, wv: torch.T
     v = lin(x, wv).view(B, L, num_kv_heads, D).transpose(1, 2)
     cos, sin = rope_table(L, D, theta)
     q, k = rope_apply(q, k, cos, sin)
+    if past_key_value is not None:
+        k = torch.cat([past_key_value[0], k], dim=2)
+        v = torch.cat([past_key_value[1], v], dim=2)
+    cache = (k, v)
     rep = num_heads // num_kv_heads
     if rep > 1:
         k = k.repeat_interleave(rep, dim=1)
         v = v.repeat_interleave(rep, dim=1)
     a = attention_standard(q, k, v, D ** -0.5)
-    return lin(a, wo)
+    out = lin(a, wo)
+    return (out, cache) if use_cache else out

@@ -49,6 +49,40 @@ def test_causal_attention(ops, gpu, B, Hq, Hkv, L, D):
     assert torch.equal(out2, out)
 
 
+@pytest.mark.parametrize("B,Hq,Hkv,L,Lk,D", [(2, 4, 2, 1, 200, 128), (1, 2, 1, 1, 1, 64), (1, 4, 4, 70, 300, 64),
+                                             (2, 8, 2, 129, 130, 128), (1, 2, 2, 256, 1024, 128), (1, 4, 1, 5, 64, 128)])
+def test_causal_attention_with_cached_keys(ops, gpu, B, Hq, Hkv, L, Lk, D):
+    """Lk - L cached keys in front of the queries: query i sees keys 0 .. i + Lk - L."""
+    print("case cached attention", B, Hq, Hkv, L, Lk, D, flush=True)
+    g = gen(94)
+    q = torch.randn(B, Hq, L, D, generator=g).bfloat16()
+    k = torch.randn(B, Hkv, Lk, D, generator=g).bfloat16()
+    v = torch.randn(B, Hkv, Lk, D, generator=g).bfloat16()
+    rep = Hq // Hkv
+    ref = O.attention_standard(q, k.repeat_interleave(rep, dim=1), v.repeat_interleave(rep, dim=1), D ** -0.5)
+    out, lse = ops.causal_attention(q.to(gpu), k.to(gpu), v.to(gpu), return_lse=True)
+    assert out.shape == (B, L, Hq * D)
+    assert rel_err(out, ref) <= BF16_TOL
+    s = torch.matmul(q.float(), k.repeat_interleave(rep, dim=1).float().transpose(-2, -1)) * D ** -0.5
+    s = s.masked_fill(torch.triu(torch.ones(L, Lk, dtype=torch.bool), diagonal=1 + Lk - L), float("-inf"))
+    assert rel_err(lse, torch.logsumexp(s, -1)) <= 1e-4
+
+
+def test_cached_attention_equals_tail_of_full_call(ops, gpu):
+    """Size-independent property at a long length: the last L rows of a full call, bit for bit per row tile
+    alignment aside -- compared at the bf16 bar since tiles start at different keys."""
+    g = gen(95)
+    B, Hq, Hkv, Lk, D, L = 1, 8, 2, 4096, 128, 1024
+    q = torch.randn(B, Hq, Lk, D, generator=g).bfloat16().to(gpu)
+    k = torch.randn(B, Hkv, Lk, D, generator=g).bfloat16().to(gpu)
+    v = torch.randn(B, Hkv, Lk, D, generator=g).bfloat16().to(gpu)
+    full = ops.causal_attention(q, k, v)
+    tail = ops.causal_attention(q[:, :, Lk - L:], k, v)
+    assert rel_err(tail, full[:, Lk - L:]) <= 1e-6      # same keys, same tile walk: identical arithmetic
+    with pytest.raises(Exception):
+        ops.causal_attention(q, k[:, :, :100], v[:, :, :100])          # fewer keys than queries
+
+
 def test_attention_is_causal(ops, gpu):
     """Changing keys / values at later positions must not change earlier outputs (bit for bit)."""
     g = gen(92)
@@ -85,3 +119,17 @@ def test_gqa_module(gpu, hidden, nh, nkv, B, L):
     assert set(att.state_dict()) == {f"{n}.weight" for n in ("q_proj", "k_proj", "v_proj", "o_proj")}
     with pytest.raises(A.AtsError):
         att(x.to(gpu).requires_grad_())
+    # prefill with use_cache, then two single-token steps fed from the cache (model.py:700-708)
+    w = [getattr(att, n).weight.detach().cpu() for n in ("q_proj", "k_proj", "v_proj", "o_proj")]
+    with torch.no_grad():
+        out_c, cache = att(x.to(gpu), use_cache=True)
+    ref_c, ref_cache = O.gqa_forward(x, *w, nh, nkv, use_cache=True)
+    assert torch.equal(out_c, out) and rel_err(cache[0], ref_cache[0]) <= BF16_TOL
+    assert rel_err(cache[1], ref_cache[1]) <= BF16_TOL
+    for step in range(2):
+        x1 = torch.randn(B, 1, hidden, generator=gen(96 + step)).bfloat16()
+        with torch.no_grad():
+            o1, cache = att(x1.to(gpu), past_key_value=cache, use_cache=True)
+        r1, ref_cache = O.gqa_forward(x1, *w, nh, nkv, past_key_value=ref_cache, use_cache=True)
+        assert cache[0].shape == (B, nkv, L + 1 + step, hidden // nh)
+        assert rel_err(o1, r1) <= BF16_TOL

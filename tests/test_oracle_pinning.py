@@ -543,6 +543,49 @@ def test_attention_standard_brute_force_and_sdpa():
     assert torch.allclose(out.view(B, L, H, D)[:, 0], v[:, :, 0].transpose(0, 1).transpose(0, 1), atol=1e-6)
 
 
+def test_attention_standard_with_cached_keys():
+    """Keys in front of the queries: the last L rows of a full-length call, one new token seeing every key
+    (the only cached case the reference's own mask admits), and a brute-force sum."""
+    g = torch.Generator().manual_seed(83)
+    B, H, Lk, D = 2, 2, 13, 8
+    q = torch.randn(B, H, Lk, D, generator=g)
+    k = torch.randn(B, H, Lk, D, generator=g)
+    v = torch.randn(B, H, Lk, D, generator=g)
+    scale = D ** -0.5
+    full = O.attention_standard(q, k, v, scale).view(B, Lk, H, D)
+    for L in (1, 4, 12):
+        part = O.attention_standard(q[:, :, Lk - L:], k, v, scale).view(B, L, H, D)
+        assert torch.allclose(part, full[:, Lk - L:], atol=1e-6)
+    one = O.attention_standard(q[:, :, -1:], k, v, scale).view(B, H, D)
+    p = torch.softmax(torch.einsum("bhd,bhjd->bhj", q[:, :, -1].double(), k.double()) * scale, -1)
+    assert torch.allclose(one.double(), torch.einsum("bhj,bhjd->bhd", p, v.double()), atol=1e-5)
+
+
+def test_gqa_forward_cache_round_trip():
+    """use_cache returns the rotated keys and the values; feeding them back with new tokens reproduces the
+    reference's quirk of rotating the new tokens at positions 0..L-1 (model.py:690-698)."""
+    g = torch.Generator().manual_seed(84)
+    B, L, Hd, nh, nkv = 1, 6, 16, 4, 2
+    D = Hd // nh
+    x = torch.randn(B, L, Hd, generator=g)
+    w = [torch.randn(n, Hd, generator=g) * 0.3 for n in (nh * D, nkv * D, nkv * D, Hd)]
+    out, (kc, vc) = O.gqa_forward(x, *w, nh, nkv, use_cache=True)
+    assert kc.shape == (B, nkv, L, D) and vc.shape == (B, nkv, L, D)
+    assert torch.equal(out, O.gqa_forward(x, *w, nh, nkv))
+    x1 = torch.randn(B, 1, Hd, generator=g)
+    out1, (kc1, vc1) = O.gqa_forward(x1, *w, nh, nkv, past_key_value=(kc, vc), use_cache=True)
+    assert kc1.shape == (B, nkv, L + 1, D) and torch.equal(kc1[:, :, :L], kc) and torch.equal(vc1[:, :, :L], vc)
+    # the new token's key is rotated at position 0, i.e. not rotated at all
+    k_new = (x1 @ w[1].T).view(B, 1, nkv, D).transpose(1, 2)
+    assert torch.allclose(kc1[:, :, L:], k_new, atol=1e-6)
+    q_new = (x1 @ w[0].T).view(B, 1, nh, D).transpose(1, 2)
+    rep = nh // nkv
+    p = torch.softmax(torch.einsum("bhd,bhjd->bhj", q_new[:, :, 0].double(),
+                                   kc1.repeat_interleave(rep, 1).double()) * D ** -0.5, -1)
+    a = torch.einsum("bhj,bhjd->bhd", p, vc1.repeat_interleave(rep, 1).double()).reshape(B, 1, nh * D)
+    assert torch.allclose(out1.double(), a @ w[3].double().T, atol=2e-5)
+
+
 def test_gqa_forward_matches_per_head_composition():
     g = torch.Generator().manual_seed(82)
     B, L, Hd, nh, nkv = 2, 9, 32, 4, 2
