@@ -214,13 +214,24 @@ def invert_token_map(token_map: torch.Tensor, n_assign: int) -> torch.Tensor:
 
 
 # --------------------------------------------------------------------------- expert FFN
+_pointer_table_cache: dict = {}
+
+
 def weight_pointer_table(weights: Sequence[torch.Tensor]) -> torch.Tensor:
     """Device array of the experts' weight base addresses (int64)."""
     for w in weights:
         _need_gpu(w)
         if not w.is_contiguous():
             raise AtsError("expert weights must be contiguous")
-    return torch.tensor([w.data_ptr() for w in weights], dtype=torch.int64, device=weights[0].device)
+    # the table holds nothing but the addresses it is keyed by, so an entry can never go stale
+    key = (weights[0].device,) + tuple(w.data_ptr() for w in weights)
+    table = _pointer_table_cache.get(key)
+    if table is None:
+        if len(_pointer_table_cache) > 256:
+            _pointer_table_cache.clear()
+        table = torch.tensor(key[1:], dtype=torch.int64, device=weights[0].device)
+        _pointer_table_cache[key] = table
+    return table
 
 
 def grouped_gateup_swiglu(a: torch.Tensor, w_gu_ptrs: torch.Tensor, row_start: torch.Tensor, row_count: torch.Tensor,
@@ -589,6 +600,22 @@ def causal_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: O
     return (out, lse) if return_lse else out
 
 
+_single_group_cache: dict = {}
+
+
+def _single_group(T: int, device: torch.device):
+    """row_start = [0], row_count = [T] of a one-group GEMM, kept per (T, device): two fill launches
+    per call are a visible share of a small projection."""
+    key = (T, device)
+    hit = _single_group_cache.get(key)
+    if hit is None:
+        if len(_single_group_cache) > 64:
+            _single_group_cache.clear()
+        hit = (torch.zeros(1, dtype=torch.int32, device=device), torch.full((1,), T, dtype=torch.int32, device=device))
+        _single_group_cache[key] = hit
+    return hit
+
+
 def linear_nt(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
     """x [T, K] @ weight[N, K]^T through the grouped GEMM kernels with a single group."""
     _need_gpu(x, weight)
@@ -597,6 +624,5 @@ def linear_nt(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
     T, K = x.shape
     N = weight.shape[0]
     x, weight = x.contiguous(), weight.contiguous()
-    start = torch.zeros(1, dtype=torch.int32, device=x.device)
-    count = torch.full((1,), T, dtype=torch.int32, device=x.device)
+    start, count = _single_group(T, x.device)
     return grouped_gemm_nt(weight_pointer_table([weight]), K, N, start, count, T, T, N, K, a=x)

@@ -326,6 +326,59 @@ def run_attention(args):
     return result
 
 
+def run_gqa_layer(args):
+    """The attention sub-layer of the headline model shape (hidden 4096, 32 query / 8 kv heads, head_dim 128) on
+    batch 8 x seq 2048: q/k/v projections, RoPE, causal attention, output projection."""
+    import adaptivetrainingsystem_amd as A
+    from adaptivetrainingsystem_amd.workloads import LayerConfig
+    from adaptivetrainingsystem_amd.profiling import StageTimer
+    dev = torch.device("cuda:0")
+    B, L, H, Hq, Hkv = 8, 2048, 4096, 32, 8
+    D = H // Hq
+    torch.manual_seed(7)
+    cfg = LayerConfig(H, 14336, 8, 2, num_heads=Hq, num_kv_heads=Hkv, seq_length=L)
+    att = A.GroupedQueryAttention(cfg).to(torch.bfloat16).to(dev).eval()
+    x = torch.randn(B, L, H, device=dev).bfloat16()
+    timer = StageTimer()
+    with torch.no_grad():
+        for _ in range(args.warmup):
+            att(x)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            with timer.range("gqa_layer"):
+                att(x)
+        torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    st = timer.summary()
+    T = B * L
+    flops = 2.0 * T * H * (Hq * D + 2 * Hkv * D + H) + 4.0 * B * Hq * D * L * (L + 1) / 2
+    achieved = flops / (st["gqa_layer"]["mean_ms"] * 1e-3) / 1e12
+    log(f"  attention sub-layer {st['gqa_layer']['mean_ms']:.3f} ms -> {achieved:.1f} TFLOP/s over projections + attention "
+        f"({achieved / PEAK_MFMA_BF16_TFLOPS:.1%} of the bf16 MFMA peak)")
+    result = {
+        "metric": "GQA attention sub-layer tokens/s", "value": T * args.steps / dt, "unit": "tokens/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": dt / args.steps * 1e3, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"gqa_layer: q/k/v/o projections + RoPE + causal attention, batch {B}, seq {L}, hidden {H}, "
+                               f"{Hq} query / {Hkv} kv heads"},
+        "roofline": {"kernel": "whole sub-layer (4 projection GEMMs + attention_fwd_kernel)", "bound": "mfma",
+                     "achieved": achieved, "peak": PEAK_MFMA_BF16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": achieved / PEAK_MFMA_BF16_TFLOPS, "traffic": None},
+        "stages_ms": {s_: round(v_["mean_ms"], 4) for s_, v_ in st.items()},
+    }
+    if not args.no_cpu_baseline:
+        from oracle import sparse_layer_oracle as O
+        w = [getattr(att, n).weight.detach().float().cpu() for n in ("q_proj", "k_proj", "v_proj", "o_proj")]
+        xc = x[:1].float().cpu()
+        t0 = time.perf_counter()
+        O.gqa_forward(xc, *w, Hq, Hkv)
+        cdt = time.perf_counter() - t0
+        result["cpu_baseline"] = {"value": L / cdt, "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
+                                  "sample": f"one sequence of the batch ({L} tokens), float32, one pass ({cdt:.2f} s)"}
+    return result
+
+
 def run_norm_rope(args):
     """Config 2: RMSNorm over x[8192, 2048] and RoPE over q[4,16,2048,128], k[4,4,2048,128], bf16."""
     from adaptivetrainingsystem_amd import ops
@@ -419,7 +472,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="c4_prefill",
                     choices=["c4_prefill", "c3_decode", "c5_finegrained_mod", "c1_cpu_reference", "c2_norm_rope",
-                             "c4_prefill_train", "c1_cpu_reference_train", "loss_clip", "attention"])
+                             "c4_prefill_train", "c1_cpu_reference_train", "loss_clip", "attention", "gqa_layer"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a 1 GiB device copy (known traffic) so hardware-counter runs can be scaled")
@@ -448,6 +501,8 @@ def main():
         result = run_loss_clip(args)
     elif args.workload == "attention":
         result = run_attention(args)
+    elif args.workload == "gqa_layer":
+        result = run_gqa_layer(args)
     elif args.workload.endswith("_train"):
         result = run_train(args)
     else:
