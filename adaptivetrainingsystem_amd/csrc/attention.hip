@@ -97,6 +97,24 @@ __device__ __forceinline__ void attention_q_tile(const bf16_t* __restrict__ q, c
 #pragma unroll
     for (int s = 0; s < KS; ++s) qf[s] = *reinterpret_cast<const au32x4_t*>(qp + s * 16 + g * 8);
 
+    // K and V^T tiles come through buffer loads: a scalar base and tile offset plus one 32-bit lane offset
+    // that never changes, so a tile costs no address arithmetic, and keys past Lk read as zeros.
+    const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<bf16_t*>(kbase), 0, (int)((int64_t)Lk * D * 2), 0x00020000);
+    const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<bf16_t*>(vbase), 0, (int)((int64_t)D * Lp * 2), 0x00020000);
+    int k_lane[KVEC], v_lane[VVEC];
+#pragma unroll
+    for (int i = 0; i < KVEC; ++i) {
+        const int idx = tid + i * 256;
+        k_lane[i] = ((idx / (D / 8)) * D + (idx % (D / 8)) * 8) * 2;
+    }
+#pragma unroll
+    for (int i = 0; i < VVEC; ++i) {
+        const int idx = tid + i * 256;
+        v_lane[i] = ((idx / (kAttBN / 8)) * Lp + (idx % (kAttBN / 8)) * 8) * 2;
+    }
+
     af32x16_t acc_o[DB];
 #pragma unroll
     for (int d = 0; d < DB; ++d)
@@ -122,18 +140,9 @@ __device__ __forceinline__ void attention_q_tile(const bf16_t* __restrict__ q, c
 
     {   // tile 0 -> stage 0
 #pragma unroll
-        for (int i = 0; i < KVEC; ++i) {
-            const int idx = tid + i * 256;
-            const int r = idx / (D / 8), c = idx % (D / 8);
-            const int key = r < Lk ? r : Lk - 1;
-            rk[i] = *reinterpret_cast<const au32x4_t*>(kbase + (int64_t)key * D + c * 8);
-        }
+        for (int i = 0; i < KVEC; ++i) rk[i] = __builtin_amdgcn_raw_buffer_load_b128(k_rsrc, k_lane[i], 0, 0);
 #pragma unroll
-        for (int i = 0; i < VVEC; ++i) {
-            const int idx = tid + i * 256;
-            const int d = idx / (kAttBN / 8), c = idx % (kAttBN / 8);
-            rv[i] = *reinterpret_cast<const au32x4_t*>(vbase + (int64_t)d * Lp + c * 8);
-        }
+        for (int i = 0; i < VVEC; ++i) rv[i] = __builtin_amdgcn_raw_buffer_load_b128(v_rsrc, v_lane[i], 0, 0);
 #pragma unroll
         for (int i = 0; i < KVEC; ++i) {
             const int idx = tid + i * 256;
@@ -164,19 +173,11 @@ __device__ __forceinline__ void attention_q_tile(const bf16_t* __restrict__ q, c
         if (has_next) {
             const int n1 = n0 + kAttBN;
 #pragma unroll
-            for (int i = 0; i < KVEC; ++i) {
-                const int idx = tid + i * 256;
-                const int r = idx / (D / 8), c = idx % (D / 8);
-                int key = n1 + r;
-                key = key < Lk ? key : Lk - 1;
-                rk[i] = *reinterpret_cast<const au32x4_t*>(kbase + (int64_t)key * D + c * 8);
-            }
+            for (int i = 0; i < KVEC; ++i)
+                rk[i] = __builtin_amdgcn_raw_buffer_load_b128(k_rsrc, k_lane[i], n1 * D * 2, 0);
 #pragma unroll
-            for (int i = 0; i < VVEC; ++i) {
-                const int idx = tid + i * 256;
-                const int d = idx / (kAttBN / 8), c = idx % (kAttBN / 8);
-                rv[i] = *reinterpret_cast<const au32x4_t*>(vbase + (int64_t)d * Lp + n1 + c * 8);
-            }
+            for (int i = 0; i < VVEC; ++i)
+                rv[i] = __builtin_amdgcn_raw_buffer_load_b128(v_rsrc, v_lane[i], n1 * 2, 0);
         }
 
         if (n0 <= q_wave_last) {   // some key of the tile is visible to this wave
@@ -344,7 +345,14 @@ __global__ __launch_bounds__(256, 2) void attention_fwd_kernel(const bf16_t* __r
 
 }  // namespace ats
 
-extern "C" int64_t ats_attention_padded_len(int L) { return ((int64_t)L + ats::kAttBN - 1) / ats::kAttBN * ats::kAttBN; }
+// Row length of V^T: whole key tiles, and a row pitch of an odd multiple of 256 bytes.  A key tile reads the
+// same 128 bytes of every row of V^T; with a power-of-two pitch (4096 bytes at 2048 keys) all those rows
+// sit in one L2 channel, which then serves every workgroup of the (batch, kv head) on its own.
+extern "C" int64_t ats_attention_padded_len(int L) {
+    int64_t tiles = ((int64_t)L + ats::kAttBN - 1) / ats::kAttBN;
+    while (tiles % 4 != 2) ++tiles;
+    return tiles * ats::kAttBN;
+}
 
 extern "C" int ats_attention_transpose_v(const void* v, int64_t sb, int64_t sl, int64_t sh, void* vt, int B, int Hkv,
                                          int L, int D, ats_stream_t stream) {
@@ -376,6 +384,8 @@ extern "C" int ats_attention_fwd(const void* q, const void* k, const void* vt, v
     ATS_REQUIRE(q && k && vt && out && aligned16(q) && aligned16(k) && aligned16(vt) && aligned16(out),
                 ATS_ERR_INVALID_ARG, "ats_attention_fwd: null or misaligned pointer");
     const int Lp = (int)ats_attention_padded_len(Lk);
+    ATS_REQUIRE((int64_t)Lp * D * 2 < 0x7fffffffLL, ATS_ERR_UNSUPPORTED,
+                "ats_attention_fwd: %d keys (one head's K or V must stay under 2 GiB)", Lk);
     const int64_t n_blocks = (int64_t)(((L + kAttBM - 1) / kAttBM + 1) / 2) * Hq * B;
     ATS_REQUIRE(n_blocks <= 0x7fffffff, ATS_ERR_UNSUPPORTED, "ats_attention_fwd: %lld workgroups", (long long)n_blocks);
     const dim3 grid((unsigned)n_blocks);
