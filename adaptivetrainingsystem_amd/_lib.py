@@ -79,6 +79,8 @@ _SIGNATURES = {
                                           c_void_p]),
     "ats_attention_fwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
                                   c_int, c_float, c_void_p]),
+    "ats_attention_delta": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
+    "ats_attention_bwd": (c_int, [c_void_p] * 12 + [c_int] * 6 + [c_float, c_void_p]),
     "ats_combine": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_int,
                             c_void_p]),
     "ats_row_dot": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_int64, c_int, c_int,

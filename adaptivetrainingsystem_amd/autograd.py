@@ -55,6 +55,64 @@ class RoPEFunction(Function):
         return gq, gk, None, None, None
 
 
+class AttentionFunction(Function):
+    """Causal grouped-query attention: q [B,Hq,L,D], k, v [B,Hkv,Lk,D] -> [B, L, Hq*D]."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, scale):
+        q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+        out, lse = ops.causal_attention(q, k, v, scale, return_lse=True)
+        ctx.save_for_backward(q, k, v, out, lse)
+        ctx.scale = scale
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        q, k, v, out, lse = ctx.saved_tensors
+        dq, dk, dv = ops.causal_attention_bwd(q, k, v, out, lse, dout, ctx.scale)
+        return dq, dk, dv, None
+
+
+class LinearFunction(Function):
+    """y = x @ weight^T for x [T, K], weight [N, K] (a bias-free nn.Linear) through the grouped GEMM kernels
+    with one group: dgrad multiplies by a transposed copy of the weight, wgrad multiplies the transposed
+    activations."""
+
+    @staticmethod
+    def forward(ctx, x, weight):
+        x = x.contiguous()
+        w = weight.detach().to(x.dtype).contiguous()
+        ctx.save_for_backward(x, w)
+        ctx.param_dtype = weight.dtype
+        return ops.linear_nt(x, w)
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, w = ctx.saved_tensors
+        T, K = x.shape
+        N = w.shape[0]
+        dy = dy.to(x.dtype).contiguous()
+        dx = dw = None
+        offsets = torch.tensor([0, T], dtype=torch.int32, device=x.device)
+        kept = offsets[1:].clone()
+        if ctx.needs_input_grad[0]:
+            wT, tab = ops.transpose_batched([w])                 # [K, N]; kept alive until the GEMM is queued
+            dx = ops.grouped_gemm_nt(tab, N, K, offsets, kept, T, T, K, N, a=dy)
+        if ctx.needs_input_grad[1]:
+            ks, kc = ops.wgrad_plan(kept)
+            ld = ops.wgrad_padded_rows(T, 1)
+            dyT = ops.transpose_grouped_rows(dy, offsets, kept, T)
+            xT = ops.transpose_grouped_rows(x, offsets, kept, T)
+            es = x.element_size()
+            a_ptrs = ks.long() * es + dyT.data_ptr()
+            b_ptrs = ks.long() * es + xT.data_ptr()
+            rs = torch.zeros(1, dtype=torch.int32, device=x.device)
+            rc = torch.full((1,), N, dtype=torch.int32, device=x.device)
+            dw = ops.grouped_gemm_nt(b_ptrs, ld, K, rs, rc, N, N, K, ld, a_ptrs=a_ptrs, lda=ld, k_count=kc,
+                                     dtype=x.dtype, out_dtype=x.dtype).to(ctx.param_dtype)
+        return dx, dw
+
+
 class SwiGLUFunction(Function):
     """out = gate * silu(up) (the dense-FFN convention of the fused wrapper)."""
 

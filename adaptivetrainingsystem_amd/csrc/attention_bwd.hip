@@ -1,0 +1,567 @@
+// Backward of the causal grouped-query attention for gfx950 (bf16, head_dim 64 or 128).
+//
+// Gradient of GroupedQueryAttention._standard_attention / _flash_attention of the reference
+// (Src/Main_Scripts/core/model.py:757-839), which the reference leaves to autograd.  With
+// P = softmax(q.k^T * scale + causal mask) (float32) and delta_i = sum_d dO[i,d] * O[i,d]:
+//     dV = P^T . dO        dP = dO . V^T        dS = P * (dP - delta) * scale
+//     dQ = dS . K          dK = dS^T . Q
+// P is recomputed from the saved log-sum-exp, the [L, Lk] matrices are never materialised, and nothing is
+// accumulated with atomics: one kernel owns query rows and walks the keys (dQ), the other owns keys and
+// walks the queries of every query head of its kv head (dK, dV), so every output element is summed by
+// one lane in a fixed order.
+//
+// Same MFMA layout trick as the forward: products are formed transposed so that a lane of the 32x32
+// accumulator owns one row of the side the block owns (a query in the dQ kernel, a key in the dK/dV
+// kernel).  The operand that changes from step to step is read from LDS as the A operand along its
+// contiguous dimension; the transposed copies this needs (K^T for dQ, Q^T and dO^T for dK/dV) are made
+// once per call by the transpose kernel of the forward.
+#include <math.h>
+
+#include "ats_common.hpp"
+
+namespace ats {
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bbf16x8_t;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float bf32x16_t;
+typedef unsigned int bu32x4_t __attribute__((ext_vector_type(4)));
+typedef unsigned int bu32x2_t __attribute__((ext_vector_type(2)));
+
+constexpr int kBwdRows = 128;   // rows a block owns: 4 waves x 32
+constexpr int kDqBN = 64;       // keys per step of the dQ kernel
+constexpr int kDkvBQ = 32;      // queries per step of the dK/dV kernel
+constexpr float kLog2e = 1.4426950408889634f;
+
+__device__ __forceinline__ bf32x16_t bwd_mma(const bu32x4_t& a, const bu32x4_t& b, bf32x16_t c) {
+    union {
+        bu32x4_t u;
+        bbf16x8_t v;
+    } x, y;
+    x.u = a;
+    y.u = b;
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(x.v, y.v, c, 0, 0, 0);
+}
+
+// delta[b, h, i] = sum_d dO[b, i, h, d] * O[b, i, h, d]; out and dout are [B, L, Hq*D].
+template <int D>
+__global__ __launch_bounds__(256) void attention_delta_kernel(const bf16_t* __restrict__ out,
+                                                              const bf16_t* __restrict__ dout,
+                                                              float* __restrict__ delta, int Hq, int L, int64_t rows) {
+    constexpr int TPR = D / 8;   // threads per (token, head) row
+    const int64_t row = (int64_t)blockIdx.x * (256 / TPR) + threadIdx.x / TPR;   // index over [B, L, Hq]
+    float s = 0.f;
+    if (row < rows) {
+        const int64_t off = row * D + (threadIdx.x % TPR) * 8;
+        const uint4 a = *reinterpret_cast<const uint4*>(out + off);
+        const uint4 b = *reinterpret_cast<const uint4*>(dout + off);
+        float fa[8], fb[8];
+        Elem<bf16_t>::unpack(a, fa);
+        Elem<bf16_t>::unpack(b, fb);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) s += fa[j] * fb[j];
+    }
+#pragma unroll
+    for (int o = TPR / 2; o > 0; o >>= 1) s += __shfl_xor(s, o, 64);
+    if (row < rows && threadIdx.x % TPR == 0) {
+        const int64_t h = row % Hq, bl = row / Hq;
+        const int64_t b = bl / L, i = bl % L;
+        delta[(b * Hq + h) * L + i] = s;
+    }
+}
+
+// ------------------------------------------------------------------------------------------ dQ
+// One 128-row query tile of one (batch, query head): lanes own queries, keys come in tiles of 64.
+template <int D>
+__device__ __forceinline__ void attention_bwd_dq_tile(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
+                                                      const bf16_t* __restrict__ v, const bf16_t* __restrict__ kt,
+                                                      const bf16_t* __restrict__ dout, const float* __restrict__ lse,
+                                                      const float* __restrict__ delta, bf16_t* __restrict__ dq, int Hq,
+                                                      int Hkv, int L, int Lk, int Lp, float scale, int qt, int hq,
+                                                      int b, unsigned char* smem) {
+    constexpr int KS = D / 16;
+    constexpr int DB = D / 32;
+    constexpr int RPITCH = D * 2 + 16;        // bytes per K / V row in LDS
+    constexpr int TPITCH = kDqBN * 2 + 8;     // bytes per K^T row in LDS
+    constexpr int RTILE = kDqBN * RPITCH;
+    constexpr int RVEC = kDqBN * (D / 8) / 256;
+    constexpr int TVEC = D * (kDqBN / 8) / 256;
+    unsigned char* const sK = smem;
+    unsigned char* const sV = smem + RTILE;
+    unsigned char* const sT = smem + 2 * RTILE;
+
+    const int hkv = hq / (Hq / Hkv);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int col = lane & 31, g = lane >> 5;
+    const int q_row = qt * kBwdRows + wave * 32 + col;
+    const int q_clamped = q_row < L ? q_row : L - 1;
+    const int off = Lk - L;
+    const int q_pos = q_row + off;
+    const float scale_log2 = scale * kLog2e;
+
+    const bf16_t* qp = q + ((int64_t)(b * Hq + hq) * L + q_clamped) * D;
+    const bf16_t* dop = dout + ((int64_t)b * L + q_clamped) * (int64_t)(Hq * D) + hq * D;
+    bu32x4_t qf[KS], dof[KS];
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+        qf[s] = *reinterpret_cast<const bu32x4_t*>(qp + s * 16 + g * 8);
+        dof[s] = *reinterpret_cast<const bu32x4_t*>(dop + s * 16 + g * 8);
+    }
+    const float lse2 = lse[(int64_t)(b * Hq + hq) * L + q_clamped] * kLog2e;
+    const float dl = delta[(int64_t)(b * Hq + hq) * L + q_clamped];
+
+    const bf16_t* kbase = k + (int64_t)(b * Hkv + hkv) * Lk * D;
+    const bf16_t* vbase = v + (int64_t)(b * Hkv + hkv) * Lk * D;
+    const bf16_t* tbase = kt + (int64_t)(b * Hkv + hkv) * D * Lp;
+    // buffer loads: keys past Lk read as zeros
+    const __amdgpu_buffer_rsrc_t k_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(kbase), 0, (int)((int64_t)Lk * D * 2), 0x00020000);
+    const __amdgpu_buffer_rsrc_t v_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(vbase), 0, (int)((int64_t)Lk * D * 2), 0x00020000);
+    const __amdgpu_buffer_rsrc_t t_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(tbase), 0, (int)((int64_t)D * Lp * 2), 0x00020000);
+
+    bf32x16_t acc_dq[DB];
+#pragma unroll
+    for (int d = 0; d < DB; ++d)
+#pragma unroll
+        for (int x = 0; x < 16; ++x) acc_dq[d][x] = 0.f;
+
+    const int q_block_last = min(qt * kBwdRows + kBwdRows - 1, L - 1) + off;
+    const int n_tiles = q_block_last / kDqBN + 1;
+    const int q_wave_first = qt * kBwdRows + wave * 32 + off;
+    const int q_wave_last = q_wave_first + 31;
+
+#pragma unroll
+    for (int s = 0; s < KS; ++s) asm volatile("" : "+v"(qf[s]), "+v"(dof[s]));
+
+    for (int t = 0; t < n_tiles; ++t) {
+        const int n0 = t * kDqBN;
+        __syncthreads();   // every wave is done with the previous tile
+        {
+            bu32x4_t rk[RVEC], rv[RVEC], rt[TVEC];
+#pragma unroll
+            for (int i = 0; i < RVEC; ++i) {
+                const int idx = tid + i * 256;
+                const int lo = ((idx / (D / 8)) * D + (idx % (D / 8)) * 8) * 2;
+                rk[i] = __builtin_amdgcn_raw_buffer_load_b128(k_rsrc, lo, n0 * D * 2, 0);
+                rv[i] = __builtin_amdgcn_raw_buffer_load_b128(v_rsrc, lo, n0 * D * 2, 0);
+            }
+#pragma unroll
+            for (int i = 0; i < TVEC; ++i) {
+                const int idx = tid + i * 256;
+                const int lo = ((idx / (kDqBN / 8)) * Lp + (idx % (kDqBN / 8)) * 8) * 2;
+                rt[i] = __builtin_amdgcn_raw_buffer_load_b128(t_rsrc, lo, n0 * 2, 0);
+            }
+#pragma unroll
+            for (int i = 0; i < RVEC; ++i) {
+                const int idx = tid + i * 256;
+                const int r = idx / (D / 8), c = idx % (D / 8);
+                *reinterpret_cast<bu32x4_t*>(sK + r * RPITCH + c * 16) = rk[i];
+                *reinterpret_cast<bu32x4_t*>(sV + r * RPITCH + c * 16) = rv[i];
+            }
+#pragma unroll
+            for (int i = 0; i < TVEC; ++i) {
+                const int idx = tid + i * 256;
+                const int d = idx / (kDqBN / 8), c = idx % (kDqBN / 8);
+                const bu32x2_t lo = {rt[i].x, rt[i].y}, hi = {rt[i].z, rt[i].w};
+                *reinterpret_cast<bu32x2_t*>(sT + d * TPITCH + c * 16) = lo;
+                *reinterpret_cast<bu32x2_t*>(sT + d * TPITCH + c * 16 + 8) = hi;
+            }
+        }
+        __syncthreads();
+        if (n0 > q_wave_last) continue;   // every key of the tile is in this wave's future
+
+        // ---- S^T = K . Q^T and dP^T = V . dO^T
+        bf32x16_t acc_s[2], acc_p[2];
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int x = 0; x < 16; ++x) {
+                acc_s[kb][x] = 0.f;
+                acc_p[kb][x] = 0.f;
+            }
+#pragma unroll
+        for (int s = 0; s < KS; ++s)
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb) {
+                const int o = (kb * 32 + col) * RPITCH + s * 32 + g * 16;
+                acc_s[kb] = bwd_mma(*reinterpret_cast<const bu32x4_t*>(sK + o), qf[s], acc_s[kb]);
+                acc_p[kb] = bwd_mma(*reinterpret_cast<const bu32x4_t*>(sV + o), dof[s], acc_p[kb]);
+            }
+        // ---- dS^T = P^T * (dP^T - delta) * scale, with P^T = exp(S^T * scale - lse)
+        const bool diagonal = n0 + kDqBN - 1 > q_wave_first;
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int x = 0; x < 16; ++x) {
+                float p = __builtin_amdgcn_exp2f(__builtin_fmaf(acc_s[kb][x], scale_log2, -lse2));
+                if (diagonal) {
+                    const int key = n0 + kb * 32 + (x >> 2) * 8 + g * 4 + (x & 3);
+                    if (key > q_pos) p = 0.f;
+                }
+                acc_s[kb][x] = p * (acc_p[kb][x] - dl) * scale;
+            }
+        bu32x4_t dsf[4];
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            const int kb = s >> 1, x0 = (s & 1) * 8;
+            dsf[s].x = pack_bf16x2(acc_s[kb][x0 + 0], acc_s[kb][x0 + 1]);
+            dsf[s].y = pack_bf16x2(acc_s[kb][x0 + 2], acc_s[kb][x0 + 3]);
+            dsf[s].z = pack_bf16x2(acc_s[kb][x0 + 4], acc_s[kb][x0 + 5]);
+            dsf[s].w = pack_bf16x2(acc_s[kb][x0 + 6], acc_s[kb][x0 + 7]);
+        }
+        // ---- dQ^T += K^T . dS^T  (keys of a k-step in accumulator order, as in the forward's second product)
+#pragma unroll
+        for (int s = 0; s < 4; ++s)
+#pragma unroll
+            for (int d = 0; d < DB; ++d) {
+                const unsigned char* tr = sT + (d * 32 + col) * TPITCH + (s * 16 + g * 4) * 2;
+                const bu32x2_t lo = *reinterpret_cast<const bu32x2_t*>(tr);
+                const bu32x2_t hi = *reinterpret_cast<const bu32x2_t*>(tr + 16);
+                acc_dq[d] = bwd_mma(bu32x4_t{lo.x, lo.y, hi.x, hi.y}, dsf[s], acc_dq[d]);
+            }
+    }
+
+    if (q_row < L) {
+        bf16_t* drow = dq + ((int64_t)(b * Hq + hq) * L + q_row) * D;
+#pragma unroll
+        for (int d = 0; d < DB; ++d)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                bu32x2_t w;
+                w.x = pack_bf16x2(acc_dq[d][r * 4 + 0], acc_dq[d][r * 4 + 1]);
+                w.y = pack_bf16x2(acc_dq[d][r * 4 + 2], acc_dq[d][r * 4 + 3]);
+                *reinterpret_cast<bu32x2_t*>(drow + d * 32 + r * 8 + g * 4) = w;
+            }
+    }
+}
+
+// A workgroup takes a long query tile and its mirror-image short one (equal work per workgroup: the
+// hardware hands workgroups out strictly in turn), and the workgroups of one (batch, kv head) share an XCD.
+template <int D>
+__global__ __launch_bounds__(256, 2) void attention_bwd_dq_kernel(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const bf16_t* __restrict__ v,
+    const bf16_t* __restrict__ kt, const bf16_t* __restrict__ dout, const float* __restrict__ lse,
+    const float* __restrict__ delta, bf16_t* __restrict__ dq, int Hq, int Hkv, int L, int Lk, int Lp, float scale,
+    int B) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    const int n_qt = (L + kBwdRows - 1) / kBwdRows;
+    const int n_pairs = (n_qt + 1) / 2;
+    const int per_group = n_pairs * (Hq / Hkv);
+    const int n_groups = B * Hkv;
+    int group, within;
+    if (n_groups % 8 == 0) {
+        const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
+        group = (idx / per_group) * 8 + xcd;
+        within = idx % per_group;
+    } else {
+        group = blockIdx.x / per_group;
+        within = blockIdx.x % per_group;
+    }
+    const int b = group / Hkv;
+    const int hq = (group % Hkv) * (Hq / Hkv) + within / n_pairs;
+    const int pair = within % n_pairs;
+    const int qt_long = n_qt - 1 - pair;
+#pragma unroll 1
+    for (int half = 0; half < 2; ++half) {
+        if (half && pair == qt_long) break;
+        attention_bwd_dq_tile<D>(q, k, v, kt, dout, lse, delta, dq, Hq, Hkv, L, Lk, Lp, scale, half ? pair : qt_long,
+                                 hq, b, smem);
+    }
+}
+
+// ------------------------------------------------------------------------------------------ dK, dV
+// One 128-row key tile of one (batch, kv head): lanes own keys; the queries of every query head of the
+// group come in steps of 32, starting at the first query that sees the tile.
+template <int D>
+__device__ __forceinline__ void attention_bwd_dkv_tile(const bf16_t* __restrict__ q, const bf16_t* __restrict__ qtr,
+                                                       const bf16_t* __restrict__ k, const bf16_t* __restrict__ v,
+                                                       const bf16_t* __restrict__ dout, const bf16_t* __restrict__ dotr,
+                                                       const float* __restrict__ lse, const float* __restrict__ delta,
+                                                       bf16_t* __restrict__ dk, bf16_t* __restrict__ dv, int Hq, int Hkv,
+                                                       int L, int Lk, int Lqp, float scale, int kt_idx, int hkv, int b,
+                                                       unsigned char* smem) {
+    constexpr int KS = D / 16;
+    constexpr int DB = D / 32;
+    constexpr int RPITCH = D * 2 + 16;        // bytes per Q / dO row in LDS
+    constexpr int TPITCH = kDkvBQ * 2 + 8;    // bytes per Q^T / dO^T row in LDS
+    constexpr int RTILE = kDkvBQ * RPITCH;
+    constexpr int TTILE = D * TPITCH;
+    constexpr int RVEC = kDkvBQ * (D / 8) / 256;   // 16-byte vectors per thread: D=128 -> 2, D=64 -> 1
+    constexpr int TVEC = D * (kDkvBQ / 8) / 256;   // D=128 -> 2, D=64 -> 1
+    unsigned char* const sQ = smem;
+    unsigned char* const sO = smem + RTILE;
+    unsigned char* const sQT = smem + 2 * RTILE;
+    unsigned char* const sOT = smem + 2 * RTILE + TTILE;
+    float* const sL = reinterpret_cast<float*>(smem + 2 * RTILE + 2 * TTILE);   // [32] lse * log2(e)
+    float* const sD = sL + kDkvBQ;                                             // [32] delta
+
+    const int rep = Hq / Hkv;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int col = lane & 31, g = lane >> 5;
+    const int key_row = kt_idx * kBwdRows + wave * 32 + col;
+    const int key_clamped = key_row < Lk ? key_row : Lk - 1;
+    const int off = Lk - L;
+    const float scale_log2 = scale * kLog2e;
+
+    const bf16_t* kp = k + ((int64_t)(b * Hkv + hkv) * Lk + key_clamped) * D;
+    const bf16_t* vp = v + ((int64_t)(b * Hkv + hkv) * Lk + key_clamped) * D;
+    bu32x4_t kf[KS], vf[KS];
+#pragma unroll
+    for (int s = 0; s < KS; ++s) {
+        kf[s] = *reinterpret_cast<const bu32x4_t*>(kp + s * 16 + g * 8);
+        vf[s] = *reinterpret_cast<const bu32x4_t*>(vp + s * 16 + g * 8);
+    }
+#pragma unroll
+    for (int s = 0; s < KS; ++s) asm volatile("" : "+v"(kf[s]), "+v"(vf[s]));
+
+    bf32x16_t acc_dk[DB], acc_dv[DB];
+#pragma unroll
+    for (int d = 0; d < DB; ++d)
+#pragma unroll
+        for (int x = 0; x < 16; ++x) {
+            acc_dk[d][x] = 0.f;
+            acc_dv[d][x] = 0.f;
+        }
+
+    const int key_block_first = kt_idx * kBwdRows;
+    const int key_wave_first = key_block_first + wave * 32;
+    const int key_wave_last = key_wave_first + 31;
+    // first query that sees any key of the block: q + off >= key_block_first
+    const int q_first = max(key_block_first - off, 0) / kDkvBQ * kDkvBQ;
+
+    for (int hh = 0; hh < rep; ++hh) {
+        const int hq = hkv * rep + hh;
+        const bf16_t* qbase = q + (int64_t)(b * Hq + hq) * L * D;
+        const bf16_t* obase = dout + (int64_t)b * L * (int64_t)(Hq * D) + hq * D;
+        const bf16_t* qtbase = qtr + (int64_t)(b * Hq + hq) * D * Lqp;
+        const bf16_t* otbase = dotr + (int64_t)(b * Hq + hq) * D * Lqp;
+        const float* lbase = lse + (int64_t)(b * Hq + hq) * L;
+        const float* dbase = delta + (int64_t)(b * Hq + hq) * L;
+        // buffer loads: query rows past L read as zeros
+        const __amdgpu_buffer_rsrc_t q_rsrc =
+            __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(qbase), 0, (int)((int64_t)L * D * 2), 0x00020000);
+        const __amdgpu_buffer_rsrc_t o_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+            const_cast<bf16_t*>(obase), 0, (int)((((int64_t)L - 1) * Hq * D + D) * 2), 0x00020000);
+        const __amdgpu_buffer_rsrc_t qt_rsrc =
+            __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(qtbase), 0, (int)((int64_t)D * Lqp * 2), 0x00020000);
+        const __amdgpu_buffer_rsrc_t ot_rsrc =
+            __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(otbase), 0, (int)((int64_t)D * Lqp * 2), 0x00020000);
+
+        for (int q0 = q_first; q0 < L; q0 += kDkvBQ) {
+            __syncthreads();   // every wave is done with the previous step
+            {
+                bu32x4_t rq[RVEC], ro[RVEC], rqt[TVEC], rot[TVEC];
+#pragma unroll
+                for (int i = 0; i < RVEC; ++i) {
+                    const int idx = tid + i * 256;
+                    const int r = idx / (D / 8), c = idx % (D / 8);
+                    rq[i] = __builtin_amdgcn_raw_buffer_load_b128(q_rsrc, (r * D + c * 8) * 2, q0 * D * 2, 0);
+                    ro[i] = __builtin_amdgcn_raw_buffer_load_b128(o_rsrc, (r * Hq * D + c * 8) * 2, q0 * Hq * D * 2, 0);
+                }
+#pragma unroll
+                for (int i = 0; i < TVEC; ++i) {
+                    const int idx = tid + i * 256;
+                    const int d = idx / (kDkvBQ / 8), c = idx % (kDkvBQ / 8);
+                    rqt[i] = __builtin_amdgcn_raw_buffer_load_b128(qt_rsrc, (d * Lqp + c * 8) * 2, q0 * 2, 0);
+                    rot[i] = __builtin_amdgcn_raw_buffer_load_b128(ot_rsrc, (d * Lqp + c * 8) * 2, q0 * 2, 0);
+                }
+                if (tid < kDkvBQ) {
+                    const int qi = q0 + tid;
+                    sL[tid] = qi < L ? lbase[qi] * kLog2e : INFINITY;   // exp2(-inf) = 0 for rows past L
+                    sD[tid] = qi < L ? dbase[qi] : 0.f;
+                }
+#pragma unroll
+                for (int i = 0; i < RVEC; ++i) {
+                    const int idx = tid + i * 256;
+                    const int r = idx / (D / 8), c = idx % (D / 8);
+                    *reinterpret_cast<bu32x4_t*>(sQ + r * RPITCH + c * 16) = rq[i];
+                    *reinterpret_cast<bu32x4_t*>(sO + r * RPITCH + c * 16) = ro[i];
+                }
+#pragma unroll
+                for (int i = 0; i < TVEC; ++i) {
+                    const int idx = tid + i * 256;
+                    const int d = idx / (kDkvBQ / 8), c = idx % (kDkvBQ / 8);
+                    const bu32x2_t a0 = {rqt[i].x, rqt[i].y}, a1 = {rqt[i].z, rqt[i].w};
+                    const bu32x2_t b0 = {rot[i].x, rot[i].y}, b1 = {rot[i].z, rot[i].w};
+                    *reinterpret_cast<bu32x2_t*>(sQT + d * TPITCH + c * 16) = a0;
+                    *reinterpret_cast<bu32x2_t*>(sQT + d * TPITCH + c * 16 + 8) = a1;
+                    *reinterpret_cast<bu32x2_t*>(sOT + d * TPITCH + c * 16) = b0;
+                    *reinterpret_cast<bu32x2_t*>(sOT + d * TPITCH + c * 16 + 8) = b1;
+                }
+            }
+            __syncthreads();
+            if (q0 + kDkvBQ - 1 + off < key_wave_first) continue;   // no query of the step sees this wave's keys
+
+            // ---- S = Q . K^T and dP = dO . V^T  (rows = queries of the step, column = this lane's key)
+            bf32x16_t acc_s, acc_p;
+#pragma unroll
+            for (int x = 0; x < 16; ++x) {
+                acc_s[x] = 0.f;
+                acc_p[x] = 0.f;
+            }
+#pragma unroll
+            for (int s = 0; s < KS; ++s) {
+                const int o = col * RPITCH + s * 32 + g * 16;
+                acc_s = bwd_mma(*reinterpret_cast<const bu32x4_t*>(sQ + o), kf[s], acc_s);
+                acc_p = bwd_mma(*reinterpret_cast<const bu32x4_t*>(sO + o), vf[s], acc_p);
+            }
+            // ---- P = exp(S * scale - lse[q]); dS = P * (dP - delta[q]) * scale; accumulator row x is
+            //      query (x / 4) * 8 + g * 4 + x % 4 of the step
+            const bool diagonal = q0 + off < key_wave_last;
+            bu32x4_t pf[2], dsf[2];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const float4 l4 = *reinterpret_cast<const float4*>(sL + r * 8 + g * 4);
+                const float4 d4 = *reinterpret_cast<const float4*>(sD + r * 8 + g * 4);
+                const float lv[4] = {l4.x, l4.y, l4.z, l4.w};
+                const float dvv[4] = {d4.x, d4.y, d4.z, d4.w};
+                float p[4], ds[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int x = r * 4 + j;
+                    float pv = __builtin_amdgcn_exp2f(__builtin_fmaf(acc_s[x], scale_log2, -lv[j]));
+                    if (diagonal) {
+                        const int qi = q0 + r * 8 + g * 4 + j;
+                        if (key_row > qi + off) pv = 0.f;
+                    }
+                    p[j] = pv;
+                    ds[j] = pv * (acc_p[x] - dvv[j]) * scale;
+                }
+                // k-step s of the second products holds accumulator values 8s .. 8s+7
+                const unsigned p01 = pack_bf16x2(p[0], p[1]), p23 = pack_bf16x2(p[2], p[3]);
+                const unsigned s01 = pack_bf16x2(ds[0], ds[1]), s23 = pack_bf16x2(ds[2], ds[3]);
+                if (r == 0) { pf[0].x = p01; pf[0].y = p23; dsf[0].x = s01; dsf[0].y = s23; }
+                if (r == 1) { pf[0].z = p01; pf[0].w = p23; dsf[0].z = s01; dsf[0].w = s23; }
+                if (r == 2) { pf[1].x = p01; pf[1].y = p23; dsf[1].x = s01; dsf[1].y = s23; }
+                if (r == 3) { pf[1].z = p01; pf[1].w = p23; dsf[1].z = s01; dsf[1].w = s23; }
+            }
+            // ---- dV^T += dO^T . P and dK^T += Q^T . dS  (queries of a k-step in accumulator order)
+#pragma unroll
+            for (int s = 0; s < 2; ++s)
+#pragma unroll
+                for (int d = 0; d < DB; ++d) {
+                    const int o = (d * 32 + col) * TPITCH + (s * 16 + g * 4) * 2;
+                    const bu32x2_t olo = *reinterpret_cast<const bu32x2_t*>(sOT + o);
+                    const bu32x2_t ohi = *reinterpret_cast<const bu32x2_t*>(sOT + o + 16);
+                    acc_dv[d] = bwd_mma(bu32x4_t{olo.x, olo.y, ohi.x, ohi.y}, pf[s], acc_dv[d]);
+                    const bu32x2_t qlo = *reinterpret_cast<const bu32x2_t*>(sQT + o);
+                    const bu32x2_t qhi = *reinterpret_cast<const bu32x2_t*>(sQT + o + 16);
+                    acc_dk[d] = bwd_mma(bu32x4_t{qlo.x, qlo.y, qhi.x, qhi.y}, dsf[s], acc_dk[d]);
+                }
+        }
+    }
+
+    if (key_row < Lk) {
+        bf16_t* krow = dk + ((int64_t)(b * Hkv + hkv) * Lk + key_row) * D;
+        bf16_t* vrow = dv + ((int64_t)(b * Hkv + hkv) * Lk + key_row) * D;
+#pragma unroll
+        for (int d = 0; d < DB; ++d)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                bu32x2_t w;
+                w.x = pack_bf16x2(acc_dk[d][r * 4 + 0], acc_dk[d][r * 4 + 1]);
+                w.y = pack_bf16x2(acc_dk[d][r * 4 + 2], acc_dk[d][r * 4 + 3]);
+                *reinterpret_cast<bu32x2_t*>(krow + d * 32 + r * 8 + g * 4) = w;
+                w.x = pack_bf16x2(acc_dv[d][r * 4 + 0], acc_dv[d][r * 4 + 1]);
+                w.y = pack_bf16x2(acc_dv[d][r * 4 + 2], acc_dv[d][r * 4 + 3]);
+                *reinterpret_cast<bu32x2_t*>(vrow + d * 32 + r * 8 + g * 4) = w;
+            }
+    }
+}
+
+// Early key tiles are seen by more queries than late ones: a workgroup takes tile j and tile n-1-j.
+template <int D>
+__global__ __launch_bounds__(256) void attention_bwd_dkv_kernel(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ qtr, const bf16_t* __restrict__ k,
+    const bf16_t* __restrict__ v, const bf16_t* __restrict__ dout, const bf16_t* __restrict__ dotr,
+    const float* __restrict__ lse, const float* __restrict__ delta, bf16_t* __restrict__ dk, bf16_t* __restrict__ dv,
+    int Hq, int Hkv, int L, int Lk, int Lqp, float scale) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    const int n_kt = (Lk + kBwdRows - 1) / kBwdRows;
+    const int n_pairs = (n_kt + 1) / 2;
+    const int pair = blockIdx.x % n_pairs;
+    const int hkv = (blockIdx.x / n_pairs) % Hkv;
+    const int b = blockIdx.x / (n_pairs * Hkv);
+    const int kt_far = n_kt - 1 - pair;
+#pragma unroll 1
+    for (int half = 0; half < 2; ++half) {
+        if (half && pair == kt_far) break;
+        attention_bwd_dkv_tile<D>(q, qtr, k, v, dout, dotr, lse, delta, dk, dv, Hq, Hkv, L, Lk, Lqp, scale,
+                                  half ? kt_far : pair, hkv, b, smem);
+    }
+}
+
+}  // namespace ats
+
+extern "C" int ats_attention_delta(const void* out, const void* dout, float* delta, int B, int Hq, int L, int D,
+                                   ats_stream_t stream) {
+    using namespace ats;
+    ATS_REQUIRE(B >= 0 && Hq > 0 && L >= 0 && (D == 64 || D == 128), ATS_ERR_UNSUPPORTED,
+                "ats_attention_delta: B=%d Hq=%d L=%d D=%d (head_dim 64 or 128)", B, Hq, L, D);
+    if (B == 0 || L == 0) return ATS_OK;
+    ATS_REQUIRE(out && dout && delta && aligned16(out) && aligned16(dout), ATS_ERR_INVALID_ARG,
+                "ats_attention_delta: null or misaligned pointer");
+    const int64_t rows = (int64_t)B * L * Hq;
+    const int rpb = 256 / (D / 8);
+    const int64_t blocks = (rows + rpb - 1) / rpb;
+    ATS_REQUIRE(blocks <= 0x7fffffff, ATS_ERR_UNSUPPORTED, "ats_attention_delta: %lld workgroups", (long long)blocks);
+    if (D == 128)
+        hipLaunchKernelGGL((attention_delta_kernel<128>), dim3((unsigned)blocks), dim3(256), 0, as_stream(stream),
+                           static_cast<const bf16_t*>(out), static_cast<const bf16_t*>(dout), delta, Hq, L, rows);
+    else
+        hipLaunchKernelGGL((attention_delta_kernel<64>), dim3((unsigned)blocks), dim3(256), 0, as_stream(stream),
+                           static_cast<const bf16_t*>(out), static_cast<const bf16_t*>(dout), delta, Hq, L, rows);
+    ATS_CHECK_LAUNCH("ats_attention_delta");
+    return ATS_OK;
+}
+
+extern "C" int ats_attention_bwd(const void* q, const void* k, const void* v, const void* qt, const void* kt,
+                                 const void* dout, const void* dot, const float* lse, const float* delta, void* dq,
+                                 void* dk, void* dv, int B, int Hq, int Hkv, int L, int Lk, int D, float scale,
+                                 ats_stream_t stream) {
+    using namespace ats;
+    ATS_REQUIRE(B >= 0 && Hq > 0 && Hkv > 0 && Hq % Hkv == 0 && L >= 0 && Lk >= L && scale > 0.f, ATS_ERR_INVALID_ARG,
+                "ats_attention_bwd: B=%d Hq=%d Hkv=%d L=%d Lk=%d scale=%g", B, Hq, Hkv, L, Lk, scale);
+    ATS_REQUIRE(D == 64 || D == 128, ATS_ERR_UNSUPPORTED, "ats_attention_bwd: head_dim %d (64 or 128)", D);
+    if (B == 0 || L == 0) return ATS_OK;
+    ATS_REQUIRE(q && k && v && qt && kt && dout && dot && lse && delta && dq && dk && dv, ATS_ERR_INVALID_ARG,
+                "ats_attention_bwd: null pointer");
+    ATS_REQUIRE(aligned16(q) && aligned16(k) && aligned16(v) && aligned16(qt) && aligned16(kt) && aligned16(dout) &&
+                    aligned16(dot) && aligned16(dq) && aligned16(dk) && aligned16(dv),
+                ATS_ERR_INVALID_ARG, "ats_attention_bwd: misaligned pointer");
+    const int Lp = (int)ats_attention_padded_len(Lk);
+    const int Lqp = (int)ats_attention_padded_len(L);
+    ATS_REQUIRE((int64_t)Lp * D * 2 < 0x7fffffffLL && (int64_t)L * Hq * D * 2 < 0x7fffffffLL, ATS_ERR_UNSUPPORTED,
+                "ats_attention_bwd: L=%d Lk=%d (one head's K or V, and one batch entry's dO, must stay under 2 GiB)", L, Lk);
+    const int n_qt = (L + kBwdRows - 1) / kBwdRows, n_kt = (Lk + kBwdRows - 1) / kBwdRows;
+    const int64_t dq_blocks = (int64_t)((n_qt + 1) / 2) * Hq * B;
+    const int64_t dkv_blocks = (int64_t)((n_kt + 1) / 2) * Hkv * B;
+    ATS_REQUIRE(dq_blocks <= 0x7fffffff && dkv_blocks <= 0x7fffffff, ATS_ERR_UNSUPPORTED, "ats_attention_bwd: grid");
+    const bf16_t* q_ = static_cast<const bf16_t*>(q);
+    const bf16_t* k_ = static_cast<const bf16_t*>(k);
+    const bf16_t* v_ = static_cast<const bf16_t*>(v);
+    const bf16_t* qt_ = static_cast<const bf16_t*>(qt);
+    const bf16_t* kt_ = static_cast<const bf16_t*>(kt);
+    const bf16_t* do_ = static_cast<const bf16_t*>(dout);
+    const bf16_t* dot_ = static_cast<const bf16_t*>(dot);
+    hipStream_t s = as_stream(stream);
+    if (D == 128) {
+        constexpr int smem_dq = 2 * kDqBN * (128 * 2 + 16) + 128 * (kDqBN * 2 + 8);
+        constexpr int smem_dkv = 2 * kDkvBQ * (128 * 2 + 16) + 2 * 128 * (kDkvBQ * 2 + 8) + 2 * kDkvBQ * 4;
+        hipLaunchKernelGGL((attention_bwd_dq_kernel<128>), dim3((unsigned)dq_blocks), dim3(256), smem_dq, s, q_, k_, v_,
+                           kt_, do_, lse, delta, static_cast<bf16_t*>(dq), Hq, Hkv, L, Lk, Lp, scale, B);
+        hipLaunchKernelGGL((attention_bwd_dkv_kernel<128>), dim3((unsigned)dkv_blocks), dim3(256), smem_dkv, s, q_, qt_,
+                           k_, v_, do_, dot_, lse, delta, static_cast<bf16_t*>(dk), static_cast<bf16_t*>(dv), Hq, Hkv, L,
+                           Lk, Lqp, scale);
+    } else {
+        constexpr int smem_dq = 2 * kDqBN * (64 * 2 + 16) + 64 * (kDqBN * 2 + 8);
+        constexpr int smem_dkv = 2 * kDkvBQ * (64 * 2 + 16) + 2 * 64 * (kDkvBQ * 2 + 8) + 2 * kDkvBQ * 4;
+        hipLaunchKernelGGL((attention_bwd_dq_kernel<64>), dim3((unsigned)dq_blocks), dim3(256), smem_dq, s, q_, k_, v_,
+                           kt_, do_, lse, delta, static_cast<bf16_t*>(dq), Hq, Hkv, L, Lk, Lp, scale, B);
+        hipLaunchKernelGGL((attention_bwd_dkv_kernel<64>), dim3((unsigned)dkv_blocks), dim3(256), smem_dkv, s, q_, qt_,
+                           k_, v_, do_, dot_, lse, delta, static_cast<bf16_t*>(dk), static_cast<bf16_t*>(dv), Hq, Hkv, L,
+                           Lk, Lqp, scale);
+    }
+    ATS_CHECK_LAUNCH("ats_attention_bwd");
+    return ATS_OK;
+}

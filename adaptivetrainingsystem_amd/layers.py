@@ -189,18 +189,22 @@ class GroupedQueryAttention(nn.Module):
             raise AtsError("GroupedQueryAttention: padding masks are not built in the gfx950 path")
         if x.dim() != 3 or x.shape[-1] != self.hidden_size:
             raise AtsError(f"GroupedQueryAttention: expected [batch, seq, {self.hidden_size}], got {tuple(x.shape)}")
-        if _wants_grad(x, *self.parameters()):
-            raise AtsError("GroupedQueryAttention: forward only (run under torch.no_grad(); the backward kernels "
-                           "of attention are not built yet)")
+        if x.dtype != torch.bfloat16:
+            raise AtsError(f"GroupedQueryAttention: the attention kernels are bfloat16 only, got {x.dtype}")
         B, L, H = x.shape
         nh, nkv, D = self.num_heads, self.num_kv_heads, self.head_dim
         x2 = x.reshape(B * L, H).contiguous()
-        q = ops.linear_nt(x2, _as_dtype(self.q_proj.weight, x.dtype)).view(B, L, nh, D).transpose(1, 2)
-        k = ops.linear_nt(x2, _as_dtype(self.k_proj.weight, x.dtype)).view(B, L, nkv, D).transpose(1, 2)
-        v = ops.linear_nt(x2, _as_dtype(self.v_proj.weight, x.dtype)).view(B, L, nkv, D).transpose(1, 2)
+        grad = _wants_grad(x, *self.parameters())
+        if grad:
+            lin = ag.LinearFunction.apply
+        else:
+            lin = lambda a, w: ops.linear_nt(a, _as_dtype(w, a.dtype))
+        q = lin(x2, self.q_proj.weight).view(B, L, nh, D).transpose(1, 2)
+        k = lin(x2, self.k_proj.weight).view(B, L, nkv, D).transpose(1, 2)
+        v = lin(x2, self.v_proj.weight).view(B, L, nkv, D).transpose(1, 2)
         # positions 0..L-1 also when a cache is passed, as the reference does (model.py:690-698)
         cos, sin = self.rope(L, x.device)
-        q, k = ops.rope(q, k, cos, sin, 0)
+        q, k = ag.RoPEFunction.apply(q, k, cos, sin, 0) if grad else ops.rope(q, k, cos, sin, 0)
         if past_key_value is not None:
             k_cache, v_cache = past_key_value
             if (k_cache.dim() != 4 or k_cache.shape[0] != B or k_cache.shape[1] != nkv or k_cache.shape[3] != D
@@ -208,8 +212,8 @@ class GroupedQueryAttention(nn.Module):
                 raise AtsError(f"GroupedQueryAttention: cache shapes {tuple(k_cache.shape)} / {tuple(v_cache.shape)}")
             k = torch.cat([k_cache.to(k.dtype), k], dim=2)
             v = torch.cat([v_cache.to(v.dtype), v], dim=2)
-        a = ops.causal_attention(q, k, v, self.scale)               # [B, L, nh*D]
-        out = ops.linear_nt(a.view(B * L, nh * D), _as_dtype(self.o_proj.weight, x.dtype)).view(B, L, H)
+        a = ag.AttentionFunction.apply(q, k, v, self.scale) if grad else ops.causal_attention(q, k, v, self.scale)
+        out = lin(a.view(B * L, nh * D), self.o_proj.weight).view(B, L, H)    # a: [B, L, nh*D]
         self._calls += 1
         if use_cache:
             return out, (k, v.contiguous())

@@ -278,6 +278,21 @@ int ats_attention_transpose_v(const void* v, int64_t sb, int64_t sl, int64_t sh,
 int ats_attention_fwd(const void* q, const void* k, const void* vt, void* out, float* lse, int B, int Hq, int Hkv,
                       int L, int Lk, int D, float scale, ats_stream_t stream);
 
+/* ---- Causal grouped-query attention (backward) ----------------------------------
+ * The reference leaves this gradient to autograd (model.py:757-839 under torch.autograd); the kernels
+ * recompute the probabilities from the forward's log-sum-exp and form
+ *   dV = P^T.dO, dP = dO.V^T, dS = P*(dP - delta)*scale, dQ = dS.K, dK = dS^T.Q
+ * without atomics (one kernel owns query rows, one owns key rows and sums over the query heads of
+ * its kv head).  ats_attention_delta: delta[B,Hq,L] = sum_d dO*O with out, dout [B,L,Hq*D].
+ * ats_attention_bwd: q [B,Hq,L,D], k, v [B,Hkv,Lk,D], dout [B,L,Hq*D] contiguous; qt, dot:
+ * [B,Hq,D,ats_attention_padded_len(L)] and kt: [B,Hkv,D,ats_attention_padded_len(Lk)] transposed copies
+ * made with ats_attention_transpose_v; lse, delta [B,Hq,L]; dq, dk, dv shaped like q, k, v. */
+int ats_attention_delta(const void* out, const void* dout, float* delta, int B, int Hq, int L, int D,
+                        ats_stream_t stream);
+int ats_attention_bwd(const void* q, const void* k, const void* v, const void* qt, const void* kt, const void* dout,
+                      const void* dot, const float* lse, const float* delta, void* dq, void* dk, void* dv, int B,
+                      int Hq, int Hkv, int L, int Lk, int D, float scale, ats_stream_t stream);
+
 /* ---- Training-step ops beside the sparse layer --------------------------------
  * Fused cross-entropy + accuracy.  Replaces fused_cross_entropy_accuracy_launcher
  * (Src/Main_Scripts/training/fused_loss.cu:179-214); numerics follow FusedLoss._pytorch_fallback

@@ -117,8 +117,6 @@ def test_gqa_module(gpu, hidden, nh, nkv, B, L):
         out = att(x.to(gpu))
     assert out.shape == x.shape and rel_err(out, ref) <= BF16_TOL
     assert set(att.state_dict()) == {f"{n}.weight" for n in ("q_proj", "k_proj", "v_proj", "o_proj")}
-    with pytest.raises(A.AtsError):
-        att(x.to(gpu).requires_grad_())
     # prefill with use_cache, then two single-token steps fed from the cache (model.py:700-708)
     w = [getattr(att, n).weight.detach().cpu() for n in ("q_proj", "k_proj", "v_proj", "o_proj")]
     with torch.no_grad():
@@ -133,3 +131,98 @@ def test_gqa_module(gpu, hidden, nh, nkv, B, L):
         r1, ref_cache = O.gqa_forward(x1, *w, nh, nkv, past_key_value=ref_cache, use_cache=True)
         assert cache[0].shape == (B, nkv, L + 1 + step, hidden // nh)
         assert rel_err(o1, r1) <= BF16_TOL
+
+
+# --------------------------------------------------------------------------- backward
+GRAD_TOL = 2e-2      # bf16 bar on gradients, relative to the oracle gradient's max-abs
+
+
+def _oracle_attention_grads(q, k, v, dout, rep):
+    """Autograd through the oracle forward on float32 leaves holding the same bf16 values."""
+    q32, k32, v32 = (t.float().requires_grad_() for t in (q, k, v))
+    D = q.shape[-1]
+    out = O.attention_standard(q32, k32.repeat_interleave(rep, dim=1), v32.repeat_interleave(rep, dim=1), D ** -0.5)
+    out.backward(dout.float())
+    return q32.grad, k32.grad, v32.grad
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,L,Lk,D", [(1, 2, 1, 64, 64, 128), (2, 4, 2, 200, 200, 128), (1, 8, 2, 300, 300, 64),
+                                             (1, 1, 1, 1, 1, 128), (2, 3, 3, 129, 129, 64), (1, 4, 1, 520, 520, 128),
+                                             (1, 4, 2, 70, 300, 64), (2, 2, 1, 1, 130, 128), (1, 2, 2, 31, 31, 64)])
+def test_causal_attention_backward(ops, gpu, B, Hq, Hkv, L, Lk, D):
+    print("case attention backward", B, Hq, Hkv, L, Lk, D, flush=True)
+    g = gen(97)
+    q = torch.randn(B, Hq, L, D, generator=g).bfloat16()
+    k = torch.randn(B, Hkv, Lk, D, generator=g).bfloat16()
+    v = torch.randn(B, Hkv, Lk, D, generator=g).bfloat16()
+    dout = torch.randn(B, L, Hq * D, generator=g).bfloat16()
+    rq, rk, rv = _oracle_attention_grads(q, k, v, dout, Hq // Hkv)
+    out, lse = ops.causal_attention(q.to(gpu), k.to(gpu), v.to(gpu), return_lse=True)
+    dq, dk, dv = ops.causal_attention_bwd(q.to(gpu), k.to(gpu), v.to(gpu), out, lse, dout.to(gpu))
+    assert dq.shape == q.shape and dk.shape == k.shape and dv.shape == v.shape
+    assert rel_err(dv, rv) <= GRAD_TOL
+    assert rel_err(dq, rq) <= GRAD_TOL
+    assert rel_err(dk, rk) <= GRAD_TOL
+
+
+def test_attention_function_autograd(gpu):
+    """The autograd Function: strided q/k/v views in, gradient accumulation through views out."""
+    from adaptivetrainingsystem_amd.autograd import AttentionFunction
+    g = gen(98)
+    B, Hq, Hkv, L, D = 2, 4, 2, 150, 64
+    base = [torch.randn(B, L, h, D, generator=g).bfloat16() for h in (Hq, Hkv, Hkv)]
+    leaves = [t.to(gpu).requires_grad_() for t in base]
+    q, k, v = (t.transpose(1, 2) for t in leaves)
+    out = AttentionFunction.apply(q, k, v, D ** -0.5)
+    w = torch.randn(B, L, Hq * D, generator=g).bfloat16()
+    (out.float() * w.to(gpu).float()).sum().backward()
+    rq, rk, rv = _oracle_attention_grads(*(t.transpose(1, 2) for t in base), w, Hq // Hkv)
+    for got, ref in zip(leaves, (rq, rk, rv)):
+        assert rel_err(got.grad.transpose(1, 2), ref) <= GRAD_TOL
+
+
+@pytest.mark.parametrize("T,K,N", [(300, 256, 192), (64, 128, 128), (1, 64, 320), (1000, 512, 64)])
+def test_linear_function_grads(gpu, T, K, N):
+    from adaptivetrainingsystem_amd.autograd import LinearFunction
+    print("case linear function", T, K, N, flush=True)
+    g = gen(99)
+    x = torch.randn(T, K, generator=g).bfloat16()
+    w = (torch.randn(N, K, generator=g) * 0.1).bfloat16()
+    dy = torch.randn(T, N, generator=g).bfloat16()
+    xg, wg = x.to(gpu).requires_grad_(), w.to(gpu).requires_grad_()
+    y = LinearFunction.apply(xg, wg)
+    y.backward(dy.to(gpu))
+    x32, w32 = x.float().requires_grad_(), w.float().requires_grad_()
+    y32 = x32 @ w32.T
+    y32.backward(dy.float())
+    assert rel_err(y, y32) <= BF16_TOL
+    assert rel_err(xg.grad, x32.grad) <= GRAD_TOL and rel_err(wg.grad, w32.grad) <= GRAD_TOL
+
+
+@pytest.mark.parametrize("hidden,nh,nkv,B,L", [(512, 4, 2, 2, 77), (256, 4, 1, 1, 200)])
+def test_gqa_module_backward(gpu, hidden, nh, nkv, B, L):
+    """Input and parameter gradients of the whole attention sub-layer against autograd over the oracle forward."""
+    import adaptivetrainingsystem_amd as A
+    from adaptivetrainingsystem_amd.workloads import LayerConfig
+    print("case gqa module backward", hidden, nh, nkv, B, L, flush=True)
+    torch.manual_seed(14)
+    cfg = LayerConfig(hidden, 4 * hidden, 1, 1, num_heads=nh, num_kv_heads=nkv, seq_length=512)
+    att = A.GroupedQueryAttention(cfg)
+    with torch.no_grad():
+        for p in att.parameters():
+            p.mul_(20.0)
+    att = att.to(torch.bfloat16).to(gpu).train()
+    x = torch.randn(B, L, hidden, generator=gen(100)).bfloat16()
+    dy = torch.randn(B, L, hidden, generator=gen(101)).bfloat16()
+    xg = x.to(gpu).requires_grad_()
+    out = att(xg)
+    out.backward(dy.to(gpu))
+    names = ("q_proj", "k_proj", "v_proj", "o_proj")
+    w32 = [getattr(att, n).weight.detach().float().cpu().requires_grad_() for n in names]
+    x32 = x.float().requires_grad_()
+    ref = O.gqa_forward(x32, *w32, nh, nkv)
+    ref.backward(dy.float())
+    assert rel_err(out, ref) <= BF16_TOL
+    assert rel_err(xg.grad, x32.grad) <= 3e-2
+    for n, w in zip(names, w32):
+        assert rel_err(getattr(att, n).weight.grad, w.grad) <= 3e-2, n
