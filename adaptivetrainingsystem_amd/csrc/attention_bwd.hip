@@ -294,6 +294,9 @@ __device__ __forceinline__ void attention_bwd_dkv_tile(const bf16_t* __restrict_
     unsigned char* const sOT = smem + 2 * RTILE + TTILE;
     float* const sL = reinterpret_cast<float*>(smem + 2 * RTILE + 2 * TTILE);   // [32] lse * log2(e)
     float* const sD = sL + kDkvBQ;                                             // [32] delta
+    // the block's own V rows stay in LDS for the whole tile: with K rows, both accumulators and V rows in
+    // registers a wave would need more than half the register file, i.e. one wave per SIMD
+    unsigned char* const sVb = smem + 2 * RTILE + 2 * TTILE + 2 * kDkvBQ * 4;    // [128][RPITCH]
 
     const int rep = Hq / Hkv;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -304,15 +307,26 @@ __device__ __forceinline__ void attention_bwd_dkv_tile(const bf16_t* __restrict_
     const float scale_log2 = scale * kLog2e;
 
     const bf16_t* kp = k + ((int64_t)(b * Hkv + hkv) * Lk + key_clamped) * D;
-    const bf16_t* vp = v + ((int64_t)(b * Hkv + hkv) * Lk + key_clamped) * D;
-    bu32x4_t kf[KS], vf[KS];
+    bu32x4_t kf[KS];
 #pragma unroll
-    for (int s = 0; s < KS; ++s) {
-        kf[s] = *reinterpret_cast<const bu32x4_t*>(kp + s * 16 + g * 8);
-        vf[s] = *reinterpret_cast<const bu32x4_t*>(vp + s * 16 + g * 8);
+    for (int s = 0; s < KS; ++s) kf[s] = *reinterpret_cast<const bu32x4_t*>(kp + s * 16 + g * 8);
+    __syncthreads();   // the previous tile of this workgroup is done with the V rows
+    {
+        const bf16_t* vblock = v + (int64_t)(b * Hkv + hkv) * Lk * D;
+        const __amdgpu_buffer_rsrc_t vb_rsrc =
+            __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(vblock), 0, (int)((int64_t)Lk * D * 2), 0x00020000);
+#pragma unroll
+        for (int i = 0; i < kBwdRows * (D / 8) / 256; ++i) {
+            const int idx = tid + i * 256;
+            const int r = idx / (D / 8), c = idx % (D / 8);
+            const bu32x4_t x = __builtin_amdgcn_raw_buffer_load_b128(vb_rsrc, (r * D + c * 8) * 2,
+                                                                     kt_idx * kBwdRows * D * 2, 0);
+            *reinterpret_cast<bu32x4_t*>(sVb + r * RPITCH + c * 16) = x;
+        }
     }
+    const unsigned char* const v_row = sVb + (wave * 32 + col) * RPITCH + g * 16;
 #pragma unroll
-    for (int s = 0; s < KS; ++s) asm volatile("" : "+v"(kf[s]), "+v"(vf[s]));
+    for (int s = 0; s < KS; ++s) asm volatile("" : "+v"(kf[s]));
 
     bf32x16_t acc_dk[DB], acc_dv[DB];
 #pragma unroll
@@ -403,7 +417,8 @@ __device__ __forceinline__ void attention_bwd_dkv_tile(const bf16_t* __restrict_
             for (int s = 0; s < KS; ++s) {
                 const int o = col * RPITCH + s * 32 + g * 16;
                 acc_s = bwd_mma(*reinterpret_cast<const bu32x4_t*>(sQ + o), kf[s], acc_s);
-                acc_p = bwd_mma(*reinterpret_cast<const bu32x4_t*>(sO + o), vf[s], acc_p);
+                acc_p = bwd_mma(*reinterpret_cast<const bu32x4_t*>(sO + o),
+                                *reinterpret_cast<const bu32x4_t*>(v_row + s * 32), acc_p);
             }
             // ---- P = exp(S * scale - lse[q]); dS = P * (dP - delta[q]) * scale; accumulator row x is
             //      query (x / 4) * 8 + g * 4 + x % 4 of the step
@@ -471,7 +486,7 @@ __device__ __forceinline__ void attention_bwd_dkv_tile(const bf16_t* __restrict_
 
 // Early key tiles are seen by more queries than late ones: a workgroup takes tile j and tile n-1-j.
 template <int D>
-__global__ __launch_bounds__(256) void attention_bwd_dkv_kernel(
+__global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ qtr, const bf16_t* __restrict__ k,
     const bf16_t* __restrict__ v, const bf16_t* __restrict__ dout, const bf16_t* __restrict__ dotr,
     const float* __restrict__ lse, const float* __restrict__ delta, bf16_t* __restrict__ dk, bf16_t* __restrict__ dv,
@@ -479,9 +494,20 @@ __global__ __launch_bounds__(256) void attention_bwd_dkv_kernel(
     extern __shared__ __align__(16) unsigned char smem[];
     const int n_kt = (Lk + kBwdRows - 1) / kBwdRows;
     const int n_pairs = (n_kt + 1) / 2;
-    const int pair = blockIdx.x % n_pairs;
-    const int hkv = (blockIdx.x / n_pairs) % Hkv;
-    const int b = blockIdx.x / (n_pairs * Hkv);
+    // consecutive ids go to different XCDs: keep the workgroups of one (batch, kv head), which read the
+    // same queries, on one XCD
+    const int n_groups = (int)gridDim.x / n_pairs;
+    int group, pair;
+    if (n_groups % 8 == 0) {
+        const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
+        group = (idx / n_pairs) * 8 + xcd;
+        pair = idx % n_pairs;
+    } else {
+        group = blockIdx.x / n_pairs;
+        pair = blockIdx.x % n_pairs;
+    }
+    const int hkv = group % Hkv;
+    const int b = group / Hkv;
     const int kt_far = n_kt - 1 - pair;
 #pragma unroll 1
     for (int half = 0; half < 2; ++half) {
@@ -547,7 +573,15 @@ extern "C" int ats_attention_bwd(const void* q, const void* k, const void* v, co
     hipStream_t s = as_stream(stream);
     if (D == 128) {
         constexpr int smem_dq = 2 * kDqBN * (128 * 2 + 16) + 128 * (kDqBN * 2 + 8);
-        constexpr int smem_dkv = 2 * kDkvBQ * (128 * 2 + 16) + 2 * 128 * (kDkvBQ * 2 + 8) + 2 * kDkvBQ * 4;
+        constexpr int smem_dkv = 2 * kDkvBQ * (128 * 2 + 16) + 2 * 128 * (kDkvBQ * 2 + 8) + 2 * kDkvBQ * 4 +
+                                 kBwdRows * (128 * 2 + 16);
+        static bool attr = false;
+        if (!attr) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(attention_bwd_dkv_kernel<128>),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, smem_dkv);
+            ATS_REQUIRE(e == hipSuccess, ATS_ERR_LAUNCH, "ats_attention_bwd: cannot reserve %d bytes of LDS", smem_dkv);
+            attr = true;
+        }
         hipLaunchKernelGGL((attention_bwd_dq_kernel<128>), dim3((unsigned)dq_blocks), dim3(256), smem_dq, s, q_, k_, v_,
                            kt_, do_, lse, delta, static_cast<bf16_t*>(dq), Hq, Hkv, L, Lk, Lp, scale, B);
         hipLaunchKernelGGL((attention_bwd_dkv_kernel<128>), dim3((unsigned)dkv_blocks), dim3(256), smem_dkv, s, q_, qt_,
@@ -555,7 +589,8 @@ extern "C" int ats_attention_bwd(const void* q, const void* k, const void* v, co
                            Lk, Lqp, scale);
     } else {
         constexpr int smem_dq = 2 * kDqBN * (64 * 2 + 16) + 64 * (kDqBN * 2 + 8);
-        constexpr int smem_dkv = 2 * kDkvBQ * (64 * 2 + 16) + 2 * 64 * (kDkvBQ * 2 + 8) + 2 * kDkvBQ * 4;
+        constexpr int smem_dkv = 2 * kDkvBQ * (64 * 2 + 16) + 2 * 64 * (kDkvBQ * 2 + 8) + 2 * kDkvBQ * 4 +
+                                 kBwdRows * (64 * 2 + 16);
         hipLaunchKernelGGL((attention_bwd_dq_kernel<64>), dim3((unsigned)dq_blocks), dim3(256), smem_dq, s, q_, k_, v_,
                            kt_, do_, lse, delta, static_cast<bf16_t*>(dq), Hq, Hkv, L, Lk, Lp, scale, B);
         hipLaunchKernelGGL((attention_bwd_dkv_kernel<64>), dim3((unsigned)dkv_blocks), dim3(256), smem_dkv, s, q_, qt_,
