@@ -9,6 +9,9 @@ its absence is an error (there is no fallback path).
 from ._lib import AtsError, LIB_PATH, is_built  # noqa: F401
 from .layers import (  # noqa: F401
     CapacityMoEFFNLayer,
+    DenseGroupedQueryAttention,
+    DenseSwiGLU,
+    DenseSwiGLUWithMoD,
     FusedRMSNorm,
     FusedRoPE,
     GroupedQueryAttention,
@@ -19,6 +22,7 @@ from .layers import (  # noqa: F401
     RMSNorm,
     RotaryEmbedding,
     SwiGLUExpert,
+    TransformerBlock,
     apply_rotary_pos_emb,
 )
 

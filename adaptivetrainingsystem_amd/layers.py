@@ -225,6 +225,9 @@ class GroupedQueryAttention(nn.Module):
                 "num_kv_heads": self.num_kv_heads, "head_dim": self.head_dim, "parameter_count": self._param_count}
 
 
+DenseGroupedQueryAttention = GroupedQueryAttention     # the reference's class name (model.py:565)
+
+
 # ============================================================================ experts
 class SwiGLUExpert(nn.Module):
     """down(silu(gate) * up) with the fused [2I, H] gate/up weight (gate = first I rows)."""
@@ -532,3 +535,94 @@ class MoDMoEBlock(nn.Module):
         ops.scatter_add_rows(out, sel, delta.view(-1, H))
         self.last_selected = sel
         return out.view(B, L, H), aux
+
+
+# ============================================================================ dense FFN and the block
+class DenseSwiGLU(SwiGLUExpert):
+    """Dense FFN of a non-MoE layer, down(silu(gate) * up) with the fused [2I, H] gate/up weight
+    (MS/core/model.py:1406-1479, its PyTorch branch: parameters gate_up_proj / down_proj)."""
+
+    def __init__(self, config):
+        super().__init__(config)
+        self.config = config
+
+    def _init_weights(self, config) -> None:
+        std = getattr(config, "init_std", 0.02)
+        nn.init.normal_(self.gate_up_proj.weight, mean=0.0, std=std)
+        nn.init.normal_(self.down_proj.weight, mean=0.0, std=std / math.sqrt(2 * getattr(config, "num_layers", 1)))
+
+
+class DenseSwiGLUWithMoD(DenseSwiGLU):
+    """Dense FFN whose output is gated per token by the MoD router (MS/core/model.py:1304-1403): every token
+    is computed, then multiplied by its routing weight.  forward -> (out, aux)."""
+
+    def __init__(self, config):
+        super().__init__(config)
+        self.use_mod = getattr(config, "use_mod", False)
+        if self.use_mod:
+            self.router = MoDRouter(config.hidden_size, capacity_factor=getattr(config, "mod_capacity_factor", 0.5),
+                                    routing_temperature=getattr(config, "mod_routing_temperature", 1.0))
+
+    def forward(self, x: torch.Tensor):
+        y = super().forward(x)
+        if not self.use_mod:
+            return y, None
+        weights, _, aux = self.router(x)
+        return y * weights.to(y.dtype), aux
+
+
+class TransformerBlock(nn.Module):
+    """Pre-norm block of the reference (MS/core/model.py:1487-1611): x + attention(input_norm(x)), then
+    x + ffn(post_attn_norm(x)) with an MoE FFN on the layers the pattern selects and a dense SwiGLU FFN
+    elsewhere.  Same sub-module names (input_norm, self_attn, post_attn_norm, ffn), so state_dicts load
+    unchanged.  forward -> (x, aux_loss or None)."""
+
+    def __init__(self, config, layer_idx: int = 0):
+        super().__init__()
+        self.config = config
+        self.layer_idx = layer_idx
+        eps = getattr(config, "rms_norm_eps", 1e-6)
+        self.input_norm = RMSNorm(config.hidden_size, eps)
+        self.self_attn = GroupedQueryAttention(config)
+        self.post_attn_norm = RMSNorm(config.hidden_size, eps)
+        self.use_moe = self._should_use_moe(layer_idx, config)
+        if self.use_moe:
+            self.ffn = MoEFFNLayer(config)
+        elif getattr(config, "use_mod", False):
+            self.ffn = DenseSwiGLUWithMoD(config)
+        else:
+            self.ffn = DenseSwiGLU(config)
+        self.gradient_checkpointing = getattr(config, "gradient_checkpointing", False)
+
+    @staticmethod
+    def _should_use_moe(layer_idx: int, config) -> bool:
+        """The layer patterns of model.py:1545-1575."""
+        if not getattr(config, "use_moe", False):
+            return False
+        pattern = getattr(config, "moe_pattern", "all")
+        if callable(pattern):
+            try:
+                return bool(pattern(layer_idx, config.num_layers))
+            except Exception:
+                return True
+        if pattern == "every_3rd":
+            return (layer_idx + 1) % 3 == 0
+        if pattern == "every_4th":
+            return (layer_idx + 1) % 4 == 0
+        if pattern == "sandwich":
+            start, end = getattr(config, "dense_start_layers", 2), getattr(config, "dense_end_layers", 2)
+            return not (layer_idx < start or layer_idx >= config.num_layers - end)
+        return pattern != "none"
+
+    def forward(self, x: torch.Tensor, attention_mask: Optional[torch.Tensor] = None):
+        if self.gradient_checkpointing and self.training:
+            return torch.utils.checkpoint.checkpoint(self._forward_impl, x, attention_mask, use_reentrant=False)
+        return self._forward_impl(x, attention_mask)
+
+    def _forward_impl(self, x: torch.Tensor, attention_mask: Optional[torch.Tensor] = None):
+        x = x + self.self_attn(self.input_norm(x), attention_mask)
+        result = self.ffn(self.post_attn_norm(x))
+        if isinstance(result, tuple):
+            out, aux = result
+            return x + out, aux
+        return x + result, None
