@@ -312,7 +312,7 @@ class MoEFFNLayer(nn.Module):
         self.router_logit_bias: Optional[torch.Tensor] = None   # optional per-expert skew (benchmarks)
         self._gate_param_count = sum(p.numel() for p in self.gate.parameters())
         self._expert_param_count = self.experts[0]._param_count
-        self._routing_stats = {"expert_usage": torch.zeros(config.num_experts), "total_routed": 0,
+        self._routing_stats = {"expert_usage": torch.zeros(config.num_experts, device="cpu"), "total_routed": 0,
                                "dropped_tokens": 0}
         self._wcache_key = None
         self._wcache = None
@@ -399,7 +399,7 @@ class MoEFFNLayer(nn.Module):
         kept = plan["kept"].cpu()
         usage = self._routing_stats["expert_usage"]
         if usage.numel() != hist.numel():       # an expert was added or pruned since the last step
-            grown = torch.zeros(hist.numel())
+            grown = torch.zeros(hist.numel(), device="cpu")
             n = min(usage.numel(), hist.numel())
             grown[:n] = usage[:n]
             self._routing_stats["expert_usage"] = grown
@@ -421,7 +421,7 @@ class MoEFFNLayer(nn.Module):
         }
 
     def reset_routing_stats(self) -> None:
-        self._routing_stats = {"expert_usage": torch.zeros(self.num_experts), "total_routed": 0,
+        self._routing_stats = {"expert_usage": torch.zeros(self.num_experts, device="cpu"), "total_routed": 0,
                                "dropped_tokens": 0}
 
 

@@ -390,6 +390,71 @@ def run_attention_train(args):
     return result
 
 
+def run_block_train(args):
+    """One transformer block of the headline model (pre-norm, GQA attention, top-2 of 8 experts MoE FFN with
+    FCFS capacity 1.25) on batch 8 x seq 2048: forward + backward with all gradients."""
+    import adaptivetrainingsystem_amd as A
+    from adaptivetrainingsystem_amd.workloads import LayerConfig
+    from adaptivetrainingsystem_amd.profiling import StageTimer
+    dev = torch.device("cuda:0")
+    B, L, H, I, E, K, Hq, Hkv = 8, 2048, 4096, 14336, 8, 2, 32, 8
+    torch.manual_seed(9)
+    cfg = LayerConfig(H, I, E, K, 1.25, num_heads=Hq, num_kv_heads=Hkv, seq_length=L, use_moe=True,
+                      moe_capacity_mode="fcfs", num_layers=32)
+    with torch.device(dev):
+        blk = A.TransformerBlock(cfg)
+    blk = blk.to(torch.bfloat16).train()
+    x = torch.randn(B, L, H, device=dev).bfloat16().requires_grad_()
+    dy = torch.randn(B, L, H, device=dev).bfloat16()
+
+    def step(timer=None):
+        blk.zero_grad(set_to_none=True)
+        x.grad = None
+        if timer is None:
+            out, aux = blk(x)
+            torch.autograd.backward([out, aux], [dy, torch.ones_like(aux)])
+            return
+        with timer.range("forward"):
+            out, aux = blk(x)
+        with timer.range("backward"):
+            torch.autograd.backward([out, aux], [dy, torch.ones_like(aux)])
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    timer = StageTimer()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step(timer)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    st = timer.summary()
+    T = B * L
+    kept = int(blk.ffn.last_plan["kept"].sum().item())
+    D = H // Hq
+    proj = 2.0 * T * H * (Hq * D + 2 * Hkv * D + H)
+    attn = 2.0 * B * Hq * D * L * (L + 1) / 2
+    ffn = 6.0 * kept * H * I
+    flops = 3.0 * (proj + ffn) + 7.0 * attn + 3.0 * 2.0 * T * H * E      # forward + dgrad + wgrad; attention 2 + 5
+    step_ms = st["forward"]["mean_ms"] + st["backward"]["mean_ms"]
+    achieved = flops / (step_ms * 1e-3) / 1e12
+    log(f"  forward {st['forward']['mean_ms']:.3f} ms, backward {st['backward']['mean_ms']:.3f} ms; kept assignments "
+        f"{kept} of {T * K}; {achieved:.1f} TFLOP/s over the step ({achieved / PEAK_MFMA_BF16_TFLOPS:.1%} of the bf16 MFMA peak); "
+        f"peak memory {torch.cuda.max_memory_allocated() / 2**30:.1f} GiB")
+    return {
+        "metric": "transformer block training tokens/s", "value": T * args.steps / dt, "unit": "tokens/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": dt / args.steps * 1e3, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"block_train: pre-norm block, GQA {Hq}/{Hkv} heads + MoE {E} experts top-{K} (I {I}, cf 1.25), "
+                               f"hidden {H}, batch {B}, seq {L}, forward + backward"},
+        "roofline": {"kernel": "whole step (grouped GEMMs, attention, HBM-bound kernels)", "bound": "mfma",
+                     "achieved": achieved, "peak": PEAK_MFMA_BF16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": achieved / PEAK_MFMA_BF16_TFLOPS, "traffic": None},
+        "stages_ms": {s_: round(v_["mean_ms"], 4) for s_, v_ in st.items()},
+        "cpu_baseline": None,
+    }
+
+
 def run_gqa_layer(args):
     """The attention sub-layer of the headline model shape (hidden 4096, 32 query / 8 kv heads, head_dim 128) on
     batch 8 x seq 2048: q/k/v projections, RoPE, causal attention, output projection."""
@@ -536,7 +601,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="c4_prefill",
                     choices=["c4_prefill", "c3_decode", "c5_finegrained_mod", "c1_cpu_reference", "c2_norm_rope",
-                             "c4_prefill_train", "c1_cpu_reference_train", "loss_clip", "attention", "attention_train", "gqa_layer"])
+                             "c4_prefill_train", "c1_cpu_reference_train", "loss_clip", "attention", "attention_train", "gqa_layer", "block_train"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a 1 GiB device copy (known traffic) so hardware-counter runs can be scaled")
@@ -567,6 +632,8 @@ def main():
         result = run_attention(args)
     elif args.workload == "attention_train":
         result = run_attention_train(args)
+    elif args.workload == "block_train":
+        result = run_block_train(args)
     elif args.workload == "gqa_layer":
         result = run_gqa_layer(args)
     elif args.workload.endswith("_train"):
