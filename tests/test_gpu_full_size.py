@@ -148,3 +148,51 @@ def test_norm_rope_config2_full(gpu):
         t = t.float()
         return t[..., :64] ** 2 + t[..., 64:] ** 2
     assert rel_err(pair_norm(q), pair_norm(w.q)) <= 4 * 2 ** -7
+
+
+def test_attention_full_size_properties_and_sampled_rows(gpu):
+    """Causal GQA attention at the headline shape (batch 8, seq 2048, 32 / 8 heads, head_dim 128): sampled
+    query rows against the oracle, and properties that hold at any size -- doubling V doubles the output
+    exactly, a prefix of the sequence gives the same rows bit for bit, a zero cotangent gives zero
+    gradients, and the key gradients of V sum to the cotangent's sum (rows of P sum to one)."""
+    from adaptivetrainingsystem_amd import ops
+    B, Hq, Hkv, L, D = 8, 32, 8, 2048, 128
+    g = torch.Generator().manual_seed(31)
+    q = torch.randn(B, Hq, L, D, generator=g).bfloat16()
+    k = torch.randn(B, Hkv, L, D, generator=g).bfloat16()
+    v = torch.randn(B, Hkv, L, D, generator=g).bfloat16()
+    qg, kg, vg = q.to(gpu), k.to(gpu), v.to(gpu)
+    out, lse = ops.causal_attention(qg, kg, vg, return_lse=True)
+    assert torch.isfinite(out.float()).all()
+    # sampled (batch, head, row) triples against the oracle's row formula
+    rows = torch.randint(0, L, (24,), generator=g).tolist() + [0, 1, 63, 64, 127, 128, L - 1]
+    o4 = out.view(B, L, Hq, D).float().cpu()
+    for n, i in enumerate(rows):
+        b, h = n % B, (7 * n) % Hq
+        kv = h // (Hq // Hkv)
+        s = (k[b, kv, :i + 1].float() @ q[b, h, i].float()) * D ** -0.5
+        p = torch.softmax(s, 0).bfloat16().float()
+        ref = p @ v[b, kv, :i + 1].float()
+        assert (o4[b, i, h] - ref).abs().max().item() <= BF16_TOL * max(ref.abs().max().item(), 1e-3), (b, h, i)
+        assert abs(lse[b, h, i].item() - torch.logsumexp(s, 0).item()) <= 1e-3
+    assert torch.equal(ops.causal_attention(qg, kg, vg * 2), out * 2)
+    half = ops.causal_attention(qg[:, :, :1024], kg[:, :, :1024], vg[:, :, :1024])
+    assert torch.equal(half, out[:, :1024])
+    # backward
+    dout = torch.randn(B, L, Hq * D, generator=g).bfloat16().to(gpu)
+    dq, dk, dv = ops.causal_attention_bwd(qg, kg, vg, out, lse, dout)
+    assert all(torch.isfinite(t.float()).all() for t in (dq, dk, dv))
+    col = dout.view(B, L, Hkv, Hq // Hkv, D).float().sum(dim=(1, 3))          # [B, Hkv, D]
+    assert rel_err(dv.float().sum(dim=2), col) <= BF16_TOL
+    z = torch.zeros_like(dout)
+    zq, zk, zv = ops.causal_attention_bwd(qg, kg, vg, out, lse, z)
+    assert not zq.any() and not zk.any() and not zv.any()
+    # sampled gradient rows: dV[j] = sum_i P[i, j] dO[i] over the queries of the group that see key j
+    for n, j in enumerate([0, 5, 700, 1500, L - 1]):
+        b, kv = n % B, (3 * n) % Hkv
+        ref = torch.zeros(D)
+        for h in range(kv * (Hq // Hkv), (kv + 1) * (Hq // Hkv)):
+            s = torch.einsum("id,d->i", q[b, h, j:].float(), k[b, kv, j].float()) * D ** -0.5
+            pj = torch.exp(s - lse[b, h, j:].cpu()).bfloat16().float()
+            ref += pj @ dout.view(B, L, Hq, D)[b, j:, h].float().cpu()
+        assert (dv[b, kv, j].float().cpu() - ref).abs().max().item() <= BF16_TOL * max(ref.abs().max().item(), 1e-3), (b, kv, j)
