@@ -27,7 +27,11 @@ typedef __attribute__((__vector_size__(16 * sizeof(float)))) float af32x16_t;
 typedef unsigned int au32x4_t __attribute__((ext_vector_type(4)));
 typedef unsigned int au32x2_t __attribute__((ext_vector_type(2)));
 
-constexpr int kAttBM = 128;   // query rows per block
+#ifndef ATT_THREADS
+#define ATT_THREADS 256
+#endif
+constexpr int kAttThreads = ATT_THREADS;          // 4 or 8 waves
+constexpr int kAttBM = kAttThreads / 64 * 32;   // query rows per block: 32 per wave
 constexpr int kAttBN = 64;    // keys per tile
 
 __device__ __forceinline__ af32x16_t att_mma(const au32x4_t& a, const au32x4_t& b, af32x16_t c) {
@@ -77,8 +81,8 @@ __device__ __forceinline__ void attention_q_tile(const bf16_t* __restrict__ q, c
     constexpr int VPITCH = kAttBN * 2 + 8;  // bytes per V^T row in LDS
     constexpr int KTILE = kAttBN * KPITCH;
     constexpr int VTILE = D * VPITCH;
-    constexpr int KVEC = kAttBN * (D / 8) / 256;   // 16-byte vectors per thread for a K tile
-    constexpr int VVEC = D * (kAttBN / 8) / 256;   // and for a V^T tile
+    constexpr int KVEC = kAttBN * (D / 8) / kAttThreads;   // 16-byte vectors per thread for a K tile
+    constexpr int VVEC = D * (kAttBN / 8) / kAttThreads;   // and for a V^T tile
     // smem: [2 stages][K tile | V^T tile]
 #define ATT_SK(stage_) (smem + (stage_) * (KTILE + VTILE))
 #define ATT_SV(stage_) (smem + (stage_) * (KTILE + VTILE) + KTILE)
@@ -106,12 +110,12 @@ __device__ __forceinline__ void attention_q_tile(const bf16_t* __restrict__ q, c
     int k_lane[KVEC], v_lane[VVEC];
 #pragma unroll
     for (int i = 0; i < KVEC; ++i) {
-        const int idx = tid + i * 256;
+        const int idx = tid + i * kAttThreads;
         k_lane[i] = ((idx / (D / 8)) * D + (idx % (D / 8)) * 8) * 2;
     }
 #pragma unroll
     for (int i = 0; i < VVEC; ++i) {
-        const int idx = tid + i * 256;
+        const int idx = tid + i * kAttThreads;
         v_lane[i] = ((idx / (kAttBN / 8)) * Lp + (idx % (kAttBN / 8)) * 8) * 2;
     }
 
@@ -145,13 +149,13 @@ __device__ __forceinline__ void attention_q_tile(const bf16_t* __restrict__ q, c
         for (int i = 0; i < VVEC; ++i) rv[i] = __builtin_amdgcn_raw_buffer_load_b128(v_rsrc, v_lane[i], 0, 0);
 #pragma unroll
         for (int i = 0; i < KVEC; ++i) {
-            const int idx = tid + i * 256;
+            const int idx = tid + i * kAttThreads;
             const int r = idx / (D / 8), c = idx % (D / 8);
             *reinterpret_cast<au32x4_t*>(ATT_SK(0) + r * KPITCH + c * 16) = rk[i];
         }
 #pragma unroll
         for (int i = 0; i < VVEC; ++i) {
-            const int idx = tid + i * 256;
+            const int idx = tid + i * kAttThreads;
             const int d = idx / (kAttBN / 8), c = idx % (kAttBN / 8);
             const au32x2_t lo = {rv[i].x, rv[i].y}, hi = {rv[i].z, rv[i].w};
             *reinterpret_cast<au32x2_t*>(ATT_SV(0) + d * VPITCH + c * 16) = lo;
@@ -170,14 +174,25 @@ __device__ __forceinline__ void attention_q_tile(const bf16_t* __restrict__ q, c
         const unsigned char* sk = ATT_SK(t & 1);
         const unsigned char* sv = ATT_SV(t & 1);
         const bool has_next = t + 1 < n_tiles;
-        if (has_next) {
-            const int n1 = n0 + kAttBN;
+        // The loads of the next tile are issued one at a time between the MFMAs of the score product: all
+        // waves of a CU leave the barrier together, and 8 loads per wave issued back to back queue up behind
+        // the CU's one address unit while no wave can reach its MFMAs.
+        const int n1 = n0 + kAttBN;
+#define ATT_LOAD_ONE(i_)                                                                               \
+    {                                                                                                  \
+        if ((i_) < KVEC)                                                                               \
+            rk[(i_) < KVEC ? (i_) : 0] =                                                               \
+                __builtin_amdgcn_raw_buffer_load_b128(k_rsrc, k_lane[(i_) < KVEC ? (i_) : 0], n1 * D * 2, 0); \
+        else                                                                                           \
+            rv[(i_) < KVEC ? 0 : (i_) - KVEC] = __builtin_amdgcn_raw_buffer_load_b128(                 \
+                v_rsrc, v_lane[(i_) < KVEC ? 0 : (i_) - KVEC], n1 * 2, 0);                             \
+    }
+        constexpr int NLOAD = KVEC + VVEC;
+        constexpr int LOAD_EVERY = 2 * KS / NLOAD;
+        static_assert(LOAD_EVERY >= 1 && LOAD_EVERY * NLOAD == 2 * KS, "one load per LOAD_EVERY score MFMAs");
+        if (has_next && n0 > q_wave_last) {   // this wave skips the tile's arithmetic but still loads its share
 #pragma unroll
-            for (int i = 0; i < KVEC; ++i)
-                rk[i] = __builtin_amdgcn_raw_buffer_load_b128(k_rsrc, k_lane[i], n1 * D * 2, 0);
-#pragma unroll
-            for (int i = 0; i < VVEC; ++i)
-                rv[i] = __builtin_amdgcn_raw_buffer_load_b128(v_rsrc, v_lane[i], n1 * 2, 0);
+            for (int i = 0; i < NLOAD; ++i) ATT_LOAD_ONE(i);
         }
 
         if (n0 <= q_wave_last) {   // some key of the tile is visible to this wave
@@ -194,9 +209,11 @@ __device__ __forceinline__ void attention_q_tile(const bf16_t* __restrict__ q, c
             for (int f = 0; f < 2 * KS; ++f) {
                 acc_s[f & 1] = att_mma(ring[f % kRing], qf[f >> 1], acc_s[f & 1]);
                 if (f + kRing < 2 * KS) ring[f % kRing] = ATT_KFRAG(f + kRing);
+                if (has_next && f % LOAD_EVERY == LOAD_EVERY - 1) ATT_LOAD_ONE(f / LOAD_EVERY);
                 __builtin_amdgcn_sched_barrier(0);   // keep the reads kRing fragments ahead of their use
             }
 #undef ATT_KFRAG
+#undef ATT_LOAD_ONE
             // first V^T fragments travel during the softmax: fragment f = (k-step f/DB, output block f%DB)
             const unsigned char* vr = sv + col * VPITCH + g * 8;
 #define ATT_VFRAG(f_, dst_)                                                                            \
@@ -270,13 +287,13 @@ __device__ __forceinline__ void attention_q_tile(const bf16_t* __restrict__ q, c
             unsigned char* dv = ATT_SV((t + 1) & 1);
 #pragma unroll
             for (int i = 0; i < KVEC; ++i) {
-                const int idx = tid + i * 256;
+                const int idx = tid + i * kAttThreads;
                 const int r = idx / (D / 8), c = idx % (D / 8);
                 *reinterpret_cast<au32x4_t*>(dk + r * KPITCH + c * 16) = rk[i];
             }
 #pragma unroll
             for (int i = 0; i < VVEC; ++i) {
-                const int idx = tid + i * 256;
+                const int idx = tid + i * kAttThreads;
                 const int d = idx / (kAttBN / 8), c = idx % (kAttBN / 8);
                 // 8-byte halves: the row pitch keeps 8-byte alignment only
                 const au32x2_t lo = {rv[i].x, rv[i].y}, hi = {rv[i].z, rv[i].w};
@@ -314,7 +331,7 @@ __device__ __forceinline__ void attention_q_tile(const bf16_t* __restrict__ q, c
 // its K and V stay in that XCD's L2.  Two waves per SIMD (register budget 256): one wave's softmax runs
 // in the shadow of the other's MFMAs.
 template <int D>
-__global__ __launch_bounds__(256, 2) void attention_fwd_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
+__global__ __launch_bounds__(kAttThreads, 512 / kAttThreads) void attention_fwd_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
                                                             const bf16_t* __restrict__ vt, bf16_t* __restrict__ out,
                                                             float* __restrict__ lse, int Hq, int Hkv, int L, int Lk, int Lp,
                                                             float scale_log2, int B) {
@@ -399,12 +416,12 @@ extern "C" int ats_attention_fwd(const void* q, const void* k, const void* vt, v
             ATS_REQUIRE(e == hipSuccess, ATS_ERR_LAUNCH, "ats_attention_fwd: cannot reserve %d bytes of LDS", smem);
             attr = true;
         }
-        hipLaunchKernelGGL((attention_fwd_kernel<128>), grid, dim3(256), smem, as_stream(stream),
+        hipLaunchKernelGGL((attention_fwd_kernel<128>), grid, dim3(kAttThreads), smem, as_stream(stream),
                            static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k), static_cast<const bf16_t*>(vt),
                            static_cast<bf16_t*>(out), lse, Hq, Hkv, L, Lk, Lp, scale_log2, B);
     } else {
         constexpr int smem = 2 * (kAttBN * (64 * 2 + 16) + 64 * (kAttBN * 2 + 8));
-        hipLaunchKernelGGL((attention_fwd_kernel<64>), grid, dim3(256), smem, as_stream(stream),
+        hipLaunchKernelGGL((attention_fwd_kernel<64>), grid, dim3(kAttThreads), smem, as_stream(stream),
                            static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k), static_cast<const bf16_t*>(vt),
                            static_cast<bf16_t*>(out), lse, Hq, Hkv, L, Lk, Lp, scale_log2, B);
     }
