@@ -43,6 +43,20 @@ def test_argument_errors_return_codes_not_exits():
     assert lib.ats_rope_fwd(None, None, None, None, None, None, 4, 4, 1, 1, 1, 4, 7, 0, 0, 0, 0, 0, 0, 0, 0,
                             None) == -1       # odd head_dim
     assert lib.ats_select_topk_per_sequence(None, 1, 10000, 5, None, None) == -1
+    # attention: head_dim outside {64, 128}, fewer keys than queries, query heads not a multiple of kv heads
+    assert lib.ats_attention_fwd(None, None, None, None, None, 1, 4, 2, 16, 16, 96, 0.1, None) == -2
+    assert b"head_dim" in lib.ats_last_error_string()
+    assert lib.ats_attention_fwd(None, None, None, None, None, 1, 4, 2, 16, 8, 128, 0.1, None) == -1
+    assert lib.ats_attention_fwd(None, None, None, None, None, 1, 3, 2, 16, 16, 128, 0.1, None) == -1
+    assert lib.ats_attention_fwd(None, None, None, None, None, 1, 4, 2, 16, 16, 128, 0.1, None) == -1     # null pointers
+    assert lib.ats_attention_fwd(None, None, None, None, None, 0, 4, 2, 16, 16, 128, 0.1, None) == 0      # empty batch
+    assert lib.ats_attention_bwd(*([None] * 12), 1, 4, 2, 16, 8, 128, 0.1, None) == -1
+    assert lib.ats_attention_bwd(*([None] * 12), 1, 4, 2, 16, 16, 32, 0.1, None) == -2
+    assert lib.ats_attention_delta(None, None, None, 1, 4, 16, 80, None) == -2
+    # V^T rows: whole 64-key tiles and a pitch that is an odd multiple of 256 bytes
+    for L in (1, 63, 64, 65, 128, 129, 2048, 4096, 5000):
+        Lp = lib.ats_attention_padded_len(L)
+        assert Lp >= L and Lp % 64 == 0 and (Lp * 2 // 256) % 2 == 1 and Lp - L < 4 * 64 + 64
     assert lib.ats_route_topk_workspace(16384, 8) > 0
     assert lib.ats_dispatch_plan_workspace(16384, 2, 8) == (32768 // 256) * 8 * 4
 
@@ -113,6 +127,20 @@ def test_no_cpu_fallback_and_module_surface():
     assert A.RMSNorm(8).state_dict()["weight"].shape == (8,)
     assert list(A.RotaryEmbedding(8).state_dict()) == []           # buffers are non-persistent
     assert A.MoECUDAOps.should_use_cuda(1, 1, 1, True, False) is False
+    # attention sub-layer and block: the reference's parameter names; CPU tensors are refused
+    cfg = LayerConfig(64, 128, 4, 2, num_heads=4, num_kv_heads=2, seq_length=32, use_moe=True)
+    att = A.GroupedQueryAttention(cfg)
+    assert {k: tuple(v.shape) for k, v in att.state_dict().items()} == {
+        "q_proj.weight": (64, 64), "k_proj.weight": (32, 64), "v_proj.weight": (32, 64), "o_proj.weight": (64, 64)}
+    with pytest.raises(A.AtsError):
+        att(torch.randn(1, 4, 64).bfloat16())
+    blk = A.TransformerBlock(cfg, layer_idx=0)
+    names = set(blk.state_dict())
+    assert {"input_norm.weight", "post_attn_norm.weight", "self_attn.o_proj.weight", "ffn.gate.weight",
+            "ffn.experts.3.down_proj.weight"} <= names
+    dense = A.TransformerBlock(LayerConfig(64, 128, 1, 1, num_heads=4, num_kv_heads=2, seq_length=32), layer_idx=0)
+    assert {"ffn.gate_up_proj.weight", "ffn.down_proj.weight"} <= set(dense.state_dict())
+    assert A.DenseGroupedQueryAttention is A.GroupedQueryAttention
 
 
 def test_workloads_are_reproducible():
