@@ -69,12 +69,16 @@ __global__ __launch_bounds__(256) void attention_vt_kernel(const bf16_t* __restr
     }
 }
 
-// One 128-row query tile of one (batch, query head) against its visible keys.
+// One tile of query rows (32 per wave) against its visible keys.  The rows are the queries of one
+// (batch, query head), or -- `pack` -- the queries of all query heads of one (batch, kv head), position
+// major: row r is position r / rep of head hkv * rep + r % rep.  Packing fills the tile when there are few
+// positions (decoding against a cache: one position, rep rows instead of one).
 template <int D>
 __device__ __forceinline__ void attention_q_tile(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
                                                  const bf16_t* __restrict__ vt, bf16_t* __restrict__ out,
                                                  float* __restrict__ lse, int Hq, int Hkv, int L, int Lk, int Lp,
-                                                 float scale_log2, int qt, int hq, int b, unsigned char* smem) {
+                                                 float scale_log2, int qt, int head, int b, bool pack,
+                                                 unsigned char* smem) {
     constexpr int KS = D / 16;              // k-steps of the score product
     constexpr int DB = D / 32;              // 32-row blocks of the output (transposed)
     constexpr int KPITCH = D * 2 + 16;      // bytes per K row in LDS
@@ -87,11 +91,17 @@ __device__ __forceinline__ void attention_q_tile(const bf16_t* __restrict__ q, c
 #define ATT_SK(stage_) (smem + (stage_) * (KTILE + VTILE))
 #define ATT_SV(stage_) (smem + (stage_) * (KTILE + VTILE) + KTILE)
 
-    const int hkv = hq / (Hq / Hkv);
+    const int rep = Hq / Hkv;
+    const int rp = pack ? rep : 1;                  // rows per position
+    const int n_rows = L * rp;
+    const int hkv = pack ? head : head / rep;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int col = lane & 31, g = lane >> 5;
-    const int q_row = qt * kAttBM + wave * 32 + col;          // this lane's query
-    const int q_clamped = q_row < L ? q_row : L - 1;
+    const int row = qt * kAttBM + wave * 32 + col;            // this lane's row
+    const int row_clamped = row < n_rows ? row : n_rows - 1;
+    const int q_clamped = row_clamped / rp;                   // its position among the queries
+    const int hq = pack ? hkv * rep + row_clamped % rp : head;
+    const bool row_valid = row < n_rows;
 
     const bf16_t* qp = q + ((int64_t)(b * Hq + hq) * L + q_clamped) * D;
     const bf16_t* kbase = k + (int64_t)(b * Hkv + hkv) * Lk * D;
@@ -128,11 +138,12 @@ __device__ __forceinline__ void attention_q_tile(const bf16_t* __restrict__ q, c
 
     // Query i sits at position i + (Lk - L): with cached keys in front the causal diagonal moves right.
     const int off = Lk - L;
-    const int q_pos = q_row + off;                              // last key this lane's query sees
-    const int q_block_last = min(qt * kAttBM + kAttBM - 1, L - 1) + off;
+    const int q_pos = row / rp + off;                           // last key this lane's query sees
+    const int q_block_last = min(qt * kAttBM + kAttBM - 1, n_rows - 1) / rp + off;
     const int n_tiles = q_block_last / kAttBN + 1;
-    const int q_wave_first = qt * kAttBM + wave * 32 + off;
-    const int q_wave_last = q_wave_first + 31;
+    const int q_wave_first = (qt * kAttBM + wave * 32) / rp + off;
+    // a wave without rows (packed tiles of a short batch) only helps to load
+    const int q_wave_last = qt * kAttBM + wave * 32 < n_rows ? (qt * kAttBM + wave * 32 + 31) / rp + off : -1;
 
     // One barrier per key tile: tile t+1 travels global -> registers while tile t is computed and lands in
     // the other LDS stage at the end of the iteration.  LDS operand fragments are read kRing MFMAs ahead
@@ -307,8 +318,8 @@ __device__ __forceinline__ void attention_q_tile(const bf16_t* __restrict__ q, c
     // ---- normalise and write [B, L, Hq*D]
     l_run += __shfl_xor(l_run, 32, 64);
     const float inv = 1.0f / l_run;
-    if (q_row < L) {
-        bf16_t* orow = out + ((int64_t)b * L + q_row) * (int64_t)(Hq * D) + hq * D;
+    if (row_valid) {
+        bf16_t* orow = out + ((int64_t)b * L + q_clamped) * (int64_t)(Hq * D) + hq * D;
 #pragma unroll
         for (int d = 0; d < DB; ++d)
 #pragma unroll
@@ -318,7 +329,7 @@ __device__ __forceinline__ void attention_q_tile(const bf16_t* __restrict__ q, c
                 w.y = pack_bf16x2(acc_o[d][r * 4 + 2] * inv, acc_o[d][r * 4 + 3] * inv);
                 *reinterpret_cast<au32x2_t*>(orow + d * 32 + r * 8 + g * 4) = w;
             }
-        if (lse && g == 0) lse[(int64_t)(b * Hq + hq) * L + q_row] = (m_run + log2f(l_run)) * 0.6931471805599453f;
+        if (lse && g == 0) lse[(int64_t)(b * Hq + hq) * L + q_clamped] = (m_run + log2f(l_run)) * 0.6931471805599453f;
     }
 #undef ATT_SK
 #undef ATT_SV
@@ -334,11 +345,12 @@ template <int D>
 __global__ __launch_bounds__(kAttThreads, 512 / kAttThreads) void attention_fwd_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
                                                             const bf16_t* __restrict__ vt, bf16_t* __restrict__ out,
                                                             float* __restrict__ lse, int Hq, int Hkv, int L, int Lk, int Lp,
-                                                            float scale_log2, int B) {
+                                                            float scale_log2, int B, int pack) {
     extern __shared__ __align__(16) unsigned char smem[];
-    const int n_qt = (L + kAttBM - 1) / kAttBM;
+    const int heads_per_group = pack ? 1 : Hq / Hkv;     // packed: the group's heads share the rows of a tile
+    const int n_qt = (L * (pack ? Hq / Hkv : 1) + kAttBM - 1) / kAttBM;
     const int n_pairs = (n_qt + 1) / 2;
-    const int per_group = n_pairs * (Hq / Hkv);          // workgroups sharing one K/V
+    const int per_group = n_pairs * heads_per_group;     // workgroups sharing one K/V
     const int n_groups = B * Hkv;
     int group, within;
     if (n_groups % 8 == 0) {
@@ -350,13 +362,14 @@ __global__ __launch_bounds__(kAttThreads, 512 / kAttThreads) void attention_fwd_
         within = blockIdx.x % per_group;
     }
     const int b = group / Hkv;
-    const int hq = (group % Hkv) * (Hq / Hkv) + within / n_pairs;
+    const int head = pack ? group % Hkv : (group % Hkv) * heads_per_group + within / n_pairs;
     const int pair = within % n_pairs;
     const int qt_long = n_qt - 1 - pair;
 #pragma unroll 1
     for (int half = 0; half < 2; ++half) {
         if (half && pair == qt_long) break;   // an odd tile count leaves the middle tile on its own
-        attention_q_tile<D>(q, k, vt, out, lse, Hq, Hkv, L, Lk, Lp, scale_log2, half ? pair : qt_long, hq, b, smem);
+        attention_q_tile<D>(q, k, vt, out, lse, Hq, Hkv, L, Lk, Lp, scale_log2, half ? pair : qt_long, head, b,
+                            pack != 0, smem);
     }
 }
 
@@ -403,7 +416,10 @@ extern "C" int ats_attention_fwd(const void* q, const void* k, const void* vt, v
     const int Lp = (int)ats_attention_padded_len(Lk);
     ATS_REQUIRE((int64_t)Lp * D * 2 < 0x7fffffffLL, ATS_ERR_UNSUPPORTED,
                 "ats_attention_fwd: %d keys (one head's K or V must stay under 2 GiB)", Lk);
-    const int64_t n_blocks = (int64_t)(((L + kAttBM - 1) / kAttBM + 1) / 2) * Hq * B;
+    // few query positions (decoding, short chunks): the query heads of a kv group share a tile's rows
+    const int pack = (L < kAttBM && Hq > Hkv) ? 1 : 0;
+    const int64_t n_blocks = pack ? (int64_t)((((int64_t)L * (Hq / Hkv) + kAttBM - 1) / kAttBM + 1) / 2) * Hkv * B
+                                  : (int64_t)(((L + kAttBM - 1) / kAttBM + 1) / 2) * Hq * B;
     ATS_REQUIRE(n_blocks <= 0x7fffffff, ATS_ERR_UNSUPPORTED, "ats_attention_fwd: %lld workgroups", (long long)n_blocks);
     const dim3 grid((unsigned)n_blocks);
     const float scale_log2 = scale * 1.4426950408889634f;
@@ -418,12 +434,12 @@ extern "C" int ats_attention_fwd(const void* q, const void* k, const void* vt, v
         }
         hipLaunchKernelGGL((attention_fwd_kernel<128>), grid, dim3(kAttThreads), smem, as_stream(stream),
                            static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k), static_cast<const bf16_t*>(vt),
-                           static_cast<bf16_t*>(out), lse, Hq, Hkv, L, Lk, Lp, scale_log2, B);
+                           static_cast<bf16_t*>(out), lse, Hq, Hkv, L, Lk, Lp, scale_log2, B, pack);
     } else {
         constexpr int smem = 2 * (kAttBN * (64 * 2 + 16) + 64 * (kAttBN * 2 + 8));
         hipLaunchKernelGGL((attention_fwd_kernel<64>), grid, dim3(kAttThreads), smem, as_stream(stream),
                            static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k), static_cast<const bf16_t*>(vt),
-                           static_cast<bf16_t*>(out), lse, Hq, Hkv, L, Lk, Lp, scale_log2, B);
+                           static_cast<bf16_t*>(out), lse, Hq, Hkv, L, Lk, Lp, scale_log2, B, pack);
     }
     ATS_CHECK_LAUNCH("ats_attention_fwd");
     return ATS_OK;

@@ -455,6 +455,56 @@ def run_block_train(args):
     }
 
 
+def run_attention_decode(args):
+    """One decoding step of the causal GQA attention: 64 sequences, one new token each, against a cache of 2048
+    keys (32 query / 8 kv heads, head_dim 128).  Bound by reading the cache once."""
+    from adaptivetrainingsystem_amd import ops
+    from adaptivetrainingsystem_amd.profiling import StageTimer
+    dev = torch.device("cuda:0")
+    B, Lk, Hq, Hkv, D = 64, 2048, 32, 8, 128
+    torch.manual_seed(10)
+    q = torch.randn(B, Hq, 1, D, device=dev).bfloat16()
+    k = torch.randn(B, Hkv, Lk, D, device=dev).bfloat16()
+    v = torch.randn(B, Hkv, Lk, D, device=dev).bfloat16()
+    for _ in range(args.warmup):
+        ops.causal_attention(q, k, v)
+    torch.cuda.synchronize()
+    timer = StageTimer()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        with timer.range("attention_decode"):
+            ops.causal_attention(q, k, v)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    st = timer.summary()
+    # K read once, V read and written once by the transpose and read once by the kernel
+    cache_bytes = 2.0 * B * Hkv * Lk * D * 2
+    achieved = cache_bytes / (st["attention_decode"]["mean_ms"] * 1e-3) / 1e9
+    log(f"  decode attention (V transpose + kernel) {st['attention_decode']['mean_ms']*1e3:.1f} us -> {achieved:.0f} GB/s of "
+        f"cache ({achieved / PEAK_HBM_GBS:.1%} of the HBM peak; the transpose moves V twice more)")
+    result = {
+        "metric": "causal GQA attention decode tokens/s", "value": B * args.steps / dt, "unit": "tokens/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": dt / args.steps * 1e3, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"attention_decode: {B} sequences x 1 new token against {Lk} cached keys, {Hq} query / "
+                               f"{Hkv} kv heads, head_dim {D}"},
+        "roofline": {"kernel": "attention_fwd_kernel, packed rows (+ V transpose)", "bound": "hbm", "achieved": achieved,
+                     "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": achieved / PEAK_HBM_GBS, "traffic": None},
+        "stages_ms": {s_: round(v_["mean_ms"], 4) for s_, v_ in st.items()},
+    }
+    if not args.no_cpu_baseline:
+        from oracle import sparse_layer_oracle as O
+        rep = Hq // Hkv
+        n = 8
+        qc, kc, vc = q[:n].float().cpu(), k[:n].float().cpu(), v[:n].float().cpu()
+        t0 = time.perf_counter()
+        O.attention_standard(qc, kc.repeat_interleave(rep, dim=1), vc.repeat_interleave(rep, dim=1), D ** -0.5)
+        cdt = time.perf_counter() - t0
+        result["cpu_baseline"] = {"value": n / cdt, "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
+                                  "sample": f"{n} of the {B} sequences, float32, one pass ({cdt:.2f} s)"}
+    return result
+
+
 def run_gqa_layer(args):
     """The attention sub-layer of the headline model shape (hidden 4096, 32 query / 8 kv heads, head_dim 128) on
     batch 8 x seq 2048: q/k/v projections, RoPE, causal attention, output projection."""
@@ -601,7 +651,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="c4_prefill",
                     choices=["c4_prefill", "c3_decode", "c5_finegrained_mod", "c1_cpu_reference", "c2_norm_rope",
-                             "c4_prefill_train", "c1_cpu_reference_train", "loss_clip", "attention", "attention_train", "gqa_layer", "block_train"])
+                             "c4_prefill_train", "c1_cpu_reference_train", "loss_clip", "attention", "attention_train", "attention_decode", "gqa_layer", "block_train"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a 1 GiB device copy (known traffic) so hardware-counter runs can be scaled")
@@ -634,6 +684,8 @@ def main():
         result = run_attention_train(args)
     elif args.workload == "block_train":
         result = run_block_train(args)
+    elif args.workload == "attention_decode":
+        result = run_attention_decode(args)
     elif args.workload == "gqa_layer":
         result = run_gqa_layer(args)
     elif args.workload.endswith("_train"):

@@ -50,6 +50,8 @@ def test_causal_attention(ops, gpu, B, Hq, Hkv, L, D):
 
 
 @pytest.mark.parametrize("B,Hq,Hkv,L,Lk,D", [(2, 4, 2, 1, 200, 128), (1, 2, 1, 1, 1, 64), (1, 4, 4, 70, 300, 64),
+                                             (3, 8, 2, 1, 513, 128), (2, 32, 8, 3, 100, 64), (1, 12, 2, 40, 77, 128),
+                                             (1, 16, 2, 127, 127, 64), (2, 6, 3, 33, 1000, 128),
                                              (2, 8, 2, 129, 130, 128), (1, 2, 2, 256, 1024, 128), (1, 4, 1, 5, 64, 128)])
 def test_causal_attention_with_cached_keys(ops, gpu, B, Hq, Hkv, L, Lk, D):
     """Lk - L cached keys in front of the queries: query i sees keys 0 .. i + Lk - L."""
