@@ -13,9 +13,9 @@
 // reductions are in-lane loops plus a single cross-lane exchange (lane ^ 32), and the accumulator of
 // S^T is already in B-operand order for the second product -- the keys a lane holds for k-step s are
 // {4g..4g+3, 8+4g..8+4g+3} + 16s (g = lane / 32); the V^T fragment is read with the same key order,
-// which is legal because the contraction over keys is a sum.  V^T ([B, Hkv, D, Lp], keys contiguous) is
-// produced once per call by a small transpose kernel, so every operand is read along its contiguous
-// dimension.
+// which is legal because the contraction over keys is a sum.  V stays as it is in memory ([key][d], any
+// batch / position / head strides) all the way into LDS; the V^T fragments come out of LDS through the
+// transposing read ds_read_b64_tr_b16, so no transposed copy of V is ever made.
 #include <math.h>
 
 #include "ats_common.hpp"
@@ -26,6 +26,8 @@ typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 abf16x8_t;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float af32x16_t;
 typedef unsigned int au32x4_t __attribute__((ext_vector_type(4)));
 typedef unsigned int au32x2_t __attribute__((ext_vector_type(2)));
+typedef short att_tr_t __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) att_tr_t* att_lds_tr_ptr_t;
 
 #ifndef ATT_THREADS
 #define ATT_THREADS 256
@@ -75,19 +77,19 @@ __global__ __launch_bounds__(256) void attention_vt_kernel(const bf16_t* __restr
 // positions (decoding against a cache: one position, rep rows instead of one).
 template <int D>
 __device__ __forceinline__ void attention_q_tile(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
-                                                 const bf16_t* __restrict__ vt, bf16_t* __restrict__ out,
-                                                 float* __restrict__ lse, int Hq, int Hkv, int L, int Lk, int Lp,
-                                                 float scale_log2, int qt, int head, int b, bool pack,
+                                                 const bf16_t* __restrict__ v, int64_t v_sb, int v_sl, int64_t v_sh,
+                                                 bf16_t* __restrict__ out, float* __restrict__ lse, int Hq, int Hkv,
+                                                 int L, int Lk, float scale_log2, int qt, int head, int b, bool pack,
                                                  unsigned char* smem) {
     constexpr int KS = D / 16;              // k-steps of the score product
     constexpr int DB = D / 32;              // 32-row blocks of the output (transposed)
     constexpr int KPITCH = D * 2 + 16;      // bytes per K row in LDS
-    constexpr int VPITCH = kAttBN * 2 + 8;  // bytes per V^T row in LDS
+    constexpr int VPITCH = D * 2 + 64;      // bytes per V row in LDS (see the transposing read below)
     constexpr int KTILE = kAttBN * KPITCH;
-    constexpr int VTILE = D * VPITCH;
+    constexpr int VTILE = kAttBN * VPITCH;
     constexpr int KVEC = kAttBN * (D / 8) / kAttThreads;   // 16-byte vectors per thread for a K tile
-    constexpr int VVEC = D * (kAttBN / 8) / kAttThreads;   // and for a V^T tile
-    // smem: [2 stages][K tile | V^T tile]
+    constexpr int VVEC = KVEC;                             // and for a V tile
+    // smem: [2 stages][K tile | V tile]
 #define ATT_SK(stage_) (smem + (stage_) * (KTILE + VTILE))
 #define ATT_SV(stage_) (smem + (stage_) * (KTILE + VTILE) + KTILE)
 
@@ -105,7 +107,7 @@ __device__ __forceinline__ void attention_q_tile(const bf16_t* __restrict__ q, c
 
     const bf16_t* qp = q + ((int64_t)(b * Hq + hq) * L + q_clamped) * D;
     const bf16_t* kbase = k + (int64_t)(b * Hkv + hkv) * Lk * D;
-    const bf16_t* vbase = vt + (int64_t)(b * Hkv + hkv) * D * Lp;
+    const bf16_t* vbase = v + b * v_sb + hkv * v_sh;          // row of key j at vbase + j * v_sl
 
     au32x4_t qf[KS];
 #pragma unroll
@@ -116,7 +118,7 @@ __device__ __forceinline__ void attention_q_tile(const bf16_t* __restrict__ q, c
     const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<bf16_t*>(kbase), 0, (int)((int64_t)Lk * D * 2), 0x00020000);
     const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<bf16_t*>(vbase), 0, (int)((int64_t)D * Lp * 2), 0x00020000);
+        const_cast<bf16_t*>(vbase), 0, (int)((((int64_t)Lk - 1) * v_sl + D) * 2), 0x00020000);
     int k_lane[KVEC], v_lane[VVEC];
 #pragma unroll
     for (int i = 0; i < KVEC; ++i) {
@@ -126,7 +128,7 @@ __device__ __forceinline__ void attention_q_tile(const bf16_t* __restrict__ q, c
 #pragma unroll
     for (int i = 0; i < VVEC; ++i) {
         const int idx = tid + i * kAttThreads;
-        v_lane[i] = ((idx / (kAttBN / 8)) * Lp + (idx % (kAttBN / 8)) * 8) * 2;
+        v_lane[i] = ((idx / (D / 8)) * v_sl + (idx % (D / 8)) * 8) * 2;
     }
 
     af32x16_t acc_o[DB];
@@ -167,10 +169,8 @@ __device__ __forceinline__ void attention_q_tile(const bf16_t* __restrict__ q, c
 #pragma unroll
         for (int i = 0; i < VVEC; ++i) {
             const int idx = tid + i * kAttThreads;
-            const int d = idx / (kAttBN / 8), c = idx % (kAttBN / 8);
-            const au32x2_t lo = {rv[i].x, rv[i].y}, hi = {rv[i].z, rv[i].w};
-            *reinterpret_cast<au32x2_t*>(ATT_SV(0) + d * VPITCH + c * 16) = lo;
-            *reinterpret_cast<au32x2_t*>(ATT_SV(0) + d * VPITCH + c * 16 + 8) = hi;
+            const int r = idx / (D / 8), c = idx % (D / 8);
+            *reinterpret_cast<au32x4_t*>(ATT_SV(0) + r * VPITCH + c * 16) = rv[i];
         }
         __syncthreads();
     }
@@ -196,7 +196,7 @@ __device__ __forceinline__ void attention_q_tile(const bf16_t* __restrict__ q, c
                 __builtin_amdgcn_raw_buffer_load_b128(k_rsrc, k_lane[(i_) < KVEC ? (i_) : 0], n1 * D * 2, 0); \
         else                                                                                           \
             rv[(i_) < KVEC ? 0 : (i_) - KVEC] = __builtin_amdgcn_raw_buffer_load_b128(                 \
-                v_rsrc, v_lane[(i_) < KVEC ? 0 : (i_) - KVEC], n1 * 2, 0);                             \
+                v_rsrc, v_lane[(i_) < KVEC ? 0 : (i_) - KVEC], n1 * v_sl * 2, 0);                      \
     }
         constexpr int NLOAD = KVEC + VVEC;
         constexpr int LOAD_EVERY = 2 * KS / NLOAD;
@@ -225,14 +225,24 @@ __device__ __forceinline__ void attention_q_tile(const bf16_t* __restrict__ q, c
             }
 #undef ATT_KFRAG
 #undef ATT_LOAD_ONE
-            // first V^T fragments travel during the softmax: fragment f = (k-step f/DB, output block f%DB)
-            const unsigned char* vr = sv + col * VPITCH + g * 8;
+            // First fragments of V^T travel during the softmax: fragment f = (k-step f/DB, output block f%DB).
+            // V sits in LDS as it does in memory ([key][d]); the A operand wants, per lane, one d and eight
+            // keys.  ds_read_b64_tr_b16 does 4x4 transposes inside groups of 16 lanes: the four lanes
+            // r = a + 4j (j = 0..3) each point at 4 consecutive d of key j, and lane 4a + c receives element
+            // c of all four, i.e. d = 4a + c for 4 consecutive keys.  With the addresses below lane l ends up
+            // with d = l % 32 and keys 4g .. 4g+3 (first read) and 8+4g .. 8+4g+3 (second read) of the
+            // k-step, which is the key order P^T has as the B operand.  The row pitch of D*2+64 bytes puts
+            // the 4 keys of a read 16 banks apart.
+            const unsigned char* vr =
+                sv + (4 * (lane >> 5) + ((lane & 15) >> 2)) * VPITCH + (16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
 #define ATT_VFRAG(f_, dst_)                                                                            \
     {                                                                                                  \
-        const unsigned char* p_ = vr + ((f_) % DB) * 32 * VPITCH + ((f_) / DB) * 32;                   \
-        const au32x2_t lo_ = *reinterpret_cast<const au32x2_t*>(p_);                                   \
-        const au32x2_t hi_ = *reinterpret_cast<const au32x2_t*>(p_ + 16);                              \
-        dst_ = au32x4_t{lo_.x, lo_.y, hi_.x, hi_.y};                                                   \
+        const unsigned char* p_ = vr + (((f_) / DB) * 16) * VPITCH + ((f_) % DB) * 64;                 \
+        const att_tr_t lo_ = __builtin_amdgcn_ds_read_tr16_b64_v4i16((att_lds_tr_ptr_t)(p_));           \
+        const att_tr_t hi_ = __builtin_amdgcn_ds_read_tr16_b64_v4i16((att_lds_tr_ptr_t)(p_ + 8 * VPITCH)); \
+        union { att_tr_t t[2]; au32x4_t u; } cv_;                                                     \
+        cv_.t[0] = lo_; cv_.t[1] = hi_;                                                                \
+        dst_ = cv_.u;                                                                                  \
     }
 #pragma unroll
             for (int f = 0; f < kRing; ++f) ATT_VFRAG(f, ring[f]);
@@ -305,11 +315,8 @@ __device__ __forceinline__ void attention_q_tile(const bf16_t* __restrict__ q, c
 #pragma unroll
             for (int i = 0; i < VVEC; ++i) {
                 const int idx = tid + i * kAttThreads;
-                const int d = idx / (kAttBN / 8), c = idx % (kAttBN / 8);
-                // 8-byte halves: the row pitch keeps 8-byte alignment only
-                const au32x2_t lo = {rv[i].x, rv[i].y}, hi = {rv[i].z, rv[i].w};
-                *reinterpret_cast<au32x2_t*>(dv + d * VPITCH + c * 16) = lo;
-                *reinterpret_cast<au32x2_t*>(dv + d * VPITCH + c * 16 + 8) = hi;
+                const int r = idx / (D / 8), c = idx % (D / 8);
+                *reinterpret_cast<au32x4_t*>(dv + r * VPITCH + c * 16) = rv[i];
             }
         }
         __syncthreads();
@@ -343,9 +350,9 @@ __device__ __forceinline__ void attention_q_tile(const bf16_t* __restrict__ q, c
 // in the shadow of the other's MFMAs.
 template <int D>
 __global__ __launch_bounds__(kAttThreads, 512 / kAttThreads) void attention_fwd_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
-                                                            const bf16_t* __restrict__ vt, bf16_t* __restrict__ out,
-                                                            float* __restrict__ lse, int Hq, int Hkv, int L, int Lk, int Lp,
-                                                            float scale_log2, int B, int pack) {
+                                                            const bf16_t* __restrict__ v, int64_t v_sb, int v_sl, int64_t v_sh,
+                                                            bf16_t* __restrict__ out, float* __restrict__ lse, int Hq, int Hkv,
+                                                            int L, int Lk, float scale_log2, int B, int pack) {
     extern __shared__ __align__(16) unsigned char smem[];
     const int heads_per_group = pack ? 1 : Hq / Hkv;     // packed: the group's heads share the rows of a tile
     const int n_qt = (L * (pack ? Hq / Hkv : 1) + kAttBM - 1) / kAttBM;
@@ -368,8 +375,8 @@ __global__ __launch_bounds__(kAttThreads, 512 / kAttThreads) void attention_fwd_
 #pragma unroll 1
     for (int half = 0; half < 2; ++half) {
         if (half && pair == qt_long) break;   // an odd tile count leaves the middle tile on its own
-        attention_q_tile<D>(q, k, vt, out, lse, Hq, Hkv, L, Lk, Lp, scale_log2, half ? pair : qt_long, head, b,
-                            pack != 0, smem);
+        attention_q_tile<D>(q, k, v, v_sb, v_sl, v_sh, out, lse, Hq, Hkv, L, Lk, scale_log2, half ? pair : qt_long,
+                            head, b, pack != 0, smem);
     }
 }
 
@@ -404,17 +411,20 @@ extern "C" int ats_attention_transpose_v(const void* v, int64_t sb, int64_t sl, 
     return ATS_OK;
 }
 
-extern "C" int ats_attention_fwd(const void* q, const void* k, const void* vt, void* out, float* lse, int B, int Hq,
-                                 int Hkv, int L, int Lk, int D, float scale, ats_stream_t stream) {
+extern "C" int ats_attention_fwd(const void* q, const void* k, const void* v, int64_t v_sb, int64_t v_sl, int64_t v_sh,
+                                 void* out, float* lse, int B, int Hq, int Hkv, int L, int Lk, int D, float scale,
+                                 ats_stream_t stream) {
     using namespace ats;
     ATS_REQUIRE(B >= 0 && Hq > 0 && Hkv > 0 && Hq % Hkv == 0 && L >= 0 && Lk >= L && scale > 0.f, ATS_ERR_INVALID_ARG,
                 "ats_attention_fwd: B=%d Hq=%d Hkv=%d L=%d Lk=%d scale=%g", B, Hq, Hkv, L, Lk, scale);
     ATS_REQUIRE(D == 64 || D == 128, ATS_ERR_UNSUPPORTED, "ats_attention_fwd: head_dim %d (64 or 128)", D);
     if (B == 0 || L == 0) return ATS_OK;
-    ATS_REQUIRE(q && k && vt && out && aligned16(q) && aligned16(k) && aligned16(vt) && aligned16(out),
+    ATS_REQUIRE(q && k && v && out && aligned16(q) && aligned16(k) && aligned16(v) && aligned16(out),
                 ATS_ERR_INVALID_ARG, "ats_attention_fwd: null or misaligned pointer");
-    const int Lp = (int)ats_attention_padded_len(Lk);
-    ATS_REQUIRE((int64_t)Lp * D * 2 < 0x7fffffffLL, ATS_ERR_UNSUPPORTED,
+    ATS_REQUIRE(v_sl >= D && v_sl % 8 == 0 && v_sb % 8 == 0 && v_sh % 8 == 0 && v_sb >= 0 && v_sh >= 0, ATS_ERR_INVALID_ARG,
+                "ats_attention_fwd: strides of v (%lld, %lld, %lld) must be multiples of 8 elements, rows apart",
+                (long long)v_sb, (long long)v_sl, (long long)v_sh);
+    ATS_REQUIRE((int64_t)Lk * D * 2 < 0x7fffffffLL && ((int64_t)Lk * v_sl + D) * 2 < 0x7fffffffLL, ATS_ERR_UNSUPPORTED,
                 "ats_attention_fwd: %d keys (one head's K or V must stay under 2 GiB)", Lk);
     // few query positions (decoding, short chunks): the query heads of a kv group share a tile's rows
     const int pack = (L < kAttBM && Hq > Hkv) ? 1 : 0;
@@ -424,7 +434,7 @@ extern "C" int ats_attention_fwd(const void* q, const void* k, const void* vt, v
     const dim3 grid((unsigned)n_blocks);
     const float scale_log2 = scale * 1.4426950408889634f;
     if (D == 128) {
-        constexpr int smem = 2 * (kAttBN * (128 * 2 + 16) + 128 * (kAttBN * 2 + 8));
+        constexpr int smem = 2 * kAttBN * ((128 * 2 + 16) + (128 * 2 + 64));
         static bool attr = false;
         if (!attr) {
             hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(attention_fwd_kernel<128>),
@@ -433,13 +443,13 @@ extern "C" int ats_attention_fwd(const void* q, const void* k, const void* vt, v
             attr = true;
         }
         hipLaunchKernelGGL((attention_fwd_kernel<128>), grid, dim3(kAttThreads), smem, as_stream(stream),
-                           static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k), static_cast<const bf16_t*>(vt),
-                           static_cast<bf16_t*>(out), lse, Hq, Hkv, L, Lk, Lp, scale_log2, B, pack);
+                           static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k), static_cast<const bf16_t*>(v),
+                           v_sb, (int)v_sl, v_sh, static_cast<bf16_t*>(out), lse, Hq, Hkv, L, Lk, scale_log2, B, pack);
     } else {
-        constexpr int smem = 2 * (kAttBN * (64 * 2 + 16) + 64 * (kAttBN * 2 + 8));
+        constexpr int smem = 2 * kAttBN * ((64 * 2 + 16) + (64 * 2 + 64));
         hipLaunchKernelGGL((attention_fwd_kernel<64>), grid, dim3(kAttThreads), smem, as_stream(stream),
-                           static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k), static_cast<const bf16_t*>(vt),
-                           static_cast<bf16_t*>(out), lse, Hq, Hkv, L, Lk, Lp, scale_log2, B, pack);
+                           static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k), static_cast<const bf16_t*>(v),
+                           v_sb, (int)v_sl, v_sh, static_cast<bf16_t*>(out), lse, Hq, Hkv, L, Lk, scale_log2, B, pack);
     }
     ATS_CHECK_LAUNCH("ats_attention_fwd");
     return ATS_OK;

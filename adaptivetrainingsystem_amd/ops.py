@@ -586,17 +586,14 @@ def causal_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: O
     if k.shape != (B, Hkv, Lk, D) or v.shape != (B, Hkv, Lk, D) or Hq % Hkv != 0 or Lk < L:
         raise AtsError(f"causal_attention: shapes q {tuple(q.shape)} k {tuple(k.shape)} v {tuple(v.shape)}")
     q, k = q.contiguous(), k.contiguous()
-    if v.stride(3) != 1 or any(st % 8 for st in v.stride()[:3]) or v.data_ptr() % 16:
+    if v.stride(3) != 1 or any(st % 8 for st in v.stride()[:3]) or v.stride(2) < D or v.data_ptr() % 16:
         v = v.contiguous()
     lib = _lib.load()
-    Lp = int(lib.ats_attention_padded_len(Lk))
-    vt = torch.empty(B, Hkv, D, Lp, dtype=q.dtype, device=q.device)
-    check(lib.ats_attention_transpose_v(v.data_ptr(), v.stride(0), v.stride(2), v.stride(1), vt.data_ptr(), B, Hkv, Lk, D,
-                                        _stream()), "ats_attention_transpose_v")
     out = torch.empty(B, L, Hq * D, dtype=q.dtype, device=q.device)
     lse = torch.empty(B, Hq, L, dtype=torch.float32, device=q.device) if return_lse else None
-    check(lib.ats_attention_fwd(q.data_ptr(), k.data_ptr(), vt.data_ptr(), out.data_ptr(), _ptr(lse), B, Hq, Hkv, L, Lk,
-                                D, float(D ** -0.5 if scale is None else scale), _stream()), "ats_attention_fwd")
+    check(lib.ats_attention_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), v.stride(0), v.stride(2), v.stride(1),
+                                out.data_ptr(), _ptr(lse), B, Hq, Hkv, L, Lk, D,
+                                float(D ** -0.5 if scale is None else scale), _stream()), "ats_attention_fwd")
     return (out, lse) if return_lse else out
 
 
