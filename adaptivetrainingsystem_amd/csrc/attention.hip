@@ -46,31 +46,6 @@ __device__ __forceinline__ af32x16_t att_mma(const au32x4_t& a, const au32x4_t& 
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(x.v, y.v, c, 0, 0, 0);
 }
 
-// v: [B, L, *] rows with element strides (batch, position, head; D contiguous) -> vt [B, Hkv, D, Lp],
-// zero padded for positions >= L.  One block per (64 positions, head, batch).
-template <int D>
-__global__ __launch_bounds__(256) void attention_vt_kernel(const bf16_t* __restrict__ v, int64_t sb, int64_t sl,
-                                                           int64_t sh, bf16_t* __restrict__ vt, int Hkv, int L,
-                                                           int Lp) {
-    __shared__ bf16_t tile[D][64 + 8];
-    const int l0 = blockIdx.x * 64, h = blockIdx.y, b = blockIdx.z;
-    const bf16_t* src = v + b * sb + h * sh;
-    for (int i = threadIdx.x; i < 64 * (D / 8); i += 256) {
-        const int r = i / (D / 8), c0 = (i % (D / 8)) * 8;
-        uint4 raw = make_uint4(0u, 0u, 0u, 0u);
-        if (l0 + r < L) raw = *reinterpret_cast<const uint4*>(src + (int64_t)(l0 + r) * sl + c0);
-        const bf16_t* e = reinterpret_cast<const bf16_t*>(&raw);
-#pragma unroll
-        for (int j = 0; j < 8; ++j) tile[c0 + j][r] = e[j];
-    }
-    __syncthreads();
-    bf16_t* dst = vt + ((int64_t)(b * Hkv + h) * D) * Lp + l0;
-    for (int i = threadIdx.x; i < D * 8; i += 256) {
-        const int d = i / 8, r0 = (i % 8) * 8;
-        *reinterpret_cast<uint4*>(dst + (int64_t)d * Lp + r0) = *reinterpret_cast<const uint4*>(&tile[d][r0]);
-    }
-}
-
 // One tile of query rows (32 per wave) against its visible keys.  The rows are the queries of one
 // (batch, query head), or -- `pack` -- the queries of all query heads of one (batch, kv head), position
 // major: row r is position r / rep of head hkv * rep + r % rep.  Packing fills the tile when there are few
@@ -381,35 +356,6 @@ __global__ __launch_bounds__(kAttThreads, 512 / kAttThreads) void attention_fwd_
 }
 
 }  // namespace ats
-
-// Row length of V^T: whole key tiles, and a row pitch of an odd multiple of 256 bytes.  A key tile reads the
-// same 128 bytes of every row of V^T; with a power-of-two pitch (4096 bytes at 2048 keys) all those rows
-// sit in one L2 channel, which then serves every workgroup of the (batch, kv head) on its own.
-extern "C" int64_t ats_attention_padded_len(int L) {
-    int64_t tiles = ((int64_t)L + ats::kAttBN - 1) / ats::kAttBN;
-    while (tiles % 4 != 2) ++tiles;
-    return tiles * ats::kAttBN;
-}
-
-extern "C" int ats_attention_transpose_v(const void* v, int64_t sb, int64_t sl, int64_t sh, void* vt, int B, int Hkv,
-                                         int L, int D, ats_stream_t stream) {
-    using namespace ats;
-    ATS_REQUIRE(B >= 0 && Hkv > 0 && L >= 0 && (D == 64 || D == 128), ATS_ERR_UNSUPPORTED,
-                "ats_attention_transpose_v: B=%d Hkv=%d L=%d D=%d (head_dim 64 or 128)", B, Hkv, L, D);
-    if (B == 0 || L == 0) return ATS_OK;
-    ATS_REQUIRE(v && vt && aligned16(v) && aligned16(vt) && sb % 8 == 0 && sl % 8 == 0 && sh % 8 == 0,
-                ATS_ERR_INVALID_ARG, "ats_attention_transpose_v: pointers and strides must be 16-byte aligned");
-    const int Lp = (int)ats_attention_padded_len(L);
-    const dim3 grid((unsigned)(Lp / 64), (unsigned)Hkv, (unsigned)B);
-    if (D == 128)
-        hipLaunchKernelGGL((attention_vt_kernel<128>), grid, dim3(256), 0, as_stream(stream),
-                           static_cast<const bf16_t*>(v), sb, sl, sh, static_cast<bf16_t*>(vt), Hkv, L, Lp);
-    else
-        hipLaunchKernelGGL((attention_vt_kernel<64>), grid, dim3(256), 0, as_stream(stream),
-                           static_cast<const bf16_t*>(v), sb, sl, sh, static_cast<bf16_t*>(vt), Hkv, L, Lp);
-    ATS_CHECK_LAUNCH("ats_attention_transpose_v");
-    return ATS_OK;
-}
 
 extern "C" int ats_attention_fwd(const void* q, const void* k, const void* v, int64_t v_sb, int64_t v_sl, int64_t v_sh,
                                  void* out, float* lse, int B, int Hq, int Hkv, int L, int Lk, int D, float scale,

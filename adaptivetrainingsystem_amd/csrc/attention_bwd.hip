@@ -12,9 +12,11 @@
 //
 // Same MFMA layout trick as the forward: products are formed transposed so that a lane of the 32x32
 // accumulator owns one row of the side the block owns (a query in the dQ kernel, a key in the dK/dV
-// kernel).  The operand that changes from step to step is read from LDS as the A operand along its
-// contiguous dimension; the transposed copies this needs (K^T for dQ, Q^T and dO^T for dK/dV) are made
-// once per call by the transpose kernel of the forward.
+// kernel).  The operand that changes from step to step is the A operand and comes from LDS, where a
+// tile is kept as it is in memory (rows of D elements): fragments along D are plain 16-byte reads,
+// fragments across rows (K^T for dQ, Q^T and dO^T for dK/dV) come out through the transposing read
+// ds_read_b64_tr_b16, so no transposed copy of any operand is made.  The two access patterns want
+// different row pitches to stay free of bank conflicts, so a tile that is read both ways is stored twice.
 #include <math.h>
 
 #include "ats_common.hpp"
@@ -25,6 +27,25 @@ typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bbf16x8_t;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float bf32x16_t;
 typedef unsigned int bu32x4_t __attribute__((ext_vector_type(4)));
 typedef unsigned int bu32x2_t __attribute__((ext_vector_type(2)));
+typedef short btr_t __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) btr_t* blds_tr_ptr_t;
+
+// A-operand fragment of X^T for one 32x32x16 MFMA from a tile stored [row][d] with pitch `pitch` bytes:
+// lane l receives d = d0 + l % 32 and rows r0 + {4g..4g+3, 8+4g..8+4g+3} (g = l / 32), the order in which a
+// 32x32 accumulator hands its rows to the next product.  `lane_base` is tr_lane_base(tile, lane, pitch).
+__device__ __forceinline__ const unsigned char* tr_lane_base(const unsigned char* tile, int lane, int pitch) {
+    return tile + (4 * (lane >> 5) + ((lane & 15) >> 2)) * pitch + (16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
+}
+__device__ __forceinline__ bu32x4_t tr_fragment(const unsigned char* lane_base, int r0, int d0, int pitch) {
+    const unsigned char* p = lane_base + r0 * pitch + d0 * 2;
+    union {
+        btr_t t[2];
+        bu32x4_t u;
+    } cv;
+    cv.t[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((blds_tr_ptr_t)(p));
+    cv.t[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((blds_tr_ptr_t)(p + 8 * pitch));
+    return cv.u;
+}
 
 constexpr int kBwdRows = 128;   // rows a block owns: 4 waves x 32
 constexpr int kDqBN = 64;       // keys per step of the dQ kernel
@@ -72,18 +93,16 @@ __global__ __launch_bounds__(256) void attention_delta_kernel(const bf16_t* __re
 // One 128-row query tile of one (batch, query head): lanes own queries, keys come in tiles of 64.
 template <int D>
 __device__ __forceinline__ void attention_bwd_dq_tile(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
-                                                      const bf16_t* __restrict__ v, const bf16_t* __restrict__ kt,
-                                                      const bf16_t* __restrict__ dout, const float* __restrict__ lse,
-                                                      const float* __restrict__ delta, bf16_t* __restrict__ dq, int Hq,
-                                                      int Hkv, int L, int Lk, int Lp, float scale, int qt, int hq,
-                                                      int b, unsigned char* smem) {
+                                                      const bf16_t* __restrict__ v, const bf16_t* __restrict__ dout,
+                                                      const float* __restrict__ lse, const float* __restrict__ delta,
+                                                      bf16_t* __restrict__ dq, int Hq, int Hkv, int L, int Lk,
+                                                      float scale, int qt, int hq, int b, unsigned char* smem) {
     constexpr int KS = D / 16;
     constexpr int DB = D / 32;
     constexpr int RPITCH = D * 2 + 16;        // bytes per K / V row in LDS
-    constexpr int TPITCH = kDqBN * 2 + 8;     // bytes per K^T row in LDS
+    constexpr int TPITCH = D * 2 + 64;        // bytes per row of the second copy of K (transposing reads)
     constexpr int RTILE = kDqBN * RPITCH;
     constexpr int RVEC = kDqBN * (D / 8) / 256;
-    constexpr int TVEC = D * (kDqBN / 8) / 256;
     unsigned char* const sK = smem;
     unsigned char* const sV = smem + RTILE;
     unsigned char* const sT = smem + 2 * RTILE;
@@ -110,14 +129,11 @@ __device__ __forceinline__ void attention_bwd_dq_tile(const bf16_t* __restrict__
 
     const bf16_t* kbase = k + (int64_t)(b * Hkv + hkv) * Lk * D;
     const bf16_t* vbase = v + (int64_t)(b * Hkv + hkv) * Lk * D;
-    const bf16_t* tbase = kt + (int64_t)(b * Hkv + hkv) * D * Lp;
     // buffer loads: keys past Lk read as zeros
     const __amdgpu_buffer_rsrc_t k_rsrc =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(kbase), 0, (int)((int64_t)Lk * D * 2), 0x00020000);
     const __amdgpu_buffer_rsrc_t v_rsrc =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(vbase), 0, (int)((int64_t)Lk * D * 2), 0x00020000);
-    const __amdgpu_buffer_rsrc_t t_rsrc =
-        __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(tbase), 0, (int)((int64_t)D * Lp * 2), 0x00020000);
 
     bf32x16_t acc_dq[DB];
 #pragma unroll
@@ -137,7 +153,7 @@ __device__ __forceinline__ void attention_bwd_dq_tile(const bf16_t* __restrict__
         const int n0 = t * kDqBN;
         __syncthreads();   // every wave is done with the previous tile
         {
-            bu32x4_t rk[RVEC], rv[RVEC], rt[TVEC];
+            bu32x4_t rk[RVEC], rv[RVEC];
 #pragma unroll
             for (int i = 0; i < RVEC; ++i) {
                 const int idx = tid + i * 256;
@@ -146,25 +162,12 @@ __device__ __forceinline__ void attention_bwd_dq_tile(const bf16_t* __restrict__
                 rv[i] = __builtin_amdgcn_raw_buffer_load_b128(v_rsrc, lo, n0 * D * 2, 0);
             }
 #pragma unroll
-            for (int i = 0; i < TVEC; ++i) {
-                const int idx = tid + i * 256;
-                const int lo = ((idx / (kDqBN / 8)) * Lp + (idx % (kDqBN / 8)) * 8) * 2;
-                rt[i] = __builtin_amdgcn_raw_buffer_load_b128(t_rsrc, lo, n0 * 2, 0);
-            }
-#pragma unroll
             for (int i = 0; i < RVEC; ++i) {
                 const int idx = tid + i * 256;
                 const int r = idx / (D / 8), c = idx % (D / 8);
                 *reinterpret_cast<bu32x4_t*>(sK + r * RPITCH + c * 16) = rk[i];
                 *reinterpret_cast<bu32x4_t*>(sV + r * RPITCH + c * 16) = rv[i];
-            }
-#pragma unroll
-            for (int i = 0; i < TVEC; ++i) {
-                const int idx = tid + i * 256;
-                const int d = idx / (kDqBN / 8), c = idx % (kDqBN / 8);
-                const bu32x2_t lo = {rt[i].x, rt[i].y}, hi = {rt[i].z, rt[i].w};
-                *reinterpret_cast<bu32x2_t*>(sT + d * TPITCH + c * 16) = lo;
-                *reinterpret_cast<bu32x2_t*>(sT + d * TPITCH + c * 16 + 8) = hi;
+                *reinterpret_cast<bu32x4_t*>(sT + r * TPITCH + c * 16) = rk[i];
             }
         }
         __syncthreads();
@@ -210,15 +213,12 @@ __device__ __forceinline__ void attention_bwd_dq_tile(const bf16_t* __restrict__
             dsf[s].w = pack_bf16x2(acc_s[kb][x0 + 6], acc_s[kb][x0 + 7]);
         }
         // ---- dQ^T += K^T . dS^T  (keys of a k-step in accumulator order, as in the forward's second product)
+        const unsigned char* t_lane = tr_lane_base(sT, lane, TPITCH);
 #pragma unroll
         for (int s = 0; s < 4; ++s)
 #pragma unroll
-            for (int d = 0; d < DB; ++d) {
-                const unsigned char* tr = sT + (d * 32 + col) * TPITCH + (s * 16 + g * 4) * 2;
-                const bu32x2_t lo = *reinterpret_cast<const bu32x2_t*>(tr);
-                const bu32x2_t hi = *reinterpret_cast<const bu32x2_t*>(tr + 16);
-                acc_dq[d] = bwd_mma(bu32x4_t{lo.x, lo.y, hi.x, hi.y}, dsf[s], acc_dq[d]);
-            }
+            for (int d = 0; d < DB; ++d)
+                acc_dq[d] = bwd_mma(tr_fragment(t_lane, s * 16, d * 32, TPITCH), dsf[s], acc_dq[d]);
     }
 
     if (q_row < L) {
@@ -240,9 +240,8 @@ __device__ __forceinline__ void attention_bwd_dq_tile(const bf16_t* __restrict__
 template <int D>
 __global__ __launch_bounds__(256, 2) void attention_bwd_dq_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const bf16_t* __restrict__ v,
-    const bf16_t* __restrict__ kt, const bf16_t* __restrict__ dout, const float* __restrict__ lse,
-    const float* __restrict__ delta, bf16_t* __restrict__ dq, int Hq, int Hkv, int L, int Lk, int Lp, float scale,
-    int B) {
+    const bf16_t* __restrict__ dout, const float* __restrict__ lse, const float* __restrict__ delta,
+    bf16_t* __restrict__ dq, int Hq, int Hkv, int L, int Lk, float scale, int B) {
     extern __shared__ __align__(16) unsigned char smem[];
     const int n_qt = (L + kBwdRows - 1) / kBwdRows;
     const int n_pairs = (n_qt + 1) / 2;
@@ -264,8 +263,8 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dq_kernel(
 #pragma unroll 1
     for (int half = 0; half < 2; ++half) {
         if (half && pair == qt_long) break;
-        attention_bwd_dq_tile<D>(q, k, v, kt, dout, lse, delta, dq, Hq, Hkv, L, Lk, Lp, scale, half ? pair : qt_long,
-                                 hq, b, smem);
+        attention_bwd_dq_tile<D>(q, k, v, dout, lse, delta, dq, Hq, Hkv, L, Lk, scale, half ? pair : qt_long, hq, b,
+                                 smem);
     }
 }
 
@@ -273,21 +272,19 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dq_kernel(
 // One 128-row key tile of one (batch, kv head): lanes own keys; the queries of every query head of the
 // group come in steps of 32, starting at the first query that sees the tile.
 template <int D>
-__device__ __forceinline__ void attention_bwd_dkv_tile(const bf16_t* __restrict__ q, const bf16_t* __restrict__ qtr,
-                                                       const bf16_t* __restrict__ k, const bf16_t* __restrict__ v,
-                                                       const bf16_t* __restrict__ dout, const bf16_t* __restrict__ dotr,
+__device__ __forceinline__ void attention_bwd_dkv_tile(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
+                                                       const bf16_t* __restrict__ v, const bf16_t* __restrict__ dout,
                                                        const float* __restrict__ lse, const float* __restrict__ delta,
                                                        bf16_t* __restrict__ dk, bf16_t* __restrict__ dv, int Hq, int Hkv,
-                                                       int L, int Lk, int Lqp, float scale, int kt_idx, int hkv, int b,
+                                                       int L, int Lk, float scale, int kt_idx, int hkv, int b,
                                                        unsigned char* smem) {
     constexpr int KS = D / 16;
     constexpr int DB = D / 32;
     constexpr int RPITCH = D * 2 + 16;        // bytes per Q / dO row in LDS
-    constexpr int TPITCH = kDkvBQ * 2 + 8;    // bytes per Q^T / dO^T row in LDS
+    constexpr int TPITCH = D * 2 + 64;        // bytes per row of the second copies (transposing reads)
     constexpr int RTILE = kDkvBQ * RPITCH;
-    constexpr int TTILE = D * TPITCH;
+    constexpr int TTILE = kDkvBQ * TPITCH;
     constexpr int RVEC = kDkvBQ * (D / 8) / 256;   // 16-byte vectors per thread: D=128 -> 2, D=64 -> 1
-    constexpr int TVEC = D * (kDkvBQ / 8) / 256;   // D=128 -> 2, D=64 -> 1
     unsigned char* const sQ = smem;
     unsigned char* const sO = smem + RTILE;
     unsigned char* const sQT = smem + 2 * RTILE;
@@ -347,8 +344,6 @@ __device__ __forceinline__ void attention_bwd_dkv_tile(const bf16_t* __restrict_
         const int hq = hkv * rep + hh;
         const bf16_t* qbase = q + (int64_t)(b * Hq + hq) * L * D;
         const bf16_t* obase = dout + (int64_t)b * L * (int64_t)(Hq * D) + hq * D;
-        const bf16_t* qtbase = qtr + (int64_t)(b * Hq + hq) * D * Lqp;
-        const bf16_t* otbase = dotr + (int64_t)(b * Hq + hq) * D * Lqp;
         const float* lbase = lse + (int64_t)(b * Hq + hq) * L;
         const float* dbase = delta + (int64_t)(b * Hq + hq) * L;
         // buffer loads: query rows past L read as zeros
@@ -356,28 +351,17 @@ __device__ __forceinline__ void attention_bwd_dkv_tile(const bf16_t* __restrict_
             __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(qbase), 0, (int)((int64_t)L * D * 2), 0x00020000);
         const __amdgpu_buffer_rsrc_t o_rsrc = __builtin_amdgcn_make_buffer_rsrc(
             const_cast<bf16_t*>(obase), 0, (int)((((int64_t)L - 1) * Hq * D + D) * 2), 0x00020000);
-        const __amdgpu_buffer_rsrc_t qt_rsrc =
-            __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(qtbase), 0, (int)((int64_t)D * Lqp * 2), 0x00020000);
-        const __amdgpu_buffer_rsrc_t ot_rsrc =
-            __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(otbase), 0, (int)((int64_t)D * Lqp * 2), 0x00020000);
 
         for (int q0 = q_first; q0 < L; q0 += kDkvBQ) {
             __syncthreads();   // every wave is done with the previous step
             {
-                bu32x4_t rq[RVEC], ro[RVEC], rqt[TVEC], rot[TVEC];
+                bu32x4_t rq[RVEC], ro[RVEC];
 #pragma unroll
                 for (int i = 0; i < RVEC; ++i) {
                     const int idx = tid + i * 256;
                     const int r = idx / (D / 8), c = idx % (D / 8);
                     rq[i] = __builtin_amdgcn_raw_buffer_load_b128(q_rsrc, (r * D + c * 8) * 2, q0 * D * 2, 0);
                     ro[i] = __builtin_amdgcn_raw_buffer_load_b128(o_rsrc, (r * Hq * D + c * 8) * 2, q0 * Hq * D * 2, 0);
-                }
-#pragma unroll
-                for (int i = 0; i < TVEC; ++i) {
-                    const int idx = tid + i * 256;
-                    const int d = idx / (kDkvBQ / 8), c = idx % (kDkvBQ / 8);
-                    rqt[i] = __builtin_amdgcn_raw_buffer_load_b128(qt_rsrc, (d * Lqp + c * 8) * 2, q0 * 2, 0);
-                    rot[i] = __builtin_amdgcn_raw_buffer_load_b128(ot_rsrc, (d * Lqp + c * 8) * 2, q0 * 2, 0);
                 }
                 if (tid < kDkvBQ) {
                     const int qi = q0 + tid;
@@ -390,17 +374,8 @@ __device__ __forceinline__ void attention_bwd_dkv_tile(const bf16_t* __restrict_
                     const int r = idx / (D / 8), c = idx % (D / 8);
                     *reinterpret_cast<bu32x4_t*>(sQ + r * RPITCH + c * 16) = rq[i];
                     *reinterpret_cast<bu32x4_t*>(sO + r * RPITCH + c * 16) = ro[i];
-                }
-#pragma unroll
-                for (int i = 0; i < TVEC; ++i) {
-                    const int idx = tid + i * 256;
-                    const int d = idx / (kDkvBQ / 8), c = idx % (kDkvBQ / 8);
-                    const bu32x2_t a0 = {rqt[i].x, rqt[i].y}, a1 = {rqt[i].z, rqt[i].w};
-                    const bu32x2_t b0 = {rot[i].x, rot[i].y}, b1 = {rot[i].z, rot[i].w};
-                    *reinterpret_cast<bu32x2_t*>(sQT + d * TPITCH + c * 16) = a0;
-                    *reinterpret_cast<bu32x2_t*>(sQT + d * TPITCH + c * 16 + 8) = a1;
-                    *reinterpret_cast<bu32x2_t*>(sOT + d * TPITCH + c * 16) = b0;
-                    *reinterpret_cast<bu32x2_t*>(sOT + d * TPITCH + c * 16 + 8) = b1;
+                    *reinterpret_cast<bu32x4_t*>(sQT + r * TPITCH + c * 16) = rq[i];
+                    *reinterpret_cast<bu32x4_t*>(sOT + r * TPITCH + c * 16) = ro[i];
                 }
             }
             __syncthreads();
@@ -451,17 +426,14 @@ __device__ __forceinline__ void attention_bwd_dkv_tile(const bf16_t* __restrict_
                 if (r == 3) { pf[1].z = p01; pf[1].w = p23; dsf[1].z = s01; dsf[1].w = s23; }
             }
             // ---- dV^T += dO^T . P and dK^T += Q^T . dS  (queries of a k-step in accumulator order)
+            const unsigned char* ot_lane = tr_lane_base(sOT, lane, TPITCH);
+            const unsigned char* qt_lane = tr_lane_base(sQT, lane, TPITCH);
 #pragma unroll
             for (int s = 0; s < 2; ++s)
 #pragma unroll
                 for (int d = 0; d < DB; ++d) {
-                    const int o = (d * 32 + col) * TPITCH + (s * 16 + g * 4) * 2;
-                    const bu32x2_t olo = *reinterpret_cast<const bu32x2_t*>(sOT + o);
-                    const bu32x2_t ohi = *reinterpret_cast<const bu32x2_t*>(sOT + o + 16);
-                    acc_dv[d] = bwd_mma(bu32x4_t{olo.x, olo.y, ohi.x, ohi.y}, pf[s], acc_dv[d]);
-                    const bu32x2_t qlo = *reinterpret_cast<const bu32x2_t*>(sQT + o);
-                    const bu32x2_t qhi = *reinterpret_cast<const bu32x2_t*>(sQT + o + 16);
-                    acc_dk[d] = bwd_mma(bu32x4_t{qlo.x, qlo.y, qhi.x, qhi.y}, dsf[s], acc_dk[d]);
+                    acc_dv[d] = bwd_mma(tr_fragment(ot_lane, s * 16, d * 32, TPITCH), pf[s], acc_dv[d]);
+                    acc_dk[d] = bwd_mma(tr_fragment(qt_lane, s * 16, d * 32, TPITCH), dsf[s], acc_dk[d]);
                 }
         }
     }
@@ -487,10 +459,9 @@ __device__ __forceinline__ void attention_bwd_dkv_tile(const bf16_t* __restrict_
 // Early key tiles are seen by more queries than late ones: a workgroup takes tile j and tile n-1-j.
 template <int D>
 __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(
-    const bf16_t* __restrict__ q, const bf16_t* __restrict__ qtr, const bf16_t* __restrict__ k,
-    const bf16_t* __restrict__ v, const bf16_t* __restrict__ dout, const bf16_t* __restrict__ dotr,
-    const float* __restrict__ lse, const float* __restrict__ delta, bf16_t* __restrict__ dk, bf16_t* __restrict__ dv,
-    int Hq, int Hkv, int L, int Lk, int Lqp, float scale) {
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const bf16_t* __restrict__ v,
+    const bf16_t* __restrict__ dout, const float* __restrict__ lse, const float* __restrict__ delta,
+    bf16_t* __restrict__ dk, bf16_t* __restrict__ dv, int Hq, int Hkv, int L, int Lk, float scale) {
     extern __shared__ __align__(16) unsigned char smem[];
     const int n_kt = (Lk + kBwdRows - 1) / kBwdRows;
     const int n_pairs = (n_kt + 1) / 2;
@@ -512,8 +483,8 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(
 #pragma unroll 1
     for (int half = 0; half < 2; ++half) {
         if (half && pair == kt_far) break;
-        attention_bwd_dkv_tile<D>(q, qtr, k, v, dout, dotr, lse, delta, dk, dv, Hq, Hkv, L, Lk, Lqp, scale,
-                                  half ? kt_far : pair, hkv, b, smem);
+        attention_bwd_dkv_tile<D>(q, k, v, dout, lse, delta, dk, dv, Hq, Hkv, L, Lk, scale, half ? kt_far : pair, hkv, b,
+                                  smem);
     }
 }
 
@@ -541,23 +512,20 @@ extern "C" int ats_attention_delta(const void* out, const void* dout, float* del
     return ATS_OK;
 }
 
-extern "C" int ats_attention_bwd(const void* q, const void* k, const void* v, const void* qt, const void* kt,
-                                 const void* dout, const void* dot, const float* lse, const float* delta, void* dq,
-                                 void* dk, void* dv, int B, int Hq, int Hkv, int L, int Lk, int D, float scale,
-                                 ats_stream_t stream) {
+extern "C" int ats_attention_bwd(const void* q, const void* k, const void* v, const void* dout, const float* lse,
+                                 const float* delta, void* dq, void* dk, void* dv, int B, int Hq, int Hkv, int L, int Lk,
+                                 int D, float scale, ats_stream_t stream) {
     using namespace ats;
     ATS_REQUIRE(B >= 0 && Hq > 0 && Hkv > 0 && Hq % Hkv == 0 && L >= 0 && Lk >= L && scale > 0.f, ATS_ERR_INVALID_ARG,
                 "ats_attention_bwd: B=%d Hq=%d Hkv=%d L=%d Lk=%d scale=%g", B, Hq, Hkv, L, Lk, scale);
     ATS_REQUIRE(D == 64 || D == 128, ATS_ERR_UNSUPPORTED, "ats_attention_bwd: head_dim %d (64 or 128)", D);
     if (B == 0 || L == 0) return ATS_OK;
-    ATS_REQUIRE(q && k && v && qt && kt && dout && dot && lse && delta && dq && dk && dv, ATS_ERR_INVALID_ARG,
+    ATS_REQUIRE(q && k && v && dout && lse && delta && dq && dk && dv, ATS_ERR_INVALID_ARG,
                 "ats_attention_bwd: null pointer");
-    ATS_REQUIRE(aligned16(q) && aligned16(k) && aligned16(v) && aligned16(qt) && aligned16(kt) && aligned16(dout) &&
-                    aligned16(dot) && aligned16(dq) && aligned16(dk) && aligned16(dv),
+    ATS_REQUIRE(aligned16(q) && aligned16(k) && aligned16(v) && aligned16(dout) && aligned16(dq) && aligned16(dk) &&
+                    aligned16(dv),
                 ATS_ERR_INVALID_ARG, "ats_attention_bwd: misaligned pointer");
-    const int Lp = (int)ats_attention_padded_len(Lk);
-    const int Lqp = (int)ats_attention_padded_len(L);
-    ATS_REQUIRE((int64_t)Lp * D * 2 < 0x7fffffffLL && (int64_t)L * Hq * D * 2 < 0x7fffffffLL, ATS_ERR_UNSUPPORTED,
+    ATS_REQUIRE((int64_t)Lk * D * 2 < 0x7fffffffLL && (int64_t)L * Hq * D * 2 < 0x7fffffffLL, ATS_ERR_UNSUPPORTED,
                 "ats_attention_bwd: L=%d Lk=%d (one head's K or V, and one batch entry's dO, must stay under 2 GiB)", L, Lk);
     const int n_qt = (L + kBwdRows - 1) / kBwdRows, n_kt = (Lk + kBwdRows - 1) / kBwdRows;
     const int64_t dq_blocks = (int64_t)((n_qt + 1) / 2) * Hq * B;
@@ -566,14 +534,11 @@ extern "C" int ats_attention_bwd(const void* q, const void* k, const void* v, co
     const bf16_t* q_ = static_cast<const bf16_t*>(q);
     const bf16_t* k_ = static_cast<const bf16_t*>(k);
     const bf16_t* v_ = static_cast<const bf16_t*>(v);
-    const bf16_t* qt_ = static_cast<const bf16_t*>(qt);
-    const bf16_t* kt_ = static_cast<const bf16_t*>(kt);
     const bf16_t* do_ = static_cast<const bf16_t*>(dout);
-    const bf16_t* dot_ = static_cast<const bf16_t*>(dot);
     hipStream_t s = as_stream(stream);
     if (D == 128) {
-        constexpr int smem_dq = 2 * kDqBN * (128 * 2 + 16) + 128 * (kDqBN * 2 + 8);
-        constexpr int smem_dkv = 2 * kDkvBQ * (128 * 2 + 16) + 2 * 128 * (kDkvBQ * 2 + 8) + 2 * kDkvBQ * 4 +
+        constexpr int smem_dq = 2 * kDqBN * (128 * 2 + 16) + kDqBN * (128 * 2 + 64);
+        constexpr int smem_dkv = 2 * kDkvBQ * (128 * 2 + 16) + 2 * kDkvBQ * (128 * 2 + 64) + 2 * kDkvBQ * 4 +
                                  kBwdRows * (128 * 2 + 16);
         static bool attr = false;
         if (!attr) {
@@ -583,19 +548,17 @@ extern "C" int ats_attention_bwd(const void* q, const void* k, const void* v, co
             attr = true;
         }
         hipLaunchKernelGGL((attention_bwd_dq_kernel<128>), dim3((unsigned)dq_blocks), dim3(256), smem_dq, s, q_, k_, v_,
-                           kt_, do_, lse, delta, static_cast<bf16_t*>(dq), Hq, Hkv, L, Lk, Lp, scale, B);
-        hipLaunchKernelGGL((attention_bwd_dkv_kernel<128>), dim3((unsigned)dkv_blocks), dim3(256), smem_dkv, s, q_, qt_,
-                           k_, v_, do_, dot_, lse, delta, static_cast<bf16_t*>(dk), static_cast<bf16_t*>(dv), Hq, Hkv, L,
-                           Lk, Lqp, scale);
+                           do_, lse, delta, static_cast<bf16_t*>(dq), Hq, Hkv, L, Lk, scale, B);
+        hipLaunchKernelGGL((attention_bwd_dkv_kernel<128>), dim3((unsigned)dkv_blocks), dim3(256), smem_dkv, s, q_, k_, v_,
+                           do_, lse, delta, static_cast<bf16_t*>(dk), static_cast<bf16_t*>(dv), Hq, Hkv, L, Lk, scale);
     } else {
-        constexpr int smem_dq = 2 * kDqBN * (64 * 2 + 16) + 64 * (kDqBN * 2 + 8);
-        constexpr int smem_dkv = 2 * kDkvBQ * (64 * 2 + 16) + 2 * 64 * (kDkvBQ * 2 + 8) + 2 * kDkvBQ * 4 +
+        constexpr int smem_dq = 2 * kDqBN * (64 * 2 + 16) + kDqBN * (64 * 2 + 64);
+        constexpr int smem_dkv = 2 * kDkvBQ * (64 * 2 + 16) + 2 * kDkvBQ * (64 * 2 + 64) + 2 * kDkvBQ * 4 +
                                  kBwdRows * (64 * 2 + 16);
         hipLaunchKernelGGL((attention_bwd_dq_kernel<64>), dim3((unsigned)dq_blocks), dim3(256), smem_dq, s, q_, k_, v_,
-                           kt_, do_, lse, delta, static_cast<bf16_t*>(dq), Hq, Hkv, L, Lk, Lp, scale, B);
-        hipLaunchKernelGGL((attention_bwd_dkv_kernel<64>), dim3((unsigned)dkv_blocks), dim3(256), smem_dkv, s, q_, qt_,
-                           k_, v_, do_, dot_, lse, delta, static_cast<bf16_t*>(dk), static_cast<bf16_t*>(dv), Hq, Hkv, L,
-                           Lk, Lqp, scale);
+                           do_, lse, delta, static_cast<bf16_t*>(dq), Hq, Hkv, L, Lk, scale, B);
+        hipLaunchKernelGGL((attention_bwd_dkv_kernel<64>), dim3((unsigned)dkv_blocks), dim3(256), smem_dkv, s, q_, k_, v_,
+                           do_, lse, delta, static_cast<bf16_t*>(dk), static_cast<bf16_t*>(dv), Hq, Hkv, L, Lk, scale);
     }
     ATS_CHECK_LAUNCH("ats_attention_bwd");
     return ATS_OK;

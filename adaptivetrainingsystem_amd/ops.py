@@ -597,16 +597,6 @@ def causal_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: O
     return (out, lse) if return_lse else out
 
 
-def _attention_transposed(x: torch.Tensor, B: int, Hn: int, L: int, D: int, sb: int, sl: int, sh: int) -> torch.Tensor:
-    """[B, Hn, D, padded L] copy of rows addressed as base + b*sb + l*sl + h*sh (+ d)."""
-    lib = _lib.load()
-    Lp = int(lib.ats_attention_padded_len(L))
-    xt = torch.empty(B, Hn, D, Lp, dtype=x.dtype, device=x.device)
-    check(lib.ats_attention_transpose_v(x.data_ptr(), sb, sl, sh, xt.data_ptr(), B, Hn, L, D, _stream()),
-          "ats_attention_transpose_v")
-    return xt
-
-
 def causal_attention_bwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Tensor, lse: torch.Tensor,
                          dout: torch.Tensor, scale: Optional[float] = None):
     """Gradients of causal_attention: q [B,Hq,L,D], k, v [B,Hkv,Lk,D], out, dout [B,L,Hq*D], lse [B,Hq,L].
@@ -624,14 +614,10 @@ def causal_attention_bwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out:
     delta = torch.empty(B, Hq, L, dtype=torch.float32, device=q.device)
     check(lib.ats_attention_delta(out.data_ptr(), dout.data_ptr(), delta.data_ptr(), B, Hq, L, D, _stream()),
           "ats_attention_delta")
-    qt = _attention_transposed(q, B, Hq, L, D, Hq * L * D, D, L * D)
-    kt = _attention_transposed(k, B, Hkv, Lk, D, Hkv * Lk * D, D, Lk * D)
-    dot = _attention_transposed(dout, B, Hq, L, D, L * Hq * D, Hq * D, D)
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
-    check(lib.ats_attention_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), qt.data_ptr(), kt.data_ptr(), dout.data_ptr(),
-                                dot.data_ptr(), lse.data_ptr(), delta.data_ptr(), dq.data_ptr(), dk.data_ptr(),
-                                dv.data_ptr(), B, Hq, Hkv, L, Lk, D, float(D ** -0.5 if scale is None else scale),
-                                _stream()), "ats_attention_bwd")
+    check(lib.ats_attention_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), dout.data_ptr(), lse.data_ptr(),
+                                delta.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), B, Hq, Hkv, L, Lk, D,
+                                float(D ** -0.5 if scale is None else scale), _stream()), "ats_attention_bwd")
     return dq, dk, dv
 
 

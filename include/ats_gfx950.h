@@ -271,12 +271,7 @@ int ats_grouped_gemm_nt(const void* a, const void* const* a_ptrs, int64_t lda, i
  * cache in front of the queries (model.py:700-704): query i sits at position i + Lk - L and sees keys up
  * to there.  The reference's masked path only runs that case for L = 1 (its [L, L] mask does not
  * broadcast otherwise); its flash path aligns the diagonal the same way.
- * lse (optional): [B,Hq,L] float32 log-sum-exp of the scaled scores per query.
- * ats_attention_transpose_v writes x^T [B,Hn,D,Lp] (Lp = ats_attention_padded_len(L), zero padded) of rows
- * addressed as base + b*sb + l*sl + h*sh; the backward pass uses it for its transposed operands. */
-int64_t ats_attention_padded_len(int L);
-int ats_attention_transpose_v(const void* v, int64_t sb, int64_t sl, int64_t sh, void* vt, int B, int Hkv, int L,
-                              int D, ats_stream_t stream);
+ * lse (optional): [B,Hq,L] float32 log-sum-exp of the scaled scores per query. */
 int ats_attention_fwd(const void* q, const void* k, const void* v, int64_t v_sb, int64_t v_sl, int64_t v_sh, void* out,
                       float* lse, int B, int Hq, int Hkv, int L, int Lk, int D, float scale, ats_stream_t stream);
 
@@ -286,14 +281,13 @@ int ats_attention_fwd(const void* q, const void* k, const void* v, int64_t v_sb,
  *   dV = P^T.dO, dP = dO.V^T, dS = P*(dP - delta)*scale, dQ = dS.K, dK = dS^T.Q
  * without atomics (one kernel owns query rows, one owns key rows and sums over the query heads of
  * its kv head).  ats_attention_delta: delta[B,Hq,L] = sum_d dO*O with out, dout [B,L,Hq*D].
- * ats_attention_bwd: q [B,Hq,L,D], k, v [B,Hkv,Lk,D], dout [B,L,Hq*D] contiguous; qt, dot:
- * [B,Hq,D,ats_attention_padded_len(L)] and kt: [B,Hkv,D,ats_attention_padded_len(Lk)] transposed copies
- * made with ats_attention_transpose_v; lse, delta [B,Hq,L]; dq, dk, dv shaped like q, k, v. */
+ * ats_attention_bwd: q [B,Hq,L,D], k, v [B,Hkv,Lk,D], dout [B,L,Hq*D] contiguous; lse, delta [B,Hq,L];
+ * dq, dk, dv shaped like q, k, v. */
 int ats_attention_delta(const void* out, const void* dout, float* delta, int B, int Hq, int L, int D,
                         ats_stream_t stream);
-int ats_attention_bwd(const void* q, const void* k, const void* v, const void* qt, const void* kt, const void* dout,
-                      const void* dot, const float* lse, const float* delta, void* dq, void* dk, void* dv, int B,
-                      int Hq, int Hkv, int L, int Lk, int D, float scale, ats_stream_t stream);
+int ats_attention_bwd(const void* q, const void* k, const void* v, const void* dout, const float* lse,
+                      const float* delta, void* dq, void* dk, void* dv, int B, int Hq, int Hkv, int L, int Lk, int D,
+                      float scale, ats_stream_t stream);
 
 /* ---- Training-step ops beside the sparse layer --------------------------------
  * Fused cross-entropy + accuracy.  Replaces fused_cross_entropy_accuracy_launcher
