@@ -143,9 +143,10 @@ def route_topk(logits: torch.Tensor, k: int, temperature: float = 1.0, variant: 
     ws_bytes = 0
     lib = _lib.load()
     if with_stats:
-        hist = torch.zeros(E, dtype=torch.int32, device=dev)
-        colsum = torch.zeros(E, dtype=torch.float32, device=dev)
-        aux = torch.zeros(1, dtype=torch.float32, device=dev)
+        zeros = torch.zeros(2 * E + 1, dtype=torch.int32, device=dev)      # one fill launch for the three outputs
+        hist = zeros[:E]
+        colsum = zeros[E:2 * E].view(torch.float32)
+        aux = zeros[2 * E:].view(torch.float32)
         ws_bytes = lib.ats_route_topk_workspace(T, E)
         ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
     check(lib.ats_route_topk(logits.data_ptr(), T, E, int(k), float(temperature), int(variant), idx.data_ptr(),
