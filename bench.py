@@ -35,7 +35,8 @@ PEAK_MFMA_BF16_TFLOPS = 2500.0   # MI355X dense bf16
 PEAK_HBM_GBS = 8000.0            # MI355X HBM3E
 # HBM-side bytes per launch of the gate/up GEMM, from separate hardware-counter runs of this script
 # (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0, factors from a 1 GiB copy; summary under profiles/).
-GATEUP_HBM_BYTES_PER_LAUNCH = {"c4_prefill": 11.56e9}
+GATEUP_HBM_BYTES_PER_LAUNCH = {"c4_prefill": 11.56e9, "c3_decode": 1.8871e9}
+ATTENTION_DECODE_HBM_BYTES_PER_LAUNCH = 538.0e6
 
 
 def log(*a):
@@ -119,7 +120,8 @@ def run_moe(args):
         gu_bytes = active * 2.0 * I * H * es + kept * (H + I) * es
         gbs = gu_bytes / (gu_ms * 1e-3) / 1e9
         roofline = {"kernel": "grouped gate/up GEMM + SwiGLU (weight streaming)", "bound": "hbm", "achieved": gbs,
-                    "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS, "traffic": None}
+                    "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS,
+                    "traffic": GATEUP_HBM_BYTES_PER_LAUNCH.get(name)}
     else:
         roofline = {"kernel": "grouped gate/up GEMM + SwiGLU", "bound": "mfma", "achieved": achieved,
                     "peak": PEAK_MFMA_BF16_TFLOPS, "unit": "TFLOP/s", "frac": achieved / PEAK_MFMA_BF16_TFLOPS,
@@ -496,7 +498,8 @@ def run_attention_decode(args):
         "config": {"workload": f"attention_decode: {B} sequences x 1 new token against {Lk} cached keys, {Hq} query / "
                                f"{Hkv} kv heads, head_dim {D}"},
         "roofline": {"kernel": "attention_fwd_kernel, packed rows", "bound": "hbm", "achieved": achieved,
-                     "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": achieved / PEAK_HBM_GBS, "traffic": None},
+                     "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": achieved / PEAK_HBM_GBS,
+                     "traffic": ATTENTION_DECODE_HBM_BYTES_PER_LAUNCH},
         "stages_ms": {s_: round(v_["mean_ms"], 4) for s_, v_ in st.items()},
     }
     if not args.no_cpu_baseline:
@@ -627,9 +630,9 @@ def run_norm_rope(args):
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "c2_norm_rope: RMSNorm x[8192,2048] + RoPE q[4,16,2048,128] k[4,4,2048,128]"},
         "roofline": {"kernel": "rope", "bound": "hbm", "achieved": rope_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                     "frac": rope_gbs / PEAK_HBM_GBS, "traffic": None},
+                     "frac": rope_gbs / PEAK_HBM_GBS, "traffic": 85.28e6},     # counter runs, see profiles/
         "rmsnorm_roofline": {"bound": "hbm", "achieved": rms_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                             "frac": rms_gbs / PEAK_HBM_GBS},
+                             "frac": rms_gbs / PEAK_HBM_GBS, "traffic": 67.22e6},
         "rmsnorm_bwd_roofline": {"bound": "hbm", "achieved": rmsb_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s",
                                  "frac": rmsb_gbs / PEAK_HBM_GBS},
         "rope_bwd_roofline": {"bound": "hbm", "achieved": ropeb_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s",
