@@ -56,21 +56,22 @@ class RoPEFunction(Function):
 
 
 class AttentionFunction(Function):
-    """Causal grouped-query attention: q [B,Hq,L,D], k, v [B,Hkv,Lk,D] -> [B, L, Hq*D]."""
+    """Causal grouped-query attention: q [B,Hq,L,D], k, v [B,Hkv,Lk,D] -> [B, L, Hq*D]; key_bias
+    [B, Lk] float32 or None (a constant: it gets no gradient)."""
 
     @staticmethod
-    def forward(ctx, q, k, v, scale):
+    def forward(ctx, q, k, v, scale, key_bias=None):
         q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
-        out, lse = ops.causal_attention(q, k, v, scale, return_lse=True)
-        ctx.save_for_backward(q, k, v, out, lse)
+        out, lse = ops.causal_attention(q, k, v, scale, return_lse=True, key_bias=key_bias)
+        ctx.save_for_backward(q, k, v, out, lse, key_bias)
         ctx.scale = scale
         return out
 
     @staticmethod
     def backward(ctx, dout):
-        q, k, v, out, lse = ctx.saved_tensors
-        dq, dk, dv = ops.causal_attention_bwd(q, k, v, out, lse, dout, ctx.scale)
-        return dq, dk, dv, None
+        q, k, v, out, lse, key_bias = ctx.saved_tensors
+        dq, dk, dv = ops.causal_attention_bwd(q, k, v, out, lse, dout, ctx.scale, key_bias=key_bias)
+        return dq, dk, dv, None, None
 
 
 class LinearFunction(Function):

@@ -50,11 +50,12 @@ __device__ __forceinline__ af32x16_t att_mma(const au32x4_t& a, const au32x4_t& 
 // (batch, query head), or -- `pack` -- the queries of all query heads of one (batch, kv head), position
 // major: row r is position r / rep of head hkv * rep + r % rep.  Packing fills the tile when there are few
 // positions (decoding against a cache: one position, rep rows instead of one).
-template <int D>
+template <int D, bool BIAS>
 __device__ __forceinline__ void attention_q_tile(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
                                                  const bf16_t* __restrict__ v, int64_t v_sb, int v_sl, int64_t v_sh,
-                                                 bf16_t* __restrict__ out, float* __restrict__ lse, int Hq, int Hkv,
-                                                 int L, int Lk, float scale_log2, int qt, int head, int b, bool pack,
+                                                 const float* __restrict__ key_bias, bf16_t* __restrict__ out,
+                                                 float* __restrict__ lse, int Hq, int Hkv, int L, int Lk,
+                                                 float scale_log2, int qt, int head, int b, bool pack,
                                                  unsigned char* smem) {
     constexpr int KS = D / 16;              // k-steps of the score product
     constexpr int DB = D / 32;              // 32-row blocks of the output (transposed)
@@ -67,6 +68,13 @@ __device__ __forceinline__ void attention_q_tile(const bf16_t* __restrict__ q, c
     // smem: [2 stages][K tile | V tile]
 #define ATT_SK(stage_) (smem + (stage_) * (KTILE + VTILE))
 #define ATT_SV(stage_) (smem + (stage_) * (KTILE + VTILE) + KTILE)
+    // optional additive bias per key (a padding mask), in log2 units: [2 stages][64] floats behind the tiles
+    float* const s_bias = reinterpret_cast<float*>(smem + 2 * (KTILE + VTILE));
+    const float* bias_row = BIAS ? key_bias + (int64_t)b * Lk : nullptr;
+    constexpr bool has_bias = BIAS;
+    // with a bias the scores are brought to log2 units before the maximum is taken (sc = 1 afterwards)
+    const float sc = has_bias ? 1.0f : scale_log2;
+    float r_bias = 0.f;
 
     const int rep = Hq / Hkv;
     const int rp = pack ? rep : 1;                  // rows per position
@@ -147,6 +155,7 @@ __device__ __forceinline__ void attention_q_tile(const bf16_t* __restrict__ q, c
             const int r = idx / (D / 8), c = idx % (D / 8);
             *reinterpret_cast<au32x4_t*>(ATT_SV(0) + r * VPITCH + c * 16) = rv[i];
         }
+        if (has_bias && tid < kAttBN) s_bias[tid] = tid < Lk ? bias_row[tid] * 1.4426950408889634f : 0.f;
         __syncthreads();
     }
 
@@ -164,6 +173,7 @@ __device__ __forceinline__ void attention_q_tile(const bf16_t* __restrict__ q, c
         // waves of a CU leave the barrier together, and 8 loads per wave issued back to back queue up behind
         // the CU's one address unit while no wave can reach its MFMAs.
         const int n1 = n0 + kAttBN;
+        if (has_bias && has_next && tid < kAttBN) r_bias = n1 + tid < Lk ? bias_row[n1 + tid] * 1.4426950408889634f : 0.f;
 #define ATT_LOAD_ONE(i_)                                                                               \
     {                                                                                                  \
         if ((i_) < KVEC)                                                                               \
@@ -223,6 +233,20 @@ __device__ __forceinline__ void attention_q_tile(const bf16_t* __restrict__ q, c
             for (int f = 0; f < kRing; ++f) ATT_VFRAG(f, ring[f]);
             __builtin_amdgcn_sched_barrier(0);
 
+            if (has_bias) {   // scores to log2 units plus the key's bias; accumulator value x of block kb is key
+                              // kb*32 + (x/4)*8 + g*4 + x%4 of the tile
+                const float* bt = s_bias + (t & 1) * kAttBN + g * 4;
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) {
+                        const float4 b4 = *reinterpret_cast<const float4*>(bt + kb * 32 + r * 8);
+                        acc_s[kb][r * 4 + 0] = __builtin_fmaf(acc_s[kb][r * 4 + 0], scale_log2, b4.x);
+                        acc_s[kb][r * 4 + 1] = __builtin_fmaf(acc_s[kb][r * 4 + 1], scale_log2, b4.y);
+                        acc_s[kb][r * 4 + 2] = __builtin_fmaf(acc_s[kb][r * 4 + 2], scale_log2, b4.z);
+                        acc_s[kb][r * 4 + 3] = __builtin_fmaf(acc_s[kb][r * 4 + 3], scale_log2, b4.w);
+                    }
+            }
             if (n0 + kAttBN - 1 > q_wave_first) {   // diagonal tile: causal mask
 #pragma unroll
                 for (int kb = 0; kb < 2; ++kb)
@@ -238,7 +262,7 @@ __device__ __forceinline__ void attention_q_tile(const bf16_t* __restrict__ q, c
 #pragma unroll
                 for (int v = 0; v < 16; ++v) mx = fmaxf(mx, acc_s[kb][v]);
             mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-            const float m_new = fmaxf(m_run, mx * scale_log2);   // scale > 0 keeps the order
+            const float m_new = fmaxf(m_run, mx * sc);   // a positive factor keeps the order
             const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);   // 0 on the first tile
             float psum = 0.f;
             // p = exp2(s * c - m * c): one fused multiply-add per element, c = scale * log2(e)
@@ -246,7 +270,7 @@ __device__ __forceinline__ void attention_q_tile(const bf16_t* __restrict__ q, c
             for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
                 for (int v = 0; v < 16; ++v) {
-                    const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(acc_s[kb][v], scale_log2, -m_new));
+                    const float p = __builtin_amdgcn_exp2f(__builtin_fmaf(acc_s[kb][v], sc, -m_new));
                     acc_s[kb][v] = p;
                     psum += p;
                 }
@@ -279,6 +303,7 @@ __device__ __forceinline__ void attention_q_tile(const bf16_t* __restrict__ q, c
         }
 
         if (has_next) {   // stage (t+1)&1 was last read in iteration t-1, before its closing barrier
+            if (has_bias && tid < kAttBN) s_bias[((t + 1) & 1) * kAttBN + tid] = r_bias;
             unsigned char* dk = ATT_SK((t + 1) & 1);
             unsigned char* dv = ATT_SV((t + 1) & 1);
 #pragma unroll
@@ -323,11 +348,12 @@ __device__ __forceinline__ void attention_q_tile(const bf16_t* __restrict__ q, c
 // Consecutive ids go to different XCDs; the blocks of one (batch, kv head) are kept on one XCD so that
 // its K and V stay in that XCD's L2.  Two waves per SIMD (register budget 256): one wave's softmax runs
 // in the shadow of the other's MFMAs.
-template <int D>
+template <int D, bool BIAS>
 __global__ __launch_bounds__(kAttThreads, 512 / kAttThreads) void attention_fwd_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
                                                             const bf16_t* __restrict__ v, int64_t v_sb, int v_sl, int64_t v_sh,
-                                                            bf16_t* __restrict__ out, float* __restrict__ lse, int Hq, int Hkv,
-                                                            int L, int Lk, float scale_log2, int B, int pack) {
+                                                            const float* __restrict__ key_bias, bf16_t* __restrict__ out,
+                                                            float* __restrict__ lse, int Hq, int Hkv, int L, int Lk,
+                                                            float scale_log2, int B, int pack) {
     extern __shared__ __align__(16) unsigned char smem[];
     const int heads_per_group = pack ? 1 : Hq / Hkv;     // packed: the group's heads share the rows of a tile
     const int n_qt = (L * (pack ? Hq / Hkv : 1) + kAttBM - 1) / kAttBM;
@@ -350,16 +376,16 @@ __global__ __launch_bounds__(kAttThreads, 512 / kAttThreads) void attention_fwd_
 #pragma unroll 1
     for (int half = 0; half < 2; ++half) {
         if (half && pair == qt_long) break;   // an odd tile count leaves the middle tile on its own
-        attention_q_tile<D>(q, k, v, v_sb, v_sl, v_sh, out, lse, Hq, Hkv, L, Lk, scale_log2, half ? pair : qt_long,
-                            head, b, pack != 0, smem);
+        attention_q_tile<D, BIAS>(q, k, v, v_sb, v_sl, v_sh, key_bias, out, lse, Hq, Hkv, L, Lk, scale_log2,
+                            half ? pair : qt_long, head, b, pack != 0, smem);
     }
 }
 
 }  // namespace ats
 
 extern "C" int ats_attention_fwd(const void* q, const void* k, const void* v, int64_t v_sb, int64_t v_sl, int64_t v_sh,
-                                 void* out, float* lse, int B, int Hq, int Hkv, int L, int Lk, int D, float scale,
-                                 ats_stream_t stream) {
+                                 const float* key_bias, void* out, float* lse, int B, int Hq, int Hkv, int L, int Lk,
+                                 int D, float scale, ats_stream_t stream) {
     using namespace ats;
     ATS_REQUIRE(B >= 0 && Hq > 0 && Hkv > 0 && Hq % Hkv == 0 && L >= 0 && Lk >= L && scale > 0.f, ATS_ERR_INVALID_ARG,
                 "ats_attention_fwd: B=%d Hq=%d Hkv=%d L=%d Lk=%d scale=%g", B, Hq, Hkv, L, Lk, scale);
@@ -379,24 +405,29 @@ extern "C" int ats_attention_fwd(const void* q, const void* k, const void* v, in
     ATS_REQUIRE(n_blocks <= 0x7fffffff, ATS_ERR_UNSUPPORTED, "ats_attention_fwd: %lld workgroups", (long long)n_blocks);
     const dim3 grid((unsigned)n_blocks);
     const float scale_log2 = scale * 1.4426950408889634f;
-    if (D == 128) {
-        constexpr int smem = 2 * kAttBN * ((128 * 2 + 16) + (128 * 2 + 64));
-        static bool attr = false;
-        if (!attr) {
-            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(attention_fwd_kernel<128>),
+    static bool reserved_lds[4] = {false, false, false, false};      // per kernel instance
+    auto launch = [&](auto kernel, int smem, bool& reserved) -> int {
+        if (smem > 64 * 1024 && !reserved) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
                                                hipFuncAttributeMaxDynamicSharedMemorySize, smem);
             ATS_REQUIRE(e == hipSuccess, ATS_ERR_LAUNCH, "ats_attention_fwd: cannot reserve %d bytes of LDS", smem);
-            attr = true;
+            reserved = true;
         }
-        hipLaunchKernelGGL((attention_fwd_kernel<128>), grid, dim3(kAttThreads), smem, as_stream(stream),
-                           static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k), static_cast<const bf16_t*>(v),
-                           v_sb, (int)v_sl, v_sh, static_cast<bf16_t*>(out), lse, Hq, Hkv, L, Lk, scale_log2, B, pack);
-    } else {
-        constexpr int smem = 2 * kAttBN * ((64 * 2 + 16) + (64 * 2 + 64));
-        hipLaunchKernelGGL((attention_fwd_kernel<64>), grid, dim3(kAttThreads), smem, as_stream(stream),
-                           static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k), static_cast<const bf16_t*>(v),
-                           v_sb, (int)v_sl, v_sh, static_cast<bf16_t*>(out), lse, Hq, Hkv, L, Lk, scale_log2, B, pack);
-    }
+        hipLaunchKernelGGL(kernel, grid, dim3(kAttThreads), smem, as_stream(stream), static_cast<const bf16_t*>(q),
+                           static_cast<const bf16_t*>(k), static_cast<const bf16_t*>(v), v_sb, (int)v_sl, v_sh, key_bias,
+                           static_cast<bf16_t*>(out), lse, Hq, Hkv, L, Lk, scale_log2, B, pack);
+        return ATS_OK;
+    };
+    // K tile, V tile (two stages each) and, with a bias, two stages of one float per key
+    const int smem = 2 * kAttBN * ((D * 2 + 16) + (D * 2 + 64)) + (key_bias ? 2 * kAttBN * 4 : 0);
+    int rc;
+    if (D == 128)
+        rc = key_bias ? launch(attention_fwd_kernel<128, true>, smem, reserved_lds[0])
+                      : launch(attention_fwd_kernel<128, false>, smem, reserved_lds[1]);
+    else
+        rc = key_bias ? launch(attention_fwd_kernel<64, true>, smem, reserved_lds[2])
+                      : launch(attention_fwd_kernel<64, false>, smem, reserved_lds[3]);
+    if (rc != ATS_OK) return rc;
     ATS_CHECK_LAUNCH("ats_attention_fwd");
     return ATS_OK;
 }

@@ -91,12 +91,13 @@ __global__ __launch_bounds__(256) void attention_delta_kernel(const bf16_t* __re
 
 // ------------------------------------------------------------------------------------------ dQ
 // One 128-row query tile of one (batch, query head): lanes own queries, keys come in tiles of 64.
-template <int D>
+template <int D, bool BIAS>
 __device__ __forceinline__ void attention_bwd_dq_tile(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
                                                       const bf16_t* __restrict__ v, const bf16_t* __restrict__ dout,
                                                       const float* __restrict__ lse, const float* __restrict__ delta,
-                                                      bf16_t* __restrict__ dq, int Hq, int Hkv, int L, int Lk,
-                                                      float scale, int qt, int hq, int b, unsigned char* smem) {
+                                                      const float* __restrict__ key_bias, bf16_t* __restrict__ dq, int Hq,
+                                                      int Hkv, int L, int Lk, float scale, int qt, int hq, int b,
+                                                      unsigned char* smem) {
     constexpr int KS = D / 16;
     constexpr int DB = D / 32;
     constexpr int RPITCH = D * 2 + 16;        // bytes per K / V row in LDS
@@ -106,6 +107,8 @@ __device__ __forceinline__ void attention_bwd_dq_tile(const bf16_t* __restrict__
     unsigned char* const sK = smem;
     unsigned char* const sV = smem + RTILE;
     unsigned char* const sT = smem + 2 * RTILE;
+    float* const sBias = reinterpret_cast<float*>(smem + 2 * RTILE + kDqBN * TPITCH);   // [64], log2 units
+    const float* bias_row = BIAS ? key_bias + (int64_t)b * Lk : nullptr;
 
     const int hkv = hq / (Hq / Hkv);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -169,6 +172,7 @@ __device__ __forceinline__ void attention_bwd_dq_tile(const bf16_t* __restrict__
                 *reinterpret_cast<bu32x4_t*>(sV + r * RPITCH + c * 16) = rv[i];
                 *reinterpret_cast<bu32x4_t*>(sT + r * TPITCH + c * 16) = rk[i];
             }
+            if (BIAS && tid < kDqBN) sBias[tid] = n0 + tid < Lk ? bias_row[n0 + tid] * kLog2e : 0.f;
         }
         __syncthreads();
         if (n0 > q_wave_last) continue;   // every key of the tile is in this wave's future
@@ -196,7 +200,9 @@ __device__ __forceinline__ void attention_bwd_dq_tile(const bf16_t* __restrict__
         for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
             for (int x = 0; x < 16; ++x) {
-                float p = __builtin_amdgcn_exp2f(__builtin_fmaf(acc_s[kb][x], scale_log2, -lse2));
+                // the key of accumulator value x is kb*32 + (x/4)*8 + g*4 + x%4 of the tile
+                const float kbias = BIAS ? sBias[kb * 32 + (x >> 2) * 8 + g * 4 + (x & 3)] : 0.f;
+                float p = __builtin_amdgcn_exp2f(__builtin_fmaf(acc_s[kb][x], scale_log2, kbias - lse2));
                 if (diagonal) {
                     const int key = n0 + kb * 32 + (x >> 2) * 8 + g * 4 + (x & 3);
                     if (key > q_pos) p = 0.f;
@@ -237,11 +243,11 @@ __device__ __forceinline__ void attention_bwd_dq_tile(const bf16_t* __restrict__
 
 // A workgroup takes a long query tile and its mirror-image short one (equal work per workgroup: the
 // hardware hands workgroups out strictly in turn), and the workgroups of one (batch, kv head) share an XCD.
-template <int D>
+template <int D, bool BIAS>
 __global__ __launch_bounds__(256, 2) void attention_bwd_dq_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const bf16_t* __restrict__ v,
     const bf16_t* __restrict__ dout, const float* __restrict__ lse, const float* __restrict__ delta,
-    bf16_t* __restrict__ dq, int Hq, int Hkv, int L, int Lk, float scale, int B) {
+    const float* __restrict__ key_bias, bf16_t* __restrict__ dq, int Hq, int Hkv, int L, int Lk, float scale, int B) {
     extern __shared__ __align__(16) unsigned char smem[];
     const int n_qt = (L + kBwdRows - 1) / kBwdRows;
     const int n_pairs = (n_qt + 1) / 2;
@@ -263,8 +269,8 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dq_kernel(
 #pragma unroll 1
     for (int half = 0; half < 2; ++half) {
         if (half && pair == qt_long) break;
-        attention_bwd_dq_tile<D>(q, k, v, dout, lse, delta, dq, Hq, Hkv, L, Lk, scale, half ? pair : qt_long, hq, b,
-                                 smem);
+        attention_bwd_dq_tile<D, BIAS>(q, k, v, dout, lse, delta, key_bias, dq, Hq, Hkv, L, Lk, scale, half ? pair : qt_long,
+                                 hq, b, smem);
     }
 }
 
@@ -275,9 +281,9 @@ template <int D>
 __device__ __forceinline__ void attention_bwd_dkv_tile(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
                                                        const bf16_t* __restrict__ v, const bf16_t* __restrict__ dout,
                                                        const float* __restrict__ lse, const float* __restrict__ delta,
-                                                       bf16_t* __restrict__ dk, bf16_t* __restrict__ dv, int Hq, int Hkv,
-                                                       int L, int Lk, float scale, int kt_idx, int hkv, int b,
-                                                       unsigned char* smem) {
+                                                       const float* __restrict__ key_bias, bf16_t* __restrict__ dk,
+                                                       bf16_t* __restrict__ dv, int Hq, int Hkv, int L, int Lk, float scale,
+                                                       int kt_idx, int hkv, int b, unsigned char* smem) {
     constexpr int KS = D / 16;
     constexpr int DB = D / 32;
     constexpr int RPITCH = D * 2 + 16;        // bytes per Q / dO row in LDS
@@ -303,6 +309,7 @@ __device__ __forceinline__ void attention_bwd_dkv_tile(const bf16_t* __restrict_
     const int off = Lk - L;
     const float scale_log2 = scale * kLog2e;
 
+    const float kbias = key_bias ? key_bias[(int64_t)b * Lk + key_clamped] * kLog2e : 0.f;   // this lane's key
     const bf16_t* kp = k + ((int64_t)(b * Hkv + hkv) * Lk + key_clamped) * D;
     bu32x4_t kf[KS];
 #pragma unroll
@@ -409,7 +416,7 @@ __device__ __forceinline__ void attention_bwd_dkv_tile(const bf16_t* __restrict_
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     const int x = r * 4 + j;
-                    float pv = __builtin_amdgcn_exp2f(__builtin_fmaf(acc_s[x], scale_log2, -lv[j]));
+                    float pv = __builtin_amdgcn_exp2f(__builtin_fmaf(acc_s[x], scale_log2, kbias - lv[j]));
                     if (diagonal) {
                         const int qi = q0 + r * 8 + g * 4 + j;
                         if (key_row > qi + off) pv = 0.f;
@@ -461,7 +468,8 @@ template <int D>
 __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const bf16_t* __restrict__ v,
     const bf16_t* __restrict__ dout, const float* __restrict__ lse, const float* __restrict__ delta,
-    bf16_t* __restrict__ dk, bf16_t* __restrict__ dv, int Hq, int Hkv, int L, int Lk, float scale) {
+    const float* __restrict__ key_bias, bf16_t* __restrict__ dk, bf16_t* __restrict__ dv, int Hq, int Hkv, int L, int Lk,
+    float scale) {
     extern __shared__ __align__(16) unsigned char smem[];
     const int n_kt = (Lk + kBwdRows - 1) / kBwdRows;
     const int n_pairs = (n_kt + 1) / 2;
@@ -483,8 +491,8 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(
 #pragma unroll 1
     for (int half = 0; half < 2; ++half) {
         if (half && pair == kt_far) break;
-        attention_bwd_dkv_tile<D>(q, k, v, dout, lse, delta, dk, dv, Hq, Hkv, L, Lk, scale, half ? kt_far : pair, hkv, b,
-                                  smem);
+        attention_bwd_dkv_tile<D>(q, k, v, dout, lse, delta, key_bias, dk, dv, Hq, Hkv, L, Lk, scale,
+                                  half ? kt_far : pair, hkv, b, smem);
     }
 }
 
@@ -513,8 +521,8 @@ extern "C" int ats_attention_delta(const void* out, const void* dout, float* del
 }
 
 extern "C" int ats_attention_bwd(const void* q, const void* k, const void* v, const void* dout, const float* lse,
-                                 const float* delta, void* dq, void* dk, void* dv, int B, int Hq, int Hkv, int L, int Lk,
-                                 int D, float scale, ats_stream_t stream) {
+                                 const float* delta, const float* key_bias, void* dq, void* dk, void* dv, int B, int Hq,
+                                 int Hkv, int L, int Lk, int D, float scale, ats_stream_t stream) {
     using namespace ats;
     ATS_REQUIRE(B >= 0 && Hq > 0 && Hkv > 0 && Hq % Hkv == 0 && L >= 0 && Lk >= L && scale > 0.f, ATS_ERR_INVALID_ARG,
                 "ats_attention_bwd: B=%d Hq=%d Hkv=%d L=%d Lk=%d scale=%g", B, Hq, Hkv, L, Lk, scale);
@@ -537,7 +545,7 @@ extern "C" int ats_attention_bwd(const void* q, const void* k, const void* v, co
     const bf16_t* do_ = static_cast<const bf16_t*>(dout);
     hipStream_t s = as_stream(stream);
     if (D == 128) {
-        constexpr int smem_dq = 2 * kDqBN * (128 * 2 + 16) + kDqBN * (128 * 2 + 64);
+        constexpr int smem_dq = 2 * kDqBN * (128 * 2 + 16) + kDqBN * (128 * 2 + 64) + kDqBN * 4;
         constexpr int smem_dkv = 2 * kDkvBQ * (128 * 2 + 16) + 2 * kDkvBQ * (128 * 2 + 64) + 2 * kDkvBQ * 4 +
                                  kBwdRows * (128 * 2 + 16);
         static bool attr = false;
@@ -547,18 +555,26 @@ extern "C" int ats_attention_bwd(const void* q, const void* k, const void* v, co
             ATS_REQUIRE(e == hipSuccess, ATS_ERR_LAUNCH, "ats_attention_bwd: cannot reserve %d bytes of LDS", smem_dkv);
             attr = true;
         }
-        hipLaunchKernelGGL((attention_bwd_dq_kernel<128>), dim3((unsigned)dq_blocks), dim3(256), smem_dq, s, q_, k_, v_,
-                           do_, lse, delta, static_cast<bf16_t*>(dq), Hq, Hkv, L, Lk, scale, B);
+        if (key_bias)
+            hipLaunchKernelGGL((attention_bwd_dq_kernel<128, true>), dim3((unsigned)dq_blocks), dim3(256), smem_dq, s, q_,
+                               k_, v_, do_, lse, delta, key_bias, static_cast<bf16_t*>(dq), Hq, Hkv, L, Lk, scale, B);
+        else
+            hipLaunchKernelGGL((attention_bwd_dq_kernel<128, false>), dim3((unsigned)dq_blocks), dim3(256), smem_dq, s, q_,
+                               k_, v_, do_, lse, delta, key_bias, static_cast<bf16_t*>(dq), Hq, Hkv, L, Lk, scale, B);
         hipLaunchKernelGGL((attention_bwd_dkv_kernel<128>), dim3((unsigned)dkv_blocks), dim3(256), smem_dkv, s, q_, k_, v_,
-                           do_, lse, delta, static_cast<bf16_t*>(dk), static_cast<bf16_t*>(dv), Hq, Hkv, L, Lk, scale);
+                           do_, lse, delta, key_bias, static_cast<bf16_t*>(dk), static_cast<bf16_t*>(dv), Hq, Hkv, L, Lk, scale);
     } else {
-        constexpr int smem_dq = 2 * kDqBN * (64 * 2 + 16) + kDqBN * (64 * 2 + 64);
+        constexpr int smem_dq = 2 * kDqBN * (64 * 2 + 16) + kDqBN * (64 * 2 + 64) + kDqBN * 4;
         constexpr int smem_dkv = 2 * kDkvBQ * (64 * 2 + 16) + 2 * kDkvBQ * (64 * 2 + 64) + 2 * kDkvBQ * 4 +
                                  kBwdRows * (64 * 2 + 16);
-        hipLaunchKernelGGL((attention_bwd_dq_kernel<64>), dim3((unsigned)dq_blocks), dim3(256), smem_dq, s, q_, k_, v_,
-                           do_, lse, delta, static_cast<bf16_t*>(dq), Hq, Hkv, L, Lk, scale, B);
+        if (key_bias)
+            hipLaunchKernelGGL((attention_bwd_dq_kernel<64, true>), dim3((unsigned)dq_blocks), dim3(256), smem_dq, s, q_,
+                               k_, v_, do_, lse, delta, key_bias, static_cast<bf16_t*>(dq), Hq, Hkv, L, Lk, scale, B);
+        else
+            hipLaunchKernelGGL((attention_bwd_dq_kernel<64, false>), dim3((unsigned)dq_blocks), dim3(256), smem_dq, s, q_,
+                               k_, v_, do_, lse, delta, key_bias, static_cast<bf16_t*>(dq), Hq, Hkv, L, Lk, scale, B);
         hipLaunchKernelGGL((attention_bwd_dkv_kernel<64>), dim3((unsigned)dkv_blocks), dim3(256), smem_dkv, s, q_, k_, v_,
-                           do_, lse, delta, static_cast<bf16_t*>(dk), static_cast<bf16_t*>(dv), Hq, Hkv, L, Lk, scale);
+                           do_, lse, delta, key_bias, static_cast<bf16_t*>(dk), static_cast<bf16_t*>(dv), Hq, Hkv, L, Lk, scale);
     }
     ATS_CHECK_LAUNCH("ats_attention_bwd");
     return ATS_OK;

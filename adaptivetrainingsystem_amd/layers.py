@@ -185,8 +185,6 @@ class GroupedQueryAttention(nn.Module):
 
     def forward(self, x: torch.Tensor, attention_mask: Optional[torch.Tensor] = None, past_key_value=None,
                 use_cache: bool = False):
-        if attention_mask is not None:
-            raise AtsError("GroupedQueryAttention: padding masks are not built in the gfx950 path")
         if x.dim() != 3 or x.shape[-1] != self.hidden_size:
             raise AtsError(f"GroupedQueryAttention: expected [batch, seq, {self.hidden_size}], got {tuple(x.shape)}")
         if x.dtype != torch.bfloat16:
@@ -212,7 +210,18 @@ class GroupedQueryAttention(nn.Module):
                 raise AtsError(f"GroupedQueryAttention: cache shapes {tuple(k_cache.shape)} / {tuple(v_cache.shape)}")
             k = torch.cat([k_cache.to(k.dtype), k], dim=2)
             v = torch.cat([v_cache.to(v.dtype), v], dim=2)
-        a = ag.AttentionFunction.apply(q, k, v, self.scale) if grad else ops.causal_attention(q, k, v, self.scale)
+        key_bias = None
+        if attention_mask is not None:
+            # [batch, keys] with 1 = real token, 0 = padding: (1 - mask) * -1e4 on that key's scores for
+            # every query and head (model.py:819-824)
+            if attention_mask.dim() != 2 or attention_mask.shape != (B, k.shape[2]):
+                raise AtsError(f"GroupedQueryAttention: attention_mask must be [batch, keys] = [{B}, {k.shape[2]}], got "
+                               f"{tuple(attention_mask.shape)} (per-query [batch, 1, seq, seq] masks are not built)")
+            key_bias = (1.0 - attention_mask.to(device=x.device, dtype=torch.float32)) * -1e4
+        if grad:
+            a = ag.AttentionFunction.apply(q, k, v, self.scale, key_bias)
+        else:
+            a = ops.causal_attention(q, k, v, self.scale, key_bias=key_bias)
         out = lin(a.view(B * L, nh * D), self.o_proj.weight).view(B, L, H)    # a: [B, L, nh*D]
         self._calls += 1
         if use_cache:

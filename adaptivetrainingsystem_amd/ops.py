@@ -573,11 +573,21 @@ def grouped_gemm_nt(b_ptrs: torch.Tensor, ldb: int, b_rows: int, row_start: torc
 
 
 # --------------------------------------------------------------------------- attention
+def _key_bias(key_bias, B: int, Lk: int, q: torch.Tensor, who: str):
+    if key_bias is None:
+        return None
+    if key_bias.shape != (B, Lk) or key_bias.dtype != torch.float32 or key_bias.device != q.device:
+        raise AtsError(f"{who}: key_bias must be float32 [batch, keys] = [{B}, {Lk}] on the inputs' device")
+    return key_bias.contiguous()
+
+
 def causal_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: Optional[float] = None,
-                     return_lse: bool = False):
+                     return_lse: bool = False, key_bias: Optional[torch.Tensor] = None):
     """Causal grouped-query attention.  q [B,Hq,L,D], k [B,Hkv,Lk,D] (made contiguous), v [B,Hkv,Lk,D] in any
     batch/head/position strides (e.g. a view of a fused projection output); bf16, D 64 or 128, Lk >= L.
     With Lk > L the leading Lk - L keys are a cache: query i sits at position i + Lk - L.
+    key_bias [B, Lk] float32 (optional) is added to the scaled scores of a key for every query and head;
+    (1 - attention_mask) * -1e4 is the reference's padding mask (MS/core/model.py:819-824).
     Returns out [B, L, Hq*D] (and lse [B,Hq,L] float32 if asked)."""
     _need_gpu(q, k, v)
     if q.dim() != 4 or k.dim() != 4 or v.dim() != 4 or q.dtype != torch.bfloat16 or k.dtype != q.dtype or v.dtype != q.dtype:
@@ -587,21 +597,22 @@ def causal_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: O
     if k.shape != (B, Hkv, Lk, D) or v.shape != (B, Hkv, Lk, D) or Hq % Hkv != 0 or Lk < L:
         raise AtsError(f"causal_attention: shapes q {tuple(q.shape)} k {tuple(k.shape)} v {tuple(v.shape)}")
     q, k = q.contiguous(), k.contiguous()
+    key_bias = _key_bias(key_bias, B, Lk, q, "causal_attention")
     if v.stride(3) != 1 or any(st % 8 for st in v.stride()[:3]) or v.stride(2) < D or v.data_ptr() % 16:
         v = v.contiguous()
     lib = _lib.load()
     out = torch.empty(B, L, Hq * D, dtype=q.dtype, device=q.device)
     lse = torch.empty(B, Hq, L, dtype=torch.float32, device=q.device) if return_lse else None
     check(lib.ats_attention_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), v.stride(0), v.stride(2), v.stride(1),
-                                out.data_ptr(), _ptr(lse), B, Hq, Hkv, L, Lk, D,
+                                _ptr(key_bias), out.data_ptr(), _ptr(lse), B, Hq, Hkv, L, Lk, D,
                                 float(D ** -0.5 if scale is None else scale), _stream()), "ats_attention_fwd")
     return (out, lse) if return_lse else out
 
 
 def causal_attention_bwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Tensor, lse: torch.Tensor,
-                         dout: torch.Tensor, scale: Optional[float] = None):
-    """Gradients of causal_attention: q [B,Hq,L,D], k, v [B,Hkv,Lk,D], out, dout [B,L,Hq*D], lse [B,Hq,L].
-    Returns (dq, dk, dv) shaped like q, k, v."""
+                         dout: torch.Tensor, scale: Optional[float] = None, key_bias: Optional[torch.Tensor] = None):
+    """Gradients of causal_attention: q [B,Hq,L,D], k, v [B,Hkv,Lk,D], out, dout [B,L,Hq*D], lse [B,Hq,L],
+    key_bias as in the forward.  Returns (dq, dk, dv) shaped like q, k, v."""
     _need_gpu(q, k, v, out, lse, dout)
     B, Hq, L, D = q.shape
     Hkv, Lk = k.shape[1], k.shape[2]
@@ -611,13 +622,15 @@ def causal_attention_bwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out:
     q, k, v, out = q.contiguous(), k.contiguous(), v.contiguous(), out.contiguous()
     dout = dout.to(q.dtype).contiguous()
     lse = lse.contiguous()
+    key_bias = _key_bias(key_bias, B, Lk, q, "causal_attention_bwd")
     lib = _lib.load()
     delta = torch.empty(B, Hq, L, dtype=torch.float32, device=q.device)
     check(lib.ats_attention_delta(out.data_ptr(), dout.data_ptr(), delta.data_ptr(), B, Hq, L, D, _stream()),
           "ats_attention_delta")
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     check(lib.ats_attention_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), dout.data_ptr(), lse.data_ptr(),
-                                delta.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), B, Hq, Hkv, L, Lk, D,
+                                delta.data_ptr(), _ptr(key_bias), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), B, Hq, Hkv,
+                                L, Lk, D,
                                 float(D ** -0.5 if scale is None else scale), _stream()), "ats_attention_bwd")
     return dq, dk, dv
 

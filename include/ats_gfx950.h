@@ -271,9 +271,12 @@ int ats_grouped_gemm_nt(const void* a, const void* const* a_ptrs, int64_t lda, i
  * cache in front of the queries (model.py:700-704): query i sits at position i + Lk - L and sees keys up
  * to there.  The reference's masked path only runs that case for L = 1 (its [L, L] mask does not
  * broadcast otherwise); its flash path aligns the diagonal the same way.
- * lse (optional): [B,Hq,L] float32 log-sum-exp of the scaled scores per query. */
-int ats_attention_fwd(const void* q, const void* k, const void* v, int64_t v_sb, int64_t v_sl, int64_t v_sh, void* out,
-                      float* lse, int B, int Hq, int Hkv, int L, int Lk, int D, float scale, ats_stream_t stream);
+ * key_bias (optional): [B,Lk] float32 added to the scaled scores of a key for every query and head; the
+ * reference's padding mask is (1 - attention_mask) * -1e4 (model.py:819-824).
+ * lse (optional): [B,Hq,L] float32 log-sum-exp of the scaled (and biased) scores per query. */
+int ats_attention_fwd(const void* q, const void* k, const void* v, int64_t v_sb, int64_t v_sl, int64_t v_sh,
+                      const float* key_bias, void* out, float* lse, int B, int Hq, int Hkv, int L, int Lk, int D,
+                      float scale, ats_stream_t stream);
 
 /* ---- Causal grouped-query attention (backward) ----------------------------------
  * The reference leaves this gradient to autograd (model.py:757-839 under torch.autograd); the kernels
@@ -282,12 +285,12 @@ int ats_attention_fwd(const void* q, const void* k, const void* v, int64_t v_sb,
  * without atomics (one kernel owns query rows, one owns key rows and sums over the query heads of
  * its kv head).  ats_attention_delta: delta[B,Hq,L] = sum_d dO*O with out, dout [B,L,Hq*D].
  * ats_attention_bwd: q [B,Hq,L,D], k, v [B,Hkv,Lk,D], dout [B,L,Hq*D] contiguous; lse, delta [B,Hq,L];
- * dq, dk, dv shaped like q, k, v. */
+ * key_bias as in the forward (optional); dq, dk, dv shaped like q, k, v. */
 int ats_attention_delta(const void* out, const void* dout, float* delta, int B, int Hq, int L, int D,
                         ats_stream_t stream);
 int ats_attention_bwd(const void* q, const void* k, const void* v, const void* dout, const float* lse,
-                      const float* delta, void* dq, void* dk, void* dv, int B, int Hq, int Hkv, int L, int Lk, int D,
-                      float scale, ats_stream_t stream);
+                      const float* delta, const float* key_bias, void* dq, void* dk, void* dv, int B, int Hq, int Hkv,
+                      int L, int Lk, int D, float scale, ats_stream_t stream);
 
 /* ---- Training-step ops beside the sparse layer --------------------------------
  * Fused cross-entropy + accuracy.  Replaces fused_cross_entropy_accuracy_launcher

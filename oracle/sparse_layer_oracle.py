@@ -502,20 +502,25 @@ def clip_grad_norm(grads, max_norm: float):
 
 
 # --------------------------------------------------------------------------- attention
-def attention_standard(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float) -> torch.Tensor:
-    """MS/core/model.py:757-823 (GroupedQueryAttention._standard_attention, no extra mask, no dropout).
+def attention_standard(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float,
+                       attention_mask=None) -> torch.Tensor:
+    """MS/core/model.py:757-838 (GroupedQueryAttention._standard_attention, no dropout).
     q [B,H,L,D], k/v [B,H,Lk,D] (already expanded to H heads), Lk >= L.  Scores and softmax in float32,
     causal positions filled with -1e4, probabilities cast to the input dtype before the second matmul,
     output [B, L, H*D] in the input dtype.
     With cached keys in front (Lk > L, model.py:700-704) query i sits at position i + Lk - L.  The
     reference's own [L, L] mask only broadcasts against [L, Lk] scores for L = 1 (one new token, which
     then sees every key); the diagonal used here is that case's generalisation, and equals what slicing
-    the last L query rows out of a full-length call gives."""
+    the last L query rows out of a full-length call gives.
+    attention_mask [B, Lk] (1 = real key, 0 = padding) adds (1 - mask) * -1e4 to every query's and head's
+    scores of a key (model.py:819-824), after the causal fill."""
     B, H, L, D = q.shape
     Lk = k.shape[2]
     scores = torch.matmul(q.float(), k.float().transpose(-2, -1)) * scale
     causal = torch.triu(torch.ones(L, Lk, dtype=torch.bool), diagonal=1 + Lk - L)
     scores = scores.masked_fill(causal, -1e4)
+    if attention_mask is not None:
+        scores = scores + (1.0 - attention_mask.float()[:, None, None, :]) * -1e4
     scores = scores - scores.detach().amax(dim=-1, keepdim=True)
     w = F.softmax(scores, dim=-1, dtype=torch.float32).to(q.dtype)
     out = torch.matmul(w.float(), v.float()).to(q.dtype)
@@ -524,7 +529,7 @@ def attention_standard(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale:
 
 def gqa_forward(x: torch.Tensor, wq: torch.Tensor, wk: torch.Tensor, wv: torch.Tensor, wo: torch.Tensor,
                 num_heads: int, num_kv_heads: int, theta: float = 10000.0, past_key_value=None,
-                use_cache: bool = False):
+                use_cache: bool = False, attention_mask=None):
     """MS/core/model.py:663-731 (GroupedQueryAttention.forward): projections (float32 accumulation,
     rounded to the input dtype like nn.Linear), RoPE at positions 0..L-1 (also with a cache, 690-698),
     cached keys/values concatenated in front (700-704), KV heads repeated, attention, o_proj.
@@ -545,6 +550,6 @@ def gqa_forward(x: torch.Tensor, wq: torch.Tensor, wk: torch.Tensor, wv: torch.T
     if rep > 1:
         k = k.repeat_interleave(rep, dim=1)
         v = v.repeat_interleave(rep, dim=1)
-    a = attention_standard(q, k, v, D ** -0.5)
+    a = attention_standard(q, k, v, D ** -0.5, attention_mask)
     out = lin(a, wo)
     return (out, cache) if use_cache else out

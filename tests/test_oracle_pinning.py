@@ -561,6 +561,43 @@ def test_attention_standard_with_cached_keys():
     assert torch.allclose(one.double(), torch.einsum("bhj,bhjd->bhd", p, v.double()), atol=1e-5)
 
 
+def test_attention_standard_padding_mask():
+    """A [B, Lk] mask of real (1) and padded (0) keys: with right padding every query sees a real key, and
+    the result equals attention over the real keys alone (the padded ones get exp(-1e4) = 0 weight);
+    an all-ones mask changes nothing; a brute-force sum with the additive -1e4 covers left padding."""
+    g = torch.Generator().manual_seed(85)
+    B, H, L, D = 2, 2, 12, 8
+    q = torch.randn(B, H, L, D, generator=g)
+    k = torch.randn(B, H, L, D, generator=g)
+    v = torch.randn(B, H, L, D, generator=g)
+    scale = D ** -0.5
+    assert torch.equal(O.attention_standard(q, k, v, scale, torch.ones(B, L)), O.attention_standard(q, k, v, scale))
+    real = [9, 5]
+    mask = torch.zeros(B, L)
+    for b, n in enumerate(real):
+        mask[b, :n] = 1
+    out = O.attention_standard(q, k, v, scale, mask).view(B, L, H, D)
+    for b, n in enumerate(real):
+        head = O.attention_standard(q[b:b + 1, :, :n], k[b:b + 1, :, :n], v[b:b + 1, :, :n], scale).view(1, n, H, D)
+        assert torch.allclose(out[b:b + 1, :n], head, atol=1e-6)
+        # a padded query position still sees every real key and nothing else
+        p = torch.softmax(torch.einsum("hid,hjd->hij", q[b, :, n:].double(), k[b, :, :n].double()) * scale, -1)
+        tail = torch.einsum("hij,hjd->ihd", p, v[b, :, :n].double())
+        assert torch.allclose(out[b, n:].double(), tail, atol=1e-5)
+    # integer masks as a tokenizer gives them
+    assert torch.equal(O.attention_standard(q, k, v, scale, mask.long()).view(B, L, H, D), out)
+    # left padding, brute force in float64 with the same additive constants; query 0 sees only a padded key
+    # and, like the reference, then spreads its weight over every key whose fill is -1e4 as well
+    mask = torch.ones(B, L)
+    mask[:, :3] = 0
+    out = O.attention_standard(q, k, v, scale, mask).view(B, L, H, D)
+    s = torch.einsum("bhid,bhjd->bhij", q.double(), k.double()) * scale
+    s = s.masked_fill(torch.triu(torch.ones(L, L, dtype=torch.bool), 1), -1e4) + (1 - mask.double())[:, None, None, :] * -1e4
+    ref = torch.einsum("bhij,bhjd->bihd", torch.softmax(s, -1), v.double())
+    assert torch.allclose(out[:, 3:].double(), ref[:, 3:], atol=1e-5)
+    assert torch.allclose(out[:, :3].double(), ref[:, :3], atol=2e-3)     # float32 scores near 1e4 resolve 1e-3
+
+
 def test_gqa_forward_cache_round_trip():
     """use_cache returns the rotated keys and the values; feeding them back with new tokens reproduces the
     reference's quirk of rotating the new tokens at positions 0..L-1 (model.py:690-698)."""
