@@ -4,6 +4,9 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+#include <initializer_list>
+
 #include "../../include/ats_gfx950.h"
 
 namespace ats {
@@ -29,6 +32,26 @@ void set_error(const char* fmt, ...);
             return ATS_ERR_LAUNCH;                                                    \
         }                                                                             \
     } while (0)
+
+// A kernel that uses more than 64 KB of dynamic LDS needs the limit raised once per device (the attribute
+// belongs to the function on the current device).  One LdsReservation per launch site remembers, as a
+// bit per device id, where that has been done; racing first calls only repeat the idempotent request.
+struct LdsReservation {
+    std::atomic<uint64_t> done{0};
+};
+inline hipError_t reserve_lds(LdsReservation& r, std::initializer_list<const void*> kernels, int bytes) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    const uint64_t bit = 1ull << (dev & 63);
+    if (dev < 64 && (r.done.load(std::memory_order_relaxed) & bit)) return hipSuccess;
+    for (const void* k : kernels) {
+        e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+        if (e != hipSuccess) return e;
+    }
+    if (dev < 64) r.done.fetch_or(bit, std::memory_order_relaxed);
+    return hipSuccess;
+}
 
 inline hipStream_t as_stream(ats_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }

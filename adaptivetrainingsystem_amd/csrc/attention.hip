@@ -405,13 +405,12 @@ extern "C" int ats_attention_fwd(const void* q, const void* k, const void* v, in
     ATS_REQUIRE(n_blocks <= 0x7fffffff, ATS_ERR_UNSUPPORTED, "ats_attention_fwd: %lld workgroups", (long long)n_blocks);
     const dim3 grid((unsigned)n_blocks);
     const float scale_log2 = scale * 1.4426950408889634f;
-    static bool reserved_lds[4] = {false, false, false, false};      // per kernel instance
-    auto launch = [&](auto kernel, int smem, bool& reserved) -> int {
-        if (smem > 64 * 1024 && !reserved) {
-            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, smem);
-            ATS_REQUIRE(e == hipSuccess, ATS_ERR_LAUNCH, "ats_attention_fwd: cannot reserve %d bytes of LDS", smem);
-            reserved = true;
+    static LdsReservation reserved_lds[4];      // one per kernel instance
+    auto launch = [&](auto kernel, int smem, LdsReservation& reserved) -> int {
+        if (smem > 64 * 1024) {
+            hipError_t e = reserve_lds(reserved, {reinterpret_cast<const void*>(kernel)}, smem);
+            ATS_REQUIRE(e == hipSuccess, ATS_ERR_LAUNCH, "ats_attention_fwd: cannot reserve %d bytes of LDS: %s", smem,
+                        hipGetErrorString(e));
         }
         hipLaunchKernelGGL(kernel, grid, dim3(kAttThreads), smem, as_stream(stream), static_cast<const bf16_t*>(q),
                            static_cast<const bf16_t*>(k), static_cast<const bf16_t*>(v), v_sb, (int)v_sl, v_sh, key_bias,

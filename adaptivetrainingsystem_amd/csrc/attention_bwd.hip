@@ -548,13 +548,10 @@ extern "C" int ats_attention_bwd(const void* q, const void* k, const void* v, co
         constexpr int smem_dq = 2 * kDqBN * (128 * 2 + 16) + kDqBN * (128 * 2 + 64) + kDqBN * 4;
         constexpr int smem_dkv = 2 * kDkvBQ * (128 * 2 + 16) + 2 * kDkvBQ * (128 * 2 + 64) + 2 * kDkvBQ * 4 +
                                  kBwdRows * (128 * 2 + 16);
-        static bool attr = false;
-        if (!attr) {
-            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(attention_bwd_dkv_kernel<128>),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, smem_dkv);
-            ATS_REQUIRE(e == hipSuccess, ATS_ERR_LAUNCH, "ats_attention_bwd: cannot reserve %d bytes of LDS", smem_dkv);
-            attr = true;
-        }
+        static LdsReservation reserved;
+        hipError_t e = reserve_lds(reserved, {reinterpret_cast<const void*>(attention_bwd_dkv_kernel<128>)}, smem_dkv);
+        ATS_REQUIRE(e == hipSuccess, ATS_ERR_LAUNCH, "ats_attention_bwd: cannot reserve %d bytes of LDS: %s", smem_dkv,
+                    hipGetErrorString(e));
         if (key_bias)
             hipLaunchKernelGGL((attention_bwd_dq_kernel<128, true>), dim3((unsigned)dq_blocks), dim3(256), smem_dq, s, q_,
                                k_, v_, do_, lse, delta, key_bias, static_cast<bf16_t*>(dq), Hq, Hkv, L, Lk, scale, B);

@@ -768,19 +768,15 @@ static int launch_cfg(const GroupedArgs& p0, int64_t max_rows, hipStream_t s) {
         if constexpr (DMA) return grouped_gemm_dma_kernel<T, TO, BM, BN, WM, WN, SM, SN, SWIGLU>;
         else return grouped_gemm_pipelined_kernel<T, TO, BM, BN, WM, WN, SM, SN, SWIGLU, true>;
     }();
-    static bool attr_done = false;
-    if (!attr_done) {
-        if (smem > 64 * 1024) {
-            for (const void* k : {reinterpret_cast<const void*>(kern_general), reinterpret_cast<const void*>(kern_pipe),
-                                  reinterpret_cast<const void*>(kern_dma)}) {
-                hipError_t e = hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-                if (e != hipSuccess) {
-                    set_error("grouped GEMM: cannot reserve %zu bytes of LDS: %s", smem, hipGetErrorString(e));
-                    return ATS_ERR_LAUNCH;
-                }
-            }
+    if (smem > 64 * 1024) {
+        static LdsReservation reserved;      // one per tile configuration (this function is a template)
+        hipError_t e = reserve_lds(reserved, {reinterpret_cast<const void*>(kern_general),
+                                              reinterpret_cast<const void*>(kern_pipe),
+                                              reinterpret_cast<const void*>(kern_dma)}, (int)smem);
+        if (e != hipSuccess) {
+            set_error("grouped GEMM: cannot reserve %zu bytes of LDS: %s", smem, hipGetErrorString(e));
+            return ATS_ERR_LAUNCH;
         }
-        attr_done = true;
     }
     const int64_t blocks = grid_blocks(max_rows, p.E, BM, p.n_tiles, SM, SN);
     if (blocks > 0x7fffffffLL) {

@@ -253,14 +253,10 @@ extern "C" int ats_select_topk_per_sequence(const float* score, int B, int L, in
     const int threads = lp2 / 2 < 64 ? 64 : (lp2 / 2 > 1024 ? 1024 : lp2 / 2);
     const size_t smem = (size_t)lp2 * 12;
     if (smem > 64 * 1024) {
-        static bool attr_done = false;
-        if (!attr_done) {
-            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(select_topk_seq_kernel),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, 8192 * 12);
-            ATS_REQUIRE(e == hipSuccess, ATS_ERR_LAUNCH, "ats_select_topk_per_sequence: LDS attribute: %s",
-                        hipGetErrorString(e));
-            attr_done = true;
-        }
+        static LdsReservation reserved;
+        hipError_t e = reserve_lds(reserved, {reinterpret_cast<const void*>(select_topk_seq_kernel)}, 8192 * 12);
+        ATS_REQUIRE(e == hipSuccess, ATS_ERR_LAUNCH, "ats_select_topk_per_sequence: LDS attribute: %s",
+                    hipGetErrorString(e));
     }
     hipLaunchKernelGGL(select_topk_seq_kernel, dim3(B), dim3(threads), smem, as_stream(stream), score, L, lp2, keep,
                        sel);
