@@ -41,6 +41,11 @@ _SIGNATURES = {
                                           c_int64, c_int, c_int, c_int, c_void_p]),
     "ats_grouped_down": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int, c_int,
                                  c_int, c_int, c_void_p]),
+    "ats_grouped_down_splitk": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64,
+                                        c_int, c_int, c_int, c_int, c_void_p]),
+    "ats_sum_partials": (c_int, [c_void_p, c_int, c_int64, c_void_p, c_int64, c_int, c_void_p]),
+    "ats_combine_partials": (c_int, [c_void_p, c_int, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int,
+                                     c_int, c_int, c_void_p]),
     "ats_rmsnorm_bwd_workspace": (c_size_t, [c_int64, c_int]),
     "ats_rmsnorm_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_float, c_int, c_int,
                                 c_void_p, c_size_t, c_void_p]),

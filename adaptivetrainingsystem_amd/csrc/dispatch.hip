@@ -327,11 +327,15 @@ __global__ __launch_bounds__(256) void combine_kernel(const TY* __restrict__ y, 
 }
 
 // Vector form: H multiple of the 16-byte vector width of both types, aligned.
-template <typename TY, typename TO, int MAXK>
+// PARTS: y is n_parts float32 partial results part_stride elements apart (a down projection split
+// along K); an expert row is their sum in slice order, rounded to the output type like the unsplit
+// projection's result, before the weighting.
+template <typename TY, typename TO, int MAXK, bool PARTS = false>
 __global__ __launch_bounds__(256) void combine_vec_kernel(const TY* __restrict__ y, const int32_t* __restrict__ row_of,
                                                           const float* __restrict__ w,
                                                           const TO* __restrict__ residual, TO* __restrict__ out,
-                                                          int64_t T, int k, int H) {
+                                                          int64_t T, int k, int H, int n_parts = 1,
+                                                          int64_t part_stride = 0) {
     constexpr int V = 8;  // columns per lane per step (one 16-byte bf16 vector or two float vectors)
     const int lane = lane_id();
     const int64_t wave = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
@@ -368,7 +372,22 @@ __global__ __launch_bounds__(256) void combine_vec_kernel(const TY* __restrict__
             for (int n = 0; n < MAXK; ++n) {
                 if (n < n_kept) {
                     const TY* yr = y + rows[n] * H + h0;
-                    if constexpr (sizeof(TY) == 2) {
+                    if constexpr (PARTS) {
+                        static_assert(sizeof(TY) == 4, "partial results are float32");
+#pragma unroll
+                        for (int j = 0; j < V; ++j) yv[n][j] = 0.f;
+                        for (int s2 = 0; s2 < n_parts; ++s2) {
+                            float pv[V];
+                            Elem<TY>::unpack(*reinterpret_cast<const uint4*>(yr + s2 * part_stride), pv);
+                            Elem<TY>::unpack(*reinterpret_cast<const uint4*>(yr + s2 * part_stride + 4), pv + 4);
+#pragma unroll
+                            for (int j = 0; j < V; ++j) yv[n][j] += pv[j];
+                        }
+                        if constexpr (sizeof(TO) == 2) {
+#pragma unroll
+                            for (int j = 0; j < V; ++j) yv[n][j] = bf16_bits_to_float(float_to_bf16_bits(yv[n][j]));
+                        }
+                    } else if constexpr (sizeof(TY) == 2) {
                         Elem<TY>::unpack(*reinterpret_cast<const uint4*>(yr), yv[n]);
                     } else {
                         Elem<TY>::unpack(*reinterpret_cast<const uint4*>(yr), yv[n]);
@@ -429,7 +448,88 @@ static void launch_combine(const void* y, const int32_t* row_of, const float* w,
                            k, H);
 }
 
+// out[i] = sum over the n_parts partial results of parts[s * part_stride + i], added in slice order.
+template <typename TO>
+__global__ __launch_bounds__(256) void sum_partials_kernel(const float* __restrict__ parts, int n_parts,
+                                                           int64_t part_stride, TO* __restrict__ out, int64_t n4) {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += (int64_t)gridDim.x * blockDim.x) {
+        float4 acc = *reinterpret_cast<const float4*>(parts + i * 4);
+        for (int s = 1; s < n_parts; ++s) {
+            const float4 v = *reinterpret_cast<const float4*>(parts + s * part_stride + i * 4);
+            acc.x += v.x;
+            acc.y += v.y;
+            acc.z += v.z;
+            acc.w += v.w;
+        }
+        if constexpr (sizeof(TO) == 2) {
+            uint2 u;
+            u.x = pack_bf16x2(acc.x, acc.y);
+            u.y = pack_bf16x2(acc.z, acc.w);
+            *reinterpret_cast<uint2*>(out + i * 4) = u;
+        } else {
+            *reinterpret_cast<float4*>(out + i * 4) = acc;
+        }
+    }
+}
+
 }  // namespace ats
+
+extern "C" int ats_sum_partials(const float* parts, int n_parts, int64_t part_stride, void* out, int64_t n,
+                                int out_dtype, ats_stream_t stream) {
+    using namespace ats;
+    ATS_REQUIRE(n_parts >= 1 && n >= 0 && n % 4 == 0 && part_stride % 4 == 0 && part_stride >= n, ATS_ERR_INVALID_ARG,
+                "ats_sum_partials: n_parts=%d n=%lld part_stride=%lld (multiples of 4 elements)", n_parts, (long long)n,
+                (long long)part_stride);
+    ATS_REQUIRE(out_dtype == ATS_F32 || out_dtype == ATS_BF16, ATS_ERR_UNSUPPORTED, "ats_sum_partials: dtype tag %d",
+                out_dtype);
+    if (n == 0) return ATS_OK;
+    ATS_REQUIRE(parts && out && aligned16(parts) && (reinterpret_cast<uintptr_t>(out) & 7u) == 0, ATS_ERR_INVALID_ARG,
+                "ats_sum_partials: null or misaligned pointer");
+    const int64_t n4 = n / 4;
+    int64_t blocks = (n4 + 255) / 256;
+    if (blocks > 4096) blocks = 4096;
+    if (out_dtype == ATS_F32)
+        hipLaunchKernelGGL((sum_partials_kernel<float>), dim3((unsigned)blocks), dim3(256), 0, as_stream(stream), parts,
+                           n_parts, part_stride, static_cast<float*>(out), n4);
+    else
+        hipLaunchKernelGGL((sum_partials_kernel<bf16_t>), dim3((unsigned)blocks), dim3(256), 0, as_stream(stream), parts,
+                           n_parts, part_stride, static_cast<bf16_t*>(out), n4);
+    ATS_CHECK_LAUNCH("ats_sum_partials");
+    return ATS_OK;
+}
+
+extern "C" int ats_combine_partials(const float* parts, int n_parts, int64_t part_stride, const int32_t* row_of,
+                                    const float* w, const void* residual, void* out, int64_t T, int k, int H,
+                                    int out_dtype, ats_stream_t stream) {
+    using namespace ats;
+    const char* name = "ats_combine_partials";
+    ATS_REQUIRE(T >= 0 && k > 0 && k <= 8 && H > 0 && H % 8 == 0 && n_parts >= 1 && part_stride % 4 == 0,
+                ATS_ERR_INVALID_ARG, "%s: T=%lld k=%d (<= 8) H=%d (multiple of 8) n_parts=%d part_stride=%lld", name,
+                (long long)T, k, H, n_parts, (long long)part_stride);
+    ATS_REQUIRE(out_dtype == ATS_F32 || out_dtype == ATS_BF16, ATS_ERR_UNSUPPORTED, "%s: dtype tag %d", name, out_dtype);
+    if (T == 0) return ATS_OK;
+    ATS_REQUIRE(parts && row_of && w && out && aligned16(parts) && aligned16(out) && (!residual || aligned16(residual)),
+                ATS_ERR_INVALID_ARG, "%s: null or misaligned pointer", name);
+    int64_t blocks = (T + 3) / 4;
+    if (blocks > 16384) blocks = 16384;
+    hipStream_t s = as_stream(stream);
+#define ATS_COMBINE_PARTS(TO_, MAXK_)                                                                              \
+    hipLaunchKernelGGL((combine_vec_kernel<float, TO_, MAXK_, true>), dim3((unsigned)blocks), dim3(256), 0, s, parts, \
+                       row_of, w, static_cast<const TO_*>(residual), static_cast<TO_*>(out), T, k, H, n_parts,       \
+                       part_stride)
+    if (out_dtype == ATS_F32) {
+        if (k <= 2) ATS_COMBINE_PARTS(float, 2);
+        else if (k <= 4) ATS_COMBINE_PARTS(float, 4);
+        else ATS_COMBINE_PARTS(float, 8);
+    } else {
+        if (k <= 2) ATS_COMBINE_PARTS(bf16_t, 2);
+        else if (k <= 4) ATS_COMBINE_PARTS(bf16_t, 4);
+        else ATS_COMBINE_PARTS(bf16_t, 8);
+    }
+#undef ATS_COMBINE_PARTS
+    ATS_CHECK_LAUNCH(name);
+    return ATS_OK;
+}
 
 extern "C" size_t ats_dispatch_plan_workspace(int64_t T, int k, int E) {
     if (T <= 0 || k <= 0 || E <= 0) return 0;

@@ -43,6 +43,10 @@ struct GroupedArgs {
     const int32_t* row_start;
     const int32_t* row_count;
     int E, K, N_out, up_offset, n_tiles;
+    // split K (register-staged kernel only): k_splits > 1 turns every expert into k_splits groups that each
+    // multiply a K / k_splits wide slice and write a partial result part_stride elements apart
+    int k_splits, k_slice;   // k_slice = K / k_splits
+    int64_t part_stride;
     // direct-to-LDS path only: bytes addressable from the A / B descriptors (0 = path not usable)
     uint32_t a_extent_bytes, b_extent_bytes;
 };
@@ -294,7 +298,8 @@ __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(
 //   LDS barrier
 //   k-step 3: MFMAs(buf 1) | read k-step 0 of slab t+1
 // Global loads therefore have a whole slab of MFMA time to land before they are needed.
-template <typename T, typename TO, int BM, int BN, int WM, int WN, int SM, int SN, bool SWIGLU, bool WARM>
+template <typename T, typename TO, int BM, int BN, int WM, int WN, int SM, int SN, bool SWIGLU, bool WARM,
+          bool SLICED = false>
 __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_pipelined_kernel(GroupedArgs p) {
     constexpr int NT = WM * WN * 64;
     constexpr int VEC = 16 / (int)sizeof(T);
@@ -314,12 +319,27 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_pipelined_kernel(Gro
     extern __shared__ __align__(16) unsigned char smem[];
 
     TileCoord tc;
-    if (!decode_tile(blockIdx.x, p.row_count, p.E, BM, p.n_tiles, SM, SN, &tc)) return;
+    // SLICED: every expert is k_splits groups, each with a K / k_splits wide slice and its own partial output
+    // (without the SwiGLU epilogue only: it is not linear)
+    static_assert(!(SLICED && SWIGLU), "slices of K need a linear epilogue");
+    constexpr bool sliced = SLICED;
+    int split = 0;
+    if constexpr (SLICED) {
+        if (!decode_tile_sliced(blockIdx.x, p.row_count, p.E, BM, p.n_tiles, SM, SN, p.k_splits, &tc, &split)) return;
+        // uniform over the block: back into scalar registers, whatever unit the walk ran on
+        tc.e = __builtin_amdgcn_readfirstlane(tc.e);
+        tc.mt = __builtin_amdgcn_readfirstlane(tc.mt);
+        tc.nt = __builtin_amdgcn_readfirstlane(tc.nt);
+        split = __builtin_amdgcn_readfirstlane(split);
+    } else {
+        if (!decode_tile(blockIdx.x, p.row_count, p.E, BM, p.n_tiles, SM, SN, &tc)) return;
+    }
     const int count = p.row_count[tc.e];
     const int row0 = p.row_start[tc.e];
-    const int K = p.k_count ? p.k_count[tc.e] : p.K;
-    const T* Bexp = static_cast<const T*>(p.b[tc.e]);
-    const T* A = static_cast<const T*>(p.a_ptrs ? p.a_ptrs[tc.e] : p.a);
+    const int K = sliced ? p.k_slice : (p.k_count ? p.k_count[tc.e] : p.K);
+    const int64_t k_first = sliced ? (int64_t)split * p.k_slice : 0;
+    const T* Bexp = static_cast<const T*>(p.b[tc.e]) + k_first;
+    const T* A = static_cast<const T*>(p.a_ptrs ? p.a_ptrs[tc.e] : p.a) + k_first;
     const int arow0 = p.a_ptrs ? 0 : row0;
 
     const int tid = threadIdx.x;
@@ -529,7 +549,7 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_pipelined_kernel(Gro
 #undef PL_LOADG
 #undef PL_ITER
 
-    TO* out = static_cast<TO*>(p.out);
+    TO* out = static_cast<TO*>(p.out) + (sliced ? (int64_t)split * p.part_stride : 0);
     if (p.E < 0) out[0] = TO{};   // never true; with the next line it keeps the warm-up loads alive
     if (p.E < 0 && junk == 0x5a5a5a5au) out[1] = TO{};
     {
@@ -763,10 +783,12 @@ static int launch_cfg(const GroupedArgs& p0, int64_t max_rows, hipStream_t s) {
     constexpr size_t smem = 2 * (size_t)(BM + BN) * kRowPitch;  // covers the unpadded DMA layout too
     constexpr int BK = 128 / (int)sizeof(T);
     auto kern_general = grouped_gemm_kernel<T, TO, BM, BN, WM, WN, SM, SN, SWIGLU>;
-    auto kern_pipe = grouped_gemm_pipelined_kernel<T, TO, BM, BN, WM, WN, SM, SN, SWIGLU, true>;
+    // the L2 warm-up touches pay where blocks share operand panels; the weight-streaming tiles share nothing
+    constexpr bool kWarm = BM != 32;
+    auto kern_pipe = grouped_gemm_pipelined_kernel<T, TO, BM, BN, WM, WN, SM, SN, SWIGLU, kWarm>;
     auto kern_dma = [] {
         if constexpr (DMA) return grouped_gemm_dma_kernel<T, TO, BM, BN, WM, WN, SM, SN, SWIGLU>;
-        else return grouped_gemm_pipelined_kernel<T, TO, BM, BN, WM, WN, SM, SN, SWIGLU, true>;
+        else return grouped_gemm_pipelined_kernel<T, TO, BM, BN, WM, WN, SM, SN, SWIGLU, kWarm>;
     }();
     if (smem > 64 * 1024) {
         static LdsReservation reserved;      // one per tile configuration (this function is a template)
@@ -778,10 +800,24 @@ static int launch_cfg(const GroupedArgs& p0, int64_t max_rows, hipStream_t s) {
             return ATS_ERR_LAUNCH;
         }
     }
-    const int64_t blocks = grid_blocks(max_rows, p.E, BM, p.n_tiles, SM, SN);
+    // slices of K: the weight-streaming tiles only, in their own instance of the register-staged kernel
+    constexpr bool kCanSlice = !DMA && !SWIGLU && BM == 32;
+    const int splits = p.k_splits > 1 ? p.k_splits : 1;
+    if (splits > 1 && (!kCanSlice || p.k_count || p.K % splits != 0 || (p.K / splits) % BK != 0)) {
+        set_error("grouped GEMM: %d slices of K=%d are not available for this tile configuration", splits, p.K);
+        return ATS_ERR_UNSUPPORTED;
+    }
+    const int64_t blocks = grid_blocks(max_rows * splits, p.E * splits, BM, p.n_tiles, SM, SN);
     if (blocks > 0x7fffffffLL) {
         set_error("grouped GEMM: grid of %lld blocks", (long long)blocks);
         return ATS_ERR_UNSUPPORTED;
+    }
+    if constexpr (kCanSlice) {
+        if (splits > 1) {
+            hipLaunchKernelGGL((grouped_gemm_pipelined_kernel<T, TO, BM, BN, WM, WN, SM, SN, SWIGLU, kWarm, true>),
+                               dim3((unsigned)blocks), dim3(WM * WN * 64), smem, s, p);
+            return ATS_OK;
+        }
     }
     // the direct-to-LDS kernel addresses its operands with 32-bit lane offsets
     const bool dma_ok = DMA && p.K % BK == 0 && p.a_extent_bytes != 0 && p.b_extent_bytes != 0;
@@ -905,6 +941,48 @@ extern "C" int ats_grouped_down(const void* h, const void* const* w_d, void* y, 
     else rc = launch_grouped<bf16_t, bf16_t, false>(p, max_rows, s);
     if (rc != ATS_OK) return rc;
     ATS_CHECK_LAUNCH("ats_grouped_down");
+    return ATS_OK;
+}
+
+extern "C" int ats_grouped_down_splitk(const void* h, const void* const* w_d, float* parts, const int32_t* row_start,
+                                       const int32_t* row_count, int E, int64_t max_rows, int64_t part_rows, int H,
+                                       int I, int k_splits, int dtype, ats_stream_t stream) {
+    using namespace ats;
+    const char* name = "ats_grouped_down_splitk";
+    int rc = check_common(name, h, w_d, parts, row_start, row_count, E, max_rows, H, I, dtype);
+    if (rc != ATS_OK) return rc;
+    ATS_REQUIRE(k_splits >= 1 && k_splits <= 64 && part_rows >= 0, ATS_ERR_INVALID_ARG, "%s: k_splits=%d part_rows=%lld",
+                name, k_splits, (long long)part_rows);
+    const int slab = dtype == ATS_F32 ? 32 : 64;
+    ATS_REQUIRE(I % (k_splits * slab) == 0, ATS_ERR_UNSUPPORTED, "%s: I=%d is not %d slices of whole %d-element slabs",
+                name, I, k_splits, slab);
+    ATS_REQUIRE(max_rows / E <= 48, ATS_ERR_UNSUPPORTED,
+                "%s: %lld rows for %d experts (slices of K are built for the weight-streaming tiles, <= 48 rows per expert)",
+                name, (long long)max_rows, E);
+    if (max_rows == 0) return ATS_OK;
+    GroupedArgs p{};
+    p.a = h;
+    p.a_row_div = 1;
+    p.lda = I;
+    p.b = w_d;
+    p.ldb = I;
+    p.out = parts;
+    p.ldo = H;
+    p.row_start = row_start;
+    p.row_count = row_count;
+    p.E = E;
+    p.K = I;
+    p.N_out = H;
+    p.k_splits = k_splits;
+    p.k_slice = I / k_splits;
+    p.part_stride = part_rows * H;
+    p.a_extent_bytes = 0xffffffffu;
+    p.b_extent_bytes = extent32(H, I, dtype == ATS_F32 ? 4 : 2);
+    hipStream_t s = as_stream(stream);
+    rc = dtype == ATS_F32 ? launch_grouped<float, float, false>(p, max_rows, s)
+                          : launch_grouped<bf16_t, float, false>(p, max_rows, s);
+    if (rc != ATS_OK) return rc;
+    ATS_CHECK_LAUNCH(name);
     return ATS_OK;
 }
 

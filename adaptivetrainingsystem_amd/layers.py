@@ -269,7 +269,12 @@ class SwiGLUExpert(nn.Module):
         start = torch.zeros(1, dtype=torch.int32, device=x.device)
         count = torch.full((1,), n, dtype=torch.int32, device=x.device)
         h = ops.grouped_gateup_swiglu(x2, ops.weight_pointer_table([wgu]), start, count, n, n, H, I)
-        y = ops.grouped_down(h, ops.weight_pointer_table([wd]), start, count, n, H, I)
+        splits = ops.down_k_splits(1, n, H, I, x2.dtype) if H % 8 == 0 else 1
+        if splits > 1:       # a few rows: slices of K keep every CU streaming the down weights
+            y = ops.sum_partials(ops.grouped_down_splitk(h, ops.weight_pointer_table([wd]), start, count, n, H, I,
+                                                         splits), x2.dtype)
+        else:
+            y = ops.grouped_down(h, ops.weight_pointer_table([wd]), start, count, n, H, I)
         return y.view(shape)
 
 
@@ -391,12 +396,19 @@ class MoEFFNLayer(nn.Module):
             with stage(tm, "gateup_swiglu"):
                 h = ops.grouped_gateup_swiglu(x_flat, wgu_ptrs, plan["offsets"], plan["kept"], rows, rows, H, I,
                                               a_rows=plan["row_src"], a_row_div=k)
+            splits = ops.down_k_splits(E, rows, H, I, x.dtype) if k <= 8 and H % 8 == 0 else 1
             with stage(tm, "down"):
-                y = ops.grouped_down(h, wd_ptrs, plan["offsets"], plan["kept"], rows, H, I)
+                if splits > 1:       # decode sizes: float32 partial results per slice of K, summed by the combine
+                    y = ops.grouped_down_splitk(h, wd_ptrs, plan["offsets"], plan["kept"], rows, H, I, splits)
+                else:
+                    y = ops.grouped_down(h, wd_ptrs, plan["offsets"], plan["kept"], rows, H, I)
         else:
             y = torch.zeros(1, H, dtype=x.dtype, device=x.device)
         with stage(tm, "combine"):
-            out = ops.combine(y, plan["row_of"], route["weights"], T, k, out_dtype=x.dtype)
+            if y.dim() == 3:
+                out = ops.combine_partials(y, plan["row_of"], route["weights"], T, k, x.dtype)
+            else:
+                out = ops.combine(y, plan["row_of"], route["weights"], T, k, out_dtype=x.dtype)
 
         self.last_plan = {"logits": logits, "capacity": C, **route, **plan}
         if self.training:

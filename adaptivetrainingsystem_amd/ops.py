@@ -266,10 +266,51 @@ def grouped_down(h: torch.Tensor, w_d_ptrs: torch.Tensor, row_start: torch.Tenso
     return out
 
 
+def down_k_splits(E: int, max_rows: int, N: int, K: int, dtype: torch.dtype) -> int:
+    """Slices of K for a weight-streaming (<= 48 rows per expert) projection: the 32 x 128 tiles give
+    E * ceil(N / 128) workgroups, and it takes several hundred of them to keep the memory system busy
+    (measured on MI355X: 8 x [4096, 14336] weights 199 -> 160 us with 2 slices; one [4096, 4096]
+    weight 50 -> 13 us with 8).  Powers of two up to 16, slices of at least 512 columns."""
+    slab = 64 if dtype == torch.bfloat16 else 32
+    if E <= 0 or max_rows <= 0 or max_rows // E > 48:
+        return 1
+    groups = E * ((N + 127) // 128)
+    s = 1
+    while s < 16 and groups * s < 384 and K % (2 * s * slab) == 0 and K // (2 * s) >= 512:
+        s *= 2
+    return s
+
+
+def grouped_down_splitk(h: torch.Tensor, w_d_ptrs: torch.Tensor, row_start: torch.Tensor, row_count: torch.Tensor,
+                        max_rows: int, H: int, I: int, k_splits: int) -> torch.Tensor:
+    """Float32 partial results [k_splits, rows, H] of grouped_down with K cut into k_splits slices
+    (decode sizes only); sum_partials or combine_partials add them up."""
+    _need_gpu(h, w_d_ptrs, row_start, row_count)
+    if h.dim() != 2 or h.shape[1] != I or not h.is_contiguous():
+        raise AtsError("grouped_down_splitk: h must be a contiguous [rows, I] tensor")
+    E = w_d_ptrs.numel()
+    parts = torch.empty(k_splits, h.shape[0], H, dtype=torch.float32, device=h.device)
+    check(_lib.load().ats_grouped_down_splitk(h.data_ptr(), w_d_ptrs.data_ptr(), parts.data_ptr(), row_start.data_ptr(),
+                                              row_count.data_ptr(), E, int(max_rows), h.shape[0], H, I, int(k_splits),
+                                              _tag(h), _stream()), "ats_grouped_down_splitk")
+    return parts
+
+
+def sum_partials(parts: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+    """parts float32 [S, ...] -> their sum over S in slice order, rounded once to out_dtype."""
+    _need_gpu(parts)
+    if parts.dtype != torch.float32 or parts.dim() < 2 or not parts.is_contiguous():
+        raise AtsError("sum_partials: parts must be a contiguous float32 [slices, ...] tensor")
+    out = torch.empty(parts.shape[1:], dtype=out_dtype, device=parts.device)
+    check(_lib.load().ats_sum_partials(parts.data_ptr(), parts.shape[0], out.numel(), out.data_ptr(), out.numel(),
+                                       _tag(out), _stream()), "ats_sum_partials")
+    return out
+
+
 # --------------------------------------------------------------------------- combine
 def combine(y: torch.Tensor, row_of: torch.Tensor, weights: torch.Tensor, num_tokens: int, k: int,
             out_dtype: Optional[torch.dtype] = None, residual: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """y [rows, H]; row_of int32 [T*k]; weights f32 [T,k] -> out [T,H]."""
+    """y [rows, H] (any leading shape); row_of int32 [T*k]; weights f32 [T,k] -> out [T,H]."""
     _need_gpu(y, row_of, weights, residual)
     if row_of.dtype != torch.int32 or weights.dtype != torch.float32:
         raise AtsError("combine: row_of must be int32 and weights float32")
@@ -285,6 +326,29 @@ def combine(y: torch.Tensor, row_of: torch.Tensor, weights: torch.Tensor, num_to
     check(_lib.load().ats_combine(y2.data_ptr(), row_of.contiguous().data_ptr(), weights.contiguous().data_ptr(),
                                   _ptr(residual), out.data_ptr(), num_tokens, int(k), H, _tag(y2), _tag(out),
                                   _stream()), "ats_combine")
+    return out
+
+
+def combine_partials(parts: torch.Tensor, row_of: torch.Tensor, weights: torch.Tensor, num_tokens: int, k: int,
+                     out_dtype: torch.dtype, residual: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """combine over the float32 partial results [S, rows, H] of grouped_down_splitk: an expert row is their
+    sum in slice order, rounded to out_dtype like the unsplit projection's result, before the weighting."""
+    _need_gpu(parts, row_of, weights, residual)
+    if row_of.dtype != torch.int32 or weights.dtype != torch.float32:
+        raise AtsError("combine_partials: row_of must be int32 and weights float32")
+    if row_of.numel() != num_tokens * k or weights.numel() != num_tokens * k:
+        raise AtsError("combine_partials: row_of/weights must have tokens*k entries")
+    if parts.dim() != 3 or parts.dtype != torch.float32 or not parts.is_contiguous():
+        raise AtsError("combine_partials: partial results must be a contiguous float32 [slices, rows, H] tensor")
+    S, rows, H = parts.shape
+    out = torch.empty(num_tokens, H, dtype=out_dtype, device=parts.device)
+    if residual is not None:
+        residual = residual.reshape(num_tokens, H).contiguous()
+        if residual.dtype != out.dtype:
+            raise AtsError("combine_partials: residual must have the output dtype")
+    check(_lib.load().ats_combine_partials(parts.data_ptr(), S, rows * H, row_of.contiguous().data_ptr(),
+                                           weights.contiguous().data_ptr(), _ptr(residual), out.data_ptr(),
+                                           num_tokens, int(k), H, _tag(out), _stream()), "ats_combine_partials")
     return out
 
 
@@ -660,4 +724,8 @@ def linear_nt(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
     N = weight.shape[0]
     x, weight = x.contiguous(), weight.contiguous()
     start, count = _single_group(T, x.device)
+    splits = down_k_splits(1, T, N, K, x.dtype) if K % 8 == 0 and N % 8 == 0 else 1
+    if splits > 1:      # a few rows against a whole weight matrix: slices of K keep every CU streaming
+        return sum_partials(grouped_down_splitk(x, weight_pointer_table([weight]), start, count, T, N, K, splits),
+                            x.dtype)
     return grouped_gemm_nt(weight_pointer_table([weight]), K, N, start, count, T, T, N, K, a=x)

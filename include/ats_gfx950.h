@@ -147,6 +147,19 @@ int ats_grouped_gateup_swiglu(const void* a, int64_t a_num_rows, const int32_t* 
 int ats_grouped_down(const void* h, const void* const* w_d, void* y, const int32_t* row_start,
                      const int32_t* row_count, int E, int64_t max_rows, int H, int I, int dtype,
                      int y_dtype, ats_stream_t stream);
+/* The down projection of weight-streaming (decode) sizes, at most 48 rows per expert, split along
+ * K so that enough workgroups stream the weights: slice s of expert e multiplies columns
+ * [s*I/k_splits, (s+1)*I/k_splits) and writes float32 parts[s][row_start[e]+m][:H]
+ * (parts: [k_splits, part_rows, H]).  The result is the sum over s, taken in slice order by
+ * ats_sum_partials or ats_combine_partials.  I must be k_splits whole K slabs (64 bf16 / 32 f32
+ * elements).  Same expert loop as ats_grouped_down (moe_cuda_wrapper.py:452-457). */
+int ats_grouped_down_splitk(const void* h, const void* const* w_d, float* parts, const int32_t* row_start,
+                            const int32_t* row_count, int E, int64_t max_rows, int64_t part_rows, int H,
+                            int I, int k_splits, int dtype, ats_stream_t stream);
+/* out[i] = sum_s parts[s*part_stride + i], i < n, added in slice order in float32 and rounded once
+ * to out_dtype (n and part_stride multiples of 4). */
+int ats_sum_partials(const float* parts, int n_parts, int64_t part_stride, void* out, int64_t n,
+                     int out_dtype, ats_stream_t stream);
 
 /* ---- Combine --------------------------------------------------------------
  * Token-major restatement of MoECUDAOps._pytorch_combine (moe_cuda_wrapper.py:328-359),
@@ -157,6 +170,12 @@ int ats_grouped_down(const void* h, const void* const* w_d, void* y, const int32
  * If residual != NULL, out[t,:] = residual[t,:] + that sum. */
 int ats_combine(const void* y, const int32_t* row_of, const float* w, const void* residual,
                 void* out, int64_t T, int k, int H, int y_dtype, int out_dtype, ats_stream_t stream);
+/* ats_combine over the partial results of ats_grouped_down_splitk: expert row r is
+ * sum_s parts[s*part_stride + r*H + :] (slice order, float32), rounded to out_dtype as the
+ * unsplit projection rounds its result, then weighted and summed as above.  k <= 8, H % 8 == 0. */
+int ats_combine_partials(const float* parts, int n_parts, int64_t part_stride, const int32_t* row_of,
+                         const float* w, const void* residual, void* out, int64_t T, int k, int H,
+                         int out_dtype, ats_stream_t stream);
 
 /* ---- Mixture-of-Depths helpers -------------------------------------------
  * score[t] = x[t,:] . w[:] (+ bias[0]); optionally prob[t] = sigmoid(score/temperature)

@@ -324,6 +324,63 @@ def test_grouped_gateup_gather_small_and_huge_source(ops, gpu):
         del src
 
 
+@pytest.mark.parametrize("counts,H,I,S", [([19, 17, 0, 14, 17, 1, 17, 13], 512, 1024, 2), ([5, 48, 20], 256, 2048, 4),
+                                          ([33], 384, 4096, 8), ([1, 0, 2, 48], 128, 512, 1)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_grouped_down_split_along_k(ops, gpu, counts, H, I, S, dtype):
+    """Decode-size down projection cut into S slices of K: the partial results add up to the unsplit
+    product (float32: to rounding of the sum order; against the float64 product with the float bar), rows
+    outside the groups are never written, and the combine over partial results gives the same bits as
+    the combine over their rounded sum."""
+    print("case split k", counts, H, I, S, dtype, flush=True)
+    g = gen(61)
+    E, rows = len(counts), sum(counts)
+    h = (torch.randn(rows, I, generator=g) * 0.5).to(dtype)
+    wd = [(torch.randn(H, I, generator=g) * 0.05).to(dtype) for _ in range(E)]
+    off = np.concatenate([[0], np.cumsum(counts)]).astype(np.int32)
+    start = torch.tensor(off[:-1], dtype=torch.int32, device=gpu)
+    count = torch.tensor(counts, dtype=torch.int32, device=gpu)
+    wd_gpu = [w.to(gpu) for w in wd]
+    tab = ops.weight_pointer_table(wd_gpu)
+    parts = ops.grouped_down_splitk(h.to(gpu), tab, start, count, rows, H, I, S)
+    assert parts.shape == (S, rows, H) and parts.dtype == torch.float32
+    ref = torch.cat([h[off[e]:off[e + 1]].double() @ wd[e].double().T for e in range(E)])
+    y32 = ops.sum_partials(parts, torch.float32)
+    assert rel_err(y32, ref) <= (F32_TOL if dtype == torch.float32 else 1e-5)
+    unsplit = ops.grouped_down(h.to(gpu), tab, start, count, rows, H, I, out_dtype=torch.float32)
+    assert rel_err(y32, unsplit) <= 1e-5
+    y = ops.sum_partials(parts, dtype)
+    assert rel_err(y, ref) <= (F32_TOL if dtype == torch.float32 else BF16_TOL)
+    # combine: two choices per token drawn from the rows
+    T, k = 11, 2
+    row_of = torch.randint(-1, rows, (T * k,), generator=g, dtype=torch.int32)
+    for t in range(T):                                   # a token does not visit a row twice
+        if row_of[2 * t] == row_of[2 * t + 1]:
+            row_of[2 * t + 1] = -1
+    w = torch.rand(T, k, generator=g)
+    res = torch.randn(T, H, generator=g).to(dtype)
+    for residual in (None, res.to(gpu)):
+        a = ops.combine_partials(parts, row_of.to(gpu), w.to(gpu), T, k, dtype, residual=residual)
+        b = ops.combine(y, row_of.to(gpu), w.to(gpu), T, k, out_dtype=dtype, residual=residual)
+        assert same_bits(a, b)
+
+
+@pytest.mark.parametrize("T,N,K", [(1, 4096, 4096), (8, 1024, 2048), (48, 512, 1536), (17, 264, 1000), (64, 2048, 4096)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_linear_nt_few_rows(ops, gpu, T, N, K, dtype):
+    """A few rows against a whole weight matrix (decode): the K-sliced path and, where K does not slice
+    (1000 columns) or the rows exceed the weight-streaming tiles (64), the plain one."""
+    print("case linear few rows", T, N, K, dtype, flush=True)
+    g = gen(62)
+    x = torch.randn(T, K, generator=g).to(dtype)
+    w = (torch.randn(N, K, generator=g) * 0.05).to(dtype)
+    got = ops.linear_nt(x.to(gpu), w.to(gpu))
+    assert got.shape == (T, N) and got.dtype == dtype
+    assert rel_err(got, x.double() @ w.double().T) <= (F32_TOL if dtype == torch.float32 else BF16_TOL)
+    expect_split = T <= 48 and K % 128 == 0
+    assert (ops.down_k_splits(1, T, N, K, dtype) > 1) == expect_split
+
+
 # ------------------------------------------------------------------ whole layer
 def _layer_vs_oracle(A, gpu, name, capacity_mode, routing, tol, scale_tokens=None, overrides=None, temperature=1.0):
     from adaptivetrainingsystem_amd import workloads as W

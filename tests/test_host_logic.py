@@ -53,6 +53,15 @@ def test_argument_errors_return_codes_not_exits():
     assert lib.ats_attention_bwd(*([None] * 10), 1, 4, 2, 16, 8, 128, 0.1, None) == -1
     assert lib.ats_attention_bwd(*([None] * 10), 1, 4, 2, 16, 16, 32, 0.1, None) == -2
     assert lib.ats_attention_delta(None, None, None, 1, 4, 16, 80, None) == -2
+    # K slices: I must be k_splits whole slabs, and only weight-streaming sizes (<= 48 rows per expert)
+    one = ctypes.c_void_p(16)
+    assert lib.ats_grouped_down_splitk(one, one, one, one, one, 8, 128, 128, 4096, 14336, 3, 1, None) == -2
+    assert b"slices" in lib.ats_last_error_string()
+    assert lib.ats_grouped_down_splitk(one, one, one, one, one, 8, 4096, 4096, 4096, 14336, 2, 1, None) == -2
+    assert lib.ats_grouped_down_splitk(one, one, one, one, one, 8, 128, 128, 4096, 14336, 0, 1, None) == -1
+    assert lib.ats_sum_partials(one, 2, 10, one, 8, 1, None) == -1          # stride not a multiple of 4
+    assert lib.ats_sum_partials(None, 2, 16, None, 0, 1, None) == 0         # nothing to add
+    assert lib.ats_combine_partials(one, 2, 64, one, one, None, one, 4, 9, 64, 1, None) == -1   # k > 8
     assert lib.ats_route_topk_workspace(16384, 8) > 0
     assert lib.ats_dispatch_plan_workspace(16384, 2, 8) == (32768 // 256) * 8 * 4
 
