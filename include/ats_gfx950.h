@@ -147,7 +147,7 @@ int ats_grouped_gateup_swiglu(const void* a, int64_t a_num_rows, const int32_t* 
 int ats_grouped_down(const void* h, const void* const* w_d, void* y, const int32_t* row_start,
                      const int32_t* row_count, int E, int64_t max_rows, int H, int I, int dtype,
                      int y_dtype, ats_stream_t stream);
-/* The down projection of weight-streaming (decode) sizes, at most 48 rows per expert, split along
+/* The down projection of weight-streaming (decode) sizes, at most 256 rows per expert, split along
  * K so that enough workgroups stream the weights: slice s of expert e multiplies columns
  * [s*I/k_splits, (s+1)*I/k_splits) and writes float32 parts[s][row_start[e]+m][:H]
  * (parts: [k_splits, part_rows, H]).  The result is the sum over s, taken in slice order by

@@ -325,7 +325,7 @@ def test_grouped_gateup_gather_small_and_huge_source(ops, gpu):
 
 
 @pytest.mark.parametrize("counts,H,I,S", [([19, 17, 0, 14, 17, 1, 17, 13], 512, 1024, 2), ([5, 48, 20], 256, 2048, 4),
-                                          ([33], 384, 4096, 8), ([1, 0, 2, 48], 128, 512, 1)])
+                                          ([33], 384, 4096, 8), ([1, 0, 2, 48], 128, 512, 1), ([200, 3, 97], 256, 1024, 2)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_grouped_down_split_along_k(ops, gpu, counts, H, I, S, dtype):
     """Decode-size down projection cut into S slices of K: the partial results add up to the unsplit
@@ -365,11 +365,12 @@ def test_grouped_down_split_along_k(ops, gpu, counts, H, I, S, dtype):
         assert same_bits(a, b)
 
 
-@pytest.mark.parametrize("T,N,K", [(1, 4096, 4096), (8, 1024, 2048), (48, 512, 1536), (17, 264, 1000), (64, 2048, 4096)])
+@pytest.mark.parametrize("T,N,K", [(1, 4096, 4096), (8, 1024, 2048), (48, 512, 1536), (17, 264, 1000), (64, 2048, 4096),
+                                   (200, 1024, 2048), (300, 512, 1024)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_linear_nt_few_rows(ops, gpu, T, N, K, dtype):
-    """A few rows against a whole weight matrix (decode): the K-sliced path and, where K does not slice
-    (1000 columns) or the rows exceed the weight-streaming tiles (64), the plain one."""
+    """A few rows against a whole weight matrix (decode): the K-sliced path (several 32-row tiles from 33
+    rows on) and, where K does not slice (1000 columns) or there are more than 256 rows, the plain one."""
     print("case linear few rows", T, N, K, dtype, flush=True)
     g = gen(62)
     x = torch.randn(T, K, generator=g).to(dtype)
@@ -377,7 +378,7 @@ def test_linear_nt_few_rows(ops, gpu, T, N, K, dtype):
     got = ops.linear_nt(x.to(gpu), w.to(gpu))
     assert got.shape == (T, N) and got.dtype == dtype
     assert rel_err(got, x.double() @ w.double().T) <= (F32_TOL if dtype == torch.float32 else BF16_TOL)
-    expect_split = T <= 48 and K % 128 == 0
+    expect_split = T <= 256 and K % 128 == 0
     assert (ops.down_k_splits(1, T, N, K, dtype) > 1) == expect_split
 
 

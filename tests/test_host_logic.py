@@ -57,7 +57,7 @@ def test_argument_errors_return_codes_not_exits():
     one = ctypes.c_void_p(16)
     assert lib.ats_grouped_down_splitk(one, one, one, one, one, 8, 128, 128, 4096, 14336, 3, 1, None) == -2
     assert b"slices" in lib.ats_last_error_string()
-    assert lib.ats_grouped_down_splitk(one, one, one, one, one, 8, 4096, 4096, 4096, 14336, 2, 1, None) == -2
+    assert lib.ats_grouped_down_splitk(one, one, one, one, one, 8, 4096, 4096, 4096, 14336, 2, 1, None) == -2   # 512 rows per expert
     assert lib.ats_grouped_down_splitk(one, one, one, one, one, 8, 128, 128, 4096, 14336, 0, 1, None) == -1
     assert lib.ats_sum_partials(one, 2, 10, one, 8, 1, None) == -1          # stride not a multiple of 4
     assert lib.ats_sum_partials(None, 2, 16, None, 0, 1, None) == 0         # nothing to add
