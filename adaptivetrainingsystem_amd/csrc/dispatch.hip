@@ -334,13 +334,19 @@ template <typename TY, typename TO, int MAXK, bool PARTS = false>
 __global__ __launch_bounds__(256) void combine_vec_kernel(const TY* __restrict__ y, const int32_t* __restrict__ row_of,
                                                           const float* __restrict__ w,
                                                           const TO* __restrict__ residual, TO* __restrict__ out,
-                                                          int64_t T, int k, int H, int n_parts = 1,
-                                                          int64_t part_stride = 0) {
+                                                          int64_t T, int k, int H, int cols_per_wave,
+                                                          int n_parts = 1, int64_t part_stride = 0) {
     constexpr int V = 8;  // columns per lane per step (one 16-byte bf16 vector or two float vectors)
     const int lane = lane_id();
     const int64_t wave = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
     const int64_t nwaves = (int64_t)gridDim.x * (blockDim.x >> 6);
-    for (int64_t t = wave; t < T; t += nwaves) {
+    // a wave owns cols_per_wave columns of one token: the whole row when there are many tokens, a
+    // 512-column piece when there are few (decoding), so that a handful of tokens still fills the chip
+    const int pieces = (H + cols_per_wave - 1) / cols_per_wave;
+    for (int64_t item = wave; item < T * pieces; item += nwaves) {
+        const int64_t t = item / pieces;
+        const int h_first = (int)(item - t * pieces) * cols_per_wave;
+        const int h_end = min(H, h_first + cols_per_wave);
         int my_row = -1;
         float my_w = 0.f;
         if (lane < k) {
@@ -363,7 +369,7 @@ __global__ __launch_bounds__(256) void combine_vec_kernel(const TY* __restrict__
             wts[n] = __shfl(my_w, src, 64);
         }
 #pragma unroll 4
-        for (int h0 = lane * V; h0 < H; h0 += kWave * V) {
+        for (int h0 = h_first + lane * V; h0 < h_end; h0 += kWave * V) {
             float acc[V];
 #pragma unroll
             for (int j = 0; j < V; ++j) acc[j] = 0.f;
@@ -425,10 +431,15 @@ __global__ __launch_bounds__(256) void combine_vec_kernel(const TY* __restrict__
     }
 }
 
+// Columns of a token that one wave combines: the row for many tokens, 512-column pieces (one step of
+// 64 lanes x 8 columns) for few.
+static int combine_cols_per_wave(int64_t T, int H) { return T >= 4096 || H <= 512 ? H : 512; }
+
 template <typename TY, typename TO>
 static void launch_combine(const void* y, const int32_t* row_of, const float* w, const void* residual, void* out,
                            int64_t T, int k, int H, hipStream_t s) {
-    int64_t blocks = (T + 3) / 4;
+    const int cols = combine_cols_per_wave(T, H);
+    int64_t blocks = (T * ((H + cols - 1) / cols) + 3) / 4;
     if (blocks > 16384) blocks = 16384;
     const TY* yp = static_cast<const TY*>(y);
     const TO* rp = static_cast<const TO*>(residual);
@@ -436,13 +447,13 @@ static void launch_combine(const void* y, const int32_t* row_of, const float* w,
     const bool vec = H % 8 == 0 && aligned16(y) && aligned16(out) && (!residual || aligned16(residual)) && k <= 8;
     if (vec && k <= 2)
         hipLaunchKernelGGL((combine_vec_kernel<TY, TO, 2>), dim3((unsigned)blocks), dim3(256), 0, s, yp, row_of, w, rp,
-                           op, T, k, H);
+                           op, T, k, H, cols);
     else if (vec && k <= 4)
         hipLaunchKernelGGL((combine_vec_kernel<TY, TO, 4>), dim3((unsigned)blocks), dim3(256), 0, s, yp, row_of, w, rp,
-                           op, T, k, H);
+                           op, T, k, H, cols);
     else if (vec)
         hipLaunchKernelGGL((combine_vec_kernel<TY, TO, 8>), dim3((unsigned)blocks), dim3(256), 0, s, yp, row_of, w, rp,
-                           op, T, k, H);
+                           op, T, k, H, cols);
     else
         hipLaunchKernelGGL((combine_kernel<TY, TO>), dim3((unsigned)blocks), dim3(256), 0, s, yp, row_of, w, rp, op, T,
                            k, H);
@@ -510,12 +521,13 @@ extern "C" int ats_combine_partials(const float* parts, int n_parts, int64_t par
     if (T == 0) return ATS_OK;
     ATS_REQUIRE(parts && row_of && w && out && aligned16(parts) && aligned16(out) && (!residual || aligned16(residual)),
                 ATS_ERR_INVALID_ARG, "%s: null or misaligned pointer", name);
-    int64_t blocks = (T + 3) / 4;
+    const int cols = combine_cols_per_wave(T, H);
+    int64_t blocks = (T * ((H + cols - 1) / cols) + 3) / 4;
     if (blocks > 16384) blocks = 16384;
     hipStream_t s = as_stream(stream);
 #define ATS_COMBINE_PARTS(TO_, MAXK_)                                                                              \
     hipLaunchKernelGGL((combine_vec_kernel<float, TO_, MAXK_, true>), dim3((unsigned)blocks), dim3(256), 0, s, parts, \
-                       row_of, w, static_cast<const TO_*>(residual), static_cast<TO_*>(out), T, k, H, n_parts,       \
+                       row_of, w, static_cast<const TO_*>(residual), static_cast<TO_*>(out), T, k, H, cols, n_parts, \
                        part_stride)
     if (out_dtype == ATS_F32) {
         if (k <= 2) ATS_COMBINE_PARTS(float, 2);
