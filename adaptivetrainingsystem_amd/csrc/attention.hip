@@ -52,6 +52,7 @@ __device__ __forceinline__ af32x16_t att_mma(const au32x4_t& a, const au32x4_t& 
 // positions (decoding against a cache: one position, rep rows instead of one).
 template <int D, bool BIAS>
 __device__ __forceinline__ void attention_q_tile(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
+                                                 int64_t k_sb, int64_t k_sh,
                                                  const bf16_t* __restrict__ v, int64_t v_sb, int v_sl, int64_t v_sh,
                                                  const float* __restrict__ key_bias, bf16_t* __restrict__ out,
                                                  float* __restrict__ lse, int Hq, int Hkv, int L, int Lk,
@@ -89,7 +90,7 @@ __device__ __forceinline__ void attention_q_tile(const bf16_t* __restrict__ q, c
     const bool row_valid = row < n_rows;
 
     const bf16_t* qp = q + ((int64_t)(b * Hq + hq) * L + q_clamped) * D;
-    const bf16_t* kbase = k + (int64_t)(b * Hkv + hkv) * Lk * D;
+    const bf16_t* kbase = k + b * k_sb + hkv * k_sh;          // rows of D elements, one after the other
     const bf16_t* vbase = v + b * v_sb + hkv * v_sh;          // row of key j at vbase + j * v_sl
 
     au32x4_t qf[KS];
@@ -350,6 +351,7 @@ __device__ __forceinline__ void attention_q_tile(const bf16_t* __restrict__ q, c
 // in the shadow of the other's MFMAs.
 template <int D, bool BIAS>
 __global__ __launch_bounds__(kAttThreads, 512 / kAttThreads) void attention_fwd_kernel(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
+                                                            int64_t k_sb, int64_t k_sh,
                                                             const bf16_t* __restrict__ v, int64_t v_sb, int v_sl, int64_t v_sh,
                                                             const float* __restrict__ key_bias, bf16_t* __restrict__ out,
                                                             float* __restrict__ lse, int Hq, int Hkv, int L, int Lk,
@@ -376,15 +378,15 @@ __global__ __launch_bounds__(kAttThreads, 512 / kAttThreads) void attention_fwd_
 #pragma unroll 1
     for (int half = 0; half < 2; ++half) {
         if (half && pair == qt_long) break;   // an odd tile count leaves the middle tile on its own
-        attention_q_tile<D, BIAS>(q, k, v, v_sb, v_sl, v_sh, key_bias, out, lse, Hq, Hkv, L, Lk, scale_log2,
+        attention_q_tile<D, BIAS>(q, k, k_sb, k_sh, v, v_sb, v_sl, v_sh, key_bias, out, lse, Hq, Hkv, L, Lk, scale_log2,
                             half ? pair : qt_long, head, b, pack != 0, smem);
     }
 }
 
 }  // namespace ats
 
-extern "C" int ats_attention_fwd(const void* q, const void* k, const void* v, int64_t v_sb, int64_t v_sl, int64_t v_sh,
-                                 const float* key_bias, void* out, float* lse, int B, int Hq, int Hkv, int L, int Lk,
+extern "C" int ats_attention_fwd(const void* q, const void* k, int64_t k_sb, int64_t k_sh, const void* v, int64_t v_sb,
+                                 int64_t v_sl, int64_t v_sh, const float* key_bias, void* out, float* lse, int B, int Hq, int Hkv, int L, int Lk,
                                  int D, float scale, ats_stream_t stream) {
     using namespace ats;
     ATS_REQUIRE(B >= 0 && Hq > 0 && Hkv > 0 && Hq % Hkv == 0 && L >= 0 && Lk >= L && scale > 0.f, ATS_ERR_INVALID_ARG,
@@ -393,6 +395,9 @@ extern "C" int ats_attention_fwd(const void* q, const void* k, const void* v, in
     if (B == 0 || L == 0) return ATS_OK;
     ATS_REQUIRE(q && k && v && out && aligned16(q) && aligned16(k) && aligned16(v) && aligned16(out),
                 ATS_ERR_INVALID_ARG, "ats_attention_fwd: null or misaligned pointer");
+    ATS_REQUIRE(k_sb % 8 == 0 && k_sh % 8 == 0 && k_sb >= 0 && k_sh >= 0, ATS_ERR_INVALID_ARG,
+                "ats_attention_fwd: batch and head strides of k (%lld, %lld) must be multiples of 8 elements",
+                (long long)k_sb, (long long)k_sh);
     ATS_REQUIRE(v_sl >= D && v_sl % 8 == 0 && v_sb % 8 == 0 && v_sh % 8 == 0 && v_sb >= 0 && v_sh >= 0, ATS_ERR_INVALID_ARG,
                 "ats_attention_fwd: strides of v (%lld, %lld, %lld) must be multiples of 8 elements, rows apart",
                 (long long)v_sb, (long long)v_sl, (long long)v_sh);
@@ -413,7 +418,8 @@ extern "C" int ats_attention_fwd(const void* q, const void* k, const void* v, in
                         hipGetErrorString(e));
         }
         hipLaunchKernelGGL(kernel, grid, dim3(kAttThreads), smem, as_stream(stream), static_cast<const bf16_t*>(q),
-                           static_cast<const bf16_t*>(k), static_cast<const bf16_t*>(v), v_sb, (int)v_sl, v_sh, key_bias,
+                           static_cast<const bf16_t*>(k), k_sb, k_sh, static_cast<const bf16_t*>(v), v_sb, (int)v_sl, v_sh,
+                           key_bias,
                            static_cast<bf16_t*>(out), lse, Hq, Hkv, L, Lk, scale_log2, B, pack);
         return ATS_OK;
     };

@@ -182,6 +182,9 @@ class GroupedQueryAttention(nn.Module):
         nn.init.normal_(self.o_proj.weight, mean=0.0, std=std * gain / math.sqrt(2 * getattr(config, "num_layers", 1)))
         self._param_count = sum(p.numel() for p in self.parameters())
         self._calls = 0
+        self._kv_buffer = None       # addresses and fill of the cache buffers handed out last (no tensor is held)
+        self._qkv_key = None
+        self._qkv = None
 
     def forward(self, x: torch.Tensor, attention_mask: Optional[torch.Tensor] = None, past_key_value=None,
                 use_cache: bool = False):
@@ -192,14 +195,21 @@ class GroupedQueryAttention(nn.Module):
         B, L, H = x.shape
         nh, nkv, D = self.num_heads, self.num_kv_heads, self.head_dim
         x2 = x.reshape(B * L, H).contiguous()
-        grad = _wants_grad(x, *self.parameters())
+        grad = torch.is_grad_enabled() and _wants_grad(x, self.q_proj.weight, self.k_proj.weight, self.v_proj.weight,
+                                                       self.o_proj.weight)
         if grad:
             lin = ag.LinearFunction.apply
+            q = lin(x2, self.q_proj.weight).view(B, L, nh, D).transpose(1, 2)
+            k = lin(x2, self.k_proj.weight).view(B, L, nkv, D).transpose(1, 2)
+            v = lin(x2, self.v_proj.weight).view(B, L, nkv, D).transpose(1, 2)
         else:
+            # one product with the three weights stacked (a copy kept until a weight changes): a third of the
+            # launches, which is what a decoding step is made of; q, k, v are column ranges of its output
             lin = lambda a, w: ops.linear_nt(a, _as_dtype(w, a.dtype))
-        q = lin(x2, self.q_proj.weight).view(B, L, nh, D).transpose(1, 2)
-        k = lin(x2, self.k_proj.weight).view(B, L, nkv, D).transpose(1, 2)
-        v = lin(x2, self.v_proj.weight).view(B, L, nkv, D).transpose(1, 2)
+            qkv = ops.linear_nt(x2, self._stacked_qkv(x.dtype))
+            q = qkv[:, :nh * D].view(B, L, nh, D).transpose(1, 2)
+            k = qkv[:, nh * D:(nh + nkv) * D].view(B, L, nkv, D).transpose(1, 2)
+            v = qkv[:, (nh + nkv) * D:].view(B, L, nkv, D).transpose(1, 2)
         # positions 0..L-1 also when a cache is passed, as the reference does (model.py:690-698)
         cos, sin = self.rope(L, x.device)
         q, k = ag.RoPEFunction.apply(q, k, cos, sin, 0) if grad else ops.rope(q, k, cos, sin, 0)
@@ -208,8 +218,11 @@ class GroupedQueryAttention(nn.Module):
             if (k_cache.dim() != 4 or k_cache.shape[0] != B or k_cache.shape[1] != nkv or k_cache.shape[3] != D
                     or v_cache.shape != k_cache.shape):
                 raise AtsError(f"GroupedQueryAttention: cache shapes {tuple(k_cache.shape)} / {tuple(v_cache.shape)}")
-            k = torch.cat([k_cache.to(k.dtype), k], dim=2)
-            v = torch.cat([v_cache.to(v.dtype), v], dim=2)
+            if use_cache and not grad:
+                k, v = self._extend_cache(k_cache, v_cache, k, v)
+            else:
+                k = torch.cat([k_cache.to(k.dtype), k], dim=2)
+                v = torch.cat([v_cache.to(v.dtype), v], dim=2)
         key_bias = None
         if attention_mask is not None:
             # [batch, keys] with 1 = real token, 0 = padding: (1 - mask) * -1e4 on that key's scores for
@@ -225,8 +238,51 @@ class GroupedQueryAttention(nn.Module):
         out = lin(a.view(B * L, nh * D), self.o_proj.weight).view(B, L, H)    # a: [B, L, nh*D]
         self._calls += 1
         if use_cache:
-            return out, (k, v.contiguous())
+            return out, (k, v if v.stride(3) == 1 and v.stride(2) == D else v.contiguous())
         return out
+
+    def _stacked_qkv(self, dtype: torch.dtype) -> torch.Tensor:
+        """[q_proj; k_proj; v_proj] weights as one [(nh + 2 nkv) * D, hidden] matrix in the compute dtype, rebuilt
+        when a weight is replaced or written to (the parameters themselves stay as the reference has them)."""
+        ws = (self.q_proj.weight, self.k_proj.weight, self.v_proj.weight)
+        key = (dtype,) + tuple((w.data_ptr(), w._version) for w in ws)
+        if self._qkv_key != key:
+            with torch.no_grad():
+                self._qkv = torch.cat([w.detach().to(dtype) for w in ws], dim=0).contiguous()
+            self._qkv_key = key
+        return self._qkv
+
+    def _extend_cache(self, k_cache, v_cache, k_new, v_new):
+        """The cache followed by the new rows, as the reference's torch.cat gives them (model.py:700-704), without
+        copying the cache on every step: the tensors handed back are the first rows of buffers
+        [batch, kv heads, capacity, head_dim] with room to grow, and when the same tensors come back as
+        past_key_value the new rows are written behind them in place.  Only the latest state is extended in
+        place (its length must be the buffer's fill), so continuing twice from one cache copies as cat does;
+        any other cache tensor is copied into a fresh buffer whose capacity is 1.5 x the new length."""
+        B, nkv, Lp, D = k_cache.shape
+        L = k_new.shape[2]
+        st = self._kv_buffer
+        cap_strides = lambda cap: (nkv * cap * D, cap * D, D, 1)
+        if (st is not None and Lp == st["length"] and Lp + L <= st["capacity"]
+                and k_cache.dtype == k_new.dtype and v_cache.dtype == v_new.dtype
+                and k_cache.data_ptr() == st["k_ptr"] and v_cache.data_ptr() == st["v_ptr"]
+                and k_cache.stride() == cap_strides(st["capacity"]) and v_cache.stride() == cap_strides(st["capacity"])
+                and k_cache.untyped_storage().nbytes() >= st["nbytes"]
+                and v_cache.untyped_storage().nbytes() >= st["nbytes"]):
+            cap = st["capacity"]
+            k_buf = k_cache.as_strided((B, nkv, cap, D), cap_strides(cap))
+            v_buf = v_cache.as_strided((B, nkv, cap, D), cap_strides(cap))
+        else:
+            cap = Lp + L + max(64, (Lp + L) // 2)
+            k_buf = torch.empty(B, nkv, cap, D, dtype=k_new.dtype, device=k_new.device)
+            v_buf = torch.empty(B, nkv, cap, D, dtype=v_new.dtype, device=v_new.device)
+            k_buf[:, :, :Lp].copy_(k_cache)
+            v_buf[:, :, :Lp].copy_(v_cache)
+        k_buf[:, :, Lp:Lp + L].copy_(k_new)
+        v_buf[:, :, Lp:Lp + L].copy_(v_new)
+        self._kv_buffer = {"k_ptr": k_buf.data_ptr(), "v_ptr": v_buf.data_ptr(), "capacity": cap, "length": Lp + L,
+                           "nbytes": k_buf.numel() * k_buf.element_size()}
+        return k_buf[:, :, :Lp + L], v_buf[:, :, :Lp + L]
 
     def get_attention_stats(self) -> Dict[str, Any]:
         return {"total_calls": self._calls, "flash_attention_calls": self._calls, "standard_attention_calls": 0,

@@ -30,7 +30,15 @@ def _need_gpu(*tensors: Optional[torch.Tensor]) -> None:
             raise AtsError("tensor is not on the GPU: the gfx950 path has no CPU fallback")
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+_raw_device = getattr(torch._C, "_cuda_getDevice", None)
+
+
 def _stream() -> int:
+    """Handle of torch's current stream on the current device.  The raw accessors skip the Stream object
+    and the device bookkeeping of torch.cuda.current_stream (8 us a call, a tenth of a decode step)."""
+    if _raw_stream is not None and _raw_device is not None:
+        return _raw_stream(_raw_device())
     return torch.cuda.current_stream().cuda_stream
 
 
@@ -657,8 +665,9 @@ def _key_bias(key_bias, B: int, Lk: int, q: torch.Tensor, who: str):
 
 def causal_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: Optional[float] = None,
                      return_lse: bool = False, key_bias: Optional[torch.Tensor] = None):
-    """Causal grouped-query attention.  q [B,Hq,L,D], k [B,Hkv,Lk,D] (made contiguous), v [B,Hkv,Lk,D] in any
-    batch/head/position strides (e.g. a view of a fused projection output); bf16, D 64 or 128, Lk >= L.
+    """Causal grouped-query attention.  q [B,Hq,L,D]; k [B,Hkv,Lk,D] with a head's rows one after the other
+    and any batch/head strides (e.g. a view of a larger cache buffer); v [B,Hkv,Lk,D] in any batch/head/position
+    strides (e.g. a view of a fused projection output); bf16, D 64 or 128, Lk >= L.
     With Lk > L the leading Lk - L keys are a cache: query i sits at position i + Lk - L.
     key_bias [B, Lk] float32 (optional) is added to the scaled scores of a key for every query and head;
     (1 - attention_mask) * -1e4 is the reference's padding mask (MS/core/model.py:819-824).
@@ -670,14 +679,17 @@ def causal_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: O
     Hkv, Lk = k.shape[1], k.shape[2]
     if k.shape != (B, Hkv, Lk, D) or v.shape != (B, Hkv, Lk, D) or Hq % Hkv != 0 or Lk < L:
         raise AtsError(f"causal_attention: shapes q {tuple(q.shape)} k {tuple(k.shape)} v {tuple(v.shape)}")
-    q, k = q.contiguous(), k.contiguous()
+    q = q.contiguous()
+    if k.stride(3) != 1 or k.stride(2) != D or k.stride(0) % 8 or k.stride(1) % 8 or k.data_ptr() % 16:
+        k = k.contiguous()        # rows of a head must follow one another; batch and head strides are free
     key_bias = _key_bias(key_bias, B, Lk, q, "causal_attention")
     if v.stride(3) != 1 or any(st % 8 for st in v.stride()[:3]) or v.stride(2) < D or v.data_ptr() % 16:
         v = v.contiguous()
     lib = _lib.load()
     out = torch.empty(B, L, Hq * D, dtype=q.dtype, device=q.device)
     lse = torch.empty(B, Hq, L, dtype=torch.float32, device=q.device) if return_lse else None
-    check(lib.ats_attention_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), v.stride(0), v.stride(2), v.stride(1),
+    check(lib.ats_attention_fwd(q.data_ptr(), k.data_ptr(), k.stride(0), k.stride(1), v.data_ptr(), v.stride(0),
+                                v.stride(2), v.stride(1),
                                 _ptr(key_bias), out.data_ptr(), _ptr(lse), B, Hq, Hkv, L, Lk, D,
                                 float(D ** -0.5 if scale is None else scale), _stream()), "ats_attention_fwd")
     return (out, lse) if return_lse else out

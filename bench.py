@@ -568,6 +568,71 @@ def run_gqa_layer(args):
     return result
 
 
+def run_gqa_decode(args):
+    """Decoding steps of the attention sub-layer of the headline model shape (hidden 4096, 32 query / 8 kv heads,
+    head_dim 128): 64 sequences, one new token each, starting from 2048 cached keys; every step feeds the cache
+    the previous one returned (q/k/v projections of 64 rows, RoPE, cache append, attention, output projection)."""
+    import adaptivetrainingsystem_amd as A
+    from adaptivetrainingsystem_amd.workloads import LayerConfig
+    dev = torch.device("cuda:0")
+    B, L0, H, Hq, Hkv = 64, 2048, 4096, 32, 8
+    D = H // Hq
+    torch.manual_seed(11)
+    cfg = LayerConfig(H, 14336, 8, 2, num_heads=Hq, num_kv_heads=Hkv, seq_length=8192)
+    att = A.GroupedQueryAttention(cfg).to(torch.bfloat16).to(dev).eval()
+    xs = torch.randn(8, B, 1, H, device=dev).bfloat16()
+
+    def fresh_cache():
+        return (torch.randn(B, Hkv, L0, D, device=dev).bfloat16(), torch.randn(B, Hkv, L0, D, device=dev).bfloat16())
+
+    with torch.no_grad():
+        cache = fresh_cache()
+        for i in range(args.warmup):
+            _, cache = att(xs[i % 8], past_key_value=cache, use_cache=True)
+        cache = fresh_cache()
+        _, cache = att(xs[0], past_key_value=cache, use_cache=True)       # moves the cache into a buffer with room
+        torch.cuda.synchronize()
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        ev0.record()
+        for i in range(args.steps):
+            _, cache = att(xs[i % 8], past_key_value=cache, use_cache=True)
+        ev1.record()
+        torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    gpu_ms = ev0.elapsed_time(ev1) / args.steps
+    keys_mid = L0 + 1 + args.steps / 2.0
+    # a step streams the four projection weights once and the filled part of the cache once
+    weight_bytes = 2.0 * H * (Hq * D + 2 * Hkv * D + H)
+    cache_bytes = 2.0 * B * Hkv * keys_mid * D * 2
+    achieved = (weight_bytes + cache_bytes) / (gpu_ms * 1e-3) / 1e9
+    log(f"  attention sub-layer decode step {gpu_ms * 1e3:.1f} us (host clock {dt / args.steps * 1e6:.1f} us) -> "
+        f"{achieved:.0f} GB/s of weights + cache ({achieved / PEAK_HBM_GBS:.1%} of the HBM peak)")
+    result = {
+        "metric": "GQA attention sub-layer decode tokens/s", "value": B * args.steps / dt, "unit": "tokens/s", "n_gpus": 1,
+        "steps": args.steps, "warmup": args.warmup, "ms_per_step": dt / args.steps * 1e3, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"gqa_decode: q/k/v/o projections + RoPE + cache append + attention, {B} sequences x 1 new "
+                               f"token, {L0} cached keys growing by one per step, hidden {H}, {Hq} query / {Hkv} kv heads"},
+        "roofline": {"kernel": "whole sub-layer step (4 K-sliced projections + attention_fwd_kernel, packed rows)",
+                     "bound": "hbm", "achieved": achieved, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": achieved / PEAK_HBM_GBS, "traffic": None},
+        "stages_ms": {"gqa_decode_step": round(gpu_ms, 4)},
+    }
+    if not args.no_cpu_baseline:
+        from oracle import sparse_layer_oracle as O
+        w = [getattr(att, n).weight.detach().float().cpu() for n in ("q_proj", "k_proj", "v_proj", "o_proj")]
+        n = 8
+        kc, vc = (t[:n, :, :L0].float().cpu() for t in cache)
+        xc = xs[0][:n].float().cpu()
+        t0 = time.perf_counter()
+        O.gqa_forward(xc, *w, Hq, Hkv, past_key_value=(kc, vc), use_cache=True)
+        cdt = time.perf_counter() - t0
+        result["cpu_baseline"] = {"value": n / cdt, "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
+                                  "sample": f"{n} of the {B} sequences, float32, one step ({cdt:.2f} s)"}
+    return result
+
+
 def run_norm_rope(args):
     """Config 2: RMSNorm over x[8192, 2048] and RoPE over q[4,16,2048,128], k[4,4,2048,128], bf16."""
     from adaptivetrainingsystem_amd import ops
@@ -661,7 +726,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="c4_prefill",
                     choices=["c4_prefill", "c3_decode", "c5_finegrained_mod", "c1_cpu_reference", "c2_norm_rope",
-                             "c4_prefill_train", "c1_cpu_reference_train", "loss_clip", "attention", "attention_train", "attention_decode", "gqa_layer", "block_train"])
+                             "c4_prefill_train", "c1_cpu_reference_train", "loss_clip", "attention", "attention_train", "attention_decode", "gqa_layer", "gqa_decode", "block_train"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a 1 GiB device copy (known traffic) so hardware-counter runs can be scaled")
@@ -698,6 +763,8 @@ def main():
         result = run_attention_decode(args)
     elif args.workload == "gqa_layer":
         result = run_gqa_layer(args)
+    elif args.workload == "gqa_decode":
+        result = run_gqa_decode(args)
     elif args.workload.endswith("_train"):
         result = run_train(args)
     else:

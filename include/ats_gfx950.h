@@ -284,18 +284,20 @@ int ats_grouped_gemm_nt(const void* a, const void* const* a_ptrs, int64_t lda, i
  * (Src/Main_Scripts/core/model.py:757-839): softmax(q.k^T * scale + causal mask) . v with float32
  * scores and softmax, probabilities rounded to bf16, output laid out [B, L, Hq*D] (the layout o_proj
  * consumes).  bf16 only, D = 64 or 128, Hq a multiple of Hkv (query head h reads kv head h / (Hq/Hkv)).
- * q: [B,Hq,L,D], k: [B,Hkv,Lk,D] contiguous, Lk >= L; v: rows of D contiguous elements addressed as
- * base + b*v_sb + j*v_sl + h*v_sh (element strides, multiples of 8), so a [B,Hkv,Lk,D] tensor or a view
- * of a fused projection output [B,Lk,Hkv,D] is read in place.  With Lk > L the first Lk - L keys are a
+ * q: [B,Hq,L,D] contiguous; k: the Lk rows of a (batch, head) follow one another (D elements each) from
+ * base + b*k_sb + h*k_sh, so a [B,Hkv,Lk,D] tensor or the first Lk rows of a larger cache buffer
+ * [B,Hkv,capacity,D] is read in place; Lk >= L; v: rows of D contiguous elements addressed as
+ * base + b*v_sb + j*v_sl + h*v_sh, so a [B,Hkv,Lk,D] tensor, a cache buffer or a view of a fused
+ * projection output [B,Lk,Hkv,D] is read in place (element strides, multiples of 8).  With Lk > L the first Lk - L keys are a
  * cache in front of the queries (model.py:700-704): query i sits at position i + Lk - L and sees keys up
  * to there.  The reference's masked path only runs that case for L = 1 (its [L, L] mask does not
  * broadcast otherwise); its flash path aligns the diagonal the same way.
  * key_bias (optional): [B,Lk] float32 added to the scaled scores of a key for every query and head; the
  * reference's padding mask is (1 - attention_mask) * -1e4 (model.py:819-824).
  * lse (optional): [B,Hq,L] float32 log-sum-exp of the scaled (and biased) scores per query. */
-int ats_attention_fwd(const void* q, const void* k, const void* v, int64_t v_sb, int64_t v_sl, int64_t v_sh,
-                      const float* key_bias, void* out, float* lse, int B, int Hq, int Hkv, int L, int Lk, int D,
-                      float scale, ats_stream_t stream);
+int ats_attention_fwd(const void* q, const void* k, int64_t k_sb, int64_t k_sh, const void* v, int64_t v_sb,
+                      int64_t v_sl, int64_t v_sh, const float* key_bias, void* out, float* lse, int B, int Hq,
+                      int Hkv, int L, int Lk, int D, float scale, ats_stream_t stream);
 
 /* ---- Causal grouped-query attention (backward) ----------------------------------
  * The reference leaves this gradient to autograd (model.py:757-839 under torch.autograd); the kernels

@@ -119,6 +119,16 @@ def test_gqa_module(gpu, hidden, nh, nkv, B, L):
         out = att(x.to(gpu))
     assert out.shape == x.shape and rel_err(out, ref) <= BF16_TOL
     assert set(att.state_dict()) == {f"{n}.weight" for n in ("q_proj", "k_proj", "v_proj", "o_proj")}
+    # the stacked q/k/v weight of the inference path follows in-place updates and replaced parameters
+    with torch.no_grad():
+        att.k_proj.weight.mul_(0.5)
+        w_k = att.k_proj.weight.detach().cpu()
+        ref2 = O.gqa_forward(x, att.q_proj.weight.detach().cpu(), w_k, att.v_proj.weight.detach().cpu(),
+                             att.o_proj.weight.detach().cpu(), nh, nkv)
+        out2 = att(x.to(gpu))
+        assert rel_err(out2, ref2) <= BF16_TOL and not torch.equal(out2, out)
+        att.k_proj.weight = torch.nn.Parameter(att.k_proj.weight.detach() * 2.0)
+        assert torch.equal(att(x.to(gpu)), out)
     # prefill with use_cache, then two single-token steps fed from the cache (model.py:700-708)
     w = [getattr(att, n).weight.detach().cpu() for n in ("q_proj", "k_proj", "v_proj", "o_proj")]
     with torch.no_grad():
@@ -231,6 +241,60 @@ def test_gqa_module_backward(gpu, hidden, nh, nkv, B, L):
 
 
 # --------------------------------------------------------------------------- the whole block
+def test_gqa_module_cache_grows_in_place(gpu):
+    """Decoding step after step: the cache handed back is the head of a buffer with room to grow, the next
+    step writes its rows behind it without copying, and outputs and cache contents equal what concatenation
+    gives (model.py:700-704).  Continuing twice from one cache, or from an older one, copies instead and
+    leaves the other continuation's cache alone."""
+    import adaptivetrainingsystem_amd as A
+    from adaptivetrainingsystem_amd.workloads import LayerConfig
+    hidden, nh, nkv, B, L = 512, 4, 2, 3, 70
+    D = hidden // nh
+    torch.manual_seed(16)
+    att = A.GroupedQueryAttention(LayerConfig(hidden, 4 * hidden, 1, 1, num_heads=nh, num_kv_heads=nkv, seq_length=512))
+    with torch.no_grad():
+        for p in att.parameters():
+            p.mul_(20.0)
+    att = att.to(torch.bfloat16).to(gpu).eval()
+    w = [getattr(att, n).weight.detach().cpu() for n in ("q_proj", "k_proj", "v_proj", "o_proj")]
+    x = torch.randn(B, L, hidden, generator=gen(120)).bfloat16()
+    with torch.no_grad():
+        _, cache = att(x.to(gpu), use_cache=True)
+    _, ref_cache = O.gqa_forward(x, *w, nh, nkv, use_cache=True)
+    ptrs = set()
+    for step in range(6):
+        x1 = torch.randn(B, 1, hidden, generator=gen(121 + step)).bfloat16()
+        with torch.no_grad():
+            plain = att(x1.to(gpu), past_key_value=cache)                    # concatenating path, no cache back
+            o1, new_cache = att(x1.to(gpu), past_key_value=cache, use_cache=True)
+        r1, ref_cache = O.gqa_forward(x1, *w, nh, nkv, past_key_value=ref_cache, use_cache=True)
+        assert torch.equal(o1, plain) and rel_err(o1, r1) <= BF16_TOL
+        assert new_cache[0].shape == (B, nkv, L + 1 + step, D) and new_cache[1].shape == new_cache[0].shape
+        assert rel_err(new_cache[0], ref_cache[0]) <= BF16_TOL and rel_err(new_cache[1], ref_cache[1]) <= BF16_TOL
+        assert torch.equal(new_cache[0][:, :, :L + step], cache[0]) and torch.equal(new_cache[1][:, :, :L + step], cache[1])
+        cache = new_cache
+        ptrs.add((cache[0].data_ptr(), cache[1].data_ptr()))
+    assert len(ptrs) == 1                         # one buffer pair served all six steps
+    # two continuations from the same state: the second one must not disturb the first one's new row
+    xa = torch.randn(B, 1, hidden, generator=gen(130)).bfloat16().to(gpu)
+    xb = torch.randn(B, 1, hidden, generator=gen(131)).bfloat16().to(gpu)
+    with torch.no_grad():
+        oa, cache_a = att(xa, past_key_value=cache, use_cache=True)
+        keep_a = [t.clone() for t in cache_a]
+        ob, cache_b = att(xb, past_key_value=cache, use_cache=True)
+        oa2 = att(xa, past_key_value=cache)
+        ob2 = att(xb, past_key_value=cache)
+    assert torch.equal(cache_a[0], keep_a[0]) and torch.equal(cache_a[1], keep_a[1])
+    assert torch.equal(oa, oa2) and torch.equal(ob, ob2) and not torch.equal(oa, ob)
+    assert cache_b[0].data_ptr() != cache_a[0].data_ptr()
+    # a chunk of several tokens on top of a cache, float32 cache tensors converted on the way in
+    x4 = torch.randn(B, 4, hidden, generator=gen(132)).bfloat16().to(gpu)
+    with torch.no_grad():
+        o4, c4 = att(x4, past_key_value=(cache_b[0].float(), cache_b[1].float()), use_cache=True)
+        o4_plain = att(x4, past_key_value=cache_b)
+    assert torch.equal(o4, o4_plain) and c4[0].shape[2] == cache_b[0].shape[2] + 4 and c4[0].dtype == torch.bfloat16
+
+
 # --------------------------------------------------------------------------- padding mask
 def _padding_mask(B, Lk, seed, left=0):
     """Right padding of a different length per batch entry (every query keeps a real key in view),
