@@ -28,7 +28,8 @@ def ops(gpu):
 
 
 @pytest.mark.parametrize("B,Hq,Hkv,L,D", [(1, 2, 1, 64, 128), (2, 4, 2, 200, 128), (1, 8, 2, 513, 64), (1, 1, 1, 1, 128),
-                                          (2, 3, 3, 129, 64), (1, 4, 1, 1024, 128), (1, 2, 2, 31, 64)])
+                                          (2, 3, 3, 129, 64), (1, 4, 1, 1024, 128), (1, 2, 2, 31, 64),
+                                          (1, 2, 1, 4100, 64), (1, 1, 1, 4300, 128)])      # 8-wave blocks from 4096 on
 def test_causal_attention(ops, gpu, B, Hq, Hkv, L, D):
     print("case attention", B, Hq, Hkv, L, D, flush=True)
     g = gen(91)
@@ -310,7 +311,7 @@ def _padding_mask(B, Lk, seed, left=0):
 
 @pytest.mark.parametrize("B,Hq,Hkv,L,Lk,D", [(2, 4, 2, 200, 200, 128), (3, 8, 2, 300, 300, 64), (1, 1, 1, 1, 1, 128),
                                              (2, 2, 2, 129, 129, 64), (2, 4, 1, 520, 520, 128), (2, 4, 2, 70, 300, 64),
-                                             (3, 32, 8, 1, 513, 128), (2, 2, 1, 31, 31, 64)])
+                                             (3, 32, 8, 1, 513, 128), (2, 2, 1, 31, 31, 64), (1, 2, 1, 4099, 4200, 128)])
 def test_causal_attention_padding_mask(ops, gpu, B, Hq, Hkv, L, Lk, D):
     """Forward and backward with (1 - mask) * -1e4 on the keys, against the oracle and autograd over it."""
     print("case attention padding mask", B, Hq, Hkv, L, Lk, D, flush=True)
