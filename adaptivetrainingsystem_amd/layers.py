@@ -153,10 +153,10 @@ class GroupedQueryAttention(nn.Module):
     """Causal grouped-query attention with the reference's constructor fields, parameter names
     (q_proj / k_proj / v_proj / o_proj, no bias) and forward(x [B, L, hidden]) -> [B, L, hidden]
     (MS/core/model.py:561-731).  Projections run through the grouped GEMM kernels (one group), RoPE and the
-    attention itself through their HIP kernels; the score matrix is never materialised.
-
-    Not built yet (raise AtsError): extra attention masks, KV cache, dropout, gradients (forward only),
-    float32 inputs."""
+    attention itself through their HIP kernels; the score matrix is never materialised.  Built: gradients of
+    every input and parameter, past_key_value / use_cache (model.py:700-708; the cache grows in place),
+    attention_mask [batch, keys] (model.py:819-824).  Not built (AtsError): per-query 4-D masks, attention
+    dropout in training mode (config.dropout > 0, model.py:622-623, 831-833), float32 inputs."""
 
     def __init__(self, config):
         super().__init__()
@@ -169,6 +169,7 @@ class GroupedQueryAttention(nn.Module):
         if self.hidden_size % self.num_heads or self.num_heads % self.num_kv_heads:
             raise AtsError("GroupedQueryAttention: hidden_size % num_heads and num_heads % num_kv_heads must be 0")
         self.scale = self.head_dim ** -0.5
+        self.dropout_p = float(getattr(config, "dropout", 0.0) or 0.0)
         self.q_proj = nn.Linear(self.hidden_size, self.num_heads * self.head_dim, bias=False)
         self.k_proj = nn.Linear(self.hidden_size, self.num_kv_heads * self.head_dim, bias=False)
         self.v_proj = nn.Linear(self.hidden_size, self.num_kv_heads * self.head_dim, bias=False)
@@ -192,6 +193,8 @@ class GroupedQueryAttention(nn.Module):
             raise AtsError(f"GroupedQueryAttention: expected [batch, seq, {self.hidden_size}], got {tuple(x.shape)}")
         if x.dtype != torch.bfloat16:
             raise AtsError(f"GroupedQueryAttention: the attention kernels are bfloat16 only, got {x.dtype}")
+        if self.training and self.dropout_p > 0:
+            raise AtsError("GroupedQueryAttention: attention dropout (config.dropout > 0 in training mode) is not built")
         B, L, H = x.shape
         nh, nkv, D = self.num_heads, self.num_kv_heads, self.head_dim
         x2 = x.reshape(B * L, H).contiguous()
