@@ -79,8 +79,10 @@ _SIGNATURES = {
     "ats_grad_clip_chunk_elems": (c_int, []),
     "ats_grad_norm_clip": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p,
                                    c_float, c_int, c_void_p]),
-    "ats_attention_fwd": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_int64, c_void_p, c_void_p, c_void_p,
-                                  c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p]),
+    "ats_attention_fwd_workspace": (c_size_t, [c_int, c_int, c_int, c_int, c_int, c_int]),
+    "ats_attention_fwd": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_int64, c_void_p,
+                                  c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p,
+                                  c_size_t, c_void_p]),
     "ats_attention_delta": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
     "ats_attention_bwd": (c_int, [c_void_p] * 10 + [c_int] * 6 + [c_float, c_void_p]),
     "ats_combine": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_int,

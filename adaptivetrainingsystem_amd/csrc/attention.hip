@@ -49,14 +49,20 @@ __device__ __forceinline__ af32x16_t att_mma(const au32x4_t& a, const au32x4_t& 
 // (batch, query head), or -- `pack` -- the queries of all query heads of one (batch, kv head), position
 // major: row r is position r / rep of head hkv * rep + r % rep.  Packing fills the tile when there are few
 // positions (decoding against a cache: one position, rep rows instead of one).
-template <int D, bool BIAS, int NT>
+// SPLIT: the tile sees the keys [key_first, key_first + key_count) only (key_first a multiple of the key tile,
+// at or before every query's position, so each row keeps a visible key) and leaves its unnormalised output,
+// running maximum and sum in part_out for attention_merge_kernel: rows of D + 4 floats at
+// ((b * Hq + hq) * L + position) * n_parts + part.
+constexpr int kPartPad = 4;
+template <int D, bool BIAS, int NT, bool SPLIT = false>
 __device__ __forceinline__ void attention_q_tile(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
                                                  int64_t k_sb, int64_t k_sh,
                                                  const bf16_t* __restrict__ v, int64_t v_sb, int v_sl, int64_t v_sh,
                                                  const float* __restrict__ key_bias, bf16_t* __restrict__ out,
                                                  float* __restrict__ lse, int Hq, int Hkv, int L, int Lk,
                                                  float scale_log2, int qt, int head, int b, bool pack,
-                                                 unsigned char* smem) {
+                                                 unsigned char* smem, float* __restrict__ part_out = nullptr,
+                                                 int part = 0, int n_parts = 1, int key_first = 0, int key_count = 0) {
     constexpr int kAttThreads = NT;
     constexpr int kAttBM = att_rows_per_block(NT);
     constexpr int KS = D / 16;              // k-steps of the score product
@@ -72,7 +78,10 @@ __device__ __forceinline__ void attention_q_tile(const bf16_t* __restrict__ q, c
 #define ATT_SV(stage_) (smem + (stage_) * (KTILE + VTILE) + KTILE)
     // optional additive bias per key (a padding mask), in log2 units: [2 stages][64] floats behind the tiles
     float* const s_bias = reinterpret_cast<float*>(smem + 2 * (KTILE + VTILE));
-    const float* bias_row = BIAS ? key_bias + (int64_t)b * Lk : nullptr;
+    const float* bias_row = BIAS ? key_bias + (int64_t)b * Lk + (SPLIT ? key_first : 0) : nullptr;
+    // Query i sits at position i + (Lk - L): with cached keys in front the causal diagonal moves right.
+    const int off = Lk - L - (SPLIT ? key_first : 0);
+    if constexpr (SPLIT) Lk = key_count;      // from here on: the keys of this part, counted from its first
     constexpr bool has_bias = BIAS;
     // with a bias the scores are brought to log2 units before the maximum is taken (sc = 1 afterwards)
     const float sc = has_bias ? 1.0f : scale_log2;
@@ -91,8 +100,8 @@ __device__ __forceinline__ void attention_q_tile(const bf16_t* __restrict__ q, c
     const bool row_valid = row < n_rows;
 
     const bf16_t* qp = q + ((int64_t)(b * Hq + hq) * L + q_clamped) * D;
-    const bf16_t* kbase = k + b * k_sb + hkv * k_sh;          // rows of D elements, one after the other
-    const bf16_t* vbase = v + b * v_sb + hkv * v_sh;          // row of key j at vbase + j * v_sl
+    const bf16_t* kbase = k + b * k_sb + hkv * k_sh + (SPLIT ? (int64_t)key_first * D : 0);     // rows of D elements
+    const bf16_t* vbase = v + b * v_sb + hkv * v_sh + (SPLIT ? (int64_t)key_first * v_sl : 0);  // key j at + j * v_sl
 
     au32x4_t qf[KS];
 #pragma unroll
@@ -123,11 +132,9 @@ __device__ __forceinline__ void attention_q_tile(const bf16_t* __restrict__ q, c
         for (int v = 0; v < 16; ++v) acc_o[d][v] = 0.f;
     float m_run = -INFINITY, l_run = 0.f;
 
-    // Query i sits at position i + (Lk - L): with cached keys in front the causal diagonal moves right.
-    const int off = Lk - L;
     const int q_pos = row / rp + off;                           // last key this lane's query sees
     const int q_block_last = min(qt * kAttBM + kAttBM - 1, n_rows - 1) / rp + off;
-    const int n_tiles = q_block_last / kAttBN + 1;
+    const int n_tiles = SPLIT ? min(q_block_last / kAttBN + 1, (Lk + kAttBN - 1) / kAttBN) : q_block_last / kAttBN + 1;
     const int q_wave_first = (qt * kAttBM + wave * 32) / rp + off;
     // a wave without rows (packed tiles of a short batch) only helps to load
     const int q_wave_last = qt * kAttBM + wave * 32 < n_rows ? (qt * kAttBM + wave * 32 + 31) / rp + off : -1;
@@ -324,8 +331,24 @@ __device__ __forceinline__ void attention_q_tile(const bf16_t* __restrict__ q, c
         __syncthreads();
     }
 
-    // ---- normalise and write [B, L, Hq*D]
     l_run += __shfl_xor(l_run, 32, 64);
+    if constexpr (SPLIT) {
+        if (row_valid) {
+            float* prow = part_out + ((((int64_t)b * Hq + hq) * L + q_clamped) * n_parts + part) * (D + kPartPad);
+#pragma unroll
+            for (int d = 0; d < DB; ++d)
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    *reinterpret_cast<float4*>(prow + d * 32 + r * 8 + g * 4) =
+                        make_float4(acc_o[d][r * 4 + 0], acc_o[d][r * 4 + 1], acc_o[d][r * 4 + 2], acc_o[d][r * 4 + 3]);
+            if (g == 0) {
+                prow[D] = m_run;
+                prow[D + 1] = l_run;
+            }
+        }
+        return;
+    }
+    // ---- normalise and write [B, L, Hq*D]
     const float inv = 1.0f / l_run;
     if (row_valid) {
         bf16_t* orow = out + ((int64_t)b * L + q_clamped) * (int64_t)(Hq * D) + hq * D;
@@ -385,11 +408,94 @@ __global__ __launch_bounds__(NT, 512 / NT) void attention_fwd_kernel(const bf16_
     }
 }
 
+// Few query rows against many keys (decoding): the keys are cut into n_parts ranges and every (batch, head
+// group, range) gets a workgroup, so that a handful of sequences still fills the chip; the ranges are merged
+// by attention_merge_kernel.  One query tile per group (rows <= 128), part p covers part_len keys from
+// p * part_len, the last one the rest.
+template <int D, bool BIAS>
+__global__ __launch_bounds__(256, 2) void attention_splitkv_kernel(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, int64_t k_sb, int64_t k_sh, const bf16_t* __restrict__ v,
+    int64_t v_sb, int v_sl, int64_t v_sh, const float* __restrict__ key_bias, float* __restrict__ part_out, int Hq, int Hkv,
+    int L, int Lk, float scale_log2, int B, int pack, int n_parts, int part_len) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    const int heads_per_group = pack ? 1 : Hq / Hkv;
+    const int n_base = B * Hkv * heads_per_group;
+    const int part = blockIdx.x / n_base;
+    const int base = blockIdx.x - part * n_base;
+    const int group = base / heads_per_group;
+    const int b = group / Hkv;
+    const int head = pack ? group % Hkv : (group % Hkv) * heads_per_group + base % heads_per_group;
+    const int key_first = part * part_len;
+    const int key_count = part == n_parts - 1 ? Lk - key_first : part_len;
+    attention_q_tile<D, BIAS, 256, true>(q, k, k_sb, k_sh, v, v_sb, v_sl, v_sh, key_bias, nullptr, nullptr, Hq, Hkv, L, Lk,
+                                         scale_log2, 0, head, b, pack != 0, smem, part_out, part, n_parts, key_first,
+                                         key_count);
+}
+
+// One wave per query row: out = sum_p 2^(m_p - M) O_p / sum_p 2^(m_p - M) l_p with M = max_p m_p, parts in order.
+template <int D>
+__global__ __launch_bounds__(256) void attention_merge_kernel(const float* __restrict__ part_out, bf16_t* __restrict__ out,
+                                                              float* __restrict__ lse, int64_t n_rows, int Hq, int L,
+                                                              int n_parts) {
+    const int lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);      // (b * Hq + hq) * L + position
+    if (row >= n_rows) return;
+    const float* p0 = part_out + row * n_parts * (D + kPartPad);
+    float M = -INFINITY;
+    for (int p = 0; p < n_parts; ++p) M = fmaxf(M, p0[p * (D + kPartPad) + D]);
+    float denom = 0.f, acc[D / 64];
+#pragma unroll
+    for (int j = 0; j < D / 64; ++j) acc[j] = 0.f;
+    for (int p = 0; p < n_parts; ++p) {
+        const float* pr = p0 + p * (D + kPartPad);
+        const float w = __builtin_amdgcn_exp2f(pr[D] - M);
+        denom += w * pr[D + 1];
+#pragma unroll
+        for (int j = 0; j < D / 64; ++j) acc[j] += w * pr[j * 64 + lane];
+    }
+    const int64_t bh = row / L, pos = row - bh * L;
+    const int64_t b = bh / Hq, hq = bh - b * Hq;
+    bf16_t* orow = out + (b * L + pos) * (int64_t)(Hq * D) + hq * D;
+    const float inv = 1.0f / denom;
+#pragma unroll
+    for (int j = 0; j < D / 64; ++j) orow[j * 64 + lane].bits = static_cast<uint16_t>(float_to_bf16_bits(acc[j] * inv));
+    if (lse && lane == 0) lse[row] = (M + log2f(denom)) * 0.6931471805599453f;
+}
+
+// Key ranges for the split: aim at ~1024 workgroups, ranges of whole key tiles and at least two tiles, every
+// range starting at or before the first query's position (so that each row sees a key of each range).
+// Measured (32 query / 8 kv heads, D 128, one new token): 1 sequence x 16384 keys 291 -> 49 us, 8 x 8192
+// 150 -> 55 us, 16 x 2048 42 -> 32 us; from 64 sequences on the single pass is as fast or faster.
+static int attention_split_plan(int B, int Hq, int Hkv, int L, int Lk, int* part_len_out) {
+    const int rep = Hq / Hkv;
+    const bool pack = L < att_rows_per_block(256) && Hq > Hkv;
+    const int64_t rows = pack ? (int64_t)L * rep : L;
+    if (rows > att_rows_per_block(256) || Lk - L < 4 * kAttBN) return 1;
+    const int64_t n_base = (int64_t)B * (pack ? Hkv : Hq);
+    if (n_base > 256) return 1;      // one workgroup per (batch, head group) already fills the chip twice over
+    int64_t want = 1024 / n_base;
+    if (want > 64) want = 64;
+    int part_len = (int)(((Lk + want - 1) / want + kAttBN - 1) / kAttBN) * kAttBN;
+    if (part_len < 2 * kAttBN) part_len = 2 * kAttBN;
+    int n_parts = (Lk + part_len - 1) / part_len;
+    while (n_parts > 1 && (int64_t)(n_parts - 1) * part_len > Lk - L) --n_parts;
+    *part_len_out = part_len;
+    return n_parts;
+}
+
 }  // namespace ats
 
+extern "C" size_t ats_attention_fwd_workspace(int B, int Hq, int Hkv, int L, int Lk, int D) {
+    if (B <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0 || L <= 0 || Lk < L || (D != 64 && D != 128)) return 0;
+    int part_len = 0;
+    const int n_parts = ats::attention_split_plan(B, Hq, Hkv, L, Lk, &part_len);
+    return n_parts > 1 ? (size_t)B * Hq * L * n_parts * (D + ats::kPartPad) * sizeof(float) : 0;
+}
+
 extern "C" int ats_attention_fwd(const void* q, const void* k, int64_t k_sb, int64_t k_sh, const void* v, int64_t v_sb,
-                                 int64_t v_sl, int64_t v_sh, const float* key_bias, void* out, float* lse, int B, int Hq, int Hkv, int L, int Lk,
-                                 int D, float scale, ats_stream_t stream) {
+                                 int64_t v_sl, int64_t v_sh, const float* key_bias, void* out, float* lse, int B, int Hq,
+                                 int Hkv, int L, int Lk, int D, float scale, void* workspace, size_t workspace_bytes,
+                                 ats_stream_t stream) {
     using namespace ats;
     ATS_REQUIRE(B >= 0 && Hq > 0 && Hkv > 0 && Hq % Hkv == 0 && L >= 0 && Lk >= L && scale > 0.f, ATS_ERR_INVALID_ARG,
                 "ats_attention_fwd: B=%d Hq=%d Hkv=%d L=%d Lk=%d scale=%g", B, Hq, Hkv, L, Lk, scale);
@@ -406,6 +512,49 @@ extern "C" int ats_attention_fwd(const void* q, const void* k, int64_t k_sb, int
     ATS_REQUIRE((int64_t)Lk * D * 2 < 0x7fffffffLL && ((int64_t)Lk * v_sl + D) * 2 < 0x7fffffffLL, ATS_ERR_UNSUPPORTED,
                 "ats_attention_fwd: %d keys (one head's K or V must stay under 2 GiB)", Lk);
     // few query positions (decoding, short chunks): the query heads of a kv group share a tile's rows
+    const float scale_log2 = scale * 1.4426950408889634f;
+    // decoding sizes with a workspace: key ranges in parallel, then a merge
+    int part_len = 0;
+    const int n_parts = workspace ? attention_split_plan(B, Hq, Hkv, L, Lk, &part_len) : 1;
+    if (n_parts > 1 && workspace_bytes >= (size_t)B * Hq * L * n_parts * (D + kPartPad) * sizeof(float) &&
+        aligned16(workspace)) {
+        const int pack = (L < att_rows_per_block(256) && Hq > Hkv) ? 1 : 0;
+        const int64_t n_base = (int64_t)B * (pack ? Hkv : Hq);
+        const int smem = 2 * kAttBN * ((D * 2 + 16) + (D * 2 + 64)) + (key_bias ? 2 * kAttBN * 4 : 0);
+        float* parts = static_cast<float*>(workspace);
+        static LdsReservation reserved_split[4];
+        auto launch_split = [&](auto kernel, LdsReservation& reserved) -> int {
+            if (smem > 64 * 1024) {
+                hipError_t e = reserve_lds(reserved, {reinterpret_cast<const void*>(kernel)}, smem);
+                ATS_REQUIRE(e == hipSuccess, ATS_ERR_LAUNCH, "ats_attention_fwd: cannot reserve %d bytes of LDS: %s", smem,
+                            hipGetErrorString(e));
+            }
+            hipLaunchKernelGGL(kernel, dim3((unsigned)(n_base * n_parts)), dim3(256), smem, as_stream(stream),
+                               static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k), k_sb, k_sh,
+                               static_cast<const bf16_t*>(v), v_sb, (int)v_sl, v_sh, key_bias, parts, Hq, Hkv, L, Lk,
+                               scale_log2, B, pack, n_parts, part_len);
+            return ATS_OK;
+        };
+        int rc;
+        if (D == 128)
+            rc = key_bias ? launch_split(attention_splitkv_kernel<128, true>, reserved_split[0])
+                          : launch_split(attention_splitkv_kernel<128, false>, reserved_split[1]);
+        else
+            rc = key_bias ? launch_split(attention_splitkv_kernel<64, true>, reserved_split[2])
+                          : launch_split(attention_splitkv_kernel<64, false>, reserved_split[3]);
+        if (rc != ATS_OK) return rc;
+        ATS_CHECK_LAUNCH("ats_attention_fwd(key ranges)");
+        const int64_t n_rows = (int64_t)B * Hq * L;
+        const dim3 mgrid((unsigned)((n_rows + 3) / 4));
+        if (D == 128)
+            hipLaunchKernelGGL((attention_merge_kernel<128>), mgrid, dim3(256), 0, as_stream(stream), parts,
+                               static_cast<bf16_t*>(out), lse, n_rows, Hq, L, n_parts);
+        else
+            hipLaunchKernelGGL((attention_merge_kernel<64>), mgrid, dim3(256), 0, as_stream(stream), parts,
+                               static_cast<bf16_t*>(out), lse, n_rows, Hq, L, n_parts);
+        ATS_CHECK_LAUNCH("ats_attention_fwd(merge)");
+        return ATS_OK;
+    }
     const int nt = L >= 4096 ? 512 : 256;
     const int kAttBM = att_rows_per_block(nt);
     const int pack = (L < kAttBM && Hq > Hkv) ? 1 : 0;
@@ -413,7 +562,6 @@ extern "C" int ats_attention_fwd(const void* q, const void* k, int64_t k_sb, int
                                   : (int64_t)(((L + kAttBM - 1) / kAttBM + 1) / 2) * Hq * B;
     ATS_REQUIRE(n_blocks <= 0x7fffffff, ATS_ERR_UNSUPPORTED, "ats_attention_fwd: %lld workgroups", (long long)n_blocks);
     const dim3 grid((unsigned)n_blocks);
-    const float scale_log2 = scale * 1.4426950408889634f;
     static LdsReservation reserved_lds[8];      // one per kernel instance
     auto launch = [&](auto kernel, int smem, LdsReservation& reserved) -> int {
         if (smem > 64 * 1024) {

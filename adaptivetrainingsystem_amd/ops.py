@@ -664,14 +664,15 @@ def _key_bias(key_bias, B: int, Lk: int, q: torch.Tensor, who: str):
 
 
 def causal_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: Optional[float] = None,
-                     return_lse: bool = False, key_bias: Optional[torch.Tensor] = None):
+                     return_lse: bool = False, key_bias: Optional[torch.Tensor] = None, split_keys: bool = True):
     """Causal grouped-query attention.  q [B,Hq,L,D]; k [B,Hkv,Lk,D] with a head's rows one after the other
     and any batch/head strides (e.g. a view of a larger cache buffer); v [B,Hkv,Lk,D] in any batch/head/position
     strides (e.g. a view of a fused projection output); bf16, D 64 or 128, Lk >= L.
     With Lk > L the leading Lk - L keys are a cache: query i sits at position i + Lk - L.
     key_bias [B, Lk] float32 (optional) is added to the scaled scores of a key for every query and head;
     (1 - attention_mask) * -1e4 is the reference's padding mask (MS/core/model.py:819-824).
-    Returns out [B, L, Hq*D] (and lse [B,Hq,L] float32 if asked)."""
+    split_keys=False keeps the single-pass kernel where few rows against many keys would otherwise be cut
+    into key ranges.  Returns out [B, L, Hq*D] (and lse [B,Hq,L] float32 if asked)."""
     _need_gpu(q, k, v)
     if q.dim() != 4 or k.dim() != 4 or v.dim() != 4 or q.dtype != torch.bfloat16 or k.dtype != q.dtype or v.dtype != q.dtype:
         raise AtsError("causal_attention: q, k, v must be 4-D bfloat16 tensors [batch, heads, seq, head_dim]")
@@ -688,10 +689,14 @@ def causal_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: O
     lib = _lib.load()
     out = torch.empty(B, L, Hq * D, dtype=q.dtype, device=q.device)
     lse = torch.empty(B, Hq, L, dtype=torch.float32, device=q.device) if return_lse else None
+    # decoding a few sequences: scratch for the partial results of key ranges that run side by side
+    ws_bytes = lib.ats_attention_fwd_workspace(B, Hq, Hkv, L, Lk, D) if split_keys else 0
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device) if ws_bytes else None
     check(lib.ats_attention_fwd(q.data_ptr(), k.data_ptr(), k.stride(0), k.stride(1), v.data_ptr(), v.stride(0),
                                 v.stride(2), v.stride(1),
                                 _ptr(key_bias), out.data_ptr(), _ptr(lse), B, Hq, Hkv, L, Lk, D,
-                                float(D ** -0.5 if scale is None else scale), _stream()), "ats_attention_fwd")
+                                float(D ** -0.5 if scale is None else scale), _ptr(ws), ws_bytes, _stream()),
+          "ats_attention_fwd")
     return (out, lse) if return_lse else out
 
 

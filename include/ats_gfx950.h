@@ -294,10 +294,17 @@ int ats_grouped_gemm_nt(const void* a, const void* const* a_ptrs, int64_t lda, i
  * broadcast otherwise); its flash path aligns the diagonal the same way.
  * key_bias (optional): [B,Lk] float32 added to the scaled scores of a key for every query and head; the
  * reference's padding mask is (1 - attention_mask) * -1e4 (model.py:819-824).
- * lse (optional): [B,Hq,L] float32 log-sum-exp of the scaled (and biased) scores per query. */
+ * lse (optional): [B,Hq,L] float32 log-sum-exp of the scaled (and biased) scores per query.
+ * workspace (optional): with few query rows against many keys (decoding a handful of sequences) one workgroup
+ * per (batch, head group) cannot fill the chip; given ats_attention_fwd_workspace(...) bytes of scratch the
+ * keys are cut into ranges that run side by side and a second kernel merges their partial softmax results
+ * (same values up to float32 rounding of the merge).  The size query returns 0 where that does not apply;
+ * NULL / too small a workspace selects the single-pass kernel. */
+size_t ats_attention_fwd_workspace(int B, int Hq, int Hkv, int L, int Lk, int D);
 int ats_attention_fwd(const void* q, const void* k, int64_t k_sb, int64_t k_sh, const void* v, int64_t v_sb,
                       int64_t v_sl, int64_t v_sh, const float* key_bias, void* out, float* lse, int B, int Hq,
-                      int Hkv, int L, int Lk, int D, float scale, ats_stream_t stream);
+                      int Hkv, int L, int Lk, int D, float scale, void* workspace, size_t workspace_bytes,
+                      ats_stream_t stream);
 
 /* ---- Causal grouped-query attention (backward) ----------------------------------
  * The reference leaves this gradient to autograd (model.py:757-839 under torch.autograd); the kernels

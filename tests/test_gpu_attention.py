@@ -71,6 +71,32 @@ def test_causal_attention_with_cached_keys(ops, gpu, B, Hq, Hkv, L, Lk, D):
     assert rel_err(lse, torch.logsumexp(s, -1)) <= 1e-4
 
 
+@pytest.mark.parametrize("B,Hq,Hkv,L,Lk,D", [(1, 32, 8, 1, 2048, 128), (2, 8, 2, 1, 4097, 64), (1, 4, 4, 1, 300, 128),
+                                             (3, 8, 2, 5, 1000, 128), (1, 16, 2, 16, 515, 64), (5, 2, 1, 64, 700, 128)])
+def test_decode_attention_over_key_ranges(ops, gpu, B, Hq, Hkv, L, Lk, D):
+    """Few query rows against many keys: the keys are cut into ranges that run side by side and are merged.
+    Same result as the single pass (to float32 rounding of the merge), the oracle's values, the log-sum-exp,
+    and the padding bias carried through the ranges."""
+    from adaptivetrainingsystem_amd import _lib
+    print("case key ranges", B, Hq, Hkv, L, Lk, D, flush=True)
+    assert _lib.load().ats_attention_fwd_workspace(B, Hq, Hkv, L, Lk, D) > 0
+    g = gen(140)
+    q = torch.randn(B, Hq, L, D, generator=g).bfloat16()
+    k = torch.randn(B, Hkv, Lk, D, generator=g).bfloat16()
+    v = torch.randn(B, Hkv, Lk, D, generator=g).bfloat16()
+    rep = Hq // Hkv
+    for mask in (None, _padding_mask(B, Lk, 141)):
+        if mask is not None:
+            mask[:, :Lk - L + 1] = 1
+            mask[:, 70:130] = 0            # a stretch of padded keys inside the cache
+        bias = None if mask is None else ((1.0 - mask) * -1e4).to(gpu)
+        ref = O.attention_standard(q, k.repeat_interleave(rep, dim=1), v.repeat_interleave(rep, dim=1), D ** -0.5, mask)
+        out, lse = ops.causal_attention(q.to(gpu), k.to(gpu), v.to(gpu), return_lse=True, key_bias=bias)
+        one, lse1 = ops.causal_attention(q.to(gpu), k.to(gpu), v.to(gpu), return_lse=True, key_bias=bias, split_keys=False)
+        assert rel_err(out, ref) <= BF16_TOL
+        assert rel_err(out, one) <= 1e-2 and rel_err(lse, lse1) <= 1e-5
+
+
 def test_cached_attention_equals_tail_of_full_call(ops, gpu):
     """Size-independent property at a long length: the last L rows of a full call, bit for bit per row tile
     alignment aside -- compared at the bf16 bar since tiles start at different keys."""

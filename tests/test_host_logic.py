@@ -44,13 +44,13 @@ def test_argument_errors_return_codes_not_exits():
                             None) == -1       # odd head_dim
     assert lib.ats_select_topk_per_sequence(None, 1, 10000, 5, None, None) == -1
     # attention: head_dim outside {64, 128}, fewer keys than queries, query heads not a multiple of kv heads
-    assert lib.ats_attention_fwd(None, None, 0, 0, None, 0, 96, 0, None, None, None, 1, 4, 2, 16, 16, 96, 0.1, None) == -2
+    assert lib.ats_attention_fwd(None, None, 0, 0, None, 0, 96, 0, None, None, None, 1, 4, 2, 16, 16, 96, 0.1, None, 0, None) == -2
     assert b"head_dim" in lib.ats_last_error_string()
-    assert lib.ats_attention_fwd(None, None, 0, 0, None, 0, 128, 0, None, None, None, 1, 4, 2, 16, 8, 128, 0.1, None) == -1
-    assert lib.ats_attention_fwd(None, None, 0, 0, None, 0, 128, 0, None, None, None, 1, 3, 2, 16, 16, 128, 0.1, None) == -1
-    assert lib.ats_attention_fwd(None, None, 0, 0, None, 0, 128, 0, None, None, None, 1, 4, 2, 16, 16, 128, 0.1, None) == -1     # null pointers
-    assert lib.ats_attention_fwd(None, None, 0, 0, None, 0, 128, 0, None, None, None, 0, 4, 2, 16, 16, 128, 0.1, None) == 0      # empty batch
-    assert lib.ats_attention_bwd(*([None] * 10), 1, 4, 2, 16, 8, 128, 0.1, None) == -1
+    assert lib.ats_attention_fwd(None, None, 0, 0, None, 0, 128, 0, None, None, None, 1, 4, 2, 16, 8, 128, 0.1, None, 0, None) == -1
+    assert lib.ats_attention_fwd(None, None, 0, 0, None, 0, 128, 0, None, None, None, 1, 3, 2, 16, 16, 128, 0.1, None, 0, None) == -1
+    assert lib.ats_attention_fwd(None, None, 0, 0, None, 0, 128, 0, None, None, None, 1, 4, 2, 16, 16, 128, 0.1, None, 0, None) == -1     # null pointers
+    assert lib.ats_attention_fwd(None, None, 0, 0, None, 0, 128, 0, None, None, None, 0, 4, 2, 16, 16, 128, 0.1, None, 0, None) == 0      # empty batch
+    assert lib.ats_attention_bwd(*([None] * 10), 1, 4, 2, 16, 8, 128, 0.1, None, 0, None) == -1
     assert lib.ats_attention_bwd(*([None] * 10), 1, 4, 2, 16, 16, 32, 0.1, None) == -2
     assert lib.ats_attention_delta(None, None, None, 1, 4, 16, 80, None) == -2
     # K slices: I must be k_splits whole slabs, and only weight-streaming sizes (<= 48 rows per expert)
