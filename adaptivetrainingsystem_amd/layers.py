@@ -182,10 +182,11 @@ class GroupedQueryAttention(nn.Module):
             nn.init.normal_(proj.weight, mean=0.0, std=std * gain)
         nn.init.normal_(self.o_proj.weight, mean=0.0, std=std * gain / math.sqrt(2 * getattr(config, "num_layers", 1)))
         self._param_count = sum(p.numel() for p in self.parameters())
-        self._calls = 0
-        self._kv_buffer = None       # addresses and fill of the cache buffers handed out last (no tensor is held)
-        self._qkv_key = None
-        self._qkv = None
+        # per-call bookkeeping lives in one dict that is mutated in place: assigning module attributes on every
+        # call goes through nn.Module.__setattr__, a visible part of a decoding step
+        #   kv: addresses and fill of the cache buffers handed out last (no tensor is held)
+        self._state: Dict[str, Any] = {"calls": 0, "kv": None, "kv_copies": 0, "kv_appends": 0, "qkv_key": None,
+                                       "qkv": None}
 
     def forward(self, x: torch.Tensor, attention_mask: Optional[torch.Tensor] = None, past_key_value=None,
                 use_cache: bool = False):
@@ -239,7 +240,7 @@ class GroupedQueryAttention(nn.Module):
         else:
             a = ops.causal_attention(q, k, v, self.scale, key_bias=key_bias)
         out = lin(a.view(B * L, nh * D), self.o_proj.weight).view(B, L, H)    # a: [B, L, nh*D]
-        self._calls += 1
+        self._state["calls"] += 1
         if use_cache:
             return out, (k, v if v.stride(3) == 1 and v.stride(2) == D else v.contiguous())
         return out
@@ -249,11 +250,12 @@ class GroupedQueryAttention(nn.Module):
         when a weight is replaced or written to (the parameters themselves stay as the reference has them)."""
         ws = (self.q_proj.weight, self.k_proj.weight, self.v_proj.weight)
         key = (dtype,) + tuple((w.data_ptr(), w._version) for w in ws)
-        if self._qkv_key != key:
+        st = self._state
+        if st["qkv_key"] != key:
             with torch.no_grad():
-                self._qkv = torch.cat([w.detach().to(dtype) for w in ws], dim=0).contiguous()
-            self._qkv_key = key
-        return self._qkv
+                st["qkv"] = torch.cat([w.detach().to(dtype) for w in ws], dim=0).contiguous()
+            st["qkv_key"] = key
+        return st["qkv"]
 
     def _extend_cache(self, k_cache, v_cache, k_new, v_new):
         """The cache followed by the new rows, as the reference's torch.cat gives them (model.py:700-704), without
@@ -264,7 +266,7 @@ class GroupedQueryAttention(nn.Module):
         any other cache tensor is copied into a fresh buffer whose capacity is 1.5 x the new length."""
         B, nkv, Lp, D = k_cache.shape
         L = k_new.shape[2]
-        st = self._kv_buffer
+        st = self._state["kv"]
         cap_strides = lambda cap: (nkv * cap * D, cap * D, D, 1)
         if (st is not None and Lp == st["length"] and Lp + L <= st["capacity"]
                 and k_cache.dtype == k_new.dtype and v_cache.dtype == v_new.dtype
@@ -275,7 +277,9 @@ class GroupedQueryAttention(nn.Module):
             cap = st["capacity"]
             k_buf = k_cache.as_strided((B, nkv, cap, D), cap_strides(cap))
             v_buf = v_cache.as_strided((B, nkv, cap, D), cap_strides(cap))
+            self._state["kv_appends"] += 1
         else:
+            self._state["kv_copies"] += 1
             cap = Lp + L + max(64, (Lp + L) // 2)
             k_buf = torch.empty(B, nkv, cap, D, dtype=k_new.dtype, device=k_new.device)
             v_buf = torch.empty(B, nkv, cap, D, dtype=v_new.dtype, device=v_new.device)
@@ -283,14 +287,16 @@ class GroupedQueryAttention(nn.Module):
             v_buf[:, :, :Lp].copy_(v_cache)
         k_buf[:, :, Lp:Lp + L].copy_(k_new)
         v_buf[:, :, Lp:Lp + L].copy_(v_new)
-        self._kv_buffer = {"k_ptr": k_buf.data_ptr(), "v_ptr": v_buf.data_ptr(), "capacity": cap, "length": Lp + L,
+        self._state["kv"] = {"k_ptr": k_buf.data_ptr(), "v_ptr": v_buf.data_ptr(), "capacity": cap, "length": Lp + L,
                            "nbytes": k_buf.numel() * k_buf.element_size()}
         return k_buf[:, :, :Lp + L], v_buf[:, :, :Lp + L]
 
     def get_attention_stats(self) -> Dict[str, Any]:
-        return {"total_calls": self._calls, "flash_attention_calls": self._calls, "standard_attention_calls": 0,
-                "flash_attention_ratio": 1.0 if self._calls else 0.0, "num_heads": self.num_heads,
-                "num_kv_heads": self.num_kv_heads, "head_dim": self.head_dim, "parameter_count": self._param_count}
+        calls = self._state["calls"]
+        return {"total_calls": calls, "flash_attention_calls": calls, "standard_attention_calls": 0,
+                "flash_attention_ratio": 1.0 if calls else 0.0, "num_heads": self.num_heads,
+                "num_kv_heads": self.num_kv_heads, "head_dim": self.head_dim, "parameter_count": self._param_count,
+                "cache_appends_in_place": self._state["kv_appends"], "cache_copies": self._state["kv_copies"]}
 
 
 DenseGroupedQueryAttention = GroupedQueryAttention     # the reference's class name (model.py:565)
