@@ -432,7 +432,9 @@ __global__ __launch_bounds__(256, 2) void attention_splitkv_kernel(
                                          key_count);
 }
 
-// One wave per query row: out = sum_p 2^(m_p - M) O_p / sum_p 2^(m_p - M) l_p with M = max_p m_p, parts in order.
+// One wave per query row: out = sum_p 2^(m_p - M) O_p / sum_p 2^(m_p - M) l_p with M = max_p m_p.  Lane p
+// holds the maximum and sum of part p (at most 64 parts), so the weights are ready before the rows of
+// partial outputs are streamed; the sums run over the parts in order.
 template <int D>
 __global__ __launch_bounds__(256) void attention_merge_kernel(const float* __restrict__ part_out, bf16_t* __restrict__ out,
                                                               float* __restrict__ lse, int64_t n_rows, int Hq, int L,
@@ -441,15 +443,20 @@ __global__ __launch_bounds__(256) void attention_merge_kernel(const float* __res
     const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);      // (b * Hq + hq) * L + position
     if (row >= n_rows) return;
     const float* p0 = part_out + row * n_parts * (D + kPartPad);
-    float M = -INFINITY;
-    for (int p = 0; p < n_parts; ++p) M = fmaxf(M, p0[p * (D + kPartPad) + D]);
+    const float2 ml = lane < n_parts ? *reinterpret_cast<const float2*>(p0 + lane * (D + kPartPad) + D)
+                                     : make_float2(-INFINITY, 0.f);
+    float M = ml.x;
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) M = fmaxf(M, __shfl_xor(M, o, 64));
+    const float w_lane = lane < n_parts ? __builtin_amdgcn_exp2f(ml.x - M) : 0.f;
     float denom = 0.f, acc[D / 64];
 #pragma unroll
     for (int j = 0; j < D / 64; ++j) acc[j] = 0.f;
+#pragma unroll 4
     for (int p = 0; p < n_parts; ++p) {
+        const float w = __shfl(w_lane, p, 64);
+        denom += w * __shfl(ml.y, p, 64);
         const float* pr = p0 + p * (D + kPartPad);
-        const float w = __builtin_amdgcn_exp2f(pr[D] - M);
-        denom += w * pr[D + 1];
 #pragma unroll
         for (int j = 0; j < D / 64; ++j) acc[j] += w * pr[j * 64 + lane];
     }
@@ -464,8 +471,8 @@ __global__ __launch_bounds__(256) void attention_merge_kernel(const float* __res
 
 // Key ranges for the split: aim at ~1024 workgroups, ranges of whole key tiles and at least two tiles, every
 // range starting at or before the first query's position (so that each row sees a key of each range).
-// Measured (32 query / 8 kv heads, D 128, one new token): 1 sequence x 16384 keys 291 -> 49 us, 8 x 8192
-// 150 -> 55 us, 16 x 2048 42 -> 32 us; from 64 sequences on the single pass is as fast or faster.
+// Measured (32 query / 8 kv heads, D 128, one new token): 1 sequence x 16384 keys 291 -> 33 us, 8 x 8192
+// 150 -> 50 us, 16 x 2048 41 -> 30 us; from 64 sequences on the single pass is as fast or faster.
 static int attention_split_plan(int B, int Hq, int Hkv, int L, int Lk, int* part_len_out) {
     const int rep = Hq / Hkv;
     const bool pack = L < att_rows_per_block(256) && Hq > Hkv;
