@@ -151,10 +151,11 @@ def route_topk(logits: torch.Tensor, k: int, temperature: float = 1.0, variant: 
     ws_bytes = 0
     lib = _lib.load()
     if with_stats:
-        zeros = torch.zeros(2 * E + 1, dtype=torch.int32, device=dev)      # one fill launch for the three outputs
-        hist = zeros[:E]
-        colsum = zeros[E:2 * E].view(torch.float32)
-        aux = zeros[2 * E:].view(torch.float32)
+        # one buffer for the three outputs; the finalize kernel writes every element (nothing runs for T == 0)
+        stats = (torch.empty if T > 0 else torch.zeros)(2 * E + 1, dtype=torch.int32, device=dev)
+        hist = stats[:E]
+        colsum = stats[E:2 * E].view(torch.float32)
+        aux = stats[2 * E:].view(torch.float32)
         ws_bytes = lib.ats_route_topk_workspace(T, E)
         ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
     check(lib.ats_route_topk(logits.data_ptr(), T, E, int(k), float(temperature), int(variant), idx.data_ptr(),
