@@ -197,10 +197,12 @@ __global__ __launch_bounds__(256) void route_topk_kernel(const float* __restrict
                                                          float temperature, int variant, int G, int iters,
                                                          int32_t* __restrict__ idx_out, float* __restrict__ w_out,
                                                          int32_t* __restrict__ part_hist,
-                                                         float* __restrict__ part_colsum) {
+                                                         float* __restrict__ part_colsum, float lbw,
+                                                         int32_t* __restrict__ hist, float* __restrict__ colsum,
+                                                         float* __restrict__ aux) {
     extern __shared__ unsigned char smem_raw[];
     int* s_hist = reinterpret_cast<int*>(smem_raw);            // [E]
-    float* s_col = reinterpret_cast<float*>(s_hist + E);        // [4][E]
+    float* s_col = reinterpret_cast<float*>(s_hist + E);        // [4][E]  (then [E] terms of the auxiliary loss)
     const bool want_stats = part_hist != nullptr;
     const int lane = lane_id();
     const int wave = threadIdx.x >> 6;
@@ -340,9 +342,31 @@ __global__ __launch_bounds__(256) void route_topk_kernel(const float* __restrict
             if (grp == 0 && e < E) s_col[wave * E + e] = c;
         }
         __syncthreads();
-        for (int e = threadIdx.x; e < E; e += 256) {
-            part_hist[(int64_t)blockIdx.x * E + e] = s_hist[e];
-            part_colsum[(int64_t)blockIdx.x * E + e] = ((s_col[e] + s_col[E + e]) + s_col[2 * E + e]) + s_col[3 * E + e];
+        if (gridDim.x > 1) {
+            for (int e = threadIdx.x; e < E; e += 256) {
+                part_hist[(int64_t)blockIdx.x * E + e] = s_hist[e];
+                part_colsum[(int64_t)blockIdx.x * E + e] =
+                    ((s_col[e] + s_col[E + e]) + s_col[2 * E + e]) + s_col[3 * E + e];
+            }
+        } else {
+            // one block holds every token (a decoding step): its partials are the totals, so the statistics
+            // and the auxiliary loss are finished here, with route_finalize_kernel's arithmetic
+            float* s_term = s_col + 4 * E;
+            for (int e = threadIdx.x; e < E; e += 256) {
+                const int hsum = s_hist[e];
+                const float csum = ((s_col[e] + s_col[E + e]) + s_col[2 * E + e]) + s_col[3 * E + e];
+                hist[e] = hsum;
+                colsum[e] = csum;
+                const float usage = (float)hsum / (float)((double)T * k + 1e-9);
+                const float importance = csum / (float)T;
+                s_term[e] = usage * importance;
+            }
+            __syncthreads();
+            if (threadIdx.x == 0 && aux) {
+                float sum = 0.f;
+                for (int e = 0; e < E; ++e) sum += s_term[e];
+                aux[0] = fminf(sum * (float)E * lbw, 1.0f);
+            }
         }
     }
 }
@@ -415,6 +439,12 @@ static int route_grid(int64_t T, int E, int* G_out, int* iters_out) {
     if (iters > 64) iters = 64;
     const int64_t per_block = (int64_t)groups_per_block * iters;
     *G_out = G;
+    // few tokens: one block takes them all in up to 16 passes and finishes the statistics itself
+    const int64_t passes = (T + groups_per_block - 1) / groups_per_block;
+    if (passes <= 16) {
+        *iters_out = (int)(passes < 1 ? 1 : passes);
+        return 1;
+    }
     *iters_out = (int)iters;
     return (int)((T + per_block - 1) / per_block);
 }
@@ -497,19 +527,22 @@ extern "C" int ats_route_topk(const float* logits, int64_t T, int E, int k, floa
         part_col = reinterpret_cast<float*>(part_hist + (size_t)nblocks * E);
     }
     hipStream_t s = as_stream(stream);
-    const size_t smem = (size_t)E * 5 * sizeof(float);
+    const size_t smem = (size_t)E * 6 * sizeof(float);
     const int vpl = (E + G - 1) / G;
     if (vpl <= 1)
         hipLaunchKernelGGL((route_topk_kernel<1>), dim3(nblocks), dim3(256), smem, s, logits, T, E, k, temperature,
-                           variant, G, iters, idx_out, w_out, part_hist, part_col);
+                           variant, G, iters, idx_out, w_out, part_hist, part_col, load_balancing_weight, hist,
+                           prob_colsum, aux);
     else if (vpl <= 4)
         hipLaunchKernelGGL((route_topk_kernel<4>), dim3(nblocks), dim3(256), smem, s, logits, T, E, k, temperature,
-                           variant, G, iters, idx_out, w_out, part_hist, part_col);
+                           variant, G, iters, idx_out, w_out, part_hist, part_col, load_balancing_weight, hist,
+                           prob_colsum, aux);
     else
         hipLaunchKernelGGL((route_topk_kernel<16>), dim3(nblocks), dim3(256), smem, s, logits, T, E, k, temperature,
-                           variant, G, iters, idx_out, w_out, part_hist, part_col);
+                           variant, G, iters, idx_out, w_out, part_hist, part_col, load_balancing_weight, hist,
+                           prob_colsum, aux);
     ATS_CHECK_LAUNCH("ats_route_topk");
-    if (stats) {
+    if (stats && nblocks > 1) {
         hipLaunchKernelGGL(route_finalize_kernel, dim3(1), dim3(256), (size_t)(E + 512) * sizeof(float), s, part_hist,
                            part_col, nblocks, E, T, k, load_balancing_weight, hist, prob_colsum, aux);
         ATS_CHECK_LAUNCH("ats_route_topk(finalize)");
