@@ -247,7 +247,9 @@ class GroupedQueryAttention(nn.Module):
 
     def _stacked_qkv(self, dtype: torch.dtype) -> torch.Tensor:
         """[q_proj; k_proj; v_proj] weights as one [(nh + 2 nkv) * D, hidden] matrix in the compute dtype, rebuilt
-        when a weight is replaced or written to (the parameters themselves stay as the reference has them)."""
+        when a weight is replaced or written to (the parameters themselves stay as the reference has them).
+        Writes are seen through the tensors' version counters: optimizers, nn.init, load_state_dict and copy_
+        advance them; a write through `weight.data` does not, and needs reset_cached_weights() afterwards."""
         ws = (self.q_proj.weight, self.k_proj.weight, self.v_proj.weight)
         key = (dtype,) + tuple((w.data_ptr(), w._version) for w in ws)
         st = self._state
@@ -256,6 +258,11 @@ class GroupedQueryAttention(nn.Module):
                 st["qkv"] = torch.cat([w.detach().to(dtype) for w in ws], dim=0).contiguous()
             st["qkv_key"] = key
         return st["qkv"]
+
+    def reset_cached_weights(self) -> None:
+        """Drops the stacked copy of the projection weights (rebuilt on the next inference call)."""
+        self._state["qkv_key"] = None
+        self._state["qkv"] = None
 
     def _extend_cache(self, k_cache, v_cache, k_new, v_new):
         """The cache followed by the new rows, as the reference's torch.cat gives them (model.py:700-704), without
@@ -400,6 +407,13 @@ class MoEFFNLayer(nn.Module):
         nn.init.normal_(self.gate.weight, mean=0.0, std=0.01)
 
     # ---- expert weight tables (device arrays of pointers; rebuilt when a weight moves or changes dtype)
+    def reset_cached_weights(self) -> None:
+        """Drops the per-expert pointer tables and compute-dtype weight copies (rebuilt on the next call).  They
+        follow replaced parameters and version-counted writes by themselves; a write through `weight.data` to
+        parameters kept in another dtype than the activations is the one case that needs this call."""
+        self._wcache_key = None
+        self._wcache = None
+
     def _weight_tables(self, dtype: torch.dtype, device: torch.device):
         params = []
         for ex in self.experts:

@@ -156,6 +156,11 @@ def test_gqa_module(gpu, hidden, nh, nkv, B, L):
         assert rel_err(out2, ref2) <= BF16_TOL and not torch.equal(out2, out)
         att.k_proj.weight = torch.nn.Parameter(att.k_proj.weight.detach() * 2.0)
         assert torch.equal(att(x.to(gpu)), out)
+        att.k_proj.weight.data.mul_(0.5)          # a write the version counter does not see
+        att.reset_cached_weights()
+        assert torch.equal(att(x.to(gpu)), out2)
+        att.k_proj.weight.data.mul_(2.0)
+        att.reset_cached_weights()
     # prefill with use_cache, then two single-token steps fed from the cache (model.py:700-708)
     w = [getattr(att, n).weight.detach().cpu() for n in ("q_proj", "k_proj", "v_proj", "o_proj")]
     with torch.no_grad():
