@@ -1,0 +1,84 @@
+"""Seeded random shapes through the attention and K-sliced product paths, against the CPU oracle.  The fixed
+cases elsewhere pin known edges; these sweep the shape space around them (tile remainders, head ratios, cache
+lengths on both sides of the thresholds that switch kernels)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import sparse_layer_oracle as O
+
+pytestmark = pytest.mark.gpu
+BF16_TOL = 2e-2
+
+
+def rel_err(got, ref) -> float:
+    got, ref = got.detach().double().cpu(), ref.detach().double().cpu()
+    denom = ref.abs().max().item()
+    return (got - ref).abs().max().item() / (denom if denom > 0 else 1.0)
+
+
+def _attention_cases(n, seed):
+    rng = np.random.default_rng(seed)
+    cases = []
+    for _ in range(n):
+        D = int(rng.choice([64, 128]))
+        Hkv = int(rng.choice([1, 2, 3, 4]))
+        Hq = Hkv * int(rng.choice([1, 2, 4, 8]))
+        B = int(rng.integers(1, 4))
+        regime = rng.integers(0, 3)
+        if regime == 0:      # prefill, no cache
+            L = int(rng.integers(1, 500)); Lk = L
+        elif regime == 1:    # a chunk on top of a cache
+            L = int(rng.integers(1, 200)); Lk = L + int(rng.integers(1, 900))
+        else:                # decoding: few rows, long cache (key ranges)
+            L = int(rng.integers(1, 5)); Lk = L + int(rng.integers(200, 1500))
+        cases.append((B, Hq, Hkv, L, Lk, D, bool(rng.integers(0, 2))))
+    return cases
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,L,Lk,D,masked", _attention_cases(36, 2024))
+def test_attention_random_shapes(gpu, B, Hq, Hkv, L, Lk, D, masked):
+    from adaptivetrainingsystem_amd import ops
+    print("case random attention", B, Hq, Hkv, L, Lk, D, masked, flush=True)
+    g = torch.Generator().manual_seed(B * 1000003 + Hq * 10007 + L * 101 + Lk)
+    q = torch.randn(B, Hq, L, D, generator=g).bfloat16()
+    k = torch.randn(B, Hkv, Lk, D, generator=g).bfloat16()
+    v = torch.randn(B, Hkv, Lk, D, generator=g).bfloat16()
+    dout = torch.randn(B, L, Hq * D, generator=g).bfloat16()
+    mask = None
+    if masked:      # right padding that leaves every query a real key, plus a padded stretch inside
+        mask = torch.ones(B, Lk)
+        for b in range(B):
+            n_real = int(torch.randint(Lk - L + 1, Lk + 1, (1,), generator=g))
+            mask[b, n_real:] = 0
+        if Lk - L > 40:
+            mask[:, 10:30] = 0
+    rep = Hq // Hkv
+    q32, k32, v32 = (t.float().requires_grad_() for t in (q, k, v))
+    ref = O.attention_standard(q32, k32.repeat_interleave(rep, dim=1), v32.repeat_interleave(rep, dim=1), D ** -0.5, mask)
+    ref.backward(dout.float())
+    bias = None if mask is None else ((1.0 - mask) * -1e4).to(gpu)
+    out, lse = ops.causal_attention(q.to(gpu), k.to(gpu), v.to(gpu), return_lse=True, key_bias=bias)
+    assert rel_err(out, ref) <= BF16_TOL
+    dq, dk, dv = ops.causal_attention_bwd(q.to(gpu), k.to(gpu), v.to(gpu), out, lse, dout.to(gpu), key_bias=bias)
+    assert rel_err(dv, v32.grad) <= BF16_TOL
+    assert rel_err(dq, q32.grad) <= BF16_TOL
+    assert rel_err(dk, k32.grad) <= BF16_TOL
+
+
+def _linear_cases(n, seed):
+    rng = np.random.default_rng(seed)
+    return [(int(rng.integers(1, 300)), int(rng.integers(1, 40)) * 8, int(rng.integers(1, 48)) * 64,
+             [torch.float32, torch.bfloat16][int(rng.integers(0, 2))]) for _ in range(n)]
+
+
+@pytest.mark.parametrize("T,N,K,dtype", _linear_cases(24, 7))
+def test_linear_random_shapes(gpu, T, N, K, dtype):
+    """Few rows against a weight matrix: plain and K-sliced tilings, whichever the shape selects."""
+    from adaptivetrainingsystem_amd import ops
+    print("case random linear", T, N, K, dtype, ops.down_k_splits(1, T, N, K, dtype), flush=True)
+    g = torch.Generator().manual_seed(T * 7919 + N * 31 + K)
+    x = torch.randn(T, K, generator=g).to(dtype)
+    w = (torch.randn(N, K, generator=g) * 0.05).to(dtype)
+    got = ops.linear_nt(x.to(gpu), w.to(gpu))
+    assert rel_err(got, x.double() @ w.double().T) <= (1e-5 if dtype == torch.float32 else BF16_TOL)
