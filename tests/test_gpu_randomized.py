@@ -82,3 +82,47 @@ def test_linear_random_shapes(gpu, T, N, K, dtype):
     w = (torch.randn(N, K, generator=g) * 0.05).to(dtype)
     got = ops.linear_nt(x.to(gpu), w.to(gpu))
     assert rel_err(got, x.double() @ w.double().T) <= (1e-5 if dtype == torch.float32 else BF16_TOL)
+
+
+def _layer_cases(n, seed):
+    rng = np.random.default_rng(seed)
+    cases = []
+    for _ in range(n):
+        E = int(rng.choice([2, 4, 8, 16, 64]))
+        k = int(rng.integers(1, min(E, 6) + 1))
+        H = int(rng.integers(2, 17)) * 64
+        I = int(rng.integers(2, 17)) * 64
+        T = int(rng.choice([1, 3, 17, 64, 130, 300, 700, 1500]))
+        cf = float(rng.choice([0.5, 1.0, 1.25, 2.0]))
+        dtype = [torch.float32, torch.bfloat16][int(rng.integers(0, 2))]
+        mode = ["fcfs", "none"][int(rng.integers(0, 2))]
+        cases.append((T, H, E, k, I, cf, dtype, mode))
+    return cases
+
+
+@pytest.mark.parametrize("T,H,E,k,I,cf,dtype,mode", _layer_cases(20, 11))
+def test_moe_layer_random_configs(gpu, T, H, E, k, I, cf, dtype, mode):
+    """The whole MoE layer on random small configurations (decode-size, mid-size and prefill tiles, sliced
+    and plain down projections, drops and no drops): integers bit for bit, output to the float bar."""
+    from adaptivetrainingsystem_amd import workloads as W
+    print("case random layer", T, H, E, k, I, cf, dtype, mode, flush=True)
+    ov = {"batch": 1, "seq": T, "hidden": H, "num_experts": E, "top_k": k, "intermediate": I, "capacity_factor": cf,
+          "dtype": dtype, "zipf_bias": 0.0}
+    w = W.make_moe_workload("c1_cpu_reference", device="cpu", overrides=ov)
+    wg = W.make_moe_workload("c1_cpu_reference", device=gpu, overrides=ov)
+    layer = W.build_layer(wg, mode)
+    out, aux = layer(wg.x)
+    p = layer.last_plan
+    logits_gpu = p["logits"].cpu()
+    kw = dict(k=k, temperature=1.0, logits_override=logits_gpu)
+    if mode == "fcfs":
+        ref = O.moe_forward_capacity(w.x, w.gate, w.gate_up, w.down, capacity_factor=cf, routing="softmax_topk", **kw)
+        assert p["capacity"] == ref["capacity"]
+        assert torch.equal(p["token_map"].cpu(), ref["token_map"]) and torch.equal(p["slot"].cpu(), ref["slot"])
+        assert torch.equal(p["kept"].cpu().long(), ref["kept"])
+    else:
+        ref = O.moe_forward_nocap(w.x, w.gate, w.gate_up, w.down, **kw)
+    assert torch.equal(p["indices"].cpu().long(), ref["indices"])
+    assert (p["weights"].cpu() - ref["weights"]).abs().max().item() <= 1e-5
+    assert rel_err(out, ref["out"]) <= (1e-5 if dtype == torch.float32 else BF16_TOL)
+    assert abs(aux.item() - ref["aux"].item()) <= 1e-6
