@@ -1,6 +1,8 @@
 """Seeded random shapes through the attention and K-sliced product paths, against the CPU oracle.  The fixed
 cases elsewhere pin known edges; these sweep the shape space around them (tile remainders, head ratios, cache
 lengths on both sides of the thresholds that switch kernels)."""
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -9,6 +11,8 @@ from oracle import sparse_layer_oracle as O
 
 pytestmark = pytest.mark.gpu
 BF16_TOL = 2e-2
+# ATS_RANDOM_SCALE=10 runs ten times as many cases from the same generators (a deeper sweep by hand)
+SCALE = max(1, int(os.environ.get("ATS_RANDOM_SCALE", "1")))
 
 
 def rel_err(got, ref) -> float:
@@ -36,7 +40,7 @@ def _attention_cases(n, seed):
     return cases
 
 
-@pytest.mark.parametrize("B,Hq,Hkv,L,Lk,D,masked", _attention_cases(36, 2024))
+@pytest.mark.parametrize("B,Hq,Hkv,L,Lk,D,masked", _attention_cases(36 * SCALE, 2024))
 def test_attention_random_shapes(gpu, B, Hq, Hkv, L, Lk, D, masked):
     from adaptivetrainingsystem_amd import ops
     print("case random attention", B, Hq, Hkv, L, Lk, D, masked, flush=True)
@@ -72,7 +76,7 @@ def _linear_cases(n, seed):
              [torch.float32, torch.bfloat16][int(rng.integers(0, 2))]) for _ in range(n)]
 
 
-@pytest.mark.parametrize("T,N,K,dtype", _linear_cases(24, 7))
+@pytest.mark.parametrize("T,N,K,dtype", _linear_cases(24 * SCALE, 7))
 def test_linear_random_shapes(gpu, T, N, K, dtype):
     """Few rows against a weight matrix: plain and K-sliced tilings, whichever the shape selects."""
     from adaptivetrainingsystem_amd import ops
@@ -100,7 +104,7 @@ def _layer_cases(n, seed):
     return cases
 
 
-@pytest.mark.parametrize("T,H,E,k,I,cf,dtype,mode", _layer_cases(20, 11))
+@pytest.mark.parametrize("T,H,E,k,I,cf,dtype,mode", _layer_cases(20 * SCALE, 11))
 def test_moe_layer_random_configs(gpu, T, H, E, k, I, cf, dtype, mode):
     """The whole MoE layer on random small configurations (decode-size, mid-size and prefill tiles, sliced
     and plain down projections, drops and no drops): integers bit for bit, output to the float bar."""
