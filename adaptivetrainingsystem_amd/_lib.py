@@ -44,6 +44,7 @@ _SIGNATURES = {
     "ats_grouped_down_splitk": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64,
                                         c_int, c_int, c_int, c_int, c_void_p]),
     "ats_sum_partials": (c_int, [c_void_p, c_int, c_int64, c_void_p, c_int64, c_int, c_void_p]),
+    "ats_swiglu_partials": (c_int, [c_void_p, c_int, c_int64, c_void_p, c_int64, c_int, c_int, c_void_p]),
     "ats_combine_partials": (c_int, [c_void_p, c_int, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int,
                                      c_int, c_int, c_void_p]),
     "ats_rmsnorm_bwd_workspace": (c_size_t, [c_int64, c_int]),

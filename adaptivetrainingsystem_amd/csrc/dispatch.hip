@@ -483,7 +483,63 @@ __global__ __launch_bounds__(256) void sum_partials_kernel(const float* __restri
     }
 }
 
+// Gate/up projection of a few rows cut along K: parts [n_parts][rows][2I] float32 (gate columns first).
+// out[r, c] = silu(sum_s gate) * (sum_s up), sums in slice order, one rounding to the output type - the
+// arithmetic of the fused gate/up epilogue on the summed accumulators.
+template <typename TO>
+__global__ __launch_bounds__(256) void swiglu_partials_kernel(const float* __restrict__ parts, int n_parts,
+                                                              int64_t part_stride, TO* __restrict__ out, int64_t rows,
+                                                              int I) {
+    const int64_t n4 = rows * (I / 4);
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n4; i += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t r = i / (I / 4);
+        const int c = (int)(i - r * (I / 4)) * 4;
+        const float* p = parts + r * 2 * I + c;
+        float4 g = *reinterpret_cast<const float4*>(p);
+        float4 u = *reinterpret_cast<const float4*>(p + I);
+        for (int s = 1; s < n_parts; ++s) {
+            const float4 gs = *reinterpret_cast<const float4*>(p + s * part_stride);
+            const float4 us = *reinterpret_cast<const float4*>(p + s * part_stride + I);
+            g.x += gs.x; g.y += gs.y; g.z += gs.z; g.w += gs.w;
+            u.x += us.x; u.y += us.y; u.z += us.z; u.w += us.w;
+        }
+        const float4 h = make_float4(silu_f(g.x) * u.x, silu_f(g.y) * u.y, silu_f(g.z) * u.z, silu_f(g.w) * u.w);
+        TO* o = out + r * I + c;
+        if constexpr (sizeof(TO) == 2) {
+            uint2 w;
+            w.x = pack_bf16x2(h.x, h.y);
+            w.y = pack_bf16x2(h.z, h.w);
+            *reinterpret_cast<uint2*>(o) = w;
+        } else {
+            *reinterpret_cast<float4*>(o) = h;
+        }
+    }
+}
+
 }  // namespace ats
+
+extern "C" int ats_swiglu_partials(const float* parts, int n_parts, int64_t part_stride, void* out, int64_t rows, int I,
+                                   int out_dtype, ats_stream_t stream) {
+    using namespace ats;
+    ATS_REQUIRE(n_parts >= 1 && rows >= 0 && I > 0 && I % 4 == 0 && part_stride % 4 == 0 && part_stride >= rows * 2 * I,
+                ATS_ERR_INVALID_ARG, "ats_swiglu_partials: n_parts=%d rows=%lld I=%d part_stride=%lld", n_parts,
+                (long long)rows, I, (long long)part_stride);
+    ATS_REQUIRE(out_dtype == ATS_F32 || out_dtype == ATS_BF16, ATS_ERR_UNSUPPORTED, "ats_swiglu_partials: dtype tag %d",
+                out_dtype);
+    if (rows == 0) return ATS_OK;
+    ATS_REQUIRE(parts && out && aligned16(parts) && (reinterpret_cast<uintptr_t>(out) & 7u) == 0, ATS_ERR_INVALID_ARG,
+                "ats_swiglu_partials: null or misaligned pointer");
+    int64_t blocks = (rows * (I / 4) + 255) / 256;
+    if (blocks > 4096) blocks = 4096;
+    if (out_dtype == ATS_F32)
+        hipLaunchKernelGGL((swiglu_partials_kernel<float>), dim3((unsigned)blocks), dim3(256), 0, as_stream(stream), parts,
+                           n_parts, part_stride, static_cast<float*>(out), rows, I);
+    else
+        hipLaunchKernelGGL((swiglu_partials_kernel<bf16_t>), dim3((unsigned)blocks), dim3(256), 0, as_stream(stream),
+                           parts, n_parts, part_stride, static_cast<bf16_t*>(out), rows, I);
+    ATS_CHECK_LAUNCH("ats_swiglu_partials");
+    return ATS_OK;
+}
 
 extern "C" int ats_sum_partials(const float* parts, int n_parts, int64_t part_stride, void* out, int64_t n,
                                 int out_dtype, ats_stream_t stream) {

@@ -74,13 +74,6 @@ __device__ __forceinline__ void mma_step<float>(const u32x4_t& wfrag, const u32x
     c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(wfrag.w), __uint_as_float(afrag.w), c, 0, 0, 0);
 }
 
-// silu(g) = g / (1 + exp(-g)) with the hardware exp2 and reciprocal (each about 1 ulp): the
-// result is within ~3e-7 relative of the correctly rounded value, far inside the float32 bar.
-__device__ __forceinline__ float silu_f(float g) {
-    const float e = __builtin_amdgcn_exp2f(g * -1.4426950408889634f);
-    return g * __builtin_amdgcn_rcpf(1.0f + e);
-}
-
 // Epilogue through LDS.  In the accumulator layout a lane owns 4 consecutive columns of one row,
 // so storing straight from registers would issue 8-byte pieces of 64 different cache lines per
 // instruction.  Instead every wave transposes 32-row blocks of its sub-tile through a private LDS

@@ -340,7 +340,12 @@ class SwiGLUExpert(nn.Module):
         wd = _as_dtype(self.down_proj.weight, x2.dtype)
         start = torch.zeros(1, dtype=torch.int32, device=x.device)
         count = torch.full((1,), n, dtype=torch.int32, device=x.device)
-        h = ops.grouped_gateup_swiglu(x2, ops.weight_pointer_table([wgu]), start, count, n, n, H, I)
+        gu_splits = ops.down_k_splits(1, n, 2 * I, H, x2.dtype) if I % 8 == 0 and n <= 32 else 1
+        if gu_splits > 1:    # a few rows: the gate/up weight streams through K slices, the activation follows the sum
+            h = ops.swiglu_partials(ops.grouped_down_splitk(x2, ops.weight_pointer_table([wgu]), start, count, n,
+                                                            2 * I, H, gu_splits), x2.dtype)
+        else:
+            h = ops.grouped_gateup_swiglu(x2, ops.weight_pointer_table([wgu]), start, count, n, n, H, I)
         splits = ops.down_k_splits(1, n, H, I, x2.dtype) if H % 8 == 0 else 1
         if splits > 1:       # a few rows: slices of K keep every CU streaming the down weights
             y = ops.sum_partials(ops.grouped_down_splitk(h, ops.weight_pointer_table([wd]), start, count, n, H, I,

@@ -326,6 +326,19 @@ def sum_partials(parts: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
     return out
 
 
+def swiglu_partials(parts: torch.Tensor, out_dtype: torch.dtype) -> torch.Tensor:
+    """parts float32 [S, rows, 2I] (a gate/up projection cut along K, gate columns first) ->
+    silu(sum gate) * (sum up) as [rows, I] of out_dtype."""
+    _need_gpu(parts)
+    if parts.dtype != torch.float32 or parts.dim() != 3 or parts.shape[2] % 8 or not parts.is_contiguous():
+        raise AtsError("swiglu_partials: parts must be a contiguous float32 [slices, rows, 2I] tensor")
+    S, rows, two_i = parts.shape
+    out = torch.empty(rows, two_i // 2, dtype=out_dtype, device=parts.device)
+    check(_lib.load().ats_swiglu_partials(parts.data_ptr(), S, rows * two_i, out.data_ptr(), rows, two_i // 2, _tag(out),
+                                          _stream()), "ats_swiglu_partials")
+    return out
+
+
 # --------------------------------------------------------------------------- combine
 def combine(y: torch.Tensor, row_of: torch.Tensor, weights: torch.Tensor, num_tokens: int, k: int,
             out_dtype: Optional[torch.dtype] = None, residual: Optional[torch.Tensor] = None) -> torch.Tensor:

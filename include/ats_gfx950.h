@@ -156,6 +156,11 @@ int ats_grouped_down(const void* h, const void* const* w_d, void* y, const int32
 int ats_grouped_down_splitk(const void* h, const void* const* w_d, float* parts, const int32_t* row_start,
                             const int32_t* row_count, int E, int64_t max_rows, int64_t part_rows, int H,
                             int I, int k_splits, int dtype, ats_stream_t stream);
+/* A gate/up projection of a few rows cut along K (ats_grouped_down_splitk run on the [2I, H] weight):
+ * parts [n_parts, rows, 2I] float32, gate columns first; out[r,c] = silu(sum_s gate) * (sum_s up), rounded
+ * once to out_dtype -- SwiGLUExpert.forward (model.py:1071-1088) on the summed accumulators.  I % 4 == 0. */
+int ats_swiglu_partials(const float* parts, int n_parts, int64_t part_stride, void* out, int64_t rows, int I,
+                        int out_dtype, ats_stream_t stream);
 /* out[i] = sum_s parts[s*part_stride + i], i < n, added in slice order in float32 and rounded once
  * to out_dtype (n and part_stride multiples of 4). */
 int ats_sum_partials(const float* parts, int n_parts, int64_t part_stride, void* out, int64_t n,

@@ -280,7 +280,7 @@ def test_dispatch_tokens_and_combine_api(A, gpu):
 
 # ------------------------------------------------------------------ expert FFN (grouped GEMMs)
 @pytest.mark.parametrize("n,H,I", [(20, 512, 1408), (70, 512, 1408), (300, 256, 200), (1000, 512, 384), (33, 72, 136),
-                                   (1, 64, 64), (2500, 128, 256)])
+                                   (1, 64, 64), (2500, 128, 256), (8, 1024, 512), (1, 2048, 256), (32, 4096, 128)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_swiglu_expert_single_group(A, gpu, n, H, I, dtype):
     print("case expert", n, H, I, dtype, flush=True)
