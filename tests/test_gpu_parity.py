@@ -543,3 +543,28 @@ def test_fused_swiglu_seam(gpu):
     gate = torch.nn.functional.linear(x, m.gate_proj.weight.cpu())
     up = torch.nn.functional.linear(x, m.up_proj.weight.cpu())
     assert rel_err(got, gate * torch.nn.functional.silu(up)) <= 1e-4   # projections run in the BLAS library
+
+
+def test_decode_ffn_step_replays_in_a_hip_graph(A, gpu):
+    """The K-sliced decode path allocates through torch and launches on the current stream, so a step can be
+    captured: three replays with eager work and synchronisation in between, each equal to the eager result."""
+    from adaptivetrainingsystem_amd.workloads import LayerConfig
+    ffn = A.DenseSwiGLU(LayerConfig(1024, 2048, 1, 1)).to(torch.bfloat16).to(gpu).eval()
+    x = torch.randn(1, 8, 1024, generator=gen(71)).bfloat16().to(gpu)
+    with torch.no_grad():
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):           # warm-up off the capturing stream: tables and caches get built
+            for _ in range(2):
+                ffn(x)
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            y = ffn(x)
+        for rep in range(3):
+            x.copy_(torch.randn(1, 8, 1024, generator=gen(72 + rep)).bfloat16())
+            ref = ffn(x)
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(y, ref), rep
