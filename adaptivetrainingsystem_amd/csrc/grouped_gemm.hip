@@ -777,7 +777,7 @@ static int launch_cfg(const GroupedArgs& p0, int64_t max_rows, hipStream_t s) {
     constexpr int BK = 128 / (int)sizeof(T);
     auto kern_general = grouped_gemm_kernel<T, TO, BM, BN, WM, WN, SM, SN, SWIGLU>;
     // the L2 warm-up touches pay where blocks share operand panels; the weight-streaming tiles share nothing
-    constexpr bool kWarm = BM != 32;
+    constexpr bool kWarm = BM > 64;
     auto kern_pipe = grouped_gemm_pipelined_kernel<T, TO, BM, BN, WM, WN, SM, SN, SWIGLU, kWarm>;
     auto kern_dma = [] {
         if constexpr (DMA) return grouped_gemm_dma_kernel<T, TO, BM, BN, WM, WN, SM, SN, SWIGLU>;
@@ -794,7 +794,7 @@ static int launch_cfg(const GroupedArgs& p0, int64_t max_rows, hipStream_t s) {
         }
     }
     // slices of K: the weight-streaming tiles only, in their own instance of the register-staged kernel
-    constexpr bool kCanSlice = !DMA && !SWIGLU && BM == 32;
+    constexpr bool kCanSlice = !DMA && !SWIGLU && (BM == 32 || BM == 64);
     const int splits = p.k_splits > 1 ? p.k_splits : 1;
     if (splits > 1 && (!kCanSlice || p.k_count || p.K % splits != 0 || (p.K / splits) % BK != 0)) {
         set_error("grouped GEMM: %d slices of K=%d are not available for this tile configuration", splits, p.K);
@@ -826,6 +826,10 @@ static int launch_grouped(const GroupedArgs& p, int64_t max_rows, hipStream_t s)
     const int64_t avg = max_rows / (p.E > 0 ? p.E : 1);
     // (33-48 rows per group would take two 32-row tiles that each stream the weights: measured 1.6x slower
     // than the 128-row tiles on the gate/up projection of 8 experts)
+    if constexpr (!SWIGLU) {
+        // K slices with more than 32 rows per group: 64-row tiles, so that up to 64 rows stream the weights once
+        if (p.k_splits > 1 && avg > 32) return launch_cfg<T, TO, 64, 128, 1, 4, 1, 32, SWIGLU>(p, max_rows, s);
+    }
     if (avg <= 32 || p.k_splits > 1) {
         // Decode: pure weight streaming, 32-row tiles.  (Measured alternatives: narrower tiles with
         // more blocks per CU, and MFMA fragments loaded straight from global memory without LDS,

@@ -97,13 +97,20 @@ class RotaryEmbedding(nn.Module):
         inv_freq = 1.0 / (theta ** (torch.arange(0, dim, 2, dtype=torch.float64) / dim))
         self.register_buffer("inv_freq", inv_freq.float(), persistent=False)
         self._tables: Dict[Any, Tuple[torch.Tensor, torch.Tensor]] = {}
+        self._last: Dict[str, Any] = {"key": None, "views": None}     # the slices handed out last (decoding asks
+                                                                      # for the same length step after step)
 
     def _extend_cache(self, seq_len: int) -> None:
         if seq_len > self.max_seq_len:
             self.max_seq_len = seq_len
             self._tables.clear()
+            self._last["key"] = None
 
     def forward(self, seq_len: int, device) -> Tuple[torch.Tensor, torch.Tensor]:
+        last = self._last
+        if last["key"] == (seq_len, device) and seq_len <= self.max_seq_len:
+            return last["views"]
+        asked = device
         device = torch.device(device)
         if device.type != "cuda":
             raise AtsError("RotaryEmbedding: tables are built on the GPU; pass a cuda device")
@@ -113,7 +120,8 @@ class RotaryEmbedding(nn.Module):
             self._tables[key] = ops.rope_table(self.max_seq_len, self.dim, self.theta, self.scaling_factor,
                                                half=False, device=device)
         cos, sin = self._tables[key]
-        return cos[:seq_len], sin[:seq_len]
+        last["key"], last["views"] = (seq_len, asked), (cos[:seq_len], sin[:seq_len])
+        return last["views"]
 
     def extra_repr(self) -> str:
         return f"dim={self.dim}, max_seq_len={self.max_seq_len}, theta={self.theta}, backend=gfx950"
@@ -210,10 +218,8 @@ class GroupedQueryAttention(nn.Module):
             # one product with the three weights stacked (a copy kept until a weight changes): a third of the
             # launches, which is what a decoding step is made of; q, k, v are column ranges of its output
             lin = lambda a, w: ops.linear_nt(a, _as_dtype(w, a.dtype))
-            qkv = ops.linear_nt(x2, self._stacked_qkv(x.dtype))
-            q = qkv[:, :nh * D].view(B, L, nh, D).transpose(1, 2)
-            k = qkv[:, nh * D:(nh + nkv) * D].view(B, L, nkv, D).transpose(1, 2)
-            v = qkv[:, (nh + nkv) * D:].view(B, L, nkv, D).transpose(1, 2)
+            qkv = ops.linear_nt(x2, self._stacked_qkv(x.dtype)).view(B, L, nh + 2 * nkv, D).transpose(1, 2)
+            q, k, v = qkv[:, :nh], qkv[:, nh:nh + nkv], qkv[:, nh + nkv:]
         # positions 0..L-1 also when a cache is passed, as the reference does (model.py:690-698)
         cos, sin = self.rope(L, x.device)
         q, k = ag.RoPEFunction.apply(q, k, cos, sin, 0) if grad else ops.rope(q, k, cos, sin, 0)

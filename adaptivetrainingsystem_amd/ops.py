@@ -279,9 +279,10 @@ def down_k_splits(E: int, max_rows: int, N: int, K: int, dtype: torch.dtype) -> 
     """Slices of K for a projection with few rows per expert.  Such a product streams its weights, and
     it takes several hundred workgroups to keep the memory system busy; the plain tilings give
     E * ceil(N / 128) of them up to 32 rows per expert and E * ceil(rows / 128) * ceil(N / 256) above.
-    When that is under 384, 32-row tiles with K cut into slices are used instead, if two or more slices
-    are needed to reach 384 (measured on MI355X: 8 x [4096, 14336] weights x 16 rows 199 -> 160 us with
-    2 slices; one [4096, 4096] weight x 64 rows 50 -> 14 us with 8, x 256 rows 51 -> 42 us with 2).
+    When that is under 384, 32-row tiles (64-row tiles above 32 rows) with K cut into slices are used
+    instead, if two or more slices are needed to fill the chip (measured on MI355X: 8 x [4096, 14336]
+    weights x 16 rows 199 -> 160 us with 2 slices; one [4096, 4096] weight x 64 rows 50 -> 10 us with 8,
+    x 256 rows 51 -> 23 us with 2; [4096, 14336] x 64 rows 156 -> 22 us with 8).
     Powers of two up to 16, slices of at least 512 columns, at most 256 rows per expert."""
     slab = 64 if dtype == torch.bfloat16 else 32
     if E <= 0 or max_rows <= 0:
@@ -293,9 +294,11 @@ def down_k_splits(E: int, max_rows: int, N: int, K: int, dtype: torch.dtype) -> 
     plain = E * n128 if max_rows // E <= 32 else E * ((rows + 127) // 128) * ((N + 255) // 256)
     if plain >= 384:
         return 1
-    groups = E * ((rows + 31) // 32) * n128
+    # 32-row tiles (three workgroups per CU) up to 32 rows, 64-row tiles (two per CU) above
+    groups = E * (1 if rows <= 32 else (rows + 63) // 64) * n128
+    enough = 384 if rows <= 32 else 256
     s = 1
-    while s < 16 and groups * s < 384 and K % (2 * s * slab) == 0 and K // (2 * s) >= 512:
+    while s < 16 and groups * s < enough and K % (2 * s * slab) == 0 and K // (2 * s) >= 512:
         s *= 2
     return s
 
