@@ -297,6 +297,145 @@ __global__ __launch_bounds__(256) void rmsnorm_bwd_rows_kernel(const T* __restri
 }
 #undef ATS_WVAL
 
+// Long rows (256-1024 vectors): the 256 lanes of a team (4 waves) share a row, so a lane holds 1-4 vectors of x
+// and of dy, few enough registers for 16 waves per CU; a block is two teams.  A team fetches its next row before
+// the current row's two sums cross its waves through LDS (one block-wide barrier per row; the slots alternate
+// with the row's parity, so a wave that runs ahead never overwrites sums still being read).  At the end team 1
+// leaves its dw slice in LDS and team 0 adds its own: one partial row per block.
+constexpr int kTeamLanes = 256;
+template <typename T, typename WT, int NV, bool HAS_W>
+__global__ __launch_bounds__(512, 2) void rmsnorm_bwd_team_kernel(const T* __restrict__ x, const WT* __restrict__ w,
+                                                                  const T* __restrict__ dy, T* __restrict__ dx,
+                                                                  float* __restrict__ dw_partial, int64_t rows,
+                                                                  int H, float eps) {
+    constexpr int V = Elem<T>::kVec;
+    extern __shared__ float dw_lds[];  // [H] when dw_partial != nullptr
+    __shared__ float red[2][2][8];     // [row parity][team][4 x sum of squares, 4 x dot]
+    const int lane = lane_id();
+    const int team = threadIdx.x >> 8, t = threadIdx.x & (kTeamLanes - 1), wv = t >> 6;
+    const int nvec = H / V;
+    const int64_t stride = (int64_t)gridDim.x * 2;
+    const int64_t first = (int64_t)blockIdx.x * 2;
+    // both teams make the same number of trips (the barrier is block-wide); team 1 may idle through the last one
+    const int64_t trips = first < rows ? (rows - first + stride - 1) / stride : 0;
+
+    float wreg[NV][V], dwacc[NV][V];
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        const int v = t + i * kTeamLanes;
+#pragma unroll
+        for (int j = 0; j < V; ++j) {
+            dwacc[i][j] = 0.f;
+            wreg[i][j] = 1.f;
+            if (HAS_W && v < nvec) wreg[i][j] = Elem<WT>::load(w + (int64_t)v * V + j);
+        }
+    }
+    uint4 xnext[NV], gnext[NV];
+    int64_t row = first + team;
+    if (row < rows) {
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int v = t + i * kTeamLanes;
+            if (v < nvec) {
+                xnext[i] = reinterpret_cast<const uint4*>(x + row * H)[v];
+                gnext[i] = reinterpret_cast<const uint4*>(dy + row * H)[v];
+            }
+        }
+    }
+    for (int64_t trip = 0; trip < trips; ++trip, row += stride) {
+        const bool active = row < rows;
+        uint4 xraw[NV], graw[NV];
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            xraw[i] = xnext[i];
+            graw[i] = gnext[i];
+        }
+        const int64_t nrow = row + stride;
+        if (nrow < rows) {
+#pragma unroll
+            for (int i = 0; i < NV; ++i) {
+                const int v = t + i * kTeamLanes;
+                if (v < nvec) {
+                    xnext[i] = reinterpret_cast<const uint4*>(x + nrow * H)[v];
+                    gnext[i] = reinterpret_cast<const uint4*>(dy + nrow * H)[v];
+                }
+            }
+        }
+        float ss = 0.f, dot = 0.f;
+        if (active) {
+#pragma unroll
+            for (int i = 0; i < NV; ++i) {
+                if (t + i * kTeamLanes < nvec) {
+                    float xf[V], gf[V];
+                    Elem<T>::unpack(xraw[i], xf);
+                    Elem<T>::unpack(graw[i], gf);
+#pragma unroll
+                    for (int j = 0; j < V; ++j) {
+                        ss += xf[j] * xf[j];
+                        dot += gf[j] * wreg[i][j] * xf[j];
+                    }
+                }
+            }
+        }
+        ss = wave_sum(ss);
+        dot = wave_sum(dot);
+        const int par = (int)(trip & 1);
+        if (lane == 0) {
+            red[par][team][wv] = ss;
+            red[par][team][4 + wv] = dot;
+        }
+        __syncthreads();
+        if (active) {
+            const float* rd = red[par][team];
+            ss = ((rd[0] + rd[1]) + rd[2]) + rd[3];
+            dot = ((rd[4] + rd[5]) + rd[6]) + rd[7];
+            const float r = 1.0f / sqrtf(ss / (float)H + eps);
+            const float c = dot / (float)H * r * r * r;
+            uint4* dxr = reinterpret_cast<uint4*>(dx + row * H);
+#pragma unroll
+            for (int i = 0; i < NV; ++i) {
+                const int v = t + i * kTeamLanes;
+                if (v < nvec) {
+                    float xf[V], gf[V], o[V];
+                    Elem<T>::unpack(xraw[i], xf);
+                    Elem<T>::unpack(graw[i], gf);
+#pragma unroll
+                    for (int j = 0; j < V; ++j) {
+                        o[j] = gf[j] * wreg[i][j] * r - xf[j] * c;
+                        dwacc[i][j] += gf[j] * xf[j] * r;
+                    }
+                    dxr[v] = Elem<T>::pack(o);
+                }
+            }
+        }
+    }
+
+    if (dw_partial) {
+        if (team == 1) {
+#pragma unroll
+            for (int i = 0; i < NV; ++i) {
+                const int v = t + i * kTeamLanes;
+                if (v < nvec) {
+#pragma unroll
+                    for (int j = 0; j < V; ++j) dw_lds[v * V + j] = dwacc[i][j];
+                }
+            }
+        }
+        __syncthreads();
+        if (team == 0) {
+            float* mine = dw_partial + (int64_t)blockIdx.x * H;
+#pragma unroll
+            for (int i = 0; i < NV; ++i) {
+                const int v = t + i * kTeamLanes;
+                if (v < nvec) {
+#pragma unroll
+                    for (int j = 0; j < V; ++j) mine[v * V + j] = dwacc[i][j] + dw_lds[v * V + j];
+                }
+            }
+        }
+    }
+}
+
 // Any hidden size / alignment: one wave per row, two scalar passes over the row; every wave owns
 // one partial row of dw in global memory and adds to it row after row.
 template <typename T, typename WT, bool HAS_W>
@@ -359,6 +498,10 @@ __global__ __launch_bounds__(256) void rmsnorm_dw_reduce_kernel(const float* __r
     }
 }
 
+static void launch_dw_reduce(const float* partial, int n_partial, float* dw, int H, hipStream_t s) {
+    hipLaunchKernelGGL(rmsnorm_dw_reduce_kernel, dim3((H + 31) / 32), dim3(256), 0, s, partial, n_partial, dw, H);
+}
+
 constexpr int kBwdBlocksVec = 512;      // vector kernel: two blocks per CU, one partial row per block
 constexpr int kBwdBlocksGeneric = 64;   // generic kernel: one partial row per wave (256 rows)
 
@@ -383,9 +526,25 @@ static int launch_rmsnorm_bwd(const void* x, const void* w, const void* dy, void
                            part, rows, H, eps);
         n_partial = blocks * 4;
     } else {
+        const size_t lds = part ? (size_t)H * sizeof(float) : 0;
+        const int nvec = H / V;
+        if (nvec >= kTeamLanes && nvec <= 4 * kTeamLanes) {
+            const int64_t want = (rows + 1) / 2;
+            const int blocks = (int)(want < kBwdBlocksVec ? want : kBwdBlocksVec);
+            const int per_team_lane = (nvec + kTeamLanes - 1) / kTeamLanes;
+#define ATS_RMSB_TEAM(NV)                                                                                        \
+    hipLaunchKernelGGL((rmsnorm_bwd_team_kernel<T, WT, NV, HAS_W>), dim3(blocks), dim3(512), lds, s, xp, wp, gp, dxp, \
+                       part, rows, H, eps)
+            if (per_team_lane <= 1) ATS_RMSB_TEAM(1);
+            else if (per_team_lane <= 2) ATS_RMSB_TEAM(2);
+            else ATS_RMSB_TEAM(4);
+#undef ATS_RMSB_TEAM
+            if (dw)
+                launch_dw_reduce(partial, blocks, dw, H, s);
+            return ATS_OK;
+        }
         const int64_t want = (rows + 3) / 4;
         const int blocks = (int)(want < kBwdBlocksVec ? want : kBwdBlocksVec);
-        const size_t lds = part ? (size_t)H * sizeof(float) : 0;
         const int per_lane = (H / V + kWave - 1) / kWave;
 #define ATS_RMSB_CASE(NV)                                                                                  \
     hipLaunchKernelGGL((rmsnorm_bwd_rows_kernel<T, WT, NV, HAS_W, (NV * V <= 32)>), dim3(blocks), dim3(256), lds, \
@@ -399,7 +558,7 @@ static int launch_rmsnorm_bwd(const void* x, const void* w, const void* dy, void
         n_partial = blocks;
     }
     if (dw)
-        hipLaunchKernelGGL(rmsnorm_dw_reduce_kernel, dim3((H + 31) / 32), dim3(256), 0, s, partial, n_partial, dw, H);
+        launch_dw_reduce(partial, n_partial, dw, H, s);
     return ATS_OK;
 }
 
