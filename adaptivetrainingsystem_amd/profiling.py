@@ -40,12 +40,13 @@ class StageTimer:
         self._events.clear()
 
     def summary(self) -> Dict[str, Dict[str, float]]:
-        """Synchronises once and returns {stage: {calls, mean_ms, min_ms, total_ms}}."""
+        """Synchronises once and returns {stage: {calls, mean_ms, min_ms, total_ms, median_ms, max_ms}}."""
         torch.cuda.synchronize()
         out = {}
         for name, pairs in self._events.items():
             ms = [a.elapsed_time(b) for a, b in pairs]
-            out[name] = {"calls": len(ms), "mean_ms": sum(ms) / len(ms), "min_ms": min(ms), "total_ms": sum(ms)}
+            out[name] = {"calls": len(ms), "mean_ms": sum(ms) / len(ms), "min_ms": min(ms), "total_ms": sum(ms),
+                         "median_ms": sorted(ms)[len(ms) // 2], "max_ms": max(ms)}
         return out
 
 
