@@ -138,9 +138,13 @@ def _ffn_forward(x, wgu, wd, offsets, kept, rows, row_src, k):
     Returns (gu [rows, 2I], h [rows, I], y [rows, H])."""
     H, I = x.shape[1], wd[0].shape[1]
     tab_gu, tab_d = ops.weight_pointer_table(wgu), ops.weight_pointer_table(wd)
-    gu = ops.grouped_gemm_nt(tab_gu, H, 2 * I, offsets, kept, rows, rows, 2 * I, H, a=x, a_rows=row_src,
-                             a_row_div=k)
-    h = ops.silu_mul(gu[:, :I], gu[:, I:], rows_dev=offsets[-1:])      # only the kept rows
+    both = ops.grouped_gateup_swiglu_save(x, tab_gu, offsets, kept, rows, rows, H, I, a_rows=row_src, a_row_div=k)
+    if both is not None:             # prefill-sized groups: one kernel writes the pre-activations and h
+        gu, h = both
+    else:
+        gu = ops.grouped_gemm_nt(tab_gu, H, 2 * I, offsets, kept, rows, rows, 2 * I, H, a=x, a_rows=row_src,
+                                 a_row_div=k)
+        h = ops.silu_mul(gu[:, :I], gu[:, I:], rows_dev=offsets[-1:])      # only the kept rows
     y = ops.grouped_down(h, tab_d, offsets, kept, rows, H, I)
     return gu, h, y
 

@@ -49,6 +49,9 @@ struct GroupedArgs {
     int64_t part_stride;
     // direct-to-LDS path only: bytes addressable from the A / B descriptors (0 = path not usable)
     uint32_t a_extent_bytes, b_extent_bytes;
+    // training forward (direct-to-LDS SwiGLU kernel only): the gate / up pre-activations, [*, 2 * N_out]
+    void* gu_out;
+    int64_t ld_gu;
 };
 
 constexpr int kRowPitch = 144;  // bytes per staged row: 128 data + 16 pad
@@ -79,9 +82,13 @@ __device__ __forceinline__ void mma_step<float>(const u32x4_t& wfrag, const u32x
 // instruction.  Instead every wave transposes 32-row blocks of its sub-tile through a private LDS
 // region and writes whole rows: 16 bytes per lane, 128-byte lines fully covered.
 // wstage: this wave's private region, 32 * (WCOLS * sizeof(TO) + 16) bytes.
-template <typename TO, int TM, int TN, bool SWIGLU>
+// SAVEGU (with SWIGLU): the gate and up accumulators themselves also go to gu[row, col] and gu[row, up_off + col]
+// (what the backward pass of a training step needs), through the same staging region.
+template <typename TO, int TM, int TN, bool SWIGLU, bool SAVEGU = false>
 __device__ __forceinline__ void epilogue_staged(f32x16_t (&acc)[TN][TM], unsigned char* wstage, TO* out, int64_t ldo,
-                                                int64_t row_base, int rows_valid, int ncol0, int n_out, int lane) {
+                                                int64_t row_base, int rows_valid, int ncol0, int n_out, int lane,
+                                                TO* gu = nullptr, int64_t ldgu = 0, int up_off = 0) {
+    static_assert(!SAVEGU || SWIGLU, "the second output exists for the SwiGLU epilogue only");
     constexpr int TNO = SWIGLU ? TN / 2 : TN;
     constexpr int WCOLS = TNO * 32;
     constexpr int ES = (int)sizeof(TO);
@@ -125,6 +132,40 @@ __device__ __forceinline__ void epilogue_staged(f32x16_t (&acc)[TN][TM], unsigne
                 *reinterpret_cast<u32x4_t*>(out + (row_base + m_local) * ldo + col) = data;
         }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        if constexpr (SAVEGU) {
+#pragma unroll
+            for (int half = 0; half < 2; ++half) {
+#pragma unroll
+                for (int j = 0; j < TNO; ++j) {
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const int jj = j + half * (TN / 2);
+                        unsigned char* dst = wstage + frow * PITCH + (j * 32 + 8 * q + 4 * fgrp) * ES;
+                        if constexpr (ES == 2) {
+                            uint2 u;
+                            u.x = pack_bf16x2(acc[jj][i][q * 4 + 0], acc[jj][i][q * 4 + 1]);
+                            u.y = pack_bf16x2(acc[jj][i][q * 4 + 2], acc[jj][i][q * 4 + 3]);
+                            *reinterpret_cast<uint2*>(dst) = u;
+                        } else {
+                            *reinterpret_cast<float4*>(dst) = make_float4(acc[jj][i][q * 4 + 0], acc[jj][i][q * 4 + 1],
+                                                                          acc[jj][i][q * 4 + 2], acc[jj][i][q * 4 + 3]);
+                        }
+                    }
+                }
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+                for (int r0 = 0; r0 < 32; r0 += RPI) {
+                    const int r = r0 + lane / LPR;
+                    const int c = lane % LPR;
+                    const u32x4_t data = *reinterpret_cast<const u32x4_t*>(wstage + r * PITCH + c * 16);
+                    const int m_local = i * 32 + r;
+                    const int col = ncol0 + c * EPC;
+                    if (m_local < rows_valid && col < n_out)
+                        *reinterpret_cast<u32x4_t*>(gu + (row_base + m_local) * ldgu + half * up_off + col) = data;
+                }
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            }
+        }
     }
 }
 
@@ -578,7 +619,7 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_pipelined_kernel(Gro
 //   issue the loads of slab t+2 into the stage slab t occupied
 //   k-step 3     : MFMAs | fragment reads of k-step 0 of slab t+1
 // so a slab has a whole slab of MFMA time to land.
-template <typename T, typename TO, int BM, int BN, int WM, int WN, int SM, int SN, bool SWIGLU>
+template <typename T, typename TO, int BM, int BN, int WM, int WN, int SM, int SN, bool SWIGLU, bool SAVEGU = false>
 __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_dma_kernel(GroupedArgs p) {
 #if defined(__HIP_DEVICE_COMPILE__)
     constexpr int NW = WM * WN;
@@ -756,8 +797,9 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_dma_kernel(GroupedAr
         constexpr int WSTAGE = 32 * (TNO_ * 32 * (int)sizeof(TO) + 16);
         const int wrow = tc.mt * BM + wm * (BM / WM);
         const int ncol0 = SWIGLU ? tc.nt * HALF + wn * (BN / WN / 2) : tc.nt * BN + wn * (BN / WN);
-        epilogue_staged<TO, TM, TN, SWIGLU>(acc, smem + wave * WSTAGE, static_cast<TO*>(p.out), p.ldo,
-                                            (int64_t)row0 + wrow, count - wrow, ncol0, p.N_out, lane);
+        epilogue_staged<TO, TM, TN, SWIGLU, SAVEGU>(acc, smem + wave * WSTAGE, static_cast<TO*>(p.out), p.ldo,
+                                                    (int64_t)row0 + wrow, count - wrow, ncol0, p.N_out, lane,
+                                                    static_cast<TO*>(p.gu_out), p.ld_gu, p.up_offset);
     }
 #endif
 }
@@ -850,6 +892,42 @@ static int launch_grouped(const GroupedArgs& p, int64_t max_rows, hipStream_t s)
     return launch_cfg<T, TO, 256, 256, 2, 4, 4, 8, SWIGLU, true>(p, max_rows, s);
 }
 
+static bool extent32_ok(int64_t rows, int64_t row_elems, int elem_size) {
+    return rows > 0 && rows <= (int64_t)0xffffffffLL / (row_elems * elem_size);
+}
+
+// Training forward: the prefill tile of the direct-to-LDS kernel with both outputs.  Other group sizes and
+// operands beyond 32-bit lane offsets take the two-kernel route (plain product, then silu(g) * u).
+constexpr int64_t kSaveGuMinAvgRows = 768;
+template <typename T>
+static bool gateup_save_supported(int64_t a_rows_total, int E, int64_t max_rows, int H, int I) {
+    constexpr int BK = 128 / (int)sizeof(T);
+    if (E <= 0 || max_rows / E <= kSaveGuMinAvgRows || H % BK != 0 || I % (16 / (int)sizeof(T)) != 0) return false;
+    return extent32_ok(a_rows_total, H, (int)sizeof(T)) && extent32_ok(2 * (int64_t)I, H, (int)sizeof(T));
+}
+
+template <typename T>
+static int launch_gateup_save(const GroupedArgs& p0, int64_t max_rows, hipStream_t s) {
+    constexpr int BM = 256, BN = 256;
+    GroupedArgs p = p0;
+    p.n_tiles = (p.N_out + BN / 2 - 1) / (BN / 2);
+    constexpr size_t smem = 2 * (size_t)(BM + BN) * kRowPitch;
+    auto kern = grouped_gemm_dma_kernel<T, T, BM, BN, 2, 4, 4, 8, true, true>;
+    static LdsReservation reserved;
+    hipError_t e = reserve_lds(reserved, {reinterpret_cast<const void*>(kern)}, (int)smem);
+    if (e != hipSuccess) {
+        set_error("grouped GEMM: cannot reserve %zu bytes of LDS: %s", smem, hipGetErrorString(e));
+        return ATS_ERR_LAUNCH;
+    }
+    const int64_t blocks = grid_blocks(max_rows, p.E, BM, p.n_tiles, 4, 8);
+    if (blocks > 0x7fffffffLL) {
+        set_error("grouped GEMM: grid of %lld blocks", (long long)blocks);
+        return ATS_ERR_UNSUPPORTED;
+    }
+    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(512), smem, s, p);
+    return ATS_OK;
+}
+
 // Bytes reachable from a buffer descriptor, or 0 when they do not fit its 32-bit range.
 static uint32_t extent32(int64_t rows, int64_t row_elems, int elem_size) {
     if (rows <= 0 || rows > (int64_t)0xffffffffLL / (row_elems * elem_size)) return 0;
@@ -871,6 +949,56 @@ static int check_common(const char* name, const void* a, const void* const* w, c
 }
 
 }  // namespace ats
+
+extern "C" int ats_grouped_gateup_swiglu_save_supported(int64_t a_num_rows, int E, int64_t max_rows, int H, int I,
+                                                        int dtype) {
+    using namespace ats;
+    if (H <= 0 || I <= 0) return 0;
+    if (dtype == ATS_F32) return gateup_save_supported<float>(a_num_rows, E, max_rows, H, I) ? 1 : 0;
+    if (dtype == ATS_BF16) return gateup_save_supported<bf16_t>(a_num_rows, E, max_rows, H, I) ? 1 : 0;
+    return 0;
+}
+
+extern "C" int ats_grouped_gateup_swiglu_save(const void* a, int64_t a_num_rows, const int32_t* a_rows, int a_row_div,
+                                              const void* const* w_gu, void* h, void* gu, const int32_t* row_start,
+                                              const int32_t* row_count, int E, int64_t max_rows, int H, int I,
+                                              int dtype, ats_stream_t stream) {
+    using namespace ats;
+    int rc = check_common("ats_grouped_gateup_swiglu_save", a, w_gu, h, row_start, row_count, E, max_rows, H, I, dtype);
+    if (rc != ATS_OK) return rc;
+    ATS_REQUIRE(gu && aligned16(gu), ATS_ERR_INVALID_ARG, "ats_grouped_gateup_swiglu_save: gu must be a 16-byte aligned buffer");
+    ATS_REQUIRE(a_num_rows > 0 && (!a_rows || a_row_div > 0), ATS_ERR_INVALID_ARG,
+                "ats_grouped_gateup_swiglu_save: a_row_div=%d a_num_rows=%lld", a_row_div, (long long)a_num_rows);
+    ATS_REQUIRE(ats_grouped_gateup_swiglu_save_supported(a_num_rows, E, max_rows, H, I, dtype), ATS_ERR_UNSUPPORTED,
+                "ats_grouped_gateup_swiglu_save: needs more than %lld rows per expert on average, H a multiple of the "
+                "K slab and operands within 4 GiB (E=%d max_rows=%lld H=%d I=%d); use the plain product and "
+                "ats_silu_mul_fwd", (long long)kSaveGuMinAvgRows, E, (long long)max_rows, H, I);
+    GroupedArgs p{};
+    p.a = a;
+    p.a_rows = a_rows;
+    p.a_row_div = a_rows ? a_row_div : 1;
+    p.lda = H;
+    p.b = w_gu;
+    p.ldb = H;
+    p.out = h;
+    p.ldo = I;
+    p.gu_out = gu;
+    p.ld_gu = 2 * (int64_t)I;
+    p.row_start = row_start;
+    p.row_count = row_count;
+    p.E = E;
+    p.K = H;
+    p.N_out = I;
+    p.up_offset = I;
+    const int es = dtype == ATS_F32 ? 4 : 2;
+    p.a_extent_bytes = extent32(a_num_rows, H, es);
+    p.b_extent_bytes = extent32(2 * (int64_t)I, H, es);
+    hipStream_t s = as_stream(stream);
+    rc = dtype == ATS_F32 ? launch_gateup_save<float>(p, max_rows, s) : launch_gateup_save<bf16_t>(p, max_rows, s);
+    if (rc != ATS_OK) return rc;
+    ATS_CHECK_LAUNCH("ats_grouped_gateup_swiglu_save");
+    return ATS_OK;
+}
 
 extern "C" int ats_grouped_gateup_swiglu(const void* a, int64_t a_num_rows, const int32_t* a_rows, int a_row_div,
                                          const void* const* w_gu, void* h, const int32_t* row_start,

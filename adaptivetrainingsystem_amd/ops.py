@@ -260,6 +260,30 @@ def grouped_gateup_swiglu(a: torch.Tensor, w_gu_ptrs: torch.Tensor, row_start: t
     return h
 
 
+def grouped_gateup_swiglu_save(a: torch.Tensor, w_gu_ptrs: torch.Tensor, row_start: torch.Tensor,
+                               row_count: torch.Tensor, n_rows_out: int, max_rows: int, H: int, I: int,
+                               a_rows: Optional[torch.Tensor] = None,
+                               a_row_div: int = 1) -> Optional[Tuple[torch.Tensor, torch.Tensor]]:
+    """Training forward of the gate/up projection: (gu [rows, 2I], h [rows, I]) from one kernel, or None when
+    the sizes are not prefill-sized (the caller then runs the plain product and silu_mul)."""
+    _need_gpu(a, w_gu_ptrs, row_start, row_count, a_rows)
+    if a.dim() != 2 or a.shape[1] != H or not a.is_contiguous():
+        raise AtsError("grouped_gateup_swiglu_save: activations must be a contiguous [rows, H] tensor")
+    E = w_gu_ptrs.numel()
+    if row_start.numel() < E or row_count.numel() < E or row_start.dtype != torch.int32 or row_count.dtype != torch.int32:
+        raise AtsError("grouped_gateup_swiglu_save: row_start/row_count must be int32 with one entry per expert")
+    lib = _lib.load()
+    if not lib.ats_grouped_gateup_swiglu_save_supported(int(a.shape[0]), E, int(max_rows), H, I, _tag(a)):
+        return None
+    h = torch.empty(n_rows_out, I, dtype=a.dtype, device=a.device)
+    gu = torch.empty(n_rows_out, 2 * I, dtype=a.dtype, device=a.device)
+    check(lib.ats_grouped_gateup_swiglu_save(a.data_ptr(), int(a.shape[0]), _ptr(a_rows), int(a_row_div),
+                                             w_gu_ptrs.data_ptr(), h.data_ptr(), gu.data_ptr(), row_start.data_ptr(),
+                                             row_count.data_ptr(), E, int(max_rows), H, I, _tag(a), _stream()),
+          "ats_grouped_gateup_swiglu_save")
+    return gu, h
+
+
 def grouped_down(h: torch.Tensor, w_d_ptrs: torch.Tensor, row_start: torch.Tensor, row_count: torch.Tensor,
                  max_rows: int, H: int, I: int, out: Optional[torch.Tensor] = None,
                  out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:

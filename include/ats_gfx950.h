@@ -147,6 +147,19 @@ int ats_grouped_gateup_swiglu(const void* a, int64_t a_num_rows, const int32_t* 
 int ats_grouped_down(const void* h, const void* const* w_d, void* y, const int32_t* row_start,
                      const int32_t* row_count, int E, int64_t max_rows, int H, int I, int dtype,
                      int y_dtype, ats_stream_t stream);
+/* The same projection for a training step: beside h it writes the gate / up pre-activations
+ * gu[r, 0:I] and gu[r, I:2I] ([rows, 2I] of dtype, rounded from the same accumulators), which the
+ * backward pass needs; replaces the plain product followed by ats_silu_mul_fwd (reference: the
+ * expert's gate_proj / up_proj outputs kept by autograd, MS/core/model.py:882-893).  Available for
+ * prefill-sized groups only: ..._save_supported returns 1 when it is (more than 768 rows per expert
+ * on average, H a multiple of the 128-byte K slab, `a` and one expert's weights within 4 GiB),
+ * otherwise the entry point fails with ATS_ERR_UNSUPPORTED. */
+int ats_grouped_gateup_swiglu_save_supported(int64_t a_num_rows, int E, int64_t max_rows, int H, int I,
+                                             int dtype);
+int ats_grouped_gateup_swiglu_save(const void* a, int64_t a_num_rows, const int32_t* a_rows, int a_row_div,
+                                   const void* const* w_gu, void* h, void* gu, const int32_t* row_start,
+                                   const int32_t* row_count, int E, int64_t max_rows, int H, int I,
+                                   int dtype, ats_stream_t stream);
 /* The down projection of weight-streaming (decode) sizes, at most 256 rows per expert, split along
  * K so that enough workgroups stream the weights: slice s of expert e multiplies columns
  * [s*I/k_splits, (s+1)*I/k_splits) and writes float32 parts[s][row_start[e]+m][:H]
