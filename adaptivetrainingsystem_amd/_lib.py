@@ -39,6 +39,9 @@ _SIGNATURES = {
     "ats_invert_token_map": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p]),
     "ats_grouped_gateup_swiglu": (c_int, [c_void_p, c_int64, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
                                           c_int64, c_int, c_int, c_int, c_void_p]),
+    "ats_grouped_down_dgrad_dsilu_supported": (c_int, [c_int, c_int64, c_int, c_int, c_int]),
+    "ats_grouped_down_dgrad_dsilu": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64,
+                                             c_int, c_int, c_int, c_void_p]),
     "ats_grouped_gateup_swiglu_save_supported": (c_int, [c_int64, c_int, c_int64, c_int, c_int, c_int]),
     "ats_grouped_gateup_swiglu_save": (c_int, [c_void_p, c_int64, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                                                c_void_p, c_int, c_int64, c_int, c_int, c_int, c_void_p]),

@@ -157,9 +157,11 @@ def _ffn_backward(dy, x, wgu, wd, gu, h, offsets, kept, rows, row_src, k, need_x
     H, I = x.shape[1], wd[0].shape[1]
     dtype, dev = x.dtype, x.device
     wdT, tab_dT = ops.transpose_batched(wd)                      # [I, H] per expert; kept alive until return
-    dh = ops.grouped_gemm_nt(tab_dT, H, I, offsets, kept, rows, rows, I, H, a=dy)
-    dgu = torch.empty_like(gu)
-    ops.silu_mul_bwd(gu[:, :I], gu[:, I:], dh, da=dgu[:, :I], db=dgu[:, I:], rows_dev=offsets[-1:])
+    dgu = ops.grouped_down_dgrad_dsilu(dy, tab_dT, gu, offsets, kept, rows, H, I)   # prefill-sized groups: one kernel
+    if dgu is None:
+        dh = ops.grouped_gemm_nt(tab_dT, H, I, offsets, kept, rows, rows, I, H, a=dy)
+        dgu = torch.empty_like(gu)
+        ops.silu_mul_bwd(gu[:, :I], gu[:, I:], dh, da=dgu[:, :I], db=dgu[:, I:], rows_dev=offsets[-1:])
     dx_rows = dwgu = dwd = None
     if need_x:
         wguT, tab_guT = ops.transpose_batched(wgu)               # [H, 2I] per expert

@@ -8,12 +8,6 @@
 
 namespace ats {
 
-// sigmoid with the hardware exp2 and reciprocal (each about 1 ulp): a few 1e-7 relative, well inside the
-// float32 bar of the gradients.
-__device__ __forceinline__ float sigmoid_f(float v) {
-    return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(v * -1.4426950408889634f));
-}
-
 // ---------------------------------------------------------------- silu(a) * b
 // out[r, c] = silu(a[r, c]) * b[r, c]; operands addressed as base + r * ld + c.
 template <typename T>

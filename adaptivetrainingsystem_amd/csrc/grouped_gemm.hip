@@ -49,7 +49,8 @@ struct GroupedArgs {
     int64_t part_stride;
     // direct-to-LDS path only: bytes addressable from the A / B descriptors (0 = path not usable)
     uint32_t a_extent_bytes, b_extent_bytes;
-    // training forward (direct-to-LDS SwiGLU kernel only): the gate / up pre-activations, [*, 2 * N_out]
+    // training (direct-to-LDS kernel only): the gate / up pre-activations, [*, 2 * N_out]; written by the
+    // forward instance, read by the instance whose epilogue turns dh into the gradients of g and u
     void* gu_out;
     int64_t ld_gu;
 };
@@ -84,11 +85,16 @@ __device__ __forceinline__ void mma_step<float>(const u32x4_t& wfrag, const u32x
 // wstage: this wave's private region, 32 * (WCOLS * sizeof(TO) + 16) bytes.
 // SAVEGU (with SWIGLU): the gate and up accumulators themselves also go to gu[row, col] and gu[row, up_off + col]
 // (what the backward pass of a training step needs), through the same staging region.
-template <typename TO, int TM, int TN, bool SWIGLU, bool SAVEGU = false>
+// DSILU (without SWIGLU): the tile is dh, the gradient of h = silu(g) * u; instead of storing it, every lane reads
+// the 16 bytes of g and of u that belong to its 16 bytes of dh (rounded to TO first, as a stored dh would be) from
+// gu and stores dg = dh * u * (s + g*s*(1-s)) and du = dh * g * s, s = sigmoid(g), to out[row, col] and
+// out[row, up_off + col]: the arithmetic of the elementwise gradient kernel, so the bits are the same.
+template <typename TO, int TM, int TN, bool SWIGLU, bool SAVEGU = false, bool DSILU = false>
 __device__ __forceinline__ void epilogue_staged(f32x16_t (&acc)[TN][TM], unsigned char* wstage, TO* out, int64_t ldo,
                                                 int64_t row_base, int rows_valid, int ncol0, int n_out, int lane,
                                                 TO* gu = nullptr, int64_t ldgu = 0, int up_off = 0) {
     static_assert(!SAVEGU || SWIGLU, "the second output exists for the SwiGLU epilogue only");
+    static_assert(!DSILU || !SWIGLU, "the SwiGLU gradient epilogue belongs to the plain product");
     constexpr int TNO = SWIGLU ? TN / 2 : TN;
     constexpr int WCOLS = TNO * 32;
     constexpr int ES = (int)sizeof(TO);
@@ -128,8 +134,27 @@ __device__ __forceinline__ void epilogue_staged(f32x16_t (&acc)[TN][TM], unsigne
             const u32x4_t data = *reinterpret_cast<const u32x4_t*>(wstage + r * PITCH + c * 16);
             const int m_local = i * 32 + r;
             const int col = ncol0 + c * EPC;
-            if (m_local < rows_valid && col < n_out)
-                *reinterpret_cast<u32x4_t*>(out + (row_base + m_local) * ldo + col) = data;
+            if constexpr (DSILU) {
+                if (m_local < rows_valid && col < n_out) {
+                    const TO* gp = gu + (row_base + m_local) * ldgu + col;
+                    TO* dp = out + (row_base + m_local) * ldo + col;
+                    float gv[EPC], uv[EPC], dv[EPC], og[EPC], ou[EPC];
+                    Elem<TO>::unpack(*reinterpret_cast<const uint4*>(gp), gv);
+                    Elem<TO>::unpack(*reinterpret_cast<const uint4*>(gp + up_off), uv);
+                    Elem<TO>::unpack(make_uint4(data[0], data[1], data[2], data[3]), dv);
+#pragma unroll
+                    for (int e = 0; e < EPC; ++e) {
+                        const float sg = sigmoid_f(gv[e]);
+                        og[e] = dv[e] * uv[e] * (sg + gv[e] * sg * (1.0f - sg));
+                        ou[e] = dv[e] * (gv[e] * sg);
+                    }
+                    *reinterpret_cast<uint4*>(dp) = Elem<TO>::pack(og);
+                    *reinterpret_cast<uint4*>(dp + up_off) = Elem<TO>::pack(ou);
+                }
+            } else {
+                if (m_local < rows_valid && col < n_out)
+                    *reinterpret_cast<u32x4_t*>(out + (row_base + m_local) * ldo + col) = data;
+            }
         }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         if constexpr (SAVEGU) {
@@ -619,7 +644,8 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_pipelined_kernel(Gro
 //   issue the loads of slab t+2 into the stage slab t occupied
 //   k-step 3     : MFMAs | fragment reads of k-step 0 of slab t+1
 // so a slab has a whole slab of MFMA time to land.
-template <typename T, typename TO, int BM, int BN, int WM, int WN, int SM, int SN, bool SWIGLU, bool SAVEGU = false>
+template <typename T, typename TO, int BM, int BN, int WM, int WN, int SM, int SN, bool SWIGLU, bool SAVEGU = false,
+          bool DSILU = false>
 __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_dma_kernel(GroupedArgs p) {
 #if defined(__HIP_DEVICE_COMPILE__)
     constexpr int NW = WM * WN;
@@ -797,7 +823,7 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_dma_kernel(GroupedAr
         constexpr int WSTAGE = 32 * (TNO_ * 32 * (int)sizeof(TO) + 16);
         const int wrow = tc.mt * BM + wm * (BM / WM);
         const int ncol0 = SWIGLU ? tc.nt * HALF + wn * (BN / WN / 2) : tc.nt * BN + wn * (BN / WN);
-        epilogue_staged<TO, TM, TN, SWIGLU, SAVEGU>(acc, smem + wave * WSTAGE, static_cast<TO*>(p.out), p.ldo,
+        epilogue_staged<TO, TM, TN, SWIGLU, SAVEGU, DSILU>(acc, smem + wave * WSTAGE, static_cast<TO*>(p.out), p.ldo,
                                                     (int64_t)row0 + wrow, count - wrow, ncol0, p.N_out, lane,
                                                     static_cast<TO*>(p.gu_out), p.ld_gu, p.up_offset);
     }
@@ -928,6 +954,37 @@ static int launch_gateup_save(const GroupedArgs& p0, int64_t max_rows, hipStream
     return ATS_OK;
 }
 
+// Training backward: dh = dy . Wd with the SwiGLU gradient in the epilogue (prefill tile of the direct-to-LDS kernel).
+constexpr int64_t kDsiluMinAvgRows = 256;
+template <typename T>
+static bool down_dgrad_dsilu_supported(int E, int64_t max_rows, int H, int I) {
+    constexpr int BK = 128 / (int)sizeof(T);
+    if (E <= 0 || max_rows / E <= kDsiluMinAvgRows || H % BK != 0 || I % (16 / (int)sizeof(T)) != 0) return false;
+    return extent32_ok(I, H, (int)sizeof(T));
+}
+
+template <typename T>
+static int launch_down_dgrad_dsilu(const GroupedArgs& p0, int64_t max_rows, hipStream_t s) {
+    constexpr int BM = 256, BN = 256;
+    GroupedArgs p = p0;
+    p.n_tiles = (p.N_out + BN - 1) / BN;
+    constexpr size_t smem = 2 * (size_t)(BM + BN) * kRowPitch;
+    auto kern = grouped_gemm_dma_kernel<T, T, BM, BN, 2, 4, 4, 8, false, false, true>;
+    static LdsReservation reserved;
+    hipError_t e = reserve_lds(reserved, {reinterpret_cast<const void*>(kern)}, (int)smem);
+    if (e != hipSuccess) {
+        set_error("grouped GEMM: cannot reserve %zu bytes of LDS: %s", smem, hipGetErrorString(e));
+        return ATS_ERR_LAUNCH;
+    }
+    const int64_t blocks = grid_blocks(max_rows, p.E, BM, p.n_tiles, 4, 8);
+    if (blocks > 0x7fffffffLL) {
+        set_error("grouped GEMM: grid of %lld blocks", (long long)blocks);
+        return ATS_ERR_UNSUPPORTED;
+    }
+    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(512), smem, s, p);
+    return ATS_OK;
+}
+
 // Bytes reachable from a buffer descriptor, or 0 when they do not fit its 32-bit range.
 static uint32_t extent32(int64_t rows, int64_t row_elems, int elem_size) {
     if (rows <= 0 || rows > (int64_t)0xffffffffLL / (row_elems * elem_size)) return 0;
@@ -997,6 +1054,52 @@ extern "C" int ats_grouped_gateup_swiglu_save(const void* a, int64_t a_num_rows,
     rc = dtype == ATS_F32 ? launch_gateup_save<float>(p, max_rows, s) : launch_gateup_save<bf16_t>(p, max_rows, s);
     if (rc != ATS_OK) return rc;
     ATS_CHECK_LAUNCH("ats_grouped_gateup_swiglu_save");
+    return ATS_OK;
+}
+
+extern "C" int ats_grouped_down_dgrad_dsilu_supported(int E, int64_t max_rows, int H, int I, int dtype) {
+    using namespace ats;
+    if (H <= 0 || I <= 0) return 0;
+    if (dtype == ATS_F32) return down_dgrad_dsilu_supported<float>(E, max_rows, H, I) ? 1 : 0;
+    if (dtype == ATS_BF16) return down_dgrad_dsilu_supported<bf16_t>(E, max_rows, H, I) ? 1 : 0;
+    return 0;
+}
+
+extern "C" int ats_grouped_down_dgrad_dsilu(const void* dy, const void* const* w_dT, const void* gu, void* dgu,
+                                            const int32_t* row_start, const int32_t* row_count, int E,
+                                            int64_t max_rows, int H, int I, int dtype, ats_stream_t stream) {
+    using namespace ats;
+    int rc = check_common("ats_grouped_down_dgrad_dsilu", dy, w_dT, dgu, row_start, row_count, E, max_rows, H, I, dtype);
+    if (rc != ATS_OK) return rc;
+    ATS_REQUIRE(gu && aligned16(gu), ATS_ERR_INVALID_ARG, "ats_grouped_down_dgrad_dsilu: gu must be a 16-byte aligned buffer");
+    ATS_REQUIRE(ats_grouped_down_dgrad_dsilu_supported(E, max_rows, H, I, dtype), ATS_ERR_UNSUPPORTED,
+                "ats_grouped_down_dgrad_dsilu: needs more than %lld rows per expert on average, H a multiple of the K "
+                "slab and one expert's weights within 4 GiB (E=%d max_rows=%lld H=%d I=%d); use ats_grouped_gemm_nt and "
+                "ats_silu_mul_bwd", (long long)kDsiluMinAvgRows, E, (long long)max_rows, H, I);
+    if (max_rows == 0) return ATS_OK;
+    GroupedArgs p{};
+    p.a = dy;
+    p.a_row_div = 1;
+    p.lda = H;
+    p.b = w_dT;
+    p.ldb = H;
+    p.out = dgu;
+    p.ldo = 2 * (int64_t)I;
+    p.gu_out = const_cast<void*>(gu);
+    p.ld_gu = 2 * (int64_t)I;
+    p.row_start = row_start;
+    p.row_count = row_count;
+    p.E = E;
+    p.K = H;
+    p.N_out = I;
+    p.up_offset = I;
+    const int es = dtype == ATS_F32 ? 4 : 2;
+    p.a_extent_bytes = 0xffffffffu;       // the descriptor starts at the tile's first row
+    p.b_extent_bytes = extent32(I, H, es);
+    hipStream_t s = as_stream(stream);
+    rc = dtype == ATS_F32 ? launch_down_dgrad_dsilu<float>(p, max_rows, s) : launch_down_dgrad_dsilu<bf16_t>(p, max_rows, s);
+    if (rc != ATS_OK) return rc;
+    ATS_CHECK_LAUNCH("ats_grouped_down_dgrad_dsilu");
     return ATS_OK;
 }
 

@@ -284,6 +284,29 @@ def grouped_gateup_swiglu_save(a: torch.Tensor, w_gu_ptrs: torch.Tensor, row_sta
     return gu, h
 
 
+def grouped_down_dgrad_dsilu(dy: torch.Tensor, w_dT_ptrs: torch.Tensor, gu: torch.Tensor, row_start: torch.Tensor,
+                             row_count: torch.Tensor, max_rows: int, H: int, I: int) -> Optional[torch.Tensor]:
+    """Training backward of the down projection and of silu(g) * u in one kernel: dgu [rows, 2I] from dy [rows, H],
+    the transposed down weights ([I, H] per expert) and the saved gu; None when the groups are not prefill-sized
+    (the caller then runs the plain product and silu_mul_bwd)."""
+    _need_gpu(dy, w_dT_ptrs, gu, row_start, row_count)
+    if dy.dim() != 2 or dy.shape[1] != H or not dy.is_contiguous():
+        raise AtsError("grouped_down_dgrad_dsilu: dy must be a contiguous [rows, H] tensor")
+    if gu.dim() != 2 or gu.shape[1] != 2 * I or not gu.is_contiguous() or gu.dtype != dy.dtype or gu.shape[0] < dy.shape[0]:
+        raise AtsError("grouped_down_dgrad_dsilu: gu must be a contiguous [rows, 2I] tensor of dy's dtype")
+    E = w_dT_ptrs.numel()
+    if row_start.numel() < E or row_count.numel() < E or row_start.dtype != torch.int32 or row_count.dtype != torch.int32:
+        raise AtsError("grouped_down_dgrad_dsilu: row_start/row_count must be int32 with one entry per expert")
+    lib = _lib.load()
+    if not lib.ats_grouped_down_dgrad_dsilu_supported(E, int(max_rows), H, I, _tag(dy)):
+        return None
+    dgu = torch.empty_like(gu)
+    check(lib.ats_grouped_down_dgrad_dsilu(dy.data_ptr(), w_dT_ptrs.data_ptr(), gu.data_ptr(), dgu.data_ptr(),
+                                           row_start.data_ptr(), row_count.data_ptr(), E, int(max_rows), H, I,
+                                           _tag(dy), _stream()), "ats_grouped_down_dgrad_dsilu")
+    return dgu
+
+
 def grouped_down(h: torch.Tensor, w_d_ptrs: torch.Tensor, row_start: torch.Tensor, row_count: torch.Tensor,
                  max_rows: int, H: int, I: int, out: Optional[torch.Tensor] = None,
                  out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:

@@ -147,6 +147,17 @@ int ats_grouped_gateup_swiglu(const void* a, int64_t a_num_rows, const int32_t* 
 int ats_grouped_down(const void* h, const void* const* w_d, void* y, const int32_t* row_start,
                      const int32_t* row_count, int E, int64_t max_rows, int H, int I, int dtype,
                      int y_dtype, ats_stream_t stream);
+/* Backward of that pair for a training step: dh = dy . w_d (as the NT product against the
+ * transposed weights w_dT[e] = [I, H]) with the gradient of h = silu(g) * u applied in the epilogue:
+ * dgu[r, 0:I] = dh * u * (s + g*s*(1-s)), dgu[r, I:2I] = dh * g * s, s = sigmoid(g), g/u read from
+ * gu [rows, 2I]; dh itself is never stored.  Same bits as ats_grouped_gemm_nt followed by
+ * ats_silu_mul_bwd (reference: SwiGLUFunction.backward, MS/core/cuda_opt_wrapper.py:237-254, after
+ * autograd's down_proj gradient).  ..._supported returns 1 for more than 256 rows per expert on
+ * average, H a multiple of the 128-byte K slab and one expert's weights within 4 GiB. */
+int ats_grouped_down_dgrad_dsilu_supported(int E, int64_t max_rows, int H, int I, int dtype);
+int ats_grouped_down_dgrad_dsilu(const void* dy, const void* const* w_dT, const void* gu, void* dgu,
+                                 const int32_t* row_start, const int32_t* row_count, int E, int64_t max_rows,
+                                 int H, int I, int dtype, ats_stream_t stream);
 /* The same projection for a training step: beside h it writes the gate / up pre-activations
  * gu[r, 0:I] and gu[r, I:2I] ([rows, 2I] of dtype, rounded from the same accumulators), which the
  * backward pass needs; replaces the plain product followed by ats_silu_mul_fwd (reference: the

@@ -654,3 +654,48 @@ def test_grouped_gateup_with_saved_preactivations(ops, gpu, counts, H, I, gather
     # below the prefill tile the caller keeps the two-kernel route
     small = torch.tensor([40] * E, dtype=torch.int32, device=gpu)
     assert ops.grouped_gateup_swiglu_save(a, tab, start, small, n, 40 * E, H, I, **kw) is None
+
+
+@pytest.mark.parametrize("counts,H,I", [([900, 0, 300, 1001], 256, 392), ([2100, 777], 512, 1024), ([300], 128, 136)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_grouped_down_dgrad_with_swiglu_gradient(ops, gpu, counts, H, I, dtype):
+    """Training backward in one kernel: dgu has the bits of the plain product dh = dy . Wd followed by the
+    elementwise gradient of silu(g) * u, agrees with the float64 formula, leaves rows outside the groups
+    alone, and declines sizes below the prefill tile."""
+    print("case dgrad dsilu", counts, H, I, dtype, flush=True)
+    g = gen(67)
+    E, n = len(counts), sum(counts)
+    wdT = [(torch.randn(I, H, generator=g) * 0.05).to(dtype).to(gpu) for _ in range(E)]     # Wd^T per expert
+    tab = ops.weight_pointer_table(wdT)
+    count = torch.tensor(counts, dtype=torch.int32)
+    start = (torch.cumsum(count, 0) - count).to(torch.int32).to(gpu)
+    count = count.to(gpu)
+    pad = 5
+    dy = torch.randn(n + pad, H, generator=g).to(dtype).to(gpu)
+    gu = torch.randn(n + pad, 2 * I, generator=g).to(dtype).to(gpu)
+    dgu = ops.grouped_down_dgrad_dsilu(dy, tab, gu, start, count, n, H, I)
+    assert dgu is not None and dgu.shape == gu.shape and dgu.dtype == dtype
+    dh = ops.grouped_gemm_nt(tab, H, I, start, count, n + pad, n, I, H, a=dy)
+    two = torch.empty_like(gu)
+    ops.silu_mul_bwd(gu[:n, :I], gu[:n, I:], dh[:n], da=two[:n, :I], db=two[:n, I:])
+    assert same_bits(dgu[:n], two[:n])
+    off = 0
+    for e, c in enumerate(counts):
+        if c:
+            dh64 = dy[off:off + c].cpu().double() @ wdT[e].cpu().double().T
+            if dtype == torch.bfloat16:
+                dh64 = dh64.bfloat16().double()                 # dh is rounded before the gradient, as when stored
+            g64, u64 = gu[off:off + c, :I].cpu().double(), gu[off:off + c, I:].cpu().double()
+            s64 = torch.sigmoid(g64)
+            ref = torch.cat([dh64 * u64 * (s64 + g64 * s64 * (1 - s64)), dh64 * g64 * s64], dim=1)
+            assert rel_err(dgu[off:off + c], ref) <= (F32_TOL if dtype == torch.float32 else BF16_TOL)
+        off += c
+    lib = __import__("adaptivetrainingsystem_amd._lib", fromlist=["load"]).load()
+    dgu.fill_(3.0)
+    rc = lib.ats_grouped_down_dgrad_dsilu(dy.data_ptr(), tab.data_ptr(), gu.data_ptr(), dgu.data_ptr(), start.data_ptr(),
+                                          count.data_ptr(), E, n, H, I, 0 if dtype == torch.float32 else 1, None)
+    assert rc == 0
+    torch.cuda.synchronize()
+    assert torch.all(dgu[n:] == 3.0) and same_bits(dgu[:n], two[:n])
+    small = torch.tensor([40] * E, dtype=torch.int32, device=gpu)
+    assert ops.grouped_down_dgrad_dsilu(dy, tab, gu, start, small, 40 * E, H, I) is None
