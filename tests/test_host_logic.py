@@ -165,3 +165,14 @@ def test_workloads_are_reproducible():
     assert torch.allclose(c.logit_bias, 1.5 * torch.log(1.0 / torch.arange(1, 9).float()))
     n = W.make_norm_rope_workload(device="cpu", batch=1, seq=8)
     assert n.q.shape == (1, 16, 8, 128) and n.k.shape == (1, 4, 8, 128) and n.norm_weight.dtype == torch.float32
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """The path runs on one GPU: asking the benchmark for more exits with a message instead of measuring."""
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    for argv, env in ((["--gpus", "2"], {}), ([], {"WORLD_SIZE": "2"})):
+        r = subprocess.run([sys.executable, os.path.join(root, "bench.py"), *argv], capture_output=True, text=True,
+                           env={**os.environ, **env}, timeout=300)
+        assert r.returncode == 2 and "one GPU" in r.stderr and r.stdout.strip() == ""
