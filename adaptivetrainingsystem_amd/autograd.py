@@ -242,8 +242,7 @@ class MoEFunction(Function):
         if logits_route is logits:
             aux = route["aux"][0]
         else:   # importance from the noise-free logits (model.py:1190-1192)
-            colsum = ops.route_topk(logits, k, 1.0, cfg["variant"], cfg["load_balancing_weight"])["prob_colsum"]
-            aux = torch.clamp((usage * (colsum / T)).sum() * (E * cfg["load_balancing_weight"]), max=1.0)
+            aux = ops.aux_loss_clean_logits(logits, route["hist"], k, cfg["variant"], cfg["load_balancing_weight"])
         plan = ops.dispatch_plan(route["indices"], E, C)
         rows = min(T * k, E * C)
         if rows > 0:

@@ -473,11 +473,15 @@ class MoEFFNLayer(nn.Module):
         tm = self.stage_timer
         with stage(tm, "router_logits"):
             logits = ops.router_logits(x_flat, _as_dtype(self.gate.weight, x.dtype), self.router_logit_bias)
+        clean_logits = logits
         if self.training and self.noise_std > 0:
             logits = logits + torch.randn_like(logits) * self.noise_std
         variant = {"softmax_topk": ROUTE_SOFTMAX_TOPK, "topk_softmax": ROUTE_TOPK_SOFTMAX}[self.routing]
         with stage(tm, "route_topk"):
             route = ops.route_topk(logits, k, self.routing_temperature, variant, self.load_balancing_weight)
+            if logits is not clean_logits:      # importance comes from the noise-free logits (model.py:1190-1192)
+                route["aux"] = ops.aux_loss_clean_logits(clean_logits, route["hist"], k, variant,
+                                                         self.load_balancing_weight).reshape(1)
         with stage(tm, "dispatch_plan"):
             plan = ops.dispatch_plan(route["indices"], E, C)
         rows = min(T * k, E * C)

@@ -164,6 +164,16 @@ def route_topk(logits: torch.Tensor, k: int, temperature: float = 1.0, variant: 
     return {"indices": idx, "weights": w, "hist": hist, "prob_colsum": colsum, "aux": aux}
 
 
+def aux_loss_clean_logits(clean_logits: torch.Tensor, hist: torch.Tensor, k: int, variant: int,
+                          load_balancing_weight: float) -> torch.Tensor:
+    """Load-balancing loss when routing ran on noisy logits: usage from the routed histogram, importance from
+    the noise-free, un-tempered logits (MS/core/model.py:1190-1192, 1244-1263).  Returns a float32 scalar."""
+    T, E = clean_logits.shape
+    colsum = route_topk(clean_logits, k, 1.0, variant, load_balancing_weight)["prob_colsum"]
+    usage = hist.float() / (T * k + 1e-9)
+    return torch.clamp((usage * (colsum / T)).sum() * (E * load_balancing_weight), max=1.0)
+
+
 # --------------------------------------------------------------------------- dispatch
 def expert_capacity(total_tokens: int, top_k: int, num_experts: int, capacity_factor: float) -> int:
     """Host-side integer, in double arithmetic then truncated, exactly as the reference computes it."""

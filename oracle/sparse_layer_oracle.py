@@ -31,7 +31,9 @@ PINNING = {
     "rmsnorm": "closed form in float64 numpy; unit row-RMS invariant; torch.nn.functional.rms_norm",
     "rope_table": "closed form with math.cos/math.sin in float64; pos 0 and d 0 special cases",
     "rope_apply": "2x2 rotation closed form per pair in float64; norm preservation; R(p)R(-p)=I; relative-position identity",
-    "fused_rope_apply": "same closed form; equals rope_apply with a half-width table and an offset",
+    "fused_rope_table": "both halves (cos and sin) against math.cos/math.sin of pos * theta^(-d/half) in float64; "
+                        "sin(1) > 0 at position 1; agreement with both halves of rope_table",
+    "fused_rope_apply": "per-element 2x2 rotation in float64 with an offset; equals rope_apply with a half-width table",
     "router_logits": "float64 matmul",
     "route_softmax_topk_renorm": "brute-force full sort on tiny inputs; index set equals route_topk_softmax; weights sum to 1",
     "route_topk_softmax": "brute-force full sort on tiny inputs; weights sum to 1",
@@ -39,10 +41,21 @@ PINNING = {
     "dispatch_loop": "literal restatement; stable-counting-sort closed form (dispatch_vectorized); C restatement; invariants",
     "combine_loop": "literal restatement; equals no-capacity formulation when nothing is dropped; linearity in weights",
     "swiglu_expert": "float64 closed form with explicit sigmoid",
-    "moe_nocap_forward": "dense brute force: sum over all experts of mask*weight*expert(x)",
+    "moe_forward_nocap": "dense brute force: sum over all experts of mask*weight*expert(x)",
     "aux_loss": "uniform routing gives exactly load_balancing_weight; float64 closed form",
+    "mod_router_probs": "float64 closed form 1/(1+exp(-(x.w+b)/T)) with bias != 0 and temperature != 1; "
+                        "w = 0 gives sigmoid(b/T); p(x)+p(-x) = 1 without bias",
     "mod_router_eval_mask": "sorted-threshold brute force",
     "mod_select_per_sequence": "argsort brute force (composition defined by the benchmark config, not a reference function)",
+    "mod_moe_block": "scores against a float64 matmul + bias; selection against a brute-force sort; skipped tokens "
+                     "bit-identical to the input, kept tokens = input + capacity layer output",
+    "dispatch_plan_vectorized": "same three-formulation check as dispatch_loop (slot, hist, kept)",
+    "dispatch_vectorized": "equals dispatch_loop element for element",
+    "combine_vectorized": "equals combine_loop",
+    "experts_on_slots": "per-slot swiglu_expert (itself pinned in float64); empty slots stay zero",
+    "moe_nocap_compute": "dense brute force over all experts",
+    "moe_forward_capacity": "composition of pinned parts; equals the no-capacity layer when nothing is dropped; "
+                            "hand-worked drop cases",
     "rmsnorm_backward": "torch.autograd of rmsnorm in float64; torch.autograd.gradcheck",
     "rope_backward": "torch.autograd of rope_apply; R(p)^T = R(-p)",
     "swiglu_backward": "torch.autograd of gate*silu(up) in float64; gradcheck",

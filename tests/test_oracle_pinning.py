@@ -142,6 +142,48 @@ def test_fused_rope_matches_full_table_form():
     assert torch.allclose(ch, c64[:, : D // 2], atol=1e-5)
 
 
+def test_fused_rope_table_both_halves_closed_form():
+    """cos AND sin of the half-width float32 table against math.cos / math.sin of pos * theta^(-d/half);
+    a negated or swapped sin half fails here (sin(1) > 0 at position 1, frequency 1)."""
+    D, theta, L = 16, 10000.0, 40
+    ch, sh = O.fused_rope_table(L, D, theta)
+    half = D // 2
+    assert ch.shape == (L, half) and sh.shape == (L, half) and ch.dtype == torch.float32
+    for pos in (0, 1, 2, 5, 17, 39):
+        for d in range(half):
+            ang = pos * theta ** (-d / half)
+            # float32 frequency and product rounding: relative 2^-23 each on an angle of up to 39
+            tol = 3e-7 + 2.5e-7 * abs(ang)
+            assert abs(ch[pos, d].item() - math.cos(ang)) <= tol, (pos, d)
+            assert abs(sh[pos, d].item() - math.sin(ang)) <= tol, (pos, d)
+    assert torch.all(ch[0] == 1) and torch.all(sh[0] == 0)
+    assert abs(sh[1, 0].item() - math.sin(1.0)) <= 1e-7 and sh[1, 0].item() > 0.8
+    assert abs(ch[1, 0].item() - math.cos(1.0)) <= 1e-7
+    # and against the float64-derived full table, both halves of it
+    c64, s64 = O.rope_table(L, D, theta)
+    assert torch.allclose(ch, c64[:, :half], atol=1e-5) and torch.allclose(ch, c64[:, half:], atol=1e-5)
+    assert torch.allclose(sh, s64[:, :half], atol=1e-5) and torch.allclose(sh, s64[:, half:], atol=1e-5)
+
+
+def test_fused_rope_apply_rotation_closed_form():
+    """The fused form rotates pair (d, d + D/2) of position p + offset by +angle: checked per element
+    in float64 with an offset, so the sign of the sin half is fixed independently of the table."""
+    B, Hq, Hkv, L, D, off, theta = 1, 2, 1, 5, 8, 3, 10000.0
+    q = torch.randn(B, Hq, L, D, generator=g(111))
+    k = torch.randn(B, Hkv, L, D, generator=g(112))
+    ch, sh = O.fused_rope_table(16, D, theta)
+    qf, kf = O.fused_rope_apply(q, k, ch, sh, off)
+    half = D // 2
+    for x, y in ((q, qf), (k, kf)):
+        for h in range(x.shape[1]):
+            for p in range(L):
+                for d in range(half):
+                    ang = (p + off) * theta ** (-d / half)
+                    a, b = x[0, h, p, d].item(), x[0, h, p, d + half].item()
+                    assert abs(y[0, h, p, d].item() - (a * math.cos(ang) - b * math.sin(ang))) <= 2e-6
+                    assert abs(y[0, h, p, d + half].item() - (a * math.sin(ang) + b * math.cos(ang))) <= 2e-6
+
+
 def test_rope_bf16_single_rounding():
     q = torch.randn(1, 2, 4, 8, generator=g(13)).bfloat16()
     k = torch.randn(1, 1, 4, 8, generator=g(14)).bfloat16()
@@ -345,6 +387,62 @@ def test_temperature_changes_weights_not_indices():
 
 
 # ------------------------------------------------------------------ MoD
+def test_mod_router_probs_closed_form_f64():
+    """sigmoid((x.w + b) / T) written out in float64 with bias != 0 and temperature != 1: a dropped
+    bias, a temperature that multiplies or sits outside the sigmoid, or a transposed weight fails."""
+    gen = g(135)
+    B, L, H = 2, 9, 24
+    x = torch.randn(B, L, H, generator=gen)
+    w = torch.randn(1, H, generator=gen) * 0.3
+    for b, T in ((0.0, 1.0), (0.7, 1.0), (-0.4, 2.5), (1.3, 0.5)):
+        bias = torch.tensor([b])
+        p = O.mod_router_probs(x, w, bias, T)
+        assert p.shape == (B, L, 1) and p.dtype == torch.float32
+        xd, wd = x.double().numpy(), w.double().numpy()[0]
+        for bi in range(B):
+            for li in range(L):
+                z = (float(np.dot(xd[bi, li], wd)) + b) / T
+                assert abs(p[bi, li, 0].item() - 1.0 / (1.0 + math.exp(-z))) <= 2e-7
+    # no bias at all == zero bias
+    assert torch.equal(O.mod_router_probs(x, w, None, 1.7), O.mod_router_probs(x, w, torch.zeros(1), 1.7))
+
+
+def test_mod_router_probs_special_cases():
+    x = torch.randn(3, 4, 8, generator=g(136))
+    # w = 0: every token gets sigmoid(b / T)
+    for b, T in ((0.9, 3.0), (-2.0, 0.25)):
+        p = O.mod_router_probs(x, torch.zeros(1, 8), torch.tensor([b]), T)
+        assert torch.allclose(p, torch.full_like(p, 1.0 / (1.0 + math.exp(-b / T))), atol=1e-7)
+    # w = 0, b = 0: exactly one half
+    assert torch.all(O.mod_router_probs(x, torch.zeros(1, 8), None, 1.0) == 0.5)
+    # monotone in the bias, antisymmetric in the sign of the input: p(x) + p(-x) = 1 without bias
+    w = torch.randn(1, 8, generator=g(137))
+    assert torch.allclose(O.mod_router_probs(x, w, None, 2.0) + O.mod_router_probs(-x, w, None, 2.0),
+                          torch.ones(3, 4, 1), atol=1e-6)
+    assert torch.all(O.mod_router_probs(x, w, torch.tensor([1.0]), 2.0) > O.mod_router_probs(x, w, None, 2.0))
+    # a larger temperature pulls every probability toward one half
+    far = (O.mod_router_probs(x, w, None, 1.0) - 0.5).abs()
+    near = (O.mod_router_probs(x, w, None, 4.0) - 0.5).abs()
+    assert torch.all(near <= far)
+
+
+def test_mod_moe_block_scores_and_selection_f64():
+    """The block's scores are x.w + b in float64 terms and its selection is the brute-force top-keep of them."""
+    gen = g(138)
+    B, L, H, I, E, keep = 2, 12, 16, 24, 4, 3
+    x = torch.randn(B, L, H, generator=gen)
+    wm = torch.randn(1, H, generator=gen)
+    bm = torch.tensor([0.25])
+    _, wg, wgu, wd = _tiny_layer(139, H=H, I=I, E=E)
+    r = O.mod_moe_block(x, wm, bm, keep, dict(gate_weight=wg, gate_up_weights=wgu, down_weights=wd,
+                                              k=2, capacity_factor=1.5))
+    ref = (x.double() @ wm.double().T).squeeze(-1) + 0.25
+    assert torch.allclose(r["scores"].double(), ref, atol=1e-5)
+    for b in range(B):
+        order = sorted(range(L), key=lambda i: (-ref[b, i].item(), i))[:keep]
+        assert r["selected"][b].tolist() == sorted(order)
+
+
 def test_mod_eval_mask_threshold():
     p = torch.rand(2, 16, 1, generator=g(35))
     mask = O.mod_router_eval_mask(p, 0.5)
@@ -646,3 +744,11 @@ def test_gqa_forward_matches_per_head_composition():
         heads.append(a[:, 0])
     ref = torch.cat(heads, dim=-1) @ wo.double().T
     assert torch.allclose(out.double(), ref, atol=2e-5)
+
+
+def test_every_oracle_function_declares_its_pin():
+    """Every function of the oracle names the independent check that fixes it; none is left out."""
+    import inspect
+    fns = [n for n, f in inspect.getmembers(O, inspect.isfunction) if f.__module__ == O.__name__]
+    assert sorted(fns) == sorted(O.PINNING), set(fns) ^ set(O.PINNING)
+    assert not [n for n, why in O.PINNING.items() if "unpinned" in why]
