@@ -100,6 +100,13 @@ _SIGNATURES = {
     "ats_scatter_add_rows": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int, c_void_p]),
     "ats_kth_value_mask": (c_int, [c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_size_t, c_void_p]),
     "ats_swiglu_mul": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int, c_void_p]),
+    # the reference's launcher names (void return, float32 only)
+    "rms_norm_launcher": (None, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_float, c_void_p]),
+    "rope_precompute_launcher": (None, [c_void_p, c_void_p, c_int, c_int, c_float, c_void_p]),
+    "rope_apply_launcher": (None, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
+                                   c_void_p]),
+    "swiglu_launcher": (None, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p]),
+    "ats_legacy_last_status": (c_int, []),
     "ats_debug_decode_tile": (c_int, [c_int64, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "ats_debug_grid_blocks": (c_int64, [c_int64, c_int, c_int, c_int, c_int, c_int]),
 }

@@ -55,6 +55,41 @@ class RoPEFunction(Function):
         return gq, gk, None, None, None
 
 
+class GatherRowsFunction(Function):
+    """out[i] = x[rows[i]] for x [N, H] and distinct int32 rows; the gradient is the scatter-add of the
+    cotangent rows onto zeros (every other row of x gets none)."""
+
+    @staticmethod
+    def forward(ctx, x, rows):
+        ctx.save_for_backward(rows)
+        ctx.n = x.shape[0]
+        return ops.gather_rows(x.contiguous(), rows)
+
+    @staticmethod
+    def backward(ctx, dout):
+        (rows,) = ctx.saved_tensors
+        dx = torch.zeros(ctx.n, dout.shape[1], dtype=dout.dtype, device=dout.device)
+        ops.scatter_add_rows(dx, rows, dout.contiguous())
+        return dx, None
+
+
+class ScatterAddRowsFunction(Function):
+    """out = x with out[rows[i]] += delta[i] (distinct rows), out of place: the cotangent passes to x
+    unchanged and its selected rows are the gradient of delta."""
+
+    @staticmethod
+    def forward(ctx, x, rows, delta):
+        ctx.save_for_backward(rows)
+        out = x.contiguous().clone()
+        ops.scatter_add_rows(out, rows, delta.to(out.dtype))
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        (rows,) = ctx.saved_tensors
+        return dout, None, ops.gather_rows(dout.contiguous(), rows)
+
+
 class AttentionFunction(Function):
     """Causal grouped-query attention: q [B,Hq,L,D], k, v [B,Hkv,Lk,D] -> [B, L, Hq*D]; key_bias
     [B, Lk] float32 or None (a constant: it gets no gradient)."""

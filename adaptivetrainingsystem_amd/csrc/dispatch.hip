@@ -306,12 +306,15 @@ __global__ __launch_bounds__(256) void combine_kernel(const TY* __restrict__ y, 
             if (rj >= 0 && (rj < my_row || (rj == my_row && j < lane))) ++my_rank;
         }
         const int n_kept = __popcll(__ballot(my_row >= 0));
-        for (int h0 = lane * 4; h0 < H; h0 += kWave * 4) {
+        // the column loop is wave-uniform (every lane makes every trip, lanes past the end with nh = 0): the
+        // ballots and shuffles inside need lanes 0..k-1 active on the last, partial trip as well
+        for (int hb = 0; hb < H; hb += kWave * 4) {
+            const int h0 = hb + lane * 4;
             float acc[4] = {0.f, 0.f, 0.f, 0.f};
-            const int nh = min(4, H - h0);
+            const int nh = max(0, min(4, H - h0));
             for (int n = 0; n < n_kept; ++n) {
                 const unsigned long long who = __ballot(my_row >= 0 && my_rank == n);
-                const int src = __ffsll((long long)who) - 1;
+                const int src = who ? __ffsll((long long)who) - 1 : 0;
                 const int64_t row = __shfl(my_row, src, 64);
                 const float wt = __shfl(my_w, src, 64);
                 const TY* yr = y + row * H + h0;

@@ -145,7 +145,8 @@ __device__ __forceinline__ uint32_t order_key(float f) {
 }
 
 __global__ __launch_bounds__(1024) void kth_value_kernel(const float* __restrict__ v, int64_t n, int64_t kth,
-                                                         uint32_t* __restrict__ key_out) {
+                                                         uint32_t* __restrict__ key_out,
+                                                         long long* __restrict__ count_out) {
     __shared__ unsigned int hist[256];
     __shared__ uint32_t s_prefix;
     __shared__ long long s_rank;
@@ -175,7 +176,12 @@ __global__ __launch_bounds__(1024) void kth_value_kernel(const float* __restrict
         }
         __syncthreads();
     }
-    if (threadIdx.x == 0) key_out[0] = s_prefix;
+    if (threadIdx.x == 0) {
+        key_out[0] = s_prefix;
+        // s_rank is now the 1-based rank of the k-th value among the values equal to it, so kth - s_rank values
+        // are strictly smaller and the mask keeps the rest
+        if (count_out) count_out[0] = (long long)n - kth + s_rank;
+    }
 }
 
 __global__ __launch_bounds__(256) void threshold_mask_kernel(const float* __restrict__ v, int64_t n,
@@ -296,7 +302,8 @@ extern "C" int ats_kth_value_mask(const float* v, int64_t n, int64_t kth, float*
                 "ats_kth_value_mask: workspace of at least 4 bytes needed");
     hipStream_t s = as_stream(stream);
     uint32_t* key = static_cast<uint32_t*>(workspace);
-    hipLaunchKernelGGL(kth_value_kernel, dim3(1), dim3(1024), 0, s, v, n, kth, key);
+    long long* count = workspace_bytes >= 16 ? reinterpret_cast<long long*>(static_cast<char*>(workspace) + 8) : nullptr;
+    hipLaunchKernelGGL(kth_value_kernel, dim3(1), dim3(1024), 0, s, v, n, kth, key, count);
     ATS_CHECK_LAUNCH("ats_kth_value_mask(select)");
     int64_t blocks = (n + 255) / 256;
     if (blocks > 4096) blocks = 4096;

@@ -600,6 +600,7 @@ class MoDRouter(nn.Module):
         self.routing_temperature = routing_temperature
         self.router = nn.Linear(hidden_size, 1, bias=True)
         self._routing_stats = {"total_tokens": 0, "computed_tokens": 0, "skipped_tokens": 0}
+        self._computed_dev = None
         nn.init.normal_(self.router.weight, mean=0.0, std=0.01)
         nn.init.zeros_(self.router.bias)
 
@@ -612,18 +613,41 @@ class MoDRouter(nn.Module):
                                self.routing_temperature, want_prob=True)
         total = B * L
         capacity = int(total * self.capacity_factor)
-        mask = ops.kth_value_mask(probs, max(1, total - capacity))
+        mask, done = ops.kth_value_mask(probs, max(1, total - capacity), return_count=True)
         self._routing_stats["total_tokens"] += total
+        # computed / skipped counts (model.py:990-995): the select kernel leaves the count on the device and it is
+        # accumulated there; it is read, with the one synchronisation that costs, only when the statistics are
+        # asked for
+        if self._computed_dev is None or self._computed_dev.device != done.device:
+            self._flush_counts()
+            self._computed_dev = done
+        else:
+            self._computed_dev += done
         return mask.view(B, L, 1), probs.view(B, L, 1), None
 
+    def _flush_counts(self) -> None:
+        if self._computed_dev is not None:
+            self._routing_stats["computed_tokens"] += float(self._computed_dev.item())
+            self._computed_dev = None
+        self._routing_stats["skipped_tokens"] = (self._routing_stats["total_tokens"]
+                                                 - self._routing_stats["computed_tokens"])
+
     def get_routing_stats(self) -> Dict[str, Any]:
+        """Keys of MS/core/model.py:998-1011."""
+        self._flush_counts()
         total = self._routing_stats["total_tokens"]
         if total == 0:
             return {"error": "No routing statistics available"}
-        return {"total_tokens_routed": total, "target_capacity": self.capacity_factor}
+        return {"total_tokens_routed": total,
+                "computed_tokens": self._routing_stats["computed_tokens"],
+                "skipped_tokens": self._routing_stats["skipped_tokens"],
+                "compute_ratio": self._routing_stats["computed_tokens"] / total,
+                "skip_ratio": self._routing_stats["skipped_tokens"] / total,
+                "target_capacity": self.capacity_factor}
 
     def reset_routing_stats(self) -> None:
         self._routing_stats = {"total_tokens": 0, "computed_tokens": 0, "skipped_tokens": 0}
+        self._computed_dev = None
 
 
 class MoDMoEBlock(nn.Module):
@@ -644,11 +668,19 @@ class MoDMoEBlock(nn.Module):
         keep = int(L * self.keep_fraction)
         scores = ops.row_dot(x, _as_dtype(self.router.weight, x.dtype))
         sel = ops.select_topk_per_sequence(scores.view(B, L), keep)
-        gathered = ops.gather_rows(x.reshape(-1, H), sel)
-        delta, aux = self.moe(gathered.view(1, B * keep, H))
-        out = x.reshape(-1, H).clone()
-        ops.scatter_add_rows(out, sel, delta.view(-1, H))
         self.last_selected = sel
+        x_rows = x.reshape(-1, H)
+        if _wants_grad(x, *self.moe.parameters()):
+            # the selection is discrete, so the score weight gets no gradient (as in the composition the
+            # benchmark defines); tokens, gate and experts get theirs through the gather / scatter pair
+            gathered = ag.GatherRowsFunction.apply(x_rows, sel)
+            delta, aux = self.moe(gathered.view(1, B * keep, H))
+            out = ag.ScatterAddRowsFunction.apply(x_rows, sel, delta.view(-1, H))
+            return out.view(B, L, H), aux
+        gathered = ops.gather_rows(x_rows, sel)
+        delta, aux = self.moe(gathered.view(1, B * keep, H))
+        out = x_rows.clone()
+        ops.scatter_add_rows(out, sel, delta.view(-1, H))
         return out.view(B, L, H), aux
 
 

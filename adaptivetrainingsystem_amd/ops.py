@@ -488,17 +488,19 @@ def scatter_add_rows(base: torch.Tensor, rows: torch.Tensor, delta: torch.Tensor
     return base
 
 
-def kth_value_mask(values: torch.Tensor, kth: int) -> torch.Tensor:
-    """float32 mask of values >= the kth smallest value (1-based), same shape as `values`."""
+def kth_value_mask(values: torch.Tensor, kth: int, return_count: bool = False):
+    """float32 mask of values >= the kth smallest value (1-based), same shape as `values`; with
+    `return_count` also the number of ones as a one-element int64 device tensor (written by the kernel)."""
     _need_gpu(values)
     if values.dtype != torch.float32:
         raise AtsError("kth_value_mask: values must be float32")
     v = values.contiguous()
     mask = torch.empty_like(v)
-    ws = torch.empty(16, dtype=torch.uint8, device=v.device)
+    ws = torch.zeros(2, dtype=torch.int64, device=v.device) if v.numel() == 0 else \
+        torch.empty(2, dtype=torch.int64, device=v.device)
     check(_lib.load().ats_kth_value_mask(v.data_ptr(), v.numel(), int(kth), mask.data_ptr(), ws.data_ptr(), 16,
                                          _stream()), "ats_kth_value_mask")
-    return mask
+    return (mask, ws[1:]) if return_count else mask
 
 
 def swiglu_mul(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:

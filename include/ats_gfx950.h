@@ -222,7 +222,9 @@ int ats_scatter_add_rows(void* base, const int32_t* rows, const void* delta, int
 
 /* mask[i] = 1.0f if v[i] >= (kth smallest of v, 1-based) else 0.0f: the inference
  * branch of MoDRouter.forward (model.py:984-990, kthvalue threshold).
- * workspace: at least 4 bytes of device memory. */
+ * workspace: at least 4 bytes of device memory, 8-byte aligned; when it holds 16 or
+ * more, the int64 at byte offset 8 receives the number of ones in the mask (the
+ * "computed tokens" statistic of model.py:990-995). */
 int ats_kth_value_mask(const float* v, int64_t n, int64_t kth, float* mask, void* workspace,
                        size_t workspace_bytes, ats_stream_t stream);
 
@@ -378,6 +380,27 @@ int ats_grad_clip_chunk_elems(void);
 int ats_grad_norm_clip(void* const* grad_ptrs, const int64_t* sizes, const int32_t* chunk_start, int n_tensors,
                        int n_chunks, int dtype, const float* extra_sumsq, float* partial, float* norm_out,
                        float max_norm, int do_clip, ats_stream_t stream);
+
+/* ---- The reference's own launcher names ---------------------------------------
+ * Exact float32 signatures of Src/Main_Scripts/core/transformer_ops.cu:331-409, so that the ctypes
+ * loader of Src/Main_Scripts/core/cuda_opt_wrapper.py:50-79 binds this library unchanged (call sites
+ * cuda_opt_wrapper.py:98-108, 156-169, 219-228, 337-344).  Thin aliases of ats_rmsnorm_fwd,
+ * ats_rope_table (half-width table), ats_rope_fwd (in place, q and k with the same head count, as
+ * that signature has it; the caller guarantees position_offset + seq_len <= max_seq_len) and
+ * ats_swiglu_mul.  They return void like the originals but never exit(): the status of the calling
+ * thread's last legacy call is ats_legacy_last_status(), its text ats_last_error_string().
+ * swiglu_fused_launcher (transformer_ops.cu:411-434) has no call site in the reference's Python
+ * and is not exported. */
+void rms_norm_launcher(const float* input, const float* weight, float* output, int batch_seq,
+                       int hidden_size, float eps, ats_stream_t stream);
+void rope_precompute_launcher(float* cos_cache, float* sin_cache, int max_seq_len, int head_dim,
+                              float theta, ats_stream_t stream);
+void rope_apply_launcher(float* q, float* k, const float* cos, const float* sin, int batch_size,
+                         int num_heads, int seq_len, int head_dim, int position_offset,
+                         ats_stream_t stream);
+void swiglu_launcher(const float* gate, const float* up, float* output, int total_tokens,
+                     int intermediate_size, ats_stream_t stream);
+int ats_legacy_last_status(void);
 
 /* ---- Host-side views of the grouped-GEMM tile schedule (no device work) ----
  * No reference counterpart; used to test the block -> (expert, m-tile, n-tile)

@@ -349,6 +349,53 @@ def test_layer_grads_bf16_skewed_drops(gpu):
     _layer_grads_vs_oracle(gpu, "c4_prefill", "fcfs", "softmax_topk", 3e-2, scale_tokens=1024)
 
 
+def test_mod_moe_block_gradients(gpu):
+    """The MoD + MoE block trains: gradients of x (identity path plus the gathered rows), the gate and every
+    expert against torch autograd over the oracle's composition, float32, fine-grained shape at reduced size.
+    The selection is discrete, so the score weight has no gradient on either side."""
+    from adaptivetrainingsystem_amd import workloads as W
+    ov = {"batch": 3, "seq": 128, "hidden": 128, "intermediate": 64, "num_experts": 8, "top_k": 3, "dtype": torch.float32}
+    w = W.make_moe_workload("c5_finegrained_mod", device="cpu", overrides=ov)
+    wg = W.make_moe_workload("c5_finegrained_mod", device=gpu, overrides=ov)
+    block = W.build_layer(wg, "fcfs")
+    for p in block.moe.parameters():
+        p.requires_grad_(True)
+    x = wg.x.clone().requires_grad_(True)
+    out, aux = block(x)
+    assert out.requires_grad and aux.requires_grad
+    cot = torch.randn(w.x.shape, generator=gen(61))
+    (out * cot.to(gpu)).sum().add(aux * 1.5).backward()
+    E, k, keep = 8, 3, int(128 * 0.125)
+    sel = block.last_selected.cpu().long()
+    plan = block.moe.last_plan
+
+    def fwd(xx, wgate, *ws):
+        r = O.mod_moe_block(xx, w.mod_weight, None, keep,
+                            dict(gate_weight=wgate, gate_up_weights=list(ws[:E]), down_weights=list(ws[E:]), k=k,
+                                 capacity_factor=w.capacity_factor, routing=wg.routing))
+        fwd.last = r
+        return r["block_out"], r["aux"]
+
+    leaves = [w.x, w.gate] + list(w.gate_up) + list(w.down)
+    grads = O.layer_grads(fwd, leaves, [cot, torch.tensor(1.5)])
+    grads = [torch.zeros_like(leaf) if g_ is None else g_ for g_, leaf in zip(grads, leaves)]
+    flat_ref = (fwd.last["selected"] + torch.arange(3).unsqueeze(1) * 128).reshape(-1)
+    assert torch.equal(sel, flat_ref), "selection differs from the oracle"
+    assert torch.equal(plan["indices"].cpu().long(), fwd.last["indices"]), "routing differs from the oracle"
+    moe = block.moe
+    errs = {"x": rel_err(x.grad, grads[0]), "gate": rel_err(moe.gate.weight.grad, grads[1]),
+            "gate_up": max(rel_err(ex.gate_up_proj.weight.grad, grads[2 + e]) for e, ex in enumerate(moe.experts)),
+            "down": max(rel_err(ex.down_proj.weight.grad, grads[2 + E + e]) for e, ex in enumerate(moe.experts))}
+    print("mod block grads", {n: f"{v:.2e}" for n, v in errs.items()}, flush=True)
+    for n, v in errs.items():
+        assert v <= 2e-5, (n, v)
+    # rows the block skipped get exactly the cotangent (identity path only)
+    skipped = torch.ones(3 * 128, dtype=torch.bool)
+    skipped[sel] = False
+    assert torch.equal(x.grad.reshape(-1, 128).cpu()[skipped], cot.reshape(-1, 128)[skipped])
+    assert block.router.weight.grad is None
+
+
 def test_training_mode_noise_and_stats(gpu):
     """Training mode: noise on the routing logits only; the auxiliary loss still uses the clean logits."""
     from adaptivetrainingsystem_amd import workloads as W
@@ -369,6 +416,15 @@ def test_training_mode_noise_and_stats(gpu):
     assert all(p.grad is not None and torch.isfinite(p.grad).all() for p in layer.parameters())
     stats = layer.get_routing_stats()
     assert stats["total_tokens_routed"] == wg.tokens
+    # the no-grad path of the same layer takes the auxiliary loss from the clean logits too: same seed, same noise
+    for p in layer.parameters():
+        p.requires_grad_(False)
+    torch.manual_seed(7)
+    with torch.no_grad():
+        out2, aux2 = layer(wg.x)
+    assert torch.equal(layer.last_plan["indices"], plan["indices"])
+    assert abs(aux2.item() - aux.item()) <= 1e-7
+    assert (out2 - out).abs().max().item() <= 1e-5 * out.abs().max().item()
 
 
 def test_module_gradients_norm_rope_expert_swiglu(gpu):

@@ -1,0 +1,83 @@
+"""The reference's launcher names, called through ctypes exactly as the reference's wrapper calls them
+(Src/Main_Scripts/core/cuda_opt_wrapper.py:98-108 RMSNorm, 156-169 RoPE apply, 219-228 SwiGLU, 337-344 RoPE
+precompute: bare CDLL handle, every argument wrapped in a ctypes type, stream as c_void_p), compared with the
+oracle.  float32 only, as those signatures are."""
+import ctypes
+import math
+
+import pytest
+import torch
+
+from oracle import sparse_layer_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def gen(seed):
+    return torch.Generator().manual_seed(seed)
+
+
+@pytest.fixture(scope="module")
+def raw(gpu):
+    from adaptivetrainingsystem_amd import _lib
+    _lib.load()
+    return ctypes.CDLL(_lib.LIB_PATH), _lib.load()
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def test_rms_norm_launcher(raw, gpu):
+    lib, typed = raw
+    x = torch.randn(37, 520, generator=gen(1)) * 2.0
+    w = torch.randn(520, generator=gen(2)) * 0.1 + 1.0
+    xg, wg = x.to(gpu), w.to(gpu)
+    out = torch.empty_like(xg)
+    lib.rms_norm_launcher(ctypes.c_void_p(xg.data_ptr()), ctypes.c_void_p(wg.data_ptr()), ctypes.c_void_p(out.data_ptr()),
+                          ctypes.c_int(37), ctypes.c_int(520), ctypes.c_float(1e-6), _stream())
+    torch.cuda.synchronize()
+    assert typed.ats_legacy_last_status() == 0
+    ref = O.rmsnorm(x, w, 1e-6)
+    assert (out.cpu() - ref).abs().max().item() <= 1e-5 * ref.abs().max().item()
+
+
+def test_rope_launchers(raw, gpu):
+    lib, typed = raw
+    B, nH, L, D, max_seq, off, theta = 2, 3, 21, 64, 64, 5, 10000.0
+    cos = torch.empty(max_seq, D // 2, device=gpu)
+    sin = torch.empty(max_seq, D // 2, device=gpu)
+    lib.rope_precompute_launcher(ctypes.c_void_p(cos.data_ptr()), ctypes.c_void_p(sin.data_ptr()), ctypes.c_int(max_seq),
+                                 ctypes.c_int(D), ctypes.c_float(theta), _stream())
+    torch.cuda.synchronize()
+    assert typed.ats_legacy_last_status() == 0
+    ch, sh = O.fused_rope_table(max_seq, D, theta)      # float32 evaluation; the kernel rounds the float64 value
+    assert (cos.cpu() - ch).abs().max().item() <= 2e-5 and (sin.cpu() - sh).abs().max().item() <= 2e-5
+    for pos, d in ((1, 0), (7, 3), (63, 31)):
+        ang = pos * theta ** (-2.0 * d / D)
+        assert abs(cos[pos, d].item() - math.cos(ang)) <= 1.2e-7 and abs(sin[pos, d].item() - math.sin(ang)) <= 1.2e-7
+    q = torch.randn(B, nH, L, D, generator=gen(3))
+    k = torch.randn(B, nH, L, D, generator=gen(4))
+    qg, kg = q.to(gpu).clone(), k.to(gpu).clone()        # the launcher rotates in place (cuda_opt_wrapper.py:153-154)
+    lib.rope_apply_launcher(ctypes.c_void_p(qg.data_ptr()), ctypes.c_void_p(kg.data_ptr()), ctypes.c_void_p(cos.data_ptr()),
+                            ctypes.c_void_p(sin.data_ptr()), ctypes.c_int(B), ctypes.c_int(nH), ctypes.c_int(L),
+                            ctypes.c_int(D), ctypes.c_int(off), _stream())
+    torch.cuda.synchronize()
+    assert typed.ats_legacy_last_status() == 0
+    rq, rk = O.fused_rope_apply(q, k, cos.cpu(), sin.cpu(), off)
+    assert torch.equal(qg.cpu(), rq) and torch.equal(kg.cpu(), rk)      # same table, same roundings: same bits
+
+
+def test_swiglu_launcher(raw, gpu):
+    lib, typed = raw
+    T, I = 19, 1408
+    gate = torch.randn(T, I, generator=gen(5))
+    up = torch.randn(T, I, generator=gen(6)) * 2.0
+    gg, ug = gate.to(gpu), up.to(gpu)
+    out = torch.empty_like(gg)
+    lib.swiglu_launcher(ctypes.c_void_p(gg.data_ptr()), ctypes.c_void_p(ug.data_ptr()), ctypes.c_void_p(out.data_ptr()),
+                        ctypes.c_int(T), ctypes.c_int(I), _stream())
+    torch.cuda.synchronize()
+    assert typed.ats_legacy_last_status() == 0
+    ref = gate * torch.nn.functional.silu(up)            # cuda_opt_wrapper.py:476-478 convention: gate * silu(up)
+    assert (out.cpu() - ref).abs().max().item() <= 1e-5 * ref.abs().max().item()

@@ -278,6 +278,27 @@ def test_dispatch_tokens_and_combine_api(A, gpu):
     assert same_bits(out2, O.combine_loop(eo2, tm_ref, w, T, k))
 
 
+@pytest.mark.parametrize("T,H,E,k,C", [(50, 260, 8, 2, 20), (40, 64, 16, 12, 40), (30, 6, 4, 3, 30), (20, 516, 8, 2, 3),
+                                       (33, 1030, 16, 9, 25)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_combine_scalar_path_tail_columns(A, gpu, T, H, E, k, C, dtype):
+    """Widths and k values that take the scalar combine kernel (H not a multiple of 8, or more than 8 choices),
+    with a last trip of the column loop that only the first lanes make: every column against the literal loop
+    (MS/core/moe_cuda_wrapper.py:328-359)."""
+    g = gen(180 + H)
+    idx = torch.topk(torch.randn(T, E, generator=g), k, -1)[1]
+    w = torch.softmax(torch.randn(T, k, generator=g), -1)
+    _, tm_ref = O.dispatch_loop(torch.zeros(T, 1), idx, E, C)
+    eo = torch.randn(E, C, H, generator=g).to(dtype)
+    ref = O.combine_loop(eo.float(), tm_ref, w, T, k)
+    out = A.MoECUDAOps.combine_expert_outputs(eo.to(gpu), tm_ref.to(gpu), w.to(gpu), T, k)
+    assert out.dtype == dtype
+    if dtype == torch.float32:
+        assert same_bits(out, ref)
+    else:
+        assert torch.equal(out.cpu(), ref.bfloat16())       # float32 sums in the same order, one rounding
+
+
 # ------------------------------------------------------------------ expert FFN (grouped GEMMs)
 @pytest.mark.parametrize("n,H,I", [(20, 512, 1408), (70, 512, 1408), (300, 256, 200), (1000, 512, 384), (33, 72, 136),
                                    (1, 64, 64), (2500, 128, 256), (8, 1024, 512), (1, 2048, 256), (32, 4096, 128)])
@@ -518,6 +539,13 @@ def test_mod_router_eval_and_selection(A, ops, gpu):
     assert aux is None and mask.shape == (3, 50, 1)
     assert (probs.cpu() - pr).abs().max().item() <= 1e-6
     assert torch.equal(mask.cpu(), O.mod_router_eval_mask(probs.cpu(), 0.5))     # threshold on bit-equal probs
+    st = m.get_routing_stats()                          # MS/core/model.py:990-995, 998-1011
+    assert st["total_tokens_routed"] == 150 and st["computed_tokens"] == mask.sum().item() == 76
+    assert st["skipped_tokens"] == 74 and abs(st["compute_ratio"] + st["skip_ratio"] - 1) < 1e-12
+    m(x.to(gpu))
+    assert m.get_routing_stats()["computed_tokens"] == 152
+    m.reset_routing_stats()
+    assert "error" in m.get_routing_stats()
     s = torch.randn(5, 700, generator=gen(22))
     s[0, 10] = s[0, 3]                                                           # a tie
     sel = ops.select_topk_per_sequence(s.to(gpu), 77).cpu().view(5, 77)

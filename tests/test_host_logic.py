@@ -14,7 +14,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 def _declared_symbols():
     text = open(os.path.join(ROOT, "include", "ats_gfx950.h")).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return sorted(set(re.findall(r"\b(ats_[a-z0-9_]+)\s*\(", text)))
+    return sorted(set(re.findall(r"\b(ats_[a-z0-9_]+|[a-z_]+_launcher)\s*\(", text)))
 
 
 def test_library_exports_every_declared_symbol():
@@ -28,6 +28,29 @@ def test_library_exports_every_declared_symbol():
         assert n in _lib._SIGNATURES, f"{n} has no ctypes signature"
     assert lib.ats_version() >= 100
     assert set(_lib._SIGNATURES) == set(names)
+
+
+def test_reference_launcher_names_are_exported_and_never_exit():
+    """The four launcher names the reference's ctypes loader binds (cuda_opt_wrapper.py:98-108, 156-169,
+    219-228, 337-344) exist with void returns; a bad argument leaves a status and a text, not an exit()."""
+    from adaptivetrainingsystem_amd import _lib
+    lib = _lib.load()
+    raw = ctypes.CDLL(_lib.LIB_PATH)        # as the reference binds it: no argtypes, explicit ctypes wrappers
+    for n in ("rms_norm_launcher", "rope_precompute_launcher", "rope_apply_launcher", "swiglu_launcher"):
+        assert hasattr(raw, n), n
+    raw.rms_norm_launcher(ctypes.c_void_p(0), ctypes.c_void_p(0), ctypes.c_void_p(0), ctypes.c_int(4), ctypes.c_int(0),
+                          ctypes.c_float(1e-6), ctypes.c_void_p(0))
+    assert lib.ats_legacy_last_status() == -1 and b"hidden" in lib.ats_last_error_string()
+    raw.rope_apply_launcher(ctypes.c_void_p(0), ctypes.c_void_p(0), ctypes.c_void_p(0), ctypes.c_void_p(0),
+                            ctypes.c_int(1), ctypes.c_int(1), ctypes.c_int(4), ctypes.c_int(7), ctypes.c_int(0),
+                            ctypes.c_void_p(0))
+    assert lib.ats_legacy_last_status() == -1           # odd head_dim
+    raw.swiglu_launcher(ctypes.c_void_p(0), ctypes.c_void_p(0), ctypes.c_void_p(0), ctypes.c_int(0), ctypes.c_int(16),
+                        ctypes.c_void_p(0))
+    assert lib.ats_legacy_last_status() == 0            # nothing to do is not an error
+    raw.rope_precompute_launcher(ctypes.c_void_p(0), ctypes.c_void_p(0), ctypes.c_int(8), ctypes.c_int(16),
+                                 ctypes.c_float(10000.0), ctypes.c_void_p(0))
+    assert lib.ats_legacy_last_status() == -1 and b"null" in lib.ats_last_error_string()
 
 
 def test_argument_errors_return_codes_not_exits():
