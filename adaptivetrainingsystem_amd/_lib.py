@@ -35,6 +35,8 @@ _SIGNATURES = {
     "ats_dispatch_plan_workspace": (c_size_t, [c_int64, c_int, c_int]),
     "ats_dispatch_plan": (c_int, [c_void_p, c_int, c_int64, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p,
                                   c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "ats_dispatch_plan_static": (c_int, [c_void_p, c_int, c_int64, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p,
+                                         c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
     "ats_gather_rows": (c_int, [c_void_p, c_void_p, c_int, c_void_p, c_int64, c_int, c_int, c_void_p]),
     "ats_invert_token_map": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p]),
     "ats_grouped_gateup_swiglu": (c_int, [c_void_p, c_int64, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int,

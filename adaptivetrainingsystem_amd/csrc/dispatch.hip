@@ -669,6 +669,58 @@ extern "C" int ats_dispatch_plan(const void* idx, int idx_dtype, int64_t T, int 
     return ATS_OK;
 }
 
+// ------------------------------------------------------------------ plan without a workspace argument
+// For callers that cannot allocate (code under HIP graph capture, tight serving loops, harnesses that forbid
+// hipMalloc): the chunk histograms of the plan live in a fixed array in device memory instead of a
+// caller-provided workspace.  Each GPU the library runs on holds its own copy of the array, at its own address,
+// until the process ends.  In host code the array's name is only a stand-in for the symbol, never a device
+// address: the address is looked up once per device with hipGetSymbolAddress and only that pointer is handed
+// to kernels.
+namespace ats {
+constexpr size_t kPlanScratchInts = (size_t)1 << 20;      // 4 MiB: chunks * E <= 1 048 576
+static __device__ __align__(256) int32_t scratch[kPlanScratchInts];
+constexpr int kPlanScratchMaxDevices = 64;
+static std::atomic<int32_t*> g_plan_scratch_ptr[kPlanScratchMaxDevices];
+
+// Device address of this GPU's copy of `scratch` (looked up on the first call on a device, with that device
+// current; racing first calls repeat the same idempotent lookup).
+static int plan_scratch_for_current_device(int32_t** out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    ATS_REQUIRE(e == hipSuccess, ATS_ERR_LAUNCH, "ats_dispatch_plan_static: hipGetDevice: %s", hipGetErrorString(e));
+    ATS_REQUIRE(dev >= 0 && dev < kPlanScratchMaxDevices, ATS_ERR_UNSUPPORTED,
+                "ats_dispatch_plan_static: device id %d (at most %d devices)", dev, kPlanScratchMaxDevices);
+    int32_t* ptr = g_plan_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!ptr) {
+        e = hipGetSymbolAddress(reinterpret_cast<void**>(&ptr), HIP_SYMBOL(scratch));
+        ATS_REQUIRE(e == hipSuccess && ptr, ATS_ERR_LAUNCH, "ats_dispatch_plan_static: hipGetSymbolAddress: %s",
+                    hipGetErrorString(e));
+        g_plan_scratch_ptr[dev].store(ptr, std::memory_order_release);
+    }
+    *out = ptr;
+    return ATS_OK;
+}
+}  // namespace ats
+
+extern "C" int ats_dispatch_plan_static(const void* idx, int idx_dtype, int64_t T, int k, int E, int C, int32_t* slot,
+                                        int32_t* token_map, int32_t* hist, int32_t* kept, int32_t* offsets,
+                                        int32_t* row_src, int32_t* row_of, int32_t* status, ats_stream_t stream) {
+    using namespace ats;
+    ATS_REQUIRE(T >= 0 && k > 0 && E > 0, ATS_ERR_INVALID_ARG, "ats_dispatch_plan_static: T=%lld k=%d E=%d",
+                (long long)T, k, E);
+    const size_t need = ats_dispatch_plan_workspace(T, k, E);
+    ATS_REQUIRE(need <= kPlanScratchInts * sizeof(int32_t), ATS_ERR_WORKSPACE,
+                "ats_dispatch_plan_static: T*k=%lld assignments over %d experts need %zu bytes of chunk histograms, "
+                "the fixed scratch array holds %zu (use ats_dispatch_plan with a workspace)",
+                (long long)(T * k), E, need, kPlanScratchInts * sizeof(int32_t));
+    int32_t* chunk_hist = nullptr;
+    const int rc = plan_scratch_for_current_device(&chunk_hist);
+    if (rc != ATS_OK) return rc;
+    // every chunk histogram the plan reads is written by its first kernel, so nothing has to start at zero
+    return ats_dispatch_plan(idx, idx_dtype, T, k, E, C, slot, token_map, hist, kept, offsets, row_src, row_of, status,
+                             chunk_hist, kPlanScratchInts * sizeof(int32_t), stream);
+}
+
 extern "C" int ats_gather_rows(const void* src, const int32_t* map, int div, void* out, int64_t n_rows, int H,
                                int dtype, ats_stream_t stream) {
     using namespace ats;

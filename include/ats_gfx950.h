@@ -117,6 +117,21 @@ int ats_dispatch_plan(const void* idx, int idx_dtype, int64_t T, int k, int E, i
                       int32_t* row_src, int32_t* row_of, int32_t* status, void* workspace,
                       size_t workspace_bytes, ats_stream_t stream);
 
+/* ats_dispatch_plan without a workspace argument, for callers that cannot allocate.  It has no
+ * counterpart in the reference; it is for code under HIP graph capture, tight serving loops and
+ * harnesses that forbid hipMalloc, which cannot provide (or size) a workspace.  Same arguments,
+ * outputs and results as ats_dispatch_plan; the chunk histograms live in a fixed 4 MiB array in
+ * device memory that each GPU the library runs on holds until the process ends, so the plan is
+ * limited to ceil(T*k / 256) * E <= 1 048 576 (larger plans return ATS_ERR_WORKSPACE: use
+ * ats_dispatch_plan).  The call allocates and frees nothing.  All calls on one GPU share that
+ * GPU's array: calls that overlap on one GPU (different streams, or threads) race; calls ordered
+ * on one stream are safe, and nothing needs clearing between them.  The first call on a device
+ * looks up the array's address (hipGetSymbolAddress) and must therefore come before any capture. */
+int ats_dispatch_plan_static(const void* idx, int idx_dtype, int64_t T, int k, int E, int C,
+                             int32_t* slot, int32_t* token_map, int32_t* hist, int32_t* kept,
+                             int32_t* offsets, int32_t* row_src, int32_t* row_of, int32_t* status,
+                             ats_stream_t stream);
+
 /* out[r,:] = src[map[r] / div, :] or zeros when map[r] < 0; r in [0, n_rows).
  * With map = token_map and div = k this fills expert_inputs[E,C,H]
  * (moe_cuda_wrapper.py:306-322); with div = 1 it is a plain row gather. */
