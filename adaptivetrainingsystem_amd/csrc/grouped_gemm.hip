@@ -635,15 +635,21 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_pipelined_kernel(Gro
 // chunk c of row R reads slot c ^ f(R).  For the 16 consecutive rows that one quarter-wave reads,
 // (R & 1, c ^ f(R)) takes 16 different values, i.e. all 64 banks are hit once.
 //
-// LDS map: [A stage 0][A stage 1][B stage 0][B stage 1]; both stages of a fragment row are
-// reachable from one address register through the 16-bit instruction offset.
+// LDS map: [A stage 0][A stage 1][A stage 2][B stage 0][B stage 1] (160 KiB for the 256 x 256 tile).  The
+// activation slabs go round a ring of three stages, the weight slabs alternate between two:
+// after the barrier that ends slab t, the weight loads of slab t+2 (into the stage slab t used) and the
+// activation loads of slab t+3 are issued, in that order.  The weight loads have one slab of MFMA time to
+// land, the activation loads two, and the wait at the end of a slab lets the youngest activation loads stay
+// in flight (s_waitcnt vmcnt(NIA)): only half of a slab's loads sit in the window that the barrier closes,
+// so the burst that the address unit has to work off after every barrier is halved.
+// The weight stage is a compile-time offset of the read instructions; the activation stage is a scalar
+// that is added to the fragment address once per k-step.
 //
 // Schedule per slab t (4 k-steps of MFMAs, fragments double buffered in registers):
 //   k-steps 0..2 : MFMAs | fragment reads of the next k-step
 //   wait for the loads of slab t+1, barrier (every wave is done reading slab t)
-//   issue the loads of slab t+2 into the stage slab t occupied
+//   issue the loads (weights of slab t+2, activations of slab t+3)
 //   k-step 3     : MFMAs | fragment reads of k-step 0 of slab t+1
-// so a slab has a whole slab of MFMA time to land.
 template <typename T, typename TO, int BM, int BN, int WM, int WN, int SM, int SN, bool SWIGLU, bool SAVEGU = false,
           bool DSILU = false>
 __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_dma_kernel(GroupedArgs p) {
@@ -657,12 +663,12 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_dma_kernel(GroupedAr
     constexpr int HALF = BN / 2;
     constexpr int A_STAGE = BM * 128;
     constexpr int B_STAGE = BN * 128;
-    constexpr int B_BASE = 2 * A_STAGE;
+    constexpr int B_BASE = 3 * A_STAGE;
     static_assert(BM % (WM * 32) == 0 && BN % (WN * 32) == 0, "wave tiling");
     static_assert(BM % (8 * NW) == 0 && BN % (8 * NW) == 0 && NW % 2 == 0, "loader tiling");
     static_assert(!SWIGLU || TN % 2 == 0, "SwiGLU needs gate and up tiles in the same wave");
     static_assert(SM * SN == kSuperBlocks, "supertile");
-    static_assert(A_STAGE + (TM - 1) * 4096 + 128 <= 65536 && B_STAGE + (BN / 2 + 32 * TN) * 128 <= 65536, "offset field");
+    static_assert((TM - 1) * 4096 + 128 <= 65536 && B_STAGE + (BN / 2 + 32 * TN) * 128 <= 65536, "offset field");
 
     extern __shared__ __align__(16) unsigned char smem[];
     typedef __attribute__((address_space(3))) void* lds_ptr_t;
@@ -743,12 +749,16 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_dma_kernel(GroupedAr
     }
     u32x4_t fa[2][TM], fb[2][TN];
 
-#define DM_ISSUE(kt_, stage_)                                                                          \
+#define DM_ISSUE_A(kt_, aoff_)                                                                         \
     {                                                                                                  \
         const int soff = (kt_) * 128;                                                                  \
         _Pragma("unroll") for (int j = 0; j < NIA; ++j)                                                \
             __builtin_amdgcn_raw_ptr_buffer_load_lds(                                                  \
-                rsrc_a, (lds_ptr_t)(dma_a + (stage_) * A_STAGE + j * NW * 1024), 16, ao[j], soff, 0, 0); \
+                rsrc_a, (lds_ptr_t)(dma_a + (aoff_) + j * NW * 1024), 16, ao[j], soff, 0, 0);          \
+    }
+#define DM_ISSUE_B(kt_, stage_)                                                                        \
+    {                                                                                                  \
+        const int soff = (kt_) * 128;                                                                  \
         _Pragma("unroll") for (int j = 0; j < NIB; ++j)                                                \
             __builtin_amdgcn_raw_ptr_buffer_load_lds(                                                  \
                 rsrc_b, (lds_ptr_t)(dma_b + (stage_) * B_STAGE + j * NW * 1024), 16, bo[j], soff, 0, 0); \
@@ -756,11 +766,12 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_dma_kernel(GroupedAr
 #define DM_B_ROW(j_) (SWIGLU ? ((j_) < TN / 2 ? (j_) * 32 : HALF + ((j_) - TN / 2) * 32) : (j_) * 32)
 // Read order = use order of the MFMAs (weight fragment 0, all activation fragments, then the
 // other weight fragments), so the first MFMAs of the next k-step wait for few reads.
-#define DM_READ(stage_, ks_, buf_)                                                                     \
+#define DM_READ(aoff_, stage_, ks_, buf_)                                                              \
     {                                                                                                  \
+        const unsigned char* fa_ = fa_addr[ks_] + (aoff_);                                             \
         fb[buf_][0] = *reinterpret_cast<const u32x4_t*>(fb_addr[ks_] + (stage_) * B_STAGE + DM_B_ROW(0) * 128); \
         _Pragma("unroll") for (int i = 0; i < TM; ++i)                                                 \
-            fa[buf_][i] = *reinterpret_cast<const u32x4_t*>(fa_addr[ks_] + (stage_) * A_STAGE + i * 4096); \
+            fa[buf_][i] = *reinterpret_cast<const u32x4_t*>(fa_ + i * 4096);                           \
         _Pragma("unroll") for (int j = 1; j < TN; ++j)                                                 \
             fb[buf_][j] = *reinterpret_cast<const u32x4_t*>(fb_addr[ks_] + (stage_) * B_STAGE + DM_B_ROW(j) * 128); \
     }
@@ -775,35 +786,43 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_dma_kernel(GroupedAr
         __builtin_amdgcn_sched_group_barrier(SG_MFMA, 1, 0);                            \
         __builtin_amdgcn_sched_group_barrier(SG_VMEM, 1, 0);                            \
     }
-// STG: stage of slab kt (compile time).  Slabs past the end are clamped to the last one: their
-// loads land in a stage nobody reads again, which keeps the loop body free of special cases.
+// STG: weight stage of slab kt (compile time); sa_cur / sa_nxt: activation stage offsets of slabs kt and
+// kt+1.  Slabs past the end are clamped to the last one: their loads land in stages nobody reads again,
+// which keeps the loop body free of special cases.
 #define DM_ITER(kt_, STG)                                                               \
     {                                                                                   \
-        DM_READ(STG, 1, 1);                                                             \
+        DM_READ(sa_cur, STG, 1, 1);                                                     \
         PL_MMA(0);                                                                      \
         PL_MIX_READS();                                                                 \
         PL_FENCE();                                                                     \
-        DM_READ(STG, 2, 0);                                                             \
+        DM_READ(sa_cur, STG, 2, 0);                                                     \
         PL_MMA(1);                                                                      \
         PL_MIX_READS();                                                                 \
         PL_FENCE();                                                                     \
-        DM_READ(STG, 3, 1);                                                             \
+        DM_READ(sa_cur, STG, 3, 1);                                                     \
         PL_MMA(0);                                                                      \
         PL_MIX_READS();                                                                 \
         PL_FENCE();                                                                     \
-        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");        \
+        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(NIA) : "memory"); \
         PL_FENCE();                                                                     \
-        DM_READ(STG ^ 1, 0, 0);                                                         \
-        DM_ISSUE(min((kt_) + 2, nk - 1), STG);                                          \
+        DM_READ(sa_nxt, STG ^ 1, 0, 0);                                                 \
+        DM_ISSUE_B(min((kt_) + 2, nk - 1), STG);                                        \
+        DM_ISSUE_A(min((kt_) + 3, nk - 1), sa_cur);                                     \
         PL_MMA(1);                                                                      \
         DM_MIX_DMA();                                                                   \
         PL_FENCE();                                                                     \
+        sa_cur = sa_nxt;                                                                \
+        sa_nxt = sa_nxt == 2 * A_STAGE ? 0 : sa_nxt + A_STAGE;                          \
     }
 
-    DM_ISSUE(0, 0);
-    DM_ISSUE(min(1, nk - 1), 1);
-    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(NIA + NIB) : "memory");
-    DM_READ(0, 0, 0);
+    DM_ISSUE_A(0, 0);
+    DM_ISSUE_B(0, 0);
+    DM_ISSUE_A(min(1, nk - 1), A_STAGE);
+    DM_ISSUE_B(min(1, nk - 1), 1);
+    DM_ISSUE_A(min(2, nk - 1), 2 * A_STAGE);
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(2 * NIA + NIB) : "memory");
+    int sa_cur = 0, sa_nxt = A_STAGE;
+    DM_READ(sa_cur, 0, 0, 0);
     int kt = 0;
     for (; kt + 1 < nk; kt += 2) {
         DM_ITER(kt, 0);
@@ -812,7 +831,8 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_dma_kernel(GroupedAr
     if (kt < nk) DM_ITER(kt, 0);
     // the clamped loads of the last slabs may still be in flight; the epilogue reuses LDS
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-#undef DM_ISSUE
+#undef DM_ISSUE_A
+#undef DM_ISSUE_B
 #undef DM_READ
 #undef DM_ITER
 #undef DM_B_ROW
@@ -836,12 +856,17 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_dma_kernel(GroupedAr
 #undef PL_FENCE
 #undef PL_MIX_READS
 
+// LDS of the direct-to-LDS kernel: three activation stages and two weight stages of unpadded 128-byte rows.
+constexpr size_t dma_lds_bytes(int BM, int BN) { return (size_t)(3 * BM + 2 * BN) * 128; }
+
 template <typename T, typename TO, int BM, int BN, int WM, int WN, int SM, int SN, bool SWIGLU, bool DMA = false>
 static int launch_cfg(const GroupedArgs& p0, int64_t max_rows, hipStream_t s) {
     GroupedArgs p = p0;
     constexpr int n_per_tile = SWIGLU ? BN / 2 : BN;
     p.n_tiles = (p.N_out + n_per_tile - 1) / n_per_tile;
-    constexpr size_t smem = 2 * (size_t)(BM + BN) * kRowPitch;  // covers the unpadded DMA layout too
+    // register-staged kernels: two padded stages; direct-to-LDS kernel: three activation + two weight stages
+    constexpr size_t smem_staged = 2 * (size_t)(BM + BN) * kRowPitch;
+    constexpr size_t smem = DMA && dma_lds_bytes(BM, BN) > smem_staged ? dma_lds_bytes(BM, BN) : smem_staged;
     constexpr int BK = 128 / (int)sizeof(T);
     auto kern_general = grouped_gemm_kernel<T, TO, BM, BN, WM, WN, SM, SN, SWIGLU>;
     // the L2 warm-up touches pay where blocks share operand panels; the weight-streaming tiles share nothing
@@ -937,7 +962,7 @@ static int launch_gateup_save(const GroupedArgs& p0, int64_t max_rows, hipStream
     constexpr int BM = 256, BN = 256;
     GroupedArgs p = p0;
     p.n_tiles = (p.N_out + BN / 2 - 1) / (BN / 2);
-    constexpr size_t smem = 2 * (size_t)(BM + BN) * kRowPitch;
+    constexpr size_t smem = dma_lds_bytes(BM, BN);
     auto kern = grouped_gemm_dma_kernel<T, T, BM, BN, 2, 4, 4, 8, true, true>;
     static LdsReservation reserved;
     hipError_t e = reserve_lds(reserved, {reinterpret_cast<const void*>(kern)}, (int)smem);
@@ -968,7 +993,7 @@ static int launch_down_dgrad_dsilu(const GroupedArgs& p0, int64_t max_rows, hipS
     constexpr int BM = 256, BN = 256;
     GroupedArgs p = p0;
     p.n_tiles = (p.N_out + BN - 1) / BN;
-    constexpr size_t smem = 2 * (size_t)(BM + BN) * kRowPitch;
+    constexpr size_t smem = dma_lds_bytes(BM, BN);
     auto kern = grouped_gemm_dma_kernel<T, T, BM, BN, 2, 4, 4, 8, false, false, true>;
     static LdsReservation reserved;
     hipError_t e = reserve_lds(reserved, {reinterpret_cast<const void*>(kern)}, (int)smem);
