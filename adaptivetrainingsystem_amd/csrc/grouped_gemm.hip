@@ -19,6 +19,8 @@
 // The permutation gather is fused into the A load (row index table).
 #include <math.h>
 
+#include <type_traits>
+
 #include "ats_common.hpp"
 #include "tile_schedule.hpp"
 
@@ -78,52 +80,81 @@ __device__ __forceinline__ void mma_step<float>(const u32x4_t& wfrag, const u32x
     c = __builtin_amdgcn_mfma_f32_32x32x2f32(__uint_as_float(wfrag.w), __uint_as_float(afrag.w), c, 0, 0, 0);
 }
 
-// Epilogue through LDS.  In the accumulator layout a lane owns 4 consecutive columns of one row,
+// Views of a wave's accumulators, 32 output rows at a time, as groups of 4 consecutive output columns
+// per lane.  ib: 32-row block of the wave's sub-tile, g: group, half: 0 = gate (or the plain product),
+// 1 = the matching up column.  All indices are compile-time constants after unrolling.
+// 32 x 32 x 16 MFMA: lane holds row (lane & 31), columns 8 q + 4 (lane >> 5) + c of each 32-column tile.
+template <int TM, int TN, bool SWIGLU>
+struct AccView32 {
+    f32x16_t (&acc)[TN][TM];
+    static constexpr int kBlocks = TM;
+    static constexpr int kColTiles = SWIGLU ? TN / 2 : TN;
+    static constexpr int kCols = kColTiles * 32;
+    static constexpr int kGroups = kColTiles * 4;
+    __device__ __forceinline__ static int row(int g, int lane) { return lane & 31; }
+    __device__ __forceinline__ static int col(int g, int lane) { return (g >> 2) * 32 + 8 * (g & 3) + 4 * (lane >> 5); }
+    __device__ __forceinline__ float val(int ib, int g, int c, int half) const {
+        return acc[(g >> 2) + half * (TN / 2)][ib][(g & 3) * 4 + c];
+    }
+};
+// 16 x 16 x 32 MFMA: lane holds row (lane & 15), columns 4 (lane >> 4) + c of each 16-column tile; a 32-row
+// block is two row tiles.
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4_t;
+template <int TM16, int TN16, bool SWIGLU>
+struct AccView16 {
+    f32x4_t (&acc)[TN16][TM16];
+    static constexpr int kBlocks = TM16 / 2;
+    static constexpr int kColTiles = SWIGLU ? TN16 / 2 : TN16;
+    static constexpr int kCols = kColTiles * 16;
+    static constexpr int kGroups = kColTiles * 2;
+    __device__ __forceinline__ static int row(int g, int lane) { return (g / kColTiles) * 16 + (lane & 15); }
+    __device__ __forceinline__ static int col(int g, int lane) { return (g % kColTiles) * 16 + 4 * (lane >> 4); }
+    __device__ __forceinline__ float val(int ib, int g, int c, int half) const {
+        return acc[(g % kColTiles) + half * (TN16 / 2)][2 * ib + g / kColTiles][c];
+    }
+};
+
+// Epilogue through LDS.  In the accumulator layouts a lane owns 4 consecutive columns of one row,
 // so storing straight from registers would issue 8-byte pieces of 64 different cache lines per
 // instruction.  Instead every wave transposes 32-row blocks of its sub-tile through a private LDS
 // region and writes whole rows: 16 bytes per lane, 128-byte lines fully covered.
-// wstage: this wave's private region, 32 * (WCOLS * sizeof(TO) + 16) bytes.
+// wstage: this wave's private region, 32 * (columns * sizeof(TO) + 16) bytes.
 // SAVEGU (with SWIGLU): the gate and up accumulators themselves also go to gu[row, col] and gu[row, up_off + col]
 // (what the backward pass of a training step needs), through the same staging region.
 // DSILU (without SWIGLU): the tile is dh, the gradient of h = silu(g) * u; instead of storing it, every lane reads
 // the 16 bytes of g and of u that belong to its 16 bytes of dh (rounded to TO first, as a stored dh would be) from
 // gu and stores dg = dh * u * (s + g*s*(1-s)) and du = dh * g * s, s = sigmoid(g), to out[row, col] and
 // out[row, up_off + col]: the arithmetic of the elementwise gradient kernel, so the bits are the same.
-template <typename TO, int TM, int TN, bool SWIGLU, bool SAVEGU = false, bool DSILU = false>
-__device__ __forceinline__ void epilogue_staged(f32x16_t (&acc)[TN][TM], unsigned char* wstage, TO* out, int64_t ldo,
-                                                int64_t row_base, int rows_valid, int ncol0, int n_out, int lane,
-                                                TO* gu = nullptr, int64_t ldgu = 0, int up_off = 0) {
+template <typename TO, typename View, bool SWIGLU, bool SAVEGU = false, bool DSILU = false>
+__device__ __forceinline__ void epilogue_view(const View av, unsigned char* wstage, TO* out, int64_t ldo,
+                                              int64_t row_base, int rows_valid, int ncol0, int n_out, int lane,
+                                              TO* gu = nullptr, int64_t ldgu = 0, int up_off = 0) {
     static_assert(!SAVEGU || SWIGLU, "the second output exists for the SwiGLU epilogue only");
     static_assert(!DSILU || !SWIGLU, "the SwiGLU gradient epilogue belongs to the plain product");
-    constexpr int TNO = SWIGLU ? TN / 2 : TN;
-    constexpr int WCOLS = TNO * 32;
+    constexpr int WCOLS = View::kCols;
     constexpr int ES = (int)sizeof(TO);
     constexpr int PITCH = WCOLS * ES + 16;
     constexpr int LPR = WCOLS * ES / 16;   // lanes per output row
     constexpr int RPI = 64 / LPR;          // rows per store instruction
     constexpr int EPC = 16 / ES;           // elements per 16-byte chunk
-    const int frow = lane & 31, fgrp = lane >> 5;
 #pragma unroll
-    for (int i = 0; i < TM; ++i) {
+    for (int i = 0; i < View::kBlocks; ++i) {
 #pragma unroll
-        for (int j = 0; j < TNO; ++j) {
+        for (int g = 0; g < View::kGroups; ++g) {
+            float v[4];
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                float v[4];
-#pragma unroll
-                for (int c = 0; c < 4; ++c) {
-                    if (SWIGLU) v[c] = silu_f(acc[j][i][q * 4 + c]) * acc[j + TN / 2][i][q * 4 + c];
-                    else v[c] = acc[j][i][q * 4 + c];
-                }
-                unsigned char* dst = wstage + frow * PITCH + (j * 32 + 8 * q + 4 * fgrp) * ES;
-                if constexpr (ES == 2) {
-                    uint2 u;
-                    u.x = pack_bf16x2(v[0], v[1]);
-                    u.y = pack_bf16x2(v[2], v[3]);
-                    *reinterpret_cast<uint2*>(dst) = u;
-                } else {
-                    *reinterpret_cast<float4*>(dst) = make_float4(v[0], v[1], v[2], v[3]);
-                }
+            for (int c = 0; c < 4; ++c) {
+                if (SWIGLU) v[c] = silu_f(av.val(i, g, c, 0)) * av.val(i, g, c, 1);
+                else v[c] = av.val(i, g, c, 0);
+            }
+            unsigned char* dst = wstage + View::row(g, lane) * PITCH + View::col(g, lane) * ES;
+            if constexpr (ES == 2) {
+                uint2 u;
+                u.x = pack_bf16x2(v[0], v[1]);
+                u.y = pack_bf16x2(v[2], v[3]);
+                *reinterpret_cast<uint2*>(dst) = u;
+            } else {
+                *reinterpret_cast<float4*>(dst) = make_float4(v[0], v[1], v[2], v[3]);
             }
         }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
@@ -161,20 +192,16 @@ __device__ __forceinline__ void epilogue_staged(f32x16_t (&acc)[TN][TM], unsigne
 #pragma unroll
             for (int half = 0; half < 2; ++half) {
 #pragma unroll
-                for (int j = 0; j < TNO; ++j) {
-#pragma unroll
-                    for (int q = 0; q < 4; ++q) {
-                        const int jj = j + half * (TN / 2);
-                        unsigned char* dst = wstage + frow * PITCH + (j * 32 + 8 * q + 4 * fgrp) * ES;
-                        if constexpr (ES == 2) {
-                            uint2 u;
-                            u.x = pack_bf16x2(acc[jj][i][q * 4 + 0], acc[jj][i][q * 4 + 1]);
-                            u.y = pack_bf16x2(acc[jj][i][q * 4 + 2], acc[jj][i][q * 4 + 3]);
-                            *reinterpret_cast<uint2*>(dst) = u;
-                        } else {
-                            *reinterpret_cast<float4*>(dst) = make_float4(acc[jj][i][q * 4 + 0], acc[jj][i][q * 4 + 1],
-                                                                          acc[jj][i][q * 4 + 2], acc[jj][i][q * 4 + 3]);
-                        }
+                for (int g = 0; g < View::kGroups; ++g) {
+                    unsigned char* dst = wstage + View::row(g, lane) * PITCH + View::col(g, lane) * ES;
+                    if constexpr (ES == 2) {
+                        uint2 u;
+                        u.x = pack_bf16x2(av.val(i, g, 0, half), av.val(i, g, 1, half));
+                        u.y = pack_bf16x2(av.val(i, g, 2, half), av.val(i, g, 3, half));
+                        *reinterpret_cast<uint2*>(dst) = u;
+                    } else {
+                        *reinterpret_cast<float4*>(dst) = make_float4(av.val(i, g, 0, half), av.val(i, g, 1, half),
+                                                                      av.val(i, g, 2, half), av.val(i, g, 3, half));
                     }
                 }
                 asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
@@ -192,6 +219,15 @@ __device__ __forceinline__ void epilogue_staged(f32x16_t (&acc)[TN][TM], unsigne
             }
         }
     }
+}
+
+template <typename TO, int TM, int TN, bool SWIGLU, bool SAVEGU = false, bool DSILU = false>
+__device__ __forceinline__ void epilogue_staged(f32x16_t (&acc)[TN][TM], unsigned char* wstage, TO* out, int64_t ldo,
+                                                int64_t row_base, int rows_valid, int ncol0, int n_out, int lane,
+                                                TO* gu = nullptr, int64_t ldgu = 0, int up_off = 0) {
+    epilogue_view<TO, AccView32<TM, TN, SWIGLU>, SWIGLU, SAVEGU, DSILU>(AccView32<TM, TN, SWIGLU>{acc}, wstage, out, ldo,
+                                                                        row_base, rows_valid, ncol0, n_out, lane, gu,
+                                                                        ldgu, up_off);
 }
 
 template <typename T, typename TO, int BM, int BN, int WM, int WN, int SM, int SN, bool SWIGLU>
@@ -850,6 +886,241 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_dma_kernel(GroupedAr
 #endif
 }
 
+// bf16 prefill tile on v_mfma_f32_16x16x32_bf16.  Same data movement as grouped_gemm_dma_kernel (256 x 256 tile,
+// 8 waves of 128 x 64, direct-to-LDS slabs, three activation stages and two weight stages, the XOR swizzle
+// also spreads the 16 rows x 4 chunks of a 16-row fragment over all banks), but the products are formed by
+// the 16 x 16 x 32 instruction: with random bf16 operands the chip, which is power limited on this kernel,
+// sustains about 14 % more of them per second than of the 32 x 32 x 16 form (measured on MFMA-only loops:
+// 2.13 vs 1.86 PFLOP/s).
+//
+// A 64-element slab is two 32-element k-steps; the wave's 128 rows are two halves of four 16-row fragments.
+// A slab is four phases of 16 MFMAs, (k-step, row half) = (0,0) (0,1) (1,0) (1,1); fragments live in two
+// buffers of four activation fragments and two buffers of four weight fragments:
+//   phase 0 : MFMAs | reads: activations (k0, half 1), weights (k1) 0..1
+//   phase 1 : MFMAs | reads: activations (k1, half 0), weights (k1) 2..3
+//   phase 2 : MFMAs | reads: activations (k1, half 1)
+//   wait for the loads of slab t+1, barrier
+//   phase 3 : MFMAs | reads: activations (k0, half 0) and weights (k0) of slab t+1 | loads: weights of slab
+//             t+2, activations of slab t+3
+template <typename TO, int SM, int SN, bool SWIGLU, bool SAVEGU = false, bool DSILU = false>
+__global__ __launch_bounds__(512) void grouped_gemm_dma16_kernel(GroupedArgs p) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    typedef bf16_t T;
+    constexpr int BM = 256, BN = 256, WM = 2, WN = 4;
+    constexpr int NW = WM * WN;
+    constexpr int ES = 2;
+    constexpr int TM = 8;   // 16-row activation fragments per wave
+    constexpr int TN = 4;   // 16-row weight fragments per wave
+    constexpr int NIA = BM / 8 / NW;
+    constexpr int NIB = BN / 8 / NW;
+    constexpr int HALF = BN / 2;
+    constexpr int A_STAGE = BM * 128;
+    constexpr int B_STAGE = BN * 128;
+    constexpr int B_BASE = 3 * A_STAGE;
+    static_assert(SM * SN == kSuperBlocks, "supertile");
+
+    extern __shared__ __align__(16) unsigned char smem[];
+    typedef __attribute__((address_space(3))) void* lds_ptr_t;
+
+    TileCoord tc;
+    if (!decode_tile(blockIdx.x, p.row_count, p.E, BM, p.n_tiles, SM, SN, &tc)) return;
+    const int count = p.row_count[tc.e];
+    const int row0 = p.row_start[tc.e];
+    const int K = p.k_count ? p.k_count[tc.e] : p.K;
+    const T* Bexp = static_cast<const T*>(p.b[tc.e]);
+    const T* A = static_cast<const T*>(p.a_ptrs ? p.a_ptrs[tc.e] : p.a);
+    const int arow0 = p.a_ptrs ? 0 : row0;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave / WN, wn = wave % WN;
+
+    // ---- load descriptors and lane offsets: instruction j of this wave covers rows (j*NW + wave)*8 .. +8
+    constexpr int kRsrcFlags = 0x00020000;  // raw buffer, 32-bit data format
+    const bool gather = p.a_rows != nullptr;
+    const T* a_base = gather ? A : A + ((int64_t)arow0 + (int64_t)tc.mt * BM) * p.lda;
+    const __amdgpu_buffer_rsrc_t rsrc_a =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(a_base), 0, (int)p.a_extent_bytes, kRsrcFlags);
+    const __amdgpu_buffer_rsrc_t rsrc_b =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(Bexp), 0, (int)p.b_extent_bytes, kRsrcFlags);
+    const int drow = lane >> 3;
+    const int dchunk = (lane & 7) ^ drow ^ (wave & 1);
+    unsigned ao[NIA], bo[NIB];
+#pragma unroll
+    for (int j = 0; j < NIA; ++j) {
+        int m = tc.mt * BM + (j * NW + wave) * 8 + drow;
+        m = m < count ? m : count - 1;
+        int64_t src = gather ? (int64_t)(p.a_rows[arow0 + m] / p.a_row_div) : (int64_t)(m - tc.mt * BM);
+        ao[j] = (unsigned)(src * p.lda * ES + dchunk * 16);
+    }
+#pragma unroll
+    for (int j = 0; j < NIB; ++j) {
+        const int rb = (j * NW + wave) * 8 + drow;
+        int n, brow;
+        if (SWIGLU) {
+            const bool up = rb >= HALF;
+            n = tc.nt * HALF + (up ? rb - HALF : rb);
+            n = n < p.N_out ? n : p.N_out - 1;
+            brow = up ? p.up_offset + n : n;
+        } else {
+            n = tc.nt * BN + rb;
+            n = n < p.N_out ? n : p.N_out - 1;
+            brow = n;
+        }
+        bo[j] = (unsigned)((int64_t)brow * p.ldb * ES + dchunk * 16);
+    }
+    unsigned char* const dma_a = smem + wave * 1024;
+    unsigned char* const dma_b = smem + B_BASE + wave * 1024;
+
+    f32x4_t acc[TN][TM];
+#pragma unroll
+    for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int i = 0; i < TM; ++i) acc[j][i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+    const int nk = K * ES / 128;
+
+    // ---- fragment addresses: one register per k-step and operand; fragments and weight stages by offset
+    const int frow = lane & 15;
+    const int kgrp = lane >> 4;
+    const int fsw = (frow & 7) ^ ((frow >> 3) & 1);
+    const unsigned char* fa_addr[2];
+    const unsigned char* fb_addr[2];
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+        const int slot = (4 * ks + kgrp) ^ fsw;
+        fa_addr[ks] = smem + (wm * (BM / WM) + frow) * 128 + slot * 16;
+        fb_addr[ks] = smem + B_BASE + (wn * (SWIGLU ? BN / WN / 2 : BN / WN) + frow) * 128 + slot * 16;
+    }
+    u32x4_t fa[2][4], fb[2][TN];
+
+#define D16_ISSUE_A(kt_, aoff_)                                                                        \
+    {                                                                                                  \
+        const int soff = (kt_) * 128;                                                                  \
+        _Pragma("unroll") for (int j = 0; j < NIA; ++j)                                                \
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(                                                  \
+                rsrc_a, (lds_ptr_t)(dma_a + (aoff_) + j * NW * 1024), 16, ao[j], soff, 0, 0);          \
+    }
+#define D16_ISSUE_B(kt_, stage_)                                                                       \
+    {                                                                                                  \
+        const int soff = (kt_) * 128;                                                                  \
+        _Pragma("unroll") for (int j = 0; j < NIB; ++j)                                                \
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(                                                  \
+                rsrc_b, (lds_ptr_t)(dma_b + (stage_) * B_STAGE + j * NW * 1024), 16, bo[j], soff, 0, 0); \
+    }
+#define D16_B_ROW(j_) (SWIGLU ? ((j_) < TN / 2 ? (j_) * 16 : HALF + ((j_) - TN / 2) * 16) : (j_) * 16)
+#define D16_READ_A(aoff_, ks_, half_, buf_)                                                            \
+    {                                                                                                  \
+        const unsigned char* fa_ = fa_addr[ks_] + (aoff_) + (half_) * 8192;                            \
+        _Pragma("unroll") for (int i = 0; i < 4; ++i)                                                  \
+            fa[buf_][i] = *reinterpret_cast<const u32x4_t*>(fa_ + i * 2048);                           \
+    }
+#define D16_READ_B(stage_, ks_, j_, buf_) \
+    fb[buf_][j_] = *reinterpret_cast<const u32x4_t*>(fb_addr[ks_] + (stage_) * B_STAGE + D16_B_ROW(j_) * 128)
+#define D16_MMA(bbuf_, abuf_, half_)                                                                   \
+    {                                                                                                  \
+        _Pragma("unroll") for (int j = 0; j < TN; ++j)                                                 \
+            _Pragma("unroll") for (int i = 0; i < 4; ++i) {                                            \
+                union {                                                                                \
+                    u32x4_t u;                                                                         \
+                    bf16x8_t v;                                                                        \
+                } w_, a_;                                                                              \
+                w_.u = fb[bbuf_][j];                                                                   \
+                a_.u = fa[abuf_][i];                                                                   \
+                acc[j][(half_) * 4 + i] =                                                              \
+                    __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_.v, a_.v, acc[j][(half_) * 4 + i], 0, 0, 0); \
+            }                                                                                          \
+    }
+// nrd fragment reads spread over the first MFMAs of a phase (16 MFMAs)
+#define D16_MIX(nrd_)                                                                   \
+    _Pragma("unroll") for (int g_ = 0; g_ < (nrd_); ++g_) {                             \
+        __builtin_amdgcn_sched_group_barrier(SG_MFMA, 16 / ((nrd_) + 2), 0);            \
+        __builtin_amdgcn_sched_group_barrier(SG_DS_RD, 1, 0);                           \
+    }
+// phase 3: one fragment read and one load per MFMA while they last
+#define D16_MIX_DMA()                                                                   \
+    _Pragma("unroll") for (int g_ = 0; g_ < 8; ++g_) {                                  \
+        __builtin_amdgcn_sched_group_barrier(SG_DS_RD, 1, 0);                           \
+        __builtin_amdgcn_sched_group_barrier(SG_MFMA, 1, 0);                            \
+        __builtin_amdgcn_sched_group_barrier(SG_VMEM, 1, 0);                            \
+    }
+// STG: weight stage of slab kt (compile time); sa_cur / sa_nxt: activation stage offsets of slabs kt, kt+1.
+// Slabs past the end are clamped to the last one (their loads land in stages nobody reads again).
+#define D16_ITER(kt_, STG)                                                              \
+    {                                                                                   \
+        D16_READ_A(sa_cur, 0, 1, 1);                                                    \
+        D16_READ_B(STG, 1, 0, 1);                                                       \
+        D16_READ_B(STG, 1, 1, 1);                                                       \
+        D16_MMA(0, 0, 0);                                                               \
+        D16_MIX(6);                                                                     \
+        PL_FENCE();                                                                     \
+        D16_READ_A(sa_cur, 1, 0, 0);                                                    \
+        D16_READ_B(STG, 1, 2, 1);                                                       \
+        D16_READ_B(STG, 1, 3, 1);                                                       \
+        D16_MMA(0, 1, 1);                                                               \
+        D16_MIX(6);                                                                     \
+        PL_FENCE();                                                                     \
+        D16_READ_A(sa_cur, 1, 1, 1);                                                    \
+        D16_MMA(1, 0, 0);                                                               \
+        D16_MIX(4);                                                                     \
+        PL_FENCE();                                                                     \
+        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(NIA) : "memory"); \
+        PL_FENCE();                                                                     \
+        D16_READ_B(STG ^ 1, 0, 0, 0);                                                   \
+        D16_READ_A(sa_nxt, 0, 0, 0);                                                    \
+        D16_READ_B(STG ^ 1, 0, 1, 0);                                                   \
+        D16_READ_B(STG ^ 1, 0, 2, 0);                                                   \
+        D16_READ_B(STG ^ 1, 0, 3, 0);                                                   \
+        D16_ISSUE_B(min((kt_) + 2, nk - 1), STG);                                       \
+        D16_ISSUE_A(min((kt_) + 3, nk - 1), sa_cur);                                    \
+        D16_MMA(1, 1, 1);                                                               \
+        D16_MIX_DMA();                                                                  \
+        PL_FENCE();                                                                     \
+        sa_cur = sa_nxt;                                                                \
+        sa_nxt = sa_nxt == 2 * A_STAGE ? 0 : sa_nxt + A_STAGE;                          \
+    }
+
+    D16_ISSUE_A(0, 0);
+    D16_ISSUE_B(0, 0);
+    D16_ISSUE_A(min(1, nk - 1), A_STAGE);
+    D16_ISSUE_B(min(1, nk - 1), 1);
+    D16_ISSUE_A(min(2, nk - 1), 2 * A_STAGE);
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(2 * NIA + NIB) : "memory");
+    int sa_cur = 0, sa_nxt = A_STAGE;
+    D16_READ_A(sa_cur, 0, 0, 0);
+#pragma unroll
+    for (int j = 0; j < TN; ++j) D16_READ_B(0, 0, j, 0);
+    int kt = 0;
+    for (; kt + 1 < nk; kt += 2) {
+        D16_ITER(kt, 0);
+        D16_ITER(kt + 1, 1);
+    }
+    if (kt < nk) D16_ITER(kt, 0);
+    // the clamped loads of the last slabs may still be in flight; the epilogue reuses LDS
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+#undef D16_ISSUE_A
+#undef D16_ISSUE_B
+#undef D16_B_ROW
+#undef D16_READ_A
+#undef D16_READ_B
+#undef D16_MMA
+#undef D16_MIX
+#undef D16_MIX_DMA
+#undef D16_ITER
+
+    {
+        typedef AccView16<TM, TN, SWIGLU> View;
+        constexpr int WSTAGE = 32 * (View::kCols * (int)sizeof(TO) + 16);
+        const int wrow = tc.mt * BM + wm * (BM / WM);
+        const int ncol0 = SWIGLU ? tc.nt * HALF + wn * (BN / WN / 2) : tc.nt * BN + wn * (BN / WN);
+        epilogue_view<TO, View, SWIGLU, SAVEGU, DSILU>(View{acc}, smem + wave * WSTAGE, static_cast<TO*>(p.out), p.ldo,
+                                                       (int64_t)row0 + wrow, count - wrow, ncol0, p.N_out, lane,
+                                                       static_cast<TO*>(p.gu_out), p.ld_gu, p.up_offset);
+    }
+#endif
+}
+
 #undef PL_STORE
 #undef PL_READ
 #undef PL_MMA
@@ -873,7 +1144,10 @@ static int launch_cfg(const GroupedArgs& p0, int64_t max_rows, hipStream_t s) {
     constexpr bool kWarm = BM > 64;
     auto kern_pipe = grouped_gemm_pipelined_kernel<T, TO, BM, BN, WM, WN, SM, SN, SWIGLU, kWarm>;
     auto kern_dma = [] {
-        if constexpr (DMA) return grouped_gemm_dma_kernel<T, TO, BM, BN, WM, WN, SM, SN, SWIGLU>;
+        if constexpr (DMA && std::is_same<T, bf16_t>::value) {
+            static_assert(BM == 256 && BN == 256 && WM == 2 && WN == 4, "the 16 x 16 x 32 kernel is the 256 x 256 tile");
+            return grouped_gemm_dma16_kernel<TO, SM, SN, SWIGLU>;
+        } else if constexpr (DMA) return grouped_gemm_dma_kernel<T, TO, BM, BN, WM, WN, SM, SN, SWIGLU>;
         else return grouped_gemm_pipelined_kernel<T, TO, BM, BN, WM, WN, SM, SN, SWIGLU, kWarm>;
     }();
     if (smem > 64 * 1024) {
@@ -963,7 +1237,10 @@ static int launch_gateup_save(const GroupedArgs& p0, int64_t max_rows, hipStream
     GroupedArgs p = p0;
     p.n_tiles = (p.N_out + BN / 2 - 1) / (BN / 2);
     constexpr size_t smem = dma_lds_bytes(BM, BN);
-    auto kern = grouped_gemm_dma_kernel<T, T, BM, BN, 2, 4, 4, 8, true, true>;
+    auto kern = [] {
+        if constexpr (std::is_same<T, bf16_t>::value) return grouped_gemm_dma16_kernel<T, 4, 8, true, true>;
+        else return grouped_gemm_dma_kernel<T, T, BM, BN, 2, 4, 4, 8, true, true>;
+    }();
     static LdsReservation reserved;
     hipError_t e = reserve_lds(reserved, {reinterpret_cast<const void*>(kern)}, (int)smem);
     if (e != hipSuccess) {
@@ -994,7 +1271,10 @@ static int launch_down_dgrad_dsilu(const GroupedArgs& p0, int64_t max_rows, hipS
     GroupedArgs p = p0;
     p.n_tiles = (p.N_out + BN - 1) / BN;
     constexpr size_t smem = dma_lds_bytes(BM, BN);
-    auto kern = grouped_gemm_dma_kernel<T, T, BM, BN, 2, 4, 4, 8, false, false, true>;
+    auto kern = [] {
+        if constexpr (std::is_same<T, bf16_t>::value) return grouped_gemm_dma16_kernel<T, 4, 8, false, false, true>;
+        else return grouped_gemm_dma_kernel<T, T, BM, BN, 2, 4, 4, 8, false, false, true>;
+    }();
     static LdsReservation reserved;
     hipError_t e = reserve_lds(reserved, {reinterpret_cast<const void*>(kern)}, (int)smem);
     if (e != hipSuccess) {
