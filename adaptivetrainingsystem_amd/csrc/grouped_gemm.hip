@@ -1047,38 +1047,61 @@ __global__ __launch_bounds__(512) void grouped_gemm_dma16_kernel(GroupedArgs p) 
     }
 // STG: weight stage of slab kt (compile time); sa_cur / sa_nxt: activation stage offsets of slabs kt, kt+1.
 // Slabs past the end are clamped to the last one (their loads land in stages nobody reads again).
-#define D16_ITER(kt_, STG)                                                              \
+// H0 / H1 (compile time): whether row half 0 / 1 of this wave holds rows of the expert at all; a half made
+// only of rows past the expert's end keeps its loads and barriers but skips its fragment reads and MFMAs.
+#define D16_ITER(kt_, STG, H0, H1)                                                      \
     {                                                                                   \
-        D16_READ_A(sa_cur, 0, 1, 1);                                                    \
-        D16_READ_B(STG, 1, 0, 1);                                                       \
-        D16_READ_B(STG, 1, 1, 1);                                                       \
-        D16_MMA(0, 0, 0);                                                               \
-        D16_MIX(6);                                                                     \
+        if (H1) D16_READ_A(sa_cur, 0, 1, 1);                                            \
+        if (H0) {                                                                       \
+            D16_READ_B(STG, 1, 0, 1);                                                   \
+            D16_READ_B(STG, 1, 1, 1);                                                   \
+            D16_MMA(0, 0, 0);                                                           \
+            D16_MIX(H1 ? 6 : 2);                                                        \
+        }                                                                               \
         PL_FENCE();                                                                     \
-        D16_READ_A(sa_cur, 1, 0, 0);                                                    \
-        D16_READ_B(STG, 1, 2, 1);                                                       \
-        D16_READ_B(STG, 1, 3, 1);                                                       \
-        D16_MMA(0, 1, 1);                                                               \
-        D16_MIX(6);                                                                     \
+        if (H0) {                                                                       \
+            D16_READ_A(sa_cur, 1, 0, 0);                                                \
+            D16_READ_B(STG, 1, 2, 1);                                                   \
+            D16_READ_B(STG, 1, 3, 1);                                                   \
+        }                                                                               \
+        if (H1) {                                                                       \
+            D16_MMA(0, 1, 1);                                                           \
+            D16_MIX(6);                                                                 \
+        }                                                                               \
         PL_FENCE();                                                                     \
-        D16_READ_A(sa_cur, 1, 1, 1);                                                    \
-        D16_MMA(1, 0, 0);                                                               \
-        D16_MIX(4);                                                                     \
+        if (H1) D16_READ_A(sa_cur, 1, 1, 1);                                            \
+        if (H0) {                                                                       \
+            D16_MMA(1, 0, 0);                                                           \
+            D16_MIX(H1 ? 4 : 0);                                                        \
+        }                                                                               \
         PL_FENCE();                                                                     \
         asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(NIA) : "memory"); \
         PL_FENCE();                                                                     \
-        D16_READ_B(STG ^ 1, 0, 0, 0);                                                   \
-        D16_READ_A(sa_nxt, 0, 0, 0);                                                    \
-        D16_READ_B(STG ^ 1, 0, 1, 0);                                                   \
-        D16_READ_B(STG ^ 1, 0, 2, 0);                                                   \
-        D16_READ_B(STG ^ 1, 0, 3, 0);                                                   \
+        if (H0) {                                                                       \
+            D16_READ_B(STG ^ 1, 0, 0, 0);                                               \
+            D16_READ_A(sa_nxt, 0, 0, 0);                                                \
+            D16_READ_B(STG ^ 1, 0, 1, 0);                                               \
+            D16_READ_B(STG ^ 1, 0, 2, 0);                                               \
+            D16_READ_B(STG ^ 1, 0, 3, 0);                                               \
+        }                                                                               \
         D16_ISSUE_B(min((kt_) + 2, nk - 1), STG);                                       \
         D16_ISSUE_A(min((kt_) + 3, nk - 1), sa_cur);                                    \
-        D16_MMA(1, 1, 1);                                                               \
-        D16_MIX_DMA();                                                                  \
+        if (H1) {                                                                       \
+            D16_MMA(1, 1, 1);                                                           \
+            D16_MIX_DMA();                                                              \
+        }                                                                               \
         PL_FENCE();                                                                     \
         sa_cur = sa_nxt;                                                                \
         sa_nxt = sa_nxt == 2 * A_STAGE ? 0 : sa_nxt + A_STAGE;                          \
+    }
+#define D16_LOOP(H0, H1)                                                                \
+    {                                                                                   \
+        int kt = 0;                                                                     \
+        for (; kt + 1 < nk; kt += 2) {                                                  \
+            D16_ITER(kt, 0, H0, H1);                                                    \
+            D16_ITER(kt + 1, 1, H0, H1);                                                \
+        }                                                                               \
+        if (kt < nk) D16_ITER(kt, 0, H0, H1);                                           \
     }
 
     D16_ISSUE_A(0, 0);
@@ -1088,17 +1111,24 @@ __global__ __launch_bounds__(512) void grouped_gemm_dma16_kernel(GroupedArgs p) 
     D16_ISSUE_A(min(2, nk - 1), 2 * A_STAGE);
     asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(2 * NIA + NIB) : "memory");
     int sa_cur = 0, sa_nxt = A_STAGE;
-    D16_READ_A(sa_cur, 0, 0, 0);
+    // rows of the expert in this wave's 128-row share of the tile (wave-uniform)
+    const int wave_rows = count - (tc.mt * BM + wm * (BM / WM));
+    if (wave_rows > 64) {
+        D16_READ_A(sa_cur, 0, 0, 0);
 #pragma unroll
-    for (int j = 0; j < TN; ++j) D16_READ_B(0, 0, j, 0);
-    int kt = 0;
-    for (; kt + 1 < nk; kt += 2) {
-        D16_ITER(kt, 0);
-        D16_ITER(kt + 1, 1);
+        for (int j = 0; j < TN; ++j) D16_READ_B(0, 0, j, 0);
+        D16_LOOP(true, true);
+    } else if (wave_rows > 0) {
+        D16_READ_A(sa_cur, 0, 0, 0);
+#pragma unroll
+        for (int j = 0; j < TN; ++j) D16_READ_B(0, 0, j, 0);
+        D16_LOOP(true, false);
+    } else {
+        D16_LOOP(false, false);
     }
-    if (kt < nk) D16_ITER(kt, 0);
     // the clamped loads of the last slabs may still be in flight; the epilogue reuses LDS
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+#undef D16_LOOP
 #undef D16_ISSUE_A
 #undef D16_ISSUE_B
 #undef D16_B_ROW
