@@ -40,13 +40,16 @@ class StageTimer:
         self._events.clear()
 
     def summary(self) -> Dict[str, Dict[str, float]]:
-        """Synchronises once and returns {stage: {calls, mean_ms, min_ms, total_ms, median_ms, max_ms}}."""
+        """Synchronises once and returns {stage: {calls, mean_ms, min_ms, total_ms, median_ms, p10_ms, p90_ms,
+        max_ms}} (percentiles by nearest rank)."""
         torch.cuda.synchronize()
         out = {}
         for name, pairs in self._events.items():
-            ms = [a.elapsed_time(b) for a, b in pairs]
-            out[name] = {"calls": len(ms), "mean_ms": sum(ms) / len(ms), "min_ms": min(ms), "total_ms": sum(ms),
-                         "median_ms": sorted(ms)[len(ms) // 2], "max_ms": max(ms)}
+            ms = sorted(a.elapsed_time(b) for a, b in pairs)
+            n = len(ms)
+            out[name] = {"calls": n, "mean_ms": sum(ms) / n, "min_ms": ms[0], "total_ms": sum(ms),
+                         "median_ms": ms[n // 2], "p10_ms": ms[min(n - 1, int(0.1 * n))],
+                         "p90_ms": ms[min(n - 1, int(0.9 * n))], "max_ms": ms[-1]}
         return out
 
 
@@ -57,3 +60,28 @@ def _null_range():
 
 def stage(timer, name: str):
     return timer.range(name) if timer is not None else _null_range()
+
+
+def calibrate_mfma(shape: str = "16x16x32", random_operands: bool = True, iters: int = 0, reps: int = 4):
+    """MFMA-only loop (operands in registers, no memory traffic): what the matrix cores sustain on this
+    machine with all-zero or with random bf16 operands.  Returns {"tflops", "core_clock_mhz", "ms"} of the
+    last of `reps` back-to-back launches (the core clock settles during the first ones)."""
+    import ctypes
+
+    from . import _lib
+    from .ops import _stream
+    code = {"32x32x16": 0, "16x16x32": 1}[shape]
+    iters = iters or (16000 if code == 0 else 8000)     # about 4 ms per launch
+    lib = _lib.load()
+    clocks = torch.zeros(2, dtype=torch.int64, device="cuda")
+    flop = ctypes.c_double(0.0)
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    for _ in range(reps):
+        ev0.record()
+        _lib.check(lib.ats_calibrate_mfma(code, int(random_operands), iters, clocks.data_ptr(), ctypes.byref(flop),
+                                          _stream()), "ats_calibrate_mfma")
+        ev1.record()
+    torch.cuda.synchronize()
+    ms = ev0.elapsed_time(ev1)
+    c = clocks.cpu().tolist()
+    return {"tflops": flop.value / (ms * 1e-3) / 1e12, "core_clock_mhz": 100.0 * c[0] / max(c[1], 1), "ms": ms}

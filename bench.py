@@ -32,11 +32,21 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 PEAK_MFMA_BF16_TFLOPS = 2500.0   # MI355X dense bf16
+PEAK_MFMA_TFLOPS = {"bf16": 2500.0, "f32": 157.3}   # MI355X dense MFMA peaks by arithmetic type
 PEAK_HBM_GBS = 8000.0            # MI355X HBM3E
-# HBM-side bytes per launch of the gate/up GEMM, from separate hardware-counter runs of this script
-# (FETCH_SIZE x 2.0 + WRITE_SIZE x 1.0, factors from a 1 GiB copy; summary under profiles/).
-GATEUP_HBM_BYTES_PER_LAUNCH = {"c4_prefill": 11.56e9, "c3_decode": 1.8871e9}
-ATTENTION_DECODE_HBM_BYTES_PER_LAUNCH = 538.0e6
+
+
+def profile_traffic(workload: str, kernel: str):
+    """HBM-side bytes per launch of a kernel, from the tracked hardware-counter summaries: lines
+    `bench-traffic <workload> <kernel> <bytes>` in profiles/*hbm_traffic.txt (None when no summary has one)."""
+    import glob
+    for path in sorted(glob.glob(os.path.join(ROOT, "profiles", "*hbm_traffic.txt"))):
+        with open(path) as f:
+            for line in f:
+                parts = line.split()
+                if len(parts) == 4 and parts[0] == "bench-traffic" and parts[1] == workload and parts[2] == kernel:
+                    return float(parts[3])
+    return None
 
 
 def log(*a):
@@ -58,9 +68,62 @@ def cpu_baseline(w, sample_tokens: int):
     r = O.moe_forward_capacity(x, gate, gu, dn, **kw)
     dt = time.perf_counter() - t0
     kept = int(r["kept"].sum())
-    return {"value": sample_tokens / dt, "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
-            "sample": f"first {sample_tokens} tokens of the workload, same weights, float32, one pass "
-                      f"({dt:.2f} s, {kept} kept assignments)"}
+    out = {"value": sample_tokens / dt, "unit": "tokens/s", "cores": torch.get_num_threads(), "kind": "port",
+           "sample": f"first {sample_tokens} tokens of the workload, same weights, float32, one pass "
+                     f"({dt:.2f} s, {kept} kept assignments)"}
+    if w.name == "c1_cpu_reference":
+        # the reference's own per-token / per-expert Python loops (moe_cuda_wrapper.py:316-324, 343-357), once
+        t0 = time.perf_counter()
+        O.moe_forward_capacity(x, gate, gu, dn, literal_loops=True, **kw)
+        out["literal_loops_c1"] = sample_tokens / (time.perf_counter() - t0)
+    return out
+
+
+def gemm_calibration(w, moe, plan, kept: int, gu_ms: float):
+    """What bounds the grouped GEMM on this machine, measured in the same process: MFMA-only loops with zero
+    and with random operands (the gap is the board's power limit), this library's gate/up kernel on all-zero
+    operands with the same row plan (its schedule without the power limit), and the vendor library's dense
+    bf16 matmul of the same M x N x K."""
+    from adaptivetrainingsystem_amd import ops
+    from adaptivetrainingsystem_amd.profiling import StageTimer, calibrate_mfma
+    H, I, E, k = w.hidden, w.intermediate, w.num_experts, w.top_k
+    out = {"mfma_only": {}}
+    for shape in ("16x16x32", "32x32x16"):
+        for rnd in (False, True):
+            r = calibrate_mfma(shape, rnd)
+            out["mfma_only"][f"{shape}_{'random' if rnd else 'zero'}_operands"] = {
+                "tflops": round(r["tflops"], 1), "core_clock_mhz": round(r["core_clock_mhz"])}
+    rows = min(plan["row_of"].numel(), E * plan["capacity"])
+    # the same launch on zero operands: the tile schedule, loads and barriers without operand-dependent power
+    x0 = torch.zeros(w.tokens, H, dtype=w.dtype, device=w.x.device)
+    wz = [torch.zeros(2 * I, H, dtype=w.dtype, device=w.x.device) for _ in range(E)]
+    ptrs = ops.weight_pointer_table(wz)
+    timer = StageTimer()
+    for i in range(6):
+        with timer.range("z" if i >= 2 else "warm"):
+            ops.grouped_gateup_swiglu(x0, ptrs, plan["offsets"], plan["kept"], rows, rows, H, I,
+                                      a_rows=plan["row_src"], a_row_div=k)
+    z_ms = timer.summary()["z"]["mean_ms"]
+    del wz, ptrs, x0
+    out["gateup_zero_operands"] = {"tflops": round(4.0 * H * I * kept / (z_ms * 1e-3) / 1e12, 1), "ms": round(z_ms, 4)}
+    out["gateup_random_operands"] = {"tflops": round(4.0 * H * I * kept / (gu_ms * 1e-3) / 1e12, 1), "ms": round(gu_ms, 4)}
+    # vendor BLAS, dense, same M x N x K as the grouped launch (M = kept rows)
+    a = torch.randn(kept, H, device=w.x.device).to(w.dtype)
+    ref = {}
+    for key, wt, flop in (("gateup_shape", w.gate_up[0], 4.0 * H * I * kept), ("down_shape", None, 2.0 * H * I * kept)):
+        if wt is None:
+            a = torch.randn(kept, I, device=w.x.device).to(w.dtype) * 0.1
+            wt = w.down[0]
+        timer = StageTimer()
+        for i in range(8):
+            with timer.range("m" if i >= 3 else "warm"):
+                torch.matmul(a, wt.t())
+        ms = timer.summary()["m"]["mean_ms"]
+        ref[key] = {"m_n_k": [kept, wt.shape[0], wt.shape[1]], "tflops": round(flop / (ms * 1e-3) / 1e12, 1),
+                    "ms": round(ms, 4)}
+    out["gemm_reference"] = {"what": "torch.matmul (vendor BLAS) on one dense bf16 problem of the grouped launch's "
+                                     "M x N x K, random operands, same process", **ref}
+    return out
 
 
 def run_moe(args):
@@ -69,12 +132,14 @@ def run_moe(args):
 
     dev = torch.device("cuda:0")
     name = args.workload
-    w = W.make_moe_workload(name, device=dev, gen_device="cuda")
+    # CPU-seeded generator where the tensors are small enough to draw on the host in seconds
+    gen_device = "cpu" if name in ("c1_cpu_reference", "c3_decode") else "cuda"
+    w = W.make_moe_workload(name, device=dev, gen_device=gen_device)
     layer = W.build_layer(w, "fcfs")
     moe = layer.moe if hasattr(layer, "moe") else layer
     T_in = w.tokens
     log(f"workload {name}: tokens={T_in} H={w.hidden} E={w.num_experts} k={w.top_k} I={w.intermediate} "
-        f"cf={w.capacity_factor} dtype={w.dtype}")
+        f"cf={w.capacity_factor} dtype={w.dtype} (inputs drawn on {gen_device})")
 
     with torch.no_grad():
         for _ in range(args.warmup):
@@ -102,11 +167,13 @@ def run_moe(args):
     T_moe = plan["row_of"].numel() // w.top_k
     dropped = T_moe * w.top_k - kept
     for s, v in stages.items():
-        log(f"  stage {s:14s} mean {v['mean_ms']:9.4f} ms  min {v['min_ms']:9.4f} ms  ({v['calls']} calls)")
+        log(f"  stage {s:14s} mean {v['mean_ms']:9.4f} ms  median {v['median_ms']:9.4f}  p10 {v['p10_ms']:9.4f}  "
+            f"p90 {v['p90_ms']:9.4f}  min {v['min_ms']:9.4f} ms  ({v['calls']} calls)")
     log(f"  kept assignments {kept} of {T_moe * w.top_k} (dropped {dropped}); capacity {plan['capacity']}; hist {hist}")
     log(f"  finite output: {bool(torch.isfinite(out.float()).all())}, aux {float(aux):.6f}")
 
     H, I = w.hidden, w.intermediate
+    dtype_name = "bf16" if w.dtype == torch.bfloat16 else "f32"
     gu_ms = stages["gateup_swiglu"]["mean_ms"]
     gu_flops = 4.0 * H * I * kept
     achieved = gu_flops / (gu_ms * 1e-3) / 1e12
@@ -114,31 +181,39 @@ def run_moe(args):
     log(f"  gate/up GEMM {achieved:.1f} TFLOP/s; down GEMM {2.0 * H * I * kept / (dn_ms * 1e-3) / 1e12:.1f} TFLOP/s")
     ms_per_step = dt / args.steps * 1e3
     es = 2 if w.dtype == torch.bfloat16 else 4
-    if kept / w.num_experts <= 48:
+    mfma_bound = kept / w.num_experts > 48
+    if not mfma_bound:
         # decode-sized groups: the gate/up kernel streams the weights of the active experts once
         active = sum(1 for c in plan["kept"].cpu().tolist() if c > 0)
         gu_bytes = active * 2.0 * I * H * es + kept * (H + I) * es
         gbs = gu_bytes / (gu_ms * 1e-3) / 1e9
         roofline = {"kernel": "grouped gate/up GEMM + SwiGLU (weight streaming)", "bound": "hbm", "achieved": gbs,
                     "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS,
-                    "traffic": GATEUP_HBM_BYTES_PER_LAUNCH.get(name)}
+                    "traffic": profile_traffic(name, "gateup")}
     else:
+        peak = PEAK_MFMA_TFLOPS[dtype_name]
         roofline = {"kernel": "grouped gate/up GEMM + SwiGLU", "bound": "mfma", "achieved": achieved,
-                    "peak": PEAK_MFMA_BF16_TFLOPS, "unit": "TFLOP/s", "frac": achieved / PEAK_MFMA_BF16_TFLOPS,
-                    "traffic": GATEUP_HBM_BYTES_PER_LAUNCH.get(name)}
+                    "peak": peak, "unit": "TFLOP/s", "frac": achieved / peak,
+                    "traffic": profile_traffic(name, "gateup")}
     result = {
-        "metric": "MoE-layer tokens/s (h4096, 8e top-2, bf16) + % of MFMA/HBM roofline",
+        "metric": f"MoE-layer tokens/s (h{H}, {w.num_experts}e top-{w.top_k}, {dtype_name}) + % of MFMA/HBM roofline",
         "value": T_in * args.steps / dt, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16" if w.dtype == torch.bfloat16 else "f32", "data": "synthetic",
+        "dtype": dtype_name, "data": "synthetic",
         "config": {"workload": f"{name}: MoE layer forward, {T_in} tokens, hidden {H}, {w.num_experts} experts, "
                                f"top-{w.top_k}, intermediate {I}, capacity_factor {w.capacity_factor}"
                                + (", Zipf-skewed router logits" if w.zipf_bias else "")
                                + (f", MoD keeps {w.mod_keep_fraction:.3f} of each sequence" if w.mod_keep_fraction else ""),
-                   "kept_assignments": kept, "dropped_assignments": dropped},
+                   "kept_assignments": kept, "dropped_assignments": dropped, "inputs_drawn_on": gen_device},
         "roofline": roofline,
         "stages_ms": {s: round(v["mean_ms"], 4) for s, v in stages.items()},
+        "stages_median_p10_p90_ms": {s: [round(v["median_ms"], 4), round(v["p10_ms"], 4), round(v["p90_ms"], 4)]
+                                     for s, v in stages.items()},
     }
+    if mfma_bound and w.dtype == torch.bfloat16 and not args.no_calibration:
+        with torch.no_grad():
+            result["calibration"] = gemm_calibration(w, moe, plan, kept, gu_ms)
+        log(f"  calibration: {json.dumps(result['calibration'])}")
     if not args.no_cpu_baseline:
         sample = min(args.cpu_sample_tokens, T_moe)
         src = w
@@ -500,7 +575,7 @@ def run_attention_decode(args):
                                f"{Hkv} kv heads, head_dim {D}"},
         "roofline": {"kernel": "attention_fwd_kernel, packed rows", "bound": "hbm", "achieved": achieved,
                      "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": achieved / PEAK_HBM_GBS,
-                     "traffic": ATTENTION_DECODE_HBM_BYTES_PER_LAUNCH},
+                     "traffic": profile_traffic("attention_decode", "attention")},
         "stages_ms": {s_: round(v_["mean_ms"], 4) for s_, v_ in st.items()},
     }
     if not args.no_cpu_baseline:
@@ -640,7 +715,7 @@ def run_norm_rope(args):
     from adaptivetrainingsystem_amd import workloads as W
     from adaptivetrainingsystem_amd.profiling import StageTimer
     dev = torch.device("cuda:0")
-    w = W.make_norm_rope_workload(device=dev, gen_device="cuda")
+    w = W.make_norm_rope_workload(device=dev, gen_device="cpu")
     cos, sin = ops.rope_table(w.seq, w.head_dim, w.theta, device=dev)
     # The inputs of one step are 75 MB: repeated over the same buffers they would be served by the 256 MB
     # memory-side cache, not by HBM.  The calls therefore rotate over 16 copies (1.2 GB of inputs).
@@ -739,9 +814,9 @@ def run_norm_rope(args):
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": "c2_norm_rope: RMSNorm x[8192,2048] + RoPE q[4,16,2048,128] k[4,4,2048,128]"},
         "roofline": {"kernel": "rope", "bound": "hbm", "achieved": rope_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                     "frac": rope_gbs / PEAK_HBM_GBS, "traffic": 85.28e6},     # counter runs, see profiles/
+                     "frac": rope_gbs / PEAK_HBM_GBS, "traffic": profile_traffic("c2_norm_rope", "rope")},
         "rmsnorm_roofline": {"bound": "hbm", "achieved": rms_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                             "frac": rms_gbs / PEAK_HBM_GBS, "traffic": 67.22e6},
+                             "frac": rms_gbs / PEAK_HBM_GBS, "traffic": profile_traffic("c2_norm_rope", "rmsnorm")},
         "copy_reference": {"what": "torch copy of x over the same rotating buffers (1.2 GB of inputs, outputs in "
                                    "distinct blocks: nothing is served by the 256 MB memory-side cache)",
                            "achieved": copy_gbs, "unit": "GB/s", "frac": copy_gbs / PEAK_HBM_GBS},
@@ -770,14 +845,16 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=None,
-                    help="timed steps (default 20; 200 for the workloads whose step is shorter than 2 ms)")
+                    help="timed steps (default 50; 200 for the workloads whose step is shorter than 2 ms)")
     ap.add_argument("--warmup", type=int, default=None,
-                    help="untimed steps first (default 5; 50 for the short workloads: with fewer the core clock "
+                    help="untimed steps first (default 10; 50 for the short workloads: with fewer the core clock "
                          "has not settled and the first kernels run up to 20 %% slower)")
     ap.add_argument("--workload", default="c4_prefill",
                     choices=["c4_prefill", "c3_decode", "c5_finegrained_mod", "c1_cpu_reference", "c2_norm_rope",
                              "c4_prefill_train", "c1_cpu_reference_train", "loss_clip", "attention", "attention_train", "attention_decode", "gqa_layer", "gqa_decode", "block_train"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-calibration", action="store_true",
+                    help="skip the MFMA-only loops, the zero-operand launch and the vendor-BLAS matmul")
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a 1 GiB device copy (known traffic) so hardware-counter runs can be scaled")
     ap.add_argument("--cpu-sample-tokens", type=int, default=16384)
@@ -785,9 +862,9 @@ def main():
     short = args.workload in ("c3_decode", "c5_finegrained_mod", "c2_norm_rope", "loss_clip", "attention",
                               "attention_train", "attention_decode", "gqa_layer", "gqa_decode")
     if args.steps is None:
-        args.steps = 200 if short else 20
+        args.steps = 200 if short else 50
     if args.warmup is None:
-        args.warmup = 50 if short else 5
+        args.warmup = 50 if short else 10
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this path runs on one GPU (experts stay resident, no collectives); use --gpus 1",
               file=sys.stderr)

@@ -425,6 +425,17 @@ int ats_debug_decode_tile(int64_t block, const int32_t* row_count_host, int E, i
                           int SM, int SN, int32_t* out3);
 int64_t ats_debug_grid_blocks(int64_t max_rows, int E, int BM, int n_tiles, int SM, int SN);
 
+/* ---- Calibration loop for the benchmark ----
+ * No reference counterpart (the reference's benchmark, Src/Main_Scripts/core/cuda_debug_script.py,
+ * reports times only).  Launches 256 workgroups of 8 waves (one per compute unit) that issue `iters` rounds of independent
+ * bf16 MFMAs on operands held in registers: shape 0 = v_mfma_f32_32x32x16_bf16, 1 =
+ * v_mfma_f32_16x16x32_bf16; random_operands 0 = all-zero bits, 1 = normal deviates of standard
+ * deviation 0.5.  *flop_out (host) receives the flop count of the launch; clocks_dev (device, two uint64,
+ * may be null) receives the core-clock cycles and the 100 MHz ticks that workgroup 0 spent in the loop.
+ * The caller times the launch with events on `stream`. */
+int ats_calibrate_mfma(int shape, int random_operands, int iters, uint64_t* clocks_dev, double* flop_out,
+                       ats_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif
