@@ -110,8 +110,8 @@ _SIGNATURES = {
     "swiglu_launcher": (None, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p]),
     "ats_legacy_last_status": (c_int, []),
     "ats_calibrate_mfma": (c_int, [c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]),
-    "ats_debug_decode_tile": (c_int, [c_int64, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p]),
-    "ats_debug_grid_blocks": (c_int64, [c_int64, c_int, c_int, c_int, c_int, c_int]),
+    "ats_debug_decode_tile": (c_int, [c_int64, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]),
+    "ats_debug_grid_blocks": (c_int64, [c_int64, c_int, c_int, c_int, c_int, c_int, c_int]),
 }
 
 _lib = None

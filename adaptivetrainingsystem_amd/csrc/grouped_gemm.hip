@@ -45,6 +45,8 @@ struct GroupedArgs {
     const int32_t* row_start;
     const int32_t* row_count;
     int E, K, N_out, up_offset, n_tiles;
+    int sm, sn;              // supertile shape of the launch (sm * sn = 32 blocks), see tile_schedule.hpp
+    int aligned_bands;       // 1: every group's tile count is rounded up to a multiple of sm
     // split K (register-staged kernel only): k_splits > 1 turns every expert into k_splits groups that each
     // multiply a K / k_splits wide slice and write a partial result part_stride elements apart
     int k_splits, k_slice;   // k_slice = K / k_splits
@@ -244,12 +246,11 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_kernel(GroupedArgs p
     static_assert(BM % (WM * 32) == 0 && BN % (WN * 32) == 0, "wave tiling");
     static_assert(BM % RPP == 0 && BN % RPP == 0, "loader tiling");
     static_assert(!SWIGLU || TN % 2 == 0, "SwiGLU needs gate and up tiles in the same wave");
-    static_assert(SM * SN == kSuperBlocks, "supertile");
 
     extern __shared__ __align__(16) unsigned char smem[];
 
     TileCoord tc;
-    if (!decode_tile(blockIdx.x, p.row_count, p.E, BM, p.n_tiles, SM, SN, &tc)) return;
+    if (!decode_tile_wave(blockIdx.x, p.row_count, p.E, BM, p.n_tiles, p.sm, p.sn, p.aligned_bands != 0, &tc)) return;
     const int count = p.row_count[tc.e];
     const int row0 = p.row_start[tc.e];
     const int K = p.K;
@@ -409,7 +410,6 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_pipelined_kernel(Gro
     static_assert(BM % (WM * 32) == 0 && BN % (WN * 32) == 0, "wave tiling");
     static_assert(BM % RPP == 0 && BN % RPP == 0, "loader tiling");
     static_assert(!SWIGLU || TN % 2 == 0, "SwiGLU needs gate and up tiles in the same wave");
-    static_assert(SM * SN == kSuperBlocks, "supertile");
 
     extern __shared__ __align__(16) unsigned char smem[];
 
@@ -420,14 +420,10 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_pipelined_kernel(Gro
     constexpr bool sliced = SLICED;
     int split = 0;
     if constexpr (SLICED) {
-        if (!decode_tile_sliced(blockIdx.x, p.row_count, p.E, BM, p.n_tiles, SM, SN, p.k_splits, &tc, &split)) return;
-        // uniform over the block: back into scalar registers, whatever unit the walk ran on
-        tc.e = __builtin_amdgcn_readfirstlane(tc.e);
-        tc.mt = __builtin_amdgcn_readfirstlane(tc.mt);
-        tc.nt = __builtin_amdgcn_readfirstlane(tc.nt);
+        if (!decode_tile_wave(blockIdx.x, p.row_count, p.E, BM, p.n_tiles, p.sm, p.sn, p.aligned_bands != 0, &tc, p.k_splits, &split)) return;
         split = __builtin_amdgcn_readfirstlane(split);
     } else {
-        if (!decode_tile(blockIdx.x, p.row_count, p.E, BM, p.n_tiles, SM, SN, &tc)) return;
+        if (!decode_tile_wave(blockIdx.x, p.row_count, p.E, BM, p.n_tiles, p.sm, p.sn, p.aligned_bands != 0, &tc)) return;
     }
     const int count = p.row_count[tc.e];
     const int row0 = p.row_start[tc.e];
@@ -703,14 +699,13 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_dma_kernel(GroupedAr
     static_assert(BM % (WM * 32) == 0 && BN % (WN * 32) == 0, "wave tiling");
     static_assert(BM % (8 * NW) == 0 && BN % (8 * NW) == 0 && NW % 2 == 0, "loader tiling");
     static_assert(!SWIGLU || TN % 2 == 0, "SwiGLU needs gate and up tiles in the same wave");
-    static_assert(SM * SN == kSuperBlocks, "supertile");
     static_assert((TM - 1) * 4096 + 128 <= 65536 && B_STAGE + (BN / 2 + 32 * TN) * 128 <= 65536, "offset field");
 
     extern __shared__ __align__(16) unsigned char smem[];
     typedef __attribute__((address_space(3))) void* lds_ptr_t;
 
     TileCoord tc;
-    if (!decode_tile(blockIdx.x, p.row_count, p.E, BM, p.n_tiles, SM, SN, &tc)) return;
+    if (!decode_tile_wave(blockIdx.x, p.row_count, p.E, BM, p.n_tiles, p.sm, p.sn, p.aligned_bands != 0, &tc)) return;
     const int count = p.row_count[tc.e];
     const int row0 = p.row_start[tc.e];
     const int K = p.k_count ? p.k_count[tc.e] : p.K;
@@ -917,13 +912,12 @@ __global__ __launch_bounds__(512) void grouped_gemm_dma16_kernel(GroupedArgs p) 
     constexpr int A_STAGE = BM * 128;
     constexpr int B_STAGE = BN * 128;
     constexpr int B_BASE = 3 * A_STAGE;
-    static_assert(SM * SN == kSuperBlocks, "supertile");
 
     extern __shared__ __align__(16) unsigned char smem[];
     typedef __attribute__((address_space(3))) void* lds_ptr_t;
 
     TileCoord tc;
-    if (!decode_tile(blockIdx.x, p.row_count, p.E, BM, p.n_tiles, SM, SN, &tc)) return;
+    if (!decode_tile_wave(blockIdx.x, p.row_count, p.E, BM, p.n_tiles, p.sm, p.sn, p.aligned_bands != 0, &tc)) return;
     const int count = p.row_count[tc.e];
     const int row0 = p.row_start[tc.e];
     const int K = p.k_count ? p.k_count[tc.e] : p.K;
@@ -1197,7 +1191,13 @@ static int launch_cfg(const GroupedArgs& p0, int64_t max_rows, hipStream_t s) {
         set_error("grouped GEMM: %d slices of K=%d are not available for this tile configuration", splits, p.K);
         return ATS_ERR_UNSUPPORTED;
     }
-    const int64_t blocks = grid_blocks(max_rows * splits, p.E * splits, BM, p.n_tiles, SM, SN);
+    // the prefill / mid-size tiles take the supertile shape that leaves the fewest n-slots unused; the
+    // weight-streaming tiles keep theirs (one m-tile per group, 32 n-tiles side by side)
+    p.sm = SM;
+    p.sn = SN;
+    if (SM == 4 && SN == 8) pick_supertile(p.n_tiles, &p.sm, &p.sn);
+    p.aligned_bands = max_rows / (p.E > 0 ? p.E : 1) >= kAlignedBandsMinAvgRows ? 1 : 0;
+    const int64_t blocks = grid_blocks(max_rows * splits, p.E * splits, BM, p.n_tiles, p.sm, p.sn, p.aligned_bands != 0);
     if (blocks > 0x7fffffffLL) {
         set_error("grouped GEMM: grid of %lld blocks", (long long)blocks);
         return ATS_ERR_UNSUPPORTED;
@@ -1234,11 +1234,11 @@ static int launch_grouped(const GroupedArgs& p, int64_t max_rows, hipStream_t s)
         if constexpr (SWIGLU) return launch_cfg<T, TO, 32, 256, 1, 4, 1, 32, SWIGLU>(p, max_rows, s);
         else return launch_cfg<T, TO, 32, 128, 1, 4, 1, 32, SWIGLU>(p, max_rows, s);
     }
-    // (without the SwiGLU epilogue the 256 x 256 tile already wins from about 256 rows per group:
-    // +12 % on the down projection of 64 experts x ~384 rows)
-    if (avg <= (SWIGLU ? 768 : 256)) {
-        // Mid-size groups are short on reuse (a weight panel serves 3-6 row tiles), so loads often
-        // miss L2: favour more resident blocks / waves over tile size.
+    // Up to kMidMaxAvgRows rows per group: 128-row tiles with more resident blocks.  Above that the 256 x 256
+    // direct-to-LDS tile wins even when a group is one and a half tiles high (64 experts x 384 rows: gate/up
+    // 745 vs 657, down 782 vs 747 TFLOP/s), because a wave skips the 64-row halves past its group's end.
+    constexpr int64_t kMidMaxAvgRows = 192;
+    if (avg <= kMidMaxAvgRows) {
         if constexpr (SWIGLU) return launch_cfg<T, TO, 128, 128, 2, 2, 4, 8, SWIGLU>(p, max_rows, s);
         else return launch_cfg<T, TO, 128, 256, 2, 4, 4, 8, SWIGLU>(p, max_rows, s);
     }
@@ -1277,7 +1277,9 @@ static int launch_gateup_save(const GroupedArgs& p0, int64_t max_rows, hipStream
         set_error("grouped GEMM: cannot reserve %zu bytes of LDS: %s", smem, hipGetErrorString(e));
         return ATS_ERR_LAUNCH;
     }
-    const int64_t blocks = grid_blocks(max_rows, p.E, BM, p.n_tiles, 4, 8);
+    pick_supertile(p.n_tiles, &p.sm, &p.sn);
+    p.aligned_bands = max_rows / (p.E > 0 ? p.E : 1) >= kAlignedBandsMinAvgRows ? 1 : 0;
+    const int64_t blocks = grid_blocks(max_rows, p.E, BM, p.n_tiles, p.sm, p.sn, p.aligned_bands != 0);
     if (blocks > 0x7fffffffLL) {
         set_error("grouped GEMM: grid of %lld blocks", (long long)blocks);
         return ATS_ERR_UNSUPPORTED;
@@ -1311,7 +1313,9 @@ static int launch_down_dgrad_dsilu(const GroupedArgs& p0, int64_t max_rows, hipS
         set_error("grouped GEMM: cannot reserve %zu bytes of LDS: %s", smem, hipGetErrorString(e));
         return ATS_ERR_LAUNCH;
     }
-    const int64_t blocks = grid_blocks(max_rows, p.E, BM, p.n_tiles, 4, 8);
+    pick_supertile(p.n_tiles, &p.sm, &p.sn);
+    p.aligned_bands = max_rows / (p.E > 0 ? p.E : 1) >= kAlignedBandsMinAvgRows ? 1 : 0;
+    const int64_t blocks = grid_blocks(max_rows, p.E, BM, p.n_tiles, p.sm, p.sn, p.aligned_bands != 0);
     if (blocks > 0x7fffffffLL) {
         set_error("grouped GEMM: grid of %lld blocks", (long long)blocks);
         return ATS_ERR_UNSUPPORTED;
@@ -1610,14 +1614,16 @@ extern "C" int ats_grouped_gemm_nt(const void* a, const void* const* a_ptrs, int
 
 // Host-side view of the tile schedule (for tests of the block -> tile map).
 extern "C" int ats_debug_decode_tile(int64_t block, const int32_t* row_count_host, int E, int BM, int n_tiles,
-                                     int SM, int SN, int32_t* out3) {
+                                     int SM, int SN, int aligned, int k_slices, int32_t* out4) {
     ats::TileCoord tc;
-    if (!ats::decode_tile(block, row_count_host, E, BM, n_tiles, SM, SN, &tc)) return 0;
-    out3[0] = tc.e;
-    out3[1] = tc.mt;
-    out3[2] = tc.nt;
+    int slice = 0;
+    if (!ats::decode_tile(block, row_count_host, E, BM, n_tiles, SM, SN, aligned != 0, &tc, k_slices, &slice)) return 0;
+    out4[0] = tc.e;
+    out4[1] = tc.mt;
+    out4[2] = tc.nt;
+    out4[3] = slice;
     return 1;
 }
-extern "C" int64_t ats_debug_grid_blocks(int64_t max_rows, int E, int BM, int n_tiles, int SM, int SN) {
-    return ats::grid_blocks(max_rows, E, BM, n_tiles, SM, SN);
+extern "C" int64_t ats_debug_grid_blocks(int64_t max_rows, int E, int BM, int n_tiles, int SM, int SN, int aligned) {
+    return ats::grid_blocks(max_rows, E, BM, n_tiles, SM, SN, aligned != 0);
 }

@@ -418,12 +418,14 @@ void swiglu_launcher(const float* gate, const float* up, float* output, int tota
 int ats_legacy_last_status(void);
 
 /* ---- Host-side views of the grouped-GEMM tile schedule (no device work) ----
- * No reference counterpart; used to test the block -> (expert, m-tile, n-tile)
- * map on the CPU.  row_count_host is a host array.  decode returns 1 and fills
- * out3 = {expert, m_tile, n_tile} when the block owns a tile, else 0. */
+ * No reference counterpart; used to test the block -> (expert, m-tile, n-tile, K slice)
+ * map on the CPU.  row_count_host is a host array; aligned = 1 rounds every group's tile
+ * count up to a multiple of SM; k_slices >= 1.  decode returns 1 and fills
+ * out4 = {expert, m_tile, n_tile, slice} when the block owns a tile, else 0.  grid_blocks
+ * takes max_rows and E already multiplied by the number of K slices. */
 int ats_debug_decode_tile(int64_t block, const int32_t* row_count_host, int E, int BM, int n_tiles,
-                          int SM, int SN, int32_t* out3);
-int64_t ats_debug_grid_blocks(int64_t max_rows, int E, int BM, int n_tiles, int SM, int SN);
+                          int SM, int SN, int aligned, int k_slices, int32_t* out4);
+int64_t ats_debug_grid_blocks(int64_t max_rows, int E, int BM, int n_tiles, int SM, int SN, int aligned);
 
 /* ---- Calibration loop for the benchmark ----
  * No reference counterpart (the reference's benchmark, Src/Main_Scripts/core/cuda_debug_script.py,

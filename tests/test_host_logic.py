@@ -89,37 +89,56 @@ def test_argument_errors_return_codes_not_exits():
     assert lib.ats_dispatch_plan_workspace(16384, 2, 8) == (32768 // 256) * 8 * 4
 
 
-@pytest.mark.parametrize("counts,BM,n_tiles,SM,SN", [
-    ([5120, 4000, 300, 0, 1, 256, 257, 77], 256, 112, 4, 8),
-    ([20, 16, 0, 3], 32, 112, 1, 32),
-    ([130, 90, 576, 1], 128, 11, 4, 8),
-    ([0, 0, 0], 128, 5, 4, 8),
-    ([1000] * 64, 128, 11, 4, 8),
+@pytest.mark.parametrize("aligned", [0, 1])
+@pytest.mark.parametrize("counts,BM,n_tiles,SM,SN,slices", [
+    ([5120, 4000, 300, 0, 1, 256, 257, 77], 256, 112, 4, 8, 1),
+    ([20, 16, 0, 3], 32, 112, 1, 32, 1),
+    ([130, 90, 576, 1], 128, 11, 8, 4, 1),
+    ([0, 0, 0], 128, 5, 4, 8, 1),
+    ([1000] * 64, 128, 11, 4, 8, 1),
+    ([384] * 70, 256, 11, 8, 4, 1),
+    ([20, 16, 0, 3], 32, 32, 1, 32, 3),
+    ([64, 33, 1], 64, 40, 1, 32, 2),
 ])
-def test_tile_schedule_covers_each_tile_once(counts, BM, n_tiles, SM, SN):
+def test_tile_schedule_covers_each_tile_once(counts, BM, n_tiles, SM, SN, slices, aligned):
     from adaptivetrainingsystem_amd import _lib
     lib = _lib.load()
     rc = np.asarray(counts, dtype=np.int32)
     E = len(counts)
-    blocks = lib.ats_debug_grid_blocks(int(rc.sum()), E, BM, n_tiles, SM, SN)
+    blocks = lib.ats_debug_grid_blocks(int(rc.sum()) * slices, E * slices, BM, n_tiles, SM, SN, aligned)
     assert blocks % 256 == 0
     seen = {}
-    out = np.zeros(3, dtype=np.int32)
+    out = np.zeros(4, dtype=np.int32)
     for b in range(blocks):
-        if lib.ats_debug_decode_tile(b, rc.ctypes.data, E, BM, n_tiles, SM, SN, out.ctypes.data):
+        if lib.ats_debug_decode_tile(b, rc.ctypes.data, E, BM, n_tiles, SM, SN, aligned, slices, out.ctypes.data):
             key = tuple(out.tolist())
             assert key not in seen, f"tile {key} given to blocks {seen[key]} and {b}"
             seen[key] = b
-    expect = {(e, mt, nt) for e in range(E) for mt in range(-(-counts[e] // BM)) for nt in range(n_tiles)}
+    expect = {(e, mt, nt, ks) for ks in range(slices) for e in range(E) for mt in range(-(-counts[e] // BM))
+              for nt in range(n_tiles)}
     assert set(seen) == expect
-    # blocks of one supertile land on one XCD (ids congruent mod 8) and cover SM x SN neighbours
+    # blocks of one supertile land on one XCD (ids congruent mod 8) and cover SN neighbouring n-tiles of one band:
+    # SM consecutive entries of the m-tile list (group 0's tiles, then group 1's, ...; a group is an expert or one
+    # K slice of it; with `aligned` every group's tile count is rounded up to a multiple of SM)
     if expect:
+        per = [-(-c // BM) for c in counts] * slices
+        if aligned:
+            per = [-(-t // SM) * SM for t in per]
+        first = np.concatenate([[0], np.cumsum(per)])
         by_xcd = {}
         for key, b in seen.items():
             by_xcd.setdefault((b % 8, (b // 8) // 32), []).append(key)
-        for keys in by_xcd.values():
-            assert len({k[0] for k in keys}) == 1
-            assert len({k[1] // SM for k in keys}) == 1 and len({k[2] // SN for k in keys}) == 1
+        order = []
+        for (xcd, li), keys in sorted(by_xcd.items(), key=lambda kv: kv[0][1] * 8 + kv[0][0]):
+            pos = {int(first[ks * E + e]) + mt for e, mt, _, ks in keys}
+            assert len({q // SM for q in pos}) == 1
+            assert len({k[2] // SN for k in keys}) == 1
+            if aligned:
+                assert len({(k[0], k[3]) for k in keys}) == 1      # one expert's weight panels per supertile
+            order.append((min(pos) // SM, keys[0][2] // SN))
+        # supertiles go group by group (by the group a band starts in), n-group by n-group, band by band
+        owner = lambda band: int(np.searchsorted(first, band * SM, side="right") - 1)
+        assert order == sorted(order, key=lambda t: (owner(t[0]), t[1], t[0]))
 
 
 def test_capacity_is_python_double_arithmetic():
