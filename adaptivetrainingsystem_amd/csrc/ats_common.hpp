@@ -131,6 +131,18 @@ __device__ __forceinline__ float sigmoid_f(float v) {
     return __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(v * -1.4426950408889634f));
 }
 
+// 16-byte accesses of data that is touched once: the non-temporal hint keeps a stream from displacing what
+// other kernels left in the caches (measured on a 67 MB copy: 1-3 % faster than plain accesses).
+typedef unsigned int ats_u32x4_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ uint4 stream_load(const uint4* p) {
+    const ats_u32x4_t v = __builtin_nontemporal_load(reinterpret_cast<const ats_u32x4_t*>(p));
+    return make_uint4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ void stream_store(uint4* p, const uint4& v) {
+    const ats_u32x4_t t = {v.x, v.y, v.z, v.w};
+    __builtin_nontemporal_store(t, reinterpret_cast<ats_u32x4_t*>(p));
+}
+
 // ---------------------------------------------------------------- wave helpers
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll

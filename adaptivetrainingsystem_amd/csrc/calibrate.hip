@@ -106,7 +106,38 @@ __global__ __launch_bounds__(512) void calibrate_mfma_kernel(int random_operands
     if (s == 1.2345678e-30f) ats_calibrate_sink[threadIdx.x & 63] = s;   // keeps the products alive
 }
 
+// Plain streaming copy, 16 bytes per lane and four loads in flight per lane: the yardstick for the
+// bandwidth-bound kernels (what a kernel that only moves its bytes reaches at the same size).
+__global__ __launch_bounds__(256) void calibrate_copy_kernel(const uint4* __restrict__ src, uint4* __restrict__ dst,
+                                                             size_t n) {
+    size_t i = (size_t)blockIdx.x * 1024 + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * 1024;
+    for (; i < n; i += stride) {
+        uint4 v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+            if (i + u * 256 < n) v[u] = stream_load(src + i + u * 256);
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+            if (i + u * 256 < n) stream_store(dst + i + u * 256, v[u]);
+    }
+}
+
 }  // namespace ats
+
+extern "C" int ats_calibrate_copy(const void* src, void* dst, size_t bytes, ats_stream_t stream) {
+    using namespace ats;
+    ATS_REQUIRE(src && dst && bytes % 16 == 0 && aligned16(src) && aligned16(dst), ATS_ERR_INVALID_ARG,
+                "ats_calibrate_copy: 16-byte aligned buffers and a multiple of 16 bytes");
+    if (bytes == 0) return ATS_OK;
+    const size_t n = bytes / 16;
+    size_t blocks = (n + 1023) / 1024;
+    if (blocks > 2048) blocks = 2048;
+    hipLaunchKernelGGL(calibrate_copy_kernel, dim3((unsigned)blocks), dim3(256), 0, as_stream(stream),
+                       static_cast<const uint4*>(src), static_cast<uint4*>(dst), n);
+    ATS_CHECK_LAUNCH("ats_calibrate_copy");
+    return ATS_OK;
+}
 
 extern "C" int ats_calibrate_mfma(int shape, int random_operands, int iters, uint64_t* clocks_dev, double* flop_out,
                                   ats_stream_t stream) {

@@ -8,6 +8,24 @@
 
 namespace ats {
 
+// V consecutive weights as float32, fetched with 16-byte loads where the alignment allows it.
+template <typename WT, int V>
+__device__ __forceinline__ void load_weight_vec(const WT* __restrict__ w, float (&out)[V]) {
+    constexpr int kPer = 16 / (int)sizeof(WT);            // weights per 16-byte load
+    if ((reinterpret_cast<uintptr_t>(w) & 15u) == 0 && V % kPer == 0) {
+#pragma unroll
+        for (int c = 0; c < V / kPer; ++c) {
+            float f[kPer];
+            Elem<WT>::unpack(reinterpret_cast<const uint4*>(w)[c], f);
+#pragma unroll
+            for (int j = 0; j < kPer; ++j) out[c * kPer + j] = f[j];
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < V; ++j) out[j] = Elem<WT>::load(w + j);
+    }
+}
+
 template <typename T, typename WT, int NV, bool HAS_W>
 __global__ __launch_bounds__(256) void rmsnorm_rows_kernel(const T* __restrict__ x,
                                                            const WT* __restrict__ w,
@@ -19,20 +37,10 @@ __global__ __launch_bounds__(256) void rmsnorm_rows_kernel(const T* __restrict__
     const int64_t wave = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
     const int64_t nwaves = (int64_t)gridDim.x * (blockDim.x >> 6);
 
-    float wreg[NV][V];
-    if (HAS_W) {
-#pragma unroll
-        for (int i = 0; i < NV; ++i) {
-            const int v = lane + i * kWave;
-            if (v < nvec) {
-#pragma unroll
-                for (int j = 0; j < V; ++j) wreg[i][j] = Elem<WT>::load(w + (int64_t)v * V + j);
-            }
-        }
-    }
-
     // the next row of this wave is fetched while the current one is reduced and written (twice the bytes in
-    // flight per wave: a 67 MB tensor is over before a one-row-at-a-time loop has filled the memory pipeline)
+    // flight per wave: a 67 MB tensor is over before a one-row-at-a-time loop has filled the memory pipeline).
+    // The first row's loads are issued before anything else: loads return in order, so whatever is asked for
+    // first delays them.
     constexpr bool kPrefetch = NV <= 8;
     uint4 ahead[kPrefetch ? NV : 1];
     if (kPrefetch && wave < rows) {
@@ -40,7 +48,16 @@ __global__ __launch_bounds__(256) void rmsnorm_rows_kernel(const T* __restrict__
 #pragma unroll
         for (int i = 0; i < NV; ++i) {
             const int v = lane + i * kWave;
-            if (v < nvec) ahead[i] = xr[v];
+            if (v < nvec) ahead[i] = stream_load(xr + v);
+        }
+    }
+
+    float wreg[NV][V];
+    if (HAS_W) {
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int v = lane + i * kWave;
+            if (v < nvec) load_weight_vec<WT, V>(w + (int64_t)v * V, wreg[i]);
         }
     }
     for (int64_t row = wave; row < rows; row += nwaves) {
@@ -54,14 +71,14 @@ __global__ __launch_bounds__(256) void rmsnorm_rows_kernel(const T* __restrict__
 #pragma unroll
                 for (int i = 0; i < NV; ++i) {
                     const int v = lane + i * kWave;
-                    if (v < nvec) ahead[kPrefetch ? i : 0] = xn[v];
+                    if (v < nvec) ahead[kPrefetch ? i : 0] = stream_load(xn + v);
                 }
             }
         } else {
 #pragma unroll
             for (int i = 0; i < NV; ++i) {
                 const int v = lane + i * kWave;
-                if (v < nvec) raw[i] = xr[v];
+                if (v < nvec) raw[i] = stream_load(xr + v);
             }
         }
         float ss = 0.f;
@@ -90,7 +107,7 @@ __global__ __launch_bounds__(256) void rmsnorm_rows_kernel(const T* __restrict__
                     if (HAS_W) t = t * wreg[i][j];
                     f[j] = t;
                 }
-                yr[v] = Elem<T>::pack(f);
+                stream_store(yr + v, Elem<T>::pack(f));
             }
         }
     }

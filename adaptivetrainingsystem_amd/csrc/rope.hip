@@ -48,6 +48,20 @@ __global__ __launch_bounds__(256) void rope_vec_kernel(RopeSeg q, RopeSeg k, con
     if (prow >= pos_per_wave || pos >= L) return;
 
     const int half = D >> 1;
+    // the rows first (they come from HBM; loads return in order), then the table slice (L2 after the first waves)
+    const int h0 = chunk * kRopeHeadsPerItem;
+    const T* in = static_cast<const T*>(seg.in);
+    T* out = static_cast<T*>(seg.out);
+    uint4 lo[kRopeHeadsPerItem], hi[kRopeHeadsPerItem];
+#pragma unroll
+    for (int i = 0; i < kRopeHeadsPerItem; ++i) {
+        const int h = h0 + i;
+        if (h < seg.heads) {
+            const T* p = in + b * seg.sb + h * seg.sh + pos * seg.sl + c * V;
+            lo[i] = stream_load(reinterpret_cast<const uint4*>(p));
+            hi[i] = stream_load(reinterpret_cast<const uint4*>(p + half));
+        }
+    }
     float cs[V], sn[V];
     {
         const float* cp = cos_tab + (int64_t)(pos_offset + pos) * table_stride + c * V;
@@ -70,19 +84,6 @@ __global__ __launch_bounds__(256) void rope_vec_kernel(RopeSeg q, RopeSeg k, con
 #pragma unroll
         for (int j = 0; j < V; ++j) sn[j] *= sin_sign;   // exact: +1 forward, -1 inverse rotation
     }
-    const int h0 = chunk * kRopeHeadsPerItem;
-    const T* in = static_cast<const T*>(seg.in);
-    T* out = static_cast<T*>(seg.out);
-    uint4 lo[kRopeHeadsPerItem], hi[kRopeHeadsPerItem];
-#pragma unroll
-    for (int i = 0; i < kRopeHeadsPerItem; ++i) {
-        const int h = h0 + i;
-        if (h < seg.heads) {
-            const T* p = in + b * seg.sb + h * seg.sh + pos * seg.sl + c * V;
-            lo[i] = *reinterpret_cast<const uint4*>(p);
-            hi[i] = *reinterpret_cast<const uint4*>(p + half);
-        }
-    }
 #pragma unroll
     for (int i = 0; i < kRopeHeadsPerItem; ++i) {
         const int h = h0 + i;
@@ -96,8 +97,8 @@ __global__ __launch_bounds__(256) void rope_vec_kernel(RopeSeg q, RopeSeg k, con
                 o2[j] = ((((a[j]) * (sn[j]))) + (((bb[j]) * (cs[j]))));
             }
             T* p = out + (((int64_t)b * seg.heads + h) * L + pos) * D + c * V;
-            *reinterpret_cast<uint4*>(p) = Elem<T>::pack(o1);
-            *reinterpret_cast<uint4*>(p + half) = Elem<T>::pack(o2);
+            stream_store(reinterpret_cast<uint4*>(p), Elem<T>::pack(o1));
+            stream_store(reinterpret_cast<uint4*>(p + half), Elem<T>::pack(o2));
         }
     }
 }

@@ -141,6 +141,86 @@ __global__ __launch_bounds__(KW * 64) void gate_gemm_bf16_kernel(const bf16_t* _
     }
 }
 
+// Up to 16 experts and a hidden size of at most 8 x 4 x 128: the same split of K over 8 waves, but a wave
+// asks for its whole K slice at once (up to 4 steps x 4 loads per token tile, plus the gate rows) before the
+// first MFMA, and a block owns MT 16-token tiles that share the gate rows' loads.  With nothing to wait for
+// between steps the block's bytes are all in flight after a few hundred cycles, which is what a kernel that
+// lives for 20 us needs.  The gate rows are fetched one step ahead of their use rather than all at once, which
+// keeps a wave at 108 registers and two blocks resident per CU.
+template <int MT>
+__global__ __launch_bounds__(512) void gate_gemm_bf16_flat_kernel(const bf16_t* __restrict__ x,
+                                                                  const bf16_t* __restrict__ wg,
+                                                                  const float* __restrict__ bias,
+                                                                  float* __restrict__ logits, int64_t T, int H, int E) {
+    constexpr int KW = 8, S = 4;
+    __shared__ float red[KW][MT][16 * 16];
+    const int lane = lane_id();
+    const int wave = threadIdx.x >> 6;
+    const int r = lane & 15;
+    const int g = lane >> 4;
+    const int64_t t0 = (int64_t)blockIdx.x * (16 * MT);
+    const int steps_total = (H + kGateKC - 1) / kGateKC;
+    const int steps_per_wave = (steps_total + KW - 1) / KW;      // <= S (host)
+    const int s_begin = wave * steps_per_wave;
+    const u32x4_t zero4 = {0u, 0u, 0u, 0u};
+    u32x4_t a[MT][S][4], b[2][4];
+    // token rows first: they come from HBM, the gate rows from L2
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+        const int64_t trow = t0 + m * 16 + r;
+        const bf16_t* xrow = x + (trow < T ? trow : 0) * (int64_t)H;
+#pragma unroll
+        for (int st = 0; st < S; ++st)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int kk = (s_begin + st) * kGateKC + g * 8 + i * 32;
+                a[m][st][i] = zero4;
+                if (st < steps_per_wave && trow < T && kk < H) a[m][st][i] = *reinterpret_cast<const u32x4_t*>(xrow + kk);
+            }
+    }
+    // the gate rows one step ahead of their use (two register sets: all of them at once would cost a resident block)
+#define GF_LOAD_B(st_, buf_)                                                                           \
+    _Pragma("unroll") for (int i = 0; i < 4; ++i) {                                                    \
+        const int kk = (s_begin + (st_)) * kGateKC + g * 8 + i * 32;                                   \
+        b[buf_][i] = zero4;                                                                            \
+        if ((st_) < steps_per_wave && r < E && kk < H)                                                 \
+            b[buf_][i] = *reinterpret_cast<const u32x4_t*>(wg + (int64_t)r * H + kk);                  \
+    }
+    GF_LOAD_B(0, 0);
+    f32x4_t acc[MT];
+#pragma unroll
+    for (int m = 0; m < MT; ++m) acc[m] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    // same order of accumulation as gate_gemm_bf16_kernel: steps ascending, the four 32-element pieces ascending
+#pragma unroll
+    for (int st = 0; st < S; ++st) {
+        if (st + 1 < S) GF_LOAD_B(st + 1, (st + 1) & 1);
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int m = 0; m < MT; ++m)
+                acc[m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a[m][st][i]), as_bf16x8(b[st & 1][i]), acc[m], 0, 0, 0);
+    }
+#undef GF_LOAD_B
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) red[wave][m][(4 * g + v) * 16 + r] = acc[m][v];
+    __syncthreads();
+    for (int i = threadIdx.x; i < MT * 256; i += KW * 64) {
+        const int m = i >> 8;
+        const int row = (i & 255) >> 4;
+        const int col = i & 15;
+        const int64_t t = t0 + m * 16 + row;
+        if (t < T && col < E) {
+            float v = red[0][m][i & 255];
+#pragma unroll
+            for (int w = 1; w < KW; ++w) v += red[w][m][i & 255];
+            if (bias) v += bias[col];
+            logits[t * E + col] = v;
+        }
+    }
+}
+
 // One wave per token, 8 experts at a time.  Works for every dtype / shape.
 template <typename T>
 __global__ __launch_bounds__(256) void gate_gemm_generic_kernel(const T* __restrict__ x, const T* __restrict__ wg,
@@ -468,7 +548,12 @@ extern "C" int ats_router_logits(const void* x, const void* wg, const float* bia
         const int nt = (E + 15) / 16;
         // Few experts: 8 waves split K (short dependent chains, 32 waves per CU resident);
         // more expert tiles need more registers per wave and use 4 waves with (NT <= 2) prefetch.
-        if (nt <= 1)
+        // prefill-sized batches of a hidden size that 8 waves cover in 4 steps each: the flat kernel (one 16-token
+        // tile per block: two blocks stay resident per CU; with two tiles per block the kernel ran 36 instead of 27 us
+        // on [16384, 4096] x 8 experts, the looped kernel 37 us)
+        if (nt <= 1 && H <= 8 * 4 * kGateKC && T >= 2048)
+            hipLaunchKernelGGL((gate_gemm_bf16_flat_kernel<1>), dim3(blocks), dim3(512), 0, s, xp, wp, bias, logits, T, H, E);
+        else if (nt <= 1)
             hipLaunchKernelGGL((gate_gemm_bf16_kernel<1, 8, false>), dim3(blocks), dim3(512), 0, s, xp, wp, bias, logits, T, H, E);
         else if (nt <= 2)
             hipLaunchKernelGGL((gate_gemm_bf16_kernel<2, 4, true>), dim3(blocks), dim3(256), 0, s, xp, wp, bias, logits, T, H, E);

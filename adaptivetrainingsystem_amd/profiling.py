@@ -85,3 +85,15 @@ def calibrate_mfma(shape: str = "16x16x32", random_operands: bool = True, iters:
     ms = ev0.elapsed_time(ev1)
     c = clocks.cpu().tolist()
     return {"tflops": flop.value / (ms * 1e-3) / 1e12, "core_clock_mhz": 100.0 * c[0] / max(c[1], 1), "ms": ms}
+
+
+def stream_copy(src: torch.Tensor, dst: torch.Tensor) -> None:
+    """The library's plain streaming copy (16 bytes per lane, four loads in flight): the yardstick for the
+    bandwidth-bound kernels."""
+    from . import _lib
+    from .ops import _stream
+    if not (src.is_cuda and dst.is_cuda and src.is_contiguous() and dst.is_contiguous()) or \
+            src.numel() * src.element_size() != dst.numel() * dst.element_size():
+        raise _lib.AtsError("stream_copy: contiguous GPU tensors of the same size")
+    _lib.check(_lib.load().ats_calibrate_copy(src.data_ptr(), dst.data_ptr(), src.numel() * src.element_size(),
+                                              _stream()), "ats_calibrate_copy")

@@ -437,6 +437,9 @@ int64_t ats_debug_grid_blocks(int64_t max_rows, int E, int BM, int n_tiles, int 
  * The caller times the launch with events on `stream`. */
 int ats_calibrate_mfma(int shape, int random_operands, int iters, uint64_t* clocks_dev, double* flop_out,
                        ats_stream_t stream);
+/* Plain streaming copy of `bytes` (a multiple of 16; both pointers 16-byte aligned): the yardstick that the
+ * benchmark prints beside the bandwidth-bound kernels.  No reference counterpart. */
+int ats_calibrate_copy(const void* src, void* dst, size_t bytes, ats_stream_t stream);
 
 #ifdef __cplusplus
 }
