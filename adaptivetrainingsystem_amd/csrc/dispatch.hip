@@ -117,7 +117,7 @@ __device__ void scan_totals(int32_t* chunk_hist, int nchunks, int E, int C, int3
     __syncthreads();
 }
 
-__global__ __launch_bounds__(256) void plan_scan_kernel(int32_t* __restrict__ chunk_hist, int nchunks, int E, int C,
+__global__ __launch_bounds__(1024) void plan_scan_kernel(int32_t* __restrict__ chunk_hist, int nchunks, int E, int C,
                                                         int32_t* __restrict__ hist, int32_t* __restrict__ kept,
                                                         int32_t* __restrict__ offsets) {
     extern __shared__ int s_tot[];
@@ -654,7 +654,8 @@ extern "C" int ats_dispatch_plan(const void* idx, int idx_dtype, int64_t T, int 
         hipLaunchKernelGGL((plan_hist_kernel<int64_t>), dim3((unsigned)nchunks), dim3(256), smem, s,
                            static_cast<const int64_t*>(idx), n, E, chunk_hist, status);
     ATS_CHECK_LAUNCH("ats_dispatch_plan(hist)");
-    hipLaunchKernelGGL(plan_scan_kernel, dim3(1), dim3(256), (size_t)E * sizeof(int), s, chunk_hist, (int)nchunks, E,
+    // 16 waves: every wave scans four experts' chunk columns, so 64 experts take one round instead of four
+    hipLaunchKernelGGL(plan_scan_kernel, dim3(1), dim3(1024), (size_t)E * sizeof(int), s, chunk_hist, (int)nchunks, E,
                        C, hist, kept, offsets);
     ATS_CHECK_LAUNCH("ats_dispatch_plan(scan)");
     if (idx_dtype == ATS_IDX_I32)

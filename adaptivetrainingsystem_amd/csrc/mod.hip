@@ -107,6 +107,126 @@ __global__ __launch_bounds__(1024) void select_topk_seq_kernel(const float* __re
     }
 }
 
+// The same selection by radix select, for sequences of up to 1024 * PER positions: thread t keeps positions
+// [t * PER, (t + 1) * PER) in registers as order-preserving keys (NaN above everything, as torch.topk ranks it).
+// Four 8-bit passes from the top byte find the key of the keep-th largest score and how many positions with
+// exactly that key are still wanted; those are the ones with the lowest positions (rank among equals by a
+// block-wide prefix sum in position order).  A second prefix sum compacts the selected positions in ascending
+// order.  No sort: 4 histogram passes + 2 scans instead of 66 compare-exchange passes over LDS.
+__device__ __forceinline__ uint32_t topk_key(float f) {
+    if (f != f) return 0xffffffffu;
+    if (f == 0.f) return 0x80000000u;       // -0 and +0 are equal scores
+    const uint32_t u = __float_as_uint(f);
+    return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+
+// Exclusive prefix sum of one int per thread over a 1024-thread block, in thread order.  s_wave: 16 ints of LDS.
+__device__ __forceinline__ int block_exclusive_scan_1024(int v, int* s_wave, int* total) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int incl = v;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const int o = __shfl_up(incl, off, 64);
+        if (lane >= off) incl += o;
+    }
+    __syncthreads();                       // s_wave may still be read from a previous call
+    if (lane == 63) s_wave[wave] = incl;
+    __syncthreads();
+    int base = 0, tot = 0;
+#pragma unroll
+    for (int w = 0; w < 16; ++w) {
+        const int c = s_wave[w];
+        if (w < wave) base += c;
+        tot += c;
+    }
+    *total = tot;
+    return base + incl - v;
+}
+
+template <int PER>
+__global__ __launch_bounds__(1024) void select_topk_radix_kernel(const float* __restrict__ score, int L, int keep,
+                                                                 int32_t* __restrict__ sel) {
+    __shared__ unsigned int s_hist[256];
+    __shared__ int s_wave[16];
+    __shared__ unsigned int s_pick[2];      // chosen bin, count still wanted inside it
+    const int b = blockIdx.x;
+    const int t = threadIdx.x;
+    uint32_t key[PER];
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+        const int i = t * PER + j;
+        key[j] = i < L ? topk_key(score[(int64_t)b * L + i]) : 0u;     // positions past L never match (see valid)
+    }
+    uint32_t prefix = 0, mask = 0;
+    unsigned int want = (unsigned int)keep;
+    for (int pass = 3; pass >= 0; --pass) {
+        if (t < 256) s_hist[t] = 0;
+        __syncthreads();
+        const int shift = pass * 8;
+#pragma unroll
+        for (int j = 0; j < PER; ++j) {
+            const int i = t * PER + j;
+            if (i < L && (key[j] & mask) == prefix) atomicAdd(&s_hist[(key[j] >> shift) & 255u], 1u);
+        }
+        __syncthreads();
+        if (t < 64) {
+            // lane l owns bins 255 - 4l ... 252 - 4l (descending); suffix sums from the top bin down
+            unsigned int c[4], sum = 0;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                c[q] = s_hist[255 - 4 * t - q];
+                sum += c[q];
+            }
+            unsigned int incl = sum;
+#pragma unroll
+            for (int off = 1; off < 64; off <<= 1) {
+                const unsigned int o = __shfl_up(incl, off, 64);
+                if (t >= off) incl += o;
+            }
+            const unsigned int before = incl - sum;          // keys in higher bins than this lane's
+            if (before < want && incl >= want) {
+                unsigned int acc = before;
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    if (acc < want && acc + c[q] >= want) {
+                        s_pick[0] = 255u - 4u * t - q;
+                        s_pick[1] = want - acc;
+                    }
+                    acc += c[q];
+                }
+            }
+        }
+        __syncthreads();
+        prefix |= s_pick[0] << shift;
+        mask |= 255u << shift;
+        want = s_pick[1];
+        __syncthreads();
+    }
+    // prefix = key of the keep-th largest; `want` positions with exactly that key are taken, lowest positions first
+    int eq = 0;
+#pragma unroll
+    for (int j = 0; j < PER; ++j) eq += (t * PER + j < L && key[j] == prefix) ? 1 : 0;
+    int tot;
+    int eq_rank = block_exclusive_scan_1024(eq, s_wave, &tot);
+    bool take[PER];
+    int ntake = 0;
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+        const bool valid = t * PER + j < L;
+        take[j] = valid && key[j] > prefix;
+        if (valid && key[j] == prefix) {
+            take[j] = eq_rank < (int)want;
+            ++eq_rank;
+        }
+        ntake += take[j] ? 1 : 0;
+    }
+    int out = block_exclusive_scan_1024(ntake, s_wave, &tot);
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+        if (take[j]) sel[(int64_t)b * keep + out++] = b * L + t * PER + j;
+    }
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void scatter_add_rows_kernel(T* __restrict__ base, const int32_t* __restrict__ rows,
                                                                const T* __restrict__ delta, int64_t n, int H,
@@ -254,6 +374,14 @@ extern "C" int ats_select_topk_per_sequence(const float* score, int B, int L, in
     ATS_REQUIRE((int64_t)B * L < INT_MAX, ATS_ERR_UNSUPPORTED, "ats_select_topk_per_sequence: B*L must fit in int32");
     if (B == 0 || keep == 0) return ATS_OK;
     ATS_REQUIRE(score && sel, ATS_ERR_INVALID_ARG, "ats_select_topk_per_sequence: null pointer");
+    hipStream_t st = as_stream(stream);
+    if (L > 512) {      // long sequences: radix select (short ones are cheap to sort and keep the sort)
+        if (L <= 2048) hipLaunchKernelGGL(select_topk_radix_kernel<2>, dim3(B), dim3(1024), 0, st, score, L, keep, sel);
+        else if (L <= 4096) hipLaunchKernelGGL(select_topk_radix_kernel<4>, dim3(B), dim3(1024), 0, st, score, L, keep, sel);
+        else hipLaunchKernelGGL(select_topk_radix_kernel<8>, dim3(B), dim3(1024), 0, st, score, L, keep, sel);
+        ATS_CHECK_LAUNCH("ats_select_topk_per_sequence");
+        return ATS_OK;
+    }
     int lp2 = 2;
     while (lp2 < L) lp2 <<= 1;
     const int threads = lp2 / 2 < 64 ? 64 : (lp2 / 2 > 1024 ? 1024 : lp2 / 2);

@@ -454,20 +454,20 @@ __global__ __launch_bounds__(256) void route_topk_kernel(const float* __restrict
 // Reduces the per-block partials in a fixed order and evaluates the auxiliary loss.
 // Thread (e, c) sums blocks c, c+TPE, ... of expert e (consecutive threads read consecutive
 // experts: coalesced); the TPE partial sums of an expert are then added in ascending c.
-__global__ __launch_bounds__(256) void route_finalize_kernel(const int32_t* __restrict__ part_hist,
+__global__ __launch_bounds__(1024) void route_finalize_kernel(const int32_t* __restrict__ part_hist,
                                                              const float* __restrict__ part_colsum, int nblocks,
                                                              int E, int64_t T, int k, float lbw,
                                                              int32_t* __restrict__ hist, float* __restrict__ colsum,
                                                              float* __restrict__ aux) {
     extern __shared__ unsigned char smem_raw[];
     float* s_term = reinterpret_cast<float*>(smem_raw);          // [E]
-    int* s_h = reinterpret_cast<int*>(s_term + E);               // [256]
-    float* s_c = reinterpret_cast<float*>(s_h + 256);            // [256]
+    int* s_h = reinterpret_cast<int*>(s_term + E);               // [1024]
+    float* s_c = reinterpret_cast<float*>(s_h + 1024);           // [1024]
     int tpe = 1;
-    while (tpe * 2 * E <= 256) tpe *= 2;   // threads per expert (power of two), 1 when E > 128
-    for (int e0 = 0; e0 < E; e0 += 256 / tpe) {
-        const int e = e0 + (int)threadIdx.x % (256 / tpe);
-        const int c = (int)threadIdx.x / (256 / tpe);
+    while (tpe * 2 * E <= 1024) tpe *= 2;  // threads per expert (power of two), 1 when E > 512
+    for (int e0 = 0; e0 < E; e0 += 1024 / tpe) {
+        const int e = e0 + (int)threadIdx.x % (1024 / tpe);
+        const int c = (int)threadIdx.x / (1024 / tpe);
         int hsum = 0;
         float csum = 0.f;
         if (e < E) {
@@ -492,8 +492,8 @@ __global__ __launch_bounds__(256) void route_finalize_kernel(const int32_t* __re
         __syncthreads();
         if (c == 0 && e < E) {
             for (int cc = 1; cc < tpe; ++cc) {
-                hsum += s_h[cc * (256 / tpe) + (int)threadIdx.x];
-                csum += s_c[cc * (256 / tpe) + (int)threadIdx.x];
+                hsum += s_h[cc * (1024 / tpe) + (int)threadIdx.x];
+                csum += s_c[cc * (1024 / tpe) + (int)threadIdx.x];
             }
             hist[e] = hsum;
             colsum[e] = csum;
@@ -628,7 +628,7 @@ extern "C" int ats_route_topk(const float* logits, int64_t T, int E, int k, floa
                            prob_colsum, aux);
     ATS_CHECK_LAUNCH("ats_route_topk");
     if (stats && nblocks > 1) {
-        hipLaunchKernelGGL(route_finalize_kernel, dim3(1), dim3(256), (size_t)(E + 512) * sizeof(float), s, part_hist,
+        hipLaunchKernelGGL(route_finalize_kernel, dim3(1), dim3(1024), (size_t)(E + 2048) * sizeof(float), s, part_hist,
                            part_col, nblocks, E, T, k, load_balancing_weight, hist, prob_colsum, aux);
         ATS_CHECK_LAUNCH("ats_route_topk(finalize)");
     }

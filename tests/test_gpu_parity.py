@@ -553,6 +553,24 @@ def test_mod_router_eval_and_selection(A, ops, gpu):
     assert torch.equal(sel.long(), ref)
 
 
+@pytest.mark.parametrize("L,keep", [(513, 1), (700, 700), (2048, 256), (2049, 300), (3000, 1), (4096, 4000),
+                                    (8192, 1024)])
+def test_select_topk_long_sequences_with_ties(ops, gpu, L, keep):
+    """Sequences above 512 positions take the radix-select kernel: heavy ties (scores from a handful of values),
+    signed zeros (equal scores) and infinities against the stable-sort oracle."""
+    g = gen(300 + L)
+    B = 3
+    s = torch.randn(B, L, generator=g)
+    s[1] = torch.randint(-2, 3, (L,), generator=g).float() * 0.5           # five distinct values, zeros included
+    s[1, ::7] = -0.0
+    s[2, : L // 3] = float("inf")
+    s[2, L // 3: L // 2] = float("-inf")
+    s[0, 5] = s[0, 400]
+    sel = ops.select_topk_per_sequence(s.to(gpu), keep).cpu().view(B, keep)
+    ref = O.mod_select_per_sequence(s, keep) + torch.arange(B).unsqueeze(1) * L
+    assert torch.equal(sel.long(), ref)
+
+
 def test_fused_swiglu_seam(gpu):
     import os
     import sys
