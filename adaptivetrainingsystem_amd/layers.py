@@ -36,7 +36,7 @@ import torch.nn as nn
 
 from . import autograd as ag
 from . import ops
-from .profiling import stage
+from .profiling import stage, timer_context
 from ._lib import ROUTE_SOFTMAX_TOPK, ROUTE_TOPK_SOFTMAX, AtsError
 
 
@@ -565,26 +565,30 @@ class MoECUDAOps:
     @staticmethod
     def topk_gating(gate_logits: torch.Tensor, k: int, temperature: float = 1.0, use_cuda: bool = True):
         """-> (indices int64 [T,k], weights float32 [T,k]); top-k of logits/temperature, softmax over the k."""
-        r = ops.route_topk(gate_logits.float(), k, temperature, ROUTE_TOPK_SOFTMAX, with_stats=False)
+        with timer_context(True, gate_logits.shape[0]):
+            r = ops.route_topk(gate_logits.float(), k, temperature, ROUTE_TOPK_SOFTMAX, with_stats=False)
         return r["indices"].long(), r["weights"]
 
     @staticmethod
     def dispatch_tokens(tokens: torch.Tensor, top_k_indices: torch.Tensor, num_experts: int, capacity: int,
                         use_cuda: bool = True):
         """-> (expert_inputs [E,C,H] zero padded, token_map [E,C] int32, -1 = empty)."""
-        plan = ops.dispatch_plan(top_k_indices, num_experts, capacity)
-        k = top_k_indices.shape[1]
-        H = tokens.shape[1]
-        expert_inputs = ops.gather_rows(tokens, plan["token_map"].view(-1), div=k)
+        with timer_context(True, tokens.shape[0]):
+            plan = ops.dispatch_plan(top_k_indices, num_experts, capacity)
+            k = top_k_indices.shape[1]
+            H = tokens.shape[1]
+            expert_inputs = ops.gather_rows(tokens, plan["token_map"].view(-1), div=k)
         return expert_inputs.view(num_experts, capacity, H), plan["token_map"]
 
     @staticmethod
     def combine_expert_outputs(expert_outputs: torch.Tensor, token_map: torch.Tensor, top_k_weights: torch.Tensor,
                                num_tokens: int, k: int, use_cuda: bool = True) -> torch.Tensor:
         """-> [num_tokens, H]; ascending expert order, dropped choices contribute nothing."""
-        row_of = ops.invert_token_map(token_map.to(torch.int32), num_tokens * k)
-        return ops.combine(expert_outputs, row_of, top_k_weights.float(), num_tokens, k,
-                           out_dtype=expert_outputs.dtype)
+        with timer_context(True, num_tokens):
+            row_of = ops.invert_token_map(token_map.to(torch.int32), num_tokens * k)
+            out = ops.combine(expert_outputs, row_of, top_k_weights.float(), num_tokens, k,
+                              out_dtype=expert_outputs.dtype)
+        return out
 
 
 # ============================================================================ Mixture of Depths

@@ -53,6 +53,125 @@ class StageTimer:
         return out
 
 
+class MoEPerformanceMonitor:
+    """The reference's monitor of its MoE operators (Src/Main_Scripts/core/moe_cuda_wrapper.py:76-136), with the
+    same fields, methods and `get_stats` keys.  The reference brackets every operator call with two device
+    synchronisations; here `timer_context` records a pair of HIP events on the launch stream and the elapsed
+    times are read only when the statistics are asked for.  There is no PyTorch fallback in this build, so
+    the `pytorch_*` side only ever moves if a caller records into it."""
+
+    def __init__(self):
+        self.reset()
+
+    def reset(self) -> None:
+        self.cuda_time = 0.0
+        self.pytorch_time = 0.0
+        self.cuda_calls = 0
+        self.pytorch_calls = 0
+        self.cuda_tokens = 0
+        self.pytorch_tokens = 0
+        self._pending: List[Tuple[torch.cuda.Event, torch.cuda.Event, bool]] = []
+
+    def record_cuda(self, time_ms: float, num_tokens: int) -> None:
+        self.cuda_time += time_ms
+        self.cuda_calls += 1
+        self.cuda_tokens += num_tokens
+
+    def record_pytorch(self, time_ms: float, num_tokens: int) -> None:
+        self.pytorch_time += time_ms
+        self.pytorch_calls += 1
+        self.pytorch_tokens += num_tokens
+
+    def _record_events(self, start, stop, use_cuda: bool, num_tokens: int) -> None:
+        self._pending.append((start, stop, use_cuda))
+        if use_cuda:
+            self.cuda_calls += 1
+            self.cuda_tokens += num_tokens
+        else:
+            self.pytorch_calls += 1
+            self.pytorch_tokens += num_tokens
+
+    def _drain(self) -> None:
+        if not self._pending:
+            return
+        torch.cuda.synchronize()
+        for start, stop, use_cuda in self._pending:
+            ms = start.elapsed_time(stop)
+            if use_cuda:
+                self.cuda_time += ms
+            else:
+                self.pytorch_time += ms
+        self._pending = []
+
+    def get_stats(self) -> Dict[str, float]:
+        self._drain()
+        total_time = self.cuda_time + self.pytorch_time
+        if total_time == 0:
+            return {"status": "No data yet"}
+        return {
+            "cuda_calls": self.cuda_calls,
+            "pytorch_calls": self.pytorch_calls,
+            "cuda_time_ms": self.cuda_time,
+            "pytorch_time_ms": self.pytorch_time,
+            "cuda_percentage": self.cuda_time / total_time * 100,
+            "estimated_speedup": (self.pytorch_time / self.cuda_time) if self.cuda_time > 0 else 1.0,
+            "tokens_per_sec_cuda": (self.cuda_tokens / (self.cuda_time / 1000)) if self.cuda_time > 0 else 0,
+            "tokens_per_sec_pytorch": (self.pytorch_tokens / (self.pytorch_time / 1000)) if self.pytorch_time > 0 else 0,
+        }
+
+    def print_summary(self) -> None:
+        stats = self.get_stats()
+        if "status" in stats:
+            print(f"\n{stats['status']}")
+            return
+        print(f"\n{'=' * 70}\nMoE operator summary (gfx950 kernels)\n{'=' * 70}")
+        print(f"Kernel calls:   {stats['cuda_calls']:,}")
+        print(f"Kernel time:    {stats['cuda_time_ms']:.2f} ms")
+        print(f"Throughput:     {stats['tokens_per_sec_cuda']:,.0f} tokens/sec")
+        if stats["pytorch_calls"]:
+            print(f"Other calls:    {stats['pytorch_calls']:,} ({stats['pytorch_time_ms']:.2f} ms)")
+        print("=" * 70)
+
+
+_GLOBAL_MONITOR = MoEPerformanceMonitor()
+_MONITOR_ENABLED = False
+
+
+def enable_performance_monitor(on: bool = True) -> None:
+    """The `MoECUDAOps` operators record into the global monitor only while this is on (an event pair per call
+    costs the stream about 10 us; the reference pays two synchronisations per call unconditionally)."""
+    global _MONITOR_ENABLED
+    _MONITOR_ENABLED = bool(on)
+
+
+@contextmanager
+def timer_context(use_cuda: bool, num_tokens: int):
+    """moe_cuda_wrapper.py:142-159 without the synchronisations: the bracket is a pair of HIP events."""
+    if not _MONITOR_ENABLED:
+        yield
+        return
+    start = torch.cuda.Event(enable_timing=True)
+    stop = torch.cuda.Event(enable_timing=True)
+    start.record()
+    try:
+        yield
+    finally:
+        stop.record()
+        _GLOBAL_MONITOR._record_events(start, stop, use_cuda, num_tokens)
+
+
+def get_performance_summary():
+    return _GLOBAL_MONITOR.get_stats()
+
+
+def print_performance_summary() -> None:
+    _GLOBAL_MONITOR.print_summary()
+
+
+def reset_performance_monitor() -> None:
+    _GLOBAL_MONITOR.reset()
+
+
 @contextmanager
 def _null_range():
     yield

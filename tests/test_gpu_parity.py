@@ -571,6 +571,33 @@ def test_select_topk_long_sequences_with_ties(ops, gpu, L, keep):
     assert torch.equal(sel.long(), ref)
 
 
+def test_performance_monitor_api(A, gpu):
+    """The monitor of the reference's operator module (moe_cuda_wrapper.py:76-159, 599-611): same keys, fed by HIP
+    events instead of synchronisations, only while it is switched on."""
+    from adaptivetrainingsystem_amd import profiling as P
+    P.reset_performance_monitor()
+    assert P.get_performance_summary() == {"status": "No data yet"}
+    logits = torch.randn(300, 8, generator=gen(41)).to(gpu)
+    A.MoECUDAOps.topk_gating(logits, 2)
+    assert P.get_performance_summary() == {"status": "No data yet"}          # off by default
+    P.enable_performance_monitor(True)
+    try:
+        idx, w = A.MoECUDAOps.topk_gating(logits, 2)
+        A.MoECUDAOps.dispatch_tokens(torch.randn(300, 64, generator=gen(42)).to(gpu), idx, 8, 100)
+    finally:
+        P.enable_performance_monitor(False)
+    st = P.get_performance_summary()
+    assert set(st) == {"cuda_calls", "pytorch_calls", "cuda_time_ms", "pytorch_time_ms", "cuda_percentage",
+                       "estimated_speedup", "tokens_per_sec_cuda", "tokens_per_sec_pytorch"}
+    assert st["cuda_calls"] == 2 and st["pytorch_calls"] == 0 and st["cuda_time_ms"] > 0
+    assert st["cuda_percentage"] == 100 and st["tokens_per_sec_cuda"] > 0
+    m = P.MoEPerformanceMonitor()
+    m.record_cuda(2.0, 100)
+    m.record_pytorch(6.0, 100)
+    assert m.get_stats()["estimated_speedup"] == 3.0 and m.get_stats()["tokens_per_sec_pytorch"] == 100 / 0.006
+    P.reset_performance_monitor()
+
+
 def test_fused_swiglu_seam(gpu):
     import os
     import sys
