@@ -112,6 +112,8 @@ _SIGNATURES = {
     "ats_calibrate_copy": (c_int, [c_void_p, c_void_p, c_size_t, c_void_p]),
     "ats_calibrate_mfma": (c_int, [c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]),
     "ats_debug_decode_tile": (c_int, [c_int64, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]),
+    "ats_debug_decode_tiles_device": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int64,
+                                              c_void_p, c_void_p]),
     "ats_debug_grid_blocks": (c_int64, [c_int64, c_int, c_int, c_int, c_int, c_int, c_int]),
 }
 

@@ -1612,6 +1612,40 @@ extern "C" int ats_grouped_gemm_nt(const void* a, const void* const* a_ptrs, int
     return ATS_OK;
 }
 
+// Device-side view of the tile schedule: one wave per block id evaluates decode_tile_wave (the search the GEMM
+// kernels run) and writes {expert, m_tile, n_tile, slice}, or -1s where the block owns no tile.
+namespace ats {
+__global__ __launch_bounds__(64) void debug_decode_tiles_kernel(const int32_t* __restrict__ row_count, int E, int BM,
+                                                                int n_tiles, int SM, int SN, int aligned, int k_slices,
+                                                                int32_t* __restrict__ out4) {
+    TileCoord tc;
+    int slice = 0;
+    const bool ok = decode_tile_wave(blockIdx.x, row_count, E, BM, n_tiles, SM, SN, aligned != 0, &tc, k_slices, &slice);
+    if (threadIdx.x == 0) {
+        int32_t* o = out4 + (int64_t)blockIdx.x * 4;
+        o[0] = ok ? tc.e : -1;
+        o[1] = ok ? tc.mt : -1;
+        o[2] = ok ? tc.nt : -1;
+        o[3] = ok ? slice : -1;
+    }
+}
+}  // namespace ats
+
+extern "C" int ats_debug_decode_tiles_device(const int32_t* row_count_dev, int E, int BM, int n_tiles, int SM, int SN,
+                                             int aligned, int k_slices, int64_t n_blocks, int32_t* out4_dev,
+                                             ats_stream_t stream) {
+    using namespace ats;
+    ATS_REQUIRE(row_count_dev && out4_dev && E > 0 && BM > 0 && n_tiles > 0 && SM > 0 && SN > 0 && SM * SN == kSuperBlocks &&
+                    k_slices >= 1 && n_blocks >= 0 && n_blocks < 0x7fffffffLL,
+                ATS_ERR_INVALID_ARG, "ats_debug_decode_tiles_device: E=%d BM=%d n_tiles=%d SM=%d SN=%d k_slices=%d", E, BM,
+                n_tiles, SM, SN, k_slices);
+    if (n_blocks == 0) return ATS_OK;
+    hipLaunchKernelGGL(debug_decode_tiles_kernel, dim3((unsigned)n_blocks), dim3(64), 0, as_stream(stream), row_count_dev,
+                       E, BM, n_tiles, SM, SN, aligned, k_slices, out4_dev);
+    ATS_CHECK_LAUNCH("ats_debug_decode_tiles_device");
+    return ATS_OK;
+}
+
 // Host-side view of the tile schedule (for tests of the block -> tile map).
 extern "C" int ats_debug_decode_tile(int64_t block, const int32_t* row_count_host, int E, int BM, int n_tiles,
                                      int SM, int SN, int aligned, int k_slices, int32_t* out4) {

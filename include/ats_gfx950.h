@@ -426,6 +426,12 @@ int ats_legacy_last_status(void);
 int ats_debug_decode_tile(int64_t block, const int32_t* row_count_host, int E, int BM, int n_tiles,
                           int SM, int SN, int aligned, int k_slices, int32_t* out4);
 int64_t ats_debug_grid_blocks(int64_t max_rows, int E, int BM, int n_tiles, int SM, int SN, int aligned);
+/* The same map as the GEMM kernels evaluate it on the device (a wave-parallel search): out4_dev
+ * [n_blocks, 4] int32 receives {expert, m_tile, n_tile, slice} per block id, -1s where the block
+ * owns no tile.  row_count_dev is a device array. */
+int ats_debug_decode_tiles_device(const int32_t* row_count_dev, int E, int BM, int n_tiles, int SM, int SN,
+                                  int aligned, int k_slices, int64_t n_blocks, int32_t* out4_dev,
+                                  ats_stream_t stream);
 
 /* ---- Calibration loop for the benchmark ----
  * No reference counterpart (the reference's benchmark, Src/Main_Scripts/core/cuda_debug_script.py,

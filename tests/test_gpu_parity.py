@@ -571,6 +571,36 @@ def test_select_topk_long_sequences_with_ties(ops, gpu, L, keep):
     assert torch.equal(sel.long(), ref)
 
 
+@pytest.mark.parametrize("aligned", [0, 1])
+@pytest.mark.parametrize("counts,BM,n_tiles,SM,SN,slices", [
+    ([5120, 4000, 300, 0, 1, 256, 257, 77], 256, 112, 4, 8, 1),
+    ([384] * 64, 256, 11, 8, 4, 1),
+    ([7, 0, 300, 129] * 40, 128, 5, 4, 8, 1),            # 160 groups: three 64-group steps of the search
+    ([20, 16, 0, 3] * 20, 32, 40, 1, 32, 2),             # 80 experts x 2 K slices
+])
+def test_tile_schedule_on_device_equals_host(gpu, counts, BM, n_tiles, SM, SN, slices, aligned):
+    """The wave-parallel search of the GEMM kernels (prefix scan by shuffles, ballot, 64 groups per step) gives
+    every block id the tile that the sequential host walk gives it."""
+    from adaptivetrainingsystem_amd import _lib
+    lib = _lib.load()
+    rc = np.asarray(counts, dtype=np.int32)
+    E = len(counts)
+    blocks = lib.ats_debug_grid_blocks(int(rc.sum()) * slices, E * slices, BM, n_tiles, SM, SN, aligned)
+    out = torch.full((blocks, 4), -7, dtype=torch.int32, device=gpu)
+    rc_dev = torch.from_numpy(rc).to(gpu)
+    assert lib.ats_debug_decode_tiles_device(rc_dev.data_ptr(), E, BM, n_tiles, SM, SN, aligned, slices, blocks,
+                                             out.data_ptr(), None) == 0
+    torch.cuda.synchronize()
+    got = out.cpu().numpy()
+    want = np.full((blocks, 4), -1, dtype=np.int32)
+    o4 = np.zeros(4, dtype=np.int32)
+    for b in range(blocks):
+        if lib.ats_debug_decode_tile(b, rc.ctypes.data, E, BM, n_tiles, SM, SN, aligned, slices, o4.ctypes.data):
+            want[b] = o4
+    assert (want[:, 0] >= 0).sum() == slices * n_tiles * sum(-(-c // BM) for c in counts)
+    assert np.array_equal(got, want)
+
+
 def test_performance_monitor_api(A, gpu):
     """The monitor of the reference's operator module (moe_cuda_wrapper.py:76-159, 599-611): same keys, fed by HIP
     events instead of synchronisations, only while it is switched on."""
