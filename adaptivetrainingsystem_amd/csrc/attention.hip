@@ -16,7 +16,14 @@
 // which is legal because the contraction over keys is a sum.  V stays as it is in memory ([key][d], any
 // batch / position / head strides) all the way into LDS; the V^T fragments come out of LDS through the
 // transposing read ds_read_b64_tr_b16, so no transposed copy of V is ever made.
+//
+// Two bodies share this layout: attention_q_tile_pipe (whole key range; the prefill / training path) loads
+// K and V straight into LDS and overlaps the score MFMAs of the next key tile with the softmax of the
+// current one inside every wave; attention_q_tile (a key range of a split, for decoding against a long
+// cache) keeps the simpler schedule with loads through registers.
 #include <math.h>
+
+#include <type_traits>
 
 #include "ats_common.hpp"
 
@@ -271,7 +278,13 @@ __device__ __forceinline__ void attention_q_tile(const bf16_t* __restrict__ q, c
 #pragma unroll
                 for (int v = 0; v < 16; ++v) mx = fmaxf(mx, acc_s[kb][v]);
             mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-            const float m_new = fmaxf(m_run, mx * sc);   // a positive factor keeps the order
+            // The reference point of the exponentials follows the running maximum lazily: it moves only when
+            // the maximum has grown by more than kLazy (log2 units), so p <= 2^kLazy, which float32 sums and
+            // bf16 operands hold without loss of relative precision, and the rescaling of the output
+            // accumulator (64 multiplies per lane) becomes rare; the result l and o / l is the same quantity.
+            constexpr float kLazy = 8.0f;
+            const float m_cand = fmaxf(m_run, mx * sc);   // a positive factor keeps the order
+            const float m_new = m_cand - m_run > kLazy ? m_cand : m_run;   // -inf on the first tile: moves
             const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);   // 0 on the first tile
             float psum = 0.f;
             // p = exp2(s * c - m * c): one fused multiply-add per element, c = scale * log2(e)
@@ -367,6 +380,345 @@ __device__ __forceinline__ void attention_q_tile(const bf16_t* __restrict__ q, c
 #undef ATT_SV
 }
 
+// Order of the MFMAs of one iteration of attention_q_tile_pipe.  NS score MFMAs (tile t+1) and 4 * DB output
+// MFMAs (tile t; DB per group of 16 keys) are dealt into four groups and a tail:
+//     group 0: NS/4 score MFMAs;   group g = 1..3: NS/4 score MFMAs, then the DB output MFMAs of key group g-1;
+//     tail: the DB output MFMAs of key group 3.
+// The exponentials of key group g are computed during group g, so the output MFMAs of a key group always find
+// their probabilities ready.
+template <int I, int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        static_for<I + 1, N>(f);
+    }
+}
+
+template <int NS, int DB>
+struct PipeSeq {
+    static constexpr int SPG = NS / 4;
+    static constexpr int GS = SPG + DB;     // slots of groups 1..3
+    static_assert(SPG * 4 == NS && 8 % SPG == 0 && 8 % GS == 0, "slots per group must divide the 8 elements of a key group");
+    static constexpr int group(int u) { return u < SPG ? 0 : 1 + (u - SPG) / GS; }      // 4 = tail
+    static constexpr int slot_in_group(int u) { return u < SPG ? u : (u - SPG) % GS; }
+    static constexpr int group_slots(int g) { return g == 0 ? SPG : GS; }
+    static constexpr bool is_s(int u) { return group(u) < 4 && slot_in_group(u) < SPG; }
+    static constexpr int idx(int u) {
+        return is_s(u) ? group(u) * SPG + slot_in_group(u)
+                       : (group(u) < 4 ? (group(u) - 1) * DB + slot_in_group(u) - SPG : 3 * DB + (u - SPG - 3 * GS));
+    }
+};
+
+// Software-pipelined variant of attention_q_tile (same arguments and results, without the key-range split).
+//
+// A wave's two units have about the same amount of work per key tile at head_dim 128: ~1000 cycles of MFMA
+// (score and output products) and ~900 cycles of vector ALU (32 exponentials per lane at a quarter rate, the
+// maximum, the sum, the conversion).  In attention_q_tile the two alternate inside a wave and overlap only
+// by the luck of the other wave on the SIMD being in the other phase.  Here the score product of tile t+1
+// is issued between the softmax instructions of tile t, so every wave keeps both units busy by itself:
+//     iteration t:   S(t+1) = K(t+1) . Q^T  interleaved with  P(t) = softmax step of S(t)
+//                    O^T   += V(t)^T . P(t)^T
+// which takes a second score accumulator (32 registers).  The registers come from the loads: K and V tiles
+// go from memory straight into LDS (buffer_load_dwordx4 ... lds, lane l of an instruction deposits its 16
+// bytes at M0 + 16 l), so no tile passes through registers and no ds_write is issued.  Such a load writes
+// 1 KiB of consecutive LDS, so rows cannot be padded; bank conflicts are avoided by an XOR swizzle applied on
+// the global side instead (which 16-byte chunk of a row a lane fetches):
+//     K: slot s of row r holds chunk s ^ fK(r); the 16 rows that a quarter wave reads with ds_read_b128 hit
+//        16 different slots (fK(r) = r % 16 for 256-byte rows; (r / 2) % 8 for 128-byte rows, where two rows
+//        share a 256-byte line),
+//     V: the transposing read takes 64 consecutive bytes from each of 4 consecutive rows per half wave; the
+//        64-byte group index is XORed with fV(r) (r % 4, or (r / 2) % 2 for 128-byte rows), so the four rows
+//        land on four different groups of 16 banks.
+// K runs one tile ahead of V: at the start of iteration t the loads of K(t+2) and V(t+1) are issued into the
+// stages that K(t) and V(t-1) occupied (everybody was done with them at the barrier that ended iteration
+// t-1) and have the whole iteration to land; two stages each, 4 x 16 KiB at head_dim 128.
+template <int D, bool BIAS, int NT>
+__device__ __forceinline__ void attention_q_tile_pipe(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
+                                                      int64_t k_sb, int64_t k_sh, const bf16_t* __restrict__ v,
+                                                      int64_t v_sb, int v_sl, int64_t v_sh,
+                                                      const float* __restrict__ key_bias, bf16_t* __restrict__ out,
+                                                      float* __restrict__ lse, int Hq, int Hkv, int L, int Lk,
+                                                      float scale_log2, int qt, int head, int b, bool pack,
+                                                      unsigned char* smem) {
+    typedef __attribute__((address_space(3))) void* lds_ptr_t;
+    typedef __attribute__((address_space(3))) unsigned char* lds_u8_t;
+    typedef __attribute__((address_space(3))) au32x4_t* lds_v4_t;
+    typedef __attribute__((address_space(3))) float* lds_f32_t;
+    typedef float att_f32x4_t __attribute__((ext_vector_type(4)));
+    typedef __attribute__((address_space(3))) att_f32x4_t* lds_f32x4_t;
+    const lds_u8_t sm = (lds_u8_t)smem;     // every LDS access below goes through this typed base
+    constexpr int NW = NT / 64;
+    constexpr int kAttBM = att_rows_per_block(NT);
+    constexpr int KS = D / 16;              // k-steps of the score product
+    constexpr int DB = D / 32;              // 32-row blocks of the output (transposed)
+    constexpr int ROWB = D * 2;             // bytes per K or V row in LDS
+    constexpr int CPR = D / 8;              // 16-byte chunks per row
+    constexpr int TILE = kAttBN * ROWB;
+    constexpr int NI = TILE / 1024 / NW;    // load instructions per wave for a K tile (and for a V tile)
+    static_assert(NI >= 1 && NI * NW * 1024 == TILE, "loader tiling");
+    constexpr int NS = 2 * KS;              // score MFMAs per tile
+    constexpr int NO = 4 * DB;              // output MFMAs per tile
+    constexpr int kRing = (BIAS && D == 128) ? 4 : 6;   // the bias variant needs the registers
+    static_assert(kRing <= NO, "the fragment ring runs through both products");
+    using SEQ = PipeSeq<NS, DB>;
+    // LDS map: [K stage 0][K stage 1][V stage 0][V stage 1][bias: 2 x 64 floats]
+    constexpr int V_BASE = 2 * TILE;
+    const lds_f32_t s_bias = (lds_f32_t)(sm + 4 * TILE);
+    const float* bias_row = BIAS ? key_bias + (int64_t)b * Lk : nullptr;
+    const int off = Lk - L;                 // query i sits at position i + (Lk - L)
+    constexpr bool has_bias = BIAS;
+    const float sc = has_bias ? 1.0f : scale_log2;
+    float r_bias = 0.f;
+
+    const int rep = Hq / Hkv;
+    const int rp = pack ? rep : 1;
+    const int n_rows = L * rp;
+    const int hkv = pack ? head : head / rep;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int col = lane & 31, g = lane >> 5;
+    const int row = qt * kAttBM + wave * 32 + col;
+    const int row_clamped = row < n_rows ? row : n_rows - 1;
+    const int q_clamped = row_clamped / rp;
+    const int hq = pack ? hkv * rep + row_clamped % rp : head;
+    const bool row_valid = row < n_rows;
+
+    const bf16_t* qp = q + ((int64_t)(b * Hq + hq) * L + q_clamped) * D;
+    const bf16_t* kbase = k + b * k_sb + hkv * k_sh;
+    const bf16_t* vbase = v + b * v_sb + hkv * v_sh;
+
+    au32x4_t qf[KS];
+#pragma unroll
+    for (int s = 0; s < KS; ++s) qf[s] = *reinterpret_cast<const au32x4_t*>(qp + s * 16 + g * 8);
+
+    const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<bf16_t*>(kbase), 0, (int)((int64_t)Lk * D * 2), 0x00020000);
+    const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<bf16_t*>(vbase), 0, (int)((((int64_t)Lk - 1) * v_sl + D) * 2), 0x00020000);
+    // load instruction j of this wave fills LDS positions (j * NW + wave) * 64 + lane (16-byte units) of a stage
+    int k_off[NI], v_off[NI];
+#pragma unroll
+    for (int j = 0; j < NI; ++j) {
+        const int p = (j * NW + wave) * 64 + lane;
+        const int r = p / CPR, s = p % CPR;
+        const int fk = D == 128 ? (r & 15) : ((r >> 1) & 7);
+        const int fv = D == 128 ? (r & 3) : ((r >> 1) & 1);
+        k_off[j] = (r * D + (s ^ fk) * 8) * 2;
+        v_off[j] = (r * v_sl + (s ^ (fv << 2)) * 8) * 2;
+    }
+#define PIPE_LOAD_K(tile_, stage_)                                                                     \
+    _Pragma("unroll") for (int j_ = 0; j_ < NI; ++j_) __builtin_amdgcn_raw_ptr_buffer_load_lds(        \
+        k_rsrc, (lds_ptr_t)(sm + (stage_) * TILE + (j_ * NW + wave) * 1024), 16, k_off[j_],            \
+        (tile_) * (kAttBN * D * 2), 0, 0)
+#define PIPE_LOAD_V(tile_, stage_)                                                                     \
+    _Pragma("unroll") for (int j_ = 0; j_ < NI; ++j_) __builtin_amdgcn_raw_ptr_buffer_load_lds(        \
+        v_rsrc, (lds_ptr_t)(sm + V_BASE + (stage_) * TILE + (j_ * NW + wave) * 1024), 16, v_off[j_],   \
+        (tile_) * kAttBN * v_sl * 2, 0, 0)
+    // Keys past Lk: their V rows must be zeros in LDS (their probabilities are exact zeros, but 0 x NaN is
+    // not); each lane clears the positions its own loads address, after those loads have landed.
+#define PIPE_CLEAR_V_TAIL(tile_, stage_)                                                               \
+    if (((tile_) + 1) * kAttBN > Lk) {                                                                 \
+        _Pragma("unroll") for (int j_ = 0; j_ < NI; ++j_) {                                            \
+            const int p_ = (j_ * NW + wave) * 64 + lane;                                               \
+            if ((tile_) * kAttBN + p_ / CPR >= Lk)                                                     \
+                *(lds_v4_t)(sm + V_BASE + (stage_) * TILE + p_ * 16) = au32x4_t{0u, 0u, 0u, 0u};       \
+        }                                                                                              \
+    }
+
+    // fragment addresses (byte offsets into smem, stage and fragment row blocks added as constants)
+    int k_addr[KS], v_addr[DB];
+    {
+        const int fk = D == 128 ? (col & 15) : ((col >> 1) & 7);
+#pragma unroll
+        for (int s = 0; s < KS; ++s) k_addr[s] = col * ROWB + (((2 * s + g) ^ fk) * 16);
+        const int rr = 4 * g + ((lane & 15) >> 2);
+        const int fv = D == 128 ? (rr & 3) : ((rr >> 1) & 1);
+        const int within = 32 * ((lane >> 4) & 1) + 8 * (lane & 3);
+#pragma unroll
+        for (int d = 0; d < DB; ++d) v_addr[d] = V_BASE + rr * ROWB + ((d ^ fv) * 64) + within;
+    }
+    // fragment f of the score product = (k-step f/2, key block f%2); fragment f of the output product =
+    // (k-step f/DB, output block f%DB), read transposed (see attention_q_tile for the lane arithmetic)
+#define PIPE_KFRAG(stage_, f_, dst_)                                                                   \
+    dst_ = *(lds_v4_t)(sm + k_addr[(f_) >> 1] + (stage_) * TILE + ((f_) & 1) * 32 * ROWB)
+#define PIPE_VFRAG(stage_, f_, dst_)                                                                   \
+    {                                                                                                  \
+        const lds_u8_t p_ = sm + v_addr[(f_) % DB] + (stage_) * TILE + ((f_) / DB) * 16 * ROWB;        \
+        const att_tr_t lo_ = __builtin_amdgcn_ds_read_tr16_b64_v4i16((att_lds_tr_ptr_t)(p_));           \
+        const att_tr_t hi_ = __builtin_amdgcn_ds_read_tr16_b64_v4i16((att_lds_tr_ptr_t)(p_ + 8 * ROWB)); \
+        union { att_tr_t t[2]; au32x4_t u; } cv_;                                                     \
+        cv_.t[0] = lo_; cv_.t[1] = hi_;                                                                \
+        dst_ = cv_.u;                                                                                  \
+    }
+    af32x16_t acc_o[DB];
+#pragma unroll
+    for (int d = 0; d < DB; ++d)
+#pragma unroll
+        for (int x = 0; x < 16; ++x) acc_o[d][x] = 0.f;
+    float m_run = -INFINITY, l_run = 0.f;
+
+    const int q_pos = row / rp + off;
+    const int q_block_last = min(qt * kAttBM + kAttBM - 1, n_rows - 1) / rp + off;
+    const int n_tiles = q_block_last / kAttBN + 1;
+    const int q_wave_first = (qt * kAttBM + wave * 32) / rp + off;
+    const int q_wave_last = qt * kAttBM + wave * 32 < n_rows ? (qt * kAttBM + wave * 32 + 31) / rp + off : -1;
+    const int my_tiles = q_wave_last >= 0 ? min(q_wave_last / kAttBN + 1, n_tiles) : 0;   // tiles this wave computes
+
+    au32x4_t ring[kRing];
+    af32x16_t acc_sa[2], acc_sb[2];
+    au32x4_t pf[4];
+
+    // ---- prologue: K(0), V(0), K(1) land; S(0)
+    PIPE_LOAD_K(0, 0);
+    PIPE_LOAD_V(0, 0);
+    if (n_tiles > 1) PIPE_LOAD_K(1, 1);
+    if (has_bias && tid < kAttBN) s_bias[tid] = tid < Lk ? bias_row[tid] * 1.4426950408889634f : 0.f;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    PIPE_CLEAR_V_TAIL(0, 0)
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+#pragma unroll
+    for (int s = 0; s < KS; ++s) asm volatile("" : "+v"(qf[s]));
+    if (my_tiles > 0) {
+#pragma unroll
+        for (int f = 0; f < kRing; ++f) PIPE_KFRAG(0, f, ring[f]);
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int x = 0; x < 16; ++x) acc_sa[kb][x] = 0.f;
+#pragma unroll
+        for (int f = 0; f < NS; ++f) {
+            acc_sa[f & 1] = att_mma(ring[f % kRing], qf[f >> 1], acc_sa[f & 1]);
+            if (f + kRing < NS) PIPE_KFRAG(0, f + kRing, ring[f % kRing]);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    // every wave is done with K stage 0 before K(2) may land there
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+
+    // Iteration t with PAR = t % 2: S(t) is in CUR, S(t+1) goes to NXT; K(t+1) sits in K stage PAR^1, V(t) in V
+    // stage PAR; K(t+2) is loaded into K stage PAR, V(t+1) into V stage PAR^1.
+    // The 64 keys of a tile form four groups of 16 (one k-step of the output product each).  After the row
+    // maximum is known, the iteration runs through NS + NO MFMA slots in the order given by PipeSeq: group g
+    // holds a quarter of the score MFMAs of tile t+1 and the output MFMAs of key group g-1 of tile t, and behind
+    // every MFMA comes a share of the exponentials of key group g; so MFMAs and vector instructions alternate
+    // through the whole iteration, and a wave that has to wait for the matrix pipe (the other wave of the SIMD
+    // is using it) is never more than one MFMA behind with its vector work.
+#define PIPE_SLOT_FRAG(kstage_, vstage_, u_, dst_)                                                     \
+    {                                                                                                  \
+        if constexpr (SEQ::is_s(u_)) { PIPE_KFRAG(kstage_, SEQ::idx(u_), dst_); }                      \
+        else PIPE_VFRAG(vstage_, SEQ::idx(u_), dst_)                                                   \
+    }
+#define PIPE_BODY(t_, PAR, CUR, NXT)                                                                   \
+    {                                                                                                  \
+        const int n0 = (t_) * kAttBN;                                                                  \
+        if ((t_) + 2 < n_tiles) PIPE_LOAD_K((t_) + 2, PAR);                           \
+        if ((t_) + 1 < n_tiles) PIPE_LOAD_V((t_) + 1, (PAR) ^ 1);                     \
+        if (has_bias && (t_) + 1 < n_tiles && tid < kAttBN)                                            \
+            r_bias = n0 + kAttBN + tid < Lk ? bias_row[n0 + kAttBN + tid] * 1.4426950408889634f : 0.f; \
+        if ((t_) < my_tiles) {                                                                         \
+            static_for<0, kRing>([&](auto uc) __attribute__((always_inline)) {                         \
+                constexpr int u = decltype(uc)::value;                                                 \
+                PIPE_SLOT_FRAG((PAR) ^ 1, PAR, u, ring[u]);                                            \
+            });                                                                                        \
+            if (has_bias) {                                                                            \
+                const lds_f32_t bt = s_bias + (PAR) * kAttBN + g * 4;                                  \
+                _Pragma("unroll") for (int kb = 0; kb < 2; ++kb)                                       \
+                _Pragma("unroll") for (int r = 0; r < 4; ++r) {                                        \
+                    const att_f32x4_t b4 = *(lds_f32x4_t)(bt + kb * 32 + r * 8);                       \
+                    CUR[kb][r * 4 + 0] = __builtin_fmaf(CUR[kb][r * 4 + 0], scale_log2, b4.x);         \
+                    CUR[kb][r * 4 + 1] = __builtin_fmaf(CUR[kb][r * 4 + 1], scale_log2, b4.y);         \
+                    CUR[kb][r * 4 + 2] = __builtin_fmaf(CUR[kb][r * 4 + 2], scale_log2, b4.z);         \
+                    CUR[kb][r * 4 + 3] = __builtin_fmaf(CUR[kb][r * 4 + 3], scale_log2, b4.w);         \
+                }                                                                                      \
+            }                                                                                          \
+            if (n0 + kAttBN - 1 > q_wave_first) {                                                      \
+                _Pragma("unroll") for (int kb = 0; kb < 2; ++kb)                                       \
+                _Pragma("unroll") for (int x = 0; x < 16; ++x) {                                       \
+                    const int key = n0 + kb * 32 + (x >> 2) * 8 + g * 4 + (x & 3);                     \
+                    if (key > q_pos) CUR[kb][x] = -INFINITY;                                           \
+                }                                                                                      \
+            }                                                                                          \
+            float mx = -INFINITY;                                                                      \
+            _Pragma("unroll") for (int kb = 0; kb < 2; ++kb)                                           \
+            _Pragma("unroll") for (int x = 0; x < 16; ++x) mx = fmaxf(mx, CUR[kb][x]);                 \
+            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));                                                    \
+            const float m_cand = fmaxf(m_run, mx * sc);                                                \
+            const float m_new = m_cand - m_run > kLazyMax ? m_cand : m_run;                            \
+            const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);                                 \
+            float psum = 0.f;                                                                          \
+            if (!__all(alpha == 1.0f)) {                                                               \
+                _Pragma("unroll") for (int d = 0; d < DB; ++d)                                         \
+                _Pragma("unroll") for (int x = 0; x < 16; ++x) acc_o[d][x] *= alpha;                   \
+            }                                                                                          \
+            __builtin_amdgcn_sched_barrier(0);                                                         \
+            static_for<0, NS + NO>([&](auto uc) __attribute__((always_inline)) {                       \
+                constexpr int u = decltype(uc)::value;                                                 \
+                constexpr int f = SEQ::idx(u);                                                         \
+                if constexpr (SEQ::is_s(u)) {                                                          \
+                    if constexpr (f < 2) {                                                             \
+                        _Pragma("unroll") for (int x = 0; x < 16; ++x) NXT[f & 1][x] = 0.f;            \
+                    }                                                                                  \
+                    NXT[f & 1] = att_mma(ring[u % kRing], qf[f >> 1], NXT[f & 1]);                     \
+                } else {                                                                               \
+                    acc_o[f % DB] = att_mma(ring[u % kRing], pf[f / DB], acc_o[f % DB]);               \
+                }                                                                                      \
+                if constexpr (u + kRing < NS + NO) PIPE_SLOT_FRAG((PAR) ^ 1, PAR, u + kRing, ring[u % kRing]); \
+                if constexpr (SEQ::group(u) < 4) {                                                     \
+                    constexpr int gq = SEQ::group(u), w = SEQ::slot_in_group(u), n = SEQ::group_slots(gq); \
+                    static_for<w * 8 / n, (w + 1) * 8 / n>([&](auto jc) __attribute__((always_inline)) { \
+                        constexpr int j = decltype(jc)::value;                                         \
+                        constexpr int kb = gq >> 1, x = (gq & 1) * 8 + j;                              \
+                        float p = __builtin_amdgcn_exp2f(__builtin_fmaf(CUR[kb][x], sc, -m_new));      \
+                        asm volatile("" : "+v"(p));   /* keeps the exponential here, between the MFMAs */ \
+                        CUR[kb][x] = p;                                                                \
+                        psum += p;                                                                     \
+                        if constexpr (j & 1) pf[gq][j >> 1] = pack_bf16x2(CUR[kb][x - 1], p);          \
+                    });                                                                                \
+                }                                                                                      \
+                __builtin_amdgcn_sched_barrier(0);                                                     \
+            });                                                                                        \
+            l_run = l_run * alpha + psum;                                                              \
+            m_run = m_new;                                                                             \
+        }                                                                                              \
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");                                               \
+        if ((t_) + 1 < n_tiles) {                                                                      \
+            PIPE_CLEAR_V_TAIL((t_) + 1, (PAR) ^ 1)                                                     \
+            if (has_bias && tid < kAttBN) s_bias[((PAR) ^ 1) * kAttBN + tid] = r_bias;                 \
+        }                                                                                              \
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");                                \
+    }
+
+    constexpr float kLazyMax = 8.0f;   // see attention_q_tile: the reference point of the exponentials moves lazily
+    for (int t = 0; t < n_tiles; t += 2) {
+        PIPE_BODY(t, 0, acc_sa, acc_sb)
+        if (t + 1 >= n_tiles) break;
+        PIPE_BODY(t + 1, 1, acc_sb, acc_sa)
+    }
+#undef PIPE_BODY
+#undef PIPE_SLOT_FRAG
+#undef PIPE_VFRAG
+#undef PIPE_KFRAG
+#undef PIPE_CLEAR_V_TAIL
+#undef PIPE_LOAD_V
+#undef PIPE_LOAD_K
+
+    l_run += __shfl_xor(l_run, 32, 64);
+    const float inv = 1.0f / l_run;
+    if (row_valid) {
+        bf16_t* orow = out + ((int64_t)b * L + q_clamped) * (int64_t)(Hq * D) + hq * D;
+#pragma unroll
+        for (int d = 0; d < DB; ++d)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                au32x2_t w;
+                w.x = pack_bf16x2(acc_o[d][r * 4 + 0] * inv, acc_o[d][r * 4 + 1] * inv);
+                w.y = pack_bf16x2(acc_o[d][r * 4 + 2] * inv, acc_o[d][r * 4 + 3] * inv);
+                *reinterpret_cast<au32x2_t*>(orow + d * 32 + r * 8 + g * 4) = w;
+            }
+        if (lse && g == 0) lse[(int64_t)(b * Hq + hq) * L + q_clamped] = (m_run + log2f(l_run)) * 0.6931471805599453f;
+    }
+}
+
 // Each workgroup takes a long query tile and its mirror-image short one, so every workgroup of a launch
 // does the same work: the hardware hands workgroups to XCDs and shader engines strictly in turn and waits
 // for the next target to have room, so workgroups of uneven length leave whole shader engines idle.
@@ -403,8 +755,8 @@ __global__ __launch_bounds__(NT, 512 / NT) void attention_fwd_kernel(const bf16_
 #pragma unroll 1
     for (int half = 0; half < 2; ++half) {
         if (half && pair == qt_long) break;   // an odd tile count leaves the middle tile on its own
-        attention_q_tile<D, BIAS, NT>(q, k, k_sb, k_sh, v, v_sb, v_sl, v_sh, key_bias, out, lse, Hq, Hkv, L, Lk, scale_log2,
-                            half ? pair : qt_long, head, b, pack != 0, smem);
+        attention_q_tile_pipe<D, BIAS, NT>(q, k, k_sb, k_sh, v, v_sb, v_sl, v_sh, key_bias, out, lse, Hq, Hkv, L, Lk,
+                                           scale_log2, half ? pair : qt_long, head, b, pack != 0, smem);
     }
 }
 
@@ -582,8 +934,8 @@ extern "C" int ats_attention_fwd(const void* q, const void* k, int64_t k_sb, int
                            static_cast<bf16_t*>(out), lse, Hq, Hkv, L, Lk, scale_log2, B, pack);
         return ATS_OK;
     };
-    // K tile, V tile (two stages each) and, with a bias, two stages of one float per key
-    const int smem = 2 * kAttBN * ((D * 2 + 16) + (D * 2 + 64)) + (key_bias ? 2 * kAttBN * 4 : 0);
+    // K tile, V tile (two stages each, rows unpadded) and, with a bias, two stages of one float per key
+    const int smem = 4 * kAttBN * D * 2 + (key_bias ? 2 * kAttBN * 4 : 0);
     int rc;
     if (D == 128 && nt == 256)
         rc = key_bias ? launch(attention_fwd_kernel<128, true, 256>, smem, reserved_lds[0])
