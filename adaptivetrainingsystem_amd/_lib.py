@@ -7,7 +7,7 @@ from __future__ import annotations
 
 import ctypes
 import os
-from ctypes import c_char_p, c_double, c_float, c_int, c_int64, c_size_t, c_void_p
+from ctypes import c_char_p, c_double, c_float, c_int, c_int64, c_uint64, c_size_t, c_void_p
 
 LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libats_gfx950.so")
 
@@ -92,6 +92,11 @@ _SIGNATURES = {
     "ats_attention_fwd": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_int64, c_void_p,
                                   c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p,
                                   c_size_t, c_void_p]),
+    "ats_attention_fwd_ex": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_int64, c_int64, c_int64, c_void_p,
+                                     c_void_p, c_int64, c_float, c_uint64, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
+                                     c_int, c_int, c_float, c_void_p, c_size_t, c_void_p]),
+    "ats_attention_bwd_ex": (c_int, [c_void_p] * 8 + [c_int64, c_float, c_uint64] + [c_void_p] * 3 + [c_int] * 6 +
+                             [c_float, c_void_p]),
     "ats_attention_delta": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
     "ats_attention_bwd": (c_int, [c_void_p] * 10 + [c_int] * 6 + [c_float, c_void_p]),
     "ats_combine": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_int,

@@ -92,21 +92,26 @@ class ScatterAddRowsFunction(Function):
 
 class AttentionFunction(Function):
     """Causal grouped-query attention: q [B,Hq,L,D], k, v [B,Hkv,Lk,D] -> [B, L, Hq*D]; key_bias
-    [B, Lk] float32 or None (a constant: it gets no gradient)."""
+    [B, Lk] / pair_bias [B or 1, L, Lk] float32 or None (constants: they get no gradient); dropout_p with the
+    seed that the backward reuses."""
 
     @staticmethod
-    def forward(ctx, q, k, v, scale, key_bias=None):
+    def forward(ctx, q, k, v, scale, key_bias=None, pair_bias=None, dropout_p=0.0, dropout_seed=0):
         q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
-        out, lse = ops.causal_attention(q, k, v, scale, return_lse=True, key_bias=key_bias)
-        ctx.save_for_backward(q, k, v, out, lse, key_bias)
+        out, lse = ops.causal_attention(q, k, v, scale, return_lse=True, key_bias=key_bias, pair_bias=pair_bias,
+                                        dropout_p=dropout_p, dropout_seed=dropout_seed)
+        ctx.save_for_backward(q, k, v, out, lse, key_bias, pair_bias)
         ctx.scale = scale
+        ctx.dropout = (float(dropout_p), int(dropout_seed))
         return out
 
     @staticmethod
     def backward(ctx, dout):
-        q, k, v, out, lse, key_bias = ctx.saved_tensors
-        dq, dk, dv = ops.causal_attention_bwd(q, k, v, out, lse, dout, ctx.scale, key_bias=key_bias)
-        return dq, dk, dv, None, None
+        q, k, v, out, lse, key_bias, pair_bias = ctx.saved_tensors
+        dq, dk, dv = ops.causal_attention_bwd(q, k, v, out, lse, dout, ctx.scale, key_bias=key_bias,
+                                              pair_bias=pair_bias, dropout_p=ctx.dropout[0],
+                                              dropout_seed=ctx.dropout[1])
+        return dq, dk, dv, None, None, None, None, None
 
 
 class LinearFunction(Function):

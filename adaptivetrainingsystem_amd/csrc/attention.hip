@@ -26,6 +26,7 @@
 #include <type_traits>
 
 #include "ats_common.hpp"
+#include "attention_extra.hpp"
 
 namespace ats {
 
@@ -61,7 +62,9 @@ __device__ __forceinline__ af32x16_t att_mma(const au32x4_t& a, const au32x4_t& 
 // running maximum and sum in part_out for attention_merge_kernel: rows of D + 4 floats at
 // ((b * Hq + hq) * L + position) * n_parts + part.
 constexpr int kPartPad = 4;
-template <int D, bool BIAS, int NT, bool SPLIT = false>
+// EXTRA: a bias per (query, key) pair and / or dropout on the weights (attention_extra.hpp); the bias is read
+// from memory in accumulator order (no LDS staging: this is the seldom-used path).
+template <int D, bool BIAS, int NT, bool SPLIT = false, bool EXTRA = false>
 __device__ __forceinline__ void attention_q_tile(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
                                                  int64_t k_sb, int64_t k_sh,
                                                  const bf16_t* __restrict__ v, int64_t v_sb, int v_sl, int64_t v_sh,
@@ -69,7 +72,9 @@ __device__ __forceinline__ void attention_q_tile(const bf16_t* __restrict__ q, c
                                                  float* __restrict__ lse, int Hq, int Hkv, int L, int Lk,
                                                  float scale_log2, int qt, int head, int b, bool pack,
                                                  unsigned char* smem, float* __restrict__ part_out = nullptr,
-                                                 int part = 0, int n_parts = 1, int key_first = 0, int key_count = 0) {
+                                                 int part = 0, int n_parts = 1, int key_first = 0, int key_count = 0,
+                                                 const AttnExtra* ex = nullptr) {
+    static_assert(!(EXTRA && (SPLIT || BIAS)), "the extras come alone: a per-key bias is folded into the pair bias");
     constexpr int kAttThreads = NT;
     constexpr int kAttBM = att_rows_per_block(NT);
     constexpr int KS = D / 16;              // k-steps of the score product
@@ -91,7 +96,7 @@ __device__ __forceinline__ void attention_q_tile(const bf16_t* __restrict__ q, c
     if constexpr (SPLIT) Lk = key_count;      // from here on: the keys of this part, counted from its first
     constexpr bool has_bias = BIAS;
     // with a bias the scores are brought to log2 units before the maximum is taken (sc = 1 afterwards)
-    const float sc = has_bias ? 1.0f : scale_log2;
+    const float sc = (has_bias || EXTRA) ? 1.0f : scale_log2;
     float r_bias = 0.f;
 
     const int rep = Hq / Hkv;
@@ -113,6 +118,22 @@ __device__ __forceinline__ void attention_q_tile(const bf16_t* __restrict__ q, c
     au32x4_t qf[KS];
 #pragma unroll
     for (int s = 0; s < KS; ++s) qf[s] = *reinterpret_cast<const au32x4_t*>(qp + s * 16 + g * 8);
+
+    // extras: this lane's row of the pair bias (a buffer descriptor over the batch entry's [L, Lk] matrix, so
+    // keys past Lk read as zeros) and the dropout key of this (batch, head)
+    __amdgpu_buffer_rsrc_t pb_rsrc;
+    int pb_row = 0;
+    bool ex_bias = false, ex_drop = false;
+    uint32_t head_key = 0, drop_counter0 = 0;
+    if constexpr (EXTRA) {
+        ex_bias = ex->bias_qk != nullptr;
+        ex_drop = ex->keep_scale > 0.f;
+        pb_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(ex_bias ? ex->bias_qk + (int64_t)b * ex->bias_sb : nullptr),
+                                                    0, ex_bias ? (int)((int64_t)L * Lk * 4) : 0, 0x00020000);
+        pb_row = q_clamped * Lk * 4;
+        head_key = attn_head_key(ex->seed_lo, ex->seed_hi, (uint32_t)(b * Hq + hq));
+        drop_counter0 = (uint32_t)q_clamped * (uint32_t)Lk;
+    }
 
     // K and V^T tiles come through buffer loads: a scalar base and tile offset plus one 32-bit lane offset
     // that never changes, so a tile costs no address arithmetic, and keys past Lk read as zeros.
@@ -263,6 +284,22 @@ __device__ __forceinline__ void attention_q_tile(const bf16_t* __restrict__ q, c
                         acc_s[kb][r * 4 + 3] = __builtin_fmaf(acc_s[kb][r * 4 + 3], scale_log2, b4.w);
                     }
             }
+            if constexpr (EXTRA) {   // scores to log2 units plus the pair bias of (this lane's query, key)
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb) {
+                    float bq[16];
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
+                        const int key = n0 + kb * 32 + (v >> 2) * 8 + g * 4 + (v & 3);
+                        bq[v] = ex_bias ? __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                                              pb_rsrc, pb_row + key * 4, 0, 0))
+                                        : 0.f;
+                    }
+#pragma unroll
+                    for (int v = 0; v < 16; ++v)
+                        acc_s[kb][v] = __builtin_fmaf(acc_s[kb][v], scale_log2, bq[v] * 1.4426950408889634f);
+                }
+            }
             if (n0 + kAttBN - 1 > q_wave_first) {   // diagonal tile: causal mask
 #pragma unroll
                 for (int kb = 0; kb < 2; ++kb)
@@ -303,6 +340,18 @@ __device__ __forceinline__ void attention_q_tile(const bf16_t* __restrict__ q, c
                 for (int d = 0; d < DB; ++d)
 #pragma unroll
                     for (int v = 0; v < 16; ++v) acc_o[d][v] *= alpha;
+            }
+            if constexpr (EXTRA) {   // dropout acts on the weights that meet V; the row sum keeps all of them
+                if (ex_drop) {
+#pragma unroll
+                    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) {
+                            const int key = n0 + kb * 32 + (v >> 2) * 8 + g * 4 + (v & 3);
+                            const bool keep = attn_drop_hash(head_key, drop_counter0 + (uint32_t)key) >= ex->drop_threshold;
+                            acc_s[kb][v] = keep ? acc_s[kb][v] * ex->keep_scale : 0.f;
+                        }
+                }
             }
             // P^T as B operand: k-step s holds accumulator values 8*(s&1) .. +7 of key block s>>1
             au32x4_t pf[4];
@@ -760,6 +809,42 @@ __global__ __launch_bounds__(NT, 512 / NT) void attention_fwd_kernel(const bf16_
     }
 }
 
+// The same launch shape for calls with a bias per (query, key) pair or dropout: the non-pipelined body with
+// the extras switched on (four waves; rows are never packed).
+template <int D>
+__global__ __launch_bounds__(256, 2) void attention_fwd_extra_kernel(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, int64_t k_sb, int64_t k_sh, const bf16_t* __restrict__ v,
+    int64_t v_sb, int v_sl, int64_t v_sh, bf16_t* __restrict__ out, float* __restrict__ lse, int Hq, int Hkv, int L, int Lk,
+    float scale_log2, int B, AttnExtra ex) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    constexpr int kAttBM = att_rows_per_block(256);
+    const int heads_per_group = Hq / Hkv;
+    const int n_qt = (L + kAttBM - 1) / kAttBM;
+    const int n_pairs = (n_qt + 1) / 2;
+    const int per_group = n_pairs * heads_per_group;
+    const int n_groups = B * Hkv;
+    int group, within;
+    if (n_groups % 8 == 0) {
+        const int xcd = blockIdx.x & 7, idx = blockIdx.x >> 3;
+        group = (idx / per_group) * 8 + xcd;
+        within = idx % per_group;
+    } else {
+        group = blockIdx.x / per_group;
+        within = blockIdx.x % per_group;
+    }
+    const int b = group / Hkv;
+    const int head = (group % Hkv) * heads_per_group + within / n_pairs;
+    const int pair = within % n_pairs;
+    const int qt_long = n_qt - 1 - pair;
+#pragma unroll 1
+    for (int half = 0; half < 2; ++half) {
+        if (half && pair == qt_long) break;
+        attention_q_tile<D, false, 256, false, true>(q, k, k_sb, k_sh, v, v_sb, v_sl, v_sh, nullptr, out, lse, Hq, Hkv, L, Lk,
+                                                     scale_log2, half ? pair : qt_long, head, b, false, smem, nullptr, 0, 1,
+                                                     0, 0, &ex);
+    }
+}
+
 // Few query rows against many keys (decoding): the keys are cut into n_parts ranges and every (batch, head
 // group, range) gets a workgroup, so that a handful of sequences still fills the chip; the ranges are merged
 // by attention_merge_kernel.  One query tile per group (rows <= 128), part p covers part_len keys from
@@ -851,10 +936,51 @@ extern "C" size_t ats_attention_fwd_workspace(int B, int Hq, int Hkv, int L, int
     return n_parts > 1 ? (size_t)B * Hq * L * n_parts * (D + ats::kPartPad) * sizeof(float) : 0;
 }
 
+// Fills the kernels' view of the optional extras; returns false (with the error text set) on bad arguments.
+namespace ats {
+bool make_attention_extra(const char* who, const float* bias_qk, int64_t bias_sb, float dropout_p, uint64_t seed, int L,
+                          int Lk, AttnExtra* ex, bool* any) {
+    *any = bias_qk != nullptr || dropout_p > 0.f;
+    ex->bias_qk = bias_qk;
+    ex->bias_sb = bias_sb;
+    ex->keep_scale = 0.f;
+    ex->drop_threshold = 0;
+    ex->seed_lo = (uint32_t)seed;
+    ex->seed_hi = (uint32_t)(seed >> 32);
+    if (!(dropout_p >= 0.f && dropout_p < 1.f)) {
+        set_error("%s: dropout probability %g (must be in [0, 1))", who, dropout_p);
+        return false;
+    }
+    if (bias_qk && (bias_sb < 0 || (reinterpret_cast<uintptr_t>(bias_qk) & 3) || (int64_t)L * Lk * 4 >= 0x7fffffffLL)) {
+        set_error("%s: pair bias (batch stride %lld; one [L, Lk] matrix must stay under 2 GiB)", who, (long long)bias_sb);
+        return false;
+    }
+    if (dropout_p > 0.f) {
+        if ((int64_t)L * Lk > 0xffffffffLL) {
+            set_error("%s: dropout needs L * Lk < 2^32", who);
+            return false;
+        }
+        ex->keep_scale = 1.0f / (1.0f - dropout_p);
+        double t = (double)dropout_p * 4294967296.0;
+        ex->drop_threshold = t >= 4294967295.0 ? 0xffffffffu : (uint32_t)t;
+    }
+    return true;
+}
+}  // namespace ats
+
 extern "C" int ats_attention_fwd(const void* q, const void* k, int64_t k_sb, int64_t k_sh, const void* v, int64_t v_sb,
                                  int64_t v_sl, int64_t v_sh, const float* key_bias, void* out, float* lse, int B, int Hq,
                                  int Hkv, int L, int Lk, int D, float scale, void* workspace, size_t workspace_bytes,
                                  ats_stream_t stream) {
+    return ats_attention_fwd_ex(q, k, k_sb, k_sh, v, v_sb, v_sl, v_sh, key_bias, nullptr, 0, 0.f, 0, out, lse, B, Hq, Hkv, L,
+                                Lk, D, scale, workspace, workspace_bytes, stream);
+}
+
+extern "C" int ats_attention_fwd_ex(const void* q, const void* k, int64_t k_sb, int64_t k_sh, const void* v, int64_t v_sb,
+                                    int64_t v_sl, int64_t v_sh, const float* key_bias, const float* bias_qk,
+                                    int64_t bias_sb, float dropout_p, uint64_t dropout_seed, void* out, float* lse, int B,
+                                    int Hq, int Hkv, int L, int Lk, int D, float scale, void* workspace,
+                                    size_t workspace_bytes, ats_stream_t stream) {
     using namespace ats;
     ATS_REQUIRE(B >= 0 && Hq > 0 && Hkv > 0 && Hq % Hkv == 0 && L >= 0 && Lk >= L && scale > 0.f, ATS_ERR_INVALID_ARG,
                 "ats_attention_fwd: B=%d Hq=%d Hkv=%d L=%d Lk=%d scale=%g", B, Hq, Hkv, L, Lk, scale);
@@ -872,6 +998,35 @@ extern "C" int ats_attention_fwd(const void* q, const void* k, int64_t k_sb, int
                 "ats_attention_fwd: %d keys (one head's K or V must stay under 2 GiB)", Lk);
     // few query positions (decoding, short chunks): the query heads of a kv group share a tile's rows
     const float scale_log2 = scale * 1.4426950408889634f;
+    AttnExtra ex;
+    bool extras = false;
+    if (!make_attention_extra("ats_attention_fwd_ex", bias_qk, bias_sb, dropout_p, dropout_seed, L, Lk, &ex, &extras))
+        return ATS_ERR_INVALID_ARG;
+    if (extras) {
+        ATS_REQUIRE(key_bias == nullptr, ATS_ERR_INVALID_ARG,
+                    "ats_attention_fwd_ex: with a pair bias or dropout the per-key bias must be folded into the pair bias");
+        const int64_t blocks = (int64_t)(((L + 127) / 128 + 1) / 2) * Hq * B;
+        ATS_REQUIRE(blocks <= 0x7fffffff, ATS_ERR_UNSUPPORTED, "ats_attention_fwd_ex: %lld workgroups", (long long)blocks);
+        const int smem_x = 2 * kAttBN * ((D * 2 + 16) + (D * 2 + 64));
+        static LdsReservation reserved_x[2];
+        auto launch_x = [&](auto kernel, LdsReservation& reserved) -> int {
+            if (smem_x > 64 * 1024) {
+                hipError_t e = reserve_lds(reserved, {reinterpret_cast<const void*>(kernel)}, smem_x);
+                ATS_REQUIRE(e == hipSuccess, ATS_ERR_LAUNCH, "ats_attention_fwd_ex: cannot reserve %d bytes of LDS: %s",
+                            smem_x, hipGetErrorString(e));
+            }
+            hipLaunchKernelGGL(kernel, dim3((unsigned)blocks), dim3(256), smem_x, as_stream(stream),
+                               static_cast<const bf16_t*>(q), static_cast<const bf16_t*>(k), k_sb, k_sh,
+                               static_cast<const bf16_t*>(v), v_sb, (int)v_sl, v_sh, static_cast<bf16_t*>(out), lse, Hq, Hkv,
+                               L, Lk, scale_log2, B, ex);
+            return ATS_OK;
+        };
+        const int rc = D == 128 ? launch_x(attention_fwd_extra_kernel<128>, reserved_x[0])
+                                : launch_x(attention_fwd_extra_kernel<64>, reserved_x[1]);
+        if (rc != ATS_OK) return rc;
+        ATS_CHECK_LAUNCH("ats_attention_fwd_ex");
+        return ATS_OK;
+    }
     // decoding sizes with a workspace: key ranges in parallel, then a merge
     int part_len = 0;
     const int n_parts = workspace ? attention_split_plan(B, Hq, Hkv, L, Lk, &part_len) : 1;

@@ -20,6 +20,7 @@
 #include <math.h>
 
 #include "ats_common.hpp"
+#include "attention_extra.hpp"
 
 namespace ats {
 
@@ -91,13 +92,15 @@ __global__ __launch_bounds__(256) void attention_delta_kernel(const bf16_t* __re
 
 // ------------------------------------------------------------------------------------------ dQ
 // One 128-row query tile of one (batch, query head): lanes own queries, keys come in tiles of 64.
-template <int D, bool BIAS>
+// EXTRA: pair bias and / or dropout (attention_extra.hpp), the same decisions as the forward made.
+template <int D, bool BIAS, bool EXTRA = false>
 __device__ __forceinline__ void attention_bwd_dq_tile(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
                                                       const bf16_t* __restrict__ v, const bf16_t* __restrict__ dout,
                                                       const float* __restrict__ lse, const float* __restrict__ delta,
                                                       const float* __restrict__ key_bias, bf16_t* __restrict__ dq, int Hq,
                                                       int Hkv, int L, int Lk, float scale, int qt, int hq, int b,
-                                                      unsigned char* smem) {
+                                                      unsigned char* smem, const AttnExtra* ex = nullptr) {
+    static_assert(!(EXTRA && BIAS), "a per-key bias is folded into the pair bias");
     constexpr int KS = D / 16;
     constexpr int DB = D / 32;
     constexpr int RPITCH = D * 2 + 16;        // bytes per K / V row in LDS
@@ -129,6 +132,19 @@ __device__ __forceinline__ void attention_bwd_dq_tile(const bf16_t* __restrict__
     }
     const float lse2 = lse[(int64_t)(b * Hq + hq) * L + q_clamped] * kLog2e;
     const float dl = delta[(int64_t)(b * Hq + hq) * L + q_clamped];
+    __amdgpu_buffer_rsrc_t pb_rsrc;
+    int pb_row = 0;
+    bool ex_bias = false, ex_drop = false;
+    uint32_t head_key = 0, drop_counter0 = 0;
+    if constexpr (EXTRA) {
+        ex_bias = ex->bias_qk != nullptr;
+        ex_drop = ex->keep_scale > 0.f;
+        pb_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(ex_bias ? ex->bias_qk + (int64_t)b * ex->bias_sb : nullptr),
+                                                    0, ex_bias ? (int)((int64_t)L * Lk * 4) : 0, 0x00020000);
+        pb_row = q_clamped * Lk * 4;
+        head_key = attn_head_key(ex->seed_lo, ex->seed_hi, (uint32_t)(b * Hq + hq));
+        drop_counter0 = (uint32_t)q_clamped * (uint32_t)Lk;
+    }
 
     const bf16_t* kbase = k + (int64_t)(b * Hkv + hkv) * Lk * D;
     const bf16_t* vbase = v + (int64_t)(b * Hkv + hkv) * Lk * D;
@@ -201,13 +217,23 @@ __device__ __forceinline__ void attention_bwd_dq_tile(const bf16_t* __restrict__
 #pragma unroll
             for (int x = 0; x < 16; ++x) {
                 // the key of accumulator value x is kb*32 + (x/4)*8 + g*4 + x%4 of the tile
-                const float kbias = BIAS ? sBias[kb * 32 + (x >> 2) * 8 + g * 4 + (x & 3)] : 0.f;
+                float kbias = BIAS ? sBias[kb * 32 + (x >> 2) * 8 + g * 4 + (x & 3)] : 0.f;
+                float dp = acc_p[kb][x];
+                if constexpr (EXTRA) {
+                    const int key = n0 + kb * 32 + (x >> 2) * 8 + g * 4 + (x & 3);
+                    if (ex_bias)
+                        kbias = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(pb_rsrc, pb_row + key * 4, 0, 0)) *
+                                kLog2e;
+                    if (ex_drop)   // dP reaches only the weights that were kept
+                        dp = attn_drop_hash(head_key, drop_counter0 + (uint32_t)key) >= ex->drop_threshold ? dp * ex->keep_scale
+                                                                                                        : 0.f;
+                }
                 float p = __builtin_amdgcn_exp2f(__builtin_fmaf(acc_s[kb][x], scale_log2, kbias - lse2));
                 if (diagonal) {
                     const int key = n0 + kb * 32 + (x >> 2) * 8 + g * 4 + (x & 3);
                     if (key > q_pos) p = 0.f;
                 }
-                acc_s[kb][x] = p * (acc_p[kb][x] - dl) * scale;
+                acc_s[kb][x] = p * (dp - dl) * scale;
             }
         bu32x4_t dsf[4];
 #pragma unroll
@@ -243,11 +269,12 @@ __device__ __forceinline__ void attention_bwd_dq_tile(const bf16_t* __restrict__
 
 // A workgroup takes a long query tile and its mirror-image short one (equal work per workgroup: the
 // hardware hands workgroups out strictly in turn), and the workgroups of one (batch, kv head) share an XCD.
-template <int D, bool BIAS>
+template <int D, bool BIAS, bool EXTRA = false>
 __global__ __launch_bounds__(256, 2) void attention_bwd_dq_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const bf16_t* __restrict__ v,
     const bf16_t* __restrict__ dout, const float* __restrict__ lse, const float* __restrict__ delta,
-    const float* __restrict__ key_bias, bf16_t* __restrict__ dq, int Hq, int Hkv, int L, int Lk, float scale, int B) {
+    const float* __restrict__ key_bias, bf16_t* __restrict__ dq, int Hq, int Hkv, int L, int Lk, float scale, int B,
+    AttnExtra ex) {
     extern __shared__ __align__(16) unsigned char smem[];
     const int n_qt = (L + kBwdRows - 1) / kBwdRows;
     const int n_pairs = (n_qt + 1) / 2;
@@ -269,21 +296,22 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dq_kernel(
 #pragma unroll 1
     for (int half = 0; half < 2; ++half) {
         if (half && pair == qt_long) break;
-        attention_bwd_dq_tile<D, BIAS>(q, k, v, dout, lse, delta, key_bias, dq, Hq, Hkv, L, Lk, scale, half ? pair : qt_long,
-                                 hq, b, smem);
+        attention_bwd_dq_tile<D, BIAS, EXTRA>(q, k, v, dout, lse, delta, key_bias, dq, Hq, Hkv, L, Lk, scale,
+                                              half ? pair : qt_long, hq, b, smem, &ex);
     }
 }
 
 // ------------------------------------------------------------------------------------------ dK, dV
 // One 128-row key tile of one (batch, kv head): lanes own keys; the queries of every query head of the
 // group come in steps of 32, starting at the first query that sees the tile.
-template <int D>
+template <int D, bool EXTRA = false>
 __device__ __forceinline__ void attention_bwd_dkv_tile(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
                                                        const bf16_t* __restrict__ v, const bf16_t* __restrict__ dout,
                                                        const float* __restrict__ lse, const float* __restrict__ delta,
                                                        const float* __restrict__ key_bias, bf16_t* __restrict__ dk,
                                                        bf16_t* __restrict__ dv, int Hq, int Hkv, int L, int Lk, float scale,
-                                                       int kt_idx, int hkv, int b, unsigned char* smem) {
+                                                       int kt_idx, int hkv, int b, unsigned char* smem,
+                                                       const AttnExtra* ex = nullptr) {
     constexpr int KS = D / 16;
     constexpr int DB = D / 32;
     constexpr int RPITCH = D * 2 + 16;        // bytes per Q / dO row in LDS
@@ -310,6 +338,15 @@ __device__ __forceinline__ void attention_bwd_dkv_tile(const bf16_t* __restrict_
     const float scale_log2 = scale * kLog2e;
 
     const float kbias = key_bias ? key_bias[(int64_t)b * Lk + key_clamped] * kLog2e : 0.f;   // this lane's key
+    __amdgpu_buffer_rsrc_t pb_rsrc;
+    bool ex_bias = false, ex_drop = false;
+    if constexpr (EXTRA) {
+        ex_bias = ex->bias_qk != nullptr;
+        ex_drop = ex->keep_scale > 0.f;
+        // queries past L read as zeros (their probabilities are zeros anyway: lse = +inf)
+        pb_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(ex_bias ? ex->bias_qk + (int64_t)b * ex->bias_sb : nullptr),
+                                                    0, ex_bias ? (int)((int64_t)L * Lk * 4) : 0, 0x00020000);
+    }
     const bf16_t* kp = k + ((int64_t)(b * Hkv + hkv) * Lk + key_clamped) * D;
     bu32x4_t kf[KS];
 #pragma unroll
@@ -353,6 +390,7 @@ __device__ __forceinline__ void attention_bwd_dkv_tile(const bf16_t* __restrict_
         const bf16_t* obase = dout + (int64_t)b * L * (int64_t)(Hq * D) + hq * D;
         const float* lbase = lse + (int64_t)(b * Hq + hq) * L;
         const float* dbase = delta + (int64_t)(b * Hq + hq) * L;
+        const uint32_t head_key = EXTRA ? attn_head_key(ex->seed_lo, ex->seed_hi, (uint32_t)(b * Hq + hq)) : 0u;
         // buffer loads: query rows past L read as zeros
         const __amdgpu_buffer_rsrc_t q_rsrc =
             __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(qbase), 0, (int)((int64_t)L * D * 2), 0x00020000);
@@ -416,13 +454,28 @@ __device__ __forceinline__ void attention_bwd_dkv_tile(const bf16_t* __restrict_
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
                     const int x = r * 4 + j;
-                    float pv = __builtin_amdgcn_exp2f(__builtin_fmaf(acc_s[x], scale_log2, kbias - lv[j]));
+                    float kb_x = kbias, dp = acc_p[x], keep_mul = 1.0f;
+                    if constexpr (EXTRA) {
+                        const int qi = q0 + r * 8 + g * 4 + j;
+                        if (ex_bias)
+                            kb_x = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                                                                 pb_rsrc, (qi * Lk + key_clamped) * 4, 0, 0)) *
+                                   kLog2e;
+                        if (ex_drop) {
+                            keep_mul = attn_drop_hash(head_key, (uint32_t)qi * (uint32_t)Lk + (uint32_t)key_clamped) >=
+                                               ex->drop_threshold
+                                           ? ex->keep_scale
+                                           : 0.f;
+                            dp *= keep_mul;
+                        }
+                    }
+                    float pv = __builtin_amdgcn_exp2f(__builtin_fmaf(acc_s[x], scale_log2, kb_x - lv[j]));
                     if (diagonal) {
                         const int qi = q0 + r * 8 + g * 4 + j;
                         if (key_row > qi + off) pv = 0.f;
                     }
-                    p[j] = pv;
-                    ds[j] = pv * (acc_p[x] - dvv[j]) * scale;
+                    p[j] = pv * keep_mul;          // the weights that met V in the forward
+                    ds[j] = pv * (dp - dvv[j]) * scale;
                 }
                 // k-step s of the second products holds accumulator values 8s .. 8s+7
                 const unsigned p01 = pack_bf16x2(p[0], p[1]), p23 = pack_bf16x2(p[2], p[3]);
@@ -464,12 +517,12 @@ __device__ __forceinline__ void attention_bwd_dkv_tile(const bf16_t* __restrict_
 }
 
 // Early key tiles are seen by more queries than late ones: a workgroup takes tile j and tile n-1-j.
-template <int D>
+template <int D, bool EXTRA = false>
 __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const bf16_t* __restrict__ v,
     const bf16_t* __restrict__ dout, const float* __restrict__ lse, const float* __restrict__ delta,
     const float* __restrict__ key_bias, bf16_t* __restrict__ dk, bf16_t* __restrict__ dv, int Hq, int Hkv, int L, int Lk,
-    float scale) {
+    float scale, AttnExtra ex) {
     extern __shared__ __align__(16) unsigned char smem[];
     const int n_kt = (Lk + kBwdRows - 1) / kBwdRows;
     const int n_pairs = (n_kt + 1) / 2;
@@ -491,8 +544,8 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dkv_kernel(
 #pragma unroll 1
     for (int half = 0; half < 2; ++half) {
         if (half && pair == kt_far) break;
-        attention_bwd_dkv_tile<D>(q, k, v, dout, lse, delta, key_bias, dk, dv, Hq, Hkv, L, Lk, scale,
-                                  half ? kt_far : pair, hkv, b, smem);
+        attention_bwd_dkv_tile<D, EXTRA>(q, k, v, dout, lse, delta, key_bias, dk, dv, Hq, Hkv, L, Lk, scale,
+                                         half ? kt_far : pair, hkv, b, smem, &ex);
     }
 }
 
@@ -523,6 +576,14 @@ extern "C" int ats_attention_delta(const void* out, const void* dout, float* del
 extern "C" int ats_attention_bwd(const void* q, const void* k, const void* v, const void* dout, const float* lse,
                                  const float* delta, const float* key_bias, void* dq, void* dk, void* dv, int B, int Hq,
                                  int Hkv, int L, int Lk, int D, float scale, ats_stream_t stream) {
+    return ats_attention_bwd_ex(q, k, v, dout, lse, delta, key_bias, nullptr, 0, 0.f, 0, dq, dk, dv, B, Hq, Hkv, L, Lk, D,
+                                scale, stream);
+}
+
+extern "C" int ats_attention_bwd_ex(const void* q, const void* k, const void* v, const void* dout, const float* lse,
+                                    const float* delta, const float* key_bias, const float* bias_qk, int64_t bias_sb,
+                                    float dropout_p, uint64_t dropout_seed, void* dq, void* dk, void* dv, int B, int Hq,
+                                    int Hkv, int L, int Lk, int D, float scale, ats_stream_t stream) {
     using namespace ats;
     ATS_REQUIRE(B >= 0 && Hq > 0 && Hkv > 0 && Hq % Hkv == 0 && L >= 0 && Lk >= L && scale > 0.f, ATS_ERR_INVALID_ARG,
                 "ats_attention_bwd: B=%d Hq=%d Hkv=%d L=%d Lk=%d scale=%g", B, Hq, Hkv, L, Lk, scale);
@@ -544,6 +605,12 @@ extern "C" int ats_attention_bwd(const void* q, const void* k, const void* v, co
     const bf16_t* v_ = static_cast<const bf16_t*>(v);
     const bf16_t* do_ = static_cast<const bf16_t*>(dout);
     hipStream_t s = as_stream(stream);
+    AttnExtra ex;
+    bool extras = false;
+    if (!make_attention_extra("ats_attention_bwd_ex", bias_qk, bias_sb, dropout_p, dropout_seed, L, Lk, &ex, &extras))
+        return ATS_ERR_INVALID_ARG;
+    ATS_REQUIRE(!extras || key_bias == nullptr, ATS_ERR_INVALID_ARG,
+                "ats_attention_bwd_ex: with a pair bias or dropout the per-key bias must be folded into the pair bias");
     if (D == 128) {
         constexpr int smem_dq = 2 * kDqBN * (128 * 2 + 16) + kDqBN * (128 * 2 + 64) + kDqBN * 4;
         constexpr int smem_dkv = 2 * kDkvBQ * (128 * 2 + 16) + 2 * kDkvBQ * (128 * 2 + 64) + 2 * kDkvBQ * 4 +
@@ -552,26 +619,50 @@ extern "C" int ats_attention_bwd(const void* q, const void* k, const void* v, co
         hipError_t e = reserve_lds(reserved, {reinterpret_cast<const void*>(attention_bwd_dkv_kernel<128>)}, smem_dkv);
         ATS_REQUIRE(e == hipSuccess, ATS_ERR_LAUNCH, "ats_attention_bwd: cannot reserve %d bytes of LDS: %s", smem_dkv,
                     hipGetErrorString(e));
-        if (key_bias)
-            hipLaunchKernelGGL((attention_bwd_dq_kernel<128, true>), dim3((unsigned)dq_blocks), dim3(256), smem_dq, s, q_,
-                               k_, v_, do_, lse, delta, key_bias, static_cast<bf16_t*>(dq), Hq, Hkv, L, Lk, scale, B);
-        else
-            hipLaunchKernelGGL((attention_bwd_dq_kernel<128, false>), dim3((unsigned)dq_blocks), dim3(256), smem_dq, s, q_,
-                               k_, v_, do_, lse, delta, key_bias, static_cast<bf16_t*>(dq), Hq, Hkv, L, Lk, scale, B);
-        hipLaunchKernelGGL((attention_bwd_dkv_kernel<128>), dim3((unsigned)dkv_blocks), dim3(256), smem_dkv, s, q_, k_, v_,
-                           do_, lse, delta, key_bias, static_cast<bf16_t*>(dk), static_cast<bf16_t*>(dv), Hq, Hkv, L, Lk, scale);
+        if (extras) {
+            static LdsReservation reserved_x;
+            e = reserve_lds(reserved_x, {reinterpret_cast<const void*>(attention_bwd_dkv_kernel<128, true>)}, smem_dkv);
+            ATS_REQUIRE(e == hipSuccess, ATS_ERR_LAUNCH, "ats_attention_bwd_ex: cannot reserve %d bytes of LDS: %s", smem_dkv,
+                        hipGetErrorString(e));
+            hipLaunchKernelGGL((attention_bwd_dq_kernel<128, false, true>), dim3((unsigned)dq_blocks), dim3(256), smem_dq, s,
+                               q_, k_, v_, do_, lse, delta, key_bias, static_cast<bf16_t*>(dq), Hq, Hkv, L, Lk, scale, B, ex);
+            hipLaunchKernelGGL((attention_bwd_dkv_kernel<128, true>), dim3((unsigned)dkv_blocks), dim3(256), smem_dkv, s, q_,
+                               k_, v_, do_, lse, delta, key_bias, static_cast<bf16_t*>(dk), static_cast<bf16_t*>(dv), Hq, Hkv,
+                               L, Lk, scale, ex);
+        } else {
+            if (key_bias)
+                hipLaunchKernelGGL((attention_bwd_dq_kernel<128, true>), dim3((unsigned)dq_blocks), dim3(256), smem_dq, s,
+                                   q_, k_, v_, do_, lse, delta, key_bias, static_cast<bf16_t*>(dq), Hq, Hkv, L, Lk, scale, B,
+                                   ex);
+            else
+                hipLaunchKernelGGL((attention_bwd_dq_kernel<128, false>), dim3((unsigned)dq_blocks), dim3(256), smem_dq, s,
+                                   q_, k_, v_, do_, lse, delta, key_bias, static_cast<bf16_t*>(dq), Hq, Hkv, L, Lk, scale, B,
+                                   ex);
+            hipLaunchKernelGGL((attention_bwd_dkv_kernel<128>), dim3((unsigned)dkv_blocks), dim3(256), smem_dkv, s, q_, k_,
+                               v_, do_, lse, delta, key_bias, static_cast<bf16_t*>(dk), static_cast<bf16_t*>(dv), Hq, Hkv, L,
+                               Lk, scale, ex);
+        }
     } else {
         constexpr int smem_dq = 2 * kDqBN * (64 * 2 + 16) + kDqBN * (64 * 2 + 64) + kDqBN * 4;
         constexpr int smem_dkv = 2 * kDkvBQ * (64 * 2 + 16) + 2 * kDkvBQ * (64 * 2 + 64) + 2 * kDkvBQ * 4 +
                                  kBwdRows * (64 * 2 + 16);
-        if (key_bias)
-            hipLaunchKernelGGL((attention_bwd_dq_kernel<64, true>), dim3((unsigned)dq_blocks), dim3(256), smem_dq, s, q_,
-                               k_, v_, do_, lse, delta, key_bias, static_cast<bf16_t*>(dq), Hq, Hkv, L, Lk, scale, B);
-        else
-            hipLaunchKernelGGL((attention_bwd_dq_kernel<64, false>), dim3((unsigned)dq_blocks), dim3(256), smem_dq, s, q_,
-                               k_, v_, do_, lse, delta, key_bias, static_cast<bf16_t*>(dq), Hq, Hkv, L, Lk, scale, B);
-        hipLaunchKernelGGL((attention_bwd_dkv_kernel<64>), dim3((unsigned)dkv_blocks), dim3(256), smem_dkv, s, q_, k_, v_,
-                           do_, lse, delta, key_bias, static_cast<bf16_t*>(dk), static_cast<bf16_t*>(dv), Hq, Hkv, L, Lk, scale);
+        if (extras) {
+            hipLaunchKernelGGL((attention_bwd_dq_kernel<64, false, true>), dim3((unsigned)dq_blocks), dim3(256), smem_dq, s,
+                               q_, k_, v_, do_, lse, delta, key_bias, static_cast<bf16_t*>(dq), Hq, Hkv, L, Lk, scale, B, ex);
+            hipLaunchKernelGGL((attention_bwd_dkv_kernel<64, true>), dim3((unsigned)dkv_blocks), dim3(256), smem_dkv, s, q_,
+                               k_, v_, do_, lse, delta, key_bias, static_cast<bf16_t*>(dk), static_cast<bf16_t*>(dv), Hq, Hkv,
+                               L, Lk, scale, ex);
+        } else {
+            if (key_bias)
+                hipLaunchKernelGGL((attention_bwd_dq_kernel<64, true>), dim3((unsigned)dq_blocks), dim3(256), smem_dq, s, q_,
+                                   k_, v_, do_, lse, delta, key_bias, static_cast<bf16_t*>(dq), Hq, Hkv, L, Lk, scale, B, ex);
+            else
+                hipLaunchKernelGGL((attention_bwd_dq_kernel<64, false>), dim3((unsigned)dq_blocks), dim3(256), smem_dq, s, q_,
+                                   k_, v_, do_, lse, delta, key_bias, static_cast<bf16_t*>(dq), Hq, Hkv, L, Lk, scale, B, ex);
+            hipLaunchKernelGGL((attention_bwd_dkv_kernel<64>), dim3((unsigned)dkv_blocks), dim3(256), smem_dkv, s, q_, k_, v_,
+                               do_, lse, delta, key_bias, static_cast<bf16_t*>(dk), static_cast<bf16_t*>(dv), Hq, Hkv, L, Lk,
+                               scale, ex);
+        }
     }
     ATS_CHECK_LAUNCH("ats_attention_bwd");
     return ATS_OK;

@@ -163,8 +163,11 @@ class GroupedQueryAttention(nn.Module):
     (MS/core/model.py:561-731).  Projections run through the grouped GEMM kernels (one group), RoPE and the
     attention itself through their HIP kernels; the score matrix is never materialised.  Built: gradients of
     every input and parameter, past_key_value / use_cache (model.py:700-708; the cache grows in place),
-    attention_mask [batch, keys] (model.py:819-824).  Not built (AtsError): per-query 4-D masks, attention
-    dropout in training mode (config.dropout > 0, model.py:622-623, 831-833), float32 inputs."""
+    attention_mask [batch, keys] or [batch, 1, queries, keys] (model.py:819-824), attention dropout in training
+    mode (config.dropout > 0, model.py:622-623, 831-833: the mask is a hash of a per-call seed drawn from
+    torch's seed and a call counter, not torch's generator stream).  Not built (AtsError): float32 inputs."""
+
+    _instances = 0      # construction order: the layers of a model draw different dropout masks
 
     def __init__(self, config):
         super().__init__()
@@ -193,8 +196,11 @@ class GroupedQueryAttention(nn.Module):
         # per-call bookkeeping lives in one dict that is mutated in place: assigning module attributes on every
         # call goes through nn.Module.__setattr__, a visible part of a decoding step
         #   kv: addresses and fill of the cache buffers handed out last (no tensor is held)
+        #   dropout_stream: tells the layers of a model apart (id-based, fixed at construction)
         self._state: Dict[str, Any] = {"calls": 0, "kv": None, "kv_copies": 0, "kv_appends": 0, "qkv_key": None,
-                                       "qkv": None}
+                                       "qkv": None, "dropout_stream": GroupedQueryAttention._instances,
+                                       "last_dropout_seed": 0}
+        GroupedQueryAttention._instances += 1
 
     def forward(self, x: torch.Tensor, attention_mask: Optional[torch.Tensor] = None, past_key_value=None,
                 use_cache: bool = False):
@@ -202,8 +208,6 @@ class GroupedQueryAttention(nn.Module):
             raise AtsError(f"GroupedQueryAttention: expected [batch, seq, {self.hidden_size}], got {tuple(x.shape)}")
         if x.dtype != torch.bfloat16:
             raise AtsError(f"GroupedQueryAttention: the attention kernels are bfloat16 only, got {x.dtype}")
-        if self.training and self.dropout_p > 0:
-            raise AtsError("GroupedQueryAttention: attention dropout (config.dropout > 0 in training mode) is not built")
         B, L, H = x.shape
         nh, nkv, D = self.num_heads, self.num_kv_heads, self.head_dim
         x2 = x.reshape(B * L, H).contiguous()
@@ -233,18 +237,32 @@ class GroupedQueryAttention(nn.Module):
             else:
                 k = torch.cat([k_cache.to(k.dtype), k], dim=2)
                 v = torch.cat([v_cache.to(v.dtype), v], dim=2)
-        key_bias = None
+        key_bias = pair_bias = None
         if attention_mask is not None:
-            # [batch, keys] with 1 = real token, 0 = padding: (1 - mask) * -1e4 on that key's scores for
-            # every query and head (model.py:819-824)
-            if attention_mask.dim() != 2 or attention_mask.shape != (B, k.shape[2]):
-                raise AtsError(f"GroupedQueryAttention: attention_mask must be [batch, keys] = [{B}, {k.shape[2]}], got "
-                               f"{tuple(attention_mask.shape)} (per-query [batch, 1, seq, seq] masks are not built)")
-            key_bias = (1.0 - attention_mask.to(device=x.device, dtype=torch.float32)) * -1e4
+            # 1 = attend, 0 = masked: (1 - mask) * -1e4 is added to the scores (model.py:819-824), for every
+            # query and head with a [batch, keys] mask, per query with a [batch, 1, queries, keys] mask
+            Lk = k.shape[2]
+            m = attention_mask.to(device=x.device, dtype=torch.float32)
+            if m.dim() == 2 and m.shape == (B, Lk):
+                key_bias = (1.0 - m) * -1e4
+            elif m.dim() == 4 and m.shape[0] in (1, B) and m.shape[1] == 1 and m.shape[2] in (1, L) and m.shape[3] == Lk:
+                pair_bias = ((1.0 - m[:, 0]) * -1e4).expand(m.shape[0], L, Lk)
+            else:
+                raise AtsError(f"GroupedQueryAttention: attention_mask must be [batch, keys] = [{B}, {Lk}] or "
+                               f"[batch, 1, queries, keys] = [{B}, 1, {L}, {Lk}], got {tuple(attention_mask.shape)} "
+                               "(one mask per head is not built)")
+        drop_p, drop_seed = 0.0, 0
+        if self.training and self.dropout_p > 0:
+            # a fresh mask per call, reproducible under torch.manual_seed: no device round trip
+            drop_p = self.dropout_p
+            drop_seed = (torch.initial_seed() + 0x9E3779B97F4A7C15 * (self._state["calls"] + 1)
+                         + 0xD1B54A32D192ED03 * self._state["dropout_stream"]) & 0xFFFFFFFFFFFFFFFF
         if grad:
-            a = ag.AttentionFunction.apply(q, k, v, self.scale, key_bias)
+            a = ag.AttentionFunction.apply(q, k, v, self.scale, key_bias, pair_bias, drop_p, drop_seed)
         else:
-            a = ops.causal_attention(q, k, v, self.scale, key_bias=key_bias)
+            a = ops.causal_attention(q, k, v, self.scale, key_bias=key_bias, pair_bias=pair_bias, dropout_p=drop_p,
+                                     dropout_seed=drop_seed)
+        self._state["last_dropout_seed"] = drop_seed
         out = lin(a.view(B * L, nh * D), self.o_proj.weight).view(B, L, H)    # a: [B, L, nh*D]
         self._state["calls"] += 1
         if use_cache:

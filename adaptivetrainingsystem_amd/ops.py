@@ -739,14 +739,41 @@ def _key_bias(key_bias, B: int, Lk: int, q: torch.Tensor, who: str):
     return key_bias.contiguous()
 
 
+def _attention_extras(key_bias, pair_bias, dropout_p: float, B: int, L: int, Lk: int, q: torch.Tensor, who: str):
+    """Arguments of the extended entry points.  Returns (key_bias, pair_bias, batch stride): with a pair bias
+    or dropout a per-key bias is folded into the pair bias (the kernels take one or the other)."""
+    key_bias = _key_bias(key_bias, B, Lk, q, who)
+    if not 0.0 <= dropout_p < 1.0:
+        raise AtsError(f"{who}: dropout_p {dropout_p} must be in [0, 1)")
+    if pair_bias is not None:
+        if pair_bias.dim() != 3 or pair_bias.shape[0] not in (1, B) or tuple(pair_bias.shape[1:]) != (L, Lk) \
+                or pair_bias.dtype != torch.float32 or pair_bias.device != q.device:
+            raise AtsError(f"{who}: pair_bias must be float32 [batch or 1, queries, keys] = [{B}, {L}, {Lk}] on the "
+                           "inputs' device")
+        if key_bias is not None:
+            pair_bias = pair_bias + key_bias[:, None, :]
+            key_bias = None
+        pair_bias = pair_bias.contiguous()
+    elif dropout_p > 0.0 and key_bias is not None:
+        pair_bias = key_bias[:, None, :].expand(B, L, Lk).contiguous()
+        key_bias = None
+    stride = 0 if pair_bias is None or pair_bias.shape[0] == 1 else L * Lk
+    return key_bias, pair_bias, stride
+
+
 def causal_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: Optional[float] = None,
-                     return_lse: bool = False, key_bias: Optional[torch.Tensor] = None, split_keys: bool = True):
+                     return_lse: bool = False, key_bias: Optional[torch.Tensor] = None, split_keys: bool = True,
+                     pair_bias: Optional[torch.Tensor] = None, dropout_p: float = 0.0, dropout_seed: int = 0):
     """Causal grouped-query attention.  q [B,Hq,L,D]; k [B,Hkv,Lk,D] with a head's rows one after the other
     and any batch/head strides (e.g. a view of a larger cache buffer); v [B,Hkv,Lk,D] in any batch/head/position
     strides (e.g. a view of a fused projection output); bf16, D 64 or 128, Lk >= L.
     With Lk > L the leading Lk - L keys are a cache: query i sits at position i + Lk - L.
     key_bias [B, Lk] float32 (optional) is added to the scaled scores of a key for every query and head;
     (1 - attention_mask) * -1e4 is the reference's padding mask (MS/core/model.py:819-824).
+    pair_bias [B or 1, L, Lk] float32 (optional) is added to the scaled scores of a (query, key) pair for
+    every head: (1 - mask[:, 0]) * -1e4 for the reference's [B,1,L,Lk] masks (same lines).
+    dropout_p > 0 drops attention weights (model.py:831-833) by a hash of (dropout_seed, batch, head, query,
+    key); causal_attention_bwd given the same seed sees the same mask.
     split_keys=False keeps the single-pass kernel where few rows against many keys would otherwise be cut
     into key ranges.  Returns out [B, L, Hq*D] (and lse [B,Hq,L] float32 if asked)."""
     _need_gpu(q, k, v)
@@ -759,7 +786,7 @@ def causal_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: O
     q = q.contiguous()
     if k.stride(3) != 1 or k.stride(2) != D or k.stride(0) % 8 or k.stride(1) % 8 or k.data_ptr() % 16:
         k = k.contiguous()        # rows of a head must follow one another; batch and head strides are free
-    key_bias = _key_bias(key_bias, B, Lk, q, "causal_attention")
+    key_bias, pair_bias, pair_stride = _attention_extras(key_bias, pair_bias, dropout_p, B, L, Lk, q, "causal_attention")
     if v.stride(3) != 1 or any(st % 8 for st in v.stride()[:3]) or v.stride(2) < D or v.data_ptr() % 16:
         v = v.contiguous()
     lib = _lib.load()
@@ -768,18 +795,20 @@ def causal_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: O
     # decoding a few sequences: scratch for the partial results of key ranges that run side by side
     ws_bytes = lib.ats_attention_fwd_workspace(B, Hq, Hkv, L, Lk, D) if split_keys else 0
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device) if ws_bytes else None
-    check(lib.ats_attention_fwd(q.data_ptr(), k.data_ptr(), k.stride(0), k.stride(1), v.data_ptr(), v.stride(0),
-                                v.stride(2), v.stride(1),
-                                _ptr(key_bias), out.data_ptr(), _ptr(lse), B, Hq, Hkv, L, Lk, D,
-                                float(D ** -0.5 if scale is None else scale), _ptr(ws), ws_bytes, _stream()),
-          "ats_attention_fwd")
+    check(lib.ats_attention_fwd_ex(q.data_ptr(), k.data_ptr(), k.stride(0), k.stride(1), v.data_ptr(), v.stride(0),
+                                   v.stride(2), v.stride(1), _ptr(key_bias), _ptr(pair_bias), pair_stride,
+                                   float(dropout_p), int(dropout_seed) & 0xFFFFFFFFFFFFFFFF, out.data_ptr(), _ptr(lse),
+                                   B, Hq, Hkv, L, Lk, D, float(D ** -0.5 if scale is None else scale), _ptr(ws),
+                                   ws_bytes, _stream()),
+          "ats_attention_fwd_ex")
     return (out, lse) if return_lse else out
 
 
 def causal_attention_bwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Tensor, lse: torch.Tensor,
-                         dout: torch.Tensor, scale: Optional[float] = None, key_bias: Optional[torch.Tensor] = None):
+                         dout: torch.Tensor, scale: Optional[float] = None, key_bias: Optional[torch.Tensor] = None,
+                         pair_bias: Optional[torch.Tensor] = None, dropout_p: float = 0.0, dropout_seed: int = 0):
     """Gradients of causal_attention: q [B,Hq,L,D], k, v [B,Hkv,Lk,D], out, dout [B,L,Hq*D], lse [B,Hq,L],
-    key_bias as in the forward.  Returns (dq, dk, dv) shaped like q, k, v."""
+    key_bias, pair_bias, dropout_p and dropout_seed as in the forward.  Returns (dq, dk, dv) shaped like q, k, v."""
     _need_gpu(q, k, v, out, lse, dout)
     B, Hq, L, D = q.shape
     Hkv, Lk = k.shape[1], k.shape[2]
@@ -789,16 +818,18 @@ def causal_attention_bwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out:
     q, k, v, out = q.contiguous(), k.contiguous(), v.contiguous(), out.contiguous()
     dout = dout.to(q.dtype).contiguous()
     lse = lse.contiguous()
-    key_bias = _key_bias(key_bias, B, Lk, q, "causal_attention_bwd")
+    key_bias, pair_bias, pair_stride = _attention_extras(key_bias, pair_bias, dropout_p, B, L, Lk, q,
+                                                         "causal_attention_bwd")
     lib = _lib.load()
     delta = torch.empty(B, Hq, L, dtype=torch.float32, device=q.device)
     check(lib.ats_attention_delta(out.data_ptr(), dout.data_ptr(), delta.data_ptr(), B, Hq, L, D, _stream()),
           "ats_attention_delta")
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
-    check(lib.ats_attention_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), dout.data_ptr(), lse.data_ptr(),
-                                delta.data_ptr(), _ptr(key_bias), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), B, Hq, Hkv,
-                                L, Lk, D,
-                                float(D ** -0.5 if scale is None else scale), _stream()), "ats_attention_bwd")
+    check(lib.ats_attention_bwd_ex(q.data_ptr(), k.data_ptr(), v.data_ptr(), dout.data_ptr(), lse.data_ptr(),
+                                   delta.data_ptr(), _ptr(key_bias), _ptr(pair_bias), pair_stride, float(dropout_p),
+                                   int(dropout_seed) & 0xFFFFFFFFFFFFFFFF, dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
+                                   B, Hq, Hkv, L, Lk, D, float(D ** -0.5 if scale is None else scale), _stream()),
+          "ats_attention_bwd_ex")
     return dq, dk, dv
 
 

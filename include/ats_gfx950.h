@@ -351,6 +351,21 @@ int ats_attention_fwd(const void* q, const void* k, int64_t k_sb, int64_t k_sh, 
                       int64_t v_sl, int64_t v_sh, const float* key_bias, void* out, float* lse, int B, int Hq,
                       int Hkv, int L, int Lk, int D, float scale, void* workspace, size_t workspace_bytes,
                       ats_stream_t stream);
+/* The same with the two options of the reference's masked path that the plain entry point leaves out
+ * (model.py:819-833):
+ *   bias_qk (optional): float32 [B, L, Lk], added to the scaled scores of (query, key) for every head; a
+ *     [B,1,L,Lk] attention mask is (1 - mask) * -1e4.  bias_sb = floats between two batch entries' matrices
+ *     (0: one matrix for the whole batch).
+ *   dropout_p in [0, 1): each attention weight is dropped with this probability and the kept ones are scaled
+ *     by 1 / (1 - p) before they meet V (nn.Dropout on the weights while training); the log-sum-exp is that of
+ *     the undropped scores.  Keep / drop is a function of (dropout_seed, batch, head, query, key) only, so
+ *     ats_attention_bwd_ex given the same seed sees the same mask; it is not torch's generator stream.
+ * With either option a per-key bias must be folded into bias_qk by the caller (key_bias must be NULL), and the
+ * single-pass kernel without the software pipeline runs.  Neither option set: identical to ats_attention_fwd. */
+int ats_attention_fwd_ex(const void* q, const void* k, int64_t k_sb, int64_t k_sh, const void* v, int64_t v_sb,
+                         int64_t v_sl, int64_t v_sh, const float* key_bias, const float* bias_qk, int64_t bias_sb,
+                         float dropout_p, uint64_t dropout_seed, void* out, float* lse, int B, int Hq, int Hkv, int L,
+                         int Lk, int D, float scale, void* workspace, size_t workspace_bytes, ats_stream_t stream);
 
 /* ---- Causal grouped-query attention (backward) ----------------------------------
  * The reference leaves this gradient to autograd (model.py:757-839 under torch.autograd); the kernels
@@ -365,6 +380,12 @@ int ats_attention_delta(const void* out, const void* dout, float* delta, int B, 
 int ats_attention_bwd(const void* q, const void* k, const void* v, const void* dout, const float* lse,
                       const float* delta, const float* key_bias, void* dq, void* dk, void* dv, int B, int Hq, int Hkv,
                       int L, int Lk, int D, float scale, ats_stream_t stream);
+/* Backward with the options of ats_attention_fwd_ex (same bias_qk, dropout_p and dropout_seed as the forward
+ * call whose lse is passed; delta from ats_attention_delta on the forward's output as usual). */
+int ats_attention_bwd_ex(const void* q, const void* k, const void* v, const void* dout, const float* lse,
+                         const float* delta, const float* key_bias, const float* bias_qk, int64_t bias_sb,
+                         float dropout_p, uint64_t dropout_seed, void* dq, void* dk, void* dv, int B, int Hq, int Hkv,
+                         int L, int Lk, int D, float scale, ats_stream_t stream);
 
 /* ---- Training-step ops beside the sparse layer --------------------------------
  * Fused cross-entropy + accuracy.  Replaces fused_cross_entropy_accuracy_launcher

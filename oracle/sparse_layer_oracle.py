@@ -61,7 +61,10 @@ PINNING = {
     "swiglu_backward": "torch.autograd of gate*silu(up) in float64; gradcheck",
     "fused_loss": "float64 logsumexp closed form; uniform logits give log(V); torch.autograd for the gradient",
     "clip_grad_norm": "closed form sqrt(sum of squares) and scaling by max_norm/(norm+1e-6)",
-    "attention_standard": "float64 brute force per query (explicit loop over allowed keys); F.scaled_dot_product_attention(is_causal=True)",
+    "attention_standard": "float64 brute force per query (explicit loop over allowed keys); F.scaled_dot_product_attention(is_causal=True); "
+                          "4-D masks and the explicit dropout mask against a float64 sum written out per element",
+    "attention_dropout_keep": "published values of MurmurHash3's fmix32 (0, 1, 2) on both sides of their thresholds; keep rate within "
+                              "4 sigma; zero correlation between seeds, heads, batch entries and neighbouring elements",
     "gqa_forward": "composition of pinned parts; equals per-head attention with repeat_interleave done by hand",
     "layer_grads": "is torch.autograd over the forward restatements above (what the reference itself trains with); "
                    "gradcheck in float64 on the no-capacity layer with fixed routing",
@@ -516,8 +519,8 @@ def clip_grad_norm(grads, max_norm: float):
 
 # --------------------------------------------------------------------------- attention
 def attention_standard(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: float,
-                       attention_mask=None) -> torch.Tensor:
-    """MS/core/model.py:757-838 (GroupedQueryAttention._standard_attention, no dropout).
+                       attention_mask=None, dropout_keep=None, dropout_p: float = 0.0) -> torch.Tensor:
+    """MS/core/model.py:757-838 (GroupedQueryAttention._standard_attention).
     q [B,H,L,D], k/v [B,H,Lk,D] (already expanded to H heads), Lk >= L.  Scores and softmax in float32,
     causal positions filled with -1e4, probabilities cast to the input dtype before the second matmul,
     output [B, L, H*D] in the input dtype.
@@ -525,19 +528,51 @@ def attention_standard(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale:
     reference's own [L, L] mask only broadcasts against [L, Lk] scores for L = 1 (one new token, which
     then sees every key); the diagonal used here is that case's generalisation, and equals what slicing
     the last L query rows out of a full-length call gives.
-    attention_mask [B, Lk] (1 = real key, 0 = padding) adds (1 - mask) * -1e4 to every query's and head's
-    scores of a key (model.py:819-824), after the causal fill."""
+    attention_mask (1 = attend, 0 = masked) adds (1 - mask) * -1e4 to the scores after the causal fill
+    (model.py:819-824): [B, Lk] for every query and head (unsqueezed as there), or 4-D [B, 1, L, Lk] as given.
+    dropout_keep [B,H,L,Lk] bool with dropout_p: nn.Dropout on the weights (model.py:831-833) with the mask
+    made explicit: kept weights are scaled by 1 / (1 - p), the others are zero."""
     B, H, L, D = q.shape
     Lk = k.shape[2]
     scores = torch.matmul(q.float(), k.float().transpose(-2, -1)) * scale
     causal = torch.triu(torch.ones(L, Lk, dtype=torch.bool), diagonal=1 + Lk - L)
     scores = scores.masked_fill(causal, -1e4)
     if attention_mask is not None:
-        scores = scores + (1.0 - attention_mask.float()[:, None, None, :]) * -1e4
+        m = attention_mask.float()
+        if m.dim() == 2:
+            m = m[:, None, None, :]
+        scores = scores + (1.0 - m) * -1e4
     scores = scores - scores.detach().amax(dim=-1, keepdim=True)
     w = F.softmax(scores, dim=-1, dtype=torch.float32).to(q.dtype)
+    if dropout_keep is not None:
+        w = (w.float() * dropout_keep.to(torch.float32) / (1.0 - dropout_p)).to(q.dtype)
     out = torch.matmul(w.float(), v.float()).to(q.dtype)
     return out.transpose(1, 2).reshape(B, L, H * D)
+
+
+def attention_dropout_keep(seed: int, B: int, H: int, L: int, Lk: int, dropout_p: float) -> torch.Tensor:
+    """The keep / drop decision of the HIP attention kernels' dropout as a bool tensor [B, H, L, Lk].  No
+    counterpart in the reference (nn.Dropout draws from torch's generator, which a tiled kernel cannot
+    replay): element (b, h, i, j) is kept iff fmix32((i * Lk + j) ^ head_key(seed, b * H + h)) >= p * 2^32,
+    fmix32 the finaliser of MurmurHash3 (csrc/attention_extra.hpp states the same function for the device)."""
+    M = 0xFFFFFFFF
+    seed &= 0xFFFFFFFFFFFFFFFF
+    lo, hi = seed & M, seed >> 32
+    bh = np.arange(B * H, dtype=np.uint64)
+    x = (np.uint64(lo) ^ ((bh * np.uint64(0x9E3779B1)) & np.uint64(M))) & np.uint64(M)
+    x ^= x >> np.uint64(15)
+    x = (x * np.uint64(0x2C1B3C6D)) & np.uint64(M)
+    x ^= np.uint64(hi)
+    x ^= x >> np.uint64(12)
+    y = (np.arange(L * Lk, dtype=np.uint64)[None, :] & np.uint64(M)) ^ x[:, None]
+    y ^= y >> np.uint64(16)
+    y = (y * np.uint64(0x85EBCA6B)) & np.uint64(M)
+    y ^= y >> np.uint64(13)
+    y = (y * np.uint64(0xC2B2AE35)) & np.uint64(M)
+    y ^= y >> np.uint64(16)
+    t = dropout_p * 4294967296.0
+    threshold = M if t >= 4294967295.0 else int(t)
+    return torch.from_numpy((y >= np.uint64(threshold)).reshape(B, H, L, Lk))
 
 
 def gqa_forward(x: torch.Tensor, wq: torch.Tensor, wk: torch.Tensor, wv: torch.Tensor, wo: torch.Tensor,

@@ -527,3 +527,157 @@ def test_transformer_block_moe_composition_and_patterns(gpu):
     assert sel("every_3rd") == [2, 5] and sel("every_4th") == [3, 7]
     assert sel("sandwich") == [2, 3, 4, 5] and sel("sandwich", dense_start_layers=1, dense_end_layers=3) == [1, 2, 3, 4]
     assert sel(lambda i, n: i % 2 == 0) == [0, 2, 4, 6]
+
+
+# --------------------------------------------------------------------------- per-query masks and dropout
+def _pair_mask(B, L, Lk, seed, p_zero=0.3):
+    """[B, 1, L, Lk] of ones and zeros in which every query keeps its own position (so no row is masked out
+    entirely: a fully masked row falls back on the -1e4 constants, which float32 scores cannot resolve)."""
+    m = (torch.rand(B, 1, L, Lk, generator=gen(seed)) >= p_zero).float()
+    i = torch.arange(L)
+    m[:, 0, i, i + (Lk - L)] = 1.0
+    return m
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,L,Lk,D", [(2, 4, 2, 200, 200, 128), (1, 8, 2, 300, 300, 64), (1, 1, 1, 1, 1, 128),
+                                             (2, 3, 3, 129, 129, 64), (1, 4, 1, 520, 520, 128), (2, 4, 2, 70, 300, 64),
+                                             (1, 2, 1, 31, 31, 64), (1, 2, 2, 130, 131, 128)])
+def test_causal_attention_pair_mask(ops, gpu, B, Hq, Hkv, L, Lk, D):
+    """[B, 1, L, Lk] masks (model.py:819-824 with a 4-D mask): forward, log-sum-exp and the three gradients
+    against the oracle and autograd over it; a 4-D mask that repeats a [B, Lk] mask for every query gives what
+    the per-key path gives; one matrix shared by the batch."""
+    print("case attention pair mask", B, Hq, Hkv, L, Lk, D, flush=True)
+    g = gen(131)
+    q = torch.randn(B, Hq, L, D, generator=g).bfloat16()
+    k = torch.randn(B, Hkv, Lk, D, generator=g).bfloat16()
+    v = torch.randn(B, Hkv, Lk, D, generator=g).bfloat16()
+    dout = torch.randn(B, L, Hq * D, generator=g).bfloat16()
+    mask = _pair_mask(B, L, Lk, 132)
+    rep = Hq // Hkv
+    q32, k32, v32 = (t.float().requires_grad_() for t in (q, k, v))
+    ref = O.attention_standard(q32, k32.repeat_interleave(rep, dim=1), v32.repeat_interleave(rep, dim=1), D ** -0.5, mask)
+    ref.backward(dout.float())
+    bias = ((1.0 - mask[:, 0]) * -1e4).to(gpu)
+    qg, kg, vg = q.to(gpu), k.to(gpu), v.to(gpu)
+    out, lse = ops.causal_attention(qg, kg, vg, return_lse=True, pair_bias=bias)
+    assert rel_err(out, ref) <= BF16_TOL
+    s = torch.matmul(q.float(), k.repeat_interleave(rep, dim=1).float().transpose(-2, -1)) * D ** -0.5
+    s = s.masked_fill(torch.triu(torch.ones(L, Lk, dtype=torch.bool), diagonal=1 + Lk - L), float("-inf"))
+    assert rel_err(lse, torch.logsumexp(s + (1.0 - mask) * -1e4, -1)) <= 1e-4
+    dq, dk, dv = ops.causal_attention_bwd(qg, kg, vg, out, lse, dout.to(gpu), pair_bias=bias)
+    assert rel_err(dv, v32.grad) <= GRAD_TOL
+    assert rel_err(dq, q32.grad) <= GRAD_TOL
+    assert rel_err(dk, k32.grad) <= GRAD_TOL
+    # the per-key mask written as a 4-D mask, alone and on top of a per-key bias
+    pad = _padding_mask(B, Lk, 133)
+    pad[:, :Lk - L + 1] = 1
+    kb = ((1.0 - pad) * -1e4).to(gpu)
+    per_key = ops.causal_attention(qg, kg, vg, key_bias=kb)
+    as_pair = ops.causal_attention(qg, kg, vg, pair_bias=kb[:, None, :].expand(B, L, Lk).contiguous())
+    assert rel_err(as_pair, per_key) <= 1e-2
+    both = ops.causal_attention(qg, kg, vg, key_bias=kb, pair_bias=torch.zeros(1, L, Lk, device=gpu))
+    assert torch.equal(both, as_pair)
+    # one matrix for the whole batch
+    shared = ops.causal_attention(qg, kg, vg, pair_bias=bias[:1])
+    assert torch.equal(shared[:1], out[:1])
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,L,Lk,D,p", [(2, 4, 2, 200, 200, 128, 0.25), (1, 8, 2, 300, 300, 64, 0.1),
+                                               (2, 3, 3, 129, 129, 64, 0.5), (1, 4, 1, 520, 520, 128, 0.3),
+                                               (2, 4, 2, 70, 300, 64, 0.25), (1, 2, 1, 31, 31, 64, 0.9)])
+def test_causal_attention_dropout(ops, gpu, B, Hq, Hkv, L, Lk, D, p):
+    """Dropout on the attention weights (model.py:831-833).  The kernels' keep / drop decisions are a function of
+    (seed, batch, head, query, key) that the oracle restates on the CPU; with that mask made explicit the
+    oracle's forward and autograd over it are the reference for output and gradients.  The log-sum-exp is that
+    of the undropped scores; another seed gives another mask; p = 0 is the plain kernel's result."""
+    print("case attention dropout", B, Hq, Hkv, L, Lk, D, p, flush=True)
+    g = gen(141)
+    q = torch.randn(B, Hq, L, D, generator=g).bfloat16()
+    k = torch.randn(B, Hkv, Lk, D, generator=g).bfloat16()
+    v = torch.randn(B, Hkv, Lk, D, generator=g).bfloat16()
+    dout = torch.randn(B, L, Hq * D, generator=g).bfloat16()
+    seed = 0x5DEECE66D1234567
+    keep = O.attention_dropout_keep(seed, B, Hq, L, Lk, p)
+    rep = Hq // Hkv
+    q32, k32, v32 = (t.float().requires_grad_() for t in (q, k, v))
+    ref = O.attention_standard(q32, k32.repeat_interleave(rep, dim=1), v32.repeat_interleave(rep, dim=1), D ** -0.5,
+                               dropout_keep=keep, dropout_p=p)
+    ref.backward(dout.float())
+    qg, kg, vg = q.to(gpu), k.to(gpu), v.to(gpu)
+    out, lse = ops.causal_attention(qg, kg, vg, return_lse=True, dropout_p=p, dropout_seed=seed)
+    assert rel_err(out, ref) <= BF16_TOL
+    plain, lse_plain = ops.causal_attention(qg, kg, vg, return_lse=True)
+    assert rel_err(lse, lse_plain) <= 1e-5
+    dq, dk, dv = ops.causal_attention_bwd(qg, kg, vg, out, lse, dout.to(gpu), dropout_p=p, dropout_seed=seed)
+    assert rel_err(dv, v32.grad) <= GRAD_TOL
+    assert rel_err(dq, q32.grad) <= GRAD_TOL
+    assert rel_err(dk, k32.grad) <= GRAD_TOL
+    other = ops.causal_attention(qg, kg, vg, dropout_p=p, dropout_seed=seed + 1)
+    if L > 1:
+        assert not torch.equal(other, out)
+    assert torch.equal(ops.causal_attention(qg, kg, vg, dropout_p=p, dropout_seed=seed), out)      # reproducible
+    # with a padding mask on top (folded into the pair bias by the host)
+    pad = _padding_mask(B, Lk, 142)
+    pad[:, :Lk - L + 1] = 1
+    ref_m = O.attention_standard(q.float(), k.float().repeat_interleave(rep, dim=1),
+                                 v.float().repeat_interleave(rep, dim=1), D ** -0.5, pad, dropout_keep=keep, dropout_p=p)
+    out_m = ops.causal_attention(qg, kg, vg, key_bias=((1.0 - pad) * -1e4).to(gpu), dropout_p=p, dropout_seed=seed)
+    assert rel_err(out_m, ref_m) <= BF16_TOL
+
+
+def test_attention_extras_errors(ops, gpu):
+    q = torch.randn(1, 2, 8, 64, device=gpu).bfloat16()
+    from adaptivetrainingsystem_amd._lib import AtsError
+    with pytest.raises(AtsError):
+        ops.causal_attention(q, q, q, dropout_p=1.0)
+    with pytest.raises(AtsError):
+        ops.causal_attention(q, q, q, pair_bias=torch.zeros(1, 8, 9, device=gpu))
+    with pytest.raises(AtsError):
+        ops.causal_attention(q, q, q, pair_bias=torch.zeros(1, 8, 8, device=gpu, dtype=torch.float64))
+
+
+def test_gqa_module_pair_mask_and_dropout(gpu):
+    """GroupedQueryAttention with a [B, 1, L, L] mask and with config.dropout > 0 in training mode, against the
+    oracle's gqa_forward / attention_standard (model.py:663-731, 819-833)."""
+    from types import SimpleNamespace
+    from adaptivetrainingsystem_amd.layers import GroupedQueryAttention
+    from adaptivetrainingsystem_amd._lib import AtsError
+    hidden, nh, nkv, B, L = 256, 4, 2, 2, 96
+    torch.manual_seed(5)
+    cfg = SimpleNamespace(hidden_size=hidden, num_heads=nh, num_kv_heads=nkv, seq_length=256, dropout=0.2)
+    att = GroupedQueryAttention(cfg).to(gpu).bfloat16()
+    w = [getattr(att, n).weight.detach().cpu() for n in ("q_proj", "k_proj", "v_proj", "o_proj")]
+    x = torch.randn(B, L, hidden, generator=gen(151)).bfloat16()
+    mask = _pair_mask(B, L, L, 152)
+    att.eval()
+    with torch.no_grad():
+        out = att(x.to(gpu), attention_mask=mask.to(gpu))
+    assert rel_err(out, O.gqa_forward(x, *w, nh, nkv, attention_mask=mask)) <= BF16_TOL
+    with pytest.raises(AtsError):
+        att(x.to(gpu), attention_mask=torch.ones(B, nh, L, L, device=gpu))      # one mask per head
+    # eval mode: dropout is off (model.py:832)
+    with torch.no_grad():
+        plain = att(x.to(gpu))
+    assert rel_err(plain, O.gqa_forward(x, *w, nh, nkv)) <= BF16_TOL
+    # training mode: a fresh mask per call, the one the recorded seed describes
+    att.train()
+    with torch.no_grad():
+        d1 = att(x.to(gpu))
+        seed1 = att._state["last_dropout_seed"]
+        d2 = att(x.to(gpu))
+    assert not torch.equal(d1, d2) and not torch.equal(d1, plain)
+    D = hidden // nh
+    keep = O.attention_dropout_keep(seed1, B, nh, L, L, 0.2)
+    lin = lambda a, m: torch.nn.functional.linear(a.float(), m.float()).to(a.dtype)
+    qh = lin(x, w[0]).view(B, L, nh, D).transpose(1, 2)
+    kh = lin(x, w[1]).view(B, L, nkv, D).transpose(1, 2)
+    vh = lin(x, w[2]).view(B, L, nkv, D).transpose(1, 2)
+    cos, sin = O.rope_table(L, D, 10000.0)
+    qh, kh = O.rope_apply(qh, kh, cos, sin)
+    a = O.attention_standard(qh, kh.repeat_interleave(nh // nkv, dim=1), vh.repeat_interleave(nh // nkv, dim=1), D ** -0.5,
+                             dropout_keep=keep, dropout_p=0.2)
+    assert rel_err(d1, lin(a, w[3]).view(B, L, hidden)) <= BF16_TOL
+    # gradients flow through the dropped attention
+    xg = x.to(gpu).requires_grad_()
+    att(xg).float().sum().backward()
+    assert xg.grad is not None and torch.isfinite(xg.grad).all() and att.q_proj.weight.grad is not None

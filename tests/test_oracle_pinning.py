@@ -752,3 +752,78 @@ def test_every_oracle_function_declares_its_pin():
     fns = [n for n, f in inspect.getmembers(O, inspect.isfunction) if f.__module__ == O.__name__]
     assert sorted(fns) == sorted(O.PINNING), set(fns) ^ set(O.PINNING)
     assert not [n for n, why in O.PINNING.items() if "unpinned" in why]
+
+
+def test_attention_standard_pair_mask_and_dropout():
+    """The 4-D mask and the explicit dropout mask of the oracle's attention against a float64 sum written out
+    per element (additive -1e4 constants, weights scaled by keep / (1 - p)); a 4-D mask that repeats a
+    [B, Lk] mask gives the 2-D path's result; keep-all with p = 0 changes nothing; keep-all with p scales the
+    output by 1 / (1 - p)."""
+    g = torch.Generator().manual_seed(87)
+    B, H, L, Lk, D = 2, 3, 7, 9, 8
+    q = torch.randn(B, H, L, D, generator=g)
+    k = torch.randn(B, H, Lk, D, generator=g)
+    v = torch.randn(B, H, Lk, D, generator=g)
+    scale = D ** -0.5
+    mask = (torch.rand(B, 1, L, Lk, generator=g) > 0.4).float()
+    i = torch.arange(L)
+    mask[:, 0, i, i + Lk - L] = 1
+    keep = torch.rand(B, H, L, Lk, generator=g) > 0.3
+    p = 0.3
+    out = O.attention_standard(q, k, v, scale, mask, dropout_keep=keep, dropout_p=p).view(B, L, H, D)
+    for b in range(B):
+        for h in range(H):
+            for qi in range(L):
+                s = []
+                for j in range(Lk):
+                    sc = float(q[b, h, qi].double() @ k[b, h, j].double()) * scale
+                    if j > qi + Lk - L:
+                        sc = -1e4
+                    sc += (1.0 - float(mask[b, 0, qi, j])) * -1e4
+                    s.append(sc)
+                mx = max(s)
+                e = [math.exp(x - mx) for x in s]
+                tot = sum(e)
+                acc = torch.zeros(D, dtype=torch.float64)
+                for j in range(Lk):
+                    if keep[b, h, qi, j]:
+                        acc += (e[j] / tot / (1.0 - p)) * v[b, h, j].double()
+                assert torch.allclose(out[b, qi, h].double(), acc, atol=2e-5), (b, h, qi)
+    pad = torch.ones(B, Lk)
+    pad[0, 2] = 0
+    pad[1, 5:7] = 0
+    assert torch.allclose(O.attention_standard(q, k, v, scale, pad[:, None, None, :].expand(B, 1, L, Lk)),
+                          O.attention_standard(q, k, v, scale, pad), atol=1e-6)
+    ones = torch.ones(B, H, L, Lk, dtype=torch.bool)
+    base = O.attention_standard(q, k, v, scale)
+    assert torch.equal(O.attention_standard(q, k, v, scale, dropout_keep=ones, dropout_p=0.0), base)
+    assert torch.allclose(O.attention_standard(q, k, v, scale, dropout_keep=ones, dropout_p=0.5), base * 2.0, atol=1e-5)
+
+
+def test_attention_dropout_keep_known_answers_and_statistics():
+    """The keep / drop function: with seed 0 the (batch 0, head 0) key is 0, so element (query 0, key j) is
+    decided by MurmurHash3's finaliser of j, whose published values fmix32(0) = 0, fmix32(1) = 0x514e28b7,
+    fmix32(2) = 0x30f4c306 fix the outcome on both sides of each threshold; the keep rate matches 1 - p within
+    4 sigma; masks of different seeds, heads and batch entries are uncorrelated; p = 0 keeps everything."""
+    for p, want in [(0.31, True), (0.32, False)]:       # 0x514e28b7 / 2^32 = 0.31760
+        assert bool(O.attention_dropout_keep(0, 1, 1, 1, 4, p)[0, 0, 0, 1]) == want
+    for p, want in [(0.19, True), (0.20, False)]:       # 0x30f4c306 / 2^32 = 0.19123
+        assert bool(O.attention_dropout_keep(0, 1, 1, 1, 4, p)[0, 0, 0, 2]) == want
+    assert not bool(O.attention_dropout_keep(0, 1, 1, 1, 4, 1e-9)[0, 0, 0, 0])      # hash 0 < any threshold >= 1
+    assert bool(O.attention_dropout_keep(0, 2, 3, 5, 7, 0.0).all())
+    B, H, L, Lk = 2, 4, 128, 160
+    n = B * H * L * Lk
+    for p in (0.1, 0.5, 0.9):
+        m = O.attention_dropout_keep(12345, B, H, L, Lk, p).float()
+        assert abs(m.mean().item() - (1 - p)) <= 4 * math.sqrt(p * (1 - p) / n)
+        per_head = m.mean(dim=(2, 3))
+        assert (per_head - (1 - p)).abs().max().item() <= 5 * math.sqrt(p * (1 - p) / (L * Lk))
+    a = O.attention_dropout_keep(1, B, H, L, Lk, 0.5).float() - 0.5
+    b = O.attention_dropout_keep(2, B, H, L, Lk, 0.5).float() - 0.5
+    bound = 5 * 0.25 / math.sqrt(L * Lk)
+    assert abs((a * b).mean().item()) <= 5 * 0.25 / math.sqrt(n)
+    assert abs((a[0, 0] * a[0, 1]).mean().item()) <= bound and abs((a[0, 0] * a[1, 0]).mean().item()) <= bound
+    # neighbouring keys and neighbouring queries of one head
+    assert abs((a[..., :-1] * a[..., 1:]).mean().item()) <= 5 * 0.25 / math.sqrt(n)
+    assert abs((a[:, :, :-1] * a[:, :, 1:]).mean().item()) <= 5 * 0.25 / math.sqrt(n)
+    assert torch.equal(O.attention_dropout_keep(1, B, H, L, Lk, 0.5), O.attention_dropout_keep(1, B, H, L, Lk, 0.5))
