@@ -114,6 +114,27 @@ class AttentionFunction(Function):
         return dq, dk, dv, None, None, None, None, None
 
 
+class AttentionF32Function(Function):
+    """The float32 route of the attention (ops.attention_f32): same arguments as AttentionFunction; the softmax
+    weights are kept for the backward, as autograd keeps them for the reference."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, scale, key_bias=None, pair_bias=None, dropout_p=0.0, dropout_seed=0):
+        out, state = ops.attention_f32(q, k, v, scale, key_bias=key_bias, pair_bias=pair_bias, dropout_p=dropout_p,
+                                       dropout_seed=dropout_seed, return_weights=True)
+        w, w_drop, qp, kp, vp = state
+        ctx.save_for_backward(w, w_drop, qp, kp, vp)
+        ctx.meta = (q.shape[0], q.shape[1], k.shape[1], q.shape[2], k.shape[2], q.shape[3], scale, float(dropout_p),
+                    int(dropout_seed))
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        B, Hq, Hkv, L, Lk, D, scale, p, seed = ctx.meta
+        dq, dk, dv = ops.attention_f32_bwd(ctx.saved_tensors, dout.contiguous(), B, Hq, Hkv, L, Lk, D, scale, p, seed)
+        return dq, dk, dv, None, None, None, None, None
+
+
 class LinearFunction(Function):
     """y = x @ weight^T for x [T, K], weight [N, K] (a bias-free nn.Linear) through the grouped GEMM kernels
     with one group: dgrad multiplies by a transposed copy of the weight, wgrad multiplies the transposed

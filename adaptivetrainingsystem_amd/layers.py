@@ -165,7 +165,8 @@ class GroupedQueryAttention(nn.Module):
     every input and parameter, past_key_value / use_cache (model.py:700-708; the cache grows in place),
     attention_mask [batch, keys] or [batch, 1, queries, keys] (model.py:819-824), attention dropout in training
     mode (config.dropout > 0, model.py:622-623, 831-833: the mask is a hash of a per-call seed drawn from
-    torch's seed and a call counter, not torch's generator stream).  Not built (AtsError): float32 inputs."""
+    torch's seed and a call counter, not torch's generator stream), float32 activations (the scores are then
+    materialised between two float32 grouped products, as the reference's _standard_attention does)."""
 
     _instances = 0      # construction order: the layers of a model draw different dropout masks
 
@@ -206,8 +207,8 @@ class GroupedQueryAttention(nn.Module):
                 use_cache: bool = False):
         if x.dim() != 3 or x.shape[-1] != self.hidden_size:
             raise AtsError(f"GroupedQueryAttention: expected [batch, seq, {self.hidden_size}], got {tuple(x.shape)}")
-        if x.dtype != torch.bfloat16:
-            raise AtsError(f"GroupedQueryAttention: the attention kernels are bfloat16 only, got {x.dtype}")
+        if x.dtype not in (torch.bfloat16, torch.float32):
+            raise AtsError(f"GroupedQueryAttention: bfloat16 or float32 activations, got {x.dtype}")
         B, L, H = x.shape
         nh, nkv, D = self.num_heads, self.num_kv_heads, self.head_dim
         x2 = x.reshape(B * L, H).contiguous()
@@ -257,7 +258,15 @@ class GroupedQueryAttention(nn.Module):
             drop_p = self.dropout_p
             drop_seed = (torch.initial_seed() + 0x9E3779B97F4A7C15 * (self._state["calls"] + 1)
                          + 0xD1B54A32D192ED03 * self._state["dropout_stream"]) & 0xFFFFFFFFFFFFFFFF
-        if grad:
+        if x.dtype == torch.float32:
+            # the reference's own route for float32 (scores materialised, model.py:807-839), on the float32 kernels
+            if grad:
+                a = ag.AttentionF32Function.apply(q.contiguous(), k.contiguous(), v.contiguous(), self.scale, key_bias,
+                                                  pair_bias, drop_p, drop_seed)
+            else:
+                a = ops.attention_f32(q.contiguous(), k.contiguous(), v.contiguous(), self.scale, key_bias=key_bias,
+                                      pair_bias=pair_bias, dropout_p=drop_p, dropout_seed=drop_seed)
+        elif grad:
             a = ag.AttentionFunction.apply(q, k, v, self.scale, key_bias, pair_bias, drop_p, drop_seed)
         else:
             a = ops.causal_attention(q, k, v, self.scale, key_bias=key_bias, pair_bias=pair_bias, dropout_p=drop_p,

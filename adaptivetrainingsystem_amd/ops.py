@@ -833,6 +833,146 @@ def causal_attention_bwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out:
     return dq, dk, dv
 
 
+# --------------------------------------------------------------------------- float32 attention
+def _ptr_table(t: torch.Tensor, index: torch.Tensor, stride_elems: int) -> torch.Tensor:
+    """Device table of addresses t.data_ptr() + index * stride_elems * itemsize (no host round trip)."""
+    return index.to(torch.int64) * (stride_elems * t.element_size()) + t.data_ptr()
+
+
+def _transpose_to(src: torch.Tensor, src_index: torch.Tensor, dst: torch.Tensor, dst_index: torch.Tensor, R: int, C: int):
+    """Matrix src_index[n] ([R, C] contiguous inside src) -> matrix dst_index[n] ([C, R] inside dst)."""
+    n = src_index.numel()
+    in_tab, out_tab = _ptr_table(src, src_index, R * C), _ptr_table(dst, dst_index, R * C)   # both alive at the launch
+    check(_lib.load().ats_transpose_batched(in_tab.data_ptr(), out_tab.data_ptr(), n, R, C, _tag(src), 1, _stream()),
+          "ats_transpose_batched")
+
+
+def _pad_rows(t: torch.Tensor, rows: int) -> torch.Tensor:
+    """[..., r, D] -> [..., rows, D] contiguous, zero rows appended."""
+    if t.shape[-2] == rows:
+        return t.contiguous()
+    out = t.new_zeros(*t.shape[:-2], rows, t.shape[-1])
+    out[..., :t.shape[-2], :] = t
+    return out
+
+
+def _f32_groups(B: int, Hq: int, Hkv: int, dev):
+    e = torch.arange(B * Hq, device=dev)
+    kv_of = (e // Hq) * Hkv + (e % Hq) // (Hq // Hkv)            # the (batch, kv head) matrix of group (batch, q head)
+    return e, kv_of
+
+
+def attention_f32(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: Optional[float] = None,
+                  key_bias: Optional[torch.Tensor] = None, pair_bias: Optional[torch.Tensor] = None,
+                  dropout_p: float = 0.0, dropout_seed: int = 0, return_weights: bool = False):
+    """Causal grouped-query attention on float32 tensors the way the reference's _standard_attention runs it
+    (MS/core/model.py:807-839): the scores of every (batch, head) are materialised by a grouped product
+    (float32 MFMA kernels), softmaxed in place (ats_attention_softmax_f32: scale, causal fill, masks, dropout)
+    and multiplied with V by a second grouped product.  q [B,Hq,L,D], k, v [B,Hkv,Lk,D], D a multiple of 4;
+    key_bias / pair_bias / dropout as in causal_attention.  Returns out [B, L, Hq*D]; with return_weights also
+    the state the backward needs (padded weights before and after dropout)."""
+    _need_gpu(q, k, v)
+    if q.dim() != 4 or k.dim() != 4 or v.dim() != 4 or q.dtype != torch.float32 or k.dtype != q.dtype or v.dtype != q.dtype:
+        raise AtsError("attention_f32: q, k, v must be 4-D float32 tensors [batch, heads, seq, head_dim]")
+    B, Hq, L, D = q.shape
+    Hkv, Lk = k.shape[1], k.shape[2]
+    if k.shape != (B, Hkv, Lk, D) or v.shape != (B, Hkv, Lk, D) or Hq % Hkv != 0 or Lk < L or D % 4 or B * Hq > 4096:
+        raise AtsError(f"attention_f32: shapes q {tuple(q.shape)} k {tuple(k.shape)} v {tuple(v.shape)} "
+                       "(head_dim a multiple of 4, at most 4096 (batch, head) pairs)")
+    key_bias = _key_bias(key_bias, B, Lk, q, "attention_f32")
+    if not 0.0 <= dropout_p < 1.0:
+        raise AtsError(f"attention_f32: dropout_p {dropout_p} must be in [0, 1)")
+    pair_stride = 0
+    if pair_bias is not None:
+        if pair_bias.dim() != 3 or pair_bias.shape[0] not in (1, B) or tuple(pair_bias.shape[1:]) != (L, Lk) \
+                or pair_bias.dtype != torch.float32 or pair_bias.device != q.device:
+            raise AtsError(f"attention_f32: pair_bias must be float32 [batch or 1, {L}, {Lk}] on the inputs' device")
+        pair_bias = pair_bias.contiguous()
+        pair_stride = 0 if pair_bias.shape[0] == 1 else L * Lk
+    scale = float(D ** -0.5 if scale is None else scale)
+    dev = q.device
+    lib = _lib.load()
+    Lp, Lkp = (L + 3) // 4 * 4, (Lk + 3) // 4 * 4
+    E = B * Hq
+    qp, kp, vp = _pad_rows(q, Lp), _pad_rows(k, Lkp), _pad_rows(v, Lkp)
+    e, kv_of = _f32_groups(B, Hq, Hkv, dev)
+    row_start = (e * Lp).to(torch.int32)
+    row_count = torch.full((E,), Lp, dtype=torch.int32, device=dev)
+    # scores[e] = q[e] . k[kv_of[e]]^T
+    w = grouped_gemm_nt(_ptr_table(kp, kv_of, Lkp * D), D, Lkp, row_start, row_count, E * Lp, E * Lp, Lkp, D,
+                        a=qp.view(E * Lp, D))
+    w_drop = torch.empty_like(w) if dropout_p > 0 else None
+    check(lib.ats_attention_softmax_f32(w.data_ptr(), _ptr(w_drop), B, Hq, L, Lp, Lk, Lkp, scale, _ptr(key_bias),
+                                        _ptr(pair_bias), pair_stride, float(dropout_p),
+                                        int(dropout_seed) & 0xFFFFFFFFFFFFFFFF, _stream()), "ats_attention_softmax_f32")
+    # out[e] = weights[e] . v[kv_of[e]]  (NT product against v^T)
+    vT = torch.empty(B * Hkv, D, Lkp, dtype=q.dtype, device=dev)
+    every_kv = torch.arange(B * Hkv, device=dev)
+    _transpose_to(vp, every_kv, vT, every_kv, Lkp, D)
+    used = w_drop if w_drop is not None else w
+    o = grouped_gemm_nt(_ptr_table(vT, kv_of, D * Lkp), Lkp, D, row_start, row_count, E * Lp, E * Lp, D, Lkp, a=used)
+    out = o.view(B, Hq, Lp, D)[:, :, :L].transpose(1, 2).reshape(B, L, Hq * D)
+    if return_weights:
+        return out, (w, w_drop, qp, kp, vp)
+    return out
+
+
+def attention_f32_bwd(state, dout: torch.Tensor, B: int, Hq: int, Hkv: int, L: int, Lk: int, D: int,
+                      scale: Optional[float] = None, dropout_p: float = 0.0, dropout_seed: int = 0):
+    """Gradients of attention_f32 from the state its forward returned: dV = P'^T.dO, dP' = dO.V^T, dS through
+    ats_attention_softmax_bwd_f32, dQ = dS.K, dK = dS^T.Q, each a grouped float32 product (transposed operands
+    are written by ats_transpose_batched; the query heads of a kv head are summed by ats_sum_partials).
+    Returns (dq [B,Hq,L,D], dk, dv [B,Hkv,Lk,D])."""
+    w, w_drop, qp, kp, vp = state
+    _need_gpu(w, dout)
+    dev = w.device
+    lib = _lib.load()
+    scale = float(D ** -0.5 if scale is None else scale)
+    Lp, Lkp = qp.shape[2], kp.shape[2]
+    E, rep = B * Hq, Hq // Hkv
+    e, kv_of = _f32_groups(B, Hq, Hkv, dev)
+    row_start = (e * Lp).to(torch.int32)
+    row_count = torch.full((E,), Lp, dtype=torch.int32, device=dev)
+    do = _pad_rows(dout.to(torch.float32).view(B, L, Hq, D).permute(0, 2, 1, 3), Lp)          # [B, Hq, Lp, D]
+    # dP' = dO . V^T, then in place to dS (gradient of the raw scores)
+    ds = grouped_gemm_nt(_ptr_table(vp, kv_of, Lkp * D), D, Lkp, row_start, row_count, E * Lp, E * Lp, Lkp, D,
+                         a=do.view(E * Lp, D))
+    check(lib.ats_attention_softmax_bwd_f32(w.data_ptr(), ds.data_ptr(), B, Hq, L, Lp, Lk, Lkp, scale, float(dropout_p),
+                                            int(dropout_seed) & 0xFFFFFFFFFFFFFFFF, _stream()),
+          "ats_attention_softmax_bwd_f32")
+    # dQ = dS . K  (NT product against K^T)
+    every_kv = torch.arange(B * Hkv, device=dev)
+    kT = torch.empty(B * Hkv, D, Lkp, dtype=w.dtype, device=dev)
+    _transpose_to(kp, every_kv, kT, every_kv, Lkp, D)
+    dq = grouped_gemm_nt(_ptr_table(kT, kv_of, D * Lkp), Lkp, D, row_start, row_count, E * Lp, E * Lp, D, Lkp, a=ds)
+    dq = dq.view(B, Hq, Lp, D)[:, :, :L].contiguous()
+    # dV and dK: per query head a product over the queries, written so that the `rep` heads of a kv head are
+    # `rep` slices of one buffer: group (b, hq) goes to slot (hq % rep) * (B * Hkv) + its kv matrix
+    slot = (e % Hq % rep) * (B * Hkv) + kv_of
+    slot_count = torch.full((E,), Lkp, dtype=torch.int32, device=dev)
+    order = torch.empty(E, dtype=torch.int64, device=dev)
+    order[slot] = e                                   # group that owns slot s
+    doT = torch.empty(E, D, Lp, dtype=w.dtype, device=dev)
+    _transpose_to(do, e, doT, e, Lp, D)
+    qT = torch.empty(E, D, Lp, dtype=w.dtype, device=dev)
+    _transpose_to(qp, e, qT, e, Lp, D)
+
+    def over_queries(mat: torch.Tensor, rhsT: torch.Tensor) -> torch.Tensor:
+        """sum over the heads of a kv group of mat[e]^T . rhs[e]: mat [E*Lp, Lkp], rhsT [E, D, Lp] -> [B,Hkv,Lkp,D]."""
+        matT = torch.empty(E, Lkp, Lp, dtype=w.dtype, device=dev)
+        _transpose_to(mat, e, matT, slot, Lp, Lkp)
+        # b_ptrs and row tables are read in group order 0..E-1 = slot order here
+        parts = grouped_gemm_nt(_ptr_table(rhsT, order, D * Lp), Lp, D, (torch.arange(E, device=dev) * Lkp).to(torch.int32),
+                                slot_count, E * Lkp, E * Lkp, D, Lp, a=matT.view(E * Lkp, Lp))
+        parts = parts.view(rep, B * Hkv * Lkp * D)
+        total = sum_partials(parts, torch.float32) if rep > 1 else parts[0]
+        return total.view(B, Hkv, Lkp, D)[:, :, :Lk].contiguous()
+
+    dv = over_queries(w_drop if w_drop is not None else w, doT)
+    dk = over_queries(ds, qT)
+    return dq, dk, dv
+
+
 _single_group_cache: dict = {}
 
 

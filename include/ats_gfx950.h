@@ -387,6 +387,23 @@ int ats_attention_bwd_ex(const void* q, const void* k, const void* v, const void
                          float dropout_p, uint64_t dropout_seed, void* dq, void* dk, void* dv, int B, int Hq, int Hkv,
                          int L, int Lk, int D, float scale, ats_stream_t stream);
 
+/* ---- Float32 attention: the row softmax between two grouped products --------------
+ * _standard_attention on float32 tensors (model.py:807-839) materialises the scores; so does this path:
+ * scores = q.k^T per (batch, head) through ats_grouped_gemm_nt, ats_attention_softmax_f32 in place, then
+ * weights.v through ats_grouped_gemm_nt again (the host mirror composes them, ops.attention_f32).
+ * scores: [B * Hq, Lp, ld] float32, row r of head e at (e * Lp + r) * ld; rows >= L and columns >= Lk are
+ * padding (written as zeros; Lp, ld multiples of 4 for the products).  Applied in the reference's order: scale,
+ * causal fill with -1e4 (query i sees keys up to i + Lk - L), + key_bias [B, Lk], + bias_qk [B, L, Lk] (both
+ * optional, as in ats_attention_fwd_ex), float32 softmax; with dropout_p > 0 weights_drop receives the weights
+ * after dropout (same keep / drop function as ats_attention_fwd_ex) and scores keeps the undropped ones.
+ * ats_attention_softmax_bwd_f32: dp = gradient of the dropped weights on entry, gradient of the raw scores on
+ * return: P * (dP' - sum_j P dP') * scale, dP' = keep * dP / (1 - p). */
+int ats_attention_softmax_f32(float* scores, float* weights_drop, int B, int Hq, int L, int Lp, int Lk, int ld,
+                              float scale, const float* key_bias, const float* bias_qk, int64_t bias_sb,
+                              float dropout_p, uint64_t dropout_seed, ats_stream_t stream);
+int ats_attention_softmax_bwd_f32(const float* weights, float* dp, int B, int Hq, int L, int Lp, int Lk, int ld,
+                                  float scale, float dropout_p, uint64_t dropout_seed, ats_stream_t stream);
+
 /* ---- Training-step ops beside the sparse layer --------------------------------
  * Fused cross-entropy + accuracy.  Replaces fused_cross_entropy_accuracy_launcher
  * (Src/Main_Scripts/training/fused_loss.cu:179-214); numerics follow FusedLoss._pytorch_fallback

@@ -432,8 +432,10 @@ def test_gqa_module_attention_mask(gpu):
     with torch.no_grad():
         assert torch.equal(att(x.to(gpu), mask.to(gpu)), out.detach())      # float mask, no-grad path
         assert not torch.equal(att(x.to(gpu)), out.detach())
+    with torch.no_grad():       # a [B, 1, L, L] mask of ones masks nothing (up to the rounding of the added zeros)
+        assert rel_err(att(x.to(gpu), torch.ones(B, 1, L, L, device=gpu)), att(x.to(gpu))) <= 1e-2
     with pytest.raises(A.AtsError):
-        att(x.to(gpu), torch.ones(B, 1, L, L, device=gpu))
+        att(x.to(gpu), torch.ones(B, L + 1, device=gpu))
     # through a block: the mask reaches the attention sub-layer (model.py:1599)
     block = A.TransformerBlock(LayerConfig(hidden, 2 * hidden, 1, 1, num_heads=nh, num_kv_heads=nkv, seq_length=512,
                                            use_moe=False)).to(torch.bfloat16).to(gpu).eval()
@@ -681,3 +683,69 @@ def test_gqa_module_pair_mask_and_dropout(gpu):
     xg = x.to(gpu).requires_grad_()
     att(xg).float().sum().backward()
     assert xg.grad is not None and torch.isfinite(xg.grad).all() and att.q_proj.weight.grad is not None
+
+
+# --------------------------------------------------------------------------- float32
+F32_TOL = 2e-4       # float32 products with float32 accumulation, relative to the oracle's max-abs
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,L,Lk,D,p", [(2, 4, 2, 64, 64, 64, 0.0), (1, 8, 2, 130, 130, 128, 0.0),
+                                               (2, 3, 3, 33, 70, 32, 0.0), (1, 1, 1, 1, 1, 64, 0.0),
+                                               (2, 4, 1, 50, 50, 64, 0.3), (1, 2, 2, 17, 29, 96, 0.5)])
+def test_attention_float32(ops, gpu, B, Hq, Hkv, L, Lk, D, p):
+    """_standard_attention on float32 tensors (model.py:807-839): output and the three gradients against the
+    oracle and autograd over it, with a padding mask, a [B, 1, L, Lk] mask and dropout."""
+    print("case attention float32", B, Hq, Hkv, L, Lk, D, p, flush=True)
+    g = gen(161)
+    q = torch.randn(B, Hq, L, D, generator=g)
+    k = torch.randn(B, Hkv, Lk, D, generator=g)
+    v = torch.randn(B, Hkv, Lk, D, generator=g)
+    dout = torch.randn(B, L, Hq * D, generator=g)
+    rep = Hq // Hkv
+    seed = 77
+    keep = O.attention_dropout_keep(seed, B, Hq, L, Lk, p) if p > 0 else None
+    pad = _padding_mask(B, Lk, 162)
+    pad[:, :Lk - L + 1] = 1
+    pair = _pair_mask(B, L, Lk, 163)
+    for mask, kw in ((None, {}), (pad, {"key_bias": ((1.0 - pad) * -1e4).to(gpu)}),
+                     (pair, {"pair_bias": ((1.0 - pair[:, 0]) * -1e4).to(gpu)})):
+        q32, k32, v32 = (t.clone().requires_grad_() for t in (q, k, v))
+        ref = O.attention_standard(q32, k32.repeat_interleave(rep, dim=1), v32.repeat_interleave(rep, dim=1), D ** -0.5,
+                                   mask, dropout_keep=keep, dropout_p=p)
+        ref.backward(dout)
+        out, state = ops.attention_f32(q.to(gpu), k.to(gpu), v.to(gpu), dropout_p=p, dropout_seed=seed, return_weights=True,
+                                       **kw)
+        assert out.shape == (B, L, Hq * D) and out.dtype == torch.float32
+        assert rel_err(out, ref) <= F32_TOL
+        dq, dk, dv = ops.attention_f32_bwd(state, dout.to(gpu), B, Hq, Hkv, L, Lk, D, None, p, seed)
+        assert dq.shape == q.shape and dk.shape == k.shape and dv.shape == v.shape
+        assert rel_err(dv, v32.grad) <= F32_TOL
+        assert rel_err(dq, q32.grad) <= F32_TOL
+        assert rel_err(dk, k32.grad) <= F32_TOL
+
+
+def test_gqa_module_float32(gpu):
+    """GroupedQueryAttention on float32 activations and weights (the reference's CPU-runnable precision):
+    forward against the oracle, gradients against autograd over it."""
+    from types import SimpleNamespace
+    from adaptivetrainingsystem_amd.layers import GroupedQueryAttention
+    hidden, nh, nkv, B, L = 128, 4, 2, 2, 40
+    torch.manual_seed(6)
+    att = GroupedQueryAttention(SimpleNamespace(hidden_size=hidden, num_heads=nh, num_kv_heads=nkv, seq_length=64)).to(gpu)
+    names = ("q_proj", "k_proj", "v_proj", "o_proj")
+    w = [getattr(att, n).weight.detach().cpu().clone().requires_grad_() for n in names]
+    x = torch.randn(B, L, hidden, generator=gen(171))
+    mask = _padding_mask(B, L, 172)
+    mask[:, 0] = 1
+    xr = x.clone().requires_grad_()
+    ref = O.gqa_forward(xr, *w, nh, nkv, attention_mask=mask)
+    ref.square().sum().backward()
+    xg = x.to(gpu).requires_grad_()
+    out = att(xg, attention_mask=mask.to(gpu))
+    assert out.dtype == torch.float32 and rel_err(out, ref) <= F32_TOL
+    out.square().sum().backward()
+    assert rel_err(xg.grad, xr.grad) <= 5 * F32_TOL
+    for n, wr in zip(names, w):
+        assert rel_err(getattr(att, n).weight.grad, wr.grad) <= 5 * F32_TOL, n
+    with torch.no_grad():
+        assert rel_err(att(x.to(gpu), attention_mask=mask.to(gpu)), ref) <= F32_TOL
