@@ -117,6 +117,9 @@ _SIGNATURES = {
     "rope_apply_launcher": (None, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
                                    c_void_p]),
     "swiglu_launcher": (None, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p]),
+    "fused_cross_entropy_accuracy_launcher": (None, [c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_int,
+                                                     c_void_p]),
+    "fused_grad_clip_launcher": (c_float, [c_void_p, c_void_p, c_int, c_float, c_void_p]),
     "ats_legacy_last_status": (c_int, []),
     "ats_calibrate_copy": (c_int, [c_void_p, c_void_p, c_size_t, c_void_p]),
     "ats_calibrate_mfma": (c_int, [c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]),

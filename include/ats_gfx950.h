@@ -453,6 +453,18 @@ void rope_apply_launcher(float* q, float* k, const float* cos, const float* sin,
                          ats_stream_t stream);
 void swiglu_launcher(const float* gate, const float* up, float* output, int total_tokens,
                      int intermediate_size, ats_stream_t stream);
+/* The training-step launchers the reference's second loader binds (Src/Main_Scripts/training/cuda_kernels.py:
+ * 60-78, call sites 154-164 and 340-346), with the signatures of training/fused_loss.cu:183-193 and
+ * training/fused_grad_clip.cu:117-123.  Aliases of ats_cross_entropy_fwd and ats_grad_norm_clip that own
+ * their scratch memory (stream-ordered allocations), as the originals do: loss_out = sum of the token losses,
+ * accuracy_out = number of correct arg-max predictions (float), valid_tokens_out = valid tokens (int64);
+ * fused_grad_clip_launcher returns the total norm (which synchronises the stream, as in the original) after
+ * scaling the float32 gradients by max_norm / (norm + 1e-6) when that is below 1. */
+void fused_cross_entropy_accuracy_launcher(const float* logits, const int64_t* labels, int64_t pad_token_id,
+                                           float* loss_out, float* accuracy_out, int64_t* valid_tokens_out,
+                                           int total_tokens, int vocab_size, ats_stream_t stream);
+float fused_grad_clip_launcher(float** grad_ptrs_device, int* grad_sizes_device, int num_tensors, float max_norm,
+                               ats_stream_t stream);
 int ats_legacy_last_status(void);
 
 /* ---- Host-side views of the grouped-GEMM tile schedule (no device work) ----

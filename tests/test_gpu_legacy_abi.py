@@ -81,3 +81,62 @@ def test_swiglu_launcher(raw, gpu):
     assert typed.ats_legacy_last_status() == 0
     ref = gate * torch.nn.functional.silu(up)            # cuda_opt_wrapper.py:476-478 convention: gate * silu(up)
     assert (out.cpu() - ref).abs().max().item() <= 1e-5 * ref.abs().max().item()
+
+
+def test_fused_cross_entropy_accuracy_launcher(raw, gpu):
+    """training/fused_loss.cu:183-193 as training/cuda_kernels.py:154-175 calls it: the three device scalars hold
+    the sum of token losses, the number of correct predictions and the number of valid tokens."""
+    lib, typed = raw
+    T, V, pad = 37, 1000, -100
+    g = gen(201)
+    logits = torch.randn(T, V, generator=g) * 3
+    labels = torch.randint(0, V, (T,), generator=g)
+    labels[[3, 11]] = pad
+    labels[20] = V + 5                       # outside the vocabulary: skipped as well (fused_loss.cu:82)
+    labels[5] = logits[5].argmax()           # a certainly correct prediction
+    ref = O.fused_loss(logits, labels, None, pad)
+    lg, lb = logits.to(gpu), labels.to(gpu)
+    loss = torch.full((1,), 7.0, device=gpu)             # the launcher clears its outputs (fused_loss.cu:195-197)
+    acc = torch.full((1,), 7.0, device=gpu)
+    valid = torch.full((1,), 7, dtype=torch.int64, device=gpu)
+    lib.fused_cross_entropy_accuracy_launcher(ctypes.c_void_p(lg.data_ptr()), ctypes.c_void_p(lb.data_ptr()),
+                                              ctypes.c_int64(pad), ctypes.c_void_p(loss.data_ptr()),
+                                              ctypes.c_void_p(acc.data_ptr()), ctypes.c_void_p(valid.data_ptr()),
+                                              ctypes.c_int(T), ctypes.c_int(V), _stream())
+    torch.cuda.synchronize()
+    assert typed.ats_legacy_last_status() == 0
+    n = int(valid.item())
+    assert n == T - 3
+    assert abs(loss.item() / n - float(ref["loss"])) <= 1e-5 * max(1.0, abs(float(ref["loss"])))
+    assert abs(acc.item() / n - float(ref["accuracy"])) <= 1e-6
+    # nothing to do is not an error and clears the outputs
+    lib.fused_cross_entropy_accuracy_launcher(ctypes.c_void_p(lg.data_ptr()), ctypes.c_void_p(lb.data_ptr()),
+                                              ctypes.c_int64(pad), ctypes.c_void_p(loss.data_ptr()),
+                                              ctypes.c_void_p(acc.data_ptr()), ctypes.c_void_p(valid.data_ptr()),
+                                              ctypes.c_int(0), ctypes.c_int(V), _stream())
+    torch.cuda.synchronize()
+    assert typed.ats_legacy_last_status() == 0 and loss.item() == 0 and valid.item() == 0
+
+
+def test_fused_grad_clip_launcher(raw, gpu):
+    """training/fused_grad_clip.cu:117-175 as training/cuda_kernels.py:320-349 calls it: device arrays of float32
+    gradient pointers and int32 sizes, the norm comes back as the return value."""
+    lib, typed = raw
+    lib.fused_grad_clip_launcher.restype = ctypes.c_float          # cuda_kernels.py:77
+    g = gen(202)
+    shapes = [(300, 70), (5,), (1,), (129, 33), (40000,)]
+    for max_norm in (0.5, 1e6):
+        grads = [torch.randn(*s, generator=g) for s in shapes]
+        want_norm, want = O.clip_grad_norm([t.clone() for t in grads], max_norm)
+        dev = [t.to(gpu) for t in grads]
+        ptrs = torch.tensor([t.data_ptr() for t in dev], dtype=torch.int64, device=gpu)
+        sizes = torch.tensor([t.numel() for t in dev], dtype=torch.int32, device=gpu)
+        norm = lib.fused_grad_clip_launcher(ctypes.c_void_p(ptrs.data_ptr()), ctypes.c_void_p(sizes.data_ptr()),
+                                            ctypes.c_int(len(dev)), ctypes.c_float(max_norm), _stream())
+        torch.cuda.synchronize()
+        assert typed.ats_legacy_last_status() == 0
+        assert abs(norm - float(want_norm)) <= 1e-5 * float(want_norm)
+        for got, ref in zip(dev, want):
+            assert torch.allclose(got.cpu(), ref, rtol=1e-5, atol=1e-7)
+    assert lib.fused_grad_clip_launcher(ctypes.c_void_p(0), ctypes.c_void_p(0), ctypes.c_int(0), ctypes.c_float(1.0),
+                                        _stream()) == 0.0
