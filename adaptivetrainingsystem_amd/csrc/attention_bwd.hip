@@ -19,6 +19,8 @@
 // different row pitches to stay free of bank conflicts, so a tile that is read both ways is stored twice.
 #include <math.h>
 
+#include <type_traits>
+
 #include "ats_common.hpp"
 #include "attention_extra.hpp"
 
@@ -90,8 +92,66 @@ __global__ __launch_bounds__(256) void attention_delta_kernel(const bf16_t* __re
     }
 }
 
+// ------------------------------------------------------------------------------------------ tiles in LDS
+// Tiles of rows of D bf16 elements go from memory straight into LDS (buffer_load_dwordx4 ... lds: lane l of an
+// instruction deposits its 16 bytes at M0 + 16 l), so rows are unpadded and a tile is stored once, although it is
+// read both ways: along D (16-byte reads, 16 consecutive rows per quarter wave) and across rows (transposing
+// 8-byte reads, 4 consecutive rows x 64 bytes per half wave).  An XOR swizzle of the 16-byte chunks, applied on the
+// global side (which chunk a lane fetches), keeps both patterns free of bank conflicts: slot s of row r holds
+// chunk s ^ g(r) with
+//     256-byte rows: g(r) = (r % 16) ^ ((r % 4) << 2)       128-byte rows: u = (r / 2) % 8, g = u ^ ((u % 2) << 2)
+// g is a bijection of the 16 rows (or 8 row pairs) a quarter wave reads along D, and it moves the 64-byte group
+// of each of 4 consecutive rows to a different quarter of the banks.
+template <int D>
+struct SwzTile {
+    static constexpr int ROWB = D * 2;      // bytes per row
+    static constexpr int CPR = D / 8;       // 16-byte chunks per row
+    static __device__ __forceinline__ int g(int r) {
+        if constexpr (D == 128) return (r & 15) ^ ((r & 3) << 2);
+        const int u = (r >> 1) & 7;
+        return u ^ ((u & 1) << 2);
+    }
+    // lane offset (bytes from the tile's first row in memory, row stride `row_bytes`) of LDS position p (16-byte units)
+    static __device__ __forceinline__ int src_offset(int p, int row_bytes) {
+        const int r = p / CPR, sl = p % CPR;
+        return r * row_bytes + ((sl ^ g(r)) * 16);
+    }
+    // LDS byte offset of the A-operand fragment along D for k-step ks: lane (row = lane % 32 of a 32-row block, half g2)
+    static __device__ __forceinline__ int row_frag(int lane, int ks) {
+        const int col = lane & 31, g2 = lane >> 5;
+        return col * ROWB + (((2 * ks + g2) ^ g(col)) * 16);
+    }
+    // LDS byte offsets of the two 8-byte transposing reads of a fragment across rows (rows r0 + 0..15 of the tile,
+    // r0 a multiple of 16, 32 d starting at 32 * G): lane l receives d = 32 G + l % 32 and rows
+    // r0 + {4h..4h+3} (lo) and r0 + 8 + {4h..4h+3} (hi), h = l / 32, the order in which a 32x32 accumulator hands
+    // its rows to the next product
+    static __device__ __forceinline__ int tr_frag(int lane, int G, bool hi) {
+        const int rr = 4 * (lane >> 5) + ((lane & 15) >> 2) + (hi ? 8 : 0);
+        const int within = 32 * ((lane >> 4) & 1) + 8 * (lane & 3);      // byte inside the 64-byte group
+        const int chunk = 4 * G + (within >> 4);
+        return rr * ROWB + ((chunk ^ g(rr)) * 16) + (within & 15);
+    }
+};
+
+typedef __attribute__((address_space(3))) unsigned char* blds_u8_t;
+typedef __attribute__((address_space(3))) bu32x4_t* blds_v4_t;
+typedef __attribute__((address_space(3))) float* blds_f32_t;
+typedef __attribute__((address_space(3))) void* blds_void_t;
+
+__device__ __forceinline__ bu32x4_t tr_fragment_swz(blds_u8_t tile, int lo_off, int hi_off, int const_off) {
+    union {
+        btr_t t[2];
+        bu32x4_t u;
+    } cv;
+    cv.t[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((blds_tr_ptr_t)(tile + lo_off + const_off));
+    cv.t[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((blds_tr_ptr_t)(tile + hi_off + const_off));
+    return cv.u;
+}
+
 // ------------------------------------------------------------------------------------------ dQ
-// One 128-row query tile of one (batch, query head): lanes own queries, keys come in tiles of 64.
+// One 128-row query tile of one (batch, query head): lanes own queries, keys come in tiles of 64.  K and V tiles
+// are double buffered: the loads of tile t+1 are issued before the arithmetic of tile t and have the whole
+// iteration to land (one barrier per tile).
 // EXTRA: pair bias and / or dropout (attention_extra.hpp), the same decisions as the forward made.
 template <int D, bool BIAS, bool EXTRA = false>
 __device__ __forceinline__ void attention_bwd_dq_tile(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
@@ -101,20 +161,21 @@ __device__ __forceinline__ void attention_bwd_dq_tile(const bf16_t* __restrict__
                                                       int Hkv, int L, int Lk, float scale, int qt, int hq, int b,
                                                       unsigned char* smem, const AttnExtra* ex = nullptr) {
     static_assert(!(EXTRA && BIAS), "a per-key bias is folded into the pair bias");
+    using SW = SwzTile<D>;
     constexpr int KS = D / 16;
     constexpr int DB = D / 32;
-    constexpr int RPITCH = D * 2 + 16;        // bytes per K / V row in LDS
-    constexpr int TPITCH = D * 2 + 64;        // bytes per row of the second copy of K (transposing reads)
-    constexpr int RTILE = kDqBN * RPITCH;
-    constexpr int RVEC = kDqBN * (D / 8) / 256;
-    unsigned char* const sK = smem;
-    unsigned char* const sV = smem + RTILE;
-    unsigned char* const sT = smem + 2 * RTILE;
-    float* const sBias = reinterpret_cast<float*>(smem + 2 * RTILE + kDqBN * TPITCH);   // [64], log2 units
+    constexpr int ROWB = SW::ROWB;
+    constexpr int TILE = kDqBN * ROWB;              // one K or V tile
+    constexpr int STAGE = 2 * TILE;                 // [K | V]
+    constexpr int NI = TILE / 1024 / 4;             // load instructions per wave and tile, K (and V)
+    static_assert(NI >= 1 && NI * 4 * 1024 == TILE, "loader tiling");
+    const blds_u8_t sm = (blds_u8_t)smem;
+    const blds_f32_t sBias = (blds_f32_t)(sm + 2 * STAGE);      // [2][64], log2 units
     const float* bias_row = BIAS ? key_bias + (int64_t)b * Lk : nullptr;
 
     const int hkv = hq / (Hq / Hkv);
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int col = lane & 31, g = lane >> 5;
     const int q_row = qt * kBwdRows + wave * 32 + col;
     const int q_clamped = q_row < L ? q_row : L - 1;
@@ -153,6 +214,36 @@ __device__ __forceinline__ void attention_bwd_dq_tile(const bf16_t* __restrict__
         __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(kbase), 0, (int)((int64_t)Lk * D * 2), 0x00020000);
     const __amdgpu_buffer_rsrc_t v_rsrc =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(vbase), 0, (int)((int64_t)Lk * D * 2), 0x00020000);
+    int ld_off[NI];
+#pragma unroll
+    for (int j = 0; j < NI; ++j) ld_off[j] = SW::src_offset((j * 4 + wave) * 64 + lane, ROWB);
+#define DQ_LOAD(tile_, stage_)                                                                         \
+    _Pragma("unroll") for (int j_ = 0; j_ < NI; ++j_) {                                                \
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(k_rsrc, (blds_void_t)(sm + (stage_) * STAGE + (j_ * 4 + wave) * 1024), 16, \
+                                                 ld_off[j_], (tile_) * (kDqBN * D * 2), 0, 0);         \
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(v_rsrc, (blds_void_t)(sm + (stage_) * STAGE + TILE + (j_ * 4 + wave) * 1024), \
+                                                 16, ld_off[j_], (tile_) * (kDqBN * D * 2), 0, 0);     \
+    }
+    // Keys past Lk: the rows of K and V that the loads address there must be zeros in LDS (they meet exact
+    // zeros of dS and P, but 0 x NaN is not 0); each lane clears the positions of its own loads once they landed.
+#define DQ_CLEAR_TAIL(tile_, stage_)                                                                   \
+    if (((tile_) + 1) * kDqBN > Lk) {                                                                  \
+        _Pragma("unroll") for (int j_ = 0; j_ < NI; ++j_) {                                            \
+            const int p_ = (j_ * 4 + wave) * 64 + lane;                                                \
+            if ((tile_) * kDqBN + p_ / SW::CPR >= Lk) {                                                \
+                *(blds_v4_t)(sm + (stage_) * STAGE + p_ * 16) = bu32x4_t{0u, 0u, 0u, 0u};              \
+                *(blds_v4_t)(sm + (stage_) * STAGE + TILE + p_ * 16) = bu32x4_t{0u, 0u, 0u, 0u};       \
+            }                                                                                          \
+        }                                                                                              \
+    }
+    int row_addr[KS], tr_lo[DB], tr_hi[DB];
+#pragma unroll
+    for (int s = 0; s < KS; ++s) row_addr[s] = SW::row_frag(lane, s);
+#pragma unroll
+    for (int d = 0; d < DB; ++d) {
+        tr_lo[d] = SW::tr_frag(lane, d, false);
+        tr_hi[d] = SW::tr_frag(lane, d, true);
+    }
 
     bf32x16_t acc_dq[DB];
 #pragma unroll
@@ -165,93 +256,94 @@ __device__ __forceinline__ void attention_bwd_dq_tile(const bf16_t* __restrict__
     const int q_wave_first = qt * kBwdRows + wave * 32 + off;
     const int q_wave_last = q_wave_first + 31;
 
+    DQ_LOAD(0, 0)
+    if (BIAS && tid < kDqBN) sBias[tid] = tid < Lk ? bias_row[tid] * kLog2e : 0.f;
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    DQ_CLEAR_TAIL(0, 0)
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 #pragma unroll
     for (int s = 0; s < KS; ++s) asm volatile("" : "+v"(qf[s]), "+v"(dof[s]));
 
+    // log2(scale) joins the exponent, so that P * scale comes out of the exponential: dS = (P * scale) * (dP - delta)
+    const float lse2s = lse2 - log2f(scale);
     for (int t = 0; t < n_tiles; ++t) {
         const int n0 = t * kDqBN;
-        __syncthreads();   // every wave is done with the previous tile
-        {
-            bu32x4_t rk[RVEC], rv[RVEC];
-#pragma unroll
-            for (int i = 0; i < RVEC; ++i) {
-                const int idx = tid + i * 256;
-                const int lo = ((idx / (D / 8)) * D + (idx % (D / 8)) * 8) * 2;
-                rk[i] = __builtin_amdgcn_raw_buffer_load_b128(k_rsrc, lo, n0 * D * 2, 0);
-                rv[i] = __builtin_amdgcn_raw_buffer_load_b128(v_rsrc, lo, n0 * D * 2, 0);
-            }
-#pragma unroll
-            for (int i = 0; i < RVEC; ++i) {
-                const int idx = tid + i * 256;
-                const int r = idx / (D / 8), c = idx % (D / 8);
-                *reinterpret_cast<bu32x4_t*>(sK + r * RPITCH + c * 16) = rk[i];
-                *reinterpret_cast<bu32x4_t*>(sV + r * RPITCH + c * 16) = rv[i];
-                *reinterpret_cast<bu32x4_t*>(sT + r * TPITCH + c * 16) = rk[i];
-            }
-            if (BIAS && tid < kDqBN) sBias[tid] = n0 + tid < Lk ? bias_row[n0 + tid] * kLog2e : 0.f;
+        const int st = (t & 1) * STAGE;             // this tile's stage; the other one receives tile t+1
+        float r_bias = 0.f;
+        if (t + 1 < n_tiles) {
+            if (t & 1) { DQ_LOAD(t + 1, 0) } else { DQ_LOAD(t + 1, 1) }
+            if (BIAS && tid < kDqBN) r_bias = n0 + kDqBN + tid < Lk ? bias_row[n0 + kDqBN + tid] * kLog2e : 0.f;
         }
-        __syncthreads();
-        if (n0 > q_wave_last) continue;   // every key of the tile is in this wave's future
-
-        // ---- S^T = K . Q^T and dP^T = V . dO^T
-        bf32x16_t acc_s[2], acc_p[2];
+        if (n0 <= q_wave_last) {   // some key of the tile is in this wave's past or present
+            // ---- S^T = K . Q^T and dP^T = V . dO^T
+            bf32x16_t acc_s[2], acc_p[2];
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
+            for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-            for (int x = 0; x < 16; ++x) {
-                acc_s[kb][x] = 0.f;
-                acc_p[kb][x] = 0.f;
-            }
-#pragma unroll
-        for (int s = 0; s < KS; ++s)
-#pragma unroll
-            for (int kb = 0; kb < 2; ++kb) {
-                const int o = (kb * 32 + col) * RPITCH + s * 32 + g * 16;
-                acc_s[kb] = bwd_mma(*reinterpret_cast<const bu32x4_t*>(sK + o), qf[s], acc_s[kb]);
-                acc_p[kb] = bwd_mma(*reinterpret_cast<const bu32x4_t*>(sV + o), dof[s], acc_p[kb]);
-            }
-        // ---- dS^T = P^T * (dP^T - delta) * scale, with P^T = exp(S^T * scale - lse)
-        const bool diagonal = n0 + kDqBN - 1 > q_wave_first;
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-            for (int x = 0; x < 16; ++x) {
-                // the key of accumulator value x is kb*32 + (x/4)*8 + g*4 + x%4 of the tile
-                float kbias = BIAS ? sBias[kb * 32 + (x >> 2) * 8 + g * 4 + (x & 3)] : 0.f;
-                float dp = acc_p[kb][x];
-                if constexpr (EXTRA) {
-                    const int key = n0 + kb * 32 + (x >> 2) * 8 + g * 4 + (x & 3);
-                    if (ex_bias)
-                        kbias = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(pb_rsrc, pb_row + key * 4, 0, 0)) *
-                                kLog2e;
-                    if (ex_drop)   // dP reaches only the weights that were kept
-                        dp = attn_drop_hash(head_key, drop_counter0 + (uint32_t)key) >= ex->drop_threshold ? dp * ex->keep_scale
-                                                                                                        : 0.f;
+                for (int x = 0; x < 16; ++x) {
+                    acc_s[kb][x] = 0.f;
+                    acc_p[kb][x] = 0.f;
                 }
-                float p = __builtin_amdgcn_exp2f(__builtin_fmaf(acc_s[kb][x], scale_log2, kbias - lse2));
-                if (diagonal) {
-                    const int key = n0 + kb * 32 + (x >> 2) * 8 + g * 4 + (x & 3);
-                    if (key > q_pos) p = 0.f;
-                }
-                acc_s[kb][x] = p * (dp - dl) * scale;
-            }
-        bu32x4_t dsf[4];
 #pragma unroll
-        for (int s = 0; s < 4; ++s) {
-            const int kb = s >> 1, x0 = (s & 1) * 8;
-            dsf[s].x = pack_bf16x2(acc_s[kb][x0 + 0], acc_s[kb][x0 + 1]);
-            dsf[s].y = pack_bf16x2(acc_s[kb][x0 + 2], acc_s[kb][x0 + 3]);
-            dsf[s].z = pack_bf16x2(acc_s[kb][x0 + 4], acc_s[kb][x0 + 5]);
-            dsf[s].w = pack_bf16x2(acc_s[kb][x0 + 6], acc_s[kb][x0 + 7]);
+            for (int s = 0; s < KS; ++s)
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb) {
+                    const blds_u8_t pk = sm + st + row_addr[s] + kb * 32 * ROWB;
+                    const bu32x4_t kf = *(blds_v4_t)(pk), vf = *(blds_v4_t)(pk + TILE);
+                    acc_s[kb] = bwd_mma(kf, qf[s], acc_s[kb]);
+                    acc_p[kb] = bwd_mma(vf, dof[s], acc_p[kb]);
+                }
+            // ---- dS^T = P^T * (dP^T - delta) * scale, with P^T = exp(S^T * scale - lse)
+            const bool diagonal = n0 + kDqBN - 1 > q_wave_first;
+            const blds_f32_t bias_t = sBias + (t & 1) * kDqBN;
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int x = 0; x < 16; ++x) {
+                    // the key of accumulator value x is kb*32 + (x/4)*8 + g*4 + x%4 of the tile
+                    float kbias = BIAS ? bias_t[kb * 32 + (x >> 2) * 8 + g * 4 + (x & 3)] : 0.f;
+                    float dp = acc_p[kb][x];
+                    if constexpr (EXTRA) {
+                        const int key = n0 + kb * 32 + (x >> 2) * 8 + g * 4 + (x & 3);
+                        if (ex_bias)
+                            kbias = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(pb_rsrc, pb_row + key * 4, 0, 0)) *
+                                    kLog2e;
+                        if (ex_drop)   // dP reaches only the weights that were kept
+                            dp = attn_drop_hash(head_key, drop_counter0 + (uint32_t)key) >= ex->drop_threshold ? dp * ex->keep_scale
+                                                                                                            : 0.f;
+                    }
+                    float p = __builtin_amdgcn_exp2f(__builtin_fmaf(acc_s[kb][x], scale_log2, kbias - lse2s));
+                    if (diagonal) {
+                        const int key = n0 + kb * 32 + (x >> 2) * 8 + g * 4 + (x & 3);
+                        if (key > q_pos) p = 0.f;
+                    }
+                    acc_s[kb][x] = p * (dp - dl);
+                }
+            bu32x4_t dsf[4];
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                const int kb = s >> 1, x0 = (s & 1) * 8;
+                dsf[s].x = pack_bf16x2(acc_s[kb][x0 + 0], acc_s[kb][x0 + 1]);
+                dsf[s].y = pack_bf16x2(acc_s[kb][x0 + 2], acc_s[kb][x0 + 3]);
+                dsf[s].z = pack_bf16x2(acc_s[kb][x0 + 4], acc_s[kb][x0 + 5]);
+                dsf[s].w = pack_bf16x2(acc_s[kb][x0 + 6], acc_s[kb][x0 + 7]);
+            }
+            // ---- dQ^T += K^T . dS^T  (keys of a k-step in accumulator order, as in the forward's second product)
+#pragma unroll
+            for (int s = 0; s < 4; ++s)
+#pragma unroll
+                for (int d = 0; d < DB; ++d)
+                    acc_dq[d] = bwd_mma(tr_fragment_swz(sm + st, tr_lo[d], tr_hi[d], s * 16 * ROWB), dsf[s], acc_dq[d]);
         }
-        // ---- dQ^T += K^T . dS^T  (keys of a k-step in accumulator order, as in the forward's second product)
-        const unsigned char* t_lane = tr_lane_base(sT, lane, TPITCH);
-#pragma unroll
-        for (int s = 0; s < 4; ++s)
-#pragma unroll
-            for (int d = 0; d < DB; ++d)
-                acc_dq[d] = bwd_mma(tr_fragment(t_lane, s * 16, d * 32, TPITCH), dsf[s], acc_dq[d]);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        if (t + 1 < n_tiles) {
+            if (t & 1) { DQ_CLEAR_TAIL(t + 1, 0) } else { DQ_CLEAR_TAIL(t + 1, 1) }
+            if (BIAS && tid < kDqBN) sBias[((t + 1) & 1) * kDqBN + tid] = r_bias;
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
     }
+#undef DQ_LOAD
+#undef DQ_CLEAR_TAIL
 
     if (q_row < L) {
         bf16_t* drow = dq + ((int64_t)(b * Hq + hq) * L + q_row) * D;
@@ -612,12 +704,19 @@ extern "C" int ats_attention_bwd_ex(const void* q, const void* k, const void* v,
     ATS_REQUIRE(!extras || key_bias == nullptr, ATS_ERR_INVALID_ARG,
                 "ats_attention_bwd_ex: with a pair bias or dropout the per-key bias must be folded into the pair bias");
     if (D == 128) {
-        constexpr int smem_dq = 2 * kDqBN * (128 * 2 + 16) + kDqBN * (128 * 2 + 64) + kDqBN * 4;
+        constexpr int smem_dq = 4 * kDqBN * 128 * 2 + 2 * kDqBN * 4;
         constexpr int smem_dkv = 2 * kDkvBQ * (128 * 2 + 16) + 2 * kDkvBQ * (128 * 2 + 64) + 2 * kDkvBQ * 4 +
                                  kBwdRows * (128 * 2 + 16);
-        static LdsReservation reserved;
+        static LdsReservation reserved, reserved_dq;
         hipError_t e = reserve_lds(reserved, {reinterpret_cast<const void*>(attention_bwd_dkv_kernel<128>)}, smem_dkv);
         ATS_REQUIRE(e == hipSuccess, ATS_ERR_LAUNCH, "ats_attention_bwd: cannot reserve %d bytes of LDS: %s", smem_dkv,
+                    hipGetErrorString(e));
+        e = reserve_lds(reserved_dq,
+                        {reinterpret_cast<const void*>(attention_bwd_dq_kernel<128, true>),
+                         reinterpret_cast<const void*>(attention_bwd_dq_kernel<128, false>),
+                         reinterpret_cast<const void*>(attention_bwd_dq_kernel<128, false, true>)},
+                        smem_dq);
+        ATS_REQUIRE(e == hipSuccess, ATS_ERR_LAUNCH, "ats_attention_bwd: cannot reserve %d bytes of LDS: %s", smem_dq,
                     hipGetErrorString(e));
         if (extras) {
             static LdsReservation reserved_x;
@@ -643,7 +742,7 @@ extern "C" int ats_attention_bwd_ex(const void* q, const void* k, const void* v,
                                Lk, scale, ex);
         }
     } else {
-        constexpr int smem_dq = 2 * kDqBN * (64 * 2 + 16) + kDqBN * (64 * 2 + 64) + kDqBN * 4;
+        constexpr int smem_dq = 4 * kDqBN * 64 * 2 + 2 * kDqBN * 4;
         constexpr int smem_dkv = 2 * kDkvBQ * (64 * 2 + 16) + 2 * kDkvBQ * (64 * 2 + 64) + 2 * kDkvBQ * 4 +
                                  kBwdRows * (64 * 2 + 16);
         if (extras) {
