@@ -67,16 +67,22 @@ class RMSNorm(nn.Module):
 
 
 class FusedRMSNorm(nn.Module):
-    """Constructor and attributes of the reference's FusedRMSNorm(hidden_size, eps)."""
+    """Constructor and attributes of the reference's FusedRMSNorm(hidden_size, eps).  The result has the input's
+    dtype, as the model's own RMSNorm gives it (MS/core/model.py:263-299); the reference's fused wrapper converts
+    its input to float32 first and returns float32 whatever came in (MS/core/cuda_opt_wrapper.py:91-117), which
+    `float32_output=True` reproduces for callers that rely on it."""
 
-    def __init__(self, hidden_size: int, eps: float = 1e-6):
+    def __init__(self, hidden_size: int, eps: float = 1e-6, float32_output: bool = False):
         super().__init__()
         self.hidden_size = hidden_size
         self.eps = eps
         self.weight = nn.Parameter(torch.ones(hidden_size))
         self.cuda_enabled = True
+        self.float32_output = float32_output
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
+        if self.float32_output and x.dtype != torch.float32:
+            x = x.float()
         if _wants_grad(x, self.weight):
             return ag.RMSNormFunction.apply(x, self.weight, self.eps)
         return ops.rmsnorm(x, self.weight, self.eps)

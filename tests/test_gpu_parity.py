@@ -601,6 +601,23 @@ def test_tile_schedule_on_device_equals_host(gpu, counts, BM, n_tiles, SM, SN, s
     assert np.array_equal(got, want)
 
 
+def test_fused_rmsnorm_float32_output(A, gpu):
+    """The reference's fused wrapper returns float32 for any input dtype (cuda_opt_wrapper.py:91-117); the module
+    follows the input dtype unless asked for that behaviour."""
+    x = torch.randn(5, 7, 96, generator=gen(61)).bfloat16()
+    w = 1.0 + 0.1 * torch.randn(96, generator=gen(62))
+    ref32 = O.rmsnorm(x.float(), w, 1e-6)
+    plain = A.FusedRMSNorm(96).to(gpu)
+    legacy = A.FusedRMSNorm(96, float32_output=True).to(gpu)
+    with torch.no_grad():
+        plain.weight.copy_(w)
+        legacy.weight.copy_(w)
+        y_plain, y_legacy = plain(x.to(gpu)), legacy(x.to(gpu))
+    assert y_plain.dtype == torch.bfloat16 and y_legacy.dtype == torch.float32
+    assert (y_legacy.cpu() - ref32).abs().max().item() <= 1e-5 * ref32.abs().max().item()
+    assert (y_plain.float().cpu() - ref32).abs().max().item() <= 2 ** -7 * ref32.abs().max().item()
+
+
 def test_performance_monitor_api(A, gpu):
     """The monitor of the reference's operator module (moe_cuda_wrapper.py:76-159, 599-611): same keys, fed by HIP
     events instead of synchronisations, only while it is switched on."""
