@@ -645,7 +645,7 @@ def test_performance_monitor_api(A, gpu):
     P.reset_performance_monitor()
 
 
-def test_fused_swiglu_seam(gpu):
+def test_fused_swiglu_seam(A, gpu):
     import os
     import sys
     seam = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "adaptivetrainingsystem_amd",
@@ -657,12 +657,55 @@ def test_fused_swiglu_seam(gpu):
     finally:
         sys.path.remove(seam)
     assert cow.TRANSFORMER_OPS_AVAILABLE
+    F = torch.nn.functional
+
+    def expect(m, x):
+        gb = None if m.gate_proj.bias is None else m.gate_proj.bias.detach().float().cpu()
+        ub = None if m.up_proj.bias is None else m.up_proj.bias.detach().float().cpu()
+        gate = F.linear(x.float(), m.gate_proj.weight.detach().float().cpu(), gb)
+        up = F.linear(x.float(), m.up_proj.weight.detach().float().cpu(), ub)
+        return gate * F.silu(up)
+
+    # float32, no biases, no autograd: one GEMM over the stacked weight with the activation in its epilogue
     m = cow.FusedSwiGLU(32, 48).to(gpu)
     x = torch.randn(2, 5, 32, generator=gen(23))
-    got = m(x.to(gpu)).cpu()
-    gate = torch.nn.functional.linear(x, m.gate_proj.weight.cpu())
-    up = torch.nn.functional.linear(x, m.up_proj.weight.cpu())
-    assert rel_err(got, gate * torch.nn.functional.silu(up)) <= 1e-4   # projections run in the BLAS library
+    with torch.no_grad():
+        got = m(x.to(gpu)).cpu()
+    assert got.shape == (2, 5, 48)
+    assert rel_err(got, expect(m, x)) <= 1e-4
+    # the stacked copy follows a write to a parameter
+    with torch.no_grad():
+        m.up_proj.weight.mul_(0.5)
+        assert rel_err(m(x.to(gpu)).cpu(), expect(m, x)) <= 1e-4
+    # bfloat16 at a prefill-sized and at a decode-sized row count (the second takes the K-sliced path)
+    mb = cow.FusedSwiGLU(256, 512).to(gpu)
+    for rows, seed in ((300, 24), (4, 25)):
+        xb = torch.randn(rows, 256, generator=gen(seed)).bfloat16()
+        with torch.no_grad():
+            got = mb(xb.to(gpu)).float().cpu()
+        wg, wu = (w.detach().bfloat16().float().cpu() for w in (mb.gate_proj.weight, mb.up_proj.weight))
+        ref = F.linear(xb.float(), wg) * F.silu(F.linear(xb.float(), wu))
+        assert rel_err(got, ref) <= 1e-2, rows
+    # biases: the projections run as single-group GEMMs, the biases and the activation follow
+    mbias = cow.FusedSwiGLU(32, 48, use_bias=True).to(gpu)
+    with torch.no_grad():
+        assert rel_err(mbias(x.to(gpu)).cpu(), expect(mbias, x)) <= 1e-4
+    # autograd: gradients of the input, both weights and both biases against torch on the CPU
+    xg = x.clone().to(gpu).requires_grad_(True)
+    y = mbias(xg)
+    dy = torch.randn(2, 5, 48, generator=gen(26))
+    y.backward(dy.to(gpu))
+    xc = x.clone().requires_grad_(True)
+    ps = [p.detach().cpu().clone().requires_grad_(True) for p in (mbias.gate_proj.weight, mbias.gate_proj.bias,
+                                                                  mbias.up_proj.weight, mbias.up_proj.bias)]
+    yc = F.linear(xc, ps[0], ps[1]) * F.silu(F.linear(xc, ps[2], ps[3]))
+    yc.backward(dy)
+    assert rel_err(y.detach().cpu(), yc.detach()) <= 1e-4
+    assert rel_err(xg.grad.cpu(), xc.grad) <= 1e-4
+    for got_p, ref_p in zip((mbias.gate_proj.weight, mbias.gate_proj.bias, mbias.up_proj.weight, mbias.up_proj.bias), ps):
+        assert rel_err(got_p.grad.cpu(), ref_p.grad) <= 1e-4
+    with pytest.raises(A.AtsError):
+        m(torch.randn(2, 31, device=gpu))
 
 
 def test_decode_ffn_step_replays_in_a_hip_graph(A, gpu):
