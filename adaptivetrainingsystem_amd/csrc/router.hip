@@ -272,6 +272,138 @@ __device__ __forceinline__ bool key_before(float va, int ia, float vb, int ib) {
 
 constexpr int kRouteMaxK = 16;
 
+// Whole-wave reductions without LDS traffic: four DPP steps leave the result of every row of 16 lanes in all of
+// its lanes (the lane pairs, the quads, the mirrored half rows, the mirrored rows), the four row results are read
+// back as scalars and folded in a fixed order.  All 64 lanes must be active.
+template <int CTRL>
+__device__ __forceinline__ unsigned dpp_u32(unsigned v) {
+    return (unsigned)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xF, 0xF, true);
+}
+template <int CTRL>
+__device__ __forceinline__ float dpp_f32(float v) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
+}
+constexpr int kDppSwapPairs = 0xB1, kDppSwapQuadHalves = 0x4E, kDppHalfMirror = 0x141, kDppRowMirror = 0x140;
+__device__ __forceinline__ unsigned wave_max_u32(unsigned v) {
+    v = max(v, dpp_u32<kDppSwapPairs>(v));
+    v = max(v, dpp_u32<kDppSwapQuadHalves>(v));
+    v = max(v, dpp_u32<kDppHalfMirror>(v));
+    v = max(v, dpp_u32<kDppRowMirror>(v));
+    const unsigned a = __builtin_amdgcn_readlane(v, 0), b = __builtin_amdgcn_readlane(v, 16);
+    const unsigned c = __builtin_amdgcn_readlane(v, 32), d = __builtin_amdgcn_readlane(v, 48);
+    return max(max(a, b), max(c, d));
+}
+__device__ __forceinline__ float wave_max_f32(float v) {
+    v = fmaxf(v, dpp_f32<kDppSwapPairs>(v));
+    v = fmaxf(v, dpp_f32<kDppSwapQuadHalves>(v));
+    v = fmaxf(v, dpp_f32<kDppHalfMirror>(v));
+    v = fmaxf(v, dpp_f32<kDppRowMirror>(v));
+    const float a = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 0));
+    const float b = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 16));
+    const float c = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 32));
+    const float d = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 48));
+    return fmaxf(fmaxf(a, b), fmaxf(c, d));
+}
+__device__ __forceinline__ float wave_sum_f32(float v) {
+    v += dpp_f32<kDppSwapPairs>(v);
+    v += dpp_f32<kDppSwapQuadHalves>(v);
+    v += dpp_f32<kDppHalfMirror>(v);
+    v += dpp_f32<kDppRowMirror>(v);
+    const float a = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 0));
+    const float b = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 16));
+    const float c = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 32));
+    const float d = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 48));
+    return ((a + b) + c) + d;
+}
+// Selection key of key_before as an unsigned number: larger key = earlier in the order.  NaN is the largest
+// key, -0 counts as +0, and 0 is below every value (used for lanes that hold no candidate).
+__device__ __forceinline__ unsigned route_order_key(float v) {
+    if (v != v) return 0xFFFFFFFFu;
+    const unsigned u = (unsigned)__float_as_int(v + 0.0f);
+    return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+
+// One token per wave, one expert per lane (32 < E <= 64): the reductions of the softmax and the k arg-max rounds
+// run on DPP and scalar reads instead of shuffles through LDS; an arg-max is the wave maximum of the keys,
+// then the lowest lane that holds it.  Same selection, weights and statistics as route_topk_kernel, except that
+// the sums of the softmax are formed in another (fixed) order.
+__global__ __launch_bounds__(256) void route_topk_wave_kernel(const float* __restrict__ logits, int64_t T, int E, int k,
+                                                              float temperature, int variant, int iters,
+                                                              int32_t* __restrict__ idx_out, float* __restrict__ w_out,
+                                                              int32_t* __restrict__ part_hist,
+                                                              float* __restrict__ part_colsum) {
+    extern __shared__ unsigned char smem_raw[];
+    int* s_hist = reinterpret_cast<int*>(smem_raw);            // [E]
+    float* s_col = reinterpret_cast<float*>(s_hist + E);        // [4][E]
+    const bool want_stats = part_hist != nullptr;
+    const int lane = lane_id();
+    const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
+    const bool has = lane < E;
+    if (want_stats) {
+        for (int i = threadIdx.x; i < E; i += 256) s_hist[i] = 0;
+        __syncthreads();
+    }
+    float col = 0.f;
+    const float neg_inf = -INFINITY;
+    for (int it = 0; it < iters; ++it) {
+        const int64_t t = ((int64_t)blockIdx.x * iters + it) * 4 + wave;
+        if (t >= T) break;                                   // wave-uniform
+        const float v = has ? logits[t * E + lane] : neg_inf;
+        const float m0 = wave_max_f32(v);
+        float p0 = has ? expf(v - m0) : 0.f;
+        p0 = p0 / wave_sum_f32(p0);
+        col += p0;
+        float sv = v, p = p0;
+        if (temperature != 1.0f) {
+            sv = has ? __fdiv_rn(v, temperature) : neg_inf;
+            const float m = wave_max_f32(sv);
+            p = has ? expf(sv - m) : 0.f;
+            p = p / wave_sum_f32(p);
+        }
+        unsigned key = has ? route_order_key(sv) : 0u;
+        float sel_val = 0.f, sel_p = 0.f;
+        int sel_idx = 0;
+        for (int j = 0; j < k; ++j) {
+            const unsigned best = wave_max_u32(key);
+            const int first = __builtin_amdgcn_readfirstlane(__ffsll((long long)__ballot(key == best)) - 1);
+            const float bv = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(sv), first));
+            const float bp = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(p), first));
+            if (lane == first) key = 0u;
+            if (lane == j) {
+                sel_val = bv;
+                sel_p = bp;
+                sel_idx = first;
+            }
+            if (want_stats && lane == 0) atomicAdd(&s_hist[first], 1);
+        }
+        float wsel;
+        const bool is_sel = lane < k;
+        if (variant == ATS_ROUTE_SOFTMAX_TOPK) {
+            float tot = 0.f;
+            for (int j = 0; j < k; ++j) tot += __int_as_float(__builtin_amdgcn_readlane(__float_as_int(sel_p), j));
+            wsel = sel_p / (tot + 1e-9f);
+        } else {
+            const float mx = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(sel_val), 0));
+            const float ex = is_sel ? expf(sel_val - mx) : 0.f;
+            float tot = 0.f;
+            for (int j = 0; j < k; ++j) tot += __int_as_float(__builtin_amdgcn_readlane(__float_as_int(ex), j));
+            wsel = ex / tot;
+        }
+        if (is_sel) {
+            idx_out[t * k + lane] = sel_idx;
+            w_out[t * k + lane] = wsel;
+        }
+    }
+    if (want_stats) {
+        if (has) s_col[wave * E + lane] = col;
+        __syncthreads();
+        for (int e = threadIdx.x; e < E; e += 256) {
+            part_hist[(int64_t)blockIdx.x * E + e] = s_hist[e];
+            part_colsum[(int64_t)blockIdx.x * E + e] = ((s_col[e] + s_col[E + e]) + s_col[2 * E + e]) + s_col[3 * E + e];
+        }
+    }
+}
+
 template <int VPL>
 __global__ __launch_bounds__(256) void route_topk_kernel(const float* __restrict__ logits, int64_t T, int E, int k,
                                                          float temperature, int variant, int G, int iters,
@@ -614,7 +746,10 @@ extern "C" int ats_route_topk(const float* logits, int64_t T, int E, int k, floa
     hipStream_t s = as_stream(stream);
     const size_t smem = (size_t)E * 6 * sizeof(float);
     const int vpl = (E + G - 1) / G;
-    if (vpl <= 1)
+    if (G == kWave && vpl <= 1 && nblocks > 1)
+        hipLaunchKernelGGL(route_topk_wave_kernel, dim3(nblocks), dim3(256), smem, s, logits, T, E, k, temperature,
+                           variant, iters, idx_out, w_out, part_hist, part_col);
+    else if (vpl <= 1)
         hipLaunchKernelGGL((route_topk_kernel<1>), dim3(nblocks), dim3(256), smem, s, logits, T, E, k, temperature,
                            variant, G, iters, idx_out, w_out, part_hist, part_col, load_balancing_weight, hist,
                            prob_colsum, aux);

@@ -174,7 +174,8 @@ def _ambiguous_rows(logits, k, temperature):
 
 
 @pytest.mark.parametrize("T,E,k,temp", [(512, 8, 2, 1.0), (1000, 64, 6, 1.0), (37, 4, 1, 1.0), (300, 128, 4, 0.7),
-                                        (129, 6, 3, 1.3), (16384, 8, 2, 1.0), (50, 300, 8, 1.0)])
+                                        (129, 6, 3, 1.3), (16384, 8, 2, 1.0), (50, 300, 8, 1.0), (700, 40, 5, 0.8),
+                                        (4096, 64, 6, 1.0), (333, 33, 16, 1.0)])
 def test_route_topk(ops, gpu, T, E, k, temp):
     print("case route", T, E, k, temp, flush=True)
     logits = torch.randn(T, E, generator=gen(15)) * 1.3
@@ -199,6 +200,31 @@ def test_route_topk_ties_go_to_lower_index(ops, gpu):
     r = ops.route_topk(logits.to(gpu), 2, 1.0, 1, with_stats=False)
     assert r["indices"].cpu().tolist() == [[0, 1], [1, 2]]
     assert torch.allclose(r["weights"].cpu(), torch.full((2, 2), 0.5))
+
+
+def test_route_topk_one_token_per_wave_order(ops, gpu):
+    """33..64 experts and more than 64 tokens take the kernel that selects with wave-wide reductions of an
+    unsigned key: ties go to the lower index, -0 equals +0, NaN ranks first, -inf last."""
+    T, E, k = 200, 64, 6
+    logits = torch.randn(T, E, generator=gen(151))
+    logits[0, :] = 1.0                                  # all equal: experts 0..5
+    logits[1, 10:20] = 7.0                              # ten equal maxima: 10..15
+    logits[2, :] = -1.0
+    logits[2, 5], logits[2, 9], logits[2, 40] = 0.0, -0.0, 0.0      # zeros of both signs tie: 5, 9, 40, then 0, 1, 2
+    logits[3, 17] = float("nan")                        # NaN first
+    logits[3, 3] = float("inf")
+    logits[4, :] = float("-inf")
+    logits[4, 60:] = torch.tensor([0.5, 0.25, 0.5, 0.125])           # 60, 62, 61, 63, then -inf ties 0, 1
+    r = ops.route_topk(logits.to(gpu), k, 1.0, 1, with_stats=False)
+    idx = r["indices"].cpu().tolist()
+    assert idx[0] == [0, 1, 2, 3, 4, 5]
+    assert idx[1] == [10, 11, 12, 13, 14, 15]
+    assert idx[2] == [5, 9, 40, 0, 1, 2]
+    assert idx[3][:2] == [17, 3]
+    assert idx[4] == [60, 62, 61, 63, 0, 1]
+    # every other row: the order of a stable sort by descending value
+    ref = torch.sort(logits[5:], dim=-1, descending=True, stable=True)[1][:, :k]
+    assert torch.equal(r["indices"].cpu().long()[5:], ref)
 
 
 def test_topk_gating_api(A, gpu):
