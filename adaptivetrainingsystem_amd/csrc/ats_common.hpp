@@ -152,4 +152,19 @@ __device__ __forceinline__ float wave_sum(float v) {
 
 __device__ __forceinline__ int lane_id() { return threadIdx.x & 63; }
 
+// Inclusive prefix sum over the 64 lanes of a wave, all of which must be active.  Four DPP row shifts scan every
+// row of 16 lanes (a lane whose source lies outside its row adds 0), the three row totals are read back as
+// scalars.  A shuffle scan costs six round trips through the LDS crossbar instead.
+__device__ __forceinline__ int wave_inclusive_scan(int v) {
+    v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xF, 0xF, false);   // row_shr:1
+    v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xF, 0xF, false);   // row_shr:2
+    v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xF, 0xF, false);   // row_shr:4
+    v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xF, 0xF, false);   // row_shr:8
+    const int r0 = __builtin_amdgcn_readlane(v, 15);
+    const int r1 = r0 + __builtin_amdgcn_readlane(v, 31);
+    const int r2 = r1 + __builtin_amdgcn_readlane(v, 47);
+    const int row = (threadIdx.x & 63) >> 4;
+    return v + (row == 0 ? 0 : row == 1 ? r0 : row == 2 ? r1 : r2);
+}
+
 }  // namespace ats

@@ -65,7 +65,7 @@ __global__ __launch_bounds__(256) void plan_hist_kernel(const IdxT* __restrict__
 }
 
 // step 2 (one block): chunk_hist -> exclusive chunk bases (in place), hist, kept, offsets.
-// One wave scans one expert at a time: 64 chunks per pass with a shuffle prefix sum, the carry
+// A wave scans four experts at a time: 64 chunks per pass with a prefix sum over the wave, the carry
 // runs across passes.
 __device__ void scan_totals(int32_t* chunk_hist, int nchunks, int E, int C, int32_t* hist, int32_t* kept,
                             int32_t* offsets, int* s_tot) {
@@ -73,24 +73,30 @@ __device__ void scan_totals(int32_t* chunk_hist, int nchunks, int E, int C, int3
     const int wave = threadIdx.x >> 6;
     const int nwaves = blockDim.x >> 6;
     constexpr int U = 4;   // experts scanned together by a wave (their loads are issued back to back)
+    constexpr int P = 2;   // passes of 64 chunks whose loads are issued together
     for (int e0 = wave * U; e0 < E; e0 += nwaves * U) {
         int carry[U];
 #pragma unroll
         for (int u = 0; u < U; ++u) carry[u] = 0;
-        for (int base = 0; base < nchunks; base += kWave) {
-            const int c = base + lane;
-            int v[U], incl[U];
+        for (int base = 0; base < nchunks; base += P * kWave) {
+            int v[P][U];
 #pragma unroll
-            for (int u = 0; u < U; ++u) v[u] = (c < nchunks && e0 + u < E) ? chunk_hist[(int64_t)c * E + e0 + u] : 0;
+            for (int q = 0; q < P; ++q) {
+                const int c = base + q * kWave + lane;
 #pragma unroll
-            for (int u = 0; u < U; ++u) {
-                incl[u] = v[u];
-                for (int off = 1; off < kWave; off <<= 1) {
-                    const int up = __shfl_up(incl[u], off, 64);
-                    if (lane >= off) incl[u] += up;
+                for (int u = 0; u < U; ++u)
+                    v[q][u] = (c < nchunks && e0 + u < E) ? chunk_hist[(int64_t)c * E + e0 + u] : 0;
+            }
+#pragma unroll
+            for (int q = 0; q < P; ++q) {
+                const int c = base + q * kWave + lane;
+                if (base + q * kWave >= nchunks) break;      // wave-uniform
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    const int incl = wave_inclusive_scan(v[q][u]);
+                    if (c < nchunks && e0 + u < E) chunk_hist[(int64_t)c * E + e0 + u] = carry[u] + incl - v[q][u];
+                    carry[u] += __builtin_amdgcn_readlane(incl, kWave - 1);
                 }
-                if (c < nchunks && e0 + u < E) chunk_hist[(int64_t)c * E + e0 + u] = carry[u] + incl[u] - v[u];
-                carry[u] += __shfl(incl[u], kWave - 1, 64);
             }
         }
         if (lane == 0) {
@@ -106,13 +112,17 @@ __device__ void scan_totals(int32_t* chunk_hist, int nchunks, int E, int C, int3
         }
     }
     __syncthreads();
-    if (threadIdx.x == 0) {
+    // offsets = exclusive prefix sums of the kept counts: the first wave, 64 experts per step
+    if (wave == 0) {
         int run = 0;
-        for (int e = 0; e < E; ++e) {
-            offsets[e] = run;
-            run += s_tot[e];
+        for (int e0 = 0; e0 < E; e0 += kWave) {
+            const int e = e0 + lane;
+            const int kp = e < E ? s_tot[e] : 0;
+            const int incl = wave_inclusive_scan(kp);
+            if (e < E) offsets[e] = run + incl - kp;
+            run += __builtin_amdgcn_readlane(incl, kWave - 1);
         }
-        offsets[E] = run;
+        if (lane == 0) offsets[E] = run;
     }
     __syncthreads();
 }
@@ -145,6 +155,9 @@ __device__ void chunk_rank_and_write(const IdxT* idx, int64_t n, int k, int E, i
     __syncthreads();
     int* my_base = s_cnt + wave * E;
     const unsigned long long lt_mask = lane == 0 ? 0ull : (~0ull >> (64 - lane));
+    // up to 64 experts: lane l keeps the running base of expert l in a register, so the loop below touches no LDS
+    const bool in_regs = E <= kWave;
+    int base_reg = (in_regs && lane < E) ? my_base[lane] : 0;
     for (int step = 0; step < PERWAVE / kWave; ++step) {
         const int64_t a = chunk_base + wave * PERWAVE + step * kWave + lane;
         bool bad = false;
@@ -152,13 +165,21 @@ __device__ void chunk_rank_and_write(const IdxT* idx, int64_t n, int k, int E, i
         int rank = -1;
         unsigned long long remaining = __ballot(e >= 0);
         while (remaining) {
-            const int leader = __ffsll((long long)remaining) - 1;
-            const int le = __shfl(e, leader, 64);
+            // the leader and its expert are the same in all lanes: scalar reads instead of shuffles
+            const int leader = __builtin_amdgcn_readfirstlane(__ffsll((long long)remaining) - 1);
+            const int le = __builtin_amdgcn_readlane(e, leader);
             const unsigned long long same = __ballot(e == le);
-            if (e == le) rank = my_base[le] + __popcll(same & lt_mask);
+            const int n_same = __popcll(same);
+            if (in_regs) {
+                const int b = __builtin_amdgcn_readlane(base_reg, le);
+                if (e == le) rank = b + __popcll(same & lt_mask);
+                if (lane == le) base_reg += n_same;
+            } else {
+                if (e == le) rank = my_base[le] + __popcll(same & lt_mask);
+                // all lanes have read my_base[le]; the leader advances it for the next step
+                if (lane == leader) my_base[le] += n_same;
+            }
             remaining &= ~same;
-            // all lanes have read my_base[le]; the leader advances it for the next step
-            if (lane == leader) my_base[le] += __popcll(same);
         }
         if (a < n) {
             if (e >= 0 && rank < C) {

@@ -123,12 +123,7 @@ __device__ __forceinline__ uint32_t topk_key(float f) {
 // Exclusive prefix sum of one int per thread over a 1024-thread block, in thread order.  s_wave: 16 ints of LDS.
 __device__ __forceinline__ int block_exclusive_scan_1024(int v, int* s_wave, int* total) {
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    int incl = v;
-#pragma unroll
-    for (int off = 1; off < 64; off <<= 1) {
-        const int o = __shfl_up(incl, off, 64);
-        if (lane >= off) incl += o;
-    }
+    const int incl = wave_inclusive_scan(v);
     __syncthreads();                       // s_wave may still be read from a previous call
     if (lane == 63) s_wave[wave] = incl;
     __syncthreads();
@@ -177,12 +172,7 @@ __global__ __launch_bounds__(1024) void select_topk_radix_kernel(const float* __
                 c[q] = s_hist[255 - 4 * t - q];
                 sum += c[q];
             }
-            unsigned int incl = sum;
-#pragma unroll
-            for (int off = 1; off < 64; off <<= 1) {
-                const unsigned int o = __shfl_up(incl, off, 64);
-                if (t >= off) incl += o;
-            }
+            const unsigned int incl = (unsigned int)wave_inclusive_scan((int)sum);
             const unsigned int before = incl - sum;          // keys in higher bins than this lane's
             if (before < want && incl >= want) {
                 unsigned int acc = before;

@@ -119,12 +119,7 @@ __device__ __forceinline__ void tile_scan64(const int32_t* __restrict__ row_coun
     const int cnt = g < G ? row_count[g % E] : 0;
     int t = cnt > 0 ? (cnt + BM - 1) / BM : 0;
     if (aligned) t = (t + SM - 1) / SM * SM;
-    int p = t;
-#pragma unroll
-    for (int off = 1; off < 64; off <<= 1) {
-        const int v = __shfl_up(p, off, 64);
-        if (lane >= off) p += v;
-    }
+    const int p = wave_inclusive_scan(t);     // ats_common.hpp
     *t_out = t;
     *p_out = p;   // inclusive prefix inside this chunk
 }
