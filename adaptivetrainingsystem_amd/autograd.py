@@ -92,7 +92,7 @@ class ScatterAddRowsFunction(Function):
 
 class AttentionFunction(Function):
     """Causal grouped-query attention: q [B,Hq,L,D], k, v [B,Hkv,Lk,D] -> [B, L, Hq*D]; key_bias
-    [B, Lk] / pair_bias [B or 1, L, Lk] float32 or None (constants: they get no gradient); dropout_p with the
+    [B, Lk] / pair_bias [B or 1, (Hq or 1,) L, Lk] float32 or None (constants: they get no gradient); dropout_p with the
     seed that the backward reuses."""
 
     @staticmethod

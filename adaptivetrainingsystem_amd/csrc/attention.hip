@@ -128,7 +128,7 @@ __device__ __forceinline__ void attention_q_tile(const bf16_t* __restrict__ q, c
     if constexpr (EXTRA) {
         ex_bias = ex->bias_qk != nullptr;
         ex_drop = ex->keep_scale > 0.f;
-        pb_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(ex_bias ? ex->bias_qk + (int64_t)b * ex->bias_sb : nullptr),
+        pb_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(ex_bias ? ex->bias_qk + (int64_t)b * ex->bias_sb + (int64_t)hq * ex->bias_sh : nullptr),
                                                     0, ex_bias ? (int)((int64_t)L * Lk * 4) : 0, 0x00020000);
         pb_row = q_clamped * Lk * 4;
         head_key = attn_head_key(ex->seed_lo, ex->seed_hi, (uint32_t)(b * Hq + hq));
@@ -938,11 +938,13 @@ extern "C" size_t ats_attention_fwd_workspace(int B, int Hq, int Hkv, int L, int
 
 // Fills the kernels' view of the optional extras; returns false (with the error text set) on bad arguments.
 namespace ats {
-bool make_attention_extra(const char* who, const float* bias_qk, int64_t bias_sb, float dropout_p, uint64_t seed, int L,
+bool make_attention_extra(const char* who, const float* bias_qk, int64_t bias_sb, int64_t bias_sh, float dropout_p,
+                          uint64_t seed, int L,
                           int Lk, AttnExtra* ex, bool* any) {
     *any = bias_qk != nullptr || dropout_p > 0.f;
     ex->bias_qk = bias_qk;
     ex->bias_sb = bias_sb;
+    ex->bias_sh = bias_sh;
     ex->keep_scale = 0.f;
     ex->drop_threshold = 0;
     ex->seed_lo = (uint32_t)seed;
@@ -951,8 +953,10 @@ bool make_attention_extra(const char* who, const float* bias_qk, int64_t bias_sb
         set_error("%s: dropout probability %g (must be in [0, 1))", who, dropout_p);
         return false;
     }
-    if (bias_qk && (bias_sb < 0 || (reinterpret_cast<uintptr_t>(bias_qk) & 3) || (int64_t)L * Lk * 4 >= 0x7fffffffLL)) {
-        set_error("%s: pair bias (batch stride %lld; one [L, Lk] matrix must stay under 2 GiB)", who, (long long)bias_sb);
+    if (bias_qk && (bias_sb < 0 || bias_sh < 0 || (reinterpret_cast<uintptr_t>(bias_qk) & 3) ||
+                    (int64_t)L * Lk * 4 >= 0x7fffffffLL)) {
+        set_error("%s: pair bias (batch stride %lld, head stride %lld; one [L, Lk] matrix must stay under 2 GiB)", who,
+                  (long long)bias_sb, (long long)bias_sh);
         return false;
     }
     if (dropout_p > 0.f) {
@@ -972,13 +976,14 @@ extern "C" int ats_attention_fwd(const void* q, const void* k, int64_t k_sb, int
                                  int64_t v_sl, int64_t v_sh, const float* key_bias, void* out, float* lse, int B, int Hq,
                                  int Hkv, int L, int Lk, int D, float scale, void* workspace, size_t workspace_bytes,
                                  ats_stream_t stream) {
-    return ats_attention_fwd_ex(q, k, k_sb, k_sh, v, v_sb, v_sl, v_sh, key_bias, nullptr, 0, 0.f, 0, out, lse, B, Hq, Hkv, L,
+    return ats_attention_fwd_ex(q, k, k_sb, k_sh, v, v_sb, v_sl, v_sh, key_bias, nullptr, 0, 0, 0.f, 0, out, lse, B, Hq, Hkv, L,
                                 Lk, D, scale, workspace, workspace_bytes, stream);
 }
 
 extern "C" int ats_attention_fwd_ex(const void* q, const void* k, int64_t k_sb, int64_t k_sh, const void* v, int64_t v_sb,
                                     int64_t v_sl, int64_t v_sh, const float* key_bias, const float* bias_qk,
-                                    int64_t bias_sb, float dropout_p, uint64_t dropout_seed, void* out, float* lse, int B,
+                                    int64_t bias_sb, int64_t bias_sh, float dropout_p, uint64_t dropout_seed, void* out,
+                                    float* lse, int B,
                                     int Hq, int Hkv, int L, int Lk, int D, float scale, void* workspace,
                                     size_t workspace_bytes, ats_stream_t stream) {
     using namespace ats;
@@ -1000,7 +1005,7 @@ extern "C" int ats_attention_fwd_ex(const void* q, const void* k, int64_t k_sb, 
     const float scale_log2 = scale * 1.4426950408889634f;
     AttnExtra ex;
     bool extras = false;
-    if (!make_attention_extra("ats_attention_fwd_ex", bias_qk, bias_sb, dropout_p, dropout_seed, L, Lk, &ex, &extras))
+    if (!make_attention_extra("ats_attention_fwd_ex", bias_qk, bias_sb, bias_sh, dropout_p, dropout_seed, L, Lk, &ex, &extras))
         return ATS_ERR_INVALID_ARG;
     if (extras) {
         ATS_REQUIRE(key_bias == nullptr, ATS_ERR_INVALID_ARG,

@@ -200,7 +200,7 @@ __device__ __forceinline__ void attention_bwd_dq_tile(const bf16_t* __restrict__
     if constexpr (EXTRA) {
         ex_bias = ex->bias_qk != nullptr;
         ex_drop = ex->keep_scale > 0.f;
-        pb_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(ex_bias ? ex->bias_qk + (int64_t)b * ex->bias_sb : nullptr),
+        pb_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(ex_bias ? ex->bias_qk + (int64_t)b * ex->bias_sb + (int64_t)hq * ex->bias_sh : nullptr),
                                                     0, ex_bias ? (int)((int64_t)L * Lk * 4) : 0, 0x00020000);
         pb_row = q_clamped * Lk * 4;
         head_key = attn_head_key(ex->seed_lo, ex->seed_hi, (uint32_t)(b * Hq + hq));
@@ -430,14 +430,10 @@ __device__ __forceinline__ void attention_bwd_dkv_tile(const bf16_t* __restrict_
     const float scale_log2 = scale * kLog2e;
 
     const float kbias = key_bias ? key_bias[(int64_t)b * Lk + key_clamped] * kLog2e : 0.f;   // this lane's key
-    __amdgpu_buffer_rsrc_t pb_rsrc;
     bool ex_bias = false, ex_drop = false;
     if constexpr (EXTRA) {
         ex_bias = ex->bias_qk != nullptr;
         ex_drop = ex->keep_scale > 0.f;
-        // queries past L read as zeros (their probabilities are zeros anyway: lse = +inf)
-        pb_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(ex_bias ? ex->bias_qk + (int64_t)b * ex->bias_sb : nullptr),
-                                                    0, ex_bias ? (int)((int64_t)L * Lk * 4) : 0, 0x00020000);
     }
     const bf16_t* kp = k + ((int64_t)(b * Hkv + hkv) * Lk + key_clamped) * D;
     bu32x4_t kf[KS];
@@ -483,6 +479,13 @@ __device__ __forceinline__ void attention_bwd_dkv_tile(const bf16_t* __restrict_
         const float* lbase = lse + (int64_t)(b * Hq + hq) * L;
         const float* dbase = delta + (int64_t)(b * Hq + hq) * L;
         const uint32_t head_key = EXTRA ? attn_head_key(ex->seed_lo, ex->seed_hi, (uint32_t)(b * Hq + hq)) : 0u;
+        // this head's [L, Lk] matrix of the pair bias; queries past L read as zeros (their probabilities are
+        // zeros anyway: lse = +inf)
+        __amdgpu_buffer_rsrc_t pb_rsrc;
+        if constexpr (EXTRA)
+            pb_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+                const_cast<float*>(ex_bias ? ex->bias_qk + (int64_t)b * ex->bias_sb + (int64_t)hq * ex->bias_sh : nullptr), 0,
+                ex_bias ? (int)((int64_t)L * Lk * 4) : 0, 0x00020000);
         // buffer loads: query rows past L read as zeros
         const __amdgpu_buffer_rsrc_t q_rsrc =
             __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(qbase), 0, (int)((int64_t)L * D * 2), 0x00020000);
@@ -668,13 +671,13 @@ extern "C" int ats_attention_delta(const void* out, const void* dout, float* del
 extern "C" int ats_attention_bwd(const void* q, const void* k, const void* v, const void* dout, const float* lse,
                                  const float* delta, const float* key_bias, void* dq, void* dk, void* dv, int B, int Hq,
                                  int Hkv, int L, int Lk, int D, float scale, ats_stream_t stream) {
-    return ats_attention_bwd_ex(q, k, v, dout, lse, delta, key_bias, nullptr, 0, 0.f, 0, dq, dk, dv, B, Hq, Hkv, L, Lk, D,
+    return ats_attention_bwd_ex(q, k, v, dout, lse, delta, key_bias, nullptr, 0, 0, 0.f, 0, dq, dk, dv, B, Hq, Hkv, L, Lk, D,
                                 scale, stream);
 }
 
 extern "C" int ats_attention_bwd_ex(const void* q, const void* k, const void* v, const void* dout, const float* lse,
                                     const float* delta, const float* key_bias, const float* bias_qk, int64_t bias_sb,
-                                    float dropout_p, uint64_t dropout_seed, void* dq, void* dk, void* dv, int B, int Hq,
+                                    int64_t bias_sh, float dropout_p, uint64_t dropout_seed, void* dq, void* dk, void* dv, int B, int Hq,
                                     int Hkv, int L, int Lk, int D, float scale, ats_stream_t stream) {
     using namespace ats;
     ATS_REQUIRE(B >= 0 && Hq > 0 && Hkv > 0 && Hq % Hkv == 0 && L >= 0 && Lk >= L && scale > 0.f, ATS_ERR_INVALID_ARG,
@@ -699,7 +702,7 @@ extern "C" int ats_attention_bwd_ex(const void* q, const void* k, const void* v,
     hipStream_t s = as_stream(stream);
     AttnExtra ex;
     bool extras = false;
-    if (!make_attention_extra("ats_attention_bwd_ex", bias_qk, bias_sb, dropout_p, dropout_seed, L, Lk, &ex, &extras))
+    if (!make_attention_extra("ats_attention_bwd_ex", bias_qk, bias_sb, bias_sh, dropout_p, dropout_seed, L, Lk, &ex, &extras))
         return ATS_ERR_INVALID_ARG;
     ATS_REQUIRE(!extras || key_bias == nullptr, ATS_ERR_INVALID_ARG,
                 "ats_attention_bwd_ex: with a pair bias or dropout the per-key bias must be folded into the pair bias");

@@ -24,6 +24,7 @@ namespace ats {
 struct AttnExtra {
     const float* bias_qk;     // [B, L, Lk] float32 added to the scaled scores, or null
     int64_t bias_sb;          // floats between the matrices of two batch entries (0: one matrix for all)
+    int64_t bias_sh;          // floats between the matrices of two query heads (0: one matrix for all heads)
     float keep_scale;         // 1 / (1 - p) with dropout, 0 without
     uint32_t drop_threshold;  // keep an element iff its hash >= threshold
     uint32_t seed_lo, seed_hi;
@@ -51,7 +52,7 @@ ATS_HD inline uint32_t attn_drop_hash(uint32_t head_key, uint32_t counter) {
 
 // Fills `ex` from the arguments of the extended entry points; false (error text set) on bad arguments.
 // `any` tells whether a pair bias or dropout was asked for at all.
-bool make_attention_extra(const char* who, const float* bias_qk, int64_t bias_sb, float dropout_p, uint64_t seed, int L,
+bool make_attention_extra(const char* who, const float* bias_qk, int64_t bias_sb, int64_t bias_sh, float dropout_p, uint64_t seed, int L,
                           int Lk, AttnExtra* ex, bool* any);
 
 }  // namespace ats

@@ -38,7 +38,7 @@ __global__ __launch_bounds__(256) void attention_softmax_f32_kernel(float* __res
     }
     const int last_key = i + (Lk - L);      // keys after it are the query's future
     const float* kb = key_bias ? key_bias + (int64_t)b * Lk : nullptr;
-    const float* pb = ex.bias_qk ? ex.bias_qk + (int64_t)b * ex.bias_sb + (int64_t)i * Lk : nullptr;
+    const float* pb = ex.bias_qk ? ex.bias_qk + (int64_t)b * ex.bias_sb + (int64_t)(e % Hq) * ex.bias_sh + (int64_t)i * Lk : nullptr;
     auto value = [&](int j) {
         float t = j > last_key ? -1e4f : srow[j] * scale;
         if (kb) t += kb[j];
@@ -101,14 +101,14 @@ __global__ __launch_bounds__(256) void attention_softmax_bwd_f32_kernel(const fl
 
 extern "C" int ats_attention_softmax_f32(float* scores, float* weights_drop, int B, int Hq, int L, int Lp, int Lk, int ld,
                                          float scale, const float* key_bias, const float* bias_qk, int64_t bias_sb,
-                                         float dropout_p, uint64_t dropout_seed, ats_stream_t stream) {
+                                         int64_t bias_sh, float dropout_p, uint64_t dropout_seed, ats_stream_t stream) {
     using namespace ats;
     ATS_REQUIRE(B >= 0 && Hq > 0 && L >= 0 && Lp >= L && Lk >= L && ld >= Lk && scale > 0.f, ATS_ERR_INVALID_ARG,
                 "ats_attention_softmax_f32: B=%d Hq=%d L=%d Lp=%d Lk=%d ld=%d scale=%g", B, Hq, L, Lp, Lk, ld, scale);
     if (B == 0 || Lp == 0) return ATS_OK;
     AttnExtra ex;
     bool extras = false;
-    if (!make_attention_extra("ats_attention_softmax_f32", bias_qk, bias_sb, dropout_p, dropout_seed, L, Lk, &ex, &extras))
+    if (!make_attention_extra("ats_attention_softmax_f32", bias_qk, bias_sb, bias_sh, dropout_p, dropout_seed, L, Lk, &ex, &extras))
         return ATS_ERR_INVALID_ARG;
     ATS_REQUIRE(scores && (dropout_p == 0.f || weights_drop), ATS_ERR_INVALID_ARG,
                 "ats_attention_softmax_f32: null pointer (dropout needs the second output)");
@@ -128,7 +128,7 @@ extern "C" int ats_attention_softmax_bwd_f32(const float* weights, float* dp, in
     if (B == 0 || Lp == 0) return ATS_OK;
     AttnExtra ex;
     bool extras = false;
-    if (!make_attention_extra("ats_attention_softmax_bwd_f32", nullptr, 0, dropout_p, dropout_seed, L, Lk, &ex, &extras))
+    if (!make_attention_extra("ats_attention_softmax_bwd_f32", nullptr, 0, 0, dropout_p, dropout_seed, L, Lk, &ex, &extras))
         return ATS_ERR_INVALID_ARG;
     ATS_REQUIRE(weights && dp, ATS_ERR_INVALID_ARG, "ats_attention_softmax_bwd_f32: null pointer");
     const int64_t n_rows = (int64_t)B * Hq * Lp;

@@ -247,17 +247,18 @@ class GroupedQueryAttention(nn.Module):
         key_bias = pair_bias = None
         if attention_mask is not None:
             # 1 = attend, 0 = masked: (1 - mask) * -1e4 is added to the scores (model.py:819-824), for every
-            # query and head with a [batch, keys] mask, per query with a [batch, 1, queries, keys] mask
+            # query and head with a [batch, keys] mask, per query (and per head) with a 4-D mask that
+            # broadcasts against [batch, heads, queries, keys]
             Lk = k.shape[2]
             m = attention_mask.to(device=x.device, dtype=torch.float32)
             if m.dim() == 2 and m.shape == (B, Lk):
                 key_bias = (1.0 - m) * -1e4
-            elif m.dim() == 4 and m.shape[0] in (1, B) and m.shape[1] == 1 and m.shape[2] in (1, L) and m.shape[3] == Lk:
-                pair_bias = ((1.0 - m[:, 0]) * -1e4).expand(m.shape[0], L, Lk)
+            elif m.dim() == 4 and m.shape[0] in (1, B) and m.shape[1] in (1, nh) and m.shape[2] in (1, L) and m.shape[3] == Lk:
+                pair_bias = ((1.0 - m) * -1e4).expand(m.shape[0], m.shape[1], L, Lk)
             else:
                 raise AtsError(f"GroupedQueryAttention: attention_mask must be [batch, keys] = [{B}, {Lk}] or "
-                               f"[batch, 1, queries, keys] = [{B}, 1, {L}, {Lk}], got {tuple(attention_mask.shape)} "
-                               "(one mask per head is not built)")
+                               f"[batch or 1, heads or 1, queries or 1, keys] = [{B}, {nh}, {L}, {Lk}], got "
+                               f"{tuple(attention_mask.shape)}")
         drop_p, drop_seed = 0.0, 0
         if self.training and self.dropout_p > 0:
             # a fresh mask per call, reproducible under torch.manual_seed: no device round trip

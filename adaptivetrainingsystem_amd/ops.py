@@ -739,26 +739,36 @@ def _key_bias(key_bias, B: int, Lk: int, q: torch.Tensor, who: str):
     return key_bias.contiguous()
 
 
-def _attention_extras(key_bias, pair_bias, dropout_p: float, B: int, L: int, Lk: int, q: torch.Tensor, who: str):
-    """Arguments of the extended entry points.  Returns (key_bias, pair_bias, batch stride): with a pair bias
-    or dropout a per-key bias is folded into the pair bias (the kernels take one or the other)."""
+def _pair_bias(pair_bias, B: int, Hq: int, L: int, Lk: int, q: torch.Tensor, who: str):
+    """Checks a pair bias, float32 [batch or 1, queries, keys] or [batch or 1, heads or 1, queries, keys], and
+    returns it as a contiguous 4-D tensor with its batch and head strides in floats (0 where it is shared)."""
+    if pair_bias.dim() == 3:
+        pair_bias = pair_bias[:, None]
+    if pair_bias.dim() != 4 or pair_bias.shape[0] not in (1, B) or pair_bias.shape[1] not in (1, Hq) \
+            or tuple(pair_bias.shape[2:]) != (L, Lk) or pair_bias.dtype != torch.float32 or pair_bias.device != q.device:
+        raise AtsError(f"{who}: pair_bias must be float32 [batch or 1, (heads or 1,) queries, keys] = "
+                       f"[{B}, {Hq}, {L}, {Lk}] on the inputs' device")
+    pair_bias = pair_bias.contiguous()
+    heads = pair_bias.shape[1]
+    return pair_bias, (0 if pair_bias.shape[0] == 1 else heads * L * Lk), (0 if heads == 1 else L * Lk)
+
+
+def _attention_extras(key_bias, pair_bias, dropout_p: float, B: int, Hq: int, L: int, Lk: int, q: torch.Tensor, who: str):
+    """Arguments of the extended entry points.  Returns (key_bias, pair_bias, batch stride, head stride): with a
+    pair bias or dropout a per-key bias is folded into the pair bias (the kernels take one or the other)."""
     key_bias = _key_bias(key_bias, B, Lk, q, who)
     if not 0.0 <= dropout_p < 1.0:
         raise AtsError(f"{who}: dropout_p {dropout_p} must be in [0, 1)")
+    sb = sh = 0
     if pair_bias is not None:
-        if pair_bias.dim() != 3 or pair_bias.shape[0] not in (1, B) or tuple(pair_bias.shape[1:]) != (L, Lk) \
-                or pair_bias.dtype != torch.float32 or pair_bias.device != q.device:
-            raise AtsError(f"{who}: pair_bias must be float32 [batch or 1, queries, keys] = [{B}, {L}, {Lk}] on the "
-                           "inputs' device")
+        pair_bias, sb, sh = _pair_bias(pair_bias, B, Hq, L, Lk, q, who)
         if key_bias is not None:
-            pair_bias = pair_bias + key_bias[:, None, :]
+            pair_bias, sb, sh = _pair_bias(pair_bias + key_bias[:, None, None, :], B, Hq, L, Lk, q, who)
             key_bias = None
-        pair_bias = pair_bias.contiguous()
     elif dropout_p > 0.0 and key_bias is not None:
-        pair_bias = key_bias[:, None, :].expand(B, L, Lk).contiguous()
+        pair_bias, sb, sh = key_bias[:, None, None, :].expand(B, 1, L, Lk).contiguous(), L * Lk, 0
         key_bias = None
-    stride = 0 if pair_bias is None or pair_bias.shape[0] == 1 else L * Lk
-    return key_bias, pair_bias, stride
+    return key_bias, pair_bias, sb, sh
 
 
 def causal_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: Optional[float] = None,
@@ -770,8 +780,8 @@ def causal_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: O
     With Lk > L the leading Lk - L keys are a cache: query i sits at position i + Lk - L.
     key_bias [B, Lk] float32 (optional) is added to the scaled scores of a key for every query and head;
     (1 - attention_mask) * -1e4 is the reference's padding mask (MS/core/model.py:819-824).
-    pair_bias [B or 1, L, Lk] float32 (optional) is added to the scaled scores of a (query, key) pair for
-    every head: (1 - mask[:, 0]) * -1e4 for the reference's [B,1,L,Lk] masks (same lines).
+    pair_bias [B or 1, L, Lk] or [B or 1, Hq or 1, L, Lk] float32 (optional) is added to the scaled scores of
+    a (query, key) pair, for every head or per head: (1 - mask) * -1e4 for the reference's 4-D masks (same lines).
     dropout_p > 0 drops attention weights (model.py:831-833) by a hash of (dropout_seed, batch, head, query,
     key); causal_attention_bwd given the same seed sees the same mask.
     split_keys=False keeps the single-pass kernel where few rows against many keys would otherwise be cut
@@ -786,7 +796,8 @@ def causal_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: O
     q = q.contiguous()
     if k.stride(3) != 1 or k.stride(2) != D or k.stride(0) % 8 or k.stride(1) % 8 or k.data_ptr() % 16:
         k = k.contiguous()        # rows of a head must follow one another; batch and head strides are free
-    key_bias, pair_bias, pair_stride = _attention_extras(key_bias, pair_bias, dropout_p, B, L, Lk, q, "causal_attention")
+    key_bias, pair_bias, pair_sb, pair_sh = _attention_extras(key_bias, pair_bias, dropout_p, B, Hq, L, Lk, q,
+                                                              "causal_attention")
     if v.stride(3) != 1 or any(st % 8 for st in v.stride()[:3]) or v.stride(2) < D or v.data_ptr() % 16:
         v = v.contiguous()
     lib = _lib.load()
@@ -796,7 +807,7 @@ def causal_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: O
     ws_bytes = lib.ats_attention_fwd_workspace(B, Hq, Hkv, L, Lk, D) if split_keys else 0
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device) if ws_bytes else None
     check(lib.ats_attention_fwd_ex(q.data_ptr(), k.data_ptr(), k.stride(0), k.stride(1), v.data_ptr(), v.stride(0),
-                                   v.stride(2), v.stride(1), _ptr(key_bias), _ptr(pair_bias), pair_stride,
+                                   v.stride(2), v.stride(1), _ptr(key_bias), _ptr(pair_bias), pair_sb, pair_sh,
                                    float(dropout_p), int(dropout_seed) & 0xFFFFFFFFFFFFFFFF, out.data_ptr(), _ptr(lse),
                                    B, Hq, Hkv, L, Lk, D, float(D ** -0.5 if scale is None else scale), _ptr(ws),
                                    ws_bytes, _stream()),
@@ -818,15 +829,15 @@ def causal_attention_bwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out:
     q, k, v, out = q.contiguous(), k.contiguous(), v.contiguous(), out.contiguous()
     dout = dout.to(q.dtype).contiguous()
     lse = lse.contiguous()
-    key_bias, pair_bias, pair_stride = _attention_extras(key_bias, pair_bias, dropout_p, B, L, Lk, q,
-                                                         "causal_attention_bwd")
+    key_bias, pair_bias, pair_sb, pair_sh = _attention_extras(key_bias, pair_bias, dropout_p, B, Hq, L, Lk, q,
+                                                              "causal_attention_bwd")
     lib = _lib.load()
     delta = torch.empty(B, Hq, L, dtype=torch.float32, device=q.device)
     check(lib.ats_attention_delta(out.data_ptr(), dout.data_ptr(), delta.data_ptr(), B, Hq, L, D, _stream()),
           "ats_attention_delta")
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     check(lib.ats_attention_bwd_ex(q.data_ptr(), k.data_ptr(), v.data_ptr(), dout.data_ptr(), lse.data_ptr(),
-                                   delta.data_ptr(), _ptr(key_bias), _ptr(pair_bias), pair_stride, float(dropout_p),
+                                   delta.data_ptr(), _ptr(key_bias), _ptr(pair_bias), pair_sb, pair_sh, float(dropout_p),
                                    int(dropout_seed) & 0xFFFFFFFFFFFFFFFF, dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
                                    B, Hq, Hkv, L, Lk, D, float(D ** -0.5 if scale is None else scale), _stream()),
           "ats_attention_bwd_ex")
@@ -882,13 +893,9 @@ def attention_f32(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: Opti
     key_bias = _key_bias(key_bias, B, Lk, q, "attention_f32")
     if not 0.0 <= dropout_p < 1.0:
         raise AtsError(f"attention_f32: dropout_p {dropout_p} must be in [0, 1)")
-    pair_stride = 0
+    pair_sb = pair_sh = 0
     if pair_bias is not None:
-        if pair_bias.dim() != 3 or pair_bias.shape[0] not in (1, B) or tuple(pair_bias.shape[1:]) != (L, Lk) \
-                or pair_bias.dtype != torch.float32 or pair_bias.device != q.device:
-            raise AtsError(f"attention_f32: pair_bias must be float32 [batch or 1, {L}, {Lk}] on the inputs' device")
-        pair_bias = pair_bias.contiguous()
-        pair_stride = 0 if pair_bias.shape[0] == 1 else L * Lk
+        pair_bias, pair_sb, pair_sh = _pair_bias(pair_bias, B, Hq, L, Lk, q, "attention_f32")
     scale = float(D ** -0.5 if scale is None else scale)
     dev = q.device
     lib = _lib.load()
@@ -903,7 +910,7 @@ def attention_f32(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, scale: Opti
                         a=qp.view(E * Lp, D))
     w_drop = torch.empty_like(w) if dropout_p > 0 else None
     check(lib.ats_attention_softmax_f32(w.data_ptr(), _ptr(w_drop), B, Hq, L, Lp, Lk, Lkp, scale, _ptr(key_bias),
-                                        _ptr(pair_bias), pair_stride, float(dropout_p),
+                                        _ptr(pair_bias), pair_sb, pair_sh, float(dropout_p),
                                         int(dropout_seed) & 0xFFFFFFFFFFFFFFFF, _stream()), "ats_attention_softmax_f32")
     # out[e] = weights[e] . v[kv_of[e]]  (NT product against v^T)
     vT = torch.empty(B * Hkv, D, Lkp, dtype=q.dtype, device=dev)

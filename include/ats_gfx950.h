@@ -353,9 +353,10 @@ int ats_attention_fwd(const void* q, const void* k, int64_t k_sb, int64_t k_sh, 
                       ats_stream_t stream);
 /* The same with the two options of the reference's masked path that the plain entry point leaves out
  * (model.py:819-833):
- *   bias_qk (optional): float32 [B, L, Lk], added to the scaled scores of (query, key) for every head; a
- *     [B,1,L,Lk] attention mask is (1 - mask) * -1e4.  bias_sb = floats between two batch entries' matrices
- *     (0: one matrix for the whole batch).
+ *   bias_qk (optional): float32 [L, Lk] matrices added to the scaled scores of (query, key); a [B,1,L,Lk]
+ *     attention mask is (1 - mask) * -1e4.  The matrix of (batch b, query head h) starts at
+ *     bias_qk + b * bias_sb + h * bias_sh floats: bias_sb = 0 shares one matrix over the batch, bias_sh = 0
+ *     over the heads ([B,1,L,Lk] masks), bias_sh = L * Lk gives every head its own ([B,H,L,Lk] masks).
  *   dropout_p in [0, 1): each attention weight is dropped with this probability and the kept ones are scaled
  *     by 1 / (1 - p) before they meet V (nn.Dropout on the weights while training); the log-sum-exp is that of
  *     the undropped scores.  Keep / drop is a function of (dropout_seed, batch, head, query, key) only, so
@@ -364,8 +365,9 @@ int ats_attention_fwd(const void* q, const void* k, int64_t k_sb, int64_t k_sh, 
  * single-pass kernel without the software pipeline runs.  Neither option set: identical to ats_attention_fwd. */
 int ats_attention_fwd_ex(const void* q, const void* k, int64_t k_sb, int64_t k_sh, const void* v, int64_t v_sb,
                          int64_t v_sl, int64_t v_sh, const float* key_bias, const float* bias_qk, int64_t bias_sb,
-                         float dropout_p, uint64_t dropout_seed, void* out, float* lse, int B, int Hq, int Hkv, int L,
-                         int Lk, int D, float scale, void* workspace, size_t workspace_bytes, ats_stream_t stream);
+                         int64_t bias_sh, float dropout_p, uint64_t dropout_seed, void* out, float* lse, int B, int Hq,
+                         int Hkv, int L, int Lk, int D, float scale, void* workspace, size_t workspace_bytes,
+                         ats_stream_t stream);
 
 /* ---- Causal grouped-query attention (backward) ----------------------------------
  * The reference leaves this gradient to autograd (model.py:757-839 under torch.autograd); the kernels
@@ -384,8 +386,8 @@ int ats_attention_bwd(const void* q, const void* k, const void* v, const void* d
  * call whose lse is passed; delta from ats_attention_delta on the forward's output as usual). */
 int ats_attention_bwd_ex(const void* q, const void* k, const void* v, const void* dout, const float* lse,
                          const float* delta, const float* key_bias, const float* bias_qk, int64_t bias_sb,
-                         float dropout_p, uint64_t dropout_seed, void* dq, void* dk, void* dv, int B, int Hq, int Hkv,
-                         int L, int Lk, int D, float scale, ats_stream_t stream);
+                         int64_t bias_sh, float dropout_p, uint64_t dropout_seed, void* dq, void* dk, void* dv, int B,
+                         int Hq, int Hkv, int L, int Lk, int D, float scale, ats_stream_t stream);
 
 /* ---- Float32 attention: the row softmax between two grouped products --------------
  * _standard_attention on float32 tensors (model.py:807-839) materialises the scores; so does this path:
@@ -393,14 +395,14 @@ int ats_attention_bwd_ex(const void* q, const void* k, const void* v, const void
  * weights.v through ats_grouped_gemm_nt again (the host mirror composes them, ops.attention_f32).
  * scores: [B * Hq, Lp, ld] float32, row r of head e at (e * Lp + r) * ld; rows >= L and columns >= Lk are
  * padding (written as zeros; Lp, ld multiples of 4 for the products).  Applied in the reference's order: scale,
- * causal fill with -1e4 (query i sees keys up to i + Lk - L), + key_bias [B, Lk], + bias_qk [B, L, Lk] (both
- * optional, as in ats_attention_fwd_ex), float32 softmax; with dropout_p > 0 weights_drop receives the weights
+ * causal fill with -1e4 (query i sees keys up to i + Lk - L), + key_bias [B, Lk], + bias_qk (both optional,
+ * bias_sb / bias_sh as in ats_attention_fwd_ex), float32 softmax; with dropout_p > 0 weights_drop receives the weights
  * after dropout (same keep / drop function as ats_attention_fwd_ex) and scores keeps the undropped ones.
  * ats_attention_softmax_bwd_f32: dp = gradient of the dropped weights on entry, gradient of the raw scores on
  * return: P * (dP' - sum_j P dP') * scale, dP' = keep * dP / (1 - p). */
 int ats_attention_softmax_f32(float* scores, float* weights_drop, int B, int Hq, int L, int Lp, int Lk, int ld,
                               float scale, const float* key_bias, const float* bias_qk, int64_t bias_sb,
-                              float dropout_p, uint64_t dropout_seed, ats_stream_t stream);
+                              int64_t bias_sh, float dropout_p, uint64_t dropout_seed, ats_stream_t stream);
 int ats_attention_softmax_bwd_f32(const float* weights, float* dp, int B, int Hq, int L, int Lp, int Lk, int ld,
                                   float scale, float dropout_p, uint64_t dropout_seed, ats_stream_t stream);
 

@@ -584,6 +584,64 @@ def test_causal_attention_pair_mask(ops, gpu, B, Hq, Hkv, L, Lk, D):
     assert torch.equal(shared[:1], out[:1])
 
 
+def _head_mask(B, H, L, Lk, seed, p_zero=0.3):
+    """[B, H, L, Lk] of ones and zeros, a different pattern per head; every query keeps its own position."""
+    m = (torch.rand(B, H, L, Lk, generator=gen(seed)) >= p_zero).float()
+    i = torch.arange(L)
+    m[:, :, i, i + (Lk - L)] = 1.0
+    return m
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,L,Lk,D", [(2, 4, 2, 200, 200, 128), (1, 8, 2, 300, 300, 64), (2, 3, 3, 129, 129, 64),
+                                             (2, 4, 1, 70, 300, 64), (1, 2, 2, 130, 131, 128)])
+def test_causal_attention_mask_per_head(ops, gpu, B, Hq, Hkv, L, Lk, D):
+    """[B, H, L, Lk] masks, which the reference's broadcast (model.py:819-824) accepts like any mask that expands
+    to the scores: forward, log-sum-exp and the three gradients (dK / dV sum over the query heads of a kv head,
+    each with its own mask) against the oracle and autograd over it; a per-head mask that repeats one matrix
+    equals the shared form bit for bit; one set of head masks shared by the batch."""
+    print("case attention head mask", B, Hq, Hkv, L, Lk, D, flush=True)
+    g = gen(171)
+    q = torch.randn(B, Hq, L, D, generator=g).bfloat16()
+    k = torch.randn(B, Hkv, Lk, D, generator=g).bfloat16()
+    v = torch.randn(B, Hkv, Lk, D, generator=g).bfloat16()
+    dout = torch.randn(B, L, Hq * D, generator=g).bfloat16()
+    mask = _head_mask(B, Hq, L, Lk, 172)
+    rep = Hq // Hkv
+    q32, k32, v32 = (t.float().requires_grad_() for t in (q, k, v))
+    ref = O.attention_standard(q32, k32.repeat_interleave(rep, dim=1), v32.repeat_interleave(rep, dim=1), D ** -0.5, mask)
+    ref.backward(dout.float())
+    bias = ((1.0 - mask) * -1e4).to(gpu)
+    qg, kg, vg = q.to(gpu), k.to(gpu), v.to(gpu)
+    out, lse = ops.causal_attention(qg, kg, vg, return_lse=True, pair_bias=bias)
+    assert rel_err(out, ref) <= BF16_TOL
+    s = torch.matmul(q.float(), k.repeat_interleave(rep, dim=1).float().transpose(-2, -1)) * D ** -0.5
+    s = s.masked_fill(torch.triu(torch.ones(L, Lk, dtype=torch.bool), diagonal=1 + Lk - L), float("-inf"))
+    assert rel_err(lse, torch.logsumexp(s + (1.0 - mask) * -1e4, -1)) <= 1e-4
+    dq, dk, dv = ops.causal_attention_bwd(qg, kg, vg, out, lse, dout.to(gpu), pair_bias=bias)
+    assert rel_err(dv, v32.grad) <= GRAD_TOL
+    assert rel_err(dq, q32.grad) <= GRAD_TOL
+    assert rel_err(dk, k32.grad) <= GRAD_TOL
+    # the same matrix for every head: the shared form's bits
+    one = bias[:, :1].contiguous()
+    shared = ops.causal_attention(qg, kg, vg, pair_bias=one)
+    repeated = ops.causal_attention(qg, kg, vg, pair_bias=one.expand(B, Hq, L, Lk).contiguous())
+    assert torch.equal(shared, repeated)
+    # head masks shared by the batch
+    first = ops.causal_attention(qg, kg, vg, pair_bias=bias[:1])
+    assert torch.equal(first[:1], out[:1])
+    # float32 route
+    if D % 4 == 0 and L <= 200:
+        q32, k32, v32 = (t.float().requires_grad_() for t in (q, k, v))
+        ref = O.attention_standard(q32, k32.repeat_interleave(rep, dim=1), v32.repeat_interleave(rep, dim=1), D ** -0.5, mask)
+        ref.backward(dout.float())
+        o32, state = ops.attention_f32(qg.float(), kg.float(), vg.float(), pair_bias=bias, return_weights=True)
+        assert rel_err(o32, ref) <= F32_TOL
+        dq, dk, dv = ops.attention_f32_bwd(state, dout.float().to(gpu), B, Hq, Hkv, L, Lk, D, None, 0.0, 0)
+        assert rel_err(dq, q32.grad) <= F32_TOL and rel_err(dk, k32.grad) <= F32_TOL and rel_err(dv, v32.grad) <= F32_TOL
+    with pytest.raises(Exception):
+        ops.causal_attention(qg, kg, vg, pair_bias=torch.zeros(B, Hq + 1, L, Lk, device=gpu))
+
+
 @pytest.mark.parametrize("B,Hq,Hkv,L,Lk,D,p", [(2, 4, 2, 200, 200, 128, 0.25), (1, 8, 2, 300, 300, 64, 0.1),
                                                (2, 3, 3, 129, 129, 64, 0.5), (1, 4, 1, 520, 520, 128, 0.3),
                                                (2, 4, 2, 70, 300, 64, 0.25), (1, 2, 1, 31, 31, 64, 0.9)])
@@ -655,8 +713,13 @@ def test_gqa_module_pair_mask_and_dropout(gpu):
     with torch.no_grad():
         out = att(x.to(gpu), attention_mask=mask.to(gpu))
     assert rel_err(out, O.gqa_forward(x, *w, nh, nkv, attention_mask=mask)) <= BF16_TOL
+    # one mask per head (the reference's broadcast takes any mask that expands to [B, H, L, L]); a wrong head count raises
+    hmask = _head_mask(B, nh, L, L, 153)
+    with torch.no_grad():
+        out_h = att(x.to(gpu), attention_mask=hmask.to(gpu))
+    assert rel_err(out_h, O.gqa_forward(x, *w, nh, nkv, attention_mask=hmask)) <= BF16_TOL
     with pytest.raises(AtsError):
-        att(x.to(gpu), attention_mask=torch.ones(B, nh, L, L, device=gpu))      # one mask per head
+        att(x.to(gpu), attention_mask=torch.ones(B, nh + 1, L, L, device=gpu))
     # eval mode: dropout is off (model.py:832)
     with torch.no_grad():
         plain = att(x.to(gpu))
