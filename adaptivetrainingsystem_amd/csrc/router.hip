@@ -272,49 +272,6 @@ __device__ __forceinline__ bool key_before(float va, int ia, float vb, int ib) {
 
 constexpr int kRouteMaxK = 16;
 
-// Whole-wave reductions without LDS traffic: four DPP steps leave the result of every row of 16 lanes in all of
-// its lanes (the lane pairs, the quads, the mirrored half rows, the mirrored rows), the four row results are read
-// back as scalars and folded in a fixed order.  All 64 lanes must be active.
-template <int CTRL>
-__device__ __forceinline__ unsigned dpp_u32(unsigned v) {
-    return (unsigned)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xF, 0xF, true);
-}
-template <int CTRL>
-__device__ __forceinline__ float dpp_f32(float v) {
-    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xF, 0xF, true));
-}
-constexpr int kDppSwapPairs = 0xB1, kDppSwapQuadHalves = 0x4E, kDppHalfMirror = 0x141, kDppRowMirror = 0x140;
-__device__ __forceinline__ unsigned wave_max_u32(unsigned v) {
-    v = max(v, dpp_u32<kDppSwapPairs>(v));
-    v = max(v, dpp_u32<kDppSwapQuadHalves>(v));
-    v = max(v, dpp_u32<kDppHalfMirror>(v));
-    v = max(v, dpp_u32<kDppRowMirror>(v));
-    const unsigned a = __builtin_amdgcn_readlane(v, 0), b = __builtin_amdgcn_readlane(v, 16);
-    const unsigned c = __builtin_amdgcn_readlane(v, 32), d = __builtin_amdgcn_readlane(v, 48);
-    return max(max(a, b), max(c, d));
-}
-__device__ __forceinline__ float wave_max_f32(float v) {
-    v = fmaxf(v, dpp_f32<kDppSwapPairs>(v));
-    v = fmaxf(v, dpp_f32<kDppSwapQuadHalves>(v));
-    v = fmaxf(v, dpp_f32<kDppHalfMirror>(v));
-    v = fmaxf(v, dpp_f32<kDppRowMirror>(v));
-    const float a = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 0));
-    const float b = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 16));
-    const float c = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 32));
-    const float d = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 48));
-    return fmaxf(fmaxf(a, b), fmaxf(c, d));
-}
-__device__ __forceinline__ float wave_sum_f32(float v) {
-    v += dpp_f32<kDppSwapPairs>(v);
-    v += dpp_f32<kDppSwapQuadHalves>(v);
-    v += dpp_f32<kDppHalfMirror>(v);
-    v += dpp_f32<kDppRowMirror>(v);
-    const float a = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 0));
-    const float b = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 16));
-    const float c = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 32));
-    const float d = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 48));
-    return ((a + b) + c) + d;
-}
 // Selection key of key_before as an unsigned number: larger key = earlier in the order.  NaN is the largest
 // key, -0 counts as +0, and 0 is below every value (used for lanes that hold no candidate).
 __device__ __forceinline__ unsigned route_order_key(float v) {
