@@ -59,12 +59,13 @@ __global__ __launch_bounds__(256) void plan_hist_kernel(const IdxT* __restrict__
     bool bad = false;
     chunk_wave_counts<IdxT, kPlanChunk / 4>(idx, n, E, (int64_t)blockIdx.x * kPlanChunk, s_cnt, &bad);
     for (int e = threadIdx.x; e < E; e += 256)
-        chunk_hist[(int64_t)blockIdx.x * E + e] = s_cnt[e] + s_cnt[E + e] + s_cnt[2 * E + e] + s_cnt[3 * E + e];
+        chunk_hist[(int64_t)e * gridDim.x + blockIdx.x] = s_cnt[e] + s_cnt[E + e] + s_cnt[2 * E + e] + s_cnt[3 * E + e];
     // the status word is cleared here and raised by the ranking kernel, which runs after this one
     if (blockIdx.x == 0 && threadIdx.x == 0) status[0] = 0;
 }
 
-// step 2 (one block): chunk_hist -> exclusive chunk bases (in place), hist, kept, offsets.
+// step 2 (one block): chunk_hist -> exclusive chunk bases (in place), hist, kept, offsets.  chunk_hist is
+// [E, nchunks]: an expert's chunk counts lie side by side, so the lanes of a scanning wave read one line.
 // A wave scans four experts at a time: 64 chunks per pass with a prefix sum over the wave, the carry
 // runs across passes.
 __device__ void scan_totals(int32_t* chunk_hist, int nchunks, int E, int C, int32_t* hist, int32_t* kept,
@@ -85,7 +86,7 @@ __device__ void scan_totals(int32_t* chunk_hist, int nchunks, int E, int C, int3
                 const int c = base + q * kWave + lane;
 #pragma unroll
                 for (int u = 0; u < U; ++u)
-                    v[q][u] = (c < nchunks && e0 + u < E) ? chunk_hist[(int64_t)c * E + e0 + u] : 0;
+                    v[q][u] = (c < nchunks && e0 + u < E) ? chunk_hist[(int64_t)(e0 + u) * nchunks + c] : 0;
             }
 #pragma unroll
             for (int q = 0; q < P; ++q) {
@@ -94,7 +95,7 @@ __device__ void scan_totals(int32_t* chunk_hist, int nchunks, int E, int C, int3
 #pragma unroll
                 for (int u = 0; u < U; ++u) {
                     const int incl = wave_inclusive_scan(v[q][u]);
-                    if (c < nchunks && e0 + u < E) chunk_hist[(int64_t)c * E + e0 + u] = carry[u] + incl - v[q][u];
+                    if (c < nchunks && e0 + u < E) chunk_hist[(int64_t)(e0 + u) * nchunks + c] = carry[u] + incl - v[q][u];
                     carry[u] += __builtin_amdgcn_readlane(incl, kWave - 1);
                 }
             }
@@ -138,14 +139,14 @@ __global__ __launch_bounds__(1024) void plan_scan_kernel(int32_t* __restrict__ c
 // (from chunk_wave_counts); they are turned into per-wave running bases.
 template <typename IdxT, int PERWAVE>
 __device__ void chunk_rank_and_write(const IdxT* idx, int64_t n, int k, int E, int C, int64_t chunk_base,
-                                     const int32_t* chunk_excl /* [E] for this chunk */,
+                                     const int32_t* chunk_excl /* this chunk's entry of expert 0 */, int chunk_pitch,
                                      const int32_t* offsets, int* s_cnt, int32_t* slot, int32_t* token_map,
                                      int32_t* row_src, int32_t* row_of) {
     const int lane = lane_id();
     const int wave = threadIdx.x >> 6;
     // per-wave running base = chunk base + counts of the earlier waves
     for (int e = threadIdx.x; e < E; e += 256) {
-        int run = chunk_excl[e];
+        int run = chunk_excl[(int64_t)e * chunk_pitch];
         for (int w = 0; w < 4; ++w) {
             const int v = s_cnt[w * E + e];
             s_cnt[w * E + e] = run;
@@ -209,7 +210,7 @@ __global__ __launch_bounds__(256) void plan_rank_kernel(const IdxT* __restrict__
     const int64_t chunk_base = (int64_t)blockIdx.x * kPlanChunk;
     chunk_wave_counts<IdxT, kPlanChunk / 4>(idx, n, E, chunk_base, s_cnt, &bad);
     if (bad) status[0] = 1;
-    chunk_rank_and_write<IdxT, kPlanChunk / 4>(idx, n, k, E, C, chunk_base, chunk_excl + (int64_t)blockIdx.x * E, offsets, s_cnt, slot,
+    chunk_rank_and_write<IdxT, kPlanChunk / 4>(idx, n, k, E, C, chunk_base, chunk_excl + blockIdx.x, (int)gridDim.x, offsets, s_cnt, slot,
                          token_map, row_src, row_of);
     // empty slots and unused compact rows
     const int64_t stride = (int64_t)gridDim.x * 256;
@@ -245,7 +246,7 @@ __global__ __launch_bounds__(256) void plan_single_kernel(const IdxT* idx, int64
     __syncthreads();
     scan_totals(chunk_hist, 1, E, C, hist, kept, offsets, s_tot);
     __threadfence_block();
-    chunk_rank_and_write<IdxT, kPlanSingle / 4>(idx, n, k, E, C, 0, chunk_hist, offsets, s_cnt, slot, token_map, row_src,
+    chunk_rank_and_write<IdxT, kPlanSingle / 4>(idx, n, k, E, C, 0, chunk_hist, 1, offsets, s_cnt, slot, token_map, row_src,
                                                 row_of);
     const int64_t ec = (int64_t)E * C;
     for (int64_t i = threadIdx.x; i < ec; i += 256) {
