@@ -107,6 +107,8 @@ _SIGNATURES = {
                             c_void_p]),
     "ats_row_dot": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_int64, c_int, c_int,
                             c_void_p]),
+    "ats_row_dot_copy": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_int64, c_int,
+                                 c_int, c_void_p]),
     "ats_select_topk_per_sequence": (c_int, [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p]),
     "ats_scatter_add_rows": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int, c_void_p]),
     "ats_kth_value_mask": (c_int, [c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_size_t, c_void_p]),

@@ -11,12 +11,13 @@
 
 namespace ats {
 
-// One wave per token row; 16-byte loads; weight vector re-read from L2.
+// One wave per token row; 16-byte loads; weight vector re-read from L2.  copy_out (optional): the rows are also
+// written there as they pass, which starts a residual output without a second pass over x.
 template <typename T>
 __global__ __launch_bounds__(256) void row_dot_kernel(const T* __restrict__ x, const T* __restrict__ w,
                                                       const float* __restrict__ bias, float* __restrict__ score,
-                                                      float* __restrict__ prob, float temperature, int64_t Tn, int H,
-                                                      bool vec) {
+                                                      float* __restrict__ prob, float temperature,
+                                                      T* __restrict__ copy_out, int64_t Tn, int H, bool vec) {
     constexpr int V = Elem<T>::kVec;
     const int lane = lane_id();
     const int64_t wave = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
@@ -26,15 +27,21 @@ __global__ __launch_bounds__(256) void row_dot_kernel(const T* __restrict__ x, c
         if (vec) {
             const uint4* xr = reinterpret_cast<const uint4*>(x + t * H);
             const uint4* wr = reinterpret_cast<const uint4*>(w);
+            uint4* cr = copy_out ? reinterpret_cast<uint4*>(copy_out + t * H) : nullptr;
             for (int v = lane; v < H / V; v += kWave) {
                 float a[V], b[V];
-                Elem<T>::unpack(xr[v], a);
+                const uint4 xv = xr[v];
+                if (cr) cr[v] = xv;
+                Elem<T>::unpack(xv, a);
                 Elem<T>::unpack(wr[v], b);
 #pragma unroll
                 for (int j = 0; j < V; ++j) acc += a[j] * b[j];
             }
         } else {
-            for (int h = lane; h < H; h += kWave) acc += Elem<T>::load(x + t * H + h) * Elem<T>::load(w + h);
+            for (int h = lane; h < H; h += kWave) {
+                if (copy_out) copy_out[t * H + h] = x[t * H + h];
+                acc += Elem<T>::load(x + t * H + h) * Elem<T>::load(w + h);
+            }
         }
         acc = wave_sum(acc);
         if (lane == 0) {
@@ -334,8 +341,14 @@ __global__ __launch_bounds__(256) void swiglu_mul_kernel(const T* __restrict__ g
 
 extern "C" int ats_row_dot(const void* x, const void* w, const float* bias, float* score, float* prob,
                            float temperature, int64_t T, int H, int dtype, ats_stream_t stream) {
+    return ats_row_dot_copy(x, w, bias, score, prob, temperature, nullptr, T, H, dtype, stream);
+}
+
+extern "C" int ats_row_dot_copy(const void* x, const void* w, const float* bias, float* score, float* prob,
+                                float temperature, void* copy_out, int64_t T, int H, int dtype, ats_stream_t stream) {
     using namespace ats;
     ATS_REQUIRE(T >= 0 && H > 0, ATS_ERR_INVALID_ARG, "ats_row_dot: T=%lld H=%d", (long long)T, H);
+    ATS_REQUIRE(!copy_out || copy_out != x, ATS_ERR_INVALID_ARG, "ats_row_dot_copy: the copy must not alias x");
     ATS_REQUIRE(dtype == ATS_F32 || dtype == ATS_BF16, ATS_ERR_UNSUPPORTED, "ats_row_dot: dtype tag %d", dtype);
     ATS_REQUIRE(!prob || temperature > 0.f, ATS_ERR_INVALID_ARG, "ats_row_dot: temperature %g", temperature);
     if (T == 0) return ATS_OK;
@@ -343,15 +356,15 @@ extern "C" int ats_row_dot(const void* x, const void* w, const float* bias, floa
     int64_t blocks = (T + 3) / 4;
     if (blocks > 16384) blocks = 16384;
     const int V = dtype == ATS_F32 ? 4 : 8;
-    const bool vec = H % V == 0 && aligned16(x) && aligned16(w);
+    const bool vec = H % V == 0 && aligned16(x) && aligned16(w) && (!copy_out || aligned16(copy_out));
     if (dtype == ATS_F32)
         hipLaunchKernelGGL((row_dot_kernel<float>), dim3((unsigned)blocks), dim3(256), 0, as_stream(stream),
                            static_cast<const float*>(x), static_cast<const float*>(w), bias, score, prob, temperature,
-                           T, H, vec);
+                           static_cast<float*>(copy_out), T, H, vec);
     else
         hipLaunchKernelGGL((row_dot_kernel<bf16_t>), dim3((unsigned)blocks), dim3(256), 0, as_stream(stream),
                            static_cast<const bf16_t*>(x), static_cast<const bf16_t*>(w), bias, score, prob,
-                           temperature, T, H, vec);
+                           temperature, static_cast<bf16_t*>(copy_out), T, H, vec);
     ATS_CHECK_LAUNCH("ats_row_dot");
     return ATS_OK;
 }

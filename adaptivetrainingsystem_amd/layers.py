@@ -704,11 +704,15 @@ class MoDMoEBlock(nn.Module):
     def forward(self, x: torch.Tensor):
         B, L, H = x.shape
         keep = int(L * self.keep_fraction)
-        scores = ops.row_dot(x, _as_dtype(self.router.weight, x.dtype))
+        grad = _wants_grad(x, *self.moe.parameters())
+        x_rows = x.reshape(-1, H)
+        if grad:
+            scores = ops.row_dot(x, _as_dtype(self.router.weight, x.dtype))
+        else:       # the pass that scores the tokens also writes the copy of x that the output starts as
+            scores, out = ops.row_dot(x, _as_dtype(self.router.weight, x.dtype), want_copy=True)
         sel = ops.select_topk_per_sequence(scores.view(B, L), keep)
         self.last_selected = sel
-        x_rows = x.reshape(-1, H)
-        if _wants_grad(x, *self.moe.parameters()):
+        if grad:
             # the selection is discrete, so the score weight gets no gradient (as in the composition the
             # benchmark defines); tokens, gate and experts get theirs through the gather / scatter pair
             gathered = ag.GatherRowsFunction.apply(x_rows, sel)
@@ -717,7 +721,6 @@ class MoDMoEBlock(nn.Module):
             return out.view(B, L, H), aux
         gathered = ops.gather_rows(x_rows, sel)
         delta, aux = self.moe(gathered.view(1, B * keep, H))
-        out = x_rows.clone()
         ops.scatter_add_rows(out, sel, delta.view(-1, H))
         return out.view(B, L, H), aux
 

@@ -446,8 +446,9 @@ def combine_partials(parts: torch.Tensor, row_of: torch.Tensor, weights: torch.T
 
 # --------------------------------------------------------------------------- MoD helpers
 def row_dot(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = None, temperature: float = 1.0,
-            want_prob: bool = False):
-    """score[t] = x[t,:] . w (+ bias); optionally sigmoid(score / temperature)."""
+            want_prob: bool = False, want_copy: bool = False):
+    """score[t] = x[t,:] . w (+ bias); optionally sigmoid(score / temperature).  want_copy: the same pass also
+    writes a copy of the rows ([T, H], returned last), the start of a residual output."""
     _need_gpu(x, w, bias)
     x2 = x.reshape(-1, x.shape[-1]).contiguous()
     T, H = x2.shape
@@ -458,9 +459,13 @@ def row_dot(x: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor] = Non
         bias = bias.reshape(-1).to(torch.float32).contiguous()
     score = torch.empty(T, dtype=torch.float32, device=x.device)
     prob = torch.empty(T, dtype=torch.float32, device=x.device) if want_prob else None
-    check(_lib.load().ats_row_dot(x2.data_ptr(), w.data_ptr(), _ptr(bias), score.data_ptr(), _ptr(prob),
-                                  float(temperature), T, H, _tag(x2), _stream()), "ats_row_dot")
-    return (score, prob) if want_prob else score
+    copy = torch.empty_like(x2) if want_copy else None
+    check(_lib.load().ats_row_dot_copy(x2.data_ptr(), w.data_ptr(), _ptr(bias), score.data_ptr(), _ptr(prob),
+                                       float(temperature), _ptr(copy), T, H, _tag(x2), _stream()), "ats_row_dot_copy")
+    res = (score, prob) if want_prob else (score,)
+    if want_copy:
+        res = res + (copy,)
+    return res if len(res) > 1 else res[0]
 
 
 def select_topk_per_sequence(scores: torch.Tensor, keep: int) -> torch.Tensor:

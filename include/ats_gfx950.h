@@ -226,6 +226,11 @@ int ats_combine_partials(const float* parts, int n_parts, int64_t part_stride, c
  * (MoDRouter.forward, model.py:926-936). */
 int ats_row_dot(const void* x, const void* w, const float* bias, float* score, float* prob,
                 float temperature, int64_t T, int H, int dtype, ats_stream_t stream);
+/* The same pass also writes the rows to copy_out [T, H] (optional, must not alias x): the residual
+ * output of a Mixture-of-Depths block starts as a copy of its input (tokens that skip the block pass
+ * through, model.py:1366-1404), and the scores read every row anyway. */
+int ats_row_dot_copy(const void* x, const void* w, const float* bias, float* score, float* prob,
+                     float temperature, void* copy_out, int64_t T, int H, int dtype, ats_stream_t stream);
 /* Per sequence, positions of the `keep` largest scores (lower position first
  * among equals), written in ascending order as flat token ids b*L+pos:
  * sel[B*keep] int32.  L <= 8192. */

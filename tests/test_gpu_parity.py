@@ -888,3 +888,21 @@ def test_grouped_down_dgrad_with_swiglu_gradient(ops, gpu, counts, H, I, dtype):
     assert torch.all(dgu[n:] == 3.0) and same_bits(dgu[:n], two[:n])
     small = torch.tensor([40] * E, dtype=torch.int32, device=gpu)
     assert ops.grouped_down_dgrad_dsilu(dy, tab, gu, start, small, 40 * E, H, I) is None
+
+
+@pytest.mark.parametrize("T,H,dtype", [(300, 2048, torch.bfloat16), (17, 33, torch.bfloat16), (64, 516, torch.float32),
+                                       (5, 7, torch.float32)])
+def test_row_dot_with_copy(ops, gpu, T, H, dtype):
+    """The MoD score pass that also writes the rows it reads: the same scores bit for bit, an exact copy."""
+    x = torch.randn(T, H, generator=gen(91)).to(dtype).to(gpu)
+    w = torch.randn(H, generator=gen(92)).to(dtype).to(gpu)
+    plain = ops.row_dot(x, w)
+    score, prob, copy = ops.row_dot(x, w, temperature=0.7, want_prob=True, want_copy=True)
+    assert same_bits(score, plain)
+    assert copy.data_ptr() != x.data_ptr() and torch.equal(copy, x)
+    assert rel_err(prob, torch.sigmoid(plain.cpu().double() / 0.7)) <= 1e-6
+    score2, copy2 = ops.row_dot(x, w, want_copy=True)
+    assert same_bits(score2, plain) and torch.equal(copy2, x)
+    lib = __import__("adaptivetrainingsystem_amd._lib", fromlist=["load"]).load()
+    assert lib.ats_row_dot_copy(x.data_ptr(), w.data_ptr(), None, score.data_ptr(), None, 1.0, x.data_ptr(), T, H,
+                                0 if dtype == torch.float32 else 1, None) != 0       # the copy may not alias x
