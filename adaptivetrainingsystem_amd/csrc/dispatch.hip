@@ -355,12 +355,16 @@ __global__ __launch_bounds__(256) void combine_kernel(const TY* __restrict__ y, 
 // PARTS: y is n_parts float32 partial results part_stride elements apart (a down projection split
 // along K); an expert row is their sum in slice order, rounded to the output type like the unsplit
 // projection's result, before the weighting.
+// out_rows (optional): token t's sum is rounded to the output type and added onto row out_rows[t] of `out`
+// (skipped where negative) instead of being written to row t: the combine followed by a scatter-add of the
+// token-major result, without the intermediate tensor.
 template <typename TY, typename TO, int MAXK, bool PARTS = false>
 __global__ __launch_bounds__(256) void combine_vec_kernel(const TY* __restrict__ y, const int32_t* __restrict__ row_of,
                                                           const float* __restrict__ w,
                                                           const TO* __restrict__ residual, TO* __restrict__ out,
                                                           int64_t T, int k, int H, int cols_per_wave,
-                                                          int n_parts = 1, int64_t part_stride = 0) {
+                                                          int n_parts = 1, int64_t part_stride = 0,
+                                                          const int32_t* __restrict__ out_rows = nullptr) {
     constexpr int V = 8;  // columns per lane per step (one 16-byte bf16 vector or two float vectors)
     const int lane = lane_id();
     const int64_t wave = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
@@ -371,6 +375,8 @@ __global__ __launch_bounds__(256) void combine_vec_kernel(const TY* __restrict__
         const int64_t t = item / pieces;
         const int h_first = (int)(item - t * pieces) * cols_per_wave;
         const int h_end = min(H, h_first + cols_per_wave);
+        const int64_t t_out = out_rows ? (int64_t)out_rows[t] : t;
+        if (t_out < 0) continue;
         int my_row = -1;
         float my_w = 0.f;
         if (lane < k) {
@@ -444,7 +450,21 @@ __global__ __launch_bounds__(256) void combine_vec_kernel(const TY* __restrict__
 #pragma unroll
                 for (int j = 0; j < V; ++j) acc[j] = ((rv[j]) + (acc[j]));
             }
-            TO* o = out + t * H + h0;
+            TO* o = out + t_out * H + h0;
+            if (out_rows) {
+                // the sum as the token-major result would hold it, then the addition a scatter-add performs
+                float ov[V];
+                if constexpr (sizeof(TO) == 2) {
+                    Elem<TO>::unpack(*reinterpret_cast<const uint4*>(o), ov);
+#pragma unroll
+                    for (int j = 0; j < V; ++j) acc[j] = ((ov[j]) + (bf16_bits_to_float(float_to_bf16_bits(acc[j]))));
+                } else {
+                    Elem<TO>::unpack(*reinterpret_cast<const uint4*>(o), ov);
+                    Elem<TO>::unpack(*reinterpret_cast<const uint4*>(o + 4), ov + 4);
+#pragma unroll
+                    for (int j = 0; j < V; ++j) acc[j] = ((ov[j]) + (acc[j]));
+                }
+            }
             if constexpr (sizeof(TO) == 2) {
                 *reinterpret_cast<uint4*>(o) = Elem<TO>::pack(acc);
             } else {
@@ -466,8 +486,8 @@ static int combine_cols_per_wave(int64_t T, int H) {
 }
 
 template <typename TY, typename TO>
-static void launch_combine(const void* y, const int32_t* row_of, const float* w, const void* residual, void* out,
-                           int64_t T, int k, int H, hipStream_t s) {
+static bool launch_combine(const void* y, const int32_t* row_of, const float* w, const void* residual, void* out,
+                           int64_t T, int k, int H, hipStream_t s, const int32_t* out_rows = nullptr) {
     const int cols = combine_cols_per_wave(T, H);
     int64_t blocks = (T * ((H + cols - 1) / cols) + 3) / 4;
     if (blocks > 16384) blocks = 16384;
@@ -475,18 +495,20 @@ static void launch_combine(const void* y, const int32_t* row_of, const float* w,
     const TO* rp = static_cast<const TO*>(residual);
     TO* op = static_cast<TO*>(out);
     const bool vec = H % 8 == 0 && aligned16(y) && aligned16(out) && (!residual || aligned16(residual)) && k <= 8;
+    if (out_rows && !vec) return false;      // the scattering form exists for the vector kernel only
     if (vec && k <= 2)
         hipLaunchKernelGGL((combine_vec_kernel<TY, TO, 2>), dim3((unsigned)blocks), dim3(256), 0, s, yp, row_of, w, rp,
-                           op, T, k, H, cols);
+                           op, T, k, H, cols, 1, (int64_t)0, out_rows);
     else if (vec && k <= 4)
         hipLaunchKernelGGL((combine_vec_kernel<TY, TO, 4>), dim3((unsigned)blocks), dim3(256), 0, s, yp, row_of, w, rp,
-                           op, T, k, H, cols);
+                           op, T, k, H, cols, 1, (int64_t)0, out_rows);
     else if (vec)
         hipLaunchKernelGGL((combine_vec_kernel<TY, TO, 8>), dim3((unsigned)blocks), dim3(256), 0, s, yp, row_of, w, rp,
-                           op, T, k, H, cols);
+                           op, T, k, H, cols, 1, (int64_t)0, out_rows);
     else
         hipLaunchKernelGGL((combine_kernel<TY, TO>), dim3((unsigned)blocks), dim3(256), 0, s, yp, row_of, w, rp, op, T,
                            k, H);
+    return true;
 }
 
 // out[i] = sum over the n_parts partial results of parts[s * part_stride + i], added in slice order.
@@ -790,6 +812,34 @@ extern "C" int ats_invert_token_map(const int32_t* token_map, int64_t n_slots, i
                            n_assign);
         ATS_CHECK_LAUNCH("ats_invert_token_map");
     }
+    return ATS_OK;
+}
+
+extern "C" int ats_combine_scatter_add(const void* y, const int32_t* row_of, const float* w, const int32_t* out_rows,
+                                       void* out, int64_t T, int k, int H, int y_dtype, int out_dtype,
+                                       ats_stream_t stream) {
+    using namespace ats;
+    ATS_REQUIRE(T >= 0 && k > 0 && H > 0, ATS_ERR_INVALID_ARG, "ats_combine_scatter_add: T=%lld k=%d H=%d", (long long)T,
+                k, H);
+    ATS_REQUIRE((y_dtype == ATS_F32 || y_dtype == ATS_BF16) && (out_dtype == ATS_F32 || out_dtype == ATS_BF16),
+                ATS_ERR_UNSUPPORTED, "ats_combine_scatter_add: dtype tags %d/%d", y_dtype, out_dtype);
+    if (T == 0) return ATS_OK;
+    ATS_REQUIRE(y && row_of && w && out && out_rows, ATS_ERR_INVALID_ARG, "ats_combine_scatter_add: null pointer");
+    ATS_REQUIRE(k <= 8 && H % 8 == 0 && aligned16(y) && aligned16(out), ATS_ERR_UNSUPPORTED,
+                "ats_combine_scatter_add: k=%d (at most 8), H=%d (a multiple of 8), 16-byte aligned operands; use "
+                "ats_combine and ats_scatter_add_rows", k, H);
+    hipStream_t s = as_stream(stream);
+    bool ok;
+    if (y_dtype == ATS_F32 && out_dtype == ATS_F32)
+        ok = launch_combine<float, float>(y, row_of, w, nullptr, out, T, k, H, s, out_rows);
+    else if (y_dtype == ATS_BF16 && out_dtype == ATS_BF16)
+        ok = launch_combine<bf16_t, bf16_t>(y, row_of, w, nullptr, out, T, k, H, s, out_rows);
+    else if (y_dtype == ATS_F32 && out_dtype == ATS_BF16)
+        ok = launch_combine<float, bf16_t>(y, row_of, w, nullptr, out, T, k, H, s, out_rows);
+    else
+        ok = launch_combine<bf16_t, float>(y, row_of, w, nullptr, out, T, k, H, s, out_rows);
+    ATS_REQUIRE(ok, ATS_ERR_UNSUPPORTED, "ats_combine_scatter_add: sizes outside the vector kernel");
+    ATS_CHECK_LAUNCH("ats_combine_scatter_add");
     return ATS_OK;
 }
 

@@ -472,7 +472,11 @@ class MoEFFNLayer(nn.Module):
             self._wcache_key = key
         return self._wcache
 
-    def forward(self, x: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    def forward(self, x: torch.Tensor, add_onto: Optional[Tuple[torch.Tensor, torch.Tensor]] = None
+                ) -> Tuple[torch.Tensor, torch.Tensor]:
+        """add_onto = (target [N, H], rows int32 [tokens]) (inference only): the layer's output for token t is
+        added onto target[rows[t]] in place, as target.index_add_ of the returned tensor would, and `target` is
+        returned in its place; for a block that runs the layer on a subset of a longer sequence."""
         if x.dim() != 3 or x.shape[-1] != self.hidden_size:
             raise AtsError(f"MoEFFNLayer: expected [batch, seq, {self.hidden_size}], got {tuple(x.shape)}")
         if len(self.experts) != self.num_experts or self.gate.weight.shape[0] != self.num_experts:
@@ -493,6 +497,8 @@ class MoEFFNLayer(nn.Module):
         params = [self.gate.weight] + [ex.gate_up_proj.weight for ex in self.experts] + \
                  [ex.down_proj.weight for ex in self.experts]
         if _wants_grad(x, *params):
+            if add_onto is not None:
+                raise AtsError("MoEFFNLayer: add_onto is an inference option (autograd adds the output itself)")
             stats: Dict[str, Any] = {}
             cfg = {"top_k": k, "temperature": self.routing_temperature, "variant": ag.moe_variant(self.routing),
                    "capacity": C, "load_balancing_weight": self.load_balancing_weight,
@@ -533,15 +539,26 @@ class MoEFFNLayer(nn.Module):
         else:
             y = torch.zeros(1, H, dtype=x.dtype, device=x.device)
         with stage(tm, "combine"):
-            if y.dim() == 3:
-                out = ops.combine_partials(y, plan["row_of"], route["weights"], T, k, x.dtype)
-            else:
-                out = ops.combine(y, plan["row_of"], route["weights"], T, k, out_dtype=x.dtype)
+            out = None
+            if add_onto is not None:
+                target, rows_to = add_onto
+                if target.dim() != 2 or target.shape[1] != H or target.dtype != x.dtype or rows_to.numel() != T:
+                    raise AtsError("MoEFFNLayer: add_onto needs a [rows, hidden] tensor of x's dtype and one row id per token")
+                if y.dim() == 2 and ops.combine_scatter_add(y, plan["row_of"], route["weights"], T, k, target, rows_to):
+                    out = target
+            if out is None:
+                if y.dim() == 3:
+                    out = ops.combine_partials(y, plan["row_of"], route["weights"], T, k, x.dtype)
+                else:
+                    out = ops.combine(y, plan["row_of"], route["weights"], T, k, out_dtype=x.dtype)
+                if add_onto is not None:        # sizes outside the fused kernel: the two-step route
+                    ops.scatter_add_rows(add_onto[0], add_onto[1], out)
+                    out = add_onto[0]
 
         self.last_plan = {"logits": logits, "capacity": C, **route, **plan}
         if self.training:
             self._update_routing_stats(plan, T)
-        return out.view(B, L, H), route["aux"][0]
+        return (out if add_onto is not None else out.view(B, L, H)), route["aux"][0]
 
     def _update_routing_stats(self, plan, total_tokens: int) -> None:
         hist = plan["hist"].cpu()
@@ -720,8 +737,7 @@ class MoDMoEBlock(nn.Module):
             out = ag.ScatterAddRowsFunction.apply(x_rows, sel, delta.view(-1, H))
             return out.view(B, L, H), aux
         gathered = ops.gather_rows(x_rows, sel)
-        delta, aux = self.moe(gathered.view(1, B * keep, H))
-        ops.scatter_add_rows(out, sel, delta.view(-1, H))
+        out, aux = self.moe(gathered.view(1, B * keep, H), add_onto=(out, sel))   # the combine adds onto the copy
         return out.view(B, L, H), aux
 
 

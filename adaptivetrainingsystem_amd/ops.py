@@ -421,6 +421,29 @@ def combine(y: torch.Tensor, row_of: torch.Tensor, weights: torch.Tensor, num_to
     return out
 
 
+def combine_scatter_add(y: torch.Tensor, row_of: torch.Tensor, weights: torch.Tensor, num_tokens: int, k: int,
+                        out: torch.Tensor, out_rows: torch.Tensor) -> bool:
+    """combine whose result is added onto rows out_rows[t] (int32, distinct, negative = skip) of `out` [N, H] in
+    place, with the bits of combine followed by scatter_add_rows.  Returns False (nothing done) when the sizes
+    are outside the vector kernel (k > 8, H not a multiple of 8, unaligned views)."""
+    _need_gpu(y, row_of, weights, out, out_rows)
+    if row_of.dtype != torch.int32 or weights.dtype != torch.float32 or out_rows.dtype != torch.int32:
+        raise AtsError("combine_scatter_add: row_of / out_rows must be int32 and weights float32")
+    if row_of.numel() != num_tokens * k or weights.numel() != num_tokens * k or out_rows.numel() != num_tokens:
+        raise AtsError("combine_scatter_add: row_of/weights must have tokens*k entries, out_rows one per token")
+    y2 = y.reshape(-1, y.shape[-1]).contiguous()
+    H = y2.shape[1]
+    if out.dim() != 2 or out.shape[1] != H or not out.is_contiguous():
+        raise AtsError("combine_scatter_add: out must be a contiguous [rows, H] tensor")
+    if k > 8 or H % 8 or y2.data_ptr() % 16 or out.data_ptr() % 16:
+        return False
+    check(_lib.load().ats_combine_scatter_add(y2.data_ptr(), row_of.contiguous().data_ptr(),
+                                              weights.contiguous().data_ptr(), out_rows.contiguous().data_ptr(),
+                                              out.data_ptr(), num_tokens, int(k), H, _tag(y2), _tag(out), _stream()),
+          "ats_combine_scatter_add")
+    return True
+
+
 def combine_partials(parts: torch.Tensor, row_of: torch.Tensor, weights: torch.Tensor, num_tokens: int, k: int,
                      out_dtype: torch.dtype, residual: Optional[torch.Tensor] = None) -> torch.Tensor:
     """combine over the float32 partial results [S, rows, H] of grouped_down_splitk: an expert row is their

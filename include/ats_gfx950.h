@@ -214,6 +214,13 @@ int ats_sum_partials(const float* parts, int n_parts, int64_t part_stride, void*
  * If residual != NULL, out[t,:] = residual[t,:] + that sum. */
 int ats_combine(const void* y, const int32_t* row_of, const float* w, const void* residual,
                 void* out, int64_t T, int k, int H, int y_dtype, int out_dtype, ats_stream_t stream);
+/* ats_combine whose token-major result is added onto rows of a larger tensor instead of being stored:
+ * out[out_rows[t], :] += round(sum_j w[t,j] * y[row_of[t*k+j], :]) for out_rows[t] >= 0 (distinct rows), the
+ * sum rounded to out_dtype first as the stored result would be; the bits of ats_combine followed by
+ * ats_scatter_add_rows.  For a block that runs the experts on a subset of the tokens and adds the result
+ * onto the residual stream at their positions.  k <= 8, H % 8 == 0, 16-byte aligned operands. */
+int ats_combine_scatter_add(const void* y, const int32_t* row_of, const float* w, const int32_t* out_rows,
+                            void* out, int64_t T, int k, int H, int y_dtype, int out_dtype, ats_stream_t stream);
 /* ats_combine over the partial results of ats_grouped_down_splitk: expert row r is
  * sum_s parts[s*part_stride + r*H + :] (slice order, float32), rounded to out_dtype as the
  * unsplit projection rounds its result, then weighted and summed as above.  k <= 8, H % 8 == 0. */

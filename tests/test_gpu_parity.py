@@ -906,3 +906,33 @@ def test_row_dot_with_copy(ops, gpu, T, H, dtype):
     lib = __import__("adaptivetrainingsystem_amd._lib", fromlist=["load"]).load()
     assert lib.ats_row_dot_copy(x.data_ptr(), w.data_ptr(), None, score.data_ptr(), None, 1.0, x.data_ptr(), T, H,
                                 0 if dtype == torch.float32 else 1, None) != 0       # the copy may not alias x
+
+
+@pytest.mark.parametrize("T,k,H,N,ydt,odt", [(300, 6, 2048, 1000, torch.bfloat16, torch.bfloat16),
+                                             (4200, 2, 2048, 5000, torch.bfloat16, torch.bfloat16),
+                                             (64, 8, 520, 64, torch.float32, torch.float32),
+                                             (129, 3, 64, 400, torch.float32, torch.bfloat16)])
+def test_combine_scatter_add_equals_combine_then_scatter_add(ops, gpu, T, k, H, N, ydt, odt):
+    """The combine that adds its token-major result onto rows of a larger tensor: the bits of combine followed
+    by scatter_add_rows, rows with a negative destination skipped, other rows of the target untouched; sizes
+    outside the vector kernel are declined."""
+    g = gen(95)
+    rows = T * k
+    y = torch.randn(rows, H, generator=g).to(ydt).to(gpu)
+    row_of = torch.randperm(rows, generator=g).int()
+    row_of[torch.rand(rows, generator=g) < 0.1] = -1                   # dropped choices
+    w = torch.rand(T, k, generator=g).to(gpu)
+    dest = torch.randperm(N, generator=g)[:T].int()
+    dest[::17] = -1
+    base = torch.randn(N, H, generator=g).to(odt).to(gpu)
+    row_of, dest = row_of.to(gpu), dest.to(gpu)
+    two = base.clone()
+    ops.scatter_add_rows(two, dest, ops.combine(y, row_of, w, T, k, out_dtype=odt))
+    one = base.clone()
+    assert ops.combine_scatter_add(y, row_of, w, T, k, one, dest)
+    assert same_bits(one, two)
+    untouched = torch.ones(N, dtype=torch.bool)
+    untouched[dest[dest >= 0].long().cpu()] = False
+    assert torch.equal(one[untouched.to(gpu)], base[untouched.to(gpu)])
+    odd = torch.zeros(N, 260, dtype=odt, device=gpu)
+    assert not ops.combine_scatter_add(torch.zeros(rows, 260, dtype=ydt, device=gpu), row_of, w, T, k, odd, dest)
