@@ -113,6 +113,7 @@ _SIGNATURES = {
                                  c_int, c_void_p]),
     "ats_select_topk_per_sequence": (c_int, [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p]),
     "ats_scatter_add_rows": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int, c_void_p]),
+    "ats_kth_value_workspace": (ctypes.c_size_t, [c_int64]),
     "ats_kth_value_mask": (c_int, [c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_size_t, c_void_p]),
     "ats_swiglu_mul": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int, c_void_p]),
     # the reference's launcher names (void return, float32 only)

@@ -261,6 +261,49 @@ __device__ __forceinline__ uint32_t order_key(float f) {
     return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
 }
 
+// One digit of the radix select, by one wave (all 64 lanes): the bin of `hist` (256 counts, ascending digits)
+// in which the running rank falls.  Lane l owns bins 4l .. 4l+3; a prefix sum over the lanes' sums finds the
+// lane, a walk over its four bins the bin.  Returns the bin and updates *rank to the rank inside it.
+__device__ __forceinline__ int kth_find_bin(const unsigned int* hist, long long* rank, int lane) {
+    unsigned int c[4];
+    unsigned int sum = 0;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        c[q] = hist[4 * lane + q];
+        sum += c[q];
+    }
+    const long long incl = (long long)(unsigned int)wave_inclusive_scan((int)sum);
+    const long long before = incl - sum;
+    const long long want = *rank;
+    // the first lane whose inclusive count reaches the rank; the last lane takes what is left (bin 255 then)
+    unsigned long long hit = __ballot(want <= incl);
+    const int owner = hit ? __ffsll((long long)hit) - 1 : 63;
+    int bin = 4 * lane + 3;
+    long long left = want - before;
+    if (lane == owner) {
+        if (left <= (long long)c[0]) {
+            bin = 4 * lane;
+        } else {
+            left -= c[0];
+            if (left <= (long long)c[1]) {
+                bin = 4 * lane + 1;
+            } else {
+                left -= c[1];
+                if (left <= (long long)c[2]) {
+                    bin = 4 * lane + 2;
+                } else {
+                    left -= c[2];
+                }
+            }
+        }
+    }
+    const int b = __builtin_amdgcn_readlane(bin, owner);
+    const int lo = __builtin_amdgcn_readlane((int)(left & 0xffffffffll), owner);
+    const int hi = __builtin_amdgcn_readlane((int)(left >> 32), owner);
+    *rank = ((long long)hi << 32) | (unsigned int)lo;
+    return b;
+}
+
 __global__ __launch_bounds__(1024) void kth_value_kernel(const float* __restrict__ v, int64_t n, int64_t kth,
                                                          uint32_t* __restrict__ key_out,
                                                          long long* __restrict__ count_out) {
@@ -281,15 +324,13 @@ __global__ __launch_bounds__(1024) void kth_value_kernel(const float* __restrict
             if ((key & hi_mask) == prefix) atomicAdd(&hist[(key >> (8 * pass)) & 255u], 1u);
         }
         __syncthreads();
-        if (threadIdx.x == 0) {
+        if (threadIdx.x < 64) {
             long long rank = s_rank;
-            int b = 0;
-            for (; b < 255; ++b) {
-                if (rank <= (long long)hist[b]) break;
-                rank -= hist[b];
+            const int b = kth_find_bin(hist, &rank, (int)threadIdx.x);
+            if (threadIdx.x == 0) {
+                s_rank = rank;
+                s_prefix = prefix | ((uint32_t)b << (8 * pass));
             }
-            s_rank = rank;
-            s_prefix = prefix | ((uint32_t)b << (8 * pass));
         }
         __syncthreads();
     }
@@ -299,6 +340,72 @@ __global__ __launch_bounds__(1024) void kth_value_kernel(const float* __restrict
         // are strictly smaller and the mask keeps the rest
         if (count_out) count_out[0] = (long long)n - kth + s_rank;
     }
+}
+
+// The same select over many workgroups, one launch per digit: every block counts the digit of its share of
+// the values that match the prefix found so far into LDS and adds its 256 counts to the pass's histogram in
+// `ghist` ([4][256], zeroed by the caller).  The prefix is not stored anywhere: the first wave of every block
+// walks the histograms of the passes above its own again (at most three 256-bin searches).
+__device__ __forceinline__ void kth_walk(const unsigned int* ghist, int upto, long long kth, int lane, uint32_t* prefix,
+                                         long long* rank) {
+    uint32_t pre = 0;
+    long long r = kth;
+    for (int q = 3; q > upto; --q) {
+        const int b = kth_find_bin(ghist + q * 256, &r, lane);
+        pre |= (uint32_t)b << (8 * q);
+    }
+    *prefix = pre;
+    *rank = r;
+}
+
+__global__ __launch_bounds__(256) void kth_digit_hist_kernel(const float* __restrict__ v, int64_t n, int64_t kth, int pass,
+                                                             unsigned int* __restrict__ ghist) {
+    __shared__ unsigned int hist[256];
+    __shared__ uint32_t s_prefix;
+    hist[threadIdx.x] = 0;
+    if (threadIdx.x < 64) {
+        uint32_t prefix;
+        long long rank;
+        kth_walk(ghist, pass, kth, (int)threadIdx.x, &prefix, &rank);
+        if (threadIdx.x == 0) s_prefix = prefix;
+    }
+    __syncthreads();
+    const uint32_t prefix = s_prefix;
+    const uint32_t hi_mask = pass == 3 ? 0u : (0xffffffffu << (8 * (pass + 1)));
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
+        const uint32_t key = order_key(v[i]);
+        if ((key & hi_mask) == prefix) atomicAdd(&hist[(key >> (8 * pass)) & 255u], 1u);
+    }
+    __syncthreads();
+    const unsigned int c = hist[threadIdx.x];
+    if (c) atomicAdd(&ghist[pass * 256 + threadIdx.x], c);
+}
+
+__global__ __launch_bounds__(256) void kth_mask_kernel(const float* __restrict__ v, int64_t n, int64_t kth,
+                                                       const unsigned int* __restrict__ ghist,
+                                                       uint32_t* __restrict__ key_out, long long* __restrict__ count_out,
+                                                       float* __restrict__ mask) {
+    __shared__ uint32_t s_thr;
+    if (threadIdx.x < 64) {
+        uint32_t prefix;
+        long long rank;
+        kth_walk(ghist, -1, kth, (int)threadIdx.x, &prefix, &rank);
+        if (threadIdx.x == 0) {
+            s_thr = prefix;
+            if (blockIdx.x == 0) {
+                key_out[0] = prefix;
+                if (count_out) count_out[0] = (long long)n - kth + rank;
+            }
+        }
+    }
+    __syncthreads();
+    const uint32_t thr = s_thr;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
+        mask[i] = order_key(v[i]) >= thr ? 1.0f : 0.0f;
+}
+
+__global__ __launch_bounds__(256) void kth_zero_kernel(unsigned int* __restrict__ ghist) {
+    for (int i = threadIdx.x; i < 4 * 256; i += 256) ghist[i] = 0;
 }
 
 __global__ __launch_bounds__(256) void threshold_mask_kernel(const float* __restrict__ v, int64_t n,
@@ -422,22 +529,44 @@ extern "C" int ats_scatter_add_rows(void* base, const int32_t* rows, const void*
     return ATS_OK;
 }
 
+// Values from which the select runs over many workgroups, and the workspace that takes:
+// key (4 bytes), pad, count (8 bytes), then the four digit histograms.
+static constexpr int64_t kKthMultiBlockMin = 16384;
+static constexpr size_t kKthMultiBlockBytes = 16 + 4 * 256 * sizeof(unsigned int);
+
+extern "C" size_t ats_kth_value_workspace(int64_t n) {
+    return n >= kKthMultiBlockMin && n < (int64_t)INT_MAX ? kKthMultiBlockBytes : 16;
+}
+
 extern "C" int ats_kth_value_mask(const float* v, int64_t n, int64_t kth, float* mask, void* workspace,
                                   size_t workspace_bytes, ats_stream_t stream) {
     using namespace ats;
     ATS_REQUIRE(n >= 0 && (n == 0 || (kth >= 1 && kth <= n)), ATS_ERR_INVALID_ARG,
                 "ats_kth_value_mask: n=%lld kth=%lld", (long long)n, (long long)kth);
     if (n == 0) return ATS_OK;
+    ATS_REQUIRE(n < (int64_t)INT_MAX, ATS_ERR_UNSUPPORTED, "ats_kth_value_mask: n=%lld (below 2^31)", (long long)n);
     ATS_REQUIRE(v && mask, ATS_ERR_INVALID_ARG, "ats_kth_value_mask: null pointer");
     ATS_REQUIRE(workspace && workspace_bytes >= sizeof(uint32_t), ATS_ERR_WORKSPACE,
                 "ats_kth_value_mask: workspace of at least 4 bytes needed");
     hipStream_t s = as_stream(stream);
     uint32_t* key = static_cast<uint32_t*>(workspace);
     long long* count = workspace_bytes >= 16 ? reinterpret_cast<long long*>(static_cast<char*>(workspace) + 8) : nullptr;
-    hipLaunchKernelGGL(kth_value_kernel, dim3(1), dim3(1024), 0, s, v, n, kth, key, count);
-    ATS_CHECK_LAUNCH("ats_kth_value_mask(select)");
     int64_t blocks = (n + 255) / 256;
     if (blocks > 4096) blocks = 4096;
+    if (n >= kKthMultiBlockMin && n < (int64_t)INT_MAX && workspace_bytes >= kKthMultiBlockBytes) {
+        // one launch per digit over many workgroups; a smaller workspace keeps the single-workgroup select
+        unsigned int* ghist = reinterpret_cast<unsigned int*>(static_cast<char*>(workspace) + 16);
+        int64_t hb = (n + 2047) / 2048;          // eight values per thread
+        if (hb > 1024) hb = 1024;
+        hipLaunchKernelGGL(kth_zero_kernel, dim3(1), dim3(256), 0, s, ghist);
+        for (int pass = 3; pass >= 0; --pass)
+            hipLaunchKernelGGL(kth_digit_hist_kernel, dim3((unsigned)hb), dim3(256), 0, s, v, n, kth, pass, ghist);
+        hipLaunchKernelGGL(kth_mask_kernel, dim3((unsigned)blocks), dim3(256), 0, s, v, n, kth, ghist, key, count, mask);
+        ATS_CHECK_LAUNCH("ats_kth_value_mask(multi)");
+        return ATS_OK;
+    }
+    hipLaunchKernelGGL(kth_value_kernel, dim3(1), dim3(1024), 0, s, v, n, kth, key, count);
+    ATS_CHECK_LAUNCH("ats_kth_value_mask(select)");
     hipLaunchKernelGGL(threshold_mask_kernel, dim3((unsigned)blocks), dim3(256), 0, s, v, n, key, mask);
     ATS_CHECK_LAUNCH("ats_kth_value_mask(mask)");
     return ATS_OK;

@@ -524,11 +524,13 @@ def kth_value_mask(values: torch.Tensor, kth: int, return_count: bool = False):
         raise AtsError("kth_value_mask: values must be float32")
     v = values.contiguous()
     mask = torch.empty_like(v)
-    ws = torch.zeros(2, dtype=torch.int64, device=v.device) if v.numel() == 0 else \
-        torch.empty(2, dtype=torch.int64, device=v.device)
-    check(_lib.load().ats_kth_value_mask(v.data_ptr(), v.numel(), int(kth), mask.data_ptr(), ws.data_ptr(), 16,
-                                         _stream()), "ats_kth_value_mask")
-    return (mask, ws[1:]) if return_count else mask
+    lib = _lib.load()
+    ws_bytes = int(lib.ats_kth_value_workspace(v.numel()))       # 16 bytes, or with room for the digit histograms
+    ws = torch.zeros(ws_bytes // 8, dtype=torch.int64, device=v.device) if v.numel() == 0 else \
+        torch.empty(ws_bytes // 8, dtype=torch.int64, device=v.device)
+    check(lib.ats_kth_value_mask(v.data_ptr(), v.numel(), int(kth), mask.data_ptr(), ws.data_ptr(), ws_bytes,
+                                 _stream()), "ats_kth_value_mask")
+    return (mask, ws[1:2]) if return_count else mask
 
 
 def swiglu_mul(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:

@@ -251,7 +251,10 @@ int ats_scatter_add_rows(void* base, const int32_t* rows, const void* delta, int
  * branch of MoDRouter.forward (model.py:984-990, kthvalue threshold).
  * workspace: at least 4 bytes of device memory, 8-byte aligned; when it holds 16 or
  * more, the int64 at byte offset 8 receives the number of ones in the mask (the
- * "computed tokens" statistic of model.py:990-995). */
+ * "computed tokens" statistic of model.py:990-995).  With the ats_kth_value_workspace(n) bytes
+ * (16, or 4112 from 16384 values on) the radix select runs over many workgroups, one launch per
+ * digit, instead of in one workgroup; n < 2^31. */
+size_t ats_kth_value_workspace(int64_t n);
 int ats_kth_value_mask(const float* v, int64_t n, int64_t kth, float* mask, void* workspace,
                        size_t workspace_bytes, ats_stream_t stream);
 

@@ -936,3 +936,31 @@ def test_combine_scatter_add_equals_combine_then_scatter_add(ops, gpu, T, k, H, 
     assert torch.equal(one[untouched.to(gpu)], base[untouched.to(gpu)])
     odd = torch.zeros(N, 260, dtype=odt, device=gpu)
     assert not ops.combine_scatter_add(torch.zeros(rows, 260, dtype=ydt, device=gpu), row_of, w, T, k, odd, dest)
+
+
+@pytest.mark.parametrize("n,kth", [(1, 1), (150, 75), (5000, 1), (5000, 5000), (16384, 8000), (40000, 1), (40000, 40000),
+                                   (100003, 50002), (300000, 299999)])
+def test_kth_value_mask_both_selects(ops, gpu, n, kth):
+    """mask = values >= the kth smallest value (model.py:984-990), by the single-workgroup radix select (small n,
+    or a 16-byte workspace) and by the one-launch-per-digit select over many workgroups (from 16384 values on):
+    against torch.kthvalue on the CPU, with heavy ties, negative values, signed zeros and infinities; the count of
+    ones is the mask's sum; both selects agree."""
+    g = gen(400 + n % 97)
+    v = torch.randn(n, generator=g)
+    v[torch.rand(n, generator=g) < 0.3] = 0.25                 # a third of the values tie
+    if n >= 150:
+        v[:4] = torch.tensor([float("inf"), float("-inf"), 0.0, -0.0])
+    thr = torch.kthvalue(v, kth).values
+    ref = (v >= thr).float()
+    mask, count = ops.kth_value_mask(v.to(gpu), kth, return_count=True)
+    assert torch.equal(mask.cpu(), ref)
+    assert count.item() == int(ref.sum().item())
+    # the single-workgroup select through the C ABI (a 16-byte workspace keeps it at any size)
+    lib = __import__("adaptivetrainingsystem_amd._lib", fromlist=["load"]).load()
+    vg = v.to(gpu)
+    m2 = torch.empty_like(vg)
+    ws = torch.empty(2, dtype=torch.int64, device=gpu)
+    assert lib.ats_kth_value_mask(vg.data_ptr(), n, kth, m2.data_ptr(), ws.data_ptr(), 16, None) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(m2.cpu(), ref) and ws[1].item() == int(ref.sum().item())
+    assert int(lib.ats_kth_value_workspace(n)) == (16 if n < 16384 else 16 + 4096)
