@@ -941,12 +941,13 @@ __global__ __launch_bounds__(512) void grouped_gemm_dma16_kernel(GroupedArgs p) 
     const int drow = lane >> 3;
     const int dchunk = (lane & 7) ^ drow ^ (wave & 1);
     unsigned ao[NIA], bo[NIB];
+    // the gather indices are asked for first: the weight loads issued below are in flight while they arrive
+    int a_idx[NIA];
 #pragma unroll
     for (int j = 0; j < NIA; ++j) {
         int m = tc.mt * BM + (j * NW + wave) * 8 + drow;
         m = m < count ? m : count - 1;
-        int64_t src = gather ? (int64_t)(p.a_rows[arow0 + m] / p.a_row_div) : (int64_t)(m - tc.mt * BM);
-        ao[j] = (unsigned)(src * p.lda * ES + dchunk * 16);
+        a_idx[j] = gather ? p.a_rows[arow0 + m] : m - tc.mt * BM;
     }
 #pragma unroll
     for (int j = 0; j < NIB; ++j) {
@@ -1098,12 +1099,17 @@ __global__ __launch_bounds__(512) void grouped_gemm_dma16_kernel(GroupedArgs p) 
         if (kt < nk) D16_ITER(kt, 0, H0, H1);                                           \
     }
 
-    D16_ISSUE_A(0, 0);
     D16_ISSUE_B(0, 0);
-    D16_ISSUE_A(min(1, nk - 1), A_STAGE);
     D16_ISSUE_B(min(1, nk - 1), 1);
+#pragma unroll
+    for (int j = 0; j < NIA; ++j) {
+        const int64_t src = gather ? (int64_t)(a_idx[j] / p.a_row_div) : (int64_t)a_idx[j];
+        ao[j] = (unsigned)(src * p.lda * ES + dchunk * 16);
+    }
+    D16_ISSUE_A(0, 0);
+    D16_ISSUE_A(min(1, nk - 1), A_STAGE);
     D16_ISSUE_A(min(2, nk - 1), 2 * A_STAGE);
-    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(2 * NIA + NIB) : "memory");
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(2 * NIA) : "memory");
     int sa_cur = 0, sa_nxt = A_STAGE;
     // rows of the expert in this wave's 128-row share of the tile (wave-uniform)
     const int wave_rows = count - (tc.mt * BM + wm * (BM / WM));
