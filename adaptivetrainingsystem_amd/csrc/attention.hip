@@ -43,6 +43,18 @@ typedef __attribute__((address_space(3))) att_tr_t* att_lds_tr_ptr_t;
 constexpr int kAttBN = 64;    // keys per tile
 constexpr int att_rows_per_block(int nt) { return nt / 64 * 32; }
 
+// Exchange with the lane 32 positions away by one VALU swap of the wave's halves (v_permlane32_swap) instead of a
+// shuffle through the LDS crossbar, whose result a wave can only wait for together with every fragment read it
+// has in flight.  All 64 lanes must be active.  Same bits as the shuffle forms (max and sum are symmetric).
+__device__ __forceinline__ float xor32_max(float v) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float xor32_sum(float v) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
 __device__ __forceinline__ af32x16_t att_mma(const au32x4_t& a, const au32x4_t& b, af32x16_t c) {
     union {
         au32x4_t u;
@@ -314,7 +326,7 @@ __device__ __forceinline__ void attention_q_tile(const bf16_t* __restrict__ q, c
             for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
                 for (int v = 0; v < 16; ++v) mx = fmaxf(mx, acc_s[kb][v]);
-            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+            mx = xor32_max(mx);
             // The reference point of the exponentials follows the running maximum lazily: it moves only when
             // the maximum has grown by more than kLazy (log2 units), so p <= 2^kLazy, which float32 sums and
             // bf16 operands hold without loss of relative precision, and the rescaling of the output
@@ -393,7 +405,7 @@ __device__ __forceinline__ void attention_q_tile(const bf16_t* __restrict__ q, c
         __syncthreads();
     }
 
-    l_run += __shfl_xor(l_run, 32, 64);
+    l_run = xor32_sum(l_run);
     if constexpr (SPLIT) {
         if (row_valid) {
             float* prow = part_out + ((((int64_t)b * Hq + hq) * L + q_clamped) * n_parts + part) * (D + kPartPad);
@@ -690,7 +702,7 @@ __device__ __forceinline__ void attention_q_tile_pipe(const bf16_t* __restrict__
             float mx = -INFINITY;                                                                      \
             _Pragma("unroll") for (int kb = 0; kb < 2; ++kb)                                           \
             _Pragma("unroll") for (int x = 0; x < 16; ++x) mx = fmaxf(mx, CUR[kb][x]);                 \
-            mx = fmaxf(mx, __shfl_xor(mx, 32, 64));                                                    \
+            mx = xor32_max(mx);                                                    \
             const float m_cand = fmaxf(m_run, mx * sc);                                                \
             const float m_new = m_cand - m_run > kLazyMax ? m_cand : m_run;                            \
             const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);                                 \
@@ -751,7 +763,7 @@ __device__ __forceinline__ void attention_q_tile_pipe(const bf16_t* __restrict__
 #undef PIPE_LOAD_V
 #undef PIPE_LOAD_K
 
-    l_run += __shfl_xor(l_run, 32, 64);
+    l_run = xor32_sum(l_run);
     const float inv = 1.0f / l_run;
     if (row_valid) {
         bf16_t* orow = out + ((int64_t)b * L + q_clamped) * (int64_t)(Hq * D) + hq * D;
