@@ -383,9 +383,10 @@ __global__ __launch_bounds__(256) void combine_vec_kernel(const TY* __restrict__
             my_row = row_of[t * k + lane];
             my_w = w[t * k + lane];
         }
+        // the source lanes below are the same for the whole wave: scalar reads, no shuffles through LDS
         int my_rank = 0;
         for (int j = 0; j < k; ++j) {
-            const int rj = __shfl(my_row, j, 64);
+            const int rj = __builtin_amdgcn_readlane(my_row, j);
             if (rj >= 0 && (rj < my_row || (rj == my_row && j < lane))) ++my_rank;
         }
         const int n_kept = __popcll(__ballot(my_row >= 0));
@@ -394,9 +395,9 @@ __global__ __launch_bounds__(256) void combine_vec_kernel(const TY* __restrict__
 #pragma unroll
         for (int n = 0; n < MAXK; ++n) {
             const unsigned long long who = __ballot(my_row >= 0 && my_rank == n);
-            const int src = who ? __ffsll((long long)who) - 1 : 0;
-            rows[n] = __shfl(my_row, src, 64);
-            wts[n] = __shfl(my_w, src, 64);
+            const int src = __builtin_amdgcn_readfirstlane(who ? __ffsll((long long)who) - 1 : 0);
+            rows[n] = __builtin_amdgcn_readlane(my_row, src);
+            wts[n] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(my_w), src));
         }
 #pragma unroll 4
         for (int h0 = h_first + lane * V; h0 < h_end; h0 += kWave * V) {
