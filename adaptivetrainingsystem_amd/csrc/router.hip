@@ -253,12 +253,45 @@ __global__ __launch_bounds__(256) void gate_gemm_generic_kernel(const T* __restr
 }
 
 // ------------------------------------------------------------------ routing pass
+// Value of the partner lane in step S of an ascending butterfly over groups of 2^(S+1) lanes, without LDS:
+// quad permutes for steps 0 and 1; mirrored half rows and rows for steps 2 and 3 (the lane 7-i or 15-i holds what
+// lane i^4 or i^8 holds once the earlier steps have made quads / half rows uniform, which an ascending butterfly
+// guarantees); swaps of 16-lane rows and of the wave's halves for steps 4 and 5.  All 64 lanes must be active.
+template <int S>
+__device__ __forceinline__ unsigned butterfly_partner(unsigned v) {
+    if constexpr (S == 0) return dpp_u32<kDppSwapPairs>(v);
+    else if constexpr (S == 1) return dpp_u32<kDppSwapQuadHalves>(v);
+    else if constexpr (S == 2) return dpp_u32<kDppHalfMirror>(v);
+    else if constexpr (S == 3) return dpp_u32<kDppRowMirror>(v);
+    else if constexpr (S == 4) {
+        const auto r = __builtin_amdgcn_permlane16_swap(v, v, false, false);     // {even rows twice, odd rows twice}
+        return (threadIdx.x & 16) ? r[0] : r[1];
+    } else {
+        const auto r = __builtin_amdgcn_permlane32_swap(v, v, false, false);     // {low half twice, high half twice}
+        return (threadIdx.x & 32) ? r[0] : r[1];
+    }
+}
+template <int S>
+__device__ __forceinline__ float butterfly_partner_f32(float v) {
+    return __uint_as_float(butterfly_partner<S>(__float_as_uint(v)));
+}
+// Reductions over groups of G lanes (a power of two), the result in every lane of the group.
 __device__ __forceinline__ float group_max(float v, int G) {
-    for (int off = G >> 1; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+    if (G > 1) v = fmaxf(v, butterfly_partner_f32<0>(v));
+    if (G > 2) v = fmaxf(v, butterfly_partner_f32<1>(v));
+    if (G > 4) v = fmaxf(v, butterfly_partner_f32<2>(v));
+    if (G > 8) v = fmaxf(v, butterfly_partner_f32<3>(v));
+    if (G > 16) v = fmaxf(v, butterfly_partner_f32<4>(v));
+    if (G > 32) v = fmaxf(v, butterfly_partner_f32<5>(v));
     return v;
 }
 __device__ __forceinline__ float group_sum(float v, int G) {
-    for (int off = G >> 1; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    if (G > 1) v += butterfly_partner_f32<0>(v);
+    if (G > 2) v += butterfly_partner_f32<1>(v);
+    if (G > 4) v += butterfly_partner_f32<2>(v);
+    if (G > 8) v += butterfly_partner_f32<3>(v);
+    if (G > 16) v += butterfly_partner_f32<4>(v);
+    if (G > 32) v += butterfly_partner_f32<5>(v);
     return v;
 }
 // Order used for selection: larger value first, lower index among equals; NaN
@@ -444,9 +477,9 @@ __global__ __launch_bounds__(256) void route_topk_kernel(const float* __restrict
         }
         // k rounds of group-wide arg-max
         unsigned taken = 0;   // bit i: v[i] already selected
-        float sel_val = 0.f;  // lane j < k of the group keeps choice j: value ...
-        float sel_p = 0.f;    // ... its softmax probability ...
+        float sel_term = 0.f; // lane j < k of the group keeps choice j: its unnormalised weight ...
         int sel_idx = 0;      // ... and expert id
+        float tot = 0.f, first_val = 0.f;
         for (int j = 0; j < k; ++j) {
             float bv = neg_inf;
             int bi = INT_MAX;
@@ -460,42 +493,43 @@ __global__ __launch_bounds__(256) void route_topk_kernel(const float* __restrict
                     bp = p[i];
                 }
             }
-            for (int off = G >> 1; off > 0; off >>= 1) {
-                const float ov = __shfl_xor(bv, off, 64);
-                const int oi = __shfl_xor(bi, off, 64);
-                const float op = __shfl_xor(bp, off, 64);
-                if (key_before(ov, oi, bv, bi)) {
-                    bv = ov;
-                    bi = oi;
-                    bp = op;
-                }
-            }
+#define ROUTE_MERGE_STEP(S_)                                                       \
+    if (G > (1 << (S_))) {                                                         \
+        const float ov = butterfly_partner_f32<S_>(bv);                            \
+        const int oi = (int)butterfly_partner<S_>((unsigned)bi);                   \
+        const float op = butterfly_partner_f32<S_>(bp);                            \
+        if (key_before(ov, oi, bv, bi)) {                                          \
+            bv = ov;                                                               \
+            bi = oi;                                                               \
+            bp = op;                                                               \
+        }                                                                          \
+    }
+            ROUTE_MERGE_STEP(0)
+            ROUTE_MERGE_STEP(1)
+            ROUTE_MERGE_STEP(2)
+            ROUTE_MERGE_STEP(3)
+            ROUTE_MERGE_STEP(4)
+            ROUTE_MERGE_STEP(5)
+#undef ROUTE_MERGE_STEP
             // owner marks its value as used
 #pragma unroll
             for (int i = 0; i < VPL; ++i)
                 if (gl + i * G == bi) taken |= 1u << i;
+            // the round's choice is the same in every lane of the group, so the normaliser of the weights is
+            // summed here, in rank order, instead of being gathered afterwards
+            if (j == 0) first_val = bv;
+            const float term = variant == ATS_ROUTE_SOFTMAX_TOPK ? bp : expf(bv - first_val);
+            tot += term;
             // k <= G always holds: G >= min(E, 64) and k <= min(E, kRouteMaxK)
             if (gl == j) {
-                sel_val = bv;
-                sel_p = bp;
+                sel_term = term;
                 sel_idx = bi;
             }
             if (want_stats && tok_ok && gl == 0) atomicAdd(&s_hist[bi], 1);
         }
         // weights: lanes 0..k-1 of the group hold the choices in rank order
-        float wsel;
         const bool is_sel = gl < k;
-        if (variant == ATS_ROUTE_SOFTMAX_TOPK) {
-            float tot = 0.f;
-            for (int j = 0; j < k; ++j) tot += __shfl(sel_p, grp * G + j, 64);
-            wsel = sel_p / (tot + 1e-9f);
-        } else {
-            const float mx = __shfl(sel_val, grp * G, 64);
-            const float ex = is_sel ? expf(sel_val - mx) : 0.f;
-            float tot = 0.f;
-            for (int j = 0; j < k; ++j) tot += __shfl(ex, grp * G + j, 64);
-            wsel = ex / tot;
-        }
+        const float wsel = variant == ATS_ROUTE_SOFTMAX_TOPK ? sel_term / (tot + 1e-9f) : sel_term / tot;
         if (tok_ok && is_sel) {
             idx_out[t * k + gl] = sel_idx;
             w_out[t * k + gl] = wsel;

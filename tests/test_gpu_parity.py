@@ -175,7 +175,8 @@ def _ambiguous_rows(logits, k, temperature):
 
 @pytest.mark.parametrize("T,E,k,temp", [(512, 8, 2, 1.0), (1000, 64, 6, 1.0), (37, 4, 1, 1.0), (300, 128, 4, 0.7),
                                         (129, 6, 3, 1.3), (16384, 8, 2, 1.0), (50, 300, 8, 1.0), (700, 40, 5, 0.8),
-                                        (4096, 64, 6, 1.0), (333, 33, 16, 1.0)])
+                                        (4096, 64, 6, 1.0), (333, 33, 16, 1.0), (500, 24, 4, 1.1), (40, 20, 3, 1.0),
+                                        (900, 12, 2, 0.9), (10, 50, 7, 1.0)])
 def test_route_topk(ops, gpu, T, E, k, temp):
     print("case route", T, E, k, temp, flush=True)
     logits = torch.randn(T, E, generator=gen(15)) * 1.3
