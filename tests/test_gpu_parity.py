@@ -760,6 +760,35 @@ def test_decode_ffn_step_replays_in_a_hip_graph(A, gpu):
             assert torch.equal(y, ref), rep
 
 
+def test_mod_moe_block_replays_in_a_hip_graph(A, gpu):
+    """The MoD + MoE block's inference path (score + copy pass, selection, gather, MoE layer whose combine adds
+    onto the copy) launches on the current stream and never synchronises: captured once, three replays with
+    eager work in between, each equal to the eager output and auxiliary loss."""
+    from adaptivetrainingsystem_amd import workloads as W
+    ov = {"batch": 4, "seq": 512, "hidden": 256, "intermediate": 128}
+    w = W.make_moe_workload("c5_finegrained_mod", device=gpu, overrides=ov)
+    block = W.build_layer(w, "fcfs")
+    x = w.x
+    with torch.no_grad():
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(2):
+                block(x)
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            y, aux = block(x)
+        for rep in range(3):
+            x.copy_(torch.randn(x.shape, generator=gen(90 + rep)).to(x.dtype))
+            ref, ref_aux = block(x)
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(y, ref), rep
+            assert torch.equal(aux, ref_aux), rep
+
+
 def test_moe_decode_step_replays_in_a_hip_graph(A, gpu):
     """The inference path of the MoE layer never synchronises (the plan stays on the device), so a decoding
     step can be captured as well: replays equal the eager output and auxiliary loss."""
