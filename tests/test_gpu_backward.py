@@ -42,7 +42,7 @@ def ops(gpu):
 
 # ------------------------------------------------------------------ RMSNorm
 @pytest.mark.parametrize("shape", [(8, 512), (3, 5, 128), (7, 100), (300, 4096), (5, 8192), (3, 12000), (1, 8), (2, 6),
-                                   (1000, 2048), (2500, 2048), (1, 4096), (3, 2056), (1027, 1024)])
+                                   (1000, 2048), (2500, 2048), (1, 4096), (3, 2056), (1027, 1024), (4099, 2048), (2051, 4096)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_rmsnorm_bwd(ops, gpu, shape, dtype):
     print("case rmsnorm_bwd", shape, dtype, flush=True)
