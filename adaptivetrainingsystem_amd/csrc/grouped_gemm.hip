@@ -394,8 +394,11 @@ __device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(
 //   LDS barrier
 //   k-step 3: MFMAs(buf 1) | read k-step 0 of slab t+1
 // Global loads therefore have a whole slab of MFMA time to land before they are needed.
+// SWZ: staged rows are 128 bytes without padding, and the 16-byte chunk c of row R sits in slot c ^ f(R),
+// f(R) = (R & 7) ^ ((R >> 3) & 1) (the 16 rows a quarter wave reads hit all 64 banks once).  The 32 x 256
+// weight-streaming tile then takes 72 KiB instead of 81, and two of its workgroups share a CU.
 template <typename T, typename TO, int BM, int BN, int WM, int WN, int SM, int SN, bool SWIGLU, bool WARM,
-          bool SLICED = false>
+          bool SLICED = false, bool SWZ = false>
 __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_pipelined_kernel(GroupedArgs p) {
     constexpr int NT = WM * WN * 64;
     constexpr int VEC = 16 / (int)sizeof(T);
@@ -405,7 +408,10 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_pipelined_kernel(Gro
     constexpr int RPP = NT / 8;
     constexpr int PA = BM / RPP;
     constexpr int PB = BN / RPP;
-    constexpr int STAGE = (BM + BN) * kRowPitch;
+    constexpr int PITCH = SWZ ? 128 : kRowPitch;
+    constexpr int STAGE = (BM + BN) * PITCH;
+    constexpr int NOFF = SWZ ? 4 : 1;   // fragment offsets per row: one per k-step when the slots are swizzled
+    static_assert(!SWZ || RPP % 16 == 0, "the loader's passes must keep a row's swizzle");
     constexpr int HALF = BN / 2;
     static_assert(BM % (WM * 32) == 0 && BN % (WN * 32) == 0, "wave tiling");
     static_assert(BM % RPP == 0 && BN % RPP == 0, "loader tiling");
@@ -505,13 +511,18 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_pipelined_kernel(Gro
 
     const int nk = K / BK;
     u32x4_t ra[PA], rb[PB];
-    const int st_off = lrow * kRowPitch + lchunk * 16;
+    const int st_off = lrow * PITCH + (SWZ ? (lchunk ^ (lrow & 7) ^ ((lrow >> 3) & 1)) : lchunk) * 16;
 
     const int frow = lane & 31;
     const int fgrp = lane >> 5;
-    int a_row_off[TM], b_row_off[TN];
+    // (tile rows of a fragment start at multiples of 32, so a lane's swizzle depends on frow alone)
+    const int fswz = (frow & 7) ^ ((frow >> 3) & 1);
+    int a_row_off[TM][NOFF], b_row_off[TN][NOFF];
 #pragma unroll
-    for (int i = 0; i < TM; ++i) a_row_off[i] = (wm * (BM / WM) + i * 32 + frow) * kRowPitch + fgrp * 16;
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int q = 0; q < NOFF; ++q)
+            a_row_off[i][q] = (wm * (BM / WM) + i * 32 + frow) * PITCH + (SWZ ? ((2 * q + fgrp) ^ fswz) : fgrp) * 16;
 #pragma unroll
     for (int j = 0; j < TN; ++j) {
         int r;
@@ -521,7 +532,9 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_pipelined_kernel(Gro
         } else {
             r = wn * (BN / WN) + j * 32;
         }
-        b_row_off[j] = BM * kRowPitch + (r + frow) * kRowPitch + fgrp * 16;
+#pragma unroll
+        for (int q = 0; q < NOFF; ++q)
+            b_row_off[j][q] = BM * PITCH + (r + frow) * PITCH + (SWZ ? ((2 * q + fgrp) ^ fswz) : fgrp) * 16;
     }
     u32x4_t fa[2][TM], fb[2][TN];
 
@@ -534,19 +547,19 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_pipelined_kernel(Gro
 #define PL_STORE(stage_)                                                                               \
     {                                                                                                  \
         unsigned char* sA_ = smem + (stage_) * STAGE + st_off;                                         \
-        unsigned char* sB_ = sA_ + BM * kRowPitch;                                                     \
+        unsigned char* sB_ = sA_ + BM * PITCH;                                                         \
         _Pragma("unroll") for (int i = 0; i < PA; ++i)                                                 \
-            *reinterpret_cast<u32x4_t*>(sA_ + i * RPP * kRowPitch) = ra[i];                              \
+            *reinterpret_cast<u32x4_t*>(sA_ + i * RPP * PITCH) = ra[i];                                  \
         _Pragma("unroll") for (int i = 0; i < PB; ++i)                                                 \
-            *reinterpret_cast<u32x4_t*>(sB_ + i * RPP * kRowPitch) = rb[i];                              \
+            *reinterpret_cast<u32x4_t*>(sB_ + i * RPP * PITCH) = rb[i];                                  \
     }
 #define PL_READ(stage_, ks_, buf_)                                                                     \
     {                                                                                                  \
-        const unsigned char* s_ = smem + (stage_) * STAGE + (ks_) * 32;                                \
+        const unsigned char* s_ = smem + (stage_) * STAGE + (SWZ ? 0 : (ks_) * 32);                    \
         _Pragma("unroll") for (int i = 0; i < TM; ++i)                                                 \
-            fa[buf_][i] = *reinterpret_cast<const u32x4_t*>(s_ + a_row_off[i]);                          \
+            fa[buf_][i] = *reinterpret_cast<const u32x4_t*>(s_ + a_row_off[i][SWZ ? (ks_) : 0]);         \
         _Pragma("unroll") for (int j = 0; j < TN; ++j)                                                 \
-            fb[buf_][j] = *reinterpret_cast<const u32x4_t*>(s_ + b_row_off[j]);                          \
+            fb[buf_][j] = *reinterpret_cast<const u32x4_t*>(s_ + b_row_off[j][SWZ ? (ks_) : 0]);         \
     }
 #define PL_MMA(buf_)                                                                                   \
     {                                                                                                  \
@@ -1172,13 +1185,16 @@ static int launch_cfg(const GroupedArgs& p0, int64_t max_rows, hipStream_t s) {
     auto kern_general = grouped_gemm_kernel<T, TO, BM, BN, WM, WN, SM, SN, SWIGLU>;
     // the L2 warm-up touches pay where blocks share operand panels; the weight-streaming tiles share nothing
     constexpr bool kWarm = BM > 64;
-    auto kern_pipe = grouped_gemm_pipelined_kernel<T, TO, BM, BN, WM, WN, SM, SN, SWIGLU, kWarm>;
+    // the gate/up weight-streaming tile: unpadded swizzled rows, so that two workgroups fit a CU
+    constexpr bool kSwz = BM == 32 && BN == 256;
+    constexpr size_t smem_pipe = kSwz ? 2 * (size_t)(BM + BN) * 128 : smem_staged;
+    auto kern_pipe = grouped_gemm_pipelined_kernel<T, TO, BM, BN, WM, WN, SM, SN, SWIGLU, kWarm, false, kSwz>;
     auto kern_dma = [] {
         if constexpr (DMA && std::is_same<T, bf16_t>::value) {
             static_assert(BM == 256 && BN == 256 && WM == 2 && WN == 4, "the 16 x 16 x 32 kernel is the 256 x 256 tile");
             return grouped_gemm_dma16_kernel<TO, SM, SN, SWIGLU>;
         } else if constexpr (DMA) return grouped_gemm_dma_kernel<T, TO, BM, BN, WM, WN, SM, SN, SWIGLU>;
-        else return grouped_gemm_pipelined_kernel<T, TO, BM, BN, WM, WN, SM, SN, SWIGLU, kWarm>;
+        else return grouped_gemm_pipelined_kernel<T, TO, BM, BN, WM, WN, SM, SN, SWIGLU, kWarm, false, kSwz>;
     }();
     if (smem > 64 * 1024) {
         static LdsReservation reserved;      // one per tile configuration (this function is a template)
@@ -1218,7 +1234,8 @@ static int launch_cfg(const GroupedArgs& p0, int64_t max_rows, hipStream_t s) {
     // the direct-to-LDS kernel addresses its operands with 32-bit lane offsets
     const bool dma_ok = DMA && p.K % BK == 0 && p.a_extent_bytes != 0 && p.b_extent_bytes != 0;
     auto kern = dma_ok ? kern_dma : (p.K % BK == 0) ? kern_pipe : kern_general;
-    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(WM * WN * 64), smem, s, p);
+    const size_t smem_launch = (!dma_ok && p.K % BK == 0) ? smem_pipe : smem;
+    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(WM * WN * 64), smem_launch, s, p);
     return ATS_OK;
 }
 
