@@ -1196,18 +1196,22 @@ static int launch_cfg(const GroupedArgs& p0, int64_t max_rows, hipStream_t s) {
         } else if constexpr (DMA) return grouped_gemm_dma_kernel<T, TO, BM, BN, WM, WN, SM, SN, SWIGLU>;
         else return grouped_gemm_pipelined_kernel<T, TO, BM, BN, WM, WN, SM, SN, SWIGLU, kWarm, false, kSwz>;
     }();
+    // slices of K: the weight-streaming tiles only, in their own instance of the register-staged kernel
+    constexpr bool kCanSlice = !DMA && !SWIGLU && (BM == 32 || BM == 64);
+    const void* kern_sliced = reinterpret_cast<const void*>(kern_pipe);
+    if constexpr (kCanSlice)
+        kern_sliced = reinterpret_cast<const void*>(
+            grouped_gemm_pipelined_kernel<T, TO, BM, BN, WM, WN, SM, SN, SWIGLU, kWarm, true, kSwz>);
     if (smem > 64 * 1024) {
         static LdsReservation reserved;      // one per tile configuration (this function is a template)
         hipError_t e = reserve_lds(reserved, {reinterpret_cast<const void*>(kern_general),
                                               reinterpret_cast<const void*>(kern_pipe),
-                                              reinterpret_cast<const void*>(kern_dma)}, (int)smem);
+                                              reinterpret_cast<const void*>(kern_dma), kern_sliced}, (int)smem);
         if (e != hipSuccess) {
             set_error("grouped GEMM: cannot reserve %zu bytes of LDS: %s", smem, hipGetErrorString(e));
             return ATS_ERR_LAUNCH;
         }
     }
-    // slices of K: the weight-streaming tiles only, in their own instance of the register-staged kernel
-    constexpr bool kCanSlice = !DMA && !SWIGLU && (BM == 32 || BM == 64);
     const int splits = p.k_splits > 1 ? p.k_splits : 1;
     if (splits > 1 && (!kCanSlice || p.k_count || p.K % splits != 0 || (p.K / splits) % BK != 0)) {
         set_error("grouped GEMM: %d slices of K=%d are not available for this tile configuration", splits, p.K);
@@ -1226,8 +1230,8 @@ static int launch_cfg(const GroupedArgs& p0, int64_t max_rows, hipStream_t s) {
     }
     if constexpr (kCanSlice) {
         if (splits > 1) {
-            hipLaunchKernelGGL((grouped_gemm_pipelined_kernel<T, TO, BM, BN, WM, WN, SM, SN, SWIGLU, kWarm, true>),
-                               dim3((unsigned)blocks), dim3(WM * WN * 64), smem, s, p);
+            hipLaunchKernelGGL((grouped_gemm_pipelined_kernel<T, TO, BM, BN, WM, WN, SM, SN, SWIGLU, kWarm, true, kSwz>),
+                               dim3((unsigned)blocks), dim3(WM * WN * 64), smem_pipe, s, p);
             return ATS_OK;
         }
     }
