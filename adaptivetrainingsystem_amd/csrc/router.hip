@@ -2,16 +2,16 @@
 // softmax / top-k / histogram / importance pass.
 //
 // Gate GEMM.  N = E is tiny, so the kernel is bound by reading x once from HBM.
-// bf16: a block owns 16 tokens; its 4 waves split the hidden dimension in
-// quarters (4x more loads in flight than one wave per tile), each feeding
-// v_mfma_f32_16x16x32_bf16 straight from global memory with 16-byte loads, and
-// the four partial tiles are summed in a fixed order through LDS.  The four lane
-// groups of a row read 64 contiguous bytes per load instruction.
+// bf16: a block owns 16 tokens; its 4 or 8 waves split the hidden dimension (that many times
+// more loads in flight than one wave per tile).  A wave loads 128 elements of its 16 token rows
+// and of 16 gate rows per step with coalesced 16-byte loads (4 rows x 256 bytes per instruction),
+// passes them through a wave-private piece of LDS into the operand layout of
+// v_mfma_f32_16x16x32_bf16, and the waves' partial tiles are summed in a fixed order through LDS.
 // f32 (and odd shapes): one wave per token with plain FMAs.
 //
 // Routing pass.  A group of G = pow2 >= min(E,64) lanes owns one token; values
-// stay in registers, maxima / sums / arg-max run over xor-shuffles inside the
-// group.  Per-block histogram and probability column sums go to a workspace and
+// stay in registers, maxima / sums / arg-max run over DPP steps and row / half-wave swaps
+// inside the group.  Per-block histogram and probability column sums go to a workspace and
 // a second tiny kernel reduces them in a fixed order (bit-reproducible, no
 // float atomics) and evaluates the auxiliary loss.
 #include <limits.h>
@@ -39,20 +39,24 @@ constexpr int kGateKC = 128;  // k elements consumed per wave per step
 
 // NT = number of 16-wide expert tiles, KW = waves per block (each owns 1/KW of the hidden
 // dimension).  With PF the loads of step s+1 are issued before the MFMAs of step s.
+// A step's 16 x 128 elements of x and, tile after tile, of the gate reach the MFMA operand layout through a
+// wave-private piece of LDS (see gate_gemm_bf16_flat_kernel: coalesced loads of whole cache lines instead of
+// 16 rows x 64 bytes per instruction); a wave's LDS accesses complete in order, so no barrier is involved.
 template <int NT, int KW, bool PF>
 __global__ __launch_bounds__(KW * 64) void gate_gemm_bf16_kernel(const bf16_t* __restrict__ x,
                                                                const bf16_t* __restrict__ wg,
                                                                const float* __restrict__ bias,
                                                                float* __restrict__ logits, int64_t T, int H,
                                                                int E) {
-    __shared__ float red[KW][NT][16 * 16];
+    static_assert(NT <= 8, "a wave's partial tiles are parked in its 8 KB stage");
+    __shared__ __align__(16) unsigned char stage[KW][2][16 * 256];   // per wave: one step of x rows, of 16 gate rows
     const int lane = lane_id();
     const int wave = threadIdx.x >> 6;
-    const int r = lane & 15;   // A: token row inside the tile; B: expert inside the tile
-    const int g = lane >> 4;   // lane group -> 8-element k slice of each 32-element MFMA step (64 contiguous bytes per row and load)
+    const int r = lane & 15;        // MFMA view: token row (A) / expert inside the tile (B) ...
+    const int g = lane >> 4;        // ... and 8-element k group of each 32-element MFMA step
+    const int lrow = lane >> 4;     // loader view: row 4 j + lrow of a 16-row tile ...
+    const int lchunk = lane & 15;   // ... and 16-byte chunk of the step's 256-byte row piece
     const int64_t t0 = (int64_t)blockIdx.x * 16;
-    const int64_t trow = t0 + r;
-    const bool row_ok = trow < T;
 
     // this wave's k range (whole steps; the tail is handled by predicates)
     const int steps_total = (H + kGateKC - 1) / kGateKC;
@@ -64,32 +68,51 @@ __global__ __launch_bounds__(KW * 64) void gate_gemm_bf16_kernel(const bf16_t* _
 #pragma unroll
     for (int n = 0; n < NT; ++n) acc[n] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-    const bf16_t* xrow = x + (row_ok ? trow : 0) * (int64_t)H;
     const u32x4_t zero4 = {0u, 0u, 0u, 0u};
     u32x4_t a[PF ? 2 : 1][4], b[PF ? 2 : 1][NT][4];
+    int woff[4], roff[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int row = 4 * j + lrow;
+        woff[j] = row * 256 + ((lchunk ^ row) << 4);
+        roff[j] = r * 256 + (((4 * j + g) ^ r) << 4);
+    }
+    unsigned char* const sx = stage[wave][0];
+    unsigned char* const sg = stage[wave][1];
 
 #define GG_LOAD(s_, buf_)                                                                              \
     {                                                                                                  \
-        const int kb_ = (s_) * kGateKC + g * 8;                                                        \
-        _Pragma("unroll") for (int i = 0; i < 4; ++i) {                                                \
-            const int kk = kb_ + i * 32;                                                               \
-            a[buf_][i] = zero4;                                                                        \
-            if (row_ok && kk < H) a[buf_][i] = *reinterpret_cast<const u32x4_t*>(xrow + kk);           \
+        const int kk = (s_) * kGateKC + lchunk * 8;                                                    \
+        _Pragma("unroll") for (int j = 0; j < 4; ++j) {                                                \
+            const int64_t trow = t0 + 4 * j + lrow;                                                    \
+            a[buf_][j] = zero4;                                                                        \
+            if (trow < T && kk < H) a[buf_][j] = *reinterpret_cast<const u32x4_t*>(x + trow * (int64_t)H + kk); \
         }                                                                                              \
         _Pragma("unroll") for (int n = 0; n < NT; ++n) {                                               \
-            const int e = n * 16 + r;                                                                  \
-            _Pragma("unroll") for (int i = 0; i < 4; ++i) {                                            \
-                const int kk = kb_ + i * 32;                                                           \
-                b[buf_][n][i] = zero4;                                                                 \
-                if (e < E && kk < H) b[buf_][n][i] = *reinterpret_cast<const u32x4_t*>(wg + (int64_t)e * H + kk); \
+            _Pragma("unroll") for (int j = 0; j < 4; ++j) {                                            \
+                const int e = n * 16 + 4 * j + lrow;                                                   \
+                b[buf_][n][j] = zero4;                                                                 \
+                if (e < E && kk < H) b[buf_][n][j] = *reinterpret_cast<const u32x4_t*>(wg + (int64_t)e * H + kk); \
             }                                                                                          \
         }                                                                                              \
     }
+// per output tile the order of accumulation is: steps ascending, the four 32-element pieces ascending
 #define GG_MMA(buf_)                                                                                   \
     {                                                                                                  \
-        _Pragma("unroll") for (int i = 0; i < 4; ++i) {                                                \
-            _Pragma("unroll") for (int n = 0; n < NT; ++n)                                             \
-                acc[n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a[buf_][i]), as_bf16x8(b[buf_][n][i]), acc[n], 0, 0, 0); \
+        u32x4_t fa[4];                                                                                 \
+        _Pragma("unroll") for (int j = 0; j < 4; ++j) *reinterpret_cast<u32x4_t*>(sx + woff[j]) = a[buf_][j]; \
+        _Pragma("unroll") for (int n = 0; n < NT; ++n) {                                               \
+            _Pragma("unroll") for (int j = 0; j < 4; ++j)                                              \
+                *reinterpret_cast<u32x4_t*>(sg + woff[j]) = b[buf_][n][j];                             \
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");                                         \
+            if (n == 0) {                                                                              \
+                _Pragma("unroll") for (int i = 0; i < 4; ++i) fa[i] = *reinterpret_cast<const u32x4_t*>(sx + roff[i]); \
+            }                                                                                          \
+            _Pragma("unroll") for (int i = 0; i < 4; ++i) {                                            \
+                const u32x4_t fb = *reinterpret_cast<const u32x4_t*>(sg + roff[i]);                    \
+                acc[n] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(fa[i]), as_bf16x8(fb), acc[n], 0, 0, 0); \
+            }                                                                                          \
+            asm volatile("" ::: "memory");                                                             \
         }                                                                                              \
     }
     if constexpr (PF) {
@@ -118,11 +141,14 @@ __global__ __launch_bounds__(KW * 64) void gate_gemm_bf16_kernel(const bf16_t* _
     }
 #undef GG_LOAD
 #undef GG_MMA
-    // D layout of the 16x16 tile: lane holds column (lane & 15), rows 4*(lane>>4) + v.
+    // D layout of the 16x16 tile: lane holds column (lane & 15), rows 4*(lane>>4) + v.  A wave parks its NT
+    // partial tiles at the front of its own stage.
+    float* const red = reinterpret_cast<float*>(stage[wave][0]);
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
 #pragma unroll
     for (int n = 0; n < NT; ++n) {
 #pragma unroll
-        for (int v = 0; v < 4; ++v) red[wave][n][(4 * g + v) * 16 + r] = acc[n][v];
+        for (int v = 0; v < 4; ++v) red[n * 256 + (4 * g + v) * 16 + r] = acc[n][v];
     }
     __syncthreads();
     for (int i = threadIdx.x; i < NT * 256; i += KW * 64) {
@@ -132,9 +158,9 @@ __global__ __launch_bounds__(KW * 64) void gate_gemm_bf16_kernel(const bf16_t* _
         const int e = n * 16 + col;
         const int64_t t = t0 + row;
         if (t < T && e < E) {
-            float v = red[0][n][i & 255];
+            float v = reinterpret_cast<const float*>(stage[0][0])[i];
 #pragma unroll
-            for (int w = 1; w < KW; ++w) v += red[w][n][i & 255];
+            for (int w = 1; w < KW; ++w) v += reinterpret_cast<const float*>(stage[w][0])[i];
             if (bias) v += bias[e];
             logits[t * E + e] = v;
         }
@@ -142,79 +168,100 @@ __global__ __launch_bounds__(KW * 64) void gate_gemm_bf16_kernel(const bf16_t* _
 }
 
 // Up to 16 experts and a hidden size of at most 8 x 4 x 128: the same split of K over 8 waves, but a wave
-// asks for its whole K slice at once (up to 4 steps x 4 loads per token tile, plus the gate rows) before the
-// first MFMA, and a block owns MT 16-token tiles that share the gate rows' loads.  With nothing to wait for
-// between steps the block's bytes are all in flight after a few hundred cycles, which is what a kernel that
-// lives for 20 us needs.  The gate rows are fetched one step ahead of their use rather than all at once, which
-// keeps a wave at 108 registers and two blocks resident per CU.
-template <int MT>
+// asks for its whole K slice of the 16 token rows at once (up to 4 steps x 4 loads) before the first MFMA, so the
+// block's bytes are all in flight after a few hundred cycles, which is what a kernel that lives for 20 us needs.
+// The loads are coalesced - an instruction covers 4 rows x 256 bytes, whole cache lines - and a step's 16 x 128
+// elements of x and of the gate go through a wave-private 4 KB piece of LDS each to reach the MFMA operand layout
+// (lane (r, g) holds 8 elements of row r): loaded directly in that layout an instruction touches 16 rows x 64
+// bytes, and the vector cache serves that pattern at a quarter of the rate (38 against 134 GB/s per CU from L2).
+// LDS slot c ^ r holds the 16-byte chunk c of row r, so the 16 rows of a fragment read hit all banks.  The gate
+// rows are fetched one step ahead of their use; order of accumulation as in gate_gemm_bf16_kernel: steps
+// ascending, the four 32-element pieces ascending, the waves' partial sums in wave order.
 __global__ __launch_bounds__(512) void gate_gemm_bf16_flat_kernel(const bf16_t* __restrict__ x,
                                                                   const bf16_t* __restrict__ wg,
                                                                   const float* __restrict__ bias,
                                                                   float* __restrict__ logits, int64_t T, int H, int E) {
     constexpr int KW = 8, S = 4;
-    __shared__ float red[KW][MT][16 * 16];
+    __shared__ __align__(16) unsigned char stage[KW][2][16 * 256];   // per wave: one step of x rows, of gate rows
     const int lane = lane_id();
     const int wave = threadIdx.x >> 6;
-    const int r = lane & 15;
-    const int g = lane >> 4;
-    const int64_t t0 = (int64_t)blockIdx.x * (16 * MT);
+    const int r = lane & 15;        // MFMA view: token row (A) / expert (B) ...
+    const int g = lane >> 4;        // ... and 8-element k group of a 32-element piece
+    const int lrow = lane >> 4;     // loader view: row 4 j + lrow of the tile ...
+    const int lchunk = lane & 15;   // ... and 16-byte chunk of the step's 256-byte row piece
+    const int64_t t0 = (int64_t)blockIdx.x * 16;
     const int steps_total = (H + kGateKC - 1) / kGateKC;
     const int steps_per_wave = (steps_total + KW - 1) / KW;      // <= S (host)
     const int s_begin = wave * steps_per_wave;
     const u32x4_t zero4 = {0u, 0u, 0u, 0u};
-    u32x4_t a[MT][S][4], b[2][4];
+    u32x4_t a[S][4], b[2][4];
     // token rows first: they come from HBM, the gate rows from L2
 #pragma unroll
-    for (int m = 0; m < MT; ++m) {
-        const int64_t trow = t0 + m * 16 + r;
-        const bf16_t* xrow = x + (trow < T ? trow : 0) * (int64_t)H;
+    for (int st = 0; st < S; ++st) {
+        const int kk = (s_begin + st) * kGateKC + lchunk * 8;
 #pragma unroll
-        for (int st = 0; st < S; ++st)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int kk = (s_begin + st) * kGateKC + g * 8 + i * 32;
-                a[m][st][i] = zero4;
-                if (st < steps_per_wave && trow < T && kk < H) a[m][st][i] = *reinterpret_cast<const u32x4_t*>(xrow + kk);
-            }
+        for (int j = 0; j < 4; ++j) {
+            const int64_t trow = t0 + 4 * j + lrow;
+            a[st][j] = zero4;
+            if (st < steps_per_wave && trow < T && kk < H)
+                a[st][j] = *reinterpret_cast<const u32x4_t*>(x + trow * (int64_t)H + kk);
+        }
     }
-    // the gate rows one step ahead of their use (two register sets: all of them at once would cost a resident block)
 #define GF_LOAD_B(st_, buf_)                                                                           \
-    _Pragma("unroll") for (int i = 0; i < 4; ++i) {                                                    \
-        const int kk = (s_begin + (st_)) * kGateKC + g * 8 + i * 32;                                   \
-        b[buf_][i] = zero4;                                                                            \
-        if ((st_) < steps_per_wave && r < E && kk < H)                                                 \
-            b[buf_][i] = *reinterpret_cast<const u32x4_t*>(wg + (int64_t)r * H + kk);                  \
+    {                                                                                                  \
+        const int kk = (s_begin + (st_)) * kGateKC + lchunk * 8;                                       \
+        _Pragma("unroll") for (int j = 0; j < 4; ++j) {                                                \
+            const int e = 4 * j + lrow;                                                                \
+            b[buf_][j] = zero4;                                                                        \
+            if ((st_) < steps_per_wave && e < E && kk < H)                                             \
+                b[buf_][j] = *reinterpret_cast<const u32x4_t*>(wg + (int64_t)e * H + kk);              \
+        }                                                                                              \
     }
     GF_LOAD_B(0, 0);
-    f32x4_t acc[MT];
+    int woff[4], roff[4];
 #pragma unroll
-    for (int m = 0; m < MT; ++m) acc[m] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-    // same order of accumulation as gate_gemm_bf16_kernel: steps ascending, the four 32-element pieces ascending
+    for (int j = 0; j < 4; ++j) {
+        const int row = 4 * j + lrow;
+        woff[j] = row * 256 + ((lchunk ^ row) << 4);
+        roff[j] = r * 256 + (((4 * j + g) ^ r) << 4);
+    }
+    unsigned char* const sx = stage[wave][0];
+    unsigned char* const sg = stage[wave][1];
+    f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int st = 0; st < S; ++st) {
         if (st + 1 < S) GF_LOAD_B(st + 1, (st + 1) & 1);
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
+        for (int j = 0; j < 4; ++j) {
+            *reinterpret_cast<u32x4_t*>(sx + woff[j]) = a[st][j];
+            *reinterpret_cast<u32x4_t*>(sg + woff[j]) = b[st & 1][j];
+        }
+        // the tile is private to the wave and a wave's LDS accesses complete in order: no barrier, the
+        // compiler only has to keep the reads behind the writes (and the next step's writes behind the reads)
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
 #pragma unroll
-            for (int m = 0; m < MT; ++m)
-                acc[m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(a[m][st][i]), as_bf16x8(b[st & 1][i]), acc[m], 0, 0, 0);
+        for (int i = 0; i < 4; ++i) {
+            const u32x4_t fa = *reinterpret_cast<const u32x4_t*>(sx + roff[i]);
+            const u32x4_t fb = *reinterpret_cast<const u32x4_t*>(sg + roff[i]);
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(as_bf16x8(fa), as_bf16x8(fb), acc, 0, 0, 0);
+        }
+        asm volatile("" ::: "memory");
     }
 #undef GF_LOAD_B
+    // the waves' partial tiles, each in the front of its own stage
+    float* const red = reinterpret_cast<float*>(stage[wave][0]);
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
 #pragma unroll
-    for (int m = 0; m < MT; ++m)
-#pragma unroll
-        for (int v = 0; v < 4; ++v) red[wave][m][(4 * g + v) * 16 + r] = acc[m][v];
+    for (int v = 0; v < 4; ++v) red[(4 * g + v) * 16 + r] = acc[v];
     __syncthreads();
-    for (int i = threadIdx.x; i < MT * 256; i += KW * 64) {
-        const int m = i >> 8;
-        const int row = (i & 255) >> 4;
+    for (int i = threadIdx.x; i < 256; i += KW * 64) {
+        const int row = i >> 4;
         const int col = i & 15;
-        const int64_t t = t0 + m * 16 + row;
+        const int64_t t = t0 + row;
         if (t < T && col < E) {
-            float v = red[0][m][i & 255];
+            float v = reinterpret_cast<const float*>(stage[0][0])[i];
 #pragma unroll
-            for (int w = 1; w < KW; ++w) v += red[w][m][i & 255];
+            for (int w = 1; w < KW; ++w) v += reinterpret_cast<const float*>(stage[w][0])[i];
             if (bias) v += bias[col];
             logits[t * E + col] = v;
         }
@@ -675,7 +722,7 @@ extern "C" int ats_router_logits(const void* x, const void* wg, const float* bia
         // tile per block: two blocks stay resident per CU; with two tiles per block the kernel ran 36 instead of 27 us
         // on [16384, 4096] x 8 experts, the looped kernel 37 us)
         if (nt <= 1 && H <= 8 * 4 * kGateKC && T >= 2048)
-            hipLaunchKernelGGL((gate_gemm_bf16_flat_kernel<1>), dim3(blocks), dim3(512), 0, s, xp, wp, bias, logits, T, H, E);
+            hipLaunchKernelGGL(gate_gemm_bf16_flat_kernel, dim3(blocks), dim3(512), 0, s, xp, wp, bias, logits, T, H, E);
         else if (nt <= 1)
             hipLaunchKernelGGL((gate_gemm_bf16_kernel<1, 8, false>), dim3(blocks), dim3(512), 0, s, xp, wp, bias, logits, T, H, E);
         else if (nt <= 2)
