@@ -163,7 +163,8 @@ def test_route_bwd(ops, gpu, T, E, k, temp, mode):
     assert (dz2.cpu() - dz_ref2).abs().max().item() <= 2e-5 * dz_ref2.abs().max().item() + noise_floor
 
 
-@pytest.mark.parametrize("T,H,E", [(512, 512, 8), (100, 1024, 64), (33, 40, 6), (1000, 2048, 128), (1, 64, 4)])
+@pytest.mark.parametrize("T,H,E", [(512, 512, 8), (100, 1024, 64), (33, 40, 6), (1000, 2048, 128), (1, 64, 4),
+                                   (1001, 2048, 5), (300, 264, 8)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_router_bwd(ops, gpu, T, H, E, dtype):
     print("case router_bwd", T, H, E, dtype, flush=True)
