@@ -264,10 +264,13 @@ __global__ __launch_bounds__(256) void router_dx_kernel(const float* __restrict_
 
 // Up to 8 experts: a thread owns V consecutive columns for a chunk of tokens and keeps its V x E gate weights in
 // registers, so the gate rows are read once per chunk instead of once per token (they made up 8/9 of the loads);
-// the next four tokens' base pieces travel while the current four are used.  Per element the same sum in the same order as above.
+// the next four tokens' base pieces travel while the current four are used.  A token's E gradients are wave
+// uniform and come in as one scalar load: nothing in the loop over the experts is conditional (absent experts
+// have zero weights and a zero gradient), since a test per expert made every value a load of its own with a
+// wait behind it.  Per element the same sum in the same order as above.
 constexpr int kDxExperts = 8;
 constexpr int kDxChunk = 64;
-template <typename T>
+template <typename T, bool FULL>   // FULL: exactly 8 experts (a token's gradients are one 32-byte scalar load)
 __global__ __launch_bounds__(256) void router_dx_cols_kernel(const float* __restrict__ dz, const T* __restrict__ wg,
                                                              const T* base, T* out, int64_t Tn, int E, int H) {
     constexpr int V = Elem<T>::kVec;
@@ -289,32 +292,35 @@ __global__ __launch_bounds__(256) void router_dx_cols_kernel(const float* __rest
         _Pragma("unroll") for (int u = 0; u < U; ++u)                                                  \
             if ((tb_) + u < t1) nxt[u] = *reinterpret_cast<const uint4*>(base + ((tb_) + u) * H + h);  \
     }
+#define ATS_DX_TOKEN(raw_, t_)                                                                         \
+    {                                                                                                  \
+        float acc[V];                                                                                  \
+        _Pragma("unroll") for (int j = 0; j < V; ++j) acc[j] = 0.f;                                    \
+        if (base) Elem<T>::unpack(raw_, acc);                                                          \
+        const float* dzt = dz + (t_) * E;                                                              \
+        float d[kDxExperts];                                                                           \
+        _Pragma("unroll") for (int e = 0; e < kDxExperts; ++e) d[e] = dzt[FULL || e < E ? e : E - 1];  \
+        _Pragma("unroll") for (int e = 0; e < kDxExperts; ++e) d[e] = FULL || e < E ? d[e] : 0.f;      \
+        _Pragma("unroll") for (int e = 0; e < kDxExperts; ++e) {                                       \
+            _Pragma("unroll") for (int j = 0; j < V; ++j) acc[j] += d[e] * wv[e][j];                   \
+        }                                                                                              \
+        *reinterpret_cast<uint4*>(out + (t_) * H + h) = Elem<T>::pack(acc);                            \
+    }
     ATS_DX_FETCH(t0);
-    for (int64_t tb = t0; tb < t1; tb += U) {
+    int64_t tb = t0;
+    for (; tb + U <= t1; tb += U) {
         uint4 raw[U];
 #pragma unroll
         for (int u = 0; u < U; ++u) raw[u] = nxt[u];
         ATS_DX_FETCH(tb + U);      // the next pieces travel while these are used
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            if (tb + u < t1) {
-                float acc[V];
-#pragma unroll
-                for (int j = 0; j < V; ++j) acc[j] = 0.f;
-                if (base) Elem<T>::unpack(raw[u], acc);
-                const float* dzt = dz + (tb + u) * E;
-#pragma unroll
-                for (int e = 0; e < kDxExperts; ++e)
-                    if (e < E) {
-                        const float d = dzt[e];
-#pragma unroll
-                        for (int j = 0; j < V; ++j) acc[j] += d * wv[e][j];
-                    }
-                *reinterpret_cast<uint4*>(out + (tb + u) * H + h) = Elem<T>::pack(acc);
-            }
-        }
+        for (int u = 0; u < U; ++u) ATS_DX_TOKEN(raw[u], tb + u);
     }
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+        if (tb + u < t1) ATS_DX_TOKEN(nxt[u], tb + u);
 #undef ATS_DX_FETCH
+#undef ATS_DX_TOKEN
 }
 
 // ---------------------------------------------------------------- router weight gradient
@@ -349,9 +355,12 @@ __global__ __launch_bounds__(256) void router_dw_partial_kernel(const float* __r
 }
 
 // The same sums with 16-byte loads: a thread owns V consecutive columns (H % V == 0, x 16-byte aligned) and asks
-// for the next 8 tokens' pieces while it uses the current 8 (16 at a time measured no faster); every column's
-// sum runs over the tokens in the same order as in the kernel above (same bits).
-template <typename T>
+// for the next 8 tokens' pieces while it uses the current 8 (16 at a time measured no faster).  A token's 8
+// gradients are wave uniform and come in as one scalar load: nothing in the loop over the experts is conditional
+// (the sums of absent experts are formed and dropped), since a test per expert made every value a load of its
+// own with a wait behind it.  Every column's sum runs over the tokens in the same order as in the kernel above
+// (same bits).
+template <typename T, bool FULL>   // FULL: E is a multiple of 8 (a token's 8 gradients are one 32-byte scalar load)
 __global__ __launch_bounds__(256) void router_dw_partial_vec_kernel(const float* __restrict__ dz,
                                                                     const T* __restrict__ x,
                                                                     float* __restrict__ partial, int64_t Tn, int E,
@@ -363,16 +372,29 @@ __global__ __launch_bounds__(256) void router_dw_partial_vec_kernel(const float*
     const int64_t t1 = t0 + chunk_tokens < Tn ? t0 + chunk_tokens : Tn;
     if (h >= H) return;
     for (int e0 = 0; e0 < E; e0 += kDwExperts) {
+        const int nv = E - e0 < kDwExperts ? E - e0 : kDwExperts;   // experts of this group that exist
         float acc[kDwExperts][V];
 #pragma unroll
         for (int i = 0; i < kDwExperts; ++i)
 #pragma unroll
             for (int j = 0; j < V; ++j) acc[i][j] = 0.f;
+#define ATS_DW_TOKEN(raw_, t_)                                                                         \
+    {                                                                                                  \
+        float xv[V];                                                                                   \
+        Elem<T>::unpack(raw_, xv);                                                                     \
+        const float* dzt = dz + (t_) * E + e0;                                                         \
+        float d[kDwExperts];                                                                           \
+        _Pragma("unroll") for (int i = 0; i < kDwExperts; ++i) d[i] = dzt[FULL || i < nv ? i : nv - 1]; \
+        _Pragma("unroll") for (int i = 0; i < kDwExperts; ++i) {                                       \
+            _Pragma("unroll") for (int j = 0; j < V; ++j) acc[i][j] += d[i] * xv[j];                   \
+        }                                                                                              \
+    }
         uint4 nxt[U];
 #pragma unroll
         for (int u = 0; u < U; ++u)
             if (t0 + u < t1) nxt[u] = *reinterpret_cast<const uint4*>(x + (t0 + u) * H + h);
-        for (int64_t tb = t0; tb < t1; tb += U) {
+        int64_t tb = t0;
+        for (; tb + U <= t1; tb += U) {
             uint4 raw[U];
 #pragma unroll
             for (int u = 0; u < U; ++u) raw[u] = nxt[u];
@@ -380,24 +402,15 @@ __global__ __launch_bounds__(256) void router_dw_partial_vec_kernel(const float*
             for (int u = 0; u < U; ++u)      // the next pieces travel while these are used
                 if (tb + U + u < t1) nxt[u] = *reinterpret_cast<const uint4*>(x + (tb + U + u) * H + h);
 #pragma unroll
-            for (int u = 0; u < U; ++u) {
-                if (tb + u < t1) {
-                    float xv[V];
-                    Elem<T>::unpack(raw[u], xv);
-                    const float* dzt = dz + (tb + u) * E + e0;
-#pragma unroll
-                    for (int i = 0; i < kDwExperts; ++i)
-                        if (e0 + i < E) {
-                            const float d = dzt[i];
-#pragma unroll
-                            for (int j = 0; j < V; ++j) acc[i][j] += d * xv[j];
-                        }
-                }
-            }
+            for (int u = 0; u < U; ++u) ATS_DW_TOKEN(raw[u], tb + u);
         }
 #pragma unroll
+        for (int u = 0; u < U; ++u)
+            if (tb + u < t1) ATS_DW_TOKEN(nxt[u], tb + u);
+#undef ATS_DW_TOKEN
+#pragma unroll
         for (int i = 0; i < kDwExperts; ++i)
-            if (e0 + i < E) {
+            if (i < nv) {
                 float* dst = partial + ((int64_t)blockIdx.y * E + e0 + i) * H + h;
 #pragma unroll
                 for (int j = 0; j < V; ++j) dst[j] = acc[i][j];
@@ -558,11 +571,15 @@ extern "C" int ats_router_bwd_dx(const float* dlogits, const void* wg, const voi
         // (base may alias out: a thread reads its piece of a row before it writes it)
         const dim3 grid((unsigned)((H / V + 255) / 256), (unsigned)((T + kDxChunk - 1) / kDxChunk));
         if (dtype == ATS_F32)
-            hipLaunchKernelGGL((router_dx_cols_kernel<float>), grid, dim3(256), 0, as_stream(stream), dlogits,
+            hipLaunchKernelGGL((router_dx_cols_kernel<float, false>), grid, dim3(256), 0, as_stream(stream), dlogits,
                                static_cast<const float*>(wg), static_cast<const float*>(base),
                                static_cast<float*>(out), T, E, H);
+        else if (E == kDxExperts)
+            hipLaunchKernelGGL((router_dx_cols_kernel<bf16_t, true>), grid, dim3(256), 0, as_stream(stream), dlogits,
+                               static_cast<const bf16_t*>(wg), static_cast<const bf16_t*>(base),
+                               static_cast<bf16_t*>(out), T, E, H);
         else
-            hipLaunchKernelGGL((router_dx_cols_kernel<bf16_t>), grid, dim3(256), 0, as_stream(stream), dlogits,
+            hipLaunchKernelGGL((router_dx_cols_kernel<bf16_t, false>), grid, dim3(256), 0, as_stream(stream), dlogits,
                                static_cast<const bf16_t*>(wg), static_cast<const bf16_t*>(base),
                                static_cast<bf16_t*>(out), T, E, H);
         ATS_CHECK_LAUNCH("ats_router_bwd_dx");
@@ -612,10 +629,13 @@ extern "C" int ats_router_bwd_dw(const float* dlogits, const void* x, float* dwg
     if (H % V == 0 && aligned16(x)) {
         const dim3 grid((unsigned)((H / V + 255) / 256), (unsigned)n_chunks);
         if (dtype == ATS_F32)
-            hipLaunchKernelGGL((router_dw_partial_vec_kernel<float>), grid, dim3(256), 0, s, dlogits,
+            hipLaunchKernelGGL((router_dw_partial_vec_kernel<float, false>), grid, dim3(256), 0, s, dlogits,
                                static_cast<const float*>(x), partial, T, E, H, chunk_tokens);
+        else if (E % kDwExperts == 0)
+            hipLaunchKernelGGL((router_dw_partial_vec_kernel<bf16_t, true>), grid, dim3(256), 0, s, dlogits,
+                               static_cast<const bf16_t*>(x), partial, T, E, H, chunk_tokens);
         else
-            hipLaunchKernelGGL((router_dw_partial_vec_kernel<bf16_t>), grid, dim3(256), 0, s, dlogits,
+            hipLaunchKernelGGL((router_dw_partial_vec_kernel<bf16_t, false>), grid, dim3(256), 0, s, dlogits,
                                static_cast<const bf16_t*>(x), partial, T, E, H, chunk_tokens);
     } else {
         const dim3 grid((unsigned)((H + 255) / 256), (unsigned)n_chunks);
