@@ -127,6 +127,7 @@ _SIGNATURES = {
     "fused_grad_clip_launcher": (c_float, [c_void_p, c_void_p, c_int, c_float, c_void_p]),
     "ats_legacy_last_status": (c_int, []),
     "ats_calibrate_copy": (c_int, [c_void_p, c_void_p, c_size_t, c_void_p]),
+    "ats_calibrate_read": (c_int, [c_void_p, c_size_t, c_void_p, c_void_p]),
     "ats_calibrate_mfma": (c_int, [c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]),
     "ats_debug_decode_tile": (c_int, [c_int64, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "ats_debug_decode_tiles_device": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int64,

@@ -123,7 +123,42 @@ __global__ __launch_bounds__(256) void calibrate_copy_kernel(const uint4* __rest
     }
 }
 
+// Plain streaming read, 16 bytes per lane and eight loads in flight per lane: the yardstick for the kernels
+// that stream weights (what a kernel that only reads its bytes, front to back, reaches).  The values are folded
+// into a word that is stored only if it takes one particular value, which keeps the loads alive.
+__global__ __launch_bounds__(256) void calibrate_read_kernel(const uint4* __restrict__ src, size_t n,
+                                                             unsigned* __restrict__ sink) {
+    size_t i = (size_t)blockIdx.x * 2048 + threadIdx.x;
+    const size_t stride = (size_t)gridDim.x * 2048;
+    unsigned acc = 0u;
+    for (; i < n; i += stride) {
+        uint4 v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            v[u] = make_uint4(0u, 0u, 0u, 0u);
+            if (i + u * 256 < n) v[u] = stream_load(src + i + u * 256);
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) acc ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
+    }
+    if (acc == 0x9e3779b9u) sink[0] = acc;
+}
+
 }  // namespace ats
+
+extern "C" int ats_calibrate_read(const void* src, size_t bytes, void* sink, ats_stream_t stream) {
+    using namespace ats;
+    ATS_REQUIRE(src && sink && bytes % 16 == 0 && aligned16(src), ATS_ERR_INVALID_ARG,
+                "ats_calibrate_read: a 16-byte aligned buffer of a multiple of 16 bytes and a 4-byte sink");
+    if (bytes == 0) return ATS_OK;
+    const size_t n = bytes / 16;
+    size_t blocks = (n + 2047) / 2048;
+    if (blocks > 2048) blocks = 2048;
+    hipLaunchKernelGGL(calibrate_read_kernel, dim3((unsigned)blocks), dim3(256), 0, as_stream(stream),
+                       static_cast<const uint4*>(src), n, static_cast<unsigned*>(sink));
+    ATS_CHECK_LAUNCH("ats_calibrate_read");
+    return ATS_OK;
+}
 
 extern "C" int ats_calibrate_copy(const void* src, void* dst, size_t bytes, ats_stream_t stream) {
     using namespace ats;

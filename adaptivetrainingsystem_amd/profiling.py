@@ -216,3 +216,14 @@ def stream_copy(src: torch.Tensor, dst: torch.Tensor) -> None:
         raise _lib.AtsError("stream_copy: contiguous GPU tensors of the same size")
     _lib.check(_lib.load().ats_calibrate_copy(src.data_ptr(), dst.data_ptr(), src.numel() * src.element_size(),
                                               _stream()), "ats_calibrate_copy")
+
+
+def stream_read(src: torch.Tensor, sink: torch.Tensor) -> None:
+    """The library's plain streaming read (16 bytes per lane, eight loads in flight): the yardstick for the
+    kernels that stream weights.  `sink`: any GPU tensor of at least 4 bytes (not written in practice)."""
+    from . import _lib
+    from .ops import _stream
+    if not (src.is_cuda and sink.is_cuda and src.is_contiguous()) or sink.numel() * sink.element_size() < 4:
+        raise _lib.AtsError("stream_read: a contiguous GPU tensor and a GPU sink of at least 4 bytes")
+    _lib.check(_lib.load().ats_calibrate_read(src.data_ptr(), src.numel() * src.element_size(), sink.data_ptr(),
+                                              _stream()), "ats_calibrate_read")

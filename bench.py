@@ -126,6 +126,28 @@ def gemm_calibration(w, moe, plan, kept: int, gu_ms: float):
     return out
 
 
+def stream_read_yardstick(nbytes, dev, reps=10):
+    """What a kernel that only reads `nbytes`, front to back, reaches (the library's plain streaming read)."""
+    from adaptivetrainingsystem_amd import profiling
+    nbytes -= nbytes % 16
+    buf = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+    buf.view(torch.int32).random_(0, 1 << 30)
+    sink = torch.zeros(16, dtype=torch.uint8, device=dev)
+    for _ in range(2):
+        profiling.stream_read(buf, sink)
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    ev0.record()
+    for _ in range(reps):
+        profiling.stream_read(buf, sink)
+    ev1.record()
+    torch.cuda.synchronize()
+    ms = ev0.elapsed_time(ev1) / reps
+    gbs = nbytes / (ms * 1e-3) / 1e9
+    return {"what": "this library's plain streaming read kernel (16 bytes per lane, eight loads in flight per lane, "
+                    "non-temporal) over as many bytes as the gate/up launch streams: what a kernel that only reads "
+                    "them reaches", "achieved": gbs, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS, "ms": ms}
+
+
 def run_moe(args):
     from adaptivetrainingsystem_amd import workloads as W
     from adaptivetrainingsystem_amd.profiling import StageTimer
@@ -190,6 +212,10 @@ def run_moe(args):
         roofline = {"kernel": "grouped gate/up GEMM + SwiGLU (weight streaming)", "bound": "hbm", "achieved": gbs,
                     "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gbs / PEAK_HBM_GBS,
                     "traffic": profile_traffic(name, "gateup")}
+        stream_read_reference = stream_read_yardstick(int(gu_bytes), dev)
+        stream_read_reference["gateup_vs_read"] = gbs / stream_read_reference["achieved"]
+        log(f"  plain streaming read of the same {gu_bytes / 1e9:.2f} GB: {stream_read_reference['achieved']:.0f} GB/s; "
+            f"the gate/up kernel reaches {stream_read_reference['gateup_vs_read']:.3f} of it")
     else:
         peak = PEAK_MFMA_TFLOPS[dtype_name]
         roofline = {"kernel": "grouped gate/up GEMM + SwiGLU", "bound": "mfma", "achieved": achieved,
@@ -210,6 +236,8 @@ def run_moe(args):
         "stages_median_p10_p90_ms": {s: [round(v["median_ms"], 4), round(v["p10_ms"], 4), round(v["p90_ms"], 4)]
                                      for s, v in stages.items()},
     }
+    if not mfma_bound:
+        result["stream_read_reference"] = stream_read_reference
     if mfma_bound and w.dtype == torch.bfloat16 and not args.no_calibration:
         with torch.no_grad():
             result["calibration"] = gemm_calibration(w, moe, plan, kept, gu_ms)

@@ -513,6 +513,10 @@ int ats_calibrate_mfma(int shape, int random_operands, int iters, uint64_t* cloc
 /* Plain streaming copy of `bytes` (a multiple of 16; both pointers 16-byte aligned): the yardstick that the
  * benchmark prints beside the bandwidth-bound kernels.  No reference counterpart. */
 int ats_calibrate_copy(const void* src, void* dst, size_t bytes, ats_stream_t stream);
+/* Plain streaming read of `bytes` (a multiple of 16; src 16-byte aligned; sink: 4 writable device bytes that are
+ * not written in practice): the yardstick that the benchmark prints beside the weight-streaming kernels of the
+ * decode-sized workloads.  No reference counterpart. */
+int ats_calibrate_read(const void* src, size_t bytes, void* sink, ats_stream_t stream);
 
 #ifdef __cplusplus
 }

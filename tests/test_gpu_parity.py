@@ -58,6 +58,22 @@ def ops(A):
     return _ops
 
 
+def test_calibration_yardsticks_move_the_bytes_they_claim(gpu):
+    """The streaming copy copies exactly, the streaming read leaves its sink alone (ragged sizes included)."""
+    from adaptivetrainingsystem_amd import profiling
+    g = torch.Generator(device=gpu)
+    g.manual_seed(11)
+    for n in (16, 4096 + 16, 3 * 1024 * 1024 + 48):
+        src = torch.randint(0, 255, (n,), dtype=torch.uint8, device=gpu, generator=g)
+        dst = torch.zeros_like(src)
+        profiling.stream_copy(src, dst)
+        assert torch.equal(src, dst)
+        sink = torch.full((16,), 7, dtype=torch.uint8, device=gpu)
+        profiling.stream_read(src, sink)
+        torch.cuda.synchronize()
+        assert bool((sink == 7).all())
+
+
 # ------------------------------------------------------------------ RMSNorm
 @pytest.mark.parametrize("shape", [(8, 512), (3, 5, 128), (7, 100), (64, 4096), (5, 8192), (3, 12000), (1, 8),
                                    (1000, 2048)])
