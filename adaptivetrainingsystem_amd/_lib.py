@@ -28,6 +28,7 @@ _SIGNATURES = {
     "ats_rope_fwd": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int,
                              c_int, c_int, c_int, c_int, c_int64, c_int64, c_int64, c_int64, c_int64, c_int64, c_int,
                              c_void_p]),
+    "ats_rope_fwd_append": (c_int, [c_void_p] * 8 + [c_int] * 8 + [c_int64] * 14 + [c_int, c_void_p]),
     "ats_router_logits": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_void_p]),
     "ats_route_topk_workspace": (c_size_t, [c_int64, c_int]),
     "ats_route_topk": (c_int, [c_void_p, c_int64, c_int, c_int, c_float, c_int, c_void_p, c_void_p, c_void_p,

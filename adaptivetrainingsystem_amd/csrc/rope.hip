@@ -22,10 +22,17 @@ struct RopeSeg {
     int64_t sb, sh, sl;  // input element strides: batch, head, position
     int heads;
     int chunks;  // ceil(heads / kRopeHeadsPerItem)
+    int64_t ob, oh, ol;  // output element strides (the position stride of a contiguous [B, H, L, D] result is D)
+    int rotate;          // 0: the rows are copied as they are (values appended to a cache beside the rotated keys)
 };
 
+static RopeSeg rope_seg(const void* in, void* out, int64_t sb, int64_t sh, int64_t sl, int heads, int L, int D) {
+    return RopeSeg{in, out, sb, sh, sl, heads, (heads + kRopeHeadsPerItem - 1) / kRopeHeadsPerItem,
+                   (int64_t)heads * L * D, (int64_t)L * D, (int64_t)D, 1};
+}
+
 template <typename T>
-__global__ __launch_bounds__(256) void rope_vec_kernel(RopeSeg q, RopeSeg k, const float* __restrict__ cos_tab,
+__global__ __launch_bounds__(256) void rope_vec_kernel(RopeSeg q, RopeSeg k, RopeSeg v3, const float* __restrict__ cos_tab,
                                                        const float* __restrict__ sin_tab, int table_stride,
                                                        int L, int D, int pos_offset, int lanes_per_row,
                                                        int pos_per_wave, int n_pos_groups, int64_t n_items, bool tab_vec,
@@ -36,11 +43,12 @@ __global__ __launch_bounds__(256) void rope_vec_kernel(RopeSeg q, RopeSeg k, con
     if (item >= n_items) return;
     const int pg = (int)(item % n_pos_groups);
     const int64_t rest = item / n_pos_groups;
-    const int total_chunks = q.chunks + k.chunks;
+    const int total_chunks = q.chunks + k.chunks + v3.chunks;
     int chunk = (int)(rest % total_chunks);
     const int b = (int)(rest / total_chunks);
-    const RopeSeg& seg = chunk < q.chunks ? q : k;
-    if (chunk >= q.chunks) chunk -= q.chunks;
+    const RopeSeg& seg = chunk < q.chunks ? q : chunk < q.chunks + k.chunks ? k : v3;
+    if (chunk >= q.chunks + k.chunks) chunk -= q.chunks + k.chunks;
+    else if (chunk >= q.chunks) chunk -= q.chunks;
 
     const int prow = lane / lanes_per_row;
     const int c = lane - prow * lanes_per_row;
@@ -96,20 +104,21 @@ __global__ __launch_bounds__(256) void rope_vec_kernel(RopeSeg q, RopeSeg k, con
                 o1[j] = ((((a[j]) * (cs[j]))) - (((bb[j]) * (sn[j]))));
                 o2[j] = ((((a[j]) * (sn[j]))) + (((bb[j]) * (cs[j]))));
             }
-            T* p = out + (((int64_t)b * seg.heads + h) * L + pos) * D + c * V;
-            stream_store(reinterpret_cast<uint4*>(p), Elem<T>::pack(o1));
-            stream_store(reinterpret_cast<uint4*>(p + half), Elem<T>::pack(o2));
+            T* p = out + b * seg.ob + h * seg.oh + pos * seg.ol + c * V;
+            stream_store(reinterpret_cast<uint4*>(p), seg.rotate ? Elem<T>::pack(o1) : lo[i]);
+            stream_store(reinterpret_cast<uint4*>(p + half), seg.rotate ? Elem<T>::pack(o2) : hi[i]);
         }
     }
 }
 
 // Any even D / alignment: one thread per rotated pair.
 template <typename T>
-__global__ __launch_bounds__(256) void rope_scalar_kernel(RopeSeg q, RopeSeg k, const float* __restrict__ cos_tab,
+__global__ __launch_bounds__(256) void rope_scalar_kernel(RopeSeg q, RopeSeg k, RopeSeg v3, const float* __restrict__ cos_tab,
                                                           const float* __restrict__ sin_tab, int table_stride,
                                                           int B, int L, int D, int pos_offset, float sin_sign) {
     const int half = D >> 1;
-    const int64_t per_b = (int64_t)(q.heads + k.heads) * L * half;
+    const int heads_all = q.heads + k.heads + v3.heads;
+    const int64_t per_b = (int64_t)heads_all * L * half;
     const int64_t total = per_b * B;
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
          i += (int64_t)gridDim.x * blockDim.x) {
@@ -117,17 +126,22 @@ __global__ __launch_bounds__(256) void rope_scalar_kernel(RopeSeg q, RopeSeg k, 
         int64_t r = i / half;
         const int pos = (int)(r % L);
         r /= L;
-        const int hh = (int)(r % (q.heads + k.heads));
-        const int b = (int)(r / (q.heads + k.heads));
-        const RopeSeg& seg = hh < q.heads ? q : k;
-        const int h = hh < q.heads ? hh : hh - q.heads;
+        const int hh = (int)(r % heads_all);
+        const int b = (int)(r / heads_all);
+        const RopeSeg& seg = hh < q.heads ? q : hh < q.heads + k.heads ? k : v3;
+        const int h = hh < q.heads ? hh : hh < q.heads + k.heads ? hh - q.heads : hh - q.heads - k.heads;
         const T* p = static_cast<const T*>(seg.in) + b * seg.sb + h * seg.sh + pos * seg.sl + d;
         const float a = Elem<T>::load(p), bb = Elem<T>::load(p + half);
         const float cs = cos_tab[(int64_t)(pos_offset + pos) * table_stride + d];
         const float sn = sin_tab[(int64_t)(pos_offset + pos) * table_stride + d] * sin_sign;
-        T* o = static_cast<T*>(seg.out) + (((int64_t)b * seg.heads + h) * L + pos) * D + d;
-        Elem<T>::store(o, ((((a) * (cs))) - (((bb) * (sn)))));
-        Elem<T>::store(o + half, ((((a) * (sn))) + (((bb) * (cs)))));
+        T* o = static_cast<T*>(seg.out) + b * seg.ob + h * seg.oh + pos * seg.ol + d;
+        if (seg.rotate) {
+            Elem<T>::store(o, ((((a) * (cs))) - (((bb) * (sn)))));
+            Elem<T>::store(o + half, ((((a) * (sn))) + (((bb) * (cs)))));
+        } else {
+            o[0] = p[0];
+            o[half] = p[half];
+        }
     }
 }
 
@@ -156,24 +170,24 @@ __global__ __launch_bounds__(256) void rope_table_kernel(float* __restrict__ cos
 }
 
 template <typename T>
-static void launch_rope(RopeSeg q, RopeSeg k, const float* cos_tab, const float* sin_tab, int table_stride, int B,
+static void launch_rope(RopeSeg q, RopeSeg k, RopeSeg v3, const float* cos_tab, const float* sin_tab, int table_stride, int B,
                         int L, int D, int pos_offset, bool vec_ok, float sin_sign, hipStream_t s) {
     constexpr int V = Elem<T>::kVec;
     if (vec_ok) {
         const int lanes_per_row = (D / 2) / V;
         const int pos_per_wave = kWave / lanes_per_row;
         const int n_pos_groups = (L + pos_per_wave - 1) / pos_per_wave;
-        const int64_t n_items = (int64_t)n_pos_groups * (q.chunks + k.chunks) * B;
+        const int64_t n_items = (int64_t)n_pos_groups * (q.chunks + k.chunks + v3.chunks) * B;
         const int64_t blocks = (n_items + 3) / 4;
         const bool tab_vec = table_stride % 4 == 0 && aligned16(cos_tab) && aligned16(sin_tab);
-        hipLaunchKernelGGL((rope_vec_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, s, q, k, cos_tab, sin_tab,
+        hipLaunchKernelGGL((rope_vec_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, s, q, k, v3, cos_tab, sin_tab,
                            table_stride, L, D, pos_offset, lanes_per_row, pos_per_wave, n_pos_groups, n_items, tab_vec,
                            sin_sign);
     } else {
-        const int64_t total = (int64_t)B * (q.heads + k.heads) * L * (D / 2);
+        const int64_t total = (int64_t)B * (q.heads + k.heads + v3.heads) * L * (D / 2);
         int64_t blocks = (total + 255) / 256;
         if (blocks > 65536) blocks = 65536;
-        hipLaunchKernelGGL((rope_scalar_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, s, q, k, cos_tab, sin_tab,
+        hipLaunchKernelGGL((rope_scalar_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, s, q, k, v3, cos_tab, sin_tab,
                            table_stride, B, L, D, pos_offset, sin_sign);
     }
 }
@@ -198,10 +212,22 @@ extern "C" int ats_rope_table(float* cos_out, float* sin_out, int seq_len, int d
     return ATS_OK;
 }
 
+// Where the rotated keys and the untouched values go when they are appended to a key / value cache
+// [B, Hkv, capacity, D] (element strides cb, ch, cl) behind its first `pos` positions.
+struct RopeCacheTarget {
+    void* k_cache;
+    void* v_cache;
+    const void* v_in;
+    int64_t v_sb, v_sh, v_sl;
+    int64_t cb, ch, cl;
+    int64_t pos;
+};
+
 static int rope_apply(const char* name, float sin_sign, const void* q_in, const void* k_in, void* q_out, void* k_out,
                       const float* cos_tab, const float* sin_tab, int table_stride, int table_len, int B, int Hq,
                       int Hkv, int L, int D, int pos_offset, int64_t q_sb, int64_t q_sh, int64_t q_sl, int64_t k_sb,
-                      int64_t k_sh, int64_t k_sl, int dtype, ats_stream_t stream) {
+                      int64_t k_sh, int64_t k_sl, int dtype, ats_stream_t stream,
+                      const RopeCacheTarget* cache = nullptr) {
     using namespace ats;
     ATS_REQUIRE(B >= 0 && Hq >= 0 && Hkv >= 0 && L >= 0 && D > 0 && D % 2 == 0, ATS_ERR_INVALID_ARG,
                 "%s: B=%d Hq=%d Hkv=%d L=%d D=%d", name, B, Hq, Hkv, L, D);
@@ -211,21 +237,31 @@ static int rope_apply(const char* name, float sin_sign, const void* q_in, const 
                 "%s: table pointers/stride (stride=%d, need >= %d)", name, table_stride, D / 2);
     ATS_REQUIRE(pos_offset >= 0 && (int64_t)pos_offset + L <= table_len, ATS_ERR_INVALID_ARG,
                 "%s: positions %d..%d exceed table length %d", name, pos_offset, pos_offset + L - 1, table_len);
-    ATS_REQUIRE((Hq == 0 || (q_in && q_out)) && (Hkv == 0 || (k_in && k_out)), ATS_ERR_INVALID_ARG,
-                "%s: null tensor pointer", name);
-    RopeSeg q{q_in, q_out, q_sb, q_sh, q_sl, Hq, (Hq + kRopeHeadsPerItem - 1) / kRopeHeadsPerItem};
-    RopeSeg k{k_in, k_out, k_sb, k_sh, k_sl, Hkv, (Hkv + kRopeHeadsPerItem - 1) / kRopeHeadsPerItem};
+    ATS_REQUIRE((Hq == 0 || (q_in && q_out)) && (Hkv == 0 || (k_in && (cache ? cache->k_cache : k_out))),
+                ATS_ERR_INVALID_ARG, "%s: null tensor pointer", name);
+    RopeSeg q = rope_seg(q_in, q_out, q_sb, q_sh, q_sl, Hq, L, D);
+    RopeSeg k = rope_seg(k_in, k_out, k_sb, k_sh, k_sl, Hkv, L, D);
+    RopeSeg v3 = rope_seg(nullptr, nullptr, 0, 0, 0, 0, L, D);
+    if (cache) {
+        // keys and values go behind the cache's first cache->pos positions instead of into a tensor of their own
+        k.out = static_cast<char*>(cache->k_cache) + cache->pos * cache->cl * (dtype == ATS_F32 ? 4 : 2);
+        k.ob = cache->cb, k.oh = cache->ch, k.ol = cache->cl;
+        v3 = rope_seg(cache->v_in, static_cast<char*>(cache->v_cache) + cache->pos * cache->cl * (dtype == ATS_F32 ? 4 : 2),
+                      cache->v_sb, cache->v_sh, cache->v_sl, Hkv, L, D);
+        v3.ob = cache->cb, v3.oh = cache->ch, v3.ol = cache->cl;
+        v3.rotate = 0;
+    }
     const int V = dtype == ATS_F32 ? 4 : 8;
     auto seg_ok = [&](const RopeSeg& sgm) {
         return sgm.heads == 0 || (aligned16(sgm.in) && aligned16(sgm.out) && sgm.sb % V == 0 && sgm.sh % V == 0 &&
-                                  sgm.sl % V == 0);
+                                  sgm.sl % V == 0 && sgm.ob % V == 0 && sgm.oh % V == 0 && sgm.ol % V == 0);
     };
     const int half = D / 2;
-    const bool vec_ok = half % V == 0 && half / V <= kWave && seg_ok(q) && seg_ok(k);
+    const bool vec_ok = half % V == 0 && half / V <= kWave && seg_ok(q) && seg_ok(k) && seg_ok(v3);
     if (dtype == ATS_F32)
-        launch_rope<float>(q, k, cos_tab, sin_tab, table_stride, B, L, D, pos_offset, vec_ok, sin_sign, as_stream(stream));
+        launch_rope<float>(q, k, v3, cos_tab, sin_tab, table_stride, B, L, D, pos_offset, vec_ok, sin_sign, as_stream(stream));
     else
-        launch_rope<bf16_t>(q, k, cos_tab, sin_tab, table_stride, B, L, D, pos_offset, vec_ok, sin_sign, as_stream(stream));
+        launch_rope<bf16_t>(q, k, v3, cos_tab, sin_tab, table_stride, B, L, D, pos_offset, vec_ok, sin_sign, as_stream(stream));
     ATS_CHECK_LAUNCH(name);
     return ATS_OK;
 }
@@ -244,4 +280,21 @@ extern "C" int ats_rope_bwd(const void* dq_out, const void* dk_out, void* dq, vo
                             int64_t k_sh, int64_t k_sl, int dtype, ats_stream_t stream) {
     return rope_apply("ats_rope_bwd", -1.0f, dq_out, dk_out, dq, dk, cos_tab, sin_tab, table_stride, table_len, B, Hq,
                       Hkv, L, D, pos_offset, q_sb, q_sh, q_sl, k_sb, k_sh, k_sl, dtype, stream);
+}
+
+extern "C" int ats_rope_fwd_append(const void* q_in, const void* k_in, const void* v_in, void* q_out, void* k_cache,
+                                   void* v_cache, const float* cos_tab, const float* sin_tab, int table_stride,
+                                   int table_len, int B, int Hq, int Hkv, int L, int D, int pos_offset, int64_t q_sb,
+                                   int64_t q_sh, int64_t q_sl, int64_t k_sb, int64_t k_sh, int64_t k_sl, int64_t v_sb,
+                                   int64_t v_sh, int64_t v_sl, int64_t cache_sb, int64_t cache_sh, int64_t cache_sl,
+                                   int64_t cache_pos, int64_t cache_capacity, int dtype, ats_stream_t stream) {
+    using namespace ats;
+    ATS_REQUIRE(Hkv > 0 && k_in && v_in && k_cache && v_cache, ATS_ERR_INVALID_ARG,
+                "ats_rope_fwd_append: keys, values and both caches are required");
+    ATS_REQUIRE(cache_pos >= 0 && L >= 0 && cache_pos + L <= cache_capacity && cache_sl >= D, ATS_ERR_INVALID_ARG,
+                "ats_rope_fwd_append: positions %lld..%lld do not fit a cache of %lld (position stride %lld, D=%d)",
+                (long long)cache_pos, (long long)(cache_pos + L - 1), (long long)cache_capacity, (long long)cache_sl, D);
+    RopeCacheTarget tgt{k_cache, v_cache, v_in, v_sb, v_sh, v_sl, cache_sb, cache_sh, cache_sl, cache_pos};
+    return rope_apply("ats_rope_fwd_append", 1.0f, q_in, k_in, q_out, nullptr, cos_tab, sin_tab, table_stride,
+                      table_len, B, Hq, Hkv, L, D, pos_offset, q_sb, q_sh, q_sl, k_sb, k_sh, k_sl, dtype, stream, &tgt);
 }

@@ -233,15 +233,17 @@ class GroupedQueryAttention(nn.Module):
             q, k, v = qkv[:, :nh], qkv[:, nh:nh + nkv], qkv[:, nh + nkv:]
         # positions 0..L-1 also when a cache is passed, as the reference does (model.py:690-698)
         cos, sin = self.rope(L, x.device)
-        q, k = ag.RoPEFunction.apply(q, k, cos, sin, 0) if grad else ops.rope(q, k, cos, sin, 0)
         if past_key_value is not None:
             k_cache, v_cache = past_key_value
             if (k_cache.dim() != 4 or k_cache.shape[0] != B or k_cache.shape[1] != nkv or k_cache.shape[3] != D
                     or v_cache.shape != k_cache.shape):
                 raise AtsError(f"GroupedQueryAttention: cache shapes {tuple(k_cache.shape)} / {tuple(v_cache.shape)}")
-            if use_cache and not grad:
-                k, v = self._extend_cache(k_cache, v_cache, k, v)
-            else:
+        if past_key_value is not None and use_cache and not grad:
+            # the rotation writes the new keys, and the values beside them, straight behind the cache
+            q, k, v = self._extend_cache(k_cache, v_cache, q, k, v, cos, sin)
+        else:
+            q, k = ag.RoPEFunction.apply(q, k, cos, sin, 0) if grad else ops.rope(q, k, cos, sin, 0)
+            if past_key_value is not None:
                 k = torch.cat([k_cache.to(k.dtype), k], dim=2)
                 v = torch.cat([v_cache.to(v.dtype), v], dim=2)
         key_bias = pair_bias = None
@@ -304,8 +306,9 @@ class GroupedQueryAttention(nn.Module):
         self._state["qkv_key"] = None
         self._state["qkv"] = None
 
-    def _extend_cache(self, k_cache, v_cache, k_new, v_new):
-        """The cache followed by the new rows, as the reference's torch.cat gives them (model.py:700-704), without
+    def _extend_cache(self, k_cache, v_cache, q, k_new, v_new, cos, sin):
+        """The rotated q, and the cache followed by the new rows (keys rotated, values as they are), as the
+        reference's rotation and torch.cat give them (model.py:690-704), without
         copying the cache on every step: the tensors handed back are the first rows of buffers
         [batch, kv heads, capacity, head_dim] with room to grow, and when the same tensors come back as
         past_key_value the new rows are written behind them in place.  Only the latest state is extended in
@@ -332,11 +335,10 @@ class GroupedQueryAttention(nn.Module):
             v_buf = torch.empty(B, nkv, cap, D, dtype=v_new.dtype, device=v_new.device)
             k_buf[:, :, :Lp].copy_(k_cache)
             v_buf[:, :, :Lp].copy_(v_cache)
-        k_buf[:, :, Lp:Lp + L].copy_(k_new)
-        v_buf[:, :, Lp:Lp + L].copy_(v_new)
+        q = ops.rope_append(q, k_new, v_new, cos, sin, k_buf, v_buf, Lp, 0)
         self._state["kv"] = {"k_ptr": k_buf.data_ptr(), "v_ptr": v_buf.data_ptr(), "capacity": cap, "length": Lp + L,
                            "nbytes": k_buf.numel() * k_buf.element_size()}
-        return k_buf[:, :, :Lp + L], v_buf[:, :, :Lp + L]
+        return q, k_buf[:, :, :Lp + L], v_buf[:, :, :Lp + L]
 
     def get_attention_stats(self) -> Dict[str, Any]:
         calls = self._state["calls"]

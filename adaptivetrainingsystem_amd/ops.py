@@ -116,6 +116,39 @@ def rope(q: torch.Tensor, k: Optional[torch.Tensor], cos: torch.Tensor, sin: tor
     return q_out, k_out
 
 
+def rope_append(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor,
+                k_cache: torch.Tensor, v_cache: torch.Tensor, cache_pos: int,
+                position_offset: int = 0) -> torch.Tensor:
+    """rope(q, k) with the rotated keys, and the values beside them, written into the cache buffers
+    k_cache / v_cache [B, Hkv, capacity, D] at positions cache_pos .. cache_pos + L - 1 (one launch instead of the
+    rotation and two strided copies).  Returns the rotated q as a new contiguous tensor."""
+    _need_gpu(q, k, v, cos, sin, k_cache, v_cache)
+    if q.dim() != 4 or k.dim() != 4 or v.shape != k.shape or k_cache.dim() != 4 or v_cache.shape != k_cache.shape:
+        raise AtsError("rope_append: q, k, v [batch, heads, seq, head_dim] and two caches of one shape")
+    B, Hq, L, D = q.shape
+    Hkv = k.shape[1]
+    if (k.shape[0] != B or k.shape[2] != L or k.shape[3] != D or k.dtype != q.dtype or v.dtype != q.dtype
+            or k_cache.dtype != q.dtype or v_cache.dtype != q.dtype or k_cache.shape[0] != B
+            or k_cache.shape[1] != Hkv or k_cache.shape[3] != D or k_cache.stride() != v_cache.stride()
+            or k_cache.stride(3) != 1):
+        raise AtsError(f"rope_append: k/v {tuple(k.shape)}, caches {tuple(k_cache.shape)} do not match q {tuple(q.shape)}")
+    if cos.dtype != torch.float32 or sin.dtype != torch.float32 or cos.shape != sin.shape or cos.dim() != 2:
+        raise AtsError("rope_append: cos/sin must be float32 2-D tables of equal shape")
+    if cos.stride(1) != 1 or sin.stride(1) != 1 or cos.stride(0) != sin.stride(0):
+        cos, sin = cos.contiguous(), sin.contiguous()
+    q, qsb, qsh, qsl = _bhl_strides(q)
+    k, ksb, ksh, ksl = _bhl_strides(k)
+    v, vsb, vsh, vsl = _bhl_strides(v)
+    q_out = torch.empty((B, Hq, L, D), dtype=q.dtype, device=q.device)
+    check(_lib.load().ats_rope_fwd_append(q.data_ptr(), k.data_ptr(), v.data_ptr(), q_out.data_ptr(),
+                                          k_cache.data_ptr(), v_cache.data_ptr(), cos.data_ptr(), sin.data_ptr(),
+                                          cos.stride(0), cos.shape[0], B, Hq, Hkv, L, D, int(position_offset),
+                                          qsb, qsh, qsl, ksb, ksh, ksl, vsb, vsh, vsl, k_cache.stride(0),
+                                          k_cache.stride(1), k_cache.stride(2), int(cache_pos), k_cache.shape[2],
+                                          _tag(q), _stream()), "ats_rope_fwd_append")
+    return q_out
+
+
 # --------------------------------------------------------------------------- router
 def router_logits(x: torch.Tensor, gate_weight: torch.Tensor, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
     """x [T,H], gate_weight [E,H] (same dtype) -> float32 logits [T,E]."""

@@ -79,6 +79,20 @@ int ats_rope_fwd(const void* q_in, const void* k_in, void* q_out, void* k_out, c
                  const float* sin_tab, int table_stride, int table_len, int B, int Hq, int Hkv, int L,
                  int D, int pos_offset, int64_t q_sb, int64_t q_sh, int64_t q_sl, int64_t k_sb,
                  int64_t k_sh, int64_t k_sl, int dtype, ats_stream_t stream);
+/* ats_rope_fwd whose rotated keys, and the values beside them, are appended to a key / value cache instead of
+ * going into tensors of their own: the in-place form of torch.cat([past_key, k], dim=2) /
+ * torch.cat([past_value, v], dim=2) in GroupedQueryAttention.forward (model.py:700-704) for a cache buffer
+ * [B, Hkv, cache_capacity, D] with element strides (cache_sb, cache_sh, cache_sl; D contiguous) that holds
+ * cache_pos positions: k (rotated) and v (copied bit for bit, addressed through v_sb / v_sh / v_sl like q and k)
+ * land at positions cache_pos .. cache_pos + L - 1; q_out is contiguous [B, Hq, L, D].  The rotation uses
+ * position pos_offset + l, independent of cache_pos (the reference rotates a decoding step's rows as positions
+ * 0 .. L-1, model.py:690-698). */
+int ats_rope_fwd_append(const void* q_in, const void* k_in, const void* v_in, void* q_out, void* k_cache,
+                        void* v_cache, const float* cos_tab, const float* sin_tab, int table_stride,
+                        int table_len, int B, int Hq, int Hkv, int L, int D, int pos_offset, int64_t q_sb,
+                        int64_t q_sh, int64_t q_sl, int64_t k_sb, int64_t k_sh, int64_t k_sl, int64_t v_sb,
+                        int64_t v_sh, int64_t v_sl, int64_t cache_sb, int64_t cache_sh, int64_t cache_sl,
+                        int64_t cache_pos, int64_t cache_capacity, int dtype, ats_stream_t stream);
 
 /* ---- Router -------------------------------------------------------------
  * logits[T,E] (float32) = x[T,H] . wg[E,H]^T (+ bias[E] if not NULL): the

@@ -273,6 +273,31 @@ def test_gqa_module_backward(gpu, hidden, nh, nkv, B, L):
 
 
 # --------------------------------------------------------------------------- the whole block
+@pytest.mark.parametrize("B,Hq,Hkv,L,D,pos,cap,dtype", [(2, 8, 2, 1, 128, 37, 64, torch.bfloat16),
+                                                        (1, 4, 4, 5, 64, 0, 5, torch.bfloat16),
+                                                        (3, 6, 2, 3, 128, 10, 13, torch.float32),
+                                                        (1, 2, 1, 4, 6, 2, 9, torch.float32)])
+def test_rope_append_equals_rope_then_copies(ops, gpu, B, Hq, Hkv, L, D, pos, cap, dtype):
+    """The rotation that writes keys and values behind a cache: the bits of rope() followed by the two copies,
+    with q, k, v as column ranges of one projection output (strided), and nothing else of the cache touched."""
+    print("case rope_append", B, Hq, Hkv, L, D, pos, cap, dtype, flush=True)
+    g = torch.Generator().manual_seed(77)
+    qkv = torch.randn(B, L, Hq + 2 * Hkv, D, generator=g).to(dtype).to(gpu).transpose(1, 2)
+    q, k, v = qkv[:, :Hq], qkv[:, Hq:Hq + Hkv], qkv[:, Hq + Hkv:]
+    cos, sin = ops.rope_table(64, D, 10000.0, None, half=True)
+    k_cache = torch.randn(B, Hkv, cap, D, generator=g).to(dtype).to(gpu)
+    v_cache = torch.randn(B, Hkv, cap, D, generator=g).to(dtype).to(gpu)
+    k_want, v_want = k_cache.clone(), v_cache.clone()
+    q_ref, k_ref = ops.rope(q, k, cos, sin, 3)
+    k_want[:, :, pos:pos + L] = k_ref
+    v_want[:, :, pos:pos + L] = v
+    q_out = ops.rope_append(q, k, v, cos, sin, k_cache, v_cache, pos, 3)
+    assert torch.equal(q_out, q_ref) and torch.equal(k_cache, k_want) and torch.equal(v_cache, v_want)
+    from adaptivetrainingsystem_amd._lib import AtsError
+    with pytest.raises(AtsError):
+        ops.rope_append(q, k, v, cos, sin, k_cache, v_cache, cap - L + 1, 3)
+
+
 def test_gqa_module_cache_grows_in_place(gpu):
     """Decoding step after step: the cache handed back is the head of a buffer with room to grow, the next
     step writes its rows behind it without copying, and outputs and cache contents equal what concatenation
