@@ -170,11 +170,10 @@ class GroupedQueryAttention(nn.Module):
     attention itself through their HIP kernels; the score matrix is never materialised.  Built: gradients of
     every input and parameter, past_key_value / use_cache (model.py:700-708; the cache grows in place),
     attention_mask [batch, keys] or [batch, 1, queries, keys] (model.py:819-824), attention dropout in training
-    mode (config.dropout > 0, model.py:622-623, 831-833: the mask is a hash of a per-call seed drawn from
-    torch's seed and a call counter, not torch's generator stream), float32 activations (the scores are then
+    mode (config.dropout > 0, model.py:622-623, 831-833: the mask is a hash of a per-call 62-bit seed drawn
+    from torch's CPU generator, so torch.manual_seed reproduces it and a checkpointed recomputation, which
+    replays that generator's state, draws the same mask again), float32 activations (the scores are then
     materialised between two float32 grouped products, as the reference's _standard_attention does)."""
-
-    _instances = 0      # construction order: the layers of a model draw different dropout masks
 
     def __init__(self, config):
         super().__init__()
@@ -203,11 +202,8 @@ class GroupedQueryAttention(nn.Module):
         # per-call bookkeeping lives in one dict that is mutated in place: assigning module attributes on every
         # call goes through nn.Module.__setattr__, a visible part of a decoding step
         #   kv: addresses and fill of the cache buffers handed out last (no tensor is held)
-        #   dropout_stream: tells the layers of a model apart (id-based, fixed at construction)
         self._state: Dict[str, Any] = {"calls": 0, "kv": None, "kv_copies": 0, "kv_appends": 0, "qkv_key": None,
-                                       "qkv": None, "dropout_stream": GroupedQueryAttention._instances,
-                                       "last_dropout_seed": 0}
-        GroupedQueryAttention._instances += 1
+                                       "qkv": None, "last_dropout_seed": 0}
 
     def forward(self, x: torch.Tensor, attention_mask: Optional[torch.Tensor] = None, past_key_value=None,
                 use_cache: bool = False):
@@ -263,10 +259,12 @@ class GroupedQueryAttention(nn.Module):
                                f"{tuple(attention_mask.shape)}")
         drop_p, drop_seed = 0.0, 0
         if self.training and self.dropout_p > 0:
-            # a fresh mask per call, reproducible under torch.manual_seed: no device round trip
+            # a fresh mask per call and layer, drawn from torch's CPU generator (no device round trip): the seed
+            # depends on torch.manual_seed and on the draws made since, not on how many modules were ever built,
+            # and torch.utils.checkpoint (preserve_rng_state) replays it in its recomputation, so the mask of the
+            # recomputed forward is the one the saved output and log-sum-exp were made with
             drop_p = self.dropout_p
-            drop_seed = (torch.initial_seed() + 0x9E3779B97F4A7C15 * (self._state["calls"] + 1)
-                         + 0xD1B54A32D192ED03 * self._state["dropout_stream"]) & 0xFFFFFFFFFFFFFFFF
+            drop_seed = int(torch.randint(0, 2 ** 62, (1,), device="cpu").item())
         if x.dtype == torch.float32:
             # the reference's own route for float32 (scores materialised, model.py:807-839), on the float32 kernels
             if grad:

@@ -82,8 +82,12 @@ class MoEPerformanceMonitor:
         self.pytorch_calls += 1
         self.pytorch_tokens += num_tokens
 
+    _PENDING_BOUND = 1024
+
     def _record_events(self, start, stop, use_cuda: bool, num_tokens: int) -> None:
         self._pending.append((start, stop, use_cuda))
+        if len(self._pending) > self._PENDING_BOUND:
+            self._collect_finished()
         if use_cuda:
             self.cuda_calls += 1
             self.cuda_tokens += num_tokens
@@ -91,16 +95,35 @@ class MoEPerformanceMonitor:
             self.pytorch_calls += 1
             self.pytorch_tokens += num_tokens
 
+    def _add_elapsed(self, start, stop, use_cuda: bool) -> None:
+        ms = start.elapsed_time(stop)
+        if use_cuda:
+            self.cuda_time += ms
+        else:
+            self.pytorch_time += ms
+
+    def _collect_finished(self) -> None:
+        """Reads the pairs whose stop event has already completed, without synchronising, so a loop that
+        monitors for a long time and seldom asks for statistics holds a bounded number of events.  If the
+        device is more than a bound's worth of calls behind the host, the oldest pair is waited for."""
+        keep = []
+        for start, stop, use_cuda in self._pending:
+            if stop.query():
+                self._add_elapsed(start, stop, use_cuda)
+            else:
+                keep.append((start, stop, use_cuda))
+        if len(keep) > self._PENDING_BOUND:
+            keep[0][1].synchronize()
+            self._add_elapsed(*keep[0])
+            keep = keep[1:]
+        self._pending = keep
+
     def _drain(self) -> None:
         if not self._pending:
             return
         torch.cuda.synchronize()
         for start, stop, use_cuda in self._pending:
-            ms = start.elapsed_time(stop)
-            if use_cuda:
-                self.cuda_time += ms
-            else:
-                self.pytorch_time += ms
+            self._add_elapsed(start, stop, use_cuda)
         self._pending = []
 
     def get_stats(self) -> Dict[str, float]:

@@ -882,13 +882,76 @@ def run_norm_rope(args):
     return result
 
 
+def _r(v, n=4):
+    return None if v is None else round(float(v), n)
+
+
+def _roof(r):
+    return {"bound": r["bound"], "achieved": _r(r["achieved"], 1), "peak": r["peak"], "unit": r["unit"],
+            "frac": _r(r["frac"]), "traffic": r.get("traffic")}
+
+
+def secondary_records(args):
+    """The other benchmark configurations, each from a short event-timed loop of its own in this process
+    (their own step and warm-up counts; no CPU leg, no calibration): config 2's RMSNorm / RoPE against the HBM
+    peak and against the streaming-copy yardstick, config 3's weight-streaming GEMMs against the HBM peak and the
+    streaming-read yardstick, config 5's step time and grouped GEMM against the MFMA peak."""
+    import copy
+    out = {}
+    sub = copy.copy(args)
+    sub.no_cpu_baseline, sub.no_calibration = True, True
+    sub.steps, sub.warmup = 200, 50
+
+    sub.workload = "c2_norm_rope"
+    r = run_norm_rope(sub)
+    out["c2_norm_rope"] = {
+        "workload": r["config"]["workload"], "ms_per_step": _r(r["ms_per_step"], 5),
+        "rmsnorm": _roof(r["rmsnorm_roofline"]), "rope": _roof(r["roofline"]),
+        "rmsnorm_bwd": _roof(r["rmsnorm_bwd_roofline"]), "rope_bwd": _roof(r["rope_bwd_roofline"]),
+        "stream_copy_reference": {k: _r(v) for k, v in r["stream_copy_reference"].items() if k != "what"},
+        "copy_reference": {k: _r(v) for k, v in r["copy_reference"].items() if k != "what"},
+        "kernel_us": {k: _r(v * 1e3, 2) for k, v in r["stages_ms"].items()}}
+    torch.cuda.empty_cache()
+
+    sub.workload = "c3_decode"
+    r = run_moe(sub)
+    st = r["stages_ms"]
+    H, I, es = 4096, 14336, 2
+    kept = r["config"]["kept_assignments"]
+    dn_bytes = 8 * H * I * es + kept * (H + I) * es            # every expert's down weight once + rows in and out
+    dn_ms = st["down"]
+    out["c3_decode"] = {
+        "workload": r["config"]["workload"], "tokens_per_s": _r(r["value"], 0), "ms_per_step": _r(r["ms_per_step"]),
+        "gateup": _roof(r["roofline"]),
+        "down": {"bound": "hbm", "achieved": _r(dn_bytes / (dn_ms * 1e-3) / 1e9, 1), "peak": PEAK_HBM_GBS,
+                 "unit": "GB/s", "frac": _r(dn_bytes / (dn_ms * 1e-3) / 1e9 / PEAK_HBM_GBS),
+                 "traffic": profile_traffic("c3_decode", "down")},
+        "stream_read_reference": {k: _r(v) for k, v in r["stream_read_reference"].items() if k != "what"},
+        "stages_ms": st}
+    torch.cuda.empty_cache()
+
+    sub.workload = "c5_finegrained_mod"
+    r = run_moe(sub)
+    st = r["stages_ms"]
+    kept = r["config"]["kept_assignments"]
+    dn_tf = 2.0 * 2048 * 1408 * kept / (st["down"] * 1e-3) / 1e12
+    out["c5_finegrained_mod"] = {
+        "workload": r["config"]["workload"], "tokens_per_s": _r(r["value"], 0), "ms_per_step": _r(r["ms_per_step"]),
+        "gateup": _roof(r["roofline"]),
+        "down": {"bound": "mfma", "achieved": _r(dn_tf, 1), "peak": PEAK_MFMA_BF16_TFLOPS, "unit": "TFLOP/s",
+                 "frac": _r(dn_tf / PEAK_MFMA_BF16_TFLOPS), "traffic": profile_traffic("c5_finegrained_mod", "down")},
+        "stages_ms": st}
+    torch.cuda.empty_cache()
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=None,
-                    help="timed steps (default 50; 200 for the workloads whose step is shorter than 2 ms)")
+                    help="timed steps (default 20; 200 for the workloads whose step is shorter than 2 ms)")
     ap.add_argument("--warmup", type=int, default=None,
-                    help="untimed steps first (default 10; 50 for the short workloads: with fewer the core clock "
+                    help="untimed steps first (default 5; 50 for the short workloads: with fewer the core clock "
                          "has not settled and the first kernels run up to 20 %% slower)")
     ap.add_argument("--workload", default="c4_prefill",
                     choices=["c4_prefill", "c3_decode", "c5_finegrained_mod", "c1_cpu_reference", "c2_norm_rope",
@@ -899,13 +962,16 @@ def main():
     ap.add_argument("--copy-probe", action="store_true",
                     help="also run a 1 GiB device copy (known traffic) so hardware-counter runs can be scaled")
     ap.add_argument("--cpu-sample-tokens", type=int, default=16384)
+    ap.add_argument("--no-secondary", action="store_true",
+                    help="with the default workload: skip the short runs of the other configurations (c2, c3, c5) "
+                         "that are appended as the `secondary` record")
     args = ap.parse_args()
     short = args.workload in ("c3_decode", "c5_finegrained_mod", "c2_norm_rope", "loss_clip", "attention",
                               "attention_train", "attention_decode", "gqa_layer", "gqa_decode")
     if args.steps is None:
-        args.steps = 200 if short else 50
+        args.steps = 200 if short else 20
     if args.warmup is None:
-        args.warmup = 50 if short else 10
+        args.warmup = 50 if short else 5
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this path runs on one GPU (experts stay resident, no collectives); use --gpus 1",
               file=sys.stderr)
@@ -948,6 +1014,12 @@ def main():
         result = run_train(args)
     else:
         result = run_moe(args)
+        if args.workload == "c4_prefill" and not args.no_secondary:
+            torch.cuda.empty_cache()
+            log("secondary records (other configurations, short loops in this process):")
+            result["secondary"] = secondary_records(args)
+            for name, rec in result["secondary"].items():
+                log(f"  secondary {name}: {json.dumps(rec)}")
     print(json.dumps(result), flush=True)
 
 

@@ -521,6 +521,49 @@ def test_transformer_block_dense_forward_backward(gpu):
     assert torch.equal(out2, out) and torch.equal(xg2.grad, xg.grad)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_transformer_block_dropout_with_and_without_checkpointing(gpu, dtype):
+    """Attention dropout under gradient checkpointing: the recomputed forward must draw the mask of the first
+    forward, or the saved output / log-sum-exp and the recomputed probabilities disagree and every gradient is
+    silently wrong.  Same torch.manual_seed, once without and once with checkpointing: outputs and all
+    gradients bit for bit; a different seed gives a different mask."""
+    import adaptivetrainingsystem_amd as A
+    from adaptivetrainingsystem_amd.workloads import LayerConfig
+    hidden, nh, nkv, B, L = 256, 4, 2, 2, 96
+    torch.manual_seed(21)
+    cfg = LayerConfig(hidden, 512, 1, 1, num_heads=nh, num_kv_heads=nkv, seq_length=512, use_moe=False, dropout=0.25)
+    blk = A.TransformerBlock(cfg)
+    with torch.no_grad():
+        for n, p in blk.named_parameters():
+            if "norm" not in n:
+                p.mul_(12.0)
+    blk = blk.to(dtype).to(gpu).train()
+    assert blk.self_attn.dropout_p == 0.25
+    x = torch.randn(B, L, hidden, generator=gen(171)).to(dtype).to(gpu)
+    dy = torch.randn(B, L, hidden, generator=gen(172)).to(dtype).to(gpu)
+
+    def run(checkpointing, seed):
+        blk.zero_grad()
+        blk.gradient_checkpointing = checkpointing
+        torch.manual_seed(seed)
+        xg = x.clone().requires_grad_()
+        out, _ = blk(xg)
+        out.backward(dy)
+        return out.detach(), xg.grad, {n: p.grad.clone() for n, p in blk.named_parameters()}
+
+    out_a, dx_a, g_a = run(False, 99)
+    out_b, dx_b, g_b = run(True, 99)
+    assert torch.equal(out_a, out_b) and torch.equal(dx_a, dx_b)
+    for n in g_a:
+        assert torch.equal(g_a[n], g_b[n]), n
+    out_c, _, _ = run(True, 100)
+    assert not torch.equal(out_a, out_c)
+    # the same mask whatever was constructed before: another attention module changes nothing
+    A.GroupedQueryAttention(cfg)
+    out_d, dx_d, _ = run(False, 99)
+    assert torch.equal(out_a, out_d) and torch.equal(dx_a, dx_d)
+
+
 def test_transformer_block_moe_composition_and_patterns(gpu):
     """The MoE block equals its own sub-modules composed by hand (the routing itself is checked against the oracle
     on bit-equal logits elsewhere), every parameter gets a finite gradient, and the layer patterns select as the

@@ -1,7 +1,8 @@
 """The benchmark configurations at their full sizes on the GPU.  Each test checks (a) every integer
 artefact bit for bit, (b) EVERY output row of the float pipeline against the oracle's whole capacity
-layer (fed the GPU's logits so that routing is compared on bit-equal inputs; the oracle runs the
-16384-token prefill layer in seconds on the host cores), and (c) size-independent properties:
+layer (fed the GPU's logits so that routing is compared on bit-equal inputs; the logits themselves are
+compared with the oracle's own router product, and the tokens that route differently on those are counted
+and must be near-ties; the oracle runs the 16384-token prefill layer in seconds on the host cores), and (c) size-independent properties:
 dispatch -> combine round trip, conservation of assignments, untouched skip tokens."""
 import numpy as np
 import pytest
@@ -33,6 +34,31 @@ def _check_routing_and_plan(p, w, T):
     assert int(kept.sum()) + dropped == T * w.top_k
     assert abs(p["aux"].item() - O.aux_loss(logits, ri, w.num_experts, 0.01).item()) <= 1e-6
     return ri, rw, tm, kept, dropped
+
+
+def _check_logits_against_own_router(p, w, x_flat, T):
+    """The GPU's logits against the oracle's OWN router product on the same inputs (MS/core/model.py:1124,1169),
+    so that a router kernel computing wrong but self-consistent logits cannot pass; then the number of tokens
+    the oracle routes differently on its own logits.  Such a token must be a near-tie: the gap between its
+    k-th and (k+1)-th own logit is within the float32 bar of the logits, anything else is a routing error."""
+    own = O.router_logits(x_flat.cpu(), w.gate.cpu())
+    if w.logit_bias is not None:
+        own = own + w.logit_bias.cpu()
+    got = p["logits"].cpu()
+    assert got.shape == own.shape == (T, w.num_experts)
+    err = rel_err(got, own)
+    own_idx = O.route_softmax_topk_renorm(own, w.top_k, 1.0)[0]
+    differs = (own_idx != p["indices"].cpu().long()).any(-1)
+    mism = int(differs.sum())
+    srt = torch.sort(own, dim=-1, descending=True)[0][:, : w.top_k + 1]
+    gap = (srt[:, :-1] - srt[:, 1:]).amin(-1)
+    bar = 2e-5 * own.abs().max().item()     # a flip needs a gap within twice the logits' 1e-5 bar
+    worst = gap[differs].max().item() if mism else 0.0
+    print(f"{w.name}: logits vs the oracle's own router rel err {err:.2e}; tokens routed differently on the "
+          f"oracle's own logits: {mism} of {T} (largest logit gap among them {worst:.2e}, bar {bar:.2e})", flush=True)
+    assert err <= 1e-5
+    assert mism <= max(1, T // 500) and worst <= bar
+    return mism
 
 
 def _check_sampled_outputs(out, x_flat, w, ri, rw, tm, kept, tokens_to_check, k):
@@ -78,6 +104,7 @@ def test_decode_config3_full(gpu):
     out, aux = layer(w.x)
     p = layer.last_plan
     ri, rw, tm, kept, dropped = _check_routing_and_plan(p, w, 64)
+    _check_logits_against_own_router(p, w, w.x.reshape(-1, 4096), 64)
     assert p["capacity"] == 20
     err = _check_sampled_outputs(out, w.x.reshape(-1, 4096), w, ri, rw, tm, kept, list(range(64)), 2)
     print("config 3 full layer rel err", err, "dropped", dropped, flush=True)
@@ -96,6 +123,7 @@ def test_prefill_config4_full(gpu):
     out, aux = layer(w.x)
     p = layer.last_plan
     ri, rw, tm, kept, dropped = _check_routing_and_plan(p, w, 16384)
+    _check_logits_against_own_router(p, w, w.x.reshape(-1, 4096), 16384)
     assert p["capacity"] == 5120 and dropped > 0 and kept.max() == 5120
     res = _oracle_layer(w, w.x.cpu(), p)
     ref = res["out"].reshape(-1, 4096)
@@ -135,6 +163,7 @@ def test_finegrained_mod_config5_full(gpu):
     ri, rw, tm, kept, dropped = _check_routing_and_plan(p, w, 4096)
     assert p["capacity"] == 576
     gathered = w.x.reshape(-1, 2048)[flat.to(gpu)]
+    _check_logits_against_own_router(p, w, gathered, 4096)
     res = _oracle_layer(w, gathered.cpu(), p)
     moe_ref = res["out"].reshape(-1, 2048)
     delta = (out.reshape(-1, 2048)[flat.to(gpu)].float() - gathered.float()).cpu()

@@ -166,7 +166,12 @@ def test_rope_strided_inputs_and_fused_module(A, ops, gpu):
 
 # ------------------------------------------------------------------ router GEMM
 @pytest.mark.parametrize("T,H,E", [(512, 512, 8), (100, 1024, 64), (33, 40, 6), (1, 4096, 8), (257, 2048, 128),
-                                   (64, 200, 8)])
+                                   (64, 200, 8),
+                                   # the instances chosen at the benchmark shapes: the flat kernel (>= 2048 tokens,
+                                   # <= 16 experts), whose 8 waves each walk a full 4-step K slice at H 4096, and
+                                   # the 4-wave kernel for 33-64 experts
+                                   (2048, 4096, 8), (16384, 4096, 8), (4096, 2048, 16), (4096, 2048, 64),
+                                   (32768, 2048, 64), (2049, 4096, 5), (3000, 1000, 16)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_router_logits(ops, gpu, T, H, E, dtype):
     print("case router", T, H, E, dtype, flush=True)
@@ -685,6 +690,18 @@ def test_performance_monitor_api(A, gpu):
     m.record_cuda(2.0, 100)
     m.record_pytorch(6.0, 100)
     assert m.get_stats()["estimated_speedup"] == 3.0 and m.get_stats()["tokens_per_sec_pytorch"] == 100 / 0.006
+    # a loop that monitors and never asks for statistics holds a bounded number of events
+    P.reset_performance_monitor()
+    P.enable_performance_monitor(True)
+    try:
+        small = torch.randn(16, 8, generator=gen(43)).to(gpu)
+        for _ in range(1500):
+            A.MoECUDAOps.topk_gating(small, 2)
+    finally:
+        P.enable_performance_monitor(False)
+    assert len(P._GLOBAL_MONITOR._pending) <= P.MoEPerformanceMonitor._PENDING_BOUND + 1
+    st = P.get_performance_summary()
+    assert st["cuda_calls"] == 1500 and st["cuda_time_ms"] > 0 and not P._GLOBAL_MONITOR._pending
     P.reset_performance_monitor()
 
 
