@@ -883,7 +883,7 @@ def run_norm_rope(args):
 
 
 def _r(v, n=4):
-    return None if v is None else round(float(v), n)
+    return round(float(v), n) if isinstance(v, (int, float)) else v
 
 
 def _roof(r):
@@ -1017,7 +1017,10 @@ def main():
         if args.workload == "c4_prefill" and not args.no_secondary:
             torch.cuda.empty_cache()
             log("secondary records (other configurations, short loops in this process):")
-            result["secondary"] = secondary_records(args)
+            try:
+                result["secondary"] = secondary_records(args)
+            except Exception as exc:       # the headline line is printed whatever happens to the short runs
+                result["secondary"] = {"error": f"{type(exc).__name__}: {exc}"}
             for name, rec in result["secondary"].items():
                 log(f"  secondary {name}: {json.dumps(rec)}")
     print(json.dumps(result), flush=True)
