@@ -116,6 +116,8 @@ _SIGNATURES = {
     "ats_scatter_add_rows": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int, c_int, c_void_p]),
     "ats_kth_value_workspace": (ctypes.c_size_t, [c_int64]),
     "ats_kth_value_mask": (c_int, [c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "ats_topk_mask_ste": (c_int, [c_void_p, c_int64, c_int64, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
+    "ats_mod_route_bwd": (c_int, [c_void_p, c_void_p, c_void_p, c_float, c_void_p, c_void_p, c_int64, c_void_p]),
     "ats_swiglu_mul": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int, c_void_p]),
     # the reference's launcher names (void return, float32 only)
     "rms_norm_launcher": (None, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_float, c_void_p]),
@@ -123,6 +125,8 @@ _SIGNATURES = {
     "rope_apply_launcher": (None, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int,
                                    c_void_p]),
     "swiglu_launcher": (None, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_void_p]),
+    "swiglu_fused_launcher": (None, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int,
+                                     ctypes.c_bool, c_void_p]),
     "fused_cross_entropy_accuracy_launcher": (None, [c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_int, c_int,
                                                      c_void_p]),
     "fused_grad_clip_launcher": (c_float, [c_void_p, c_void_p, c_int, c_float, c_void_p]),

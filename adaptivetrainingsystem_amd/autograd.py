@@ -370,5 +370,39 @@ class MoEFunction(Function):
         return (dx_out if need_x else None, dwg.to(gate_dtype) if need_wg else None, None, *grads_w)
 
 
+class MoDRouteFunction(Function):
+    """Training branch of the reference's MoDRouter (MS/core/model.py:923-952): probabilities
+    sigmoid((x . w + b) / temperature), a mask with exactly `capacity` ones at the largest of them over all
+    tokens of the batch, and the straight-through weights (mask - p) + p, whose gradient goes to p unchanged.
+    Returns (weights [T], probs [T], mask [T]), float32; the mask carries no gradient."""
+
+    @staticmethod
+    def forward(ctx, x, weight, bias, temperature, capacity):
+        x2 = x.reshape(-1, x.shape[-1])
+        w = weight if weight.dtype == x2.dtype else weight.to(x2.dtype)
+        _, probs = ops.row_dot(x2, w, None if bias is None else bias.detach(), temperature, want_prob=True)
+        mask, ste = ops.topk_mask_ste(probs, capacity)
+        ctx.save_for_backward(x2, w, probs)
+        ctx.temperature = temperature
+        ctx.x_shape = x.shape
+        ctx.weight_dtype = weight.dtype
+        ctx.has_bias = bias is not None
+        ctx.mark_non_differentiable(mask)
+        return ste, probs, mask
+
+    @staticmethod
+    def backward(ctx, d_weights, d_probs, _d_mask):
+        x2, w, probs = ctx.saved_tensors
+        need_x, need_w = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
+        need_b = ctx.has_bias and ctx.needs_input_grad[2]
+        gw = None if d_weights is None else d_weights.float()
+        gp = None if d_probs is None else d_probs.float()
+        gl, db = ops.mod_route_bwd(probs, gw, gp, ctx.temperature, need_bias=need_b)
+        dx, dw = ops.router_bwd(gl.view(-1, 1), x2, w.reshape(1, -1), need_dx=need_x, need_dw=need_w)
+        return (dx.view(ctx.x_shape) if need_x else None,
+                dw.to(ctx.weight_dtype) if need_w else None,
+                db if need_b else None, None, None)
+
+
 def moe_variant(routing: str) -> int:
     return {"softmax_topk": ROUTE_SOFTMAX_TOPK, "topk_softmax": ROUTE_TOPK_SOFTMAX}[routing]

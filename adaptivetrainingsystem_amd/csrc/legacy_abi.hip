@@ -1,7 +1,7 @@
 // The reference's own launcher names, exported with their exact float32 signatures so that the ctypes
 // loader of Src/Main_Scripts/core/cuda_opt_wrapper.py:50-79 binds this library unchanged:
-//   rms_norm_launcher, rope_precompute_launcher, rope_apply_launcher, swiglu_launcher
-//   (Src/Main_Scripts/core/transformer_ops.cu:331-409; call sites cuda_opt_wrapper.py:98-108, 156-169,
+//   rms_norm_launcher, rope_precompute_launcher, rope_apply_launcher, swiglu_launcher, swiglu_fused_launcher
+//   (Src/Main_Scripts/core/transformer_ops.cu:331-434; call sites cuda_opt_wrapper.py:98-108, 156-169,
 //   219-228, 337-344).
 // Each is a thin alias of the ats_* entry point beside it.  They return void like the originals; where the
 // originals print and exit() on a failed launch (transformer_ops.cu:321-329) these never terminate the
@@ -59,6 +59,74 @@ extern "C" void swiglu_launcher(const float* gate, const float* up, float* outpu
     }
     ats::g_legacy_status =
         ats_swiglu_mul(gate, up, output, (int64_t)total_tokens * intermediate_size, ATS_F32, stream);
+}
+
+namespace ats {
+// Tables of the two products below, written on the device so that the launcher neither copies from host
+// memory nor waits: one group of total_tokens rows, multiplied by the gate weight and by the up weight.
+__global__ void legacy_swiglu_tables_kernel(const float* gate_weight, const float* up_weight, int total_tokens,
+                                            const void** b_ptrs, int32_t* row_start, int32_t* row_count) {
+    if (threadIdx.x == 0 && blockIdx.x == 0) {
+        b_ptrs[0] = gate_weight;
+        b_ptrs[1] = up_weight;
+        row_start[0] = 0;
+        row_count[0] = total_tokens;
+    }
+}
+}  // namespace ats
+
+// output[t, j] = (x[t] . gate_weight[j]) * silu(x[t] . up_weight[j]) over [total_tokens, intermediate_size],
+// float32, weights [intermediate_size, hidden_size] (Src/Main_Scripts/core/transformer_ops.cu:268-313, 411-434;
+// no call site in the reference's Python).  As in the original the biases are accepted and not applied
+// (transformer_ops.cu:427-431 passes neither to its kernel).  Two float32 products on the matrix cores into
+// a stream-ordered scratch buffer, then the elementwise activation; hidden_size and intermediate_size must be
+// multiples of 4 (16-byte rows, which the original's float4 loads assume as well).
+extern "C" void swiglu_fused_launcher(const float* input, const float* gate_weight, const float* up_weight,
+                                      const float* gate_bias, const float* up_bias, float* output, int total_tokens,
+                                      int hidden_size, int intermediate_size, bool use_bias, ats_stream_t stream) {
+    using namespace ats;
+    (void)gate_bias;
+    (void)up_bias;
+    (void)use_bias;
+    const char* who = "swiglu_fused_launcher";
+    if (total_tokens < 0 || hidden_size <= 0 || intermediate_size <= 0 ||
+        (total_tokens > 0 && (!input || !gate_weight || !up_weight || !output))) {
+        set_error("%s: total_tokens=%d hidden_size=%d intermediate_size=%d or a null pointer", who, total_tokens,
+                  hidden_size, intermediate_size);
+        g_legacy_status = ATS_ERR_INVALID_ARG;
+        return;
+    }
+    if (total_tokens == 0) {
+        g_legacy_status = ATS_OK;
+        return;
+    }
+    hipStream_t s = as_stream(stream);
+    const size_t n_out = (size_t)total_tokens * (size_t)intermediate_size;
+    const size_t off_tables = 2 * n_out * sizeof(float);
+    const size_t bytes = off_tables + 32;
+    unsigned char* dev = nullptr;
+    hipError_t e = hipMallocAsync(reinterpret_cast<void**>(&dev), bytes, s);
+    if (e != hipSuccess) {
+        set_error("%s: scratch allocation of %zu bytes failed: %s", who, bytes, hipGetErrorString(e));
+        g_legacy_status = ATS_ERR_LAUNCH;
+        return;
+    }
+    float* gu = reinterpret_cast<float*>(dev);
+    const void** b_ptrs = reinterpret_cast<const void**>(dev + off_tables);
+    int32_t* row_start = reinterpret_cast<int32_t*>(dev + off_tables + 16);
+    int32_t* row_count = reinterpret_cast<int32_t*>(dev + off_tables + 24);
+    hipLaunchKernelGGL(legacy_swiglu_tables_kernel, dim3(1), dim3(64), 0, s, gate_weight, up_weight, total_tokens, b_ptrs,
+                       row_start, row_count);
+    int rc = hipGetLastError() == hipSuccess ? ATS_OK : ATS_ERR_LAUNCH;
+    if (rc != ATS_OK) set_error("%s: launch failed", who);
+    for (int half = 0; half < 2 && rc == ATS_OK; ++half)
+        rc = ats_grouped_gemm_nt(input, nullptr, hidden_size, total_tokens, nullptr, 1,
+                                 reinterpret_cast<const void* const*>(b_ptrs + half), hidden_size, intermediate_size,
+                                 gu + half * n_out, intermediate_size, row_start, row_count, nullptr, 1, total_tokens,
+                                 intermediate_size, hidden_size, ATS_F32, ATS_F32, stream);
+    if (rc == ATS_OK) rc = ats_swiglu_mul(gu, gu + n_out, output, (int64_t)n_out, ATS_F32, stream);
+    (void)hipFreeAsync(dev, s);
+    g_legacy_status = rc;
 }
 
 // ---- training-step launchers (Src/Main_Scripts/training/fused_loss.cu:183-214, fused_grad_clip.cu:117-175;

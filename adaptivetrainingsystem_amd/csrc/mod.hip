@@ -257,7 +257,8 @@ __global__ __launch_bounds__(256) void scatter_add_rows_kernel(T* __restrict__ b
 // block, then a threshold mask.  Keys are the usual order-preserving unsigned
 // image of the float bits.
 __device__ __forceinline__ uint32_t order_key(float f) {
-    const uint32_t u = __float_as_uint(f);
+    // -0.0 and +0.0 compare equal as floats, so they share a key
+    const uint32_t u = f == 0.0f ? 0u : __float_as_uint(f);
     return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
 }
 
@@ -404,6 +405,17 @@ __global__ __launch_bounds__(256) void kth_mask_kernel(const float* __restrict__
         mask[i] = order_key(v[i]) >= thr ? 1.0f : 0.0f;
 }
 
+__global__ __launch_bounds__(64) void kth_key_kernel(int64_t n, int64_t kth, const unsigned int* __restrict__ ghist,
+                                                     uint32_t* __restrict__ key_out, long long* __restrict__ count_out) {
+    uint32_t prefix;
+    long long rank;
+    kth_walk(ghist, -1, kth, (int)threadIdx.x, &prefix, &rank);
+    if (threadIdx.x == 0) {
+        key_out[0] = prefix;
+        count_out[0] = (long long)n - kth + rank;
+    }
+}
+
 __global__ __launch_bounds__(256) void kth_zero_kernel(unsigned int* __restrict__ ghist) {
     for (int i = threadIdx.x; i < 4 * 256; i += 256) ghist[i] = 0;
 }
@@ -413,6 +425,109 @@ __global__ __launch_bounds__(256) void threshold_mask_kernel(const float* __rest
     const uint32_t thr = key[0];
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
         mask[i] = order_key(v[i]) >= thr ? 1.0f : 0.0f;
+}
+
+// Training branch of the MoD router (MS/core/model.py:941-965): a 0/1 mask with exactly k ones at the k
+// largest values, and the straight-through weights (mask - p) + p formed in float32 in the reference's order.
+// `thr` is the order key of the k-th largest value and `count_ge` the number of values >= it (both from the
+// radix select).  When count_ge == k every value at the threshold is in; otherwise only the first
+// k - (number above) of them in index order are (the lower index wins among equals, the rule of the routing
+// kernels), which the second kernel settles in one workgroup that walks the values in order.
+__device__ __forceinline__ float ste_weight(float m, float p) { return (m - p) + p; }
+
+__global__ __launch_bounds__(256) void topk_mask_kernel(const float* __restrict__ v, int64_t n, int64_t k,
+                                                        const uint32_t* __restrict__ key,
+                                                        const long long* __restrict__ count_ge,
+                                                        float* __restrict__ mask, float* __restrict__ ste) {
+    const uint32_t thr = key[0];
+    const bool all_ties_in = count_ge[0] == (long long)k;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
+        const float p = v[i];
+        const uint32_t kk = order_key(p);
+        const float m = (kk > thr || (kk == thr && all_ties_in)) ? 1.0f : 0.0f;
+        mask[i] = m;
+        if (ste) ste[i] = ste_weight(m, p);
+    }
+}
+
+__global__ __launch_bounds__(1024) void topk_ties_kernel(const float* __restrict__ v, int64_t n, int64_t k,
+                                                         const uint32_t* __restrict__ key,
+                                                         const long long* __restrict__ count_ge,
+                                                         float* __restrict__ mask, float* __restrict__ ste) {
+    if (count_ge[0] == (long long)k) return;          // uniform: nothing to settle
+    __shared__ int wave_cnt[16];
+    __shared__ long long s_total;
+    const uint32_t thr = key[0];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    // values equal to the threshold
+    long long mine = 0;
+    for (int64_t i = threadIdx.x; i < n; i += blockDim.x) mine += order_key(v[i]) == thr ? 1 : 0;
+    int w = wave_inclusive_scan((int)mine);
+    if (lane == 63) wave_cnt[wave] = w;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        long long t = 0;
+        for (int q = 0; q < 16; ++q) t += wave_cnt[q];
+        s_total = t;
+    }
+    __syncthreads();
+    // ones still to hand out: k minus the values above the threshold
+    long long need = (long long)k - (count_ge[0] - s_total);
+    long long base = 0;
+    for (int64_t i0 = 0; i0 < n && base < need; i0 += blockDim.x) {
+        const int64_t i = i0 + threadIdx.x;
+        const bool eq = i < n && order_key(v[i]) == thr;
+        const unsigned long long b = __ballot(eq);
+        __syncthreads();                              // wave_cnt of the previous chunk has been read
+        if (lane == 0) wave_cnt[wave] = __popcll(b);
+        __syncthreads();
+        int before = 0, chunk = 0;
+        for (int q = 0; q < 16; ++q) {
+            const int c = wave_cnt[q];
+            before += q < wave ? c : 0;
+            chunk += c;
+        }
+        if (eq) {
+            const long long rank = base + before + __popcll(b & ((1ull << lane) - 1ull));
+            if (rank < need) {
+                mask[i] = 1.0f;
+                if (ste) ste[i] = ste_weight(1.0f, v[i]);
+            }
+        }
+        base += chunk;
+    }
+}
+
+__global__ __launch_bounds__(256) void fill_mask_kernel(const float* __restrict__ v, int64_t n, float m,
+                                                        float* __restrict__ mask, float* __restrict__ ste) {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) {
+        mask[i] = m;
+        if (ste) ste[i] = ste_weight(m, v[i]);
+    }
+}
+
+// Gradient of the router's logits: gl = (dL/dweights + dL/dprobs) * p * (1 - p) / temperature (the
+// straight-through weights pass their gradient to the probabilities unchanged; sigmoid' = p (1 - p)), and the
+// gradient of the bias, their sum, added in a fixed order by one workgroup.
+__global__ __launch_bounds__(1024) void mod_route_bwd_kernel(const float* __restrict__ gw, const float* __restrict__ gp,
+                                                             const float* __restrict__ prob, float inv_temperature,
+                                                             float* __restrict__ gl, float* __restrict__ dbias,
+                                                             int64_t n) {
+    __shared__ float part[1024];
+    float acc = 0.f;
+    for (int64_t i = threadIdx.x; i < n; i += blockDim.x) {
+        const float p = prob[i];
+        const float g = ((gw ? gw[i] : 0.f) + (gp ? gp[i] : 0.f)) * (p * (1.0f - p)) * inv_temperature;
+        gl[i] = g;
+        acc += g;
+    }
+    part[threadIdx.x] = acc;
+    __syncthreads();
+    for (int s2 = 512; s2 > 0; s2 >>= 1) {
+        if ((int)threadIdx.x < s2) part[threadIdx.x] += part[threadIdx.x + s2];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0 && dbias) dbias[0] = part[0];
 }
 
 // Dense-FFN activation of the fused wrapper: out = gate * silu(up).
@@ -569,6 +684,59 @@ extern "C" int ats_kth_value_mask(const float* v, int64_t n, int64_t kth, float*
     ATS_CHECK_LAUNCH("ats_kth_value_mask(select)");
     hipLaunchKernelGGL(threshold_mask_kernel, dim3((unsigned)blocks), dim3(256), 0, s, v, n, key, mask);
     ATS_CHECK_LAUNCH("ats_kth_value_mask(mask)");
+    return ATS_OK;
+}
+
+extern "C" int ats_topk_mask_ste(const float* v, int64_t n, int64_t k, float* mask, float* ste, void* workspace,
+                                 size_t workspace_bytes, ats_stream_t stream) {
+    using namespace ats;
+    ATS_REQUIRE(n >= 0 && k >= 0, ATS_ERR_INVALID_ARG, "ats_topk_mask_ste: n=%lld k=%lld", (long long)n, (long long)k);
+    if (n == 0) return ATS_OK;
+    ATS_REQUIRE(n < (int64_t)INT_MAX, ATS_ERR_UNSUPPORTED, "ats_topk_mask_ste: n=%lld (below 2^31)", (long long)n);
+    ATS_REQUIRE(v && mask, ATS_ERR_INVALID_ARG, "ats_topk_mask_ste: null pointer");
+    hipStream_t s = as_stream(stream);
+    int64_t blocks = (n + 255) / 256;
+    if (blocks > 4096) blocks = 4096;
+    if (k == 0 || k >= n) {
+        hipLaunchKernelGGL(fill_mask_kernel, dim3((unsigned)blocks), dim3(256), 0, s, v, n, k == 0 ? 0.0f : 1.0f, mask, ste);
+        ATS_CHECK_LAUNCH("ats_topk_mask_ste(fill)");
+        return ATS_OK;
+    }
+    ATS_REQUIRE(workspace && workspace_bytes >= ats_kth_value_workspace(n), ATS_ERR_WORKSPACE,
+                "ats_topk_mask_ste: workspace of ats_kth_value_workspace(n) = %zu bytes needed, got %zu",
+                ats_kth_value_workspace(n), workspace_bytes);
+    // the k-th largest is the (n - k + 1)-th smallest; the select leaves its key and the count of values >= it
+    const int64_t kth = n - k + 1;
+    uint32_t* key = static_cast<uint32_t*>(workspace);
+    long long* count = reinterpret_cast<long long*>(static_cast<char*>(workspace) + 8);
+    if (n >= kKthMultiBlockMin) {
+        unsigned int* ghist = reinterpret_cast<unsigned int*>(static_cast<char*>(workspace) + 16);
+        int64_t hb = (n + 2047) / 2048;
+        if (hb > 1024) hb = 1024;
+        hipLaunchKernelGGL(kth_zero_kernel, dim3(1), dim3(256), 0, s, ghist);
+        for (int pass = 3; pass >= 0; --pass)
+            hipLaunchKernelGGL(kth_digit_hist_kernel, dim3((unsigned)hb), dim3(256), 0, s, v, n, kth, pass, ghist);
+        hipLaunchKernelGGL(kth_key_kernel, dim3(1), dim3(64), 0, s, n, kth, ghist, key, count);
+    } else {
+        hipLaunchKernelGGL(kth_value_kernel, dim3(1), dim3(1024), 0, s, v, n, kth, key, count);
+    }
+    ATS_CHECK_LAUNCH("ats_topk_mask_ste(select)");
+    hipLaunchKernelGGL(topk_mask_kernel, dim3((unsigned)blocks), dim3(256), 0, s, v, n, k, key, count, mask, ste);
+    hipLaunchKernelGGL(topk_ties_kernel, dim3(1), dim3(1024), 0, s, v, n, k, key, count, mask, ste);
+    ATS_CHECK_LAUNCH("ats_topk_mask_ste");
+    return ATS_OK;
+}
+
+extern "C" int ats_mod_route_bwd(const float* grad_weights, const float* grad_probs, const float* prob,
+                                 float temperature, float* grad_logits, float* grad_bias, int64_t n,
+                                 ats_stream_t stream) {
+    using namespace ats;
+    ATS_REQUIRE(n >= 0 && temperature > 0.f, ATS_ERR_INVALID_ARG, "ats_mod_route_bwd: n=%lld temperature=%g",
+                (long long)n, temperature);
+    ATS_REQUIRE(n == 0 || (prob && grad_logits), ATS_ERR_INVALID_ARG, "ats_mod_route_bwd: null pointer");
+    hipLaunchKernelGGL(mod_route_bwd_kernel, dim3(1), dim3(1024), 0, as_stream(stream), grad_weights, grad_probs, prob,
+                       1.0f / temperature, grad_logits, grad_bias, n);
+    ATS_CHECK_LAUNCH("ats_mod_route_bwd");
     return ATS_OK;
 }
 

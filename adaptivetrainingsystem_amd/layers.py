@@ -644,9 +644,14 @@ class MoECUDAOps:
 
 # ============================================================================ Mixture of Depths
 class MoDRouter(nn.Module):
-    """Token-level compute/skip router: sigmoid(Linear(H,1)(x) / temperature), inference branch
-    (k-th value threshold over all tokens of the batch).  forward -> (routing_weights [B,L,1],
-    routing_probs [B,L,1], None)."""
+    """Token-level compute/skip router of the reference (MS/core/model.py:884-1011):
+    sigmoid(Linear(H,1)(x) / temperature).  In evaluation mode the k-th value of all probabilities of the
+    batch is the threshold (model.py:984-995): forward -> (routing_weights [B,L,1], routing_probs [B,L,1],
+    None).  In training mode (model.py:941-965) exactly int(B*L*capacity_factor) tokens, those with the
+    largest probabilities, get a 1 in the mask, the routing weights are the straight-through form
+    mask - p.detach() + p (value of the mask, gradient of p), and the auxiliary loss is the squared
+    distance of the mask's mean from capacity_factor; the reference's branch continues into placeholder code
+    that cannot run (model.py:967-982: calls with a literal `...`), which is where this one stops."""
 
     def __init__(self, hidden_size: int, capacity_factor: float = 0.5, routing_temperature: float = 1.0):
         super().__init__()
@@ -660,10 +665,21 @@ class MoDRouter(nn.Module):
         nn.init.zeros_(self.router.bias)
 
     def forward(self, x: torch.Tensor):
-        if self.training:
-            raise NotImplementedError("MoDRouter: the training branch needs autograd, which this forward-only "
-                                      "path does not provide")
         B, L, H = x.shape
+        if self.training:
+            total = B * L
+            capacity = min(int(total * self.capacity_factor), total)
+            weights, probs, mask = ag.MoDRouteFunction.apply(x, self.router.weight, self.router.bias,
+                                                             self.routing_temperature, capacity)
+            # exactly `capacity` ones by construction, so the statistics need no device round trip
+            self._routing_stats["total_tokens"] += total
+            self._routing_stats["computed_tokens"] += float(capacity)
+            self._routing_stats["skipped_tokens"] = (self._routing_stats["total_tokens"]
+                                                     - self._routing_stats["computed_tokens"])
+            # mse(mask.mean(), capacity_factor): the mask is a constant of the graph, and so is this loss
+            ratio = capacity / total if total else 0.0
+            aux = torch.full((), (ratio - self.capacity_factor) ** 2, dtype=torch.float32, device=x.device)
+            return weights.view(B, L, 1), probs.view(B, L, 1), aux
         _, probs = ops.row_dot(x, _as_dtype(self.router.weight, x.dtype), self.router.bias.detach(),
                                self.routing_temperature, want_prob=True)
         total = B * L

@@ -566,6 +566,43 @@ def kth_value_mask(values: torch.Tensor, kth: int, return_count: bool = False):
     return (mask, ws[1:2]) if return_count else mask
 
 
+def topk_mask_ste(values: torch.Tensor, k: int, want_ste: bool = True):
+    """float32 mask with exactly min(k, n) ones at the k largest of `values` (lower index first among equals)
+    and, with `want_ste`, the straight-through weights (mask - values) + values; both of `values`' shape."""
+    _need_gpu(values)
+    if values.dtype != torch.float32:
+        raise AtsError("topk_mask_ste: values must be float32")
+    v = values.contiguous()
+    mask = torch.empty_like(v)
+    ste = torch.empty_like(v) if want_ste else None
+    lib = _lib.load()
+    ws_bytes = int(lib.ats_kth_value_workspace(v.numel()))
+    ws = torch.empty(max(ws_bytes // 8, 2), dtype=torch.int64, device=v.device)
+    check(lib.ats_topk_mask_ste(v.data_ptr(), v.numel(), int(k), mask.data_ptr(), _ptr(ste), ws.data_ptr(), ws_bytes,
+                                _stream()), "ats_topk_mask_ste")
+    return (mask, ste) if want_ste else mask
+
+
+def mod_route_bwd(prob: torch.Tensor, grad_weights: Optional[torch.Tensor], grad_probs: Optional[torch.Tensor],
+                  temperature: float = 1.0, need_bias: bool = True):
+    """Gradient of the MoD router's logits, float32 [n], and of its bias, float32 [1] (or None)."""
+    _need_gpu(prob, grad_weights, grad_probs)
+    p = prob.reshape(-1).contiguous()
+    n = p.numel()
+    for g in (grad_weights, grad_probs):
+        if g is not None and (g.dtype != torch.float32 or g.numel() != n):
+            raise AtsError("mod_route_bwd: gradients must be float32 with one value per token")
+    if p.dtype != torch.float32:
+        raise AtsError("mod_route_bwd: probabilities must be float32")
+    gw = None if grad_weights is None else grad_weights.reshape(-1).contiguous()
+    gp = None if grad_probs is None else grad_probs.reshape(-1).contiguous()
+    gl = torch.empty(n, dtype=torch.float32, device=p.device)
+    db = torch.empty(1, dtype=torch.float32, device=p.device) if need_bias else None
+    check(_lib.load().ats_mod_route_bwd(_ptr(gw), _ptr(gp), p.data_ptr(), float(temperature), gl.data_ptr(), _ptr(db), n,
+                                        _stream()), "ats_mod_route_bwd")
+    return gl, db
+
+
 def swiglu_mul(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
     """gate * silu(up) (dense-FFN convention of the fused wrapper)."""
     _need_gpu(gate, up)

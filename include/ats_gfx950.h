@@ -21,6 +21,7 @@
 #ifndef ATS_GFX950_H
 #define ATS_GFX950_H
 
+#include <stdbool.h>
 #include <stddef.h>
 #include <stdint.h>
 
@@ -272,6 +273,20 @@ size_t ats_kth_value_workspace(int64_t n);
 int ats_kth_value_mask(const float* v, int64_t n, int64_t kth, float* mask, void* workspace,
                        size_t workspace_bytes, ats_stream_t stream);
 
+/* Training branch of MoDRouter.forward (model.py:941-952): mask[i] = 1.0f at exactly min(k, n) positions, the
+ * k largest of v (among equal values the lower index first; torch.topk leaves that order to the library),
+ * else 0.0f; ste (may be null) receives the straight-through weights (mask - v) + v, float32 in the
+ * reference's order of operations.  workspace: ats_kth_value_workspace(n) bytes, 8-byte aligned.  n < 2^31. */
+int ats_topk_mask_ste(const float* v, int64_t n, int64_t k, float* mask, float* ste, void* workspace,
+                      size_t workspace_bytes, ats_stream_t stream);
+/* Backward of that branch, which the reference leaves to autograd over model.py:923-952:
+ * grad_logits[i] = (grad_weights[i] + grad_probs[i]) * p (1 - p) / temperature with p = prob[i] (either
+ * gradient may be null), grad_bias[0] (may be null) = their sum, added in a fixed order.  The gradients of
+ * the router's weight and of x follow from grad_logits through ats_router_bwd_dw / ats_router_bwd_dx
+ * with one "expert". */
+int ats_mod_route_bwd(const float* grad_weights, const float* grad_probs, const float* prob,
+                      float temperature, float* grad_logits, float* grad_bias, int64_t n, ats_stream_t stream);
+
 /* out = gate * silu(up), elementwise over n values: replaces swiglu_launcher
  * (transformer_ops.cu:394-409), the activation of the dense FusedSwiGLU wrapper
  * (cuda_opt_wrapper.py:476-478; note the convention differs from the experts'). */
@@ -473,8 +488,10 @@ int ats_grad_norm_clip(void* const* grad_ptrs, const int64_t* sizes, const int32
  * that signature has it; the caller guarantees position_offset + seq_len <= max_seq_len) and
  * ats_swiglu_mul.  They return void like the originals but never exit(): the status of the calling
  * thread's last legacy call is ats_legacy_last_status(), its text ats_last_error_string().
- * swiglu_fused_launcher (transformer_ops.cu:411-434) has no call site in the reference's Python
- * and is not exported. */
+ * swiglu_fused_launcher (transformer_ops.cu:411-434; no call site in the reference's Python) is the
+ * product x . gate_weight^T times silu(x . up_weight^T) with float32 weights [intermediate, hidden]; like
+ * the original it accepts the biases and does not apply them.  It owns a stream-ordered scratch
+ * allocation of 2 * total_tokens * intermediate_size floats. */
 void rms_norm_launcher(const float* input, const float* weight, float* output, int batch_seq,
                        int hidden_size, float eps, ats_stream_t stream);
 void rope_precompute_launcher(float* cos_cache, float* sin_cache, int max_seq_len, int head_dim,
@@ -484,6 +501,9 @@ void rope_apply_launcher(float* q, float* k, const float* cos, const float* sin,
                          ats_stream_t stream);
 void swiglu_launcher(const float* gate, const float* up, float* output, int total_tokens,
                      int intermediate_size, ats_stream_t stream);
+void swiglu_fused_launcher(const float* input, const float* gate_weight, const float* up_weight,
+                           const float* gate_bias, const float* up_bias, float* output, int total_tokens,
+                           int hidden_size, int intermediate_size, bool use_bias, ats_stream_t stream);
 /* The training-step launchers the reference's second loader binds (Src/Main_Scripts/training/cuda_kernels.py:
  * 60-78, call sites 154-164 and 340-346), with the signatures of training/fused_loss.cu:183-193 and
  * training/fused_grad_clip.cu:117-123.  Aliases of ats_cross_entropy_fwd and ats_grad_norm_clip that own

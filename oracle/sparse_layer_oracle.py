@@ -46,6 +46,9 @@ PINNING = {
     "mod_router_probs": "float64 closed form 1/(1+exp(-(x.w+b)/T)) with bias != 0 and temperature != 1; "
                         "w = 0 gives sigmoid(b/T); p(x)+p(-x) = 1 without bias",
     "mod_router_eval_mask": "sorted-threshold brute force",
+    "mod_router_train": "mask = brute-force ranking (exactly int(N*cf) ones, at the largest probabilities); the weights' value "
+                        "is the mask to one ulp; d weights / d logit = p(1-p)/T against the float64 closed form, with a "
+                        "non-constant cotangent; aux = (k/N - cf)^2 closed form and no gradient",
     "mod_select_per_sequence": "argsort brute force (composition defined by the benchmark config, not a reference function)",
     "mod_moe_block": "scores against a float64 matmul + bias; selection against a brute-force sort; skipped tokens "
                      "bit-identical to the input, kept tokens = input + capacity layer output",
@@ -402,6 +405,26 @@ def mod_router_eval_mask(probs: torch.Tensor, capacity_factor: float):
     cap = int(n * capacity_factor)
     thr = probs.flatten().kthvalue(max(1, n - cap))[0]
     return (probs >= thr).float()
+
+
+def mod_router_train(x, router_weight, router_bias, temperature: float = 1.0, capacity_factor: float = 0.5):
+    """MS/core/model.py:923-965 (MoDRouter.forward, training branch, up to where its placeholder code begins).
+
+    -> (routing_weights [B,L,1] = mask - p.detach() + p, routing_probs [B,L,1], mask [B,L,1], aux_loss).
+    The mask has exactly min(int(B*L*cf), B*L) ones, at the largest probabilities over the whole batch
+    (torch.topk; among equal probabilities the library picks).  aux = mse(mask.mean(), cf)."""
+    B, L, _ = x.shape
+    probs = mod_router_probs(x, router_weight, router_bias, temperature)     # [B, L, 1]
+    total = B * L
+    cap = int(total * capacity_factor)
+    flat = probs.view(-1)
+    _, top = torch.topk(flat, k=min(cap, total))
+    mask = torch.zeros_like(flat)
+    mask[top] = 1.0
+    mask = mask.view(B, L, 1).detach()
+    weights = mask - probs.detach() + probs
+    aux = F.mse_loss(mask.mean(), torch.tensor(capacity_factor))
+    return weights, probs, mask, aux
 
 
 def mod_select_per_sequence(scores: torch.Tensor, keep: int) -> torch.Tensor:

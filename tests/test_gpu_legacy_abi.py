@@ -83,6 +83,31 @@ def test_swiglu_launcher(raw, gpu):
     assert (out.cpu() - ref).abs().max().item() <= 1e-5 * ref.abs().max().item()
 
 
+@pytest.mark.parametrize("T,H,I", [(19, 512, 1408), (300, 264, 100), (1, 64, 4)])
+def test_swiglu_fused_launcher(raw, gpu, T, H, I):
+    """transformer_ops.cu:268-313, 411-434: (x . gate_w^T) * silu(x . up_w^T) in float32; the biases are accepted
+    and, as in the original, not applied."""
+    lib, typed = raw
+    g = gen(7)
+    x = torch.randn(T, H, generator=g)
+    wg = torch.randn(I, H, generator=g) * 0.1
+    wu = torch.randn(I, H, generator=g) * 0.1
+    bias = torch.randn(I, generator=g)
+    xg, wgg, wug, bg = x.to(gpu), wg.to(gpu), wu.to(gpu), bias.to(gpu)
+    out = torch.full((T, I), 9.0, device=gpu)
+    p = lambda t: ctypes.c_void_p(t.data_ptr())
+    lib.swiglu_fused_launcher(p(xg), p(wgg), p(wug), p(bg), p(bg), p(out), ctypes.c_int(T), ctypes.c_int(H),
+                              ctypes.c_int(I), ctypes.c_bool(True), _stream())
+    torch.cuda.synchronize()
+    assert typed.ats_legacy_last_status() == 0
+    ref = (x.double() @ wg.double().T) * torch.nn.functional.silu(x.double() @ wu.double().T)
+    assert (out.cpu().double() - ref).abs().max().item() <= 1e-5 * ref.abs().max().item()
+    # sizes that do not describe 16-byte rows are refused with a status, not a crash
+    lib.swiglu_fused_launcher(p(xg), p(wgg), p(wug), None, None, p(out), ctypes.c_int(1), ctypes.c_int(H - 1),
+                              ctypes.c_int(I), ctypes.c_bool(False), _stream())
+    assert typed.ats_legacy_last_status() != 0
+
+
 def test_fused_cross_entropy_accuracy_launcher(raw, gpu):
     """training/fused_loss.cu:183-193 as training/cuda_kernels.py:154-175 calls it: the three device scalars hold
     the sum of token losses, the number of correct predictions and the number of valid tokens."""

@@ -601,6 +601,121 @@ def test_mod_router_eval_and_selection(A, ops, gpu):
     assert torch.equal(sel.long(), ref)
 
 
+def _lowest_index_topk_mask(v, k):
+    """Exactly k ones at the k largest values; among equal values the lower index first."""
+    order = torch.sort(-v.double(), stable=True)[1][:k]
+    m = torch.zeros_like(v)
+    m[order] = 1.0
+    return m
+
+
+@pytest.mark.parametrize("n,k", [(150, 75), (1, 1), (1, 0), (1000, 0), (1000, 1000), (1000, 1500), (5000, 1), (16383, 4000),
+                                 (16384, 8192), (70000, 123), (524288, 65536)])
+def test_topk_mask_ste_exact_count_and_ties(ops, gpu, n, k):
+    """The mask of the MoD router's training branch: exactly min(k, n) ones, at the largest values, the lower
+    index first among equals (one workgroup up to 16383 values, digit passes over many workgroups above);
+    heavy ties, a tie that straddles the threshold, signed zeros and infinities; and the straight-through
+    weights (mask - v) + v bit for bit."""
+    print("case topk_mask", n, k, flush=True)
+    g = gen(400 + n % 97 + k % 13)
+    kk = min(k, n)
+    cases = [torch.rand(n, generator=g)]
+    tied = torch.randint(0, 5, (n,), generator=g).float() * 0.25            # five distinct values
+    cases.append(tied)
+    half = torch.rand(n, generator=g)
+    half[::3] = 0.5                                                         # a third of the values are equal
+    cases.append(half)
+    sgn = torch.randn(n, generator=g)
+    sgn[::5] = 0.0
+    sgn[1::5] = -0.0
+    if n > 10:
+        sgn[2], sgn[7] = float("inf"), float("-inf")
+    cases.append(sgn)
+    for v in cases:
+        mask, ste = ops.topk_mask_ste(v.to(gpu), k)
+        want = _lowest_index_topk_mask(v, kk)
+        assert int(mask.sum().item()) == kk
+        assert torch.equal(mask.cpu(), want)
+        fin = torch.isfinite(v)
+        assert torch.equal(ste.cpu()[fin], ((want - v) + v)[fin])
+        assert torch.equal(ops.topk_mask_ste(v.to(gpu), k, want_ste=False).cpu(), want)
+
+
+def test_mod_router_training_branch(A, ops, gpu):
+    """MoDRouter in training mode (MS/core/model.py:941-965) against the oracle's restatement: probabilities,
+    mask (on bit-equal probabilities), straight-through weights, auxiliary loss, statistics, and the gradients of
+    x, the router weight and the bias under a per-token cotangent on both outputs."""
+    for dtype, tol in ((torch.float32, 1e-5), (torch.bfloat16, 2e-2)):
+        m = A.MoDRouter(96, capacity_factor=0.3, routing_temperature=1.7).to(gpu).train()
+        with torch.no_grad():
+            m.router.weight.copy_(torch.randn(1, 96, generator=gen(51)) * 0.3)
+            m.router.bias.fill_(-0.2)
+        x = torch.randn(4, 70, 96, generator=gen(52)).to(dtype)
+        cw = torch.randn(4, 70, 1, generator=gen(53))
+        cp = torch.randn(4, 70, 1, generator=gen(54))
+        xg = x.to(gpu).requires_grad_()
+        weights, probs, aux = m(xg)
+        assert weights.shape == probs.shape == (4, 70, 1) and weights.dtype == torch.float32
+        xr = x.float().requires_grad_()
+        wr = m.router.weight.detach().cpu().to(dtype).float().requires_grad_()
+        br = m.router.bias.detach().cpu().clone().requires_grad_()
+        rw, rp, rmask, raux = O.mod_router_train(xr, wr, br, 1.7, 0.3)
+        assert (probs.detach().cpu() - rp.detach()).abs().max().item() <= (2e-6 if dtype == torch.float32 else 2e-6)
+        k = int(280 * 0.3)
+        mask_gpu = (weights.detach() > 0.5).float().cpu()
+        assert int(mask_gpu.sum()) == k
+        assert torch.equal(mask_gpu.view(-1), _lowest_index_topk_mask(probs.detach().cpu().view(-1), k))   # bit-equal probs
+        differs = int((mask_gpu != rmask).sum())
+        assert differs <= 2                         # only a near-tie of the two sets of probabilities may differ
+        assert (weights.detach().cpu() - mask_gpu).abs().max().item() <= 1.2e-7
+        assert abs(aux.item() - raux.item()) <= 1e-7 and not aux.requires_grad
+        st = m.get_routing_stats()
+        assert st["total_tokens_routed"] == 280 and st["computed_tokens"] == k and st["skipped_tokens"] == 280 - k
+        torch.autograd.backward([weights, probs], [cw.to(gpu), cp.to(gpu)])
+        torch.autograd.backward([rw, rp], [cw, cp])
+        assert rel_err(xg.grad, xr.grad) <= tol
+        assert rel_err(m.router.weight.grad, wr.grad) <= max(tol, 2e-5)
+        assert rel_err(m.router.bias.grad, br.grad) <= 2e-5
+        # capacity_factor >= 1: every token computed, weights of one, zero auxiliary loss
+        m2 = A.MoDRouter(96, capacity_factor=1.0).to(gpu).train()
+        w2, _, aux2 = m2(x.to(gpu))
+        assert (w2 - 1.0).abs().max().item() <= 1.2e-7 and aux2.item() == 0.0
+
+
+def test_dense_swiglu_with_mod_trains(A, gpu):
+    """DenseSwiGLUWithMoD (MS/core/model.py:1304-1403) in training mode: the FFN output of every token times
+    its straight-through routing weight; output and all gradients against the oracle's pieces."""
+    from adaptivetrainingsystem_amd.workloads import LayerConfig
+    torch.manual_seed(23)
+    cfg = LayerConfig(128, 256, 1, 1, use_mod=True, mod_capacity_factor=0.5, mod_routing_temperature=1.0)
+    ffn = A.DenseSwiGLUWithMoD(cfg)
+    with torch.no_grad():
+        ffn.gate_up_proj.weight.mul_(6.0)
+        ffn.down_proj.weight.mul_(6.0)
+        ffn.router.router.weight.copy_(torch.randn(1, 128, generator=gen(55)) * 0.2)
+    ffn = ffn.to(gpu).train()
+    x = torch.randn(2, 48, 128, generator=gen(56))
+    dy = torch.randn(2, 48, 128, generator=gen(57))
+    xg = x.to(gpu).requires_grad_()
+    out, aux = ffn(xg)
+    out.backward(dy.to(gpu))
+    p = {n: t.detach().cpu().clone().requires_grad_() for n, t in ffn.named_parameters()}
+    xr = x.clone().requires_grad_()
+    rw, _, rmask, raux = O.mod_router_train(xr, p["router.router.weight"], p["router.router.bias"], 1.0, 0.5)
+    ref = O.swiglu_expert(xr, p["gate_up_proj.weight"], p["down_proj.weight"]) * rw
+    ref.backward(dy)
+    assert int((out.detach().abs().amax(-1) > 0).sum()) == 48          # half of the 96 tokens are computed
+    assert rel_err(out, ref) <= 1e-5 and abs(aux.item() - raux.item()) <= 1e-7
+    assert rel_err(xg.grad, xr.grad) <= 2e-5
+    for n, t in ffn.named_parameters():
+        assert t.grad is not None and rel_err(t.grad, p[n].grad) <= 3e-5, n
+    # evaluation mode keeps the threshold branch
+    ffn.eval()
+    with torch.no_grad():
+        out_e, aux_e = ffn(x.to(gpu))
+    assert aux_e is None and torch.isfinite(out_e).all()
+
+
 @pytest.mark.parametrize("L,keep", [(513, 1), (700, 700), (2048, 256), (2049, 300), (3000, 1), (4096, 4000),
                                     (8192, 1024)])
 def test_select_topk_long_sequences_with_ties(ops, gpu, L, keep):

@@ -36,7 +36,7 @@ def test_reference_launcher_names_are_exported_and_never_exit():
     from adaptivetrainingsystem_amd import _lib
     lib = _lib.load()
     raw = ctypes.CDLL(_lib.LIB_PATH)        # as the reference binds it: no argtypes, explicit ctypes wrappers
-    for n in ("rms_norm_launcher", "rope_precompute_launcher", "rope_apply_launcher", "swiglu_launcher",
+    for n in ("rms_norm_launcher", "rope_precompute_launcher", "rope_apply_launcher", "swiglu_launcher", "swiglu_fused_launcher",
               "fused_cross_entropy_accuracy_launcher", "fused_grad_clip_launcher"):      # training/cuda_kernels.py:60-78
         assert hasattr(raw, n), n
     raw.rms_norm_launcher(ctypes.c_void_p(0), ctypes.c_void_p(0), ctypes.c_void_p(0), ctypes.c_int(4), ctypes.c_int(0),

@@ -426,6 +426,40 @@ def test_mod_router_probs_special_cases():
     assert torch.all(near <= far)
 
 
+def test_mod_router_train_mask_ste_gradient_and_aux():
+    """Training branch of the MoD router: the mask is the brute-force ranking with exactly int(N*cf) ones; the
+    routing weights have the mask's value (to one ulp of the float32 (m - p) + p) and the gradient of the
+    probabilities, p(1-p)/T per logit in float64 terms; the auxiliary loss is (k/N - cf)^2 and a constant."""
+    gen = g(141)
+    B, L, H = 3, 11, 20
+    x = torch.randn(B, L, H, generator=gen)
+    for cf, b, T in ((0.5, 0.3, 1.0), (0.125, -0.2, 2.0), (0.9, 0.0, 0.7)):
+        w = (torch.randn(1, H, generator=gen) * 0.4).requires_grad_()
+        bias = torch.tensor([b], requires_grad=True)
+        xg = x.clone().requires_grad_()
+        weights, probs, mask, aux = O.mod_router_train(xg, w, bias, T, cf)
+        n, k = B * L, int(B * L * cf)
+        assert weights.shape == probs.shape == mask.shape == (B, L, 1)
+        pd = 1.0 / (1.0 + np.exp(-((x.double().numpy() @ w.detach().double().numpy()[0]) + b) / T))   # [B, L]
+        order = sorted(range(n), key=lambda i: -pd.reshape(-1)[i])
+        want = np.zeros(n)
+        want[order[:k]] = 1.0
+        assert int(mask.sum()) == k and np.array_equal(mask.reshape(-1).numpy(), want)
+        assert (weights.detach() - mask).abs().max().item() <= 1.2e-7
+        assert not mask.requires_grad and not aux.requires_grad
+        assert abs(aux.item() - (k / n - cf) ** 2) <= 1e-7
+        # a cotangent that differs per token: a gradient that ignored it, or used the mask's, would fail
+        cot = torch.randn(B, L, 1, generator=gen)
+        weights.backward(cot)
+        gl = cot.double().numpy()[..., 0] * pd * (1.0 - pd) / T                       # d loss / d logit
+        assert np.allclose(bias.grad.double().numpy(), gl.sum(), atol=1e-5)
+        assert np.allclose(w.grad.double().numpy()[0], np.einsum("bl,blh->h", gl, x.double().numpy()), atol=1e-5)
+        assert np.allclose(xg.grad.double().numpy(), gl[..., None] * w.detach().double().numpy()[0], atol=1e-6)
+    # capacity_factor of one or more: every token is computed
+    weights, _, mask, aux = O.mod_router_train(x, torch.randn(1, H, generator=gen), None, 1.0, 1.0)
+    assert mask.all() and abs(aux.item()) <= 1e-12
+
+
 def test_mod_moe_block_scores_and_selection_f64():
     """The block's scores are x.w + b in float64 terms and its selection is the brute-force top-keep of them."""
     gen = g(138)
