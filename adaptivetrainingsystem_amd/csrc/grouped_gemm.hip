@@ -3,20 +3,28 @@
 //   gate/up + SwiGLU : h[r, i] = silu(a_r . Wgu[e][i,:]) * (a_r . Wgu[e][I+i,:])
 //   down             : y[r, :] = h[r,:] . Wd[e]^T
 //
-// Both are "NT" products: activations [rows, K] and weights [N, K] have K
-// contiguous, so both operands are fetched with 16-byte loads along K and fed to
-// v_mfma_f32_32x32x16_bf16 (bf16) or v_mfma_f32_32x32x2_f32 (f32) without any
-// transpose.  The weight fragment is passed as the first MFMA operand, so the
-// accumulator of a lane holds 4 consecutive output columns of one output row
-// and the epilogue stores 8/16 contiguous bytes per lane.
+// Both are "NT" products: activations [rows, K] and weights [N, K] have K contiguous, so both operands are
+// fetched with 16-byte loads along K and fed to the matrix cores without any transpose.  The weight fragment
+// is the first MFMA operand, so the accumulator of a lane holds 4 consecutive output columns of one output
+// row.  With SwiGLU a tile holds BN/2 gate rows and the matching BN/2 up rows, so silu(g)*u is formed in
+// registers and the [rows, 2I] intermediate never exists.  The permutation gather is fused into the A load
+// (row index table).  One launch covers all experts: tile_schedule.hpp maps a block id to (expert, m-tile,
+// n-tile) so that the 32 workgroups of an XCD share operand panels in that XCD's L2.
 //
-// Block tile BM x BN (BN counts weight rows; with SwiGLU the tile holds BN/2
-// gate rows and the matching BN/2 up rows, so silu(g)*u is formed in registers
-// and the [rows, 2I] intermediate never exists).  K is consumed in 128-byte
-// slabs per row, staged through LDS with a 144-byte row pitch (bank-conflict
-// free for 16-byte reads), double buffered: the global loads of slab t+1 are in
-// flight while slab t feeds the matrix cores; one barrier per slab.
-// The permutation gather is fused into the A load (row index table).
+// Kernels, by the rows per expert the host sees (launch_grouped):
+//   grouped_gemm_dma16_kernel     bf16, groups above 192 rows (prefill and fine-grained shapes; also the
+//                                 training instances that save g/u or apply the SwiGLU gradient).  256 x 256
+//                                 tile, 8 waves of 128 x 64 on v_mfma_f32_16x16x32_bf16, K in 64-element
+//                                 slabs that go from memory straight into LDS (buffer_load ... lds: unpadded
+//                                 128-byte rows, XOR swizzle on the global side), three activation stages and
+//                                 two weight stages in the 160 KiB of LDS, one barrier per slab, fragment
+//                                 reads and loads placed among the MFMAs with sched_group_barrier.
+//   grouped_gemm_dma_kernel       the same data path for float32 operands on v_mfma_f32_32x32x2_f32.
+//   grouped_gemm_pipelined_kernel register-staged, two padded (144-byte pitch) or swizzled stages: the
+//                                 128-row tiles of mid-sized groups, the 32 / 64-row weight-streaming tiles of
+//                                 decode-sized groups (optionally sliced along K), and gather sources whose
+//                                 lane offsets do not fit 32 bits.
+//   grouped_gemm_kernel           general fallback for K that is not a multiple of a slab (bounds-checked loads).
 #include <math.h>
 
 #include <type_traits>
@@ -904,12 +912,17 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_dma_kernel(GroupedAr
 // A 64-element slab is two 32-element k-steps; the wave's 128 rows are two halves of four 16-row fragments.
 // A slab is four phases of 16 MFMAs, (k-step, row half) = (0,0) (0,1) (1,0) (1,1); fragments live in two
 // buffers of four activation fragments and two buffers of four weight fragments:
-//   phase 0 : MFMAs | reads: activations (k0, half 1), weights (k1) 0..1
-//   phase 1 : MFMAs | reads: activations (k1, half 0), weights (k1) 2..3
-//   phase 2 : MFMAs | reads: activations (k1, half 1)
+//   phase 0 : MFMAs | reads: activations (k0, half 1), weights (k1) 0..1 | loads: activations of slab t+2, 2 of 4
+//   phase 1 : MFMAs | reads: activations (k1, half 0), weights (k1) 2..3 | loads: activations of slab t+2, 1 of 4
+//   phase 2 : MFMAs | reads: activations (k1, half 1)                    | loads: activations of slab t+2, 1 of 4
 //   wait for the loads of slab t+1, barrier
-//   phase 3 : MFMAs | reads: activations (k0, half 0) and weights (k0) of slab t+1 | loads: weights of slab
-//             t+2, activations of slab t+3
+//   phase 3 : MFMAs | reads: activations (k0, half 0) and weights (k0) of slab t+1 | loads: weights of slab t+2
+// The activation ring has three stages, so the stage that slab t+2 goes into was given up at the previous
+// barrier and its loads can be issued anywhere in slab t; the weights have two stages, so theirs have to
+// follow the barrier.  With all eight loads of a wave behind the barrier the 64 loads of the workgroup
+// reached the texture addresser within a few hundred cycles, its queue filled up (it takes one 1 KiB load in
+// about 16 cycles) and the waves, which issue in order, stood at their next load with MFMAs behind it:
+// spreading the activation loads over the slab is worth 3-4 % at the prefill and at the fine-grained shape.
 template <typename TO, int SM, int SN, bool SWIGLU, bool SAVEGU = false, bool DSILU = false>
 __global__ __launch_bounds__(512) void grouped_gemm_dma16_kernel(GroupedArgs p) {
 #if defined(__HIP_DEVICE_COMPILE__)
@@ -1010,6 +1023,9 @@ __global__ __launch_bounds__(512) void grouped_gemm_dma16_kernel(GroupedArgs p) 
             __builtin_amdgcn_raw_ptr_buffer_load_lds(                                                  \
                 rsrc_a, (lds_ptr_t)(dma_a + (aoff_) + j * NW * 1024), 16, ao[j], soff, 0, 0);          \
     }
+#define D16_ISSUE_A1(kt_, aoff_, j_)                                                                   \
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc_a, (lds_ptr_t)(dma_a + (aoff_) + (j_) * NW * 1024), 16, \
+                                             ao[j_], (kt_) * 128, 0, 0)
 #define D16_ISSUE_B(kt_, stage_)                                                                       \
     {                                                                                                  \
         const int soff = (kt_) * 128;                                                                  \
@@ -1040,33 +1056,40 @@ __global__ __launch_bounds__(512) void grouped_gemm_dma16_kernel(GroupedArgs p) 
                     __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_.v, a_.v, acc[j][(half_) * 4 + i], 0, 0, 0); \
             }                                                                                          \
     }
-// nrd fragment reads spread over the first MFMAs of a phase (16 MFMAs)
-#define D16_MIX(nrd_)                                                                   \
+// nrd fragment reads and nvm loads spread over the first MFMAs of a phase (16 MFMAs)
+#define D16_MIX(nrd_, nvm_)                                                             \
     _Pragma("unroll") for (int g_ = 0; g_ < (nrd_); ++g_) {                             \
         __builtin_amdgcn_sched_group_barrier(SG_MFMA, 16 / ((nrd_) + 2), 0);            \
         __builtin_amdgcn_sched_group_barrier(SG_DS_RD, 1, 0);                           \
+        if (g_ < (nvm_)) __builtin_amdgcn_sched_group_barrier(SG_VMEM, 1, 0);           \
     }
-// phase 3: one fragment read and one load per MFMA while they last
+// phase 3: a fragment read per two MFMAs, a load per four
 #define D16_MIX_DMA()                                                                   \
     _Pragma("unroll") for (int g_ = 0; g_ < 8; ++g_) {                                  \
         __builtin_amdgcn_sched_group_barrier(SG_DS_RD, 1, 0);                           \
-        __builtin_amdgcn_sched_group_barrier(SG_MFMA, 1, 0);                            \
-        __builtin_amdgcn_sched_group_barrier(SG_VMEM, 1, 0);                            \
+        __builtin_amdgcn_sched_group_barrier(SG_MFMA, 2, 0);                            \
+        if (g_ % 2 == 0) __builtin_amdgcn_sched_group_barrier(SG_VMEM, 1, 0);           \
     }
-// STG: weight stage of slab kt (compile time); sa_cur / sa_nxt: activation stage offsets of slabs kt, kt+1.
-// Slabs past the end are clamped to the last one (their loads land in stages nobody reads again).
+// STG: weight stage of slab kt (compile time); sa_cur / sa_nxt: activation stage offsets of slabs kt, kt+1
+// (the third stage takes slab kt+2).  Slabs past the end are clamped to the last one (their loads land in
+// stages nobody reads again).
 // H0 / H1 (compile time): whether row half 0 / 1 of this wave holds rows of the expert at all; a half made
 // only of rows past the expert's end keeps its loads and barriers but skips its fragment reads and MFMAs.
 #define D16_ITER(kt_, STG, H0, H1)                                                      \
     {                                                                                   \
+        const int sa_far = 3 * A_STAGE - sa_cur - sa_nxt;                               \
+        const int ka_ = min((kt_) + 2, nk - 1);                                         \
         if (H1) D16_READ_A(sa_cur, 0, 1, 1);                                            \
+        D16_ISSUE_A1(ka_, sa_far, 0);                                                   \
+        D16_ISSUE_A1(ka_, sa_far, 1);                                                   \
         if (H0) {                                                                       \
             D16_READ_B(STG, 1, 0, 1);                                                   \
             D16_READ_B(STG, 1, 1, 1);                                                   \
             D16_MMA(0, 0, 0);                                                           \
-            D16_MIX(H1 ? 6 : 2);                                                        \
+            D16_MIX(H1 ? 6 : 2, 2);                                                     \
         }                                                                               \
         PL_FENCE();                                                                     \
+        D16_ISSUE_A1(ka_, sa_far, 2);                                                   \
         if (H0) {                                                                       \
             D16_READ_A(sa_cur, 1, 0, 0);                                                \
             D16_READ_B(STG, 1, 2, 1);                                                   \
@@ -1074,13 +1097,14 @@ __global__ __launch_bounds__(512) void grouped_gemm_dma16_kernel(GroupedArgs p) 
         }                                                                               \
         if (H1) {                                                                       \
             D16_MMA(0, 1, 1);                                                           \
-            D16_MIX(6);                                                                 \
+            D16_MIX(6, 1);                                                              \
         }                                                                               \
         PL_FENCE();                                                                     \
+        D16_ISSUE_A1(ka_, sa_far, 3);                                                   \
         if (H1) D16_READ_A(sa_cur, 1, 1, 1);                                            \
         if (H0) {                                                                       \
             D16_MMA(1, 0, 0);                                                           \
-            D16_MIX(H1 ? 4 : 0);                                                        \
+            D16_MIX(H1 ? 4 : 1, 1);                                                     \
         }                                                                               \
         PL_FENCE();                                                                     \
         asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(NIA) : "memory"); \
@@ -1093,7 +1117,6 @@ __global__ __launch_bounds__(512) void grouped_gemm_dma16_kernel(GroupedArgs p) 
             D16_READ_B(STG ^ 1, 0, 3, 0);                                               \
         }                                                                               \
         D16_ISSUE_B(min((kt_) + 2, nk - 1), STG);                                       \
-        D16_ISSUE_A(min((kt_) + 3, nk - 1), sa_cur);                                    \
         if (H1) {                                                                       \
             D16_MMA(1, 1, 1);                                                           \
             D16_MIX_DMA();                                                              \
@@ -1121,8 +1144,7 @@ __global__ __launch_bounds__(512) void grouped_gemm_dma16_kernel(GroupedArgs p) 
     }
     D16_ISSUE_A(0, 0);
     D16_ISSUE_A(min(1, nk - 1), A_STAGE);
-    D16_ISSUE_A(min(2, nk - 1), 2 * A_STAGE);
-    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(2 * NIA) : "memory");
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(NIA) : "memory");
     int sa_cur = 0, sa_nxt = A_STAGE;
     // rows of the expert in this wave's 128-row share of the tile (wave-uniform)
     const int wave_rows = count - (tc.mt * BM + wm * (BM / WM));
@@ -1143,6 +1165,7 @@ __global__ __launch_bounds__(512) void grouped_gemm_dma16_kernel(GroupedArgs p) 
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
 #undef D16_LOOP
 #undef D16_ISSUE_A
+#undef D16_ISSUE_A1
 #undef D16_ISSUE_B
 #undef D16_B_ROW
 #undef D16_READ_A
