@@ -10,7 +10,8 @@
 //   3. per-chunk ranking: inside a wave the rank among equal ids comes from
 //      ballots; across the steps of a wave and the waves of a block from small
 //      LDS counters that are only ever advanced in program order.
-// Small plans (T*k <= kPlanSingle) run all three steps in one block, one launch.
+// Small plans (T*k <= kPlanSingle) run all three steps in one block, one launch; plans of up to kPlanFused
+// assignments run in one launch of many blocks that each count the chunks before their own themselves.
 #include <limits.h>
 
 #include "ats_common.hpp"
@@ -221,6 +222,138 @@ __global__ __launch_bounds__(256) void plan_rank_kernel(const IdxT* __restrict__
         if (pos >= kept[e]) token_map[i] = -1;
     }
     const int total = offsets[E];
+    for (int64_t i = total + (int64_t)blockIdx.x * 256 + threadIdx.x; i < row_src_len; i += stride) row_src[i] = -1;
+}
+
+// Plans of up to kPlanFused assignments in ONE launch of many blocks and no workspace: a block does not wait
+// for the histograms of the chunks before its own, it counts them itself.  Every block walks the whole
+// index list once (at most 128 KiB from L2; 16-byte loads when the list is int32): the assignments before
+// its chunk give the chunk's exclusive bases, all of them give the totals, from which every block forms
+// kept / offsets for itself; then it ranks its chunk as the third kernel of the long form does.  Three
+// dependent launches (4.5 + 4.7 + 7.7 us at 24576 assignments over 64 experts) become one.  Same integers
+// by construction: the bases are counts of the same sets.
+constexpr int kPlanFused = 32768;
+
+// Replicas of a wave's counters in the counting pass: with few experts most lanes of a wave hit the same
+// counter and the LDS atomics of an instruction run one after the other (with Zipf-skewed routing over 8
+// experts two fifths of the lanes hit expert 0's).
+__host__ __device__ inline int plan_count_replicas(int E) { return E <= 16 ? 8 : (E <= 64 ? 2 : 1); }
+
+// One pass over all n indices into two counter sets: assignments before `split` (a multiple of 4) into
+// cnt, the others into cnt + set_stride.  cnt: [4 waves][E][R] counters per set.
+template <typename IdxT>
+__device__ __forceinline__ void count_split(const IdxT* __restrict__ idx, int64_t n, int64_t split, int E, int R,
+                                            int* cnt, int set_stride, bool* bad) {
+    int* mine = cnt + (threadIdx.x >> 6) * E * R + (threadIdx.x & (R - 1));
+    int64_t tail_from = 0;
+    if (sizeof(IdxT) == 4 && (reinterpret_cast<uintptr_t>(idx) & 15) == 0) {
+        // sixteen 16-byte loads in flight per thread: one at a time, the L2 round trips of the 24-32 loads a
+        // thread makes were the whole cost of the pass
+        const int4* v = reinterpret_cast<const int4*>(idx);
+        constexpr int U = 16;
+        const int64_t qend = n / 4, qsplit = split / 4;
+        for (int64_t q0 = threadIdx.x; q0 < qend; q0 += 256 * U) {
+            int4 w[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int64_t q = q0 + (int64_t)u * 256;
+                w[u] = v[q < qend ? q : q0];
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int64_t q = q0 + (int64_t)u * 256;
+                if (q >= qend) break;
+                int* set = mine + (q >= qsplit ? set_stride : 0);
+                const int ids[4] = {w[u].x, w[u].y, w[u].z, w[u].w};
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    if (ids[j] < 0 || ids[j] >= E) *bad = true;
+                    else atomicAdd(&set[ids[j] * R], 1);
+                }
+            }
+        }
+        tail_from = qend * 4;
+    }
+    for (int64_t a = tail_from + threadIdx.x; a < n; a += 256) {
+        const int e = load_expert(idx, a, n, E, bad);
+        if (e >= 0) atomicAdd(&mine[(a >= split ? set_stride : 0) + e * R], 1);
+    }
+}
+
+__device__ __forceinline__ int count_total(const int* cnt, int E, int R, int e) {
+    int t = 0;
+    for (int w = 0; w < 4; ++w)
+        for (int r = 0; r < R; ++r) t += cnt[(w * E + e) * R + r];
+    return t;
+}
+
+template <typename IdxT>
+__global__ __launch_bounds__(256) void plan_fused_kernel(const IdxT* __restrict__ idx, int64_t n, int k, int E, int C,
+                                                         int32_t* __restrict__ hist, int32_t* __restrict__ kept,
+                                                         int32_t* __restrict__ offsets, int32_t* __restrict__ slot,
+                                                         int32_t* __restrict__ token_map, int32_t* __restrict__ row_src,
+                                                         int32_t* __restrict__ row_of, int64_t row_src_len,
+                                                         int32_t* __restrict__ status) {
+    extern __shared__ int s_all[];
+    const int R = plan_count_replicas(E);
+    int* s_cnt = s_all;               // [4 * E] per-wave counters of the chunk
+    int* s_pre = s_all + 4 * E;       // [E] assignments before this chunk
+    int* s_kept = s_all + 5 * E;      // [E]
+    int* s_off = s_all + 6 * E;       // [E + 1]
+    int* s_rep = s_all + 7 * E + 1;   // [2][4 * E * R] counters of the counting pass
+    const int lane = lane_id();
+    const int wave = threadIdx.x >> 6;
+    const int64_t chunk_base = (int64_t)blockIdx.x * kPlanChunk;
+    bool bad = false;
+    // one pass over the whole list: assignments before the chunk into the first counter set (the chunk's
+    // exclusive bases), the chunk and everything after it into the second (with the first: the totals)
+    const int set = 4 * E * R;
+    for (int i = threadIdx.x; i < 2 * set; i += 256) s_rep[i] = 0;
+    __syncthreads();
+    count_split<IdxT>(idx, n, chunk_base, E, R, s_rep, set, &bad);
+    __syncthreads();
+    for (int e = threadIdx.x; e < E; e += 256) {
+        const int pre = count_total(s_rep, E, R, e);
+        const int tot = pre + count_total(s_rep + set, E, R, e);
+        const int kp = tot < C ? tot : C;
+        s_pre[e] = pre;
+        s_kept[e] = kp;
+        if (blockIdx.x == 0) {
+            hist[e] = tot;
+            kept[e] = kp;
+        }
+    }
+    __syncthreads();
+    if (wave == 0) {
+        int run = 0;
+        for (int e0 = 0; e0 < E; e0 += kWave) {
+            const int e = e0 + lane;
+            const int kp = e < E ? s_kept[e] : 0;
+            const int incl = wave_inclusive_scan(kp);
+            if (e < E) s_off[e] = run + incl - kp;
+            run += __builtin_amdgcn_readlane(incl, kWave - 1);
+        }
+        if (lane == 0) s_off[E] = run;
+    }
+    __syncthreads();
+    if (blockIdx.x == 0) {
+        for (int e = threadIdx.x; e <= E; e += 256) offsets[e] = s_off[e];
+        // block 0 has seen every index: it alone writes the status word
+        const int any_bad = __syncthreads_or(bad ? 1 : 0);
+        if (threadIdx.x == 0) status[0] = any_bad;
+    }
+    // ranks of the chunk
+    chunk_wave_counts<IdxT, kPlanChunk / 4>(idx, n, E, chunk_base, s_cnt, &bad);
+    chunk_rank_and_write<IdxT, kPlanChunk / 4>(idx, n, k, E, C, chunk_base, s_pre, 1, s_off, s_cnt, slot, token_map,
+                                               row_src, row_of);
+    const int64_t stride = (int64_t)gridDim.x * 256;
+    const int64_t ec = (int64_t)E * C;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < ec; i += stride) {
+        const int e = (int)(i / C);
+        const int pos = (int)(i - (int64_t)e * C);
+        if (pos >= s_kept[e]) token_map[i] = -1;
+    }
+    const int total = s_off[E];
     for (int64_t i = total + (int64_t)blockIdx.x * 256 + threadIdx.x; i < row_src_len; i += stride) row_src[i] = -1;
 }
 
@@ -676,15 +809,29 @@ extern "C" int ats_dispatch_plan(const void* idx, int idx_dtype, int64_t T, int 
     ATS_REQUIRE(T == 0 || idx, ATS_ERR_INVALID_ARG, "ats_dispatch_plan: null idx");
     const int64_t n = T * k;
     const bool single = n <= kPlanSingle;
+    const bool fused = !single && n <= kPlanFused;
     const int64_t nchunks = single ? 1 : (n + kPlanChunk - 1) / kPlanChunk;
-    const size_t need = (size_t)nchunks * E * sizeof(int32_t);
-    ATS_REQUIRE(workspace && workspace_bytes >= need, ATS_ERR_WORKSPACE,
+    const size_t need = fused ? 0 : (size_t)nchunks * E * sizeof(int32_t);
+    ATS_REQUIRE(fused || (workspace && workspace_bytes >= need), ATS_ERR_WORKSPACE,
                 "ats_dispatch_plan: workspace %zu bytes, need %zu", workspace_bytes, need);
     hipStream_t s = as_stream(stream);
     int32_t* chunk_hist = static_cast<int32_t*>(workspace);
     int64_t row_src_len = n < (int64_t)E * C ? n : (int64_t)E * C;
     if (row_src_len < 1) row_src_len = 1;
     const size_t smem = (size_t)5 * E * sizeof(int);
+    if (fused) {
+        const size_t smem_fused = ((size_t)7 * E + 1 + (size_t)8 * E * plan_count_replicas(E)) * sizeof(int);
+        if (idx_dtype == ATS_IDX_I32)
+            hipLaunchKernelGGL((plan_fused_kernel<int32_t>), dim3((unsigned)nchunks), dim3(256), smem_fused, s,
+                               static_cast<const int32_t*>(idx), n, k, E, C, hist, kept, offsets, slot, token_map,
+                               row_src, row_of, row_src_len, status);
+        else
+            hipLaunchKernelGGL((plan_fused_kernel<int64_t>), dim3((unsigned)nchunks), dim3(256), smem_fused, s,
+                               static_cast<const int64_t*>(idx), n, k, E, C, hist, kept, offsets, slot, token_map,
+                               row_src, row_of, row_src_len, status);
+        ATS_CHECK_LAUNCH("ats_dispatch_plan(fused)");
+        return ATS_OK;
+    }
     if (single) {
         if (idx_dtype == ATS_IDX_I32)
             hipLaunchKernelGGL((plan_single_kernel<int32_t>), dim3(1), dim3(256), smem, s,

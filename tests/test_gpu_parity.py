@@ -283,7 +283,10 @@ def _check_plan(ops, gpu, idx, E, C, idx_dtype=torch.int32):
 
 
 @pytest.mark.parametrize("T,E,k,C", [(16, 4, 2, 5), (512, 8, 2, 160), (64, 8, 2, 20), (300, 8, 3, 0), (1500, 8, 2, 1000000 // 8),
-                                     (4096, 64, 6, 576), (16384, 8, 2, 5120), (32768, 64, 6, 4608), (700, 300, 4, 7)])
+                                     (4096, 64, 6, 576), (16384, 8, 2, 5120), (32768, 64, 6, 4608), (700, 300, 4, 7),
+                                     # the one-launch form (1025 .. 32768 assignments): ragged ends, replica counts
+                                     (513, 8, 2, 100), (3001, 5, 3, 2000), (10922, 20, 3, 1500), (8000, 70, 4, 600),
+                                     (16385, 8, 2, 5120)])
 def test_dispatch_plan_bit_exact(ops, gpu, T, E, k, C):
     print("case plan", T, E, k, C, flush=True)
     g = gen(17 + T)
