@@ -300,7 +300,7 @@ int ats_swiglu_mul(const void* gate, const void* up, void* out, int64_t n, int d
  * RMSNormFunction.backward (cuda_opt_wrapper.py:119-142): with g = dy*w,
  * r = rsqrt(mean(x^2)+eps):  dx = r*g - x*r^3*mean(g*x),  dw[h] = sum_rows dy*x*r
  * (float32, fixed summation order).  dw may be NULL; otherwise workspace must hold
- * ats_rmsnorm_bwd_workspace(rows, hidden) bytes. */
+ * ats_rmsnorm_bwd_workspace(rows, hidden) bytes, 16-byte aligned. */
 size_t ats_rmsnorm_bwd_workspace(int64_t rows, int hidden);
 int ats_rmsnorm_bwd(const void* x, const void* w, const void* dy, void* dx, float* dw, int64_t rows,
                     int hidden, float eps, int x_dtype, int w_dtype, void* workspace,
