@@ -40,6 +40,25 @@ from .profiling import stage, timer_context
 from ._lib import ROUTE_SOFTMAX_TOPK, ROUTE_TOPK_SOFTMAX, AtsError
 
 
+# float16 activations: the gfx950 kernels take float32 and bfloat16.  The reference's fused wrappers convert
+# whatever comes in to float32, run their kernel and convert back (MS/core/cuda_opt_wrapper.py:92, 117, 153, 217),
+# and its RMSNorm computes in float32 for every dtype (MS/core/model.py:263-299); float16 is served the same
+# way here: up-cast, the float32 kernels, one rounding back to float16.  The casts are torch's (differentiable),
+# so RMSNorm and RoPE also train that way; the layers with weight matrices take float16 for inference only.
+def _is_f16(*tensors: Optional[torch.Tensor]) -> bool:
+    return any(t is not None and t.dtype == torch.float16 for t in tensors)
+
+
+def _f32(t: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
+    return t if t is None or t.dtype == torch.float32 else t.float()
+
+
+def _no_f16_training(name: str, *tensors: Optional[torch.Tensor]) -> None:
+    if _wants_grad(*tensors):
+        raise AtsError(f"{name}: float16 activations are served through the float32 kernels for inference only; "
+                       "train in bfloat16 or float32")
+
+
 # ============================================================================ normalisation
 class RMSNorm(nn.Module):
     """y = x * rsqrt(mean(x^2) + eps) * weight, float32 math, result in x's dtype."""
@@ -58,6 +77,10 @@ class RMSNorm(nn.Module):
         if x.shape[-1] != self.dim:
             raise AtsError(f"RMSNorm: last dimension {x.shape[-1]} != {self.dim}")
         w = self.weight if self.elementwise_affine else None
+        if _is_f16(x, w):
+            xf, wf = _f32(x), _f32(w)
+            y = ag.RMSNormFunction.apply(xf, wf, self.eps) if _wants_grad(xf, wf) else ops.rmsnorm(xf, wf, self.eps)
+            return y.to(x.dtype)
         if _wants_grad(x, w):
             return ag.RMSNormFunction.apply(x, w, self.eps)
         return ops.rmsnorm(x, w, self.eps)
@@ -83,6 +106,10 @@ class FusedRMSNorm(nn.Module):
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         if self.float32_output and x.dtype != torch.float32:
             x = x.float()
+        if _is_f16(x, self.weight):
+            xf, wf = _f32(x), _f32(self.weight)
+            y = ag.RMSNormFunction.apply(xf, wf, self.eps) if _wants_grad(xf, wf) else ops.rmsnorm(xf, wf, self.eps)
+            return y.to(x.dtype)
         if _wants_grad(x, self.weight):
             return ag.RMSNormFunction.apply(x, self.weight, self.eps)
         return ops.rmsnorm(x, self.weight, self.eps)
@@ -136,6 +163,9 @@ class RotaryEmbedding(nn.Module):
 def apply_rotary_pos_emb(q: torch.Tensor, k: torch.Tensor, cos: torch.Tensor,
                          sin: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
     """q [B,Hq,L,D], k [B,Hkv,L,D], cos/sin [L, D] -> rotated (q, k) in the input dtype."""
+    if _is_f16(q, k):
+        qo, ko = apply_rotary_pos_emb(_f32(q), _f32(k), cos, sin)
+        return qo.to(q.dtype), ko.to(k.dtype)
     if _wants_grad(q, k):
         return ag.RoPEFunction.apply(q, k, cos, sin, 0)
     return ops.rope(q, k, cos, sin, 0)
@@ -157,6 +187,9 @@ class FusedRoPE(nn.Module):
         if self.cos_cache.device != q.device:
             self.cos_cache = self.cos_cache.to(q.device)
             self.sin_cache = self.sin_cache.to(q.device)
+        if _is_f16(q, k):
+            qo, ko = self.forward(_f32(q), _f32(k), position_offset)
+            return qo.to(q.dtype), ko.to(k.dtype)
         if _wants_grad(q, k):
             return ag.RoPEFunction.apply(q, k, self.cos_cache, self.sin_cache, position_offset)
         return ops.rope(q, k, self.cos_cache, self.sin_cache, position_offset)
@@ -209,8 +242,15 @@ class GroupedQueryAttention(nn.Module):
                 use_cache: bool = False):
         if x.dim() != 3 or x.shape[-1] != self.hidden_size:
             raise AtsError(f"GroupedQueryAttention: expected [batch, seq, {self.hidden_size}], got {tuple(x.shape)}")
+        if x.dtype == torch.float16:
+            _no_f16_training("GroupedQueryAttention", x, *self.parameters())
+            past = None if past_key_value is None else tuple(_f32(t) for t in past_key_value)
+            res = self.forward(x.float(), attention_mask, past, use_cache)
+            if use_cache:
+                return res[0].to(x.dtype), tuple(t.to(x.dtype) for t in res[1])
+            return res.to(x.dtype)
         if x.dtype not in (torch.bfloat16, torch.float32):
-            raise AtsError(f"GroupedQueryAttention: bfloat16 or float32 activations, got {x.dtype}")
+            raise AtsError(f"GroupedQueryAttention: bfloat16, float16 or float32 activations, got {x.dtype}")
         B, L, H = x.shape
         nh, nkv, D = self.num_heads, self.num_kv_heads, self.head_dim
         x2 = x.reshape(B * L, H).contiguous()
@@ -370,6 +410,9 @@ class SwiGLUExpert(nn.Module):
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         """One expert over every row of x, through the grouped kernels with a single group."""
+        if x.dtype == torch.float16:
+            _no_f16_training(type(self).__name__, x, *self.parameters())
+            return SwiGLUExpert.forward(self, x.float()).to(x.dtype)
         shape = x.shape
         x2 = x.reshape(-1, shape[-1]).contiguous()
         n = x2.shape[0]
@@ -479,6 +522,12 @@ class MoEFFNLayer(nn.Module):
         returned in its place; for a block that runs the layer on a subset of a longer sequence."""
         if x.dim() != 3 or x.shape[-1] != self.hidden_size:
             raise AtsError(f"MoEFFNLayer: expected [batch, seq, {self.hidden_size}], got {tuple(x.shape)}")
+        if x.dtype == torch.float16:
+            _no_f16_training("MoEFFNLayer", x, *self.parameters())
+            if add_onto is not None:
+                raise AtsError("MoEFFNLayer: add_onto takes bfloat16 or float32 activations")
+            out, aux = self.forward(x.float())
+            return out.to(x.dtype), aux
         if len(self.experts) != self.num_experts or self.gate.weight.shape[0] != self.num_experts:
             raise AtsError("MoEFFNLayer: num_experts, experts and gate disagree")
         B, L, H = x.shape

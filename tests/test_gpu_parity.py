@@ -1145,3 +1145,62 @@ def test_kth_value_mask_both_selects(ops, gpu, n, kth):
     torch.cuda.synchronize()
     assert torch.equal(m2.cpu(), ref) and ws[1].item() == int(ref.sum().item())
     assert int(lib.ats_kth_value_workspace(n)) == (16 if n < 16384 else 16 + 4096)
+
+
+# ------------------------------------------------------------------ float16 activations
+def test_float16_activations_run_through_the_float32_kernels(A, gpu):
+    """float16 is served as the reference's fused wrappers serve every dtype (cuda_opt_wrapper.py:92, 117, 153, 217):
+    up-cast, float32 kernels, one rounding back.  Norm and RoPE also train that way; the layers with weight
+    matrices take float16 for inference and refuse to train in it."""
+    from adaptivetrainingsystem_amd.workloads import LayerConfig
+    g = gen(91)
+    x = torch.randn(3, 17, 256, generator=g).half()
+    norm = A.RMSNorm(256).to(gpu)
+    with torch.no_grad():
+        norm.weight.copy_(torch.randn(256, generator=g) * 0.1 + 1.0)
+    y = norm(x.to(gpu))
+    ref = O.rmsnorm(x.float(), norm.weight.detach().cpu(), 1e-6)
+    assert y.dtype == torch.float16 and rel_err(y, ref) <= 2 ** -10
+    xg = x.to(gpu).requires_grad_()
+    norm(xg).float().sum().backward()
+    xr = x.float().requires_grad_()
+    O.rmsnorm(xr, norm.weight.detach().cpu(), 1e-6).sum().backward()
+    assert xg.grad.dtype == torch.float16 and rel_err(xg.grad, xr.grad) <= 2e-3
+    fused = A.FusedRMSNorm(256).to(gpu).half()
+    assert fused(x.to(gpu)).dtype == torch.float16
+    q = torch.randn(2, 4, 33, 64, generator=g).half()
+    k = torch.randn(2, 2, 33, 64, generator=g).half()
+    cos, sin = A.RotaryEmbedding(64, max_seq_len=64)(33, gpu)
+    gq, gk = A.apply_rotary_pos_emb(q.to(gpu), k.to(gpu), cos, sin)
+    rq, rk = O.rope_apply(q.float(), k.float(), cos.cpu(), sin.cpu())
+    assert gq.dtype == torch.float16 and rel_err(gq, rq) <= 2 ** -10 and rel_err(gk, rk) <= 2 ** -10
+    fq, fk = A.FusedRoPE(64, max_seq_len=64)(q.to(gpu), k.to(gpu), 3)
+    assert fq.dtype == torch.float16 and fk.shape == k.shape
+    # MoE layer, dense FFN and attention: float16 inference against the oracle on float32 copies
+    cfg = LayerConfig(128, 256, 4, 2, 1.25, num_heads=4, num_kv_heads=2, seq_length=64, moe_capacity_mode="fcfs")
+    torch.manual_seed(3)
+    moe = A.MoEFFNLayer(cfg).to(gpu).half().eval()
+    xm = torch.randn(2, 24, 128, generator=g).half()
+    with torch.no_grad():
+        out, aux = moe(xm.to(gpu))
+    p = moe.last_plan
+    refm = O.moe_forward_capacity(xm.float(), moe.gate.weight.detach().float().cpu(),
+                                  [e.gate_up_proj.weight.detach().float().cpu() for e in moe.experts],
+                                  [e.down_proj.weight.detach().float().cpu() for e in moe.experts], k=2,
+                                  capacity_factor=1.25, logits_override=p["logits"].cpu())
+    assert out.dtype == torch.float16 and rel_err(out, refm["out"].reshape(out.shape)) <= 2e-3
+    ffn = A.DenseSwiGLU(cfg).to(gpu).half().eval()
+    with torch.no_grad():
+        yf = ffn(xm.to(gpu))
+    assert yf.dtype == torch.float16
+    assert rel_err(yf, O.swiglu_expert(xm.float(), ffn.gate_up_proj.weight.detach().float().cpu(),
+                                       ffn.down_proj.weight.detach().float().cpu())) <= 2e-3
+    att = A.GroupedQueryAttention(cfg).to(gpu).half().eval()
+    with torch.no_grad():
+        ya, (kc, vc) = att(xm.to(gpu), use_cache=True)
+    w = [getattr(att, n).weight.detach().float().cpu() for n in ("q_proj", "k_proj", "v_proj", "o_proj")]
+    assert ya.dtype == kc.dtype == vc.dtype == torch.float16
+    assert rel_err(ya, O.gqa_forward(xm.float(), *w, 4, 2)) <= 5e-3
+    moe.train()
+    with pytest.raises(A.AtsError):
+        moe(xm.to(gpu).requires_grad_())
