@@ -60,6 +60,13 @@ class FusedSwiGLU(nn.Module):
         H, I = self.hidden_size, self.intermediate_size
         if x.shape[-1] != H:
             raise _lib.AtsError(f"FusedSwiGLU: last dimension {x.shape[-1]} != hidden_size {H}")
+        if x.dtype == torch.float16:
+            # as the reference's wrapper serves every dtype (cuda_opt_wrapper.py:217): up-cast, float32 kernels,
+            # one rounding back; inference only (the matrices would need float32 master copies to train)
+            if _wants_grad(x, *self.parameters()):
+                raise _lib.AtsError("FusedSwiGLU: float16 activations are served through the float32 kernels for "
+                                    "inference only; train in bfloat16 or float32")
+            return self.forward(x.float()).to(x.dtype)
         out_shape = x.shape[:-1] + (I,)
         x2 = x.reshape(-1, H).contiguous()
         n = x2.shape[0]

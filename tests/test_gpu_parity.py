@@ -1204,3 +1204,12 @@ def test_float16_activations_run_through_the_float32_kernels(A, gpu):
     moe.train()
     with pytest.raises(A.AtsError):
         moe(xm.to(gpu).requires_grad_())
+    from adaptivetrainingsystem_amd.seams import cuda_opt_wrapper as cow
+    sw = cow.FusedSwiGLU(128, 192).to(gpu).half().eval()
+    with torch.no_grad():
+        ys = sw(xm.to(gpu))
+    gate = xm.float() @ sw.gate_proj.weight.detach().float().cpu().t()
+    up = xm.float() @ sw.up_proj.weight.detach().float().cpu().t()
+    assert ys.dtype == torch.float16 and rel_err(ys, torch.nn.functional.silu(gate) * up) <= 2e-3
+    with pytest.raises(A.AtsError):
+        sw(xm.to(gpu).requires_grad_())
