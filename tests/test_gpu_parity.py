@@ -1210,6 +1210,6 @@ def test_float16_activations_run_through_the_float32_kernels(A, gpu):
         ys = sw(xm.to(gpu))
     gate = xm.float() @ sw.gate_proj.weight.detach().float().cpu().t()
     up = xm.float() @ sw.up_proj.weight.detach().float().cpu().t()
-    assert ys.dtype == torch.float16 and rel_err(ys, torch.nn.functional.silu(gate) * up) <= 2e-3
+    assert ys.dtype == torch.float16 and rel_err(ys, gate * torch.nn.functional.silu(up)) <= 2e-3
     with pytest.raises(A.AtsError):
         sw(xm.to(gpu).requires_grad_())
