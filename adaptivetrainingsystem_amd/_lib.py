@@ -44,10 +44,11 @@ _SIGNATURES = {
                                           c_int64, c_int, c_int, c_int, c_void_p]),
     "ats_grouped_down_dgrad_dsilu_supported": (c_int, [c_int, c_int64, c_int, c_int, c_int]),
     "ats_grouped_down_dgrad_dsilu": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64,
-                                             c_int, c_int, c_int, c_void_p]),
+                                             c_int, c_int, c_int, c_void_p, c_int64, c_void_p, c_void_p]),
     "ats_grouped_gateup_swiglu_save_supported": (c_int, [c_int64, c_int, c_int64, c_int, c_int, c_int]),
     "ats_grouped_gateup_swiglu_save": (c_int, [c_void_p, c_int64, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
-                                               c_void_p, c_int, c_int64, c_int, c_int, c_int, c_void_p]),
+                                               c_void_p, c_int, c_int64, c_int, c_int, c_int, c_void_p, c_int64,
+                                               c_void_p, c_void_p]),
     "ats_grouped_down": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int, c_int,
                                  c_int, c_int, c_void_p]),
     "ats_grouped_down_splitk": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64, c_int64,
@@ -77,6 +78,7 @@ _SIGNATURES = {
     "ats_transpose_batched": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "ats_wgrad_padded_rows": (c_int64, [c_int64, c_int]),
     "ats_wgrad_plan": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p]),
+    "ats_transposed_zero_empty_groups": (c_int, [c_void_p, c_int64, c_int, c_void_p, c_void_p, c_int, c_int, c_void_p]),
     "ats_transpose_grouped_rows": (c_int, [c_void_p, c_int64, c_int, c_void_p, c_int, c_void_p, c_void_p, c_int,
                                            c_int64, c_void_p, c_int64, c_int, c_void_p]),
     "ats_grouped_gemm_nt": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_void_p, c_int, c_void_p, c_int64, c_int64,

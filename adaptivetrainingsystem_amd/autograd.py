@@ -194,31 +194,50 @@ class SwiGLUFunction(Function):
         return dg.view(ctx.shape), du.view(ctx.shape)
 
 
-def _ffn_forward(x, wgu, wd, offsets, kept, rows, row_src, k):
+# Whether the fused bfloat16 training kernels also write the transposed copies of h and dgu that the weight-gradient
+# products contract over (otherwise separate transposing passes produce them; same bits either way).
+FUSE_TRANSPOSED_COPIES = True
+
+
+def _ffn_forward(x, wgu, wd, offsets, kept, rows, row_src, k, want_wgrad=False):
     """Expert FFN over the grouped rows, keeping the gate/up pre-activations for the backward pass.
-    Returns (gu [rows, 2I], h [rows, I], y [rows, H])."""
+    Returns (gu [rows, 2I], h [rows, I], y [rows, H], hT, wplan): with want_wgrad, wplan = the weight-gradient
+    layout of these groups (ops.wgrad_plan) and, where the fused bfloat16 kernel runs, hT = h already transposed
+    into it by that kernel (the backward pass then keeps hT instead of h); otherwise None."""
     H, I = x.shape[1], wd[0].shape[1]
     tab_gu, tab_d = ops.weight_pointer_table(wgu), ops.weight_pointer_table(wd)
-    both = ops.grouped_gateup_swiglu_save(x, tab_gu, offsets, kept, rows, rows, H, I, a_rows=row_src, a_row_div=k)
+    wplan = ops.wgrad_plan(kept) if want_wgrad and rows > 0 else None
+    hT = None
+    both = ops.grouped_gateup_swiglu_save(x, tab_gu, offsets, kept, rows, rows, H, I, a_rows=row_src, a_row_div=k,
+                                          t_col0=wplan[0] if wplan is not None and FUSE_TRANSPOSED_COPIES else None)
     if both is not None:             # prefill-sized groups: one kernel writes the pre-activations and h
-        gu, h = both
+        gu, h, hT = both
     else:
         gu = ops.grouped_gemm_nt(tab_gu, H, 2 * I, offsets, kept, rows, rows, 2 * I, H, a=x, a_rows=row_src,
                                  a_row_div=k)
         h = ops.silu_mul(gu[:, :I], gu[:, I:], rows_dev=offsets[-1:])      # only the kept rows
     y = ops.grouped_down(h, tab_d, offsets, kept, rows, H, I)
-    return gu, h, y
+    return gu, h, y, hT, wplan
 
 
-def _ffn_backward(dy, x, wgu, wd, gu, h, offsets, kept, rows, row_src, k, need_x, need_w):
+def _ffn_backward(dy, x, wgu, wd, gu, h, offsets, kept, rows, row_src, k, need_x, need_w, hT=None, wplan=None):
     """Gradients of _ffn_forward: dx_rows [rows, H] (or None), dWgu [E, 2I, H], dWd [E, H, I] (or None).
     dgrad multiplies by per-step transposed copies of the weights; wgrad multiplies the transposed,
-    zero-padded activations of each expert (K = its padded row count)."""
+    zero-padded activations of each expert (K = its padded row count).  h may be None when hT, its transposed
+    copy from the forward kernel, is given; the fused bfloat16 dgrad kernel likewise hands back dgu and its
+    transposed copy, so only dy and the gathered x go through a transposing pass."""
     E = len(wd)
     H, I = x.shape[1], wd[0].shape[1]
     dtype, dev = x.dtype, x.device
+    if need_w and wplan is None:
+        wplan = ops.wgrad_plan(kept)
     wdT, tab_dT = ops.transpose_batched(wd)                      # [I, H] per expert; kept alive until return
-    dgu = ops.grouped_down_dgrad_dsilu(dy, tab_dT, gu, offsets, kept, rows, H, I)   # prefill-sized groups: one kernel
+    dguT = None
+    pair = ops.grouped_down_dgrad_dsilu(dy, tab_dT, gu, offsets, kept, rows, H, I,       # prefill-sized groups:
+                                        t_col0=wplan[0] if need_w and FUSE_TRANSPOSED_COPIES else None)   # one kernel
+    dgu = None
+    if pair is not None:
+        dgu, dguT = pair
     if dgu is None:
         dh = ops.grouped_gemm_nt(tab_dT, H, I, offsets, kept, rows, rows, I, H, a=dy)
         dgu = torch.empty_like(gu)
@@ -228,13 +247,15 @@ def _ffn_backward(dy, x, wgu, wd, gu, h, offsets, kept, rows, row_src, k, need_x
         wguT, tab_guT = ops.transpose_batched(wgu)               # [H, 2I] per expert
         dx_rows = ops.grouped_gemm_nt(tab_guT, 2 * I, H, offsets, kept, rows, rows, H, 2 * I, a=dgu)
     if need_w:
-        ks, kc = ops.wgrad_plan(kept)
+        ks, kc = wplan
         ld = ops.wgrad_padded_rows(rows, E)
         es = x.element_size()
 
-        def wgrad(lhs, rhs, M, N, gather=None):
-            lhsT = ops.transpose_grouped_rows(lhs, offsets, kept, rows)
-            rhsT = ops.transpose_grouped_rows(rhs, offsets, kept, rows, gather=gather, gather_div=k)
+        def wgrad(lhs, rhs, M, N, gather=None, lhsT=None, rhsT=None):
+            if lhsT is None:
+                lhsT = ops.transpose_grouped_rows(lhs, offsets, kept, rows)
+            if rhsT is None:
+                rhsT = ops.transpose_grouped_rows(rhs, offsets, kept, rows, gather=gather, gather_div=k)
             a_ptrs = ks.long() * es + lhsT.data_ptr()
             b_ptrs = ks.long() * es + rhsT.data_ptr()
             rs = torch.arange(E, dtype=torch.int32, device=dev) * M
@@ -243,8 +264,8 @@ def _ffn_backward(dy, x, wgu, wd, gu, h, offsets, kept, rows, row_src, k, need_x
                                     dtype=dtype, out_dtype=dtype)
             return g.view(E, M, N)
 
-        dwd = wgrad(dy, h, H, I)
-        dwgu = wgrad(dgu, x, 2 * I, H, gather=row_src)
+        dwd = wgrad(dy, h, H, I, rhsT=hT)
+        dwgu = wgrad(dgu, x, 2 * I, H, gather=row_src, lhsT=dguT)
     return dx_rows, dwgu, dwd
 
 
@@ -259,18 +280,25 @@ class ExpertFFNFunction(Function):
         n = x.shape[0]
         offsets = torch.tensor([0, n], dtype=torch.int32, device=x.device)
         kept = offsets[1:].clone()
-        gu, h, y = _ffn_forward(x, wgu, wd, offsets, kept, n, None, 1)
-        ctx.save_for_backward(x, offsets, kept, gu, h)
+        gu, h, y, hT, wplan = _ffn_forward(x, wgu, wd, offsets, kept, n, None, 1,
+                                           want_wgrad=ctx.needs_input_grad[1] or ctx.needs_input_grad[2])
+        ctx.h_transposed = hT is not None
+        ctx.has_wplan = wplan is not None
+        ctx.save_for_backward(x, offsets, kept, gu, hT if hT is not None else h, *(wplan or ()))
         ctx.wgu, ctx.wd = wgu, wd
         ctx.param_dtypes = (w_gate_up.dtype, w_down.dtype)
         return y
 
     @staticmethod
     def backward(ctx, dy):
-        x, offsets, kept, gu, h = ctx.saved_tensors
+        x, offsets, kept, gu, h = ctx.saved_tensors[:5]
+        wplan = tuple(ctx.saved_tensors[5:7]) if ctx.has_wplan else None
+        hT = None
+        if ctx.h_transposed:
+            h, hT = None, h
         need_x, need_w = ctx.needs_input_grad[0], ctx.needs_input_grad[1] or ctx.needs_input_grad[2]
         dx, dwgu, dwd = _ffn_backward(dy.to(x.dtype).contiguous(), x, ctx.wgu, ctx.wd, gu, h, offsets, kept,
-                                      x.shape[0], None, 1, need_x, need_w)
+                                      x.shape[0], None, 1, need_x, need_w, hT=hT, wplan=wplan)
         return (dx, dwgu[0].to(ctx.param_dtypes[0]) if need_w else None,
                 dwd[0].to(ctx.param_dtypes[1]) if need_w else None)
 
@@ -306,8 +334,10 @@ class MoEFunction(Function):
             aux = ops.aux_loss_clean_logits(logits, route["hist"], k, cfg["variant"], cfg["load_balancing_weight"])
         plan = ops.dispatch_plan(route["indices"], E, C)
         rows = min(T * k, E * C)
+        hT = wplan = None
         if rows > 0:
-            gu, h, y = _ffn_forward(x, wgu, wd, plan["offsets"], plan["kept"], rows, plan["row_src"], k)
+            gu, h, y, hT, wplan = _ffn_forward(x, wgu, wd, plan["offsets"], plan["kept"], rows, plan["row_src"], k,
+                                               want_wgrad=any(ctx.needs_input_grad[3:]))
         else:
             gu = torch.zeros(1, 2 * I, dtype=dtype, device=x.device)
             h = torch.zeros(1, I, dtype=dtype, device=x.device)
@@ -318,8 +348,11 @@ class MoEFunction(Function):
         ctx.dims = (T, H, I, E, rows)
         ctx.n_weights = len(expert_weights)
         ctx.wgu, ctx.wd = wgu, wd          # dtype copies (or the parameters' own storage); not graph tensors
+        ctx.h_transposed = hT is not None       # then the kernel's transposed copy of h is kept instead of h
+        ctx.has_wplan = wplan is not None
         ctx.save_for_backward(x, wg, logits, logits_route, route["indices"], route["weights"], usage, aux.detach(),
-                              plan["offsets"], plan["kept"], plan["row_src"], plan["row_of"], gu, h, y)
+                              plan["offsets"], plan["kept"], plan["row_src"], plan["row_of"], gu,
+                              hT if hT is not None else h, y, *(wplan or ()))
         ctx.param_dtypes = (gate_weight.dtype, [w.dtype for w in expert_weights])
         if cfg.get("stats") is not None:
             cfg["stats"].update({"logits": logits, "capacity": C, **route, **plan, "aux": aux.detach().reshape(1)})
@@ -327,7 +360,11 @@ class MoEFunction(Function):
 
     @staticmethod
     def backward(ctx, dout, daux):
-        (x, wg, logits, logits_route, idx, w, usage, aux, offsets, kept, row_src, row_of, gu, h, y) = ctx.saved_tensors
+        (x, wg, logits, logits_route, idx, w, usage, aux, offsets, kept, row_src, row_of, gu, h, y) = ctx.saved_tensors[:15]
+        wplan = tuple(ctx.saved_tensors[15:17]) if ctx.has_wplan else None
+        hT = None
+        if ctx.h_transposed:
+            h, hT = None, h
         T, H, I, E, rows = ctx.dims
         k = ctx.cfg["top_k"]
         dtype = x.dtype
@@ -340,7 +377,7 @@ class MoEFunction(Function):
         if rows > 0:
             dy, dw = ops.combine_bwd(dout, y, row_src, w, k)
             dx_rows, dwgu, dwd = _ffn_backward(dy, x, ctx.wgu, ctx.wd, gu, h, offsets, kept, rows, row_src, k, need_x,
-                                               need_w)
+                                               need_w, hT=hT, wplan=wplan)
             if need_x:
                 ones = torch.ones(T, k, dtype=torch.float32, device=dev)
                 dx = ops.combine(dx_rows, row_of, ones, T, k, out_dtype=dtype)

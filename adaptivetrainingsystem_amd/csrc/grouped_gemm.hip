@@ -65,6 +65,13 @@ struct GroupedArgs {
     // forward instance, read by the instance whose epilogue turns dh into the gradients of g and u
     void* gu_out;
     int64_t ld_gu;
+    // training, bf16 instances of the direct-to-LDS kernel, optional: the tile's result also goes, transposed,
+    // into t_out[column, t_col0[group] + row inside the group] (row stride ld_t elements), zero in the columns
+    // between a group's last row and the next multiple of 64: the layout that the weight-gradient product
+    // contracts over (see ats_wgrad_plan), so that no transposing pass over the activations is needed
+    void* t_out;
+    int64_t ld_t;
+    const int32_t* t_col0;
 };
 
 constexpr int kRowPitch = 144;  // bytes per staged row: 128 data + 16 pad
@@ -135,10 +142,28 @@ struct AccView16 {
 // the 16 bytes of g and of u that belong to its 16 bytes of dh (rounded to TO first, as a stored dh would be) from
 // gu and stores dg = dh * u * (s + g*s*(1-s)) and du = dh * g * s, s = sigmoid(g), to out[row, col] and
 // out[row, up_off + col]: the arithmetic of the elementwise gradient kernel, so the bits are the same.
+// tout (SAVEGU or DSILU, 16-bit TO, optional): the same values once more, transposed, for the weight-gradient
+// product: tout[col, tcol + row] for the wave's rows, zeros from the group's last row to the next multiple of 64
+// (tcol: the wave's first row inside the group + the group's first column; ldt: row stride).  The values are
+// staged in a second wave-private LDS region, tstage, with rows along the fast axis:
+//   SAVEGU: the accumulator layout already has 16 lanes on 16 consecutive rows, so h goes from the registers
+//     into [32 columns][128 rows] (pitch 272 bytes: the lanes of a write land on 64 different banks) and
+//     leaves as 256-byte row segments after the last 32-row block;
+//   DSILU: dg and du exist only in the row-major phase (a lane holds 8 columns of one row), so every 32-row
+//     block goes into [2][64 columns][32 rows] (pitch 80 bytes, the 16-byte row chunk XORed with bits of the
+//     column so that the lanes of a write land on 64 different banks) and leaves as 64-byte segments.
+// In both, two lanes that hold neighbouring rows first exchange half of their values (one DPP move per word), so
+// that every LDS write is a whole word holding rows m and m + 1 of one column.
+constexpr int kTransPitchH = 128 * 2 + 16;
+constexpr int kTransPitchD = 32 * 2 + 16;
+constexpr int kTransStageH = 32 * kTransPitchH;         // bytes per wave, SAVEGU
+constexpr int kTransStageD = 2 * 64 * kTransPitchD;     // bytes per wave, DSILU
 template <typename TO, typename View, bool SWIGLU, bool SAVEGU = false, bool DSILU = false>
 __device__ __forceinline__ void epilogue_view(const View av, unsigned char* wstage, TO* out, int64_t ldo,
                                               int64_t row_base, int rows_valid, int ncol0, int n_out, int lane,
-                                              TO* gu = nullptr, int64_t ldgu = 0, int up_off = 0) {
+                                              TO* gu = nullptr, int64_t ldgu = 0, int up_off = 0,
+                                              TO* tout = nullptr, int64_t ldt = 0, int64_t tcol = 0,
+                                              unsigned char* tstage = nullptr) {
     static_assert(!SAVEGU || SWIGLU, "the second output exists for the SwiGLU epilogue only");
     static_assert(!DSILU || !SWIGLU, "the SwiGLU gradient epilogue belongs to the plain product");
     constexpr int WCOLS = View::kCols;
@@ -147,6 +172,10 @@ __device__ __forceinline__ void epilogue_view(const View av, unsigned char* wsta
     constexpr int LPR = WCOLS * ES / 16;   // lanes per output row
     constexpr int RPI = 64 / LPR;          // rows per store instruction
     constexpr int EPC = 16 / ES;           // elements per 16-byte chunk
+    constexpr bool kTrans = (SAVEGU || DSILU) && ES == 2 && View::kBlocks * 32 == 128;
+    // rows of the wave that the transposed copy covers: the valid ones and the zero columns after them
+    const int t_rows = !kTrans || tout == nullptr || rows_valid <= 0 ? 0
+                       : (rows_valid >= 128 ? 128 : (rows_valid + 63) / 64 * 64);
 #pragma unroll
     for (int i = 0; i < View::kBlocks; ++i) {
 #pragma unroll
@@ -163,6 +192,21 @@ __device__ __forceinline__ void epilogue_view(const View av, unsigned char* wsta
                 u.x = pack_bf16x2(v[0], v[1]);
                 u.y = pack_bf16x2(v[2], v[3]);
                 *reinterpret_cast<uint2*>(dst) = u;
+                if constexpr (kTrans && SAVEGU) {
+                    if (t_rows > 0) {
+                        // Neighbouring lanes hold neighbouring rows: the even lane takes its neighbour's first two
+                        // columns, the odd lane its neighbour's last two, and each writes two whole words (rows m,
+                        // m + 1 of one column).
+                        const bool odd = (lane & 1) != 0;
+                        const uint32_t rcv = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(odd ? u.x : u.y), 0xB1, 0xf, 0xf, false);
+                        const int m_even = i * 32 + (View::row(g, lane) & ~1);
+                        const uint32_t lo = m_even < rows_valid ? (odd ? rcv : u.x) : 0u;
+                        const uint32_t hi = m_even + 1 < rows_valid ? (odd ? u.y : rcv) : 0u;
+                        unsigned char* td = tstage + (View::col(g, lane) + (odd ? 2 : 0)) * kTransPitchH + m_even * 2;
+                        *reinterpret_cast<uint32_t*>(td) = (lo & 0xffffu) | (hi << 16);
+                        *reinterpret_cast<uint32_t*>(td + kTransPitchH) = (lo >> 16) | (hi & 0xffff0000u);
+                    }
+                }
             } else {
                 *reinterpret_cast<float4*>(dst) = make_float4(v[0], v[1], v[2], v[3]);
             }
@@ -176,6 +220,7 @@ __device__ __forceinline__ void epilogue_view(const View av, unsigned char* wsta
             const int m_local = i * 32 + r;
             const int col = ncol0 + c * EPC;
             if constexpr (DSILU) {
+                uint4 pg = make_uint4(0u, 0u, 0u, 0u), pu = make_uint4(0u, 0u, 0u, 0u);
                 if (m_local < rows_valid && col < n_out) {
                     const TO* gp = gu + (row_base + m_local) * ldgu + col;
                     TO* dp = out + (row_base + m_local) * ldo + col;
@@ -189,8 +234,36 @@ __device__ __forceinline__ void epilogue_view(const View av, unsigned char* wsta
                         og[e] = dv[e] * uv[e] * (sg + gv[e] * sg * (1.0f - sg));
                         ou[e] = dv[e] * (gv[e] * sg);
                     }
-                    *reinterpret_cast<uint4*>(dp) = Elem<TO>::pack(og);
-                    *reinterpret_cast<uint4*>(dp + up_off) = Elem<TO>::pack(ou);
+                    pg = Elem<TO>::pack(og);
+                    pu = Elem<TO>::pack(ou);
+                    *reinterpret_cast<uint4*>(dp) = pg;
+                    *reinterpret_cast<uint4*>(dp + up_off) = pu;
+                }
+                if constexpr (kTrans) {
+                    if (i * 32 < t_rows) {
+                        // rows past the group's end were left at zero above: they are the zero columns.
+                        // Lanes 8 apart hold neighbouring rows of the same 8 columns: the lane of the even row takes
+                        // its neighbour's first four columns, the other its neighbour's last four, and each writes
+                        // whole words (rows m, m + 1 of one column).
+                        const bool odd = (r & 1) != 0;
+                        constexpr int kRor8 = 0x128;     // DPP row_ror:8, lane ^ 8 inside a row of 16 lanes
+                        const uint32_t rg0 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(odd ? pg.x : pg.z), kRor8, 0xf, 0xf, false);
+                        const uint32_t rg1 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(odd ? pg.y : pg.w), kRor8, 0xf, 0xf, false);
+                        const uint32_t ru0 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(odd ? pu.x : pu.z), kRor8, 0xf, 0xf, false);
+                        const uint32_t ru1 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(odd ? pu.y : pu.w), kRor8, 0xf, 0xf, false);
+                        const uint32_t lo[2][2] = {{odd ? rg0 : pg.x, odd ? rg1 : pg.y}, {odd ? ru0 : pu.x, odd ? ru1 : pu.y}};
+                        const uint32_t hi[2][2] = {{odd ? pg.z : rg0, odd ? pg.w : rg1}, {odd ? pu.z : ru0, odd ? pu.w : ru1}};
+                        const int nb = c * 8 + (odd ? 4 : 0);
+                        unsigned char* td = tstage + nb * kTransPitchD + (((r >> 3) ^ ((c >> 1) & 3)) * 16) + ((r & 7) >> 1) * 4;
+#pragma unroll
+                        for (int half = 0; half < 2; ++half)
+#pragma unroll
+                            for (int w2 = 0; w2 < 2; ++w2) {
+                                unsigned char* t2 = td + (half * 64 + 2 * w2) * kTransPitchD;
+                                *reinterpret_cast<uint32_t*>(t2) = (lo[half][w2] & 0xffffu) | (hi[half][w2] << 16);
+                                *reinterpret_cast<uint32_t*>(t2 + kTransPitchD) = (lo[half][w2] >> 16) | (hi[half][w2] & 0xffff0000u);
+                            }
+                    }
                 }
             } else {
                 if (m_local < rows_valid && col < n_out)
@@ -198,6 +271,22 @@ __device__ __forceinline__ void epilogue_view(const View av, unsigned char* wsta
             }
         }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        if constexpr (kTrans && DSILU) {
+            if (i * 32 < t_rows) {
+#pragma unroll
+                for (int it = 0; it < 8; ++it) {
+                    const int idx = it * 64 + lane;
+                    const int rowid = idx >> 2, j = idx & 3;          // 128 staged rows (dg 0..63, du 64..127) x 4 chunks
+                    const int n_l = rowid & 63, half = rowid >> 6;
+                    const u32x4_t data = *reinterpret_cast<const u32x4_t*>(
+                        tstage + rowid * kTransPitchD + ((j ^ ((n_l >> 4) & 3)) * 16));
+                    const int m0 = i * 32 + j * 8;
+                    if (m0 < t_rows && ncol0 + n_l < n_out)
+                        *reinterpret_cast<u32x4_t*>(tout + (int64_t)(half * up_off + ncol0 + n_l) * ldt + tcol + m0) = data;
+                }
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            }
+        }
         if constexpr (SAVEGU) {
 #pragma unroll
             for (int half = 0; half < 2; ++half) {
@@ -226,6 +315,18 @@ __device__ __forceinline__ void epilogue_view(const View av, unsigned char* wsta
                         *reinterpret_cast<u32x4_t*>(gu + (row_base + m_local) * ldgu + half * up_off + col) = data;
                 }
                 asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            }
+        }
+    }
+    if constexpr (kTrans && SAVEGU) {
+        if (t_rows > 0) {
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+            for (int r0 = 0; r0 < 32; r0 += 4) {
+                const int n_l = r0 + (lane >> 4), ch = lane & 15;
+                const u32x4_t data = *reinterpret_cast<const u32x4_t*>(tstage + n_l * kTransPitchH + ch * 16);
+                if (ch * 8 < t_rows && ncol0 + n_l < n_out)
+                    *reinterpret_cast<u32x4_t*>(tout + (int64_t)(ncol0 + n_l) * ldt + tcol + ch * 8) = data;
             }
         }
     }
@@ -1180,9 +1281,20 @@ __global__ __launch_bounds__(512) void grouped_gemm_dma16_kernel(GroupedArgs p) 
         constexpr int WSTAGE = 32 * (View::kCols * (int)sizeof(TO) + 16);
         const int wrow = tc.mt * BM + wm * (BM / WM);
         const int ncol0 = SWIGLU ? tc.nt * HALF + wn * (BN / WN / 2) : tc.nt * BN + wn * (BN / WN);
-        epilogue_view<TO, View, SWIGLU, SAVEGU, DSILU>(View{acc}, smem + wave * WSTAGE, static_cast<TO*>(p.out), p.ldo,
-                                                       (int64_t)row0 + wrow, count - wrow, ncol0, p.N_out, lane,
-                                                       static_cast<TO*>(p.gu_out), p.ld_gu, p.up_offset);
+        if constexpr (SAVEGU || DSILU) {
+            constexpr int TSTAGE = SAVEGU ? kTransStageH : kTransStageD;
+            static_assert(NW * (WSTAGE + TSTAGE) <= (3 * BM + 2 * BN) * 128, "epilogue staging exceeds the tile's LDS");
+            TO* tout = static_cast<TO*>(p.t_out);
+            const int64_t tcol = tout ? (int64_t)p.t_col0[tc.e] + wrow : 0;
+            epilogue_view<TO, View, SWIGLU, SAVEGU, DSILU>(View{acc}, smem + wave * WSTAGE, static_cast<TO*>(p.out), p.ldo,
+                                                           (int64_t)row0 + wrow, count - wrow, ncol0, p.N_out, lane,
+                                                           static_cast<TO*>(p.gu_out), p.ld_gu, p.up_offset, tout,
+                                                           p.ld_t, tcol, smem + NW * WSTAGE + wave * TSTAGE);
+        } else {
+            epilogue_view<TO, View, SWIGLU, SAVEGU, DSILU>(View{acc}, smem + wave * WSTAGE, static_cast<TO*>(p.out), p.ldo,
+                                                           (int64_t)row0 + wrow, count - wrow, ncol0, p.N_out, lane,
+                                                           static_cast<TO*>(p.gu_out), p.ld_gu, p.up_offset);
+        }
     }
 #endif
 }
@@ -1405,12 +1517,28 @@ extern "C" int ats_grouped_gateup_swiglu_save_supported(int64_t a_num_rows, int 
     return 0;
 }
 
+// The optional transposed copy of a training launch: bf16 only, a 16-byte aligned buffer whose row stride holds
+// every group's padded columns (ats_wgrad_padded_rows), and the groups' first columns from ats_wgrad_plan.
+static int check_transposed(const char* name, const void* t_out, int64_t ld_t, const int32_t* t_col0, int64_t max_rows,
+                            int E, int dtype) {
+    if (!t_out) return ATS_OK;
+    ATS_REQUIRE(dtype == ATS_BF16, ATS_ERR_UNSUPPORTED, "%s: the transposed copy is written for bfloat16 only", name);
+    ATS_REQUIRE(t_col0 && ats::aligned16(t_out) && ld_t % 64 == 0 && ld_t >= ats_wgrad_padded_rows(max_rows, E),
+                ATS_ERR_INVALID_ARG, "%s: transposed copy needs the groups' first columns, a 16-byte aligned buffer and "
+                "a row stride that is a multiple of 64 and at least %lld (got %lld)", name,
+                (long long)ats_wgrad_padded_rows(max_rows, E), (long long)ld_t);
+    return ATS_OK;
+}
+
 extern "C" int ats_grouped_gateup_swiglu_save(const void* a, int64_t a_num_rows, const int32_t* a_rows, int a_row_div,
                                               const void* const* w_gu, void* h, void* gu, const int32_t* row_start,
                                               const int32_t* row_count, int E, int64_t max_rows, int H, int I,
-                                              int dtype, ats_stream_t stream) {
+                                              int dtype, void* h_t, int64_t ld_t, const int32_t* t_col0,
+                                              ats_stream_t stream) {
     using namespace ats;
     int rc = check_common("ats_grouped_gateup_swiglu_save", a, w_gu, h, row_start, row_count, E, max_rows, H, I, dtype);
+    if (rc != ATS_OK) return rc;
+    rc = check_transposed("ats_grouped_gateup_swiglu_save", h_t, ld_t, t_col0, max_rows, E, dtype);
     if (rc != ATS_OK) return rc;
     ATS_REQUIRE(gu && aligned16(gu), ATS_ERR_INVALID_ARG, "ats_grouped_gateup_swiglu_save: gu must be a 16-byte aligned buffer");
     ATS_REQUIRE(a_num_rows > 0 && (!a_rows || a_row_div > 0), ATS_ERR_INVALID_ARG,
@@ -1430,6 +1558,9 @@ extern "C" int ats_grouped_gateup_swiglu_save(const void* a, int64_t a_num_rows,
     p.ldo = I;
     p.gu_out = gu;
     p.ld_gu = 2 * (int64_t)I;
+    p.t_out = h_t;
+    p.ld_t = ld_t;
+    p.t_col0 = t_col0;
     p.row_start = row_start;
     p.row_count = row_count;
     p.E = E;
@@ -1456,9 +1587,12 @@ extern "C" int ats_grouped_down_dgrad_dsilu_supported(int E, int64_t max_rows, i
 
 extern "C" int ats_grouped_down_dgrad_dsilu(const void* dy, const void* const* w_dT, const void* gu, void* dgu,
                                             const int32_t* row_start, const int32_t* row_count, int E,
-                                            int64_t max_rows, int H, int I, int dtype, ats_stream_t stream) {
+                                            int64_t max_rows, int H, int I, int dtype, void* dgu_t, int64_t ld_t,
+                                            const int32_t* t_col0, ats_stream_t stream) {
     using namespace ats;
     int rc = check_common("ats_grouped_down_dgrad_dsilu", dy, w_dT, dgu, row_start, row_count, E, max_rows, H, I, dtype);
+    if (rc != ATS_OK) return rc;
+    rc = check_transposed("ats_grouped_down_dgrad_dsilu", dgu_t, ld_t, t_col0, max_rows, E, dtype);
     if (rc != ATS_OK) return rc;
     ATS_REQUIRE(gu && aligned16(gu), ATS_ERR_INVALID_ARG, "ats_grouped_down_dgrad_dsilu: gu must be a 16-byte aligned buffer");
     ATS_REQUIRE(ats_grouped_down_dgrad_dsilu_supported(E, max_rows, H, I, dtype), ATS_ERR_UNSUPPORTED,
@@ -1476,6 +1610,9 @@ extern "C" int ats_grouped_down_dgrad_dsilu(const void* dy, const void* const* w
     p.ldo = 2 * (int64_t)I;
     p.gu_out = const_cast<void*>(gu);
     p.ld_gu = 2 * (int64_t)I;
+    p.t_out = dgu_t;
+    p.ld_t = ld_t;
+    p.t_col0 = t_col0;
     p.row_start = row_start;
     p.row_count = row_count;
     p.E = E;

@@ -124,7 +124,44 @@ __global__ __launch_bounds__(256) void transpose_grouped_kernel(const T* __restr
                       out + (int64_t)c0 * ld_out + kstart + i0, ld_out, kTile, tile, vec);
 }
 
+// The 64 columns of every group without rows, zeroed (the kernels that write a transposed copy from their
+// epilogue never visit such a group).  grid.x: groups, grid.y: blocks of 32 rows of the transposed matrix.
+template <typename T>
+__global__ __launch_bounds__(256) void zero_empty_groups_kernel(T* __restrict__ out, int64_t ld, int C,
+                                                                const int32_t* __restrict__ row_count,
+                                                                const int32_t* __restrict__ k_start) {
+    const int e = blockIdx.x;
+    if (row_count[e] > 0) return;
+    constexpr int V = Elem<T>::kVec;               // elements per 16 bytes
+    constexpr int LPR = kKPad / V;                 // lanes per row of 64 zero columns
+    const int c = blockIdx.y * (256 / LPR) + (int)threadIdx.x / LPR;
+    if (c >= C) return;
+    T* dst = out + (int64_t)c * ld + k_start[e] + ((int)threadIdx.x % LPR) * V;
+    *reinterpret_cast<uint4*>(dst) = make_uint4(0u, 0u, 0u, 0u);
+}
+
 }  // namespace ats
+
+extern "C" int ats_transposed_zero_empty_groups(void* out, int64_t ld, int C, const int32_t* row_count,
+                                                const int32_t* k_start, int E, int dtype, ats_stream_t stream) {
+    using namespace ats;
+    ATS_REQUIRE(E > 0 && C > 0 && out && row_count && k_start && ld % kKPad == 0 && aligned16(out), ATS_ERR_INVALID_ARG,
+                "ats_transposed_zero_empty_groups: E=%d C=%d ld=%lld (a multiple of %d, 16-byte aligned buffer)", E, C,
+                (long long)ld, kKPad);
+    ATS_REQUIRE(dtype == ATS_F32 || dtype == ATS_BF16, ATS_ERR_UNSUPPORTED,
+                "ats_transposed_zero_empty_groups: dtype tag %d", dtype);
+    const int rows_per_block = dtype == ATS_F32 ? 256 / (kKPad / 4) : 256 / (kKPad / 8);
+    const dim3 grid((unsigned)E, (unsigned)((C + rows_per_block - 1) / rows_per_block));
+    ATS_REQUIRE(grid.y <= 65535, ATS_ERR_UNSUPPORTED, "ats_transposed_zero_empty_groups: grid");
+    if (dtype == ATS_F32)
+        hipLaunchKernelGGL((zero_empty_groups_kernel<float>), grid, dim3(256), 0, as_stream(stream),
+                           static_cast<float*>(out), ld, C, row_count, k_start);
+    else
+        hipLaunchKernelGGL((zero_empty_groups_kernel<bf16_t>), grid, dim3(256), 0, as_stream(stream),
+                           static_cast<bf16_t*>(out), ld, C, row_count, k_start);
+    ATS_CHECK_LAUNCH("ats_transposed_zero_empty_groups");
+    return ATS_OK;
+}
 
 extern "C" int ats_transpose_batched(const void* const* in_ptrs, void* const* out_ptrs, int E, int R, int C, int dtype,
                                      int aligned_bases, ats_stream_t stream) {

@@ -305,10 +305,13 @@ def grouped_gateup_swiglu(a: torch.Tensor, w_gu_ptrs: torch.Tensor, row_start: t
 
 def grouped_gateup_swiglu_save(a: torch.Tensor, w_gu_ptrs: torch.Tensor, row_start: torch.Tensor,
                                row_count: torch.Tensor, n_rows_out: int, max_rows: int, H: int, I: int,
-                               a_rows: Optional[torch.Tensor] = None,
-                               a_row_div: int = 1) -> Optional[Tuple[torch.Tensor, torch.Tensor]]:
-    """Training forward of the gate/up projection: (gu [rows, 2I], h [rows, I]) from one kernel, or None when
-    the sizes are not prefill-sized (the caller then runs the plain product and silu_mul)."""
+                               a_rows: Optional[torch.Tensor] = None, a_row_div: int = 1,
+                               t_col0: Optional[torch.Tensor] = None
+                               ) -> Optional[Tuple[torch.Tensor, torch.Tensor, Optional[torch.Tensor]]]:
+    """Training forward of the gate/up projection: (gu [rows, 2I], h [rows, I], hT) from one kernel, or None when
+    the sizes are not prefill-sized (the caller then runs the plain product and silu_mul).  hT is None unless
+    t_col0 (the k_start of wgrad_plan) is given and the dtype is bfloat16: then it is h transposed into the
+    weight-gradient layout [I, wgrad_padded_rows] (see transpose_grouped_rows), written by the same kernel."""
     _need_gpu(a, w_gu_ptrs, row_start, row_count, a_rows)
     if a.dim() != 2 or a.shape[1] != H or not a.is_contiguous():
         raise AtsError("grouped_gateup_swiglu_save: activations must be a contiguous [rows, H] tensor")
@@ -320,18 +323,40 @@ def grouped_gateup_swiglu_save(a: torch.Tensor, w_gu_ptrs: torch.Tensor, row_sta
         return None
     h = torch.empty(n_rows_out, I, dtype=a.dtype, device=a.device)
     gu = torch.empty(n_rows_out, 2 * I, dtype=a.dtype, device=a.device)
+    hT, ld = _transposed_copy_buffer(I, row_count, t_col0, max_rows, E, a.dtype, a.device)
     check(lib.ats_grouped_gateup_swiglu_save(a.data_ptr(), int(a.shape[0]), _ptr(a_rows), int(a_row_div),
                                              w_gu_ptrs.data_ptr(), h.data_ptr(), gu.data_ptr(), row_start.data_ptr(),
-                                             row_count.data_ptr(), E, int(max_rows), H, I, _tag(a), _stream()),
+                                             row_count.data_ptr(), E, int(max_rows), H, I, _tag(a), _ptr(hT), ld,
+                                             _ptr(t_col0) if hT is not None else None, _stream()),
           "ats_grouped_gateup_swiglu_save")
-    return gu, h
+    return gu, h, hT
+
+
+def _transposed_copy_buffer(C: int, row_count: torch.Tensor, t_col0: Optional[torch.Tensor], max_rows: int, E: int,
+                            dtype: torch.dtype, device) -> Tuple[Optional[torch.Tensor], int]:
+    """The [C, padded rows] buffer that a training launch fills with the transposed copy of its result (bfloat16
+    launches with the experts' first columns given), the columns of experts without rows already cleared."""
+    if t_col0 is None or dtype != torch.bfloat16:
+        return None, 0
+    _need_gpu(t_col0)
+    if t_col0.dtype != torch.int32 or t_col0.numel() < E:
+        raise AtsError("transposed copy: t_col0 must be int32 with one entry per expert")
+    ld = wgrad_padded_rows(max_rows, E)
+    out = torch.empty(C, ld, dtype=dtype, device=device)
+    check(_lib.load().ats_transposed_zero_empty_groups(out.data_ptr(), ld, C, row_count.data_ptr(), t_col0.data_ptr(), E,
+                                                       _tag(out), _stream()), "ats_transposed_zero_empty_groups")
+    return out, ld
 
 
 def grouped_down_dgrad_dsilu(dy: torch.Tensor, w_dT_ptrs: torch.Tensor, gu: torch.Tensor, row_start: torch.Tensor,
-                             row_count: torch.Tensor, max_rows: int, H: int, I: int) -> Optional[torch.Tensor]:
-    """Training backward of the down projection and of silu(g) * u in one kernel: dgu [rows, 2I] from dy [rows, H],
-    the transposed down weights ([I, H] per expert) and the saved gu; None when the groups are not prefill-sized
-    (the caller then runs the plain product and silu_mul_bwd)."""
+                             row_count: torch.Tensor, max_rows: int, H: int, I: int,
+                             t_col0: Optional[torch.Tensor] = None
+                             ) -> Optional[Tuple[torch.Tensor, Optional[torch.Tensor]]]:
+    """Training backward of the down projection and of silu(g) * u in one kernel: (dgu [rows, 2I], dguT) from
+    dy [rows, H], the transposed down weights ([I, H] per expert) and the saved gu; None when the groups are not
+    prefill-sized (the caller then runs the plain product and silu_mul_bwd).  dguT is None unless t_col0 (the
+    k_start of wgrad_plan) is given and the dtype is bfloat16: then it is dgu transposed into the weight-gradient
+    layout [2I, wgrad_padded_rows], written by the same kernel."""
     _need_gpu(dy, w_dT_ptrs, gu, row_start, row_count)
     if dy.dim() != 2 or dy.shape[1] != H or not dy.is_contiguous():
         raise AtsError("grouped_down_dgrad_dsilu: dy must be a contiguous [rows, H] tensor")
@@ -344,10 +369,12 @@ def grouped_down_dgrad_dsilu(dy: torch.Tensor, w_dT_ptrs: torch.Tensor, gu: torc
     if not lib.ats_grouped_down_dgrad_dsilu_supported(E, int(max_rows), H, I, _tag(dy)):
         return None
     dgu = torch.empty_like(gu)
+    dguT, ld = _transposed_copy_buffer(2 * I, row_count, t_col0, max_rows, E, dy.dtype, dy.device)
     check(lib.ats_grouped_down_dgrad_dsilu(dy.data_ptr(), w_dT_ptrs.data_ptr(), gu.data_ptr(), dgu.data_ptr(),
                                            row_start.data_ptr(), row_count.data_ptr(), E, int(max_rows), H, I,
-                                           _tag(dy), _stream()), "ats_grouped_down_dgrad_dsilu")
-    return dgu
+                                           _tag(dy), _ptr(dguT), ld, _ptr(t_col0) if dguT is not None else None,
+                                           _stream()), "ats_grouped_down_dgrad_dsilu")
+    return dgu, dguT
 
 
 def grouped_down(h: torch.Tensor, w_d_ptrs: torch.Tensor, row_start: torch.Tensor, row_count: torch.Tensor,

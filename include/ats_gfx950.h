@@ -183,11 +183,19 @@ int ats_grouped_down(const void* h, const void* const* w_d, void* y, const int32
  * gu [rows, 2I]; dh itself is never stored.  Same bits as ats_grouped_gemm_nt followed by
  * ats_silu_mul_bwd (reference: SwiGLUFunction.backward, MS/core/cuda_opt_wrapper.py:237-254, after
  * autograd's down_proj gradient).  ..._supported returns 1 for more than 256 rows per expert on
- * average, H a multiple of the 128-byte K slab and one expert's weights within 4 GiB. */
+ * average, H a multiple of the 128-byte K slab and one expert's weights within 4 GiB.
+ * dgu_t (optional, bfloat16 only; also h_t of ats_grouped_gateup_swiglu_save): the result once more,
+ * transposed, in the layout of ats_transpose_grouped_rows -- dgu_t[c, t_col0[e] + m] for row m of
+ * expert e, zeros up to the next multiple of 64 columns, row stride ld_t >= ats_wgrad_padded_rows,
+ * t_col0 = the k_start of ats_wgrad_plan -- written from the same registers, so that the weight
+ * gradient (autograd's dW = dY^T . X for nn.Linear, MS/core/model.py:882-893) needs no transposing
+ * pass over this operand.  The columns of experts without rows are not written
+ * (ats_transposed_zero_empty_groups clears them). */
 int ats_grouped_down_dgrad_dsilu_supported(int E, int64_t max_rows, int H, int I, int dtype);
 int ats_grouped_down_dgrad_dsilu(const void* dy, const void* const* w_dT, const void* gu, void* dgu,
                                  const int32_t* row_start, const int32_t* row_count, int E, int64_t max_rows,
-                                 int H, int I, int dtype, ats_stream_t stream);
+                                 int H, int I, int dtype, void* dgu_t, int64_t ld_t, const int32_t* t_col0,
+                                 ats_stream_t stream);
 /* The same projection for a training step: beside h it writes the gate / up pre-activations
  * gu[r, 0:I] and gu[r, I:2I] ([rows, 2I] of dtype, rounded from the same accumulators), which the
  * backward pass needs; replaces the plain product followed by ats_silu_mul_fwd (reference: the
@@ -200,7 +208,8 @@ int ats_grouped_gateup_swiglu_save_supported(int64_t a_num_rows, int E, int64_t 
 int ats_grouped_gateup_swiglu_save(const void* a, int64_t a_num_rows, const int32_t* a_rows, int a_row_div,
                                    const void* const* w_gu, void* h, void* gu, const int32_t* row_start,
                                    const int32_t* row_count, int E, int64_t max_rows, int H, int I,
-                                   int dtype, ats_stream_t stream);
+                                   int dtype, void* h_t, int64_t ld_t, const int32_t* t_col0,
+                                   ats_stream_t stream);
 /* The down projection of weight-streaming (decode) sizes, at most 256 rows per expert, split along
  * K so that enough workgroups stream the weights: slice s of expert e multiplies columns
  * [s*I/k_splits, (s+1)*I/k_splits) and writes float32 parts[s][row_start[e]+m][:H]
@@ -357,6 +366,9 @@ int ats_wgrad_plan(const int32_t* row_count, int E, int32_t* k_start, int32_t* k
 int ats_transpose_grouped_rows(const void* in, int64_t ld_in, int C, const int32_t* gather, int gather_div,
                                const int32_t* row_start, const int32_t* row_count, int E, int64_t max_rows,
                                void* out, int64_t ld_out, int dtype, ats_stream_t stream);
+/* Clears the 64 columns that every expert without rows owns in a transposed matrix [C, ld] of that layout. */
+int ats_transposed_zero_empty_groups(void* out, int64_t ld, int C, const int32_t* row_count,
+                                     const int32_t* k_start, int E, int dtype, ats_stream_t stream);
 /* General grouped product with K contiguous in both operands:
  * out[row_start[e]+m, n] = sum_k A_e[m,k] * B_e[n,k], m < row_count[e], n < N.
  * A_e = rows row_start[e].. of `a` (optionally gathered through a_rows), or a_ptrs[e] with rows

@@ -967,7 +967,7 @@ def test_moe_decode_step_replays_in_a_hip_graph(A, gpu):
 
 
 @pytest.mark.parametrize("counts,H,I,gather", [([900, 0, 1300, 1001], 256, 392, True), ([2100, 777], 512, 1024, False),
-                                               ([800], 128, 136, True)])
+                                               ([800], 128, 136, True), ([1100, 1, 2303, 64, 0, 1216], 128, 200, False)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_grouped_gateup_with_saved_preactivations(ops, gpu, counts, H, I, gather, dtype):
     """Training forward of the gate/up projection in one kernel: h has the bits of the inference kernel, the
@@ -992,10 +992,23 @@ def test_grouped_gateup_with_saved_preactivations(ops, gpu, counts, H, I, gather
     else:
         a, kw = rows.to(gpu), {}
     start, count = start.to(gpu), count.to(gpu)
-    both = ops.grouped_gateup_swiglu_save(a, tab, start, count, n + pad, n, H, I, **kw)
+    ks, kc = ops.wgrad_plan(count)
+    both = ops.grouped_gateup_swiglu_save(a, tab, start, count, n + pad, n, H, I, t_col0=ks, **kw)
     assert both is not None
-    gu, h = both
+    gu, h, hT = both
     assert gu.shape == (n + pad, 2 * I) and h.shape == (n + pad, I) and gu.dtype == dtype and h.dtype == dtype
+    # the transposed copy for the weight gradient: bfloat16 launches write it, with the bits of h and zero padding
+    assert (hT is not None) == (dtype == torch.bfloat16)
+    if hT is not None:
+        want = ops.transpose_grouped_rows(h[:n], start, count, n)
+        assert hT.shape == want.shape
+        for e, c in enumerate(counts):
+            lo, width = int(ks[e]), int(kc[e])
+            assert width == max(64, (c + 63) // 64 * 64)
+            assert same_bits(hT[:, lo:lo + width], want[:, lo:lo + width]), e
+            assert torch.all(hT[:, lo + c:lo + width] == 0)
+        plain = ops.grouped_gateup_swiglu_save(a, tab, start, count, n + pad, n, H, I, **kw)
+        assert plain[2] is None and same_bits(plain[1][:n], h[:n]) and same_bits(plain[0][:n], gu[:n])
     h_inf = ops.grouped_gateup_swiglu(a, tab, start, count, n + pad, n, H, I, **kw)
     assert same_bits(h[:n], h_inf[:n])
     gu_plain = ops.grouped_gemm_nt(tab, H, 2 * I, start, count, n + pad, n, 2 * I, H, a=a, **kw)
@@ -1016,7 +1029,7 @@ def test_grouped_gateup_with_saved_preactivations(ops, gpu, counts, H, I, gather
     rc = lib.ats_grouped_gateup_swiglu_save(a.data_ptr(), a.shape[0], kw["a_rows"].data_ptr() if gather else None,
                                             kw.get("a_row_div", 1), tab.data_ptr(), h.data_ptr(), gu.data_ptr(),
                                             start.data_ptr(), count.data_ptr(), E, n, H, I,
-                                            0 if dtype == torch.float32 else 1, None)
+                                            0 if dtype == torch.float32 else 1, None, 0, None, None)
     assert rc == 0
     torch.cuda.synchronize()
     assert torch.all(gu[n:] == 3.0) and torch.all(h[n:] == 5.0)
@@ -1026,7 +1039,8 @@ def test_grouped_gateup_with_saved_preactivations(ops, gpu, counts, H, I, gather
     assert ops.grouped_gateup_swiglu_save(a, tab, start, small, n, 40 * E, H, I, **kw) is None
 
 
-@pytest.mark.parametrize("counts,H,I", [([900, 0, 300, 1001], 256, 392), ([2100, 777], 512, 1024), ([300], 128, 136)])
+@pytest.mark.parametrize("counts,H,I", [([900, 0, 300, 1001], 256, 392), ([2100, 777], 512, 1024), ([300], 128, 136),
+                                        ([1024, 1, 1279, 64, 0, 193], 128, 200)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_grouped_down_dgrad_with_swiglu_gradient(ops, gpu, counts, H, I, dtype):
     """Training backward in one kernel: dgu has the bits of the plain product dh = dy . Wd followed by the
@@ -1043,8 +1057,21 @@ def test_grouped_down_dgrad_with_swiglu_gradient(ops, gpu, counts, H, I, dtype):
     pad = 5
     dy = torch.randn(n + pad, H, generator=g).to(dtype).to(gpu)
     gu = torch.randn(n + pad, 2 * I, generator=g).to(dtype).to(gpu)
-    dgu = ops.grouped_down_dgrad_dsilu(dy, tab, gu, start, count, n, H, I)
-    assert dgu is not None and dgu.shape == gu.shape and dgu.dtype == dtype
+    ks, kc = ops.wgrad_plan(count)
+    pair = ops.grouped_down_dgrad_dsilu(dy, tab, gu, start, count, n, H, I, t_col0=ks)
+    assert pair is not None
+    dgu, dguT = pair
+    assert dgu.shape == gu.shape and dgu.dtype == dtype
+    assert (dguT is not None) == (dtype == torch.bfloat16)
+    if dguT is not None:
+        want = ops.transpose_grouped_rows(dgu[:n], start, count, n)
+        assert dguT.shape == want.shape
+        for e, c in enumerate(counts):
+            lo, width = int(ks[e]), int(kc[e])
+            assert same_bits(dguT[:, lo:lo + width], want[:, lo:lo + width]), e
+            assert torch.all(dguT[:, lo + c:lo + width] == 0)
+        plain = ops.grouped_down_dgrad_dsilu(dy, tab, gu, start, count, n, H, I)
+        assert plain[1] is None and same_bits(plain[0][:n], dgu[:n])
     dh = ops.grouped_gemm_nt(tab, H, I, start, count, n + pad, n, I, H, a=dy)
     two = torch.empty_like(gu)
     ops.silu_mul_bwd(gu[:n, :I], gu[:n, I:], dh[:n], da=two[:n, :I], db=two[:n, I:])
@@ -1063,7 +1090,8 @@ def test_grouped_down_dgrad_with_swiglu_gradient(ops, gpu, counts, H, I, dtype):
     lib = __import__("adaptivetrainingsystem_amd._lib", fromlist=["load"]).load()
     dgu.fill_(3.0)
     rc = lib.ats_grouped_down_dgrad_dsilu(dy.data_ptr(), tab.data_ptr(), gu.data_ptr(), dgu.data_ptr(), start.data_ptr(),
-                                          count.data_ptr(), E, n, H, I, 0 if dtype == torch.float32 else 1, None)
+                                          count.data_ptr(), E, n, H, I, 0 if dtype == torch.float32 else 1,
+                                          None, 0, None, None)
     assert rc == 0
     torch.cuda.synchronize()
     assert torch.all(dgu[n:] == 3.0) and same_bits(dgu[:n], two[:n])
