@@ -149,15 +149,24 @@ struct AccView16 {
 //   SAVEGU: the accumulator layout already has 16 lanes on 16 consecutive rows, so h goes from the registers
 //     into [32 columns][128 rows] (pitch 272 bytes: the lanes of a write land on 64 different banks) and
 //     leaves as 256-byte row segments after the last 32-row block;
-//   DSILU: dg and du exist only in the row-major phase (a lane holds 8 columns of one row), so every 32-row
-//     block goes into [2][64 columns][32 rows] (pitch 80 bytes, the 16-byte row chunk XORed with bits of the
-//     column so that the lanes of a write land on 64 different banks) and leaves as 64-byte segments.
+//   DSILU: dg and du exist only in the row-major phase (a lane holds 8 columns of one row), so two 32-row
+//     blocks at a time go into [2][64 columns][64 rows] and leave as whole 128-byte lines (64-byte pieces of
+//     lines cost three times as much at the memory side).  That region takes 16 KiB per wave, which fits
+//     beside the row-major staging only without padding, so both are unpadded 128-byte rows with XOR swizzles:
+//     in the transposed region the 16-byte chunk of a row is XORed with bits 3-5 of the column and columns with
+//     bit 2 set trade places with their neighbour (the lanes of a write land on 64 different banks); in the
+//     row-major region the chunk is XORed with the low bits of the row.
 // In both, two lanes that hold neighbouring rows first exchange half of their values (one DPP move per word), so
 // that every LDS write is a whole word holding rows m and m + 1 of one column.
 constexpr int kTransPitchH = 128 * 2 + 16;
-constexpr int kTransPitchD = 32 * 2 + 16;
 constexpr int kTransStageH = 32 * kTransPitchH;         // bytes per wave, SAVEGU
-constexpr int kTransStageD = 2 * 64 * kTransPitchD;     // bytes per wave, DSILU
+constexpr int kTransStageD = 2 * 64 * 128;              // bytes per wave, DSILU
+// Bytes of the row-major staging region of one wave.
+template <typename TO, typename View, bool DSILU>
+constexpr int epilogue_wstage_bytes() {
+    return DSILU && sizeof(TO) == 2 && View::kCols == 64 && View::kBlocks == 4
+               ? 32 * 128 : 32 * (View::kCols * (int)sizeof(TO) + 16);
+}
 template <typename TO, typename View, bool SWIGLU, bool SAVEGU = false, bool DSILU = false>
 __device__ __forceinline__ void epilogue_view(const View av, unsigned char* wstage, TO* out, int64_t ldo,
                                               int64_t row_base, int rows_valid, int ncol0, int n_out, int lane,
@@ -168,11 +177,13 @@ __device__ __forceinline__ void epilogue_view(const View av, unsigned char* wsta
     static_assert(!DSILU || !SWIGLU, "the SwiGLU gradient epilogue belongs to the plain product");
     constexpr int WCOLS = View::kCols;
     constexpr int ES = (int)sizeof(TO);
-    constexpr int PITCH = WCOLS * ES + 16;
+    constexpr bool kSwzStage = DSILU && ES == 2 && WCOLS == 64 && View::kBlocks == 4;   // unpadded, swizzled rows
+    constexpr int PITCH = kSwzStage ? 128 : WCOLS * ES + 16;
+    static_assert(32 * PITCH == epilogue_wstage_bytes<TO, View, DSILU>(), "staging size");
     constexpr int LPR = WCOLS * ES / 16;   // lanes per output row
     constexpr int RPI = 64 / LPR;          // rows per store instruction
     constexpr int EPC = 16 / ES;           // elements per 16-byte chunk
-    constexpr bool kTrans = (SAVEGU || DSILU) && ES == 2 && View::kBlocks * 32 == 128;
+    constexpr bool kTrans = (SAVEGU || DSILU) && ES == 2 && View::kBlocks * 32 == 128 && (SAVEGU || kSwzStage);
     // rows of the wave that the transposed copy covers: the valid ones and the zero columns after them
     const int t_rows = !kTrans || tout == nullptr || rows_valid <= 0 ? 0
                        : (rows_valid >= 128 ? 128 : (rows_valid + 63) / 64 * 64);
@@ -187,6 +198,9 @@ __device__ __forceinline__ void epilogue_view(const View av, unsigned char* wsta
                 else v[c] = av.val(i, g, c, 0);
             }
             unsigned char* dst = wstage + View::row(g, lane) * PITCH + View::col(g, lane) * ES;
+            if constexpr (kSwzStage)
+                dst = wstage + View::row(g, lane) * 128 + (((View::col(g, lane) >> 3) ^ (View::row(g, lane) & 7)) * 16) +
+                      (View::col(g, lane) & 7) * 2;
             if constexpr (ES == 2) {
                 uint2 u;
                 u.x = pack_bf16x2(v[0], v[1]);
@@ -216,7 +230,8 @@ __device__ __forceinline__ void epilogue_view(const View av, unsigned char* wsta
         for (int r0 = 0; r0 < 32; r0 += RPI) {
             const int r = r0 + lane / LPR;
             const int c = lane % LPR;
-            const u32x4_t data = *reinterpret_cast<const u32x4_t*>(wstage + r * PITCH + c * 16);
+            const u32x4_t data =
+                *reinterpret_cast<const u32x4_t*>(wstage + r * PITCH + (kSwzStage ? (c ^ (r & 7)) : c) * 16);
             const int m_local = i * 32 + r;
             const int col = ncol0 + c * EPC;
             if constexpr (DSILU) {
@@ -253,15 +268,20 @@ __device__ __forceinline__ void epilogue_view(const View av, unsigned char* wsta
                         const uint32_t ru1 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(odd ? pu.y : pu.w), kRor8, 0xf, 0xf, false);
                         const uint32_t lo[2][2] = {{odd ? rg0 : pg.x, odd ? rg1 : pg.y}, {odd ? ru0 : pu.x, odd ? ru1 : pu.y}};
                         const uint32_t hi[2][2] = {{odd ? pg.z : rg0, odd ? pg.w : rg1}, {odd ? pu.z : ru0, odd ? pu.w : ru1}};
+                        // staged row of column n: n ^ 1 for the columns with bit 2 set (the odd lane's), chunk
+                        // (rows / 8 inside the pair of blocks) ^ (n >> 3)
                         const int nb = c * 8 + (odd ? 4 : 0);
-                        unsigned char* td = tstage + nb * kTransPitchD + (((r >> 3) ^ ((c >> 1) & 3)) * 16) + ((r & 7) >> 1) * 4;
+                        const int q = (i & 1) * 4 + (r >> 3);
+                        unsigned char* td = tstage + ((q ^ c) * 16) + ((r & 7) >> 1) * 4;
 #pragma unroll
                         for (int half = 0; half < 2; ++half)
 #pragma unroll
                             for (int w2 = 0; w2 < 2; ++w2) {
-                                unsigned char* t2 = td + (half * 64 + 2 * w2) * kTransPitchD;
-                                *reinterpret_cast<uint32_t*>(t2) = (lo[half][w2] & 0xffffu) | (hi[half][w2] << 16);
-                                *reinterpret_cast<uint32_t*>(t2 + kTransPitchD) = (lo[half][w2] >> 16) | (hi[half][w2] & 0xffff0000u);
+                                const int n0 = half * 64 + nb + 2 * w2;
+                                *reinterpret_cast<uint32_t*>(td + (odd ? n0 + 1 : n0) * 128) =
+                                    (lo[half][w2] & 0xffffu) | (hi[half][w2] << 16);
+                                *reinterpret_cast<uint32_t*>(td + (odd ? n0 : n0 + 1) * 128) =
+                                    (lo[half][w2] >> 16) | (hi[half][w2] & 0xffff0000u);
                             }
                     }
                 }
@@ -272,17 +292,17 @@ __device__ __forceinline__ void epilogue_view(const View av, unsigned char* wsta
         }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         if constexpr (kTrans && DSILU) {
-            if (i * 32 < t_rows) {
+            if ((i & 1) && i * 32 < t_rows) {          // t_rows is 64 or 128: both blocks of a pair are in or out
 #pragma unroll
-                for (int it = 0; it < 8; ++it) {
+                for (int it = 0; it < 16; ++it) {
                     const int idx = it * 64 + lane;
-                    const int rowid = idx >> 2, j = idx & 3;          // 128 staged rows (dg 0..63, du 64..127) x 4 chunks
+                    const int rowid = idx >> 3, j = idx & 7;          // 128 columns (dg 0..63, du 64..127) x 8 chunks
                     const int n_l = rowid & 63, half = rowid >> 6;
                     const u32x4_t data = *reinterpret_cast<const u32x4_t*>(
-                        tstage + rowid * kTransPitchD + ((j ^ ((n_l >> 4) & 3)) * 16));
-                    const int m0 = i * 32 + j * 8;
-                    if (m0 < t_rows && ncol0 + n_l < n_out)
-                        *reinterpret_cast<u32x4_t*>(tout + (int64_t)(half * up_off + ncol0 + n_l) * ldt + tcol + m0) = data;
+                        tstage + (rowid ^ ((rowid >> 2) & 1)) * 128 + ((j ^ ((n_l >> 3) & 7)) * 16));
+                    const int m0 = (i - 1) * 32 + j * 8;
+                    if (ncol0 + n_l < n_out)
+                        __builtin_nontemporal_store(data, reinterpret_cast<u32x4_t*>(tout + (int64_t)(half * up_off + ncol0 + n_l) * ldt + tcol + m0));
                 }
                 asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
             }
@@ -326,7 +346,7 @@ __device__ __forceinline__ void epilogue_view(const View av, unsigned char* wsta
                 const int n_l = r0 + (lane >> 4), ch = lane & 15;
                 const u32x4_t data = *reinterpret_cast<const u32x4_t*>(tstage + n_l * kTransPitchH + ch * 16);
                 if (ch * 8 < t_rows && ncol0 + n_l < n_out)
-                    *reinterpret_cast<u32x4_t*>(tout + (int64_t)(ncol0 + n_l) * ldt + tcol + ch * 8) = data;
+                    __builtin_nontemporal_store(data, reinterpret_cast<u32x4_t*>(tout + (int64_t)(ncol0 + n_l) * ldt + tcol + ch * 8));
             }
         }
     }
@@ -1278,7 +1298,7 @@ __global__ __launch_bounds__(512) void grouped_gemm_dma16_kernel(GroupedArgs p) 
 
     {
         typedef AccView16<TM, TN, SWIGLU> View;
-        constexpr int WSTAGE = 32 * (View::kCols * (int)sizeof(TO) + 16);
+        constexpr int WSTAGE = epilogue_wstage_bytes<TO, View, DSILU>();
         const int wrow = tc.mt * BM + wm * (BM / WM);
         const int ncol0 = SWIGLU ? tc.nt * HALF + wn * (BN / WN / 2) : tc.nt * BN + wn * (BN / WN);
         if constexpr (SAVEGU || DSILU) {
