@@ -291,8 +291,9 @@ class ExpertFFNFunction(Function):
 
     @staticmethod
     def backward(ctx, dy):
-        x, offsets, kept, gu, h = ctx.saved_tensors[:5]
-        wplan = tuple(ctx.saved_tensors[5:7]) if ctx.has_wplan else None
+        saved = ctx.saved_tensors                    # read once: activation checkpointing unpacks on every access
+        x, offsets, kept, gu, h = saved[:5]
+        wplan = tuple(saved[5:7]) if ctx.has_wplan else None
         hT = None
         if ctx.h_transposed:
             h, hT = None, h
@@ -360,8 +361,9 @@ class MoEFunction(Function):
 
     @staticmethod
     def backward(ctx, dout, daux):
-        (x, wg, logits, logits_route, idx, w, usage, aux, offsets, kept, row_src, row_of, gu, h, y) = ctx.saved_tensors[:15]
-        wplan = tuple(ctx.saved_tensors[15:17]) if ctx.has_wplan else None
+        saved = ctx.saved_tensors                    # read once: activation checkpointing unpacks on every access
+        (x, wg, logits, logits_route, idx, w, usage, aux, offsets, kept, row_src, row_of, gu, h, y) = saved[:15]
+        wplan = tuple(saved[15:17]) if ctx.has_wplan else None
         hT = None
         if ctx.h_transposed:
             h, hT = None, h
