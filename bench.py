@@ -866,9 +866,11 @@ def run_norm_rope(args):
                                   "achieved": scopy_gbs, "unit": "GB/s", "frac": scopy_gbs / PEAK_HBM_GBS,
                                   "rmsnorm_vs_copy": rms_gbs / scopy_gbs, "rope_vs_copy": rope_gbs / scopy_gbs},
         "rmsnorm_bwd_roofline": {"bound": "hbm", "achieved": rmsb_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                                 "frac": rmsb_gbs / PEAK_HBM_GBS},
+                                 "frac": rmsb_gbs / PEAK_HBM_GBS,
+                                 "traffic": profile_traffic("c2_norm_rope", "rmsnorm_bwd")},
         "rope_bwd_roofline": {"bound": "hbm", "achieved": ropeb_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                              "frac": ropeb_gbs / PEAK_HBM_GBS},
+                              "frac": ropeb_gbs / PEAK_HBM_GBS,
+                              "traffic": profile_traffic("c2_norm_rope", "rope_bwd")},
         "stages_ms": {s: round(v["mean_ms"], 5) for s, v in st.items()},
     }
     if not args.no_cpu_baseline:
