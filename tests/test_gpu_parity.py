@@ -1241,3 +1241,25 @@ def test_float16_activations_run_through_the_float32_kernels(A, gpu):
     assert ys.dtype == torch.float16 and rel_err(ys, gate * torch.nn.functional.silu(up)) <= 2e-3
     with pytest.raises(A.AtsError):
         sw(xm.to(gpu).requires_grad_())
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_transposed_zero_empty_groups(ops, gpu, dtype):
+    """The 64 columns of every expert without rows are cleared in a transposed [C, ld] matrix; nothing else is touched."""
+    lib = __import__("adaptivetrainingsystem_amd._lib", fromlist=["load"]).load()
+    counts = torch.tensor([5, 0, 130, 0, 0, 64], dtype=torch.int32, device=gpu)
+    ks, kc = ops.wgrad_plan(counts)
+    E, C = counts.numel(), 37
+    ld = ops.wgrad_padded_rows(int(counts.sum()), E)
+    buf = torch.full((C, ld), 7.0, dtype=dtype, device=gpu)
+    rc = lib.ats_transposed_zero_empty_groups(buf.data_ptr(), ld, C, counts.data_ptr(), ks.data_ptr(), E,
+                                              0 if dtype == torch.float32 else 1, None)
+    assert rc == 0
+    torch.cuda.synchronize()
+    want = torch.full((C, ld), 7.0, dtype=dtype)
+    for e in range(E):
+        if int(counts[e]) == 0:
+            assert int(kc[e]) == 64
+            want[:, int(ks[e]):int(ks[e]) + 64] = 0
+    assert torch.equal(buf.cpu(), want)
+    assert lib.ats_transposed_zero_empty_groups(buf.data_ptr(), ld + 1, C, counts.data_ptr(), ks.data_ptr(), E, 1, None) != 0
