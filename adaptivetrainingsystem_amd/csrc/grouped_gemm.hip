@@ -1044,6 +1044,10 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_dma_kernel(GroupedAr
 // reached the texture addresser within a few hundred cycles, its queue filled up (it takes one 1 KiB load in
 // about 16 cycles) and the waves, which issue in order, stood at their next load with MFMAs behind it:
 // spreading the activation loads over the slab is worth 3-4 % at the prefill and at the fine-grained shape.
+// A wave runs phase 3 (the weight loads of slab t+2 and the first fragment reads of slab t+1, right behind the
+// barrier) at raised priority and drops back at the top of the next slab: 1 % at both shapes and on the training
+// step (s_setprio 1, 2 or 3, and keeping it through phase 0, measure the same at the prefill shape; raising it for
+// phases 0-2 instead loses 0.2 %).
 template <typename TO, int SM, int SN, bool SWIGLU, bool SAVEGU = false, bool DSILU = false>
 __global__ __launch_bounds__(512) void grouped_gemm_dma16_kernel(GroupedArgs p) {
 #if defined(__HIP_DEVICE_COMPILE__)
@@ -1199,6 +1203,7 @@ __global__ __launch_bounds__(512) void grouped_gemm_dma16_kernel(GroupedArgs p) 
 #define D16_ITER(kt_, STG, H0, H1)                                                      \
     {                                                                                   \
         const int sa_far = 3 * A_STAGE - sa_cur - sa_nxt;                               \
+        __builtin_amdgcn_s_setprio(0);                                                  \
         const int ka_ = min((kt_) + 2, nk - 1);                                         \
         if (H1) D16_READ_A(sa_cur, 0, 1, 1);                                            \
         D16_ISSUE_A1(ka_, sa_far, 0);                                                   \
@@ -1229,6 +1234,7 @@ __global__ __launch_bounds__(512) void grouped_gemm_dma16_kernel(GroupedArgs p) 
         }                                                                               \
         PL_FENCE();                                                                     \
         asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(NIA) : "memory"); \
+        __builtin_amdgcn_s_setprio(2);                                                  \
         PL_FENCE();                                                                     \
         if (H0) {                                                                       \
             D16_READ_B(STG ^ 1, 0, 0, 0);                                               \
@@ -1282,6 +1288,7 @@ __global__ __launch_bounds__(512) void grouped_gemm_dma16_kernel(GroupedArgs p) 
     } else {
         D16_LOOP(false, false);
     }
+    __builtin_amdgcn_s_setprio(0);
     // the clamped loads of the last slabs may still be in flight; the epilogue reuses LDS
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
 #undef D16_LOOP
