@@ -1033,9 +1033,9 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_dma_kernel(GroupedAr
 // A 64-element slab is two 32-element k-steps; the wave's 128 rows are two halves of four 16-row fragments.
 // A slab is four phases of 16 MFMAs, (k-step, row half) = (0,0) (0,1) (1,0) (1,1); fragments live in two
 // buffers of four activation fragments and two buffers of four weight fragments:
-//   phase 0 : MFMAs | reads: activations (k0, half 1), weights (k1) 0..1 | loads: activations of slab t+2, 2 of 4
+//   phase 0 : MFMAs | reads: activations (k0, half 1), weights (k1) 0..1 | loads: activations of slab t+2, 1 of 4
 //   phase 1 : MFMAs | reads: activations (k1, half 0), weights (k1) 2..3 | loads: activations of slab t+2, 1 of 4
-//   phase 2 : MFMAs | reads: activations (k1, half 1)                    | loads: activations of slab t+2, 1 of 4
+//   phase 2 : MFMAs | reads: activations (k1, half 1)                    | loads: activations of slab t+2, 2 of 4
 //   wait for the loads of slab t+1, barrier
 //   phase 3 : MFMAs | reads: activations (k0, half 0) and weights (k0) of slab t+1 | loads: weights of slab t+2
 // The activation ring has three stages, so the stage that slab t+2 goes into was given up at the previous
@@ -1044,6 +1044,11 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_dma_kernel(GroupedAr
 // reached the texture addresser within a few hundred cycles, its queue filled up (it takes one 1 KiB load in
 // about 16 cycles) and the waves, which issue in order, stood at their next load with MFMAs behind it:
 // spreading the activation loads over the slab is worth 3-4 % at the prefill and at the fine-grained shape.
+// Inside a phase the fragment reads go between its first MFMAs and the loads between the MFMAs behind them
+// (in phase 3: eight reads over the first eight MFMAs, four loads over the last eight).  With the loads at the
+// head of their phase, next to the reads, the prefill step was 3.3 % slower and the training step 3.4 %
+// (alternating runs on one box: 5.70 -> 5.51 ms and 19.69 -> 19.03 ms); loads of one array bunched into one
+// phase, or weight loads held back until after the next slab has begun, lose it again.
 // A wave runs phase 3 (the weight loads of slab t+2 and the first fragment reads of slab t+1, right behind the
 // barrier) at raised priority and drops back at the top of the next slab: 1 % at both shapes and on the training
 // step (s_setprio 1, 2 or 3, and keeping it through phase 0, measure the same at the prefill shape; raising it for
@@ -1181,19 +1186,26 @@ __global__ __launch_bounds__(512) void grouped_gemm_dma16_kernel(GroupedArgs p) 
                     __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_.v, a_.v, acc[j][(half_) * 4 + i], 0, 0, 0); \
             }                                                                                          \
     }
-// nrd fragment reads and nvm loads spread over the first MFMAs of a phase (16 MFMAs)
+// Order inside a phase of 16 MFMAs: its nrd fragment reads go between the first MFMAs, its nvm loads between
+// the MFMAs behind them
 #define D16_MIX(nrd_, nvm_)                                                             \
     _Pragma("unroll") for (int g_ = 0; g_ < (nrd_); ++g_) {                             \
         __builtin_amdgcn_sched_group_barrier(SG_MFMA, 16 / ((nrd_) + 2), 0);            \
         __builtin_amdgcn_sched_group_barrier(SG_DS_RD, 1, 0);                           \
-        if (g_ < (nvm_)) __builtin_amdgcn_sched_group_barrier(SG_VMEM, 1, 0);           \
+    }                                                                                   \
+    _Pragma("unroll") for (int g_ = 0; g_ < (nvm_); ++g_) {                             \
+        __builtin_amdgcn_sched_group_barrier(SG_MFMA, 1, 0);                            \
+        __builtin_amdgcn_sched_group_barrier(SG_VMEM, 1, 0);                            \
     }
-// phase 3: a fragment read per two MFMAs, a load per four
+// phase 3: a fragment read per MFMA over the first half, a load per two MFMAs over the second
 #define D16_MIX_DMA()                                                                   \
     _Pragma("unroll") for (int g_ = 0; g_ < 8; ++g_) {                                  \
         __builtin_amdgcn_sched_group_barrier(SG_DS_RD, 1, 0);                           \
+        __builtin_amdgcn_sched_group_barrier(SG_MFMA, 1, 0);                            \
+    }                                                                                   \
+    _Pragma("unroll") for (int g_ = 0; g_ < 4; ++g_) {                                  \
+        __builtin_amdgcn_sched_group_barrier(SG_VMEM, 1, 0);                            \
         __builtin_amdgcn_sched_group_barrier(SG_MFMA, 2, 0);                            \
-        if (g_ % 2 == 0) __builtin_amdgcn_sched_group_barrier(SG_VMEM, 1, 0);           \
     }
 // STG: weight stage of slab kt (compile time); sa_cur / sa_nxt: activation stage offsets of slabs kt, kt+1
 // (the third stage takes slab kt+2).  Slabs past the end are clamped to the last one (their loads land in
@@ -1207,15 +1219,14 @@ __global__ __launch_bounds__(512) void grouped_gemm_dma16_kernel(GroupedArgs p) 
         const int ka_ = min((kt_) + 2, nk - 1);                                         \
         if (H1) D16_READ_A(sa_cur, 0, 1, 1);                                            \
         D16_ISSUE_A1(ka_, sa_far, 0);                                                   \
-        D16_ISSUE_A1(ka_, sa_far, 1);                                                   \
         if (H0) {                                                                       \
             D16_READ_B(STG, 1, 0, 1);                                                   \
             D16_READ_B(STG, 1, 1, 1);                                                   \
             D16_MMA(0, 0, 0);                                                           \
-            D16_MIX(H1 ? 6 : 2, 2);                                                     \
+            D16_MIX(H1 ? 6 : 2, 1);                                                     \
         }                                                                               \
         PL_FENCE();                                                                     \
-        D16_ISSUE_A1(ka_, sa_far, 2);                                                   \
+        D16_ISSUE_A1(ka_, sa_far, 1);                                                   \
         if (H0) {                                                                       \
             D16_READ_A(sa_cur, 1, 0, 0);                                                \
             D16_READ_B(STG, 1, 2, 1);                                                   \
@@ -1226,11 +1237,12 @@ __global__ __launch_bounds__(512) void grouped_gemm_dma16_kernel(GroupedArgs p) 
             D16_MIX(6, 1);                                                              \
         }                                                                               \
         PL_FENCE();                                                                     \
+        D16_ISSUE_A1(ka_, sa_far, 2);                                                   \
         D16_ISSUE_A1(ka_, sa_far, 3);                                                   \
         if (H1) D16_READ_A(sa_cur, 1, 1, 1);                                            \
         if (H0) {                                                                       \
             D16_MMA(1, 0, 0);                                                           \
-            D16_MIX(H1 ? 4 : 1, 1);                                                     \
+            D16_MIX(H1 ? 4 : 1, 2);                                                     \
         }                                                                               \
         PL_FENCE();                                                                     \
         asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(NIA) : "memory"); \
