@@ -15,8 +15,8 @@
 // kernel).  The operand that changes from step to step is the A operand and comes from LDS, where a
 // tile is kept as it is in memory (rows of D elements): fragments along D are plain 16-byte reads,
 // fragments across rows (K^T for dQ, Q^T and dO^T for dK/dV) come out through the transposing read
-// ds_read_b64_tr_b16, so no transposed copy of any operand is made.  The two access patterns want
-// different row pitches to stay free of bank conflicts, so a tile that is read both ways is stored twice.
+// ds_read_b64_tr_b16, so no transposed copy of any operand is made.  A tile is stored once, unpadded, with
+// its 16-byte chunks swizzled so that both access patterns stay free of bank conflicts (SwzTile below).
 #include <math.h>
 
 #include <type_traits>
@@ -33,23 +33,7 @@ typedef unsigned int bu32x2_t __attribute__((ext_vector_type(2)));
 typedef short btr_t __attribute__((ext_vector_type(4)));
 typedef __attribute__((address_space(3))) btr_t* blds_tr_ptr_t;
 
-// A-operand fragment of X^T for one 32x32x16 MFMA from a tile stored [row][d] with pitch `pitch` bytes:
-// lane l receives d = d0 + l % 32 and rows r0 + {4g..4g+3, 8+4g..8+4g+3} (g = l / 32), the order in which a
-// 32x32 accumulator hands its rows to the next product.  `lane_base` is tr_lane_base(tile, lane, pitch).
-__device__ __forceinline__ const unsigned char* tr_lane_base(const unsigned char* tile, int lane, int pitch) {
-    return tile + (4 * (lane >> 5) + ((lane & 15) >> 2)) * pitch + (16 * ((lane >> 4) & 1) + 4 * (lane & 3)) * 2;
-}
-__device__ __forceinline__ bu32x4_t tr_fragment(const unsigned char* lane_base, int r0, int d0, int pitch) {
-    const unsigned char* p = lane_base + r0 * pitch + d0 * 2;
-    union {
-        btr_t t[2];
-        bu32x4_t u;
-    } cv;
-    cv.t[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((blds_tr_ptr_t)(p));
-    cv.t[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((blds_tr_ptr_t)(p + 8 * pitch));
-    return cv.u;
-}
-
+constexpr int kSgMfma = 0x008, kSgDsRead = 0x100;   // instruction classes of sched_group_barrier
 constexpr int kBwdRows = 128;   // rows a block owns: 4 waves x 32
 constexpr int kDqBN = 64;       // keys per step of the dQ kernel
 constexpr int kDkvBQ = 32;      // queries per step of the dK/dV kernel
@@ -342,6 +326,15 @@ __device__ __forceinline__ void attention_bwd_dq_tile(const bf16_t* __restrict__
 #pragma unroll
                 for (int d = 0; d < DB; ++d)
                     acc_dq[d] = bwd_mma(tr_fragment_swz(sm + st, tr_lo[d], tr_hi[d], s * 16 * ROWB), dsf[s], acc_dq[d]);
+            // the transposing reads run two fragments ahead of the MFMAs (unconstrained, the compiler issues all
+            // 32 reads first and the first MFMAs wait for the tail of that burst)
+            __builtin_amdgcn_sched_group_barrier(kSgDsRead, 4, 0);
+#pragma unroll
+            for (int i = 0; i + 2 < 4 * DB; ++i) {
+                __builtin_amdgcn_sched_group_barrier(kSgDsRead, 2, 0);
+                __builtin_amdgcn_sched_group_barrier(kSgMfma, 1, 0);
+            }
+            __builtin_amdgcn_sched_group_barrier(kSgMfma, 2, 0);
             __builtin_amdgcn_s_setprio(0);
         }
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -404,7 +397,12 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dq_kernel(
 
 // ------------------------------------------------------------------------------------------ dK, dV
 // One 128-row key tile of one (batch, kv head): lanes own keys; the queries of every query head of the
-// group come in steps of 32, starting at the first query that sees the tile.
+// group come in steps of 32, starting at the first query that sees the tile.  The steps of all heads form one
+// sequence; the Q and dO rows of step i+1 go from memory straight into the LDS stage that step i-1 used
+// (swizzled tiles as in the dQ kernel, read along D for the first two products and across rows for the last
+// two) while step i is computed: one barrier per step, and the loads have the whole step to land.
+typedef float bf32x4_t __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) bf32x4_t* blds_f4_t;
 template <int D, bool EXTRA = false>
 __device__ __forceinline__ void attention_bwd_dkv_tile(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
                                                        const bf16_t* __restrict__ v, const bf16_t* __restrict__ dout,
@@ -413,25 +411,25 @@ __device__ __forceinline__ void attention_bwd_dkv_tile(const bf16_t* __restrict_
                                                        bf16_t* __restrict__ dv, int Hq, int Hkv, int L, int Lk, float scale,
                                                        int kt_idx, int hkv, int b, unsigned char* smem,
                                                        const AttnExtra* ex = nullptr) {
+    using SW = SwzTile<D>;
     constexpr int KS = D / 16;
     constexpr int DB = D / 32;
-    constexpr int RPITCH = D * 2 + 16;        // bytes per Q / dO row in LDS
-    constexpr int TPITCH = D * 2 + 64;        // bytes per row of the second copies (transposing reads)
-    constexpr int RTILE = kDkvBQ * RPITCH;
-    constexpr int TTILE = kDkvBQ * TPITCH;
-    constexpr int RVEC = kDkvBQ * (D / 8) / 256;   // 16-byte vectors per thread: D=128 -> 2, D=64 -> 1
-    unsigned char* const sQ = smem;
-    unsigned char* const sO = smem + RTILE;
-    unsigned char* const sQT = smem + 2 * RTILE;
-    unsigned char* const sOT = smem + 2 * RTILE + TTILE;
-    float* const sL = reinterpret_cast<float*>(smem + 2 * RTILE + 2 * TTILE);   // [32] lse * log2(e)
-    float* const sD = sL + kDkvBQ;                                             // [32] delta
+    constexpr int ROWB = SW::ROWB;
+    constexpr int TILE = kDkvBQ * ROWB;              // one Q or dO tile
+    constexpr int STAGE = 2 * TILE;                  // [Q | dO]
+    constexpr int NI = TILE / 1024 / 4;              // load instructions per wave and tile, Q (and dO)
+    static_assert(NI >= 1 && NI * 4 * 1024 == TILE, "loader tiling");
+    constexpr int RPITCH = D * 2 + 16;               // bytes per V row in LDS
+    const blds_u8_t sm = (blds_u8_t)smem;
+    const blds_f32_t sL = (blds_f32_t)(sm + 2 * STAGE);   // [2][32] lse * log2(e)
+    const blds_f32_t sD = sL + 2 * kDkvBQ;                // [2][32] delta
     // the block's own V rows stay in LDS for the whole tile: with K rows, both accumulators and V rows in
     // registers a wave would need more than half the register file, i.e. one wave per SIMD
-    unsigned char* const sVb = smem + 2 * RTILE + 2 * TTILE + 2 * kDkvBQ * 4;    // [128][RPITCH]
+    unsigned char* const sVb = smem + 2 * STAGE + 4 * kDkvBQ * 4;    // [128][RPITCH]
 
     const int rep = Hq / Hkv;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int col = lane & 31, g = lane >> 5;
     const int key_row = kt_idx * kBwdRows + wave * 32 + col;
     const int key_clamped = key_row < Lk ? key_row : Lk - 1;
@@ -448,7 +446,7 @@ __device__ __forceinline__ void attention_bwd_dkv_tile(const bf16_t* __restrict_
     bu32x4_t kf[KS];
 #pragma unroll
     for (int s = 0; s < KS; ++s) kf[s] = *reinterpret_cast<const bu32x4_t*>(kp + s * 16 + g * 8);
-    __syncthreads();   // the previous tile of this workgroup is done with the V rows
+    __syncthreads();   // the previous tile of this workgroup is done with the V rows and the stages
     {
         const bf16_t* vblock = v + (int64_t)(b * Hkv + hkv) * Lk * D;
         const __amdgpu_buffer_rsrc_t vb_rsrc =
@@ -466,6 +464,63 @@ __device__ __forceinline__ void attention_bwd_dkv_tile(const bf16_t* __restrict_
 #pragma unroll
     for (int s = 0; s < KS; ++s) asm volatile("" : "+v"(kf[s]));
 
+    // lane offsets of the loads (Q rows are D elements apart, dO rows Hq * D) and of the fragment reads
+    int ld_q[NI], ld_o[NI];
+#pragma unroll
+    for (int j = 0; j < NI; ++j) {
+        ld_q[j] = SW::src_offset((j * 4 + wave) * 64 + lane, ROWB);
+        ld_o[j] = SW::src_offset((j * 4 + wave) * 64 + lane, Hq * ROWB);
+    }
+    // fragment offsets of k-step s / d block G differ from those of k-step 0 / block 0 in the chunk bits only:
+    // off(s) = off(0) ^ (s << 5), off(G) = off(0) ^ (G << 6); they are formed per step from three registers
+    // (sixteen kept across the loop would not fit beside the accumulators)
+    const int row_base = SW::row_frag(lane, 0), tr_lo_base = SW::tr_frag(lane, 0, false),
+              tr_hi_base = SW::tr_frag(lane, 0, true);
+    // buffer loads: query rows past L are outside the descriptors
+#define DKV_LOAD(hh_, q0_, stage_)                                                                     \
+    {                                                                                                  \
+        const int hq_ = hkv * rep + (hh_);                                                             \
+        const __amdgpu_buffer_rsrc_t q_rsrc_ = __builtin_amdgcn_make_buffer_rsrc(                      \
+            const_cast<bf16_t*>(q + (int64_t)(b * Hq + hq_) * L * D), 0, (int)((int64_t)L * D * 2), 0x00020000); \
+        const __amdgpu_buffer_rsrc_t o_rsrc_ = __builtin_amdgcn_make_buffer_rsrc(                      \
+            const_cast<bf16_t*>(dout + (int64_t)b * L * (int64_t)(Hq * D) + hq_ * D), 0,              \
+            (int)((((int64_t)L - 1) * Hq * D + D) * 2), 0x00020000);                                   \
+        _Pragma("unroll") for (int j_ = 0; j_ < NI; ++j_) {                                            \
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(q_rsrc_, (blds_void_t)(sm + (stage_) * STAGE + (j_ * 4 + wave) * 1024), \
+                                                     16, ld_q[j_], (q0_) * (D * 2), 0, 0);             \
+            __builtin_amdgcn_raw_ptr_buffer_load_lds(o_rsrc_, (blds_void_t)(sm + (stage_) * STAGE + TILE + (j_ * 4 + wave) * 1024), \
+                                                     16, ld_o[j_], (q0_) * (Hq * D * 2), 0, 0);        \
+        }                                                                                              \
+    }
+    // Queries past L: their rows of Q and dO must be zeros in LDS (they meet exact zeros of P and dS, but
+    // 0 x NaN is not 0); each lane clears the positions of its own loads once they landed.
+#define DKV_CLEAR_TAIL(q0_, stage_)                                                                    \
+    if ((q0_) + kDkvBQ > L) {                                                                          \
+        _Pragma("unroll") for (int j_ = 0; j_ < NI; ++j_) {                                            \
+            const int p_ = (j_ * 4 + wave) * 64 + lane;                                                \
+            if ((q0_) + p_ / SW::CPR >= L) {                                                           \
+                *(blds_v4_t)(sm + (stage_) * STAGE + p_ * 16) = bu32x4_t{0u, 0u, 0u, 0u};              \
+                *(blds_v4_t)(sm + (stage_) * STAGE + TILE + p_ * 16) = bu32x4_t{0u, 0u, 0u, 0u};       \
+            }                                                                                          \
+        }                                                                                              \
+    }
+    // lse and delta of the step's queries: thread t < 32 fetches those of query q0 + t (raw values: nothing may
+    // wait for them before the step's arithmetic is done) and finishes them when it stores them
+#define DKV_ROW_SCALARS(hh_, q0_, l_, d_)                                                              \
+    if (tid < kDkvBQ) {                                                                                \
+        const int qc_ = min((q0_) + tid, L - 1);                                                       \
+        const int64_t base_ = (int64_t)(b * Hq + hkv * rep + (hh_)) * L;                               \
+        l_ = lse[base_ + qc_];                                                                         \
+        d_ = delta[base_ + qc_];                                                                       \
+    }
+#define DKV_STORE_SCALARS(q0_, par_, l_, d_)                                                           \
+    asm volatile("" : "+v"(l_), "+v"(d_));   /* the wait for the two values stays down here */          \
+    if (tid < kDkvBQ) {                                                                                \
+        const bool in_ = (q0_) + tid < L;                                                              \
+        sL[(par_) * kDkvBQ + tid] = in_ ? l_ * kLog2e : INFINITY;   /* exp2(-inf) = 0 for rows past L */ \
+        sD[(par_) * kDkvBQ + tid] = in_ ? d_ : 0.f;                                                    \
+    }
+
     bf32x16_t acc_dk[DB], acc_dv[DB];
 #pragma unroll
     for (int d = 0; d < DB; ++d)
@@ -480,56 +535,48 @@ __device__ __forceinline__ void attention_bwd_dkv_tile(const bf16_t* __restrict_
     const int key_wave_last = key_wave_first + 31;
     // first query that sees any key of the block: q + off >= key_block_first
     const int q_first = max(key_block_first - off, 0) / kDkvBQ * kDkvBQ;
+    const int n_steps = rep * ((L - q_first + kDkvBQ - 1) / kDkvBQ);
 
-    for (int hh = 0; hh < rep; ++hh) {
-        const int hq = hkv * rep + hh;
-        const bf16_t* qbase = q + (int64_t)(b * Hq + hq) * L * D;
-        const bf16_t* obase = dout + (int64_t)b * L * (int64_t)(Hq * D) + hq * D;
-        const float* lbase = lse + (int64_t)(b * Hq + hq) * L;
-        const float* dbase = delta + (int64_t)(b * Hq + hq) * L;
-        const uint32_t head_key = EXTRA ? attn_head_key(ex->seed_lo, ex->seed_hi, (uint32_t)(b * Hq + hq)) : 0u;
-        // this head's [L, Lk] matrix of the pair bias; queries past L read as zeros (their probabilities are
-        // zeros anyway: lse = +inf)
-        __amdgpu_buffer_rsrc_t pb_rsrc;
-        if constexpr (EXTRA)
-            pb_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-                const_cast<float*>(ex_bias ? ex->bias_qk + (int64_t)b * ex->bias_sb + (int64_t)hq * ex->bias_sh : nullptr), 0,
-                ex_bias ? (int)((int64_t)L * Lk * 4) : 0, 0x00020000);
-        // buffer loads: query rows past L read as zeros
-        const __amdgpu_buffer_rsrc_t q_rsrc =
-            __builtin_amdgcn_make_buffer_rsrc(const_cast<bf16_t*>(qbase), 0, (int)((int64_t)L * D * 2), 0x00020000);
-        const __amdgpu_buffer_rsrc_t o_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-            const_cast<bf16_t*>(obase), 0, (int)((((int64_t)L - 1) * Hq * D + D) * 2), 0x00020000);
+    DKV_LOAD(0, q_first, 0)
+    {
+        float l0 = 0.f, d0 = 0.f;
+        DKV_ROW_SCALARS(0, q_first, l0, d0)
+        DKV_STORE_SCALARS(q_first, 0, l0, d0)
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    DKV_CLEAR_TAIL(q_first, 0)
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
 
-        for (int q0 = q_first; q0 < L; q0 += kDkvBQ) {
-            __syncthreads();   // every wave is done with the previous step
-            {
-                bu32x4_t rq[RVEC], ro[RVEC];
-#pragma unroll
-                for (int i = 0; i < RVEC; ++i) {
-                    const int idx = tid + i * 256;
-                    const int r = idx / (D / 8), c = idx % (D / 8);
-                    rq[i] = __builtin_amdgcn_raw_buffer_load_b128(q_rsrc, (r * D + c * 8) * 2, q0 * D * 2, 0);
-                    ro[i] = __builtin_amdgcn_raw_buffer_load_b128(o_rsrc, (r * Hq * D + c * 8) * 2, q0 * Hq * D * 2, 0);
-                }
-                if (tid < kDkvBQ) {
-                    const int qi = q0 + tid;
-                    sL[tid] = qi < L ? lbase[qi] * kLog2e : INFINITY;   // exp2(-inf) = 0 for rows past L
-                    sD[tid] = qi < L ? dbase[qi] : 0.f;
-                }
-#pragma unroll
-                for (int i = 0; i < RVEC; ++i) {
-                    const int idx = tid + i * 256;
-                    const int r = idx / (D / 8), c = idx % (D / 8);
-                    *reinterpret_cast<bu32x4_t*>(sQ + r * RPITCH + c * 16) = rq[i];
-                    *reinterpret_cast<bu32x4_t*>(sO + r * RPITCH + c * 16) = ro[i];
-                    *reinterpret_cast<bu32x4_t*>(sQT + r * TPITCH + c * 16) = rq[i];
-                    *reinterpret_cast<bu32x4_t*>(sOT + r * TPITCH + c * 16) = ro[i];
-                }
-            }
-            __syncthreads();
-            if (q0 + kDkvBQ - 1 + off < key_wave_first) continue;   // no query of the step sees this wave's keys
-
+    int hh = 0, q0 = q_first;
+    for (int i = 0; i < n_steps; ++i) {
+        const int par = i & 1;
+        const blds_u8_t st = sm + par * STAGE;     // this step's stage; the other one receives step i+1
+        int hh_n = hh, q0_n = q0 + kDkvBQ;
+        if (q0_n >= L) {
+            hh_n = hh + 1;
+            q0_n = q_first;
+        }
+        const bool more = i + 1 < n_steps;
+        const bool active = q0 + kDkvBQ - 1 + off >= key_wave_first;   // some query of the step sees this wave's keys
+        float r_l = 0.f, r_d = 0.f;
+        int rb = row_base, tlb = tr_lo_base, thb = tr_hi_base;
+        asm volatile("" : "+v"(rb), "+v"(tlb), "+v"(thb));   // keeps the offsets below inside the step
+#define DKV_PREFETCH()                                                                                 \
+        if (more) {                                                                                    \
+            if (par) { DKV_LOAD(hh_n, q0_n, 0) } else { DKV_LOAD(hh_n, q0_n, 1) }                      \
+            DKV_ROW_SCALARS(hh_n, q0_n, r_l, r_d)                                                      \
+        }
+        DKV_PREFETCH()
+        if (active) {
+            const int hq = hkv * rep + hh;
+            const uint32_t head_key = EXTRA ? attn_head_key(ex->seed_lo, ex->seed_hi, (uint32_t)(b * Hq + hq)) : 0u;
+            // this head's [L, Lk] matrix of the pair bias; queries past L read as zeros (their probabilities are
+            // zeros anyway: lse = +inf)
+            __amdgpu_buffer_rsrc_t pb_rsrc;
+            if constexpr (EXTRA)
+                pb_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+                    const_cast<float*>(ex_bias ? ex->bias_qk + (int64_t)b * ex->bias_sb + (int64_t)hq * ex->bias_sh : nullptr), 0,
+                    ex_bias ? (int)((int64_t)L * Lk * 4) : 0, 0x00020000);
             // ---- S = Q . K^T and dP = dO . V^T  (rows = queries of the step, column = this lane's key)
             __builtin_amdgcn_s_setprio(1);
             bf32x16_t acc_s, acc_p;
@@ -540,11 +587,19 @@ __device__ __forceinline__ void attention_bwd_dkv_tile(const bf16_t* __restrict_
             }
 #pragma unroll
             for (int s = 0; s < KS; ++s) {
-                const int o = col * RPITCH + s * 32 + g * 16;
-                acc_s = bwd_mma(*reinterpret_cast<const bu32x4_t*>(sQ + o), kf[s], acc_s);
-                acc_p = bwd_mma(*reinterpret_cast<const bu32x4_t*>(sO + o),
-                                *reinterpret_cast<const bu32x4_t*>(v_row + s * 32), acc_p);
+                const int ra = rb ^ (s << 5);
+                const bu32x4_t qa = *(blds_v4_t)(st + ra), oa = *(blds_v4_t)(st + TILE + ra);
+                acc_s = bwd_mma(qa, kf[s], acc_s);
+                acc_p = bwd_mma(oa, *reinterpret_cast<const bu32x4_t*>(v_row + s * 32), acc_p);
             }
+            // the three reads of k-step s+1 go out before the MFMAs of k-step s
+            __builtin_amdgcn_sched_group_barrier(kSgDsRead, 3, 0);
+#pragma unroll
+            for (int s = 0; s + 1 < KS; ++s) {
+                __builtin_amdgcn_sched_group_barrier(kSgDsRead, 3, 0);
+                __builtin_amdgcn_sched_group_barrier(kSgMfma, 2, 0);
+            }
+            __builtin_amdgcn_sched_group_barrier(kSgMfma, 2, 0);
             // ---- P = exp(S * scale - lse[q]); dS = P * (dP - delta[q]) * scale; accumulator row x is
             //      query (x / 4) * 8 + g * 4 + x % 4 of the step
             __builtin_amdgcn_s_setprio(0);
@@ -552,8 +607,8 @@ __device__ __forceinline__ void attention_bwd_dkv_tile(const bf16_t* __restrict_
             bu32x4_t pf[2], dsf[2];
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                const float4 l4 = *reinterpret_cast<const float4*>(sL + r * 8 + g * 4);
-                const float4 d4 = *reinterpret_cast<const float4*>(sD + r * 8 + g * 4);
+                const bf32x4_t l4 = *(blds_f4_t)(sL + par * kDkvBQ + r * 8 + g * 4);
+                const bf32x4_t d4 = *(blds_f4_t)(sD + par * kDkvBQ + r * 8 + g * 4);
                 const float lv[4] = {l4.x, l4.y, l4.z, l4.w};
                 const float dvv[4] = {d4.x, d4.y, d4.z, d4.w};
                 float p[4], ds[4];
@@ -591,20 +646,51 @@ __device__ __forceinline__ void attention_bwd_dkv_tile(const bf16_t* __restrict_
                 if (r == 2) { pf[1].x = p01; pf[1].y = p23; dsf[1].x = s01; dsf[1].y = s23; }
                 if (r == 3) { pf[1].z = p01; pf[1].w = p23; dsf[1].z = s01; dsf[1].w = s23; }
             }
-            // ---- dV^T += dO^T . P and dK^T += Q^T . dS  (queries of a k-step in accumulator order)
+            // ---- dV^T += dO^T . P and dK^T += Q^T . dS  (queries of a k-step in accumulator order).  The
+            //      transposing reads of pair i+1 (a fragment of dO^T and one of Q^T) are issued before the MFMAs
+            //      of pair i: left to itself the compiler reuses one set of registers for every fragment and
+            //      each MFMA waits a full LDS latency
             __builtin_amdgcn_s_setprio(1);
-            const unsigned char* ot_lane = tr_lane_base(sOT, lane, TPITCH);
-            const unsigned char* qt_lane = tr_lane_base(sQT, lane, TPITCH);
+            {
+                constexpr int NP = 2 * DB;   // pairs: (k-step s, d block) = (i / DB, i % DB)
+                bu32x4_t fo[2], fq[2];
+                fo[0] = tr_fragment_swz(st + TILE, tlb, thb, 0);
+                fq[0] = tr_fragment_swz(st, tlb, thb, 0);
 #pragma unroll
-            for (int s = 0; s < 2; ++s)
-#pragma unroll
-                for (int d = 0; d < DB; ++d) {
-                    acc_dv[d] = bwd_mma(tr_fragment(ot_lane, s * 16, d * 32, TPITCH), pf[s], acc_dv[d]);
-                    acc_dk[d] = bwd_mma(tr_fragment(qt_lane, s * 16, d * 32, TPITCH), dsf[s], acc_dk[d]);
+                for (int i = 0; i < NP; ++i) {
+                    if (i + 1 < NP) {
+                        const int s1 = (i + 1) / DB, d1 = (i + 1) % DB;
+                        const int tl = tlb ^ (d1 << 6), th = thb ^ (d1 << 6);
+                        fo[(i + 1) & 1] = tr_fragment_swz(st + TILE, tl, th, s1 * 16 * ROWB);
+                        fq[(i + 1) & 1] = tr_fragment_swz(st, tl, th, s1 * 16 * ROWB);
+                    }
+                    acc_dv[i % DB] = bwd_mma(fo[i & 1], pf[i / DB], acc_dv[i % DB]);
+                    acc_dk[i % DB] = bwd_mma(fq[i & 1], dsf[i / DB], acc_dk[i % DB]);
                 }
+                __builtin_amdgcn_sched_group_barrier(kSgDsRead, 8, 0);
+#pragma unroll
+                for (int i = 0; i + 2 < NP; ++i) {
+                    __builtin_amdgcn_sched_group_barrier(kSgMfma, 2, 0);
+                    __builtin_amdgcn_sched_group_barrier(kSgDsRead, 4, 0);
+                }
+                __builtin_amdgcn_sched_group_barrier(kSgMfma, 4, 0);
+            }
             __builtin_amdgcn_s_setprio(0);
         }
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        if (more) {
+            if (par) { DKV_CLEAR_TAIL(q0_n, 0) } else { DKV_CLEAR_TAIL(q0_n, 1) }
+            DKV_STORE_SCALARS(q0_n, par ^ 1, r_l, r_d)
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        hh = hh_n;
+        q0 = q0_n;
     }
+#undef DKV_LOAD
+#undef DKV_CLEAR_TAIL
+#undef DKV_ROW_SCALARS
+#undef DKV_STORE_SCALARS
+#undef DKV_PREFETCH
 
     if (key_row < Lk) {
         bf16_t* krow = dk + ((int64_t)(b * Hkv + hkv) * Lk + key_row) * D;
@@ -721,8 +807,7 @@ extern "C" int ats_attention_bwd_ex(const void* q, const void* k, const void* v,
                 "ats_attention_bwd_ex: with a pair bias or dropout the per-key bias must be folded into the pair bias");
     if (D == 128) {
         constexpr int smem_dq = 4 * kDqBN * 128 * 2 + 2 * kDqBN * 4;
-        constexpr int smem_dkv = 2 * kDkvBQ * (128 * 2 + 16) + 2 * kDkvBQ * (128 * 2 + 64) + 2 * kDkvBQ * 4 +
-                                 kBwdRows * (128 * 2 + 16);
+        constexpr int smem_dkv = 4 * kDkvBQ * 128 * 2 + 4 * kDkvBQ * 4 + kBwdRows * (128 * 2 + 16);
         static LdsReservation reserved, reserved_dq;
         hipError_t e = reserve_lds(reserved, {reinterpret_cast<const void*>(attention_bwd_dkv_kernel<128>)}, smem_dkv);
         ATS_REQUIRE(e == hipSuccess, ATS_ERR_LAUNCH, "ats_attention_bwd: cannot reserve %d bytes of LDS: %s", smem_dkv,
@@ -759,8 +844,7 @@ extern "C" int ats_attention_bwd_ex(const void* q, const void* k, const void* v,
         }
     } else {
         constexpr int smem_dq = 4 * kDqBN * 64 * 2 + 2 * kDqBN * 4;
-        constexpr int smem_dkv = 2 * kDkvBQ * (64 * 2 + 16) + 2 * kDkvBQ * (64 * 2 + 64) + 2 * kDkvBQ * 4 +
-                                 kBwdRows * (64 * 2 + 16);
+        constexpr int smem_dkv = 4 * kDkvBQ * 64 * 2 + 4 * kDkvBQ * 4 + kBwdRows * (64 * 2 + 16);
         if (extras) {
             hipLaunchKernelGGL((attention_bwd_dq_kernel<64, false, true>), dim3((unsigned)dq_blocks), dim3(256), smem_dq, s,
                                q_, k_, v_, do_, lse, delta, key_bias, static_cast<bf16_t*>(dq), Hq, Hkv, L, Lk, scale, B, ex);
