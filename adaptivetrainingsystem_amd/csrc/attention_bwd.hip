@@ -605,8 +605,8 @@ __device__ __forceinline__ void attention_bwd_dkv_tile(const bf16_t* __restrict_
             __builtin_amdgcn_s_setprio(0);
             const bool diagonal = q0 + off < key_wave_last;
             bu32x4_t pf[2], dsf[2];
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
+            // rows r of the accumulators (queries r*8 + g*4 + 0..3 of the step) -> words r%2*2, r%2*2+1 of pf / dsf [r/2]
+            auto exp_rows = [&](int r) {
                 const bf32x4_t l4 = *(blds_f4_t)(sL + par * kDkvBQ + r * 8 + g * 4);
                 const bf32x4_t d4 = *(blds_f4_t)(sD + par * kDkvBQ + r * 8 + g * 4);
                 const float lv[4] = {l4.x, l4.y, l4.z, l4.w};
@@ -645,11 +645,14 @@ __device__ __forceinline__ void attention_bwd_dkv_tile(const bf16_t* __restrict_
                 if (r == 1) { pf[0].z = p01; pf[0].w = p23; dsf[0].z = s01; dsf[0].w = s23; }
                 if (r == 2) { pf[1].x = p01; pf[1].y = p23; dsf[1].x = s01; dsf[1].y = s23; }
                 if (r == 3) { pf[1].z = p01; pf[1].w = p23; dsf[1].z = s01; dsf[1].w = s23; }
-            }
+            };
+            exp_rows(0);
+            exp_rows(1);
             // ---- dV^T += dO^T . P and dK^T += Q^T . dS  (queries of a k-step in accumulator order).  The
             //      transposing reads of pair i+1 (a fragment of dO^T and one of Q^T) are issued before the MFMAs
             //      of pair i: left to itself the compiler reuses one set of registers for every fragment and
-            //      each MFMA waits a full LDS latency
+            //      each MFMA waits a full LDS latency.  The exponentials of the second half of the step's queries
+            //      run between the MFMAs of the first half.
             __builtin_amdgcn_s_setprio(1);
             {
                 constexpr int NP = 2 * DB;   // pairs: (k-step s, d block) = (i / DB, i % DB)
@@ -658,6 +661,8 @@ __device__ __forceinline__ void attention_bwd_dkv_tile(const bf16_t* __restrict_
                 fq[0] = tr_fragment_swz(st, tlb, thb, 0);
 #pragma unroll
                 for (int i = 0; i < NP; ++i) {
+                    if (i == 0) exp_rows(2);
+                    if (i == DB / 2) exp_rows(3);
                     if (i + 1 < NP) {
                         const int s1 = (i + 1) / DB, d1 = (i + 1) % DB;
                         const int tl = tlb ^ (d1 << 6), th = thb ^ (d1 << 6);
