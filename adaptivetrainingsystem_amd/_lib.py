@@ -100,6 +100,8 @@ _SIGNATURES = {
                                      c_int, c_int, c_int, c_float, c_void_p, c_size_t, c_void_p]),
     "ats_attention_bwd_ex": (c_int, [c_void_p] * 8 + [c_int64, c_int64, c_float, c_uint64] + [c_void_p] * 3 + [c_int] * 6 +
                              [c_float, c_void_p]),
+    "ats_attention_bwd_out": (c_int, [c_void_p] * 9 + [c_int64, c_int64, c_float, c_uint64] + [c_void_p] * 3 + [c_int] * 6 +
+                              [c_float, c_void_p]),
     "ats_attention_softmax_f32": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_void_p,
                                           c_void_p, c_int64, c_int64, c_float, c_uint64, c_void_p]),
     "ats_attention_softmax_bwd_f32": (c_int, [c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_float,

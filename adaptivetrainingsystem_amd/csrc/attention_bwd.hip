@@ -148,7 +148,9 @@ __device__ __forceinline__ void attention_bwd_dq_tile(const bf16_t* __restrict__
                                                       const float* __restrict__ lse, const float* __restrict__ delta,
                                                       const float* __restrict__ key_bias, bf16_t* __restrict__ dq, int Hq,
                                                       int Hkv, int L, int Lk, float scale, int qt, int hq, int b,
-                                                      unsigned char* smem, const AttnExtra* ex = nullptr) {
+                                                      unsigned char* smem, const AttnExtra* ex = nullptr,
+                                                      const bf16_t* __restrict__ out_rows = nullptr,
+                                                      float* __restrict__ delta_w = nullptr) {
     static_assert(!(EXTRA && BIAS), "a per-key bias is folded into the pair bias");
     using SW = SwzTile<D>;
     constexpr int KS = D / 16;
@@ -181,7 +183,27 @@ __device__ __forceinline__ void attention_bwd_dq_tile(const bf16_t* __restrict__
         dof[s] = *reinterpret_cast<const bu32x4_t*>(dop + s * 16 + g * 8);
     }
     const float lse2 = lse[(int64_t)(b * Hq + hq) * L + q_clamped] * kLog2e;
-    const float dl = delta[(int64_t)(b * Hq + hq) * L + q_clamped];
+    // delta of this lane's query: given, or formed here from the forward's output row and the dO row that the
+    // lane holds anyway (lanes l and l + 32 hold the two halves of a row) and left behind for the dK/dV kernel
+    float dl;
+    if (out_rows != nullptr) {
+        const bf16_t* orow = out_rows + ((int64_t)b * L + q_clamped) * (int64_t)(Hq * D) + hq * D;
+        float part = 0.f;
+#pragma unroll
+        for (int s = 0; s < KS; ++s) {
+            const uint4 ov = *reinterpret_cast<const uint4*>(orow + s * 16 + g * 8);
+            const uint4 dv4 = make_uint4(dof[s].x, dof[s].y, dof[s].z, dof[s].w);
+            float fo[8], fd[8];
+            Elem<bf16_t>::unpack(ov, fo);
+            Elem<bf16_t>::unpack(dv4, fd);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) part += fo[j] * fd[j];
+        }
+        dl = part + __shfl_xor(part, 32, 64);
+        if (g == 0 && q_row < L) delta_w[(int64_t)(b * Hq + hq) * L + q_row] = dl;
+    } else {
+        dl = delta[(int64_t)(b * Hq + hq) * L + q_clamped];
+    }
     __amdgpu_buffer_rsrc_t pb_rsrc;
     int pb_row = 0;
     bool ex_bias = false, ex_drop = false;
@@ -368,7 +390,7 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dq_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k, const bf16_t* __restrict__ v,
     const bf16_t* __restrict__ dout, const float* __restrict__ lse, const float* __restrict__ delta,
     const float* __restrict__ key_bias, bf16_t* __restrict__ dq, int Hq, int Hkv, int L, int Lk, float scale, int B,
-    AttnExtra ex) {
+    AttnExtra ex, const bf16_t* __restrict__ out_rows, float* __restrict__ delta_w) {
     extern __shared__ __align__(16) unsigned char smem[];
     const int n_qt = (L + kBwdRows - 1) / kBwdRows;
     const int n_pairs = (n_qt + 1) / 2;
@@ -391,7 +413,7 @@ __global__ __launch_bounds__(256, 2) void attention_bwd_dq_kernel(
     for (int half = 0; half < 2; ++half) {
         if (half && pair == qt_long) break;
         attention_bwd_dq_tile<D, BIAS, EXTRA>(q, k, v, dout, lse, delta, key_bias, dq, Hq, Hkv, L, Lk, scale,
-                                              half ? pair : qt_long, hq, b, smem, &ex);
+                                              half ? pair : qt_long, hq, b, smem, &ex, out_rows, delta_w);
     }
 }
 
@@ -779,17 +801,23 @@ extern "C" int ats_attention_bwd(const void* q, const void* k, const void* v, co
                                 scale, stream);
 }
 
-extern "C" int ats_attention_bwd_ex(const void* q, const void* k, const void* v, const void* dout, const float* lse,
-                                    const float* delta, const float* key_bias, const float* bias_qk, int64_t bias_sb,
-                                    int64_t bias_sh, float dropout_p, uint64_t dropout_seed, void* dq, void* dk, void* dv, int B, int Hq,
-                                    int Hkv, int L, int Lk, int D, float scale, ats_stream_t stream) {
+// out == nullptr: delta is given.  Otherwise the dQ kernel forms delta from out and dout and writes it to
+// delta_ws, where the dK/dV kernel (launched behind it on the same stream) reads it.
+static int attention_bwd_launch(const void* q, const void* k, const void* v, const void* out, const void* dout,
+                                const float* lse, const float* delta, float* delta_ws, const float* key_bias,
+                                const float* bias_qk, int64_t bias_sb, int64_t bias_sh, float dropout_p,
+                                uint64_t dropout_seed, void* dq, void* dk, void* dv, int B, int Hq, int Hkv, int L, int Lk,
+                                int D, float scale, ats_stream_t stream) {
     using namespace ats;
     ATS_REQUIRE(B >= 0 && Hq > 0 && Hkv > 0 && Hq % Hkv == 0 && L >= 0 && Lk >= L && scale > 0.f, ATS_ERR_INVALID_ARG,
                 "ats_attention_bwd: B=%d Hq=%d Hkv=%d L=%d Lk=%d scale=%g", B, Hq, Hkv, L, Lk, scale);
     ATS_REQUIRE(D == 64 || D == 128, ATS_ERR_UNSUPPORTED, "ats_attention_bwd: head_dim %d (64 or 128)", D);
     if (B == 0 || L == 0) return ATS_OK;
-    ATS_REQUIRE(q && k && v && dout && lse && delta && dq && dk && dv, ATS_ERR_INVALID_ARG,
-                "ats_attention_bwd: null pointer");
+    ATS_REQUIRE(q && k && v && dout && lse && (out ? delta_ws != nullptr : delta != nullptr) && dq && dk && dv,
+                ATS_ERR_INVALID_ARG, "ats_attention_bwd: null pointer");
+    ATS_REQUIRE(!out || aligned16(out), ATS_ERR_INVALID_ARG, "ats_attention_bwd: misaligned pointer");
+    const bf16_t* out_ = static_cast<const bf16_t*>(out);
+    const float* delta_kv = out ? delta_ws : delta;   // what the dK/dV kernel reads
     ATS_REQUIRE(aligned16(q) && aligned16(k) && aligned16(v) && aligned16(dout) && aligned16(dq) && aligned16(dk) &&
                     aligned16(dv),
                 ATS_ERR_INVALID_ARG, "ats_attention_bwd: misaligned pointer");
@@ -830,21 +858,21 @@ extern "C" int ats_attention_bwd_ex(const void* q, const void* k, const void* v,
             ATS_REQUIRE(e == hipSuccess, ATS_ERR_LAUNCH, "ats_attention_bwd_ex: cannot reserve %d bytes of LDS: %s", smem_dkv,
                         hipGetErrorString(e));
             hipLaunchKernelGGL((attention_bwd_dq_kernel<128, false, true>), dim3((unsigned)dq_blocks), dim3(256), smem_dq, s,
-                               q_, k_, v_, do_, lse, delta, key_bias, static_cast<bf16_t*>(dq), Hq, Hkv, L, Lk, scale, B, ex);
+                               q_, k_, v_, do_, lse, delta, key_bias, static_cast<bf16_t*>(dq), Hq, Hkv, L, Lk, scale, B, ex, out_, delta_ws);
             hipLaunchKernelGGL((attention_bwd_dkv_kernel<128, true>), dim3((unsigned)dkv_blocks), dim3(256), smem_dkv, s, q_,
-                               k_, v_, do_, lse, delta, key_bias, static_cast<bf16_t*>(dk), static_cast<bf16_t*>(dv), Hq, Hkv,
+                               k_, v_, do_, lse, delta_kv, key_bias, static_cast<bf16_t*>(dk), static_cast<bf16_t*>(dv), Hq, Hkv,
                                L, Lk, scale, ex);
         } else {
             if (key_bias)
                 hipLaunchKernelGGL((attention_bwd_dq_kernel<128, true>), dim3((unsigned)dq_blocks), dim3(256), smem_dq, s,
                                    q_, k_, v_, do_, lse, delta, key_bias, static_cast<bf16_t*>(dq), Hq, Hkv, L, Lk, scale, B,
-                                   ex);
+                                   ex, out_, delta_ws);
             else
                 hipLaunchKernelGGL((attention_bwd_dq_kernel<128, false>), dim3((unsigned)dq_blocks), dim3(256), smem_dq, s,
                                    q_, k_, v_, do_, lse, delta, key_bias, static_cast<bf16_t*>(dq), Hq, Hkv, L, Lk, scale, B,
-                                   ex);
+                                   ex, out_, delta_ws);
             hipLaunchKernelGGL((attention_bwd_dkv_kernel<128>), dim3((unsigned)dkv_blocks), dim3(256), smem_dkv, s, q_, k_,
-                               v_, do_, lse, delta, key_bias, static_cast<bf16_t*>(dk), static_cast<bf16_t*>(dv), Hq, Hkv, L,
+                               v_, do_, lse, delta_kv, key_bias, static_cast<bf16_t*>(dk), static_cast<bf16_t*>(dv), Hq, Hkv, L,
                                Lk, scale, ex);
         }
     } else {
@@ -852,22 +880,40 @@ extern "C" int ats_attention_bwd_ex(const void* q, const void* k, const void* v,
         constexpr int smem_dkv = 4 * kDkvBQ * 64 * 2 + 4 * kDkvBQ * 4 + kBwdRows * (64 * 2 + 16);
         if (extras) {
             hipLaunchKernelGGL((attention_bwd_dq_kernel<64, false, true>), dim3((unsigned)dq_blocks), dim3(256), smem_dq, s,
-                               q_, k_, v_, do_, lse, delta, key_bias, static_cast<bf16_t*>(dq), Hq, Hkv, L, Lk, scale, B, ex);
+                               q_, k_, v_, do_, lse, delta, key_bias, static_cast<bf16_t*>(dq), Hq, Hkv, L, Lk, scale, B, ex, out_, delta_ws);
             hipLaunchKernelGGL((attention_bwd_dkv_kernel<64, true>), dim3((unsigned)dkv_blocks), dim3(256), smem_dkv, s, q_,
-                               k_, v_, do_, lse, delta, key_bias, static_cast<bf16_t*>(dk), static_cast<bf16_t*>(dv), Hq, Hkv,
+                               k_, v_, do_, lse, delta_kv, key_bias, static_cast<bf16_t*>(dk), static_cast<bf16_t*>(dv), Hq, Hkv,
                                L, Lk, scale, ex);
         } else {
             if (key_bias)
                 hipLaunchKernelGGL((attention_bwd_dq_kernel<64, true>), dim3((unsigned)dq_blocks), dim3(256), smem_dq, s, q_,
-                                   k_, v_, do_, lse, delta, key_bias, static_cast<bf16_t*>(dq), Hq, Hkv, L, Lk, scale, B, ex);
+                                   k_, v_, do_, lse, delta, key_bias, static_cast<bf16_t*>(dq), Hq, Hkv, L, Lk, scale, B, ex, out_, delta_ws);
             else
                 hipLaunchKernelGGL((attention_bwd_dq_kernel<64, false>), dim3((unsigned)dq_blocks), dim3(256), smem_dq, s, q_,
-                                   k_, v_, do_, lse, delta, key_bias, static_cast<bf16_t*>(dq), Hq, Hkv, L, Lk, scale, B, ex);
+                                   k_, v_, do_, lse, delta, key_bias, static_cast<bf16_t*>(dq), Hq, Hkv, L, Lk, scale, B, ex, out_, delta_ws);
             hipLaunchKernelGGL((attention_bwd_dkv_kernel<64>), dim3((unsigned)dkv_blocks), dim3(256), smem_dkv, s, q_, k_, v_,
-                               do_, lse, delta, key_bias, static_cast<bf16_t*>(dk), static_cast<bf16_t*>(dv), Hq, Hkv, L, Lk,
+                               do_, lse, delta_kv, key_bias, static_cast<bf16_t*>(dk), static_cast<bf16_t*>(dv), Hq, Hkv, L, Lk,
                                scale, ex);
         }
     }
     ATS_CHECK_LAUNCH("ats_attention_bwd");
     return ATS_OK;
+}
+
+extern "C" int ats_attention_bwd_ex(const void* q, const void* k, const void* v, const void* dout, const float* lse,
+                                    const float* delta, const float* key_bias, const float* bias_qk, int64_t bias_sb,
+                                    int64_t bias_sh, float dropout_p, uint64_t dropout_seed, void* dq, void* dk, void* dv, int B, int Hq,
+                                    int Hkv, int L, int Lk, int D, float scale, ats_stream_t stream) {
+    return attention_bwd_launch(q, k, v, nullptr, dout, lse, delta, nullptr, key_bias, bias_qk, bias_sb, bias_sh, dropout_p,
+                                dropout_seed, dq, dk, dv, B, Hq, Hkv, L, Lk, D, scale, stream);
+}
+
+extern "C" int ats_attention_bwd_out(const void* q, const void* k, const void* v, const void* out, const void* dout,
+                                     const float* lse, float* delta_ws, const float* key_bias, const float* bias_qk,
+                                     int64_t bias_sb, int64_t bias_sh, float dropout_p, uint64_t dropout_seed, void* dq,
+                                     void* dk, void* dv, int B, int Hq, int Hkv, int L, int Lk, int D, float scale,
+                                     ats_stream_t stream) {
+    ATS_REQUIRE(out != nullptr || B == 0 || L == 0, ATS_ERR_INVALID_ARG, "ats_attention_bwd_out: null pointer");
+    return attention_bwd_launch(q, k, v, out, dout, lse, nullptr, delta_ws, key_bias, bias_qk, bias_sb, bias_sh, dropout_p,
+                                dropout_seed, dq, dk, dv, B, Hq, Hkv, L, Lk, D, scale, stream);
 }

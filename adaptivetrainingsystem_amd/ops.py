@@ -959,15 +959,15 @@ def causal_attention_bwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out:
     key_bias, pair_bias, pair_sb, pair_sh = _attention_extras(key_bias, pair_bias, dropout_p, B, Hq, L, Lk, q,
                                                               "causal_attention_bwd")
     lib = _lib.load()
+    # delta = rowsum(dO * O) is formed inside the dQ kernel and handed to the dK/dV kernel through this buffer
     delta = torch.empty(B, Hq, L, dtype=torch.float32, device=q.device)
-    check(lib.ats_attention_delta(out.data_ptr(), dout.data_ptr(), delta.data_ptr(), B, Hq, L, D, _stream()),
-          "ats_attention_delta")
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
-    check(lib.ats_attention_bwd_ex(q.data_ptr(), k.data_ptr(), v.data_ptr(), dout.data_ptr(), lse.data_ptr(),
-                                   delta.data_ptr(), _ptr(key_bias), _ptr(pair_bias), pair_sb, pair_sh, float(dropout_p),
-                                   int(dropout_seed) & 0xFFFFFFFFFFFFFFFF, dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
-                                   B, Hq, Hkv, L, Lk, D, float(D ** -0.5 if scale is None else scale), _stream()),
-          "ats_attention_bwd_ex")
+    check(lib.ats_attention_bwd_out(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), dout.data_ptr(),
+                                    lse.data_ptr(), delta.data_ptr(), _ptr(key_bias), _ptr(pair_bias), pair_sb, pair_sh,
+                                    float(dropout_p), int(dropout_seed) & 0xFFFFFFFFFFFFFFFF, dq.data_ptr(), dk.data_ptr(),
+                                    dv.data_ptr(), B, Hq, Hkv, L, Lk, D, float(D ** -0.5 if scale is None else scale),
+                                    _stream()),
+          "ats_attention_bwd_out")
     return dq, dk, dv
 
 

@@ -444,6 +444,14 @@ int ats_attention_bwd_ex(const void* q, const void* k, const void* v, const void
                          const float* delta, const float* key_bias, const float* bias_qk, int64_t bias_sb,
                          int64_t bias_sh, float dropout_p, uint64_t dropout_seed, void* dq, void* dk, void* dv, int B,
                          int Hq, int Hkv, int L, int Lk, int D, float scale, ats_stream_t stream);
+/* ats_attention_bwd_ex without the separate ats_attention_delta launch: the dQ kernel, whose lanes hold the dO
+ * rows already, forms delta from them and the forward's output `out` [B,L,Hq*D] and writes it to delta_ws
+ * [B,Hq,L] (float32, caller's), where the dK/dV kernel behind it reads it.  Same gradient as autograd's for
+ * model.py:757-839; delta is summed in another order than ats_attention_delta sums it (float32 rounding). */
+int ats_attention_bwd_out(const void* q, const void* k, const void* v, const void* out, const void* dout,
+                          const float* lse, float* delta_ws, const float* key_bias, const float* bias_qk,
+                          int64_t bias_sb, int64_t bias_sh, float dropout_p, uint64_t dropout_seed, void* dq, void* dk,
+                          void* dv, int B, int Hq, int Hkv, int L, int Lk, int D, float scale, ats_stream_t stream);
 
 /* ---- Float32 attention: the row softmax between two grouped products --------------
  * _standard_attention on float32 tensors (model.py:807-839) materialises the scores; so does this path:

@@ -209,6 +209,44 @@ def test_causal_attention_backward(ops, gpu, B, Hq, Hkv, L, Lk, D):
     assert rel_err(dk, rk) <= GRAD_TOL
 
 
+@pytest.mark.parametrize("B,Hq,Hkv,L,Lk,D", [(2, 4, 2, 200, 200, 128), (1, 8, 2, 300, 300, 64), (1, 4, 2, 70, 300, 64),
+                                             (1, 2, 2, 31, 31, 64)])
+def test_causal_attention_backward_given_delta(ops, gpu, B, Hq, Hkv, L, Lk, D):
+    """ats_attention_delta + ats_attention_bwd (delta computed by its own kernel and passed in) against the oracle
+    and against the entry point that forms delta inside the dQ kernel (what ops.causal_attention_bwd calls)."""
+    from adaptivetrainingsystem_amd import _lib
+    print("case attention backward, given delta", B, Hq, Hkv, L, Lk, D, flush=True)
+    g = gen(197)
+    q = torch.randn(B, Hq, L, D, generator=g).bfloat16()
+    k = torch.randn(B, Hkv, Lk, D, generator=g).bfloat16()
+    v = torch.randn(B, Hkv, Lk, D, generator=g).bfloat16()
+    dout = torch.randn(B, L, Hq * D, generator=g).bfloat16()
+    rq, rk, rv = _oracle_attention_grads(q, k, v, dout, Hq // Hkv)
+    qg, kg, vg, dg = q.to(gpu), k.to(gpu), v.to(gpu), dout.to(gpu)
+    out, lse = ops.causal_attention(qg, kg, vg, return_lse=True)
+    lib = _lib.load()
+    stream = torch.cuda.current_stream().cuda_stream
+    delta = torch.empty(B, Hq, L, dtype=torch.float32, device=gpu)
+    assert lib.ats_attention_delta(out.data_ptr(), dg.data_ptr(), delta.data_ptr(), B, Hq, L, D, stream) == 0
+    ref_delta = (out.float() * dg.float()).view(B, L, Hq, D).sum(-1).permute(0, 2, 1)
+    assert rel_err(delta, ref_delta) <= 1e-5
+    dq, dk, dv = torch.empty_like(qg), torch.empty_like(kg), torch.empty_like(vg)
+    assert lib.ats_attention_bwd(qg.data_ptr(), kg.data_ptr(), vg.data_ptr(), dg.data_ptr(), lse.data_ptr(),
+                                 delta.data_ptr(), None, dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), B, Hq, Hkv, L, Lk, D,
+                                 float(D ** -0.5), stream) == 0
+    for got, ref in ((dq, rq), (dk, rk), (dv, rv)):
+        assert rel_err(got, ref) <= GRAD_TOL
+    # the fused entry point leaves the same delta behind (summed in another order) and the same gradients
+    delta2 = torch.full((B, Hq, L), float("nan"), dtype=torch.float32, device=gpu)
+    dq2, dk2, dv2 = torch.empty_like(qg), torch.empty_like(kg), torch.empty_like(vg)
+    assert lib.ats_attention_bwd_out(qg.data_ptr(), kg.data_ptr(), vg.data_ptr(), out.data_ptr(), dg.data_ptr(),
+                                     lse.data_ptr(), delta2.data_ptr(), None, None, 0, 0, 0.0, 0, dq2.data_ptr(),
+                                     dk2.data_ptr(), dv2.data_ptr(), B, Hq, Hkv, L, Lk, D, float(D ** -0.5), stream) == 0
+    assert rel_err(delta2, ref_delta) <= 1e-5
+    for got, ref in ((dq2, dq), (dk2, dk), (dv2, dv)):
+        assert rel_err(got, ref) <= 1e-2
+
+
 def test_attention_function_autograd(gpu):
     """The autograd Function: strided q/k/v views in, gradient accumulation through views out."""
     from adaptivetrainingsystem_amd.autograd import AttentionFunction

@@ -77,6 +77,8 @@ def test_argument_errors_return_codes_not_exits():
     assert lib.ats_attention_bwd(*([None] * 10), 1, 4, 2, 16, 8, 128, 0.1, None, 0, None) == -1
     assert lib.ats_attention_bwd(*([None] * 10), 1, 4, 2, 16, 16, 32, 0.1, None) == -2
     assert lib.ats_attention_delta(None, None, None, 1, 4, 16, 80, None) == -2
+    assert lib.ats_attention_bwd_out(*([None] * 9), 0, 0, 0.0, 0, None, None, None, 1, 4, 2, 16, 16, 128, 0.1, None) == -1
+    assert lib.ats_attention_bwd_out(*([None] * 9), 0, 0, 0.0, 0, None, None, None, 0, 4, 2, 16, 16, 128, 0.1, None) == 0
     # K slices: I must be k_splits whole slabs, and only weight-streaming sizes (<= 48 rows per expert)
     one = ctypes.c_void_p(16)
     assert lib.ats_grouped_down_splitk(one, one, one, one, one, 8, 128, 128, 4096, 14336, 3, 1, None) == -2
