@@ -487,8 +487,8 @@ def run_attention_train(args):
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": {"workload": f"attention_train: causal GQA forward + backward, batch {B}, seq {L}, {Hq} query / "
                                f"{Hkv} kv heads, head_dim {D}"},
-        "roofline": {"kernel": "attention_fwd_kernel + attention_bwd_dq_kernel + attention_bwd_dkv_kernel (with the "
-                               "transposes and the delta kernel)", "bound": "mfma", "achieved": achieved,
+        "roofline": {"kernel": "attention_fwd_kernel + attention_bwd_dq_kernel (forms delta) + "
+                               "attention_bwd_dkv_kernel", "bound": "mfma", "achieved": achieved,
                      "peak": PEAK_MFMA_BF16_TFLOPS, "unit": "TFLOP/s", "frac": achieved / PEAK_MFMA_BF16_TFLOPS,
                      "traffic": None},
         "stages_ms": {s_: round(v_["mean_ms"], 4) for s_, v_ in st.items()},

@@ -245,3 +245,32 @@ def test_attention_full_size_properties_and_sampled_rows(gpu):
             pj = torch.exp(s - lse[b, h, j:].cpu()).bfloat16().float()
             ref += pj @ dout.view(B, L, Hq, D)[b, j:, h].float().cpu()
         assert (dv[b, kv, j].float().cpu() - ref).abs().max().item() <= BF16_TOL * max(ref.abs().max().item(), 1e-3), (b, kv, j)
+    # the gradients are linear in dout, and doubling is exact in every format on the way
+    q2, k2, v2 = ops.causal_attention_bwd(qg, kg, vg, out, lse, dout * 2)
+    assert torch.equal(q2, dq * 2) and torch.equal(k2, dk * 2) and torch.equal(v2, dv * 2)
+    # sampled rows of dQ and dK from float32 arithmetic on the host:
+    # dS[i, j] = P[i, j] (dO[i].V[j] - dO[i].O[i]) scale, dQ[i] = sum_j dS[i, j] K[j], dK[j] = sum_{h, i} dS[i, j] Q[i]
+    out_c, lse_c, do_c = out.float().cpu().view(B, L, Hq, D), lse.cpu(), dout.float().cpu().view(B, L, Hq, D)
+    scale = D ** -0.5
+
+    def ds_block(b, h, kv, rows, cols):
+        s_ = q[b, h, rows].float() @ k[b, kv, cols].float().T * scale
+        p_ = torch.exp(s_ - lse_c[b, h, rows][:, None])
+        p_ = torch.where(cols[None, :] <= rows[:, None], p_, torch.zeros(()))
+        dp_ = do_c[b, rows, h] @ v[b, kv, cols].float().T
+        dl_ = (do_c[b, rows, h] * out_c[b, rows, h]).sum(-1, keepdim=True)
+        return p_ * (dp_ - dl_) * scale
+
+    for n, i in enumerate([0, 63, 1000, L - 1]):
+        b, h = (n + 1) % B, (5 * n + 2) % Hq
+        kv = h // (Hq // Hkv)
+        rows, cols = torch.tensor([i]), torch.arange(i + 1)
+        ref = (ds_block(b, h, kv, rows, cols) @ k[b, kv, cols].float())[0]
+        assert (dq[b, h, i].float().cpu() - ref).abs().max().item() <= BF16_TOL * max(ref.abs().max().item(), 1e-3), (b, h, i)
+    for n, j in enumerate([0, 129, 1200, L - 1]):
+        b, kv = (n + 2) % B, (3 * n + 1) % Hkv
+        rows, cols = torch.arange(j, L), torch.tensor([j])
+        ref = torch.zeros(D)
+        for h in range(kv * (Hq // Hkv), (kv + 1) * (Hq // Hkv)):
+            ref += (ds_block(b, h, kv, rows, cols).T @ q[b, h, rows].float())[0]
+        assert (dk[b, kv, j].float().cpu() - ref).abs().max().item() <= BF16_TOL * max(ref.abs().max().item(), 1e-3), (b, kv, j)
