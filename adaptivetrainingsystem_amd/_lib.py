@@ -45,6 +45,12 @@ _SIGNATURES = {
     "ats_grouped_down_dgrad_dsilu_supported": (c_int, [c_int, c_int64, c_int, c_int, c_int]),
     "ats_grouped_down_dgrad_dsilu": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64,
                                              c_int, c_int, c_int, c_void_p, c_int64, c_void_p, c_void_p]),
+    "ats_grouped_down_dgrad_dsilu_nn_supported": (c_int, [c_int, c_int64, c_int, c_int, c_int]),
+    "ats_grouped_down_dgrad_dsilu_nn": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int64,
+                                                c_int, c_int, c_int, c_void_p, c_int64, c_void_p, c_void_p]),
+    "ats_grouped_gemm_nn_supported": (c_int, [c_int, c_int64, c_int, c_int, c_int64, c_int]),
+    "ats_grouped_gemm_nn": (c_int, [c_void_p, c_int64, c_int64, c_void_p, c_int, c_void_p, c_int64, c_void_p, c_int64,
+                                    c_void_p, c_void_p, c_int, c_int64, c_int, c_int, c_int, c_int, c_void_p]),
     "ats_grouped_gateup_swiglu_save_supported": (c_int, [c_int64, c_int, c_int64, c_int, c_int, c_int]),
     "ats_grouped_gateup_swiglu_save": (c_int, [c_void_p, c_int64, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
                                                c_void_p, c_int, c_int64, c_int, c_int, c_int, c_void_p, c_int64,

@@ -197,6 +197,10 @@ class SwiGLUFunction(Function):
 # Whether the fused bfloat16 training kernels also write the transposed copies of h and dgu that the weight-gradient
 # products contract over (otherwise separate transposing passes produce them; same bits either way).
 FUSE_TRANSPOSED_COPIES = True
+# Data gradients of the expert products read the weights as the forward holds them ([out, in], the reduction
+# index along the rows) where the K-major kernel applies (bfloat16, prefill-sized groups), instead of multiplying
+# by a transposed copy made per step.
+DGRAD_FROM_FORWARD_WEIGHTS = True
 
 
 def _ffn_forward(x, wgu, wd, offsets, kept, rows, row_src, k, want_wgrad=False):
@@ -231,21 +235,29 @@ def _ffn_backward(dy, x, wgu, wd, gu, h, offsets, kept, rows, row_src, k, need_x
     dtype, dev = x.dtype, x.device
     if need_w and wplan is None:
         wplan = ops.wgrad_plan(kept)
-    wdT, tab_dT = ops.transpose_batched(wd)                      # [I, H] per expert; kept alive until return
     dguT = None
-    pair = ops.grouped_down_dgrad_dsilu(dy, tab_dT, gu, offsets, kept, rows, H, I,       # prefill-sized groups:
-                                        t_col0=wplan[0] if need_w and FUSE_TRANSPOSED_COPIES else None)   # one kernel
+    t_col0 = wplan[0] if need_w and FUSE_TRANSPOSED_COPIES else None
+    if DGRAD_FROM_FORWARD_WEIGHTS and ops.grouped_down_dgrad_dsilu_supported(E, rows, H, I, dtype, transposed_weights=False):
+        # prefill-sized bfloat16 groups: one kernel, reading the down weights as the forward holds them
+        pair = ops.grouped_down_dgrad_dsilu(dy, ops.weight_pointer_table(list(wd)), gu, offsets, kept, rows, H, I,
+                                            t_col0=t_col0, transposed_weights=False)
+    else:
+        wdT, tab_dT = ops.transpose_batched(wd)                  # [I, H] per expert; kept alive until return
+        pair = ops.grouped_down_dgrad_dsilu(dy, tab_dT, gu, offsets, kept, rows, H, I, t_col0=t_col0)   # one kernel
     dgu = None
     if pair is not None:
         dgu, dguT = pair
-    if dgu is None:
+    if dgu is None:                                              # smaller groups, float32: two kernels
         dh = ops.grouped_gemm_nt(tab_dT, H, I, offsets, kept, rows, rows, I, H, a=dy)
         dgu = torch.empty_like(gu)
         ops.silu_mul_bwd(gu[:, :I], gu[:, I:], dh, da=dgu[:, :I], db=dgu[:, I:], rows_dev=offsets[-1:])
     dx_rows = dwgu = dwd = None
     if need_x:
-        wguT, tab_guT = ops.transpose_batched(wgu)               # [H, 2I] per expert
-        dx_rows = ops.grouped_gemm_nt(tab_guT, 2 * I, H, offsets, kept, rows, rows, H, 2 * I, a=dgu)
+        if DGRAD_FROM_FORWARD_WEIGHTS and ops.grouped_gemm_nn_supported(E, rows, H, 2 * I, H, dtype):
+            dx_rows = ops.grouped_gemm_nn(ops.weight_pointer_table(list(wgu)), H, offsets, kept, rows, rows, H, 2 * I, dgu)
+        else:
+            wguT, tab_guT = ops.transpose_batched(wgu)           # [H, 2I] per expert
+            dx_rows = ops.grouped_gemm_nt(tab_guT, 2 * I, H, offsets, kept, rows, rows, H, 2 * I, a=dgu)
     if need_w:
         ks, kc = wplan
         ld = ops.wgrad_padded_rows(rows, E)

@@ -1024,11 +1024,16 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_dma_kernel(GroupedAr
 }
 
 // bf16 prefill tile on v_mfma_f32_16x16x32_bf16.  Same data movement as grouped_gemm_dma_kernel (256 x 256 tile,
-// 8 waves of 128 x 64, direct-to-LDS slabs, three activation stages and two weight stages, the XOR swizzle
-// also spreads the 16 rows x 4 chunks of a 16-row fragment over all banks), but the products are formed by
-// the 16 x 16 x 32 instruction: with random bf16 operands the chip, which is power limited on this kernel,
-// sustains about 14 % more of them per second than of the 32 x 32 x 16 form (measured on MFMA-only loops:
+// 8 waves of 128 x 64, direct-to-LDS slabs, three activation stages and two weight stages), but the products
+// are formed by the 16 x 16 x 32 instruction: with random bf16 operands the chip, which is power limited on this
+// kernel, sustains about 14 % more of them per second than of the 32 x 32 x 16 form (measured on MFMA-only loops:
 // 2.13 vs 1.86 PFLOP/s).
+// Swizzle: slot s of row R holds chunk s ^ (R & 7).  A fragment read has lane l on row l % 16 and chunk
+// 4 ks + l / 16; measured with the bank-conflict counter on a stand-alone kernel that issues only this read, the
+// hardware serves it in 4 cycles (no conflict), while the f(R) = (R & 7) ^ ((R >> 3) & 1) of the 32 x 32 x 16 kernel,
+// which a model of 16 consecutive lanes per cycle prefers, takes 8 (SQ_LDS_BANK_CONFLICT = half of
+// SQ_LDS_IDX_ACTIVE, also over the whole GEMM launch): the lanes that share a cycle are not 16 consecutive ones.
+// LDS was busy 60 % of this kernel's cycles with that conflict; without it the prefill step is 0.45 % faster.
 //
 // A 64-element slab is two 32-element k-steps; the wave's 128 rows are two halves of four 16-row fragments.
 // A slab is four phases of 16 MFMAs, (k-step, row half) = (0,0) (0,1) (1,0) (1,1); fragments live in two
@@ -1053,9 +1058,22 @@ __global__ __launch_bounds__(WM* WN * 64) void grouped_gemm_dma_kernel(GroupedAr
 // barrier) at raised priority and drops back at the top of the next slab: 1 % at both shapes and on the training
 // step (s_setprio 1, 2 or 3, and keeping it through phase 0, measure the same at the prefill shape; raising it for
 // phases 0-2 instead loses 0.2 %).
-template <typename TO, int SM, int SN, bool SWIGLU, bool SAVEGU = false, bool DSILU = false>
-__global__ __launch_bounds__(512) void grouped_gemm_dma16_kernel(GroupedArgs p) {
+//
+// BKM: the weight operand is stored [K][N] (K-major: the reduction index walks rows of p.ldb elements) instead
+// of [N][K].  That is the layout of the forward's own weights as the backward's data gradients need them
+// (dx = dy . W with W [N_fwd = K][K_fwd = N]), so no transposed copy of the weights is made per step.  A slab of
+// it is 64 rows of 256 output columns (512 bytes, again 32 KiB a stage); a weight fragment (16 output columns x
+// 32 reduction steps) comes out through the transposing read ds_read_b64_tr_b16: a group of 16 lanes reads a
+// block of 4 rows x 32 bytes and lane i receives its column i, two reads give a lane its 8 consecutive reduction
+// steps - the same register contents as the 16-byte read of the [N][K] layout, so both layouts give the same
+// bits.  The 32-byte chunks of a row are swizzled on the global side, chunk c of stage row r lands in slot
+// c ^ f(r), f(r) = (r % 4) | ((r / 8) % 4) << 2: the 16 row pieces that one read instruction touches fall on 16
+// different slots, i.e. on all banks once.
+template <typename TO, int SM, int SN, bool SWIGLU, bool SAVEGU = false, bool DSILU = false, bool BKM = false>
+__device__ __forceinline__ void grouped_gemm_dma16_body(const GroupedArgs& p, unsigned char* smem,
+                                                         const int32_t* __restrict__ row_count) {
 #if defined(__HIP_DEVICE_COMPILE__)
+    static_assert(!BKM || (!SWIGLU && !SAVEGU), "the K-major weight layout serves the plain product and the dgrad epilogue");
     typedef bf16_t T;
     constexpr int BM = 256, BN = 256, WM = 2, WN = 4;
     constexpr int NW = WM * WN;
@@ -1069,12 +1087,11 @@ __global__ __launch_bounds__(512) void grouped_gemm_dma16_kernel(GroupedArgs p) 
     constexpr int B_STAGE = BN * 128;
     constexpr int B_BASE = 3 * A_STAGE;
 
-    extern __shared__ __align__(16) unsigned char smem[];
     typedef __attribute__((address_space(3))) void* lds_ptr_t;
 
     TileCoord tc;
     if (!decode_tile_wave(blockIdx.x, p.row_count, p.E, BM, p.n_tiles, p.sm, p.sn, p.aligned_bands != 0, &tc)) return;
-    const int count = p.row_count[tc.e];
+    const int count = row_count[tc.e];
     const int row0 = p.row_start[tc.e];
     const int K = p.k_count ? p.k_count[tc.e] : p.K;
     const T* Bexp = static_cast<const T*>(p.b[tc.e]);
@@ -1095,7 +1112,7 @@ __global__ __launch_bounds__(512) void grouped_gemm_dma16_kernel(GroupedArgs p) 
     const __amdgpu_buffer_rsrc_t rsrc_b =
         __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(Bexp), 0, (int)p.b_extent_bytes, kRsrcFlags);
     const int drow = lane >> 3;
-    const int dchunk = (lane & 7) ^ drow ^ (wave & 1);
+    const int dchunk = (lane & 7) ^ drow;
     unsigned ao[NIA], bo[NIB];
     // the gather indices are asked for first: the weight loads issued below are in flight while they arrive
     int a_idx[NIA];
@@ -1107,6 +1124,15 @@ __global__ __launch_bounds__(512) void grouped_gemm_dma16_kernel(GroupedArgs p) 
     }
 #pragma unroll
     for (int j = 0; j < NIB; ++j) {
+        if constexpr (BKM) {
+            // instruction j of this wave fills stage rows 2 (j NW + wave), + 1: lane l the 16 bytes l % 32 of row l / 32
+            const int r = 2 * (j * NW + wave) + (lane >> 5);
+            const int f = (r & 3) | (((r >> 3) & 3) << 2);
+            int n = tc.nt * BN + ((lane & 31) ^ (f << 1)) * 8;
+            n = n <= p.N_out - 8 ? n : p.N_out - 8;      // columns past the end repeat the last eight (never stored)
+            bo[j] = (unsigned)(((int64_t)r * p.ldb + n) * ES);
+            continue;
+        }
         const int rb = (j * NW + wave) * 8 + drow;
         int n, brow;
         if (SWIGLU) {
@@ -1135,7 +1161,7 @@ __global__ __launch_bounds__(512) void grouped_gemm_dma16_kernel(GroupedArgs p) 
     // ---- fragment addresses: one register per k-step and operand; fragments and weight stages by offset
     const int frow = lane & 15;
     const int kgrp = lane >> 4;
-    const int fsw = (frow & 7) ^ ((frow >> 3) & 1);
+    const int fsw = frow & 7;
     const unsigned char* fa_addr[2];
     const unsigned char* fb_addr[2];
 #pragma unroll
@@ -1144,6 +1170,20 @@ __global__ __launch_bounds__(512) void grouped_gemm_dma16_kernel(GroupedArgs p) 
         fa_addr[ks] = smem + (wm * (BM / WM) + frow) * 128 + slot * 16;
         fb_addr[ks] = smem + B_BASE + (wn * (SWIGLU ? BN / WN / 2 : BN / WN) + frow) * 128 + slot * 16;
     }
+    // K-major weights: fragment j of a k-step sits in slot ((wn ^ q) << 2 | (j ^ t)) of rows 8 q + t (+ 4), lane
+    // 16 q + i, t = i / 4, 8 (i % 4) bytes in; k-step and stage are immediate offsets
+    typedef short tr4_t __attribute__((ext_vector_type(4)));
+    typedef __attribute__((address_space(3))) tr4_t* lds_tr_ptr_t;
+    typedef __attribute__((address_space(3))) unsigned char* lds_u8_t;
+    lds_u8_t fb_tr[TN];
+    if constexpr (BKM) {
+        const int t4 = frow >> 2;
+        const int base0 = B_BASE + (8 * kgrp + t4) * 512 + 8 * (frow & 3) + (((wn ^ kgrp) & 3) << 2) * 32;
+#pragma unroll
+        for (int j = 0; j < TN; ++j) fb_tr[j] = (lds_u8_t)smem + base0 + ((j ^ t4) * 32);
+    }
+    const int b_slab = BKM ? (int)(p.ldb * 128) : 128;   // bytes from one slab of the weight operand to the next
+    constexpr int RB2 = BKM ? 4 : 2;   // read instructions of two weight fragments
     u32x4_t fa[2][4], fb[2][TN];
 
 #define D16_ISSUE_A(kt_, aoff_)                                                                        \
@@ -1158,7 +1198,7 @@ __global__ __launch_bounds__(512) void grouped_gemm_dma16_kernel(GroupedArgs p) 
                                              ao[j_], (kt_) * 128, 0, 0)
 #define D16_ISSUE_B(kt_, stage_)                                                                       \
     {                                                                                                  \
-        const int soff = (kt_) * 128;                                                                  \
+        const int soff = (kt_) * b_slab;                                                               \
         _Pragma("unroll") for (int j = 0; j < NIB; ++j)                                                \
             __builtin_amdgcn_raw_ptr_buffer_load_lds(                                                  \
                 rsrc_b, (lds_ptr_t)(dma_b + (stage_) * B_STAGE + j * NW * 1024), 16, bo[j], soff, 0, 0); \
@@ -1170,8 +1210,18 @@ __global__ __launch_bounds__(512) void grouped_gemm_dma16_kernel(GroupedArgs p) 
         _Pragma("unroll") for (int i = 0; i < 4; ++i)                                                  \
             fa[buf_][i] = *reinterpret_cast<const u32x4_t*>(fa_ + i * 2048);                           \
     }
-#define D16_READ_B(stage_, ks_, j_, buf_) \
-    fb[buf_][j_] = *reinterpret_cast<const u32x4_t*>(fb_addr[ks_] + (stage_) * B_STAGE + D16_B_ROW(j_) * 128)
+#define D16_READ_B(stage_, ks_, j_, buf_)                                                              \
+    if constexpr (BKM) {                                                                               \
+        union {                                                                                        \
+            tr4_t t[2];                                                                                \
+            u32x4_t u;                                                                                 \
+        } cv_;                                                                                         \
+        const lds_u8_t pb_ = fb_tr[j_] + (stage_) * B_STAGE + (ks_) * (32 * 512);                      \
+        cv_.t[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr_t)(pb_));                       \
+        cv_.t[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_tr_ptr_t)(pb_ + 4 * 512));             \
+        fb[buf_][j_] = cv_.u;                                                                          \
+    } else                                                                                             \
+        fb[buf_][j_] = *reinterpret_cast<const u32x4_t*>(fb_addr[ks_] + (stage_) * B_STAGE + D16_B_ROW(j_) * 128)
 #define D16_MMA(bbuf_, abuf_, half_)                                                                   \
     {                                                                                                  \
         _Pragma("unroll") for (int j = 0; j < TN; ++j)                                                 \
@@ -1197,9 +1247,14 @@ __global__ __launch_bounds__(512) void grouped_gemm_dma16_kernel(GroupedArgs p) 
         __builtin_amdgcn_sched_group_barrier(SG_MFMA, 1, 0);                            \
         __builtin_amdgcn_sched_group_barrier(SG_VMEM, 1, 0);                            \
     }
-// phase 3: a fragment read per MFMA over the first half, a load per two MFMAs over the second
+// phase 3: a fragment read per MFMA over the first half (K-major weights: their four fragments take two read
+// instructions each), a load per two MFMAs over the second
 #define D16_MIX_DMA()                                                                   \
-    _Pragma("unroll") for (int g_ = 0; g_ < 8; ++g_) {                                  \
+    _Pragma("unroll") for (int g_ = 0; g_ < 4; ++g_) {                                  \
+        __builtin_amdgcn_sched_group_barrier(SG_DS_RD, BKM ? 2 : 1, 0);                 \
+        __builtin_amdgcn_sched_group_barrier(SG_MFMA, 1, 0);                            \
+    }                                                                                   \
+    _Pragma("unroll") for (int g_ = 0; g_ < 4; ++g_) {                                  \
         __builtin_amdgcn_sched_group_barrier(SG_DS_RD, 1, 0);                           \
         __builtin_amdgcn_sched_group_barrier(SG_MFMA, 1, 0);                            \
     }                                                                                   \
@@ -1223,7 +1278,7 @@ __global__ __launch_bounds__(512) void grouped_gemm_dma16_kernel(GroupedArgs p) 
             D16_READ_B(STG, 1, 0, 1);                                                   \
             D16_READ_B(STG, 1, 1, 1);                                                   \
             D16_MMA(0, 0, 0);                                                           \
-            D16_MIX(H1 ? 6 : 2, 1);                                                     \
+            D16_MIX((H1 ? 4 : 0) + RB2, 1);                                             \
         }                                                                               \
         PL_FENCE();                                                                     \
         D16_ISSUE_A1(ka_, sa_far, 1);                                                   \
@@ -1234,7 +1289,7 @@ __global__ __launch_bounds__(512) void grouped_gemm_dma16_kernel(GroupedArgs p) 
         }                                                                               \
         if (H1) {                                                                       \
             D16_MMA(0, 1, 1);                                                           \
-            D16_MIX(6, 1);                                                              \
+            D16_MIX(4 + RB2, 1);                                                        \
         }                                                                               \
         PL_FENCE();                                                                     \
         D16_ISSUE_A1(ka_, sa_far, 2);                                                   \
@@ -1336,6 +1391,18 @@ __global__ __launch_bounds__(512) void grouped_gemm_dma16_kernel(GroupedArgs p) 
         }
     }
 #endif
+}
+
+template <typename TO, int SM, int SN, bool SWIGLU, bool SAVEGU = false, bool DSILU = false, bool BKM = false>
+__global__ __launch_bounds__(512) void grouped_gemm_dma16_kernel(GroupedArgs p) {
+    // The body is a function of its own for one reason: a __restrict__ parameter that it reads through gives every
+    // other memory access in it (the transposing LDS reads among them) "does not alias that parameter" metadata once
+    // it is inlined here, and the compiler's wait insertion takes an LDS read that carries alias metadata but no
+    // scope of a direct-to-LDS load as independent of the loads in flight.  Without it every ds_read_b64_tr_b16 of
+    // the K-major variant is preceded by s_waitcnt vmcnt(0), i.e. waits for all of the slab loads just issued (the
+    // plain 16-byte fragment reads carry type-based alias metadata and never had that wait): 27-37 % slower.
+    extern __shared__ __align__(16) unsigned char smem_k[];
+    grouped_gemm_dma16_body<TO, SM, SN, SWIGLU, SAVEGU, DSILU, BKM>(p, smem_k, p.row_count);
 }
 
 #undef PL_STORE
@@ -1525,6 +1592,39 @@ static int launch_down_dgrad_dsilu(const GroupedArgs& p0, int64_t max_rows, hipS
     return ATS_OK;
 }
 
+// Products against weights stored [K][N] (the forward's own weights in the backward's data gradients): the
+// prefill tile of the bfloat16 direct-to-LDS kernel only; other group sizes and types multiply by a transposed copy.
+static bool kmajor_supported(int E, int64_t max_rows, int N, int K, int64_t ldb, int64_t min_avg_rows) {
+    if (E <= 0 || max_rows / E <= min_avg_rows || K % 64 != 0 || N % 8 != 0 || N < 8 || ldb % 8 != 0 || ldb < N) return false;
+    return extent32_ok(K, ldb, 2);
+}
+
+template <typename TO, bool DSILU>
+static int launch_kmajor(const GroupedArgs& p0, int64_t max_rows, hipStream_t s) {
+    constexpr int BM = 256, BN = 256;
+    GroupedArgs p = p0;
+    p.n_tiles = (p.N_out + BN - 1) / BN;
+    constexpr size_t smem = dma_lds_bytes(BM, BN);
+    auto kern = grouped_gemm_dma16_kernel<TO, 4, 8, false, false, DSILU, true>;
+    static LdsReservation reserved;
+    hipError_t e = reserve_lds(reserved, {reinterpret_cast<const void*>(kern)}, (int)smem);
+    if (e != hipSuccess) {
+        set_error("grouped GEMM: cannot reserve %zu bytes of LDS: %s", smem, hipGetErrorString(e));
+        return ATS_ERR_LAUNCH;
+    }
+    p.sm = 4;
+    p.sn = 8;
+    pick_supertile(p.n_tiles, &p.sm, &p.sn);
+    p.aligned_bands = max_rows / (p.E > 0 ? p.E : 1) >= kAlignedBandsMinAvgRows ? 1 : 0;
+    const int64_t blocks = grid_blocks(max_rows, p.E, BM, p.n_tiles, p.sm, p.sn, p.aligned_bands != 0);
+    if (blocks > 0x7fffffffLL) {
+        set_error("grouped GEMM: grid of %lld blocks", (long long)blocks);
+        return ATS_ERR_UNSUPPORTED;
+    }
+    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(512), smem, s, p);
+    return ATS_OK;
+}
+
 // Bytes reachable from a buffer descriptor, or 0 when they do not fit its 32-bit range.
 static uint32_t extent32(int64_t rows, int64_t row_elems, int elem_size) {
     if (rows <= 0 || rows > (int64_t)0xffffffffLL / (row_elems * elem_size)) return 0;
@@ -1665,6 +1765,108 @@ extern "C" int ats_grouped_down_dgrad_dsilu(const void* dy, const void* const* w
     rc = dtype == ATS_F32 ? launch_down_dgrad_dsilu<float>(p, max_rows, s) : launch_down_dgrad_dsilu<bf16_t>(p, max_rows, s);
     if (rc != ATS_OK) return rc;
     ATS_CHECK_LAUNCH("ats_grouped_down_dgrad_dsilu");
+    return ATS_OK;
+}
+
+extern "C" int ats_grouped_down_dgrad_dsilu_nn_supported(int E, int64_t max_rows, int H, int I, int dtype) {
+    using namespace ats;
+    if (H <= 0 || I <= 0 || dtype != ATS_BF16) return 0;
+    return kmajor_supported(E, max_rows, I, H, I, kDsiluMinAvgRows) ? 1 : 0;
+}
+extern "C" int ats_grouped_down_dgrad_dsilu_nn(const void* dy, const void* const* w_d, const void* gu, void* dgu,
+                                               const int32_t* row_start, const int32_t* row_count, int E,
+                                               int64_t max_rows, int H, int I, int dtype, void* dgu_t, int64_t ld_t,
+                                               const int32_t* t_col0, ats_stream_t stream) {
+    using namespace ats;
+    const char* name = "ats_grouped_down_dgrad_dsilu_nn";
+    int rc = check_common(name, dy, w_d, dgu, row_start, row_count, E, max_rows, H, I, dtype);
+    if (rc != ATS_OK) return rc;
+    rc = check_transposed(name, dgu_t, ld_t, t_col0, max_rows, E, dtype);
+    if (rc != ATS_OK) return rc;
+    ATS_REQUIRE(gu && aligned16(gu), ATS_ERR_INVALID_ARG, "%s: gu must be a 16-byte aligned buffer", name);
+    ATS_REQUIRE(ats_grouped_down_dgrad_dsilu_nn_supported(E, max_rows, H, I, dtype), ATS_ERR_UNSUPPORTED,
+                "%s: bfloat16 with more than %lld rows per expert on average, H a multiple of 64, I of 8 and one expert's "
+                "weights within 4 GiB (E=%d max_rows=%lld H=%d I=%d dtype=%d); use ats_grouped_down_dgrad_dsilu on "
+                "transposed weights", name, (long long)kDsiluMinAvgRows, E, (long long)max_rows, H, I, dtype);
+    if (max_rows == 0) return ATS_OK;
+    GroupedArgs p{};
+    p.a = dy;
+    p.a_row_div = 1;
+    p.lda = H;
+    p.b = w_d;
+    p.ldb = I;
+    p.out = dgu;
+    p.ldo = 2 * (int64_t)I;
+    p.gu_out = const_cast<void*>(gu);
+    p.ld_gu = 2 * (int64_t)I;
+    p.t_out = dgu_t;
+    p.ld_t = ld_t;
+    p.t_col0 = t_col0;
+    p.row_start = row_start;
+    p.row_count = row_count;
+    p.E = E;
+    p.K = H;
+    p.N_out = I;
+    p.up_offset = I;
+    p.a_extent_bytes = 0xffffffffu;       // the descriptor starts at the tile's first row
+    p.b_extent_bytes = extent32(H, I, 2);
+    rc = launch_kmajor<bf16_t, true>(p, max_rows, as_stream(stream));
+    if (rc != ATS_OK) return rc;
+    ATS_CHECK_LAUNCH(name);
+    return ATS_OK;
+}
+
+extern "C" int ats_grouped_gemm_nn_supported(int E, int64_t max_rows, int N, int K, int64_t ldb, int dtype) {
+    using namespace ats;
+    if (N <= 0 || K <= 0 || dtype != ATS_BF16) return 0;
+    return kmajor_supported(E, max_rows, N, K, ldb, 192) ? 1 : 0;
+}
+extern "C" int ats_grouped_gemm_nn(const void* a, int64_t lda, int64_t a_num_rows, const int32_t* a_rows, int a_row_div,
+                                   const void* const* b_ptrs, int64_t ldb, void* out, int64_t ldo,
+                                   const int32_t* row_start, const int32_t* row_count, int E, int64_t max_rows, int N,
+                                   int K, int dtype, int out_dtype, ats_stream_t stream) {
+    using namespace ats;
+    const char* name = "ats_grouped_gemm_nn";
+    ATS_REQUIRE(E > 0 && E <= 4096 && max_rows >= 0 && N > 0 && K > 0, ATS_ERR_INVALID_ARG,
+                "%s: E=%d max_rows=%lld N=%d K=%d", name, E, (long long)max_rows, N, K);
+    ATS_REQUIRE(dtype == ATS_BF16 && (out_dtype == ATS_F32 || out_dtype == ATS_BF16), ATS_ERR_UNSUPPORTED,
+                "%s: dtype tags %d -> %d (bfloat16 operands, bfloat16 or float32 out)", name, dtype, out_dtype);
+    ATS_REQUIRE(a && b_ptrs && out && row_start && row_count, ATS_ERR_INVALID_ARG, "%s: null pointer", name);
+    ATS_REQUIRE(!a_rows || (a_row_div > 0 && a_num_rows > 0), ATS_ERR_INVALID_ARG, "%s: a_row_div=%d a_num_rows=%lld",
+                name, a_row_div, (long long)a_num_rows);
+    const int ovec = out_dtype == ATS_F32 ? 4 : 8;
+    ATS_REQUIRE(lda % 8 == 0 && lda >= K && N % ovec == 0 && ldo % ovec == 0 && ldo >= N, ATS_ERR_UNSUPPORTED,
+                "%s: K=%d N=%d lda=%lld ldo=%lld must describe 16-byte aligned rows", name, K, N, (long long)lda,
+                (long long)ldo);
+    ATS_REQUIRE(aligned16(a) && aligned16(out), ATS_ERR_INVALID_ARG, "%s: operands must be 16-byte aligned", name);
+    ATS_REQUIRE(ats_grouped_gemm_nn_supported(E, max_rows, N, K, ldb, dtype), ATS_ERR_UNSUPPORTED,
+                "%s: more than 192 rows per expert on average, K a multiple of 64, N and ldb of 8 and one expert's weights "
+                "within 4 GiB (E=%d max_rows=%lld N=%d K=%d ldb=%lld); use ats_grouped_gemm_nt on transposed weights", name,
+                E, (long long)max_rows, N, K, (long long)ldb);
+    if (max_rows == 0) return ATS_OK;
+    GroupedArgs p{};
+    p.a = a;
+    p.a_rows = a_rows;
+    p.a_row_div = a_rows ? a_row_div : 1;
+    p.lda = lda;
+    p.b = b_ptrs;
+    p.ldb = ldb;
+    p.out = out;
+    p.ldo = ldo;
+    p.row_start = row_start;
+    p.row_count = row_count;
+    p.E = E;
+    p.K = K;
+    p.N_out = N;
+    p.up_offset = 0;
+    p.a_extent_bytes = a_rows ? extent32(a_num_rows, lda, 2) : 0xffffffffu;
+    p.b_extent_bytes = extent32(K, ldb, 2);
+    ATS_REQUIRE(p.a_extent_bytes != 0, ATS_ERR_UNSUPPORTED, "%s: the gathered operand must stay within 4 GiB", name);
+    hipStream_t s = as_stream(stream);
+    const int rc = out_dtype == ATS_F32 ? launch_kmajor<float, false>(p, max_rows, s)
+                                        : launch_kmajor<bf16_t, false>(p, max_rows, s);
+    if (rc != ATS_OK) return rc;
+    ATS_CHECK_LAUNCH(name);
     return ATS_OK;
 }
 

@@ -348,15 +348,24 @@ def _transposed_copy_buffer(C: int, row_count: torch.Tensor, t_col0: Optional[to
     return out, ld
 
 
+def grouped_down_dgrad_dsilu_supported(E: int, max_rows: int, H: int, I: int, dtype: torch.dtype,
+                                       transposed_weights: bool = True) -> bool:
+    """Whether grouped_down_dgrad_dsilu has a kernel for these sizes (with the transposed, or the forward's own, weights)."""
+    lib = _lib.load()
+    fn = lib.ats_grouped_down_dgrad_dsilu_supported if transposed_weights else lib.ats_grouped_down_dgrad_dsilu_nn_supported
+    return bool(fn(int(E), int(max_rows), int(H), int(I), _DT[dtype]))
+
+
 def grouped_down_dgrad_dsilu(dy: torch.Tensor, w_dT_ptrs: torch.Tensor, gu: torch.Tensor, row_start: torch.Tensor,
                              row_count: torch.Tensor, max_rows: int, H: int, I: int,
-                             t_col0: Optional[torch.Tensor] = None
+                             t_col0: Optional[torch.Tensor] = None, transposed_weights: bool = True
                              ) -> Optional[Tuple[torch.Tensor, Optional[torch.Tensor]]]:
     """Training backward of the down projection and of silu(g) * u in one kernel: (dgu [rows, 2I], dguT) from
     dy [rows, H], the transposed down weights ([I, H] per expert) and the saved gu; None when the groups are not
     prefill-sized (the caller then runs the plain product and silu_mul_bwd).  dguT is None unless t_col0 (the
     k_start of wgrad_plan) is given and the dtype is bfloat16: then it is dgu transposed into the weight-gradient
-    layout [2I, wgrad_padded_rows], written by the same kernel."""
+    layout [2I, wgrad_padded_rows], written by the same kernel.  transposed_weights=False: the pointer table holds
+    the forward's own down weights ([H, I] per expert; bfloat16, ats_grouped_down_dgrad_dsilu_nn)."""
     _need_gpu(dy, w_dT_ptrs, gu, row_start, row_count)
     if dy.dim() != 2 or dy.shape[1] != H or not dy.is_contiguous():
         raise AtsError("grouped_down_dgrad_dsilu: dy must be a contiguous [rows, H] tensor")
@@ -366,14 +375,15 @@ def grouped_down_dgrad_dsilu(dy: torch.Tensor, w_dT_ptrs: torch.Tensor, gu: torc
     if row_start.numel() < E or row_count.numel() < E or row_start.dtype != torch.int32 or row_count.dtype != torch.int32:
         raise AtsError("grouped_down_dgrad_dsilu: row_start/row_count must be int32 with one entry per expert")
     lib = _lib.load()
-    if not lib.ats_grouped_down_dgrad_dsilu_supported(E, int(max_rows), H, I, _tag(dy)):
+    if not grouped_down_dgrad_dsilu_supported(E, max_rows, H, I, dy.dtype, transposed_weights):
         return None
     dgu = torch.empty_like(gu)
     dguT, ld = _transposed_copy_buffer(2 * I, row_count, t_col0, max_rows, E, dy.dtype, dy.device)
-    check(lib.ats_grouped_down_dgrad_dsilu(dy.data_ptr(), w_dT_ptrs.data_ptr(), gu.data_ptr(), dgu.data_ptr(),
-                                           row_start.data_ptr(), row_count.data_ptr(), E, int(max_rows), H, I,
-                                           _tag(dy), _ptr(dguT), ld, _ptr(t_col0) if dguT is not None else None,
-                                           _stream()), "ats_grouped_down_dgrad_dsilu")
+    fn = lib.ats_grouped_down_dgrad_dsilu if transposed_weights else lib.ats_grouped_down_dgrad_dsilu_nn
+    check(fn(dy.data_ptr(), w_dT_ptrs.data_ptr(), gu.data_ptr(), dgu.data_ptr(), row_start.data_ptr(),
+             row_count.data_ptr(), E, int(max_rows), H, I, _tag(dy), _ptr(dguT), ld,
+             _ptr(t_col0) if dguT is not None else None, _stream()),
+          "ats_grouped_down_dgrad_dsilu" if transposed_weights else "ats_grouped_down_dgrad_dsilu_nn")
     return dgu, dguT
 
 
@@ -854,6 +864,31 @@ def grouped_gemm_nt(b_ptrs: torch.Tensor, ldb: int, b_rows: int, row_start: torc
                                           out.data_ptr(), N, row_start.data_ptr(), row_count.data_ptr(), _ptr(k_count),
                                           E, int(max_rows), int(N), int(K), _DT[dtype], _DT[out_dtype], _stream()),
           "ats_grouped_gemm_nt")
+    return out
+
+
+def grouped_gemm_nn_supported(E: int, max_rows: int, N: int, K: int, ldb: int, dtype: torch.dtype) -> bool:
+    """Whether grouped_gemm_nn has a kernel for these sizes (bfloat16, prefill-sized groups)."""
+    if dtype not in _DT:
+        return False
+    return bool(_lib.load().ats_grouped_gemm_nn_supported(int(E), int(max_rows), int(N), int(K), int(ldb), _DT[dtype]))
+
+
+def grouped_gemm_nn(b_ptrs: torch.Tensor, ldb: int, row_start: torch.Tensor, row_count: torch.Tensor, n_rows_out: int,
+                    max_rows: int, N: int, K: int, a: torch.Tensor, a_rows: Optional[torch.Tensor] = None,
+                    a_row_div: int = 1, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """out[row_start[e]+m, :N] = A_e[m, :K] @ B_e[:K, :N] with B_e = b_ptrs[e] stored [K, ldb] (see
+    ats_grouped_gemm_nn): the data gradient of a linear layer against the weights as the forward holds them."""
+    _need_gpu(a, b_ptrs, row_start, row_count, a_rows)
+    a = _rows_2d(a, "grouped_gemm_nn")
+    out_dtype = a.dtype if out_dtype is None else out_dtype
+    E = b_ptrs.numel()
+    out = torch.empty(n_rows_out, N, dtype=out_dtype, device=b_ptrs.device)
+    check(_lib.load().ats_grouped_gemm_nn(a.data_ptr(), int(a.stride(0)), int(a.shape[0]), _ptr(a_rows), int(a_row_div),
+                                          b_ptrs.data_ptr(), int(ldb), out.data_ptr(), N, row_start.data_ptr(),
+                                          row_count.data_ptr(), E, int(max_rows), int(N), int(K), _DT[a.dtype],
+                                          _DT[out_dtype], _stream()),
+          "ats_grouped_gemm_nn")
     return out
 
 

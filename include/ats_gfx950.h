@@ -196,6 +196,14 @@ int ats_grouped_down_dgrad_dsilu(const void* dy, const void* const* w_dT, const 
                                  const int32_t* row_start, const int32_t* row_count, int E, int64_t max_rows,
                                  int H, int I, int dtype, void* dgu_t, int64_t ld_t, const int32_t* t_col0,
                                  ats_stream_t stream);
+/* The same kernel reading the forward's own weights w_d[e] = [H, I] (reduction index H along the rows): no
+ * transposed copy of the weights per step, the same bits.  bfloat16 only; ..._supported as above with H a
+ * multiple of 64 and I of 8 (reference: autograd's down_proj input gradient, MS/core/model.py:882-893). */
+int ats_grouped_down_dgrad_dsilu_nn_supported(int E, int64_t max_rows, int H, int I, int dtype);
+int ats_grouped_down_dgrad_dsilu_nn(const void* dy, const void* const* w_d, const void* gu, void* dgu,
+                                    const int32_t* row_start, const int32_t* row_count, int E, int64_t max_rows,
+                                    int H, int I, int dtype, void* dgu_t, int64_t ld_t, const int32_t* t_col0,
+                                    ats_stream_t stream);
 /* The same projection for a training step: beside h it writes the gate / up pre-activations
  * gu[r, 0:I] and gu[r, I:2I] ([rows, 2I] of dtype, rounded from the same accumulators), which the
  * backward pass needs; replaces the plain product followed by ats_silu_mul_fwd (reference: the
@@ -380,6 +388,18 @@ int ats_grouped_gemm_nt(const void* a, const void* const* a_ptrs, int64_t lda, i
                         int64_t b_rows, void* out, int64_t ldo, const int32_t* row_start,
                         const int32_t* row_count, const int32_t* k_count, int E, int64_t max_rows, int N,
                         int K, int dtype, int out_dtype, ats_stream_t stream);
+/* Grouped product against weights stored with the reduction index along their rows:
+ * out[row_start[e]+m, n] = sum_k A_e[m,k] * B_e[k,n], B_e = b_ptrs[e] ([K, ldb >= N]).
+ * The data gradient of a linear layer, dX = dY . W with W = [out_features, in_features] as the forward holds it
+ * (autograd's input gradient of nn.Linear, MS/core/model.py:882-893), without a transposed copy of W; same bits
+ * as ats_grouped_gemm_nt on the transposed copy.  bfloat16 operands, prefill-sized groups only: ..._supported
+ * returns 1 for more than 192 rows per expert on average, K a multiple of 64, N and ldb multiples of 8 and one
+ * expert's weights within 4 GiB; otherwise transpose (ats_transpose_batched) and call ats_grouped_gemm_nt. */
+int ats_grouped_gemm_nn_supported(int E, int64_t max_rows, int N, int K, int64_t ldb, int dtype);
+int ats_grouped_gemm_nn(const void* a, int64_t lda, int64_t a_num_rows, const int32_t* a_rows, int a_row_div,
+                        const void* const* b_ptrs, int64_t ldb, void* out, int64_t ldo, const int32_t* row_start,
+                        const int32_t* row_count, int E, int64_t max_rows, int N, int K, int dtype, int out_dtype,
+                        ats_stream_t stream);
 
 /* ---- Causal grouped-query attention (forward) -----------------------------------
  * Replaces GroupedQueryAttention._standard_attention / _flash_attention

@@ -1039,6 +1039,54 @@ def test_grouped_gateup_with_saved_preactivations(ops, gpu, counts, H, I, gather
     assert ops.grouped_gateup_swiglu_save(a, tab, start, small, n, 40 * E, H, I, **kw) is None
 
 
+@pytest.mark.parametrize("counts,K,N", [([900, 0, 300, 1001], 256, 392), ([2100, 777], 1024, 512), ([300], 128, 136),
+                                        ([1024, 1, 1279, 64, 0, 193], 192, 200), ([513], 64, 8), ([700, 700], 448, 1000)])
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
+def test_grouped_gemm_against_k_major_weights(ops, gpu, counts, K, N, out_dtype):
+    """out = A . B with B stored [K, N] (the forward's weights in a data gradient): the bits of the NT product
+    against the transposed copy, agreement with float64, rows outside the groups untouched, gathered A rows,
+    and the sizes it declines."""
+    print("case gemm nn", counts, K, N, out_dtype, flush=True)
+    g = gen(167)
+    E, n = len(counts), sum(counts)
+    w = [(torch.randn(K, N, generator=g) * 0.05).bfloat16().to(gpu) for _ in range(E)]
+    wT = [x.t().contiguous() for x in w]
+    tab, tabT = ops.weight_pointer_table(w), ops.weight_pointer_table(wT)
+    count = torch.tensor(counts, dtype=torch.int32)
+    start = (torch.cumsum(count, 0) - count).to(torch.int32).to(gpu)
+    count = count.to(gpu)
+    a = torch.randn(n + 3, K, generator=g).bfloat16().to(gpu)
+    assert ops.grouped_gemm_nn_supported(E, n, N, K, N, torch.bfloat16)
+    out = ops.grouped_gemm_nn(tab, N, start, count, n + 3, n, N, K, a, out_dtype=out_dtype)
+    ref = ops.grouped_gemm_nt(tabT, K, N, start, count, n + 3, n, N, K, a=a, out_dtype=out_dtype)
+    assert out.dtype == out_dtype and same_bits(out[:n], ref[:n])
+    off = 0
+    for e, c in enumerate(counts):
+        if c:
+            r64 = a[off:off + c].cpu().double() @ w[e].cpu().double()
+            assert rel_err(out[off:off + c], r64) <= BF16_TOL
+        off += c
+    # gathered rows of A (row m of the product reads a[src[m] // 2])
+    src = torch.randint(0, 2 * (n + 3), (n,), generator=g).to(torch.int32).to(gpu)
+    got = ops.grouped_gemm_nn(tab, N, start, count, n, n, N, K, a, a_rows=src, a_row_div=2, out_dtype=out_dtype)
+    want = ops.grouped_gemm_nn(tab, N, start, count, n, n, N, K, a[(src // 2).long()].contiguous(), out_dtype=out_dtype)
+    assert same_bits(got, want)
+    # rows beyond the groups are not written
+    lib = __import__("adaptivetrainingsystem_amd._lib", fromlist=["load"]).load()
+    buf = torch.full((n + 3, N), 7.0, dtype=out_dtype, device=gpu)
+    rc = lib.ats_grouped_gemm_nn(a.data_ptr(), K, n + 3, None, 1, tab.data_ptr(), N, buf.data_ptr(), N, start.data_ptr(),
+                                 count.data_ptr(), E, n, N, K, 1, 0 if out_dtype == torch.float32 else 1, None)
+    assert rc == 0
+    torch.cuda.synchronize()
+    assert torch.all(buf[n:] == 7.0) and same_bits(buf[:n], ref[:n])
+    # declined: decode-sized groups, float32 operands, K not a multiple of 64
+    assert not ops.grouped_gemm_nn_supported(E, 40 * E, N, K, N, torch.bfloat16)
+    assert not ops.grouped_gemm_nn_supported(E, n, N, K, N, torch.float32)
+    assert not ops.grouped_gemm_nn_supported(E, n, N, K + 8, N, torch.bfloat16)
+    assert lib.ats_grouped_gemm_nn(a.data_ptr(), K, n + 3, None, 1, tab.data_ptr(), N, buf.data_ptr(), N, start.data_ptr(),
+                                   count.data_ptr(), E, 40 * E, N, K, 1, 1, None) == -2
+
+
 @pytest.mark.parametrize("counts,H,I", [([900, 0, 300, 1001], 256, 392), ([2100, 777], 512, 1024), ([300], 128, 136),
                                         ([1024, 1, 1279, 64, 0, 193], 128, 200)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -1087,6 +1135,16 @@ def test_grouped_down_dgrad_with_swiglu_gradient(ops, gpu, counts, H, I, dtype):
             ref = torch.cat([dh64 * u64 * (s64 + g64 * s64 * (1 - s64)), dh64 * g64 * s64], dim=1)
             assert rel_err(dgu[off:off + c], ref) <= (F32_TOL if dtype == torch.float32 else BF16_TOL)
         off += c
+    # the forward's own weights ([H, I] per expert) instead of the transposed copy: bfloat16, H a multiple of 64
+    wd = [x.t().contiguous() for x in wdT]
+    nn = ops.grouped_down_dgrad_dsilu(dy, ops.weight_pointer_table(wd), gu, start, count, n, H, I, t_col0=ks,
+                                      transposed_weights=False)
+    assert (nn is not None) == (dtype == torch.bfloat16 and H % 64 == 0)
+    if nn is not None:
+        assert same_bits(nn[0][:n], dgu[:n])
+        for e in range(E):
+            lo, width = int(ks[e]), int(kc[e])
+            assert same_bits(nn[1][:, lo:lo + width], dguT[:, lo:lo + width]), e
     lib = __import__("adaptivetrainingsystem_amd._lib", fromlist=["load"]).load()
     dgu.fill_(3.0)
     rc = lib.ats_grouped_down_dgrad_dsilu(dy.data_ptr(), tab.data_ptr(), gu.data_ptr(), dgu.data_ptr(), start.data_ptr(),
