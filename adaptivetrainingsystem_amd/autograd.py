@@ -137,8 +137,8 @@ class AttentionF32Function(Function):
 
 class LinearFunction(Function):
     """y = x @ weight^T for x [T, K], weight [N, K] (a bias-free nn.Linear) through the grouped GEMM kernels
-    with one group: dgrad multiplies by a transposed copy of the weight, wgrad multiplies the transposed
-    activations."""
+    with one group: dgrad reads the weight as it is where the K-major kernel applies (bfloat16, more than 192
+    rows) and multiplies by a transposed copy otherwise, wgrad multiplies the transposed activations."""
 
     @staticmethod
     def forward(ctx, x, weight):
@@ -158,8 +158,11 @@ class LinearFunction(Function):
         offsets = torch.tensor([0, T], dtype=torch.int32, device=x.device)
         kept = offsets[1:].clone()
         if ctx.needs_input_grad[0]:
-            wT, tab = ops.transpose_batched([w])                 # [K, N]; kept alive until the GEMM is queued
-            dx = ops.grouped_gemm_nt(tab, N, K, offsets, kept, T, T, K, N, a=dy)
+            if DGRAD_FROM_FORWARD_WEIGHTS and ops.grouped_gemm_nn_supported(1, T, K, N, K, x.dtype):
+                dx = ops.grouped_gemm_nn(ops.weight_pointer_table([w]), K, offsets, kept, T, T, K, N, dy)
+            else:
+                wT, tab = ops.transpose_batched([w])             # [K, N]; kept alive until the GEMM is queued
+                dx = ops.grouped_gemm_nt(tab, N, K, offsets, kept, T, T, K, N, a=dy)
         if ctx.needs_input_grad[1]:
             ks, kc = ops.wgrad_plan(kept)
             ld = ops.wgrad_padded_rows(T, 1)
