@@ -88,6 +88,54 @@ def test_linear_random_shapes(gpu, T, N, K, dtype):
     assert rel_err(got, x.double() @ w.double().T) <= (1e-5 if dtype == torch.float32 else BF16_TOL)
 
 
+def _kmajor_cases(n, seed):
+    rng = np.random.default_rng(seed)
+    cases = []
+    for _ in range(n):
+        E = int(rng.integers(1, 7))
+        counts = [int(c) for c in rng.integers(0, 900, E)]
+        counts[int(rng.integers(0, E))] += 193 * E        # the K-major kernel serves groups above 192 rows on average
+        K = int(rng.integers(1, 17)) * 64
+        N = int(rng.integers(1, 150)) * 8
+        pad = int(rng.choice([0, 0, 8, 64]))
+        cases.append((counts, K, N, pad, bool(rng.integers(0, 2)), bool(rng.integers(0, 2))))
+    return cases
+
+
+@pytest.mark.parametrize("counts,K,N,pad,gather,f32_out", _kmajor_cases(16 * SCALE, 23))
+def test_kmajor_product_random_shapes(gpu, counts, K, N, pad, gather, f32_out):
+    """Grouped product against weights stored [K, N] (row stride N + pad): float64 reference and the bits of the NT
+    product against a transposed copy, over random group sizes, tile remainders in N, K from one slab upwards."""
+    from adaptivetrainingsystem_amd import ops
+    print("case random k-major", counts, K, N, pad, gather, f32_out, flush=True)
+    E, n = len(counts), sum(counts)
+    g = torch.Generator().manual_seed(n * 31 + K * 7 + N)
+    ldb = N + pad
+    store = [(torch.randn(K, ldb, generator=g) * 0.05).bfloat16().to(gpu) for _ in range(E)]
+    w = [x[:, :N] for x in store]                                   # [K, N] views with row stride ldb
+    wT = [x.t().contiguous() for x in w]
+    tab = torch.tensor([x.data_ptr() for x in store], dtype=torch.int64, device=gpu)
+    tabT = ops.weight_pointer_table(wT)
+    count = torch.tensor(counts, dtype=torch.int32)
+    start = (torch.cumsum(count, 0) - count).to(torch.int32).to(gpu)
+    count = count.to(gpu)
+    src_rows = n + 5
+    a = torch.randn(src_rows, K, generator=g).bfloat16().to(gpu)
+    rows = torch.randint(0, 3 * src_rows, (n,), generator=g).to(torch.int32).to(gpu) if gather else None
+    a_used = a[(rows // 3).long()] if gather else a[:n]
+    out_dtype = torch.float32 if f32_out else torch.bfloat16
+    assert ops.grouped_gemm_nn_supported(E, n, N, K, ldb, torch.bfloat16)
+    out = ops.grouped_gemm_nn(tab, ldb, start, count, n, n, N, K, a, a_rows=rows, a_row_div=3, out_dtype=out_dtype)
+    ref = ops.grouped_gemm_nt(tabT, K, N, start, count, n, n, N, K, a=a_used.contiguous(), out_dtype=out_dtype)
+    assert torch.equal(out, ref)
+    off = 0
+    for e, c in enumerate(counts):
+        if c:
+            r64 = a_used[off:off + c].cpu().double() @ w[e].cpu().double()
+            assert rel_err(out[off:off + c], r64) <= BF16_TOL
+        off += c
+
+
 def _layer_cases(n, seed):
     rng = np.random.default_rng(seed)
     cases = []
