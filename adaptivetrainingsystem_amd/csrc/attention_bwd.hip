@@ -142,6 +142,10 @@ __device__ __forceinline__ bu32x4_t tr_fragment_swz(blds_u8_t tile, int lo_off, 
 // are double buffered: the loads of tile t+1 are issued before the arithmetic of tile t and have the whole
 // iteration to land (one barrier per tile).
 // EXTRA: pair bias and / or dropout (attention_extra.hpp), the same decisions as the forward made.
+// The tile functions of both kernels are inlined functions with __restrict__ pointer parameters, and that is load
+// bearing: it gives the transposing LDS reads alias metadata, without which the compiler waits for every
+// direct-to-LDS load in flight (s_waitcnt vmcnt(0)) before each ds_read_b64_tr_b16 (see grouped_gemm.hip, where the
+// same builtin first came without it).
 template <int D, bool BIAS, bool EXTRA = false>
 __device__ __forceinline__ void attention_bwd_dq_tile(const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
                                                       const bf16_t* __restrict__ v, const bf16_t* __restrict__ dout,
